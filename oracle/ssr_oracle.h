@@ -1,0 +1,107 @@
+/* ssr_oracle.h -- C interface of the CPU oracle.
+ *
+ * TEST INFRASTRUCTURE ONLY. This library restates, on the CPU, the algorithm of the reference's
+ * Gaussian-splat hot path (projection + SH colour, tile keys, sort, tile ranges, compositing
+ * forward, compositing backward, projection backward). It exists to check the HIP kernels; the
+ * product library never links, loads or calls it. Only tests, the smoke check and the
+ * cpu_baseline leg of the benchmark may use it.
+ *
+ * Every pointer is a host pointer. Arrays use the reference's layouts
+ * (src/primitives/PrimitiveBase3DGS.cuh:87-139,187-225):
+ *   world:  means[N,3] quats[N,4](w,x,y,z) log_scales[N,3] opacity_logits[N] features_dc[N,3]
+ *           features_sh[N,15,3]
+ *   screen: xy[N,2] depth[N] conic[N,3] opac[N] rgb[N,3]
+ */
+#pragma once
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { OR_CAM_PINHOLE = 0, OR_CAM_EQUIRECT = 3 };            /* src/core/Common.cuh CameraModelType */
+enum { OR_SH_F32 = 0, OR_SH_REF_Q8 = 1, OR_SH_REF_Q16 = 2, OR_SH_I8_F16SCALE = 3 };
+
+typedef struct {
+    int32_t model;          /* OR_CAM_* */
+    uint32_t width, height;
+    float viewmat[16];      /* row-major world->camera [R t; 0 1] */
+    float fx, fy, cx, cy;
+} or_camera;
+
+typedef struct {
+    int32_t codec;          /* OR_SH_* */
+    const float* sh_f32;    /* [N,15,3] when codec == OR_SH_F32 */
+    const uint8_t* packed;  /* ref q8: uint8[N*3*num_sh_buffer]; ref q16: uint16; i8: int8[N*45] */
+    const float* bounds;    /* ref codecs: float2[n_bounds] (min,max) */
+    int64_t bounds_stride;  /* cells per bound; 0 selects 256*3*num_sh_buffer */
+    uint32_t num_sh_buffer; /* coefficients per splat in the packed buffer (15 for SH3) */
+    const uint16_t* scale_f16; /* i8 codec: fp16 bits, one per splat */
+} or_sh_source;
+
+/* K1. Outputs: aabb[N,4], sort_depth[N], radii[N] (max-accumulated), screen rows. Rows of culled
+ * splats are left untouched, as the reference leaves them. Returns the number of visible splats. */
+int64_t or_projection_fwd(int64_t N, int sh_degree,
+    const float* means, const float* quats, const float* log_scales, const float* opacity_logits,
+    const float* features_dc, const or_sh_source* sh, const or_camera* cam,
+    float* aabb, float* sort_depth, float* radii,
+    float* xy, float* depth, float* conic, float* opac, float* rgb);
+
+/* K2 */
+void or_tile_count(int64_t N, const float* aabb, const float* xy, const float* conic,
+    const float* opac, uint32_t width, uint32_t height, int64_t* tiles_per_splat);
+/* K3 */
+void or_inclusive_sum_i64(int64_t n, const int64_t* in, int64_t* out);
+/* K4. Returns the number of 0xffffffff pad keys written (0 when count and write agree). */
+int64_t or_tile_write(int64_t N, const float* aabb, const float* sort_depth, const float* xy,
+    const float* conic, const float* opac, const int64_t* cum_tiles, uint32_t width,
+    uint32_t height, int64_t* isect_ids, int32_t* flatten_ids);
+/* K5: stable sort on bits [begin_bit, end_bit) of the key. */
+void or_sort_pairs(int64_t n, const int64_t* keys_in, const int32_t* vals_in, int begin_bit,
+    int end_bit, int64_t* keys_out, int32_t* vals_out);
+/* K6 */
+void or_tile_offsets(int64_t n_isects, const int64_t* sorted_ids, uint32_t n_tiles,
+    int32_t* offsets);
+
+/* K7. stats (optional, 2 entries): K_f and K_b as defined for the bandwidth model. */
+void or_raster_fwd(int64_t N, const float* xy, const float* depth, const float* conic,
+    const float* opac, const float* rgb, uint32_t width, uint32_t height,
+    const int32_t* tile_offsets, const int32_t* flatten_ids, int64_t n_isects,
+    float* out_rgb, float* out_depth, float* out_T, int32_t* out_last_ids, int64_t* stats);
+
+/* K8. v_* outputs are ACCUMULATED into (caller zero-fills). abs_* (optional, may be NULL) receive
+ * the sum of absolute values of the same terms in double, as an error scale for comparisons. */
+void or_raster_bwd(int64_t N, const float* xy, const float* depth, const float* conic,
+    const float* opac, const float* rgb, uint32_t width, uint32_t height,
+    const int32_t* tile_offsets, const int32_t* flatten_ids, int64_t n_isects,
+    const float* render_T, const int32_t* last_ids, const float* render_depth,
+    const float* v_rgb, const float* v_depth, const float* v_T,
+    float* v_xy, float* v_sdepth, float* v_conic, float* v_opac, float* v_srgb,
+    double* abs_terms /* [N,10] or NULL */);
+
+/* K9. Gradients are ACCUMULATED into v_* (caller zero-fills). */
+void or_projection_bwd(int64_t N, int sh_degree,
+    const float* means, const float* quats, const float* log_scales, const float* opacity_logits,
+    const float* features_dc, const or_sh_source* sh, const or_camera* cam, const float* aabb,
+    const float* v_xy, const float* v_sdepth, const float* v_conic, const float* v_opac,
+    const float* v_srgb,
+    float* v_means, float* v_quats, float* v_scales, float* v_opacities, float* v_dc, float* v_sh);
+
+/* Codecs (src/core/Tensor.h:1364-1392): block-wise (min,max) + uint8/uint16 codes. */
+void or_quantize_ref(int bits, int64_t n_cells, int64_t bounds_stride, const float* values,
+    uint8_t* packed, float* bounds /* float2[ceil(n_cells/stride)] */);
+/* int8 codes with one fp16 scale per splat: v = code * scale. */
+void or_quantize_i8_f16(int64_t N, int cells_per_splat, const float* values, int8_t* codes,
+    uint16_t* scale_f16);
+void or_decode_sh(int64_t gid, const or_sh_source* sh, float* out45);
+
+/* Transcendentals of include/ssr_math.h evaluated elementwise (op: 0 exp, 1 log, 2 atan2(a,b),
+ * 3 sigmoid), for checking them against libm and against the device. */
+void or_math(int op, int64_t n, const float* a, const float* b, float* out);
+
+int or_num_threads(void);
+void or_set_num_threads(int n);
+
+#ifdef __cplusplus
+}
+#endif

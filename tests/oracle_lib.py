@@ -1,0 +1,216 @@
+"""ctypes binding of the CPU oracle (oracle/libssr_oracle.so). Test infrastructure only."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+_SO = os.path.join(_ROOT, "oracle", "libssr_oracle.so")
+
+
+class OrCamera(C.Structure):
+    _fields_ = [("model", C.c_int32), ("width", C.c_uint32), ("height", C.c_uint32),
+                ("viewmat", C.c_float * 16), ("fx", C.c_float), ("fy", C.c_float),
+                ("cx", C.c_float), ("cy", C.c_float)]
+
+
+class OrShSource(C.Structure):
+    _fields_ = [("codec", C.c_int32), ("sh_f32", C.c_void_p), ("packed", C.c_void_p),
+                ("bounds", C.c_void_p), ("bounds_stride", C.c_int64),
+                ("num_sh_buffer", C.c_uint32), ("scale_f16", C.c_void_p)]
+
+
+def build():
+    subprocess.check_call(["make", "-s", "-C", os.path.join(_ROOT, "oracle")])
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            build()
+        _lib = C.CDLL(_SO)
+        _lib.or_projection_fwd.restype = C.c_int64
+        _lib.or_tile_write.restype = C.c_int64
+        _lib.or_num_threads.restype = C.c_int
+    return _lib
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def camera_of(scene) -> OrCamera:
+    cam = OrCamera()
+    cam.model = scene.camera_model
+    cam.width, cam.height = scene.width, scene.height
+    vm = np.ascontiguousarray(scene.viewmat, np.float32).reshape(-1)
+    for i in range(16):
+        cam.viewmat[i] = float(vm[i])
+    cam.fx, cam.fy, cam.cx, cam.cy = [float(v) for v in scene.intrins]
+    return cam
+
+
+def sh_source_of(scene, keep):
+    """keep: list that receives arrays which must outlive the struct."""
+    s = OrShSource()
+    s.codec = scene.sh_codec
+    s.num_sh_buffer = 15
+    s.bounds_stride = scene.sh_bounds_stride
+    if scene.sh_codec == 0:
+        a = np.ascontiguousarray(scene.features_sh, np.float32)
+        keep.append(a)
+        s.sh_f32 = a.ctypes.data
+    else:
+        a = np.ascontiguousarray(scene.sh_packed)
+        keep.append(a)
+        s.packed = a.ctypes.data
+        if scene.sh_bounds is not None:
+            b = np.ascontiguousarray(scene.sh_bounds, np.float32)
+            keep.append(b)
+            s.bounds = b.ctypes.data
+        if scene.sh_scale_f16 is not None:
+            h = np.ascontiguousarray(scene.sh_scale_f16.view(np.uint16))
+            keep.append(h)
+            s.scale_f16 = h.ctypes.data
+    return s
+
+
+def math(op, a, b=None):
+    a = np.ascontiguousarray(a, np.float32)
+    b = np.ascontiguousarray(a if b is None else b, np.float32)
+    out = np.empty_like(a)
+    lib().or_math(C.c_int(op), C.c_int64(a.size), _p(a), _p(b), _p(out))
+    return out
+
+
+def projection_fwd(scene, sh_degree=3):
+    n = scene.n
+    keep = []
+    cam, sh = camera_of(scene), sh_source_of(scene, keep)
+    o = dict(aabb=np.zeros((n, 4), np.float32), sort_depth=np.zeros(n, np.float32),
+             radii=np.zeros(n, np.float32), xy=np.zeros((n, 2), np.float32),
+             depth=np.zeros(n, np.float32), conic=np.zeros((n, 3), np.float32),
+             opac=np.zeros(n, np.float32), rgb=np.zeros((n, 3), np.float32))
+    o["visible"] = lib().or_projection_fwd(
+        C.c_int64(n), C.c_int(sh_degree), _p(scene.means), _p(scene.quats), _p(scene.log_scales),
+        _p(scene.opacity_logits), _p(scene.features_dc), C.byref(sh), C.byref(cam),
+        _p(o["aabb"]), _p(o["sort_depth"]), _p(o["radii"]), _p(o["xy"]), _p(o["depth"]),
+        _p(o["conic"]), _p(o["opac"]), _p(o["rgb"]))
+    return o
+
+
+def tile_count(n, aabb, xy, conic, opac, w, h):
+    out = np.zeros(n, np.int64)
+    lib().or_tile_count(C.c_int64(n), _p(aabb), _p(xy), _p(conic), _p(opac), C.c_uint32(w),
+                        C.c_uint32(h), _p(out))
+    return out
+
+
+def inclusive_sum(a):
+    a = np.ascontiguousarray(a, np.int64)
+    out = np.empty_like(a)
+    lib().or_inclusive_sum_i64(C.c_int64(a.size), _p(a), _p(out))
+    return out
+
+
+def tile_write(n, aabb, sort_depth, xy, conic, opac, cum, w, h):
+    k = int(cum[-1]) if n else 0
+    ids = np.zeros(k, np.int64)
+    flat = np.zeros(k, np.int32)
+    pads = lib().or_tile_write(C.c_int64(n), _p(aabb), _p(sort_depth), _p(xy), _p(conic), _p(opac),
+                               _p(cum), C.c_uint32(w), C.c_uint32(h), _p(ids), _p(flat))
+    return ids, flat, pads
+
+
+def sort_pairs(keys, vals, begin_bit, end_bit):
+    keys = np.ascontiguousarray(keys, np.int64)
+    vals = np.ascontiguousarray(vals, np.int32)
+    ko, vo = np.empty_like(keys), np.empty_like(vals)
+    lib().or_sort_pairs(C.c_int64(keys.size), _p(keys), _p(vals), C.c_int(begin_bit),
+                        C.c_int(end_bit), _p(ko), _p(vo))
+    return ko, vo
+
+
+def tile_offsets(sorted_ids, n_tiles):
+    out = np.full(n_tiles, -1, np.int32)
+    lib().or_tile_offsets(C.c_int64(sorted_ids.size), _p(sorted_ids), C.c_uint32(n_tiles), _p(out))
+    return out
+
+
+def tile_n_bits(n_tiles):
+    b = 0
+    while (1 << b) <= n_tiles:   # src/kernels/tile/IntersectTile.cu:489-490
+        b += 1
+    return b
+
+
+def raster_fwd(n, scr, w, h, offsets, flat):
+    o = dict(rgb=np.zeros((h, w, 3), np.float32), depth=np.zeros((h, w), np.float32),
+             T=np.zeros((h, w), np.float32), last_ids=np.zeros((h, w), np.int32))
+    stats = np.zeros(2, np.int64)
+    lib().or_raster_fwd(C.c_int64(n), _p(scr["xy"]), _p(scr["depth"]), _p(scr["conic"]),
+                        _p(scr["opac"]), _p(scr["rgb"]), C.c_uint32(w), C.c_uint32(h), _p(offsets),
+                        _p(flat), C.c_int64(flat.size), _p(o["rgb"]), _p(o["depth"]), _p(o["T"]),
+                        _p(o["last_ids"]), _p(stats))
+    o["K_f"], o["K_b"] = int(stats[0]), int(stats[1])
+    return o
+
+
+def raster_bwd(n, scr, w, h, offsets, flat, fwd, v_rgb, v_depth, v_T, with_abs=True):
+    g = dict(v_xy=np.zeros((n, 2), np.float32), v_depth=np.zeros(n, np.float32),
+             v_conic=np.zeros((n, 3), np.float32), v_opac=np.zeros(n, np.float32),
+             v_rgb=np.zeros((n, 3), np.float32))
+    abs_terms = np.zeros((n, 10), np.float64) if with_abs else None
+    lib().or_raster_bwd(C.c_int64(n), _p(scr["xy"]), _p(scr["depth"]), _p(scr["conic"]),
+                        _p(scr["opac"]), _p(scr["rgb"]), C.c_uint32(w), C.c_uint32(h), _p(offsets),
+                        _p(flat), C.c_int64(flat.size), _p(fwd["T"]), _p(fwd["last_ids"]),
+                        _p(fwd["depth"]), _p(np.ascontiguousarray(v_rgb, np.float32)),
+                        _p(np.ascontiguousarray(v_depth, np.float32)),
+                        _p(np.ascontiguousarray(v_T, np.float32)),
+                        _p(g["v_xy"]), _p(g["v_depth"]), _p(g["v_conic"]), _p(g["v_opac"]),
+                        _p(g["v_rgb"]), _p(abs_terms))
+    g["abs_terms"] = abs_terms
+    return g
+
+
+def projection_bwd(scene, aabb, vs, sh_degree=3):
+    n = scene.n
+    keep = []
+    cam, sh = camera_of(scene), sh_source_of(scene, keep)
+    g = dict(v_means=np.zeros((n, 3), np.float32), v_quats=np.zeros((n, 4), np.float32),
+             v_scales=np.zeros((n, 3), np.float32), v_opacities=np.zeros(n, np.float32),
+             v_dc=np.zeros((n, 3), np.float32), v_sh=np.zeros((n, 15, 3), np.float32))
+    lib().or_projection_bwd(
+        C.c_int64(n), C.c_int(sh_degree), _p(scene.means), _p(scene.quats), _p(scene.log_scales),
+        _p(scene.opacity_logits), _p(scene.features_dc), C.byref(sh), C.byref(cam), _p(aabb),
+        _p(vs["v_xy"]), _p(vs["v_depth"]), _p(vs["v_conic"]), _p(vs["v_opac"]), _p(vs["v_rgb"]),
+        _p(g["v_means"]), _p(g["v_quats"]), _p(g["v_scales"]), _p(g["v_opacities"]), _p(g["v_dc"]),
+        _p(g["v_sh"]))
+    return g
+
+
+def pipeline(scene, sh_degree=3, backward=True):
+    """The whole iteration in the reference's order (src/engine/EngineForward.cpp:166-293,
+    src/engine/EngineLoss.cpp:138-240,359-368)."""
+    n, w, h = scene.n, scene.width, scene.height
+    p = projection_fwd(scene, sh_degree)
+    counts = tile_count(n, p["aabb"], p["xy"], p["conic"], p["opac"], w, h)
+    cum = inclusive_sum(counts)
+    ids, flat, pads = tile_write(n, p["aabb"], p["sort_depth"], p["xy"], p["conic"], p["opac"], cum, w, h)
+    n_tiles = scene.tile_w * scene.tile_h
+    sk, sv = sort_pairs(ids, flat, 0, 32 + tile_n_bits(n_tiles))
+    offs = tile_offsets(sk, n_tiles)
+    f = raster_fwd(n, p, w, h, offs, sv)
+    out = dict(proj=p, counts=counts, cum=cum, isect_ids=ids, flatten_ids=flat, pads=pads,
+               sorted_ids=sk, sorted_flat=sv, offsets=offs, fwd=f)
+    if backward:
+        out["vscreen"] = raster_bwd(n, p, w, h, offs, sv, f, scene.v_rgb, scene.v_depth, scene.v_T)
+        out["grads"] = projection_bwd(scene, p["aabb"], out["vscreen"], sh_degree)
+    return out

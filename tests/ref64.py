@@ -1,0 +1,114 @@
+"""Independent float64 restatements (numpy) used to pin the oracle: matrix-form projection,
+textbook real spherical harmonics, brute-force per-pixel compositing. None of this code is shared
+with the oracle or the kernels; finite differences of these functions pin the backward passes."""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+
+ALPHA_T = 1.0 / 255.0
+
+
+def quat_rot(q):
+    w, x, y, z = q / np.linalg.norm(q)
+    return np.array([
+        [1 - 2 * (y * y + z * z), 2 * (x * y - w * z), 2 * (x * z + w * y)],
+        [2 * (x * y + w * z), 1 - 2 * (x * x + z * z), 2 * (y * z - w * x)],
+        [2 * (x * z - w * y), 2 * (y * z + w * x), 1 - 2 * (x * x + y * y)]])
+
+
+def project(mean, quat, log_scale, logit, viewmat, intr, width, model, f32_consts=True):
+    """Returns xy(2), depth, conic(3), opac, plus cov2d (blurred) and the tile extents."""
+    R, t = viewmat[:3, :3].astype(np.float64), viewmat[:3, 3].astype(np.float64)
+    fx, fy, cx, cy = [float(v) for v in intr]
+    pc = R @ mean + t
+    x, y, z = pc
+    Rq = quat_rot(quat)
+    S = np.diag(np.exp(log_scale))
+    cov = Rq @ S @ S @ Rq.T
+    covc = R @ cov @ R.T
+    if model == 0:
+        xy = np.array([fx * x / z + cx, fy * y / z + cy])
+        J = np.array([[fx / z, 0, -fx * x / z ** 2], [0, fy / z, -fy * y / z ** 2]])
+        c03 = float(np.float32(0.3)) if f32_consts else 0.3
+        lim_pos = width + c03 * (0.5 * width)
+        lim_neg = c03 * (0.5 * width)
+        # y limits reuse the x limits (src/shaders/primitive_3dgs.slang:92-93)
+        J[0, 2] = min(max(J[0, 2], -(lim_pos - cx) / z), (lim_neg + cx) / z)
+        J[1, 2] = min(max(J[1, 2], -(lim_pos - cy) / z), (lim_neg + cy) / z)
+    else:
+        h = math.hypot(x, z)
+        r2 = x * x + y * y + z * z
+        xy = np.array([fx * math.atan2(x, z) + cx, fy * math.atan2(y, h) + cy])
+        J = np.array([[fx * z / h ** 2, 0, -fx * x / h ** 2],
+                      [-fy * x * y / (h * r2), fy * h / r2, -fy * z * y / (h * r2)]])
+    c2 = J @ covc @ J.T
+    eps = float(np.float32(0.3)) if f32_consts else 0.3
+    c2 = c2 + eps * np.eye(2)
+    inv = np.linalg.inv(c2)
+    opac = 1.0 / (1.0 + math.exp(-logit))
+    depth = float(np.linalg.norm(pc))
+    return dict(xy=xy, depth=depth, conic=np.array([inv[0, 0], inv[0, 1], inv[1, 1]]), opac=opac,
+                cov2d=c2, pc=pc)
+
+
+def real_sh_deg3(d):
+    """Textbook real spherical harmonics l=1..3 (Cartesian forms, unit vector d), multiplied by the
+    Condon-Shortley sign (-1)^m that the reference's basis carries
+    (src/shaders/harmonics.slang:172-217). Order: l=1 m=-1,0,1; l=2 m=-2..2; l=3 m=-3..3."""
+    x, y, z = d / np.linalg.norm(d)
+    pi = math.pi
+    Y = [
+        -math.sqrt(3 / (4 * pi)) * y, math.sqrt(3 / (4 * pi)) * z, -math.sqrt(3 / (4 * pi)) * x,
+        0.5 * math.sqrt(15 / pi) * x * y, -0.5 * math.sqrt(15 / pi) * y * z,
+        0.25 * math.sqrt(5 / pi) * (3 * z * z - 1), -0.5 * math.sqrt(15 / pi) * x * z,
+        0.25 * math.sqrt(15 / pi) * (x * x - y * y),
+        -0.25 * math.sqrt(35 / (2 * pi)) * y * (3 * x * x - y * y),
+        0.5 * math.sqrt(105 / pi) * x * y * z,
+        -0.25 * math.sqrt(21 / (2 * pi)) * y * (5 * z * z - 1),
+        0.25 * math.sqrt(7 / pi) * (5 * z ** 3 - 3 * z),
+        -0.25 * math.sqrt(21 / (2 * pi)) * x * (5 * z * z - 1),
+        0.25 * math.sqrt(105 / pi) * (x * x - y * y) * z,
+        -0.25 * math.sqrt(35 / (2 * pi)) * x * (x * x - 3 * y * y),
+    ]
+    return np.array(Y)
+
+
+def sh_color(mean, viewmat, dc, coeffs, degree=3, clamp=True):
+    R, t = viewmat[:3, :3].astype(np.float64), viewmat[:3, 3].astype(np.float64)
+    d = mean + R.T @ t            # mean - campos
+    Y = real_sh_deg3(d)
+    ncoef = degree * (degree + 2)
+    col = 0.5 * math.sqrt(1 / math.pi) * dc + (Y[:ncoef, None] * coeffs[:ncoef]).sum(axis=0)
+    col = col + 0.5
+    return np.maximum(col, 0.0) if clamp else col
+
+
+def composite(px, py, frags, with_state=False):
+    """Front-to-back compositing of one pixel over `frags` (already in sorted order):
+    dict arrays xy[K,2], conic[K,3], opac[K], rgb[K,3], depth[K]. Returns rgb, depth, T, last."""
+    T = 1.0
+    rgb = np.zeros(3)
+    dsum = 0.0
+    last = 0
+    for k in range(len(frags["opac"])):
+        dx = frags["xy"][k, 0] - px
+        dy = frags["xy"][k, 1] - py
+        a, b, c = frags["conic"][k]
+        sigma = 0.5 * (a * dx * dx + c * dy * dy) + b * dx * dy
+        if sigma < 0:
+            continue
+        alpha = min(0.999, frags["opac"][k] * math.exp(-sigma))
+        if alpha <= ALPHA_T:
+            continue
+        nT = T * (1 - alpha)
+        if nT <= 1e-4:
+            break
+        w = alpha * T
+        rgb = rgb + w * frags["rgb"][k]
+        dsum += w * frags["depth"][k]
+        T = nT
+        last = k
+    depth = dsum / max(1 - T, 1e-10)
+    return rgb, depth, T, last
