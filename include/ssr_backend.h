@@ -1,0 +1,218 @@
+/* ssr_backend.h -- C ABI of the MI355X (gfx950) Gaussian-splat rasterizer hot path.
+ *
+ * One shared library, libssr_hip.so, exports exactly the entry points below. They are what a
+ * third backend of the reference (beside its CUDA and Vulkan ones) binds for this path: each
+ * replaces one launch function or runtime call of the reference's backend seam
+ * (src/backend/api/{Projection,TileIntersect,Rasterization}.h, src/backend/api/BackendRuntime.h,
+ * src/backend/common/SortScan.h). The C++ adapter in spirula-studio_amd/host/ re-creates the
+ * reference's own C++ signatures on top of these.
+ *
+ * Conventions
+ *  - Every data pointer is a DEVICE pointer unless named host_*. Sizes are element counts unless
+ *    named *_bytes. No entry point allocates device memory; scratch is passed in by the caller
+ *    (sizes from the *_scratch_bytes functions). No entry point synchronises except
+ *    ssr_read_i64, ssr_*_synchronize, ssr_memcpy (sync form) and ssr_event_elapsed_ms.
+ *  - `stream` is a hipStream_t passed as void*; NULL is the default stream, which is what the
+ *    reference launches on (src/core/Common.cuh:207).
+ *  - Return value 0 = success. Non-zero = error; the message is kept per thread and returned (and
+ *    cleared) by ssr_last_error(), like the reference's sticky backend::last_error()
+ *    (src/backend/api/BackendRuntime.h:98). Nothing calls exit().
+ *  - Supported variant: primitive "3dgs" (not antialiased), camera PINHOLE or EQUIRECTANGULAR,
+ *    distortion NONE, one camera (C = 1), SH degree 0..3, dist_type None, no median, no
+ *    accumulation weights, non-packed. Anything else is rejected with an error, as the reference
+ *    rejects an uncompiled variant (src/kernels/projection/ProjectionFwd.cu:84-89).
+ *  - Layouts are the reference's (src/primitives/PrimitiveBase3DGS.cuh:87-139,187-225).
+ */
+#ifndef SSR_BACKEND_H
+#define SSR_BACKEND_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* ssr_stream_t;
+typedef void* ssr_event_t;
+
+enum { SSR_CAM_PINHOLE = 0, SSR_CAM_EQUIRECT = 3 };       /* CameraModelType, src/core/Common.cuh */
+enum { SSR_SH_F32 = 0, SSR_SH_REF_Q8 = 1, SSR_SH_REF_Q16 = 2, SSR_SH_I8_F16SCALE = 3 };
+enum { SSR_MEMCPY_H2D = 0, SSR_MEMCPY_D2H = 1, SSR_MEMCPY_D2D = 2, SSR_MEMCPY_H2H = 3,
+       SSR_MEMCPY_AUTO = 4 };                             /* backend::MemcpyKind */
+
+/* WorldBuffer = TensorArray<6> (src/primitives/PrimitiveBase3DGS.cuh:87-139). */
+typedef struct {
+    float* means;           /* [N,3] */
+    float* quats;           /* [N,4] w,x,y,z */
+    float* log_scales;      /* [N,3] */
+    float* opacity_logits;  /* [N] */
+    float* features_dc;     /* [N,3] */
+    float* features_sh;     /* [N,sh_stride] coefficient-major, channel innermost */
+    int32_t sh_stride;      /* floats per splat in features_sh (45 for SH3) */
+} ssr_world;
+
+/* ScreenBuffer = TensorArray<5> (src/primitives/PrimitiveBase3DGS.cuh:187-225). */
+typedef struct {
+    float* xy;      /* [N,2] */
+    float* depth;   /* [N]   */
+    float* conic;   /* [N,3] */
+    float* opac;    /* [N]   */
+    float* rgb;     /* [N,3] */
+} ssr_screen;
+
+/* Quantized SH source. REF_Q8/REF_Q16: the reference's codec, uint8/uint16 codes plus float2
+ * (min,max) per `bounds_stride` cells, cell = gid*3*num_sh_buffer + 3*j + ch
+ * (src/shaders/harmonics.slang:92-140; launcher args src/kernels/projection/ProjectionFwd.cuh:27-35;
+ * bounds_stride 0 selects 256*3*num_sh_buffer as there). I8_F16SCALE: int8 codes [N,45] times one
+ * fp16 scale per splat (the benchmark's storage format; no counterpart in the reference). */
+typedef struct {
+    int32_t codec;              /* SSR_SH_* ; SSR_SH_F32 reads ssr_world.features_sh */
+    const void* packed;
+    const float* bounds;        /* float2[n_bounds] */
+    int64_t bounds_stride;
+    uint32_t num_sh_buffer;
+    const uint16_t* scale_f16;  /* [N] */
+} ssr_sh_quant;
+
+typedef struct {
+    int32_t camera_model;   /* SSR_CAM_* */
+    uint32_t num_cameras;   /* must be 1 */
+    uint32_t width, height;
+    const float* viewmats;  /* device [C,4,4] row-major world->camera */
+    const float* intrins;   /* device [C,4] fx,fy,cx,cy */
+} ssr_camera;
+
+/* ---- K1: projection_3dgs_forward (src/kernels/projection/ProjectionFwd.cuh:18-36,
+ * kernel src/kernels/projection/ProjectionFwd_kernel.cuh:17-111). Writes aabb/sort_depth for every
+ * splat, the screen row and atomic-max radii only for visible ones. If tiles_per_splat is
+ * non-NULL the tile count of K2 is produced in the same pass. */
+typedef struct {
+    int64_t num_splats;
+    int32_t sh_degree;
+    ssr_world world;
+    ssr_sh_quant sh;
+    ssr_camera camera;
+    float* aabb;            /* [C,N,4] */
+    float* sort_depth;      /* [C,N] */
+    float* radii;           /* [N], caller zero-fills (src/engine/EngineForward.cpp:66-69) */
+    ssr_screen screen;
+    int64_t* tiles_per_splat; /* optional [C*N] */
+} ssr_projection_fwd_params;
+int ssr_projection_fwd(const ssr_projection_fwd_params* p, ssr_stream_t stream);
+
+/* ---- K2..K6: do_intersect_tile_generic, ellipse mode (src/kernels/tile/IntersectTile.cuh:25-41,
+ * src/kernels/tile/IntersectTile.cu:376-509) split at its data-dependent allocation. */
+int ssr_tile_count(int64_t n, const float* aabb, const float* xy, const float* conic,
+                   const float* opac, uint32_t width, uint32_t height, int64_t* tiles_per_splat,
+                   ssr_stream_t stream);
+/* inclusive_sum<int64> (src/backend/common/SortScan.h:58-72; IntersectTile.cu:425-428). */
+size_t ssr_scan_scratch_bytes(int64_t n);
+int ssr_inclusive_sum_i64(const int64_t* in, int64_t* out, int64_t n, void* scratch,
+                          size_t scratch_bytes, ssr_stream_t stream);
+/* The reference's blocking 8-byte readback of n_isects (IntersectTile.cu:432-436). */
+int ssr_read_i64(const int64_t* device_value, int64_t* host_value, ssr_stream_t stream);
+int ssr_tile_write(int64_t n, const float* aabb, const float* sort_depth, const float* xy,
+                   const float* conic, const float* opac, const int64_t* cum_tiles,
+                   uint32_t width, uint32_t height, int64_t* isect_ids, int32_t* flatten_ids,
+                   ssr_stream_t stream);
+/* sort_pairs<int64,int32> with CUB DoubleBuffer semantics (src/backend/common/SortScan.h:42-56;
+ * call site IntersectTile.cu:486-493): stable on bits [begin_bit,end_bit); *selector says which
+ * of the (a,b) buffers holds the result. */
+size_t ssr_sort_scratch_bytes(int64_t n);
+int ssr_sort_pairs_u64_i32(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, int32_t* vals_b,
+                           int64_t n, int begin_bit, int end_bit, int* selector, void* scratch,
+                           size_t scratch_bytes, ssr_stream_t stream);
+/* intersect_offset_kernel (IntersectTile.cu:271-307); zero-fills when n_isects == 0 (:448-451). */
+int ssr_tile_offsets(int64_t n_isects, const int64_t* sorted_ids, uint32_t n_tiles,
+                     int32_t* offsets, ssr_stream_t stream);
+/* Number of key bits the sort must cover: 32 + tile_n_bits (IntersectTile.cu:489-490). */
+int ssr_sort_end_bit(uint32_t n_tiles);
+
+/* ---- K7: rasterize_to_pixels_3dgs_fwd (src/kernels/raster/RasterizationFwd.cuh:18-38, kernel
+ * src/kernels/raster/RasterizationEval3DFwd_kernel.cuh:48-313, IS_EVAL3D=0). */
+typedef struct {
+    int64_t num_splats;
+    ssr_screen screen;          /* read */
+    uint32_t width, height;
+    const int32_t* tile_offsets;  /* [tile_h,tile_w] */
+    const int32_t* flatten_ids;   /* [n_isects] */
+    int64_t n_isects;
+    float* render_rgb;      /* [H,W,3] */
+    float* render_depth;    /* [H,W] */
+    float* render_T;        /* [H,W] */
+    int32_t* last_ids;      /* [H,W] */
+} ssr_raster_fwd_params;
+int ssr_raster_fwd(const ssr_raster_fwd_params* p, ssr_stream_t stream);
+
+/* ---- K8: rasterize_to_pixels_3dgs_bwd (src/kernels/raster/RasterizationBwd.cuh:18-48, kernel
+ * src/kernels/raster/RasterizationEval3DBwd_kernel.cuh:48-636, IS_EVAL3D=0). Gradients are ADDED
+ * into v_screen with float atomics; the caller zero-fills it first, as the reference's launcher
+ * does (src/kernels/raster/RasterizationBwd.cu:143-146). */
+typedef struct {
+    int64_t num_splats;
+    ssr_screen screen;
+    uint32_t width, height;
+    const int32_t* tile_offsets;
+    const int32_t* flatten_ids;
+    int64_t n_isects;
+    const float* render_T;
+    const int32_t* last_ids;
+    const float* render_depth;
+    const float* v_render_rgb;    /* [H,W,3] */
+    const float* v_render_depth;  /* [H,W] */
+    const float* v_render_T;      /* [H,W] */
+    ssr_screen v_screen;          /* accumulated into */
+} ssr_raster_bwd_params;
+int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t stream);
+
+/* ---- K9: projection_3dgs_backward (src/kernels/projection/ProjectionBwd.cuh:18-46, kernel
+ * src/kernels/projection/ProjectionBwd_kernel.cuh:16-130), v_viewmats = NULL. accumulate != 0:
+ * gradients are added into v_world (the reference's behaviour; caller zero-fills,
+ * src/engine/EngineLoss.cpp:120-127). accumulate == 0: every row of v_world is overwritten
+ * (zeros for culled splats), which gives the same values with C = 1 and needs no zero-fill. */
+typedef struct {
+    int64_t num_splats;
+    int32_t sh_degree;
+    ssr_world world;
+    ssr_sh_quant sh;
+    ssr_camera camera;
+    const float* aabb;
+    ssr_screen v_screen;    /* read */
+    ssr_world v_world;      /* written / accumulated */
+    int32_t accumulate;
+} ssr_projection_bwd_params;
+int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream_t stream);
+
+/* ---- K10 and runtime (src/backend/api/BackendRuntime.h:29-168). */
+int ssr_fill_u32(void* dst, uint32_t value, int64_t count, ssr_stream_t stream);
+int ssr_init(int device);                       /* select the device, warm the context */
+int ssr_device_count(void);
+const char* ssr_device_name(void);
+void* ssr_device_malloc(size_t bytes);          /* 0 bytes -> NULL; failure -> NULL */
+int ssr_device_free(void* ptr);                 /* drains in-flight work first */
+void* ssr_host_malloc_pinned(size_t bytes);
+int ssr_host_free_pinned(void* ptr);
+int ssr_memcpy(void* dst, const void* src, size_t bytes, int kind, ssr_stream_t stream, int async);
+int ssr_memset(void* dst, int byte_value, size_t bytes, ssr_stream_t stream, int async);
+int ssr_is_device_pointer(const void* ptr);     /* pinned host memory is NOT a device pointer */
+int ssr_device_synchronize(void);
+int ssr_stream_synchronize(ssr_stream_t stream);
+ssr_stream_t ssr_stream_create(void);
+int ssr_stream_destroy(ssr_stream_t stream);
+ssr_event_t ssr_event_create(void);
+int ssr_event_record(ssr_event_t ev, ssr_stream_t stream);
+int ssr_event_synchronize(ssr_event_t ev);
+int ssr_event_elapsed_ms(ssr_event_t start, ssr_event_t stop, float* ms);
+int ssr_event_destroy(ssr_event_t ev);
+const char* ssr_last_error(void);               /* returns and clears; "" when none */
+
+/* Diagnostics: include/ssr_math.h evaluated on the device (op: 0 exp, 1 log, 2 atan2(a,b),
+ * 3 sigmoid), to check that host and device produce identical bits. */
+int ssr_debug_math(int op, int64_t n, const float* a, const float* b, float* out,
+                   ssr_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SSR_BACKEND_H */

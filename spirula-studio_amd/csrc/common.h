@@ -1,0 +1,38 @@
+// common.h -- shared host/device helpers of libssr_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string>
+
+#include "../../include/ssr_backend.h"
+#include "../../include/ssr_math.h"
+
+namespace ssr {
+
+constexpr int kTile = 16;    // binning tile: TILE_SIZE_X * MACRO_TILE_SIZE_X (src/core/Common.cuh:36-39)
+constexpr int kMicro = 8;    // compositing sub-tile: TILE_SIZE_X
+constexpr float kAlphaThreshold = 1.0f / 255.0f;   // src/core/Common.cuh:47
+constexpr float kTransmitThreshold = 1e-4f;        // src/kernels/tile/IntersectTile.cu:25
+
+// Per-thread sticky error (returned and cleared by ssr_last_error()).
+void set_error(const std::string& msg);
+int fail(const char* where, const std::string& msg);
+int check_hip(hipError_t e, const char* where);
+
+inline hipStream_t as_stream(ssr_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+}  // namespace ssr
+
+#define SSR_CHECK_LAUNCH(where)                                       \
+    do {                                                              \
+        int _e = ssr::check_hip(hipGetLastError(), where);            \
+        if (_e) return _e;                                            \
+    } while (0)
+
+#define SSR_REQUIRE(cond, where, msg)                                 \
+    do {                                                              \
+        if (!(cond)) return ssr::fail(where, msg);                    \
+    } while (0)

@@ -1,0 +1,423 @@
+// projection.hip -- K1 (projection + SH colour, optional fused tile count) and K9 (their VJP).
+//
+// K1 follows projection_fused_fwd_kernel (src/kernels/projection/ProjectionFwd_kernel.cuh:17-111)
+// with World::project (src/primitives/Primitive3DGS.cuh:56-110). K9 follows
+// projection_fused_bwd_kernel (src/kernels/projection/ProjectionBwd_kernel.cuh:16-130) with
+// World::project_vjp (src/primitives/Primitive3DGS.cuh:119-201); the projection VJP is written out
+// by hand with the conventions of the reference's generated derivative
+// (src/generated/primitive_3dgs.cuh:12782-13230): a clamped Jacobian entry sends its gradient to
+// the violated bound, v_conic enters as [[vx, vy],[0, vz]], normalize(quat) and length() are
+// differentiated, extents / sorting depth / radius carry no gradient.
+//
+// One thread per Gaussian, 256 threads (4 wavefronts) per workgroup. Both kernels are bound by
+// HBM traffic (236 B in, 60 B out per visible splat forward; 472 B in/out backward).
+#include "projection_device.h"
+
+namespace ssr {
+
+constexpr int kProjBlock = 256;
+
+__device__ __forceinline__ void load_splat(const ssr_world& w, int64_t g, float mean[3], float quat[4],
+                                           float ls[3], float& logit) {
+    const float* m = w.means + 3 * g;
+    mean[0] = m[0]; mean[1] = m[1]; mean[2] = m[2];
+    const float4 q = *reinterpret_cast<const float4*>(w.quats + 4 * g);
+    quat[0] = q.x; quat[1] = q.y; quat[2] = q.z; quat[3] = q.w;
+    const float* s = w.log_scales + 3 * g;
+    ls[0] = s[0]; ls[1] = s[1]; ls[2] = s[2];
+    logit = w.opacity_logits[g];
+}
+
+// atomicMax for non-negative floats through the integer ordering (src/core/Common.cuh:785-789)
+__device__ __forceinline__ void atomic_max_nonneg(float* p, float v) {
+    atomicMax(reinterpret_cast<int*>(p), __float_as_int(v));
+}
+
+template <int kDegree>
+__global__ __launch_bounds__(kProjBlock) void projection_fwd_kernel(ssr_projection_fwd_params P) {
+    const int64_t g = (int64_t)blockIdx.x * kProjBlock + threadIdx.x;
+    if (g >= P.num_splats) return;
+    const CamD cam = load_camera(P.camera);
+    float mean[3], quat[4], ls[3], logit;
+    load_splat(P.world, g, mean, quat, ls, logit);
+    ProjD p;
+    project<false>(cam, mean, quat, ls, logit, p);
+
+    float col[3] = {0.f, 0.f, 0.f};
+    float bb[4] = {p.aabb[0], p.aabb[1], p.aabb[2], p.aabb[3]};
+    if (bb[2] > bb[0] && bb[3] > bb[1]) {
+        constexpr int kCoef = kDegree * (kDegree + 2);
+        float coef[kCoef > 0 ? 3 * kCoef : 1];
+        if (kCoef > 0) decode_sh<kCoef>(P.world, P.sh, g, coef);
+        float dir[3];
+        view_dir(cam, mean, dir);
+        ShBasisD b;
+        sh_basis<kDegree>(dir, b);
+        const float* dcp = P.world.features_dc + 3 * g;
+        const float dc[3] = {dcp[0], dcp[1], dcp[2]};
+        float raw[3];
+        sh_color_raw<kDegree>(b, dc, coef, raw);
+#pragma unroll
+        for (int c = 0; c < 3; c++) col[c] = ssr_max(raw[c] + 0.5f, 0.0f);
+    }
+    bb[0] = ssr_min(ssr_max(bb[0], 0.0f), cam.Wf - 1.0f);
+    bb[1] = ssr_min(ssr_max(bb[1], 0.0f), cam.Hf - 1.0f);
+    bb[2] = ssr_min(ssr_max(bb[2], 0.0f), cam.Wf - 1.0f);
+    bb[3] = ssr_min(ssr_max(bb[3], 0.0f), cam.Hf - 1.0f);
+    float4* aabb_out = reinterpret_cast<float4*>(P.aabb);
+    if (bb[2] - bb[0] > 1e-3f && bb[3] - bb[1] > 1e-3f) {
+        *reinterpret_cast<float2*>(P.screen.xy + 2 * g) = make_float2(p.xy[0], p.xy[1]);
+        P.screen.depth[g] = p.depth;
+        float* cn = P.screen.conic + 3 * g;
+        cn[0] = p.conic[0]; cn[1] = p.conic[1]; cn[2] = p.conic[2];
+        P.screen.opac[g] = p.opac;
+        float* rg = P.screen.rgb + 3 * g;
+        rg[0] = col[0]; rg[1] = col[1]; rg[2] = col[2];
+        aabb_out[g] = make_float4(bb[0], bb[1], bb[2], bb[3]);
+        P.sort_depth[g] = p.sort_depth;
+        atomic_max_nonneg(P.radii + g, p.radius);
+        if (P.tiles_per_splat) {
+            const int tw = (int)((P.camera.width + kTile - 1) / kTile), th = (int)((P.camera.height + kTile - 1) / kTile);
+            TileGeomD tg;
+            tile_geom(bb, p.xy, p.conic, p.opac, tw, th, tg);
+            P.tiles_per_splat[g] = count_tiles(tg);
+        }
+    } else {
+        aabb_out[g] = make_float4(0.f, 0.f, 0.f, 0.f);
+        P.sort_depth[g] = 0.0f;
+        if (P.tiles_per_splat) P.tiles_per_splat[g] = 0;
+    }
+}
+
+__device__ __forceinline__ float fin(float v) { return ssr_isfinite(v) ? v : 0.0f; }
+
+template <bool kAccumulate>
+__device__ __forceinline__ void put(float* p, float v) {
+    if (kAccumulate) { if (v != 0.0f) atomicAdd(p, v); }
+    else *p = v;
+}
+
+template <int kDegree, bool kAccumulate>
+__global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projection_bwd_params P) {
+    const int64_t g = (int64_t)blockIdx.x * kProjBlock + threadIdx.x;
+    if (g >= P.num_splats) return;
+    constexpr int kCoef = kDegree * (kDegree + 2);
+    const float4 bb = reinterpret_cast<const float4*>(P.aabb)[g];
+    ssr_world& V = P.v_world;
+    if (bb.z <= bb.x || bb.w <= bb.y) {   // ProjectionBwd_kernel.cuh:58
+        if (!kAccumulate) {
+#pragma unroll
+            for (int i = 0; i < 3; i++) { V.means[3 * g + i] = 0.f; V.log_scales[3 * g + i] = 0.f; V.features_dc[3 * g + i] = 0.f; }
+            *reinterpret_cast<float4*>(V.quats + 4 * g) = make_float4(0.f, 0.f, 0.f, 0.f);
+            V.opacity_logits[g] = 0.f;
+            float* vs = V.features_sh + g * (int64_t)V.sh_stride;
+            for (int i = 0; i < V.sh_stride; i++) vs[i] = 0.f;
+        }
+        return;
+    }
+    const CamD cam = load_camera(P.camera);
+    float mean[3], quat[4], ls[3], logit;
+    load_splat(P.world, g, mean, quat, ls, logit);
+    ProjD p;
+    project<true>(cam, mean, quat, ls, logit, p);
+    const float x = p.mc[0], y = p.mc[1], z = p.mc[2];
+    float vmc[3] = {0.f, 0.f, 0.f};
+    // conic = inverse(cov2d)
+    const float c00 = p.c2[0][0], c01 = p.c2[0][1], c10 = p.c2[1][0], c11 = p.c2[1][1];
+    const float det = c00 * c11 - c01 * c10, inv = 1.0f / det;
+    const float* vcn = P.v_screen.conic + 3 * g;
+    const float g00 = vcn[0], g01 = vcn[1], g11 = vcn[2];
+    const float v_inv = (c11 * g00 - c01 * g01) + c00 * g11;
+    const float v_det = -(v_inv / (det * det));
+    float vC[2][2];
+    vC[0][0] = inv * g11 + c11 * v_det;
+    vC[1][1] = inv * g00 + c00 * v_det;
+    vC[0][1] = -(inv * g01) - c10 * v_det;
+    vC[1][0] = -(c01 * v_det);
+    // cov2d = J covc J^T
+    float vJ[2][3], vS[3][3];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int k = 0; k < 3; k++) {
+            float s = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int l = 0; l < 3; l++)
+                    s += vC[i][j] * p.J[j][l] * p.covc[k][l] + vC[j][i] * p.J[j][l] * p.covc[l][k];
+            vJ[i][k] = s;
+        }
+#pragma unroll
+    for (int k = 0; k < 3; k++)
+#pragma unroll
+        for (int l = 0; l < 3; l++) {
+            float s = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) s += p.J[i][k] * vC[i][j] * p.J[j][l];
+            vS[k][l] = s;
+        }
+    const float vm0 = P.v_screen.xy[2 * g], vm1 = P.v_screen.xy[2 * g + 1];
+    if (cam.model == SSR_CAM_PINHOLE) {
+        const float z2 = z * z, iz = 1.0f / z, iz2 = 1.0f / z2;
+        vmc[2] += vJ[0][0] * (-cam.fx * iz2) + vJ[1][1] * (-cam.fy * iz2);
+        const float lim_pos = cam.Wf + 0.3f * (0.5f * cam.Wf), lim_neg = 0.3f * (0.5f * cam.Wf);
+        const float cmaxx = lim_neg + cam.cx, cminx = -(lim_pos - cam.cx);
+        const float cmaxy = lim_neg + cam.cy, cminy = -(lim_pos - cam.cy);
+        if (p.clamp_lo[0]) vmc[2] += vJ[0][2] * cminx * (-iz2);
+        else if (p.clamp_hi[0]) vmc[2] += vJ[0][2] * cmaxx * (-iz2);
+        else { vmc[0] += vJ[0][2] * (-cam.fx * iz2); vmc[2] += vJ[0][2] * (2.0f * cam.fx * x * iz2 * iz); }
+        if (p.clamp_lo[1]) vmc[2] += vJ[1][2] * cminy * (-iz2);
+        else if (p.clamp_hi[1]) vmc[2] += vJ[1][2] * cmaxy * (-iz2);
+        else { vmc[1] += vJ[1][2] * (-cam.fy * iz2); vmc[2] += vJ[1][2] * (2.0f * cam.fy * y * iz2 * iz); }
+        vmc[0] += vm0 * cam.fx * iz;
+        vmc[1] += vm1 * cam.fy * iz;
+        vmc[2] += -(vm0 * cam.fx * x + vm1 * cam.fy * y) * iz2;
+    } else {
+        const float h2 = x * x + z * z, h = ssr_sqrt(h2), r2 = h2 + y * y;
+        const float A = 1.0f / h2, B = 1.0f / (h * r2);
+        const float dAx = -2.0f * x * A * A, dAz = -2.0f * z * A * A;
+        const float dBx = -B * B * (x * r2 / h + 2.0f * x * h);
+        const float dBy = -B * B * (2.0f * y * h);
+        const float dBz = -B * B * (z * r2 / h + 2.0f * z * h);
+        const float fx = cam.fx, fy = cam.fy;
+        const float ir2 = 1.0f / r2, ir4 = ir2 * ir2;
+        vmc[0] += vJ[0][0] * fx * z * dAx + vJ[0][2] * (-fx) * (A + x * dAx);
+        vmc[2] += vJ[0][0] * fx * (A + z * dAz) + vJ[0][2] * (-fx) * x * dAz;
+        vmc[0] += vJ[1][0] * (-fy) * (y * B + x * y * dBx) + vJ[1][2] * (-fy) * (z * y * dBx) +
+                  vJ[1][1] * fy * ((x / h) * ir2 - h * 2.0f * x * ir4);
+        vmc[1] += vJ[1][0] * (-fy) * (x * B + x * y * dBy) + vJ[1][2] * (-fy) * (z * B + z * y * dBy) +
+                  vJ[1][1] * fy * (-h * 2.0f * y * ir4);
+        vmc[2] += vJ[1][0] * (-fy) * (x * y * dBz) + vJ[1][2] * (-fy) * (y * B + z * y * dBz) +
+                  vJ[1][1] * fy * ((z / h) * ir2 - h * 2.0f * z * ir4);
+        vmc[0] += vm0 * fx * z * A + vm1 * fy * (-(x * y) * B);
+        vmc[1] += vm1 * fy * h * ir2;
+        vmc[2] += vm0 * fx * (-x * A) + vm1 * fy * (-(z * y) * B);
+    }
+    {   // depth = length(mean_c); the sqrt derivative is guarded at 1e-7
+        const float s2 = dot3(p.mc, p.mc);
+        const float vs = P.v_screen.depth[g] * (0.5f / ssr_sqrt(ssr_max(1e-7f, s2)));
+#pragma unroll
+        for (int i = 0; i < 3; i++) vmc[i] += 2.0f * p.mc[i] * vs;
+    }
+    float vmean[3];
+#pragma unroll
+    for (int i = 0; i < 3; i++) vmean[i] = (cam.R[0][i] * vmc[0] + cam.R[1][i] * vmc[1]) + cam.R[2][i] * vmc[2];
+    float t1[3][3], vcov[3][3], vM[3][3];
+#pragma unroll
+    for (int i = 0; i < 3; i++)
+#pragma unroll
+        for (int j = 0; j < 3; j++)
+            t1[i][j] = (cam.R[0][i] * vS[0][j] + cam.R[1][i] * vS[1][j]) + cam.R[2][i] * vS[2][j];
+#pragma unroll
+    for (int i = 0; i < 3; i++)
+#pragma unroll
+        for (int j = 0; j < 3; j++)
+            vcov[i][j] = (t1[i][0] * cam.R[0][j] + t1[i][1] * cam.R[1][j]) + t1[i][2] * cam.R[2][j];
+#pragma unroll
+    for (int i = 0; i < 3; i++)
+#pragma unroll
+        for (int j = 0; j < 3; j++) {
+            float s = 0.0f;
+#pragma unroll
+            for (int k = 0; k < 3; k++) s += (vcov[i][k] + vcov[k][i]) * p.M[k][j];
+            vM[i][j] = s;
+        }
+    float vRq[3][3], vscale[3];
+#pragma unroll
+    for (int j = 0; j < 3; j++) {
+        float s = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 3; i++) { vRq[i][j] = vM[i][j] * p.s[j]; s += vM[i][j] * p.Rq[i][j]; }
+        vscale[j] = s * p.s[j];
+    }
+    const float qw = p.qn[0], qx = p.qn[1], qy = p.qn[2], qz = p.qn[3];
+    float vqn[4];
+    vqn[0] = 2.0f * (qx * (vRq[2][1] - vRq[1][2]) + qy * (vRq[0][2] - vRq[2][0]) + qz * (vRq[1][0] - vRq[0][1]));
+    vqn[1] = 2.0f * (-2.0f * qx * (vRq[1][1] + vRq[2][2]) + qy * (vRq[0][1] + vRq[1][0]) +
+                     qz * (vRq[0][2] + vRq[2][0]) + qw * (vRq[2][1] - vRq[1][2]));
+    vqn[2] = 2.0f * (-2.0f * qy * (vRq[0][0] + vRq[2][2]) + qx * (vRq[0][1] + vRq[1][0]) +
+                     qz * (vRq[1][2] + vRq[2][1]) + qw * (vRq[0][2] - vRq[2][0]));
+    vqn[3] = 2.0f * (-2.0f * qz * (vRq[0][0] + vRq[1][1]) + qx * (vRq[0][2] + vRq[2][0]) +
+                     qy * (vRq[1][2] + vRq[2][1]) + qw * (vRq[1][0] - vRq[0][1]));
+    const float qd = ((p.qn[0] * vqn[0] + p.qn[1] * vqn[1]) + p.qn[2] * vqn[2]) + p.qn[3] * vqn[3];
+    float vquat[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) vquat[i] = (vqn[i] - p.qn[i] * qd) * p.qinv;
+    const float vlogit = P.v_screen.opac[g] * (p.opac * (1.0f - p.opac));
+
+    // SH colour VJP (src/shaders/harmonics.slang:373-649,1087-1126)
+    float coef[kCoef > 0 ? 3 * kCoef : 1];
+    if (kCoef > 0) decode_sh<kCoef>(P.world, P.sh, g, coef);
+    float dir[3];
+    view_dir(cam, mean, dir);
+    ShBasisD b;
+    sh_basis<kDegree>(dir, b);
+    const float* dcp = P.world.features_dc + 3 * g;
+    const float dc[3] = {dcp[0], dcp[1], dcp[2]};
+    float raw[3];
+    sh_color_raw<kDegree>(b, dc, coef, raw);
+    const float* vrg = P.v_screen.rgb + 3 * g;
+    float vc[3];
+#pragma unroll
+    for (int c = 0; c < 3; c++) vc[c] = vrg[c] * (raw[c] >= -0.5f ? 1.0f : 0.0f);
+    float vdir[3] = {0.f, 0.f, 0.f};
+    float* vsh = V.features_sh + g * (int64_t)V.sh_stride;
+    if (kDegree >= 1) {
+#pragma unroll
+        for (int j = 0; j < kCoef; j++) {
+            const float tv[3] = {b.Y[j] * vc[0], b.Y[j] * vc[1], b.Y[j] * vc[2]};
+            const float d2 = dot3(tv, tv);
+            const bool ok = ssr_isfinite(d2) && d2 != 0.0f;   // harmonics.slang:397-403
+#pragma unroll
+            for (int c = 0; c < 3; c++) {
+                if (kAccumulate) { if (ok) atomicAdd(vsh + 3 * j + c, tv[c]); }
+                else vsh[3 * j + c] = ok ? tv[c] : 0.0f;
+            }
+        }
+        auto cd = [&](int j) { return (coef[3 * j] * vc[0] + coef[3 * j + 1] * vc[1]) + coef[3 * j + 2] * vc[2]; };
+        const float X = b.x, Y = b.y, Z = b.z;
+        float vx = -0.48860251190292f * cd(2), vy = -0.48860251190292f * cd(0), vz = 0.48860251190292f * cd(1);
+        if (kDegree >= 2) {
+            const float z2 = Z * Z;
+            const float fTmp0B = -1.092548430592079f * Z;
+            const float fC1 = X * X - Y * Y, fS1 = 2.f * X * Y;
+            const float fC1_x = 2.f * X, fC1_y = -2.f * Y, fS1_x = 2.f * Y, fS1_y = 2.f * X;
+            const float pSH6_z = 2.f * 0.9461746957575601f * Z;
+            const float pSH7_x = fTmp0B, pSH7_z = -1.092548430592079f * X;
+            const float pSH5_y = fTmp0B, pSH5_z = -1.092548430592079f * Y;
+            const float pSH8_x = 0.5462742152960395f * fC1_x, pSH8_y = 0.5462742152960395f * fC1_y;
+            const float pSH4_x = 0.5462742152960395f * fS1_x, pSH4_y = 0.5462742152960395f * fS1_y;
+            vx += pSH4_x * cd(3) + pSH8_x * cd(7) + pSH7_x * cd(6);
+            vy += pSH4_y * cd(3) + pSH8_y * cd(7) + pSH5_y * cd(4);
+            vz += pSH6_z * cd(5) + pSH7_z * cd(6) + pSH5_z * cd(4);
+            if (kDegree >= 3) {
+                const float fTmp0C = -2.285228997322329f * z2 + 0.4570457994644658f;
+                const float fTmp1B = 1.445305721320277f * Z;
+                const float fTmp0C_z = -2.285228997322329f * 2.f * Z;
+                const float fTmp1B_z = 1.445305721320277f;
+                const float fC2_x = fC1 + X * fC1_x - Y * fS1_x;
+                const float fC2_y = X * fC1_y - fS1 - Y * fS1_y;
+                const float fS2_x = fS1 + X * fS1_x + Y * fC1_x;
+                const float fS2_y = X * fS1_y + fC1 + Y * fC1_y;
+                const float pSH12_z = 3.f * 1.865881662950577f * z2 - 1.119528997770346f;
+                const float pSH13_x = fTmp0C, pSH13_z = fTmp0C_z * X;
+                const float pSH11_y = fTmp0C, pSH11_z = fTmp0C_z * Y;
+                const float pSH14_x = fTmp1B * fC1_x, pSH14_y = fTmp1B * fC1_y, pSH14_z = fTmp1B_z * fC1;
+                const float pSH10_x = fTmp1B * fS1_x, pSH10_y = fTmp1B * fS1_y, pSH10_z = fTmp1B_z * fS1;
+                const float pSH15_x = -0.5900435899266435f * fC2_x, pSH15_y = -0.5900435899266435f * fC2_y;
+                const float pSH9_x = -0.5900435899266435f * fS2_x, pSH9_y = -0.5900435899266435f * fS2_y;
+                vx += pSH9_x * cd(8) + pSH15_x * cd(14) + pSH10_x * cd(9) + pSH14_x * cd(13) + pSH13_x * cd(12);
+                vy += pSH9_y * cd(8) + pSH15_y * cd(14) + pSH10_y * cd(9) + pSH14_y * cd(13) + pSH11_y * cd(10);
+                vz += pSH12_z * cd(11) + pSH13_z * cd(12) + pSH11_z * cd(10) + pSH14_z * cd(13) + pSH10_z * cd(9);
+            }
+        }
+        const float dn = (vx * X + vy * Y) + vz * Z;
+        vdir[0] = (vx - dn * X) * b.inorm;
+        vdir[1] = (vy - dn * Y) * b.inorm;
+        vdir[2] = (vz - dn * Z) * b.inorm;
+    }
+    if (!kAccumulate) {   // coefficients above the active degree receive nothing
+        for (int i = 3 * kCoef; i < V.sh_stride; i++) vsh[i] = 0.0f;
+    }
+    // World::atomicStore (src/primitives/PrimitiveBase3DGS.cuh:75-83): per-component finite filter
+#pragma unroll
+    for (int i = 0; i < 3; i++) put<kAccumulate>(V.means + 3 * g + i, fin(vmean[i] + vdir[i]));
+#pragma unroll
+    for (int i = 0; i < 4; i++) put<kAccumulate>(V.quats + 4 * g + i, fin(vquat[i]));
+#pragma unroll
+    for (int i = 0; i < 3; i++) put<kAccumulate>(V.log_scales + 3 * g + i, fin(vscale[i]));
+    put<kAccumulate>(V.opacity_logits + g, fin(vlogit));
+#pragma unroll
+    for (int i = 0; i < 3; i++) put<kAccumulate>(V.features_dc + 3 * g + i, fin(0.2820947917738781f * vc[i]));
+}
+
+static int check_common(const char* where, int64_t n, int sh_degree, const ssr_world& w, const ssr_sh_quant& sh,
+                        const ssr_camera& cam) {
+    SSR_REQUIRE(n >= 0 && n < (int64_t)1 << 31, where, "num_splats must be in [0, 2^31)");
+    SSR_REQUIRE(sh_degree >= 0 && sh_degree <= 3, where, "SH degree must be 0..3");
+    SSR_REQUIRE(cam.camera_model == SSR_CAM_PINHOLE || cam.camera_model == SSR_CAM_EQUIRECT, where,
+                "unsupported camera model (PINHOLE and EQUIRECTANGULAR without distortion are built)");
+    SSR_REQUIRE(cam.num_cameras == 1, where, "exactly one camera per call is supported");
+    SSR_REQUIRE(cam.width > 0 && cam.height > 0, where, "empty image");
+    SSR_REQUIRE(cam.viewmats && cam.intrins, where, "null camera pointer");
+    if (n == 0) return 0;
+    SSR_REQUIRE(w.means && w.quats && w.log_scales && w.opacity_logits && w.features_dc, where, "null world buffer");
+    if (sh_degree > 0) {
+        switch (sh.codec) {
+            case SSR_SH_F32:
+                SSR_REQUIRE(w.features_sh, where, "null features_sh");
+                SSR_REQUIRE(w.sh_stride >= 3 * sh_degree * (sh_degree + 2), where, "sh_stride too small for the SH degree");
+                break;
+            case SSR_SH_REF_Q8: case SSR_SH_REF_Q16:
+                SSR_REQUIRE(sh.packed && sh.bounds, where, "null quantized SH buffer");
+                SSR_REQUIRE(sh.num_sh_buffer >= (uint32_t)(sh_degree * (sh_degree + 2)), where, "num_sh_buffer too small");
+                SSR_REQUIRE(sh.bounds_stride >= 0, where, "negative bounds stride");
+                break;
+            case SSR_SH_I8_F16SCALE:
+                SSR_REQUIRE(sh.packed && sh.scale_f16, where, "null quantized SH buffer");
+                break;
+            default: return fail(where, "unknown SH codec");
+        }
+    }
+    return 0;
+}
+
+}  // namespace ssr
+
+using namespace ssr;
+
+extern "C" int ssr_projection_fwd(const ssr_projection_fwd_params* p, ssr_stream_t stream) {
+    SSR_REQUIRE(p, "ssr_projection_fwd", "null params");
+    int e = check_common("ssr_projection_fwd", p->num_splats, p->sh_degree, p->world, p->sh, p->camera);
+    if (e) return e;
+    if (p->num_splats == 0) return 0;
+    SSR_REQUIRE(p->aabb && p->sort_depth && p->radii, "ssr_projection_fwd", "null output");
+    SSR_REQUIRE(p->screen.xy && p->screen.depth && p->screen.conic && p->screen.opac && p->screen.rgb,
+                "ssr_projection_fwd", "null screen buffer");
+    SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->aabb) & 15) == 0 && (reinterpret_cast<uintptr_t>(p->world.quats) & 15) == 0,
+                "ssr_projection_fwd", "aabb and quats must be 16-byte aligned");
+    SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->screen.xy) & 7) == 0, "ssr_projection_fwd", "screen.xy must be 8-byte aligned");
+    const dim3 grid((unsigned)ceil_div(p->num_splats, kProjBlock)), block(kProjBlock);
+    hipStream_t s = as_stream(stream);
+    switch (p->sh_degree) {
+        case 0: hipLaunchKernelGGL(projection_fwd_kernel<0>, grid, block, 0, s, *p); break;
+        case 1: hipLaunchKernelGGL(projection_fwd_kernel<1>, grid, block, 0, s, *p); break;
+        case 2: hipLaunchKernelGGL(projection_fwd_kernel<2>, grid, block, 0, s, *p); break;
+        default: hipLaunchKernelGGL(projection_fwd_kernel<3>, grid, block, 0, s, *p); break;
+    }
+    SSR_CHECK_LAUNCH("ssr_projection_fwd");
+    return 0;
+}
+
+extern "C" int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream_t stream) {
+    SSR_REQUIRE(p, "ssr_projection_bwd", "null params");
+    int e = check_common("ssr_projection_bwd", p->num_splats, p->sh_degree, p->world, p->sh, p->camera);
+    if (e) return e;
+    if (p->num_splats == 0) return 0;   // src/kernels/projection/ProjectionBwd.cu:86-87
+    SSR_REQUIRE(p->aabb, "ssr_projection_bwd", "null aabb");   // ProjectionBwd.cu:89-97
+    SSR_REQUIRE(p->v_screen.xy && p->v_screen.depth && p->v_screen.conic && p->v_screen.opac && p->v_screen.rgb,
+                "ssr_projection_bwd", "null v_screen buffer");
+    const ssr_world& v = p->v_world;
+    SSR_REQUIRE(v.means && v.quats && v.log_scales && v.opacity_logits && v.features_dc && v.features_sh,
+                "ssr_projection_bwd", "null v_world buffer");
+    SSR_REQUIRE(v.sh_stride >= 3 * p->sh_degree * (p->sh_degree + 2), "ssr_projection_bwd", "v_world.sh_stride too small");
+    SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->aabb) & 15) == 0 && (reinterpret_cast<uintptr_t>(p->world.quats) & 15) == 0 &&
+                (reinterpret_cast<uintptr_t>(v.quats) & 15) == 0, "ssr_projection_bwd", "aabb and quats must be 16-byte aligned");
+    const dim3 grid((unsigned)ceil_div(p->num_splats, kProjBlock)), block(kProjBlock);
+    hipStream_t s = as_stream(stream);
+#define SSR_LAUNCH_BWD(D)                                                                          \
+    if (p->accumulate) hipLaunchKernelGGL((projection_bwd_kernel<D, true>), grid, block, 0, s, *p); \
+    else hipLaunchKernelGGL((projection_bwd_kernel<D, false>), grid, block, 0, s, *p)
+    switch (p->sh_degree) {
+        case 0: SSR_LAUNCH_BWD(0); break;
+        case 1: SSR_LAUNCH_BWD(1); break;
+        case 2: SSR_LAUNCH_BWD(2); break;
+        default: SSR_LAUNCH_BWD(3); break;
+    }
+#undef SSR_LAUNCH_BWD
+    SSR_CHECK_LAUNCH("ssr_projection_bwd");
+    return 0;
+}

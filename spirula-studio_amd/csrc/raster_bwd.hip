@@ -1,0 +1,192 @@
+// raster_bwd.hip -- K8: compositing backward. Replays each tile's sorted range back to front,
+// undoing the transmittance recursion, and accumulates per-Gaussian screen-space gradients.
+//
+// Follows rasterize_to_pixels_bwd_kernel with IS_EVAL3D=0, dist_type=None, no median, no
+// accumulation weights (src/kernels/raster/RasterizationEval3DBwd_kernel.cuh:48-636) and the
+// fragment VJPs of src/primitives/Primitive3DGS.cuh:262-300:
+//   per pixel   v_T <- v_T + depth_out * v_depth / W,  v_depth <- v_depth / W,  W = max(1-T,1e-10)
+//   per splat k <= last_id with alpha > 1/255:
+//     T0 = T1/(1-alpha); v_alpha = T0 (c.v_c) - v_T1 T0; v_c_k = alpha T0 v_c;
+//     v_T0 = alpha (c.v_c) + v_T1 (1-alpha)
+//
+// Native schedule instead of the reference's 32-lane systolic sweep: a wavefront holds the 64
+// pixels of one 8x8 sub-tile in its lanes (state in registers, no LDS traffic for it); fragments
+// are staged per 16x16 tile in LDS, back to front, shared by the tile's 4 wavefronts; each
+// wavefront walks the fragments whose footprint bit is set. The ten per-splat sums are reduced
+// across the wavefront with DPP (quad permutes, row mirrors, row broadcasts) and issued as ONE
+// 10-lane float atomic instruction per (splat, sub-tile) -- the same number of atomic operations
+// as the reference (src/primitives/PrimitiveBase3DGS.cuh:177-183), non-finite sums dropped and
+// zeros skipped as there (src/core/Common.cuh:791-856). The scan starts at the tile's largest
+// last_id rather than at the end of the range; splats beyond it are skipped by every pixel anyway.
+#include "raster_device.h"
+
+namespace ssr {
+
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ float dpp_get(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, kRowMask, 0xf, false));
+}
+
+// Sum over the 64 lanes; the total is valid in lanes 48..63.
+__device__ __forceinline__ float wave_sum_row3(float v) {
+    v += dpp_get<0xB1, 0xf>(v);    // quad_perm [1,0,3,2]
+    v += dpp_get<0x4E, 0xf>(v);    // quad_perm [2,3,0,1]
+    v += dpp_get<0x141, 0xf>(v);   // row_half_mirror
+    v += dpp_get<0x140, 0xf>(v);   // row_mirror: every lane of a row holds the row sum
+    v += dpp_get<0x142, 0xa>(v);   // row_bcast15 into rows 1 and 3
+    v += dpp_get<0x143, 0xc>(v);   // row_bcast31 into rows 2 and 3
+    return v;
+}
+
+__device__ __forceinline__ int wave_max_i32(int v) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) v = max(v, __shfl_xor(v, d, 64));
+    return v;
+}
+
+__global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd_params P, int tile_w, int tile_h) {
+    __shared__ FragLds frags[kBatch];
+    __shared__ int32_t s_ids[kBatch];
+    __shared__ int s_wave_max[4];
+    const int n_tiles = tile_w * tile_h;
+    const int tile = xcd_tile_of(blockIdx.x, n_tiles);
+    if (tile >= n_tiles) return;
+    const int tid = threadIdx.x, lane = tid & 63, mt = tid >> 6;
+    const int ty = tile / tile_w, tx = tile - ty * tile_w;
+    const int j = tx * kTile + (mt & 1) * kMicro + (lane & 7);
+    const int i = ty * kTile + (mt >> 1) * kMicro + (lane >> 3);
+    const float px = (float)j + 0.5f, py = (float)i + 0.5f;
+    const bool inside = (uint32_t)i < P.height && (uint32_t)j < P.width;
+    const int64_t pid = (int64_t)i * P.width + j;
+
+    // per-pixel state (RasterizationEval3DBwd_kernel.cuh:186-232)
+    const int32_t bin_final = inside ? P.last_ids[pid] : -1;
+    float T1 = inside ? P.render_T[pid] : 0.0f;
+    float vT1 = inside ? P.v_render_T[pid] : 0.0f;
+    float vr = 0.f, vg = 0.f, vb = 0.f, vd = 0.f;
+    if (inside) {
+        const float* v = P.v_render_rgb + 3 * pid;
+        vr = v[0]; vg = v[1]; vb = v[2];
+        vd = P.v_render_depth[pid];
+    }
+    {
+        const float inv_alpha = 1.0f / ssr_max(1.0f - T1, 1e-10f);
+        const float exp_depth = inside ? P.render_depth[pid] : 0.0f;
+        vT1 = vT1 + (exp_depth * vd) * inv_alpha;
+        vd = vd * inv_alpha;
+    }
+
+    const int32_t range_start = P.tile_offsets[tile];
+    const int32_t range_end = (tile == n_tiles - 1) ? (int32_t)P.n_isects : P.tile_offsets[tile + 1];
+    const int wave_last = wave_max_i32(bin_final);
+    if (lane == 0) s_wave_max[mt] = wave_last;
+    __syncthreads();
+    const int tile_last = max(max(s_wave_max[0], s_wave_max[1]), max(s_wave_max[2], s_wave_max[3]));
+    const float tile_x0 = (float)(tx * kTile), tile_y0 = (float)(ty * kTile);
+
+    for (int32_t hi = min(range_end - 1, tile_last); hi >= range_start; hi -= kBatch) {
+        __syncthreads();   // previous batch fully consumed
+        const int32_t idx = hi - tid;   // LDS slot t holds sorted index hi - t: ascending t is back to front
+        if (idx >= range_start) {
+            const int32_t g = P.flatten_ids[idx];
+            s_ids[tid] = g;
+            frags[tid] = stage_fragment(P.screen, g, tile_x0, tile_y0);
+        } else {
+            frags[tid].q2 = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        __syncthreads();
+        const int n_batch = min(kBatch, hi - range_start + 1);
+        for (int c = 0; c * 64 < n_batch; c++) {
+            if (hi - c * 64 - 63 > wave_last) continue;   // nothing in this chunk is <= any last_id here
+            const uint32_t my_hits = __float_as_uint(frags[c * 64 + lane].q2.z);
+            uint64_t m = __ballot((my_hits >> mt) & 1u);
+            while (m) {
+                const int t = __builtin_ctzll(m);
+                m &= m - 1;
+                const int k = c * 64 + t;
+                const int32_t sorted_idx = hi - k;
+                if (sorted_idx > wave_last) continue;
+                const float4 q0 = frags[k].q0, q1 = frags[k].q1;
+                float dx, dy, vis, sigma;
+                const float alpha = eval_alpha(q0, q1, px, py, dx, dy, vis, sigma);
+                const bool active = sorted_idx <= bin_final && alpha > kAlphaThreshold;
+                if (__ballot(active) == 0ull) continue;
+                const float4 q2 = frags[k].q2;
+                const float opac = q1.y, cr = q1.z, cg = q1.w, cb = q2.x, cdp = q2.y;
+                float t_x = 0.f, t_y = 0.f, t_d = 0.f, t_ca = 0.f, t_cb = 0.f, t_cc = 0.f, t_o = 0.f, t_r = 0.f,
+                      t_g = 0.f, t_b = 0.f;
+                if (active) {
+                    const float ra = 1.0f / (1.0f - alpha);
+                    const float T0 = T1 * ra;
+                    const float dotcv = ssr_fma(cdp, vd, ssr_fma(cb, vb, ssr_fma(cg, vg, cr * vr)));
+                    const float v_alpha = T0 * dotcv - vT1 * T0;
+                    const float w = alpha * T0;
+                    const float v_T0 = alpha * dotcv + vT1 * (1.0f - alpha);
+                    if (sigma >= 0.f && opac * vis <= 0.999f) {
+                        const float v_sigma = (-opac) * vis * v_alpha;
+                        const float conx = q0.z + q0.z, conz = q1.x + q1.x, cony = q0.w;   // full conic
+                        t_ca = 0.5f * v_sigma * dx * dx;
+                        t_cb = v_sigma * dx * dy;
+                        t_cc = 0.5f * v_sigma * dy * dy;
+                        t_x = v_sigma * (conx * dx + cony * dy);
+                        t_y = v_sigma * (cony * dx + conz * dy);
+                        t_o = vis * v_alpha;
+                    }
+                    t_r = vr * w; t_g = vg * w; t_b = vb * w; t_d = vd * w;
+                    T1 = T0; vT1 = v_T0;
+                }
+                // wavefront reduction, then lanes 48..57 each own one of the ten sums
+                const float s0 = wave_sum_row3(t_x), s1 = wave_sum_row3(t_y), s2 = wave_sum_row3(t_d),
+                            s3 = wave_sum_row3(t_ca), s4 = wave_sum_row3(t_cb), s5 = wave_sum_row3(t_cc),
+                            s6 = wave_sum_row3(t_o), s7 = wave_sum_row3(t_r), s8 = wave_sum_row3(t_g),
+                            s9 = wave_sum_row3(t_b);
+                const int q = lane - 48;
+                float mine = s0;
+                mine = q == 1 ? s1 : mine; mine = q == 2 ? s2 : mine; mine = q == 3 ? s3 : mine;
+                mine = q == 4 ? s4 : mine; mine = q == 5 ? s5 : mine; mine = q == 6 ? s6 : mine;
+                mine = q == 7 ? s7 : mine; mine = q == 8 ? s8 : mine; mine = q == 9 ? s9 : mine;
+                if (q >= 0 && q < 10 && ssr_isfinite(mine) && mine != 0.0f) {
+                    const int64_t g = s_ids[k];
+                    float* dst;
+                    switch (q) {
+                        case 0: dst = P.v_screen.xy + 2 * g; break;
+                        case 1: dst = P.v_screen.xy + 2 * g + 1; break;
+                        case 2: dst = P.v_screen.depth + g; break;
+                        case 3: dst = P.v_screen.conic + 3 * g; break;
+                        case 4: dst = P.v_screen.conic + 3 * g + 1; break;
+                        case 5: dst = P.v_screen.conic + 3 * g + 2; break;
+                        case 6: dst = P.v_screen.opac + g; break;
+                        case 7: dst = P.v_screen.rgb + 3 * g; break;
+                        case 8: dst = P.v_screen.rgb + 3 * g + 1; break;
+                        default: dst = P.v_screen.rgb + 3 * g + 2; break;
+                    }
+                    atomicAdd(dst, mine);
+                }
+            }
+        }
+    }
+}
+
+}  // namespace ssr
+
+using namespace ssr;
+
+extern "C" int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t stream) {
+    SSR_REQUIRE(p, "ssr_raster_bwd", "null params");
+    SSR_REQUIRE(p->width > 0 && p->height > 0, "ssr_raster_bwd", "empty image");
+    SSR_REQUIRE(p->n_isects >= 0 && p->n_isects < (int64_t)1 << 31, "ssr_raster_bwd", "n_isects out of range");
+    if (p->n_isects == 0) return 0;   // nothing contributed anywhere
+    SSR_REQUIRE(p->tile_offsets && p->flatten_ids, "ssr_raster_bwd", "null tile data");
+    SSR_REQUIRE(p->render_T && p->last_ids && p->render_depth, "ssr_raster_bwd", "null forward output");
+    SSR_REQUIRE(p->v_render_rgb && p->v_render_depth && p->v_render_T, "ssr_raster_bwd", "null output gradient");
+    SSR_REQUIRE(p->screen.xy && p->screen.depth && p->screen.conic && p->screen.opac && p->screen.rgb,
+                "ssr_raster_bwd", "null screen buffer");
+    SSR_REQUIRE(p->v_screen.xy && p->v_screen.depth && p->v_screen.conic && p->v_screen.opac && p->v_screen.rgb,
+                "ssr_raster_bwd", "null v_screen buffer");
+    SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->screen.xy) & 7) == 0, "ssr_raster_bwd", "screen.xy must be 8-byte aligned");
+    const int tw = (int)ceil_div(p->width, kTile), th = (int)ceil_div(p->height, kTile);
+    hipLaunchKernelGGL(raster_bwd_kernel, dim3((unsigned)xcd_grid_size(tw * th)), dim3(kRasterBlock), 0, as_stream(stream),
+                       *p, tw, th);
+    SSR_CHECK_LAUNCH("ssr_raster_bwd");
+    return 0;
+}

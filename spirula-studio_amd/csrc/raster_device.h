@@ -1,0 +1,87 @@
+// raster_device.h -- fragment staging and alpha evaluation shared by the compositing forward (K7)
+// and backward (K8) kernels.
+//
+// Work decomposition (native to 64-wide wavefronts): one 256-thread workgroup per 16x16 binning
+// tile; each of its 4 wavefronts owns one 8x8 sub-tile, one lane per pixel. The tile's sorted
+// range is staged through LDS in batches of 256 fragments (one fragment per thread, read once per
+// tile instead of once per sub-tile), together with a 4-bit footprint mask: bit m says whether
+// the splat's alpha >= 1/255 ellipse reaches sub-tile m. That is the reference's per-sub-tile
+// cull (src/kernels/raster/RasterizationEval3DFwd_kernel.cuh:203-209,
+// src/kernels/raster/RasterizationEval3DBwd_kernel.cuh:336-342 with ellipse_box_overlap_test,
+// src/core/Common.cuh:55-77); a wavefront walks only the fragments whose bit is set, with a
+// scalar bit-scan over a 64-bit ballot, so the skip costs no vector work.
+#pragma once
+#include "common.h"
+
+namespace ssr {
+
+constexpr int kRasterBlock = 256;
+constexpr int kBatch = 256;
+
+// One staged fragment: 3 x 16 bytes, read back with broadcast 128-bit LDS loads.
+//   q0 = (x, y, 0.5*conic.x, conic.y)   q1 = (0.5*conic.z, opac, r, g)   q2 = (b, depth, hitmask, -)
+struct FragLds {
+    float4 q0, q1, q2;
+};
+
+__device__ __forceinline__ bool ellipse_box_overlap(const float ic[3], float x0, float x1, float y0, float y1) {
+    float a = ic[0], b = ic[1], c = ic[2];
+    const float wx = (-b) / c, wy = (-b) / a;
+    const float u0 = ssr_min(ssr_max(x0 * wx, y0), y1);
+    const float u1 = ssr_min(ssr_max(x1 * wx, y0), y1);
+    const float v0 = ssr_min(ssr_max(y0 * wy, x0), x1);
+    const float v1 = ssr_min(ssr_max(y1 * wy, x0), x1);
+    b = b * 2.0f;
+    const float mx = ssr_min(((a * x0) * x0 + (b * x0) * u0) + (c * u0) * u0,
+                             ((a * x1) * x1 + (b * x1) * u1) + (c * u1) * u1);
+    const float my = ssr_min(((a * v0) * v0 + (b * v0) * y0) + (c * y0) * y0,
+                             ((a * v1) * v1 + (b * v1) * y1) + (c * y1) * y1);
+    const float mc = ssr_max(ssr_max(x0, -x1), ssr_max(y0, -y1));
+    return ssr_min(mc, ssr_min(mx, my) - 1.0f) < 0.f;
+}
+
+// Gathers splat `g` from the screen buffers and computes its sub-tile footprint mask.
+__device__ __forceinline__ FragLds stage_fragment(const ssr_screen& s, int32_t g, float tile_x0, float tile_y0) {
+    const float2 xy = *reinterpret_cast<const float2*>(s.xy + 2 * (int64_t)g);
+    const float* cn = s.conic + 3 * (int64_t)g;
+    const float cx = cn[0], cy = cn[1], cz = cn[2];
+    const float opac = s.opac[g];
+    const float* rg = s.rgb + 3 * (int64_t)g;
+    uint32_t hits = 0;
+    if (opac > kAlphaThreshold) {
+        const float kk = 0.5f / ssr_log(opac / kAlphaThreshold);
+        const float ic[3] = {cx * kk, cy * kk, cz * kk};
+#pragma unroll
+        for (int m = 0; m < 4; m++) {
+            const float bx0 = tile_x0 + (float)((m & 1) * kMicro), by0 = tile_y0 + (float)((m >> 1) * kMicro);
+            if (ellipse_box_overlap(ic, bx0 - xy.x, (bx0 + (float)kMicro) - xy.x, by0 - xy.y, (by0 + (float)kMicro) - xy.y))
+                hits |= 1u << m;
+        }
+    }
+    FragLds f;
+    f.q0 = make_float4(xy.x, xy.y, 0.5f * cx, cy);
+    f.q1 = make_float4(0.5f * cz, opac, rg[0], rg[1]);
+    f.q2 = make_float4(rg[2], s.depth[g], __uint_as_float(hits), 0.0f);
+    return f;
+}
+
+// FragmentFwd::evaluate_alpha (src/primitives/Primitive3DGS.cuh:250-260):
+// sigma = 0.5 (a dx^2 + c dy^2) + b dx dy with the fused operations placed as written here.
+__device__ __forceinline__ float eval_alpha(const float4& q0, const float4& q1, float px, float py, float& dx,
+                                            float& dy, float& vis, float& sigma) {
+    dx = q0.x - px; dy = q0.y - py;
+    sigma = ssr_fma(q0.z * dx, dx, ssr_fma(q1.x * dy, dy, (q0.w * dx) * dy));
+    vis = ssr_exp(-sigma);
+    const float alpha = ssr_min(0.999f, q1.y * vis);
+    return sigma < 0.f ? 0.f : alpha;
+}
+
+// Workgroup id -> tile id so that each of the 8 XCDs (workgroups are dealt to them round-robin)
+// works on one contiguous band of tiles and its L2 keeps that band's splat rows.
+__device__ __forceinline__ int xcd_tile_of(int wg, int n_tiles) {
+    const int chunk = (n_tiles + 7) >> 3;
+    return (wg & 7) * chunk + (wg >> 3);
+}
+inline int xcd_grid_size(int n_tiles) { return ((n_tiles + 7) >> 3) * 8; }
+
+}  // namespace ssr

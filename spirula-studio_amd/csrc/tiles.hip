@@ -1,0 +1,231 @@
+// tiles.hip -- K2 (tiles per splat), K3 (int64 inclusive scan), K4 (key write), K6 (tile offsets).
+//
+// K2/K4 follow intersect_tile_kernel<count, ellipse=true> (src/kernels/tile/IntersectTile.cu:104-267),
+// K6 follows intersect_offset_kernel (:271-307). Keys are (tile_id << 32) | depth bits with
+// depth bits = bits(|sorting depth|) ^ 0x80000000 (:190-196); values are flat splat indices.
+#include "projection_device.h"
+
+namespace ssr {
+
+constexpr int kTileBlock = 256;
+
+__global__ __launch_bounds__(kTileBlock) void tile_count_kernel(
+    int64_t n, const float4* __restrict__ aabb, const float2* __restrict__ xy,
+    const float* __restrict__ conic, const float* __restrict__ opac, int tile_w, int tile_h,
+    int64_t* __restrict__ tiles_per_splat) {
+    const int64_t g = (int64_t)blockIdx.x * kTileBlock + threadIdx.x;
+    if (g >= n) return;
+    const float4 a = aabb[g];
+    if (a.z <= a.x || a.w <= a.y) { tiles_per_splat[g] = 0; return; }
+    const float bb[4] = {a.x, a.y, a.z, a.w};
+    const float2 c = xy[g];
+    const float cxy[2] = {c.x, c.y};
+    const float cn[3] = {conic[3 * g], conic[3 * g + 1], conic[3 * g + 2]};
+    TileGeomD tg;
+    tile_geom(bb, cxy, cn, opac[g], tile_w, tile_h, tg);
+    tiles_per_splat[g] = count_tiles(tg);
+}
+
+__global__ __launch_bounds__(kTileBlock) void tile_write_kernel(
+    int64_t n, const float4* __restrict__ aabb, const float* __restrict__ sort_depth,
+    const float2* __restrict__ xy, const float* __restrict__ conic, const float* __restrict__ opac,
+    const int64_t* __restrict__ cum, int tile_w, int tile_h, int64_t* __restrict__ isect_ids,
+    int32_t* __restrict__ flatten_ids) {
+    const int64_t g = (int64_t)blockIdx.x * kTileBlock + threadIdx.x;
+    if (g >= n) return;
+    int64_t cur = g == 0 ? 0 : cum[g - 1];
+    const int64_t end = cum[g];
+    const float4 a = aabb[g];
+    if (!(a.z <= a.x || a.w <= a.y)) {
+        const float bb[4] = {a.x, a.y, a.z, a.w};
+        const float2 c = xy[g];
+        const float cxy[2] = {c.x, c.y};
+        const float cn[3] = {conic[3 * g], conic[3 * g + 1], conic[3 * g + 2]};
+        TileGeomD tg;
+        tile_geom(bb, cxy, cn, opac[g], tile_w, tile_h, tg);
+        uint32_t du = ssr_f2u(ssr_fabs(sort_depth[g]));
+        du = (du >> 31) ? ~du : (du ^ 0x80000000u);
+        for_each_tile(tg, [&](int lo, int hi, int fixed, bool rows) {
+            for (int v = lo; v < hi && cur < end; v++) {
+                const int64_t tile_id = rows ? ((int64_t)fixed * tile_w + v) : ((int64_t)v * tile_w + fixed);
+                isect_ids[cur] = (int64_t)(((uint64_t)tile_id << 32) | (uint64_t)du);
+                flatten_ids[cur] = (int32_t)g;
+                ++cur;
+            }
+        });
+    }
+    while (cur < end) {   // IntersectTile.cu:261-266; unreachable when count and write agree
+        isect_ids[cur] = (int64_t)0xffffffffull;
+        flatten_ids[cur] = (int32_t)g;
+        ++cur;
+    }
+}
+
+// ---- int64 inclusive scan: per-block reduce, single-block scan of the block sums, downsweep ----
+
+constexpr int kScanBlock = 256;
+constexpr int kScanItems = 8;
+constexpr int kScanTile = kScanBlock * kScanItems;
+
+__device__ __forceinline__ int64_t wave_inclusive_scan(int64_t v, int lane) {
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int64_t o = __shfl_up(v, d, 64);
+        if (lane >= d) v += o;
+    }
+    return v;
+}
+
+// Exclusive prefix of `v` over the block plus the block total; 4 wavefronts.
+__device__ __forceinline__ int64_t block_exclusive_scan(int64_t v, int64_t& total, int64_t* lds /* [4] */) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t inc = wave_inclusive_scan(v, lane);
+    if (lane == 63) lds[wave] = inc;
+    __syncthreads();
+    int64_t base = 0;
+#pragma unroll
+    for (int w = 0; w < kScanBlock / 64; w++) { if (w < wave) base += lds[w]; }
+    total = lds[0] + lds[1] + lds[2] + lds[3];
+    __syncthreads();
+    return base + inc - v;
+}
+
+__global__ __launch_bounds__(kScanBlock) void scan_reduce_kernel(const int64_t* __restrict__ in, int64_t n,
+                                                                 int64_t* __restrict__ block_sums) {
+    __shared__ int64_t lds[4];
+    const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
+    int64_t s = 0;
+#pragma unroll
+    for (int i = 0; i < kScanItems; i++) { if (base + i < n) s += in[base + i]; }
+    int64_t total;
+    block_exclusive_scan(s, total, lds);
+    if (threadIdx.x == 0) block_sums[blockIdx.x] = total;
+}
+
+__global__ __launch_bounds__(kScanBlock) void scan_spine_kernel(int64_t* __restrict__ block_sums, int64_t n_blocks) {
+    __shared__ int64_t lds[4];
+    int64_t carry = 0;
+    for (int64_t start = 0; start < n_blocks; start += kScanBlock) {
+        const int64_t i = start + threadIdx.x;
+        const int64_t v = i < n_blocks ? block_sums[i] : 0;
+        int64_t total;
+        const int64_t ex = block_exclusive_scan(v, total, lds);
+        if (i < n_blocks) block_sums[i] = carry + ex;   // exclusive prefix
+        carry += total;
+    }
+}
+
+__global__ __launch_bounds__(kScanBlock) void scan_down_kernel(const int64_t* __restrict__ in, int64_t n,
+                                                               const int64_t* __restrict__ block_prefix,
+                                                               int64_t* __restrict__ out) {
+    __shared__ int64_t lds[4];
+    const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
+    int64_t v[kScanItems];
+    int64_t s = 0;
+#pragma unroll
+    for (int i = 0; i < kScanItems; i++) { v[i] = base + i < n ? in[base + i] : 0; s += v[i]; }
+    int64_t total;
+    int64_t run = block_prefix[blockIdx.x] + block_exclusive_scan(s, total, lds);
+#pragma unroll
+    for (int i = 0; i < kScanItems; i++) { run += v[i]; if (base + i < n) out[base + i] = run; }
+}
+
+// ---- K6 ----
+
+__global__ __launch_bounds__(kTileBlock) void tile_offsets_kernel(int64_t n_isects, const int64_t* __restrict__ ids,
+                                                                  int64_t n_tiles, int32_t* __restrict__ offsets) {
+    const int64_t idx = (int64_t)blockIdx.x * kTileBlock + threadIdx.x;
+    if (idx >= n_isects) return;
+    const int64_t tile = ids[idx] >> 32;
+    if (idx == 0)
+        for (int64_t i = 0; i < tile + 1 && i < n_tiles; ++i) offsets[i] = 0;
+    if (idx == n_isects - 1)
+        for (int64_t i = tile + 1; i < n_tiles; ++i) offsets[i] = (int32_t)n_isects;
+    if (idx > 0) {
+        const int64_t prev = ids[idx - 1] >> 32;
+        if (prev != tile)
+            for (int64_t i = prev + 1; i < tile + 1 && i < n_tiles; ++i) offsets[i] = (int32_t)idx;
+    }
+}
+
+}  // namespace ssr
+
+using namespace ssr;
+
+extern "C" {
+
+int ssr_tile_count(int64_t n, const float* aabb, const float* xy, const float* conic, const float* opac,
+                   uint32_t width, uint32_t height, int64_t* tiles_per_splat, ssr_stream_t stream) {
+    SSR_REQUIRE(n >= 0 && n < (int64_t)1 << 31, "ssr_tile_count", "count out of range");
+    if (n == 0) return 0;
+    SSR_REQUIRE(aabb && xy && conic && opac && tiles_per_splat, "ssr_tile_count", "null pointer");
+    SSR_REQUIRE(width > 0 && height > 0, "ssr_tile_count", "empty image");
+    SSR_REQUIRE((reinterpret_cast<uintptr_t>(aabb) & 15) == 0 && (reinterpret_cast<uintptr_t>(xy) & 7) == 0,
+                "ssr_tile_count", "aabb must be 16-byte and xy 8-byte aligned");
+    const int tw = (int)ceil_div(width, kTile), th = (int)ceil_div(height, kTile);
+    hipLaunchKernelGGL(tile_count_kernel, dim3((unsigned)ceil_div(n, kTileBlock)), dim3(kTileBlock), 0, as_stream(stream),
+                       n, reinterpret_cast<const float4*>(aabb), reinterpret_cast<const float2*>(xy), conic, opac, tw, th,
+                       tiles_per_splat);
+    SSR_CHECK_LAUNCH("ssr_tile_count");
+    return 0;
+}
+
+size_t ssr_scan_scratch_bytes(int64_t n) {
+    if (n <= 0) return 0;
+    return (size_t)ceil_div(n, kScanTile) * sizeof(int64_t);
+}
+
+int ssr_inclusive_sum_i64(const int64_t* in, int64_t* out, int64_t n, void* scratch, size_t scratch_bytes,
+                          ssr_stream_t stream) {
+    SSR_REQUIRE(n >= 0, "ssr_inclusive_sum_i64", "negative count");
+    if (n == 0) return 0;
+    SSR_REQUIRE(in && out, "ssr_inclusive_sum_i64", "null pointer");
+    SSR_REQUIRE(scratch && scratch_bytes >= ssr_scan_scratch_bytes(n), "ssr_inclusive_sum_i64", "scratch too small");
+    const int64_t nb = ceil_div(n, kScanTile);
+    int64_t* sums = reinterpret_cast<int64_t*>(scratch);
+    hipStream_t s = as_stream(stream);
+    hipLaunchKernelGGL(scan_reduce_kernel, dim3((unsigned)nb), dim3(kScanBlock), 0, s, in, n, sums);
+    hipLaunchKernelGGL(scan_spine_kernel, dim3(1), dim3(kScanBlock), 0, s, sums, nb);
+    hipLaunchKernelGGL(scan_down_kernel, dim3((unsigned)nb), dim3(kScanBlock), 0, s, in, n, sums, out);
+    SSR_CHECK_LAUNCH("ssr_inclusive_sum_i64");
+    return 0;
+}
+
+int ssr_tile_write(int64_t n, const float* aabb, const float* sort_depth, const float* xy, const float* conic,
+                   const float* opac, const int64_t* cum_tiles, uint32_t width, uint32_t height, int64_t* isect_ids,
+                   int32_t* flatten_ids, ssr_stream_t stream) {
+    SSR_REQUIRE(n >= 0 && n < (int64_t)1 << 31, "ssr_tile_write", "count out of range");
+    if (n == 0) return 0;
+    SSR_REQUIRE(aabb && sort_depth && xy && conic && opac && cum_tiles, "ssr_tile_write", "null pointer");
+    SSR_REQUIRE(isect_ids && flatten_ids, "ssr_tile_write", "null output (n_isects == 0 needs no call)");
+    SSR_REQUIRE(width > 0 && height > 0, "ssr_tile_write", "empty image");
+    SSR_REQUIRE((reinterpret_cast<uintptr_t>(aabb) & 15) == 0 && (reinterpret_cast<uintptr_t>(xy) & 7) == 0,
+                "ssr_tile_write", "aabb must be 16-byte and xy 8-byte aligned");
+    const int tw = (int)ceil_div(width, kTile), th = (int)ceil_div(height, kTile);
+    hipLaunchKernelGGL(tile_write_kernel, dim3((unsigned)ceil_div(n, kTileBlock)), dim3(kTileBlock), 0, as_stream(stream),
+                       n, reinterpret_cast<const float4*>(aabb), sort_depth, reinterpret_cast<const float2*>(xy), conic, opac,
+                       cum_tiles, tw, th, isect_ids, flatten_ids);
+    SSR_CHECK_LAUNCH("ssr_tile_write");
+    return 0;
+}
+
+int ssr_sort_end_bit(uint32_t n_tiles) {
+    int b = 0;
+    while (b < 32 && (1u << b) <= n_tiles) ++b;   // src/kernels/tile/IntersectTile.cu:489-490
+    return 32 + b;
+}
+
+int ssr_tile_offsets(int64_t n_isects, const int64_t* sorted_ids, uint32_t n_tiles, int32_t* offsets,
+                     ssr_stream_t stream) {
+    SSR_REQUIRE(n_isects >= 0 && n_isects < (int64_t)1 << 31, "ssr_tile_offsets", "n_isects out of range");
+    if (n_tiles == 0) return 0;
+    SSR_REQUIRE(offsets, "ssr_tile_offsets", "null offsets");
+    if (n_isects == 0) return ssr_fill_u32(offsets, 0u, n_tiles, stream);   // IntersectTile.cu:448-451
+    SSR_REQUIRE(sorted_ids, "ssr_tile_offsets", "null keys");
+    hipLaunchKernelGGL(tile_offsets_kernel, dim3((unsigned)ceil_div(n_isects, kTileBlock)), dim3(kTileBlock), 0,
+                       as_stream(stream), n_isects, sorted_ids, (int64_t)n_tiles, offsets);
+    SSR_CHECK_LAUNCH("ssr_tile_offsets");
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,190 @@
+"""Drives the hot path stage by stage through the C ABI (libssr_hip.so) from Python, for the GPU
+parity tests. Mirrors the call order of the reference's engine
+(src/engine/EngineForward.cpp:166-293, src/engine/EngineLoss.cpp:138-240,359-368)."""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+
+class GpuRun:
+    def __init__(self, pkg, scene, sh_degree=3):
+        self.L = pkg.lib
+        self.lib = self.L.load()
+        self.check = self.L.check
+        self.sc = scene
+        self.sh_degree = sh_degree
+        D = self.L.DeviceArray
+        sc = scene
+        n = sc.n
+        self.n = n
+        self.d = {}
+        for k in ["means", "quats", "log_scales", "opacity_logits", "features_dc"]:
+            self.d[k] = D.from_host(getattr(sc, k).astype(np.float32))
+        if sc.sh_codec == 0:
+            self.d["features_sh"] = D.from_host(sc.features_sh.astype(np.float32))
+        else:
+            self.d["sh_packed"] = D.from_host(sc.sh_packed)
+            if sc.sh_bounds is not None:
+                self.d["sh_bounds"] = D.from_host(sc.sh_bounds.astype(np.float32))
+            if sc.sh_scale_f16 is not None:
+                self.d["sh_scale"] = D.from_host(sc.sh_scale_f16.view(np.uint16))
+        self.d["viewmat"] = D.from_host(sc.viewmat.astype(np.float32))
+        self.d["intrins"] = D.from_host(sc.intrins.astype(np.float32))
+        for k, shape in [("aabb", (n, 4)), ("sort_depth", (n,)), ("radii", (n,)), ("xy", (n, 2)),
+                         ("depth", (n,)), ("conic", (n, 3)), ("opac", (n,)), ("rgb", (n, 3))]:
+            self.d[k] = D(shape, np.float32)
+        self.d["counts"] = D((n,), np.int64)
+        self.d["cum"] = D((n,), np.int64)
+
+    def ptr(self, k):
+        a = self.d.get(k)
+        return a.ptr if a is not None else None
+
+    def world(self, prefix=""):
+        w = self.L.World()
+        w.means, w.quats, w.log_scales = self.ptr(prefix + "means"), self.ptr(prefix + "quats"), self.ptr(prefix + "log_scales")
+        w.opacity_logits, w.features_dc = self.ptr(prefix + "opacity_logits"), self.ptr(prefix + "features_dc")
+        w.features_sh = self.ptr(prefix + "features_sh")
+        w.sh_stride = 45
+        return w
+
+    def shq(self):
+        q = self.L.ShQuant()
+        q.codec = self.sc.sh_codec
+        q.packed, q.bounds, q.scale_f16 = self.ptr("sh_packed"), self.ptr("sh_bounds"), self.ptr("sh_scale")
+        q.bounds_stride = self.sc.sh_bounds_stride
+        q.num_sh_buffer = 15
+        return q
+
+    def camera(self):
+        c = self.L.Camera()
+        c.camera_model, c.num_cameras = self.sc.camera_model, 1
+        c.width, c.height = self.sc.width, self.sc.height
+        c.viewmats, c.intrins = self.ptr("viewmat"), self.ptr("intrins")
+        return c
+
+    def screen(self, prefix=""):
+        s = self.L.Screen()
+        s.xy, s.depth, s.conic = self.ptr(prefix + "xy"), self.ptr(prefix + "depth"), self.ptr(prefix + "conic")
+        s.opac, s.rgb = self.ptr(prefix + "opac"), self.ptr(prefix + "rgb")
+        return s
+
+    # ---- stages ----
+    def projection_fwd(self, fused_count=False):
+        for k in ["radii"]:
+            self.d[k].fill_zero()
+        p = self.L.ProjectionFwdParams()
+        p.num_splats, p.sh_degree = self.n, self.sh_degree
+        p.world, p.sh, p.camera = self.world(), self.shq(), self.camera()
+        p.aabb, p.sort_depth, p.radii = self.ptr("aabb"), self.ptr("sort_depth"), self.ptr("radii")
+        p.screen = self.screen()
+        p.tiles_per_splat = self.ptr("counts") if fused_count else None
+        self.check(self.lib.ssr_projection_fwd(C.byref(p), None))
+
+    def tiles(self, fused_count=False):
+        sc, D = self.sc, self.L.DeviceArray
+        n = self.n
+        if not fused_count:
+            self.check(self.lib.ssr_tile_count(n, self.ptr("aabb"), self.ptr("xy"), self.ptr("conic"),
+                                               self.ptr("opac"), sc.width, sc.height, self.ptr("counts"), None))
+        sb = self.lib.ssr_scan_scratch_bytes(n)
+        self.d["scan_scratch"] = D((max(sb, 8),), np.uint8)
+        self.check(self.lib.ssr_inclusive_sum_i64(self.ptr("counts"), self.ptr("cum"), n,
+                                                  self.ptr("scan_scratch"), sb, None))
+        k = C.c_int64(0)
+        if n:
+            self.check(self.lib.ssr_read_i64(self.d["cum"].ptr + 8 * (n - 1), C.byref(k), None))
+        self.K = K = int(k.value)
+        n_tiles = sc.tile_w * sc.tile_h
+        self.d["offsets"] = D((n_tiles,), np.int32)
+        for nm in ["keys_a", "keys_b"]:
+            self.d[nm] = D((K,), np.int64)
+        for nm in ["vals_a", "vals_b"]:
+            self.d[nm] = D((K,), np.int32)
+        self.sel = 0
+        if K:
+            self.check(self.lib.ssr_tile_write(n, self.ptr("aabb"), self.ptr("sort_depth"), self.ptr("xy"),
+                                               self.ptr("conic"), self.ptr("opac"), self.ptr("cum"), sc.width,
+                                               sc.height, self.ptr("keys_a"), self.ptr("vals_a"), None))
+            self.unsorted_keys = self.d["keys_a"].to_host()
+            self.unsorted_vals = self.d["vals_a"].to_host()
+            sb = self.lib.ssr_sort_scratch_bytes(K)
+            self.d["sort_scratch"] = D((sb,), np.uint8)
+            sel = C.c_int(0)
+            self.check(self.lib.ssr_sort_pairs_u64_i32(self.ptr("keys_a"), self.ptr("keys_b"), self.ptr("vals_a"),
+                                                       self.ptr("vals_b"), K, 0, self.lib.ssr_sort_end_bit(n_tiles),
+                                                       C.byref(sel), self.ptr("sort_scratch"), sb, None))
+            self.sel = sel.value
+        else:
+            self.unsorted_keys = np.zeros(0, np.int64)
+            self.unsorted_vals = np.zeros(0, np.int32)
+        self.keys = "keys_b" if self.sel else "keys_a"
+        self.vals = "vals_b" if self.sel else "vals_a"
+        self.check(self.lib.ssr_tile_offsets(K, self.ptr(self.keys), n_tiles, self.ptr("offsets"), None))
+
+    def raster_fwd(self):
+        sc, D = self.sc, self.L.DeviceArray
+        h, w = sc.height, sc.width
+        for k, shape, dt in [("r_rgb", (h, w, 3), np.float32), ("r_depth", (h, w), np.float32),
+                             ("r_T", (h, w), np.float32), ("r_last", (h, w), np.int32)]:
+            self.d[k] = D(shape, dt)
+        p = self.L.RasterFwdParams()
+        p.num_splats, p.screen, p.width, p.height = self.n, self.screen(), w, h
+        p.tile_offsets, p.flatten_ids, p.n_isects = self.ptr("offsets"), self.ptr(self.vals), self.K
+        p.render_rgb, p.render_depth, p.render_T, p.last_ids = (self.ptr("r_rgb"), self.ptr("r_depth"),
+                                                                self.ptr("r_T"), self.ptr("r_last"))
+        self.check(self.lib.ssr_raster_fwd(C.byref(p), None))
+
+    def raster_bwd(self, v_rgb=None, v_depth=None, v_T=None):
+        sc, D = self.sc, self.L.DeviceArray
+        n = self.n
+        self.d["g_rgb"] = D.from_host(np.asarray(sc.v_rgb if v_rgb is None else v_rgb, np.float32))
+        self.d["g_depth"] = D.from_host(np.asarray(sc.v_depth if v_depth is None else v_depth, np.float32))
+        self.d["g_T"] = D.from_host(np.asarray(sc.v_T if v_T is None else v_T, np.float32))
+        for k, shape in [("v_xy", (n, 2)), ("v_depth", (n,)), ("v_conic", (n, 3)), ("v_opac", (n,)), ("v_rgb", (n, 3))]:
+            if k not in self.d:
+                self.d[k] = D(shape, np.float32)
+            self.d[k].fill_zero()
+        p = self.L.RasterBwdParams()
+        p.num_splats, p.screen, p.width, p.height = n, self.screen(), sc.width, sc.height
+        p.tile_offsets, p.flatten_ids, p.n_isects = self.ptr("offsets"), self.ptr(self.vals), self.K
+        p.render_T, p.last_ids, p.render_depth = self.ptr("r_T"), self.ptr("r_last"), self.ptr("r_depth")
+        p.v_render_rgb, p.v_render_depth, p.v_render_T = self.ptr("g_rgb"), self.ptr("g_depth"), self.ptr("g_T")
+        p.v_screen = self.screen("v_")
+        self.check(self.lib.ssr_raster_bwd(C.byref(p), None))
+
+    def projection_bwd(self, accumulate=True, poison=False):
+        D = self.L.DeviceArray
+        n = self.n
+        for k, shape in [("w_means", (n, 3)), ("w_quats", (n, 4)), ("w_log_scales", (n, 3)),
+                         ("w_opacity_logits", (n,)), ("w_features_dc", (n, 3)), ("w_features_sh", (n, 15, 3))]:
+            if k not in self.d:
+                self.d[k] = D(shape, np.float32)
+            if poison:
+                self.check(self.lib.ssr_fill_u32(self.d[k].ptr, 0x7fc00000, self.d[k].nbytes // 4, None))
+            else:
+                self.d[k].fill_zero()
+        p = self.L.ProjectionBwdParams()
+        p.num_splats, p.sh_degree = n, self.sh_degree
+        p.world, p.sh, p.camera = self.world(), self.shq(), self.camera()
+        p.aabb, p.v_screen, p.v_world = self.ptr("aabb"), self.screen("v_"), self.world("w_")
+        p.accumulate = 1 if accumulate else 0
+        self.check(self.lib.ssr_projection_bwd(C.byref(p), None))
+
+    def run_all(self, backward=True, fused_count=False):
+        self.projection_fwd(fused_count)
+        self.tiles(fused_count)
+        self.raster_fwd()
+        if backward:
+            self.raster_bwd()
+            self.projection_bwd()
+        self.check(self.lib.ssr_device_synchronize())
+        return self
+
+    def host(self, k):
+        return self.d[k].to_host()
+
+    def proj_host(self):
+        return {k: self.host(k) for k in ["aabb", "sort_depth", "radii", "xy", "depth", "conic", "opac", "rgb"]}

@@ -1,0 +1,134 @@
+"""GPU parity: the HIP path, called through the C ABI, against the CPU oracle on the same seeded
+inputs. Bars: tile keys / sorted ids / tile ranges bit-exact; images max-abs 1e-4 per channel;
+gradients 1e-3 relative (with a floor proportional to the sum of |terms|, since float atomics add
+in a different order)."""
+import numpy as np
+import pytest
+
+from gpu_pipeline import GpuRun
+
+pytestmark = pytest.mark.gpu
+
+IMG_TOL = 1e-4
+GRAD_RTOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def gpu(pkg):
+    from spirula_studio_amd import lib
+    pkg.lib = lib
+    lib.check(lib.load().ssr_init(0))
+    return pkg
+
+
+def _grad_close(got, ref, abs_scale, name):
+    got, ref = got.astype(np.float64), ref.astype(np.float64)
+    tol = GRAD_RTOL * np.abs(ref) + 2e-6 * abs_scale + 1e-9
+    bad = np.abs(got - ref) > tol
+    assert not bad.any(), (name, int(bad.sum()), float(np.abs(got - ref).max()),
+                           got[bad][:4], ref[bad][:4])
+
+
+def _compare(gpu, oracle, sc, label, fused_count=False):
+    r = oracle.pipeline(sc)
+    print(f"[{label}] N={sc.n} {sc.width}x{sc.height} visible={r['proj']['visible']} K={r['isect_ids'].size}", flush=True)
+    g = GpuRun(gpu, sc).run_all(fused_count=fused_count)
+    vis = r["proj"]["aabb"][:, 2] > r["proj"]["aabb"][:, 0]
+    # K1: bit-exact on every compared array (culled screen rows are not written by either side)
+    p = g.proj_host()
+    for k in ["aabb", "sort_depth", "radii"]:
+        assert np.array_equal(p[k].view(np.uint32), r["proj"][k].view(np.uint32)), k
+    for k in ["xy", "depth", "conic", "opac", "rgb"]:
+        assert np.array_equal(p[k][vis].view(np.uint32), r["proj"][k][vis].view(np.uint32)), k
+    # K2..K6: bit-exact
+    assert np.array_equal(g.host("counts"), r["counts"])
+    assert np.array_equal(g.host("cum"), r["cum"])
+    assert g.K == r["isect_ids"].size
+    assert np.array_equal(g.unsorted_keys, r["isect_ids"])
+    assert np.array_equal(g.unsorted_vals, r["flatten_ids"])
+    assert np.array_equal(g.host(g.keys), r["sorted_ids"])
+    assert np.array_equal(g.host(g.vals), r["sorted_flat"])
+    assert np.array_equal(g.host("offsets"), r["offsets"])
+    # K7
+    f = r["fwd"]
+    assert np.abs(g.host("r_rgb") - f["rgb"]).max() <= IMG_TOL
+    assert np.abs(g.host("r_T") - f["T"]).max() <= IMG_TOL
+    dd = np.abs(g.host("r_depth") - f["depth"])
+    assert (dd <= IMG_TOL * np.maximum(1.0, np.abs(f["depth"]))).all()
+    assert np.array_equal(g.host("r_last"), f["last_ids"])
+    # K8
+    vs = r["vscreen"]
+    ab = vs["abs_terms"]
+    _grad_close(g.host("v_xy"), vs["v_xy"], ab[:, 0:2], "v_xy")
+    _grad_close(g.host("v_depth"), vs["v_depth"], ab[:, 2], "v_depth")
+    _grad_close(g.host("v_conic"), vs["v_conic"], ab[:, 3:6], "v_conic")
+    _grad_close(g.host("v_opac"), vs["v_opac"], ab[:, 6], "v_opac")
+    _grad_close(g.host("v_rgb"), vs["v_rgb"], ab[:, 7:10], "v_rgb")
+    # K9, fed its own K8 output: compare with the oracle chain under a norm-relative bar
+    gr = r["grads"]
+    for k, o in [("w_means", "v_means"), ("w_quats", "v_quats"), ("w_log_scales", "v_scales"),
+                 ("w_opacity_logits", "v_opacities"), ("w_features_dc", "v_dc"), ("w_features_sh", "v_sh")]:
+        got, ref = g.host(k).astype(np.float64), gr[o].astype(np.float64)
+        rows = ref.reshape(sc.n, -1)
+        scale = np.abs(rows).max(axis=1, keepdims=True) + 1e-30
+        err = np.abs(got.reshape(sc.n, -1) - rows)
+        # per-row relative bar, with a floor for rows whose inputs cancel
+        floor = 2e-5 * (np.abs(rows).mean() + 1e-12)
+        assert (err <= 2 * GRAD_RTOL * scale + floor).all(), (k, float((err / scale).max()))
+        assert not np.any(got[~vis]), k
+    return g, r
+
+
+def test_device_math_is_bit_identical_to_host(gpu, oracle):
+    lib, L = gpu.lib.load(), gpu.lib
+    rng = np.random.default_rng(0)
+    a = np.concatenate([rng.uniform(-100, 100, 300000), rng.normal(0, 3, 300000),
+                        [0.0, -0.0, 1.0, 88.7, -87.3, 1e-40, 255.0]]).astype(np.float32)
+    b = rng.normal(0, 3, a.size).astype(np.float32)
+    db, do = L.DeviceArray.from_host(b), L.DeviceArray(a.shape, np.float32)
+    for op in range(4):
+        x = np.abs(a) if op == 1 else a
+        da = L.DeviceArray.from_host(x)
+        L.check(lib.ssr_debug_math(op, a.size, da.ptr, db.ptr, do.ptr, None))
+        got = do.to_host()
+        want = oracle.math(op, x, b)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), op
+
+
+def test_tiny_pinhole(gpu, oracle):
+    _compare(gpu, oracle, gpu.scenes.tiny_scene(n=400, width=72, height=56, seed=3), "tiny")
+
+
+def test_tiny_fused_count(gpu, oracle):
+    _compare(gpu, oracle, gpu.scenes.tiny_scene(n=500, width=64, height=64, seed=5), "tiny-fused", fused_count=True)
+
+
+def test_tiny_equirect(gpu, oracle):
+    _compare(gpu, oracle, gpu.scenes.tiny_scene(n=600, width=128, height=64, seed=4, camera_model=3), "tiny-eq")
+
+
+def test_config1_reduced(gpu, oracle):
+    _compare(gpu, oracle, gpu.scenes.make_scene(1, n=20000, width=400, height=400, parity_variant=True), "cfg1/5")
+
+
+def test_config1_full(gpu, oracle):
+    _compare(gpu, oracle, gpu.scenes.make_scene(1), "cfg1")
+
+
+@pytest.mark.parametrize("codec,stride", [(1, 256), (1, 0), (2, 256), (3, 0)])
+def test_quantized_sh(gpu, oracle, codec, stride):
+    sc = gpu.scenes.make_scene(3, n=30000, width=480, height=270, sh_codec=0)
+    gpu.scenes.apply_sh_codec(sc, codec, bounds_stride=stride)
+    _compare(gpu, oracle, sc, f"cfg3-codec{codec}-stride{stride}")
+
+
+def test_config5_reduced_equirect(gpu, oracle):
+    _compare(gpu, oracle, gpu.scenes.make_scene(5, n=40000, width=512, height=256, parity_variant=True), "cfg5/150")
+
+
+def test_empty_and_culled(gpu, oracle):
+    sc = gpu.scenes.tiny_scene(n=64, width=40, height=24, seed=1)
+    sc.means[:, 2] = -10.0
+    g, r = _compare(gpu, oracle, sc, "all-culled")
+    assert g.K == 0 and not np.any(g.host("offsets"))
+    assert np.all(g.host("r_T") == 1.0)
