@@ -1,0 +1,195 @@
+#!/usr/bin/env python3
+"""Benchmark of the splat-raster hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2]
+
+One step = one forward+backward iteration of the path on a seeded synthetic scene whose inputs
+and pixel cotangents are already resident in HBM: zero radii -> projection+SH (with the tile
+count fused) -> int64 scan + 8-byte count readback -> key write -> 64-bit radix sort -> tile
+offsets -> compositing forward -> zero v_screen -> compositing backward -> projection backward.
+Prints ONE JSON line: the metric of BASELINE.json (iterations/s), a `roofline` object for the
+kernel that takes the most time, and a `cpu_baseline` object (the CPU oracle timed on this host).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E peak
+
+
+def algorithmic_bytes(N, V, K, K_f, K_b, P, T, S):
+    """Minimum HBM bytes per stage for one iteration: every array an algorithm of this shape must
+    read or write once. N splats, V visible, K splat-tile pairs, K_f / K_b pairs the forward /
+    backward actually need, P pixels, T tiles, S bytes of higher-order SH storage per splat."""
+    return {
+        "K1": N * (44 + 20) + V * (12 + S + 40 + 4),
+        "K2": N * 16 + V * (24 + 8) + (N - V) * 8,
+        "K3": N * 16,
+        "K4": N * 16 + V * (24 + 4 + 16) + K * 12,
+        "K5": 6 * K * 24,
+        "K6": K * 8 + T * 4,
+        "K7": K_f * 44 + P * 24,
+        "K8": P * 32 + K_b * 44 + K_b * 40 + N * 40,
+        "K9": N * 16 + V * (56 + S + 40) + V * 236 + N * 236,
+    }
+
+
+def tile_need(offsets, last_ids, n_isects, width, height):
+    """K_b: per tile, (largest last_id over its pixels) - range start + 1, summed over tiles."""
+    import numpy as np
+    tw, th = (width + 15) // 16, (height + 15) // 16
+    pad = np.full((th * 16, tw * 16), -1, np.int64)
+    pad[:height, :width] = last_ids.reshape(height, width)
+    tmax = pad.reshape(th, 16, tw, 16).max(axis=(1, 3)).reshape(-1)
+    start = offsets.astype(np.int64)
+    end = np.concatenate([start[1:], [n_isects]])
+    need = np.clip(np.minimum(tmax, end - 1) - start + 1, 0, None)
+    need[end <= start] = 0
+    return int(need.sum())
+
+
+def cpu_baseline(pkg, cfg, budget_s=20.0):
+    """The CPU oracle on this host's cores, on a bounded sample of the same workload."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_lib
+    full = pkg.scenes.CONFIGS[cfg]
+    # sample: the same scene at 1/8 of the splats and 1/8 of the pixels keeps the per-tile load
+    frac = 8
+    n = max(1000, full["n"] // frac)
+    w = max(64, int(full["w"] / frac ** 0.5) // 16 * 16)
+    h = max(64, int(full["h"] / frac ** 0.5) // 16 * 16)
+    sc = pkg.scenes.make_scene(cfg, n=n, width=w, height=h)
+    oracle_lib.lib()
+    cores = oracle_lib.lib().or_num_threads()
+    t0 = time.time()
+    iters = 0
+    while True:
+        oracle_lib.pipeline(sc)
+        iters += 1
+        if time.time() - t0 > budget_s or iters >= 50:
+            break
+    dt = (time.time() - t0) / iters
+    # whole-config rate estimated from the sample: work scales with splats and with pixels
+    est = 1.0 / (dt * frac)
+    return {"value": est, "unit": "iters/s", "cores": cores, "kind": "port",
+            "sample": f"{iters} iteration(s) of config {cfg} at N={n}, {w}x{h} (1/{frac} of the splats and of "
+                      f"the pixels): {dt * 1e3:.1f} ms each; value = sample rate / {frac}"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", type=int, default=2, help="1..5 (BASELINE.json configs; 2 is the headline)")
+    ap.add_argument("--n", type=int, default=None, help="override the number of Gaussians")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--reference-order", action="store_true",
+                    help="run the stages exactly as the reference does (separate count pass, atomic K9 into zero-filled buffers)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run device copies / fills of known size (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE) and exit")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus must be 1 (the path has no multi-GPU part)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+
+    import ssr_pkg
+    pkg = ssr_pkg.load()
+    from spirula_studio_amd import host, lib
+
+    if args.copy_calibration:
+        L = lib.load()
+        lib.check(L.ssr_init(0))
+        nbytes = 1 << 30
+        a, b = lib.DeviceArray((nbytes,), np.uint8), lib.DeviceArray((nbytes,), np.uint8)
+        for _ in range(5):
+            lib.check(L.ssr_fill_u32(a.ptr, 1, nbytes // 4, None))          # writes 1 GiB
+            lib.check(L.ssr_memcpy(b.ptr, a.ptr, nbytes, lib.D2D, None, 1))  # reads 1 GiB, writes 1 GiB
+        lib.check(L.ssr_device_synchronize())
+        print(json.dumps({"copy_calibration_bytes": nbytes, "launches": 5}))
+        return
+
+    cfg = args.config
+    t_gen = time.time()
+    sc = pkg.scenes.make_scene(cfg, n=args.n)
+    t_gen = time.time() - t_gen
+    native = not args.reference_order
+    eng = host.Engine(sc, fuse_tile_count=native, overwrite_world_grads=native)
+    L = lib.load()
+
+    eng.time_iterations(max(args.warmup, 1))
+    lib.check(L.ssr_device_synchronize())
+    t0 = time.perf_counter()
+    ms = eng.time_iterations(args.steps)
+    lib.check(L.ssr_device_synchronize())
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+
+    # per-stage device times, outside the timed region (events around every stage)
+    lib.check(host.load().ssrh_set_options(int(native), int(native), int(sc.sh_codec == 3), 1))
+    acc = {}
+    reps = 5
+    for _ in range(reps):
+        eng.forward()
+        eng.backward()
+        for k, v in eng.stage_times().items():
+            acc[k] = acc.get(k, 0.0) + v / reps
+    lib.check(host.load().ssrh_set_options(int(native), int(native), int(sc.sh_codec == 3), 0))
+
+    # problem sizes from the device results
+    aabb = eng.cache("aabb").reshape(-1, 4)
+    V = int((aabb[:, 2] > aabb[:, 0]).sum())
+    K = eng.n_isects
+    P = sc.width * sc.height
+    T = sc.tile_w * sc.tile_h
+    K_b = tile_need(eng.cache("offsets"), eng.cache("last_ids"), K, sc.width, sc.height)
+    K_f = K_b   # lower bound of the forward's need (it also reads the splat that ends a pixel)
+    S = 180 if sc.sh_codec == 0 else (47 if sc.sh_codec == 3 else 45 + 8 * 45 / 256)
+    ab = algorithmic_bytes(sc.n, V, K, K_f, K_b, P, T, S)
+    total_bytes = sum(ab.values())
+    dom = max(acc, key=acc.get)
+    dom_gbs = ab[dom] / (acc[dom] * 1e-3) / 1e9 if acc[dom] > 0 else 0.0
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get(f"config{cfg}", {}).get(dom)
+        except Exception:
+            traffic = None
+
+    out = {
+        "metric": "fwd+bwd raster iters/sec at 1M SH3 1080p; % of HBM roofline",
+        "value": args.steps / wall,
+        "unit": "iters/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"config {cfg}: {sc.name}, N={sc.n}, {sc.width}x{sc.height}, "
+                               f"{'pinhole' if sc.camera_model == 0 else 'equirectangular'}, SH3 "
+                               f"{['fp32', 'ref-q8', 'ref-q16', 'int8*fp16scale'][sc.sh_codec]}, tile 16x16, seed {pkg.scenes.CONFIGS[cfg]['seed']:#x}",
+                   "visible": V, "n_isects": K, "K_b": K_b, "tiles": T, "pixels": P,
+                   "stage_order": "fused-count + overwrite-grads" if native else "reference order",
+                   "device_ms_per_iter_median": float(np.median(ms))},
+        "hbm_roofline_frac_whole_iteration": total_bytes / (float(np.median(ms)) * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "algorithmic_bytes_per_iter": total_bytes,
+        "stage_ms": {k: round(v, 4) for k, v in acc.items()},
+        "stage_algorithmic_GBs": {k: round(ab[k] / (acc[k] * 1e-3) / 1e9, 1) if acc[k] > 0 else None for k in acc},
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": dom_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": dom_gbs / HBM_PEAK_GBS, "traffic": traffic,
+                     "algorithmic_bytes_per_launch": ab[dom], "avg_launch_ms": acc[dom]},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(pkg, cfg)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

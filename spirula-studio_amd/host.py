@@ -1,0 +1,146 @@
+"""ctypes binding of libssr_host.so: the C++ host layer that mirrors the reference's backend
+interface and engine call order (spirula-studio_amd/host/ssr_engine.hpp). Fails loudly when the
+library is not built."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import numpy as np
+
+from . import lib as _lib
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+SO_PATH = os.path.join(_HERE, "host", "libssr_host.so")
+
+vp = C.c_void_p
+SYMBOLS = {
+    "ssrh_last_error": (C.c_char_p, []),
+    "ssrh_init": (C.c_int, [C.c_int]),
+    "ssrh_reset": (C.c_int, []),
+    "ssrh_set_options": (C.c_int, [C.c_int] * 4),
+    "ssrh_set_data_3dgs": (C.c_int, [C.c_int64, vp, vp, vp, vp, vp, vp, C.c_int]),
+    "ssrh_set_sh_value_quant": (C.c_int, [C.c_int, vp, C.c_int64, C.c_int, vp, C.c_int64, C.c_int, C.c_int64]),
+    "ssrh_set_camera_params": (C.c_int, [C.c_int, C.c_int, C.c_char_p, C.c_char_p, vp, vp, C.c_int]),
+    "ssrh_forward_3dgs": (C.c_int, [C.c_char_p, C.c_int, C.c_int, C.c_int, C.c_int]),
+    "ssrh_backward_from_render_grad": (C.c_int, [vp, vp, vp]),
+    "ssrh_copy_render_to_host": (C.c_int, [vp, vp, vp]),
+    "ssrh_copy_grads_to_host": (C.c_int, [vp] * 6),
+    "ssrh_cache_pointer": (C.c_int, [C.c_int, C.POINTER(vp), C.POINTER(C.c_int64)]),
+    "ssrh_last_n_isects": (C.c_int64, []),
+    "ssrh_last_stage_times": (C.c_int, [vp]),
+    "ssrh_time_iterations": (C.c_int, [C.c_int, vp, vp, vp, C.c_int, vp]),
+    "ssrh_pool_bytes": (C.c_size_t, []),
+}
+
+_h = None
+
+
+def load():
+    global _h
+    if _h is None:
+        _lib.load()   # libssr_hip.so first: the host library links against it
+        if not os.path.exists(SO_PATH):
+            raise _lib.SsrError(f"{SO_PATH} is not built; run `make -C {os.path.dirname(SO_PATH)}`")
+        h = C.CDLL(SO_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(h, name)
+            fn.restype, fn.argtypes = res, args
+        _h = h
+    return _h
+
+
+def check(rc):
+    if rc != 0:
+        raise _lib.SsrError(load().ssrh_last_error().decode() or f"host error {rc}")
+
+
+_MODEL = {0: b"PINHOLE", 3: b"EQUIRECTANGULAR"}
+
+CACHE = dict(aabb=(0, np.float32), sort_depth=(1, np.float32), xy=(2, np.float32), depth=(3, np.float32),
+             conic=(4, np.float32), opac=(5, np.float32), rgb=(6, np.float32), sorted_ids=(7, np.int64),
+             sorted_flat=(8, np.int32), offsets=(9, np.int32), last_ids=(10, np.int32), radii=(11, np.float32),
+             v_xy=(12, np.float32), v_depth=(13, np.float32), v_conic=(14, np.float32), v_opac=(15, np.float32),
+             v_rgb=(16, np.float32))
+
+
+class Engine:
+    """Drives the engine harness for one scene: upload once, then forward / backward."""
+
+    def __init__(self, scene, device=0, fuse_tile_count=True, overwrite_world_grads=True,
+                 stage_profiling=False, sh_degree=3):
+        self.h = load()
+        self.sc = scene
+        self.sh_degree = sh_degree
+        check(self.h.ssrh_init(device))
+        check(self.h.ssrh_reset())
+        check(self.h.ssrh_set_options(int(fuse_tile_count), int(overwrite_world_grads),
+                                      int(scene.sh_codec == 3), int(stage_profiling)))
+        f32 = lambda a: np.ascontiguousarray(a, np.float32)
+        self._keep = [f32(scene.means), f32(scene.quats), f32(scene.log_scales), f32(scene.opacity_logits),
+                      f32(scene.features_dc), f32(scene.features_sh)]
+        p = [a.ctypes.data for a in self._keep]
+        check(self.h.ssrh_set_data_3dgs(scene.n, *p, 15))
+        if scene.sh_codec != 0:
+            packed = np.ascontiguousarray(scene.sh_packed)
+            if scene.sh_codec == 3:
+                bounds = np.ascontiguousarray(scene.sh_scale_f16.view(np.uint16))
+                bits = 8
+            else:
+                bounds = np.ascontiguousarray(scene.sh_bounds, np.float32).reshape(-1, 2)
+                bits = 8 if scene.sh_codec == 1 else 16
+            be = bounds.itemsize if scene.sh_codec == 3 else 8
+            check(self.h.ssrh_set_sh_value_quant(bits, packed.ctypes.data, packed.size, packed.itemsize,
+                                                 bounds.ctypes.data, bounds.shape[0], be, scene.sh_bounds_stride))
+        vm, it = f32(scene.viewmat), f32(scene.intrins)
+        check(self.h.ssrh_set_camera_params(scene.width, scene.height, _MODEL[scene.camera_model], b"NONE",
+                                            vm.ctypes.data, it.ctypes.data, 1))
+        # cotangents resident on the device
+        self.d_vrgb = _lib.DeviceArray.from_host(f32(scene.v_rgb))
+        self.d_vdepth = _lib.DeviceArray.from_host(f32(scene.v_depth))
+        self.d_vT = _lib.DeviceArray.from_host(f32(scene.v_T))
+
+    def forward(self):
+        check(self.h.ssrh_forward_3dgs(b"3dgs", self.sh_degree, 0, 0, 0))
+
+    def backward(self):
+        check(self.h.ssrh_backward_from_render_grad(self.d_vrgb.ptr, self.d_vdepth.ptr, self.d_vT.ptr))
+
+    def time_iterations(self, iters):
+        ms = np.zeros(iters, np.float32)
+        check(self.h.ssrh_time_iterations(self.sh_degree, self.d_vrgb.ptr, self.d_vdepth.ptr, self.d_vT.ptr,
+                                          iters, ms.ctypes.data))
+        return ms
+
+    def stage_times(self):
+        t = np.zeros(9, np.float32)
+        check(self.h.ssrh_last_stage_times(t.ctypes.data))
+        return dict(zip(["K1", "K2", "K3", "K4", "K5", "K6", "K7", "K8", "K9"], [float(v) for v in t]))
+
+    @property
+    def n_isects(self):
+        return int(self.h.ssrh_last_n_isects())
+
+    def render(self):
+        h, w = self.sc.height, self.sc.width
+        rgb, depth, T = np.zeros((h, w, 3), np.float32), np.zeros((h, w), np.float32), np.zeros((h, w), np.float32)
+        check(self.h.ssrh_copy_render_to_host(rgb.ctypes.data, depth.ctypes.data, T.ctypes.data))
+        return rgb, depth, T
+
+    def grads(self):
+        n = self.sc.n
+        g = dict(v_means=np.zeros((n, 3), np.float32), v_quats=np.zeros((n, 4), np.float32),
+                 v_scales=np.zeros((n, 3), np.float32), v_opacities=np.zeros(n, np.float32),
+                 v_dc=np.zeros((n, 3), np.float32), v_sh=np.zeros((n, 15, 3), np.float32))
+        check(self.h.ssrh_copy_grads_to_host(*[g[k].ctypes.data for k in
+                                               ["v_means", "v_quats", "v_scales", "v_opacities", "v_dc", "v_sh"]]))
+        return g
+
+    def cache(self, name):
+        which, dt = CACHE[name]
+        ptr, cnt = vp(), C.c_int64()
+        check(self.h.ssrh_cache_pointer(which, C.byref(ptr), C.byref(cnt)))
+        out = np.zeros(cnt.value, dt)
+        if cnt.value:
+            _lib.check(_lib.load().ssr_memcpy(out.ctypes.data, ptr, out.nbytes, _lib.D2H, None, 0))
+        return out

@@ -1,0 +1,402 @@
+// ssr_backend_api.cpp -- the reference-shaped launch functions and runtime, implemented on the C
+// ABI of libssr_hip.so. This file contains no device code and needs no HIP headers.
+#include "ssr_backend_api.hpp"
+
+#include <cstring>
+
+#include "../../include/ssr_backend.h"
+
+namespace {
+
+[[noreturn]] void throw_last(const char* where) {
+    const char* e = ssr_last_error();
+    throw std::runtime_error(std::string(where) + ": " + ((e && e[0]) ? e : "unknown backend error"));
+}
+inline void ok(int rc, const char* where) { if (rc != 0) throw_last(where); }
+
+thread_local std::string g_sticky;   // backend::last_error(): returned once, then cleared
+
+ssr_ext::Options g_opts;
+bool g_profile = false;
+ssr_ext::StageTimes g_times;
+int64_t g_n_isects = 0;
+bool g_counts_fused = false;         // the last projection already produced tile counts
+
+struct StageTimer {
+    ssr_event_t a = nullptr, b = nullptr;
+    float* out;
+    explicit StageTimer(float* o) : out(o) {
+        if (!g_profile) return;
+        a = ssr_event_create(); b = ssr_event_create();
+        ssr_event_record(a, nullptr);
+    }
+    ~StageTimer() {
+        if (!g_profile) return;
+        ssr_event_record(b, nullptr);
+        float ms = 0;
+        ssr_event_elapsed_ms(a, b, &ms);
+        *out = ms;
+        ssr_event_destroy(a); ssr_event_destroy(b);
+    }
+};
+
+int camera_model_of(const std::string& m) {
+    if (m == "PINHOLE" || m == "pinhole") return SSR_CAM_PINHOLE;
+    if (m == "EQUIRECTANGULAR" || m == "equirectangular" || m == "EQUIRECT") return SSR_CAM_EQUIRECT;
+    throw std::runtime_error("projection: camera model '" + m + "' is not built in this backend "
+                             "(PINHOLE and EQUIRECTANGULAR are)");
+}
+void require_no_distortion(const std::string& d) {
+    if (!(d == "NONE" || d == "none" || d.empty()))
+        throw std::runtime_error("projection: distortion tier '" + d + "' is not built in this backend (NONE is)");
+}
+
+ssr_world world_of(const std::vector<DeviceTensorFloatND>& s) {
+    if (s.size() != 6) throw std::runtime_error("expected 6 world tensors (means, quats, scales, opacities, dc, sh)");
+    ssr_world w;
+    w.means = s[0].data_ptr(); w.quats = s[1].data_ptr(); w.log_scales = s[2].data_ptr();
+    w.opacity_logits = s[3].data_ptr(); w.features_dc = s[4].data_ptr(); w.features_sh = s[5].data_ptr();
+    w.sh_stride = (int32_t)s[5].channels();
+    return w;
+}
+ssr_screen screen_of(const std::vector<DeviceTensorFloatND>& s) {
+    if (s.size() != 5) throw std::runtime_error("expected 5 screen tensors (xy, depth, conic, opac, rgb)");
+    ssr_screen r;
+    r.xy = s[0].data_ptr(); r.depth = s[1].data_ptr(); r.conic = s[2].data_ptr(); r.opac = s[3].data_ptr();
+    r.rgb = s[4].data_ptr();
+    return r;
+}
+ssr_sh_quant sh_of(const std::optional<TorchTensorView>& packed, const std::optional<TorchTensorView>& bounds,
+                   uint32_t num_sh_buffer, int bits, int64_t stride) {
+    ssr_sh_quant q;
+    std::memset(&q, 0, sizeof(q));
+    q.codec = SSR_SH_F32;
+    q.num_sh_buffer = num_sh_buffer;
+    q.bounds_stride = stride;
+    if (bits == 32) return q;
+    if (bits != 8 && bits != 16) throw std::runtime_error("projection: sh_value_bits must be 32, 16 or 8");
+    if (!packed || !bounds) throw std::runtime_error("projection: quantized SH needs packed codes and bounds");
+    q.packed = (const void*)std::get<0>(*packed);
+    if (g_opts.sh_int8_f16scale && bits == 8) {
+        q.codec = SSR_SH_I8_F16SCALE;
+        q.scale_f16 = (const uint16_t*)std::get<0>(*bounds);
+    } else {
+        q.codec = bits == 8 ? SSR_SH_REF_Q8 : SSR_SH_REF_Q16;
+        q.bounds = (const float*)std::get<0>(*bounds);
+    }
+    return q;
+}
+ssr_camera camera_of(const std::string& model, const TorchTensorView& viewmats, const TorchTensorView& intrins,
+                     uint32_t w, uint32_t h) {
+    ssr_camera c;
+    c.camera_model = camera_model_of(model);
+    const auto& shape = std::get<2>(viewmats);
+    c.num_cameras = shape.empty() ? 0u : (uint32_t)shape[0];
+    if (c.num_cameras != 1) throw std::runtime_error("this backend runs one camera per call (got " + std::to_string(c.num_cameras) + ")");
+    c.width = w; c.height = h;
+    c.viewmats = (const float*)std::get<0>(viewmats);
+    c.intrins = (const float*)std::get<0>(intrins);
+    return c;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------
+namespace backend {
+
+struct Event { ssr_event_t ev; };
+
+int device_count() { return ssr_device_count(); }
+bool device_select(int index) {
+    if (ssr_init(index) != 0) { g_sticky = ssr_last_error(); return false; }
+    return true;
+}
+void* device_malloc(size_t bytes) {
+    void* p = ssr_device_malloc(bytes);
+    if (!p && bytes) g_sticky = ssr_last_error();
+    return p;
+}
+void* device_malloc_checked(size_t bytes, const char* what) {
+    void* p = device_malloc(bytes);
+    if (!p && bytes > 0) {
+        char buf[64];
+        std::snprintf(buf, sizeof buf, "%.0f MiB", (double)bytes / (1024.0 * 1024.0));
+        std::string msg = std::string("GPU allocation failed: ") + last_error() + "; could not allocate " + buf;
+        if (what && what[0]) { msg += " for "; msg += what; }
+        msg += ". Try a smaller model (fewer splats / SH) or a lower image resolution.";
+        throw std::runtime_error(msg);
+    }
+    return p;
+}
+void device_free(void* ptr) { if (ssr_device_free(ptr) != 0) g_sticky = ssr_last_error(); }
+void* host_malloc_pinned(size_t bytes) {
+    void* p = ssr_host_malloc_pinned(bytes);
+    if (!p && bytes) g_sticky = ssr_last_error();
+    return p;
+}
+void host_free_pinned(void* ptr) { if (ssr_host_free_pinned(ptr) != 0) g_sticky = ssr_last_error(); }
+const char* last_error() {
+    static thread_local std::string out;
+    out.swap(g_sticky);
+    g_sticky.clear();
+    return out.c_str();
+}
+static int kind_of(MemcpyKind k) {
+    switch (k) {
+        case MemcpyKind::HostToDevice: return SSR_MEMCPY_H2D;
+        case MemcpyKind::DeviceToHost: return SSR_MEMCPY_D2H;
+        case MemcpyKind::DeviceToDevice: return SSR_MEMCPY_D2D;
+        default: return SSR_MEMCPY_AUTO;
+    }
+}
+void memcpy_sync(void* d, const void* s, size_t n, MemcpyKind k) { if (ssr_memcpy(d, s, n, kind_of(k), nullptr, 0)) g_sticky = ssr_last_error(); }
+void memcpy_async(void* d, const void* s, size_t n, MemcpyKind k, Stream st) { if (ssr_memcpy(d, s, n, kind_of(k), st, 1)) g_sticky = ssr_last_error(); }
+void memset_sync(void* d, int v, size_t n) { if (ssr_memset(d, v, n, nullptr, 0)) g_sticky = ssr_last_error(); }
+void memset_async(void* d, int v, size_t n, Stream st) { if (ssr_memset(d, v, n, st, 1)) g_sticky = ssr_last_error(); }
+bool is_device_pointer(const void* p) { return ssr_is_device_pointer(p) != 0; }
+void device_synchronize() { if (ssr_device_synchronize()) g_sticky = ssr_last_error(); }
+void stream_synchronize(Stream st) { if (ssr_stream_synchronize(st)) g_sticky = ssr_last_error(); }
+Event* event_create(bool) { Event* e = new Event{ssr_event_create()}; return e; }
+void event_record(Event* e, Stream st) { if (e && ssr_event_record(e->ev, st)) g_sticky = ssr_last_error(); }
+void event_synchronize(Event* e) { if (e && ssr_event_synchronize(e->ev)) g_sticky = ssr_last_error(); }
+void event_destroy(Event* e) { if (e) { ssr_event_destroy(e->ev); delete e; } }
+float event_elapsed_ms(Event* a, Event* b) {
+    float ms = 0;
+    if (!a || !b || ssr_event_elapsed_ms(a->ev, b->ev, &ms)) g_sticky = ssr_last_error();
+    return ms;
+}
+
+}  // namespace backend
+
+namespace ssr_ext {
+Options& options() { return g_opts; }
+void set_stage_profiling(bool on) { g_profile = on; }
+StageTimes last_stage_times() { return g_times; }
+int64_t last_n_isects() { return g_n_isects; }
+}  // namespace ssr_ext
+
+// ---------------------------------------------------------------------------------------------
+std::tuple<DeviceTensor2D<float4>, DeviceTensor2D<float>, std::vector<DeviceTensorFloatND>>
+projection_3dgs_forward(const int64_t num_splats, const int max_sh_degree,
+                        const std::vector<DeviceTensorFloatND>& in_splats, TorchTensorView viewmats,
+                        TorchTensorView intrins, const uint32_t image_width, const uint32_t image_height,
+                        const std::string camera_model, const std::string distortion, const TorchTensorView,
+                        DeviceVector<float> radii, const std::optional<TorchTensorView> sh_value_packed,
+                        const std::optional<TorchTensorView> sh_value_bounds, const uint32_t num_sh_buffer,
+                        const int sh_value_bits, const int64_t sh_bounds_stride) {
+    require_no_distortion(distortion);
+    ssr_projection_fwd_params p;
+    std::memset(&p, 0, sizeof(p));
+    p.num_splats = num_splats;
+    p.sh_degree = max_sh_degree;
+    p.world = world_of(in_splats);
+    p.sh = sh_of(sh_value_packed, sh_value_bounds, num_sh_buffer, sh_value_bits, sh_bounds_stride);
+    p.camera = camera_of(camera_model, viewmats, intrins, image_width, image_height);
+    const int64_t C = 1, N = num_splats;
+
+    DeviceTensor2D<float4> aabb; aabb.resize(PoolSlot::ProjAabb, C, N);
+    DeviceTensor2D<float> depths; depths.resize(PoolSlot::ProjDepths, C, N);
+    float* xy = DevicePool::global().acquire<float>(PoolSlot::ProjScreenXy, (size_t)(C * N * 2));
+    float* dp = DevicePool::global().acquire<float>(PoolSlot::ProjScreenDepth, (size_t)(C * N));
+    float* cn = DevicePool::global().acquire<float>(PoolSlot::ProjScreenConic, (size_t)(C * N * 3));
+    float* op = DevicePool::global().acquire<float>(PoolSlot::ProjScreenOpac, (size_t)(C * N));
+    float* rg = DevicePool::global().acquire<float>(PoolSlot::ProjScreenRgb, (size_t)(C * N * 3));
+    p.aabb = (float*)aabb.data_ptr(); p.sort_depth = depths.data_ptr(); p.radii = radii.data_ptr();
+    p.screen.xy = xy; p.screen.depth = dp; p.screen.conic = cn; p.screen.opac = op; p.screen.rgb = rg;
+    g_counts_fused = false;
+    if (g_opts.fuse_tile_count) {
+        p.tiles_per_splat = DevicePool::global().acquire<int64_t>(PoolSlot::IsectTilesPerSplat, (size_t)(C * N));
+        g_counts_fused = true;
+    }
+    {
+        StageTimer t(&g_times.k1);
+        ok(ssr_projection_fwd(&p, nullptr), "projection_3dgs_forward");
+    }
+    std::vector<DeviceTensorFloatND> screen = {
+        DeviceTensorFloatND(xy, {C * N, 2}), DeviceTensorFloatND(dp, {C * N, 1}), DeviceTensorFloatND(cn, {C * N, 3}),
+        DeviceTensorFloatND(op, {C * N, 1}), DeviceTensorFloatND(rg, {C * N, 3})};
+    return std::make_tuple(aabb, depths, screen);
+}
+
+int64_t intersect_tile_count(int width, int height) {
+    return (int64_t)((width + 15) / 16) * (int64_t)((height + 15) / 16);
+}
+
+std::tuple<DeviceVector<int64_t>, DeviceVector<int32_t>, DeviceTensor3D<int32_t>>
+do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, DeviceTensorFloatND* proj_xy,
+                          DeviceTensorFloatND* proj_conic, DeviceTensorFloatND* proj_opac, const uint32_t I,
+                          TorchTensorView, const uint32_t image_width, const uint32_t image_height,
+                          DeviceVector<int32_t>* image_ids, const int32_t* tile_active) {
+    if (image_ids) throw std::runtime_error("do_intersect_tile_generic: packed mode is not built in this backend");
+    if (tile_active) throw std::runtime_error("do_intersect_tile_generic: the tile-skip mask is not built in this backend");
+    if (!proj_xy || !proj_conic || !proj_opac)
+        throw std::runtime_error("do_intersect_tile_generic: AABB mode is not built in this backend (ellipse mode is)");
+    if (I != 1) throw std::runtime_error("do_intersect_tile_generic: this backend runs one image per call");
+    const int64_t total = depths.numel();
+    const uint32_t tile_w = (image_width + 15) / 16, tile_h = (image_height + 15) / 16;
+    const uint32_t n_tiles = tile_w * tile_h * I;
+
+    DeviceVector<int64_t> tiles_per_splat; tiles_per_splat.resize(PoolSlot::IsectTilesPerSplat, total);
+    if (!g_counts_fused) {
+        StageTimer t(&g_times.k2);
+        ok(ssr_tile_count(total, aabb.data_ptr(), proj_xy->data_ptr(), proj_conic->data_ptr(), proj_opac->data_ptr(),
+                          image_width, image_height, tiles_per_splat.data_ptr(), nullptr), "do_intersect_tile_generic/count");
+    } else {
+        g_times.k2 = 0;
+    }
+    g_counts_fused = false;
+    DeviceVector<int64_t> cum; cum.resize(PoolSlot::IsectCumTiles, total);
+    int64_t n_isects = 0;
+    {
+        StageTimer t(&g_times.k3);
+        const size_t sb = ssr_scan_scratch_bytes(total);
+        void* scratch = DevicePool::global().acquire<uint8_t>(PoolSlot::IsectScanScratch, sb);
+        ok(ssr_inclusive_sum_i64(tiles_per_splat.data_ptr(), cum.data_ptr(), total, scratch, sb, nullptr),
+           "do_intersect_tile_generic/scan");
+        if (total > 0) ok(ssr_read_i64(cum.data_ptr() + (total - 1), &n_isects, nullptr), "do_intersect_tile_generic/readback");
+    }
+    g_n_isects = n_isects;
+    DeviceTensor3D<int32_t> offsets; offsets.resize(PoolSlot::IsectOffsets, I, tile_h, tile_w);
+    if (n_isects == 0) {
+        offsets.zero();
+        return std::make_tuple(DeviceVector<int64_t>{}, DeviceVector<int32_t>{}, offsets);
+    }
+    if (n_isects >= ((int64_t)1 << 31)) throw std::runtime_error("do_intersect_tile_generic: more than 2^31-1 intersections");
+    DeviceVector<int64_t> ids_a, ids_b; ids_a.resize(PoolSlot::IsectIdsA, n_isects); ids_b.resize(PoolSlot::IsectIdsB, n_isects);
+    DeviceVector<int32_t> flat_a, flat_b; flat_a.resize(PoolSlot::IsectFlatA, n_isects); flat_b.resize(PoolSlot::IsectFlatB, n_isects);
+    {
+        StageTimer t(&g_times.k4);
+        ok(ssr_tile_write(total, aabb.data_ptr(), depths.data_ptr(), proj_xy->data_ptr(), proj_conic->data_ptr(),
+                          proj_opac->data_ptr(), cum.data_ptr(), image_width, image_height, ids_a.data_ptr(),
+                          flat_a.data_ptr(), nullptr), "do_intersect_tile_generic/write");
+    }
+    int selector = 0;
+    {
+        StageTimer t(&g_times.k5);
+        const size_t sb = ssr_sort_scratch_bytes(n_isects);
+        void* scratch = DevicePool::global().acquire<uint8_t>(PoolSlot::IsectSortScratch, sb);
+        ok(ssr_sort_pairs_u64_i32(ids_a.data_ptr(), ids_b.data_ptr(), flat_a.data_ptr(), flat_b.data_ptr(), n_isects, 0,
+                                  ssr_sort_end_bit(n_tiles), &selector, scratch, sb, nullptr), "do_intersect_tile_generic/sort");
+    }
+    DeviceVector<int64_t> ids_out = selector ? ids_b : ids_a;
+    DeviceVector<int32_t> flat_out = selector ? flat_b : flat_a;
+    {
+        StageTimer t(&g_times.k6);
+        ok(ssr_tile_offsets(n_isects, ids_out.data_ptr(), n_tiles, offsets.data_ptr(), nullptr), "do_intersect_tile_generic/offsets");
+    }
+    return std::make_tuple(ids_out, flat_out, offsets);
+}
+
+std::tuple<RenderOutput::TensorTuple, DeviceTensor3D<float>, DeviceTensor3D<int32_t>, RenderOutput::TensorTuple,
+           DeviceTensor3D<float>>
+rasterize_to_pixels_3dgs_fwd(int64_t num_splats, std::vector<DeviceTensorFloatND>, std::vector<DeviceTensorFloatND> splats_s,
+                             DeviceVector<int32_t> gaussian_ids, const uint32_t image_width, const uint32_t image_height,
+                             const DeviceTensor3D<int32_t> tile_offsets, const DeviceVector<int32_t> flatten_ids,
+                             DistortionType dist_type, bool output_median) {
+    if (gaussian_ids.data_ptr()) throw std::runtime_error("rasterize_to_pixels_3dgs_fwd: packed mode is not built in this backend");
+    if (dist_type != DistortionType::None) throw std::runtime_error("rasterize_to_pixels_3dgs_fwd: depth distortion is not built in this backend");
+    if (output_median) throw std::runtime_error("rasterize_to_pixels_3dgs_fwd: median depth is not built in this backend");
+    const int64_t I = tile_offsets.size<0>();
+    if (I != 1) throw std::runtime_error("rasterize_to_pixels_3dgs_fwd: this backend runs one image per call");
+    RenderOutput::TensorTuple renders;
+    std::get<0>(renders).resize(PoolSlot::RendersRgb, I, image_height, image_width);
+    std::get<1>(renders).resize(PoolSlot::RendersDepth, I, image_height, image_width);
+    DeviceTensor3D<float> Ts; Ts.resize(PoolSlot::RenderTs, I, image_height, image_width);
+    DeviceTensor3D<int32_t> last; last.resize(PoolSlot::RenderLastIds, I, image_height, image_width);
+    ssr_raster_fwd_params p;
+    std::memset(&p, 0, sizeof(p));
+    p.num_splats = num_splats;
+    if (flatten_ids.size() > 0) p.screen = screen_of(splats_s);
+    p.width = image_width; p.height = image_height;
+    p.tile_offsets = tile_offsets.data_ptr(); p.flatten_ids = flatten_ids.data_ptr(); p.n_isects = flatten_ids.size();
+    p.render_rgb = (float*)std::get<0>(renders).data_ptr(); p.render_depth = std::get<1>(renders).data_ptr();
+    p.render_T = Ts.data_ptr(); p.last_ids = last.data_ptr();
+    {
+        StageTimer t(&g_times.k7);
+        ok(ssr_raster_fwd(&p, nullptr), "rasterize_to_pixels_3dgs_fwd");
+    }
+    return std::make_tuple(renders, Ts, last, RenderOutput::TensorTuple{}, DeviceTensor3D<float>{});
+}
+
+std::tuple<std::vector<DeviceTensorFloatND>, std::vector<DeviceTensorFloatND>, DeviceVector<float>>
+rasterize_to_pixels_3dgs_bwd(int64_t num_splats, std::vector<DeviceTensorFloatND> splats_w,
+                             std::vector<DeviceTensorFloatND> splats_s, DeviceVector<int32_t> gaussian_ids,
+                             const uint32_t image_width, const uint32_t image_height,
+                             const DeviceTensor3D<int32_t> tile_offsets, const DeviceVector<int32_t> flatten_ids,
+                             const DeviceTensor3D<float> render_Ts, const DeviceTensor3D<int32_t> last_ids,
+                             RenderOutput::TensorTuple render_outputs_tuple, std::optional<RenderOutput::TensorTuple>,
+                             DistortionType dist_type, DeviceTensor3D<float> accum_weight_map, DensifyAccumMode accum_mode,
+                             RenderOutput::TensorTuple v_render_outputs, const DeviceTensor3D<float> v_render_Ts,
+                             const DeviceTensor3D<float> v_median, std::optional<RenderOutput::TensorTuple>,
+                             std::optional<std::vector<DeviceTensorFloatND>> v_splats_w,
+                             std::optional<std::vector<DeviceTensorFloatND>> v_splats_s) {
+    if (gaussian_ids.data_ptr()) throw std::runtime_error("rasterize_to_pixels_3dgs_bwd: packed mode is not built in this backend");
+    if (dist_type != DistortionType::None) throw std::runtime_error("rasterize_to_pixels_3dgs_bwd: depth distortion is not built in this backend");
+    if (accum_mode != DensifyAccumMode::None || accum_weight_map.data_ptr())
+        throw std::runtime_error("rasterize_to_pixels_3dgs_bwd: accumulation weights are not built in this backend");
+    if (v_median.data_ptr()) throw std::runtime_error("rasterize_to_pixels_3dgs_bwd: median depth is not built in this backend");
+    std::vector<DeviceTensorFloatND> vs;
+    if (v_splats_s) {
+        vs = *v_splats_s;   // caller-provided accumulators are added into as they are
+    } else {
+        // the launcher owns and zero-fills v_screen (src/kernels/raster/RasterizationBwd.cu:143-146)
+        const int64_t n = splats_s.empty() ? 0 : splats_s[0].rows();
+        const PoolSlot slots[5] = {PoolSlot::RasterBwdVScreenXy, PoolSlot::RasterBwdVScreenDepth, PoolSlot::RasterBwdVScreenConic,
+                                   PoolSlot::RasterBwdVScreenOpac, PoolSlot::RasterBwdVScreenRgb};
+        const int ch[5] = {2, 1, 3, 1, 3};
+        for (int i = 0; i < 5; i++) {
+            float* p = DevicePool::global().acquire<float>(slots[i], (size_t)(n * ch[i]));
+            backend::memset_async(p, 0, (size_t)(n * ch[i]) * sizeof(float));
+            vs.emplace_back(p, std::vector<int64_t>{n, ch[i]});
+        }
+    }
+    ssr_raster_bwd_params p;
+    std::memset(&p, 0, sizeof(p));
+    p.num_splats = num_splats;
+    p.screen = screen_of(splats_s);
+    p.width = image_width; p.height = image_height;
+    p.tile_offsets = tile_offsets.data_ptr(); p.flatten_ids = flatten_ids.data_ptr(); p.n_isects = flatten_ids.size();
+    p.render_T = render_Ts.data_ptr(); p.last_ids = last_ids.data_ptr(); p.render_depth = std::get<1>(render_outputs_tuple).data_ptr();
+    p.v_render_rgb = (const float*)std::get<0>(v_render_outputs).data_ptr();
+    p.v_render_depth = std::get<1>(v_render_outputs).data_ptr();
+    p.v_render_T = v_render_Ts.data_ptr();
+    p.v_screen = screen_of(vs);
+    {
+        StageTimer t(&g_times.k8);
+        ok(ssr_raster_bwd(&p, nullptr), "rasterize_to_pixels_3dgs_bwd");
+    }
+    std::vector<DeviceTensorFloatND> vw = v_splats_w ? *v_splats_w : std::vector<DeviceTensorFloatND>{};
+    (void)splats_w;
+    return std::make_tuple(vw, vs, DeviceVector<float>{});
+}
+
+void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
+                              const std::vector<DeviceTensorFloatND>& splats_world, TorchTensorView viewmats,
+                              TorchTensorView intrins, const uint32_t image_width, const uint32_t image_height,
+                              const std::string camera_model, const std::string distortion, const TorchTensorView,
+                              const DeviceVector<int32_t> camera_ids, const DeviceVector<int32_t> gaussian_ids,
+                              const DeviceTensor2D<float4> aabb, const std::vector<DeviceTensorFloatND>& v_splats_screen,
+                              const std::vector<DeviceTensorFloatND>& v_splats_world, DeviceTensor2D<float>* v_viewmats,
+                              const std::optional<TorchTensorView> sh_value_packed,
+                              const std::optional<TorchTensorView> sh_value_bounds, const uint32_t num_sh_buffer,
+                              const int sh_value_bits, const int64_t sh_bounds_stride) {
+    require_no_distortion(distortion);
+    if (camera_ids.data_ptr() || gaussian_ids.data_ptr())
+        throw std::runtime_error("projection_3dgs_backward: packed mode is not built in this backend");
+    if (v_viewmats) throw std::runtime_error("projection_3dgs_backward: camera pose gradients are not built in this backend");
+    if (num_splats == 0) return;   // src/kernels/projection/ProjectionBwd.cu:86-87
+    if (!aabb.data_ptr()) throw std::runtime_error("projection_3dgs_backward: aabb is null");   // :89-97
+    ssr_projection_bwd_params p;
+    std::memset(&p, 0, sizeof(p));
+    p.num_splats = num_splats;
+    p.sh_degree = max_sh_degree;
+    p.world = world_of(splats_world);
+    p.sh = sh_of(sh_value_packed, sh_value_bounds, num_sh_buffer, sh_value_bits, sh_bounds_stride);
+    p.camera = camera_of(camera_model, viewmats, intrins, image_width, image_height);
+    p.aabb = (const float*)aabb.data_ptr();
+    p.v_screen = screen_of(v_splats_screen);
+    p.v_world = world_of(v_splats_world);
+    p.accumulate = g_opts.overwrite_world_grads ? 0 : 1;
+    StageTimer t(&g_times.k9);
+    ok(ssr_projection_bwd(&p, nullptr), "projection_3dgs_backward");
+}

@@ -1,0 +1,110 @@
+// ssr_backend_api.hpp -- the reference's launch functions for the projection / tile / raster path,
+// re-declared with the reference's own names, argument order and meaning, implemented on the C ABI
+// of libssr_hip.so. A maintainer of the reference adds this backend by compiling these
+// definitions in place of the CUDA (src/kernels/**) or Vulkan (src/backend/vulkan/kernels/**) ones.
+//
+//   projection_3dgs_forward        src/kernels/projection/ProjectionFwd.cuh:18-36
+//   do_intersect_tile_generic      src/kernels/tile/IntersectTile.cuh:25-41
+//   rasterize_to_pixels_3dgs_fwd   src/kernels/raster/RasterizationFwd.cuh:18-38
+//   rasterize_to_pixels_3dgs_bwd   src/kernels/raster/RasterizationBwd.cuh:18-48
+//   projection_3dgs_backward       src/kernels/projection/ProjectionBwd.cuh:18-46
+//
+// Outputs are slots of the process-global grow-only DevicePool, returned as non-owning views that
+// stay valid until the same function runs again; the caller never frees. Unsupported variants
+// throw std::runtime_error, as the reference does (src/kernels/projection/ProjectionFwd.cu:84-89).
+// Not thread-safe across concurrent calls (one in-order stream, shared scratch), like the
+// reference's sort scratch (src/backend/vulkan/SortScanVulkan.cpp:4-6).
+#pragma once
+#include "ssr_host_types.hpp"
+
+std::tuple<DeviceTensor2D<float4>, DeviceTensor2D<float>, std::vector<DeviceTensorFloatND>>
+projection_3dgs_forward(
+    const int64_t num_splats, const int max_sh_degree,
+    const std::vector<DeviceTensorFloatND>& in_splats,
+    TorchTensorView viewmats, TorchTensorView intrins,
+    const uint32_t image_width, const uint32_t image_height,
+    const std::string camera_model, const std::string distortion,
+    const TorchTensorView dist_coeffs,
+    DeviceVector<float> radii,
+    const std::optional<TorchTensorView> sh_value_packed,
+    const std::optional<TorchTensorView> sh_value_bounds,
+    const uint32_t num_sh_buffer,
+    const int sh_value_bits,
+    const int64_t sh_bounds_stride);
+
+int64_t intersect_tile_count(int width, int height);
+
+std::tuple<DeviceVector<int64_t>, DeviceVector<int32_t>, DeviceTensor3D<int32_t>>
+do_intersect_tile_generic(
+    DeviceTensorFloatND aabb, DeviceTensorFloatND depths,
+    DeviceTensorFloatND* proj_xy, DeviceTensorFloatND* proj_conic, DeviceTensorFloatND* proj_opac,
+    const uint32_t I, TorchTensorView intrins,
+    const uint32_t image_width, const uint32_t image_height,
+    DeviceVector<int32_t>* image_ids, const int32_t* tile_active);
+
+std::tuple<RenderOutput::TensorTuple, DeviceTensor3D<float>, DeviceTensor3D<int32_t>,
+           RenderOutput::TensorTuple, DeviceTensor3D<float>>
+rasterize_to_pixels_3dgs_fwd(
+    int64_t num_splats,
+    std::vector<DeviceTensorFloatND> splats_w, std::vector<DeviceTensorFloatND> splats_s,
+    DeviceVector<int32_t> gaussian_ids,
+    const uint32_t image_width, const uint32_t image_height,
+    const DeviceTensor3D<int32_t> tile_offsets, const DeviceVector<int32_t> flatten_ids,
+    DistortionType dist_type, bool output_median);
+
+std::tuple<std::vector<DeviceTensorFloatND>, std::vector<DeviceTensorFloatND>, DeviceVector<float>>
+rasterize_to_pixels_3dgs_bwd(
+    int64_t num_splats,
+    std::vector<DeviceTensorFloatND> splats_w, std::vector<DeviceTensorFloatND> splats_s,
+    DeviceVector<int32_t> gaussian_ids,
+    const uint32_t image_width, const uint32_t image_height,
+    const DeviceTensor3D<int32_t> tile_offsets, const DeviceVector<int32_t> flatten_ids,
+    const DeviceTensor3D<float> render_Ts, const DeviceTensor3D<int32_t> last_ids,
+    RenderOutput::TensorTuple render_outputs_tuple,
+    std::optional<RenderOutput::TensorTuple> distortion_fwd_outputs,
+    DistortionType dist_type,
+    DeviceTensor3D<float> accum_weight_map, DensifyAccumMode accum_mode,
+    RenderOutput::TensorTuple v_render_outputs,
+    const DeviceTensor3D<float> v_render_Ts, const DeviceTensor3D<float> v_median,
+    std::optional<RenderOutput::TensorTuple> v_distortion_outputs,
+    std::optional<std::vector<DeviceTensorFloatND>> v_splats_w,
+    std::optional<std::vector<DeviceTensorFloatND>> v_splats_s);
+
+void projection_3dgs_backward(
+    const int64_t num_splats, const int max_sh_degree,
+    const std::vector<DeviceTensorFloatND>& splats_world,
+    TorchTensorView viewmats, TorchTensorView intrins,
+    const uint32_t image_width, const uint32_t image_height,
+    const std::string camera_model, const std::string distortion,
+    const TorchTensorView dist_coeffs,
+    const DeviceVector<int32_t> camera_ids, const DeviceVector<int32_t> gaussian_ids,
+    const DeviceTensor2D<float4> aabb,
+    const std::vector<DeviceTensorFloatND>& v_splats_screen,
+    const std::vector<DeviceTensorFloatND>& v_splats_world,
+    DeviceTensor2D<float>* v_viewmats,
+    const std::optional<TorchTensorView> sh_value_packed,
+    const std::optional<TorchTensorView> sh_value_bounds,
+    const uint32_t num_sh_buffer, const int sh_value_bits, const int64_t sh_bounds_stride);
+
+// ---- extensions of this backend (no counterpart in the reference) ----
+namespace ssr_ext {
+// Work the reference does that this backend can skip with identical results:
+struct Options {
+    // K1 also produces the per-splat tile count, so do_intersect_tile_generic skips its count
+    // pass when the projection that produced `aabb` ran with this set.
+    bool fuse_tile_count = false;
+    // K9 overwrites every gradient row (zeros for culled splats) instead of atomically adding into
+    // zero-filled buffers; valid for one camera per call, which is all this backend accepts.
+    bool overwrite_world_grads = false;
+    // int8 codes x per-splat fp16 scale as SH storage (the benchmark's format): sh_value_bits == 8
+    // with sh_value_bounds holding the fp16 scales when this is set.
+    bool sh_int8_f16scale = false;
+};
+Options& options();
+// Per-stage device time of the most recent calls (ms), measured with events on the launch stream
+// when profiling is on.
+struct StageTimes { float k1 = 0, k2 = 0, k3 = 0, k4 = 0, k5 = 0, k6 = 0, k7 = 0, k8 = 0, k9 = 0; };
+void set_stage_profiling(bool on);
+StageTimes last_stage_times();
+int64_t last_n_isects();
+}  // namespace ssr_ext

@@ -1,0 +1,335 @@
+// ssr_engine.cpp -- engine harness (see ssr_engine.hpp) and its C entry points for Python.
+#include "ssr_engine.hpp"
+
+#include <cstring>
+
+#include "../../include/ssr_backend.h"
+
+static EngineState g_engine;
+EngineState& engine() { return g_engine; }
+void engine_reset() { g_engine = EngineState{}; }
+
+namespace {
+
+// host memory is copied into the slot, a device address is aliased (EngineCommon.h:90-105)
+template <typename T>
+DeviceVector<T> hv_to_dv(PoolSlot slot, const TorchTensorView& tv) {
+    DeviceVector<T> view(tv);   // validates element size
+    void* src = (void*)std::get<0>(tv);
+    if (view.size() == 0 || backend::is_device_pointer(src)) return view;
+    DeviceVector<T> out; out.resize(slot, view.size());
+    backend::memcpy_sync(out.data_ptr(), src, (size_t)view.size() * sizeof(T), backend::MemcpyKind::HostToDevice);
+    return out;
+}
+
+TorchTensorView device_copy_tv(PoolSlot slot, const TorchTensorView& tv) {
+    void* src = (void*)std::get<0>(tv);
+    int64_t n = 1;
+    for (auto s : std::get<2>(tv)) n *= s;
+    const size_t bytes = (size_t)n * std::get<1>(tv);
+    if (bytes == 0 || backend::is_device_pointer(src)) return tv;
+    uint8_t* p = DevicePool::global().acquire<uint8_t>(slot, bytes);
+    backend::memcpy_sync(p, src, bytes, backend::MemcpyKind::HostToDevice);
+    return TorchTensorView((uint64_t)p, std::get<1>(tv), std::get<2>(tv));
+}
+
+void alloc_grad_buffers() {
+    // _alloc_grad_buffers: six fp32 world-gradient buffers, zeroed (src/engine/EngineLoss.cpp:20-127)
+    auto& g = engine().grad;
+    const int64_t n = engine().max_num_splats;
+    g.means.resize(PoolSlot::GradMeans, n); g.quats.resize(PoolSlot::GradQuats, n);
+    g.scales.resize(PoolSlot::GradScales, n); g.opacities.resize(PoolSlot::GradOpacities, n);
+    g.features_dc.resize(PoolSlot::GradFeaturesDc, n); g.features_sh.resize(PoolSlot::GradFeaturesSh, n, engine().num_sh);
+    if (!engine().optim.skip_grad_zero && !ssr_ext::options().overwrite_world_grads) {
+        g.means.zero(); g.quats.zero(); g.scales.zero(); g.opacities.zero(); g.features_dc.zero(); g.features_sh.zero();
+    }
+}
+
+}  // namespace
+
+void set_data_3dgs(int64_t num_splats, TorchTensorView means, TorchTensorView quats, TorchTensorView scales,
+                   TorchTensorView opacities, TorchTensorView features_dc, TorchTensorView features_sh) {
+    const int64_t max_num_splats = std::get<2>(means)[0];
+    if (std::get<2>(quats)[0] != max_num_splats || std::get<2>(scales)[0] != max_num_splats ||
+        std::get<2>(opacities)[0] != max_num_splats || std::get<2>(features_dc)[0] != max_num_splats ||
+        std::get<2>(features_sh)[0] != max_num_splats)
+        throw std::runtime_error("setData3DGS: max_num_splats mismatch across splat tensors");
+    if (max_num_splats < num_splats) throw std::runtime_error("setData3DGS: tensor size smaller than num_splats");
+    engine().cur_num_splats = num_splats;
+    engine().max_num_splats = max_num_splats;
+    auto sh_shape = std::get<2>(features_sh);
+    engine().num_sh = sh_shape.size() >= 2 ? (int)sh_shape[1] : 0;
+    if (engine().world.initialized) return;   // set once; later calls are no-ops (EngineSetup.cpp:36-37)
+    auto& w = engine().world;
+    w.means = hv_to_dv<float3>(PoolSlot::WorldMeans, means);
+    w.quats = hv_to_dv<float4>(PoolSlot::WorldQuats, quats);
+    w.scales = hv_to_dv<float3>(PoolSlot::WorldScales, scales);
+    w.opacities = hv_to_dv<float>(PoolSlot::WorldOpacities, opacities);
+    w.features_dc = hv_to_dv<float3>(PoolSlot::WorldFeaturesDc, features_dc);
+    {
+        TorchTensorView d = device_copy_tv(PoolSlot::WorldFeaturesSh, features_sh);
+        w.features_sh = DeviceTensor2D<float3>((float3*)std::get<0>(d), max_num_splats, engine().num_sh);
+    }
+    w.initialized = true;
+}
+
+void set_sh_value_quant(int sh_value_bits, TorchTensorView packed, TorchTensorView bounds, int64_t bounds_stride) {
+    auto& w = engine().world;
+    w.sh_value_bits = sh_value_bits;
+    if (sh_value_bits == 32) { w.sh_packed.reset(); w.sh_bounds.reset(); return; }
+    // codes and bounds given from the host are copied into pool slots; device addresses are aliased
+    packed = device_copy_tv(PoolSlot::WorldShQuantPacked, packed);
+    bounds = device_copy_tv(PoolSlot::WorldShQuantBounds, bounds);
+    w.sh_packed = packed; w.sh_bounds = bounds; w.sh_bounds_stride = bounds_stride;
+}
+
+void set_camera_params(int width, int height, std::string camera_model, std::string distortion,
+                       TorchTensorView viewmats, TorchTensorView intrins, TorchTensorView dist_coeffs) {
+    auto& c = engine().camera;
+    c.width = width; c.height = height;
+    c.model_str = camera_model; c.distortion_str = distortion;
+    c.num = (int)std::get<2>(viewmats)[0];
+    if (std::get<2>(intrins)[0] != c.num || std::get<2>(dist_coeffs)[0] != c.num)
+        throw std::runtime_error("setCameraParams: num_cameras mismatch");
+    c.viewmats = device_copy_tv(PoolSlot::CamViewmats, viewmats);
+    c.intrins = device_copy_tv(PoolSlot::CamIntrins, intrins);
+    c.dist_coeffs = device_copy_tv(PoolSlot::CamDistCoeffs, dist_coeffs);
+}
+
+void forward_3dgs(std::string primitive, int sh_degree, bool packed, bool output_median, int dist_type_int) {
+    if (primitive != "3dgs") throw std::runtime_error("forward_3dgs: primitive '" + primitive + "' is not built in this backend");
+    if (packed) throw std::runtime_error("forward_3dgs: packed projection is not built in this backend");
+    auto& E = engine();
+    if (!E.world.initialized) throw std::runtime_error("forward_3dgs: set_data_3dgs must be called first");
+    E.primitive = primitive; E.sh_degree = sh_degree; E.packed = packed;
+    const int64_t N = E.cur_num_splats;
+    std::vector<DeviceTensorFloatND> in_splats = {
+        DeviceTensorFloatND(E.world.means), DeviceTensorFloatND(E.world.quats), DeviceTensorFloatND(E.world.scales),
+        DeviceTensorFloatND((float*)E.world.opacities.data_ptr(), {E.world.opacities.size(), 1}),
+        DeviceTensorFloatND(E.world.features_dc), DeviceTensorFloatND(E.world.features_sh)};
+    E.fwd.splats_w = in_splats;
+    // radii: zeroed before projection, which accumulates with atomic max (EngineForward.cpp:66-69)
+    E.optim.radii.resize(PoolSlot::EngRadii, E.max_num_splats);
+    if (!E.optim.skip_grad_zero) E.optim.radii.zero();
+
+    auto [aabb, depths, screen] = projection_3dgs_forward(
+        N, sh_degree, in_splats, E.camera.viewmats, E.camera.intrins, (uint32_t)E.camera.width,
+        (uint32_t)E.camera.height, E.camera.model_str, E.camera.distortion_str, E.camera.dist_coeffs, E.optim.radii,
+        E.world.sh_packed, E.world.sh_bounds, (uint32_t)E.num_sh, E.world.sh_value_bits, E.world.sh_bounds_stride);
+    E.fwd.aabb = aabb; E.fwd.depths = depths; E.fwd.splats_s = screen;
+
+    DeviceTensorFloatND aabb_nd((float*)aabb.data_ptr(), {aabb.numel(), 4});
+    DeviceTensorFloatND depths_nd(depths.data_ptr(), {depths.numel()});
+    auto [ids, flat, offsets] = do_intersect_tile_generic(
+        aabb_nd, depths_nd, &screen[0], &screen[2], &screen[3], (uint32_t)E.camera.num, E.camera.intrins,
+        (uint32_t)E.camera.width, (uint32_t)E.camera.height, nullptr, nullptr);
+    E.fwd.isect_ids = ids; E.fwd.flatten_ids = flat; E.fwd.tile_offsets = offsets;
+
+    auto [renders, Ts, last, dist, median] = rasterize_to_pixels_3dgs_fwd(
+        N, in_splats, screen, DeviceVector<int32_t>{}, (uint32_t)E.camera.width, (uint32_t)E.camera.height, offsets, flat,
+        (DistortionType)dist_type_int, output_median);
+    E.fwd.renders = renders; E.fwd.render_Ts = Ts; E.fwd.last_ids = last;
+}
+
+void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
+                                      TorchTensorView v_render_Ts) {
+    auto& E = engine();
+    if (std::get<0>(E.fwd.renders).data_ptr() == nullptr)
+        throw std::runtime_error("engine_backward_from_render_grad: forward_3dgs must be called first");
+    alloc_grad_buffers();
+    const int64_t C = E.camera.num, H = E.camera.height, W = E.camera.width;
+    // stage the cotangents into pool buffers; Auto routes host and device sources alike
+    // (src/engine/EngineLoss.cpp:420-428). A device source is used in place.
+    auto stage = [&](PoolSlot slot, const TorchTensorView& src, int ch) -> float* {
+        void* s = (void*)std::get<0>(src);
+        if (backend::is_device_pointer(s)) return (float*)s;
+        float* d = DevicePool::global().acquire<float>(slot, (size_t)(C * H * W * ch));
+        backend::memcpy_sync(d, s, (size_t)(C * H * W * ch) * sizeof(float), backend::MemcpyKind::Auto);
+        return d;
+    };
+    float* v_rgb = stage(PoolSlot::EngVRgb, v_render_rgb, 3);
+    float* v_depth = stage(PoolSlot::EngVDepth, v_render_depth, 1);
+    float* v_Ts = stage(PoolSlot::EngVTs, v_render_Ts, 1);
+    RenderOutput::TensorTuple v_renders;
+    std::get<0>(v_renders) = DeviceTensor3D<float3>((float3*)v_rgb, C, H, W);
+    std::get<1>(v_renders) = DeviceTensor3D<float>(v_depth, C, H, W);
+    DeviceTensor3D<float> v_Ts_t(v_Ts, C, H, W);
+
+    // _engine_raster_proj_backward, non-fused branch (src/engine/EngineLoss.cpp:218-240,294-390)
+    auto [vw, vs, accum] = rasterize_to_pixels_3dgs_bwd(
+        E.cur_num_splats, E.fwd.splats_w, E.fwd.splats_s, DeviceVector<int32_t>{}, (uint32_t)W, (uint32_t)H,
+        E.fwd.tile_offsets, E.fwd.flatten_ids, E.fwd.render_Ts, E.fwd.last_ids, E.fwd.renders, std::nullopt,
+        DistortionType::None, DeviceTensor3D<float>{}, DensifyAccumMode::None, v_renders, v_Ts_t, DeviceTensor3D<float>{},
+        std::nullopt, std::nullopt, std::nullopt);
+    E.grad.v_screen = vs;
+    std::vector<DeviceTensorFloatND> v_world = {
+        DeviceTensorFloatND(E.grad.means), DeviceTensorFloatND(E.grad.quats), DeviceTensorFloatND(E.grad.scales),
+        DeviceTensorFloatND((float*)E.grad.opacities.data_ptr(), {E.grad.opacities.size(), 1}),
+        DeviceTensorFloatND(E.grad.features_dc), DeviceTensorFloatND(E.grad.features_sh)};
+    projection_3dgs_backward(
+        E.cur_num_splats, E.sh_degree, E.fwd.splats_w, E.camera.viewmats, E.camera.intrins, (uint32_t)W, (uint32_t)H,
+        E.camera.model_str, E.camera.distortion_str, E.camera.dist_coeffs, DeviceVector<int32_t>{}, DeviceVector<int32_t>{},
+        E.fwd.aabb, vs, v_world, nullptr, E.world.sh_packed, E.world.sh_bounds, (uint32_t)E.num_sh, E.world.sh_value_bits,
+        E.world.sh_bounds_stride);
+}
+
+void engine_copy_render_to_host(TorchTensorView out_rgb, TorchTensorView out_depth, TorchTensorView out_Ts,
+                                TorchTensorView, TorchTensorView) {
+    auto& f = engine().fwd;
+    auto& rgb = std::get<0>(f.renders);
+    auto& depth = std::get<1>(f.renders);
+    if (rgb.data_ptr() && std::get<0>(out_rgb))
+        backend::memcpy_sync((void*)std::get<0>(out_rgb), rgb.data_ptr(), rgb.numel() * sizeof(float3), backend::MemcpyKind::DeviceToHost);
+    if (depth.data_ptr() && std::get<0>(out_depth))
+        backend::memcpy_sync((void*)std::get<0>(out_depth), depth.data_ptr(), depth.numel() * sizeof(float), backend::MemcpyKind::DeviceToHost);
+    if (f.render_Ts.data_ptr() && std::get<0>(out_Ts))
+        backend::memcpy_sync((void*)std::get<0>(out_Ts), f.render_Ts.data_ptr(), f.render_Ts.numel() * sizeof(float), backend::MemcpyKind::DeviceToHost);
+}
+
+void engine_copy_grads_to_host(TorchTensorView means, TorchTensorView quats, TorchTensorView scales,
+                               TorchTensorView opacities, TorchTensorView features_dc, TorchTensorView features_sh) {
+    auto& g = engine().grad;
+    auto put = [](void* dst, const void* src, size_t bytes) {
+        if (dst && src && bytes) backend::memcpy_sync(dst, src, bytes, backend::MemcpyKind::DeviceToHost);
+    };
+    put((void*)std::get<0>(means), g.means.data_ptr(), g.means.size() * sizeof(float3));
+    put((void*)std::get<0>(quats), g.quats.data_ptr(), g.quats.size() * sizeof(float4));
+    put((void*)std::get<0>(scales), g.scales.data_ptr(), g.scales.size() * sizeof(float3));
+    put((void*)std::get<0>(opacities), g.opacities.data_ptr(), g.opacities.size() * sizeof(float));
+    put((void*)std::get<0>(features_dc), g.features_dc.data_ptr(), g.features_dc.size() * sizeof(float3));
+    put((void*)std::get<0>(features_sh), g.features_sh.data_ptr(), g.features_sh.numel() * sizeof(float3));
+}
+
+// ---------------------------------------------------------------------------------------------
+// C entry points for Python (tests, smoke, bench). Exceptions become a return code and a message.
+namespace {
+thread_local std::string g_host_error;
+template <class F> int guard(F&& f) {
+    try { f(); return 0; }
+    catch (const std::exception& e) { g_host_error = e.what(); return 1; }
+}
+TorchTensorView tv(const void* p, uint32_t elem, std::vector<int64_t> shape) { return TorchTensorView((uint64_t)p, elem, std::move(shape)); }
+}  // namespace
+
+extern "C" {
+
+const char* ssrh_last_error(void) { static thread_local std::string out; out.swap(g_host_error); g_host_error.clear(); return out.c_str(); }
+
+int ssrh_init(int device) { return guard([&] { if (!backend::device_select(device)) throw std::runtime_error(std::string("device_select failed: ") + backend::last_error()); }); }
+
+int ssrh_reset(void) { return guard([&] { engine_reset(); }); }
+
+int ssrh_set_options(int fuse_tile_count, int overwrite_world_grads, int sh_int8_f16scale, int stage_profiling) {
+    return guard([&] {
+        auto& o = ssr_ext::options();
+        o.fuse_tile_count = fuse_tile_count != 0; o.overwrite_world_grads = overwrite_world_grads != 0;
+        o.sh_int8_f16scale = sh_int8_f16scale != 0;
+        ssr_ext::set_stage_profiling(stage_profiling != 0);
+    });
+}
+
+// host or device pointers; num_sh = coefficients per splat excluding DC (15 for SH3)
+int ssrh_set_data_3dgs(int64_t n, const float* means, const float* quats, const float* scales, const float* opacities,
+                       const float* dc, const float* sh, int num_sh) {
+    return guard([&] {
+        set_data_3dgs(n, tv(means, 4, {n, 3}), tv(quats, 4, {n, 4}), tv(scales, 4, {n, 3}), tv(opacities, 4, {n, 1}),
+                      tv(dc, 4, {n, 3}), tv(sh, 4, {n, num_sh, 3}));
+    });
+}
+
+int ssrh_set_sh_value_quant(int bits, const void* packed, int64_t packed_count, int packed_elem, const void* bounds,
+                            int64_t bounds_count, int bounds_elem, int64_t bounds_stride) {
+    return guard([&] { set_sh_value_quant(bits, tv(packed, (uint32_t)packed_elem, {packed_count}), tv(bounds, (uint32_t)bounds_elem, {bounds_count}), bounds_stride); });
+}
+
+int ssrh_set_camera_params(int width, int height, const char* model, const char* distortion, const float* viewmats,
+                           const float* intrins, int num_cameras) {
+    return guard([&] {
+        static const float zero_coeffs[8 * 16] = {0};
+        set_camera_params(width, height, model, distortion, tv(viewmats, 4, {num_cameras, 4, 4}), tv(intrins, 4, {num_cameras, 4}),
+                          tv(zero_coeffs, 4, {num_cameras, 8}));
+    });
+}
+
+int ssrh_forward_3dgs(const char* primitive, int sh_degree, int packed, int output_median, int dist_type) {
+    return guard([&] { forward_3dgs(primitive, sh_degree, packed != 0, output_median != 0, dist_type); });
+}
+
+int ssrh_backward_from_render_grad(const float* v_rgb, const float* v_depth, const float* v_Ts) {
+    return guard([&] {
+        const int64_t C = engine().camera.num, H = engine().camera.height, W = engine().camera.width;
+        engine_backward_from_render_grad(tv(v_rgb, 4, {C, H, W, 3}), tv(v_depth, 4, {C, H, W, 1}), tv(v_Ts, 4, {C, H, W, 1}));
+    });
+}
+
+int ssrh_copy_render_to_host(float* rgb, float* depth, float* Ts) {
+    return guard([&] {
+        const int64_t C = engine().camera.num, H = engine().camera.height, W = engine().camera.width;
+        engine_copy_render_to_host(tv(rgb, 4, {C, H, W, 3}), tv(depth, 4, {C, H, W, 1}), tv(Ts, 4, {C, H, W, 1}), tv(nullptr, 4, {0}), tv(nullptr, 4, {0}));
+    });
+}
+
+int ssrh_copy_grads_to_host(float* means, float* quats, float* scales, float* opacities, float* dc, float* sh) {
+    return guard([&] {
+        const int64_t n = engine().max_num_splats;
+        engine_copy_grads_to_host(tv(means, 4, {n, 3}), tv(quats, 4, {n, 4}), tv(scales, 4, {n, 3}), tv(opacities, 4, {n, 1}),
+                                  tv(dc, 4, {n, 3}), tv(sh, 4, {n, engine().num_sh, 3}));
+    });
+}
+
+// Device addresses of the forward cache, for tests that compare intermediate buffers.
+//   which: 0 aabb, 1 sort depths, 2..6 screen xy/depth/conic/opac/rgb, 7 sorted keys, 8 sorted ids,
+//          9 tile offsets, 10 last_ids, 11 radii, 12..16 v_screen xy/depth/conic/opac/rgb
+int ssrh_cache_pointer(int which, void** ptr, int64_t* count) {
+    return guard([&] {
+        auto& E = engine();
+        auto nd = [&](const DeviceTensorFloatND& t) { *ptr = t.data_ptr(); *count = t.numel(); };
+        switch (which) {
+            case 0: *ptr = E.fwd.aabb.data_ptr(); *count = E.fwd.aabb.numel() * 4; break;
+            case 1: *ptr = E.fwd.depths.data_ptr(); *count = E.fwd.depths.numel(); break;
+            case 2: case 3: case 4: case 5: case 6: nd(E.fwd.splats_s.at(which - 2)); break;
+            case 7: *ptr = E.fwd.isect_ids.data_ptr(); *count = E.fwd.isect_ids.size(); break;
+            case 8: *ptr = E.fwd.flatten_ids.data_ptr(); *count = E.fwd.flatten_ids.size(); break;
+            case 9: *ptr = E.fwd.tile_offsets.data_ptr(); *count = E.fwd.tile_offsets.numel(); break;
+            case 10: *ptr = E.fwd.last_ids.data_ptr(); *count = E.fwd.last_ids.numel(); break;
+            case 11: *ptr = E.optim.radii.data_ptr(); *count = E.optim.radii.size(); break;
+            case 12: case 13: case 14: case 15: case 16: nd(E.grad.v_screen.at(which - 12)); break;
+            default: throw std::runtime_error("unknown cache buffer");
+        }
+    });
+}
+
+int64_t ssrh_last_n_isects(void) { return ssr_ext::last_n_isects(); }
+
+int ssrh_last_stage_times(float* out9) {
+    return guard([&] {
+        auto t = ssr_ext::last_stage_times();
+        const float v[9] = {t.k1, t.k2, t.k3, t.k4, t.k5, t.k6, t.k7, t.k8, t.k9};
+        std::memcpy(out9, v, sizeof(v));
+    });
+}
+
+// Runs `iters` forward+backward iterations back to back with device-resident cotangents and
+// returns the elapsed device time of each (events on the launch stream, one synchronise per
+// iteration at its end).
+int ssrh_time_iterations(int sh_degree, const float* v_rgb_dev, const float* v_depth_dev, const float* v_Ts_dev, int iters,
+                         float* ms_out) {
+    return guard([&] {
+        ssr_event_t a = ssr_event_create(), b = ssr_event_create();
+        for (int i = 0; i < iters; i++) {
+            ssr_event_record(a, nullptr);
+            forward_3dgs("3dgs", sh_degree, false, false, 0);
+            const int64_t C = engine().camera.num, H = engine().camera.height, W = engine().camera.width;
+            engine_backward_from_render_grad(tv(v_rgb_dev, 4, {C, H, W, 3}), tv(v_depth_dev, 4, {C, H, W, 1}), tv(v_Ts_dev, 4, {C, H, W, 1}));
+            ssr_event_record(b, nullptr);
+            float ms = 0;
+            if (ssr_event_elapsed_ms(a, b, &ms)) throw std::runtime_error(ssr_last_error());
+            ms_out[i] = ms;
+        }
+        ssr_event_destroy(a); ssr_event_destroy(b);
+    });
+}
+
+size_t ssrh_pool_bytes(void) { return DevicePool::global().total_bytes(); }
+
+}  // extern "C"

@@ -1,0 +1,63 @@
+// ssr_engine.hpp -- the caller side of the path: a process-global engine state that drives the
+// launch functions in the reference's order, with the reference's zero-fills and buffer lifetimes.
+//
+//   set_data_3dgs                     src/engine/EngineSetup.cpp:11-47
+//   set_camera_params                 src/engine/EngineSetup.cpp:50-87
+//   forward_3dgs                      src/engine/EngineForward.cpp:24-311
+//   engine_backward_from_render_grad  src/engine/EngineLoss.cpp:400-433 (-> :138-391, non-fused branch)
+//   engine_copy_render_to_host        src/engine/EngineQuery.cpp:36-76
+//   engine_copy_grads_to_host         src/engine/EngineQuery.cpp:122-140
+//
+// Inputs that are already device addresses are used in place; host memory is copied once
+// (src/engine/EngineCommon.h:90-105). The forward cache is retained for the backward
+// (src/engine/EngineState.h:127-160).
+#pragma once
+#include "ssr_backend_api.hpp"
+
+struct EngineState {
+    int64_t cur_num_splats = 0, max_num_splats = 0;
+    int num_sh = 0, sh_degree = 0;
+    std::string primitive;
+    bool packed = false;
+    struct {
+        bool initialized = false;
+        DeviceVector<float3> means; DeviceVector<float4> quats; DeviceVector<float3> scales;
+        DeviceVector<float> opacities; DeviceVector<float3> features_dc; DeviceTensor2D<float3> features_sh;
+        int sh_value_bits = 32;
+        std::optional<TorchTensorView> sh_packed, sh_bounds;
+        int64_t sh_bounds_stride = 0;
+    } world;
+    struct {
+        int width = 0, height = 0, num = 0;
+        std::string model_str = "PINHOLE", distortion_str = "NONE";
+        TorchTensorView viewmats, intrins, dist_coeffs;
+    } camera;
+    struct { DeviceVector<float> radii; bool skip_grad_zero = false; } optim;
+    struct {
+        std::vector<DeviceTensorFloatND> splats_w, splats_s;
+        DeviceTensor2D<float4> aabb; DeviceTensor2D<float> depths;
+        DeviceVector<int64_t> isect_ids; DeviceVector<int32_t> flatten_ids; DeviceTensor3D<int32_t> tile_offsets;
+        RenderOutput::TensorTuple renders; DeviceTensor3D<float> render_Ts; DeviceTensor3D<int32_t> last_ids;
+    } fwd;
+    struct {
+        DeviceVector<float3> means; DeviceVector<float4> quats; DeviceVector<float3> scales;
+        DeviceVector<float> opacities; DeviceVector<float3> features_dc; DeviceTensor2D<float3> features_sh;
+        std::vector<DeviceTensorFloatND> v_screen;
+    } grad;
+};
+EngineState& engine();
+void engine_reset();   // drop all state (not the pool)
+
+void set_data_3dgs(int64_t num_splats, TorchTensorView means, TorchTensorView quats, TorchTensorView scales,
+                   TorchTensorView opacities, TorchTensorView features_dc, TorchTensorView features_sh);
+// quantized SH storage (engine().world.features_sh_quant*, src/engine/EngineForward.cpp:76-116)
+void set_sh_value_quant(int sh_value_bits, TorchTensorView packed, TorchTensorView bounds, int64_t bounds_stride);
+void set_camera_params(int width, int height, std::string camera_model, std::string distortion,
+                       TorchTensorView viewmats, TorchTensorView intrins, TorchTensorView dist_coeffs);
+void forward_3dgs(std::string primitive, int sh_degree, bool packed, bool output_median, int dist_type_int);
+void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
+                                      TorchTensorView v_render_Ts);
+void engine_copy_render_to_host(TorchTensorView out_rgb, TorchTensorView out_depth, TorchTensorView out_Ts,
+                                TorchTensorView out_rgb_raw, TorchTensorView out_median);
+void engine_copy_grads_to_host(TorchTensorView means, TorchTensorView quats, TorchTensorView scales,
+                               TorchTensorView opacities, TorchTensorView features_dc, TorchTensorView features_sh);

@@ -1,0 +1,127 @@
+"""GPU: the C++ host layer (reference-shaped launch functions + engine call order) against the
+oracle, in both stage orders, and the behaviours the engine relies on."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def H(pkg):
+    from spirula_studio_amd import host, lib
+    host.load()
+    return host, lib
+
+
+def _check(eng, ref, sc):
+    assert np.array_equal(eng.cache("sorted_ids"), ref["sorted_ids"])
+    assert np.array_equal(eng.cache("sorted_flat"), ref["sorted_flat"])
+    assert np.array_equal(eng.cache("offsets"), ref["offsets"])
+    assert np.array_equal(eng.cache("aabb").reshape(-1, 4), ref["proj"]["aabb"])
+    assert np.array_equal(eng.cache("radii"), ref["proj"]["radii"])
+    rgb, depth, T = eng.render()
+    assert np.abs(rgb - ref["fwd"]["rgb"]).max() <= 1e-4
+    assert np.abs(T - ref["fwd"]["T"]).max() <= 1e-4
+    assert np.array_equal(eng.cache("last_ids").reshape(sc.height, sc.width), ref["fwd"]["last_ids"])
+    g = eng.grads()
+    for k, v in g.items():
+        r = ref["grads"][k].astype(np.float64).reshape(sc.n, -1)
+        scale = np.abs(r).max(axis=1, keepdims=True)
+        err = np.abs(v.reshape(sc.n, -1) - r)
+        assert (err <= 2e-3 * scale + 2e-5 * (np.abs(r).mean() + 1e-12)).all(), k
+    return g
+
+
+@pytest.mark.parametrize("native", [False, True])
+def test_engine_matches_oracle(pkg, oracle, H, native):
+    host, lib = H
+    sc = pkg.scenes.make_scene(1, n=30000, width=320, height=240, parity_variant=True)
+    ref = oracle.pipeline(sc)
+    eng = host.Engine(sc, fuse_tile_count=native, overwrite_world_grads=native)
+    eng.forward()
+    eng.backward()
+    g1 = _check(eng, ref, sc)
+    # a second forward+backward on the same inputs: zero-fills honoured, nothing accumulates
+    eng.forward()
+    eng.backward()
+    g2 = _check(eng, ref, sc)
+    for k in g1:
+        assert np.allclose(g1[k], g2[k], rtol=2e-3, atol=1e-6)
+
+
+def test_engine_quantized_and_equirect(pkg, oracle, H):
+    host, lib = H
+    for cfg, kw in [(3, dict(n=20000, width=320, height=192)), (5, dict(n=30000, width=512, height=256))]:
+        sc = pkg.scenes.make_scene(cfg, **kw)
+        ref = oracle.pipeline(sc)
+        eng = host.Engine(sc)
+        eng.forward()
+        eng.backward()
+        _check(eng, ref, sc)
+    sc = pkg.scenes.make_scene(3, n=20000, width=320, height=192, sh_codec=0)
+    pkg.scenes.apply_sh_codec(sc, 1, bounds_stride=256)
+    ref = oracle.pipeline(sc)
+    eng = host.Engine(sc)
+    eng.forward()
+    eng.backward()
+    _check(eng, ref, sc)
+
+
+def test_unsupported_variants_raise(pkg, H):
+    host, lib = H
+    sc = pkg.scenes.tiny_scene(n=50, width=32, height=32)
+    eng = host.Engine(sc)
+    h = host.load()
+    for args in [(b"3dgut", 3, 0, 0, 0), (b"3dgs", 3, 1, 0, 0), (b"3dgs", 3, 0, 1, 0), (b"3dgs", 3, 0, 0, 1)]:
+        assert h.ssrh_forward_3dgs(*args) != 0
+        assert b"not built" in h.ssrh_last_error()
+    assert h.ssrh_set_camera_params(32, 32, b"FISHEYE", b"NONE", None, None, 1) == 0
+    assert h.ssrh_forward_3dgs(b"3dgs", 3, 0, 0, 0) != 0
+    assert b"FISHEYE" in h.ssrh_last_error()
+
+
+def test_runtime_contract(pkg, H):
+    """The checklist of src/backend/vulkan/tests/vk_runtime_smoke.cpp:44-160."""
+    host, lib = H
+    L = lib.load()
+    lib.check(L.ssr_init(0))
+    assert L.ssr_device_malloc(0) is None
+    d = L.ssr_device_malloc(1 << 20)
+    assert d and L.ssr_is_device_pointer(d) == 1 and L.ssr_is_device_pointer(d + 4096) == 1
+    p = L.ssr_host_malloc_pinned(4096)
+    assert p and L.ssr_is_device_pointer(p) == 0            # pinned host memory is not a device pointer
+    a = np.arange(1000, dtype=np.int32)
+    assert L.ssr_is_device_pointer(a.ctypes.data) == 0
+    # all copy kinds, including Auto routing
+    lib.check(L.ssr_memcpy(d, a.ctypes.data, a.nbytes, lib.H2D, None, 0))
+    d2 = L.ssr_device_malloc(a.nbytes)
+    lib.check(L.ssr_memcpy(d2, d, a.nbytes, lib.AUTO, None, 0))
+    b = np.zeros_like(a)
+    lib.check(L.ssr_memcpy(b.ctypes.data, d2, a.nbytes, lib.AUTO, None, 0))
+    assert np.array_equal(a, b)
+    # memset with an unaligned byte tail
+    lib.check(L.ssr_memset(d + 1, 0xAB, 1001, None, 0))
+    c = np.zeros(1004, np.uint8)
+    lib.check(L.ssr_memcpy(c.ctypes.data, d, 1004, lib.D2H, None, 0))
+    assert c[0] == 0 and np.all(c[1:1002] == 0xAB) and c[1002] != 0xAB
+    # pinned async readback fenced by an event
+    ev = L.ssr_event_create()
+    lib.check(L.ssr_memcpy(p, d2, 4000, lib.D2H, None, 1))
+    lib.check(L.ssr_event_record(ev, None))
+    lib.check(L.ssr_event_synchronize(ev))
+    import ctypes as C
+    assert np.array_equal(np.frombuffer((C.c_int32 * 1000).from_address(p), np.int32), a)
+    # timing events
+    e0, e1 = L.ssr_event_create(), L.ssr_event_create()
+    lib.check(L.ssr_event_record(e0, None))
+    lib.check(L.ssr_fill_u32(d, 7, (1 << 20) // 4, None))
+    lib.check(L.ssr_event_record(e1, None))
+    ms = C.c_float(-1)
+    lib.check(L.ssr_event_elapsed_ms(e0, e1, C.byref(ms)))
+    assert ms.value >= 0
+    # sticky error: reported once, cleared by the read
+    assert L.ssr_memcpy(None, None, 16, lib.H2D, None, 0) != 0
+    assert L.ssr_last_error() != b"" and L.ssr_last_error() == b""
+    for e in (ev, e0, e1):
+        L.ssr_event_destroy(e)
+    L.ssr_device_free(d); L.ssr_device_free(d2); L.ssr_host_free_pinned(p)
