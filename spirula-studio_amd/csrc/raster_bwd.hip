@@ -13,28 +13,39 @@
 // pixels of one 8x8 sub-tile in its lanes (state in registers, no LDS traffic for it); fragments
 // are staged per 16x16 tile in LDS, back to front, shared by the tile's 4 wavefronts; each
 // wavefront walks the fragments whose footprint bit is set. The ten per-splat sums are reduced
-// across the wavefront with DPP (quad permutes, row mirrors, row broadcasts) and issued as ONE
-// 10-lane float atomic instruction per (splat, sub-tile) -- the same number of atomic operations
-// as the reference (src/primitives/PrimitiveBase3DGS.cuh:177-183), non-finite sums dropped and
-// zeros skipped as there (src/core/Common.cuh:791-856). The scan starts at the tile's largest
+// across the wavefront by a transposing reduction: v_permlane32_swap and v_permlane16_swap (gfx950)
+// each fold one level of TWO channels at once, leaving 3 registers that hold one channel per
+// 16-lane row; 4 DPP steps per register finish the rows (28 operations instead of 60). Ten lanes
+// then issue ONE float atomic instruction per (splat, sub-tile) -- the same number of atomic
+// operations as the reference (src/primitives/PrimitiveBase3DGS.cuh:177-183), non-finite sums
+// dropped and zeros skipped as there (src/core/Common.cuh:791-856). The scan starts at the tile's largest
 // last_id rather than at the end of the range; splats beyond it are skipped by every pixel anyway.
 #include "raster_device.h"
 
 namespace ssr {
 
-template <int kCtrl, int kRowMask>
+template <int kCtrl>
 __device__ __forceinline__ float dpp_get(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, kRowMask, 0xf, false));
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, 0xf, 0xf, false));
 }
 
-// Sum over the 64 lanes; the total is valid in lanes 48..63.
-__device__ __forceinline__ float wave_sum_row3(float v) {
-    v += dpp_get<0xB1, 0xf>(v);    // quad_perm [1,0,3,2]
-    v += dpp_get<0x4E, 0xf>(v);    // quad_perm [2,3,0,1]
-    v += dpp_get<0x141, 0xf>(v);   // row_half_mirror
-    v += dpp_get<0x140, 0xf>(v);   // row_mirror: every lane of a row holds the row sum
-    v += dpp_get<0x142, 0xa>(v);   // row_bcast15 into rows 1 and 3
-    v += dpp_get<0x143, 0xc>(v);   // row_bcast31 into rows 2 and 3
+// lanes 0..31: a[l] + a[l+32]; lanes 32..63: b[l-32] + b[l]
+__device__ __forceinline__ float fold32(float a, float b) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+// rows (16 lanes each): row0 = a.row0 + a.row1, row1 = b.row0 + b.row1, row2 = a.row2 + a.row3,
+// row3 = b.row2 + b.row3
+__device__ __forceinline__ float fold16(float a, float b) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+// every lane of a row receives the sum over its row
+__device__ __forceinline__ float row_sum(float v) {
+    v += dpp_get<0xB1>(v);     // quad_perm [1,0,3,2]
+    v += dpp_get<0x4E>(v);     // quad_perm [2,3,0,1]
+    v += dpp_get<0x141>(v);    // row_half_mirror
+    v += dpp_get<0x140>(v);    // row_mirror
     return v;
 }
 
@@ -84,6 +95,30 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
     const int tile_last = max(max(s_wave_max[0], s_wave_max[1]), max(s_wave_max[2], s_wave_max[3]));
     const float tile_x0 = (float)(tx * kTile), tile_y0 = (float)(ty * kTile);
 
+    // After the reduction, row r of register j holds channel kChan[j][r] in all its lanes; lane
+    // 16 r + j (j < 3) adds that channel. Destination = base + stride * splat, fixed per lane.
+    //   channels: 0,1 xy  2 depth  3,4,5 conic  6 opac  7,8,9 rgb
+    const int row = lane >> 4, sub = lane & 15;
+    int chan = -1;
+    if (sub == 0) chan = row == 0 ? 0 : row == 1 ? 2 : row == 2 ? 1 : 3;
+    else if (sub == 1) chan = row == 0 ? 4 : row == 1 ? 6 : row == 2 ? 5 : 7;
+    else if (sub == 2 && (row & 1) == 0) chan = row == 0 ? 8 : 9;
+    float* abase = nullptr;
+    int astride = 0;
+    switch (chan) {
+        case 0: abase = P.v_screen.xy; astride = 2; break;
+        case 1: abase = P.v_screen.xy + 1; astride = 2; break;
+        case 2: abase = P.v_screen.depth; astride = 1; break;
+        case 3: abase = P.v_screen.conic; astride = 3; break;
+        case 4: abase = P.v_screen.conic + 1; astride = 3; break;
+        case 5: abase = P.v_screen.conic + 2; astride = 3; break;
+        case 6: abase = P.v_screen.opac; astride = 1; break;
+        case 7: abase = P.v_screen.rgb; astride = 3; break;
+        case 8: abase = P.v_screen.rgb + 1; astride = 3; break;
+        case 9: abase = P.v_screen.rgb + 2; astride = 3; break;
+        default: break;
+    }
+
     for (int32_t hi = min(range_end - 1, tile_last); hi >= range_start; hi -= kBatch) {
         __syncthreads();   // previous batch fully consumed
         const int32_t idx = hi - tid;   // LDS slot t holds sorted index hi - t: ascending t is back to front
@@ -106,62 +141,45 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
                 const int k = c * 64 + t;
                 const int32_t sorted_idx = hi - k;
                 if (sorted_idx > wave_last) continue;
-                const float4 q0 = frags[k].q0, q1 = frags[k].q1;
+                const float4 q0 = frags[k].q0, q1 = frags[k].q1, q2 = frags[k].q2;
                 float dx, dy, vis, sigma;
-                const float alpha = eval_alpha(q0, q1, px, py, dx, dy, vis, sigma);
+                const float alpha = eval_alpha_fast(q0, q1, q2.w, px, py, dx, dy, vis, sigma);
                 const bool active = sorted_idx <= bin_final && alpha > kAlphaThreshold;
                 if (__ballot(active) == 0ull) continue;
-                const float4 q2 = frags[k].q2;
                 const float opac = q1.y, cr = q1.z, cg = q1.w, cb = q2.x, cdp = q2.y;
                 float t_x = 0.f, t_y = 0.f, t_d = 0.f, t_ca = 0.f, t_cb = 0.f, t_cc = 0.f, t_o = 0.f, t_r = 0.f,
                       t_g = 0.f, t_b = 0.f;
                 if (active) {
-                    const float ra = 1.0f / (1.0f - alpha);
+                    // 1/(1-alpha) by the hardware reciprocal (1 ulp): gradients are compared at 1e-3
+                    const float ra = __builtin_amdgcn_rcpf(1.0f - alpha);
                     const float T0 = T1 * ra;
                     const float dotcv = ssr_fma(cdp, vd, ssr_fma(cb, vb, ssr_fma(cg, vg, cr * vr)));
-                    const float v_alpha = T0 * dotcv - vT1 * T0;
+                    const float v_alpha = T0 * (dotcv - vT1);
                     const float w = alpha * T0;
-                    const float v_T0 = alpha * dotcv + vT1 * (1.0f - alpha);
-                    if (sigma >= 0.f && opac * vis <= 0.999f) {
+                    const float v_T0 = ssr_fma(alpha, dotcv - vT1, vT1);
+                    if (opac * vis <= 0.999f) {   // sigma >= 0 holds for every active lane
                         const float v_sigma = (-opac) * vis * v_alpha;
-                        const float conx = q0.z + q0.z, conz = q1.x + q1.x, cony = q0.w;   // full conic
-                        t_ca = 0.5f * v_sigma * dx * dx;
-                        t_cb = v_sigma * dx * dy;
-                        t_cc = 0.5f * v_sigma * dy * dy;
-                        t_x = v_sigma * (conx * dx + cony * dy);
-                        t_y = v_sigma * (cony * dx + conz * dy);
+                        const float vsx = v_sigma * dx, vsy = v_sigma * dy;
+                        t_ca = 0.5f * vsx * dx;
+                        t_cb = vsx * dy;
+                        t_cc = 0.5f * vsy * dy;
+                        // conic.x = 2 * (0.5 conic.x), conic.z likewise
+                        t_x = ssr_fma(q0.z + q0.z, vsx, q0.w * vsy);
+                        t_y = ssr_fma(q0.w, vsx, (q1.x + q1.x) * vsy);
                         t_o = vis * v_alpha;
                     }
                     t_r = vr * w; t_g = vg * w; t_b = vb * w; t_d = vd * w;
                     T1 = T0; vT1 = v_T0;
                 }
-                // wavefront reduction, then lanes 48..57 each own one of the ten sums
-                const float s0 = wave_sum_row3(t_x), s1 = wave_sum_row3(t_y), s2 = wave_sum_row3(t_d),
-                            s3 = wave_sum_row3(t_ca), s4 = wave_sum_row3(t_cb), s5 = wave_sum_row3(t_cc),
-                            s6 = wave_sum_row3(t_o), s7 = wave_sum_row3(t_r), s8 = wave_sum_row3(t_g),
-                            s9 = wave_sum_row3(t_b);
-                const int q = lane - 48;
-                float mine = s0;
-                mine = q == 1 ? s1 : mine; mine = q == 2 ? s2 : mine; mine = q == 3 ? s3 : mine;
-                mine = q == 4 ? s4 : mine; mine = q == 5 ? s5 : mine; mine = q == 6 ? s6 : mine;
-                mine = q == 7 ? s7 : mine; mine = q == 8 ? s8 : mine; mine = q == 9 ? s9 : mine;
-                if (q >= 0 && q < 10 && ssr_isfinite(mine) && mine != 0.0f) {
-                    const int64_t g = s_ids[k];
-                    float* dst;
-                    switch (q) {
-                        case 0: dst = P.v_screen.xy + 2 * g; break;
-                        case 1: dst = P.v_screen.xy + 2 * g + 1; break;
-                        case 2: dst = P.v_screen.depth + g; break;
-                        case 3: dst = P.v_screen.conic + 3 * g; break;
-                        case 4: dst = P.v_screen.conic + 3 * g + 1; break;
-                        case 5: dst = P.v_screen.conic + 3 * g + 2; break;
-                        case 6: dst = P.v_screen.opac + g; break;
-                        case 7: dst = P.v_screen.rgb + 3 * g; break;
-                        case 8: dst = P.v_screen.rgb + 3 * g + 1; break;
-                        default: dst = P.v_screen.rgb + 3 * g + 2; break;
-                    }
-                    atomicAdd(dst, mine);
-                }
+                // transposing reduction: 10 channels -> 3 registers with one channel per row
+                const float ra_ = fold32(t_x, t_y), rb_ = fold32(t_d, t_ca), rc_ = fold32(t_cb, t_cc),
+                            rd_ = fold32(t_o, t_r), re_ = fold32(t_g, t_b);
+                const float s1 = row_sum(fold16(ra_, rb_));   // rows: x, d, y, ca      -> channels 0,2,1,3
+                const float s2 = row_sum(fold16(rc_, rd_));   // rows: cb, o, cc, r     -> channels 4,6,5,7
+                const float s3 = row_sum(fold16(re_, re_));   // rows: g, g, b, b       -> channels 8,8,9,9
+                float mine = sub == 0 ? s1 : (sub == 1 ? s2 : s3);
+                if (chan >= 0 && ssr_isfinite(mine) && mine != 0.0f)
+                    atomicAdd(abase + (int64_t)astride * s_ids[k], mine);
             }
         }
     }

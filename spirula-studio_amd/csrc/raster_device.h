@@ -19,7 +19,7 @@ constexpr int kRasterBlock = 256;
 constexpr int kBatch = 256;
 
 // One staged fragment: 3 x 16 bytes, read back with broadcast 128-bit LDS loads.
-//   q0 = (x, y, 0.5*conic.x, conic.y)   q1 = (0.5*conic.z, opac, r, g)   q2 = (b, depth, hitmask, -)
+//   q0 = (x, y, 0.5*conic.x, conic.y)   q1 = (0.5*conic.z, opac, r, g)   q2 = (b, depth, hitmask, sigma cut)
 struct FragLds {
     float4 q0, q1, q2;
 };
@@ -61,7 +61,10 @@ __device__ __forceinline__ FragLds stage_fragment(const ssr_screen& s, int32_t g
     FragLds f;
     f.q0 = make_float4(xy.x, xy.y, 0.5f * cx, cy);
     f.q1 = make_float4(0.5f * cz, opac, rg[0], rg[1]);
-    f.q2 = make_float4(rg[2], s.depth[g], __uint_as_float(hits), 0.0f);
+    // sigma above which alpha <= 1/255 for certain: exp(-5.55) = 0.003888 < 1/255 = 0.003922 and
+    // opac <= 1 for anything the projection produced; a caller-supplied opac > 1 disables the cut.
+    const float cut = opac <= 1.0f ? 5.55f : __uint_as_float(0x7f800000u);
+    f.q2 = make_float4(rg[2], s.depth[g], __uint_as_float(hits), cut);
     return f;
 }
 
@@ -74,6 +77,37 @@ __device__ __forceinline__ float eval_alpha(const float4& q0, const float4& q1, 
     vis = ssr_exp(-sigma);
     const float alpha = ssr_min(0.999f, q1.y * vis);
     return sigma < 0.f ? 0.f : alpha;
+}
+
+// exp(x) for x in [-5.55, 0] (and NaN): the same operations as ssr_exp() on that range, where its
+// overflow / underflow branches are dead and 2^k (k in [-9, 0]) can be applied by adding k to the
+// exponent field -- exact, so the bits equal ssr_exp(x).
+__device__ __forceinline__ float exp_neg_small(float x) {
+    const float k = ssr_rint(x * 1.44269504088896341f);
+    float r = ssr_fma(k, -0.693359375f, x);
+    r = ssr_fma(k, 2.12194440e-4f, r);
+    const float z = r * r;
+    float p = 1.9875691500e-4f;
+    p = ssr_fma(p, r, 1.3981999507e-3f);
+    p = ssr_fma(p, r, 8.3334519073e-3f);
+    p = ssr_fma(p, r, 4.1665795894e-2f);
+    p = ssr_fma(p, r, 1.6666665459e-1f);
+    p = ssr_fma(p, r, 5.0000001201e-1f);
+    const float y = ssr_fma(p, z, r) + 1.0f;
+    int ki;   // hardware conversion: saturating, NaN -> 0 (a C cast of NaN would be undefined)
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(ki) : "v"(k));
+    return __uint_as_float(__float_as_uint(y) + ((uint32_t)ki << 23));
+}
+
+// eval_alpha() without the transcendental's range handling: identical results wherever
+// alpha > 1/255 can hold (0 <= sigma <= cut), and alpha = 0 -- the skipped case -- elsewhere.
+__device__ __forceinline__ float eval_alpha_fast(const float4& q0, const float4& q1, float cut, float px, float py,
+                                                 float& dx, float& dy, float& vis, float& sigma) {
+    dx = q0.x - px; dy = q0.y - py;
+    sigma = ssr_fma(q0.z * dx, dx, ssr_fma(q1.x * dy, dy, (q0.w * dx) * dy));
+    vis = exp_neg_small(-sigma);
+    const float alpha = ssr_min(0.999f, q1.y * vis);
+    return (sigma < 0.f || sigma > cut) ? 0.f : alpha;
 }
 
 // Workgroup id -> tile id so that each of the 8 XCDs (workgroups are dealt to them round-robin)

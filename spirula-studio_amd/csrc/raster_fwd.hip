@@ -49,13 +49,12 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_kernel(ssr_raster_fwd
                 const int t = __builtin_ctzll(m);
                 m &= m - 1;
                 const int k = c * 64 + t;
-                const float4 q0 = frags[k].q0, q1 = frags[k].q1;
+                const float4 q0 = frags[k].q0, q1 = frags[k].q1, q2 = frags[k].q2;
                 float dx, dy, vis, sigma;
-                const float alpha = eval_alpha(q0, q1, px, py, dx, dy, vis, sigma);
+                const float alpha = eval_alpha_fast(q0, q1, q2.w, px, py, dx, dy, vis, sigma);
                 if (!done && alpha > kAlphaThreshold) {
                     const float next_T = T * (1.0f - alpha);
                     if (next_T > kTransmitThreshold) {
-                        const float4 q2 = frags[k].q2;
                         const float w = alpha * T;
                         cr = ssr_fma(q1.z, w, cr); cg = ssr_fma(q1.w, w, cg); cb = ssr_fma(q2.x, w, cb);
                         cd = ssr_fma(q2.y, w, cd);
