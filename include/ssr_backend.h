@@ -98,6 +98,11 @@ typedef struct {
     float* radii;           /* [N], caller zero-fills (src/engine/EngineForward.cpp:66-69) */
     ssr_screen screen;
     int64_t* tiles_per_splat; /* optional [C*N] */
+    /* Optional work list (no counterpart in the reference's non-packed path): the indices of the
+     * splats whose screen row was written, in no particular order, appended at *visible_count
+     * (which the caller zeroes). Later stages can then run over V entries instead of N. */
+    int32_t* visible_ids;     /* optional [C*N] */
+    int64_t* visible_count;   /* required when visible_ids is given */
 } ssr_projection_fwd_params;
 int ssr_projection_fwd(const ssr_projection_fwd_params* p, ssr_stream_t stream);
 
@@ -108,14 +113,19 @@ int ssr_tile_count(int64_t n, const float* aabb, const float* xy, const float* c
                    ssr_stream_t stream);
 /* inclusive_sum<int64> (src/backend/common/SortScan.h:58-72; IntersectTile.cu:425-428). */
 size_t ssr_scan_scratch_bytes(int64_t n);
-int ssr_inclusive_sum_i64(const int64_t* in, int64_t* out, int64_t n, void* scratch,
-                          size_t scratch_bytes, ssr_stream_t stream);
-/* The reference's blocking 8-byte readback of n_isects (IntersectTile.cu:432-436). */
-int ssr_read_i64(const int64_t* device_value, int64_t* host_value, ssr_stream_t stream);
+/* total_out (optional) also receives out[n-1], so that it can sit next to other counters and be
+ * read back in one copy. */
+int ssr_inclusive_sum_i64(const int64_t* in, int64_t* out, int64_t n, int64_t* total_out,
+                          void* scratch, size_t scratch_bytes, ssr_stream_t stream);
+/* The reference's blocking readback of n_isects (8 bytes, IntersectTile.cu:432-436); `count`
+ * consecutive values are copied. */
+int ssr_read_i64(const int64_t* device_values, int64_t* host_values, int count, ssr_stream_t stream);
+/* visible_ids (optional, with n_visible entries): run over that work list instead of all n splats;
+ * the keys written are the same. */
 int ssr_tile_write(int64_t n, const float* aabb, const float* sort_depth, const float* xy,
                    const float* conic, const float* opac, const int64_t* cum_tiles,
                    uint32_t width, uint32_t height, int64_t* isect_ids, int32_t* flatten_ids,
-                   ssr_stream_t stream);
+                   const int32_t* visible_ids, int64_t n_visible, ssr_stream_t stream);
 /* sort_pairs<int64,int32> with CUB DoubleBuffer semantics (src/backend/common/SortScan.h:42-56;
  * call site IntersectTile.cu:486-493): stable on bits [begin_bit,end_bit); *selector says which
  * of the (a,b) buffers holds the result. */
@@ -181,6 +191,11 @@ typedef struct {
     ssr_screen v_screen;    /* read */
     ssr_world v_world;      /* written / accumulated */
     int32_t accumulate;
+    /* Optional work list from ssr_projection_fwd: only these splats are processed. With
+     * accumulate == 0 their rows are overwritten and rows of other splats are NOT touched (the
+     * caller zero-fills v_world once, as the reference does). */
+    const int32_t* visible_ids;
+    int64_t n_visible;
 } ssr_projection_bwd_params;
 int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream_t stream);
 

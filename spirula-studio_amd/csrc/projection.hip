@@ -33,60 +33,81 @@ __device__ __forceinline__ void atomic_max_nonneg(float* p, float v) {
     atomicMax(reinterpret_cast<int*>(p), __float_as_int(v));
 }
 
+// Two phases per workgroup of 256 splats. Phase 1: every thread projects its splat (44 B in) and
+// writes aabb / sorting depth / geometry row / tile count; splats that stay visible are appended
+// to a list in LDS. Phase 2: the first n_visible threads evaluate SH colour (192 B in) for the
+// listed splats, so the expensive part runs on dense wavefronts however sparse visibility is.
 template <int kDegree>
 __global__ __launch_bounds__(kProjBlock) void projection_fwd_kernel(ssr_projection_fwd_params P) {
-    const int64_t g = (int64_t)blockIdx.x * kProjBlock + threadIdx.x;
-    if (g >= P.num_splats) return;
+    __shared__ int s_list[kProjBlock];
+    __shared__ int s_count;
+    __shared__ long long s_base;
+    if (threadIdx.x == 0) s_count = 0;
+    __syncthreads();
+    const int64_t block0 = (int64_t)blockIdx.x * kProjBlock;
+    const int64_t g = block0 + threadIdx.x;
     const CamD cam = load_camera(P.camera);
-    float mean[3], quat[4], ls[3], logit;
-    load_splat(P.world, g, mean, quat, ls, logit);
-    ProjD p;
-    project<false>(cam, mean, quat, ls, logit, p);
-
-    float col[3] = {0.f, 0.f, 0.f};
-    float bb[4] = {p.aabb[0], p.aabb[1], p.aabb[2], p.aabb[3]};
-    if (bb[2] > bb[0] && bb[3] > bb[1]) {
-        constexpr int kCoef = kDegree * (kDegree + 2);
-        float coef[kCoef > 0 ? 3 * kCoef : 1];
-        if (kCoef > 0) decode_sh<kCoef>(P.world, P.sh, g, coef);
-        float dir[3];
-        view_dir(cam, mean, dir);
-        ShBasisD b;
-        sh_basis<kDegree>(dir, b);
-        const float* dcp = P.world.features_dc + 3 * g;
-        const float dc[3] = {dcp[0], dcp[1], dcp[2]};
-        float raw[3];
-        sh_color_raw<kDegree>(b, dc, coef, raw);
-#pragma unroll
-        for (int c = 0; c < 3; c++) col[c] = ssr_max(raw[c] + 0.5f, 0.0f);
-    }
-    bb[0] = ssr_min(ssr_max(bb[0], 0.0f), cam.Wf - 1.0f);
-    bb[1] = ssr_min(ssr_max(bb[1], 0.0f), cam.Hf - 1.0f);
-    bb[2] = ssr_min(ssr_max(bb[2], 0.0f), cam.Wf - 1.0f);
-    bb[3] = ssr_min(ssr_max(bb[3], 0.0f), cam.Hf - 1.0f);
-    float4* aabb_out = reinterpret_cast<float4*>(P.aabb);
-    if (bb[2] - bb[0] > 1e-3f && bb[3] - bb[1] > 1e-3f) {
-        *reinterpret_cast<float2*>(P.screen.xy + 2 * g) = make_float2(p.xy[0], p.xy[1]);
-        P.screen.depth[g] = p.depth;
-        float* cn = P.screen.conic + 3 * g;
-        cn[0] = p.conic[0]; cn[1] = p.conic[1]; cn[2] = p.conic[2];
-        P.screen.opac[g] = p.opac;
-        float* rg = P.screen.rgb + 3 * g;
-        rg[0] = col[0]; rg[1] = col[1]; rg[2] = col[2];
-        aabb_out[g] = make_float4(bb[0], bb[1], bb[2], bb[3]);
-        P.sort_depth[g] = p.sort_depth;
-        atomic_max_nonneg(P.radii + g, p.radius);
-        if (P.tiles_per_splat) {
-            const int tw = (int)((P.camera.width + kTile - 1) / kTile), th = (int)((P.camera.height + kTile - 1) / kTile);
-            TileGeomD tg;
-            tile_geom(bb, p.xy, p.conic, p.opac, tw, th, tg);
-            P.tiles_per_splat[g] = count_tiles(tg);
+    if (g < P.num_splats) {
+        float mean[3], quat[4], ls[3], logit;
+        load_splat(P.world, g, mean, quat, ls, logit);
+        ProjD p;
+        project<false>(cam, mean, quat, ls, logit, p);
+        float bb[4] = {p.aabb[0], p.aabb[1], p.aabb[2], p.aabb[3]};
+        bb[0] = ssr_min(ssr_max(bb[0], 0.0f), cam.Wf - 1.0f);
+        bb[1] = ssr_min(ssr_max(bb[1], 0.0f), cam.Hf - 1.0f);
+        bb[2] = ssr_min(ssr_max(bb[2], 0.0f), cam.Wf - 1.0f);
+        bb[3] = ssr_min(ssr_max(bb[3], 0.0f), cam.Hf - 1.0f);
+        float4* aabb_out = reinterpret_cast<float4*>(P.aabb);
+        // a clamped extent > 1e-3 implies the unclamped aabb is non-empty, which is the reference's
+        // condition for evaluating the colour (src/primitives/Primitive3DGS.cuh:74)
+        if (bb[2] - bb[0] > 1e-3f && bb[3] - bb[1] > 1e-3f) {
+            *reinterpret_cast<float2*>(P.screen.xy + 2 * g) = make_float2(p.xy[0], p.xy[1]);
+            P.screen.depth[g] = p.depth;
+            float* cn = P.screen.conic + 3 * g;
+            cn[0] = p.conic[0]; cn[1] = p.conic[1]; cn[2] = p.conic[2];
+            P.screen.opac[g] = p.opac;
+            aabb_out[g] = make_float4(bb[0], bb[1], bb[2], bb[3]);
+            P.sort_depth[g] = p.sort_depth;
+            atomic_max_nonneg(P.radii + g, p.radius);
+            if (P.tiles_per_splat) {
+                const int tw = (int)((P.camera.width + kTile - 1) / kTile), th = (int)((P.camera.height + kTile - 1) / kTile);
+                TileGeomD tg;
+                tile_geom(bb, p.xy, p.conic, p.opac, tw, th, tg);
+                P.tiles_per_splat[g] = count_tiles(tg);
+            }
+            s_list[atomicAdd(&s_count, 1)] = threadIdx.x;
+        } else {
+            aabb_out[g] = make_float4(0.f, 0.f, 0.f, 0.f);
+            P.sort_depth[g] = 0.0f;
+            if (P.tiles_per_splat) P.tiles_per_splat[g] = 0;
         }
-    } else {
-        aabb_out[g] = make_float4(0.f, 0.f, 0.f, 0.f);
-        P.sort_depth[g] = 0.0f;
-        if (P.tiles_per_splat) P.tiles_per_splat[g] = 0;
     }
+    __syncthreads();
+    const int n_vis = s_count;
+    if (P.visible_ids) {
+        if (threadIdx.x == 0 && n_vis > 0)
+            s_base = (long long)atomicAdd(reinterpret_cast<unsigned long long*>(P.visible_count), (unsigned long long)n_vis);
+        __syncthreads();
+        if ((int)threadIdx.x < n_vis) P.visible_ids[s_base + threadIdx.x] = (int32_t)(block0 + s_list[threadIdx.x]);
+    }
+    if ((int)threadIdx.x >= n_vis) return;
+    const int64_t v = block0 + s_list[threadIdx.x];
+    const float* mp = P.world.means + 3 * v;
+    const float mean[3] = {mp[0], mp[1], mp[2]};
+    constexpr int kCoef = kDegree * (kDegree + 2);
+    float coef[kCoef > 0 ? 3 * kCoef : 1];
+    if (kCoef > 0) decode_sh<kCoef>(P.world, P.sh, v, coef);
+    float dir[3];
+    view_dir(cam, mean, dir);
+    ShBasisD b;
+    sh_basis<kDegree>(dir, b);
+    const float* dcp = P.world.features_dc + 3 * v;
+    const float dc[3] = {dcp[0], dcp[1], dcp[2]};
+    float raw[3];
+    sh_color_raw<kDegree>(b, dc, coef, raw);
+    float* rg = P.screen.rgb + 3 * v;
+#pragma unroll
+    for (int c = 0; c < 3; c++) rg[c] = ssr_max(raw[c] + 0.5f, 0.0f);
 }
 
 __device__ __forceinline__ float fin(float v) { return ssr_isfinite(v) ? v : 0.0f; }
@@ -99,13 +120,14 @@ __device__ __forceinline__ void put(float* p, float v) {
 
 template <int kDegree, bool kAccumulate>
 __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projection_bwd_params P) {
-    const int64_t g = (int64_t)blockIdx.x * kProjBlock + threadIdx.x;
-    if (g >= P.num_splats) return;
+    const int64_t i = (int64_t)blockIdx.x * kProjBlock + threadIdx.x;
+    if (i >= (P.visible_ids ? P.n_visible : P.num_splats)) return;
+    const int64_t g = P.visible_ids ? (int64_t)P.visible_ids[i] : i;
     constexpr int kCoef = kDegree * (kDegree + 2);
     const float4 bb = reinterpret_cast<const float4*>(P.aabb)[g];
     ssr_world& V = P.v_world;
     if (bb.z <= bb.x || bb.w <= bb.y) {   // ProjectionBwd_kernel.cuh:58
-        if (!kAccumulate) {
+        if (!kAccumulate && !P.visible_ids) {
 #pragma unroll
             for (int i = 0; i < 3; i++) { V.means[3 * g + i] = 0.f; V.log_scales[3 * g + i] = 0.f; V.features_dc[3 * g + i] = 0.f; }
             *reinterpret_cast<float4*>(V.quats + 4 * g) = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -380,6 +402,7 @@ extern "C" int ssr_projection_fwd(const ssr_projection_fwd_params* p, ssr_stream
     SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->aabb) & 15) == 0 && (reinterpret_cast<uintptr_t>(p->world.quats) & 15) == 0,
                 "ssr_projection_fwd", "aabb and quats must be 16-byte aligned");
     SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->screen.xy) & 7) == 0, "ssr_projection_fwd", "screen.xy must be 8-byte aligned");
+    SSR_REQUIRE(!p->visible_ids || p->visible_count, "ssr_projection_fwd", "visible_ids needs visible_count");
     const dim3 grid((unsigned)ceil_div(p->num_splats, kProjBlock)), block(kProjBlock);
     hipStream_t s = as_stream(stream);
     switch (p->sh_degree) {
@@ -406,7 +429,11 @@ extern "C" int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream
     SSR_REQUIRE(v.sh_stride >= 3 * p->sh_degree * (p->sh_degree + 2), "ssr_projection_bwd", "v_world.sh_stride too small");
     SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->aabb) & 15) == 0 && (reinterpret_cast<uintptr_t>(p->world.quats) & 15) == 0 &&
                 (reinterpret_cast<uintptr_t>(v.quats) & 15) == 0, "ssr_projection_bwd", "aabb and quats must be 16-byte aligned");
-    const dim3 grid((unsigned)ceil_div(p->num_splats, kProjBlock)), block(kProjBlock);
+    if (p->visible_ids) {
+        SSR_REQUIRE(p->n_visible >= 0 && p->n_visible <= p->num_splats, "ssr_projection_bwd", "visible count out of range");
+        if (p->n_visible == 0) return 0;
+    }
+    const dim3 grid((unsigned)ceil_div(p->visible_ids ? p->n_visible : p->num_splats, kProjBlock)), block(kProjBlock);
     hipStream_t s = as_stream(stream);
 #define SSR_LAUNCH_BWD(D)                                                                          \
     if (p->accumulate) hipLaunchKernelGGL((projection_bwd_kernel<D, true>), grid, block, 0, s, *p); \

@@ -146,31 +146,27 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
                 const float alpha = eval_alpha_fast(q0, q1, q2.w, px, py, dx, dy, vis, sigma);
                 const bool active = sorted_idx <= bin_final && alpha > kAlphaThreshold;
                 if (__ballot(active) == 0ull) continue;
-                const float opac = q1.y, cr = q1.z, cg = q1.w, cb = q2.x, cdp = q2.y;
-                float t_x = 0.f, t_y = 0.f, t_d = 0.f, t_ca = 0.f, t_cb = 0.f, t_cc = 0.f, t_o = 0.f, t_r = 0.f,
-                      t_g = 0.f, t_b = 0.f;
-                if (active) {
-                    // 1/(1-alpha) by the hardware reciprocal (1 ulp): gradients are compared at 1e-3
-                    const float ra = __builtin_amdgcn_rcpf(1.0f - alpha);
-                    const float T0 = T1 * ra;
-                    const float dotcv = ssr_fma(cdp, vd, ssr_fma(cb, vb, ssr_fma(cg, vg, cr * vr)));
-                    const float v_alpha = T0 * (dotcv - vT1);
-                    const float w = alpha * T0;
-                    const float v_T0 = ssr_fma(alpha, dotcv - vT1, vT1);
-                    if (opac * vis <= 0.999f) {   // sigma >= 0 holds for every active lane
-                        const float v_sigma = (-opac) * vis * v_alpha;
-                        const float vsx = v_sigma * dx, vsy = v_sigma * dy;
-                        t_ca = 0.5f * vsx * dx;
-                        t_cb = vsx * dy;
-                        t_cc = 0.5f * vsy * dy;
-                        // conic.x = 2 * (0.5 conic.x), conic.z likewise
-                        t_x = ssr_fma(q0.z + q0.z, vsx, q0.w * vsy);
-                        t_y = ssr_fma(q0.w, vsx, (q1.x + q1.x) * vsy);
-                        t_o = vis * v_alpha;
-                    }
-                    t_r = vr * w; t_g = vg * w; t_b = vb * w; t_d = vd * w;
-                    T1 = T0; vT1 = v_T0;
-                }
+                // Branch-free per-lane terms: an inactive lane runs with alpha = 0 and v_alpha = 0, which
+                // leaves its T and v_T unchanged (T/(1-0) = T, v_T + 0*(..) = v_T) and makes every term zero.
+                const float cr = q1.z, cg = q1.w, cb = q2.x, cdp = q2.y;
+                const float a = active ? alpha : 0.0f;
+                // 1/(1-alpha) by the hardware reciprocal (1 ulp): gradients are compared at 1e-3
+                const float T0 = T1 * __builtin_amdgcn_rcpf(1.0f - a);
+                const float dv = ssr_fma(cdp, vd, ssr_fma(cb, vb, ssr_fma(cg, vg, cr * vr))) - vT1;
+                const float w = a * T0;
+                const float ov = q1.y * vis;
+                // evaluate_alpha_vjp gate (src/primitives/Primitive3DGS.cuh:273); sigma >= 0 holds when active
+                const float v_alpha = (active && ov <= 0.999f) ? T0 * dv : 0.0f;
+                vT1 = ssr_fma(a, dv, vT1);
+                T1 = T0;
+                const float v_sigma = (-ov) * v_alpha;
+                const float vsx = v_sigma * dx, vsy = v_sigma * dy;
+                const float t_ca = (0.5f * vsx) * dx, t_cb = vsx * dy, t_cc = (0.5f * vsy) * dy;
+                // conic.x = 2 * (0.5 conic.x), conic.z likewise
+                const float t_x = ssr_fma(q0.z + q0.z, vsx, q0.w * vsy);
+                const float t_y = ssr_fma(q0.w, vsx, (q1.x + q1.x) * vsy);
+                const float t_o = vis * v_alpha;
+                const float t_r = vr * w, t_g = vg * w, t_b = vb * w, t_d = vd * w;
                 // transposing reduction: 10 channels -> 3 registers with one channel per row
                 const float ra_ = fold32(t_x, t_y), rb_ = fold32(t_d, t_ca), rc_ = fold32(t_cb, t_cc),
                             rd_ = fold32(t_o, t_r), re_ = fold32(t_g, t_b);

@@ -105,9 +105,11 @@ __device__ __forceinline__ float eval_alpha_fast(const float4& q0, const float4&
                                                  float& dx, float& dy, float& vis, float& sigma) {
     dx = q0.x - px; dy = q0.y - py;
     sigma = ssr_fma(q0.z * dx, dx, ssr_fma(q1.x * dy, dy, (q0.w * dx) * dy));
-    vis = exp_neg_small(-sigma);
-    const float alpha = ssr_min(0.999f, q1.y * vis);
-    return (sigma < 0.f || sigma > cut) ? 0.f : alpha;
+    // outside [0, cut] the exponent arithmetic of exp_neg_small is meaningless: force vis = 0 there,
+    // which also makes alpha 0 and keeps every product formed from vis finite
+    const float e = exp_neg_small(-sigma);
+    vis = (sigma < 0.f || sigma > cut) ? 0.f : e;
+    return ssr_min(0.999f, q1.y * vis);
 }
 
 // Workgroup id -> tile id so that each of the 8 XCDs (workgroups are dealt to them round-robin)

@@ -232,9 +232,10 @@ int ssr_event_destroy(ssr_event_t ev) {
     return check_hip(hipEventDestroy(reinterpret_cast<hipEvent_t>(ev)), "ssr_event_destroy");
 }
 
-int ssr_read_i64(const int64_t* device_value, int64_t* host_value, ssr_stream_t stream) {
+int ssr_read_i64(const int64_t* device_value, int64_t* host_value, int count, ssr_stream_t stream) {
     SSR_REQUIRE(device_value && host_value, "ssr_read_i64", "null pointer");
-    int e = check_hip(hipMemcpyAsync(host_value, device_value, sizeof(int64_t), hipMemcpyDeviceToHost, as_stream(stream)),
+    SSR_REQUIRE(count > 0 && count <= 1024, "ssr_read_i64", "count out of range");
+    int e = check_hip(hipMemcpyAsync(host_value, device_value, sizeof(int64_t) * (size_t)count, hipMemcpyDeviceToHost, as_stream(stream)),
                       "ssr_read_i64");
     if (e) return e;
     return check_hip(hipStreamSynchronize(as_stream(stream)), "ssr_read_i64/sync");

@@ -30,9 +30,10 @@ __global__ __launch_bounds__(kTileBlock) void tile_write_kernel(
     int64_t n, const float4* __restrict__ aabb, const float* __restrict__ sort_depth,
     const float2* __restrict__ xy, const float* __restrict__ conic, const float* __restrict__ opac,
     const int64_t* __restrict__ cum, int tile_w, int tile_h, int64_t* __restrict__ isect_ids,
-    int32_t* __restrict__ flatten_ids) {
-    const int64_t g = (int64_t)blockIdx.x * kTileBlock + threadIdx.x;
-    if (g >= n) return;
+    int32_t* __restrict__ flatten_ids, const int32_t* __restrict__ visible_ids) {
+    const int64_t i = (int64_t)blockIdx.x * kTileBlock + threadIdx.x;
+    if (i >= n) return;
+    const int64_t g = visible_ids ? (int64_t)visible_ids[i] : i;
     int64_t cur = g == 0 ? 0 : cum[g - 1];
     const int64_t end = cum[g];
     const float4 a = aabb[g];
@@ -117,7 +118,7 @@ __global__ __launch_bounds__(kScanBlock) void scan_spine_kernel(int64_t* __restr
 
 __global__ __launch_bounds__(kScanBlock) void scan_down_kernel(const int64_t* __restrict__ in, int64_t n,
                                                                const int64_t* __restrict__ block_prefix,
-                                                               int64_t* __restrict__ out) {
+                                                               int64_t* __restrict__ out, int64_t* __restrict__ total_out) {
     __shared__ int64_t lds[4];
     const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
     int64_t v[kScanItems];
@@ -127,7 +128,13 @@ __global__ __launch_bounds__(kScanBlock) void scan_down_kernel(const int64_t* __
     int64_t total;
     int64_t run = block_prefix[blockIdx.x] + block_exclusive_scan(s, total, lds);
 #pragma unroll
-    for (int i = 0; i < kScanItems; i++) { run += v[i]; if (base + i < n) out[base + i] = run; }
+    for (int i = 0; i < kScanItems; i++) {
+        run += v[i];
+        if (base + i < n) {
+            out[base + i] = run;
+            if (total_out && base + i == n - 1) *total_out = run;
+        }
+    }
 }
 
 // ---- K6 ----
@@ -175,8 +182,8 @@ size_t ssr_scan_scratch_bytes(int64_t n) {
     return (size_t)ceil_div(n, kScanTile) * sizeof(int64_t);
 }
 
-int ssr_inclusive_sum_i64(const int64_t* in, int64_t* out, int64_t n, void* scratch, size_t scratch_bytes,
-                          ssr_stream_t stream) {
+int ssr_inclusive_sum_i64(const int64_t* in, int64_t* out, int64_t n, int64_t* total_out, void* scratch,
+                          size_t scratch_bytes, ssr_stream_t stream) {
     SSR_REQUIRE(n >= 0, "ssr_inclusive_sum_i64", "negative count");
     if (n == 0) return 0;
     SSR_REQUIRE(in && out, "ssr_inclusive_sum_i64", "null pointer");
@@ -186,15 +193,19 @@ int ssr_inclusive_sum_i64(const int64_t* in, int64_t* out, int64_t n, void* scra
     hipStream_t s = as_stream(stream);
     hipLaunchKernelGGL(scan_reduce_kernel, dim3((unsigned)nb), dim3(kScanBlock), 0, s, in, n, sums);
     hipLaunchKernelGGL(scan_spine_kernel, dim3(1), dim3(kScanBlock), 0, s, sums, nb);
-    hipLaunchKernelGGL(scan_down_kernel, dim3((unsigned)nb), dim3(kScanBlock), 0, s, in, n, sums, out);
+    hipLaunchKernelGGL(scan_down_kernel, dim3((unsigned)nb), dim3(kScanBlock), 0, s, in, n, sums, out, total_out);
     SSR_CHECK_LAUNCH("ssr_inclusive_sum_i64");
     return 0;
 }
 
 int ssr_tile_write(int64_t n, const float* aabb, const float* sort_depth, const float* xy, const float* conic,
                    const float* opac, const int64_t* cum_tiles, uint32_t width, uint32_t height, int64_t* isect_ids,
-                   int32_t* flatten_ids, ssr_stream_t stream) {
+                   int32_t* flatten_ids, const int32_t* visible_ids, int64_t n_visible, ssr_stream_t stream) {
     SSR_REQUIRE(n >= 0 && n < (int64_t)1 << 31, "ssr_tile_write", "count out of range");
+    if (visible_ids) {
+        SSR_REQUIRE(n_visible >= 0 && n_visible <= n, "ssr_tile_write", "visible count out of range");
+        if (n_visible == 0) return 0;
+    }
     if (n == 0) return 0;
     SSR_REQUIRE(aabb && sort_depth && xy && conic && opac && cum_tiles, "ssr_tile_write", "null pointer");
     SSR_REQUIRE(isect_ids && flatten_ids, "ssr_tile_write", "null output (n_isects == 0 needs no call)");
@@ -202,9 +213,10 @@ int ssr_tile_write(int64_t n, const float* aabb, const float* sort_depth, const 
     SSR_REQUIRE((reinterpret_cast<uintptr_t>(aabb) & 15) == 0 && (reinterpret_cast<uintptr_t>(xy) & 7) == 0,
                 "ssr_tile_write", "aabb must be 16-byte and xy 8-byte aligned");
     const int tw = (int)ceil_div(width, kTile), th = (int)ceil_div(height, kTile);
-    hipLaunchKernelGGL(tile_write_kernel, dim3((unsigned)ceil_div(n, kTileBlock)), dim3(kTileBlock), 0, as_stream(stream),
-                       n, reinterpret_cast<const float4*>(aabb), sort_depth, reinterpret_cast<const float2*>(xy), conic, opac,
-                       cum_tiles, tw, th, isect_ids, flatten_ids);
+    const int64_t work = visible_ids ? n_visible : n;
+    hipLaunchKernelGGL(tile_write_kernel, dim3((unsigned)ceil_div(work, kTileBlock)), dim3(kTileBlock), 0, as_stream(stream),
+                       work, reinterpret_cast<const float4*>(aabb), sort_depth, reinterpret_cast<const float2*>(xy), conic, opac,
+                       cum_tiles, tw, th, isect_ids, flatten_ids, visible_ids);
     SSR_CHECK_LAUNCH("ssr_tile_write");
     return 0;
 }

@@ -20,7 +20,10 @@ ssr_ext::Options g_opts;
 bool g_profile = false;
 ssr_ext::StageTimes g_times;
 int64_t g_n_isects = 0;
+int64_t g_n_visible = -1;
 bool g_counts_fused = false;         // the last projection already produced tile counts
+int64_t* g_counters = nullptr;       // device [n_isects, n_visible], one readback for both
+int32_t* g_visible_ids = nullptr;    // device work list of the last projection (null: off)
 
 struct StageTimer {
     ssr_event_t a = nullptr, b = nullptr;
@@ -173,6 +176,7 @@ Options& options() { return g_opts; }
 void set_stage_profiling(bool on) { g_profile = on; }
 StageTimes last_stage_times() { return g_times; }
 int64_t last_n_isects() { return g_n_isects; }
+int64_t last_n_visible() { return g_n_visible; }
 }  // namespace ssr_ext
 
 // ---------------------------------------------------------------------------------------------
@@ -207,6 +211,15 @@ projection_3dgs_forward(const int64_t num_splats, const int max_sh_degree,
     if (g_opts.fuse_tile_count) {
         p.tiles_per_splat = DevicePool::global().acquire<int64_t>(PoolSlot::IsectTilesPerSplat, (size_t)(C * N));
         g_counts_fused = true;
+    }
+    g_counters = DevicePool::global().acquire<int64_t>(PoolSlot::IsectCounters, 2);
+    g_visible_ids = nullptr;
+    g_n_visible = -1;
+    if (g_opts.visible_list) {
+        g_visible_ids = DevicePool::global().acquire<int32_t>(PoolSlot::ProjVisibleIds, (size_t)(C * N));
+        backend::memset_async(g_counters, 0, 2 * sizeof(int64_t));
+        p.visible_ids = g_visible_ids;
+        p.visible_count = g_counters + 1;
     }
     {
         StageTimer t(&g_times.k1);
@@ -251,9 +264,15 @@ do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, 
         StageTimer t(&g_times.k3);
         const size_t sb = ssr_scan_scratch_bytes(total);
         void* scratch = DevicePool::global().acquire<uint8_t>(PoolSlot::IsectScanScratch, sb);
-        ok(ssr_inclusive_sum_i64(tiles_per_splat.data_ptr(), cum.data_ptr(), total, scratch, sb, nullptr),
+        if (!g_counters) g_counters = DevicePool::global().acquire<int64_t>(PoolSlot::IsectCounters, 2);
+        ok(ssr_inclusive_sum_i64(tiles_per_splat.data_ptr(), cum.data_ptr(), total, g_counters, scratch, sb, nullptr),
            "do_intersect_tile_generic/scan");
-        if (total > 0) ok(ssr_read_i64(cum.data_ptr() + (total - 1), &n_isects, nullptr), "do_intersect_tile_generic/readback");
+        if (total > 0) {
+            int64_t both[2] = {0, 0};
+            ok(ssr_read_i64(g_counters, both, g_visible_ids ? 2 : 1, nullptr), "do_intersect_tile_generic/readback");
+            n_isects = both[0];
+            if (g_visible_ids) g_n_visible = both[1];
+        }
     }
     g_n_isects = n_isects;
     DeviceTensor3D<int32_t> offsets; offsets.resize(PoolSlot::IsectOffsets, I, tile_h, tile_w);
@@ -268,7 +287,8 @@ do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, 
         StageTimer t(&g_times.k4);
         ok(ssr_tile_write(total, aabb.data_ptr(), depths.data_ptr(), proj_xy->data_ptr(), proj_conic->data_ptr(),
                           proj_opac->data_ptr(), cum.data_ptr(), image_width, image_height, ids_a.data_ptr(),
-                          flat_a.data_ptr(), nullptr), "do_intersect_tile_generic/write");
+                          flat_a.data_ptr(), g_visible_ids, g_visible_ids ? g_n_visible : 0, nullptr),
+           "do_intersect_tile_generic/write");
     }
     int selector = 0;
     {
@@ -397,6 +417,7 @@ void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
     p.v_screen = screen_of(v_splats_screen);
     p.v_world = world_of(v_splats_world);
     p.accumulate = g_opts.overwrite_world_grads ? 0 : 1;
+    if (g_visible_ids && g_n_visible >= 0) { p.visible_ids = g_visible_ids; p.n_visible = g_n_visible; }
     StageTimer t(&g_times.k9);
     ok(ssr_projection_bwd(&p, nullptr), "projection_3dgs_backward");
 }

@@ -93,8 +93,13 @@ struct Options {
     // K1 also produces the per-splat tile count, so do_intersect_tile_generic skips its count
     // pass when the projection that produced `aabb` ran with this set.
     bool fuse_tile_count = false;
-    // K9 overwrites every gradient row (zeros for culled splats) instead of atomically adding into
-    // zero-filled buffers; valid for one camera per call, which is all this backend accepts.
+    // K1 also emits the list of visible splats; the key write (K4) and the projection backward (K9)
+    // then run over that list instead of all N splats.
+    bool visible_list = false;
+    // K9 stores gradients instead of atomically adding them; valid for one camera per call, which
+    // is all this backend accepts. Without the visible list every row is overwritten (zeros for
+    // culled splats) and the caller may skip its zero-fill; with the list only visible rows are
+    // stored and the zero-fill is still needed.
     bool overwrite_world_grads = false;
     // int8 codes x per-splat fp16 scale as SH storage (the benchmark's format): sh_value_bits == 8
     // with sh_value_bounds holding the fp16 scales when this is set.
@@ -107,4 +112,5 @@ struct StageTimes { float k1 = 0, k2 = 0, k3 = 0, k4 = 0, k5 = 0, k6 = 0, k7 = 0
 void set_stage_profiling(bool on);
 StageTimes last_stage_times();
 int64_t last_n_isects();
+int64_t last_n_visible();   // -1 when the visible list is off
 }  // namespace ssr_ext

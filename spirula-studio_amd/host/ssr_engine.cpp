@@ -40,7 +40,8 @@ void alloc_grad_buffers() {
     g.means.resize(PoolSlot::GradMeans, n); g.quats.resize(PoolSlot::GradQuats, n);
     g.scales.resize(PoolSlot::GradScales, n); g.opacities.resize(PoolSlot::GradOpacities, n);
     g.features_dc.resize(PoolSlot::GradFeaturesDc, n); g.features_sh.resize(PoolSlot::GradFeaturesSh, n, engine().num_sh);
-    if (!engine().optim.skip_grad_zero && !ssr_ext::options().overwrite_world_grads) {
+    const auto& o = ssr_ext::options();
+    if (!engine().optim.skip_grad_zero && !(o.overwrite_world_grads && !o.visible_list)) {
         g.means.zero(); g.quats.zero(); g.scales.zero(); g.opacities.zero(); g.features_dc.zero(); g.features_sh.zero();
     }
 }
@@ -219,10 +220,12 @@ int ssrh_init(int device) { return guard([&] { if (!backend::device_select(devic
 
 int ssrh_reset(void) { return guard([&] { engine_reset(); }); }
 
-int ssrh_set_options(int fuse_tile_count, int overwrite_world_grads, int sh_int8_f16scale, int stage_profiling) {
+int ssrh_set_options(int fuse_tile_count, int visible_list, int overwrite_world_grads, int sh_int8_f16scale,
+                     int stage_profiling) {
     return guard([&] {
         auto& o = ssr_ext::options();
-        o.fuse_tile_count = fuse_tile_count != 0; o.overwrite_world_grads = overwrite_world_grads != 0;
+        o.fuse_tile_count = fuse_tile_count != 0; o.visible_list = visible_list != 0;
+        o.overwrite_world_grads = overwrite_world_grads != 0;
         o.sh_int8_f16scale = sh_int8_f16scale != 0;
         ssr_ext::set_stage_profiling(stage_profiling != 0);
     });
@@ -300,6 +303,7 @@ int ssrh_cache_pointer(int which, void** ptr, int64_t* count) {
 }
 
 int64_t ssrh_last_n_isects(void) { return ssr_ext::last_n_isects(); }
+int64_t ssrh_last_n_visible(void) { return ssr_ext::last_n_visible(); }
 
 int ssrh_last_stage_times(float* out9) {
     return guard([&] {

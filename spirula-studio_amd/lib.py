@@ -42,7 +42,8 @@ class Camera(C.Structure):
 class ProjectionFwdParams(C.Structure):
     _fields_ = [("num_splats", C.c_int64), ("sh_degree", C.c_int32), ("world", World),
                 ("sh", ShQuant), ("camera", Camera), ("aabb", vp), ("sort_depth", vp),
-                ("radii", vp), ("screen", Screen), ("tiles_per_splat", vp)]
+                ("radii", vp), ("screen", Screen), ("tiles_per_splat", vp), ("visible_ids", vp),
+                ("visible_count", vp)]
 
 
 class RasterFwdParams(C.Structure):
@@ -63,7 +64,8 @@ class RasterBwdParams(C.Structure):
 class ProjectionBwdParams(C.Structure):
     _fields_ = [("num_splats", C.c_int64), ("sh_degree", C.c_int32), ("world", World),
                 ("sh", ShQuant), ("camera", Camera), ("aabb", vp), ("v_screen", Screen),
-                ("v_world", World), ("accumulate", C.c_int32)]
+                ("v_world", World), ("accumulate", C.c_int32), ("visible_ids", vp),
+                ("n_visible", C.c_int64)]
 
 
 # every symbol include/ssr_backend.h declares: (name, restype, argtypes)
@@ -72,9 +74,9 @@ SYMBOLS = {
     "ssr_projection_fwd": (_i32, [C.POINTER(ProjectionFwdParams), vp]),
     "ssr_tile_count": (_i32, [_i64, vp, vp, vp, vp, _u32, _u32, vp, vp]),
     "ssr_scan_scratch_bytes": (_sz, [_i64]),
-    "ssr_inclusive_sum_i64": (_i32, [vp, vp, _i64, vp, _sz, vp]),
-    "ssr_read_i64": (_i32, [vp, C.POINTER(C.c_int64), vp]),
-    "ssr_tile_write": (_i32, [_i64, vp, vp, vp, vp, vp, vp, _u32, _u32, vp, vp, vp]),
+    "ssr_inclusive_sum_i64": (_i32, [vp, vp, _i64, vp, vp, _sz, vp]),
+    "ssr_read_i64": (_i32, [vp, C.POINTER(C.c_int64), _i32, vp]),
+    "ssr_tile_write": (_i32, [_i64, vp, vp, vp, vp, vp, vp, _u32, _u32, vp, vp, vp, _i64, vp]),
     "ssr_sort_scratch_bytes": (_sz, [_i64]),
     "ssr_sort_pairs_u64_i32": (_i32, [vp, vp, vp, vp, _i64, _i32, _i32, C.POINTER(C.c_int), vp, _sz, vp]),
     "ssr_tile_offsets": (_i32, [_i64, vp, _u32, vp, vp]),

@@ -11,8 +11,10 @@ features_sh [N,15,3]; cameras as viewmats [4,4] row-major world->camera and (fx,
 """
 from __future__ import annotations
 
+import ctypes
 import dataclasses
 import math
+import os
 
 import numpy as np
 
@@ -44,12 +46,46 @@ def _u01(seed: int, stream: int, idx: np.ndarray) -> np.ndarray:
     return (h >> np.uint64(11)).astype(np.float64) * (1.0 / 9007199254740992.0)
 
 
+def _native():
+    """The same generators in native code (libssr_host.so), used when that library is built."""
+    global _NATIVE
+    if _NATIVE is None:
+        _NATIVE = False
+        so = os.path.join(os.path.dirname(os.path.abspath(__file__)), "host", "libssr_host.so")
+        hip = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libssr_hip.so")
+        if os.path.exists(so) and os.path.exists(hip):
+            try:
+                ctypes.CDLL(hip, mode=ctypes.RTLD_GLOBAL)
+                h = ctypes.CDLL(so)
+                h.ssrh_rng_uniform.argtypes = [ctypes.c_uint64, ctypes.c_uint64, ctypes.c_int64, ctypes.c_int64,
+                                               ctypes.c_double, ctypes.c_double, ctypes.c_void_p]
+                h.ssrh_rng_normal.argtypes = [ctypes.c_uint64, ctypes.c_uint64, ctypes.c_int64, ctypes.c_double,
+                                              ctypes.c_double, ctypes.c_void_p]
+                _NATIVE = h
+            except OSError:
+                _NATIVE = False
+    return _NATIVE
+
+
+_NATIVE = None
+
+
 def uniform(seed: int, stream: int, n: int, lo: float, hi: float, start: int = 0) -> np.ndarray:
+    h = _native()
+    if h:
+        out = np.empty(n, np.float32)
+        h.ssrh_rng_uniform(seed, stream, start, n, lo, hi, out.ctypes.data)
+        return out
     idx = np.arange(start, start + n, dtype=np.uint64)
     return (lo + (hi - lo) * _u01(seed, stream, idx)).astype(np.float32)
 
 
 def normal(seed: int, stream: int, n: int, mean: float, sigma: float) -> np.ndarray:
+    h = _native()
+    if h:
+        out = np.empty(n, np.float32)
+        h.ssrh_rng_normal(seed, stream, n, mean, sigma, out.ctypes.data)
+        return out
     idx = np.arange(n, dtype=np.uint64)
     pair = idx >> np.uint64(1)
     u1 = 1.0 - _u01(seed, stream, pair * np.uint64(2))

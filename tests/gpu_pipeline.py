@@ -9,7 +9,8 @@ import numpy as np
 
 
 class GpuRun:
-    def __init__(self, pkg, scene, sh_degree=3):
+    def __init__(self, pkg, scene, sh_degree=3, use_list=False):
+        self.use_list = use_list
         self.L = pkg.lib
         self.lib = self.L.load()
         self.check = self.L.check
@@ -37,6 +38,9 @@ class GpuRun:
             self.d[k] = D(shape, np.float32)
         self.d["counts"] = D((n,), np.int64)
         self.d["cum"] = D((n,), np.int64)
+        self.d["vis_ids"] = D((n,), np.int32)
+        self.d["counters"] = D((2,), np.int64)     # [n_isects, n_visible]
+        self.V = None
 
     def ptr(self, k):
         a = self.d.get(k)
@@ -81,6 +85,10 @@ class GpuRun:
         p.aabb, p.sort_depth, p.radii = self.ptr("aabb"), self.ptr("sort_depth"), self.ptr("radii")
         p.screen = self.screen()
         p.tiles_per_splat = self.ptr("counts") if fused_count else None
+        if self.use_list:
+            self.d["counters"].fill_zero()
+            p.visible_ids = self.ptr("vis_ids")
+            p.visible_count = self.d["counters"].ptr + 8
         self.check(self.lib.ssr_projection_fwd(C.byref(p), None))
 
     def tiles(self, fused_count=False):
@@ -91,12 +99,13 @@ class GpuRun:
                                                self.ptr("opac"), sc.width, sc.height, self.ptr("counts"), None))
         sb = self.lib.ssr_scan_scratch_bytes(n)
         self.d["scan_scratch"] = D((max(sb, 8),), np.uint8)
-        self.check(self.lib.ssr_inclusive_sum_i64(self.ptr("counts"), self.ptr("cum"), n,
+        self.check(self.lib.ssr_inclusive_sum_i64(self.ptr("counts"), self.ptr("cum"), n, self.ptr("counters"),
                                                   self.ptr("scan_scratch"), sb, None))
-        k = C.c_int64(0)
+        k = (C.c_int64 * 2)(0, 0)
         if n:
-            self.check(self.lib.ssr_read_i64(self.d["cum"].ptr + 8 * (n - 1), C.byref(k), None))
-        self.K = K = int(k.value)
+            self.check(self.lib.ssr_read_i64(self.ptr("counters"), k, 2, None))
+        self.K = K = int(k[0])
+        self.V = int(k[1]) if self.use_list else None
         n_tiles = sc.tile_w * sc.tile_h
         self.d["offsets"] = D((n_tiles,), np.int32)
         for nm in ["keys_a", "keys_b"]:
@@ -107,7 +116,9 @@ class GpuRun:
         if K:
             self.check(self.lib.ssr_tile_write(n, self.ptr("aabb"), self.ptr("sort_depth"), self.ptr("xy"),
                                                self.ptr("conic"), self.ptr("opac"), self.ptr("cum"), sc.width,
-                                               sc.height, self.ptr("keys_a"), self.ptr("vals_a"), None))
+                                               sc.height, self.ptr("keys_a"), self.ptr("vals_a"),
+                                               self.ptr("vis_ids") if self.use_list else None,
+                                               self.V if self.use_list else 0, None))
             self.unsorted_keys = self.d["keys_a"].to_host()
             self.unsorted_vals = self.d["vals_a"].to_host()
             sb = self.lib.ssr_sort_scratch_bytes(K)
@@ -171,6 +182,8 @@ class GpuRun:
         p.world, p.sh, p.camera = self.world(), self.shq(), self.camera()
         p.aabb, p.v_screen, p.v_world = self.ptr("aabb"), self.screen("v_"), self.world("w_")
         p.accumulate = 1 if accumulate else 0
+        if self.use_list:
+            p.visible_ids, p.n_visible = self.ptr("vis_ids"), self.V
         self.check(self.lib.ssr_projection_bwd(C.byref(p), None))
 
     def run_all(self, backward=True, fused_count=False):

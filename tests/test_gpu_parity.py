@@ -29,10 +29,13 @@ def _grad_close(got, ref, abs_scale, name):
                            got[bad][:4], ref[bad][:4])
 
 
-def _compare(gpu, oracle, sc, label, fused_count=False):
+def _compare(gpu, oracle, sc, label, fused_count=False, use_list=False):
     r = oracle.pipeline(sc)
     print(f"[{label}] N={sc.n} {sc.width}x{sc.height} visible={r['proj']['visible']} K={r['isect_ids'].size}", flush=True)
-    g = GpuRun(gpu, sc).run_all(fused_count=fused_count)
+    g = GpuRun(gpu, sc, use_list=use_list).run_all(fused_count=fused_count)
+    if use_list:
+        assert g.V == r['proj']['visible']
+        assert np.array_equal(np.sort(g.host('vis_ids')[:g.V]), np.nonzero(r['proj']['aabb'][:, 2] > r['proj']['aabb'][:, 0])[0])
     vis = r["proj"]["aabb"][:, 2] > r["proj"]["aabb"][:, 0]
     # K1: bit-exact on every compared array (culled screen rows are not written by either side)
     p = g.proj_host()
@@ -101,6 +104,13 @@ def test_tiny_pinhole(gpu, oracle):
 
 def test_tiny_fused_count(gpu, oracle):
     _compare(gpu, oracle, gpu.scenes.tiny_scene(n=500, width=64, height=64, seed=5), "tiny-fused", fused_count=True)
+
+
+def test_visible_work_list(gpu, oracle):
+    """K4 and K9 driven by the list of visible splats that K1 emits: same keys, same gradients."""
+    sc = gpu.scenes.make_scene(4, n=60000, width=480, height=270, sh_codec=0)   # mostly culled
+    _compare(gpu, oracle, sc, "cfg4-list", fused_count=True, use_list=True)
+    _compare(gpu, oracle, gpu.scenes.tiny_scene(n=700, width=96, height=64, seed=8), "tiny-list", use_list=True)
 
 
 def test_tiny_equirect(gpu, oracle):
