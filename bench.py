@@ -121,7 +121,7 @@ def main():
     sc = pkg.scenes.make_scene(cfg, n=args.n)
     t_gen = time.time() - t_gen
     native = not args.reference_order
-    eng = host.Engine(sc, fuse_tile_count=native, visible_list=native, overwrite_world_grads=native)
+    eng = host.Engine(sc, fuse_tile_count=native, visible_list=native, packed_rows=native, overwrite_world_grads=native)
     L = lib.load()
 
     eng.time_iterations(max(args.warmup, 1))
@@ -176,7 +176,7 @@ def main():
                                f"{'pinhole' if sc.camera_model == 0 else 'equirectangular'}, SH3 "
                                f"{['fp32', 'ref-q8', 'ref-q16', 'int8*fp16scale'][sc.sh_codec]}, tile 16x16, seed {pkg.scenes.CONFIGS[cfg]['seed']:#x}",
                    "visible": V, "n_isects": K, "K_b": K_b, "tiles": T, "pixels": P,
-                   "stage_order": "fused tile count, visible-splat work list, plain-store gradients" if native else "reference order",
+                   "stage_order": "fused tile count, visible-splat work list, packed fragment rows, plain-store gradients" if native else "reference order",
                    "device_ms_per_iter_median": float(np.median(ms))},
         "hbm_roofline_frac_whole_iteration": total_bytes / (float(np.median(ms)) * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "algorithmic_bytes_per_iter": total_bytes,

@@ -103,6 +103,11 @@ typedef struct {
      * (which the caller zeroes). Later stages can then run over V entries instead of N. */
     int32_t* visible_ids;     /* optional [C*N] */
     int64_t* visible_count;   /* required when visible_ids is given */
+    /* Optional second copy of the visible screen rows as one 48-byte record per splat,
+     * (x, y, conic.x/2, conic.y | conic.z/2, opac, r, g | b, depth, sigma cut, footprint scale),
+     * 16-byte aligned, [C*N,12]. The compositing kernels gather a splat from it with one or two
+     * cache lines instead of five (same values, so same results). */
+    float* packed_rows;
 } ssr_projection_fwd_params;
 int ssr_projection_fwd(const ssr_projection_fwd_params* p, ssr_stream_t stream);
 
@@ -152,6 +157,8 @@ typedef struct {
     float* render_depth;    /* [H,W] */
     float* render_T;        /* [H,W] */
     int32_t* last_ids;      /* [H,W] */
+    const float* packed_rows; /* optional: rows written by ssr_projection_fwd for this screen;
+                                 when given, `screen` is not read */
 } ssr_raster_fwd_params;
 int ssr_raster_fwd(const ssr_raster_fwd_params* p, ssr_stream_t stream);
 
@@ -173,6 +180,7 @@ typedef struct {
     const float* v_render_depth;  /* [H,W] */
     const float* v_render_T;      /* [H,W] */
     ssr_screen v_screen;          /* accumulated into */
+    const float* packed_rows;     /* optional, as in ssr_raster_fwd_params */
 } ssr_raster_bwd_params;
 int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t stream);
 

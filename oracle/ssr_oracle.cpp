@@ -630,8 +630,8 @@ void or_raster_fwd(int64_t N, const float* xy, const float* depth, const float* 
     (void)N;
     const int tw = (int)((width + kTile - 1) / kTile), th = (int)((height + kTile - 1) / kTile);
     const int n_tiles = tw * th;
-    int64_t kf = 0, kb = 0;
-#pragma omp parallel for schedule(dynamic, 4) reduction(+ : kf, kb)
+    int64_t kf = 0, kb = 0, vis_f = 0, vis_b = 0, prod_b = 0;
+#pragma omp parallel for schedule(dynamic, 4) reduction(+ : kf, kb, vis_f, vis_b, prod_b)
     for (int tile = 0; tile < n_tiles; tile++) {
         const int ty = tile / tw, tx = tile % tw;
         const int32_t start = tile_offsets[tile];
@@ -650,6 +650,8 @@ void or_raster_fwd(int64_t N, const float* xy, const float* depth, const float* 
         }
         int32_t max_eval = start - 1, max_last = start - 1;
         bool any_pixel = false;
+        int32_t mt_eval[4] = {start - 1, start - 1, start - 1, start - 1}, mt_last[4] = {-1, -1, -1, -1};
+        std::vector<uint8_t> used(frags.size(), 0);   // bit m: some pixel of sub-tile m composited it
         for (int py_ = 0; py_ < kTile; py_++) {
             for (int px_ = 0; px_ < kTile; px_++) {
                 const uint32_t i = ty * kTile + py_, j = tx * kTile + px_;
@@ -674,6 +676,7 @@ void or_raster_fwd(int64_t N, const float* xy, const float* depth, const float* 
                         cd = ssr_fma(f.d, w, cd);
                         cur_idx = (uint32_t)k;
                         T = next_T;
+                        used[k - start] |= (uint8_t)(1u << mt);
                     } else {
                         break;   // done: the crossing splat is not added
                     }
@@ -687,14 +690,25 @@ void or_raster_fwd(int64_t N, const float* xy, const float* depth, const float* 
                 out_last_ids[pid] = (int32_t)cur_idx;
                 max_eval = std::max(max_eval, last_eval);
                 max_last = std::max(max_last, (int32_t)cur_idx);
+                mt_eval[mt] = std::max(mt_eval[mt], last_eval);
+                mt_last[mt] = std::max(mt_last[mt], (int32_t)cur_idx);
             }
         }
+        for (int32_t k = start; k < end; k++)
+            for (int mt = 0; mt < 4; mt++) {
+                if (!((hits[k - start] >> mt) & 1)) continue;
+                if (k <= mt_eval[mt]) vis_f++;
+                if (k <= mt_last[mt]) vis_b++;
+                if ((used[k - start] >> mt) & 1) prod_b++;
+            }
         if (any_pixel && end > start) {
             kf += std::max(0, max_eval - start + 1);
             kb += std::max(0, std::min(max_last, end - 1) - start + 1);
         }
     }
-    if (stats) { stats[0] = kf; stats[1] = kb; }
+    // [2..4]: (splat, 8x8 sub-tile) visits of the forward, of the backward, and those of the
+    // backward in which at least one pixel composited the splat
+    if (stats) { stats[0] = kf; stats[1] = kb; stats[2] = vis_f; stats[3] = vis_b; stats[4] = prod_b; }
 }
 
 // rasterize_to_pixels_bwd_kernel (IS_EVAL3D=0, dist_type=None, no median, no accum weights),

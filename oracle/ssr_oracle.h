@@ -63,7 +63,9 @@ void or_sort_pairs(int64_t n, const int64_t* keys_in, const int32_t* vals_in, in
 void or_tile_offsets(int64_t n_isects, const int64_t* sorted_ids, uint32_t n_tiles,
     int32_t* offsets);
 
-/* K7. stats (optional, 2 entries): K_f and K_b as defined for the bandwidth model. */
+/* K7. stats (optional, 5 entries): K_f and K_b as defined for the bandwidth model, then the
+ * number of (splat, 8x8 sub-tile) visits of the forward, of the backward, and of the backward
+ * visits in which some pixel composited the splat. */
 void or_raster_fwd(int64_t N, const float* xy, const float* depth, const float* conic,
     const float* opac, const float* rgb, uint32_t width, uint32_t height,
     const int32_t* tile_offsets, const int32_t* flatten_ids, int64_t n_isects,

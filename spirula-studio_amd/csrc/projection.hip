@@ -12,6 +12,7 @@
 // One thread per Gaussian, 256 threads (4 wavefronts) per workgroup. Both kernels are bound by
 // HBM traffic (236 B in, 60 B out per visible splat forward; 472 B in/out backward).
 #include "projection_device.h"
+#include "raster_device.h"
 
 namespace ssr {
 
@@ -75,6 +76,15 @@ __global__ __launch_bounds__(kProjBlock) void projection_fwd_kernel(ssr_projecti
                 tile_geom(bb, p.xy, p.conic, p.opac, tw, th, tg);
                 P.tiles_per_splat[g] = count_tiles(tg);
             }
+            if (P.packed_rows) {   // geometry part of the row; phase 2 adds the colour
+                float cut, kk;
+                fragment_constants(p.opac, cut, kk);
+                float4* row = reinterpret_cast<float4*>(P.packed_rows) + 3 * g;
+                row[0] = make_float4(p.xy[0], p.xy[1], 0.5f * p.conic[0], p.conic[1]);
+                *reinterpret_cast<float2*>(&row[1]) = make_float2(0.5f * p.conic[2], p.opac);
+                float* r2 = reinterpret_cast<float*>(&row[2]);
+                r2[1] = p.depth; r2[2] = cut; r2[3] = kk;
+            }
             s_list[atomicAdd(&s_count, 1)] = threadIdx.x;
         } else {
             aabb_out[g] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -106,8 +116,14 @@ __global__ __launch_bounds__(kProjBlock) void projection_fwd_kernel(ssr_projecti
     float raw[3];
     sh_color_raw<kDegree>(b, dc, coef, raw);
     float* rg = P.screen.rgb + 3 * v;
+    float col[3];
 #pragma unroll
-    for (int c = 0; c < 3; c++) rg[c] = ssr_max(raw[c] + 0.5f, 0.0f);
+    for (int c = 0; c < 3; c++) { col[c] = ssr_max(raw[c] + 0.5f, 0.0f); rg[c] = col[c]; }
+    if (P.packed_rows) {
+        float* row = P.packed_rows + kPackedRowFloats * v;
+        *reinterpret_cast<float2*>(row + 6) = make_float2(col[0], col[1]);
+        row[8] = col[2];
+    }
 }
 
 __device__ __forceinline__ float fin(float v) { return ssr_isfinite(v) ? v : 0.0f; }
@@ -403,6 +419,7 @@ extern "C" int ssr_projection_fwd(const ssr_projection_fwd_params* p, ssr_stream
                 "ssr_projection_fwd", "aabb and quats must be 16-byte aligned");
     SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->screen.xy) & 7) == 0, "ssr_projection_fwd", "screen.xy must be 8-byte aligned");
     SSR_REQUIRE(!p->visible_ids || p->visible_count, "ssr_projection_fwd", "visible_ids needs visible_count");
+    SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->packed_rows) & 15) == 0, "ssr_projection_fwd", "packed_rows must be 16-byte aligned");
     const dim3 grid((unsigned)ceil_div(p->num_splats, kProjBlock)), block(kProjBlock);
     hipStream_t s = as_stream(stream);
     switch (p->sh_degree) {

@@ -125,7 +125,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
         if (idx >= range_start) {
             const int32_t g = P.flatten_ids[idx];
             s_ids[tid] = g;
-            frags[tid] = stage_fragment(P.screen, g, tile_x0, tile_y0);
+            frags[tid] = stage_fragment(P.screen, P.packed_rows, g, tile_x0, tile_y0);
         } else {
             frags[tid].q2 = make_float4(0.f, 0.f, 0.f, 0.f);
         }
@@ -193,11 +193,15 @@ extern "C" int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t strea
     SSR_REQUIRE(p->tile_offsets && p->flatten_ids, "ssr_raster_bwd", "null tile data");
     SSR_REQUIRE(p->render_T && p->last_ids && p->render_depth, "ssr_raster_bwd", "null forward output");
     SSR_REQUIRE(p->v_render_rgb && p->v_render_depth && p->v_render_T, "ssr_raster_bwd", "null output gradient");
-    SSR_REQUIRE(p->screen.xy && p->screen.depth && p->screen.conic && p->screen.opac && p->screen.rgb,
-                "ssr_raster_bwd", "null screen buffer");
+    if (p->packed_rows) {
+        SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->packed_rows) & 15) == 0, "ssr_raster_bwd", "packed_rows must be 16-byte aligned");
+    } else {
+        SSR_REQUIRE(p->screen.xy && p->screen.depth && p->screen.conic && p->screen.opac && p->screen.rgb,
+                    "ssr_raster_bwd", "null screen buffer");
+        SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->screen.xy) & 7) == 0, "ssr_raster_bwd", "screen.xy must be 8-byte aligned");
+    }
     SSR_REQUIRE(p->v_screen.xy && p->v_screen.depth && p->v_screen.conic && p->v_screen.opac && p->v_screen.rgb,
                 "ssr_raster_bwd", "null v_screen buffer");
-    SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->screen.xy) & 7) == 0, "ssr_raster_bwd", "screen.xy must be 8-byte aligned");
     const int tw = (int)ceil_div(p->width, kTile), th = (int)ceil_div(p->height, kTile);
     hipLaunchKernelGGL(raster_bwd_kernel, dim3((unsigned)xcd_grid_size(tw * th)), dim3(kRasterBlock), 0, as_stream(stream),
                        *p, tw, th);

@@ -40,31 +40,59 @@ __device__ __forceinline__ bool ellipse_box_overlap(const float ic[3], float x0,
     return ssr_min(mc, ssr_min(mx, my) - 1.0f) < 0.f;
 }
 
-// Gathers splat `g` from the screen buffers and computes its sub-tile footprint mask.
-__device__ __forceinline__ FragLds stage_fragment(const ssr_screen& s, int32_t g, float tile_x0, float tile_y0) {
-    const float2 xy = *reinterpret_cast<const float2*>(s.xy + 2 * (int64_t)g);
-    const float* cn = s.conic + 3 * (int64_t)g;
-    const float cx = cn[0], cy = cn[1], cz = cn[2];
-    const float opac = s.opac[g];
-    const float* rg = s.rgb + 3 * (int64_t)g;
-    uint32_t hits = 0;
+// Per-splat values that do not depend on the tile: the sigma cut (above it alpha <= 1/255 for
+// certain: ln(255 opac) plus a margin far larger than the rounding of log/exp, so no lane is
+// skipped that the reference would keep) and the conic scale of the footprint ellipse.
+__device__ __forceinline__ void fragment_constants(float opac, float& cut, float& kk) {
+    cut = 0.0f; kk = 0.0f;
     if (opac > kAlphaThreshold) {
-        const float kk = 0.5f / ssr_log(opac / kAlphaThreshold);
-        const float ic[3] = {cx * kk, cy * kk, cz * kk};
+        const float lg = ssr_log(opac / kAlphaThreshold);
+        // exp_neg_small() is exact down to -87; only a caller-supplied opac beyond e^80 exceeds that
+        cut = ssr_min(lg + 1e-3f, 80.0f);
+        kk = 0.5f / lg;
+    }
+}
+
+// A fragment row as K1 can lay it out in HBM: 48 contiguous bytes per splat,
+//   (x, y, 0.5 conic.x, conic.y | 0.5 conic.z, opac, r, g | b, depth, sigma cut, footprint scale),
+// one or two cache lines per gather instead of five.
+constexpr int kPackedRowFloats = 12;
+
+// Brings splat `g` into the staged form and computes its sub-tile footprint mask, either from a
+// packed row or by gathering the five screen arrays.
+__device__ __forceinline__ FragLds stage_fragment(const ssr_screen& s, const float* __restrict__ packed, int32_t g,
+                                                  float tile_x0, float tile_y0) {
+    FragLds f;
+    float cut, kk;
+    if (packed) {
+        const float4* row = reinterpret_cast<const float4*>(packed) + 3 * (int64_t)g;
+        f.q0 = row[0]; f.q1 = row[1];
+        const float4 r2 = row[2];
+        f.q2 = make_float4(r2.x, r2.y, 0.0f, r2.z);
+        cut = r2.z; kk = r2.w;
+    } else {
+        const float2 xy = *reinterpret_cast<const float2*>(s.xy + 2 * (int64_t)g);
+        const float* cn = s.conic + 3 * (int64_t)g;
+        const float opac = s.opac[g];
+        const float* rg = s.rgb + 3 * (int64_t)g;
+        fragment_constants(opac, cut, kk);
+        f.q0 = make_float4(xy.x, xy.y, 0.5f * cn[0], cn[1]);
+        f.q1 = make_float4(0.5f * cn[2], opac, rg[0], rg[1]);
+        f.q2 = make_float4(rg[2], s.depth[g], 0.0f, cut);
+    }
+    uint32_t hits = 0;
+    if (f.q1.y > kAlphaThreshold) {
+        // conic.x = 2 * (0.5 conic.x) exactly, conic.z likewise
+        const float ic[3] = {(f.q0.z + f.q0.z) * kk, f.q0.w * kk, (f.q1.x + f.q1.x) * kk};
+        const float x = f.q0.x, y = f.q0.y;
 #pragma unroll
         for (int m = 0; m < 4; m++) {
             const float bx0 = tile_x0 + (float)((m & 1) * kMicro), by0 = tile_y0 + (float)((m >> 1) * kMicro);
-            if (ellipse_box_overlap(ic, bx0 - xy.x, (bx0 + (float)kMicro) - xy.x, by0 - xy.y, (by0 + (float)kMicro) - xy.y))
+            if (ellipse_box_overlap(ic, bx0 - x, (bx0 + (float)kMicro) - x, by0 - y, (by0 + (float)kMicro) - y))
                 hits |= 1u << m;
         }
     }
-    FragLds f;
-    f.q0 = make_float4(xy.x, xy.y, 0.5f * cx, cy);
-    f.q1 = make_float4(0.5f * cz, opac, rg[0], rg[1]);
-    // sigma above which alpha <= 1/255 for certain: exp(-5.55) = 0.003888 < 1/255 = 0.003922 and
-    // opac <= 1 for anything the projection produced; a caller-supplied opac > 1 disables the cut.
-    const float cut = opac <= 1.0f ? 5.55f : __uint_as_float(0x7f800000u);
-    f.q2 = make_float4(rg[2], s.depth[g], __uint_as_float(hits), cut);
+    f.q2.z = __uint_as_float(hits);
     return f;
 }
 
@@ -79,9 +107,9 @@ __device__ __forceinline__ float eval_alpha(const float4& q0, const float4& q1, 
     return sigma < 0.f ? 0.f : alpha;
 }
 
-// exp(x) for x in [-5.55, 0] (and NaN): the same operations as ssr_exp() on that range, where its
-// overflow / underflow branches are dead and 2^k (k in [-9, 0]) can be applied by adding k to the
-// exponent field -- exact, so the bits equal ssr_exp(x).
+// exp(x) for x in [-87, 0] (and NaN): the same operations as ssr_exp() on that range, where its
+// overflow / underflow branches are dead and 2^k (k in [-126, 0], result normal) can be applied by
+// adding k to the exponent field -- exact, so the bits equal ssr_exp(x).
 __device__ __forceinline__ float exp_neg_small(float x) {
     const float k = ssr_rint(x * 1.44269504088896341f);
     float r = ssr_fma(k, -0.693359375f, x);
@@ -101,6 +129,15 @@ __device__ __forceinline__ float exp_neg_small(float x) {
 
 // eval_alpha() without the transcendental's range handling: identical results wherever
 // alpha > 1/255 can hold (0 <= sigma <= cut), and alpha = 0 -- the skipped case -- elsewhere.
+__device__ __forceinline__ float eval_sigma(const float4& q0, const float4& q1, float px, float py, float& dx, float& dy) {
+    dx = q0.x - px; dy = q0.y - py;
+    return ssr_fma(q0.z * dx, dx, ssr_fma(q1.x * dy, dy, (q0.w * dx) * dy));
+}
+__device__ __forceinline__ float alpha_of_sigma(const float4& q1, float cut, float sigma, float& vis) {
+    const float e = exp_neg_small(-sigma);
+    vis = (sigma < 0.f || sigma > cut) ? 0.f : e;
+    return ssr_min(0.999f, q1.y * vis);
+}
 __device__ __forceinline__ float eval_alpha_fast(const float4& q0, const float4& q1, float cut, float px, float py,
                                                  float& dx, float& dy, float& vis, float& sigma) {
     dx = q0.x - px; dy = q0.y - py;

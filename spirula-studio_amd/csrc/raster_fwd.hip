@@ -35,7 +35,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_kernel(ssr_raster_fwd
         if (__syncthreads_count(done) >= kRasterBlock) break;
         const int32_t idx = batch_start + tid;
         if (idx < range_end) {
-            frags[tid] = stage_fragment(P.screen, P.flatten_ids[idx], tile_x0, tile_y0);
+            frags[tid] = stage_fragment(P.screen, P.packed_rows, P.flatten_ids[idx], tile_x0, tile_y0);
         } else {
             frags[tid].q2 = make_float4(0.f, 0.f, 0.f, 0.f);   // empty footprint mask
         }
@@ -90,9 +90,13 @@ extern "C" int ssr_raster_fwd(const ssr_raster_fwd_params* p, ssr_stream_t strea
     SSR_REQUIRE(p->tile_offsets, "ssr_raster_fwd", "null tile offsets");
     if (p->n_isects > 0) {
         SSR_REQUIRE(p->flatten_ids, "ssr_raster_fwd", "null flatten_ids");
-        SSR_REQUIRE(p->screen.xy && p->screen.depth && p->screen.conic && p->screen.opac && p->screen.rgb,
-                    "ssr_raster_fwd", "null screen buffer");
-        SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->screen.xy) & 7) == 0, "ssr_raster_fwd", "screen.xy must be 8-byte aligned");
+        if (p->packed_rows) {
+            SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->packed_rows) & 15) == 0, "ssr_raster_fwd", "packed_rows must be 16-byte aligned");
+        } else {
+            SSR_REQUIRE(p->screen.xy && p->screen.depth && p->screen.conic && p->screen.opac && p->screen.rgb,
+                        "ssr_raster_fwd", "null screen buffer");
+            SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->screen.xy) & 7) == 0, "ssr_raster_fwd", "screen.xy must be 8-byte aligned");
+        }
     }
     const int tw = (int)ceil_div(p->width, kTile), th = (int)ceil_div(p->height, kTile);
     hipLaunchKernelGGL(raster_fwd_kernel, dim3((unsigned)xcd_grid_size(tw * th)), dim3(kRasterBlock), 0, as_stream(stream),

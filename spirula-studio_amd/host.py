@@ -18,7 +18,7 @@ SYMBOLS = {
     "ssrh_last_error": (C.c_char_p, []),
     "ssrh_init": (C.c_int, [C.c_int]),
     "ssrh_reset": (C.c_int, []),
-    "ssrh_set_options": (C.c_int, [C.c_int] * 5),
+    "ssrh_set_options": (C.c_int, [C.c_int] * 6),
     "ssrh_set_data_3dgs": (C.c_int, [C.c_int64, vp, vp, vp, vp, vp, vp, C.c_int]),
     "ssrh_set_sh_value_quant": (C.c_int, [C.c_int, vp, C.c_int64, C.c_int, vp, C.c_int64, C.c_int, C.c_int64]),
     "ssrh_set_camera_params": (C.c_int, [C.c_int, C.c_int, C.c_char_p, C.c_char_p, vp, vp, C.c_int]),
@@ -68,14 +68,15 @@ CACHE = dict(aabb=(0, np.float32), sort_depth=(1, np.float32), xy=(2, np.float32
 class Engine:
     """Drives the engine harness for one scene: upload once, then forward / backward."""
 
-    def __init__(self, scene, device=0, fuse_tile_count=True, visible_list=True, overwrite_world_grads=True,
+    def __init__(self, scene, device=0, fuse_tile_count=True, visible_list=True, packed_rows=True, overwrite_world_grads=True,
                  stage_profiling=False, sh_degree=3):
         self.h = load()
         self.sc = scene
         self.sh_degree = sh_degree
         check(self.h.ssrh_init(device))
         check(self.h.ssrh_reset())
-        self.opts = [int(fuse_tile_count), int(visible_list), int(overwrite_world_grads), int(scene.sh_codec == 3)]
+        self.opts = [int(fuse_tile_count), int(visible_list), int(packed_rows), int(overwrite_world_grads),
+                     int(scene.sh_codec == 3)]
         check(self.h.ssrh_set_options(*self.opts, int(stage_profiling)))
         f32 = lambda a: np.ascontiguousarray(a, np.float32)
         self._keep = [f32(scene.means), f32(scene.quats), f32(scene.log_scales), f32(scene.opacity_logits),

@@ -24,6 +24,8 @@ int64_t g_n_visible = -1;
 bool g_counts_fused = false;         // the last projection already produced tile counts
 int64_t* g_counters = nullptr;       // device [n_isects, n_visible], one readback for both
 int32_t* g_visible_ids = nullptr;    // device work list of the last projection (null: off)
+float* g_packed_rows = nullptr;      // packed screen rows of the last projection (null: off)
+const float* g_packed_for_xy = nullptr;   // the screen.xy buffer those rows mirror
 
 struct StageTimer {
     ssr_event_t a = nullptr, b = nullptr;
@@ -221,6 +223,13 @@ projection_3dgs_forward(const int64_t num_splats, const int max_sh_degree,
         p.visible_ids = g_visible_ids;
         p.visible_count = g_counters + 1;
     }
+    g_packed_rows = nullptr;
+    g_packed_for_xy = nullptr;
+    if (g_opts.packed_rows) {
+        g_packed_rows = DevicePool::global().acquire<float>(PoolSlot::ProjPackedRows, (size_t)(C * N * 12));
+        g_packed_for_xy = xy;
+        p.packed_rows = g_packed_rows;
+    }
     {
         StageTimer t(&g_times.k1);
         ok(ssr_projection_fwd(&p, nullptr), "projection_3dgs_forward");
@@ -331,6 +340,7 @@ rasterize_to_pixels_3dgs_fwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     p.tile_offsets = tile_offsets.data_ptr(); p.flatten_ids = flatten_ids.data_ptr(); p.n_isects = flatten_ids.size();
     p.render_rgb = (float*)std::get<0>(renders).data_ptr(); p.render_depth = std::get<1>(renders).data_ptr();
     p.render_T = Ts.data_ptr(); p.last_ids = last.data_ptr();
+    if (g_packed_rows && p.screen.xy == g_packed_for_xy) p.packed_rows = g_packed_rows;
     {
         StageTimer t(&g_times.k7);
         ok(ssr_raster_fwd(&p, nullptr), "rasterize_to_pixels_3dgs_fwd");
@@ -381,6 +391,7 @@ rasterize_to_pixels_3dgs_bwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     p.v_render_depth = std::get<1>(v_render_outputs).data_ptr();
     p.v_render_T = v_render_Ts.data_ptr();
     p.v_screen = screen_of(vs);
+    if (g_packed_rows && p.screen.xy == g_packed_for_xy) p.packed_rows = g_packed_rows;
     {
         StageTimer t(&g_times.k8);
         ok(ssr_raster_bwd(&p, nullptr), "rasterize_to_pixels_3dgs_bwd");

@@ -96,6 +96,9 @@ struct Options {
     // K1 also emits the list of visible splats; the key write (K4) and the projection backward (K9)
     // then run over that list instead of all N splats.
     bool visible_list = false;
+    // K1 also writes each visible screen row as one 48-byte record; the compositing kernels gather
+    // from it when they are handed the screen buffers of that same projection.
+    bool packed_rows = false;
     // K9 stores gradients instead of atomically adding them; valid for one camera per call, which
     // is all this backend accepts. Without the visible list every row is overwritten (zeros for
     // culled splats) and the caller may skip its zero-fill; with the list only visible rows are

@@ -43,14 +43,14 @@ class ProjectionFwdParams(C.Structure):
     _fields_ = [("num_splats", C.c_int64), ("sh_degree", C.c_int32), ("world", World),
                 ("sh", ShQuant), ("camera", Camera), ("aabb", vp), ("sort_depth", vp),
                 ("radii", vp), ("screen", Screen), ("tiles_per_splat", vp), ("visible_ids", vp),
-                ("visible_count", vp)]
+                ("visible_count", vp), ("packed_rows", vp)]
 
 
 class RasterFwdParams(C.Structure):
     _fields_ = [("num_splats", C.c_int64), ("screen", Screen), ("width", C.c_uint32),
                 ("height", C.c_uint32), ("tile_offsets", vp), ("flatten_ids", vp),
                 ("n_isects", C.c_int64), ("render_rgb", vp), ("render_depth", vp),
-                ("render_T", vp), ("last_ids", vp)]
+                ("render_T", vp), ("last_ids", vp), ("packed_rows", vp)]
 
 
 class RasterBwdParams(C.Structure):
@@ -58,7 +58,7 @@ class RasterBwdParams(C.Structure):
                 ("height", C.c_uint32), ("tile_offsets", vp), ("flatten_ids", vp),
                 ("n_isects", C.c_int64), ("render_T", vp), ("last_ids", vp), ("render_depth", vp),
                 ("v_render_rgb", vp), ("v_render_depth", vp), ("v_render_T", vp),
-                ("v_screen", Screen)]
+                ("v_screen", Screen), ("packed_rows", vp)]
 
 
 class ProjectionBwdParams(C.Structure):

@@ -9,8 +9,9 @@ import numpy as np
 
 
 class GpuRun:
-    def __init__(self, pkg, scene, sh_degree=3, use_list=False):
+    def __init__(self, pkg, scene, sh_degree=3, use_list=False, use_packed=False):
         self.use_list = use_list
+        self.use_packed = use_packed
         self.L = pkg.lib
         self.lib = self.L.load()
         self.check = self.L.check
@@ -40,6 +41,7 @@ class GpuRun:
         self.d["cum"] = D((n,), np.int64)
         self.d["vis_ids"] = D((n,), np.int32)
         self.d["counters"] = D((2,), np.int64)     # [n_isects, n_visible]
+        self.d["packed"] = D((n, 12), np.float32)
         self.V = None
 
     def ptr(self, k):
@@ -85,6 +87,8 @@ class GpuRun:
         p.aabb, p.sort_depth, p.radii = self.ptr("aabb"), self.ptr("sort_depth"), self.ptr("radii")
         p.screen = self.screen()
         p.tiles_per_splat = self.ptr("counts") if fused_count else None
+        if self.use_packed:
+            p.packed_rows = self.ptr("packed")
         if self.use_list:
             self.d["counters"].fill_zero()
             p.visible_ids = self.ptr("vis_ids")
@@ -146,6 +150,9 @@ class GpuRun:
         p.tile_offsets, p.flatten_ids, p.n_isects = self.ptr("offsets"), self.ptr(self.vals), self.K
         p.render_rgb, p.render_depth, p.render_T, p.last_ids = (self.ptr("r_rgb"), self.ptr("r_depth"),
                                                                 self.ptr("r_T"), self.ptr("r_last"))
+        if self.use_packed:
+            p.packed_rows = self.ptr("packed")
+            p.screen = self.L.Screen()   # not read
         self.check(self.lib.ssr_raster_fwd(C.byref(p), None))
 
     def raster_bwd(self, v_rgb=None, v_depth=None, v_T=None):
@@ -164,6 +171,9 @@ class GpuRun:
         p.render_T, p.last_ids, p.render_depth = self.ptr("r_T"), self.ptr("r_last"), self.ptr("r_depth")
         p.v_render_rgb, p.v_render_depth, p.v_render_T = self.ptr("g_rgb"), self.ptr("g_depth"), self.ptr("g_T")
         p.v_screen = self.screen("v_")
+        if self.use_packed:
+            p.packed_rows = self.ptr("packed")
+            p.screen = self.L.Screen()
         self.check(self.lib.ssr_raster_bwd(C.byref(p), None))
 
     def projection_bwd(self, accumulate=True, poison=False):

@@ -154,12 +154,13 @@ def tile_n_bits(n_tiles):
 def raster_fwd(n, scr, w, h, offsets, flat):
     o = dict(rgb=np.zeros((h, w, 3), np.float32), depth=np.zeros((h, w), np.float32),
              T=np.zeros((h, w), np.float32), last_ids=np.zeros((h, w), np.int32))
-    stats = np.zeros(2, np.int64)
+    stats = np.zeros(5, np.int64)
     lib().or_raster_fwd(C.c_int64(n), _p(scr["xy"]), _p(scr["depth"]), _p(scr["conic"]),
                         _p(scr["opac"]), _p(scr["rgb"]), C.c_uint32(w), C.c_uint32(h), _p(offsets),
                         _p(flat), C.c_int64(flat.size), _p(o["rgb"]), _p(o["depth"]), _p(o["T"]),
                         _p(o["last_ids"]), _p(stats))
     o["K_f"], o["K_b"] = int(stats[0]), int(stats[1])
+    o["visits_fwd"], o["visits_bwd"], o["visits_bwd_productive"] = int(stats[2]), int(stats[3]), int(stats[4])
     return o
 
 

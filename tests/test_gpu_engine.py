@@ -37,7 +37,7 @@ def test_engine_matches_oracle(pkg, oracle, H, native):
     host, lib = H
     sc = pkg.scenes.make_scene(1, n=30000, width=320, height=240, parity_variant=True)
     ref = oracle.pipeline(sc)
-    eng = host.Engine(sc, fuse_tile_count=native, visible_list=native, overwrite_world_grads=native)
+    eng = host.Engine(sc, fuse_tile_count=native, visible_list=native, packed_rows=native, overwrite_world_grads=native)
     eng.forward()
     eng.backward()
     g1 = _check(eng, ref, sc)
@@ -71,7 +71,7 @@ def test_engine_overwrite_without_list(pkg, oracle, H):
     host, lib = H
     sc = pkg.scenes.make_scene(4, n=40000, width=480, height=270)
     ref = oracle.pipeline(sc)
-    eng = host.Engine(sc, fuse_tile_count=True, visible_list=False, overwrite_world_grads=True)
+    eng = host.Engine(sc, fuse_tile_count=True, visible_list=False, packed_rows=False, overwrite_world_grads=True)
     eng.forward()
     eng.backward()
     _check(eng, ref, sc)

@@ -29,10 +29,10 @@ def _grad_close(got, ref, abs_scale, name):
                            got[bad][:4], ref[bad][:4])
 
 
-def _compare(gpu, oracle, sc, label, fused_count=False, use_list=False):
+def _compare(gpu, oracle, sc, label, fused_count=False, use_list=False, use_packed=False):
     r = oracle.pipeline(sc)
     print(f"[{label}] N={sc.n} {sc.width}x{sc.height} visible={r['proj']['visible']} K={r['isect_ids'].size}", flush=True)
-    g = GpuRun(gpu, sc, use_list=use_list).run_all(fused_count=fused_count)
+    g = GpuRun(gpu, sc, use_list=use_list, use_packed=use_packed).run_all(fused_count=fused_count)
     if use_list:
         assert g.V == r['proj']['visible']
         assert np.array_equal(np.sort(g.host('vis_ids')[:g.V]), np.nonzero(r['proj']['aabb'][:, 2] > r['proj']['aabb'][:, 0])[0])
@@ -111,6 +111,13 @@ def test_visible_work_list(gpu, oracle):
     sc = gpu.scenes.make_scene(4, n=60000, width=480, height=270, sh_codec=0)   # mostly culled
     _compare(gpu, oracle, sc, "cfg4-list", fused_count=True, use_list=True)
     _compare(gpu, oracle, gpu.scenes.tiny_scene(n=700, width=96, height=64, seed=8), "tiny-list", use_list=True)
+
+
+def test_packed_fragment_rows(gpu, oracle):
+    """The compositing kernels fed from K1's 48-byte packed rows: identical results."""
+    _compare(gpu, oracle, gpu.scenes.tiny_scene(n=700, width=96, height=64, seed=9), "tiny-packed", use_packed=True)
+    sc = gpu.scenes.make_scene(2, n=50000, width=480, height=270, parity_variant=True)
+    _compare(gpu, oracle, sc, "cfg2-packed", fused_count=True, use_list=True, use_packed=True)
 
 
 def test_tiny_equirect(gpu, oracle):
