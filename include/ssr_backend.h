@@ -207,6 +207,14 @@ typedef struct {
 } ssr_projection_bwd_params;
 int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream_t stream);
 
+/* Zeroes the gradient rows of the listed splats only (the rows a previous ssr_projection_bwd run
+ * over that list wrote), instead of refilling all N rows. No counterpart in the reference, which
+ * always refills (src/engine/EngineLoss.cpp:120-127).
+ * skip_visible_aabb (optional, [N,4]): rows of splats whose aabb is non-empty are left alone, for use
+ * right before an ssr_projection_bwd in store mode that overwrites exactly those rows. */
+int ssr_zero_world_rows(const ssr_world* v_world, const int32_t* ids, int64_t n,
+                        const float* skip_visible_aabb, ssr_stream_t stream);
+
 /* ---- K10 and runtime (src/backend/api/BackendRuntime.h:29-168). */
 int ssr_fill_u32(void* dst, uint32_t value, int64_t count, ssr_stream_t stream);
 int ssr_init(int device);                       /* select the device, warm the context */

@@ -34,10 +34,15 @@ __device__ __forceinline__ void atomic_max_nonneg(float* p, float v) {
     atomicMax(reinterpret_cast<int*>(p), __float_as_int(v));
 }
 
+template <int kDegree>
+__device__ __forceinline__ void sh_colour(const ssr_projection_fwd_params& P, const CamD& cam, int64_t v);
+
 // Two phases per workgroup of 256 splats. Phase 1: every thread projects its splat (44 B in) and
 // writes aabb / sorting depth / geometry row / tile count; splats that stay visible are appended
 // to a list in LDS. Phase 2: the first n_visible threads evaluate SH colour (192 B in) for the
 // listed splats, so the expensive part runs on dense wavefronts however sparse visibility is.
+// (Running phase 2 as a kernel of its own over the global list was measured and is slower in every
+// configuration, sparse or dense.)
 template <int kDegree>
 __global__ __launch_bounds__(kProjBlock) void projection_fwd_kernel(ssr_projection_fwd_params P) {
     __shared__ int s_list[kProjBlock];
@@ -102,6 +107,12 @@ __global__ __launch_bounds__(kProjBlock) void projection_fwd_kernel(ssr_projecti
     }
     if ((int)threadIdx.x >= n_vis) return;
     const int64_t v = block0 + s_list[threadIdx.x];
+    sh_colour<kDegree>(P, cam, v);
+}
+
+// SH colour of one visible splat: max(0.5 + sum_j Y_j c_j, 0) (src/shaders/harmonics.slang:1055-1066)
+template <int kDegree>
+__device__ __forceinline__ void sh_colour(const ssr_projection_fwd_params& P, const CamD& cam, int64_t v) {
     const float* mp = P.world.means + 3 * v;
     const float mean[3] = {mp[0], mp[1], mp[2]};
     constexpr int kCoef = kDegree * (kDegree + 2);
@@ -372,6 +383,28 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
     for (int i = 0; i < 3; i++) put<kAccumulate>(V.features_dc + 3 * g + i, fin(0.2820947917738781f * vc[i]));
 }
 
+// One wavefront per listed splat: lane l zeroes float l of its 59-float gradient row
+// (3 mean, 4 quat, 3 scale, 1 opacity, 3 dc, sh_stride SH).
+// Rows of splats that are visible now (non-empty aabb) are skipped when `aabb` is given: the
+// projection backward that follows overwrites them.
+__global__ __launch_bounds__(kProjBlock) void zero_world_rows_kernel(ssr_world V, const int32_t* __restrict__ ids, int64_t n,
+                                                                     const float4* __restrict__ aabb) {
+    const int64_t row = (int64_t)blockIdx.x * (kProjBlock / 64) + (threadIdx.x >> 6);
+    if (row >= n) return;
+    const int lane = threadIdx.x & 63;
+    const int64_t g = ids[row];
+    if (aabb) {
+        const float4 bb = aabb[g];
+        if (!(bb.z <= bb.x || bb.w <= bb.y)) return;
+    }
+    if (lane < 3) V.means[3 * g + lane] = 0.f;
+    else if (lane < 7) V.quats[4 * g + lane - 3] = 0.f;
+    else if (lane < 10) V.log_scales[3 * g + lane - 7] = 0.f;
+    else if (lane < 11) V.opacity_logits[g] = 0.f;
+    else if (lane < 14) V.features_dc[3 * g + lane - 11] = 0.f;
+    for (int k = lane; k < V.sh_stride; k += 64) V.features_sh[g * (int64_t)V.sh_stride + k] = 0.f;
+}
+
 static int check_common(const char* where, int64_t n, int sh_degree, const ssr_world& w, const ssr_sh_quant& sh,
                         const ssr_camera& cam) {
     SSR_REQUIRE(n >= 0 && n < (int64_t)1 << 31, where, "num_splats must be in [0, 2^31)");
@@ -463,5 +496,20 @@ extern "C" int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream
     }
 #undef SSR_LAUNCH_BWD
     SSR_CHECK_LAUNCH("ssr_projection_bwd");
+    return 0;
+}
+
+extern "C" int ssr_zero_world_rows(const ssr_world* v_world, const int32_t* ids, int64_t n, const float* skip_visible_aabb,
+                                   ssr_stream_t stream) {
+    SSR_REQUIRE(v_world, "ssr_zero_world_rows", "null world");
+    SSR_REQUIRE(n >= 0 && n < (int64_t)1 << 31, "ssr_zero_world_rows", "count out of range");
+    if (n == 0) return 0;
+    SSR_REQUIRE(ids, "ssr_zero_world_rows", "null ids");
+    const ssr_world& v = *v_world;
+    SSR_REQUIRE(v.means && v.quats && v.log_scales && v.opacity_logits && v.features_dc && (v.features_sh || v.sh_stride == 0),
+                "ssr_zero_world_rows", "null buffer");
+    hipLaunchKernelGGL(zero_world_rows_kernel, dim3((unsigned)ceil_div(n, kProjBlock / 64)), dim3(kProjBlock), 0, as_stream(stream),
+                       v, ids, n, reinterpret_cast<const float4*>(skip_visible_aabb));
+    SSR_CHECK_LAUNCH("ssr_zero_world_rows");
     return 0;
 }

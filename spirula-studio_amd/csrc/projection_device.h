@@ -332,31 +332,35 @@ __device__ __forceinline__ void tile_geom(const float aabb[4], const float xy[2]
     g.by_rows = (g.ymax - g.ymin) * kTile <= (g.xmax - g.xmin) * kTile;
 }
 
-// Visits every tile the ellipse touches in the reference's enumeration order
-// (count pass IntersectTile.cu:55-101, write pass :198-247).
-template <class F>
-__device__ __forceinline__ void for_each_tile(const TileGeomD& g, F&& emit) {
+// Tile interval [lo, hi) that the ellipse covers in one band: band index `r` is a tile row when
+// g.by_rows (the interval is then over tile columns) and a tile column otherwise. Same arithmetic
+// as the reference's count pass (IntersectTile.cu:55-101) and write pass (:198-247).
+__device__ __forceinline__ void tile_band_interval(const TileGeomD& g, int r, int& lo, int& hi) {
+    float bd[2];
     if (g.by_rows) {
-        for (int y = g.ymin; y < g.ymax; y++) {
-            const float y0 = (float)(y * kTile) - g.xy[1];
-            const float y1 = y0 + (float)kTile;
-            float bd[2];
-            ellipse_range_bound(g.ic, y0, y1, bd);
-            const int x0 = clampi(ssr_f2i_sat(ssr_floor((bd[0] + g.xy[0]) / (float)kTile)), g.xmin, g.xmax);
-            const int x1 = clampi(ssr_f2i_sat(ssr_ceil((bd[1] + g.xy[0]) / (float)kTile)), g.xmin, g.xmax);
-            emit(x0, x1, y, true);
-        }
+        const float y0 = (float)(r * kTile) - g.xy[1];
+        const float y1 = y0 + (float)kTile;
+        ellipse_range_bound(g.ic, y0, y1, bd);
+        lo = clampi(ssr_f2i_sat(ssr_floor((bd[0] + g.xy[0]) / (float)kTile)), g.xmin, g.xmax);
+        hi = clampi(ssr_f2i_sat(ssr_ceil((bd[1] + g.xy[0]) / (float)kTile)), g.xmin, g.xmax);
     } else {
         const float sw[3] = {g.ic[2], g.ic[1], g.ic[0]};
-        for (int x = g.xmin; x < g.xmax; x++) {
-            const float x0 = (float)(x * kTile) - g.xy[0];
-            const float x1 = x0 + (float)kTile;
-            float bd[2];
-            ellipse_range_bound(sw, x0, x1, bd);
-            const int y0 = clampi(ssr_f2i_sat(ssr_floor((bd[0] + g.xy[1]) / (float)kTile)), g.ymin, g.ymax);
-            const int y1 = clampi(ssr_f2i_sat(ssr_ceil((bd[1] + g.xy[1]) / (float)kTile)), g.ymin, g.ymax);
-            emit(y0, y1, x, false);
-        }
+        const float x0 = (float)(r * kTile) - g.xy[0];
+        const float x1 = x0 + (float)kTile;
+        ellipse_range_bound(sw, x0, x1, bd);
+        lo = clampi(ssr_f2i_sat(ssr_floor((bd[0] + g.xy[1]) / (float)kTile)), g.ymin, g.ymax);
+        hi = clampi(ssr_f2i_sat(ssr_ceil((bd[1] + g.xy[1]) / (float)kTile)), g.ymin, g.ymax);
+    }
+}
+
+// Visits every band the ellipse touches in the reference's enumeration order: emit(lo, hi, band, by_rows).
+template <class F>
+__device__ __forceinline__ void for_each_tile(const TileGeomD& g, F&& emit) {
+    const int b0 = g.by_rows ? g.ymin : g.xmin, b1 = g.by_rows ? g.ymax : g.xmax;
+    for (int r = b0; r < b1; r++) {
+        int lo, hi;
+        tile_band_interval(g, r, lo, hi);
+        emit(lo, hi, r, g.by_rows);
     }
 }
 

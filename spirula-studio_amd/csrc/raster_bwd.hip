@@ -26,7 +26,7 @@ namespace ssr {
 
 template <int kCtrl>
 __device__ __forceinline__ float dpp_get(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, 0xf, 0xf, false));
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, 0xf, 0xf, true));
 }
 
 // lanes 0..31: a[l] + a[l+32]; lanes 32..63: b[l-32] + b[l]
@@ -175,7 +175,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
                 const float s3 = row_sum(fold16(re_, re_));   // rows: g, g, b, b       -> channels 8,8,9,9
                 float mine = sub == 0 ? s1 : (sub == 1 ? s2 : s3);
                 if (chan >= 0 && ssr_isfinite(mine) && mine != 0.0f)
-                    atomicAdd(abase + (int64_t)astride * s_ids[k], mine);
+                    atomicAdd(abase + (uint32_t)astride * (uint32_t)s_ids[k], mine);   // < 2^32 elements per array
             }
         }
     }
@@ -189,6 +189,7 @@ extern "C" int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t strea
     SSR_REQUIRE(p, "ssr_raster_bwd", "null params");
     SSR_REQUIRE(p->width > 0 && p->height > 0, "ssr_raster_bwd", "empty image");
     SSR_REQUIRE(p->n_isects >= 0 && p->n_isects < (int64_t)1 << 31, "ssr_raster_bwd", "n_isects out of range");
+    SSR_REQUIRE(p->num_splats >= 0 && p->num_splats < ((int64_t)1 << 30), "ssr_raster_bwd", "num_splats must be below 2^30");
     if (p->n_isects == 0) return 0;   // nothing contributed anywhere
     SSR_REQUIRE(p->tile_offsets && p->flatten_ids, "ssr_raster_bwd", "null tile data");
     SSR_REQUIRE(p->render_T && p->last_ids && p->render_depth, "ssr_raster_bwd", "null forward output");

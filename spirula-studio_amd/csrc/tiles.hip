@@ -26,26 +26,51 @@ __global__ __launch_bounds__(kTileBlock) void tile_count_kernel(
     tiles_per_splat[g] = count_tiles(tg);
 }
 
+// Splats that touch more than kCoopTiles tiles (a splat close to the camera can cover thousands)
+// are not written by their own thread: the wavefront takes them one at a time, 64 bands per step,
+// with a wavefront scan placing each band's run of keys, so no lane loops over thousands of tiles
+// while the other 63 wait.
+constexpr int kCoopTiles = 96;
+
+__device__ __forceinline__ int wave_inclusive_scan_i32(int v, int lane) {
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int o = __shfl_up(v, d, 64);
+        if (lane >= d) v += o;
+    }
+    return v;
+}
+
 __global__ __launch_bounds__(kTileBlock) void tile_write_kernel(
     int64_t n, const float4* __restrict__ aabb, const float* __restrict__ sort_depth,
     const float2* __restrict__ xy, const float* __restrict__ conic, const float* __restrict__ opac,
     const int64_t* __restrict__ cum, int tile_w, int tile_h, int64_t* __restrict__ isect_ids,
     int32_t* __restrict__ flatten_ids, const int32_t* __restrict__ visible_ids) {
     const int64_t i = (int64_t)blockIdx.x * kTileBlock + threadIdx.x;
-    if (i >= n) return;
-    const int64_t g = visible_ids ? (int64_t)visible_ids[i] : i;
-    int64_t cur = g == 0 ? 0 : cum[g - 1];
-    const int64_t end = cum[g];
-    const float4 a = aabb[g];
-    if (!(a.z <= a.x || a.w <= a.y)) {
-        const float bb[4] = {a.x, a.y, a.z, a.w};
-        const float2 c = xy[g];
-        const float cxy[2] = {c.x, c.y};
-        const float cn[3] = {conic[3 * g], conic[3 * g + 1], conic[3 * g + 2]};
-        TileGeomD tg;
-        tile_geom(bb, cxy, cn, opac[g], tile_w, tile_h, tg);
-        uint32_t du = ssr_f2u(ssr_fabs(sort_depth[g]));
-        du = (du >> 31) ? ~du : (du ^ 0x80000000u);
+    const int lane = threadIdx.x & 63;
+    const bool in_range = i < n;
+    const int64_t g = in_range ? (visible_ids ? (int64_t)visible_ids[i] : i) : 0;
+    int64_t cur = 0, end = 0;
+    TileGeomD tg;
+    uint32_t du = 0;
+    bool visible = false;
+    if (in_range) {
+        cur = g == 0 ? 0 : cum[g - 1];
+        end = cum[g];
+        const float4 a = aabb[g];
+        visible = !(a.z <= a.x || a.w <= a.y);
+        if (visible) {
+            const float bb[4] = {a.x, a.y, a.z, a.w};
+            const float2 c = xy[g];
+            const float cxy[2] = {c.x, c.y};
+            const float cn[3] = {conic[3 * g], conic[3 * g + 1], conic[3 * g + 2]};
+            tile_geom(bb, cxy, cn, opac[g], tile_w, tile_h, tg);
+            du = ssr_f2u(ssr_fabs(sort_depth[g]));
+            du = (du >> 31) ? ~du : (du ^ 0x80000000u);
+        }
+    }
+    const bool coop = visible && (end - cur) > kCoopTiles;
+    if (visible && !coop) {
         for_each_tile(tg, [&](int lo, int hi, int fixed, bool rows) {
             for (int v = lo; v < hi && cur < end; v++) {
                 const int64_t tile_id = rows ? ((int64_t)fixed * tile_w + v) : ((int64_t)v * tile_w + fixed);
@@ -55,10 +80,47 @@ __global__ __launch_bounds__(kTileBlock) void tile_write_kernel(
             }
         });
     }
-    while (cur < end) {   // IntersectTile.cu:261-266; unreachable when count and write agree
-        isect_ids[cur] = (int64_t)0xffffffffull;
-        flatten_ids[cur] = (int32_t)g;
-        ++cur;
+    if (in_range && !coop) {
+        while (cur < end) {   // IntersectTile.cu:261-266; unreachable when count and write agree
+            isect_ids[cur] = (int64_t)0xffffffffull;
+            flatten_ids[cur] = (int32_t)g;
+            ++cur;
+        }
+    }
+    // cooperative part: the whole wavefront stays converged here
+    uint64_t todo = __ballot(coop);
+    while (todo) {
+        const int src = __builtin_ctzll(todo);
+        todo &= todo - 1;
+        TileGeomD sg;
+        sg.xy[0] = __shfl(tg.xy[0], src, 64); sg.xy[1] = __shfl(tg.xy[1], src, 64);
+        sg.ic[0] = __shfl(tg.ic[0], src, 64); sg.ic[1] = __shfl(tg.ic[1], src, 64); sg.ic[2] = __shfl(tg.ic[2], src, 64);
+        sg.xmin = __shfl(tg.xmin, src, 64); sg.xmax = __shfl(tg.xmax, src, 64);
+        sg.ymin = __shfl(tg.ymin, src, 64); sg.ymax = __shfl(tg.ymax, src, 64);
+        sg.by_rows = __shfl((int)tg.by_rows, src, 64) != 0;
+        const uint32_t sdu = (uint32_t)__shfl((int)du, src, 64);
+        const int32_t sgid = (int32_t)__shfl((int)g, src, 64);
+        int64_t scur = ((int64_t)__shfl((int)(cur >> 32), src, 64) << 32) | (uint32_t)__shfl((int)(uint32_t)cur, src, 64);
+        const int64_t send = ((int64_t)__shfl((int)(end >> 32), src, 64) << 32) | (uint32_t)__shfl((int)(uint32_t)end, src, 64);
+        const int b0 = sg.by_rows ? sg.ymin : sg.xmin, b1 = sg.by_rows ? sg.ymax : sg.xmax;
+        for (int base = b0; base < b1; base += 64) {
+            const int r = base + lane;
+            int lo = 0, hi = 0;
+            if (r < b1) tile_band_interval(sg, r, lo, hi);
+            const int c = max(hi - lo, 0);
+            const int inc = wave_inclusive_scan_i32(c, lane);
+            int64_t pos = scur + (inc - c);
+            for (int v = lo; v < hi && pos < send; v++, pos++) {
+                const int64_t tile_id = sg.by_rows ? ((int64_t)r * tile_w + v) : ((int64_t)v * tile_w + r);
+                isect_ids[pos] = (int64_t)(((uint64_t)tile_id << 32) | (uint64_t)sdu);
+                flatten_ids[pos] = sgid;
+            }
+            scur += __shfl(inc, 63, 64);
+        }
+        for (int64_t pos = scur + lane; pos < send; pos += 64) {   // pad keys, as above
+            isect_ids[pos] = (int64_t)0xffffffffull;
+            flatten_ids[pos] = sgid;
+        }
     }
 }
 

@@ -26,6 +26,9 @@ int64_t* g_counters = nullptr;       // device [n_isects, n_visible], one readba
 int32_t* g_visible_ids = nullptr;    // device work list of the last projection (null: off)
 float* g_packed_rows = nullptr;      // packed screen rows of the last projection (null: off)
 const float* g_packed_for_xy = nullptr;   // the screen.xy buffer those rows mirror
+int g_list_toggle = 0;               // which of the two visible-list buffers the last projection used
+const int32_t* g_bwd_list = nullptr; // list of the last projection backward
+int64_t g_bwd_count = 0;
 
 struct StageTimer {
     ssr_event_t a = nullptr, b = nullptr;
@@ -179,6 +182,12 @@ void set_stage_profiling(bool on) { g_profile = on; }
 StageTimes last_stage_times() { return g_times; }
 int64_t last_n_isects() { return g_n_isects; }
 int64_t last_n_visible() { return g_n_visible; }
+const int32_t* last_backward_list(int64_t* count) { if (count) *count = g_bwd_count; return g_bwd_list; }
+void zero_world_rows(const std::vector<DeviceTensorFloatND>& v, const int32_t* ids, int64_t n,
+                     const DeviceTensor2D<float4>* aabb) {
+    ssr_world w = world_of(v);
+    ok(ssr_zero_world_rows(&w, ids, n, aabb ? (const float*)aabb->data_ptr() : nullptr, nullptr), "zero_world_rows");
+}
 }  // namespace ssr_ext
 
 // ---------------------------------------------------------------------------------------------
@@ -218,7 +227,9 @@ projection_3dgs_forward(const int64_t num_splats, const int max_sh_degree,
     g_visible_ids = nullptr;
     g_n_visible = -1;
     if (g_opts.visible_list) {
-        g_visible_ids = DevicePool::global().acquire<int32_t>(PoolSlot::ProjVisibleIds, (size_t)(C * N));
+        g_list_toggle ^= 1;
+        g_visible_ids = DevicePool::global().acquire<int32_t>(
+            g_list_toggle ? PoolSlot::ProjVisibleIdsB : PoolSlot::ProjVisibleIds, (size_t)(C * N));
         backend::memset_async(g_counters, 0, 2 * sizeof(int64_t));
         p.visible_ids = g_visible_ids;
         p.visible_count = g_counters + 1;
@@ -428,7 +439,11 @@ void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
     p.v_screen = screen_of(v_splats_screen);
     p.v_world = world_of(v_splats_world);
     p.accumulate = g_opts.overwrite_world_grads ? 0 : 1;
-    if (g_visible_ids && g_n_visible >= 0) { p.visible_ids = g_visible_ids; p.n_visible = g_n_visible; }
+    g_bwd_list = nullptr; g_bwd_count = 0;
+    if (g_visible_ids && g_n_visible >= 0) {
+        p.visible_ids = g_visible_ids; p.n_visible = g_n_visible;
+        g_bwd_list = g_visible_ids; g_bwd_count = g_n_visible;
+    }
     StageTimer t(&g_times.k9);
     ok(ssr_projection_bwd(&p, nullptr), "projection_3dgs_backward");
 }

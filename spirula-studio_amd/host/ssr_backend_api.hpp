@@ -116,4 +116,11 @@ void set_stage_profiling(bool on);
 StageTimes last_stage_times();
 int64_t last_n_isects();
 int64_t last_n_visible();   // -1 when the visible list is off
+// The list the last projection_3dgs_backward ran over (device pointer) and its length; it stays
+// intact until the projection after next (the two list buffers alternate). Null when it had none.
+const int32_t* last_backward_list(int64_t* count);
+// Zeroes the rows of `ids` in six world-gradient tensors (ordered as v_splats_world).
+// With `aabb` given, rows of currently visible splats are skipped (a store-mode backward overwrites them).
+void zero_world_rows(const std::vector<DeviceTensorFloatND>& v_splats_world, const int32_t* ids, int64_t n,
+                     const DeviceTensor2D<float4>* aabb);
 }  // namespace ssr_ext

@@ -41,9 +41,20 @@ void alloc_grad_buffers() {
     g.scales.resize(PoolSlot::GradScales, n); g.opacities.resize(PoolSlot::GradOpacities, n);
     g.features_dc.resize(PoolSlot::GradFeaturesDc, n); g.features_sh.resize(PoolSlot::GradFeaturesSh, n, engine().num_sh);
     const auto& o = ssr_ext::options();
-    if (!engine().optim.skip_grad_zero && !(o.overwrite_world_grads && !o.visible_list)) {
-        g.means.zero(); g.quats.zero(); g.scales.zero(); g.opacities.zero(); g.features_dc.zero(); g.features_sh.zero();
+    if (engine().optim.skip_grad_zero) return;
+    if (o.overwrite_world_grads && !o.visible_list) return;   // K9 overwrites every row itself
+    // Every row is zero except those the last backward wrote through its visible list: when that
+    // list is short, zero just those rows instead of refilling all N (the refill is 236 B per splat).
+    if (o.visible_list && o.overwrite_world_grads && g.dirty_list && g.dirty_key == (const void*)g.means.data_ptr() &&
+        g.dirty_count * 2 < n) {
+        std::vector<DeviceTensorFloatND> v_world = {
+            DeviceTensorFloatND(g.means), DeviceTensorFloatND(g.quats), DeviceTensorFloatND(g.scales),
+            DeviceTensorFloatND((float*)g.opacities.data_ptr(), {g.opacities.size(), 1}),
+            DeviceTensorFloatND(g.features_dc), DeviceTensorFloatND(g.features_sh)};
+        ssr_ext::zero_world_rows(v_world, g.dirty_list, g.dirty_count, &engine().fwd.aabb);
+        return;
     }
+    g.means.zero(); g.quats.zero(); g.scales.zero(); g.opacities.zero(); g.features_dc.zero(); g.features_sh.zero();
 }
 
 }  // namespace
@@ -172,6 +183,8 @@ void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorV
         E.camera.model_str, E.camera.distortion_str, E.camera.dist_coeffs, DeviceVector<int32_t>{}, DeviceVector<int32_t>{},
         E.fwd.aabb, vs, v_world, nullptr, E.world.sh_packed, E.world.sh_bounds, (uint32_t)E.num_sh, E.world.sh_value_bits,
         E.world.sh_bounds_stride);
+    E.grad.dirty_list = ssr_ext::last_backward_list(&E.grad.dirty_count);
+    E.grad.dirty_key = (const void*)E.grad.means.data_ptr();
 }
 
 void engine_copy_render_to_host(TorchTensorView out_rgb, TorchTensorView out_depth, TorchTensorView out_Ts,

@@ -43,6 +43,11 @@ struct EngineState {
         DeviceVector<float3> means; DeviceVector<float4> quats; DeviceVector<float3> scales;
         DeviceVector<float> opacities; DeviceVector<float3> features_dc; DeviceTensor2D<float3> features_sh;
         std::vector<DeviceTensorFloatND> v_screen;
+        // rows that are not zero: those of the list the last backward wrote (valid while the
+        // gradient buffers stay where they are and nobody else writes them)
+        const int32_t* dirty_list = nullptr;
+        int64_t dirty_count = 0;
+        const void* dirty_key = nullptr;
     } grad;
 };
 EngineState& engine();

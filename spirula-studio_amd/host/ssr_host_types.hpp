@@ -62,7 +62,7 @@ enum class PoolSlot : int {
     EngRadii,
     ProjAabb, ProjDepths, ProjScreenXy, ProjScreenDepth, ProjScreenConic, ProjScreenOpac, ProjScreenRgb,
     IsectTilesPerSplat, IsectCumTiles, IsectIdsA, IsectIdsB, IsectFlatA, IsectFlatB, IsectOffsets,
-    IsectScanScratch, IsectSortScratch, IsectCounters, ProjVisibleIds, ProjPackedRows,
+    IsectScanScratch, IsectSortScratch, IsectCounters, ProjVisibleIds, ProjVisibleIdsB, ProjPackedRows,
     RendersRgb, RendersDepth, RenderTs, RenderLastIds,
     RasterBwdVScreenXy, RasterBwdVScreenDepth, RasterBwdVScreenConic, RasterBwdVScreenOpac, RasterBwdVScreenRgb,
     EngVRgb, EngVDepth, EngVTs,

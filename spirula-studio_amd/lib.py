@@ -84,6 +84,7 @@ SYMBOLS = {
     "ssr_raster_fwd": (_i32, [C.POINTER(RasterFwdParams), vp]),
     "ssr_raster_bwd": (_i32, [C.POINTER(RasterBwdParams), vp]),
     "ssr_projection_bwd": (_i32, [C.POINTER(ProjectionBwdParams), vp]),
+    "ssr_zero_world_rows": (_i32, [C.POINTER(World), vp, _i64, vp, vp]),
     "ssr_fill_u32": (_i32, [vp, _u32, _i64, vp]),
     "ssr_init": (_i32, [_i32]),
     "ssr_device_count": (_i32, []),

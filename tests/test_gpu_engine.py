@@ -77,6 +77,33 @@ def test_engine_overwrite_without_list(pkg, oracle, H):
     _check(eng, ref, sc)
 
 
+def test_lazy_gradient_zeroing_follows_the_camera(pkg, oracle, H):
+    """With few visible splats only the rows written by the previous backward are re-zeroed; after a
+    camera move the rows of splats that left the view must read zero again."""
+    host, lib = H
+    import ctypes as C
+    sc = pkg.scenes.make_scene(4, n=60000, width=480, height=270)
+    eng = host.Engine(sc)
+    for _ in range(2):
+        eng.forward()
+        eng.backward()
+    ref = oracle.pipeline(sc)
+    assert ref["proj"]["visible"] * 2 < sc.n
+    _check(eng, ref, sc)
+    # look the other way: a different set of splats is visible
+    sc.viewmat = np.array([[-1, 0, 0, 0], [0, 1, 0, 0], [0, 0, -1, 0.5], [0, 0, 0, 1]], np.float32)
+    vm, it = np.ascontiguousarray(sc.viewmat), np.ascontiguousarray(sc.intrins, np.float32)
+    host.check(eng.h.ssrh_set_camera_params(sc.width, sc.height, b"PINHOLE", b"NONE", vm.ctypes.data, it.ctypes.data, 1))
+    eng.forward()
+    eng.backward()
+    ref2 = oracle.pipeline(sc)
+    vis1 = ref["proj"]["aabb"][:, 2] > ref["proj"]["aabb"][:, 0]
+    vis2 = ref2["proj"]["aabb"][:, 2] > ref2["proj"]["aabb"][:, 0]
+    assert (vis1 & ~vis2).sum() > 1000
+    g = _check(eng, ref2, sc)
+    assert not np.any(g["v_sh"][~vis2]) and not np.any(g["v_means"][~vis2])
+
+
 def test_unsupported_variants_raise(pkg, H):
     host, lib = H
     sc = pkg.scenes.tiny_scene(n=50, width=32, height=32)

@@ -120,6 +120,16 @@ def test_packed_fragment_rows(gpu, oracle):
     _compare(gpu, oracle, sc, "cfg2-packed", fused_count=True, use_list=True, use_packed=True)
 
 
+def test_huge_splats_cooperative_key_write(gpu, oracle):
+    """Splats that cover hundreds of tiles take the wavefront-cooperative path of the key write."""
+    sc = gpu.scenes.tiny_scene(n=600, width=640, height=400, seed=13)
+    sc.log_scales[::7] += 2.5          # every 7th splat becomes very large
+    sc.means[::50, 2] = -3.6           # a few right in front of the camera (camera at z = -4)
+    g, r = _compare(gpu, oracle, sc, "huge", fused_count=True, use_list=True)
+    assert r["counts"].max() > 500
+    _compare(gpu, oracle, sc, "huge-nolist")
+
+
 def test_tiny_equirect(gpu, oracle):
     _compare(gpu, oracle, gpu.scenes.tiny_scene(n=600, width=128, height=64, seed=4, camera_model=3), "tiny-eq")
 
