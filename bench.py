@@ -91,6 +91,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--reference-order", action="store_true",
                     help="run the stages exactly as the reference does (separate count pass, atomic K9 into zero-filled buffers)")
+    ap.add_argument("--packed-projection", action="store_true",
+                    help="run the packed form of the projection (compacted nnz-row outputs; the reference's training default)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run device copies / fills of known size (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE) and exit")
     args = ap.parse_args()
@@ -121,7 +123,8 @@ def main():
     sc = pkg.scenes.make_scene(cfg, n=args.n)
     t_gen = time.time() - t_gen
     native = not args.reference_order
-    eng = host.Engine(sc, fuse_tile_count=native, visible_list=native, packed_rows=native, overwrite_world_grads=native)
+    eng = host.Engine(sc, fuse_tile_count=native, visible_list=native and not args.packed_projection, packed_rows=native,
+                      overwrite_world_grads=native, packed_projection=args.packed_projection)
     L = lib.load()
 
     eng.time_iterations(max(args.warmup, 1))
@@ -145,7 +148,7 @@ def main():
 
     # problem sizes from the device results
     aabb = eng.cache("aabb").reshape(-1, 4)
-    V = int((aabb[:, 2] > aabb[:, 0]).sum())
+    V = int((aabb[:, 2] > aabb[:, 0]).sum())   # packed form: every one of its nnz rows
     K = eng.n_isects
     P = sc.width * sc.height
     T = sc.tile_w * sc.tile_h
@@ -176,7 +179,8 @@ def main():
                                f"{'pinhole' if sc.camera_model == 0 else 'equirectangular'}, SH3 "
                                f"{['fp32', 'ref-q8', 'ref-q16', 'int8*fp16scale'][sc.sh_codec]}, tile 16x16, seed {pkg.scenes.CONFIGS[cfg]['seed']:#x}",
                    "visible": V, "n_isects": K, "K_b": K_b, "tiles": T, "pixels": P,
-                   "stage_order": "fused tile count, visible-splat work list, packed fragment rows, plain-store gradients" if native else "reference order",
+                   "stage_order": ("fused tile count, visible-splat work list, packed fragment rows, plain-store gradients" if native else "reference order")
+                                  + (", packed projection outputs" if args.packed_projection else ""),
                    "device_ms_per_iter_median": float(np.median(ms))},
         "hbm_roofline_frac_whole_iteration": total_bytes / (float(np.median(ms)) * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "algorithmic_bytes_per_iter": total_bytes,

@@ -19,7 +19,8 @@
  *    (src/backend/api/BackendRuntime.h:98). Nothing calls exit().
  *  - Supported variant: primitive "3dgs" (not antialiased), camera PINHOLE or EQUIRECTANGULAR,
  *    distortion NONE, one camera (C = 1), SH degree 0..3, dist_type None, no median, no
- *    accumulation weights, non-packed. Anything else is rejected with an error, as the reference
+ *    accumulation weights; both the [C,N] layout and the packed (compacted, nnz rows) layout of
+ *    the projection outputs. Anything else is rejected with an error, as the reference
  *    rejects an uncompiled variant (src/kernels/projection/ProjectionFwd.cu:84-89).
  *  - Layouts are the reference's (src/primitives/PrimitiveBase3DGS.cuh:87-139,187-225).
  */
@@ -110,6 +111,40 @@ typedef struct {
     float* packed_rows;
 } ssr_projection_fwd_params;
 int ssr_projection_fwd(const ssr_projection_fwd_params* p, ssr_stream_t stream);
+
+/* ---- K1, packed form: projection_3dgs_packed_forward (src/kernels/projection/ProjectionPackedFwd.cuh:18-37;
+ * kernels src/kernels/projection/ProjectionPackedFwd_kernel.cuh:17-184; launcher
+ * src/kernels/projection/ProjectionPackedFwd.cu:64-158). The outputs hold one row per VISIBLE
+ * splat, in ascending splat order: camera_ids / gaussian_ids / aabb / sort_depth / screen, nnz rows.
+ * The reference runs mask -> inclusive scan -> blocking readback of nnz -> a second full projection
+ * that writes the compacted rows. Here the first call projects every splat once, compacts the
+ * visible ones inside each 256-splat workgroup into `scratch`, and scans the workgroup counts into
+ * *nnz; the second call evaluates SH colour for the nnz staged rows and places them. Between the
+ * two the caller may read *nnz back (ssr_read_i64) to size its outputs, or skip the readback and
+ * pass capacity num_splats as max_rows. Rows past *nnz are not written. radii is max-accumulated
+ * by splat index, as in the non-packed form. */
+typedef struct {
+    int64_t num_splats;
+    int32_t sh_degree;
+    ssr_world world;
+    ssr_sh_quant sh;
+    ssr_camera camera;
+    float* radii;               /* [N], caller zero-fills */
+    void* scratch;              /* ssr_projection_packed_scratch_bytes(num_splats), 16-byte aligned */
+    size_t scratch_bytes;
+    int64_t* nnz;               /* device scalar: written by _mask, read by _emit */
+    int64_t max_rows;           /* _emit: capacity of the arrays below, in rows (>= *nnz) */
+    int32_t* camera_ids;        /* [nnz] all zero with one camera */
+    int32_t* gaussian_ids;      /* [nnz] ascending */
+    float* aabb;                /* [nnz,4] */
+    float* sort_depth;          /* [nnz] */
+    ssr_screen screen;          /* [nnz] rows */
+    int64_t* tiles_per_splat;   /* optional [nnz]: fused K2 */
+    float* packed_rows;         /* optional [nnz,12]: 48-byte fragment rows, as in ssr_projection_fwd_params */
+} ssr_projection_packed_params;
+size_t ssr_projection_packed_scratch_bytes(int64_t num_splats);
+int ssr_projection_packed_mask(const ssr_projection_packed_params* p, ssr_stream_t stream);
+int ssr_projection_packed_emit(const ssr_projection_packed_params* p, ssr_stream_t stream);
 
 /* ---- K2..K6: do_intersect_tile_generic, ellipse mode (src/kernels/tile/IntersectTile.cuh:25-41,
  * src/kernels/tile/IntersectTile.cu:376-509) split at its data-dependent allocation. */
@@ -204,6 +239,12 @@ typedef struct {
      * caller zero-fills v_world once, as the reference does). */
     const int32_t* visible_ids;
     int64_t n_visible;
+    /* Packed mode (src/kernels/projection/ProjectionBwd_kernel.cuh:51-56, launcher
+     * src/kernels/projection/ProjectionBwd.cu:80-84): v_screen holds num_packed rows, row i belongs
+     * to splat packed_gaussian_ids[i]; aabb is not consulted and visible_ids must be NULL.
+     * num_packed == 0 with the pointer set is a no-op (ProjectionBwd.cu:89-97). */
+    const int32_t* packed_gaussian_ids;
+    int64_t num_packed;
 } ssr_projection_bwd_params;
 int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream_t stream);
 

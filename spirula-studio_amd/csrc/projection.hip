@@ -35,7 +35,8 @@ __device__ __forceinline__ void atomic_max_nonneg(float* p, float v) {
 }
 
 template <int kDegree>
-__device__ __forceinline__ void sh_colour(const ssr_projection_fwd_params& P, const CamD& cam, int64_t v);
+__device__ __forceinline__ void sh_colour(const ssr_world& W, const ssr_sh_quant& Q, const CamD& cam, int64_t g,
+                                          float* rgb_row, float* packed_row);
 
 // Two phases per workgroup of 256 splats. Phase 1: every thread projects its splat (44 B in) and
 // writes aabb / sorting depth / geometry row / tile count; splats that stay visible are appended
@@ -107,34 +108,207 @@ __global__ __launch_bounds__(kProjBlock) void projection_fwd_kernel(ssr_projecti
     }
     if ((int)threadIdx.x >= n_vis) return;
     const int64_t v = block0 + s_list[threadIdx.x];
-    sh_colour<kDegree>(P, cam, v);
+    sh_colour<kDegree>(P.world, P.sh, cam, v, P.screen.rgb + 3 * v,
+                       P.packed_rows ? P.packed_rows + kPackedRowFloats * v : nullptr);
 }
 
-// SH colour of one visible splat: max(0.5 + sum_j Y_j c_j, 0) (src/shaders/harmonics.slang:1055-1066)
+// SH colour of one visible splat g: max(0.5 + sum_j Y_j c_j, 0) (src/shaders/harmonics.slang:1055-1066),
+// written to rgb_row[0..2] and, when given, to the colour slots of its 48-byte fragment row.
 template <int kDegree>
-__device__ __forceinline__ void sh_colour(const ssr_projection_fwd_params& P, const CamD& cam, int64_t v) {
-    const float* mp = P.world.means + 3 * v;
+__device__ __forceinline__ void sh_colour(const ssr_world& W, const ssr_sh_quant& Q, const CamD& cam, int64_t g,
+                                          float* rgb_row, float* packed_row) {
+    const float* mp = W.means + 3 * g;
     const float mean[3] = {mp[0], mp[1], mp[2]};
     constexpr int kCoef = kDegree * (kDegree + 2);
     float coef[kCoef > 0 ? 3 * kCoef : 1];
-    if (kCoef > 0) decode_sh<kCoef>(P.world, P.sh, v, coef);
+    if (kCoef > 0) decode_sh<kCoef>(W, Q, g, coef);
     float dir[3];
     view_dir(cam, mean, dir);
     ShBasisD b;
     sh_basis<kDegree>(dir, b);
-    const float* dcp = P.world.features_dc + 3 * v;
+    const float* dcp = W.features_dc + 3 * g;
     const float dc[3] = {dcp[0], dcp[1], dcp[2]};
     float raw[3];
     sh_color_raw<kDegree>(b, dc, coef, raw);
-    float* rg = P.screen.rgb + 3 * v;
     float col[3];
 #pragma unroll
-    for (int c = 0; c < 3; c++) { col[c] = ssr_max(raw[c] + 0.5f, 0.0f); rg[c] = col[c]; }
-    if (P.packed_rows) {
-        float* row = P.packed_rows + kPackedRowFloats * v;
-        *reinterpret_cast<float2*>(row + 6) = make_float2(col[0], col[1]);
-        row[8] = col[2];
+    for (int c = 0; c < 3; c++) { col[c] = ssr_max(raw[c] + 0.5f, 0.0f); rgb_row[c] = col[c]; }
+    if (packed_row) {
+        *reinterpret_cast<float2*>(packed_row + 6) = make_float2(col[0], col[1]);
+        packed_row[8] = col[2];
     }
+}
+
+// ---- packed form -------------------------------------------------------------------------------
+// Staging area of the packed projection inside the caller's scratch buffer: per-workgroup visible
+// counts, their exclusive scan, and the geometry of the visible splats compacted within each
+// workgroup's own 256-row segment (structure of arrays, so both passes access it coalesced).
+struct PackedStage {
+    int32_t* block_counts;    // [nb]
+    int64_t* block_offsets;   // [nb + 1], block_offsets[nb] = nnz
+    float4* aabb;             // [N]
+    float2* xy;               // [N]
+    float* conic;             // [3][N], component-major
+    float* sort_depth;        // [N]
+    float* depth;             // [N]
+    float* opac;              // [N]
+    int32_t* gid;             // [N]
+};
+
+__host__ __device__ inline size_t align16(size_t b) { return (b + 15) & ~(size_t)15; }
+
+inline size_t packed_stage_layout(int64_t n, void* base, PackedStage* st) {
+    const size_t nb = (size_t)ceil_div(n, kProjBlock), N = (size_t)n;
+    char* p = static_cast<char*>(base);
+    size_t off = 0;
+    auto take = [&](size_t bytes) { char* r = p ? p + off : nullptr; off += align16(bytes); return r; };
+    char* a0 = take(N * 16); char* a1 = take(N * 8); char* a2 = take(N * 12); char* a3 = take(N * 4);
+    char* a4 = take(N * 4); char* a5 = take(N * 4); char* a6 = take(N * 4);
+    char* a7 = take((nb + 1) * 8); char* a8 = take(nb * 4);
+    if (st) {
+        st->aabb = reinterpret_cast<float4*>(a0); st->xy = reinterpret_cast<float2*>(a1);
+        st->conic = reinterpret_cast<float*>(a2); st->sort_depth = reinterpret_cast<float*>(a3);
+        st->depth = reinterpret_cast<float*>(a4); st->opac = reinterpret_cast<float*>(a5);
+        st->gid = reinterpret_cast<int32_t*>(a6); st->block_offsets = reinterpret_cast<int64_t*>(a7);
+        st->block_counts = reinterpret_cast<int32_t*>(a8);
+    }
+    return off;
+}
+
+// Pass 1 of the packed projection (projection_packed_mask_kernel,
+// src/kernels/projection/ProjectionPackedFwd_kernel.cuh:17-94): the visibility rule is the clamped
+// aabb extent test. Unlike the reference, which keeps only the mask and projects again later, the
+// projected geometry of the visible splats is kept: compacted in splat order within the
+// workgroup's segment of the staging area (ballot ranks inside a wavefront, wavefront totals through
+// LDS), so that the second pass never touches a culled splat.
+__global__ __launch_bounds__(kProjBlock) void projection_packed_mask_kernel(ssr_projection_packed_params P, PackedStage S) {
+    __shared__ int s_wave[kProjBlock / 64];
+    const int64_t block0 = (int64_t)blockIdx.x * kProjBlock;
+    const int64_t g = block0 + threadIdx.x;
+    const CamD cam = load_camera(P.camera);
+    bool vis = false;
+    ProjD p;
+    float bb[4] = {0.f, 0.f, 0.f, 0.f};
+    if (g < P.num_splats) {
+        float mean[3], quat[4], ls[3], logit;
+        load_splat(P.world, g, mean, quat, ls, logit);
+        project<false>(cam, mean, quat, ls, logit, p);
+        bb[0] = ssr_min(ssr_max(p.aabb[0], 0.0f), cam.Wf - 1.0f);
+        bb[1] = ssr_min(ssr_max(p.aabb[1], 0.0f), cam.Hf - 1.0f);
+        bb[2] = ssr_min(ssr_max(p.aabb[2], 0.0f), cam.Wf - 1.0f);
+        bb[3] = ssr_min(ssr_max(p.aabb[3], 0.0f), cam.Hf - 1.0f);
+        vis = bb[2] - bb[0] > 1e-3f && bb[3] - bb[1] > 1e-3f;   // ProjectionPackedFwd_kernel.cuh:93
+    }
+    const unsigned long long m = __ballot(vis);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int rank = __popcll(m & ((1ull << lane) - 1ull));
+    if (lane == 0) s_wave[wave] = __popcll(m);
+    __syncthreads();
+    int base = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < kProjBlock / 64; w++) { if (w < wave) base += s_wave[w]; total += s_wave[w]; }
+    if (threadIdx.x == 0) S.block_counts[blockIdx.x] = total;
+    if (!vis) return;
+    const int64_t d = block0 + base + rank;
+    const int64_t N = P.num_splats;
+    S.aabb[d] = make_float4(bb[0], bb[1], bb[2], bb[3]);
+    S.xy[d] = make_float2(p.xy[0], p.xy[1]);
+    S.conic[d] = p.conic[0]; S.conic[N + d] = p.conic[1]; S.conic[2 * N + d] = p.conic[2];
+    S.sort_depth[d] = p.sort_depth;
+    S.depth[d] = p.depth;
+    S.opac[d] = p.opac;
+    S.gid[d] = (int32_t)g;
+    atomic_max_nonneg(P.radii + g, p.radius);   // ProjectionPackedFwd_kernel.cuh:183
+}
+
+// Exclusive scan of the workgroup counts by ONE workgroup: each thread sums a contiguous run, the
+// 1024 run totals are scanned in LDS, then each thread writes its run's offsets. The counts are
+// N/256 values (39k for ten million splats), so one workgroup is enough and saves two launches.
+constexpr int kScanOneBlock = 1024;
+__global__ __launch_bounds__(kScanOneBlock) void packed_block_scan_kernel(const int32_t* __restrict__ counts, int64_t nb,
+                                                                          int64_t* __restrict__ offsets, int64_t* __restrict__ nnz) {
+    __shared__ long long s_part[kScanOneBlock];
+    const int64_t run = (nb + kScanOneBlock - 1) / kScanOneBlock;
+    const int64_t lo = (int64_t)threadIdx.x * run, hi = lo + run < nb ? lo + run : nb;
+    long long sum = 0;
+    for (int64_t i = lo; i < hi; i++) sum += counts[i];
+    s_part[threadIdx.x] = sum;
+    __syncthreads();
+    for (int d = 1; d < kScanOneBlock; d <<= 1) {   // Hillis-Steele inclusive scan
+        const long long v = (int)threadIdx.x >= d ? s_part[threadIdx.x - d] : 0;
+        __syncthreads();
+        s_part[threadIdx.x] += v;
+        __syncthreads();
+    }
+    long long acc = s_part[threadIdx.x] - sum;
+    for (int64_t i = lo; i < hi; i++) { offsets[i] = acc; acc += counts[i]; }
+    if (threadIdx.x == kScanOneBlock - 1) { offsets[nb] = s_part[threadIdx.x]; *nnz = s_part[threadIdx.x]; }
+}
+
+// Pass 2 (projection_packed_fwd_kernel, ProjectionPackedFwd_kernel.cuh:97-184): one thread per
+// OUTPUT row j < nnz. The source workgroup of row j is found by bisection over the scanned
+// offsets: two searches with uniform arguments bracket the workgroups this 256-row span touches, a
+// short per-thread search finishes inside the bracket.
+__device__ __forceinline__ int64_t last_block_at_or_before(const int64_t* __restrict__ off, int64_t nb, int64_t j) {
+    int64_t lo = 0, hi = nb;   // invariant: off[lo] <= j < off[hi]
+    while (hi - lo > 1) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (off[mid] <= j) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+template <int kDegree>
+__global__ __launch_bounds__(kProjBlock) void projection_packed_emit_kernel(ssr_projection_packed_params P, PackedStage S) {
+    const int64_t nnz = *P.nnz < P.max_rows ? *P.nnz : P.max_rows;
+    const int64_t j0 = (int64_t)blockIdx.x * kProjBlock;
+    if (j0 >= nnz) return;
+    const int64_t nb = (P.num_splats + kProjBlock - 1) / kProjBlock;
+    const int64_t j1 = j0 + kProjBlock - 1 < nnz - 1 ? j0 + kProjBlock - 1 : nnz - 1;
+    int64_t lo = last_block_at_or_before(S.block_offsets, nb, j0);
+    int64_t hi = last_block_at_or_before(S.block_offsets, nb, j1) + 1;
+    const int64_t j = j0 + threadIdx.x;
+    if (j >= nnz) return;
+    while (hi - lo > 1) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (S.block_offsets[mid] <= j) lo = mid; else hi = mid;
+    }
+    const int64_t src = lo * kProjBlock + (j - S.block_offsets[lo]);
+    const int64_t N = P.num_splats;
+    const CamD cam = load_camera(P.camera);
+    const float4 bb4 = S.aabb[src];
+    const float2 xy = S.xy[src];
+    const float conic[3] = {S.conic[src], S.conic[N + src], S.conic[2 * N + src]};
+    const float opac = S.opac[src], depth = S.depth[src];
+    const int32_t g = S.gid[src];
+    P.camera_ids[j] = 0;
+    P.gaussian_ids[j] = g;
+    reinterpret_cast<float4*>(P.aabb)[j] = bb4;
+    P.sort_depth[j] = S.sort_depth[src];
+    *reinterpret_cast<float2*>(P.screen.xy + 2 * j) = xy;
+    P.screen.depth[j] = depth;
+    float* cn = P.screen.conic + 3 * j;
+    cn[0] = conic[0]; cn[1] = conic[1]; cn[2] = conic[2];
+    P.screen.opac[j] = opac;
+    if (P.tiles_per_splat) {
+        const int tw = (int)((P.camera.width + kTile - 1) / kTile), th = (int)((P.camera.height + kTile - 1) / kTile);
+        const float bb[4] = {bb4.x, bb4.y, bb4.z, bb4.w};
+        const float c2[2] = {xy.x, xy.y};
+        TileGeomD tg;
+        tile_geom(bb, c2, conic, opac, tw, th, tg);
+        P.tiles_per_splat[j] = count_tiles(tg);
+    }
+    float* prow = nullptr;
+    if (P.packed_rows) {
+        float cut, kk;
+        fragment_constants(opac, cut, kk);
+        prow = P.packed_rows + kPackedRowFloats * j;
+        float4* row = reinterpret_cast<float4*>(prow);
+        row[0] = make_float4(xy.x, xy.y, 0.5f * conic[0], conic[1]);
+        *reinterpret_cast<float2*>(&row[1]) = make_float2(0.5f * conic[2], opac);
+        prow[9] = depth; prow[10] = cut; prow[11] = kk;
+    }
+    sh_colour<kDegree>(P.world, P.sh, cam, g, P.screen.rgb + 3 * j, prow);
 }
 
 __device__ __forceinline__ float fin(float v) { return ssr_isfinite(v) ? v : 0.0f; }
@@ -148,10 +322,13 @@ __device__ __forceinline__ void put(float* p, float v) {
 template <int kDegree, bool kAccumulate>
 __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projection_bwd_params P) {
     const int64_t i = (int64_t)blockIdx.x * kProjBlock + threadIdx.x;
-    if (i >= (P.visible_ids ? P.n_visible : P.num_splats)) return;
-    const int64_t g = P.visible_ids ? (int64_t)P.visible_ids[i] : i;
+    if (i >= (P.packed_gaussian_ids ? P.num_packed : (P.visible_ids ? P.n_visible : P.num_splats))) return;
+    // g: row of the splat in world / v_world; r: its row in v_screen (ProjectionBwd_kernel.cuh:51-63)
+    const int64_t g = P.packed_gaussian_ids ? (int64_t)P.packed_gaussian_ids[i] : (P.visible_ids ? (int64_t)P.visible_ids[i] : i);
+    const int64_t r = P.packed_gaussian_ids ? i : g;
     constexpr int kCoef = kDegree * (kDegree + 2);
-    const float4 bb = reinterpret_cast<const float4*>(P.aabb)[g];
+    float4 bb = make_float4(0.f, 0.f, 1.f, 1.f);
+    if (!P.packed_gaussian_ids) bb = reinterpret_cast<const float4*>(P.aabb)[g];
     ssr_world& V = P.v_world;
     if (bb.z <= bb.x || bb.w <= bb.y) {   // ProjectionBwd_kernel.cuh:58
         if (!kAccumulate && !P.visible_ids) {
@@ -174,7 +351,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
     // conic = inverse(cov2d)
     const float c00 = p.c2[0][0], c01 = p.c2[0][1], c10 = p.c2[1][0], c11 = p.c2[1][1];
     const float det = c00 * c11 - c01 * c10, inv = 1.0f / det;
-    const float* vcn = P.v_screen.conic + 3 * g;
+    const float* vcn = P.v_screen.conic + 3 * r;
     const float g00 = vcn[0], g01 = vcn[1], g11 = vcn[2];
     const float v_inv = (c11 * g00 - c01 * g01) + c00 * g11;
     const float v_det = -(v_inv / (det * det));
@@ -208,7 +385,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
                 for (int j = 0; j < 2; j++) s += p.J[i][k] * vC[i][j] * p.J[j][l];
             vS[k][l] = s;
         }
-    const float vm0 = P.v_screen.xy[2 * g], vm1 = P.v_screen.xy[2 * g + 1];
+    const float vm0 = P.v_screen.xy[2 * r], vm1 = P.v_screen.xy[2 * r + 1];
     if (cam.model == SSR_CAM_PINHOLE) {
         const float z2 = z * z, iz = 1.0f / z, iz2 = 1.0f / z2;
         vmc[2] += vJ[0][0] * (-cam.fx * iz2) + vJ[1][1] * (-cam.fy * iz2);
@@ -247,7 +424,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
     }
     {   // depth = length(mean_c); the sqrt derivative is guarded at 1e-7
         const float s2 = dot3(p.mc, p.mc);
-        const float vs = P.v_screen.depth[g] * (0.5f / ssr_sqrt(ssr_max(1e-7f, s2)));
+        const float vs = P.v_screen.depth[r] * (0.5f / ssr_sqrt(ssr_max(1e-7f, s2)));
 #pragma unroll
         for (int i = 0; i < 3; i++) vmc[i] += 2.0f * p.mc[i] * vs;
     }
@@ -295,7 +472,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
     float vquat[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) vquat[i] = (vqn[i] - p.qn[i] * qd) * p.qinv;
-    const float vlogit = P.v_screen.opac[g] * (p.opac * (1.0f - p.opac));
+    const float vlogit = P.v_screen.opac[r] * (p.opac * (1.0f - p.opac));
 
     // SH colour VJP (src/shaders/harmonics.slang:373-649,1087-1126)
     float coef[kCoef > 0 ? 3 * kCoef : 1];
@@ -308,7 +485,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
     const float dc[3] = {dcp[0], dcp[1], dcp[2]};
     float raw[3];
     sh_color_raw<kDegree>(b, dc, coef, raw);
-    const float* vrg = P.v_screen.rgb + 3 * g;
+    const float* vrg = P.v_screen.rgb + 3 * r;
     float vc[3];
 #pragma unroll
     for (int c = 0; c < 3; c++) vc[c] = vrg[c] * (raw[c] >= -0.5f ? 1.0f : 0.0f);
@@ -465,12 +642,84 @@ extern "C" int ssr_projection_fwd(const ssr_projection_fwd_params* p, ssr_stream
     return 0;
 }
 
+extern "C" size_t ssr_projection_packed_scratch_bytes(int64_t num_splats) {
+    if (num_splats <= 0) return 16;
+    return packed_stage_layout(num_splats, nullptr, nullptr);
+}
+
+static int check_packed(const char* where, const ssr_projection_packed_params* p) {
+    SSR_REQUIRE(p, where, "null params");
+    int e = check_common(where, p->num_splats, p->sh_degree, p->world, p->sh, p->camera);
+    if (e) return e;
+    SSR_REQUIRE(p->nnz, where, "null nnz");
+    if (p->num_splats == 0) return 0;
+    SSR_REQUIRE(p->scratch && (reinterpret_cast<uintptr_t>(p->scratch) & 15) == 0, where, "scratch must be non-null and 16-byte aligned");
+    SSR_REQUIRE(p->scratch_bytes >= ssr_projection_packed_scratch_bytes(p->num_splats), where, "scratch too small");
+    SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->world.quats) & 15) == 0, where, "quats must be 16-byte aligned");
+    return 0;
+}
+
+extern "C" int ssr_projection_packed_mask(const ssr_projection_packed_params* p, ssr_stream_t stream) {
+    const char* where = "ssr_projection_packed_mask";
+    int e = check_packed(where, p);
+    if (e) return e;
+    hipStream_t s = as_stream(stream);
+    if (p->num_splats == 0) {   // nnz = 0 without touching the scratch
+        hipLaunchKernelGGL(packed_block_scan_kernel, dim3(1), dim3(kScanOneBlock), 0, s, (const int32_t*)nullptr, (int64_t)0,
+                           p->nnz, p->nnz);
+        SSR_CHECK_LAUNCH(where);
+        return 0;
+    }
+    SSR_REQUIRE(p->radii, where, "null radii");
+    PackedStage st;
+    packed_stage_layout(p->num_splats, p->scratch, &st);
+    const int64_t nb = ceil_div(p->num_splats, kProjBlock);
+    hipLaunchKernelGGL(projection_packed_mask_kernel, dim3((unsigned)nb), dim3(kProjBlock), 0, s, *p, st);
+    SSR_CHECK_LAUNCH(where);
+    hipLaunchKernelGGL(packed_block_scan_kernel, dim3(1), dim3(kScanOneBlock), 0, s, (const int32_t*)st.block_counts, nb,
+                       st.block_offsets, p->nnz);
+    SSR_CHECK_LAUNCH(where);
+    return 0;
+}
+
+extern "C" int ssr_projection_packed_emit(const ssr_projection_packed_params* p, ssr_stream_t stream) {
+    const char* where = "ssr_projection_packed_emit";
+    int e = check_packed(where, p);
+    if (e) return e;
+    SSR_REQUIRE(p->max_rows >= 0 && p->max_rows <= p->num_splats, where, "max_rows must be in [0, num_splats]");
+    if (p->num_splats == 0 || p->max_rows == 0) return 0;
+    SSR_REQUIRE(p->camera_ids && p->gaussian_ids && p->aabb && p->sort_depth, where, "null output");
+    SSR_REQUIRE(p->screen.xy && p->screen.depth && p->screen.conic && p->screen.opac && p->screen.rgb, where, "null screen buffer");
+    SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->aabb) & 15) == 0, where, "aabb must be 16-byte aligned");
+    SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->screen.xy) & 7) == 0, where, "screen.xy must be 8-byte aligned");
+    SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->packed_rows) & 15) == 0, where, "packed_rows must be 16-byte aligned");
+    PackedStage st;
+    packed_stage_layout(p->num_splats, p->scratch, &st);
+    const dim3 grid((unsigned)ceil_div(p->max_rows, kProjBlock)), block(kProjBlock);
+    hipStream_t s = as_stream(stream);
+    switch (p->sh_degree) {
+        case 0: hipLaunchKernelGGL(projection_packed_emit_kernel<0>, grid, block, 0, s, *p, st); break;
+        case 1: hipLaunchKernelGGL(projection_packed_emit_kernel<1>, grid, block, 0, s, *p, st); break;
+        case 2: hipLaunchKernelGGL(projection_packed_emit_kernel<2>, grid, block, 0, s, *p, st); break;
+        default: hipLaunchKernelGGL(projection_packed_emit_kernel<3>, grid, block, 0, s, *p, st); break;
+    }
+    SSR_CHECK_LAUNCH(where);
+    return 0;
+}
+
 extern "C" int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream_t stream) {
     SSR_REQUIRE(p, "ssr_projection_bwd", "null params");
     int e = check_common("ssr_projection_bwd", p->num_splats, p->sh_degree, p->world, p->sh, p->camera);
     if (e) return e;
     if (p->num_splats == 0) return 0;   // src/kernels/projection/ProjectionBwd.cu:86-87
-    SSR_REQUIRE(p->aabb, "ssr_projection_bwd", "null aabb");   // ProjectionBwd.cu:89-97
+    const bool packed = p->packed_gaussian_ids != nullptr;
+    if (packed) {
+        SSR_REQUIRE(!p->visible_ids, "ssr_projection_bwd", "packed mode takes no visible list");
+        SSR_REQUIRE(p->num_packed >= 0 && p->num_packed <= p->num_splats, "ssr_projection_bwd", "num_packed out of range");
+        if (p->num_packed == 0) return 0;
+    } else {
+        SSR_REQUIRE(p->aabb, "ssr_projection_bwd", "null aabb");   // ProjectionBwd.cu:89-97
+    }
     SSR_REQUIRE(p->v_screen.xy && p->v_screen.depth && p->v_screen.conic && p->v_screen.opac && p->v_screen.rgb,
                 "ssr_projection_bwd", "null v_screen buffer");
     const ssr_world& v = p->v_world;
@@ -483,7 +732,8 @@ extern "C" int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream
         SSR_REQUIRE(p->n_visible >= 0 && p->n_visible <= p->num_splats, "ssr_projection_bwd", "visible count out of range");
         if (p->n_visible == 0) return 0;
     }
-    const dim3 grid((unsigned)ceil_div(p->visible_ids ? p->n_visible : p->num_splats, kProjBlock)), block(kProjBlock);
+    const int64_t work = packed ? p->num_packed : (p->visible_ids ? p->n_visible : p->num_splats);
+    const dim3 grid((unsigned)ceil_div(work, kProjBlock)), block(kProjBlock);
     hipStream_t s = as_stream(stream);
 #define SSR_LAUNCH_BWD(D)                                                                          \
     if (p->accumulate) hipLaunchKernelGGL((projection_bwd_kernel<D, true>), grid, block, 0, s, *p); \

@@ -30,7 +30,7 @@ SYMBOLS = {
     "ssrh_last_n_isects": (C.c_int64, []),
     "ssrh_last_n_visible": (C.c_int64, []),
     "ssrh_last_stage_times": (C.c_int, [vp]),
-    "ssrh_time_iterations": (C.c_int, [C.c_int, vp, vp, vp, C.c_int, vp]),
+    "ssrh_time_iterations": (C.c_int, [C.c_int, C.c_int, vp, vp, vp, C.c_int, vp]),
     "ssrh_pool_bytes": (C.c_size_t, []),
 }
 
@@ -62,15 +62,18 @@ CACHE = dict(aabb=(0, np.float32), sort_depth=(1, np.float32), xy=(2, np.float32
              conic=(4, np.float32), opac=(5, np.float32), rgb=(6, np.float32), sorted_ids=(7, np.int64),
              sorted_flat=(8, np.int32), offsets=(9, np.int32), last_ids=(10, np.int32), radii=(11, np.float32),
              v_xy=(12, np.float32), v_depth=(13, np.float32), v_conic=(14, np.float32), v_opac=(15, np.float32),
-             v_rgb=(16, np.float32))
+             v_rgb=(16, np.float32), gaussian_ids=(17, np.int32), camera_ids=(18, np.int32))
 
 
 class Engine:
     """Drives the engine harness for one scene: upload once, then forward / backward."""
 
     def __init__(self, scene, device=0, fuse_tile_count=True, visible_list=True, packed_rows=True, overwrite_world_grads=True,
-                 stage_profiling=False, sh_degree=3):
+                 stage_profiling=False, sh_degree=3, packed_projection=False):
+        """packed_projection: forward_3dgs(packed=true), the compacted projection outputs of
+        projection_3dgs_packed_forward (the visible-splat work list then has no role)."""
         self.h = load()
+        self.packed_projection = bool(packed_projection)
         self.sc = scene
         self.sh_degree = sh_degree
         check(self.h.ssrh_init(device))
@@ -106,14 +109,14 @@ class Engine:
         check(self.h.ssrh_set_options(*self.opts, int(on)))
 
     def forward(self):
-        check(self.h.ssrh_forward_3dgs(b"3dgs", self.sh_degree, 0, 0, 0))
+        check(self.h.ssrh_forward_3dgs(b"3dgs", self.sh_degree, int(self.packed_projection), 0, 0))
 
     def backward(self):
         check(self.h.ssrh_backward_from_render_grad(self.d_vrgb.ptr, self.d_vdepth.ptr, self.d_vT.ptr))
 
     def time_iterations(self, iters):
         ms = np.zeros(iters, np.float32)
-        check(self.h.ssrh_time_iterations(self.sh_degree, self.d_vrgb.ptr, self.d_vdepth.ptr, self.d_vT.ptr,
+        check(self.h.ssrh_time_iterations(self.sh_degree, int(self.packed_projection), self.d_vrgb.ptr, self.d_vdepth.ptr, self.d_vT.ptr,
                                           iters, ms.ctypes.data))
         return ms
 

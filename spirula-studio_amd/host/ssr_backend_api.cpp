@@ -251,6 +251,77 @@ projection_3dgs_forward(const int64_t num_splats, const int max_sh_degree,
     return std::make_tuple(aabb, depths, screen);
 }
 
+std::tuple<DeviceVector<int32_t>, DeviceVector<int32_t>, DeviceVector<float4>, DeviceVector<float>,
+           std::vector<DeviceTensorFloatND>>
+projection_3dgs_packed_forward(const int64_t num_splats, const int max_sh_degree,
+                               const std::vector<DeviceTensorFloatND>& in_splats, TorchTensorView viewmats,
+                               TorchTensorView intrins, const uint32_t image_width, const uint32_t image_height,
+                               const std::string camera_model, const std::string distortion, const TorchTensorView,
+                               DeviceVector<float> radii, const std::optional<TorchTensorView> sh_value_packed,
+                               const std::optional<TorchTensorView> sh_value_bounds, const uint32_t num_sh_buffer,
+                               const int sh_value_bits, const int64_t sh_bounds_stride) {
+    require_no_distortion(distortion);
+    ssr_projection_packed_params p;
+    std::memset(&p, 0, sizeof(p));
+    p.num_splats = num_splats;
+    p.sh_degree = max_sh_degree;
+    p.world = world_of(in_splats);
+    p.sh = sh_of(sh_value_packed, sh_value_bounds, num_sh_buffer, sh_value_bits, sh_bounds_stride);
+    p.camera = camera_of(camera_model, viewmats, intrins, image_width, image_height);
+    p.radii = radii.data_ptr();
+    p.scratch_bytes = ssr_projection_packed_scratch_bytes(num_splats);
+    p.scratch = DevicePool::global().acquire<uint8_t>(PoolSlot::ProjPackedScratch, p.scratch_bytes);
+    p.nnz = DevicePool::global().acquire<int64_t>(PoolSlot::ProjPackedNnz, 1);
+    // the work list and its counters belong to the non-packed form
+    g_visible_ids = nullptr; g_n_visible = -1; g_counters = nullptr;
+    g_counts_fused = false; g_packed_rows = nullptr; g_packed_for_xy = nullptr;
+    StageTimer t(&g_times.k1);
+    ok(ssr_projection_packed_mask(&p, nullptr), "projection_3dgs_packed_forward/mask");
+    int64_t nnz = 0;
+    if (num_splats > 0) ok(ssr_read_i64(p.nnz, &nnz, 1, nullptr), "projection_3dgs_packed_forward/readback");
+    g_n_visible = nnz;
+    DeviceVector<int32_t> camera_ids, gaussian_ids;
+    DeviceVector<float4> aabb;
+    DeviceVector<float> depths;
+    if (nnz == 0) {   // nothing visible: empty (null) views, which every later stage treats as "no work"
+        std::vector<DeviceTensorFloatND> none = {
+            DeviceTensorFloatND(nullptr, {0, 2}), DeviceTensorFloatND(nullptr, {0, 1}), DeviceTensorFloatND(nullptr, {0, 3}),
+            DeviceTensorFloatND(nullptr, {0, 1}), DeviceTensorFloatND(nullptr, {0, 3})};
+        return std::make_tuple(camera_ids, gaussian_ids, aabb, depths, none);
+    }
+    camera_ids.resize(PoolSlot::ProjCameraIds, nnz);
+    // two id buffers alternate, so that the list a backward ran over outlives the next projection
+    g_list_toggle ^= 1;
+    gaussian_ids.resize(g_list_toggle ? PoolSlot::ProjGaussianIdsB : PoolSlot::ProjGaussianIds, nnz);
+    aabb.resize(PoolSlot::ProjAabb, nnz);
+    depths.resize(PoolSlot::ProjDepths, nnz);
+    float* xy = DevicePool::global().acquire<float>(PoolSlot::ProjScreenXy, (size_t)(nnz * 2));
+    float* dp = DevicePool::global().acquire<float>(PoolSlot::ProjScreenDepth, (size_t)nnz);
+    float* cn = DevicePool::global().acquire<float>(PoolSlot::ProjScreenConic, (size_t)(nnz * 3));
+    float* op = DevicePool::global().acquire<float>(PoolSlot::ProjScreenOpac, (size_t)nnz);
+    float* rg = DevicePool::global().acquire<float>(PoolSlot::ProjScreenRgb, (size_t)(nnz * 3));
+    std::vector<DeviceTensorFloatND> screen = {
+        DeviceTensorFloatND(xy, {nnz, 2}), DeviceTensorFloatND(dp, {nnz, 1}), DeviceTensorFloatND(cn, {nnz, 3}),
+        DeviceTensorFloatND(op, {nnz, 1}), DeviceTensorFloatND(rg, {nnz, 3})};
+    {
+        p.max_rows = nnz;
+        p.camera_ids = camera_ids.data_ptr(); p.gaussian_ids = gaussian_ids.data_ptr();
+        p.aabb = (float*)aabb.data_ptr(); p.sort_depth = depths.data_ptr();
+        p.screen.xy = xy; p.screen.depth = dp; p.screen.conic = cn; p.screen.opac = op; p.screen.rgb = rg;
+        if (g_opts.fuse_tile_count) {
+            p.tiles_per_splat = DevicePool::global().acquire<int64_t>(PoolSlot::IsectTilesPerSplat, (size_t)nnz);
+            g_counts_fused = true;
+        }
+        if (g_opts.packed_rows) {
+            g_packed_rows = DevicePool::global().acquire<float>(PoolSlot::ProjPackedRows, (size_t)(nnz * 12));
+            g_packed_for_xy = xy;
+            p.packed_rows = g_packed_rows;
+        }
+        ok(ssr_projection_packed_emit(&p, nullptr), "projection_3dgs_packed_forward/emit");
+    }
+    return std::make_tuple(camera_ids, gaussian_ids, aabb, depths, screen);
+}
+
 int64_t intersect_tile_count(int width, int height) {
     return (int64_t)((width + 15) / 16) * (int64_t)((height + 15) / 16);
 }
@@ -260,7 +331,9 @@ do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, 
                           DeviceTensorFloatND* proj_conic, DeviceTensorFloatND* proj_opac, const uint32_t I,
                           TorchTensorView, const uint32_t image_width, const uint32_t image_height,
                           DeviceVector<int32_t>* image_ids, const int32_t* tile_active) {
-    if (image_ids) throw std::runtime_error("do_intersect_tile_generic: packed mode is not built in this backend");
+    // Packed mode (image_ids given): `total` rows, one per visible (camera, splat) pair, and the
+    // values written to flatten_ids are row numbers (src/kernels/tile/IntersectTile.cu:386-409). With
+    // the single camera this backend runs, every image id is 0 and the array itself is not read.
     if (tile_active) throw std::runtime_error("do_intersect_tile_generic: the tile-skip mask is not built in this backend");
     if (!proj_xy || !proj_conic || !proj_opac)
         throw std::runtime_error("do_intersect_tile_generic: AABB mode is not built in this backend (ellipse mode is)");
@@ -333,7 +406,10 @@ rasterize_to_pixels_3dgs_fwd(int64_t num_splats, std::vector<DeviceTensorFloatND
                              DeviceVector<int32_t> gaussian_ids, const uint32_t image_width, const uint32_t image_height,
                              const DeviceTensor3D<int32_t> tile_offsets, const DeviceVector<int32_t> flatten_ids,
                              DistortionType dist_type, bool output_median) {
-    if (gaussian_ids.data_ptr()) throw std::runtime_error("rasterize_to_pixels_3dgs_fwd: packed mode is not built in this backend");
+    // gaussian_ids (packed mode) maps a screen row to its world row; the 3dgs fragment is read from
+    // the screen row alone (src/kernels/raster/RasterizationEval3DFwd_kernel.cuh:183-184), so it is
+    // accepted and not read.
+    if (gaussian_ids.data_ptr()) num_splats = gaussian_ids.size();
     if (dist_type != DistortionType::None) throw std::runtime_error("rasterize_to_pixels_3dgs_fwd: depth distortion is not built in this backend");
     if (output_median) throw std::runtime_error("rasterize_to_pixels_3dgs_fwd: median depth is not built in this backend");
     const int64_t I = tile_offsets.size<0>();
@@ -371,7 +447,7 @@ rasterize_to_pixels_3dgs_bwd(int64_t num_splats, std::vector<DeviceTensorFloatND
                              const DeviceTensor3D<float> v_median, std::optional<RenderOutput::TensorTuple>,
                              std::optional<std::vector<DeviceTensorFloatND>> v_splats_w,
                              std::optional<std::vector<DeviceTensorFloatND>> v_splats_s) {
-    if (gaussian_ids.data_ptr()) throw std::runtime_error("rasterize_to_pixels_3dgs_bwd: packed mode is not built in this backend");
+    if (gaussian_ids.data_ptr()) num_splats = gaussian_ids.size();   // packed: v_screen has one row per screen row
     if (dist_type != DistortionType::None) throw std::runtime_error("rasterize_to_pixels_3dgs_bwd: depth distortion is not built in this backend");
     if (accum_mode != DensifyAccumMode::None || accum_weight_map.data_ptr())
         throw std::runtime_error("rasterize_to_pixels_3dgs_bwd: accumulation weights are not built in this backend");
@@ -423,11 +499,12 @@ void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
                               const std::optional<TorchTensorView> sh_value_bounds, const uint32_t num_sh_buffer,
                               const int sh_value_bits, const int64_t sh_bounds_stride) {
     require_no_distortion(distortion);
-    if (camera_ids.data_ptr() || gaussian_ids.data_ptr())
-        throw std::runtime_error("projection_3dgs_backward: packed mode is not built in this backend");
     if (v_viewmats) throw std::runtime_error("projection_3dgs_backward: camera pose gradients are not built in this backend");
-    if (num_splats == 0) return;   // src/kernels/projection/ProjectionBwd.cu:86-87
-    if (!aabb.data_ptr()) throw std::runtime_error("projection_3dgs_backward: aabb is null");   // :89-97
+    const bool is_packed = camera_ids.data_ptr() && gaussian_ids.data_ptr();   // src/kernels/projection/ProjectionBwd.cu:80
+    g_bwd_list = nullptr; g_bwd_count = 0;
+    if (num_splats == 0) return;   // ProjectionBwd.cu:86-87
+    // a packed forward with no visible splat leaves ids and aabb null: nothing to do (ProjectionBwd.cu:89-97)
+    if (!is_packed && !aabb.data_ptr()) return;
     ssr_projection_bwd_params p;
     std::memset(&p, 0, sizeof(p));
     p.num_splats = num_splats;
@@ -439,8 +516,11 @@ void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
     p.v_screen = screen_of(v_splats_screen);
     p.v_world = world_of(v_splats_world);
     p.accumulate = g_opts.overwrite_world_grads ? 0 : 1;
-    g_bwd_list = nullptr; g_bwd_count = 0;
-    if (g_visible_ids && g_n_visible >= 0) {
+    if (is_packed) {
+        p.aabb = nullptr;
+        p.packed_gaussian_ids = gaussian_ids.data_ptr(); p.num_packed = camera_ids.size();
+        g_bwd_list = gaussian_ids.data_ptr(); g_bwd_count = camera_ids.size();
+    } else if (g_visible_ids && g_n_visible >= 0) {
         p.visible_ids = g_visible_ids; p.n_visible = g_n_visible;
         g_bwd_list = g_visible_ids; g_bwd_count = g_n_visible;
     }

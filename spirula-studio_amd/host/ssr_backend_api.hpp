@@ -4,6 +4,7 @@
 // definitions in place of the CUDA (src/kernels/**) or Vulkan (src/backend/vulkan/kernels/**) ones.
 //
 //   projection_3dgs_forward        src/kernels/projection/ProjectionFwd.cuh:18-36
+//   projection_3dgs_packed_forward src/kernels/projection/ProjectionPackedFwd.cuh:18-37
 //   do_intersect_tile_generic      src/kernels/tile/IntersectTile.cuh:25-41
 //   rasterize_to_pixels_3dgs_fwd   src/kernels/raster/RasterizationFwd.cuh:18-38
 //   rasterize_to_pixels_3dgs_bwd   src/kernels/raster/RasterizationBwd.cuh:18-48
@@ -19,6 +20,25 @@
 
 std::tuple<DeviceTensor2D<float4>, DeviceTensor2D<float>, std::vector<DeviceTensorFloatND>>
 projection_3dgs_forward(
+    const int64_t num_splats, const int max_sh_degree,
+    const std::vector<DeviceTensorFloatND>& in_splats,
+    TorchTensorView viewmats, TorchTensorView intrins,
+    const uint32_t image_width, const uint32_t image_height,
+    const std::string camera_model, const std::string distortion,
+    const TorchTensorView dist_coeffs,
+    DeviceVector<float> radii,
+    const std::optional<TorchTensorView> sh_value_packed,
+    const std::optional<TorchTensorView> sh_value_bounds,
+    const uint32_t num_sh_buffer,
+    const int sh_value_bits,
+    const int64_t sh_bounds_stride);
+
+// Packed form: (camera_ids[nnz], gaussian_ids[nnz], aabb[nnz], sorting depths[nnz], screen[5] with
+// nnz rows), visible splats only, in ascending splat order. Blocks on the readback of nnz, as the
+// reference does (src/kernels/projection/ProjectionPackedFwd.cu:112-119).
+std::tuple<DeviceVector<int32_t>, DeviceVector<int32_t>, DeviceVector<float4>, DeviceVector<float>,
+           std::vector<DeviceTensorFloatND>>
+projection_3dgs_packed_forward(
     const int64_t num_splats, const int max_sh_degree,
     const std::vector<DeviceTensorFloatND>& in_splats,
     TorchTensorView viewmats, TorchTensorView intrins,

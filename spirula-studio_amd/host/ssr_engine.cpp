@@ -42,16 +42,19 @@ void alloc_grad_buffers() {
     g.features_dc.resize(PoolSlot::GradFeaturesDc, n); g.features_sh.resize(PoolSlot::GradFeaturesSh, n, engine().num_sh);
     const auto& o = ssr_ext::options();
     if (engine().optim.skip_grad_zero) return;
-    if (o.overwrite_world_grads && !o.visible_list) return;   // K9 overwrites every row itself
-    // Every row is zero except those the last backward wrote through its visible list: when that
-    // list is short, zero just those rows instead of refilling all N (the refill is 236 B per splat).
-    if (o.visible_list && o.overwrite_world_grads && g.dirty_list && g.dirty_key == (const void*)g.means.data_ptr() &&
+    const bool listed = o.visible_list || engine().packed;   // the backward touches listed rows only
+    if (o.overwrite_world_grads && !listed) return;   // K9 overwrites every row itself
+    // Every row is zero except those the last backward wrote through its list (the visible-splat
+    // list, or gaussian_ids in packed mode): when that list is short, zero just those rows instead
+    // of refilling all N (the refill is 236 B per splat).
+    if (listed && o.overwrite_world_grads && g.dirty_valid && g.dirty_key == (const void*)g.means.data_ptr() &&
         g.dirty_count * 2 < n) {
         std::vector<DeviceTensorFloatND> v_world = {
             DeviceTensorFloatND(g.means), DeviceTensorFloatND(g.quats), DeviceTensorFloatND(g.scales),
             DeviceTensorFloatND((float*)g.opacities.data_ptr(), {g.opacities.size(), 1}),
             DeviceTensorFloatND(g.features_dc), DeviceTensorFloatND(g.features_sh)};
-        ssr_ext::zero_world_rows(v_world, g.dirty_list, g.dirty_count, &engine().fwd.aabb);
+        if (g.dirty_count > 0)
+            ssr_ext::zero_world_rows(v_world, g.dirty_list, g.dirty_count, engine().packed ? nullptr : &engine().fwd.aabb);
         return;
     }
     g.means.zero(); g.quats.zero(); g.scales.zero(); g.opacities.zero(); g.features_dc.zero(); g.features_sh.zero();
@@ -110,7 +113,6 @@ void set_camera_params(int width, int height, std::string camera_model, std::str
 
 void forward_3dgs(std::string primitive, int sh_degree, bool packed, bool output_median, int dist_type_int) {
     if (primitive != "3dgs") throw std::runtime_error("forward_3dgs: primitive '" + primitive + "' is not built in this backend");
-    if (packed) throw std::runtime_error("forward_3dgs: packed projection is not built in this backend");
     auto& E = engine();
     if (!E.world.initialized) throw std::runtime_error("forward_3dgs: set_data_3dgs must be called first");
     E.primitive = primitive; E.sh_degree = sh_degree; E.packed = packed;
@@ -124,21 +126,41 @@ void forward_3dgs(std::string primitive, int sh_degree, bool packed, bool output
     E.optim.radii.resize(PoolSlot::EngRadii, E.max_num_splats);
     if (!E.optim.skip_grad_zero) E.optim.radii.zero();
 
-    auto [aabb, depths, screen] = projection_3dgs_forward(
-        N, sh_degree, in_splats, E.camera.viewmats, E.camera.intrins, (uint32_t)E.camera.width,
-        (uint32_t)E.camera.height, E.camera.model_str, E.camera.distortion_str, E.camera.dist_coeffs, E.optim.radii,
-        E.world.sh_packed, E.world.sh_bounds, (uint32_t)E.num_sh, E.world.sh_value_bits, E.world.sh_bounds_stride);
-    E.fwd.aabb = aabb; E.fwd.depths = depths; E.fwd.splats_s = screen;
+    DeviceTensorFloatND aabb_nd, depths_nd;
+    std::vector<DeviceTensorFloatND> screen;
+    if (packed) {   // src/engine/EngineForward.cpp:119-165
+        auto [cam_ids, gauss_ids, aabb_vec, depths_vec, scr] = projection_3dgs_packed_forward(
+            N, sh_degree, in_splats, E.camera.viewmats, E.camera.intrins, (uint32_t)E.camera.width,
+            (uint32_t)E.camera.height, E.camera.model_str, E.camera.distortion_str, E.camera.dist_coeffs, E.optim.radii,
+            E.world.sh_packed, E.world.sh_bounds, (uint32_t)E.num_sh, E.world.sh_value_bits, E.world.sh_bounds_stride);
+        E.fwd.camera_ids = cam_ids; E.fwd.gaussian_ids = gauss_ids;
+        E.fwd.aabb = DeviceTensor2D<float4>(aabb_vec.data_ptr(), aabb_vec.size(), 1);   // [nnz, 1] view for backward
+        E.fwd.depths = DeviceTensor2D<float>(depths_vec.data_ptr(), 1, depths_vec.size());
+        screen = scr;
+        aabb_nd = DeviceTensorFloatND((float*)aabb_vec.data_ptr(), {aabb_vec.size(), 4});
+        depths_nd = DeviceTensorFloatND(depths_vec.data_ptr(), {depths_vec.size()});
+    } else {
+        auto [aabb, depths, scr] = projection_3dgs_forward(
+            N, sh_degree, in_splats, E.camera.viewmats, E.camera.intrins, (uint32_t)E.camera.width,
+            (uint32_t)E.camera.height, E.camera.model_str, E.camera.distortion_str, E.camera.dist_coeffs, E.optim.radii,
+            E.world.sh_packed, E.world.sh_bounds, (uint32_t)E.num_sh, E.world.sh_value_bits, E.world.sh_bounds_stride);
+        E.fwd.camera_ids = DeviceVector<int32_t>(); E.fwd.gaussian_ids = DeviceVector<int32_t>();
+        E.fwd.aabb = aabb; E.fwd.depths = depths;
+        screen = scr;
+        aabb_nd = DeviceTensorFloatND((float*)aabb.data_ptr(), {aabb.numel(), 4});
+        depths_nd = DeviceTensorFloatND(depths.data_ptr(), {depths.numel()});
+    }
+    E.fwd.splats_s = screen;
 
-    DeviceTensorFloatND aabb_nd((float*)aabb.data_ptr(), {aabb.numel(), 4});
-    DeviceTensorFloatND depths_nd(depths.data_ptr(), {depths.numel()});
+    DeviceVector<int32_t>* image_ids_ptr = nullptr;   // EngineForward.cpp:215-217
+    if (packed && E.fwd.camera_ids.data_ptr() != nullptr) image_ids_ptr = &E.fwd.camera_ids;
     auto [ids, flat, offsets] = do_intersect_tile_generic(
         aabb_nd, depths_nd, &screen[0], &screen[2], &screen[3], (uint32_t)E.camera.num, E.camera.intrins,
-        (uint32_t)E.camera.width, (uint32_t)E.camera.height, nullptr, nullptr);
+        (uint32_t)E.camera.width, (uint32_t)E.camera.height, image_ids_ptr, nullptr);
     E.fwd.isect_ids = ids; E.fwd.flatten_ids = flat; E.fwd.tile_offsets = offsets;
 
     auto [renders, Ts, last, dist, median] = rasterize_to_pixels_3dgs_fwd(
-        N, in_splats, screen, DeviceVector<int32_t>{}, (uint32_t)E.camera.width, (uint32_t)E.camera.height, offsets, flat,
+        N, in_splats, screen, E.fwd.gaussian_ids, (uint32_t)E.camera.width, (uint32_t)E.camera.height, offsets, flat,
         (DistortionType)dist_type_int, output_median);
     E.fwd.renders = renders; E.fwd.render_Ts = Ts; E.fwd.last_ids = last;
 }
@@ -169,7 +191,7 @@ void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorV
 
     // _engine_raster_proj_backward, non-fused branch (src/engine/EngineLoss.cpp:218-240,294-390)
     auto [vw, vs, accum] = rasterize_to_pixels_3dgs_bwd(
-        E.cur_num_splats, E.fwd.splats_w, E.fwd.splats_s, DeviceVector<int32_t>{}, (uint32_t)W, (uint32_t)H,
+        E.cur_num_splats, E.fwd.splats_w, E.fwd.splats_s, E.fwd.gaussian_ids, (uint32_t)W, (uint32_t)H,
         E.fwd.tile_offsets, E.fwd.flatten_ids, E.fwd.render_Ts, E.fwd.last_ids, E.fwd.renders, std::nullopt,
         DistortionType::None, DeviceTensor3D<float>{}, DensifyAccumMode::None, v_renders, v_Ts_t, DeviceTensor3D<float>{},
         std::nullopt, std::nullopt, std::nullopt);
@@ -180,11 +202,13 @@ void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorV
         DeviceTensorFloatND(E.grad.features_dc), DeviceTensorFloatND(E.grad.features_sh)};
     projection_3dgs_backward(
         E.cur_num_splats, E.sh_degree, E.fwd.splats_w, E.camera.viewmats, E.camera.intrins, (uint32_t)W, (uint32_t)H,
-        E.camera.model_str, E.camera.distortion_str, E.camera.dist_coeffs, DeviceVector<int32_t>{}, DeviceVector<int32_t>{},
+        E.camera.model_str, E.camera.distortion_str, E.camera.dist_coeffs, E.fwd.camera_ids, E.fwd.gaussian_ids,
         E.fwd.aabb, vs, v_world, nullptr, E.world.sh_packed, E.world.sh_bounds, (uint32_t)E.num_sh, E.world.sh_value_bits,
         E.world.sh_bounds_stride);
     E.grad.dirty_list = ssr_ext::last_backward_list(&E.grad.dirty_count);
     E.grad.dirty_key = (const void*)E.grad.means.data_ptr();
+    // with no list the backward may have written any row; with one, exactly the listed rows
+    E.grad.dirty_valid = E.grad.dirty_list != nullptr || (E.packed && E.fwd.gaussian_ids.size() == 0);
 }
 
 void engine_copy_render_to_host(TorchTensorView out_rgb, TorchTensorView out_depth, TorchTensorView out_Ts,
@@ -296,7 +320,8 @@ int ssrh_copy_grads_to_host(float* means, float* quats, float* scales, float* op
 
 // Device addresses of the forward cache, for tests that compare intermediate buffers.
 //   which: 0 aabb, 1 sort depths, 2..6 screen xy/depth/conic/opac/rgb, 7 sorted keys, 8 sorted ids,
-//          9 tile offsets, 10 last_ids, 11 radii, 12..16 v_screen xy/depth/conic/opac/rgb
+//          9 tile offsets, 10 last_ids, 11 radii, 12..16 v_screen xy/depth/conic/opac/rgb,
+//          17 gaussian_ids, 18 camera_ids (packed projection)
 int ssrh_cache_pointer(int which, void** ptr, int64_t* count) {
     return guard([&] {
         auto& E = engine();
@@ -311,6 +336,8 @@ int ssrh_cache_pointer(int which, void** ptr, int64_t* count) {
             case 10: *ptr = E.fwd.last_ids.data_ptr(); *count = E.fwd.last_ids.numel(); break;
             case 11: *ptr = E.optim.radii.data_ptr(); *count = E.optim.radii.size(); break;
             case 12: case 13: case 14: case 15: case 16: nd(E.grad.v_screen.at(which - 12)); break;
+            case 17: *ptr = E.fwd.gaussian_ids.data_ptr(); *count = E.fwd.gaussian_ids.size(); break;
+            case 18: *ptr = E.fwd.camera_ids.data_ptr(); *count = E.fwd.camera_ids.size(); break;
             default: throw std::runtime_error("unknown cache buffer");
         }
     });
@@ -330,13 +357,13 @@ int ssrh_last_stage_times(float* out9) {
 // Runs `iters` forward+backward iterations back to back with device-resident cotangents and
 // returns the elapsed device time of each (events on the launch stream, one synchronise per
 // iteration at its end).
-int ssrh_time_iterations(int sh_degree, const float* v_rgb_dev, const float* v_depth_dev, const float* v_Ts_dev, int iters,
-                         float* ms_out) {
+int ssrh_time_iterations(int sh_degree, int packed, const float* v_rgb_dev, const float* v_depth_dev, const float* v_Ts_dev,
+                         int iters, float* ms_out) {
     return guard([&] {
         ssr_event_t a = ssr_event_create(), b = ssr_event_create();
         for (int i = 0; i < iters; i++) {
             ssr_event_record(a, nullptr);
-            forward_3dgs("3dgs", sh_degree, false, false, 0);
+            forward_3dgs("3dgs", sh_degree, packed != 0, false, 0);
             const int64_t C = engine().camera.num, H = engine().camera.height, W = engine().camera.width;
             engine_backward_from_render_grad(tv(v_rgb_dev, 4, {C, H, W, 3}), tv(v_depth_dev, 4, {C, H, W, 1}), tv(v_Ts_dev, 4, {C, H, W, 1}));
             ssr_event_record(b, nullptr);

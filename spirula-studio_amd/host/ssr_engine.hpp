@@ -36,6 +36,7 @@ struct EngineState {
     struct {
         std::vector<DeviceTensorFloatND> splats_w, splats_s;
         DeviceTensor2D<float4> aabb; DeviceTensor2D<float> depths;
+        DeviceVector<int32_t> camera_ids, gaussian_ids;   // packed projection only
         DeviceVector<int64_t> isect_ids; DeviceVector<int32_t> flatten_ids; DeviceTensor3D<int32_t> tile_offsets;
         RenderOutput::TensorTuple renders; DeviceTensor3D<float> render_Ts; DeviceTensor3D<int32_t> last_ids;
     } fwd;
@@ -48,6 +49,7 @@ struct EngineState {
         const int32_t* dirty_list = nullptr;
         int64_t dirty_count = 0;
         const void* dirty_key = nullptr;
+        bool dirty_valid = false;
     } grad;
 };
 EngineState& engine();

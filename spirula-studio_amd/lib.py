@@ -65,13 +65,24 @@ class ProjectionBwdParams(C.Structure):
     _fields_ = [("num_splats", C.c_int64), ("sh_degree", C.c_int32), ("world", World),
                 ("sh", ShQuant), ("camera", Camera), ("aabb", vp), ("v_screen", Screen),
                 ("v_world", World), ("accumulate", C.c_int32), ("visible_ids", vp),
-                ("n_visible", C.c_int64)]
+                ("n_visible", C.c_int64), ("packed_gaussian_ids", vp), ("num_packed", C.c_int64)]
+
+
+class ProjectionPackedParams(C.Structure):
+    _fields_ = [("num_splats", C.c_int64), ("sh_degree", C.c_int32), ("world", World),
+                ("sh", ShQuant), ("camera", Camera), ("radii", vp), ("scratch", vp),
+                ("scratch_bytes", C.c_size_t), ("nnz", vp), ("max_rows", C.c_int64),
+                ("camera_ids", vp), ("gaussian_ids", vp), ("aabb", vp), ("sort_depth", vp),
+                ("screen", Screen), ("tiles_per_splat", vp), ("packed_rows", vp)]
 
 
 # every symbol include/ssr_backend.h declares: (name, restype, argtypes)
 _i64, _u32, _i32, _sz = C.c_int64, C.c_uint32, C.c_int, C.c_size_t
 SYMBOLS = {
     "ssr_projection_fwd": (_i32, [C.POINTER(ProjectionFwdParams), vp]),
+    "ssr_projection_packed_scratch_bytes": (_sz, [_i64]),
+    "ssr_projection_packed_mask": (_i32, [C.POINTER(ProjectionPackedParams), vp]),
+    "ssr_projection_packed_emit": (_i32, [C.POINTER(ProjectionPackedParams), vp]),
     "ssr_tile_count": (_i32, [_i64, vp, vp, vp, vp, _u32, _u32, vp, vp]),
     "ssr_scan_scratch_bytes": (_sz, [_i64]),
     "ssr_inclusive_sum_i64": (_i32, [vp, vp, _i64, vp, vp, _sz, vp]),

@@ -9,9 +9,16 @@ import numpy as np
 
 
 class GpuRun:
-    def __init__(self, pkg, scene, sh_degree=3, use_list=False, use_packed=False):
+    def __init__(self, pkg, scene, sh_degree=3, use_list=False, use_packed=False, packed_projection=False,
+                 read_nnz=True):
+        """use_packed: 48-byte fragment rows for the compositing kernels. packed_projection: the
+        compacted (nnz-row) projection outputs of projection_3dgs_packed_forward; read_nnz=False
+        sizes the outputs for all N splats instead of reading nnz back between the two calls."""
         self.use_list = use_list
         self.use_packed = use_packed
+        self.packed_projection = packed_projection
+        self.read_nnz = read_nnz
+        assert not (packed_projection and use_list)
         self.L = pkg.lib
         self.lib = self.L.load()
         self.check = self.L.check
@@ -43,6 +50,7 @@ class GpuRun:
         self.d["counters"] = D((2,), np.int64)     # [n_isects, n_visible]
         self.d["packed"] = D((n, 12), np.float32)
         self.V = None
+        self.rows = n          # rows of the projection outputs: N, or nnz in packed mode
 
     def ptr(self, k):
         a = self.d.get(k)
@@ -78,7 +86,48 @@ class GpuRun:
         return s
 
     # ---- stages ----
+    def projection_packed_fwd(self, fused_count=False):
+        D = self.L.DeviceArray
+        n = self.n
+        self.d["radii"].fill_zero()
+        sb = self.lib.ssr_projection_packed_scratch_bytes(n)
+        self.d["pk_scratch"] = D((sb,), np.uint8)
+        self.d["nnz"] = D((1,), np.int64)
+        p = self.L.ProjectionPackedParams()
+        p.num_splats, p.sh_degree = n, self.sh_degree
+        p.world, p.sh, p.camera = self.world(), self.shq(), self.camera()
+        p.radii, p.scratch, p.scratch_bytes, p.nnz = self.ptr("radii"), self.ptr("pk_scratch"), sb, self.ptr("nnz")
+        self.check(self.lib.ssr_projection_packed_mask(C.byref(p), None))
+        if self.read_nnz:
+            k = (C.c_int64 * 1)(0)
+            self.check(self.lib.ssr_read_i64(self.ptr("nnz"), k, 1, None))
+            cap = int(k[0])
+        else:
+            cap = n
+        for nm, shape, dt in [("camera_ids", (cap,), np.int32), ("gaussian_ids", (cap,), np.int32),
+                              ("aabb", (cap, 4), np.float32), ("sort_depth", (cap,), np.float32),
+                              ("xy", (cap, 2), np.float32), ("depth", (cap,), np.float32),
+                              ("conic", (cap, 3), np.float32), ("opac", (cap,), np.float32),
+                              ("rgb", (cap, 3), np.float32), ("counts", (cap,), np.int64),
+                              ("cum", (cap,), np.int64), ("packed", (cap, 12), np.float32)]:
+            self.d[nm] = D(shape, dt)
+            if cap:   # poison, so that rows past nnz are seen to stay untouched
+                self.check(self.lib.ssr_fill_u32(self.d[nm].ptr, 0x7fc12345, self.d[nm].nbytes // 4, None))
+        p.max_rows = cap
+        p.camera_ids, p.gaussian_ids = self.ptr("camera_ids"), self.ptr("gaussian_ids")
+        p.aabb, p.sort_depth, p.screen = self.ptr("aabb"), self.ptr("sort_depth"), self.screen()
+        p.tiles_per_splat = self.ptr("counts") if fused_count else None
+        p.packed_rows = self.ptr("packed") if self.use_packed else None
+        self.check(self.lib.ssr_projection_packed_emit(C.byref(p), None))
+        if not self.read_nnz:
+            k = (C.c_int64 * 1)(0)
+            self.check(self.lib.ssr_read_i64(self.ptr("nnz"), k, 1, None))
+        self.nnz = self.rows = int(k[0])
+        self.cap = cap
+
     def projection_fwd(self, fused_count=False):
+        if self.packed_projection:
+            return self.projection_packed_fwd(fused_count)
         for k in ["radii"]:
             self.d[k].fill_zero()
         p = self.L.ProjectionFwdParams()
@@ -97,7 +146,7 @@ class GpuRun:
 
     def tiles(self, fused_count=False):
         sc, D = self.sc, self.L.DeviceArray
-        n = self.n
+        n = self.rows
         if not fused_count:
             self.check(self.lib.ssr_tile_count(n, self.ptr("aabb"), self.ptr("xy"), self.ptr("conic"),
                                                self.ptr("opac"), sc.width, sc.height, self.ptr("counts"), None))
@@ -146,7 +195,7 @@ class GpuRun:
                              ("r_T", (h, w), np.float32), ("r_last", (h, w), np.int32)]:
             self.d[k] = D(shape, dt)
         p = self.L.RasterFwdParams()
-        p.num_splats, p.screen, p.width, p.height = self.n, self.screen(), w, h
+        p.num_splats, p.screen, p.width, p.height = self.rows, self.screen(), w, h
         p.tile_offsets, p.flatten_ids, p.n_isects = self.ptr("offsets"), self.ptr(self.vals), self.K
         p.render_rgb, p.render_depth, p.render_T, p.last_ids = (self.ptr("r_rgb"), self.ptr("r_depth"),
                                                                 self.ptr("r_T"), self.ptr("r_last"))
@@ -157,7 +206,7 @@ class GpuRun:
 
     def raster_bwd(self, v_rgb=None, v_depth=None, v_T=None):
         sc, D = self.sc, self.L.DeviceArray
-        n = self.n
+        n = self.rows
         self.d["g_rgb"] = D.from_host(np.asarray(sc.v_rgb if v_rgb is None else v_rgb, np.float32))
         self.d["g_depth"] = D.from_host(np.asarray(sc.v_depth if v_depth is None else v_depth, np.float32))
         self.d["g_T"] = D.from_host(np.asarray(sc.v_T if v_T is None else v_T, np.float32))
@@ -194,6 +243,11 @@ class GpuRun:
         p.accumulate = 1 if accumulate else 0
         if self.use_list:
             p.visible_ids, p.n_visible = self.ptr("vis_ids"), self.V
+        if self.packed_projection:
+            if self.rows == 0:   # nothing visible: the launcher has nothing to run (ProjectionBwd.cu:86-97)
+                return
+            p.aabb = None
+            p.packed_gaussian_ids, p.num_packed = self.ptr("gaussian_ids"), self.rows
         self.check(self.lib.ssr_projection_bwd(C.byref(p), None))
 
     def run_all(self, backward=True, fused_count=False):

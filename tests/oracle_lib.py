@@ -215,3 +215,50 @@ def pipeline(scene, sh_degree=3, backward=True):
         out["vscreen"] = raster_bwd(n, p, w, h, offs, sv, f, scene.v_rgb, scene.v_depth, scene.v_T)
         out["grads"] = projection_bwd(scene, p["aabb"], out["vscreen"], sh_degree)
     return out
+
+
+def pack_projection(p):
+    """projection_3dgs_packed_forward restated on the unpacked oracle outputs: the visibility mask
+    is the clamped-extent test (src/kernels/projection/ProjectionPackedFwd_kernel.cuh:89-93), which
+    is exactly the rule under which the unpacked kernel keeps a non-zero aabb
+    (src/kernels/projection/ProjectionFwd_kernel.cuh:97-110); the packed arrays are the visible rows
+    in ascending splat order (inclusive scan of the mask, ProjectionPackedFwd.cu:112-119)."""
+    a = p["aabb"]
+    mask = (a[:, 2] - a[:, 0] > np.float32(1e-3)) & (a[:, 3] - a[:, 1] > np.float32(1e-3))
+    gids = np.nonzero(mask)[0].astype(np.int32)
+    q = {k: np.ascontiguousarray(p[k][gids]) for k in ["aabb", "sort_depth", "xy", "depth", "conic", "opac", "rgb"]}
+    q["gaussian_ids"] = gids
+    q["camera_ids"] = np.zeros(gids.size, np.int32)
+    q["radii"] = p["radii"]
+    q["visible"] = int(gids.size)
+    return q
+
+
+def pipeline_packed(scene, sh_degree=3, backward=True):
+    """The iteration with packed projection outputs (engine path with packed=true,
+    src/engine/EngineForward.cpp:119-162,215-217): every later stage sees nnz rows, flatten ids are
+    packed row numbers, v_screen has nnz rows, and the projection backward maps row i to splat
+    gaussian_ids[i] (src/kernels/projection/ProjectionBwd_kernel.cuh:51-56)."""
+    n, w, h = scene.n, scene.width, scene.height
+    full = projection_fwd(scene, sh_degree)
+    p = pack_projection(full)
+    m = p["visible"]
+    counts = tile_count(m, p["aabb"], p["xy"], p["conic"], p["opac"], w, h)
+    cum = inclusive_sum(counts)
+    ids, flat, pads = tile_write(m, p["aabb"], p["sort_depth"], p["xy"], p["conic"], p["opac"], cum, w, h)
+    n_tiles = scene.tile_w * scene.tile_h
+    sk, sv = sort_pairs(ids, flat, 0, 32 + tile_n_bits(n_tiles))
+    offs = tile_offsets(sk, n_tiles)
+    f = raster_fwd(m, p, w, h, offs, sv)
+    out = dict(proj=p, full_proj=full, counts=counts, cum=cum, isect_ids=ids, flatten_ids=flat, pads=pads,
+               sorted_ids=sk, sorted_flat=sv, offsets=offs, fwd=f)
+    if backward:
+        vs = raster_bwd(m, p, w, h, offs, sv, f, scene.v_rgb, scene.v_depth, scene.v_T)
+        out["vscreen"] = vs
+        shapes = dict(v_xy=(n, 2), v_depth=(n,), v_conic=(n, 3), v_opac=(n,), v_rgb=(n, 3))
+        spread = {}
+        for k, shp in shapes.items():
+            spread[k] = np.zeros(shp, np.float32)
+            spread[k][p["gaussian_ids"]] = vs[k]
+        out["grads"] = projection_bwd(scene, full["aabb"], spread, sh_degree)
+    return out

@@ -82,6 +82,56 @@ def _compare(gpu, oracle, sc, label, fused_count=False, use_list=False, use_pack
     return g, r
 
 
+def _compare_packed(gpu, oracle, sc, label, fused_count=False, use_packed=False, read_nnz=True):
+    """Packed projection outputs (nnz compacted rows) through every later stage."""
+    r = oracle.pipeline_packed(sc)
+    q = r["proj"]
+    m = q["visible"]
+    print(f"[{label}] N={sc.n} {sc.width}x{sc.height} nnz={m} K={r['isect_ids'].size}", flush=True)
+    g = GpuRun(gpu, sc, use_packed=use_packed, packed_projection=True, read_nnz=read_nnz).run_all(fused_count=fused_count)
+    assert g.nnz == m
+    # K1 packed: ids exact and ascending, rows bit-exact, rows past nnz untouched
+    assert np.array_equal(g.host("gaussian_ids")[:m], q["gaussian_ids"])
+    assert not np.any(g.host("camera_ids")[:m])
+    assert np.array_equal(g.host("radii").view(np.uint32), q["radii"].view(np.uint32))
+    for k in ["aabb", "sort_depth", "xy", "depth", "conic", "opac", "rgb"]:
+        got = g.host(k)
+        assert np.array_equal(got[:m].view(np.uint32), q[k].view(np.uint32)), k
+        assert np.all(got[m:].view(np.uint32) == 0x7fc12345), k
+    # K2..K6: bit-exact, flatten ids are packed row numbers
+    assert np.array_equal(g.host("counts")[:m], r["counts"])
+    assert np.array_equal(g.host("cum")[:m], r["cum"])
+    assert g.K == r["isect_ids"].size
+    assert np.array_equal(g.unsorted_keys, r["isect_ids"])
+    assert np.array_equal(g.unsorted_vals, r["flatten_ids"])
+    assert np.array_equal(g.host(g.keys), r["sorted_ids"])
+    assert np.array_equal(g.host(g.vals), r["sorted_flat"])
+    assert np.array_equal(g.host("offsets"), r["offsets"])
+    f = r["fwd"]
+    assert np.abs(g.host("r_rgb") - f["rgb"]).max() <= IMG_TOL
+    assert np.abs(g.host("r_T") - f["T"]).max() <= IMG_TOL
+    dd = np.abs(g.host("r_depth") - f["depth"])
+    assert (dd <= IMG_TOL * np.maximum(1.0, np.abs(f["depth"]))).all()
+    assert np.array_equal(g.host("r_last"), f["last_ids"])
+    vs = r["vscreen"]
+    ab = vs["abs_terms"]
+    for k, cols in [("v_xy", slice(0, 2)), ("v_depth", 2), ("v_conic", slice(3, 6)), ("v_opac", 6), ("v_rgb", slice(7, 10))]:
+        _grad_close(g.host(k)[:m], vs[k], ab[:, cols], k)
+    gr = r["grads"]
+    vis = np.zeros(sc.n, bool)
+    vis[q["gaussian_ids"]] = True
+    for k, o in [("w_means", "v_means"), ("w_quats", "v_quats"), ("w_log_scales", "v_scales"),
+                 ("w_opacity_logits", "v_opacities"), ("w_features_dc", "v_dc"), ("w_features_sh", "v_sh")]:
+        got, ref = g.host(k).astype(np.float64), gr[o].astype(np.float64)
+        rows = ref.reshape(sc.n, -1)
+        scale = np.abs(rows).max(axis=1, keepdims=True) + 1e-30
+        err = np.abs(got.reshape(sc.n, -1) - rows)
+        floor = 2e-5 * (np.abs(rows).mean() + 1e-12)
+        assert (err <= 2 * GRAD_RTOL * scale + floor).all(), (k, float((err / scale).max()))
+        assert not np.any(got[~vis]), k
+    return g, r
+
+
 def test_device_math_is_bit_identical_to_host(gpu, oracle):
     lib, L = gpu.lib.load(), gpu.lib
     rng = np.random.default_rng(0)
@@ -159,3 +209,42 @@ def test_empty_and_culled(gpu, oracle):
     g, r = _compare(gpu, oracle, sc, "all-culled")
     assert g.K == 0 and not np.any(g.host("offsets"))
     assert np.all(g.host("r_T") == 1.0)
+
+
+def test_packed_projection_tiny(gpu, oracle):
+    """projection_3dgs_packed_forward: compacted rows in ascending splat order, then the whole chain."""
+    _compare_packed(gpu, oracle, gpu.scenes.tiny_scene(n=700, width=96, height=64, seed=21), "pk-tiny")
+    _compare_packed(gpu, oracle, gpu.scenes.tiny_scene(n=900, width=80, height=48, seed=22), "pk-tiny-fused",
+                    fused_count=True, use_packed=True)
+
+
+def test_packed_projection_without_readback(gpu, oracle):
+    """Outputs sized for all N splats, nnz read only afterwards: rows past nnz stay untouched."""
+    _compare_packed(gpu, oracle, gpu.scenes.tiny_scene(n=1300, width=96, height=64, seed=23), "pk-noread",
+                    fused_count=True, read_nnz=False)
+
+
+def test_packed_projection_sparse_and_dense(gpu, oracle):
+    sc = gpu.scenes.make_scene(4, n=80000, width=480, height=270, sh_codec=3)     # mostly culled, int8 SH
+    g, r = _compare_packed(gpu, oracle, sc, "pk-cfg4", fused_count=True, use_packed=True)
+    assert 0 < g.nnz < sc.n // 2
+    sc = gpu.scenes.make_scene(2, n=50000, width=480, height=270, parity_variant=True)   # mostly visible
+    _compare_packed(gpu, oracle, sc, "pk-cfg2", fused_count=True)
+    sc = gpu.scenes.make_scene(5, n=40000, width=512, height=256)                 # equirect
+    _compare_packed(gpu, oracle, sc, "pk-cfg5")
+
+
+def test_packed_projection_all_culled_and_empty(gpu, oracle):
+    sc = gpu.scenes.tiny_scene(n=300, width=40, height=24, seed=1)
+    sc.means[:, 2] = -10.0
+    g, r = _compare_packed(gpu, oracle, sc, "pk-all-culled")
+    assert g.nnz == 0 and g.K == 0 and np.all(g.host("r_T") == 1.0)
+
+
+def test_packed_projection_block_boundaries(gpu, oracle):
+    """Visibility patterns that leave whole 256-splat workgroups empty or full."""
+    sc = gpu.scenes.tiny_scene(n=256 * 9 + 17, width=96, height=64, seed=24)
+    blk = np.arange(sc.n) // 256
+    sc.means[(blk == 0) | (blk == 3) | (blk == 4) | (blk == 9), 2] = -10.0   # culled blocks, incl. first and last
+    g, r = _compare_packed(gpu, oracle, sc, "pk-blocks", fused_count=True)
+    assert 0 < g.nnz < sc.n
