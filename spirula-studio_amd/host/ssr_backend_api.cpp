@@ -456,15 +456,16 @@ rasterize_to_pixels_3dgs_bwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     if (v_splats_s) {
         vs = *v_splats_s;   // caller-provided accumulators are added into as they are
     } else {
-        // the launcher owns and zero-fills v_screen (src/kernels/raster/RasterizationBwd.cu:143-146)
+        // the launcher owns and zero-fills v_screen (src/kernels/raster/RasterizationBwd.cu:143-146);
+        // the five arrays sit back to back in one slot so that one fill clears them all
         const int64_t n = splats_s.empty() ? 0 : splats_s[0].rows();
-        const PoolSlot slots[5] = {PoolSlot::RasterBwdVScreenXy, PoolSlot::RasterBwdVScreenDepth, PoolSlot::RasterBwdVScreenConic,
-                                   PoolSlot::RasterBwdVScreenOpac, PoolSlot::RasterBwdVScreenRgb};
         const int ch[5] = {2, 1, 3, 1, 3};
+        float* base = DevicePool::global().acquire<float>(PoolSlot::RasterBwdVScreenXy, (size_t)(n * 10));
+        backend::memset_async(base, 0, (size_t)(n * 10) * sizeof(float));
+        int64_t off = 0;
         for (int i = 0; i < 5; i++) {
-            float* p = DevicePool::global().acquire<float>(slots[i], (size_t)(n * ch[i]));
-            backend::memset_async(p, 0, (size_t)(n * ch[i]) * sizeof(float));
-            vs.emplace_back(p, std::vector<int64_t>{n, ch[i]});
+            vs.emplace_back(base + off, std::vector<int64_t>{n, ch[i]});
+            off += n * ch[i];
         }
     }
     ssr_raster_bwd_params p;
