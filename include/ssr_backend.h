@@ -148,9 +148,17 @@ int ssr_projection_packed_emit(const ssr_projection_packed_params* p, ssr_stream
 
 /* ---- K2..K6: do_intersect_tile_generic, ellipse mode (src/kernels/tile/IntersectTile.cuh:25-41,
  * src/kernels/tile/IntersectTile.cu:376-509) split at its data-dependent allocation. */
+/* tile_active (optional, [tile_h,tile_w], 0 = skip): a tile the loss never reads is left out by
+ * both passes, so that compositing sees an empty range for it (IntersectTile.cu:117-119,165-166). */
 int ssr_tile_count(int64_t n, const float* aabb, const float* xy, const float* conic,
-                   const float* opac, uint32_t width, uint32_t height, int64_t* tiles_per_splat,
-                   ssr_stream_t stream);
+                   const float* opac, uint32_t width, uint32_t height, const int32_t* tile_active,
+                   int64_t* tiles_per_splat, ssr_stream_t stream);
+/* compute_tile_active (IntersectTile.cu:316-368): tile_active[t] = 1 when any pixel of tile t,
+ * grown by one pixel, is unmasked; `mask` is [mask_height, mask_width] bytes (non-zero = keep),
+ * sampled at the nearest source pixel (src/core/Interpolation.cuh:108-120). */
+int ssr_compute_tile_active(const uint8_t* mask, int32_t mask_height, int32_t mask_width,
+                            uint32_t width, uint32_t height, int32_t* tile_active,
+                            ssr_stream_t stream);
 /* inclusive_sum<int64> (src/backend/common/SortScan.h:58-72; IntersectTile.cu:425-428). */
 size_t ssr_scan_scratch_bytes(int64_t n);
 /* total_out (optional) also receives out[n-1], so that it can sit next to other counters and be
@@ -165,7 +173,8 @@ int ssr_read_i64(const int64_t* device_values, int64_t* host_values, int count, 
 int ssr_tile_write(int64_t n, const float* aabb, const float* sort_depth, const float* xy,
                    const float* conic, const float* opac, const int64_t* cum_tiles,
                    uint32_t width, uint32_t height, int64_t* isect_ids, int32_t* flatten_ids,
-                   const int32_t* visible_ids, int64_t n_visible, ssr_stream_t stream);
+                   const int32_t* visible_ids, int64_t n_visible, const int32_t* tile_active,
+                   ssr_stream_t stream);
 /* sort_pairs<int64,int32> with CUB DoubleBuffer semantics (src/backend/common/SortScan.h:42-56;
  * call site IntersectTile.cu:486-493): stable on bits [begin_bit,end_bit); *selector says which
  * of the (a,b) buffers holds the result. */

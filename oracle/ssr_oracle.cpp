@@ -543,17 +543,50 @@ int64_t or_projection_fwd(int64_t N, int sh_degree, const float* means, const fl
     return visible;
 }
 
-// intersect_tile_kernel<count=true, ellipse=true>, src/kernels/tile/IntersectTile.cu:104-186
-void or_tile_count(int64_t N, const float* aabb, const float* xy, const float* conic,
-    const float* opac, uint32_t width, uint32_t height, int64_t* tiles_per_splat) {
+// intersect_tile_kernel<count=true, ellipse=true>, src/kernels/tile/IntersectTile.cu:104-186;
+// tile_active (may be NULL): tiles marked 0 are not counted (:62,76-80,95-98)
+void or_tile_count_masked(int64_t N, const float* aabb, const float* xy, const float* conic,
+    const float* opac, uint32_t width, uint32_t height, const int32_t* tile_active, int64_t* tiles_per_splat) {
     const int tw = (int)((width + kTile - 1) / kTile), th = (int)((height + kTile - 1) / kTile);
 #pragma omp parallel for schedule(static)
     for (int64_t g = 0; g < N; g++) {
         TileGeom tg = tile_geom(aabb + 4 * g, xy + 2 * g, conic + 3 * g, opac[g], tw, th);
         int64_t n = 0;
-        if (tg.visible) for_each_tile(tg, [&](int, int) { n++; });
+        if (tg.visible) for_each_tile(tg, [&](int x, int y) { if (!tile_active || tile_active[(int64_t)y * tw + x]) n++; });
         tiles_per_splat[g] = n;
     }
+}
+void or_tile_count(int64_t N, const float* aabb, const float* xy, const float* conic,
+    const float* opac, uint32_t width, uint32_t height, int64_t* tiles_per_splat) {
+    or_tile_count_masked(N, aabb, xy, conic, opac, width, height, nullptr, tiles_per_splat);
+}
+
+// tile_active_kernel, src/kernels/tile/IntersectTile.cu:316-347, with nearest_sample_b
+// (src/core/Interpolation.cuh:108-120); kMaskPad = 1 (IntersectTile.cu:311)
+void or_compute_tile_active(const uint8_t* mask, int32_t h_mask, int32_t w_mask, uint32_t width, uint32_t height,
+    int32_t* tile_active) {
+    const int tw = (int)((width + kTile - 1) / kTile), th = (int)((height + kTile - 1) / kTile);
+    const int W = (int)width, H = (int)height;
+    for (int ty = 0; ty < th; ty++)
+        for (int tx = 0; tx < tw; tx++) {
+            bool live = false;
+            for (int dy = -1; dy < kTile + 1 && !live; ++dy) {
+                const int y = ty * kTile + dy;
+                if (y >= H) break;
+                if (y < 0) continue;
+                for (int dx = -1; dx < kTile + 1; ++dx) {
+                    const int x = tx * kTile + dx;
+                    if (x >= W) break;
+                    if (x < 0) continue;
+                    const float u = (((float)x + 0.5f) * (float)w_mask) / (float)W - 0.5f;
+                    const float v = (((float)y + 0.5f) * (float)h_mask) / (float)H - 0.5f;
+                    const int sx = std::max(0, std::min(w_mask - 1, ssr_f2i_sat(ssr_floor(u + 0.5f))));
+                    const int sy = std::max(0, std::min(h_mask - 1, ssr_f2i_sat(ssr_floor(v + 0.5f))));
+                    if (mask[(size_t)sy * w_mask + sx]) { live = true; break; }
+                }
+            }
+            tile_active[ty * tw + tx] = live ? 1 : 0;
+        }
 }
 
 void or_inclusive_sum_i64(int64_t n, const int64_t* in, int64_t* out) {
@@ -565,6 +598,12 @@ void or_inclusive_sum_i64(int64_t n, const int64_t* in, int64_t* out) {
 int64_t or_tile_write(int64_t N, const float* aabb, const float* sort_depth, const float* xy,
     const float* conic, const float* opac, const int64_t* cum, uint32_t width, uint32_t height,
     int64_t* isect_ids, int32_t* flatten_ids) {
+    return or_tile_write_masked(N, aabb, sort_depth, xy, conic, opac, cum, width, height, nullptr, isect_ids, flatten_ids);
+}
+// tile_active (may be NULL): skipped tiles are left out (IntersectTile.cu:225,240)
+int64_t or_tile_write_masked(int64_t N, const float* aabb, const float* sort_depth, const float* xy,
+    const float* conic, const float* opac, const int64_t* cum, uint32_t width, uint32_t height,
+    const int32_t* tile_active, int64_t* isect_ids, int32_t* flatten_ids) {
     const int tw = (int)((width + kTile - 1) / kTile), th = (int)((height + kTile - 1) / kTile);
     int64_t pads = 0;
 #pragma omp parallel for schedule(static) reduction(+ : pads)
@@ -576,6 +615,7 @@ int64_t or_tile_write(int64_t N, const float* aabb, const float* sort_depth, con
             uint32_t du = ssr_f2u(ssr_fabs(sort_depth[g]));
             du = (du >> 31) ? ~du : (du ^ 0x80000000u);
             for_each_tile(tg, [&](int x, int y) {
+                if (tile_active && !tile_active[(int64_t)y * tw + x]) return;
                 if (cur < end) {
                     int64_t tile_id = (int64_t)y * tw + (int64_t)x;
                     isect_ids[cur] = (int64_t)(((uint64_t)tile_id << 32) | (uint64_t)du);

@@ -50,6 +50,15 @@ int64_t or_projection_fwd(int64_t N, int sh_degree,
 /* K2 */
 void or_tile_count(int64_t N, const float* aabb, const float* xy, const float* conic,
     const float* opac, uint32_t width, uint32_t height, int64_t* tiles_per_splat);
+/* K2/K4 with the tile-skip map (tile_active[tile_h*tile_w], 0 = skip; NULL = all live), and the
+ * map itself from a [h_mask,w_mask] byte mask (src/kernels/tile/IntersectTile.cu:316-368). */
+void or_tile_count_masked(int64_t N, const float* aabb, const float* xy, const float* conic,
+    const float* opac, uint32_t width, uint32_t height, const int32_t* tile_active, int64_t* tiles_per_splat);
+int64_t or_tile_write_masked(int64_t N, const float* aabb, const float* sort_depth, const float* xy,
+    const float* conic, const float* opac, const int64_t* cum_tiles, uint32_t width,
+    uint32_t height, const int32_t* tile_active, int64_t* isect_ids, int32_t* flatten_ids);
+void or_compute_tile_active(const uint8_t* mask, int32_t h_mask, int32_t w_mask, uint32_t width, uint32_t height,
+    int32_t* tile_active);
 /* K3 */
 void or_inclusive_sum_i64(int64_t n, const int64_t* in, int64_t* out);
 /* K4. Returns the number of 0xffffffff pad keys written (0 when count and write agree). */

@@ -370,4 +370,22 @@ __device__ __forceinline__ int64_t count_tiles(const TileGeomD& g) {
     return n;
 }
 
+// Tile-skip map (src/kernels/tile/IntersectTile.cu:62,76-80,95-98,225): live[y * tile_w + x] == 0
+// marks a tile that neither pass emits.
+__device__ __forceinline__ bool tile_is_live(const int32_t* __restrict__ live, int tile_w, int fixed, int v, bool rows) {
+    return live[rows ? ((int64_t)fixed * tile_w + v) : ((int64_t)v * tile_w + fixed)] != 0;
+}
+
+__device__ __forceinline__ int count_live(const int32_t* __restrict__ live, int tile_w, int lo, int hi, int fixed, bool rows) {
+    int n = 0;
+    for (int v = lo; v < hi; v++) n += tile_is_live(live, tile_w, fixed, v, rows) ? 1 : 0;
+    return n;
+}
+
+__device__ __forceinline__ int64_t count_tiles_masked(const TileGeomD& g, const int32_t* __restrict__ live, int tile_w) {
+    int64_t n = 0;
+    for_each_tile(g, [&](int lo, int hi, int fixed, bool rows) { n += count_live(live, tile_w, lo, hi, fixed, rows); });
+    return n;
+}
+
 }  // namespace ssr

@@ -12,7 +12,7 @@ constexpr int kTileBlock = 256;
 __global__ __launch_bounds__(kTileBlock) void tile_count_kernel(
     int64_t n, const float4* __restrict__ aabb, const float2* __restrict__ xy,
     const float* __restrict__ conic, const float* __restrict__ opac, int tile_w, int tile_h,
-    int64_t* __restrict__ tiles_per_splat) {
+    const int32_t* __restrict__ live, int64_t* __restrict__ tiles_per_splat) {
     const int64_t g = (int64_t)blockIdx.x * kTileBlock + threadIdx.x;
     if (g >= n) return;
     const float4 a = aabb[g];
@@ -23,7 +23,36 @@ __global__ __launch_bounds__(kTileBlock) void tile_count_kernel(
     const float cn[3] = {conic[3 * g], conic[3 * g + 1], conic[3 * g + 2]};
     TileGeomD tg;
     tile_geom(bb, cxy, cn, opac[g], tile_w, tile_h, tg);
-    tiles_per_splat[g] = count_tiles(tg);
+    tiles_per_splat[g] = live ? count_tiles_masked(tg, live, tile_w) : count_tiles(tg);
+}
+
+// tile_active_kernel (src/kernels/tile/IntersectTile.cu:316-347): a tile is live when any pixel of
+// it, grown by one pixel (the depth-to-normal stencil of the loss reads one pixel past its own),
+// is unmasked; the mask is sampled at the nearest source pixel (src/core/Interpolation.cuh:108-120).
+__global__ __launch_bounds__(kTileBlock) void tile_active_kernel(const uint8_t* __restrict__ mask, int h_mask, int w_mask,
+                                                                 int width, int height, int tile_w, int tile_h,
+                                                                 int32_t* __restrict__ tile_active) {
+    const int t = blockIdx.x * kTileBlock + threadIdx.x;
+    if (t >= tile_w * tile_h) return;
+    const int tx = t % tile_w, ty = t / tile_w;
+    constexpr int kPad = 1;
+    bool live = false;
+    for (int dy = -kPad; dy < kTile + kPad && !live; ++dy) {
+        const int y = ty * kTile + dy;
+        if (y >= height) break;
+        if (y < 0) continue;
+        for (int dx = -kPad; dx < kTile + kPad; ++dx) {
+            const int x = tx * kTile + dx;
+            if (x >= width) break;
+            if (x < 0) continue;
+            const float u = (((float)x + 0.5f) * (float)w_mask) / (float)width - 0.5f;
+            const float v = (((float)y + 0.5f) * (float)h_mask) / (float)height - 0.5f;
+            const int sx = max(0, min(w_mask - 1, ssr_f2i_sat(ssr_floor(u + 0.5f))));
+            const int sy = max(0, min(h_mask - 1, ssr_f2i_sat(ssr_floor(v + 0.5f))));
+            if (mask[(size_t)sy * w_mask + sx]) { live = true; break; }
+        }
+    }
+    tile_active[t] = live ? 1 : 0;
 }
 
 // Splats that touch more than kCoopTiles tiles (a splat close to the camera can cover thousands)
@@ -45,7 +74,7 @@ __global__ __launch_bounds__(kTileBlock) void tile_write_kernel(
     int64_t n, const float4* __restrict__ aabb, const float* __restrict__ sort_depth,
     const float2* __restrict__ xy, const float* __restrict__ conic, const float* __restrict__ opac,
     const int64_t* __restrict__ cum, int tile_w, int tile_h, int64_t* __restrict__ isect_ids,
-    int32_t* __restrict__ flatten_ids, const int32_t* __restrict__ visible_ids) {
+    int32_t* __restrict__ flatten_ids, const int32_t* __restrict__ visible_ids, const int32_t* __restrict__ live) {
     const int64_t i = (int64_t)blockIdx.x * kTileBlock + threadIdx.x;
     const int lane = threadIdx.x & 63;
     const bool in_range = i < n;
@@ -73,6 +102,7 @@ __global__ __launch_bounds__(kTileBlock) void tile_write_kernel(
     if (visible && !coop) {
         for_each_tile(tg, [&](int lo, int hi, int fixed, bool rows) {
             for (int v = lo; v < hi && cur < end; v++) {
+                if (live && !tile_is_live(live, tile_w, fixed, v, rows)) continue;
                 const int64_t tile_id = rows ? ((int64_t)fixed * tile_w + v) : ((int64_t)v * tile_w + fixed);
                 isect_ids[cur] = (int64_t)(((uint64_t)tile_id << 32) | (uint64_t)du);
                 flatten_ids[cur] = (int32_t)g;
@@ -107,13 +137,15 @@ __global__ __launch_bounds__(kTileBlock) void tile_write_kernel(
             const int r = base + lane;
             int lo = 0, hi = 0;
             if (r < b1) tile_band_interval(sg, r, lo, hi);
-            const int c = max(hi - lo, 0);
+            const int c = live ? count_live(live, tile_w, lo, hi, r, sg.by_rows) : max(hi - lo, 0);
             const int inc = wave_inclusive_scan_i32(c, lane);
             int64_t pos = scur + (inc - c);
-            for (int v = lo; v < hi && pos < send; v++, pos++) {
+            for (int v = lo; v < hi && pos < send; v++) {
+                if (live && !tile_is_live(live, tile_w, r, v, sg.by_rows)) continue;
                 const int64_t tile_id = sg.by_rows ? ((int64_t)r * tile_w + v) : ((int64_t)v * tile_w + r);
                 isect_ids[pos] = (int64_t)(((uint64_t)tile_id << 32) | (uint64_t)sdu);
                 flatten_ids[pos] = sgid;
+                pos++;
             }
             scur += __shfl(inc, 63, 64);
         }
@@ -223,8 +255,21 @@ using namespace ssr;
 
 extern "C" {
 
+int ssr_compute_tile_active(const uint8_t* mask, int32_t mask_height, int32_t mask_width, uint32_t width, uint32_t height,
+                            int32_t* tile_active, ssr_stream_t stream) {
+    SSR_REQUIRE(mask && tile_active, "ssr_compute_tile_active", "null pointer");
+    SSR_REQUIRE(mask_height > 0 && mask_width > 0 && width > 0 && height > 0, "ssr_compute_tile_active", "empty mask or image");
+    SSR_REQUIRE(width < (1u << 30) && height < (1u << 30), "ssr_compute_tile_active", "image too large");
+    const int tw = (int)ceil_div(width, kTile), th = (int)ceil_div(height, kTile);
+    hipLaunchKernelGGL(tile_active_kernel, dim3((unsigned)ceil_div((int64_t)tw * th, kTileBlock)), dim3(kTileBlock), 0,
+                       as_stream(stream), mask, mask_height, mask_width, (int)width, (int)height, tw, th, tile_active);
+    SSR_CHECK_LAUNCH("ssr_compute_tile_active");
+    return 0;
+}
+
 int ssr_tile_count(int64_t n, const float* aabb, const float* xy, const float* conic, const float* opac,
-                   uint32_t width, uint32_t height, int64_t* tiles_per_splat, ssr_stream_t stream) {
+                   uint32_t width, uint32_t height, const int32_t* tile_active, int64_t* tiles_per_splat,
+                   ssr_stream_t stream) {
     SSR_REQUIRE(n >= 0 && n < (int64_t)1 << 31, "ssr_tile_count", "count out of range");
     if (n == 0) return 0;
     SSR_REQUIRE(aabb && xy && conic && opac && tiles_per_splat, "ssr_tile_count", "null pointer");
@@ -234,7 +279,7 @@ int ssr_tile_count(int64_t n, const float* aabb, const float* xy, const float* c
     const int tw = (int)ceil_div(width, kTile), th = (int)ceil_div(height, kTile);
     hipLaunchKernelGGL(tile_count_kernel, dim3((unsigned)ceil_div(n, kTileBlock)), dim3(kTileBlock), 0, as_stream(stream),
                        n, reinterpret_cast<const float4*>(aabb), reinterpret_cast<const float2*>(xy), conic, opac, tw, th,
-                       tiles_per_splat);
+                       tile_active, tiles_per_splat);
     SSR_CHECK_LAUNCH("ssr_tile_count");
     return 0;
 }
@@ -262,7 +307,8 @@ int ssr_inclusive_sum_i64(const int64_t* in, int64_t* out, int64_t n, int64_t* t
 
 int ssr_tile_write(int64_t n, const float* aabb, const float* sort_depth, const float* xy, const float* conic,
                    const float* opac, const int64_t* cum_tiles, uint32_t width, uint32_t height, int64_t* isect_ids,
-                   int32_t* flatten_ids, const int32_t* visible_ids, int64_t n_visible, ssr_stream_t stream) {
+                   int32_t* flatten_ids, const int32_t* visible_ids, int64_t n_visible, const int32_t* tile_active,
+                   ssr_stream_t stream) {
     SSR_REQUIRE(n >= 0 && n < (int64_t)1 << 31, "ssr_tile_write", "count out of range");
     if (visible_ids) {
         SSR_REQUIRE(n_visible >= 0 && n_visible <= n, "ssr_tile_write", "visible count out of range");
@@ -278,7 +324,7 @@ int ssr_tile_write(int64_t n, const float* aabb, const float* sort_depth, const 
     const int64_t work = visible_ids ? n_visible : n;
     hipLaunchKernelGGL(tile_write_kernel, dim3((unsigned)ceil_div(work, kTileBlock)), dim3(kTileBlock), 0, as_stream(stream),
                        work, reinterpret_cast<const float4*>(aabb), sort_depth, reinterpret_cast<const float2*>(xy), conic, opac,
-                       cum_tiles, tw, th, isect_ids, flatten_ids, visible_ids);
+                       cum_tiles, tw, th, isect_ids, flatten_ids, visible_ids, tile_active);
     SSR_CHECK_LAUNCH("ssr_tile_write");
     return 0;
 }

@@ -22,6 +22,7 @@ SYMBOLS = {
     "ssrh_set_data_3dgs": (C.c_int, [C.c_int64, vp, vp, vp, vp, vp, vp, C.c_int]),
     "ssrh_set_sh_value_quant": (C.c_int, [C.c_int, vp, C.c_int64, C.c_int, vp, C.c_int64, C.c_int, C.c_int64]),
     "ssrh_set_camera_params": (C.c_int, [C.c_int, C.c_int, C.c_char_p, C.c_char_p, vp, vp, C.c_int]),
+    "ssrh_set_tile_mask": (C.c_int, [vp, C.c_int, C.c_int]),
     "ssrh_forward_3dgs": (C.c_int, [C.c_char_p, C.c_int, C.c_int, C.c_int, C.c_int]),
     "ssrh_backward_from_render_grad": (C.c_int, [vp, vp, vp]),
     "ssrh_copy_render_to_host": (C.c_int, [vp, vp, vp]),
@@ -107,6 +108,11 @@ class Engine:
 
     def set_stage_profiling(self, on):
         check(self.h.ssrh_set_options(*self.opts, int(on)))
+
+    def set_tile_mask(self, mask):
+        """Tile-skip map for the next forward only, from a [h_mask, w_mask] byte mask."""
+        mask = np.ascontiguousarray(mask, np.uint8)
+        check(self.h.ssrh_set_tile_mask(mask.ctypes.data, mask.shape[0], mask.shape[1]))
 
     def forward(self):
         check(self.h.ssrh_forward_3dgs(b"3dgs", self.sh_degree, int(self.packed_projection), 0, 0))

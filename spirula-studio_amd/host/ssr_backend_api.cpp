@@ -326,6 +326,14 @@ int64_t intersect_tile_count(int width, int height) {
     return (int64_t)((width + 15) / 16) * (int64_t)((height + 15) / 16);
 }
 
+void compute_tile_active(TorchTensorView mask, int I, int width, int height, int32_t* tile_active) {
+    if (I != 1) throw std::runtime_error("compute_tile_active: this backend runs one image per call");
+    const auto& ms = std::get<2>(mask);
+    if (ms.size() != 3) throw std::runtime_error("compute_tile_active: mask must be [I, H_mask, W_mask]");
+    ok(ssr_compute_tile_active((const uint8_t*)std::get<0>(mask), (int32_t)ms[1], (int32_t)ms[2], (uint32_t)width,
+                               (uint32_t)height, tile_active, nullptr), "compute_tile_active");
+}
+
 std::tuple<DeviceVector<int64_t>, DeviceVector<int32_t>, DeviceTensor3D<int32_t>>
 do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, DeviceTensorFloatND* proj_xy,
                           DeviceTensorFloatND* proj_conic, DeviceTensorFloatND* proj_opac, const uint32_t I,
@@ -334,7 +342,6 @@ do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, 
     // Packed mode (image_ids given): `total` rows, one per visible (camera, splat) pair, and the
     // values written to flatten_ids are row numbers (src/kernels/tile/IntersectTile.cu:386-409). With
     // the single camera this backend runs, every image id is 0 and the array itself is not read.
-    if (tile_active) throw std::runtime_error("do_intersect_tile_generic: the tile-skip mask is not built in this backend");
     if (!proj_xy || !proj_conic || !proj_opac)
         throw std::runtime_error("do_intersect_tile_generic: AABB mode is not built in this backend (ellipse mode is)");
     if (I != 1) throw std::runtime_error("do_intersect_tile_generic: this backend runs one image per call");
@@ -343,10 +350,11 @@ do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, 
     const uint32_t n_tiles = tile_w * tile_h * I;
 
     DeviceVector<int64_t> tiles_per_splat; tiles_per_splat.resize(PoolSlot::IsectTilesPerSplat, total);
-    if (!g_counts_fused) {
+    // counts fused into the projection know nothing of a tile-skip map: count again when one is given
+    if (!g_counts_fused || tile_active) {
         StageTimer t(&g_times.k2);
         ok(ssr_tile_count(total, aabb.data_ptr(), proj_xy->data_ptr(), proj_conic->data_ptr(), proj_opac->data_ptr(),
-                          image_width, image_height, tiles_per_splat.data_ptr(), nullptr), "do_intersect_tile_generic/count");
+                          image_width, image_height, tile_active, tiles_per_splat.data_ptr(), nullptr), "do_intersect_tile_generic/count");
     } else {
         g_times.k2 = 0;
     }
@@ -380,7 +388,7 @@ do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, 
         StageTimer t(&g_times.k4);
         ok(ssr_tile_write(total, aabb.data_ptr(), depths.data_ptr(), proj_xy->data_ptr(), proj_conic->data_ptr(),
                           proj_opac->data_ptr(), cum.data_ptr(), image_width, image_height, ids_a.data_ptr(),
-                          flat_a.data_ptr(), g_visible_ids, g_visible_ids ? g_n_visible : 0, nullptr),
+                          flat_a.data_ptr(), g_visible_ids, g_visible_ids ? g_n_visible : 0, tile_active, nullptr),
            "do_intersect_tile_generic/write");
     }
     int selector = 0;

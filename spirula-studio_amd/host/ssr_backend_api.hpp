@@ -53,6 +53,8 @@ projection_3dgs_packed_forward(
     const int64_t sh_bounds_stride);
 
 int64_t intersect_tile_count(int width, int height);
+// src/kernels/tile/IntersectTile.cu:349-368; mask is [I, H_mask, W_mask] bool on the device
+void compute_tile_active(TorchTensorView mask, int I, int width, int height, int32_t* tile_active);
 
 std::tuple<DeviceVector<int64_t>, DeviceVector<int32_t>, DeviceTensor3D<int32_t>>
 do_intersect_tile_generic(

@@ -111,6 +111,14 @@ void set_camera_params(int width, int height, std::string camera_model, std::str
     c.dist_coeffs = device_copy_tv(PoolSlot::CamDistCoeffs, dist_coeffs);
 }
 
+void engine_set_tile_mask(TorchTensorView mask) {
+    auto& E = engine();
+    if (E.camera.width <= 0) throw std::runtime_error("engine_set_tile_mask: set_camera_params must be called first");
+    TorchTensorView dm = device_copy_tv(PoolSlot::EngTileMask, mask);
+    E.fwd.tile_active.resize(PoolSlot::IsectTileActive, intersect_tile_count(E.camera.width, E.camera.height) * E.camera.num);
+    compute_tile_active(dm, E.camera.num, E.camera.width, E.camera.height, E.fwd.tile_active.data_ptr());
+}
+
 void forward_3dgs(std::string primitive, int sh_degree, bool packed, bool output_median, int dist_type_int) {
     if (primitive != "3dgs") throw std::runtime_error("forward_3dgs: primitive '" + primitive + "' is not built in this backend");
     auto& E = engine();
@@ -156,8 +164,9 @@ void forward_3dgs(std::string primitive, int sh_degree, bool packed, bool output
     if (packed && E.fwd.camera_ids.data_ptr() != nullptr) image_ids_ptr = &E.fwd.camera_ids;
     auto [ids, flat, offsets] = do_intersect_tile_generic(
         aabb_nd, depths_nd, &screen[0], &screen[2], &screen[3], (uint32_t)E.camera.num, E.camera.intrins,
-        (uint32_t)E.camera.width, (uint32_t)E.camera.height, image_ids_ptr, nullptr);
+        (uint32_t)E.camera.width, (uint32_t)E.camera.height, image_ids_ptr, E.fwd.tile_active.data_ptr());
     E.fwd.isect_ids = ids; E.fwd.flatten_ids = flat; E.fwd.tile_offsets = offsets;
+    E.fwd.tile_active = DeviceVector<int32_t>();   // one shot
 
     auto [renders, Ts, last, dist, median] = rasterize_to_pixels_3dgs_fwd(
         N, in_splats, screen, E.fwd.gaussian_ids, (uint32_t)E.camera.width, (uint32_t)E.camera.height, offsets, flat,
@@ -290,6 +299,10 @@ int ssrh_set_camera_params(int width, int height, const char* model, const char*
         set_camera_params(width, height, model, distortion, tv(viewmats, 4, {num_cameras, 4, 4}), tv(intrins, 4, {num_cameras, 4}),
                           tv(zero_coeffs, 4, {num_cameras, 8}));
     });
+}
+
+int ssrh_set_tile_mask(const uint8_t* mask, int h_mask, int w_mask) {
+    return guard([&] { engine_set_tile_mask(tv(mask, 1, {1, h_mask, w_mask})); });
 }
 
 int ssrh_forward_3dgs(const char* primitive, int sh_degree, int packed, int output_median, int dist_type) {

@@ -37,6 +37,9 @@ struct EngineState {
         std::vector<DeviceTensorFloatND> splats_w, splats_s;
         DeviceTensor2D<float4> aabb; DeviceTensor2D<float> depths;
         DeviceVector<int32_t> camera_ids, gaussian_ids;   // packed projection only
+        // Tile-skip map for the NEXT forward only: whoever wants tiles skipped sets it right before,
+        // so a later render cannot inherit it (src/engine/EngineForward.cpp:245-252).
+        DeviceVector<int32_t> tile_active;
         DeviceVector<int64_t> isect_ids; DeviceVector<int32_t> flatten_ids; DeviceTensor3D<int32_t> tile_offsets;
         RenderOutput::TensorTuple renders; DeviceTensor3D<float> render_Ts; DeviceTensor3D<int32_t> last_ids;
     } fwd;
@@ -61,6 +64,9 @@ void set_data_3dgs(int64_t num_splats, TorchTensorView means, TorchTensorView qu
 void set_sh_value_quant(int sh_value_bits, TorchTensorView packed, TorchTensorView bounds, int64_t bounds_stride);
 void set_camera_params(int width, int height, std::string camera_model, std::string distortion,
                        TorchTensorView viewmats, TorchTensorView intrins, TorchTensorView dist_coeffs);
+// computes engine().fwd.tile_active from a [1, H_mask, W_mask] bool mask (host or device), as the
+// training step does from the ground-truth alpha (src/engine/EngineTrainStep.cpp:100-104)
+void engine_set_tile_mask(TorchTensorView mask);
 void forward_3dgs(std::string primitive, int sh_degree, bool packed, bool output_median, int dist_type_int);
 void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
                                       TorchTensorView v_render_Ts);

@@ -63,7 +63,7 @@ enum class PoolSlot : int {
     ProjAabb, ProjDepths, ProjScreenXy, ProjScreenDepth, ProjScreenConic, ProjScreenOpac, ProjScreenRgb,
     IsectTilesPerSplat, IsectCumTiles, IsectIdsA, IsectIdsB, IsectFlatA, IsectFlatB, IsectOffsets,
     IsectScanScratch, IsectSortScratch, IsectCounters, ProjVisibleIds, ProjVisibleIdsB, ProjPackedRows,
-    ProjCameraIds, ProjGaussianIds, ProjGaussianIdsB, ProjPackedScratch, ProjPackedNnz,
+    IsectTileActive, EngTileMask, ProjCameraIds, ProjGaussianIds, ProjGaussianIdsB, ProjPackedScratch, ProjPackedNnz,
     RendersRgb, RendersDepth, RenderTs, RenderLastIds,
     RasterBwdVScreenXy, RasterBwdVScreenDepth, RasterBwdVScreenConic, RasterBwdVScreenOpac, RasterBwdVScreenRgb,
     EngVRgb, EngVDepth, EngVTs,

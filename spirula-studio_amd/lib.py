@@ -83,11 +83,12 @@ SYMBOLS = {
     "ssr_projection_packed_scratch_bytes": (_sz, [_i64]),
     "ssr_projection_packed_mask": (_i32, [C.POINTER(ProjectionPackedParams), vp]),
     "ssr_projection_packed_emit": (_i32, [C.POINTER(ProjectionPackedParams), vp]),
-    "ssr_tile_count": (_i32, [_i64, vp, vp, vp, vp, _u32, _u32, vp, vp]),
+    "ssr_tile_count": (_i32, [_i64, vp, vp, vp, vp, _u32, _u32, vp, vp, vp]),
+    "ssr_compute_tile_active": (_i32, [vp, _i32, _i32, _u32, _u32, vp, vp]),
     "ssr_scan_scratch_bytes": (_sz, [_i64]),
     "ssr_inclusive_sum_i64": (_i32, [vp, vp, _i64, vp, vp, _sz, vp]),
     "ssr_read_i64": (_i32, [vp, C.POINTER(C.c_int64), _i32, vp]),
-    "ssr_tile_write": (_i32, [_i64, vp, vp, vp, vp, vp, vp, _u32, _u32, vp, vp, vp, _i64, vp]),
+    "ssr_tile_write": (_i32, [_i64, vp, vp, vp, vp, vp, vp, _u32, _u32, vp, vp, vp, _i64, vp, vp]),
     "ssr_sort_scratch_bytes": (_sz, [_i64]),
     "ssr_sort_pairs_u64_i32": (_i32, [vp, vp, vp, vp, _i64, _i32, _i32, C.POINTER(C.c_int), vp, _sz, vp]),
     "ssr_tile_offsets": (_i32, [_i64, vp, _u32, vp, vp]),

@@ -51,6 +51,7 @@ class GpuRun:
         self.d["packed"] = D((n, 12), np.float32)
         self.V = None
         self.rows = n          # rows of the projection outputs: N, or nnz in packed mode
+        self.tile_active = None   # device tile-skip map (set_tile_mask)
 
     def ptr(self, k):
         a = self.d.get(k)
@@ -84,6 +85,16 @@ class GpuRun:
         s.xy, s.depth, s.conic = self.ptr(prefix + "xy"), self.ptr(prefix + "depth"), self.ptr(prefix + "conic")
         s.opac, s.rgb = self.ptr(prefix + "opac"), self.ptr(prefix + "rgb")
         return s
+
+    def set_tile_mask(self, mask):
+        """compute_tile_active on the device from a [h_mask, w_mask] byte mask."""
+        D = self.L.DeviceArray
+        mask = np.ascontiguousarray(mask, np.uint8)
+        self.d["mask"] = D.from_host(mask)
+        self.d["tile_active"] = D((self.sc.tile_w * self.sc.tile_h,), np.int32)
+        self.check(self.lib.ssr_compute_tile_active(self.ptr("mask"), mask.shape[0], mask.shape[1], self.sc.width,
+                                                    self.sc.height, self.ptr("tile_active"), None))
+        self.tile_active = self.ptr("tile_active")
 
     # ---- stages ----
     def projection_packed_fwd(self, fused_count=False):
@@ -147,9 +158,10 @@ class GpuRun:
     def tiles(self, fused_count=False):
         sc, D = self.sc, self.L.DeviceArray
         n = self.rows
-        if not fused_count:
+        if not fused_count or self.tile_active:   # fused counts know nothing of the tile-skip map
             self.check(self.lib.ssr_tile_count(n, self.ptr("aabb"), self.ptr("xy"), self.ptr("conic"),
-                                               self.ptr("opac"), sc.width, sc.height, self.ptr("counts"), None))
+                                               self.ptr("opac"), sc.width, sc.height, self.tile_active,
+                                               self.ptr("counts"), None))
         sb = self.lib.ssr_scan_scratch_bytes(n)
         self.d["scan_scratch"] = D((max(sb, 8),), np.uint8)
         self.check(self.lib.ssr_inclusive_sum_i64(self.ptr("counts"), self.ptr("cum"), n, self.ptr("counters"),
@@ -171,7 +183,7 @@ class GpuRun:
                                                self.ptr("conic"), self.ptr("opac"), self.ptr("cum"), sc.width,
                                                sc.height, self.ptr("keys_a"), self.ptr("vals_a"),
                                                self.ptr("vis_ids") if self.use_list else None,
-                                               self.V if self.use_list else 0, None))
+                                               self.V if self.use_list else 0, self.tile_active, None))
             self.unsorted_keys = self.d["keys_a"].to_host()
             self.unsorted_vals = self.d["vals_a"].to_host()
             sb = self.lib.ssr_sort_scratch_bytes(K)

@@ -106,10 +106,18 @@ def projection_fwd(scene, sh_degree=3):
     return o
 
 
-def tile_count(n, aabb, xy, conic, opac, w, h):
+def tile_count(n, aabb, xy, conic, opac, w, h, tile_active=None):
     out = np.zeros(n, np.int64)
-    lib().or_tile_count(C.c_int64(n), _p(aabb), _p(xy), _p(conic), _p(opac), C.c_uint32(w),
-                        C.c_uint32(h), _p(out))
+    lib().or_tile_count_masked(C.c_int64(n), _p(aabb), _p(xy), _p(conic), _p(opac), C.c_uint32(w),
+                               C.c_uint32(h), _p(tile_active), _p(out))
+    return out
+
+
+def compute_tile_active(mask, w, h):
+    mask = np.ascontiguousarray(mask, np.uint8)
+    out = np.zeros(((h + 15) // 16) * ((w + 15) // 16), np.int32)
+    lib().or_compute_tile_active(_p(mask), C.c_int32(mask.shape[0]), C.c_int32(mask.shape[1]), C.c_uint32(w),
+                                 C.c_uint32(h), _p(out))
     return out
 
 
@@ -120,12 +128,13 @@ def inclusive_sum(a):
     return out
 
 
-def tile_write(n, aabb, sort_depth, xy, conic, opac, cum, w, h):
+def tile_write(n, aabb, sort_depth, xy, conic, opac, cum, w, h, tile_active=None):
     k = int(cum[-1]) if n else 0
     ids = np.zeros(k, np.int64)
     flat = np.zeros(k, np.int32)
-    pads = lib().or_tile_write(C.c_int64(n), _p(aabb), _p(sort_depth), _p(xy), _p(conic), _p(opac),
-                               _p(cum), C.c_uint32(w), C.c_uint32(h), _p(ids), _p(flat))
+    lib().or_tile_write_masked.restype = C.c_int64
+    pads = lib().or_tile_write_masked(C.c_int64(n), _p(aabb), _p(sort_depth), _p(xy), _p(conic), _p(opac),
+                                      _p(cum), C.c_uint32(w), C.c_uint32(h), _p(tile_active), _p(ids), _p(flat))
     return ids, flat, pads
 
 
@@ -197,14 +206,14 @@ def projection_bwd(scene, aabb, vs, sh_degree=3):
     return g
 
 
-def pipeline(scene, sh_degree=3, backward=True):
+def pipeline(scene, sh_degree=3, backward=True, tile_active=None):
     """The whole iteration in the reference's order (src/engine/EngineForward.cpp:166-293,
-    src/engine/EngineLoss.cpp:138-240,359-368)."""
+    src/engine/EngineLoss.cpp:138-240,359-368). tile_active: optional tile-skip map for the tile stage."""
     n, w, h = scene.n, scene.width, scene.height
     p = projection_fwd(scene, sh_degree)
-    counts = tile_count(n, p["aabb"], p["xy"], p["conic"], p["opac"], w, h)
+    counts = tile_count(n, p["aabb"], p["xy"], p["conic"], p["opac"], w, h, tile_active)
     cum = inclusive_sum(counts)
-    ids, flat, pads = tile_write(n, p["aabb"], p["sort_depth"], p["xy"], p["conic"], p["opac"], cum, w, h)
+    ids, flat, pads = tile_write(n, p["aabb"], p["sort_depth"], p["xy"], p["conic"], p["opac"], cum, w, h, tile_active)
     n_tiles = scene.tile_w * scene.tile_h
     sk, sv = sort_pairs(ids, flat, 0, 32 + tile_n_bits(n_tiles))
     offs = tile_offsets(sk, n_tiles)
@@ -234,7 +243,7 @@ def pack_projection(p):
     return q
 
 
-def pipeline_packed(scene, sh_degree=3, backward=True):
+def pipeline_packed(scene, sh_degree=3, backward=True, tile_active=None):
     """The iteration with packed projection outputs (engine path with packed=true,
     src/engine/EngineForward.cpp:119-162,215-217): every later stage sees nnz rows, flatten ids are
     packed row numbers, v_screen has nnz rows, and the projection backward maps row i to splat
@@ -243,9 +252,9 @@ def pipeline_packed(scene, sh_degree=3, backward=True):
     full = projection_fwd(scene, sh_degree)
     p = pack_projection(full)
     m = p["visible"]
-    counts = tile_count(m, p["aabb"], p["xy"], p["conic"], p["opac"], w, h)
+    counts = tile_count(m, p["aabb"], p["xy"], p["conic"], p["opac"], w, h, tile_active)
     cum = inclusive_sum(counts)
-    ids, flat, pads = tile_write(m, p["aabb"], p["sort_depth"], p["xy"], p["conic"], p["opac"], cum, w, h)
+    ids, flat, pads = tile_write(m, p["aabb"], p["sort_depth"], p["xy"], p["conic"], p["opac"], cum, w, h, tile_active)
     n_tiles = scene.tile_w * scene.tile_h
     sk, sv = sort_pairs(ids, flat, 0, 32 + tile_n_bits(n_tiles))
     offs = tile_offsets(sk, n_tiles)

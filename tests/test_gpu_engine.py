@@ -177,6 +177,30 @@ def test_engine_packed_follows_the_camera_and_handles_nothing_visible(pkg, oracl
     look([[1, 0, 0, 0], [0, 1, 0, 0], [0, 0, 1, 0], [0, 0, 0, 1]])             # and back
 
 
+def test_engine_tile_mask_is_one_shot(pkg, oracle, H):
+    host, lib = H
+    sc = pkg.scenes.make_scene(1, n=20000, width=320, height=240, parity_variant=True)
+    mask = np.zeros((240, 320), np.uint8)
+    mask[60:150, 100:260] = 1
+    live = oracle.compute_tile_active(mask, sc.width, sc.height)
+    assert 0 < live.sum() < live.size
+    for packed in (False, True):
+        eng = host.Engine(sc, packed_projection=packed)
+        eng.set_tile_mask(mask)
+        eng.forward()
+        eng.backward()
+        if packed:
+            _check_packed(eng, oracle.pipeline_packed(sc, tile_active=live), sc)
+        else:
+            _check(eng, oracle.pipeline(sc, tile_active=live), sc)
+        eng.forward()          # the map is not inherited by the next forward
+        eng.backward()
+        if packed:
+            _check_packed(eng, oracle.pipeline_packed(sc), sc)
+        else:
+            _check(eng, oracle.pipeline(sc), sc)
+
+
 def test_unsupported_variants_raise(pkg, H):
     host, lib = H
     sc = pkg.scenes.tiny_scene(n=50, width=32, height=32)

@@ -29,10 +29,15 @@ def _grad_close(got, ref, abs_scale, name):
                            got[bad][:4], ref[bad][:4])
 
 
-def _compare(gpu, oracle, sc, label, fused_count=False, use_list=False, use_packed=False):
-    r = oracle.pipeline(sc)
+def _compare(gpu, oracle, sc, label, fused_count=False, use_list=False, use_packed=False, mask=None):
+    live = None if mask is None else oracle.compute_tile_active(mask, sc.width, sc.height)
+    r = oracle.pipeline(sc, tile_active=live)
     print(f"[{label}] N={sc.n} {sc.width}x{sc.height} visible={r['proj']['visible']} K={r['isect_ids'].size}", flush=True)
-    g = GpuRun(gpu, sc, use_list=use_list, use_packed=use_packed).run_all(fused_count=fused_count)
+    g = GpuRun(gpu, sc, use_list=use_list, use_packed=use_packed)
+    if mask is not None:
+        g.set_tile_mask(mask)
+        assert np.array_equal(g.host("tile_active"), live)
+    g.run_all(fused_count=fused_count)
     if use_list:
         assert g.V == r['proj']['visible']
         assert np.array_equal(np.sort(g.host('vis_ids')[:g.V]), np.nonzero(r['proj']['aabb'][:, 2] > r['proj']['aabb'][:, 0])[0])
@@ -248,3 +253,25 @@ def test_packed_projection_block_boundaries(gpu, oracle):
     sc.means[(blk == 0) | (blk == 3) | (blk == 4) | (blk == 9), 2] = -10.0   # culled blocks, incl. first and last
     g, r = _compare_packed(gpu, oracle, sc, "pk-blocks", fused_count=True)
     assert 0 < g.nnz < sc.n
+
+
+def test_tile_skip_mask(gpu, oracle):
+    """compute_tile_active + the tile_active argument of both tile passes: skipped tiles get an empty
+    range, everything else is unchanged (src/kernels/tile/IntersectTile.cu:309-368)."""
+    rng = np.random.default_rng(3)
+    sc = gpu.scenes.tiny_scene(n=900, width=160, height=96, seed=41)
+    sc.log_scales[::9] += 1.5
+    mask = np.zeros((40, 67), np.uint8)          # a mask at another resolution than the image
+    mask[5:30, 10:50] = rng.random((25, 40)) < 0.02
+    g, r = _compare(gpu, oracle, sc, "mask-tiny", mask=mask)
+    live = g.host("tile_active")
+    assert 0 < live.sum() < live.size
+    _compare(gpu, oracle, sc, "mask-tiny-list", fused_count=True, use_list=True, use_packed=True, mask=mask)
+    _compare(gpu, oracle, sc, "mask-none-live", mask=np.zeros((8, 8), np.uint8))
+    # huge splats: the wavefront-cooperative key write under a mask
+    sc = gpu.scenes.tiny_scene(n=600, width=640, height=400, seed=13)
+    sc.log_scales[::7] += 2.5
+    sc.means[::50, 2] = -3.6
+    mask = (rng.random((400, 640)) < 0.0005).astype(np.uint8)
+    g, r = _compare(gpu, oracle, sc, "mask-huge", fused_count=True, use_list=True, mask=mask)
+    assert r["counts"].max() > 96
