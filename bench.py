@@ -93,6 +93,9 @@ def main():
                     help="run the stages exactly as the reference does (separate count pass, atomic K9 into zero-filled buffers)")
     ap.add_argument("--packed-projection", action="store_true",
                     help="run the packed form of the projection (compacted nnz-row outputs; the reference's training default)")
+    ap.add_argument("--fused-optimizer", action="store_true",
+                    help="backward = compositing backward + projection backward fused with the Adam step "
+                         "(the reference's FPBO mode); K9 then includes the optimizer's 1.4 kB/splat of traffic")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run device copies / fills of known size (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE) and exit")
     args = ap.parse_args()
@@ -127,10 +130,32 @@ def main():
                       overwrite_world_grads=native, packed_projection=args.packed_projection)
     L = lib.load()
 
-    eng.time_iterations(max(args.warmup, 1))
+    hyper = dict(lr_means=1.6e-6, lr_quats=1e-5, lr_scales=5e-5, lr_opacs=5e-4, lr_features_dc=2.5e-5, lr_features_sh=1.25e-6)
+    adam_step = [0]
+
+    def backward():
+        if args.fused_optimizer:
+            adam_step[0] += 1
+            eng.backward_fused_optimizer(hyper, adam_step[0])
+        else:
+            eng.backward()
+
+    def run(iters):
+        if not args.fused_optimizer:
+            return eng.time_iterations(iters)
+        out = np.zeros(iters, np.float32)
+        for i in range(iters):
+            t = time.perf_counter()
+            eng.forward()
+            backward()
+            lib.check(L.ssr_device_synchronize())
+            out[i] = (time.perf_counter() - t) * 1e3
+        return out
+
+    run(max(args.warmup, 1))
     lib.check(L.ssr_device_synchronize())
     t0 = time.perf_counter()
-    ms = eng.time_iterations(args.steps)
+    ms = run(args.steps)
     lib.check(L.ssr_device_synchronize())
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
@@ -141,7 +166,7 @@ def main():
     reps = 5
     for _ in range(reps):
         eng.forward()
-        eng.backward()
+        backward()
         for k, v in eng.stage_times().items():
             acc[k] = acc.get(k, 0.0) + v / reps
     eng.set_stage_profiling(False)
@@ -180,7 +205,8 @@ def main():
                                f"{['fp32', 'ref-q8', 'ref-q16', 'int8*fp16scale'][sc.sh_codec]}, tile 16x16, seed {pkg.scenes.CONFIGS[cfg]['seed']:#x}",
                    "visible": V, "n_isects": K, "K_b": K_b, "tiles": T, "pixels": P,
                    "stage_order": ("fused tile count, visible-splat work list, packed fragment rows, plain-store gradients" if native else "reference order")
-                                  + (", packed projection outputs" if args.packed_projection else ""),
+                                  + (", packed projection outputs" if args.packed_projection else "")
+                                  + (", projection backward fused with Adam" if args.fused_optimizer else ""),
                    "device_ms_per_iter_median": float(np.median(ms))},
         "hbm_roofline_frac_whole_iteration": total_bytes / (float(np.median(ms)) * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "algorithmic_bytes_per_iter": total_bytes,

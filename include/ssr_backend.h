@@ -257,6 +257,38 @@ typedef struct {
 } ssr_projection_bwd_params;
 int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream_t stream);
 
+/* ---- K9 fused with the optimizer step: fused_projection_bwd_optimizer_3dgs
+ * (src/kernels/optim/FusedProjectionBwdOptim.cuh:18-62; kernel
+ * src/kernels/optim/FusedProjectionBwdOptim_kernel.cuh:146-1030, the fp32-state branch). One pass
+ * over ALL num_splats splats: the projection VJP of the visible ones (aabb test as in K9) is kept in
+ * registers, the per-splat regularizer gradients are added, and Adam (beta1 0.9, beta2 0.999,
+ * eps 1e-15, bias-corrected) updates the six parameter arrays and both moment sets in place --
+ * the 236 B/splat gradient round trip through HBM disappears. Quaternions take the Riemannian
+ * step (gradient projected on the tangent of the unit sphere, result re-normalised). Splats that
+ * are not visible still decay their moments, as in the reference.
+ * Built: fp32 parameters and moments, one camera, non-packed, regularizers mcmc_opacity,
+ * mcmc_scale, scale ratio, quaternion norm and SH/DC magnitude. Not built (rejected): quantized
+ * Adam state, value-quantized SH, effective-rank regularizer, scale-agnostic mean step,
+ * colour trust region. */
+typedef struct {
+    int64_t num_splats;
+    int32_t sh_degree;
+    ssr_world world;            /* parameters, updated in place; features_sh fp32 */
+    ssr_camera camera;
+    const float* aabb;          /* [N,4] of the forward */
+    ssr_screen v_screen;        /* read: output of ssr_raster_bwd */
+    ssr_world v_world_in;       /* optional gradient contributions already accumulated (any member may
+                                   be NULL = zero; features_sh is not read, as in the reference) */
+    ssr_world g1, g2;           /* Adam first / second moments, same shapes as world, updated in place */
+    float* densify_score;       /* optional [N]: exp(max log-scale) * |dL/dmean| */
+    float lr_means, lr_quats, lr_scales, lr_opacs, lr_features_dc, lr_features_sh;
+    float max_gauss_ratio, scale_regularization_weight;
+    float mcmc_opacity_reg_weight, mcmc_scale_reg_weight, quat_norm_reg_weight, sh_reg_weight;
+    int32_t step;               /* Adam step (>= 1) when `steps` is NULL */
+    const int32_t* steps;       /* optional per-splat step [N] */
+} ssr_fpbo_params;
+int ssr_fused_projection_bwd_optimizer(const ssr_fpbo_params* p, ssr_stream_t stream);
+
 /* Zeroes the gradient rows of the listed splats only (the rows a previous ssr_projection_bwd run
  * over that list wrote), instead of refilling all N rows. No counterpart in the reference, which
  * always refills (src/engine/EngineLoss.cpp:120-127).

@@ -461,6 +461,104 @@ void or_math(int op, int64_t n, const float* a, const float* b, float* out) {
 
 void or_decode_sh(int64_t gid, const or_sh_source* sh, float* out45) { decode_sh(gid, sh, 15, out45); }
 
+// Fused projection backward + Adam, fp32 state (src/kernels/optim/FusedProjectionBwdOptim_kernel.cuh:232-710
+// with BLOCK_SIZE == 0, VALUE_BITS == 32, use_scale_agnostic_mean = color_trust_linear = false).
+// The data gradient is or_projection_bwd's; the regularizers are the closed-form derivatives of
+// src/shaders/per_splat_losses.slang:30-81 (effective-rank terms not included: weight 0).
+void or_fused_projection_bwd_optimizer(int64_t N, int sh_degree,
+    float* means, float* quats, float* log_scales, float* opacity_logits, float* features_dc, float* features_sh,
+    const or_camera* cam, const float* aabb,
+    const float* v_xy, const float* v_sdepth, const float* v_conic, const float* v_opac, const float* v_srgb,
+    const float* const* v_in, float* const* g1, float* const* g2, float* densify_score,
+    const float* hyper, int32_t step, const int32_t* steps) {
+    const int n_coef = sh_degree * (sh_degree + 2);
+    std::vector<float> vm((size_t)N * 3), vq((size_t)N * 4), vs((size_t)N * 3), vo((size_t)N), vd((size_t)N * 3),
+        vsh((size_t)N * 45);
+    or_sh_source src;
+    memset(&src, 0, sizeof(src));
+    src.codec = OR_SH_F32; src.sh_f32 = features_sh; src.num_sh_buffer = 15;
+    or_projection_bwd(N, sh_degree, means, quats, log_scales, opacity_logits, features_dc, &src, cam, aabb, v_xy, v_sdepth,
+                      v_conic, v_opac, v_srgb, vm.data(), vq.data(), vs.data(), vo.data(), vd.data(), vsh.data());
+    const float lr_means = hyper[0], lr_quats = hyper[1], lr_scales = hyper[2], lr_opacs = hyper[3], lr_dc = hyper[4],
+                lr_sh = hyper[5], max_ratio = hyper[6], scale_w = hyper[7], mcmc_o = hyper[8], mcmc_s = hyper[9],
+                qnorm_w = hyper[10], sh_w = hyper[11];
+    const float kBeta1 = 0.9f, kBeta2 = 0.999f, kEps = 1e-15f;
+    const float sh_reg = sh_w * (1.0f / (float)(n_coef > 0 ? n_coef : 1));
+#pragma omp parallel for schedule(static)
+    for (int64_t g = 0; g < N; g++) {
+        float b1c, b2c;
+        if (steps) {
+            const float t = (float)steps[g];
+            b1c = 1.0f / (1.0f - ssr_exp(t * -0.105360515657826301f));
+            b2c = 1.0f / (1.0f - ssr_exp(t * -0.00100050033358353350f));
+        } else {
+            b1c = (float)(1.0 / (1.0 - pow(0.9, (double)step)));
+            b2c = (float)(1.0 / (1.0 - pow(0.999, (double)step)));
+        }
+        auto adam = [&](float x, float v, float lr, float* g1p, float* g2p) {
+            const float a = kBeta1 * *g1p + (1.f - kBeta1) * v;
+            const float b = kBeta2 * *g2p + (1.f - kBeta2) * (v * v);
+            *g1p = a; *g2p = b;
+            return x - ((lr * b1c) * a) / (ssr_sqrt(b * b2c) + kEps);
+        };
+        auto vin = [&](int k, int64_t i) { return v_in && v_in[k] ? v_in[k][i] : 0.0f; };
+        float gm[3], gq[4], gs[3], go, gd[3];
+        for (int i = 0; i < 3; i++) {
+            gm[i] = vin(0, 3 * g + i) + vm[3 * g + i];
+            gs[i] = vin(2, 3 * g + i) + vs[3 * g + i];
+            gd[i] = vin(4, 3 * g + i) + vd[3 * g + i];
+        }
+        for (int i = 0; i < 4; i++) gq[i] = vin(1, 4 * g + i) + vq[4 * g + i];
+        go = vin(3, g) + vo[g];
+        // SH
+        for (int i = 0; i < 3 * n_coef; i++) {
+            float* x = features_sh + 45 * g + i;
+            *x = adam(*x, vsh[45 * g + i] + sh_reg * *x, lr_sh, g1[5] + 45 * g + i, g2[5] + 45 * g + i);
+        }
+        const float* ls = log_scales + 3 * g;
+        const float* q0 = quats + 4 * g;
+        const float logit = opacity_logits[g];
+        // regularizers
+        const float sg = ssr_sigmoid(logit);
+        go += mcmc_o * (sg * (1.0f - sg));
+        const float ms = (mcmc_s * 1e-2f) / 3.0f;
+        const float e[3] = {ssr_exp(ls[0]), ssr_exp(ls[1]), ssr_exp(ls[2])};
+        int imax = 0, imin = 0;
+        for (int i = 1; i < 3; i++) { if (e[i] > e[imax]) imax = i; if (e[i] < e[imin]) imin = i; }
+        const float ratio = e[imax] / e[imin];
+        const float rg = ratio > max_ratio ? scale_w * ratio : 0.0f;
+        for (int i = 0; i < 3; i++) gs[i] += ms + (i == imax ? rg : 0.f) - (i == imin ? rg : 0.f);
+        const float qn = ssr_sqrt((q0[0] * q0[0] + q0[1] * q0[1]) + (q0[2] * q0[2] + q0[3] * q0[3]));
+        const float qg = qnorm_w * ((1.0f - 1.0f / qn) / qn);
+        for (int i = 0; i < 4; i++) gq[i] += qg * q0[i];
+        const float lim = 0.5f / 0.28209479177387814f;
+        for (int i = 0; i < 3; i++)
+            gd[i] += sh_w * (ssr_max(features_dc[3 * g + i] - lim, 0.0f) + ssr_min(features_dc[3 * g + i] + lim, 0.0f));
+        const float smax = ssr_max(ssr_max(ls[0], ls[1]), ls[2]);
+        // scales
+        float new_ls[3];
+        for (int i = 0; i < 3; i++) new_ls[i] = adam(ls[i], gs[i], lr_scales, g1[2] + 3 * g + i, g2[2] + 3 * g + i);
+        // quats, Riemannian
+        {
+            const float inv = 1.0f / qn;
+            float q[4], v[4];
+            for (int i = 0; i < 4; i++) q[i] = q0[i] * inv;
+            const float d = (q[0] * gq[0] + q[1] * gq[1]) + (q[2] * gq[2] + q[3] * gq[3]);
+            for (int i = 0; i < 4; i++) v[i] = gq[i] - d * q[i];
+            for (int i = 0; i < 4; i++) q[i] = adam(q[i], v[i], lr_quats, g1[1] + 4 * g + i, g2[1] + 4 * g + i);
+            const float minv = 1.0f / ssr_sqrt((q[0] * q[0] + q[1] * q[1]) + (q[2] * q[2] + q[3] * q[3]));
+            for (int i = 0; i < 4; i++) quats[4 * g + i] = q[i] * minv;
+        }
+        for (int i = 0; i < 3; i++) log_scales[3 * g + i] = new_ls[i];
+        opacity_logits[g] = adam(logit, go, lr_opacs, g1[3] + g, g2[3] + g);
+        if (densify_score) densify_score[g] = ssr_exp(smax) * ssr_sqrt(dot3(gm, gm));
+        for (int i = 0; i < 3; i++) means[3 * g + i] = adam(means[3 * g + i], gm[i], lr_means, g1[0] + 3 * g + i, g2[0] + 3 * g + i);
+        for (int i = 0; i < 3; i++)
+            features_dc[3 * g + i] = adam(features_dc[3 * g + i], gd[i], lr_dc, g1[4] + 3 * g + i, g2[4] + 3 * g + i);
+    }
+}
+
+
 // QuantizedTensor<BITS,256>::encode_v with block-reduced bounds, src/core/Tensor.h:1364-1392
 void or_quantize_ref(int bits, int64_t n_cells, int64_t stride, const float* v, uint8_t* packed,
                      float* bounds) {

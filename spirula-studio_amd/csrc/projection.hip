@@ -11,6 +11,9 @@
 //
 // One thread per Gaussian, 256 threads (4 wavefronts) per workgroup. Both kernels are bound by
 // HBM traffic (236 B in, 60 B out per visible splat forward; 472 B in/out backward).
+#include <math.h>
+#include <string.h>
+
 #include "projection_device.h"
 #include "raster_device.h"
 
@@ -319,31 +322,17 @@ __device__ __forceinline__ void put(float* p, float v) {
     else *p = v;
 }
 
-template <int kDegree, bool kAccumulate>
-__global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projection_bwd_params P) {
-    const int64_t i = (int64_t)blockIdx.x * kProjBlock + threadIdx.x;
-    if (i >= (P.packed_gaussian_ids ? P.num_packed : (P.visible_ids ? P.n_visible : P.num_splats))) return;
-    // g: row of the splat in world / v_world; r: its row in v_screen (ProjectionBwd_kernel.cuh:51-63)
-    const int64_t g = P.packed_gaussian_ids ? (int64_t)P.packed_gaussian_ids[i] : (P.visible_ids ? (int64_t)P.visible_ids[i] : i);
-    const int64_t r = P.packed_gaussian_ids ? i : g;
+// Gradient of one splat's screen row with respect to its world row (everything K9 computes before
+// it stores): g is the splat's row in `W`, r its row in `VS`. sh_sink(j, Yj, vc) receives the two
+// factors of the gradient of SH coefficient j (j < kDegree (kDegree + 2)), which is Yj * vc[0..2].
+struct WorldGradD { float mean[3], quat[4], scale[3], logit, dc[3]; };
+
+template <int kDegree, class ShSink>
+__device__ __forceinline__ void projection_vjp(const CamD& cam, const ssr_world& W, const ssr_sh_quant& Q, int64_t g,
+                                               const ssr_screen& VS, int64_t r, WorldGradD& out, ShSink&& sh_sink) {
     constexpr int kCoef = kDegree * (kDegree + 2);
-    float4 bb = make_float4(0.f, 0.f, 1.f, 1.f);
-    if (!P.packed_gaussian_ids) bb = reinterpret_cast<const float4*>(P.aabb)[g];
-    ssr_world& V = P.v_world;
-    if (bb.z <= bb.x || bb.w <= bb.y) {   // ProjectionBwd_kernel.cuh:58
-        if (!kAccumulate && !P.visible_ids) {
-#pragma unroll
-            for (int i = 0; i < 3; i++) { V.means[3 * g + i] = 0.f; V.log_scales[3 * g + i] = 0.f; V.features_dc[3 * g + i] = 0.f; }
-            *reinterpret_cast<float4*>(V.quats + 4 * g) = make_float4(0.f, 0.f, 0.f, 0.f);
-            V.opacity_logits[g] = 0.f;
-            float* vs = V.features_sh + g * (int64_t)V.sh_stride;
-            for (int i = 0; i < V.sh_stride; i++) vs[i] = 0.f;
-        }
-        return;
-    }
-    const CamD cam = load_camera(P.camera);
     float mean[3], quat[4], ls[3], logit;
-    load_splat(P.world, g, mean, quat, ls, logit);
+    load_splat(W, g, mean, quat, ls, logit);
     ProjD p;
     project<true>(cam, mean, quat, ls, logit, p);
     const float x = p.mc[0], y = p.mc[1], z = p.mc[2];
@@ -351,7 +340,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
     // conic = inverse(cov2d)
     const float c00 = p.c2[0][0], c01 = p.c2[0][1], c10 = p.c2[1][0], c11 = p.c2[1][1];
     const float det = c00 * c11 - c01 * c10, inv = 1.0f / det;
-    const float* vcn = P.v_screen.conic + 3 * r;
+    const float* vcn = VS.conic + 3 * r;
     const float g00 = vcn[0], g01 = vcn[1], g11 = vcn[2];
     const float v_inv = (c11 * g00 - c01 * g01) + c00 * g11;
     const float v_det = -(v_inv / (det * det));
@@ -385,7 +374,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
                 for (int j = 0; j < 2; j++) s += p.J[i][k] * vC[i][j] * p.J[j][l];
             vS[k][l] = s;
         }
-    const float vm0 = P.v_screen.xy[2 * r], vm1 = P.v_screen.xy[2 * r + 1];
+    const float vm0 = VS.xy[2 * r], vm1 = VS.xy[2 * r + 1];
     if (cam.model == SSR_CAM_PINHOLE) {
         const float z2 = z * z, iz = 1.0f / z, iz2 = 1.0f / z2;
         vmc[2] += vJ[0][0] * (-cam.fx * iz2) + vJ[1][1] * (-cam.fy * iz2);
@@ -424,7 +413,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
     }
     {   // depth = length(mean_c); the sqrt derivative is guarded at 1e-7
         const float s2 = dot3(p.mc, p.mc);
-        const float vs = P.v_screen.depth[r] * (0.5f / ssr_sqrt(ssr_max(1e-7f, s2)));
+        const float vs = VS.depth[r] * (0.5f / ssr_sqrt(ssr_max(1e-7f, s2)));
 #pragma unroll
         for (int i = 0; i < 3; i++) vmc[i] += 2.0f * p.mc[i] * vs;
     }
@@ -472,36 +461,28 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
     float vquat[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) vquat[i] = (vqn[i] - p.qn[i] * qd) * p.qinv;
-    const float vlogit = P.v_screen.opac[r] * (p.opac * (1.0f - p.opac));
+    const float vlogit = VS.opac[r] * (p.opac * (1.0f - p.opac));
 
     // SH colour VJP (src/shaders/harmonics.slang:373-649,1087-1126)
     float coef[kCoef > 0 ? 3 * kCoef : 1];
-    if (kCoef > 0) decode_sh<kCoef>(P.world, P.sh, g, coef);
+    if (kCoef > 0) decode_sh<kCoef>(W, Q, g, coef);
     float dir[3];
     view_dir(cam, mean, dir);
     ShBasisD b;
     sh_basis<kDegree>(dir, b);
-    const float* dcp = P.world.features_dc + 3 * g;
+    const float* dcp = W.features_dc + 3 * g;
     const float dc[3] = {dcp[0], dcp[1], dcp[2]};
     float raw[3];
     sh_color_raw<kDegree>(b, dc, coef, raw);
-    const float* vrg = P.v_screen.rgb + 3 * r;
+    const float* vrg = VS.rgb + 3 * r;
     float vc[3];
 #pragma unroll
     for (int c = 0; c < 3; c++) vc[c] = vrg[c] * (raw[c] >= -0.5f ? 1.0f : 0.0f);
     float vdir[3] = {0.f, 0.f, 0.f};
-    float* vsh = V.features_sh + g * (int64_t)V.sh_stride;
     if (kDegree >= 1) {
 #pragma unroll
         for (int j = 0; j < kCoef; j++) {
-            const float tv[3] = {b.Y[j] * vc[0], b.Y[j] * vc[1], b.Y[j] * vc[2]};
-            const float d2 = dot3(tv, tv);
-            const bool ok = ssr_isfinite(d2) && d2 != 0.0f;   // harmonics.slang:397-403
-#pragma unroll
-            for (int c = 0; c < 3; c++) {
-                if (kAccumulate) { if (ok) atomicAdd(vsh + 3 * j + c, tv[c]); }
-                else vsh[3 * j + c] = ok ? tv[c] : 0.0f;
-            }
+            sh_sink(j, b.Y[j], vc);
         }
         auto cd = [&](int j) { return (coef[3 * j] * vc[0] + coef[3 * j + 1] * vc[1]) + coef[3 * j + 2] * vc[2]; };
         const float X = b.x, Y = b.y, Z = b.z;
@@ -545,19 +526,206 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
         vdir[1] = (vy - dn * Y) * b.inorm;
         vdir[2] = (vz - dn * Z) * b.inorm;
     }
+#pragma unroll
+    for (int i = 0; i < 3; i++) { out.mean[i] = vmean[i] + vdir[i]; out.scale[i] = vscale[i]; out.dc[i] = 0.2820947917738781f * vc[i]; }
+#pragma unroll
+    for (int i = 0; i < 4; i++) out.quat[i] = vquat[i];
+    out.logit = vlogit;
+}
+
+template <int kDegree, bool kAccumulate>
+__global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projection_bwd_params P) {
+    const int64_t i = (int64_t)blockIdx.x * kProjBlock + threadIdx.x;
+    if (i >= (P.packed_gaussian_ids ? P.num_packed : (P.visible_ids ? P.n_visible : P.num_splats))) return;
+    // g: row of the splat in world / v_world; r: its row in v_screen (ProjectionBwd_kernel.cuh:51-63)
+    const int64_t g = P.packed_gaussian_ids ? (int64_t)P.packed_gaussian_ids[i] : (P.visible_ids ? (int64_t)P.visible_ids[i] : i);
+    const int64_t r = P.packed_gaussian_ids ? i : g;
+    constexpr int kCoef = kDegree * (kDegree + 2);
+    float4 bb = make_float4(0.f, 0.f, 1.f, 1.f);
+    if (!P.packed_gaussian_ids) bb = reinterpret_cast<const float4*>(P.aabb)[g];
+    ssr_world& V = P.v_world;
+    if (bb.z <= bb.x || bb.w <= bb.y) {   // ProjectionBwd_kernel.cuh:58
+        if (!kAccumulate && !P.visible_ids) {
+#pragma unroll
+            for (int i = 0; i < 3; i++) { V.means[3 * g + i] = 0.f; V.log_scales[3 * g + i] = 0.f; V.features_dc[3 * g + i] = 0.f; }
+            *reinterpret_cast<float4*>(V.quats + 4 * g) = make_float4(0.f, 0.f, 0.f, 0.f);
+            V.opacity_logits[g] = 0.f;
+            float* vs = V.features_sh + g * (int64_t)V.sh_stride;
+            for (int i = 0; i < V.sh_stride; i++) vs[i] = 0.f;
+        }
+        return;
+    }
+    const CamD cam = load_camera(P.camera);
+    WorldGradD wg;
+    float* vsh = V.features_sh + g * (int64_t)V.sh_stride;
+    projection_vjp<kDegree>(cam, P.world, P.sh, g, P.v_screen, r, wg, [&](int j, float Yj, const float vc[3]) {
+        const float tv[3] = {Yj * vc[0], Yj * vc[1], Yj * vc[2]};
+        const float d2 = dot3(tv, tv);
+        const bool ok = ssr_isfinite(d2) && d2 != 0.0f;   // harmonics.slang:397-403
+#pragma unroll
+        for (int c = 0; c < 3; c++) {
+            if (kAccumulate) { if (ok) atomicAdd(vsh + 3 * j + c, tv[c]); }
+            else vsh[3 * j + c] = ok ? tv[c] : 0.0f;
+        }
+    });
     if (!kAccumulate) {   // coefficients above the active degree receive nothing
         for (int i = 3 * kCoef; i < V.sh_stride; i++) vsh[i] = 0.0f;
     }
     // World::atomicStore (src/primitives/PrimitiveBase3DGS.cuh:75-83): per-component finite filter
 #pragma unroll
-    for (int i = 0; i < 3; i++) put<kAccumulate>(V.means + 3 * g + i, fin(vmean[i] + vdir[i]));
+    for (int i = 0; i < 3; i++) put<kAccumulate>(V.means + 3 * g + i, fin(wg.mean[i]));
 #pragma unroll
-    for (int i = 0; i < 4; i++) put<kAccumulate>(V.quats + 4 * g + i, fin(vquat[i]));
+    for (int i = 0; i < 4; i++) put<kAccumulate>(V.quats + 4 * g + i, fin(wg.quat[i]));
 #pragma unroll
-    for (int i = 0; i < 3; i++) put<kAccumulate>(V.log_scales + 3 * g + i, fin(vscale[i]));
-    put<kAccumulate>(V.opacity_logits + g, fin(vlogit));
+    for (int i = 0; i < 3; i++) put<kAccumulate>(V.log_scales + 3 * g + i, fin(wg.scale[i]));
+    put<kAccumulate>(V.opacity_logits + g, fin(wg.logit));
 #pragma unroll
-    for (int i = 0; i < 3; i++) put<kAccumulate>(V.features_dc + 3 * g + i, fin(0.2820947917738781f * vc[i]));
+    for (int i = 0; i < 3; i++) put<kAccumulate>(V.features_dc + 3 * g + i, fin(wg.dc[i]));
+}
+
+// ---- projection backward fused with Adam ---------------------------------------------------------
+struct AdamD { float b1c, b2c; };   // 1/(1-beta1^t), 1/(1-beta2^t)
+
+__device__ __forceinline__ float adam_step(float x, float v, float lr, const AdamD& a, float* g1p, float* g2p) {
+    constexpr float kBeta1 = 0.9f, kBeta2 = 0.999f, kEps = 1e-15f;
+    const float g1 = kBeta1 * *g1p + (1.f - kBeta1) * v;
+    const float g2 = kBeta2 * *g2p + (1.f - kBeta2) * (v * v);
+    *g1p = g1; *g2p = g2;
+    return x - ((lr * a.b1c) * g1) / (ssr_sqrt(g2 * a.b2c) + kEps);
+}
+
+// Two phases per workgroup of 256 splats. Phase 1, one thread per splat: projection VJP in
+// registers, regularizers, Adam on the 14 non-SH parameters; the SH gradient is rank one
+// (Y_j * v_colour), so only its factors (15 + 3 floats) go to LDS. Phase 2, the workgroup streams
+// over its 256 x 3 kCoef SH coefficients in memory order: parameter and both moments are read and
+// written fully coalesced, the gradient is rebuilt from the factors in LDS.
+template <int kDegree>
+__global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_kernel(ssr_fpbo_params P, AdamD scalar_adam) {
+    constexpr int kCoef = kDegree * (kDegree + 2);
+    constexpr int kY = kCoef > 0 ? kCoef : 1;
+    __shared__ float s_Y[kProjBlock][kY + 1];   // +1: odd row pitch, conflict-free column reads
+    __shared__ float s_vc[kProjBlock][3];
+    __shared__ float s_b1c[kProjBlock], s_b2c[kProjBlock];
+    const int64_t block0 = (int64_t)blockIdx.x * kProjBlock;
+    const int64_t g = block0 + threadIdx.x;
+    const ssr_world& W = P.world;
+    AdamD ad = scalar_adam;
+#pragma unroll
+    for (int j = 0; j < kY; j++) s_Y[threadIdx.x][j] = 0.f;
+    s_vc[threadIdx.x][0] = s_vc[threadIdx.x][1] = s_vc[threadIdx.x][2] = 0.f;
+    if (g < P.num_splats) {
+        if (P.steps) {   // per-splat step: beta^t = exp(t ln beta)
+            const float t = (float)P.steps[g];
+            ad.b1c = 1.0f / (1.0f - ssr_exp(t * -0.105360515657826301f));
+            ad.b2c = 1.0f / (1.0f - ssr_exp(t * -0.00100050033358353350f));
+        }
+        // gradient contributions that are already there (World::atomicLoad, FusedProjectionBwdOptim_kernel.cuh:250-251)
+        WorldGradD wg;
+        const ssr_world& VI = P.v_world_in;
+#pragma unroll
+        for (int i = 0; i < 3; i++) {
+            wg.mean[i] = VI.means ? VI.means[3 * g + i] : 0.f;
+            wg.scale[i] = VI.log_scales ? VI.log_scales[3 * g + i] : 0.f;
+            wg.dc[i] = VI.features_dc ? VI.features_dc[3 * g + i] : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) wg.quat[i] = VI.quats ? VI.quats[4 * g + i] : 0.f;
+        wg.logit = VI.opacity_logits ? VI.opacity_logits[g] : 0.f;
+
+        const float4 bb = reinterpret_cast<const float4*>(P.aabb)[g];
+        if (!(bb.z <= bb.x || bb.w <= bb.y)) {   // FusedProjectionBwdOptim_kernel.cuh:271-272
+            const CamD cam = load_camera(P.camera);
+            WorldGradD pg;
+            ssr_sh_quant none;
+            none.codec = SSR_SH_F32; none.packed = nullptr; none.bounds = nullptr; none.bounds_stride = 0;
+            none.num_sh_buffer = 0; none.scale_f16 = nullptr;
+            projection_vjp<kDegree>(cam, W, none, g, P.v_screen, g, pg, [&](int j, float Yj, const float vc[3]) {
+                s_Y[threadIdx.x][j] = Yj;
+                if (j == 0) { s_vc[threadIdx.x][0] = vc[0]; s_vc[threadIdx.x][1] = vc[1]; s_vc[threadIdx.x][2] = vc[2]; }
+            });
+#pragma unroll
+            for (int i = 0; i < 3; i++) { wg.mean[i] += pg.mean[i]; wg.scale[i] += pg.scale[i]; wg.dc[i] += pg.dc[i]; }
+#pragma unroll
+            for (int i = 0; i < 4; i++) wg.quat[i] += pg.quat[i];
+            wg.logit += pg.logit;
+        }
+        // parameters as they were before this step
+        float mean[3], quat[4], ls[3], logit;
+        load_splat(W, g, mean, quat, ls, logit);
+        const float* dcp = W.features_dc + 3 * g;
+        const float dc[3] = {dcp[0], dcp[1], dcp[2]};
+
+        // per-splat regularizers (src/shaders/per_splat_losses.slang:30-81, v_loss = 1)
+        {
+            const float sg = ssr_sigmoid(logit);
+            wg.logit += P.mcmc_opacity_reg_weight * (sg * (1.0f - sg));
+            const float ms = (P.mcmc_scale_reg_weight * 1e-2f) / 3.0f;
+            const float e[3] = {ssr_exp(ls[0]), ssr_exp(ls[1]), ssr_exp(ls[2])};
+            int imax = 0, imin = 0;
+            for (int i = 1; i < 3; i++) { if (e[i] > e[imax]) imax = i; if (e[i] < e[imin]) imin = i; }
+            const float ratio = e[imax] / e[imin];
+            const float rg = ratio > P.max_gauss_ratio ? P.scale_regularization_weight * ratio : 0.0f;
+#pragma unroll
+            for (int i = 0; i < 3; i++) wg.scale[i] += ms + (i == imax ? rg : 0.f) - (i == imin ? rg : 0.f);
+            const float qn = ssr_sqrt((quat[0] * quat[0] + quat[1] * quat[1]) + (quat[2] * quat[2] + quat[3] * quat[3]));
+            const float qg = P.quat_norm_reg_weight * ((1.0f - 1.0f / qn) / qn);
+#pragma unroll
+            for (int i = 0; i < 4; i++) wg.quat[i] += qg * quat[i];
+            const float lim = 0.5f / 0.28209479177387814f;   // FusedProjectionBwdOptim_kernel.cuh:354-357
+#pragma unroll
+            for (int i = 0; i < 3; i++) wg.dc[i] += P.sh_reg_weight * (ssr_max(dc[i] - lim, 0.0f) + ssr_min(dc[i] + lim, 0.0f));
+        }
+
+        // scales, quats (Riemannian), opacity, means, dc -- FusedProjectionBwdOptim_kernel.cuh:390-612
+#pragma unroll
+        for (int i = 0; i < 3; i++)
+            W.log_scales[3 * g + i] = adam_step(ls[i], wg.scale[i], P.lr_scales, ad, P.g1.log_scales + 3 * g + i, P.g2.log_scales + 3 * g + i);
+        {
+            const float n2 = (quat[0] * quat[0] + quat[1] * quat[1]) + (quat[2] * quat[2] + quat[3] * quat[3]);
+            const float inv = 1.0f / ssr_sqrt(n2);
+            float q[4], v[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) q[i] = quat[i] * inv;
+            const float d = (q[0] * wg.quat[0] + q[1] * wg.quat[1]) + (q[2] * wg.quat[2] + q[3] * wg.quat[3]);
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[i] = wg.quat[i] - d * q[i];
+#pragma unroll
+            for (int i = 0; i < 4; i++) q[i] = adam_step(q[i], v[i], P.lr_quats, ad, P.g1.quats + 4 * g + i, P.g2.quats + 4 * g + i);
+            const float m2 = (q[0] * q[0] + q[1] * q[1]) + (q[2] * q[2] + q[3] * q[3]);
+            const float minv = 1.0f / ssr_sqrt(m2);
+            *reinterpret_cast<float4*>(W.quats + 4 * g) = make_float4(q[0] * minv, q[1] * minv, q[2] * minv, q[3] * minv);
+        }
+        W.opacity_logits[g] = adam_step(logit, wg.logit, P.lr_opacs, ad, P.g1.opacity_logits + g, P.g2.opacity_logits + g);
+        if (P.densify_score) {
+            const float smax = ssr_max(ssr_max(ls[0], ls[1]), ls[2]);
+            P.densify_score[g] = ssr_exp(smax) * ssr_sqrt(dot3(wg.mean, wg.mean));
+        }
+#pragma unroll
+        for (int i = 0; i < 3; i++)
+            W.means[3 * g + i] = adam_step(mean[i], wg.mean[i], P.lr_means, ad, P.g1.means + 3 * g + i, P.g2.means + 3 * g + i);
+#pragma unroll
+        for (int i = 0; i < 3; i++)
+            W.features_dc[3 * g + i] = adam_step(dc[i], wg.dc[i], P.lr_features_dc, ad, P.g1.features_dc + 3 * g + i, P.g2.features_dc + 3 * g + i);
+    }
+    s_b1c[threadIdx.x] = ad.b1c; s_b2c[threadIdx.x] = ad.b2c;
+    if (kCoef == 0) return;
+    __syncthreads();
+    // phase 2: SH coefficients of the workgroup's splats in memory order (FusedProjectionBwdOptim_kernel.cuh:667-710)
+    const int64_t rest = P.num_splats - block0;
+    const int n_here = rest < kProjBlock ? (int)rest : kProjBlock;
+    const float sh_reg = P.sh_reg_weight * (1.0f / (float)kY);
+    constexpr int kPer = 3 * kCoef;
+    for (int e = threadIdx.x; e < n_here * kPer; e += kProjBlock) {
+        const int sp = e / kPer, i = e - sp * kPer;
+        const int j = i / 3, c = i - 3 * j;
+        const int64_t row = block0 + sp;
+        float* xp = W.features_sh + row * W.sh_stride + i;
+        const float x = *xp;
+        const float v = s_Y[sp][j] * s_vc[sp][c] + sh_reg * x;
+        AdamD a;
+        a.b1c = s_b1c[sp]; a.b2c = s_b2c[sp];
+        *xp = adam_step(x, v, P.lr_features_sh, a, P.g1.features_sh + row * P.g1.sh_stride + i, P.g2.features_sh + row * P.g2.sh_stride + i);
+    }
 }
 
 // One wavefront per listed splat: lane l zeroes float l of its 59-float gradient row
@@ -746,6 +914,39 @@ extern "C" int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream
     }
 #undef SSR_LAUNCH_BWD
     SSR_CHECK_LAUNCH("ssr_projection_bwd");
+    return 0;
+}
+
+extern "C" int ssr_fused_projection_bwd_optimizer(const ssr_fpbo_params* p, ssr_stream_t stream) {
+    const char* where = "ssr_fused_projection_bwd_optimizer";
+    SSR_REQUIRE(p, where, "null params");
+    ssr_sh_quant none;
+    memset(&none, 0, sizeof(none));
+    int e = check_common(where, p->num_splats, p->sh_degree, p->world, none, p->camera);
+    if (e) return e;
+    if (p->num_splats == 0) return 0;
+    SSR_REQUIRE(p->aabb && (reinterpret_cast<uintptr_t>(p->aabb) & 15) == 0, where, "aabb must be non-null and 16-byte aligned");
+    SSR_REQUIRE(p->v_screen.xy && p->v_screen.depth && p->v_screen.conic && p->v_screen.opac && p->v_screen.rgb, where,
+                "null v_screen buffer");
+    for (const ssr_world* w : {&p->world, &p->g1, &p->g2}) {
+        SSR_REQUIRE(w->means && w->quats && w->log_scales && w->opacity_logits && w->features_dc, where, "null parameter or moment buffer");
+        SSR_REQUIRE(p->sh_degree == 0 || (w->features_sh && w->sh_stride >= 3 * p->sh_degree * (p->sh_degree + 2)), where,
+                    "features_sh missing or sh_stride too small");
+    }
+    SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->world.quats) & 15) == 0, where, "quats must be 16-byte aligned");
+    SSR_REQUIRE(p->steps || p->step >= 1, where, "Adam step must be >= 1");
+    AdamD ad;
+    ad.b1c = (float)(1.0 / (1.0 - pow(0.9, (double)p->step)));
+    ad.b2c = (float)(1.0 / (1.0 - pow(0.999, (double)p->step)));
+    const dim3 grid((unsigned)ceil_div(p->num_splats, kProjBlock)), block(kProjBlock);
+    hipStream_t s = as_stream(stream);
+    switch (p->sh_degree) {
+        case 0: hipLaunchKernelGGL(fused_projection_bwd_optimizer_kernel<0>, grid, block, 0, s, *p, ad); break;
+        case 1: hipLaunchKernelGGL(fused_projection_bwd_optimizer_kernel<1>, grid, block, 0, s, *p, ad); break;
+        case 2: hipLaunchKernelGGL(fused_projection_bwd_optimizer_kernel<2>, grid, block, 0, s, *p, ad); break;
+        default: hipLaunchKernelGGL(fused_projection_bwd_optimizer_kernel<3>, grid, block, 0, s, *p, ad); break;
+    }
+    SSR_CHECK_LAUNCH(where);
     return 0;
 }
 

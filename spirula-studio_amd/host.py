@@ -22,6 +22,8 @@ SYMBOLS = {
     "ssrh_set_data_3dgs": (C.c_int, [C.c_int64, vp, vp, vp, vp, vp, vp, C.c_int]),
     "ssrh_set_sh_value_quant": (C.c_int, [C.c_int, vp, C.c_int64, C.c_int, vp, C.c_int64, C.c_int, C.c_int64]),
     "ssrh_set_camera_params": (C.c_int, [C.c_int, C.c_int, C.c_char_p, C.c_char_p, vp, vp, C.c_int]),
+    "ssrh_backward_fused_optimizer": (C.c_int, [vp, vp, vp, vp, C.c_int]),
+    "ssrh_copy_params_to_host": (C.c_int, [vp, vp, vp, vp, vp, vp]),
     "ssrh_set_tile_mask": (C.c_int, [vp, C.c_int, C.c_int]),
     "ssrh_forward_3dgs": (C.c_int, [C.c_char_p, C.c_int, C.c_int, C.c_int, C.c_int]),
     "ssrh_backward_from_render_grad": (C.c_int, [vp, vp, vp]),
@@ -119,6 +121,25 @@ class Engine:
 
     def backward(self):
         check(self.h.ssrh_backward_from_render_grad(self.d_vrgb.ptr, self.d_vdepth.ptr, self.d_vT.ptr))
+
+    HYPER = ["lr_means", "lr_quats", "lr_scales", "lr_opacs", "lr_features_dc", "lr_features_sh", "max_gauss_ratio",
+             "scale_regularization_weight", "mcmc_opacity_reg_weight", "mcmc_scale_reg_weight", "quat_norm_reg_weight",
+             "sh_reg_weight"]
+
+    def backward_fused_optimizer(self, hyper, step):
+        """Compositing backward, then the projection backward fused with the Adam step: the engine's
+        parameters and its Adam moments are updated in place (fp32 SH only)."""
+        hv = np.array([hyper.get(k, 0.0) for k in self.HYPER], np.float32)
+        check(self.h.ssrh_backward_fused_optimizer(self.d_vrgb.ptr, self.d_vdepth.ptr, self.d_vT.ptr, hv.ctypes.data, int(step)))
+
+    def params(self):
+        n = self.sc.n
+        g = dict(means=np.zeros((n, 3), np.float32), quats=np.zeros((n, 4), np.float32),
+                 log_scales=np.zeros((n, 3), np.float32), opacity_logits=np.zeros(n, np.float32),
+                 features_dc=np.zeros((n, 3), np.float32), features_sh=np.zeros((n, 15, 3), np.float32))
+        check(self.h.ssrh_copy_params_to_host(*[g[k].ctypes.data for k in
+                                                ["means", "quats", "log_scales", "opacity_logits", "features_dc", "features_sh"]]))
+        return g
 
     def time_iterations(self, iters):
         ms = np.zeros(iters, np.float32)

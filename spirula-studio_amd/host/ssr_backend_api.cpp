@@ -536,3 +536,54 @@ void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
     StageTimer t(&g_times.k9);
     ok(ssr_projection_bwd(&p, nullptr), "projection_3dgs_backward");
 }
+
+void fused_projection_bwd_optimizer_3dgs(
+    const int64_t num_splats, const int max_sh_degree, std::vector<DeviceTensorFloatND> splats_world,
+    TorchTensorView viewmats, TorchTensorView intrins, const uint32_t image_width, const uint32_t image_height,
+    const std::string camera_model, const std::string distortion, const TorchTensorView,
+    const DeviceVector<int32_t> camera_ids, const DeviceVector<int32_t> gaussian_ids, DeviceTensorFloatND aabb,
+    const std::vector<DeviceTensorFloatND> v_splats_world, const std::vector<DeviceTensorFloatND> v_splats_screen,
+    const std::vector<DeviceTensorFloatND> g1_splats_world, const std::vector<DeviceTensorFloatND> g2_splats_world,
+    const std::optional<TorchTensorView> sh_packed, const std::optional<TorchTensorView>,
+    const std::optional<TorchTensorView> sh_value_packed, const std::optional<TorchTensorView>, NonShQuantState non_sh,
+    DeviceVector<float>, DeviceVector<float> densify_score, const float lr_means, const float lr_quats,
+    const float lr_scales, const float lr_opacs, const float lr_features_dc, const float lr_features_sh,
+    const float max_gauss_ratio, const float scale_regularization_weight, const float mcmc_opacity_reg_weight,
+    const float mcmc_scale_reg_weight, const float erank_reg_weight, const float erank_reg_weight_s3,
+    const float quat_norm_reg_weight, const float sh_reg_weight, bool use_scale_agnostic_mean, bool color_trust_linear,
+    float, std::variant<int32_t, TorchTensorView> step, int quantization_level) {
+    const char* w = "fused_projection_bwd_optimizer_3dgs: ";
+    require_no_distortion(distortion);
+    if (camera_ids.data_ptr() || gaussian_ids.data_ptr()) throw std::runtime_error(std::string(w) + "packed mode is not built in this backend");
+    if (sh_packed || non_sh.enabled || quantization_level != 0) throw std::runtime_error(std::string(w) + "quantized Adam state is not built in this backend");
+    if (sh_value_packed) throw std::runtime_error(std::string(w) + "value-quantized SH is not built in this backend");
+    if (erank_reg_weight != 0.0f || erank_reg_weight_s3 != 0.0f) throw std::runtime_error(std::string(w) + "the effective-rank regularizer is not built in this backend");
+    if (use_scale_agnostic_mean) throw std::runtime_error(std::string(w) + "the scale-agnostic mean step is not built in this backend");
+    if (color_trust_linear) throw std::runtime_error(std::string(w) + "the colour trust region is not built in this backend");
+    if (num_splats == 0) return;
+    ssr_fpbo_params p;
+    std::memset(&p, 0, sizeof(p));
+    p.num_splats = num_splats;
+    p.sh_degree = max_sh_degree;
+    p.world = world_of(splats_world);
+    p.camera = camera_of(camera_model, viewmats, intrins, image_width, image_height);
+    p.aabb = aabb.data_ptr();
+    p.v_screen = screen_of(v_splats_screen);
+    if (!v_splats_world.empty()) p.v_world_in = world_of(v_splats_world);
+    p.v_world_in.features_sh = nullptr;   // not read (FusedProjectionBwdOptim_kernel.cuh:250-255)
+    p.g1 = world_of(g1_splats_world);
+    p.g2 = world_of(g2_splats_world);
+    p.densify_score = densify_score.data_ptr();
+    p.lr_means = lr_means; p.lr_quats = lr_quats; p.lr_scales = lr_scales; p.lr_opacs = lr_opacs;
+    p.lr_features_dc = lr_features_dc; p.lr_features_sh = lr_features_sh;
+    p.max_gauss_ratio = max_gauss_ratio; p.scale_regularization_weight = scale_regularization_weight;
+    p.mcmc_opacity_reg_weight = mcmc_opacity_reg_weight; p.mcmc_scale_reg_weight = mcmc_scale_reg_weight;
+    p.quat_norm_reg_weight = quat_norm_reg_weight; p.sh_reg_weight = sh_reg_weight;
+    if (const int32_t* s = std::get_if<int32_t>(&step)) {
+        p.step = *s;
+    } else {
+        p.steps = (const int32_t*)std::get<0>(std::get<TorchTensorView>(step));
+    }
+    StageTimer t(&g_times.k9);
+    ok(ssr_fused_projection_bwd_optimizer(&p, nullptr), "fused_projection_bwd_optimizer_3dgs");
+}

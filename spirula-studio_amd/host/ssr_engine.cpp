@@ -174,15 +174,12 @@ void forward_3dgs(std::string primitive, int sh_degree, bool packed, bool output
     E.fwd.renders = renders; E.fwd.render_Ts = Ts; E.fwd.last_ids = last;
 }
 
-void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
-                                      TorchTensorView v_render_Ts) {
+namespace {
+// stage the pixel cotangents and run the compositing backward; returns v_screen
+std::vector<DeviceTensorFloatND> raster_backward(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
+                                                 TorchTensorView v_render_Ts) {
     auto& E = engine();
-    if (std::get<0>(E.fwd.renders).data_ptr() == nullptr)
-        throw std::runtime_error("engine_backward_from_render_grad: forward_3dgs must be called first");
-    alloc_grad_buffers();
     const int64_t C = E.camera.num, H = E.camera.height, W = E.camera.width;
-    // stage the cotangents into pool buffers; Auto routes host and device sources alike
-    // (src/engine/EngineLoss.cpp:420-428). A device source is used in place.
     auto stage = [&](PoolSlot slot, const TorchTensorView& src, int ch) -> float* {
         void* s = (void*)std::get<0>(src);
         if (backend::is_device_pointer(s)) return (float*)s;
@@ -197,13 +194,24 @@ void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorV
     std::get<0>(v_renders) = DeviceTensor3D<float3>((float3*)v_rgb, C, H, W);
     std::get<1>(v_renders) = DeviceTensor3D<float>(v_depth, C, H, W);
     DeviceTensor3D<float> v_Ts_t(v_Ts, C, H, W);
-
-    // _engine_raster_proj_backward, non-fused branch (src/engine/EngineLoss.cpp:218-240,294-390)
     auto [vw, vs, accum] = rasterize_to_pixels_3dgs_bwd(
         E.cur_num_splats, E.fwd.splats_w, E.fwd.splats_s, E.fwd.gaussian_ids, (uint32_t)W, (uint32_t)H,
         E.fwd.tile_offsets, E.fwd.flatten_ids, E.fwd.render_Ts, E.fwd.last_ids, E.fwd.renders, std::nullopt,
         DistortionType::None, DeviceTensor3D<float>{}, DensifyAccumMode::None, v_renders, v_Ts_t, DeviceTensor3D<float>{},
         std::nullopt, std::nullopt, std::nullopt);
+    return vs;
+}
+}  // namespace
+
+void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
+                                      TorchTensorView v_render_Ts) {
+    auto& E = engine();
+    if (std::get<0>(E.fwd.renders).data_ptr() == nullptr)
+        throw std::runtime_error("engine_backward_from_render_grad: forward_3dgs must be called first");
+    alloc_grad_buffers();
+    const int64_t H = E.camera.height, W = E.camera.width;
+    // _engine_raster_proj_backward, non-fused branch (src/engine/EngineLoss.cpp:218-240,294-390)
+    auto vs = raster_backward(v_render_rgb, v_render_depth, v_render_Ts);
     E.grad.v_screen = vs;
     std::vector<DeviceTensorFloatND> v_world = {
         DeviceTensorFloatND(E.grad.means), DeviceTensorFloatND(E.grad.quats), DeviceTensorFloatND(E.grad.scales),
@@ -218,6 +226,57 @@ void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorV
     E.grad.dirty_key = (const void*)E.grad.means.data_ptr();
     // with no list the backward may have written any row; with one, exactly the listed rows
     E.grad.dirty_valid = E.grad.dirty_list != nullptr || (E.packed && E.fwd.gaussian_ids.size() == 0);
+}
+
+
+void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
+                                     TorchTensorView v_render_Ts, const float hyper[12], int step) {
+    auto& E = engine();
+    if (std::get<0>(E.fwd.renders).data_ptr() == nullptr)
+        throw std::runtime_error("engine_backward_fused_optimizer: forward_3dgs must be called first");
+    if (E.packed) throw std::runtime_error("engine_backward_fused_optimizer: packed projection is not built for the fused optimizer");
+    const int64_t n = E.max_num_splats;
+    if (!E.optim.adam_ready) {
+        const PoolSlot s1[6] = {PoolSlot::AdamG1Means, PoolSlot::AdamG1Quats, PoolSlot::AdamG1Scales, PoolSlot::AdamG1Opacities,
+                                PoolSlot::AdamG1FeaturesDc, PoolSlot::AdamG1FeaturesSh};
+        const PoolSlot s2[6] = {PoolSlot::AdamG2Means, PoolSlot::AdamG2Quats, PoolSlot::AdamG2Scales, PoolSlot::AdamG2Opacities,
+                                PoolSlot::AdamG2FeaturesDc, PoolSlot::AdamG2FeaturesSh};
+        const int64_t ch[6] = {3, 4, 3, 1, 3, 3 * (int64_t)E.num_sh};
+        E.optim.g1.clear(); E.optim.g2.clear();
+        for (int i = 0; i < 6; i++) {
+            float* a = DevicePool::global().acquire<float>(s1[i], (size_t)(n * ch[i]));
+            float* b = DevicePool::global().acquire<float>(s2[i], (size_t)(n * ch[i]));
+            backend::memset_async(a, 0, (size_t)(n * ch[i]) * sizeof(float));
+            backend::memset_async(b, 0, (size_t)(n * ch[i]) * sizeof(float));
+            E.optim.g1.emplace_back(a, std::vector<int64_t>{n, ch[i]});
+            E.optim.g2.emplace_back(b, std::vector<int64_t>{n, ch[i]});
+        }
+        E.optim.densify_score.resize(PoolSlot::EngDensifyScore, n);
+        E.optim.adam_ready = true;
+    }
+    E.grad.v_screen = raster_backward(v_render_rgb, v_render_depth, v_render_Ts);
+    const int64_t W = E.camera.width, H = E.camera.height;
+    fused_projection_bwd_optimizer_3dgs(
+        E.cur_num_splats, E.sh_degree, E.fwd.splats_w, E.camera.viewmats, E.camera.intrins, (uint32_t)W, (uint32_t)H,
+        E.camera.model_str, E.camera.distortion_str, E.camera.dist_coeffs, DeviceVector<int32_t>{}, DeviceVector<int32_t>{},
+        DeviceTensorFloatND((float*)E.fwd.aabb.data_ptr(), {E.fwd.aabb.numel(), 4}), {}, E.grad.v_screen, E.optim.g1, E.optim.g2,
+        std::nullopt, std::nullopt, E.world.sh_packed, E.world.sh_bounds, NonShQuantState{}, E.optim.radii,
+        E.optim.densify_score, hyper[0], hyper[1], hyper[2], hyper[3], hyper[4], hyper[5], hyper[6], hyper[7], hyper[8],
+        hyper[9], 0.0f, 0.0f, hyper[10], hyper[11], false, false, 0.0f, (int32_t)step, 0);
+}
+
+void engine_copy_params_to_host(TorchTensorView means, TorchTensorView quats, TorchTensorView scales,
+                                TorchTensorView opacities, TorchTensorView features_dc, TorchTensorView features_sh) {
+    auto& w = engine().world;
+    auto put = [](void* dst, const void* src, size_t bytes) {
+        if (dst && src && bytes) backend::memcpy_sync(dst, src, bytes, backend::MemcpyKind::DeviceToHost);
+    };
+    put((void*)std::get<0>(means), w.means.data_ptr(), w.means.size() * sizeof(float3));
+    put((void*)std::get<0>(quats), w.quats.data_ptr(), w.quats.size() * sizeof(float4));
+    put((void*)std::get<0>(scales), w.scales.data_ptr(), w.scales.size() * sizeof(float3));
+    put((void*)std::get<0>(opacities), w.opacities.data_ptr(), w.opacities.size() * sizeof(float));
+    put((void*)std::get<0>(features_dc), w.features_dc.data_ptr(), w.features_dc.size() * sizeof(float3));
+    put((void*)std::get<0>(features_sh), w.features_sh.data_ptr(), w.features_sh.numel() * sizeof(float3));
 }
 
 void engine_copy_render_to_host(TorchTensorView out_rgb, TorchTensorView out_depth, TorchTensorView out_Ts,
@@ -313,6 +372,21 @@ int ssrh_backward_from_render_grad(const float* v_rgb, const float* v_depth, con
     return guard([&] {
         const int64_t C = engine().camera.num, H = engine().camera.height, W = engine().camera.width;
         engine_backward_from_render_grad(tv(v_rgb, 4, {C, H, W, 3}), tv(v_depth, 4, {C, H, W, 1}), tv(v_Ts, 4, {C, H, W, 1}));
+    });
+}
+
+int ssrh_backward_fused_optimizer(const float* v_rgb, const float* v_depth, const float* v_Ts, const float* hyper12, int step) {
+    return guard([&] {
+        const int64_t C = engine().camera.num, H = engine().camera.height, W = engine().camera.width;
+        engine_backward_fused_optimizer(tv(v_rgb, 4, {C, H, W, 3}), tv(v_depth, 4, {C, H, W, 1}), tv(v_Ts, 4, {C, H, W, 1}), hyper12, step);
+    });
+}
+
+int ssrh_copy_params_to_host(float* means, float* quats, float* scales, float* opacities, float* dc, float* sh) {
+    return guard([&] {
+        const int64_t n = engine().max_num_splats;
+        engine_copy_params_to_host(tv(means, 4, {n, 3}), tv(quats, 4, {n, 4}), tv(scales, 4, {n, 3}), tv(opacities, 4, {n, 1}),
+                                   tv(dc, 4, {n, 3}), tv(sh, 4, {n, engine().num_sh, 3}));
     });
 }
 

@@ -32,7 +32,12 @@ struct EngineState {
         std::string model_str = "PINHOLE", distortion_str = "NONE";
         TorchTensorView viewmats, intrins, dist_coeffs;
     } camera;
-    struct { DeviceVector<float> radii; bool skip_grad_zero = false; } optim;
+    struct {
+        DeviceVector<float> radii; bool skip_grad_zero = false;
+        bool adam_ready = false;
+        std::vector<DeviceTensorFloatND> g1, g2;   // Adam moments, shaped like the world tensors
+        DeviceVector<float> densify_score;
+    } optim;
     struct {
         std::vector<DeviceTensorFloatND> splats_w, splats_s;
         DeviceTensor2D<float4> aabb; DeviceTensor2D<float> depths;
@@ -70,6 +75,15 @@ void engine_set_tile_mask(TorchTensorView mask);
 void forward_3dgs(std::string primitive, int sh_degree, bool packed, bool output_median, int dist_type_int);
 void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
                                       TorchTensorView v_render_Ts);
+// Backward with the projection backward folded into the optimizer step
+// (engine().optim.use_fused_proj_bwd_optim, src/engine/EngineLoss.cpp:286-290): compositing backward,
+// then fused_projection_bwd_optimizer_3dgs on the engine's parameters with Adam moments kept in pool
+// slots (zero on first use). hyper: lr_means, lr_quats, lr_scales, lr_opacs, lr_dc, lr_sh,
+// max_gauss_ratio, scale_reg_w, mcmc_opacity_w, mcmc_scale_w, quat_norm_w, sh_reg_w.
+void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
+                                     TorchTensorView v_render_Ts, const float hyper[12], int step);
+void engine_copy_params_to_host(TorchTensorView means, TorchTensorView quats, TorchTensorView scales,
+                                TorchTensorView opacities, TorchTensorView features_dc, TorchTensorView features_sh);
 void engine_copy_render_to_host(TorchTensorView out_rgb, TorchTensorView out_depth, TorchTensorView out_Ts,
                                 TorchTensorView out_rgb_raw, TorchTensorView out_median);
 void engine_copy_grads_to_host(TorchTensorView means, TorchTensorView quats, TorchTensorView scales,

@@ -13,6 +13,7 @@
 #include <stdexcept>
 #include <string>
 #include <tuple>
+#include <variant>
 #include <vector>
 
 // ---- vector PODs with the device layout (BackendTypes.h:34-49) ----
@@ -63,7 +64,9 @@ enum class PoolSlot : int {
     ProjAabb, ProjDepths, ProjScreenXy, ProjScreenDepth, ProjScreenConic, ProjScreenOpac, ProjScreenRgb,
     IsectTilesPerSplat, IsectCumTiles, IsectIdsA, IsectIdsB, IsectFlatA, IsectFlatB, IsectOffsets,
     IsectScanScratch, IsectSortScratch, IsectCounters, ProjVisibleIds, ProjVisibleIdsB, ProjPackedRows,
-    IsectTileActive, EngTileMask, ProjCameraIds, ProjGaussianIds, ProjGaussianIdsB, ProjPackedScratch, ProjPackedNnz,
+    IsectTileActive, EngTileMask,
+    AdamG1Means, AdamG1Quats, AdamG1Scales, AdamG1Opacities, AdamG1FeaturesDc, AdamG1FeaturesSh,
+    AdamG2Means, AdamG2Quats, AdamG2Scales, AdamG2Opacities, AdamG2FeaturesDc, AdamG2FeaturesSh, EngDensifyScore, ProjCameraIds, ProjGaussianIds, ProjGaussianIdsB, ProjPackedScratch, ProjPackedNnz,
     RendersRgb, RendersDepth, RenderTs, RenderLastIds,
     RasterBwdVScreenXy, RasterBwdVScreenDepth, RasterBwdVScreenConic, RasterBwdVScreenOpac, RasterBwdVScreenRgb,
     EngVRgb, EngVDepth, EngVTs,
@@ -174,6 +177,9 @@ public:
     int64_t rows() const { return shape_.empty() ? 0 : shape_[0]; }
     int64_t channels() const { return rows() ? numel() / rows() : 0; }
 };
+
+// src/core/NonShQuantState.h:16-28 (only `enabled` is consulted here: quantized Adam state is not built)
+struct NonShQuantState { bool enabled = false; };
 
 struct RenderOutput {
     // (rgb [I,H,W] float3, depth [I,H,W] float, normal -- unused by the 3dgs primitive)

@@ -76,6 +76,18 @@ class ProjectionPackedParams(C.Structure):
                 ("screen", Screen), ("tiles_per_splat", vp), ("packed_rows", vp)]
 
 
+class FpboParams(C.Structure):
+    _fields_ = [("num_splats", C.c_int64), ("sh_degree", C.c_int32), ("world", World), ("camera", Camera),
+                ("aabb", vp), ("v_screen", Screen), ("v_world_in", World), ("g1", World), ("g2", World),
+                ("densify_score", vp),
+                ("lr_means", C.c_float), ("lr_quats", C.c_float), ("lr_scales", C.c_float), ("lr_opacs", C.c_float),
+                ("lr_features_dc", C.c_float), ("lr_features_sh", C.c_float),
+                ("max_gauss_ratio", C.c_float), ("scale_regularization_weight", C.c_float),
+                ("mcmc_opacity_reg_weight", C.c_float), ("mcmc_scale_reg_weight", C.c_float),
+                ("quat_norm_reg_weight", C.c_float), ("sh_reg_weight", C.c_float),
+                ("step", C.c_int32), ("steps", vp)]
+
+
 # every symbol include/ssr_backend.h declares: (name, restype, argtypes)
 _i64, _u32, _i32, _sz = C.c_int64, C.c_uint32, C.c_int, C.c_size_t
 SYMBOLS = {
@@ -96,6 +108,7 @@ SYMBOLS = {
     "ssr_raster_fwd": (_i32, [C.POINTER(RasterFwdParams), vp]),
     "ssr_raster_bwd": (_i32, [C.POINTER(RasterBwdParams), vp]),
     "ssr_projection_bwd": (_i32, [C.POINTER(ProjectionBwdParams), vp]),
+    "ssr_fused_projection_bwd_optimizer": (_i32, [C.POINTER(FpboParams), vp]),
     "ssr_zero_world_rows": (_i32, [C.POINTER(World), vp, _i64, vp, vp]),
     "ssr_fill_u32": (_i32, [vp, _u32, _i64, vp]),
     "ssr_init": (_i32, [_i32]),

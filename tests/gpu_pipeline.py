@@ -262,6 +262,34 @@ class GpuRun:
             p.packed_gaussian_ids, p.num_packed = self.ptr("gaussian_ids"), self.rows
         self.check(self.lib.ssr_projection_bwd(C.byref(p), None))
 
+    def fused_optimizer(self, g1, g2, hyper, step=1, steps=None, v_in=None):
+        """ssr_fused_projection_bwd_optimizer on the device copies of the parameters (fp32 SH);
+        g1 / g2 are host dicts keyed like the world arrays. Returns (params, g1, g2, score) from the device."""
+        D = self.L.DeviceArray
+        keys = ["means", "quats", "log_scales", "opacity_logits", "features_dc", "features_sh"]
+        for pre, src in (("m1_", g1), ("m2_", g2)):
+            for k in keys:
+                self.d[pre + k] = D.from_host(np.ascontiguousarray(src[k], np.float32))
+        for k in keys:
+            a = None if v_in is None else v_in.get(k)
+            self.d["vi_" + k] = None if a is None else D.from_host(np.ascontiguousarray(a, np.float32))
+        self.d["score"] = D((self.n,), np.float32)
+        p = self.L.FpboParams()
+        p.num_splats, p.sh_degree = self.n, self.sh_degree
+        p.world, p.camera, p.aabb = self.world(), self.camera(), self.ptr("aabb")
+        p.v_screen, p.v_world_in, p.g1, p.g2 = self.screen("v_"), self.world("vi_"), self.world("m1_"), self.world("m2_")
+        p.densify_score = self.ptr("score")
+        for k, v in hyper.items():
+            setattr(p, k, v)
+        p.step = step
+        if steps is not None:
+            self.d["steps"] = D.from_host(np.ascontiguousarray(steps, np.int32))
+            p.steps = self.ptr("steps")
+        self.check(self.lib.ssr_fused_projection_bwd_optimizer(C.byref(p), None))
+        self.check(self.lib.ssr_device_synchronize())
+        out = lambda pre: {k: self.host(pre + k) for k in keys}
+        return out(""), out("m1_"), out("m2_"), self.host("score")
+
     def run_all(self, backward=True, fused_count=False):
         self.projection_fwd(fused_count)
         self.tiles(fused_count)

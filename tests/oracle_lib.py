@@ -206,6 +206,39 @@ def projection_bwd(scene, aabb, vs, sh_degree=3):
     return g
 
 
+HYPER = ["lr_means", "lr_quats", "lr_scales", "lr_opacs", "lr_features_dc", "lr_features_sh", "max_gauss_ratio",
+         "scale_regularization_weight", "mcmc_opacity_reg_weight", "mcmc_scale_reg_weight", "quat_norm_reg_weight",
+         "sh_reg_weight"]
+WORLD_KEYS = ["means", "quats", "log_scales", "opacity_logits", "features_dc", "features_sh"]
+
+
+def fused_projection_bwd_optimizer(scene, aabb, vs, params, g1, g2, hyper, step=1, steps=None, v_in=None,
+                                   sh_degree=3, densify=True):
+    """Updates params / g1 / g2 (dicts of float32 arrays keyed by WORLD_KEYS, fp32 SH [N,15,3]) in place
+    and returns the densification score."""
+    n = scene.n
+    cam = camera_of(scene)
+    PF = C.POINTER(C.c_float)
+
+    def ptrs(d):
+        arr = (C.c_void_p * 6)()
+        for i, k in enumerate(WORLD_KEYS):
+            a = None if d is None else d.get(k)
+            arr[i] = None if a is None else a.ctypes.data
+        return arr
+    hv = np.array([hyper.get(k, 0.0) for k in HYPER], np.float32)
+    score = np.zeros(n, np.float32) if densify else None
+    for d in (params, g1, g2):
+        for k in WORLD_KEYS:
+            assert d[k].dtype == np.float32 and d[k].flags.c_contiguous
+    lib().or_fused_projection_bwd_optimizer(
+        C.c_int64(n), C.c_int(sh_degree), *[_p(params[k]) for k in WORLD_KEYS], C.byref(cam), _p(aabb),
+        _p(vs["v_xy"]), _p(vs["v_depth"]), _p(vs["v_conic"]), _p(vs["v_opac"]), _p(vs["v_rgb"]),
+        ptrs(v_in) if v_in is not None else None, ptrs(g1), ptrs(g2), _p(score), _p(hv), C.c_int32(step),
+        _p(None if steps is None else np.ascontiguousarray(steps, np.int32)))
+    return score
+
+
 def pipeline(scene, sh_degree=3, backward=True, tile_active=None):
     """The whole iteration in the reference's order (src/engine/EngineForward.cpp:166-293,
     src/engine/EngineLoss.cpp:138-240,359-368). tile_active: optional tile-skip map for the tile stage."""

@@ -201,6 +201,47 @@ def test_engine_tile_mask_is_one_shot(pkg, oracle, H):
             _check(eng, oracle.pipeline(sc), sc)
 
 
+def test_engine_fused_optimizer_training_steps(pkg, oracle, H):
+    """Three training steps with the projection backward folded into Adam, against the oracle running
+    the same loop (forward, compositing backward, fused optimizer) on its own copy of the parameters."""
+    import copy
+    host, lib = H
+    sc = pkg.scenes.make_scene(1, n=20000, width=320, height=240, parity_variant=True)
+    ref_sc = copy.deepcopy(sc)
+    h = dict(lr_means=1.6e-4, lr_quats=1e-3, lr_scales=5e-3, lr_opacs=5e-2, lr_features_dc=2.5e-3,
+             lr_features_sh=1.25e-4, max_gauss_ratio=6.0, scale_regularization_weight=0.01,
+             mcmc_opacity_reg_weight=0.01, mcmc_scale_reg_weight=0.01, quat_norm_reg_weight=0.02, sh_reg_weight=0.05)
+    lrs = dict(means="lr_means", quats="lr_quats", log_scales="lr_scales", opacity_logits="lr_opacs",
+               features_dc="lr_features_dc", features_sh="lr_features_sh")
+    eng = host.Engine(sc)
+    P = {k: np.ascontiguousarray(getattr(ref_sc, k), np.float32).copy() for k in oracle.WORLD_KEYS}
+    g1 = {k: np.zeros_like(v) for k, v in P.items()}
+    g2 = {k: np.zeros_like(v) for k, v in P.items()}
+    for step in (1, 2, 3):
+        eng.forward()
+        eng.backward_fused_optimizer(h, step)
+        for k in oracle.WORLD_KEYS:
+            setattr(ref_sc, k, P[k])
+        r = oracle.pipeline(ref_sc, backward=True)
+        oracle.fused_projection_bwd_optimizer(ref_sc, r["proj"]["aabb"], r["vscreen"], P, g1, g2, h, step=step)
+        got = eng.params()
+        for k in oracle.WORLD_KEYS:
+            d = np.abs(got[k].astype(np.float64) - P[k])
+            lr = h[lrs[k]]
+            # first steps move every parameter by about lr * sign(gradient): a gradient that rounds to the
+            # other side of zero moves it the other way, so a few elements may differ by a step or two
+            far = d > 0.05 * lr + 1e-6
+            assert far.mean() < 2e-3, (step, k, float(far.mean()))
+            assert d.max() <= 2.5 * step * lr + 1e-6, (step, k, float(d.max()))
+    # the render of the updated model still matches
+    eng.forward()
+    for k in oracle.WORLD_KEYS:
+        setattr(ref_sc, k, P[k])
+    r = oracle.pipeline(ref_sc, backward=False)
+    rgb, depth, T = eng.render()
+    assert np.abs(rgb - r["fwd"]["rgb"]).max() < 0.02
+
+
 def test_unsupported_variants_raise(pkg, H):
     host, lib = H
     sc = pkg.scenes.tiny_scene(n=50, width=32, height=32)

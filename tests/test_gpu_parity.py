@@ -275,3 +275,45 @@ def test_tile_skip_mask(gpu, oracle):
     mask = (rng.random((400, 640)) < 0.0005).astype(np.uint8)
     g, r = _compare(gpu, oracle, sc, "mask-huge", fused_count=True, use_list=True, mask=mask)
     assert r["counts"].max() > 96
+
+
+@pytest.mark.parametrize("cfg", ["tiny", "cfg2", "equirect-steps"])
+def test_fused_projection_bwd_optimizer(gpu, oracle, cfg):
+    """K9 fused with Adam (fused_projection_bwd_optimizer_3dgs, fp32 state): both sides are fed the
+    SAME screen gradients (the device's), so only the arithmetic of the fused kernel is compared."""
+    rng = np.random.default_rng(11)
+    if cfg == "tiny":
+        sc = gpu.scenes.tiny_scene(n=900, width=96, height=64, seed=61)
+        sc.means[::4, 2] = -10.0
+        sc.log_scales[5] = [-2.0, -4.5, -3.0]
+        sc.features_dc[7] = [2.5, -2.2, 0.1]
+        sc.quats *= np.linspace(0.5, 2.0, sc.n)[:, None].astype(np.float32)
+    elif cfg == "cfg2":
+        sc = gpu.scenes.make_scene(2, n=40000, width=480, height=270, parity_variant=True)
+    else:
+        sc = gpu.scenes.make_scene(5, n=30000, width=512, height=256)
+    g = GpuRun(gpu, sc)
+    g.projection_fwd(); g.tiles(); g.raster_fwd(); g.raster_bwd()
+    vs = {k: g.host(k) for k in ["v_xy", "v_depth", "v_conic", "v_opac", "v_rgb"]}
+    aabb = g.host("aabb")
+    P = {k: np.ascontiguousarray(getattr(sc, k), np.float32).copy() for k in oracle.WORLD_KEYS}
+    g1 = {k: rng.normal(0, 1e-3, P[k].shape).astype(np.float32) for k in oracle.WORLD_KEYS}
+    g2 = {k: rng.uniform(1e-7, 1e-5, P[k].shape).astype(np.float32) for k in oracle.WORLD_KEYS}
+    v_in = {"means": rng.normal(0, 1e-3, (sc.n, 3)).astype(np.float32)}
+    h = dict(lr_means=1.6e-4, lr_quats=1e-3, lr_scales=5e-3, lr_opacs=5e-2, lr_features_dc=2.5e-3,
+             lr_features_sh=1.25e-4, max_gauss_ratio=6.0, scale_regularization_weight=0.01,
+             mcmc_opacity_reg_weight=0.01, mcmc_scale_reg_weight=0.01, quat_norm_reg_weight=0.02, sh_reg_weight=0.05)
+    steps = rng.integers(1, 400, sc.n).astype(np.int32) if cfg == "equirect-steps" else None
+    dP, d1, d2, dscore = g.fused_optimizer(g1, g2, h, step=37, steps=steps, v_in=v_in)
+    score = oracle.fused_projection_bwd_optimizer(sc, aabb, vs, P, g1, g2, h, step=37, steps=steps, v_in=v_in)
+    lrs = dict(means="lr_means", quats="lr_quats", log_scales="lr_scales", opacity_logits="lr_opacs",
+               features_dc="lr_features_dc", features_sh="lr_features_sh")
+    for k in oracle.WORLD_KEYS:
+        # moments: relative to the row's gradient scale; parameters: a fraction of one learning-rate step
+        a, b = d1[k].reshape(sc.n, -1).astype(np.float64), g1[k].reshape(sc.n, -1).astype(np.float64)
+        assert (np.abs(a - b) <= 1e-3 * np.abs(b) + 1e-4 * (np.abs(b).max(axis=1, keepdims=True) + 1e-12)).all(), ("g1", k)
+        a, b = d2[k].reshape(sc.n, -1).astype(np.float64), g2[k].reshape(sc.n, -1).astype(np.float64)
+        assert (np.abs(a - b) <= 2e-3 * np.abs(b) + 1e-12).all(), ("g2", k)
+        a, b = dP[k].astype(np.float64), P[k].astype(np.float64)
+        assert np.abs(a - b).max() <= 0.02 * h[lrs[k]] * 40 + 1e-6, (k, float(np.abs(a - b).max()))
+    assert np.allclose(dscore, score, rtol=1e-3, atol=1e-9)

@@ -1,0 +1,112 @@
+"""Projection backward fused with Adam (oracle restatement of the fp32-state branch of
+src/kernels/optim/FusedProjectionBwdOptim_kernel.cuh:232-710), pinned against a float64 numpy Adam fed
+the (separately pinned) projection gradient, with the regularizer gradients taken by central finite
+differences of the loss definitions of src/shaders/per_splat_losses.slang:30-81."""
+import numpy as np
+import pytest
+
+B1, B2, EPS = 0.9, 0.999, 1e-15
+KSH0 = 0.28209479177387814
+
+
+def _losses64(ls, logit, quat, dc, sh, h, n_coef):
+    """Sum of the per-splat regularizers with v_loss = 1, in float64."""
+    e = np.exp(ls)
+    ratio = e.max() / e.min()
+    loss = h["mcmc_opacity_reg_weight"] / (1 + np.exp(-logit))
+    loss += h["mcmc_scale_reg_weight"] * 1e-2 * ls.sum() / 3.0
+    loss += h["scale_regularization_weight"] * (max(ratio, h["max_gauss_ratio"]) - h["max_gauss_ratio"])
+    qn = np.linalg.norm(quat)
+    loss += h["quat_norm_reg_weight"] * (qn - 1 - np.log(qn))
+    # dc / sh magnitude: the kernel adds w (relu(dc - lim) + min(dc + lim, 0)) and (w / n_coef) sh to the gradients,
+    # i.e. the losses w/2 (relu(|dc| - lim))^2 and w / (2 n_coef) |sh|^2
+    lim = 0.5 / KSH0
+    loss += 0.5 * h["sh_reg_weight"] * (np.maximum(np.abs(dc) - lim, 0) ** 2).sum()
+    loss += 0.5 * h["sh_reg_weight"] / max(n_coef, 1) * (sh ** 2).sum()
+    return loss
+
+
+def _fd(f, x, eps=1e-6):
+    g = np.zeros_like(x)
+    for i in range(x.size):
+        d = np.zeros_like(x)
+        d.flat[i] = eps
+        g.flat[i] = (f(x + d) - f(x - d)) / (2 * eps)
+    return g
+
+
+@pytest.mark.parametrize("per_splat_steps", [False, True])
+def test_fused_optimizer_against_float64_adam(pkg, oracle, per_splat_steps):
+    sc = pkg.scenes.tiny_scene(n=120, width=96, height=64, seed=51)
+    sc.means[::4, 2] = -10.0                     # culled splats still decay their moments
+    sc.log_scales[5] = [-2.0, -4.5, -3.0]        # ratio e^2.5 > max_gauss_ratio
+    sc.features_dc[7] = [2.5, -2.2, 0.1]         # beyond +-0.5/kSh0
+    sc.quats *= np.linspace(0.5, 2.0, sc.n)[:, None].astype(np.float32)   # non-unit quaternions
+    r = oracle.pipeline(sc)
+    rng = np.random.default_rng(2)
+    P = {k: np.ascontiguousarray(getattr(sc, k), np.float32).copy() for k in oracle.WORLD_KEYS}
+    g1 = {k: (rng.normal(0, 1e-3, P[k].shape)).astype(np.float32) for k in oracle.WORLD_KEYS}
+    g2 = {k: (rng.uniform(1e-7, 1e-5, P[k].shape)).astype(np.float32) for k in oracle.WORLD_KEYS}
+    v_in = {"means": rng.normal(0, 1e-3, (sc.n, 3)).astype(np.float32), "opacity_logits": None}
+    h = dict(lr_means=1.6e-4, lr_quats=1e-3, lr_scales=5e-3, lr_opacs=5e-2, lr_features_dc=2.5e-3,
+             lr_features_sh=1.25e-4, max_gauss_ratio=6.0, scale_regularization_weight=0.01,
+             mcmc_opacity_reg_weight=0.01, mcmc_scale_reg_weight=0.01, quat_norm_reg_weight=0.02, sh_reg_weight=0.05)
+    steps = rng.integers(1, 400, sc.n).astype(np.int32) if per_splat_steps else None
+    step = 37
+    P0 = {k: v.astype(np.float64) for k, v in P.items()}
+    G1 = {k: v.astype(np.float64) for k, v in g1.items()}
+    G2 = {k: v.astype(np.float64) for k, v in g2.items()}
+    score = oracle.fused_projection_bwd_optimizer(sc, r["proj"]["aabb"], r["vscreen"], P, g1, g2, h, step=step,
+                                                  steps=steps, v_in=v_in)
+    # ---- float64 expectation ----
+    gr = r["grads"]
+    data = dict(means=gr["v_means"] + v_in["means"], quats=gr["v_quats"], log_scales=gr["v_scales"],
+                opacity_logits=gr["v_opacities"], features_dc=gr["v_dc"], features_sh=gr["v_sh"])
+    data = {k: v.astype(np.float64) for k, v in data.items()}
+    t = (steps if per_splat_steps else np.full(sc.n, step)).astype(np.float64)
+    c1, c2 = 1 / (1 - B1 ** t), 1 / (1 - B2 ** t)
+    exp_score = np.exp(P0["log_scales"].max(axis=1)) * np.linalg.norm(data["means"], axis=1)
+    assert np.allclose(score, exp_score, rtol=1e-5, atol=1e-12)
+    for g in range(sc.n):
+        ls, lo, q, dc, sh = (P0["log_scales"][g], P0["opacity_logits"][g], P0["quats"][g], P0["features_dc"][g],
+                             P0["features_sh"][g])
+        reg = dict(
+            log_scales=_fd(lambda x: _losses64(x, lo, q, dc, sh, h, 15), ls),
+            opacity_logits=_fd(lambda x: _losses64(ls, x[0], q, dc, sh, h, 15), np.array([lo]))[0],
+            quats=_fd(lambda x: _losses64(ls, lo, x, dc, sh, h, 15), q),
+            features_dc=_fd(lambda x: _losses64(ls, lo, q, x, sh, h, 15), dc),
+            features_sh=_fd(lambda x: _losses64(ls, lo, q, dc, x, h, 15), sh), means=0.0)
+        for k in oracle.WORLD_KEYS:
+            v = data[k][g] + reg[k]
+            x = P0[k][g]
+            if k == "quats":
+                x = x / np.linalg.norm(x)
+                v = v - np.dot(x, v) * x
+            m1 = B1 * G1[k][g] + (1 - B1) * v
+            m2 = B2 * G2[k][g] + (1 - B2) * v * v
+            lr = h["lr_" + {"log_scales": "scales", "opacity_logits": "opacs"}.get(k, k)]
+            new = x - lr * c1[g] * m1 / (np.sqrt(m2 * c2[g]) + EPS)
+            if k == "quats":
+                new = new / np.linalg.norm(new)
+            scale = np.abs(v).max() + 1e-12
+            assert np.allclose(g1[k][g], m1, rtol=2e-5, atol=2e-6 * scale), (k, g)
+            assert np.allclose(g2[k][g], m2, rtol=5e-5, atol=1e-12), (k, g)
+            assert np.allclose(P[k][g], new, rtol=1e-5, atol=2e-5 * lr * 50 + 1e-7), (k, g, P[k][g], new)
+
+
+def test_zero_learning_rates_and_weights_leave_parameters_alone(pkg, oracle):
+    sc = pkg.scenes.tiny_scene(n=60, width=64, height=48, seed=52)
+    r = oracle.pipeline(sc)
+    P = {k: np.ascontiguousarray(getattr(sc, k), np.float32).copy() for k in oracle.WORLD_KEYS}
+    keep = {k: v.copy() for k, v in P.items()}
+    g1 = {k: np.zeros_like(v) for k, v in P.items()}
+    g2 = {k: np.zeros_like(v) for k, v in P.items()}
+    oracle.fused_projection_bwd_optimizer(sc, r["proj"]["aabb"], r["vscreen"], P, g1, g2, {}, step=1)
+    for k in P:
+        if k == "quats":   # re-normalised
+            assert np.allclose(P[k], keep[k] / np.linalg.norm(keep[k], axis=1, keepdims=True), atol=1e-6)
+        else:
+            assert np.array_equal(P[k], keep[k]), k
+    # moments took the gradient: g1 = 0.1 v
+    assert np.allclose(g1["means"], 0.1 * r["grads"]["v_means"], rtol=1e-5, atol=1e-12)
+    assert np.allclose(g2["features_sh"], 0.001 * r["grads"]["v_sh"] ** 2, rtol=1e-4, atol=1e-20)
