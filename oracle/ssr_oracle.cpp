@@ -765,7 +765,23 @@ void or_raster_fwd(int64_t N, const float* xy, const float* depth, const float* 
     const float* opac, const float* rgb, uint32_t width, uint32_t height,
     const int32_t* tile_offsets, const int32_t* flatten_ids, int64_t n_isects,
     float* out_rgb, float* out_depth, float* out_T, int32_t* out_last_ids, int64_t* stats) {
+    or_raster_fwd_ex(N, xy, depth, conic, opac, rgb, width, height, tile_offsets, flatten_ids, n_isects, out_rgb, out_depth,
+                     out_T, out_last_ids, stats, 0, nullptr, nullptr, nullptr);
+}
+
+// The same kernel with its variants (RasterizationEval3DFwd_kernel.cuh:143-148,245-307):
+// dist_type 1 (D) / 2 (RGB_D): the depth channel is accumulated as ln(max(z, 1e-6)), second moments
+// S = sum w c^2 are accumulated next to C = sum w c, the distortion image D = W S - C^2 (W = 1 - T)
+// is written for the active channels and the rendered depth becomes exp(C_lnz / W).
+// out_median (non-NULL): depth at which the post-splat transmittance crosses 1/2, interpolated
+// linearly in ln T between the two bracketing splats (0 when it never does).
+void or_raster_fwd_ex(int64_t N, const float* xy, const float* depth, const float* conic,
+    const float* opac, const float* rgb, uint32_t width, uint32_t height,
+    const int32_t* tile_offsets, const int32_t* flatten_ids, int64_t n_isects,
+    float* out_rgb, float* out_depth, float* out_T, int32_t* out_last_ids, int64_t* stats,
+    int dist_type, float* out_dist_rgb, float* out_dist_depth, float* out_median) {
     (void)N;
+    const bool dist = dist_type != 0, dist_rgb = dist_type == 2;
     const int tw = (int)((width + kTile - 1) / kTile), th = (int)((height + kTile - 1) / kTile);
     const int n_tiles = tw * th;
     int64_t kf = 0, kb = 0, vis_f = 0, vis_b = 0, prod_b = 0;
@@ -798,6 +814,8 @@ void or_raster_fwd(int64_t N, const float* xy, const float* depth, const float* 
                 const int mt = (py_ / kMicro) * 2 + (px_ / kMicro);
                 const float px = (float)j + 0.5f, py = (float)i + 0.5f;
                 float T = 1.0f, cr = 0, cg = 0, cb = 0, cd = 0;
+                float s2r = 0, s2g = 0, s2b = 0, s2d = 0;
+                float median = 0.0f, med_prev_z = 0.0f, med_prev_T = 1.0f;
                 uint32_t cur_idx = 0;
                 int32_t last_eval = start - 1;
                 for (int32_t k = start; k < end; k++) {
@@ -808,10 +826,26 @@ void or_raster_fwd(int64_t N, const float* xy, const float* depth, const float* 
                     last_eval = k;
                     if (alpha <= kAlphaThreshold) continue;
                     const float next_T = T * (1.0f - alpha);
+                    if (out_median) {   // before the 1e-4 early-out, RasterizationEval3DFwd_kernel.cuh:245-259
+                        if (med_prev_T >= 0.5f && next_T < 0.5f) {
+                            const float a = ssr_log(med_prev_T), b = ssr_log(next_T), d = b - a;
+                            const float fr = (ssr_fabs(d) > 1e-20f) ? (-0.6931471805599453f - a) / d : 0.0f;
+                            median = med_prev_z + (f.d - med_prev_z) * fr;
+                        }
+                        med_prev_T = next_T;
+                        med_prev_z = f.d;
+                    }
                     if (next_T > 1e-4f) {
                         const float w = alpha * T;
+                        const float zd = dist ? ssr_log(ssr_max(f.d, 1e-6f)) : f.d;
+                        if (dist) {
+                            if (dist_rgb) {
+                                s2r = ssr_fma(f.r * f.r, w, s2r); s2g = ssr_fma(f.g * f.g, w, s2g); s2b = ssr_fma(f.b * f.b, w, s2b);
+                            }
+                            s2d = ssr_fma(zd * zd, w, s2d);
+                        }
                         cr = ssr_fma(f.r, w, cr); cg = ssr_fma(f.g, w, cg); cb = ssr_fma(f.b, w, cb);
-                        cd = ssr_fma(f.d, w, cd);
+                        cd = ssr_fma(zd, w, cd);
                         cur_idx = (uint32_t)k;
                         T = next_T;
                         used[k - start] |= (uint8_t)(1u << mt);
@@ -824,7 +858,19 @@ void or_raster_fwd(int64_t N, const float* xy, const float* depth, const float* 
                 out_T[pid] = T;
                 const float invW = 1.0f / ssr_max(1.0f - T, 1e-10f);
                 out_rgb[3 * pid] = cr; out_rgb[3 * pid + 1] = cg; out_rgb[3 * pid + 2] = cb;
-                out_depth[pid] = cd * invW;
+                if (out_median) out_median[pid] = median;
+                if (dist) {   // D = W S - C^2 on the raw accumulators, :291-295
+                    const float W = 1.0f - T;
+                    if (dist_rgb) {
+                        out_dist_rgb[3 * pid] = s2r * W - cr * cr;
+                        out_dist_rgb[3 * pid + 1] = s2g * W - cg * cg;
+                        out_dist_rgb[3 * pid + 2] = s2b * W - cb * cb;
+                    }
+                    out_dist_depth[pid] = s2d * W - cd * cd;
+                    out_depth[pid] = ssr_exp(cd * invW);
+                } else {
+                    out_depth[pid] = cd * invW;
+                }
                 out_last_ids[pid] = (int32_t)cur_idx;
                 max_eval = std::max(max_eval, last_eval);
                 max_last = std::max(max_last, (int32_t)cur_idx);
@@ -859,7 +905,26 @@ void or_raster_bwd(int64_t N, const float* xy, const float* depth, const float* 
     const float* render_T, const int32_t* last_ids, const float* render_depth,
     const float* v_rgb, const float* v_depth, const float* v_T,
     float* v_xy, float* v_sdepth, float* v_conic, float* v_opac, float* v_srgb, double* abs_terms) {
-    (void)N;
+    or_raster_bwd_ex(N, xy, depth, conic, opac, rgb, width, height, tile_offsets, flatten_ids, n_isects, render_T, last_ids,
+                     render_depth, v_rgb, v_depth, v_T, v_xy, v_sdepth, v_conic, v_opac, v_srgb, abs_terms,
+                     0, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, nullptr, nullptr, 0, nullptr);
+}
+
+// The same kernel with its variants (RasterizationEval3DBwd_kernel.cuh:150-172,207-257,268-279,433-550,574-585):
+// depth distortion / median / per-splat accumulation of a pixel weight map. gaussian_ids (packed
+// mode, may be NULL) maps a screen row to the world row that accum_weight is indexed by; with
+// accum_mode 3 (Avg) accum_weight holds n_world numerators followed by n_world denominators.
+void or_raster_bwd_ex(int64_t N, const float* xy, const float* depth, const float* conic,
+    const float* opac, const float* rgb, uint32_t width, uint32_t height,
+    const int32_t* tile_offsets, const int32_t* flatten_ids, int64_t n_isects,
+    const float* render_T, const int32_t* last_ids, const float* render_depth,
+    const float* v_rgb, const float* v_depth, const float* v_T,
+    float* v_xy, float* v_sdepth, float* v_conic, float* v_opac, float* v_srgb, double* abs_terms,
+    int dist_type, const float* render_rgb, const float* dist_rgb_img, const float* dist_depth_img,
+    const float* v_dist_rgb, const float* v_dist_depth, const float* v_median,
+    int accum_mode, const float* accum_map, const int32_t* gaussian_ids, int64_t n_world, float* accum_weight) {
+    const bool dist = dist_type != 0, dist_rgb = dist_type == 2;
+    std::vector<float> awpart(accum_mode ? (size_t)n_isects * 2 : 0, 0.0f);
     const int tw = (int)((width + kTile - 1) / kTile), th = (int)((height + kTile - 1) / kTile);
     const int n_tiles = tw * th;
     std::vector<float> part((size_t)n_isects * 10, 0.0f);
@@ -875,6 +940,8 @@ void or_raster_bwd(int64_t N, const float* xy, const float* depth, const float* 
             // per-pixel state, RasterizationEval3DBwd_kernel.cuh:186-232
             float T1[64], vT1[64], vc[64][4];
             int32_t bin_final[64];
+            float Cc[64][4], Sc[64][4], vD[64][4], Wd[64], amap[64];
+            float med_v[64], pend_zgrad[64], pend_zfar[64], pend_Tfar[64];
             for (int p = 0; p < 64; p++) {
                 const int pxi = bx + p % kMicro, pyi = by + p / kMicro;
                 const bool inside = pxi < (int)width && pyi < (int)height;
@@ -886,10 +953,33 @@ void or_raster_bwd(int64_t N, const float* xy, const float* depth, const float* 
                       vb = inside ? v_rgb[3 * pid + 2] : 0.f, vd = inside ? v_depth[pid] : 0.f;
                 float inv_alpha = 1.0f / ssr_max(1.0f - Tf, 1e-10f);
                 float exp_depth = inside ? render_depth[pid] : 0.0f;
-                vT = vT + (exp_depth * vd) * inv_alpha;
-                vd = vd * inv_alpha;
+                if (dist) {   // log-depth render: depth = exp(C_lnz / W), RasterizationEval3DBwd_kernel.cuh:212-218
+                    const float m = ssr_log(ssr_max(exp_depth, 1e-6f));
+                    vT = vT + ((exp_depth * vd) * m) * inv_alpha;
+                    vd = vd * (exp_depth * inv_alpha);
+                } else {
+                    vT = vT + (exp_depth * vd) * inv_alpha;
+                    vd = vd * inv_alpha;
+                }
                 T1[p] = Tf; vT1[p] = vT;
                 vc[p][0] = vr; vc[p][1] = vg; vc[p][2] = vb; vc[p][3] = vd;
+                if (dist) {   // :228-257
+                    for (int q = 0; q < 3; q++) Cc[p][q] = (inside && dist_rgb) ? render_rgb[3 * pid + q] : 0.0f;
+                    Cc[p][3] = ssr_log(ssr_max(exp_depth, 1e-6f)) * ssr_max(1.0f - Tf, 1e-10f);
+                    const float W = inside ? (1.0f - Tf) : 0.0f;
+                    const float invW = W > 1e-10f ? (1.0f / W) : 0.0f;
+                    float Dv[4] = {0, 0, 0, 0};
+                    for (int q = 0; q < 4; q++) vD[p][q] = 0.0f;
+                    if (inside) {
+                        if (dist_rgb) for (int q = 0; q < 3; q++) { Dv[q] = dist_rgb_img[3 * pid + q]; vD[p][q] = v_dist_rgb[3 * pid + q]; }
+                        Dv[3] = dist_depth_img[pid]; vD[p][3] = v_dist_depth[pid];
+                    }
+                    for (int q = 0; q < 4; q++) Sc[p][q] = (Dv[q] + Cc[p][q] * Cc[p][q]) * invW;
+                    Wd[p] = W;
+                }
+                amap[p] = (accum_mode && accum_map && inside) ? accum_map[pid] : 0.0f;
+                med_v[p] = (v_median && inside) ? v_median[pid] : 0.0f;
+                pend_zgrad[p] = pend_zfar[p] = pend_Tfar[p] = 0.0f;
             }
             for (int32_t k = end - 1; k >= start; k--) {
                 const int32_t g = flatten_ids[k];
@@ -898,6 +988,7 @@ void or_raster_bwd(int64_t N, const float* xy, const float* depth, const float* 
                 float acc[10] = {0};   // xy(2) depth conic(3) opac rgb(3)
                 double aacc[10] = {0};
                 bool any = false;
+                float aw = 0.0f, aw_den = 0.0f;
                 for (int p = 0; p < 64; p++) {
                     if (k > bin_final[p]) continue;
                     const float px = (float)(bx + p % kMicro) + 0.5f, py = (float)(by + p / kMicro) + 0.5f;
@@ -908,10 +999,46 @@ void or_raster_bwd(int64_t N, const float* xy, const float* depth, const float* 
                     const float ra = 1.0f / (1.0f - alpha);
                     const float T0 = T1[p] * ra;
                     const float* c = vc[p];
-                    const float dotcv = ssr_fma(f.d, c[3], ssr_fma(f.b, c[2], ssr_fma(f.g, c[1], f.r * c[0])));
-                    const float v_alpha = T0 * dotcv - vT1[p] * T0;
+                    float vT1p = vT1[p];
+                    float v_depth_median = 0.0f;
+                    if (v_median) {   // :433-470
+                        const float vm = med_v[p];
+                        if (pend_Tfar[p] > 0.0f) {   // this splat is the near member of the crossing found one step ago
+                            v_depth_median += pend_zgrad[p];
+                            const float a_ln = ssr_log(T1[p]), b_ln = ssr_log(pend_Tfar[p]);
+                            const float dba = b_ln - a_ln;
+                            const float inv = (ssr_fabs(dba) > 1e-20f) ? (-1.0f / dba) : 0.0f;
+                            const float Sg = (vm * (pend_zfar[p] - f.d)) * inv;
+                            vT1p += Sg / T1[p];
+                            pend_Tfar[p] = 0.0f;
+                        }
+                        if (T0 >= 0.5f && T1[p] < 0.5f) {   // far member: the post-splat T drops below 1/2 here
+                            const float a = ssr_log(T0), b = ssr_log(T1[p]), d = b - a;
+                            const float fr = (ssr_fabs(d) > 1e-20f) ? (-0.6931471805599453f - a) / d : 0.0f;
+                            v_depth_median += fr * vm;
+                            pend_zgrad[p] = (1.0f - fr) * vm;
+                            pend_zfar[p] = f.d;
+                            pend_Tfar[p] = T1[p];
+                        }
+                    }
+                    const float zd = dist ? ssr_log(ssr_max(f.d, 1e-6f)) : f.d;
+                    const float dotcv = ssr_fma(zd, c[3], ssr_fma(f.b, c[2], ssr_fma(f.g, c[1], f.r * c[0])));
+                    float v_alpha = T0 * dotcv - vT1p * T0;
                     const float w = alpha * T0;
-                    const float v_T0 = alpha * dotcv + vT1[p] * (1.0f - alpha);
+                    float v_T0 = alpha * dotcv + vT1p * (1.0f - alpha);
+                    float vcol[4] = {c[0] * w, c[1] * w, c[2] * w, c[3] * w};
+                    if (dist) {   // closed form D = W S - C^2, :497-517
+                        const float col[4] = {f.r, f.g, f.b, zd};
+                        float gsum = 0.0f;
+                        for (int q = dist_rgb ? 0 : 3; q < 4; q++) {
+                            vcol[q] += ((col[q] * Wd[p] - Cc[p][q]) * vD[p][q]) * (2.0f * w);
+                            gsum += ((Sc[p][q] + (col[q] * col[q]) * Wd[p]) - (col[q] * Cc[p][q]) * 2.0f) * vD[p][q];
+                        }
+                        v_alpha += T0 * gsum;
+                        v_T0 += alpha * gsum;
+                        vcol[3] *= 1.0f / ssr_max(f.d, 1e-6f);
+                    }
+                    vcol[3] += v_depth_median;
                     float t[10] = {0};
                     if (sigma >= 0.f && f.opac * vis <= 0.999f) {
                         const float v_sigma = (-f.opac) * vis * v_alpha;
@@ -922,9 +1049,11 @@ void or_raster_bwd(int64_t N, const float* xy, const float* depth, const float* 
                         t[1] = v_sigma * (f.cy * dx + f.cz * dy);
                         t[6] = vis * v_alpha;
                     }
-                    t[7] = c[0] * w; t[8] = c[1] * w; t[9] = c[2] * w; t[2] = c[3] * w;
+                    t[7] = vcol[0]; t[8] = vcol[1]; t[9] = vcol[2]; t[2] = vcol[3];
                     for (int q = 0; q < 10; q++) acc[q] += t[q];
                     if (abs_terms) for (int q = 0; q < 10; q++) aacc[q] += std::fabs((double)t[q]);
+                    if (accum_mode == 1) aw = ssr_max(aw, amap[p] * w);   // :553-562
+                    else if (accum_mode) { aw += amap[p] * w; if (accum_mode == 3) aw_den += w; }
                     T1[p] = T0; vT1[p] = v_T0;
                 }
                 if (any) {
@@ -933,6 +1062,8 @@ void or_raster_bwd(int64_t N, const float* xy, const float* depth, const float* 
                         part[(size_t)k * 10 + q] += v;
                         if (abs_terms) apart[(size_t)k * 10 + q] += aacc[q];
                     }
+                    if (accum_mode == 1) awpart[(size_t)k * 2] = ssr_max(awpart[(size_t)k * 2], aw);
+                    else if (accum_mode) { awpart[(size_t)k * 2] += aw; awpart[(size_t)k * 2 + 1] += aw_den; }
                 }
             }
         }
@@ -946,6 +1077,14 @@ void or_raster_bwd(int64_t N, const float* xy, const float* depth, const float* 
         v_opac[g] += p[6];
         v_srgb[3 * g] += p[7]; v_srgb[3 * g + 1] += p[8]; v_srgb[3 * g + 2] += p[9];
         if (abs_terms) for (int q = 0; q < 10; q++) abs_terms[(size_t)g * 10 + q] += apart[(size_t)k * 10 + q];
+        if (accum_mode) {
+            const int64_t wid = gaussian_ids ? gaussian_ids[g] : g;
+            if (accum_mode == 1) accum_weight[wid] = ssr_max(accum_weight[wid], awpart[(size_t)k * 2]);
+            else {
+                accum_weight[wid] += awpart[(size_t)k * 2];
+                if (accum_mode == 3) accum_weight[n_world + wid] += awpart[(size_t)k * 2 + 1];
+            }
+        }
     }
 }
 

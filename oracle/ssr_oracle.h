@@ -90,6 +90,27 @@ void or_raster_bwd(int64_t N, const float* xy, const float* depth, const float* 
     float* v_xy, float* v_sdepth, float* v_conic, float* v_opac, float* v_srgb,
     double* abs_terms /* [N,10] or NULL */);
 
+/* K7 / K8 with their variants. dist_type: 0 none, 1 depth (D), 2 rgb + depth (RGB_D).
+ * Forward: out_dist_rgb [H,W,3] (RGB_D), out_dist_depth [H,W] (D, RGB_D), out_median [H,W] or NULL.
+ * Backward: render_rgb / dist_*_img are the forward's outputs, v_dist_* and v_median (NULL = no
+ * median) the cotangents; accum_mode 0 none, 1 max, 2 sum, 3 avg (numerators then denominators,
+ * n_world rows each; gaussian_ids, or NULL, maps a screen row to its world row);
+ * accum_weight is max-/add-accumulated into (caller zero-fills). */
+void or_raster_fwd_ex(int64_t N, const float* xy, const float* depth, const float* conic,
+    const float* opac, const float* rgb, uint32_t width, uint32_t height,
+    const int32_t* tile_offsets, const int32_t* flatten_ids, int64_t n_isects,
+    float* out_rgb, float* out_depth, float* out_T, int32_t* out_last_ids, int64_t* stats,
+    int dist_type, float* out_dist_rgb, float* out_dist_depth, float* out_median);
+void or_raster_bwd_ex(int64_t N, const float* xy, const float* depth, const float* conic,
+    const float* opac, const float* rgb, uint32_t width, uint32_t height,
+    const int32_t* tile_offsets, const int32_t* flatten_ids, int64_t n_isects,
+    const float* render_T, const int32_t* last_ids, const float* render_depth,
+    const float* v_rgb, const float* v_depth, const float* v_T,
+    float* v_xy, float* v_sdepth, float* v_conic, float* v_opac, float* v_srgb, double* abs_terms,
+    int dist_type, const float* render_rgb, const float* dist_rgb_img, const float* dist_depth_img,
+    const float* v_dist_rgb, const float* v_dist_depth, const float* v_median,
+    int accum_mode, const float* accum_map, const int32_t* gaussian_ids, int64_t n_world, float* accum_weight);
+
 /* K9. Gradients are ACCUMULATED into v_* (caller zero-fills). */
 void or_projection_bwd(int64_t N, int sh_degree,
     const float* means, const float* quats, const float* log_scales, const float* opacity_logits,

@@ -160,32 +160,48 @@ def tile_n_bits(n_tiles):
     return b
 
 
-def raster_fwd(n, scr, w, h, offsets, flat):
+def raster_fwd(n, scr, w, h, offsets, flat, dist_type=0, median=False):
+    """dist_type 0 none / 1 depth / 2 rgb+depth distortion; median: also the median depth image."""
     o = dict(rgb=np.zeros((h, w, 3), np.float32), depth=np.zeros((h, w), np.float32),
              T=np.zeros((h, w), np.float32), last_ids=np.zeros((h, w), np.int32))
+    if dist_type:
+        o["dist_depth"] = np.zeros((h, w), np.float32)
+        if dist_type == 2:
+            o["dist_rgb"] = np.zeros((h, w, 3), np.float32)
+    if median:
+        o["median"] = np.zeros((h, w), np.float32)
     stats = np.zeros(5, np.int64)
-    lib().or_raster_fwd(C.c_int64(n), _p(scr["xy"]), _p(scr["depth"]), _p(scr["conic"]),
-                        _p(scr["opac"]), _p(scr["rgb"]), C.c_uint32(w), C.c_uint32(h), _p(offsets),
-                        _p(flat), C.c_int64(flat.size), _p(o["rgb"]), _p(o["depth"]), _p(o["T"]),
-                        _p(o["last_ids"]), _p(stats))
+    lib().or_raster_fwd_ex(C.c_int64(n), _p(scr["xy"]), _p(scr["depth"]), _p(scr["conic"]),
+                           _p(scr["opac"]), _p(scr["rgb"]), C.c_uint32(w), C.c_uint32(h), _p(offsets),
+                           _p(flat), C.c_int64(flat.size), _p(o["rgb"]), _p(o["depth"]), _p(o["T"]),
+                           _p(o["last_ids"]), _p(stats), C.c_int(dist_type), _p(o.get("dist_rgb")),
+                           _p(o.get("dist_depth")), _p(o.get("median")))
     o["K_f"], o["K_b"] = int(stats[0]), int(stats[1])
     o["visits_fwd"], o["visits_bwd"], o["visits_bwd_productive"] = int(stats[2]), int(stats[3]), int(stats[4])
     return o
 
 
-def raster_bwd(n, scr, w, h, offsets, flat, fwd, v_rgb, v_depth, v_T, with_abs=True):
+def raster_bwd(n, scr, w, h, offsets, flat, fwd, v_rgb, v_depth, v_T, with_abs=True, dist_type=0,
+               v_dist_rgb=None, v_dist_depth=None, v_median=None, accum_mode=0, accum_map=None,
+               gaussian_ids=None, n_world=None):
     g = dict(v_xy=np.zeros((n, 2), np.float32), v_depth=np.zeros(n, np.float32),
              v_conic=np.zeros((n, 3), np.float32), v_opac=np.zeros(n, np.float32),
              v_rgb=np.zeros((n, 3), np.float32))
     abs_terms = np.zeros((n, 10), np.float64) if with_abs else None
-    lib().or_raster_bwd(C.c_int64(n), _p(scr["xy"]), _p(scr["depth"]), _p(scr["conic"]),
-                        _p(scr["opac"]), _p(scr["rgb"]), C.c_uint32(w), C.c_uint32(h), _p(offsets),
-                        _p(flat), C.c_int64(flat.size), _p(fwd["T"]), _p(fwd["last_ids"]),
-                        _p(fwd["depth"]), _p(np.ascontiguousarray(v_rgb, np.float32)),
-                        _p(np.ascontiguousarray(v_depth, np.float32)),
-                        _p(np.ascontiguousarray(v_T, np.float32)),
-                        _p(g["v_xy"]), _p(g["v_depth"]), _p(g["v_conic"]), _p(g["v_opac"]),
-                        _p(g["v_rgb"]), _p(abs_terms))
+    n_world = n if n_world is None else n_world
+    if accum_mode:
+        g["accum_weight"] = np.zeros(n_world * (2 if accum_mode == 3 else 1), np.float32)
+    f32 = lambda a: None if a is None else np.ascontiguousarray(a, np.float32)
+    keep = [f32(v_rgb), f32(v_depth), f32(v_T), f32(v_dist_rgb), f32(v_dist_depth), f32(v_median), f32(accum_map),
+            None if gaussian_ids is None else np.ascontiguousarray(gaussian_ids, np.int32)]
+    lib().or_raster_bwd_ex(C.c_int64(n), _p(scr["xy"]), _p(scr["depth"]), _p(scr["conic"]),
+                           _p(scr["opac"]), _p(scr["rgb"]), C.c_uint32(w), C.c_uint32(h), _p(offsets),
+                           _p(flat), C.c_int64(flat.size), _p(fwd["T"]), _p(fwd["last_ids"]),
+                           _p(fwd["depth"]), _p(keep[0]), _p(keep[1]), _p(keep[2]),
+                           _p(g["v_xy"]), _p(g["v_depth"]), _p(g["v_conic"]), _p(g["v_opac"]),
+                           _p(g["v_rgb"]), _p(abs_terms), C.c_int(dist_type), _p(fwd["rgb"]), _p(fwd.get("dist_rgb")),
+                           _p(fwd.get("dist_depth")), _p(keep[3]), _p(keep[4]), _p(keep[5]), C.c_int(accum_mode),
+                           _p(keep[6]), _p(keep[7]), C.c_int64(n_world), _p(g.get("accum_weight")))
     g["abs_terms"] = abs_terms
     return g
 
@@ -239,7 +255,7 @@ def fused_projection_bwd_optimizer(scene, aabb, vs, params, g1, g2, hyper, step=
     return score
 
 
-def pipeline(scene, sh_degree=3, backward=True, tile_active=None):
+def pipeline(scene, sh_degree=3, backward=True, tile_active=None, variant=None):
     """The whole iteration in the reference's order (src/engine/EngineForward.cpp:166-293,
     src/engine/EngineLoss.cpp:138-240,359-368). tile_active: optional tile-skip map for the tile stage."""
     n, w, h = scene.n, scene.width, scene.height
@@ -250,11 +266,16 @@ def pipeline(scene, sh_degree=3, backward=True, tile_active=None):
     n_tiles = scene.tile_w * scene.tile_h
     sk, sv = sort_pairs(ids, flat, 0, 32 + tile_n_bits(n_tiles))
     offs = tile_offsets(sk, n_tiles)
-    f = raster_fwd(n, p, w, h, offs, sv)
+    # variant: dict(dist_type=, median=bool, v_dist_rgb=, v_dist_depth=, v_median=, accum_mode=, accum_map=)
+    va = variant or {}
+    f = raster_fwd(n, p, w, h, offs, sv, va.get("dist_type", 0), va.get("median", False))
     out = dict(proj=p, counts=counts, cum=cum, isect_ids=ids, flatten_ids=flat, pads=pads,
                sorted_ids=sk, sorted_flat=sv, offsets=offs, fwd=f)
     if backward:
-        out["vscreen"] = raster_bwd(n, p, w, h, offs, sv, f, scene.v_rgb, scene.v_depth, scene.v_T)
+        out["vscreen"] = raster_bwd(n, p, w, h, offs, sv, f, scene.v_rgb, scene.v_depth, scene.v_T,
+                                    dist_type=va.get("dist_type", 0), v_dist_rgb=va.get("v_dist_rgb"),
+                                    v_dist_depth=va.get("v_dist_depth"), v_median=va.get("v_median") if va.get("median") else None,
+                                    accum_mode=va.get("accum_mode", 0), accum_map=va.get("accum_map"))
         out["grads"] = projection_bwd(scene, p["aabb"], out["vscreen"], sh_degree)
     return out
 

@@ -112,3 +112,53 @@ def composite(px, py, frags, with_state=False):
         last = k
     depth = dsum / max(1 - T, 1e-10)
     return rgb, depth, T, last
+
+
+def composite_ex(px, py, frags, dist_type=0):
+    """composite() plus the variant outputs, each from its definition rather than from the kernel's
+    accumulators: per-splat weights w_k = alpha_k T_k; with distortion on, the depth channel is
+    c = ln(max(z, 1e-6)), rendered depth = exp(sum w c / W), and the distortion image is
+    1/2 sum_ij w_i w_j (c_i - c_j)^2 per channel (which equals W S - C^2); the median depth is where
+    the post-splat transmittance first drops below 1/2, interpolated linearly in ln T from the
+    previous splat (virtual first point z = 0, T = 1). Returns a dict."""
+    K = len(frags["opac"])
+    T = 1.0
+    ws, ks = [], []
+    median, prev_T, prev_z, found = 0.0, 1.0, 0.0, False
+    for k in range(K):
+        dx = frags["xy"][k, 0] - px
+        dy = frags["xy"][k, 1] - py
+        a, b, c = frags["conic"][k]
+        sigma = 0.5 * (a * dx * dx + c * dy * dy) + b * dx * dy
+        if sigma < 0:
+            continue
+        alpha = min(0.999, frags["opac"][k] * math.exp(-sigma))
+        if alpha <= ALPHA_T:
+            continue
+        nT = T * (1 - alpha)
+        if not found and prev_T >= 0.5 and nT < 0.5:
+            la, lb = math.log(prev_T), math.log(nT)
+            f = (math.log(0.5) - la) / (lb - la) if abs(lb - la) > 1e-20 else 0.0
+            median = prev_z + (frags["depth"][k] - prev_z) * f
+            found = True
+        prev_T, prev_z = nT, frags["depth"][k]
+        if nT <= 1e-4:
+            break
+        ws.append(alpha * T)
+        ks.append(k)
+        T = nT
+    w = np.array(ws)
+    ks = np.array(ks, int)
+    rgbs = frags["rgb"][ks] if len(ks) else np.zeros((0, 3))
+    z = frags["depth"][ks] if len(ks) else np.zeros(0)
+    W = max(1 - T, 1e-10)
+    out = dict(T=T, last=int(ks[-1]) if len(ks) else 0, rgb=(w[:, None] * rgbs).sum(axis=0), median=median, w=w, ks=ks)
+    if dist_type:
+        lz = np.log(np.maximum(z, 1e-6))
+        out["depth"] = math.exp((w * lz).sum() / W)
+        pair = lambda c: 0.5 * (w[:, None] * w[None, :] * (c[:, None] - c[None, :]) ** 2).sum()
+        out["dist_depth"] = pair(lz)
+        out["dist_rgb"] = np.array([pair(rgbs[:, q]) for q in range(3)]) if len(ks) else np.zeros(3)
+    else:
+        out["depth"] = (w * z).sum() / W
+    return out
