@@ -18,8 +18,8 @@
  *    cleared) by ssr_last_error(), like the reference's sticky backend::last_error()
  *    (src/backend/api/BackendRuntime.h:98). Nothing calls exit().
  *  - Supported variant: primitive "3dgs" (not antialiased), camera PINHOLE or EQUIRECTANGULAR,
- *    distortion NONE, one camera (C = 1), SH degree 0..3, dist_type None, no median, no
- *    accumulation weights; both the [C,N] layout and the packed (compacted, nnz rows) layout of
+ *    distortion NONE, one camera (C = 1), SH degree 0..3, dist_type None / D / RGB_D, median
+ *    depth, accumulation weights; both the [C,N] layout and the packed (compacted, nnz rows) layout of
  *    the projection outputs. Anything else is rejected with an error, as the reference
  *    rejects an uncompiled variant (src/kernels/projection/ProjectionFwd.cu:84-89).
  *  - Layouts are the reference's (src/primitives/PrimitiveBase3DGS.cuh:87-139,187-225).
@@ -39,6 +39,8 @@ typedef void* ssr_event_t;
 
 enum { SSR_CAM_PINHOLE = 0, SSR_CAM_EQUIRECT = 3 };       /* CameraModelType, src/core/Common.cuh */
 enum { SSR_SH_F32 = 0, SSR_SH_REF_Q8 = 1, SSR_SH_REF_Q16 = 2, SSR_SH_I8_F16SCALE = 3 };
+enum { SSR_DIST_NONE = 0, SSR_DIST_D = 1, SSR_DIST_RGB_D = 2 };   /* DistortionType, src/primitives/Primitive.cuh:24-32 */
+enum { SSR_ACCUM_NONE = 0, SSR_ACCUM_MAX = 1, SSR_ACCUM_SUM = 2, SSR_ACCUM_AVG = 3 };   /* DensifyAccumMode, :37-42 */
 enum { SSR_MEMCPY_H2D = 0, SSR_MEMCPY_D2H = 1, SSR_MEMCPY_D2D = 2, SSR_MEMCPY_H2H = 3,
        SSR_MEMCPY_AUTO = 4 };                             /* backend::MemcpyKind */
 
@@ -203,6 +205,15 @@ typedef struct {
     int32_t* last_ids;      /* [H,W] */
     const float* packed_rows; /* optional: rows written by ssr_projection_fwd for this screen;
                                  when given, `screen` is not read */
+    /* Variants (RasterizationEval3DFwd_kernel.cuh:143-148,245-307). dist_type SSR_DIST_D / _RGB_D:
+     * the depth channel is composited as ln(max(z, 1e-6)) and rendered as exp(mean), and the
+     * distortion image D = W S - C^2 (W = 1 - T, C / S first / second moments of the weights) is
+     * written for depth (and rgb). render_median non-NULL: depth where the post-splat
+     * transmittance crosses 1/2, interpolated in ln T; 0 where it never does. */
+    int32_t dist_type;          /* SSR_DIST_* */
+    float* distortion_rgb;      /* [H,W,3], RGB_D */
+    float* distortion_depth;    /* [H,W], D and RGB_D */
+    float* render_median;       /* optional [H,W] */
 } ssr_raster_fwd_params;
 int ssr_raster_fwd(const ssr_raster_fwd_params* p, ssr_stream_t stream);
 
@@ -225,6 +236,24 @@ typedef struct {
     const float* v_render_T;      /* [H,W] */
     ssr_screen v_screen;          /* accumulated into */
     const float* packed_rows;     /* optional, as in ssr_raster_fwd_params */
+    /* Variants (RasterizationEval3DBwd_kernel.cuh:150-172,207-279,433-585). With dist_type set:
+     * render_rgb and distortion_* are the forward's outputs, v_distortion_* the cotangents of the
+     * distortion image. v_render_median non-NULL: cotangent of the median depth. accum_mode
+     * SSR_ACCUM_*: accum_weight[w] receives max / sum over pixels of accum_weight_map[pixel] *
+     * alpha * T for world row w = gaussian_ids ? gaussian_ids[row] : row; AVG adds the sum of
+     * alpha * T at accum_weight[num_world + w]. The caller zero-fills accum_weight. */
+    int32_t dist_type;
+    const float* render_rgb;          /* [H,W,3], RGB_D */
+    const float* distortion_rgb;      /* [H,W,3], RGB_D */
+    const float* distortion_depth;    /* [H,W] */
+    const float* v_distortion_rgb;    /* [H,W,3], RGB_D */
+    const float* v_distortion_depth;  /* [H,W] */
+    const float* v_render_median;     /* optional [H,W] */
+    int32_t accum_mode;
+    const float* accum_weight_map;    /* [H,W] */
+    const int32_t* gaussian_ids;      /* optional [num_splats] (packed projection) */
+    int64_t num_world;                /* rows per lane of accum_weight */
+    float* accum_weight;              /* [num_world] or [2 num_world] (AVG) */
 } ssr_raster_bwd_params;
 int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t stream);
 

@@ -55,6 +55,26 @@ __device__ __forceinline__ int wave_max_i32(int v) {
     return v;
 }
 
+__device__ __forceinline__ float wave_sum_f32(float v) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max_f32(float v) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) v = ssr_max(v, __shfl_xor(v, d, 64));
+    return v;
+}
+// float atomic max through the integer orderings (src/core/Common.cuh:784-788)
+__device__ __forceinline__ void atomic_max_f32(float* p, float v) {
+    if (__float_as_int(v) >= 0) atomicMax(reinterpret_cast<int*>(p), __float_as_int(v));
+    else atomicMin(reinterpret_cast<unsigned*>(p), __float_as_uint(v));
+}
+
+// kDist (SSR_DIST_*), kMedian and kAccum (SSR_ACCUM_*) select the variants
+// (RasterizationEval3DBwd_kernel.cuh:150-172,207-279,433-585); <0, false, 0> is the plain kernel and
+// compiles to exactly the code it had without them.
+template <int kDist, bool kMedian, int kAccum>
 __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd_params P, int tile_w, int tile_h) {
     __shared__ FragLds frags[kBatch];
     __shared__ int32_t s_ids[kBatch];
@@ -80,11 +100,41 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
         vr = v[0]; vg = v[1]; vb = v[2];
         vd = P.v_render_depth[pid];
     }
+    // totals of the forward held constant during the sweep (distortion), median state, weight map
+    [[maybe_unused]] float Cr = 0.f, Cg = 0.f, Cb = 0.f, Cd = 0.f, Sr = 0.f, Sg = 0.f, Sb = 0.f, Sd = 0.f;
+    [[maybe_unused]] float vDr = 0.f, vDg = 0.f, vDb = 0.f, vDd = 0.f, Wd = 0.f;
+    [[maybe_unused]] float med_v = 0.f, pend_zgrad = 0.f, pend_zfar = 0.f, pend_Tfar = 0.f, amap = 0.f;
     {
         const float inv_alpha = 1.0f / ssr_max(1.0f - T1, 1e-10f);
         const float exp_depth = inside ? P.render_depth[pid] : 0.0f;
-        vT1 = vT1 + (exp_depth * vd) * inv_alpha;
-        vd = vd * inv_alpha;
+        if constexpr (kDist != SSR_DIST_NONE) {
+            // log-depth render: depth = exp(C_lnz / W)  (RasterizationEval3DBwd_kernel.cuh:212-218)
+            const float m = ssr_log(ssr_max(exp_depth, 1e-6f));
+            vT1 = vT1 + ((exp_depth * vd) * m) * inv_alpha;
+            vd = vd * (exp_depth * inv_alpha);
+            // C, S = (D + C^2) / W, W and the distortion cotangent (:228-257)
+            Cd = m * ssr_max(1.0f - T1, 1e-10f);
+            Wd = inside ? (1.0f - T1) : 0.0f;
+            const float invW = Wd > 1e-10f ? (1.0f / Wd) : 0.0f;
+            float Dd = 0.f, Dr = 0.f, Dg = 0.f, Db = 0.f;
+            if (inside) {
+                Dd = P.distortion_depth[pid]; vDd = P.v_distortion_depth[pid];
+                if constexpr (kDist == SSR_DIST_RGB_D) {
+                    const float* c = P.render_rgb + 3 * pid; Cr = c[0]; Cg = c[1]; Cb = c[2];
+                    const float* d = P.distortion_rgb + 3 * pid; Dr = d[0]; Dg = d[1]; Db = d[2];
+                    const float* v = P.v_distortion_rgb + 3 * pid; vDr = v[0]; vDg = v[1]; vDb = v[2];
+                }
+            }
+            Sd = (Dd + Cd * Cd) * invW;
+            if constexpr (kDist == SSR_DIST_RGB_D) {
+                Sr = (Dr + Cr * Cr) * invW; Sg = (Dg + Cg * Cg) * invW; Sb = (Db + Cb * Cb) * invW;
+            }
+        } else {
+            vT1 = vT1 + (exp_depth * vd) * inv_alpha;
+            vd = vd * inv_alpha;
+        }
+        if constexpr (kMedian) med_v = inside ? P.v_render_median[pid] : 0.0f;
+        if constexpr (kAccum != SSR_ACCUM_NONE) amap = inside ? P.accum_weight_map[pid] : 0.0f;
     }
 
     const int32_t range_start = P.tile_offsets[tile];
@@ -148,12 +198,46 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
                 if (__ballot(active) == 0ull) continue;
                 // Branch-free per-lane terms: an inactive lane runs with alpha = 0 and v_alpha = 0, which
                 // leaves its T and v_T unchanged (T/(1-0) = T, v_T + 0*(..) = v_T) and makes every term zero.
-                const float cr = q1.z, cg = q1.w, cb = q2.x, cdp = q2.y;
+                const float cr = q1.z, cg = q1.w, cb = q2.x;
+                float cdp = q2.y;
                 const float a = active ? alpha : 0.0f;
                 // 1/(1-alpha) by the hardware reciprocal (1 ulp): gradients are compared at 1e-3
                 const float T0 = T1 * __builtin_amdgcn_rcpf(1.0f - a);
-                const float dv = ssr_fma(cdp, vd, ssr_fma(cb, vb, ssr_fma(cg, vg, cr * vr))) - vT1;
+                [[maybe_unused]] float v_depth_median = 0.0f;
+                if constexpr (kMedian) {   // RasterizationEval3DBwd_kernel.cuh:433-470
+                    if (active && pend_Tfar > 0.0f) {   // near member of the crossing found at the previous active splat
+                        v_depth_median += pend_zgrad;
+                        const float dba = ssr_log(pend_Tfar) - ssr_log(T1);
+                        const float inv = (ssr_fabs(dba) > 1e-20f) ? (-1.0f / dba) : 0.0f;
+                        vT1 += ((med_v * (pend_zfar - q2.y)) * inv) / T1;
+                        pend_Tfar = 0.0f;
+                    }
+                    if (active && T0 >= 0.5f && T1 < 0.5f) {   // far member: post-splat T drops below 1/2 here
+                        const float la = ssr_log(T0), d = ssr_log(T1) - la;
+                        const float fr = (ssr_fabs(d) > 1e-20f) ? (-0.6931471805599453f - la) / d : 0.0f;
+                        v_depth_median += fr * med_v;
+                        pend_zgrad = (1.0f - fr) * med_v;
+                        pend_zfar = q2.y;
+                        pend_Tfar = T1;
+                    }
+                }
+                if constexpr (kDist != SSR_DIST_NONE) cdp = ssr_log(ssr_max(q2.y, 1e-6f));
+                float dv = ssr_fma(cdp, vd, ssr_fma(cb, vb, ssr_fma(cg, vg, cr * vr))) - vT1;
                 const float w = a * T0;
+                [[maybe_unused]] float xr = 0.f, xg = 0.f, xb = 0.f, xd = 0.f;   // distortion part of the colour gradient
+                if constexpr (kDist != SSR_DIST_NONE) {   // closed form D = W S - C^2 (:497-517)
+                    float gsum = 0.0f;
+                    const float w2 = 2.0f * w;
+                    if constexpr (kDist == SSR_DIST_RGB_D) {
+                        xr = ((cr * Wd - Cr) * vDr) * w2; xg = ((cg * Wd - Cg) * vDg) * w2; xb = ((cb * Wd - Cb) * vDb) * w2;
+                        gsum += ((Sr + (cr * cr) * Wd) - (cr * Cr) * 2.0f) * vDr;
+                        gsum += ((Sg + (cg * cg) * Wd) - (cg * Cg) * 2.0f) * vDg;
+                        gsum += ((Sb + (cb * cb) * Wd) - (cb * Cb) * 2.0f) * vDb;
+                    }
+                    xd = ((cdp * Wd - Cd) * vDd) * w2;
+                    gsum += ((Sd + (cdp * cdp) * Wd) - (cdp * Cd) * 2.0f) * vDd;
+                    dv += gsum;   // v_alpha gains T0 g and v_T0 gains alpha g, exactly where dv enters
+                }
                 const float ov = q1.y * vis;
                 // evaluate_alpha_vjp gate (src/primitives/Primitive3DGS.cuh:273); sigma >= 0 holds when active
                 const float v_alpha = (active && ov <= 0.999f) ? T0 * dv : 0.0f;
@@ -166,7 +250,26 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
                 const float t_x = ssr_fma(q0.z + q0.z, vsx, q0.w * vsy);
                 const float t_y = ssr_fma(q0.w, vsx, (q1.x + q1.x) * vsy);
                 const float t_o = vis * v_alpha;
-                const float t_r = vr * w, t_g = vg * w, t_b = vb * w, t_d = vd * w;
+                float t_r = vr * w, t_g = vg * w, t_b = vb * w, t_d = vd * w;
+                if constexpr (kDist != SSR_DIST_NONE) {
+                    if constexpr (kDist == SSR_DIST_RGB_D) { t_r += xr; t_g += xg; t_b += xb; }
+                    t_d = (t_d + xd) * (1.0f / ssr_max(q2.y, 1e-6f));   // d/d ln z -> d/dz
+                }
+                if constexpr (kMedian) t_d += v_depth_median;
+                if constexpr (kAccum != SSR_ACCUM_NONE) {   // :553-562,574-585
+                    const int64_t wid = P.gaussian_ids ? (int64_t)P.gaussian_ids[s_ids[k]] : (int64_t)s_ids[k];
+                    if constexpr (kAccum == SSR_ACCUM_MAX) {
+                        const float mx = wave_max_f32(amap * w);   // inactive lanes contribute map * 0; the running max starts at 0
+                        if (lane == 0) atomic_max_f32(P.accum_weight + wid, ssr_max(mx, 0.0f));
+                    } else {
+                        const float sm = wave_sum_f32(amap * w);
+                        if (lane == 0 && sm != 0.0f) atomicAdd(P.accum_weight + wid, sm);
+                        if constexpr (kAccum == SSR_ACCUM_AVG) {
+                            const float dn = wave_sum_f32(w);
+                            if (lane == 0 && dn != 0.0f) atomicAdd(P.accum_weight + P.num_world + wid, dn);
+                        }
+                    }
+                }
                 // transposing reduction: 10 channels -> 3 registers with one channel per row
                 const float ra_ = fold32(t_x, t_y), rb_ = fold32(t_d, t_ca), rc_ = fold32(t_cb, t_cc),
                             rd_ = fold32(t_o, t_r), re_ = fold32(t_g, t_b);
@@ -203,9 +306,38 @@ extern "C" int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t strea
     }
     SSR_REQUIRE(p->v_screen.xy && p->v_screen.depth && p->v_screen.conic && p->v_screen.opac && p->v_screen.rgb,
                 "ssr_raster_bwd", "null v_screen buffer");
+    SSR_REQUIRE(p->dist_type >= SSR_DIST_NONE && p->dist_type <= SSR_DIST_RGB_D, "ssr_raster_bwd",
+                "dist_type must be NONE, D or RGB_D (the 3dgs pixel has no normal channel)");
+    if (p->dist_type != SSR_DIST_NONE)
+        SSR_REQUIRE(p->distortion_depth && p->v_distortion_depth, "ssr_raster_bwd", "null depth distortion image or cotangent");
+    if (p->dist_type == SSR_DIST_RGB_D)
+        SSR_REQUIRE(p->render_rgb && p->distortion_rgb && p->v_distortion_rgb, "ssr_raster_bwd", "null rgb distortion input");
+    SSR_REQUIRE(p->accum_mode >= SSR_ACCUM_NONE && p->accum_mode <= SSR_ACCUM_AVG, "ssr_raster_bwd", "unknown accum_mode");
+    if (p->accum_mode != SSR_ACCUM_NONE) {
+        SSR_REQUIRE(p->accum_weight_map && p->accum_weight, "ssr_raster_bwd", "null accumulation buffer");
+        SSR_REQUIRE(p->num_world > 0, "ssr_raster_bwd", "num_world must be positive");
+    }
     const int tw = (int)ceil_div(p->width, kTile), th = (int)ceil_div(p->height, kTile);
-    hipLaunchKernelGGL(raster_bwd_kernel, dim3((unsigned)xcd_grid_size(tw * th)), dim3(kRasterBlock), 0, as_stream(stream),
-                       *p, tw, th);
+    const dim3 grid((unsigned)xcd_grid_size(tw * th)), block(kRasterBlock);
+    hipStream_t st = as_stream(stream);
+    const bool med = p->v_render_median != nullptr;
+#define SSR_BWD(D, M, A) hipLaunchKernelGGL((raster_bwd_kernel<D, M, A>), grid, block, 0, st, *p, tw, th)
+#define SSR_BWD_A(D, M)                                        \
+    switch (p->accum_mode) {                                   \
+        case SSR_ACCUM_MAX: SSR_BWD(D, M, SSR_ACCUM_MAX); break; \
+        case SSR_ACCUM_SUM: SSR_BWD(D, M, SSR_ACCUM_SUM); break; \
+        case SSR_ACCUM_AVG: SSR_BWD(D, M, SSR_ACCUM_AVG); break; \
+        default: SSR_BWD(D, M, SSR_ACCUM_NONE); break;           \
+    }
+#define SSR_BWD_M(D) if (med) { SSR_BWD_A(D, true) } else { SSR_BWD_A(D, false) }
+    switch (p->dist_type) {
+        case SSR_DIST_D: SSR_BWD_M(SSR_DIST_D) break;
+        case SSR_DIST_RGB_D: SSR_BWD_M(SSR_DIST_RGB_D) break;
+        default: SSR_BWD_M(SSR_DIST_NONE) break;
+    }
+#undef SSR_BWD_M
+#undef SSR_BWD_A
+#undef SSR_BWD
     SSR_CHECK_LAUNCH("ssr_raster_bwd");
     return 0;
 }

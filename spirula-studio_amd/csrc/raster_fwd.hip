@@ -10,6 +10,9 @@
 
 namespace ssr {
 
+// kDist (SSR_DIST_*) and kMedian select the variants (RasterizationEval3DFwd_kernel.cuh:143-148,245-307);
+// <0, false> is the plain kernel and compiles to exactly the code it had without them.
+template <int kDist, bool kMedian>
 __global__ __launch_bounds__(kRasterBlock) void raster_fwd_kernel(ssr_raster_fwd_params P, int tile_w, int tile_h) {
     __shared__ FragLds frags[kBatch];
     const int n_tiles = tile_w * tile_h;
@@ -27,6 +30,8 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_kernel(ssr_raster_fwd
     const int32_t range_end = (tile == n_tiles - 1) ? (int32_t)P.n_isects : P.tile_offsets[tile + 1];
 
     float T = 1.0f, cr = 0.f, cg = 0.f, cb = 0.f, cd = 0.f;
+    [[maybe_unused]] float s2r = 0.f, s2g = 0.f, s2b = 0.f, s2d = 0.f;           // second moments (distortion)
+    [[maybe_unused]] float median = 0.f, med_prev_z = 0.f, med_prev_T = 1.0f;   // median depth
     uint32_t cur_idx = 0;
     const float tile_x0 = (float)(tx * kTile), tile_y0 = (float)(ty * kTile);
 
@@ -54,10 +59,28 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_kernel(ssr_raster_fwd
                 const float alpha = eval_alpha_fast(q0, q1, q2.w, px, py, dx, dy, vis, sigma);
                 if (!done && alpha > kAlphaThreshold) {
                     const float next_T = T * (1.0f - alpha);
+                    if constexpr (kMedian) {   // before the early-out, so a splat that ends the pixel still counts
+                        if (med_prev_T >= 0.5f && next_T < 0.5f) {
+                            const float a = ssr_log(med_prev_T), b = ssr_log(next_T), d = b - a;
+                            const float fr = (ssr_fabs(d) > 1e-20f) ? (-0.6931471805599453f - a) / d : 0.0f;
+                            median = med_prev_z + (q2.y - med_prev_z) * fr;
+                        }
+                        med_prev_T = next_T;
+                        med_prev_z = q2.y;
+                    }
                     if (next_T > kTransmitThreshold) {
                         const float w = alpha * T;
+                        float zd = q2.y;
+                        if constexpr (kDist != SSR_DIST_NONE) {
+                            zd = ssr_log(ssr_max(q2.y, 1e-6f));
+                            if constexpr (kDist == SSR_DIST_RGB_D) {
+                                s2r = ssr_fma(q1.z * q1.z, w, s2r); s2g = ssr_fma(q1.w * q1.w, w, s2g);
+                                s2b = ssr_fma(q2.x * q2.x, w, s2b);
+                            }
+                            s2d = ssr_fma(zd * zd, w, s2d);
+                        }
                         cr = ssr_fma(q1.z, w, cr); cg = ssr_fma(q1.w, w, cg); cb = ssr_fma(q2.x, w, cb);
-                        cd = ssr_fma(q2.y, w, cd);
+                        cd = ssr_fma(zd, w, cd);
                         cur_idx = (uint32_t)(batch_start + k);
                         T = next_T;
                     } else {
@@ -73,7 +96,18 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_kernel(ssr_raster_fwd
         const float invW = 1.0f / ssr_max(1.0f - T, 1e-10f);
         float* o = P.render_rgb + 3 * pid;
         o[0] = cr; o[1] = cg; o[2] = cb;
-        P.render_depth[pid] = cd * invW;
+        if constexpr (kMedian) P.render_median[pid] = median;
+        if constexpr (kDist != SSR_DIST_NONE) {   // D = W S - C^2 on the raw accumulators
+            const float W = 1.0f - T;
+            if constexpr (kDist == SSR_DIST_RGB_D) {
+                float* d = P.distortion_rgb + 3 * pid;
+                d[0] = s2r * W - cr * cr; d[1] = s2g * W - cg * cg; d[2] = s2b * W - cb * cb;
+            }
+            P.distortion_depth[pid] = s2d * W - cd * cd;
+            P.render_depth[pid] = ssr_exp(cd * invW);
+        } else {
+            P.render_depth[pid] = cd * invW;
+        }
         P.last_ids[pid] = (int32_t)cur_idx;
     }
 }
@@ -98,9 +132,21 @@ extern "C" int ssr_raster_fwd(const ssr_raster_fwd_params* p, ssr_stream_t strea
             SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->screen.xy) & 7) == 0, "ssr_raster_fwd", "screen.xy must be 8-byte aligned");
         }
     }
+    SSR_REQUIRE(p->dist_type >= SSR_DIST_NONE && p->dist_type <= SSR_DIST_RGB_D, "ssr_raster_fwd",
+                "dist_type must be NONE, D or RGB_D (the 3dgs pixel has no normal channel)");
+    SSR_REQUIRE(p->dist_type == SSR_DIST_NONE || p->distortion_depth, "ssr_raster_fwd", "null distortion_depth");
+    SSR_REQUIRE(p->dist_type != SSR_DIST_RGB_D || p->distortion_rgb, "ssr_raster_fwd", "null distortion_rgb");
     const int tw = (int)ceil_div(p->width, kTile), th = (int)ceil_div(p->height, kTile);
-    hipLaunchKernelGGL(raster_fwd_kernel, dim3((unsigned)xcd_grid_size(tw * th)), dim3(kRasterBlock), 0, as_stream(stream),
-                       *p, tw, th);
+    const dim3 grid((unsigned)xcd_grid_size(tw * th)), block(kRasterBlock);
+    hipStream_t s = as_stream(stream);
+#define SSR_FWD(D, M) hipLaunchKernelGGL((raster_fwd_kernel<D, M>), grid, block, 0, s, *p, tw, th)
+    const bool med = p->render_median != nullptr;
+    switch (p->dist_type) {
+        case SSR_DIST_D: if (med) SSR_FWD(SSR_DIST_D, true); else SSR_FWD(SSR_DIST_D, false); break;
+        case SSR_DIST_RGB_D: if (med) SSR_FWD(SSR_DIST_RGB_D, true); else SSR_FWD(SSR_DIST_RGB_D, false); break;
+        default: if (med) SSR_FWD(SSR_DIST_NONE, true); else SSR_FWD(SSR_DIST_NONE, false); break;
+    }
+#undef SSR_FWD
     SSR_CHECK_LAUNCH("ssr_raster_fwd");
     return 0;
 }

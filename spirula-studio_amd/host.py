@@ -22,6 +22,7 @@ SYMBOLS = {
     "ssrh_set_data_3dgs": (C.c_int, [C.c_int64, vp, vp, vp, vp, vp, vp, C.c_int]),
     "ssrh_set_sh_value_quant": (C.c_int, [C.c_int, vp, C.c_int64, C.c_int, vp, C.c_int64, C.c_int, C.c_int64]),
     "ssrh_set_camera_params": (C.c_int, [C.c_int, C.c_int, C.c_char_p, C.c_char_p, vp, vp, C.c_int]),
+    "ssrh_backward_with_variants": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, C.c_int]),
     "ssrh_backward_fused_optimizer": (C.c_int, [vp, vp, vp, vp, C.c_int]),
     "ssrh_copy_params_to_host": (C.c_int, [vp, vp, vp, vp, vp, vp]),
     "ssrh_set_tile_mask": (C.c_int, [vp, C.c_int, C.c_int]),
@@ -65,7 +66,9 @@ CACHE = dict(aabb=(0, np.float32), sort_depth=(1, np.float32), xy=(2, np.float32
              conic=(4, np.float32), opac=(5, np.float32), rgb=(6, np.float32), sorted_ids=(7, np.int64),
              sorted_flat=(8, np.int32), offsets=(9, np.int32), last_ids=(10, np.int32), radii=(11, np.float32),
              v_xy=(12, np.float32), v_depth=(13, np.float32), v_conic=(14, np.float32), v_opac=(15, np.float32),
-             v_rgb=(16, np.float32), gaussian_ids=(17, np.int32), camera_ids=(18, np.int32))
+             v_rgb=(16, np.float32), gaussian_ids=(17, np.int32), camera_ids=(18, np.int32),
+             dist_rgb=(19, np.float32), dist_depth=(20, np.float32), median=(21, np.float32),
+             accum_weight=(22, np.float32))
 
 
 class Engine:
@@ -77,6 +80,7 @@ class Engine:
         projection_3dgs_packed_forward (the visible-splat work list then has no role)."""
         self.h = load()
         self.packed_projection = bool(packed_projection)
+        self.dist_type, self.output_median = 0, False   # variants of the next forward (set_variants)
         self.sc = scene
         self.sh_degree = sh_degree
         check(self.h.ssrh_init(device))
@@ -117,7 +121,19 @@ class Engine:
         check(self.h.ssrh_set_tile_mask(mask.ctypes.data, mask.shape[0], mask.shape[1]))
 
     def forward(self):
-        check(self.h.ssrh_forward_3dgs(b"3dgs", self.sh_degree, int(self.packed_projection), 0, 0))
+        check(self.h.ssrh_forward_3dgs(b"3dgs", self.sh_degree, int(self.packed_projection), int(self.output_median),
+                                       int(self.dist_type)))
+
+    def set_variants(self, dist_type=0, median=False):
+        """dist_type 0 none / 1 depth / 2 rgb+depth distortion; median: also render the median depth."""
+        self.dist_type, self.output_median = int(dist_type), bool(median)
+
+    def backward_with_variants(self, v_dist_rgb=None, v_dist_depth=None, v_median=None, accum_map=None, accum_mode=0):
+        f32 = lambda a: None if a is None else np.ascontiguousarray(a, np.float32)
+        keep = [f32(v_dist_rgb), f32(v_dist_depth), f32(v_median), f32(accum_map)]
+        ptr = lambda a: None if a is None else a.ctypes.data
+        check(self.h.ssrh_backward_with_variants(self.d_vrgb.ptr, self.d_vdepth.ptr, self.d_vT.ptr, ptr(keep[0]), ptr(keep[1]),
+                                                 ptr(keep[2]), ptr(keep[3]), int(accum_mode)))
 
     def backward(self):
         check(self.h.ssrh_backward_from_render_grad(self.d_vrgb.ptr, self.d_vdepth.ptr, self.d_vT.ptr))

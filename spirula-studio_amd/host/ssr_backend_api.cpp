@@ -418,8 +418,8 @@ rasterize_to_pixels_3dgs_fwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     // the screen row alone (src/kernels/raster/RasterizationEval3DFwd_kernel.cuh:183-184), so it is
     // accepted and not read.
     if (gaussian_ids.data_ptr()) num_splats = gaussian_ids.size();
-    if (dist_type != DistortionType::None) throw std::runtime_error("rasterize_to_pixels_3dgs_fwd: depth distortion is not built in this backend");
-    if (output_median) throw std::runtime_error("rasterize_to_pixels_3dgs_fwd: median depth is not built in this backend");
+    if (dist_type == DistortionType::DN || dist_type == DistortionType::RGB_DN)
+        throw std::runtime_error("rasterize_to_pixels_3dgs_fwd: normal distortion needs a normal channel, which the 3dgs pixel does not have");
     const int64_t I = tile_offsets.size<0>();
     if (I != 1) throw std::runtime_error("rasterize_to_pixels_3dgs_fwd: this backend runs one image per call");
     RenderOutput::TensorTuple renders;
@@ -436,11 +436,27 @@ rasterize_to_pixels_3dgs_fwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     p.render_rgb = (float*)std::get<0>(renders).data_ptr(); p.render_depth = std::get<1>(renders).data_ptr();
     p.render_T = Ts.data_ptr(); p.last_ids = last.data_ptr();
     if (g_packed_rows && p.screen.xy == g_packed_for_xy) p.packed_rows = g_packed_rows;
+    // distortion channels present in dist_type only (RenderOutput::resizeDistortion, src/primitives/Primitive.cuh:88-101)
+    RenderOutput::TensorTuple distortions;
+    DeviceTensor3D<float> median;
+    p.dist_type = (int32_t)dist_type;
+    if (dist_type != DistortionType::None) {
+        std::get<1>(distortions).resize(PoolSlot::RenderDistortionDepth, I, image_height, image_width);
+        p.distortion_depth = std::get<1>(distortions).data_ptr();
+        if (dist_type == DistortionType::RGB_D) {
+            std::get<0>(distortions).resize(PoolSlot::RenderDistortionRgb, I, image_height, image_width);
+            p.distortion_rgb = (float*)std::get<0>(distortions).data_ptr();
+        }
+    }
+    if (output_median) {
+        median.resize(PoolSlot::RenderMedian, I, image_height, image_width);
+        p.render_median = median.data_ptr();
+    }
     {
         StageTimer t(&g_times.k7);
         ok(ssr_raster_fwd(&p, nullptr), "rasterize_to_pixels_3dgs_fwd");
     }
-    return std::make_tuple(renders, Ts, last, RenderOutput::TensorTuple{}, DeviceTensor3D<float>{});
+    return std::make_tuple(renders, Ts, last, distortions, median);
 }
 
 std::tuple<std::vector<DeviceTensorFloatND>, std::vector<DeviceTensorFloatND>, DeviceVector<float>>
@@ -449,17 +465,20 @@ rasterize_to_pixels_3dgs_bwd(int64_t num_splats, std::vector<DeviceTensorFloatND
                              const uint32_t image_width, const uint32_t image_height,
                              const DeviceTensor3D<int32_t> tile_offsets, const DeviceVector<int32_t> flatten_ids,
                              const DeviceTensor3D<float> render_Ts, const DeviceTensor3D<int32_t> last_ids,
-                             RenderOutput::TensorTuple render_outputs_tuple, std::optional<RenderOutput::TensorTuple>,
-                             DistortionType dist_type, DeviceTensor3D<float> accum_weight_map, DensifyAccumMode accum_mode,
+                             RenderOutput::TensorTuple render_outputs_tuple,
+                             std::optional<RenderOutput::TensorTuple> distortion_fwd_outputs, DistortionType dist_type, DeviceTensor3D<float> accum_weight_map, DensifyAccumMode accum_mode,
                              RenderOutput::TensorTuple v_render_outputs, const DeviceTensor3D<float> v_render_Ts,
-                             const DeviceTensor3D<float> v_median, std::optional<RenderOutput::TensorTuple>,
+                             const DeviceTensor3D<float> v_median,
+                             std::optional<RenderOutput::TensorTuple> v_distortion_outputs,
                              std::optional<std::vector<DeviceTensorFloatND>> v_splats_w,
                              std::optional<std::vector<DeviceTensorFloatND>> v_splats_s) {
+    const int64_t num_world = num_splats;   // rows of accum_weight (src/kernels/raster/RasterizationBwd.cu:82-84)
     if (gaussian_ids.data_ptr()) num_splats = gaussian_ids.size();   // packed: v_screen has one row per screen row
-    if (dist_type != DistortionType::None) throw std::runtime_error("rasterize_to_pixels_3dgs_bwd: depth distortion is not built in this backend");
-    if (accum_mode != DensifyAccumMode::None || accum_weight_map.data_ptr())
-        throw std::runtime_error("rasterize_to_pixels_3dgs_bwd: accumulation weights are not built in this backend");
-    if (v_median.data_ptr()) throw std::runtime_error("rasterize_to_pixels_3dgs_bwd: median depth is not built in this backend");
+    if (dist_type == DistortionType::DN || dist_type == DistortionType::RGB_DN)
+        throw std::runtime_error("rasterize_to_pixels_3dgs_bwd: normal distortion needs a normal channel, which the 3dgs pixel does not have");
+    if (dist_type != DistortionType::None && (!distortion_fwd_outputs || !v_distortion_outputs))
+        throw std::runtime_error("rasterize_to_pixels_3dgs_bwd: distortion needs the forward distortion image and its gradient");
+    if (accum_weight_map.data_ptr() == nullptr) accum_mode = DensifyAccumMode::None;   // src/kernels/raster/RasterizationBwd.cu:234
     std::vector<DeviceTensorFloatND> vs;
     if (v_splats_s) {
         vs = *v_splats_s;   // caller-provided accumulators are added into as they are
@@ -488,13 +507,34 @@ rasterize_to_pixels_3dgs_bwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     p.v_render_T = v_render_Ts.data_ptr();
     p.v_screen = screen_of(vs);
     if (g_packed_rows && p.screen.xy == g_packed_for_xy) p.packed_rows = g_packed_rows;
+    p.dist_type = (int32_t)dist_type;
+    if (dist_type != DistortionType::None) {
+        p.distortion_depth = std::get<1>(*distortion_fwd_outputs).data_ptr();
+        p.v_distortion_depth = std::get<1>(*v_distortion_outputs).data_ptr();
+        if (dist_type == DistortionType::RGB_D) {
+            p.render_rgb = (const float*)std::get<0>(render_outputs_tuple).data_ptr();
+            p.distortion_rgb = (const float*)std::get<0>(*distortion_fwd_outputs).data_ptr();
+            p.v_distortion_rgb = (const float*)std::get<0>(*v_distortion_outputs).data_ptr();
+        }
+    }
+    p.v_render_median = v_median.data_ptr();
+    DeviceVector<float> accum;
+    p.accum_mode = (int32_t)accum_mode;
+    if (accum_mode != DensifyAccumMode::None) {   // RasterizationBwd.cu:157-163
+        accum.resize(PoolSlot::RasterBwdAccumWeight, num_world * (accum_mode == DensifyAccumMode::Avg ? 2 : 1));
+        accum.zero();
+        p.accum_weight_map = accum_weight_map.data_ptr();
+        p.accum_weight = accum.data_ptr();
+        p.num_world = num_world;
+        p.gaussian_ids = gaussian_ids.data_ptr();
+    }
     {
         StageTimer t(&g_times.k8);
         ok(ssr_raster_bwd(&p, nullptr), "rasterize_to_pixels_3dgs_bwd");
     }
     std::vector<DeviceTensorFloatND> vw = v_splats_w ? *v_splats_w : std::vector<DeviceTensorFloatND>{};
     (void)splats_w;
-    return std::make_tuple(vw, vs, DeviceVector<float>{});
+    return std::make_tuple(vw, vs, accum);
 }
 
 void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,

@@ -172,12 +172,18 @@ void forward_3dgs(std::string primitive, int sh_degree, bool packed, bool output
         N, in_splats, screen, E.fwd.gaussian_ids, (uint32_t)E.camera.width, (uint32_t)E.camera.height, offsets, flat,
         (DistortionType)dist_type_int, output_median);
     E.fwd.renders = renders; E.fwd.render_Ts = Ts; E.fwd.last_ids = last;
+    E.fwd.distortions = dist; E.fwd.dist_type = (DistortionType)dist_type_int; E.fwd.render_median = median;
 }
 
 namespace {
 // stage the pixel cotangents and run the compositing backward; returns v_screen
+struct VariantGrads {
+    TorchTensorView v_dist_rgb{0, 4, {}}, v_dist_depth{0, 4, {}}, v_median{0, 4, {}}, accum_map{0, 4, {}};
+    DensifyAccumMode accum_mode = DensifyAccumMode::None;
+};
+
 std::vector<DeviceTensorFloatND> raster_backward(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
-                                                 TorchTensorView v_render_Ts) {
+                                                 TorchTensorView v_render_Ts, const VariantGrads& vg = VariantGrads{}) {
     auto& E = engine();
     const int64_t C = E.camera.num, H = E.camera.height, W = E.camera.width;
     auto stage = [&](PoolSlot slot, const TorchTensorView& src, int ch) -> float* {
@@ -194,11 +200,26 @@ std::vector<DeviceTensorFloatND> raster_backward(TorchTensorView v_render_rgb, T
     std::get<0>(v_renders) = DeviceTensor3D<float3>((float3*)v_rgb, C, H, W);
     std::get<1>(v_renders) = DeviceTensor3D<float>(v_depth, C, H, W);
     DeviceTensor3D<float> v_Ts_t(v_Ts, C, H, W);
+    // cotangents of the variants that the forward produced
+    std::optional<RenderOutput::TensorTuple> dist_fwd, v_dist;
+    if (E.fwd.dist_type != DistortionType::None) {
+        if (!std::get<0>(vg.v_dist_depth)) throw std::runtime_error("backward: the forward ran with distortion; its gradient is required");
+        RenderOutput::TensorTuple vd;
+        std::get<1>(vd) = DeviceTensor3D<float>(stage(PoolSlot::EngVDistDepth, vg.v_dist_depth, 1), C, H, W);
+        if (E.fwd.dist_type == DistortionType::RGB_D)
+            std::get<0>(vd) = DeviceTensor3D<float3>((float3*)stage(PoolSlot::EngVDistRgb, vg.v_dist_rgb, 3), C, H, W);
+        dist_fwd = E.fwd.distortions; v_dist = vd;
+    }
+    DeviceTensor3D<float> v_med, amap;
+    if (E.fwd.render_median.data_ptr() && std::get<0>(vg.v_median))
+        v_med = DeviceTensor3D<float>(stage(PoolSlot::EngVMedian, vg.v_median, 1), C, H, W);
+    if (vg.accum_mode != DensifyAccumMode::None && std::get<0>(vg.accum_map))
+        amap = DeviceTensor3D<float>(stage(PoolSlot::EngAccumMap, vg.accum_map, 1), C, H, W);
     auto [vw, vs, accum] = rasterize_to_pixels_3dgs_bwd(
         E.cur_num_splats, E.fwd.splats_w, E.fwd.splats_s, E.fwd.gaussian_ids, (uint32_t)W, (uint32_t)H,
-        E.fwd.tile_offsets, E.fwd.flatten_ids, E.fwd.render_Ts, E.fwd.last_ids, E.fwd.renders, std::nullopt,
-        DistortionType::None, DeviceTensor3D<float>{}, DensifyAccumMode::None, v_renders, v_Ts_t, DeviceTensor3D<float>{},
-        std::nullopt, std::nullopt, std::nullopt);
+        E.fwd.tile_offsets, E.fwd.flatten_ids, E.fwd.render_Ts, E.fwd.last_ids, E.fwd.renders, dist_fwd,
+        E.fwd.dist_type, amap, vg.accum_mode, v_renders, v_Ts_t, v_med, v_dist, std::nullopt, std::nullopt);
+    if (accum.data_ptr()) { E.fwd.accum_weight = accum; E.fwd.accum_mode = vg.accum_mode; }   // EngineLoss.cpp:243-246
     return vs;
 }
 }  // namespace
@@ -228,6 +249,32 @@ void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorV
     E.grad.dirty_valid = E.grad.dirty_list != nullptr || (E.packed && E.fwd.gaussian_ids.size() == 0);
 }
 
+
+void engine_backward_with_variants(TorchTensorView v_render_rgb, TorchTensorView v_render_depth, TorchTensorView v_render_Ts,
+                                   TorchTensorView v_dist_rgb, TorchTensorView v_dist_depth, TorchTensorView v_median,
+                                   TorchTensorView accum_map, int accum_mode) {
+    auto& E = engine();
+    if (std::get<0>(E.fwd.renders).data_ptr() == nullptr)
+        throw std::runtime_error("engine_backward_with_variants: forward_3dgs must be called first");
+    alloc_grad_buffers();
+    VariantGrads vg;
+    vg.v_dist_rgb = v_dist_rgb; vg.v_dist_depth = v_dist_depth; vg.v_median = v_median; vg.accum_map = accum_map;
+    vg.accum_mode = (DensifyAccumMode)accum_mode;
+    auto vs = raster_backward(v_render_rgb, v_render_depth, v_render_Ts, vg);
+    E.grad.v_screen = vs;
+    std::vector<DeviceTensorFloatND> v_world = {
+        DeviceTensorFloatND(E.grad.means), DeviceTensorFloatND(E.grad.quats), DeviceTensorFloatND(E.grad.scales),
+        DeviceTensorFloatND((float*)E.grad.opacities.data_ptr(), {E.grad.opacities.size(), 1}),
+        DeviceTensorFloatND(E.grad.features_dc), DeviceTensorFloatND(E.grad.features_sh)};
+    projection_3dgs_backward(
+        E.cur_num_splats, E.sh_degree, E.fwd.splats_w, E.camera.viewmats, E.camera.intrins, (uint32_t)E.camera.width,
+        (uint32_t)E.camera.height, E.camera.model_str, E.camera.distortion_str, E.camera.dist_coeffs, E.fwd.camera_ids,
+        E.fwd.gaussian_ids, E.fwd.aabb, vs, v_world, nullptr, E.world.sh_packed, E.world.sh_bounds, (uint32_t)E.num_sh,
+        E.world.sh_value_bits, E.world.sh_bounds_stride);
+    E.grad.dirty_list = ssr_ext::last_backward_list(&E.grad.dirty_count);
+    E.grad.dirty_key = (const void*)E.grad.means.data_ptr();
+    E.grad.dirty_valid = E.grad.dirty_list != nullptr || (E.packed && E.fwd.gaussian_ids.size() == 0);
+}
 
 void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
                                      TorchTensorView v_render_Ts, const float hyper[12], int step) {
@@ -375,6 +422,16 @@ int ssrh_backward_from_render_grad(const float* v_rgb, const float* v_depth, con
     });
 }
 
+int ssrh_backward_with_variants(const float* v_rgb, const float* v_depth, const float* v_Ts, const float* v_dist_rgb,
+                                const float* v_dist_depth, const float* v_median, const float* accum_map, int accum_mode) {
+    return guard([&] {
+        const int64_t C = engine().camera.num, H = engine().camera.height, W = engine().camera.width;
+        engine_backward_with_variants(tv(v_rgb, 4, {C, H, W, 3}), tv(v_depth, 4, {C, H, W, 1}), tv(v_Ts, 4, {C, H, W, 1}),
+                                      tv(v_dist_rgb, 4, {C, H, W, 3}), tv(v_dist_depth, 4, {C, H, W, 1}), tv(v_median, 4, {C, H, W, 1}),
+                                      tv(accum_map, 4, {C, H, W, 1}), accum_mode);
+    });
+}
+
 int ssrh_backward_fused_optimizer(const float* v_rgb, const float* v_depth, const float* v_Ts, const float* hyper12, int step) {
     return guard([&] {
         const int64_t C = engine().camera.num, H = engine().camera.height, W = engine().camera.width;
@@ -408,7 +465,8 @@ int ssrh_copy_grads_to_host(float* means, float* quats, float* scales, float* op
 // Device addresses of the forward cache, for tests that compare intermediate buffers.
 //   which: 0 aabb, 1 sort depths, 2..6 screen xy/depth/conic/opac/rgb, 7 sorted keys, 8 sorted ids,
 //          9 tile offsets, 10 last_ids, 11 radii, 12..16 v_screen xy/depth/conic/opac/rgb,
-//          17 gaussian_ids, 18 camera_ids (packed projection)
+//          17 gaussian_ids, 18 camera_ids (packed projection), 19/20 distortion rgb/depth, 21 median depth,
+//          22 accumulated weights
 int ssrh_cache_pointer(int which, void** ptr, int64_t* count) {
     return guard([&] {
         auto& E = engine();
@@ -423,6 +481,10 @@ int ssrh_cache_pointer(int which, void** ptr, int64_t* count) {
             case 10: *ptr = E.fwd.last_ids.data_ptr(); *count = E.fwd.last_ids.numel(); break;
             case 11: *ptr = E.optim.radii.data_ptr(); *count = E.optim.radii.size(); break;
             case 12: case 13: case 14: case 15: case 16: nd(E.grad.v_screen.at(which - 12)); break;
+            case 19: *ptr = std::get<0>(E.fwd.distortions).data_ptr(); *count = std::get<0>(E.fwd.distortions).numel() * 3; break;
+            case 20: *ptr = std::get<1>(E.fwd.distortions).data_ptr(); *count = std::get<1>(E.fwd.distortions).numel(); break;
+            case 21: *ptr = E.fwd.render_median.data_ptr(); *count = E.fwd.render_median.numel(); break;
+            case 22: *ptr = E.fwd.accum_weight.data_ptr(); *count = E.fwd.accum_weight.size(); break;
             case 17: *ptr = E.fwd.gaussian_ids.data_ptr(); *count = E.fwd.gaussian_ids.size(); break;
             case 18: *ptr = E.fwd.camera_ids.data_ptr(); *count = E.fwd.camera_ids.size(); break;
             default: throw std::runtime_error("unknown cache buffer");

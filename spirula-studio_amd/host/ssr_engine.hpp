@@ -47,6 +47,9 @@ struct EngineState {
         DeviceVector<int32_t> tile_active;
         DeviceVector<int64_t> isect_ids; DeviceVector<int32_t> flatten_ids; DeviceTensor3D<int32_t> tile_offsets;
         RenderOutput::TensorTuple renders; DeviceTensor3D<float> render_Ts; DeviceTensor3D<int32_t> last_ids;
+        RenderOutput::TensorTuple distortions; DistortionType dist_type = DistortionType::None;   // EngineForward.cpp:287-291
+        DeviceTensor3D<float> render_median;
+        DeviceVector<float> accum_weight; DensifyAccumMode accum_mode = DensifyAccumMode::None;    // EngineLoss.cpp:243-246
     } fwd;
     struct {
         DeviceVector<float3> means; DeviceVector<float4> quats; DeviceVector<float3> scales;
@@ -82,6 +85,12 @@ void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorV
 // max_gauss_ratio, scale_reg_w, mcmc_opacity_w, mcmc_scale_w, quat_norm_w, sh_reg_w.
 void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
                                      TorchTensorView v_render_Ts, const float hyper[12], int step);
+// engine_backward_from_render_grad with the cotangents of the variants of the forward that ran
+// (any may be a null view): distortion image, median depth, and a pixel weight map to accumulate
+// per splat (the reference feeds these from its loss, src/engine/EngineLoss.cpp:138-216).
+void engine_backward_with_variants(TorchTensorView v_render_rgb, TorchTensorView v_render_depth, TorchTensorView v_render_Ts,
+                                   TorchTensorView v_dist_rgb, TorchTensorView v_dist_depth, TorchTensorView v_median,
+                                   TorchTensorView accum_map, int accum_mode);
 void engine_copy_params_to_host(TorchTensorView means, TorchTensorView quats, TorchTensorView scales,
                                 TorchTensorView opacities, TorchTensorView features_dc, TorchTensorView features_sh);
 void engine_copy_render_to_host(TorchTensorView out_rgb, TorchTensorView out_depth, TorchTensorView out_Ts,

@@ -25,8 +25,8 @@ static_assert(sizeof(float3) == 12 && sizeof(float4) == 16 && alignof(float4) ==
 // (data_ptr, element_size, shape): host or device memory, decided by the address
 typedef std::tuple<uint64_t, uint32_t, std::vector<int64_t>> TorchTensorView;
 
-enum class DistortionType : int { None = 0, D = 1, RGB_D = 2, DN = 3 };
-enum class DensifyAccumMode : int { None = 0, Sum = 1, Max = 2, Avg = 3 };
+enum class DistortionType : int { None = 0, D = 1, RGB_D = 2, DN = 3, RGB_DN = 4 };   // src/primitives/Primitive.cuh:24-26
+enum class DensifyAccumMode : int { None = 0, Max = 1, Sum = 2, Avg = 3 };        // src/primitives/Primitive.cuh:37-39
 
 namespace backend {
 enum class MemcpyKind { HostToDevice, DeviceToHost, DeviceToDevice, Auto };
@@ -67,7 +67,8 @@ enum class PoolSlot : int {
     IsectTileActive, EngTileMask,
     AdamG1Means, AdamG1Quats, AdamG1Scales, AdamG1Opacities, AdamG1FeaturesDc, AdamG1FeaturesSh,
     AdamG2Means, AdamG2Quats, AdamG2Scales, AdamG2Opacities, AdamG2FeaturesDc, AdamG2FeaturesSh, EngDensifyScore, ProjCameraIds, ProjGaussianIds, ProjGaussianIdsB, ProjPackedScratch, ProjPackedNnz,
-    RendersRgb, RendersDepth, RenderTs, RenderLastIds,
+    RendersRgb, RendersDepth, RenderTs, RenderLastIds, RenderDistortionRgb, RenderDistortionDepth, RenderMedian,
+    RasterBwdAccumWeight, EngVDistRgb, EngVDistDepth, EngVMedian, EngAccumMap,
     RasterBwdVScreenXy, RasterBwdVScreenDepth, RasterBwdVScreenConic, RasterBwdVScreenOpac, RasterBwdVScreenRgb,
     EngVRgb, EngVDepth, EngVTs,
     GradMeans, GradQuats, GradScales, GradOpacities, GradFeaturesDc, GradFeaturesSh,

@@ -50,7 +50,8 @@ class RasterFwdParams(C.Structure):
     _fields_ = [("num_splats", C.c_int64), ("screen", Screen), ("width", C.c_uint32),
                 ("height", C.c_uint32), ("tile_offsets", vp), ("flatten_ids", vp),
                 ("n_isects", C.c_int64), ("render_rgb", vp), ("render_depth", vp),
-                ("render_T", vp), ("last_ids", vp), ("packed_rows", vp)]
+                ("render_T", vp), ("last_ids", vp), ("packed_rows", vp), ("dist_type", C.c_int32),
+                ("distortion_rgb", vp), ("distortion_depth", vp), ("render_median", vp)]
 
 
 class RasterBwdParams(C.Structure):
@@ -58,7 +59,10 @@ class RasterBwdParams(C.Structure):
                 ("height", C.c_uint32), ("tile_offsets", vp), ("flatten_ids", vp),
                 ("n_isects", C.c_int64), ("render_T", vp), ("last_ids", vp), ("render_depth", vp),
                 ("v_render_rgb", vp), ("v_render_depth", vp), ("v_render_T", vp),
-                ("v_screen", Screen), ("packed_rows", vp)]
+                ("v_screen", Screen), ("packed_rows", vp), ("dist_type", C.c_int32), ("render_rgb", vp),
+                ("distortion_rgb", vp), ("distortion_depth", vp), ("v_distortion_rgb", vp),
+                ("v_distortion_depth", vp), ("v_render_median", vp), ("accum_mode", C.c_int32),
+                ("accum_weight_map", vp), ("gaussian_ids", vp), ("num_world", C.c_int64), ("accum_weight", vp)]
 
 
 class ProjectionBwdParams(C.Structure):

@@ -52,6 +52,9 @@ class GpuRun:
         self.V = None
         self.rows = n          # rows of the projection outputs: N, or nnz in packed mode
         self.tile_active = None   # device tile-skip map (set_tile_mask)
+        # variants of the compositing kernels: dict(dist_type=, median=bool, v_dist_rgb=, v_dist_depth=,
+        # v_median=, accum_mode=, accum_map=)
+        self.variant = {}
 
     def ptr(self, k):
         a = self.d.get(k)
@@ -214,6 +217,17 @@ class GpuRun:
         if self.use_packed:
             p.packed_rows = self.ptr("packed")
             p.screen = self.L.Screen()   # not read
+        va = self.variant
+        p.dist_type = va.get("dist_type", 0)
+        if p.dist_type:
+            self.d["r_dist_depth"] = D((h, w), np.float32)
+            p.distortion_depth = self.ptr("r_dist_depth")
+            if p.dist_type == 2:
+                self.d["r_dist_rgb"] = D((h, w, 3), np.float32)
+                p.distortion_rgb = self.ptr("r_dist_rgb")
+        if va.get("median"):
+            self.d["r_median"] = D((h, w), np.float32)
+            p.render_median = self.ptr("r_median")
         self.check(self.lib.ssr_raster_fwd(C.byref(p), None))
 
     def raster_bwd(self, v_rgb=None, v_depth=None, v_T=None):
@@ -235,6 +249,26 @@ class GpuRun:
         if self.use_packed:
             p.packed_rows = self.ptr("packed")
             p.screen = self.L.Screen()
+        va = self.variant
+        f32 = lambda a: D.from_host(np.ascontiguousarray(a, np.float32))
+        p.dist_type = va.get("dist_type", 0)
+        if p.dist_type:
+            self.d["g_dist_depth"] = f32(va["v_dist_depth"])
+            p.distortion_depth, p.v_distortion_depth = self.ptr("r_dist_depth"), self.ptr("g_dist_depth")
+            if p.dist_type == 2:
+                self.d["g_dist_rgb"] = f32(va["v_dist_rgb"])
+                p.render_rgb, p.distortion_rgb, p.v_distortion_rgb = self.ptr("r_rgb"), self.ptr("r_dist_rgb"), self.ptr("g_dist_rgb")
+        if va.get("median"):
+            self.d["g_median"] = f32(va["v_median"])
+            p.v_render_median = self.ptr("g_median")
+        p.accum_mode = va.get("accum_mode", 0)
+        if p.accum_mode:
+            self.d["accum_map"] = f32(va["accum_map"])
+            self.d["accum_weight"] = D((self.n * (2 if p.accum_mode == 3 else 1),), np.float32)
+            self.d["accum_weight"].fill_zero()
+            p.accum_weight_map, p.accum_weight, p.num_world = self.ptr("accum_map"), self.ptr("accum_weight"), self.n
+            if self.packed_projection:
+                p.gaussian_ids = self.ptr("gaussian_ids")
         self.check(self.lib.ssr_raster_bwd(C.byref(p), None))
 
     def projection_bwd(self, accumulate=True, poison=False):

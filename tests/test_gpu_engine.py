@@ -242,14 +242,55 @@ def test_engine_fused_optimizer_training_steps(pkg, oracle, H):
     assert np.abs(rgb - r["fwd"]["rgb"]).max() < 0.02
 
 
+@pytest.mark.parametrize("packed", [False, True])
+def test_engine_compositing_variants(pkg, oracle, H, packed):
+    """forward_3dgs(output_median, dist_type) and a backward fed the distortion / median cotangents and
+    a pixel weight map to accumulate per splat (indexed by world row also in packed mode)."""
+    host, lib = H
+    sc = pkg.scenes.make_scene(1, n=20000, width=240, height=160, parity_variant=True)
+    sc.means[::3, 2] = -10.0
+    rng = np.random.default_rng(5)
+    h, w = sc.height, sc.width
+    cot = dict(v_dist_rgb=rng.uniform(-1, 1, (h, w, 3)).astype(np.float32), v_dist_depth=rng.uniform(-1, 1, (h, w)).astype(np.float32),
+               v_median=rng.uniform(-1, 1, (h, w)).astype(np.float32), accum_map=rng.uniform(0, 1, (h, w)).astype(np.float32))
+    va = dict(dist_type=2, median=False, accum_mode=3, **cot)
+    eng = host.Engine(sc, packed_projection=packed)
+    eng.set_variants(dist_type=2, median=True)
+    eng.forward()
+    eng.backward_with_variants(cot["v_dist_rgb"], cot["v_dist_depth"], None, cot["accum_map"], accum_mode=3)
+    # oracle: unpacked chain; packing only renumbers rows, the accumulated weights are per world row
+    r = oracle.pipeline(sc, variant=va)
+    rm = oracle.pipeline(sc, backward=False, variant=dict(median=True))
+    assert np.abs(eng.cache("dist_rgb").reshape(h, w, 3) - r["fwd"]["dist_rgb"]).max() <= 1e-4
+    assert np.abs(eng.cache("dist_depth").reshape(h, w) - r["fwd"]["dist_depth"]).max() <= 1e-4
+    med = rm["fwd"]["median"]
+    assert (np.abs(eng.cache("median").reshape(h, w) - med) <= 1e-4 * np.maximum(1, np.abs(med))).all()
+    rgb, depth, T = eng.render()
+    assert (np.abs(depth - r["fwd"]["depth"]) <= 1e-4 * np.maximum(1, r["fwd"]["depth"])).all()
+    aw = eng.cache("accum_weight")
+    assert aw.size == 2 * sc.n
+    assert np.allclose(aw, r["vscreen"]["accum_weight"], rtol=1e-3, atol=1e-6) and (aw[:sc.n] > 0).sum() > 100
+    g = eng.grads()
+    for k, v in g.items():
+        ref = r["grads"][k].astype(np.float64).reshape(sc.n, -1)
+        scale = np.abs(ref).max(axis=1, keepdims=True)
+        err = np.abs(v.reshape(sc.n, -1) - ref)
+        assert (err <= 2e-3 * scale + 2e-5 * (np.abs(ref).mean() + 1e-12)).all(), k
+    # a forward with distortion needs its cotangent in the backward
+    assert eng.h.ssrh_backward_from_render_grad(eng.d_vrgb.ptr, eng.d_vdepth.ptr, eng.d_vT.ptr) != 0
+    assert b"distortion" in eng.h.ssrh_last_error()
+
+
 def test_unsupported_variants_raise(pkg, H):
     host, lib = H
     sc = pkg.scenes.tiny_scene(n=50, width=32, height=32)
     eng = host.Engine(sc)
     h = host.load()
-    for args in [(b"3dgut", 3, 0, 0, 0), (b"3dgs", 3, 0, 1, 0), (b"3dgs", 3, 0, 0, 1)]:
-        assert h.ssrh_forward_3dgs(*args) != 0
-        assert b"not built" in h.ssrh_last_error()
+    assert h.ssrh_forward_3dgs(b"3dgut", 3, 0, 0, 0) != 0
+    assert b"not built" in h.ssrh_last_error()
+    for dist in (3, 4):   # DN, RGB_DN: the 3dgs pixel has no normal channel
+        assert h.ssrh_forward_3dgs(b"3dgs", 3, 0, 0, dist) != 0
+        assert b"normal" in h.ssrh_last_error()
     assert h.ssrh_set_camera_params(32, 32, b"FISHEYE", b"NONE", None, None, 1) == 0
     assert h.ssrh_forward_3dgs(b"3dgs", 3, 0, 0, 0) != 0
     assert b"FISHEYE" in h.ssrh_last_error()
