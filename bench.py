@@ -96,6 +96,9 @@ def main():
     ap.add_argument("--fused-optimizer", action="store_true",
                     help="backward = compositing backward + projection backward fused with the Adam step "
                          "(the reference's FPBO mode); K9 then includes the optimizer's 1.4 kB/splat of traffic")
+    ap.add_argument("--dist-type", type=int, default=0, help="compositing variant: 1 depth distortion, 2 rgb + depth distortion")
+    ap.add_argument("--median", action="store_true", help="compositing variant: also render the median depth and back-propagate it")
+    ap.add_argument("--accum-mode", type=int, default=0, help="compositing variant: accumulate a pixel weight map per splat (1 max, 2 sum, 3 avg)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run device copies / fills of known size (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE) and exit")
     args = ap.parse_args()
@@ -133,15 +136,27 @@ def main():
     hyper = dict(lr_means=1.6e-6, lr_quats=1e-5, lr_scales=5e-5, lr_opacs=5e-4, lr_features_dc=2.5e-5, lr_features_sh=1.25e-6)
     adam_step = [0]
 
+    variants = args.dist_type or args.median or args.accum_mode
+    if variants:
+        rng = np.random.default_rng(1)
+        eng.set_variants(args.dist_type, args.median)
+        u = lambda *shape: lib.DeviceArray.from_host(rng.uniform(-1, 1, shape).astype(np.float32))
+        vcot = dict(rgb=u(sc.height, sc.width, 3), depth=u(sc.height, sc.width), med=u(sc.height, sc.width),
+                    amap=lib.DeviceArray.from_host(rng.uniform(0, 1, (sc.height, sc.width)).astype(np.float32)))
+
     def backward():
-        if args.fused_optimizer:
+        if variants:
+            host.check(eng.h.ssrh_backward_with_variants(eng.d_vrgb.ptr, eng.d_vdepth.ptr, eng.d_vT.ptr, vcot["rgb"].ptr,
+                                                         vcot["depth"].ptr, vcot["med"].ptr if args.median else None,
+                                                         vcot["amap"].ptr if args.accum_mode else None, args.accum_mode))
+        elif args.fused_optimizer:
             adam_step[0] += 1
             eng.backward_fused_optimizer(hyper, adam_step[0])
         else:
             eng.backward()
 
     def run(iters):
-        if not args.fused_optimizer:
+        if not (args.fused_optimizer or variants):
             return eng.time_iterations(iters)
         out = np.zeros(iters, np.float32)
         for i in range(iters):
@@ -206,7 +221,8 @@ def main():
                    "visible": V, "n_isects": K, "K_b": K_b, "tiles": T, "pixels": P,
                    "stage_order": ("fused tile count, visible-splat work list, packed fragment rows, plain-store gradients" if native else "reference order")
                                   + (", packed projection outputs" if args.packed_projection else "")
-                                  + (", projection backward fused with Adam" if args.fused_optimizer else ""),
+                                  + (", projection backward fused with Adam" if args.fused_optimizer else "")
+                                  + (f", compositing variants dist_type={args.dist_type} median={int(args.median)} accum_mode={args.accum_mode}" if variants else ""),
                    "device_ms_per_iter_median": float(np.median(ms))},
         "hbm_roofline_frac_whole_iteration": total_bytes / (float(np.median(ms)) * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "algorithmic_bytes_per_iter": total_bytes,

@@ -79,6 +79,8 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
     __shared__ FragLds frags[kBatch];
     __shared__ int32_t s_ids[kBatch];
     __shared__ int s_wave_max[4];
+    // distortion composites ln(max(z, 1e-6)): a per-splat value, taken once when the fragment is staged
+    [[maybe_unused]] __shared__ float s_lz[kDist != SSR_DIST_NONE ? kBatch : 1];
     const int n_tiles = tile_w * tile_h;
     const int tile = xcd_tile_of(blockIdx.x, n_tiles);
     if (tile >= n_tiles) return;
@@ -153,6 +155,8 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
     if (sub == 0) chan = row == 0 ? 0 : row == 1 ? 2 : row == 2 ? 1 : 3;
     else if (sub == 1) chan = row == 0 ? 4 : row == 1 ? 6 : row == 2 ? 5 : 7;
     else if (sub == 2 && (row & 1) == 0) chan = row == 0 ? 8 : 9;
+    else if (sub == 2 && (kAccum == SSR_ACCUM_SUM || kAccum == SSR_ACCUM_AVG) && (row == 1 || kAccum == SSR_ACCUM_AVG))
+        chan = row == 1 ? 10 : 11;   // the weight sums ride in the two spare rows of the third register
     float* abase = nullptr;
     int astride = 0;
     switch (chan) {
@@ -166,6 +170,8 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
         case 7: abase = P.v_screen.rgb; astride = 3; break;
         case 8: abase = P.v_screen.rgb + 1; astride = 3; break;
         case 9: abase = P.v_screen.rgb + 2; astride = 3; break;
+        case 10: abase = P.accum_weight; astride = 1; break;
+        case 11: abase = P.accum_weight + P.num_world; astride = 1; break;
         default: break;
     }
 
@@ -176,6 +182,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
             const int32_t g = P.flatten_ids[idx];
             s_ids[tid] = g;
             frags[tid] = stage_fragment(P.screen, P.packed_rows, g, tile_x0, tile_y0);
+            if constexpr (kDist != SSR_DIST_NONE) s_lz[tid] = ssr_log(ssr_max(frags[tid].q2.y, 1e-6f));
         } else {
             frags[tid].q2 = make_float4(0.f, 0.f, 0.f, 0.f);
         }
@@ -221,7 +228,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
                         pend_Tfar = T1;
                     }
                 }
-                if constexpr (kDist != SSR_DIST_NONE) cdp = ssr_log(ssr_max(q2.y, 1e-6f));
+                if constexpr (kDist != SSR_DIST_NONE) cdp = s_lz[k];
                 float dv = ssr_fma(cdp, vd, ssr_fma(cb, vb, ssr_fma(cg, vg, cr * vr))) - vT1;
                 const float w = a * T0;
                 [[maybe_unused]] float xr = 0.f, xg = 0.f, xb = 0.f, xd = 0.f;   // distortion part of the colour gradient
@@ -256,18 +263,12 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
                     t_d = (t_d + xd) * (1.0f / ssr_max(q2.y, 1e-6f));   // d/d ln z -> d/dz
                 }
                 if constexpr (kMedian) t_d += v_depth_median;
+                [[maybe_unused]] int64_t wid = 0;
                 if constexpr (kAccum != SSR_ACCUM_NONE) {   // :553-562,574-585
-                    const int64_t wid = P.gaussian_ids ? (int64_t)P.gaussian_ids[s_ids[k]] : (int64_t)s_ids[k];
+                    wid = P.gaussian_ids ? (int64_t)P.gaussian_ids[s_ids[k]] : (int64_t)s_ids[k];
                     if constexpr (kAccum == SSR_ACCUM_MAX) {
                         const float mx = wave_max_f32(amap * w);   // inactive lanes contribute map * 0; the running max starts at 0
                         if (lane == 0) atomic_max_f32(P.accum_weight + wid, ssr_max(mx, 0.0f));
-                    } else {
-                        const float sm = wave_sum_f32(amap * w);
-                        if (lane == 0 && sm != 0.0f) atomicAdd(P.accum_weight + wid, sm);
-                        if constexpr (kAccum == SSR_ACCUM_AVG) {
-                            const float dn = wave_sum_f32(w);
-                            if (lane == 0 && dn != 0.0f) atomicAdd(P.accum_weight + P.num_world + wid, dn);
-                        }
                     }
                 }
                 // transposing reduction: 10 channels -> 3 registers with one channel per row
@@ -275,10 +276,19 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
                             rd_ = fold32(t_o, t_r), re_ = fold32(t_g, t_b);
                 const float s1 = row_sum(fold16(ra_, rb_));   // rows: x, d, y, ca      -> channels 0,2,1,3
                 const float s2 = row_sum(fold16(rc_, rd_));   // rows: cb, o, cc, r     -> channels 4,6,5,7
-                const float s3 = row_sum(fold16(re_, re_));   // rows: g, g, b, b       -> channels 8,8,9,9
+                float s3;
+                if constexpr (kAccum == SSR_ACCUM_SUM || kAccum == SSR_ACCUM_AVG) {
+                    // the weight sums ride in the two spare rows of the third register
+                    const float rf_ = fold32(amap * w, w);
+                    s3 = row_sum(fold16(re_, rf_));           // rows: g, sum map w, b, sum w -> channels 8,10,9,11
+                } else {
+                    s3 = row_sum(fold16(re_, re_));           // rows: g, g, b, b       -> channels 8,8,9,9
+                }
                 float mine = sub == 0 ? s1 : (sub == 1 ? s2 : s3);
+                uint32_t dst_row = (uint32_t)s_ids[k];
+                if constexpr (kAccum == SSR_ACCUM_SUM || kAccum == SSR_ACCUM_AVG) { if (chan >= 10) dst_row = (uint32_t)wid; }
                 if (chan >= 0 && ssr_isfinite(mine) && mine != 0.0f)
-                    atomicAdd(abase + (uint32_t)astride * (uint32_t)s_ids[k], mine);   // < 2^32 elements per array
+                    atomicAdd(abase + (uint32_t)astride * dst_row, mine);   // < 2^32 elements per array
             }
         }
     }

@@ -15,6 +15,8 @@ namespace ssr {
 template <int kDist, bool kMedian>
 __global__ __launch_bounds__(kRasterBlock) void raster_fwd_kernel(ssr_raster_fwd_params P, int tile_w, int tile_h) {
     __shared__ FragLds frags[kBatch];
+    // distortion composites ln(max(z, 1e-6)): a per-splat value, taken once when the fragment is staged
+    [[maybe_unused]] __shared__ float s_lz[kDist != SSR_DIST_NONE ? kBatch : 1];
     const int n_tiles = tile_w * tile_h;
     const int tile = xcd_tile_of(blockIdx.x, n_tiles);
     if (tile >= n_tiles) return;   // whole workgroup leaves together
@@ -41,6 +43,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_kernel(ssr_raster_fwd
         const int32_t idx = batch_start + tid;
         if (idx < range_end) {
             frags[tid] = stage_fragment(P.screen, P.packed_rows, P.flatten_ids[idx], tile_x0, tile_y0);
+            if constexpr (kDist != SSR_DIST_NONE) s_lz[tid] = ssr_log(ssr_max(frags[tid].q2.y, 1e-6f));
         } else {
             frags[tid].q2 = make_float4(0.f, 0.f, 0.f, 0.f);   // empty footprint mask
         }
@@ -72,7 +75,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_kernel(ssr_raster_fwd
                         const float w = alpha * T;
                         float zd = q2.y;
                         if constexpr (kDist != SSR_DIST_NONE) {
-                            zd = ssr_log(ssr_max(q2.y, 1e-6f));
+                            zd = s_lz[k];
                             if constexpr (kDist == SSR_DIST_RGB_D) {
                                 s2r = ssr_fma(q1.z * q1.z, w, s2r); s2g = ssr_fma(q1.w * q1.w, w, s2g);
                                 s2b = ssr_fma(q2.x * q2.x, w, s2b);
