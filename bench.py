@@ -130,7 +130,7 @@ def main():
     t_gen = time.time() - t_gen
     native = not args.reference_order
     eng = host.Engine(sc, fuse_tile_count=native, visible_list=native and not args.packed_projection, packed_rows=native,
-                      overwrite_world_grads=native, packed_projection=args.packed_projection)
+                      overwrite_world_grads=native, packed_projection=args.packed_projection, packed_vscreen=native)
     L = lib.load()
 
     hyper = dict(lr_means=1.6e-6, lr_quats=1e-5, lr_scales=5e-5, lr_opacs=5e-4, lr_features_dc=2.5e-5, lr_features_sh=1.25e-6)
@@ -219,7 +219,7 @@ def main():
                                f"{'pinhole' if sc.camera_model == 0 else 'equirectangular'}, SH3 "
                                f"{['fp32', 'ref-q8', 'ref-q16', 'int8*fp16scale'][sc.sh_codec]}, tile 16x16, seed {pkg.scenes.CONFIGS[cfg]['seed']:#x}",
                    "visible": V, "n_isects": K, "K_b": K_b, "tiles": T, "pixels": P,
-                   "stage_order": ("fused tile count, visible-splat work list, packed fragment rows, plain-store gradients" if native else "reference order")
+                   "stage_order": ("fused tile count, visible-splat work list, packed fragment rows, packed gradient rows, plain-store gradients" if native else "reference order")
                                   + (", packed projection outputs" if args.packed_projection else "")
                                   + (", projection backward fused with Adam" if args.fused_optimizer else "")
                                   + (f", compositing variants dist_type={args.dist_type} median={int(args.median)} accum_mode={args.accum_mode}" if variants else ""),

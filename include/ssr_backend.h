@@ -236,6 +236,12 @@ typedef struct {
     const float* v_render_T;      /* [H,W] */
     ssr_screen v_screen;          /* accumulated into */
     const float* packed_rows;     /* optional, as in ssr_raster_fwd_params */
+    /* Optional [num_splats,12] (16-byte aligned, caller zero-fills): the ten gradient channels of a
+     * splat as ONE row (x, y, depth, conic[3], opac, rgb[3], 2 pad) instead of five arrays, so that
+     * its atomics land in one or two cache lines instead of five. When given, v_screen is not
+     * written; ssr_projection_bwd / ssr_fused_projection_bwd_optimizer read the rows through their
+     * own v_rows field. No counterpart in the reference. */
+    float* v_rows;
     /* Variants (RasterizationEval3DBwd_kernel.cuh:150-172,207-279,433-585). With dist_type set:
      * render_rgb and distortion_* are the forward's outputs, v_distortion_* the cotangents of the
      * distortion image. v_render_median non-NULL: cotangent of the median depth. accum_mode
@@ -283,6 +289,7 @@ typedef struct {
      * num_packed == 0 with the pointer set is a no-op (ProjectionBwd.cu:89-97). */
     const int32_t* packed_gaussian_ids;
     int64_t num_packed;
+    const float* v_rows;    /* optional: ssr_raster_bwd's row output; when given, v_screen is not read */
 } ssr_projection_bwd_params;
 int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream_t stream);
 
@@ -306,6 +313,7 @@ typedef struct {
     ssr_camera camera;
     const float* aabb;          /* [N,4] of the forward */
     ssr_screen v_screen;        /* read: output of ssr_raster_bwd */
+    const float* v_rows;        /* optional: ssr_raster_bwd's row output; when given, v_screen is not read */
     ssr_world v_world_in;       /* optional gradient contributions already accumulated (any member may
                                    be NULL = zero; features_sh is not read, as in the reference) */
     ssr_world g1, g2;           /* Adam first / second moments, same shapes as world, updated in place */

@@ -327,9 +327,20 @@ __device__ __forceinline__ void put(float* p, float v) {
 // factors of the gradient of SH coefficient j (j < kDegree (kDegree + 2)), which is Yj * vc[0..2].
 struct WorldGradD { float mean[3], quat[4], scale[3], logit, dc[3]; };
 
+// Where the screen-space gradient of row r lives: five arrays (the reference's layout) or one
+// 12-float row per splat (x, y, depth, conic[3], opac, rgb[3], pad[2]) written by the compositing backward.
+struct VScreenD {
+    const float *xy, *depth, *conic, *opac, *rgb;
+    int s_xy, s_depth, s_conic, s_opac, s_rgb;   // floats between consecutive rows
+};
+__device__ __forceinline__ VScreenD vscreen_of(const ssr_screen& s, const float* rows) {
+    if (rows) return VScreenD{rows, rows + 2, rows + 3, rows + 6, rows + 7, 12, 12, 12, 12, 12};
+    return VScreenD{s.xy, s.depth, s.conic, s.opac, s.rgb, 2, 1, 3, 1, 3};
+}
+
 template <int kDegree, class ShSink>
 __device__ __forceinline__ void projection_vjp(const CamD& cam, const ssr_world& W, const ssr_sh_quant& Q, int64_t g,
-                                               const ssr_screen& VS, int64_t r, WorldGradD& out, ShSink&& sh_sink) {
+                                               const VScreenD& VS, int64_t r, WorldGradD& out, ShSink&& sh_sink) {
     constexpr int kCoef = kDegree * (kDegree + 2);
     float mean[3], quat[4], ls[3], logit;
     load_splat(W, g, mean, quat, ls, logit);
@@ -340,7 +351,7 @@ __device__ __forceinline__ void projection_vjp(const CamD& cam, const ssr_world&
     // conic = inverse(cov2d)
     const float c00 = p.c2[0][0], c01 = p.c2[0][1], c10 = p.c2[1][0], c11 = p.c2[1][1];
     const float det = c00 * c11 - c01 * c10, inv = 1.0f / det;
-    const float* vcn = VS.conic + 3 * r;
+    const float* vcn = VS.conic + VS.s_conic * r;
     const float g00 = vcn[0], g01 = vcn[1], g11 = vcn[2];
     const float v_inv = (c11 * g00 - c01 * g01) + c00 * g11;
     const float v_det = -(v_inv / (det * det));
@@ -374,7 +385,7 @@ __device__ __forceinline__ void projection_vjp(const CamD& cam, const ssr_world&
                 for (int j = 0; j < 2; j++) s += p.J[i][k] * vC[i][j] * p.J[j][l];
             vS[k][l] = s;
         }
-    const float vm0 = VS.xy[2 * r], vm1 = VS.xy[2 * r + 1];
+    const float vm0 = VS.xy[VS.s_xy * r], vm1 = VS.xy[VS.s_xy * r + 1];
     if (cam.model == SSR_CAM_PINHOLE) {
         const float z2 = z * z, iz = 1.0f / z, iz2 = 1.0f / z2;
         vmc[2] += vJ[0][0] * (-cam.fx * iz2) + vJ[1][1] * (-cam.fy * iz2);
@@ -413,7 +424,7 @@ __device__ __forceinline__ void projection_vjp(const CamD& cam, const ssr_world&
     }
     {   // depth = length(mean_c); the sqrt derivative is guarded at 1e-7
         const float s2 = dot3(p.mc, p.mc);
-        const float vs = VS.depth[r] * (0.5f / ssr_sqrt(ssr_max(1e-7f, s2)));
+        const float vs = VS.depth[VS.s_depth * r] * (0.5f / ssr_sqrt(ssr_max(1e-7f, s2)));
 #pragma unroll
         for (int i = 0; i < 3; i++) vmc[i] += 2.0f * p.mc[i] * vs;
     }
@@ -461,7 +472,7 @@ __device__ __forceinline__ void projection_vjp(const CamD& cam, const ssr_world&
     float vquat[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) vquat[i] = (vqn[i] - p.qn[i] * qd) * p.qinv;
-    const float vlogit = VS.opac[r] * (p.opac * (1.0f - p.opac));
+    const float vlogit = VS.opac[VS.s_opac * r] * (p.opac * (1.0f - p.opac));
 
     // SH colour VJP (src/shaders/harmonics.slang:373-649,1087-1126)
     float coef[kCoef > 0 ? 3 * kCoef : 1];
@@ -474,7 +485,7 @@ __device__ __forceinline__ void projection_vjp(const CamD& cam, const ssr_world&
     const float dc[3] = {dcp[0], dcp[1], dcp[2]};
     float raw[3];
     sh_color_raw<kDegree>(b, dc, coef, raw);
-    const float* vrg = VS.rgb + 3 * r;
+    const float* vrg = VS.rgb + VS.s_rgb * r;
     float vc[3];
 #pragma unroll
     for (int c = 0; c < 3; c++) vc[c] = vrg[c] * (raw[c] >= -0.5f ? 1.0f : 0.0f);
@@ -558,7 +569,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
     const CamD cam = load_camera(P.camera);
     WorldGradD wg;
     float* vsh = V.features_sh + g * (int64_t)V.sh_stride;
-    projection_vjp<kDegree>(cam, P.world, P.sh, g, P.v_screen, r, wg, [&](int j, float Yj, const float vc[3]) {
+    projection_vjp<kDegree>(cam, P.world, P.sh, g, vscreen_of(P.v_screen, P.v_rows), r, wg, [&](int j, float Yj, const float vc[3]) {
         const float tv[3] = {Yj * vc[0], Yj * vc[1], Yj * vc[2]};
         const float d2 = dot3(tv, tv);
         const bool ok = ssr_isfinite(d2) && d2 != 0.0f;   // harmonics.slang:397-403
@@ -639,7 +650,7 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
             ssr_sh_quant none;
             none.codec = SSR_SH_F32; none.packed = nullptr; none.bounds = nullptr; none.bounds_stride = 0;
             none.num_sh_buffer = 0; none.scale_f16 = nullptr;
-            projection_vjp<kDegree>(cam, W, none, g, P.v_screen, g, pg, [&](int j, float Yj, const float vc[3]) {
+            projection_vjp<kDegree>(cam, W, none, g, vscreen_of(P.v_screen, P.v_rows), g, pg, [&](int j, float Yj, const float vc[3]) {
                 s_Y[threadIdx.x][j] = Yj;
                 if (j == 0) { s_vc[threadIdx.x][0] = vc[0]; s_vc[threadIdx.x][1] = vc[1]; s_vc[threadIdx.x][2] = vc[2]; }
             });
@@ -888,7 +899,7 @@ extern "C" int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream
     } else {
         SSR_REQUIRE(p->aabb, "ssr_projection_bwd", "null aabb");   // ProjectionBwd.cu:89-97
     }
-    SSR_REQUIRE(p->v_screen.xy && p->v_screen.depth && p->v_screen.conic && p->v_screen.opac && p->v_screen.rgb,
+    SSR_REQUIRE(p->v_rows || (p->v_screen.xy && p->v_screen.depth && p->v_screen.conic && p->v_screen.opac && p->v_screen.rgb),
                 "ssr_projection_bwd", "null v_screen buffer");
     const ssr_world& v = p->v_world;
     SSR_REQUIRE(v.means && v.quats && v.log_scales && v.opacity_logits && v.features_dc && v.features_sh,
@@ -926,7 +937,7 @@ extern "C" int ssr_fused_projection_bwd_optimizer(const ssr_fpbo_params* p, ssr_
     if (e) return e;
     if (p->num_splats == 0) return 0;
     SSR_REQUIRE(p->aabb && (reinterpret_cast<uintptr_t>(p->aabb) & 15) == 0, where, "aabb must be non-null and 16-byte aligned");
-    SSR_REQUIRE(p->v_screen.xy && p->v_screen.depth && p->v_screen.conic && p->v_screen.opac && p->v_screen.rgb, where,
+    SSR_REQUIRE(p->v_rows || (p->v_screen.xy && p->v_screen.depth && p->v_screen.conic && p->v_screen.opac && p->v_screen.rgb), where,
                 "null v_screen buffer");
     for (const ssr_world* w : {&p->world, &p->g1, &p->g2}) {
         SSR_REQUIRE(w->means && w->quats && w->log_scales && w->opacity_logits && w->features_dc, where, "null parameter or moment buffer");

@@ -79,6 +79,11 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
     __shared__ FragLds frags[kBatch];
     __shared__ int32_t s_ids[kBatch];
     __shared__ int s_wave_max[4];
+    // Per-fragment gradient sums of the whole tile: the four wavefronts (sub-tiles) add their reduced
+    // sums here with LDS atomics, and each staged fragment goes to global memory once per batch --
+    // one set of global atomics per (splat, tile) instead of one per (splat, sub-tile).
+    constexpr int kAccCh = (kAccum == SSR_ACCUM_SUM || kAccum == SSR_ACCUM_AVG) ? 12 : 10;
+    __shared__ float s_acc[kBatch * kAccCh];
     // distortion composites ln(max(z, 1e-6)): a per-splat value, taken once when the fragment is staged
     [[maybe_unused]] __shared__ float s_lz[kDist != SSR_DIST_NONE ? kBatch : 1];
     const int n_tiles = tile_w * tile_h;
@@ -157,26 +162,60 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
     else if (sub == 2 && (row & 1) == 0) chan = row == 0 ? 8 : 9;
     else if (sub == 2 && (kAccum == SSR_ACCUM_SUM || kAccum == SSR_ACCUM_AVG) && (row == 1 || kAccum == SSR_ACCUM_AVG))
         chan = row == 1 ? 10 : 11;   // the weight sums ride in the two spare rows of the third register
-    float* abase = nullptr;
-    int astride = 0;
-    switch (chan) {
-        case 0: abase = P.v_screen.xy; astride = 2; break;
-        case 1: abase = P.v_screen.xy + 1; astride = 2; break;
-        case 2: abase = P.v_screen.depth; astride = 1; break;
-        case 3: abase = P.v_screen.conic; astride = 3; break;
-        case 4: abase = P.v_screen.conic + 1; astride = 3; break;
-        case 5: abase = P.v_screen.conic + 2; astride = 3; break;
-        case 6: abase = P.v_screen.opac; astride = 1; break;
-        case 7: abase = P.v_screen.rgb; astride = 3; break;
-        case 8: abase = P.v_screen.rgb + 1; astride = 3; break;
-        case 9: abase = P.v_screen.rgb + 2; astride = 3; break;
-        case 10: abase = P.accum_weight; astride = 1; break;
-        case 11: abase = P.accum_weight + P.num_world; astride = 1; break;
-        default: break;
-    }
+#pragma unroll
+    for (int c = 0; c < kAccCh; c++) s_acc[tid * kAccCh + c] = 0.0f;
+    // Thread t owns fragment slot t: it moves that slot's sums to global memory (zeros skipped, as in
+    // src/core/Common.cuh:791-856) and clears them. Called between two barriers.
+    auto flush_slot = [&]() {
+        if (P.v_rows) {
+            // all 256 slots x 10 channels in memory order of the destination rows: the lanes of one
+            // instruction cover whole rows, so a row's atomics travel as one or two requests
+            __syncthreads();   // slot owners differ from readers here: wait for every wavefront's sums
+            for (int e = tid; e < kBatch * 10; e += kRasterBlock) {
+                const int slot = e / 10, ch = e - slot * 10;
+                const float x = s_acc[slot * kAccCh + ch];
+                if (x != 0.0f) {
+                    s_acc[slot * kAccCh + ch] = 0.0f;
+                    atomicAdd(P.v_rows + 12u * (uint32_t)s_ids[slot] + (uint32_t)ch, x);
+                }
+            }
+            if constexpr (kAccCh == 12) {
+                const float a = s_acc[tid * kAccCh + 10], b = s_acc[tid * kAccCh + 11];
+                if (a != 0.0f || b != 0.0f) {
+                    s_acc[tid * kAccCh + 10] = 0.0f; s_acc[tid * kAccCh + 11] = 0.0f;
+                    const uint32_t g = (uint32_t)s_ids[tid];
+                    const int64_t wid = P.gaussian_ids ? (int64_t)P.gaussian_ids[g] : (int64_t)g;
+                    if (a != 0.0f) atomicAdd(P.accum_weight + wid, a);
+                    if (kAccum == SSR_ACCUM_AVG && b != 0.0f) atomicAdd(P.accum_weight + P.num_world + wid, b);
+                }
+            }
+            __syncthreads();   // s_ids and s_acc are free for the next batch
+            return;
+        }
+        float v[kAccCh];
+        bool any = false;
+#pragma unroll
+        for (int c = 0; c < kAccCh; c++) { v[c] = s_acc[tid * kAccCh + c]; any |= v[c] != 0.0f; }
+        if (!any) return;
+#pragma unroll
+        for (int c = 0; c < kAccCh; c++) s_acc[tid * kAccCh + c] = 0.0f;
+        const uint32_t g = (uint32_t)s_ids[tid];   // < 2^30 rows, so every index below fits 32 bits
+        auto add = [](float* p, float x) { if (x != 0.0f) atomicAdd(p, x); };
+        add(P.v_screen.xy + 2u * g, v[0]); add(P.v_screen.xy + 2u * g + 1u, v[1]);
+        add(P.v_screen.depth + g, v[2]);
+        add(P.v_screen.conic + 3u * g, v[3]); add(P.v_screen.conic + 3u * g + 1u, v[4]); add(P.v_screen.conic + 3u * g + 2u, v[5]);
+        add(P.v_screen.opac + g, v[6]);
+        add(P.v_screen.rgb + 3u * g, v[7]); add(P.v_screen.rgb + 3u * g + 1u, v[8]); add(P.v_screen.rgb + 3u * g + 2u, v[9]);
+        if constexpr (kAccCh == 12) {
+            const int64_t wid = P.gaussian_ids ? (int64_t)P.gaussian_ids[g] : (int64_t)g;
+            add(P.accum_weight + wid, v[10]);
+            if constexpr (kAccum == SSR_ACCUM_AVG) add(P.accum_weight + P.num_world + wid, v[11]);
+        }
+    };
 
     for (int32_t hi = min(range_end - 1, tile_last); hi >= range_start; hi -= kBatch) {
         __syncthreads();   // previous batch fully consumed
+        flush_slot();      // its sums leave before the slot is reused (first pass: all zero)
         const int32_t idx = hi - tid;   // LDS slot t holds sorted index hi - t: ascending t is back to front
         if (idx >= range_start) {
             const int32_t g = P.flatten_ids[idx];
@@ -285,13 +324,12 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
                     s3 = row_sum(fold16(re_, re_));           // rows: g, g, b, b       -> channels 8,8,9,9
                 }
                 float mine = sub == 0 ? s1 : (sub == 1 ? s2 : s3);
-                uint32_t dst_row = (uint32_t)s_ids[k];
-                if constexpr (kAccum == SSR_ACCUM_SUM || kAccum == SSR_ACCUM_AVG) { if (chan >= 10) dst_row = (uint32_t)wid; }
-                if (chan >= 0 && ssr_isfinite(mine) && mine != 0.0f)
-                    atomicAdd(abase + (uint32_t)astride * dst_row, mine);   // < 2^32 elements per array
+                if (chan >= 0 && ssr_isfinite(mine) && mine != 0.0f) atomicAdd(&s_acc[k * kAccCh + chan], mine);
             }
         }
     }
+    __syncthreads();
+    flush_slot();
 }
 
 }  // namespace ssr
@@ -314,8 +352,9 @@ extern "C" int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t strea
                     "ssr_raster_bwd", "null screen buffer");
         SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->screen.xy) & 7) == 0, "ssr_raster_bwd", "screen.xy must be 8-byte aligned");
     }
-    SSR_REQUIRE(p->v_screen.xy && p->v_screen.depth && p->v_screen.conic && p->v_screen.opac && p->v_screen.rgb,
+    SSR_REQUIRE(p->v_rows || (p->v_screen.xy && p->v_screen.depth && p->v_screen.conic && p->v_screen.opac && p->v_screen.rgb),
                 "ssr_raster_bwd", "null v_screen buffer");
+    SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->v_rows) & 15) == 0, "ssr_raster_bwd", "v_rows must be 16-byte aligned");
     SSR_REQUIRE(p->dist_type >= SSR_DIST_NONE && p->dist_type <= SSR_DIST_RGB_D, "ssr_raster_bwd",
                 "dist_type must be NONE, D or RGB_D (the 3dgs pixel has no normal channel)");
     if (p->dist_type != SSR_DIST_NONE)

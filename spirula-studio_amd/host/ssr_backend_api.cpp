@@ -27,6 +27,8 @@ int32_t* g_visible_ids = nullptr;    // device work list of the last projection 
 float* g_packed_rows = nullptr;      // packed screen rows of the last projection (null: off)
 const float* g_packed_for_xy = nullptr;   // the screen.xy buffer those rows mirror
 int g_list_toggle = 0;               // which of the two visible-list buffers the last projection used
+float* g_vrows = nullptr;             // packed gradient rows of the last compositing backward (null: off)
+const float* g_vrows_for_xy = nullptr; // the v_screen.xy buffer they stand in for
 const int32_t* g_bwd_list = nullptr; // list of the last projection backward
 int64_t g_bwd_count = 0;
 
@@ -481,6 +483,7 @@ rasterize_to_pixels_3dgs_bwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     if (accum_weight_map.data_ptr() == nullptr) accum_mode = DensifyAccumMode::None;   // src/kernels/raster/RasterizationBwd.cu:234
     std::vector<DeviceTensorFloatND> vs;
     if (v_splats_s) {
+        g_vrows = nullptr; g_vrows_for_xy = nullptr;
         vs = *v_splats_s;   // caller-provided accumulators are added into as they are
     } else {
         // the launcher owns and zero-fills v_screen (src/kernels/raster/RasterizationBwd.cu:143-146);
@@ -488,7 +491,14 @@ rasterize_to_pixels_3dgs_bwd(int64_t num_splats, std::vector<DeviceTensorFloatND
         const int64_t n = splats_s.empty() ? 0 : splats_s[0].rows();
         const int ch[5] = {2, 1, 3, 1, 3};
         float* base = DevicePool::global().acquire<float>(PoolSlot::RasterBwdVScreenXy, (size_t)(n * 10));
-        backend::memset_async(base, 0, (size_t)(n * 10) * sizeof(float));
+        g_vrows = nullptr; g_vrows_for_xy = nullptr;
+        if (g_opts.packed_vscreen) {   // the rows take the gradients; the five arrays stay unfilled
+            g_vrows = DevicePool::global().acquire<float>(PoolSlot::RasterBwdVRows, (size_t)(n * 12));
+            g_vrows_for_xy = base;
+            backend::memset_async(g_vrows, 0, (size_t)(n * 12) * sizeof(float));
+        } else {
+            backend::memset_async(base, 0, (size_t)(n * 10) * sizeof(float));
+        }
         int64_t off = 0;
         for (int i = 0; i < 5; i++) {
             vs.emplace_back(base + off, std::vector<int64_t>{n, ch[i]});
@@ -507,6 +517,7 @@ rasterize_to_pixels_3dgs_bwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     p.v_render_T = v_render_Ts.data_ptr();
     p.v_screen = screen_of(vs);
     if (g_packed_rows && p.screen.xy == g_packed_for_xy) p.packed_rows = g_packed_rows;
+    if (g_vrows && p.v_screen.xy == g_vrows_for_xy) p.v_rows = g_vrows;
     p.dist_type = (int32_t)dist_type;
     if (dist_type != DistortionType::None) {
         p.distortion_depth = std::get<1>(*distortion_fwd_outputs).data_ptr();
@@ -563,6 +574,7 @@ void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
     p.camera = camera_of(camera_model, viewmats, intrins, image_width, image_height);
     p.aabb = (const float*)aabb.data_ptr();
     p.v_screen = screen_of(v_splats_screen);
+    if (g_vrows && p.v_screen.xy == g_vrows_for_xy) p.v_rows = g_vrows;
     p.v_world = world_of(v_splats_world);
     p.accumulate = g_opts.overwrite_world_grads ? 0 : 1;
     if (is_packed) {
@@ -609,6 +621,7 @@ void fused_projection_bwd_optimizer_3dgs(
     p.camera = camera_of(camera_model, viewmats, intrins, image_width, image_height);
     p.aabb = aabb.data_ptr();
     p.v_screen = screen_of(v_splats_screen);
+    if (g_vrows && p.v_screen.xy == g_vrows_for_xy) p.v_rows = g_vrows;
     if (!v_splats_world.empty()) p.v_world_in = world_of(v_splats_world);
     p.v_world_in.features_sh = nullptr;   // not read (FusedProjectionBwdOptim_kernel.cuh:250-255)
     p.g1 = world_of(g1_splats_world);

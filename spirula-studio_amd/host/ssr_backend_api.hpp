@@ -157,6 +157,11 @@ struct Options {
     // culled splats) and the caller may skip its zero-fill; with the list only visible rows are
     // stored and the zero-fill is still needed.
     bool overwrite_world_grads = false;
+    // The compositing backward writes each splat's ten gradient channels as one 12-float row (its
+    // atomics then touch one or two cache lines instead of five) and the projection backward / fused
+    // optimizer read those rows when handed the v_splats_screen of that call; the five returned
+    // tensors are then allocated but NOT filled.
+    bool packed_vscreen = false;
     // int8 codes x per-splat fp16 scale as SH storage (the benchmark's format): sh_value_bits == 8
     // with sh_value_bounds holding the fp16 scales when this is set.
     bool sh_int8_f16scale = false;

@@ -68,7 +68,7 @@ enum class PoolSlot : int {
     AdamG1Means, AdamG1Quats, AdamG1Scales, AdamG1Opacities, AdamG1FeaturesDc, AdamG1FeaturesSh,
     AdamG2Means, AdamG2Quats, AdamG2Scales, AdamG2Opacities, AdamG2FeaturesDc, AdamG2FeaturesSh, EngDensifyScore, ProjCameraIds, ProjGaussianIds, ProjGaussianIdsB, ProjPackedScratch, ProjPackedNnz,
     RendersRgb, RendersDepth, RenderTs, RenderLastIds, RenderDistortionRgb, RenderDistortionDepth, RenderMedian,
-    RasterBwdAccumWeight, EngVDistRgb, EngVDistDepth, EngVMedian, EngAccumMap,
+    RasterBwdAccumWeight, RasterBwdVRows, EngVDistRgb, EngVDistDepth, EngVMedian, EngAccumMap,
     RasterBwdVScreenXy, RasterBwdVScreenDepth, RasterBwdVScreenConic, RasterBwdVScreenOpac, RasterBwdVScreenRgb,
     EngVRgb, EngVDepth, EngVTs,
     GradMeans, GradQuats, GradScales, GradOpacities, GradFeaturesDc, GradFeaturesSh,

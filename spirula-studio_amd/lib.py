@@ -59,7 +59,7 @@ class RasterBwdParams(C.Structure):
                 ("height", C.c_uint32), ("tile_offsets", vp), ("flatten_ids", vp),
                 ("n_isects", C.c_int64), ("render_T", vp), ("last_ids", vp), ("render_depth", vp),
                 ("v_render_rgb", vp), ("v_render_depth", vp), ("v_render_T", vp),
-                ("v_screen", Screen), ("packed_rows", vp), ("dist_type", C.c_int32), ("render_rgb", vp),
+                ("v_screen", Screen), ("packed_rows", vp), ("v_rows", vp), ("dist_type", C.c_int32), ("render_rgb", vp),
                 ("distortion_rgb", vp), ("distortion_depth", vp), ("v_distortion_rgb", vp),
                 ("v_distortion_depth", vp), ("v_render_median", vp), ("accum_mode", C.c_int32),
                 ("accum_weight_map", vp), ("gaussian_ids", vp), ("num_world", C.c_int64), ("accum_weight", vp)]
@@ -69,7 +69,7 @@ class ProjectionBwdParams(C.Structure):
     _fields_ = [("num_splats", C.c_int64), ("sh_degree", C.c_int32), ("world", World),
                 ("sh", ShQuant), ("camera", Camera), ("aabb", vp), ("v_screen", Screen),
                 ("v_world", World), ("accumulate", C.c_int32), ("visible_ids", vp),
-                ("n_visible", C.c_int64), ("packed_gaussian_ids", vp), ("num_packed", C.c_int64)]
+                ("n_visible", C.c_int64), ("packed_gaussian_ids", vp), ("num_packed", C.c_int64), ("v_rows", vp)]
 
 
 class ProjectionPackedParams(C.Structure):
@@ -82,7 +82,7 @@ class ProjectionPackedParams(C.Structure):
 
 class FpboParams(C.Structure):
     _fields_ = [("num_splats", C.c_int64), ("sh_degree", C.c_int32), ("world", World), ("camera", Camera),
-                ("aabb", vp), ("v_screen", Screen), ("v_world_in", World), ("g1", World), ("g2", World),
+                ("aabb", vp), ("v_screen", Screen), ("v_rows", vp), ("v_world_in", World), ("g1", World), ("g2", World),
                 ("densify_score", vp),
                 ("lr_means", C.c_float), ("lr_quats", C.c_float), ("lr_scales", C.c_float), ("lr_opacs", C.c_float),
                 ("lr_features_dc", C.c_float), ("lr_features_sh", C.c_float),

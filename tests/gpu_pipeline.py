@@ -10,7 +10,7 @@ import numpy as np
 
 class GpuRun:
     def __init__(self, pkg, scene, sh_degree=3, use_list=False, use_packed=False, packed_projection=False,
-                 read_nnz=True):
+                 read_nnz=True, use_vrows=False):
         """use_packed: 48-byte fragment rows for the compositing kernels. packed_projection: the
         compacted (nnz-row) projection outputs of projection_3dgs_packed_forward; read_nnz=False
         sizes the outputs for all N splats instead of reading nnz back between the two calls."""
@@ -18,6 +18,7 @@ class GpuRun:
         self.use_packed = use_packed
         self.packed_projection = packed_projection
         self.read_nnz = read_nnz
+        self.use_vrows = use_vrows   # one 12-float gradient row per splat between K8 and K9
         assert not (packed_projection and use_list)
         self.L = pkg.lib
         self.lib = self.L.load()
@@ -249,6 +250,13 @@ class GpuRun:
         if self.use_packed:
             p.packed_rows = self.ptr("packed")
             p.screen = self.L.Screen()
+        if self.use_vrows:
+            self.d["v_rows"] = D((n, 12), np.float32)
+            self.d["v_rows"].fill_zero()
+            p.v_rows = self.ptr("v_rows")
+            if n:   # the five arrays must stay untouched
+                for k in ["v_xy", "v_depth", "v_conic", "v_opac", "v_rgb"]:
+                    self.check(self.lib.ssr_fill_u32(self.d[k].ptr, 0x7fc12345, self.d[k].nbytes // 4, None))
         va = self.variant
         f32 = lambda a: D.from_host(np.ascontiguousarray(a, np.float32))
         p.dist_type = va.get("dist_type", 0)
@@ -270,6 +278,13 @@ class GpuRun:
             if self.packed_projection:
                 p.gaussian_ids = self.ptr("gaussian_ids")
         self.check(self.lib.ssr_raster_bwd(C.byref(p), None))
+        if self.use_vrows and n:   # unpack for the comparisons, after checking the arrays were left alone
+            for k in ["v_xy", "v_depth", "v_conic", "v_opac", "v_rgb"]:
+                assert np.all(self.host(k).view(np.uint32) == 0x7fc12345), k
+            rows = self.host("v_rows")
+            assert not np.any(rows[:, 10:])
+            for k, sl in [("v_xy", slice(0, 2)), ("v_depth", 2), ("v_conic", slice(3, 6)), ("v_opac", 6), ("v_rgb", slice(7, 10))]:
+                self.d[k] = D.from_host(np.ascontiguousarray(rows[:, sl]))
 
     def projection_bwd(self, accumulate=True, poison=False):
         D = self.L.DeviceArray
@@ -289,6 +304,9 @@ class GpuRun:
         p.accumulate = 1 if accumulate else 0
         if self.use_list:
             p.visible_ids, p.n_visible = self.ptr("vis_ids"), self.V
+        if self.use_vrows:
+            p.v_rows = self.ptr("v_rows")
+            p.v_screen = self.L.Screen()   # not read
         if self.packed_projection:
             if self.rows == 0:   # nothing visible: the launcher has nothing to run (ProjectionBwd.cu:86-97)
                 return

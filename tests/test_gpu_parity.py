@@ -29,11 +29,12 @@ def _grad_close(got, ref, abs_scale, name, max_bad=0, rtol=GRAD_RTOL, afrac=2e-6
                                   got[bad][:4], ref[bad][:4])
 
 
-def _compare(gpu, oracle, sc, label, fused_count=False, use_list=False, use_packed=False, mask=None, variant=None):
+def _compare(gpu, oracle, sc, label, fused_count=False, use_list=False, use_packed=False, mask=None, variant=None,
+             use_vrows=False):
     live = None if mask is None else oracle.compute_tile_active(mask, sc.width, sc.height)
     r = oracle.pipeline(sc, tile_active=live, variant=variant)
     print(f"[{label}] N={sc.n} {sc.width}x{sc.height} visible={r['proj']['visible']} K={r['isect_ids'].size}", flush=True)
-    g = GpuRun(gpu, sc, use_list=use_list, use_packed=use_packed)
+    g = GpuRun(gpu, sc, use_list=use_list, use_packed=use_packed, use_vrows=use_vrows)
     if mask is not None:
         g.set_tile_mask(mask)
         assert np.array_equal(g.host("tile_active"), live)
@@ -88,6 +89,10 @@ def _compare(gpu, oracle, sc, label, fused_count=False, use_list=False, use_pack
     # terms are compared at that conditioning rather than at the bar of the plain path.
     mb = 8 if va.get("median") else 0
     kw = dict(rtol=1e-2, afrac=1e-3) if mb else {}
+    if va.get("dist_type") and not mb:
+        # the distortion terms contain (c W - C), a difference of nearly equal numbers whose rounding is
+        # not part of the |term| sums that set the floor: widen the floor for these runs
+        kw = dict(afrac=3e-5)
     _grad_close(g.host("v_xy"), vs["v_xy"], ab[:, 0:2], "v_xy", 2 * mb, **kw)
     _grad_close(g.host("v_depth"), vs["v_depth"], ab[:, 2], "v_depth", mb, **kw)
     _grad_close(g.host("v_conic"), vs["v_conic"], ab[:, 3:6], "v_conic", 3 * mb, **kw)
@@ -362,3 +367,16 @@ def test_compositing_variants(gpu, oracle, dist_type, median, accum):
     sc = gpu.scenes.tiny_scene(n=700, width=96, height=64, seed=9)
     va = dict(dist_type=dist_type, median=median, accum_mode=accum, **_variant_cotangents(sc, 2))
     _compare(gpu, oracle, sc, "variant-tiny", variant=va)
+
+
+def test_packed_gradient_rows(gpu, oracle):
+    """K8 writing one 12-float gradient row per splat and K9 reading it: same gradients, the five
+    v_screen arrays untouched."""
+    _compare(gpu, oracle, gpu.scenes.tiny_scene(n=700, width=96, height=64, seed=9), "vrows-tiny", use_vrows=True)
+    sc = gpu.scenes.make_scene(2, n=50000, width=480, height=270, parity_variant=True)
+    _compare(gpu, oracle, sc, "vrows-cfg2", fused_count=True, use_list=True, use_packed=True, use_vrows=True)
+    va = dict(dist_type=2, median=False, accum_mode=3, **_variant_cotangents(sc))
+    _compare(gpu, oracle, sc, "vrows-variants", fused_count=True, use_list=True, use_packed=True, use_vrows=True, variant=va)
+    sc = gpu.scenes.tiny_scene(n=64, width=40, height=24, seed=1)
+    sc.means[:, 2] = -10.0
+    _compare(gpu, oracle, sc, "vrows-culled", use_vrows=True)
