@@ -26,6 +26,7 @@ int64_t* g_counters = nullptr;       // device [n_isects, n_visible], one readba
 int32_t* g_visible_ids = nullptr;    // device work list of the last projection (null: off)
 float* g_packed_rows = nullptr;      // packed screen rows of the last projection (null: off)
 const float* g_packed_for_xy = nullptr;   // the screen.xy buffer those rows mirror
+bool g_packed_mode = false;          // the last projection was the packed form
 int g_list_toggle = 0;               // which of the two visible-list buffers the last projection used
 float* g_vrows = nullptr;             // packed gradient rows of the last compositing backward (null: off)
 const float* g_vrows_for_xy = nullptr; // the v_screen.xy buffer they stand in for
@@ -184,6 +185,12 @@ void set_stage_profiling(bool on) { g_profile = on; }
 StageTimes last_stage_times() { return g_times; }
 int64_t last_n_isects() { return g_n_isects; }
 int64_t last_n_visible() { return g_n_visible; }
+bool backward_overwrites_all_rows(int64_t num_splats) {
+    if (!g_opts.overwrite_world_grads) return false;
+    if (g_packed_mode) return false;                       // packed rows: only listed splats are written
+    if (!g_visible_ids || g_n_visible < 0) return true;    // no list: every row is visited
+    return g_n_visible * 2 >= num_splats;
+}
 const int32_t* last_backward_list(int64_t* count) { if (count) *count = g_bwd_count; return g_bwd_list; }
 void zero_world_rows(const std::vector<DeviceTensorFloatND>& v, const int32_t* ids, int64_t n,
                      const DeviceTensor2D<float4>* aabb) {
@@ -221,6 +228,7 @@ projection_3dgs_forward(const int64_t num_splats, const int max_sh_degree,
     p.aabb = (float*)aabb.data_ptr(); p.sort_depth = depths.data_ptr(); p.radii = radii.data_ptr();
     p.screen.xy = xy; p.screen.depth = dp; p.screen.conic = cn; p.screen.opac = op; p.screen.rgb = rg;
     g_counts_fused = false;
+    g_packed_mode = false;
     if (g_opts.fuse_tile_count) {
         p.tiles_per_splat = DevicePool::global().acquire<int64_t>(PoolSlot::IsectTilesPerSplat, (size_t)(C * N));
         g_counts_fused = true;
@@ -275,6 +283,7 @@ projection_3dgs_packed_forward(const int64_t num_splats, const int max_sh_degree
     p.scratch = DevicePool::global().acquire<uint8_t>(PoolSlot::ProjPackedScratch, p.scratch_bytes);
     p.nnz = DevicePool::global().acquire<int64_t>(PoolSlot::ProjPackedNnz, 1);
     // the work list and its counters belong to the non-packed form
+    g_packed_mode = true;
     g_visible_ids = nullptr; g_n_visible = -1; g_counters = nullptr;
     g_counts_fused = false; g_packed_rows = nullptr; g_packed_for_xy = nullptr;
     StageTimer t(&g_times.k1);
@@ -582,8 +591,9 @@ void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
         p.packed_gaussian_ids = gaussian_ids.data_ptr(); p.num_packed = camera_ids.size();
         g_bwd_list = gaussian_ids.data_ptr(); g_bwd_count = camera_ids.size();
     } else if (g_visible_ids && g_n_visible >= 0) {
-        p.visible_ids = g_visible_ids; p.n_visible = g_n_visible;
+        // the rows that end up non-zero are the listed ones either way
         g_bwd_list = g_visible_ids; g_bwd_count = g_n_visible;
+        if (!ssr_ext::backward_overwrites_all_rows(num_splats)) { p.visible_ids = g_visible_ids; p.n_visible = g_n_visible; }
     }
     StageTimer t(&g_times.k9);
     ok(ssr_projection_bwd(&p, nullptr), "projection_3dgs_backward");

@@ -177,6 +177,11 @@ int64_t last_n_visible();   // -1 when the visible list is off
 // The list the last projection_3dgs_backward ran over (device pointer) and its length; it stays
 // intact until the projection after next (the two list buffers alternate). Null when it had none.
 const int32_t* last_backward_list(int64_t* count);
+// True when the next projection_3dgs_backward (after the forward that just ran) will overwrite EVERY
+// row of v_splats_world -- store mode, and either no work list or so many visible splats (half or
+// more) that walking all rows is cheaper than a zero-fill plus the list. The caller may then skip
+// its zero-fill.
+bool backward_overwrites_all_rows(int64_t num_splats);
 // Zeroes the rows of `ids` in six world-gradient tensors (ordered as v_splats_world).
 // With `aabb` given, rows of currently visible splats are skipped (a store-mode backward overwrites them).
 void zero_world_rows(const std::vector<DeviceTensorFloatND>& v_splats_world, const int32_t* ids, int64_t n,

@@ -43,7 +43,8 @@ void alloc_grad_buffers() {
     const auto& o = ssr_ext::options();
     if (engine().optim.skip_grad_zero) return;
     const bool listed = o.visible_list || engine().packed;   // the backward touches listed rows only
-    if (o.overwrite_world_grads && !listed) return;   // K9 overwrites every row itself
+    // K9 overwrites every row itself (rows past cur_num_splats, if any, are not its business: fill then)
+    if (engine().cur_num_splats == n && ssr_ext::backward_overwrites_all_rows(n)) return;
     // Every row is zero except those the last backward wrote through its list (the visible-splat
     // list, or gaussian_ids in packed mode): when that list is short, zero just those rows instead
     // of refilling all N (the refill is 236 B per splat).
