@@ -6,8 +6,8 @@
 // 8-bit-digit sort, src/backend/vulkan/SortScanVulkan.cpp:84-146). The result is the unique
 // stable order on the masked key, so any correct stable sort is bit-identical to either.
 //
-// Per 8-bit digit pass: (1) per-workgroup digit histogram, (2) per-digit scan across workgroups
-// plus a scan of the 256 digit totals, (3) stable scatter. In (3) each wavefront owns a contiguous
+// Per 8-bit digit pass: (1) per-workgroup digit histogram, (2) per-digit scan across workgroups,
+// (3) stable scatter (which first scans the 256 digit totals for itself). In (3) each wavefront owns a contiguous
 // run of keys and ranks them 64 at a time with ballot-based digit matching (wave64: one 64-bit
 // ballot per digit bit), so order inside a workgroup is wave, round, lane = input order.
 #include "common.h"
@@ -69,34 +69,33 @@ __global__ __launch_bounds__(kSortBlock) void sort_scan_rows_kernel(uint32_t* __
     if (threadIdx.x == 0) totals[blockIdx.x] = carry;
 }
 
-// Exclusive scan of the 256 digit totals (one workgroup).
-__global__ __launch_bounds__(kRadix) void sort_scan_totals_kernel(uint32_t* __restrict__ totals) {
-    __shared__ uint32_t ws[kRadix / 64];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t v = totals[threadIdx.x];
-    uint32_t inc = v;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const uint32_t o = __shfl_up(inc, d, 64);
-        if (lane >= d) inc += o;
-    }
-    if (lane == 63) ws[wave] = inc;
-    __syncthreads();
-    uint32_t base = 0;
-#pragma unroll
-    for (int w = 0; w < kRadix / 64; w++) { if (w < wave) base += ws[w]; }
-    totals[threadIdx.x] = base + inc - v;
-}
-
 __global__ __launch_bounds__(kSortBlock) void sort_scatter_kernel(
     const uint64_t* __restrict__ keys_in, const int32_t* __restrict__ vals_in, uint64_t* __restrict__ keys_out,
     int32_t* __restrict__ vals_out, int64_t n, int shift, uint32_t mask, int n_bits, uint32_t n_blocks,
-    const uint32_t* __restrict__ hist, const uint32_t* __restrict__ digit_base) {
+    const uint32_t* __restrict__ hist, const uint32_t* __restrict__ totals) {
     __shared__ uint32_t wcount[kSortWaves][kRadix];   // per-wave running digit counts, then bases
+    __shared__ uint32_t ws[kSortWaves];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
     for (int w = 0; w < kSortWaves; w++) wcount[w][threadIdx.x] = 0;
-    __syncthreads();
+    // exclusive scan of the 256 digit totals, done by every workgroup for itself (a kernel of its own
+    // for these 1 KB would cost a launch per pass): thread t ends up with the first position of digit t
+    uint32_t digit_base;
+    {
+        const uint32_t v = totals[threadIdx.x];
+        uint32_t inc = v;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t o = __shfl_up(inc, d, 64);
+            if (lane >= d) inc += o;
+        }
+        if (lane == 63) ws[wave] = inc;
+        __syncthreads();
+        uint32_t base = 0;
+#pragma unroll
+        for (int w = 0; w < kSortWaves; w++) { if (w < wave) base += ws[w]; }
+        digit_base = base + inc - v;
+    }
 
     const int64_t wave_base = (int64_t)blockIdx.x * kSortTile + (int64_t)wave * (kSortRounds * 64);
     uint64_t key[kSortRounds];
@@ -129,7 +128,7 @@ __global__ __launch_bounds__(kSortBlock) void sort_scatter_kernel(
     __syncthreads();
     {   // thread t owns digit t: turn per-wave counts into global positions of each wave's first key
         const uint32_t d = threadIdx.x;
-        uint32_t run = digit_base[d] + hist[(size_t)d * n_blocks + blockIdx.x];
+        uint32_t run = digit_base + hist[(size_t)d * n_blocks + blockIdx.x];
 #pragma unroll
         for (int w = 0; w < kSortWaves; w++) {
             const uint32_t c = wcount[w][d];
@@ -183,7 +182,6 @@ int ssr_sort_pairs_u64_i32(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, in
         const uint32_t mask = (1u << bits) - 1u;
         hipLaunchKernelGGL(sort_hist_kernel, dim3(nb), dim3(kSortBlock), 0, s, k[cur], n, shift, mask, nb, hist);
         hipLaunchKernelGGL(sort_scan_rows_kernel, dim3(kRadix), dim3(kSortBlock), 0, s, hist, nb, totals);
-        hipLaunchKernelGGL(sort_scan_totals_kernel, dim3(1), dim3(kRadix), 0, s, totals);
         hipLaunchKernelGGL(sort_scatter_kernel, dim3(nb), dim3(kSortBlock), 0, s, k[cur], v[cur], k[cur ^ 1], v[cur ^ 1], n,
                            shift, mask, bits, nb, hist, totals);
         cur ^= 1;
