@@ -6,6 +6,12 @@
  * product library never links, loads or calls it. Only tests, the smoke check and the
  * cpu_baseline leg of the benchmark may use it.
  *
+ * Parity unpinned: the opacity side of the median-depth gradient in or_raster_bwd_ex. The reference's
+ * backward omits the far splat's own opacity term by its own statement
+ * (src/kernels/raster/RasterizationEval3DBwd_kernel.cuh:433-440), so it is not the derivative of the
+ * forward and no finite difference can check it; it is restated as read. Every other function is
+ * checked against closed forms, float64 restatements or finite differences by tests/test_oracle_*.py.
+ *
  * Every pointer is a host pointer. Arrays use the reference's layouts
  * (src/primitives/PrimitiveBase3DGS.cuh:87-139,187-225):
  *   world:  means[N,3] quats[N,4](w,x,y,z) log_scales[N,3] opacity_logits[N] features_dc[N,3]
