@@ -96,17 +96,6 @@ __device__ __forceinline__ FragLds stage_fragment(const ssr_screen& s, const flo
     return f;
 }
 
-// FragmentFwd::evaluate_alpha (src/primitives/Primitive3DGS.cuh:250-260):
-// sigma = 0.5 (a dx^2 + c dy^2) + b dx dy with the fused operations placed as written here.
-__device__ __forceinline__ float eval_alpha(const float4& q0, const float4& q1, float px, float py, float& dx,
-                                            float& dy, float& vis, float& sigma) {
-    dx = q0.x - px; dy = q0.y - py;
-    sigma = ssr_fma(q0.z * dx, dx, ssr_fma(q1.x * dy, dy, (q0.w * dx) * dy));
-    vis = ssr_exp(-sigma);
-    const float alpha = ssr_min(0.999f, q1.y * vis);
-    return sigma < 0.f ? 0.f : alpha;
-}
-
 // exp(x) for x in [-87, 0] (and NaN): the same operations as ssr_exp() on that range, where its
 // overflow / underflow branches are dead and 2^k (k in [-126, 0], result normal) can be applied by
 // adding k to the exponent field -- exact, so the bits equal ssr_exp(x).
@@ -127,17 +116,10 @@ __device__ __forceinline__ float exp_neg_small(float x) {
     return __uint_as_float(__float_as_uint(y) + ((uint32_t)ki << 23));
 }
 
-// eval_alpha() without the transcendental's range handling: identical results wherever
+// FragmentFwd::evaluate_alpha (src/primitives/Primitive3DGS.cuh:250-260): sigma = 0.5 (a dx^2 + c dy^2)
+// + b dx dy with the fused operations placed as written here, alpha = min(0.999, opac exp(-sigma)),
+// 0 for sigma < 0. The exponential is taken without its range handling: identical results wherever
 // alpha > 1/255 can hold (0 <= sigma <= cut), and alpha = 0 -- the skipped case -- elsewhere.
-__device__ __forceinline__ float eval_sigma(const float4& q0, const float4& q1, float px, float py, float& dx, float& dy) {
-    dx = q0.x - px; dy = q0.y - py;
-    return ssr_fma(q0.z * dx, dx, ssr_fma(q1.x * dy, dy, (q0.w * dx) * dy));
-}
-__device__ __forceinline__ float alpha_of_sigma(const float4& q1, float cut, float sigma, float& vis) {
-    const float e = exp_neg_small(-sigma);
-    vis = (sigma < 0.f || sigma > cut) ? 0.f : e;
-    return ssr_min(0.999f, q1.y * vis);
-}
 __device__ __forceinline__ float eval_alpha_fast(const float4& q0, const float4& q1, float cut, float px, float py,
                                                  float& dx, float& dy, float& vis, float& sigma) {
     dx = q0.x - px; dy = q0.y - py;

@@ -75,7 +75,7 @@ class Engine:
     """Drives the engine harness for one scene: upload once, then forward / backward."""
 
     def __init__(self, scene, device=0, fuse_tile_count=True, visible_list=True, packed_rows=True, overwrite_world_grads=True,
-                 stage_profiling=False, sh_degree=3, packed_projection=False, packed_vscreen=False):
+                 stage_profiling=False, sh_degree=3, packed_projection=False, packed_vscreen=True):
         """packed_projection: forward_3dgs(packed=true), the compacted projection outputs of
         projection_3dgs_packed_forward (the visible-splat work list then has no role)."""
         self.h = load()
