@@ -155,6 +155,16 @@ def quantize_ref(values: np.ndarray, bits: int, stride: int):
 def quantize_i8_f16(values: np.ndarray):
     """int8 codes with one fp16 scale per Gaussian: v = code * scale."""
     v = values.reshape(values.shape[0], -1).astype(np.float32)
+    nat = _native()
+    if nat is not None and hasattr(nat, "ssrh_quantize_i8_f16") and v.shape[0] >= 100000:
+        v = np.ascontiguousarray(v)
+        q = np.empty(v.shape, np.int8)
+        scale = np.empty(v.shape[0], np.uint16)
+        dec = np.empty(v.shape, np.float32)
+        nat.ssrh_quantize_i8_f16(ctypes.c_int64(v.shape[0]), ctypes.c_int(v.shape[1]), v.ctypes.data_as(ctypes.c_void_p),
+                                 q.ctypes.data_as(ctypes.c_void_p), scale.ctypes.data_as(ctypes.c_void_p),
+                                 dec.ctypes.data_as(ctypes.c_void_p))
+        return q.reshape(-1), scale.view(np.float16), dec.reshape(values.shape)
     amax = np.abs(v).max(axis=1)
     scale = (amax / np.float32(127.0)).astype(np.float16)
     scale = np.where((scale == 0) & (amax > 0), np.float16(6e-8), scale).astype(np.float16)
@@ -274,6 +284,23 @@ def apply_sh_codec(sc: Scene, codec: int, bounds_stride: int = 256) -> None:
         sc.features_sh = dec
     else:
         raise ValueError(f"unknown SH codec {codec}")
+
+
+def subset(sc: Scene, idx: np.ndarray) -> Scene:
+    """The scene restricted to the splats `idx` (same camera and cotangents). Per-splat codecs keep
+    their codes; the block-wise reference codecs become fp32 storage of the decoded values, which
+    projects to the same bits."""
+    idx = np.asarray(idx, np.int64)
+    out = dataclasses.replace(
+        sc, n=int(idx.size), means=np.ascontiguousarray(sc.means[idx]), quats=np.ascontiguousarray(sc.quats[idx]),
+        log_scales=np.ascontiguousarray(sc.log_scales[idx]), opacity_logits=np.ascontiguousarray(sc.opacity_logits[idx]),
+        features_dc=np.ascontiguousarray(sc.features_dc[idx]), features_sh=np.ascontiguousarray(sc.features_sh[idx]))
+    if sc.sh_codec == SH_I8_F16SCALE:
+        out.sh_packed = np.ascontiguousarray(sc.sh_packed.reshape(sc.n, -1)[idx])
+        out.sh_scale_f16 = np.ascontiguousarray(sc.sh_scale_f16[idx])
+    elif sc.sh_codec != SH_F32:
+        out.sh_codec, out.sh_packed, out.sh_bounds, out.sh_bounds_stride = SH_F32, None, None, 0
+    return out
 
 
 def tiny_scene(n: int = 300, width: int = 64, height: int = 48, seed: int = 7,
