@@ -91,6 +91,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--reference-order", action="store_true",
                     help="run the stages exactly as the reference does (separate count pass, atomic K9 into zero-filled buffers)")
+    ap.add_argument("--whole-key-sort", action="store_true",
+                    help="six whole-array digit passes + the offsets kernel instead of the tile-segmented sort")
     ap.add_argument("--packed-projection", action="store_true",
                     help="run the packed form of the projection (compacted nnz-row outputs; the reference's training default)")
     ap.add_argument("--fused-optimizer", action="store_true",
@@ -130,7 +132,8 @@ def main():
     t_gen = time.time() - t_gen
     native = not args.reference_order
     eng = host.Engine(sc, fuse_tile_count=native, visible_list=native and not args.packed_projection, packed_rows=native,
-                      overwrite_world_grads=native, packed_projection=args.packed_projection, packed_vscreen=native)
+                      overwrite_world_grads=native, packed_projection=args.packed_projection, packed_vscreen=native,
+                      tile_sort=native and not args.whole_key_sort)
     L = lib.load()
 
     hyper = dict(lr_means=1.6e-6, lr_quats=1e-5, lr_scales=5e-5, lr_opacs=5e-4, lr_features_dc=2.5e-5, lr_features_sh=1.25e-6)

@@ -189,6 +189,16 @@ int ssr_tile_offsets(int64_t n_isects, const int64_t* sorted_ids, uint32_t n_til
                      int32_t* offsets, ssr_stream_t stream);
 /* Number of key bits the sort must cover: 32 + tile_n_bits (IntersectTile.cu:489-490). */
 int ssr_sort_end_bit(uint32_t n_tiles);
+/* The sort of IntersectTile.cu:486-493 and the offsets of :271-307 in one call, for keys of the
+ * form (tile << 32) | depth_bits with tile < n_tiles: partitions by tile (stable, tile bits only),
+ * writes tile_offsets, then sorts every tile's range on the depth bits with one workgroup per
+ * tile. Result (in the buffer pair *selector names) and tile_offsets are bit-identical to
+ * ssr_sort_pairs_u64_i32 on bits [0, ssr_sort_end_bit(n_tiles)) followed by ssr_tile_offsets.
+ * The other buffer pair is used as working space. */
+size_t ssr_sort_tile_scratch_bytes(int64_t n, uint32_t n_tiles);
+int ssr_sort_tile_pairs(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, int32_t* vals_b,
+                        int64_t n, uint32_t n_tiles, int32_t* tile_offsets, int* selector,
+                        void* scratch, size_t scratch_bytes, ssr_stream_t stream);
 
 /* ---- K7: rasterize_to_pixels_3dgs_fwd (src/kernels/raster/RasterizationFwd.cuh:18-38, kernel
  * src/kernels/raster/RasterizationEval3DFwd_kernel.cuh:48-313, IS_EVAL3D=0). */

@@ -24,11 +24,33 @@ __device__ __forceinline__ uint32_t digit_of(uint64_t key, int shift, uint32_t m
     return (uint32_t)(key >> shift) & mask;
 }
 
+// For each lane: the number of live lanes below it that hold the same 8-bit digit (its rank among its
+// peers), and the size of that peer group. One ballot per digit bit set in `varying` (the caller knows
+// the other bits to be the same in every live lane); a lane differs from this one when any bit's vote
+// disagrees with its own bit (vote XOR own bit, OR-ed over the bits).
+__device__ __forceinline__ void wave_match_digit(uint32_t d, uint32_t varying, bool live, uint32_t& rank, uint32_t& group) {
+    uint32_t differ_lo = 0, differ_hi = 0;
+#pragma unroll
+    for (int b = 0; b < 8; b++) {
+        if ((varying >> b) & 1u) {
+            const uint32_t own = (uint32_t)__builtin_amdgcn_sbfe((int)d, (uint32_t)b, 1u);   // 0 or ~0
+            const uint64_t vote = __ballot(own != 0u);
+            differ_lo |= (uint32_t)vote ^ own;
+            differ_hi |= (uint32_t)(vote >> 32) ^ own;
+        }
+    }
+    const uint64_t alive = __ballot(live);
+    const uint32_t peers_lo = ~differ_lo & (uint32_t)alive, peers_hi = ~differ_hi & (uint32_t)(alive >> 32);
+    rank = __builtin_amdgcn_mbcnt_hi(peers_hi, __builtin_amdgcn_mbcnt_lo(peers_lo, 0u));
+    group = (uint32_t)__popc(peers_lo) + (uint32_t)__popc(peers_hi);
+}
+
 // hist[d * n_blocks + block]
 __global__ __launch_bounds__(kSortBlock) void sort_hist_kernel(const uint64_t* __restrict__ keys, int64_t n, int shift,
                                                                uint32_t mask, uint32_t n_blocks,
-                                                               uint32_t* __restrict__ hist) {
+                                                               uint32_t* __restrict__ hist, uint32_t* clear4) {
     __shared__ uint32_t lh[kRadix];
+    if (clear4 && blockIdx.x == 0 && threadIdx.x < 4) clear4[threadIdx.x] = 0;   // counters of a later kernel on this stream
     lh[threadIdx.x] = 0;
     __syncthreads();
     const int64_t base = (int64_t)blockIdx.x * kSortTile;
@@ -74,7 +96,10 @@ __global__ __launch_bounds__(kSortBlock) void sort_scatter_kernel(
     int32_t* __restrict__ vals_out, int64_t n, int shift, uint32_t mask, int n_bits, uint32_t n_blocks,
     const uint32_t* __restrict__ hist, const uint32_t* __restrict__ totals) {
     __shared__ uint32_t wcount[kSortWaves][kRadix];   // per-wave running digit counts, then bases
-    __shared__ uint32_t ws[kSortWaves];
+    __shared__ uint32_t ws[kSortWaves], ws2[kSortWaves];
+    __shared__ uint32_t s_shift[kRadix];
+    __shared__ uint64_t s_key[kSortTile];
+    __shared__ int32_t s_val[kSortTile];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
     for (int w = 0; w < kSortWaves; w++) wcount[w][threadIdx.x] = 0;
@@ -101,7 +126,6 @@ __global__ __launch_bounds__(kSortBlock) void sort_scatter_kernel(
     uint64_t key[kSortRounds];
     int32_t val[kSortRounds];
     uint32_t off[kSortRounds];
-    const uint64_t lt_mask = (1ull << lane) - 1ull;
 #pragma unroll
     for (int r = 0; r < kSortRounds; r++) {
         const int64_t i = wave_base + r * 64 + lane;
@@ -109,42 +133,350 @@ __global__ __launch_bounds__(kSortBlock) void sort_scatter_kernel(
         key[r] = live ? keys_in[i] : 0;
         val[r] = live ? vals_in[i] : 0;
         const uint32_t d = digit_of(key[r], shift, mask);
-        // lanes holding the same digit (and alive): intersect one ballot per digit bit
-        uint64_t peers = __ballot(live);
-        for (int b = 0; b < n_bits; b++) {
-            const uint64_t vote = __ballot((d >> b) & 1u);
-            peers &= ((d >> b) & 1u) ? vote : ~vote;
-        }
+        uint32_t rank, group;
+        wave_match_digit(d, mask, live, rank, group);
         uint32_t prev = 0;
         if (live) {
             prev = wcount[wave][d];          // count from earlier rounds of this wave
         }
         // every peer has read before the leader updates: same wavefront, program order on LDS
         __builtin_amdgcn_wave_barrier();
-        if (live && (peers & lt_mask) == 0) wcount[wave][d] = prev + (uint32_t)__popcll(peers);
+        if (live && rank == 0) wcount[wave][d] = prev + group;
         __builtin_amdgcn_wave_barrier();
-        off[r] = prev + (uint32_t)__popcll(peers & lt_mask);
+        off[r] = prev + rank;
     }
     __syncthreads();
-    {   // thread t owns digit t: turn per-wave counts into global positions of each wave's first key
+    {   // thread t owns digit t: per-wave counts become positions, inside this workgroup's 4096 keys in digit
+        // order, of each wave's first key of the digit; s_shift[t] = where the digit's run goes in the output
+        // minus where it starts in that order
         const uint32_t d = threadIdx.x;
-        uint32_t run = digit_base + hist[(size_t)d * n_blocks + blockIdx.x];
+        uint32_t c[kSortWaves], block_count = 0;
 #pragma unroll
-        for (int w = 0; w < kSortWaves; w++) {
-            const uint32_t c = wcount[w][d];
-            wcount[w][d] = run;
-            run += c;
+        for (int w = 0; w < kSortWaves; w++) { c[w] = wcount[w][d]; block_count += c[w]; }
+        uint32_t inc = block_count;
+#pragma unroll
+        for (int k = 1; k < 64; k <<= 1) {
+            const uint32_t o = __shfl_up(inc, k, 64);
+            if (lane >= k) inc += o;
         }
+        if (lane == 63) ws2[wave] = inc;
+        __syncthreads();
+        uint32_t local = inc - block_count;
+#pragma unroll
+        for (int w = 0; w < kSortWaves; w++) { if (w < wave) local += ws2[w]; }
+        s_shift[d] = digit_base + hist[(size_t)d * n_blocks + blockIdx.x] - local;
+        uint32_t run = local;
+#pragma unroll
+        for (int w = 0; w < kSortWaves; w++) { wcount[w][d] = run; run += c[w]; }
     }
     __syncthreads();
+    // stage the pairs in digit order, then write them out in that order: neighbouring lanes write
+    // neighbouring addresses wherever a digit's run is longer than one key
 #pragma unroll
     for (int r = 0; r < kSortRounds; r++) {
         const int64_t i = wave_base + r * 64 + lane;
         if (i < n) {
             const uint32_t pos = wcount[wave][digit_of(key[r], shift, mask)] + off[r];
-            keys_out[pos] = key[r];
-            vals_out[pos] = val[r];
+            s_key[pos] = key[r];
+            s_val[pos] = val[r];
         }
+    }
+    __syncthreads();
+    const int64_t block_base = (int64_t)blockIdx.x * kSortTile;
+    const int block_n = (int)(n - block_base < kSortTile ? n - block_base : kSortTile);
+#pragma unroll
+    for (int r = 0; r < kSortRounds; r++) {
+        const int j = r * kSortBlock + threadIdx.x;
+        if (j < block_n) {
+            const uint64_t k = s_key[j];
+            const uint32_t pos = s_shift[digit_of(k, shift, mask)] + (uint32_t)j;
+            keys_out[pos] = k;
+            vals_out[pos] = s_val[j];
+        }
+    }
+}
+
+// ---- Tile-segmented variant ---------------------------------------------------------------------
+// Keys are (tile id << 32) | depth bits. A stable sort on the tile bits alone leaves every tile's
+// entries contiguous and in input order; a stable sort of each such segment on the depth bits then
+// gives the same order as a stable sort on the whole key. Only the tile-bit passes stream the whole
+// key array through HBM; a segment is sorted by one workgroup, in LDS when it fits.
+
+// Ranks the wave's 64 keys of one round by `d` (8 bits): returns the number of earlier keys of this wave
+// with the same digit, and advances the wave's running count (wcount_row = this wave's 256 counters).
+__device__ __forceinline__ uint32_t seg_rank_round(uint32_t d, uint32_t varying, bool live, uint32_t* wcount_row) {
+    uint32_t rank, group;
+    wave_match_digit(d, varying, live, rank, group);
+    uint32_t prev = 0;
+    if (live) prev = wcount_row[d];
+    __builtin_amdgcn_wave_barrier();
+    if (live && rank == 0) wcount_row[d] = prev + group;
+    __builtin_amdgcn_wave_barrier();
+    return prev + rank;
+}
+
+// Threads 0..255 own one digit each: per-wave counts become the segment-local position of each wave's
+// first key of that digit. Called by the whole workgroup (two barriers inside).
+template <int kWaves>
+__device__ __forceinline__ void seg_digit_bases(uint32_t (*wcount)[kRadix], uint32_t* ws) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if constexpr (kWaves == 1) {   // a lone wavefront: lane l owns digits 4l..4l+3, nothing to wait for
+        uint4 c = reinterpret_cast<uint4*>(wcount[0])[lane];
+        const uint32_t total = c.x + c.y + c.z + c.w;
+        uint32_t inc = total;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t o = __shfl_up(inc, d, 64);
+            if (lane >= d) inc += o;
+        }
+        uint4 b;
+        b.x = inc - total; b.y = b.x + c.x; b.z = b.y + c.y; b.w = b.z + c.z;
+        reinterpret_cast<uint4*>(wcount[0])[lane] = b;
+        __syncthreads();
+        return;
+    }
+    const bool owner = threadIdx.x < kRadix;
+    uint32_t total = 0, inc = 0;
+    if (owner) {
+#pragma unroll
+        for (int w = 0; w < kWaves; w++) total += wcount[w][threadIdx.x];
+        inc = total;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t o = __shfl_up(inc, d, 64);
+            if (lane >= d) inc += o;
+        }
+        if (lane == 63) ws[wave] = inc;
+    }
+    __syncthreads();
+    if (owner) {
+        uint32_t run = inc - total;
+#pragma unroll
+        for (int w = 0; w < kRadix / 64; w++) { if (w < wave) run += ws[w]; }
+#pragma unroll
+        for (int w = 0; w < kWaves; w++) {
+            const uint32_t c = wcount[w][threadIdx.x];
+            wcount[w][threadIdx.x] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+}
+
+// OR over the workgroup of `x` (the key bits that differ inside the segment): a digit whose bits are
+// all clear in it is the same for every key, and its pass moves nothing.
+template <int kWaves>
+__device__ __forceinline__ uint32_t seg_or_all(uint32_t x, uint32_t* wor) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) x |= __shfl_xor(x, d, 64);
+    if ((threadIdx.x & 63) == 0) wor[threadIdx.x >> 6] = x;
+    __syncthreads();
+    uint32_t all = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; w++) all |= wor[w];
+    return all;
+}
+
+// The workgroup (kWaves wavefronts) sorts keys[s, s + len), len <= 64 * kWaves * kRounds, in place on the
+// low 32 key bits: keys in registers, one LDS round trip per digit pass.
+template <int kWaves, int kRounds>
+__device__ __forceinline__ void seg_sort_lds(uint64_t* keys, int32_t* vals, int64_t s, int len, uint32_t (*wcount)[kRadix],
+                                             uint32_t* ws, uint32_t* wor, uint2* buf) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int per_wave = ((len + kWaves - 1) / kWaves + 63) & ~63;   // contiguous run per wave
+    const int rounds = per_wave >> 6;
+    const int first = wave * per_wave + lane;
+    const uint64_t key0 = keys[s];
+    const uint32_t hi = (uint32_t)(key0 >> 32);
+
+    uint32_t key[kRounds], off[kRounds];
+    int32_t val[kRounds];
+    uint32_t differ = 0;
+#pragma unroll
+    for (int r = 0; r < kRounds; r++) {
+        const int i = first + r * 64;
+        const bool live = r < rounds && i < len;
+        key[r] = live ? (uint32_t)keys[s + i] : (uint32_t)key0;
+        val[r] = live ? vals[s + i] : 0;
+        differ |= key[r] ^ (uint32_t)key0;
+    }
+    differ = seg_or_all<kWaves>(differ, wor);
+    int last_shift = -1;   // the last pass that moves anything writes straight to the output
+#pragma unroll
+    for (int shift = 0; shift < 32; shift += 8) { if ((differ >> shift) & 255u) last_shift = shift; }
+    if (last_shift < 0) return;   // all keys equal: already in order
+#pragma unroll 1
+    for (int shift = 0; shift <= last_shift; shift += 8) {
+        if (((differ >> shift) & 255u) == 0) continue;
+        wcount[wave][lane] = wcount[wave][lane + 64] = wcount[wave][lane + 128] = wcount[wave][lane + 192] = 0;
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < kRounds; r++) {
+            if (r < rounds) {
+                const bool live = first + r * 64 < len;
+                off[r] = seg_rank_round((key[r] >> shift) & 255u, (differ >> shift) & 255u, live, wcount[wave]);
+            }
+        }
+        __syncthreads();
+        seg_digit_bases<kWaves>(wcount, ws);
+        if (shift == last_shift) {
+#pragma unroll
+            for (int r = 0; r < kRounds; r++) {
+                if (r < rounds && first + r * 64 < len) {
+                    const uint32_t pos = wcount[wave][(key[r] >> shift) & 255u] + off[r];
+                    keys[s + pos] = ((uint64_t)hi << 32) | key[r];
+                    vals[s + pos] = val[r];
+                }
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < kRounds; r++) {
+                if (r < rounds && first + r * 64 < len) {
+                    const uint32_t pos = wcount[wave][(key[r] >> shift) & 255u] + off[r];
+                    buf[pos] = make_uint2(key[r], (uint32_t)val[r]);
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < kRounds; r++) {
+                if (r < rounds && first + r * 64 < len) {
+                    const uint2 kv = buf[first + r * 64];
+                    key[r] = kv.x;
+                    val[r] = (int32_t)kv.y;
+                }
+            }
+            // the barrier after the next pass's clearing of wcount also orders these reads of buf before
+            // that pass's writes to it
+        }
+    }
+}
+
+// Work lists of the tiles whose segments are too long for the direct kernel, by size class:
+// counts[c] entries in list[c]; class 0 up to kSegCap0 keys, class 1 up to kSegCap1, class 2 beyond.
+struct SegLists { uint32_t* counts; uint32_t* list[3]; };
+constexpr int kSegCap0 = 4 * 64 * 4;           // four wavefronts, 4 keys per lane
+constexpr int kSegCap1 = 16 * 64 * 8;          // sixteen wavefronts, 8 keys per lane
+
+// One workgroup of kWaves wavefronts per tile: sorts segments of 2..64*kWaves*kRounds keys, lists the
+// longer ones. These kernels are bound by instruction issue: one wavefront per tile executes the fewest
+// instructions per key, but its tiles take long, so it pays only when there are several rounds of
+// workgroups to balance the compute units; four wavefronts per tile otherwise.
+template <int kWaves, int kRounds>
+__global__ __launch_bounds__(kWaves * 64) void sort_segments_direct_kernel(uint64_t* keys, int32_t* vals,
+                                                                           const int32_t* __restrict__ tile_offsets,
+                                                                           uint32_t n_tiles, int64_t n, SegLists lists) {
+    constexpr int kCap = kWaves * 64 * kRounds;
+    static_assert(kCap <= kSegCap0, "class 0 starts above the direct kernel's capacity");
+    __shared__ __attribute__((aligned(16))) uint32_t wcount[kWaves][kRadix];
+    __shared__ uint32_t ws[kRadix / 64];
+    __shared__ uint32_t wor[kWaves];
+    __shared__ uint2 buf[kCap];
+    const uint32_t tile = blockIdx.x;
+    const int64_t s = tile_offsets[tile];
+    const int64_t e = tile + 1 < n_tiles ? (int64_t)tile_offsets[tile + 1] : n;
+    const int len = (int)(e - s);
+    if (len <= 1) return;
+    if (len > kCap) {
+        if (threadIdx.x == 0) {
+            const int c = len > kSegCap1 ? 2 : len > kSegCap0 ? 1 : 0;
+            lists.list[c][atomicAdd(&lists.counts[c], 1u)] = tile;
+        }
+        return;
+    }
+    seg_sort_lds<kWaves, kRounds>(keys, vals, s, len, wcount, ws, wor, buf);
+}
+
+// Workgroups of four wavefronts take the listed segments of class 0 in turn.
+__global__ __launch_bounds__(256) void sort_segments_small_kernel(uint64_t* keys, int32_t* vals,
+                                                                  const int32_t* __restrict__ tile_offsets, uint32_t n_tiles,
+                                                                  int64_t n, SegLists lists) {
+    __shared__ uint32_t wcount[4][kRadix];
+    __shared__ uint32_t ws[kRadix / 64];
+    __shared__ uint32_t wor[4];
+    __shared__ uint2 buf[kSegCap0];
+    const uint32_t count = lists.counts[0];
+    for (uint32_t idx = blockIdx.x; idx < count; idx += gridDim.x) {
+        const uint32_t tile = lists.list[0][idx];
+        const int64_t s = tile_offsets[tile];
+        const int64_t e = tile + 1 < n_tiles ? (int64_t)tile_offsets[tile + 1] : n;
+        seg_sort_lds<4, 4>(keys, vals, s, (int)(e - s), wcount, ws, wor, buf);
+        __syncthreads();   // LDS is reused by the next segment
+    }
+}
+
+// The workgroup (16 wavefronts) sorts keys[s, s + len) of any length on the low 32 key bits: four digit
+// passes through global memory, between that range of (keys, vals) and the same range of the second
+// buffer pair; the result ends where it started.
+constexpr int kSegGlobalWaves = 16;
+__device__ __forceinline__ void seg_sort_global(uint64_t* keys, int32_t* vals, uint64_t* keys_alt, int32_t* vals_alt, int64_t s,
+                                                int len, uint32_t (*wcount)[kRadix], uint32_t* ws) {
+    constexpr int kWaves = kSegGlobalWaves;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int per_wave = ((len + kWaves - 1) / kWaves + 63) & ~63;
+    const int w_begin = wave * per_wave;
+    const int w_end = min(len, w_begin + per_wave);
+    uint64_t* k_src = keys + s; uint64_t* k_dst = keys_alt + s;
+    int32_t* v_src = vals + s; int32_t* v_dst = vals_alt + s;
+#pragma unroll 1
+    for (int shift = 0; shift < 32; shift += 8) {
+        wcount[wave][lane] = wcount[wave][lane + 64] = wcount[wave][lane + 128] = wcount[wave][lane + 192] = 0;
+        __syncthreads();
+#pragma unroll 4
+        for (int i = w_begin + lane; i < w_end; i += 64) {
+            const uint64_t k = __hip_atomic_load(k_src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            atomicAdd(&wcount[wave][(uint32_t)(k >> shift) & 255u], 1u);
+        }
+        __syncthreads();
+        seg_digit_bases<kWaves>(wcount, ws);
+        // wcount[wave][d] now runs: the next free position of digit d for this wave
+        uint64_t k_next = 0; int32_t v_next = 0;
+        if (w_begin + lane < w_end) {
+            k_next = __hip_atomic_load(k_src + w_begin + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            v_next = __hip_atomic_load(v_src + w_begin + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+        for (int i0 = w_begin; i0 < w_end; i0 += 64) {
+            const uint64_t k = k_next; const int32_t v = v_next;
+            const bool live = i0 + lane < w_end;
+            const int j = i0 + 64 + lane;   // the next round's pair is in flight while this one is ranked
+            if (j < w_end) {
+                k_next = __hip_atomic_load(k_src + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                v_next = __hip_atomic_load(v_src + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+            const uint32_t pos = seg_rank_round((uint32_t)(k >> shift) & 255u, 255u, live, wcount[wave]);
+            if (live) {
+                __hip_atomic_store(k_dst + pos, k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_store(v_dst + pos, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+        }
+        __syncthreads();   // workgroup-scope release/acquire: the next pass reads what this one wrote
+        uint64_t* tk = k_src; k_src = k_dst; k_dst = tk;
+        int32_t* tv = v_src; v_src = v_dst; v_dst = tv;
+    }
+}
+
+// Workgroups of sixteen wavefronts take the listed segments of class 1 (in LDS), then of class 2
+// (through global memory), in turn.
+__global__ __launch_bounds__(kSegGlobalWaves * 64) void sort_segments_long_kernel(
+    uint64_t* keys, int32_t* vals, uint64_t* keys_alt, int32_t* vals_alt, const int32_t* __restrict__ tile_offsets,
+    uint32_t n_tiles, int64_t n, SegLists lists) {
+    __shared__ uint32_t wcount[kSegGlobalWaves][kRadix];
+    __shared__ uint32_t ws[kRadix / 64];
+    __shared__ uint32_t wor[kSegGlobalWaves];
+    __shared__ uint2 buf[kSegCap1];
+    static_assert(kSegCap1 == kSegGlobalWaves * 64 * 8, "class 1 is sorted by sixteen wavefronts with 8 keys per lane");
+    const uint32_t count1 = lists.counts[1], count2 = lists.counts[2];
+    for (uint32_t idx = blockIdx.x; idx < count1; idx += gridDim.x) {
+        const uint32_t tile = lists.list[1][idx];
+        const int64_t s = tile_offsets[tile];
+        const int64_t e = tile + 1 < n_tiles ? (int64_t)tile_offsets[tile + 1] : n;
+        seg_sort_lds<kSegGlobalWaves, 8>(keys, vals, s, (int)(e - s), wcount, ws, wor, buf);
+        __syncthreads();   // LDS is reused by the next segment
+    }
+    for (uint32_t idx = blockIdx.x; idx < count2; idx += gridDim.x) {
+        const uint32_t tile = lists.list[2][idx];
+        const int64_t s = tile_offsets[tile];
+        const int64_t e = tile + 1 < n_tiles ? (int64_t)tile_offsets[tile + 1] : n;
+        seg_sort_global(keys, vals, keys_alt, vals_alt, s, (int)(e - s), wcount, ws);
     }
 }
 
@@ -160,9 +492,15 @@ size_t ssr_sort_scratch_bytes(int64_t n) {
     return (nb * kRadix + kRadix) * sizeof(uint32_t);
 }
 
-int ssr_sort_pairs_u64_i32(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, int32_t* vals_b, int64_t n,
-                           int begin_bit, int end_bit, int* selector, void* scratch, size_t scratch_bytes,
-                           ssr_stream_t stream) {
+size_t ssr_sort_tile_scratch_bytes(int64_t n, uint32_t n_tiles) {
+    if (n <= 0) return 0;
+    return ((ssr_sort_scratch_bytes(n) + 15) & ~(size_t)15) + (4 + 3 * (size_t)n_tiles) * sizeof(uint32_t);
+}
+
+// clear4 (optional): four counters that the first kernel launched here sets to zero
+static int sort_pairs_impl(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, int32_t* vals_b, int64_t n, int begin_bit,
+                           int end_bit, int* selector, void* scratch, size_t scratch_bytes, ssr_stream_t stream,
+                           uint32_t* clear4) {
     SSR_REQUIRE(selector, "ssr_sort_pairs_u64_i32", "null selector");
     *selector = 0;
     SSR_REQUIRE(n >= 0 && n < (int64_t)1 << 31, "ssr_sort_pairs_u64_i32", "count out of range");
@@ -180,7 +518,8 @@ int ssr_sort_pairs_u64_i32(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, in
     for (int shift = begin_bit; shift < end_bit; shift += 8) {
         const int bits = end_bit - shift < 8 ? end_bit - shift : 8;
         const uint32_t mask = (1u << bits) - 1u;
-        hipLaunchKernelGGL(sort_hist_kernel, dim3(nb), dim3(kSortBlock), 0, s, k[cur], n, shift, mask, nb, hist);
+        hipLaunchKernelGGL(sort_hist_kernel, dim3(nb), dim3(kSortBlock), 0, s, k[cur], n, shift, mask, nb, hist,
+                           shift == begin_bit ? clear4 : nullptr);
         hipLaunchKernelGGL(sort_scan_rows_kernel, dim3(kRadix), dim3(kSortBlock), 0, s, hist, nb, totals);
         hipLaunchKernelGGL(sort_scatter_kernel, dim3(nb), dim3(kSortBlock), 0, s, k[cur], v[cur], k[cur ^ 1], v[cur ^ 1], n,
                            shift, mask, bits, nb, hist, totals);
@@ -188,6 +527,63 @@ int ssr_sort_pairs_u64_i32(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, in
     }
     SSR_CHECK_LAUNCH("ssr_sort_pairs_u64_i32");
     *selector = cur;
+    return 0;
+}
+
+int ssr_sort_pairs_u64_i32(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, int32_t* vals_b, int64_t n,
+                           int begin_bit, int end_bit, int* selector, void* scratch, size_t scratch_bytes,
+                           ssr_stream_t stream) {
+    return sort_pairs_impl(keys_a, keys_b, vals_a, vals_b, n, begin_bit, end_bit, selector, scratch, scratch_bytes, stream,
+                           nullptr);
+}
+
+int ssr_sort_tile_pairs(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, int32_t* vals_b, int64_t n,
+                        uint32_t n_tiles, int32_t* tile_offsets, int* selector, void* scratch, size_t scratch_bytes,
+                        ssr_stream_t stream) {
+    SSR_REQUIRE(selector, "ssr_sort_tile_pairs", "null selector");
+    *selector = 0;
+    SSR_REQUIRE(n >= 0 && n < (int64_t)1 << 31, "ssr_sort_tile_pairs", "count out of range");
+    if (n_tiles == 0) return 0;
+    SSR_REQUIRE(tile_offsets, "ssr_sort_tile_pairs", "null offsets");
+    SSR_REQUIRE(n == 0 || (scratch && scratch_bytes >= ssr_sort_tile_scratch_bytes(n, n_tiles)), "ssr_sort_tile_pairs",
+                "scratch too small");
+    SegLists lists = {};
+    if (n > 0) {
+        lists.counts = reinterpret_cast<uint32_t*>(static_cast<char*>(scratch) + ((ssr_sort_scratch_bytes(n) + 15) & ~(size_t)15));
+        for (int c = 0; c < 3; c++) lists.list[c] = lists.counts + 4 + (size_t)c * n_tiles;
+    }
+    const int end_bit = ssr_sort_end_bit(n_tiles);
+    if (n > 0 && end_bit > 32) {   // partition by tile: stable on the tile bits only
+        if (sort_pairs_impl(keys_a, keys_b, vals_a, vals_b, n, 32, end_bit, selector, scratch, scratch_bytes, stream, lists.counts))
+            return 1;
+    } else if (n > 0) {
+        SSR_REQUIRE(keys_a && keys_b && vals_a && vals_b, "ssr_sort_tile_pairs", "null buffer");
+        if (ssr_fill_u32(lists.counts, 0u, 4, stream)) return 1;
+    }
+    const int cur = *selector;
+    int64_t* k[2] = {keys_a, keys_b};
+    int32_t* v[2] = {vals_a, vals_b};
+    if (ssr_tile_offsets(n, k[cur], n_tiles, tile_offsets, stream)) return 1;
+    if (n <= 1) return 0;
+    hipStream_t s = as_stream(stream);
+    uint64_t* kc = reinterpret_cast<uint64_t*>(k[cur]);
+    uint64_t* ka = reinterpret_cast<uint64_t*>(k[cur ^ 1]);
+    const bool lone_waves = n_tiles >= 16384;   // at least two rounds of one-wavefront workgroups on 256 compute units
+    if (lone_waves) {
+        hipLaunchKernelGGL((sort_segments_direct_kernel<1, 8>), dim3(n_tiles), dim3(64), 0, s, kc, v[cur], tile_offsets, n_tiles,
+                           n, lists);
+        // the listed segments: fixed grids, a workgroup with no list entry ends at once
+        if (n > 512)
+            hipLaunchKernelGGL(sort_segments_small_kernel, dim3(n_tiles < 2048 ? n_tiles : 2048), dim3(256), 0, s, kc, v[cur],
+                               tile_offsets, n_tiles, n, lists);
+    } else {
+        hipLaunchKernelGGL((sort_segments_direct_kernel<4, 4>), dim3(n_tiles), dim3(256), 0, s, kc, v[cur], tile_offsets,
+                           n_tiles, n, lists);
+    }
+    if (n > kSegCap0)
+        hipLaunchKernelGGL(sort_segments_long_kernel, dim3(n_tiles < 512 ? n_tiles : 512), dim3(kSegGlobalWaves * 64), 0, s, kc,
+                           v[cur], ka, v[cur ^ 1], tile_offsets, n_tiles, n, lists);
+    SSR_CHECK_LAUNCH("ssr_sort_tile_pairs");
     return 0;
 }
 

@@ -18,7 +18,7 @@ SYMBOLS = {
     "ssrh_last_error": (C.c_char_p, []),
     "ssrh_init": (C.c_int, [C.c_int]),
     "ssrh_reset": (C.c_int, []),
-    "ssrh_set_options": (C.c_int, [C.c_int] * 7),
+    "ssrh_set_options": (C.c_int, [C.c_int] * 8),
     "ssrh_set_data_3dgs": (C.c_int, [C.c_int64, vp, vp, vp, vp, vp, vp, C.c_int]),
     "ssrh_set_sh_value_quant": (C.c_int, [C.c_int, vp, C.c_int64, C.c_int, vp, C.c_int64, C.c_int, C.c_int64]),
     "ssrh_set_camera_params": (C.c_int, [C.c_int, C.c_int, C.c_char_p, C.c_char_p, vp, vp, C.c_int]),
@@ -75,7 +75,8 @@ class Engine:
     """Drives the engine harness for one scene: upload once, then forward / backward."""
 
     def __init__(self, scene, device=0, fuse_tile_count=True, visible_list=True, packed_rows=True, overwrite_world_grads=True,
-                 stage_profiling=False, sh_degree=3, packed_projection=False, packed_vscreen=True):
+                 stage_profiling=False, sh_degree=3, packed_projection=False, packed_vscreen=True,
+                 tile_sort=True):
         """packed_projection: forward_3dgs(packed=true), the compacted projection outputs of
         projection_3dgs_packed_forward (the visible-splat work list then has no role)."""
         self.h = load()
@@ -88,7 +89,8 @@ class Engine:
         self.opts = [int(fuse_tile_count), int(visible_list), int(packed_rows), int(overwrite_world_grads),
                      int(scene.sh_codec == 3)]
         self.packed_vscreen = int(packed_vscreen)
-        check(self.h.ssrh_set_options(*self.opts, int(stage_profiling), self.packed_vscreen))
+        self.tile_sort = int(tile_sort)
+        check(self.h.ssrh_set_options(*self.opts, int(stage_profiling), self.packed_vscreen, self.tile_sort))
         f32 = lambda a: np.ascontiguousarray(a, np.float32)
         self._keep = [f32(scene.means), f32(scene.quats), f32(scene.log_scales), f32(scene.opacity_logits),
                       f32(scene.features_dc), f32(scene.features_sh)]
@@ -114,7 +116,7 @@ class Engine:
         self.d_vT = _lib.DeviceArray.from_host(f32(scene.v_T))
 
     def set_stage_profiling(self, on):
-        check(self.h.ssrh_set_options(*self.opts, int(on), self.packed_vscreen))
+        check(self.h.ssrh_set_options(*self.opts, int(on), self.packed_vscreen, self.tile_sort))
 
     def set_tile_mask(self, mask):
         """Tile-skip map for the next forward only, from a [h_mask, w_mask] byte mask."""

@@ -405,14 +405,18 @@ do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, 
     int selector = 0;
     {
         StageTimer t(&g_times.k5);
-        const size_t sb = ssr_sort_scratch_bytes(n_isects);
+        const size_t sb = g_opts.tile_sort ? ssr_sort_tile_scratch_bytes(n_isects, n_tiles) : ssr_sort_scratch_bytes(n_isects);
         void* scratch = DevicePool::global().acquire<uint8_t>(PoolSlot::IsectSortScratch, sb);
-        ok(ssr_sort_pairs_u64_i32(ids_a.data_ptr(), ids_b.data_ptr(), flat_a.data_ptr(), flat_b.data_ptr(), n_isects, 0,
-                                  ssr_sort_end_bit(n_tiles), &selector, scratch, sb, nullptr), "do_intersect_tile_generic/sort");
+        if (g_opts.tile_sort)   // also writes the offsets
+            ok(ssr_sort_tile_pairs(ids_a.data_ptr(), ids_b.data_ptr(), flat_a.data_ptr(), flat_b.data_ptr(), n_isects, n_tiles,
+                                   offsets.data_ptr(), &selector, scratch, sb, nullptr), "do_intersect_tile_generic/tile_sort");
+        else
+            ok(ssr_sort_pairs_u64_i32(ids_a.data_ptr(), ids_b.data_ptr(), flat_a.data_ptr(), flat_b.data_ptr(), n_isects, 0,
+                                      ssr_sort_end_bit(n_tiles), &selector, scratch, sb, nullptr), "do_intersect_tile_generic/sort");
     }
     DeviceVector<int64_t> ids_out = selector ? ids_b : ids_a;
     DeviceVector<int32_t> flat_out = selector ? flat_b : flat_a;
-    {
+    if (!g_opts.tile_sort) {
         StageTimer t(&g_times.k6);
         ok(ssr_tile_offsets(n_isects, ids_out.data_ptr(), n_tiles, offsets.data_ptr(), nullptr), "do_intersect_tile_generic/offsets");
     }

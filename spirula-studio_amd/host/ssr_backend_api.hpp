@@ -162,6 +162,9 @@ struct Options {
     // optimizer read those rows when handed the v_splats_screen of that call; the five returned
     // tensors are then allocated but NOT filled.
     bool packed_vscreen = false;
+    // The key sort partitions by tile (the tile bits only) and then sorts each tile's range on the
+    // depth bits with one workgroup per tile, instead of six whole-array digit passes; same result.
+    bool tile_sort = false;
     // int8 codes x per-splat fp16 scale as SH storage (the benchmark's format): sh_value_bits == 8
     // with sh_value_bounds holding the fp16 scales when this is set.
     bool sh_int8_f16scale = false;

@@ -374,7 +374,7 @@ int ssrh_init(int device) { return guard([&] { if (!backend::device_select(devic
 int ssrh_reset(void) { return guard([&] { engine_reset(); }); }
 
 int ssrh_set_options(int fuse_tile_count, int visible_list, int packed_rows, int overwrite_world_grads,
-                     int sh_int8_f16scale, int stage_profiling, int packed_vscreen) {
+                     int sh_int8_f16scale, int stage_profiling, int packed_vscreen, int tile_sort) {
     return guard([&] {
         auto& o = ssr_ext::options();
         o.fuse_tile_count = fuse_tile_count != 0; o.visible_list = visible_list != 0;
@@ -382,6 +382,7 @@ int ssrh_set_options(int fuse_tile_count, int visible_list, int packed_rows, int
         o.overwrite_world_grads = overwrite_world_grads != 0;
         o.sh_int8_f16scale = sh_int8_f16scale != 0;
         o.packed_vscreen = packed_vscreen != 0;
+        o.tile_sort = tile_sort != 0;
         ssr_ext::set_stage_profiling(stage_profiling != 0);
     });
 }

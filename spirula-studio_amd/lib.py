@@ -109,6 +109,8 @@ SYMBOLS = {
     "ssr_sort_pairs_u64_i32": (_i32, [vp, vp, vp, vp, _i64, _i32, _i32, C.POINTER(C.c_int), vp, _sz, vp]),
     "ssr_tile_offsets": (_i32, [_i64, vp, _u32, vp, vp]),
     "ssr_sort_end_bit": (_i32, [_u32]),
+    "ssr_sort_tile_scratch_bytes": (_sz, [_i64, _u32]),
+    "ssr_sort_tile_pairs": (_i32, [vp, vp, vp, vp, _i64, _u32, vp, C.POINTER(C.c_int), vp, _sz, vp]),
     "ssr_raster_fwd": (_i32, [C.POINTER(RasterFwdParams), vp]),
     "ssr_raster_bwd": (_i32, [C.POINTER(RasterBwdParams), vp]),
     "ssr_projection_bwd": (_i32, [C.POINTER(ProjectionBwdParams), vp]),

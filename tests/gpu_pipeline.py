@@ -10,7 +10,7 @@ import numpy as np
 
 class GpuRun:
     def __init__(self, pkg, scene, sh_degree=3, use_list=False, use_packed=False, packed_projection=False,
-                 read_nnz=True, use_vrows=False):
+                 read_nnz=True, use_vrows=False, tile_sort=False):
         """use_packed: 48-byte fragment rows for the compositing kernels. packed_projection: the
         compacted (nnz-row) projection outputs of projection_3dgs_packed_forward; read_nnz=False
         sizes the outputs for all N splats instead of reading nnz back between the two calls."""
@@ -18,6 +18,7 @@ class GpuRun:
         self.use_packed = use_packed
         self.packed_projection = packed_projection
         self.read_nnz = read_nnz
+        self.tile_sort = tile_sort   # ssr_sort_tile_pairs instead of the whole-key sort + ssr_tile_offsets
         self.use_vrows = use_vrows   # one 12-float gradient row per splat between K8 and K9
         assert not (packed_projection and use_list)
         self.L = pkg.lib
@@ -190,19 +191,25 @@ class GpuRun:
                                                self.V if self.use_list else 0, self.tile_active, None))
             self.unsorted_keys = self.d["keys_a"].to_host()
             self.unsorted_vals = self.d["vals_a"].to_host()
-            sb = self.lib.ssr_sort_scratch_bytes(K)
+            sb = (self.lib.ssr_sort_tile_scratch_bytes(K, n_tiles) if self.tile_sort else self.lib.ssr_sort_scratch_bytes(K))
             self.d["sort_scratch"] = D((sb,), np.uint8)
             sel = C.c_int(0)
-            self.check(self.lib.ssr_sort_pairs_u64_i32(self.ptr("keys_a"), self.ptr("keys_b"), self.ptr("vals_a"),
-                                                       self.ptr("vals_b"), K, 0, self.lib.ssr_sort_end_bit(n_tiles),
-                                                       C.byref(sel), self.ptr("sort_scratch"), sb, None))
+            if self.tile_sort:
+                self.check(self.lib.ssr_sort_tile_pairs(self.ptr("keys_a"), self.ptr("keys_b"), self.ptr("vals_a"),
+                                                        self.ptr("vals_b"), K, n_tiles, self.ptr("offsets"),
+                                                        C.byref(sel), self.ptr("sort_scratch"), sb, None))
+            else:
+                self.check(self.lib.ssr_sort_pairs_u64_i32(self.ptr("keys_a"), self.ptr("keys_b"), self.ptr("vals_a"),
+                                                           self.ptr("vals_b"), K, 0, self.lib.ssr_sort_end_bit(n_tiles),
+                                                           C.byref(sel), self.ptr("sort_scratch"), sb, None))
             self.sel = sel.value
         else:
             self.unsorted_keys = np.zeros(0, np.int64)
             self.unsorted_vals = np.zeros(0, np.int32)
         self.keys = "keys_b" if self.sel else "keys_a"
         self.vals = "vals_b" if self.sel else "vals_a"
-        self.check(self.lib.ssr_tile_offsets(K, self.ptr(self.keys), n_tiles, self.ptr("offsets"), None))
+        if not (self.tile_sort and K):
+            self.check(self.lib.ssr_tile_offsets(K, self.ptr(self.keys), n_tiles, self.ptr("offsets"), None))
 
     def raster_fwd(self):
         sc, D = self.sc, self.L.DeviceArray

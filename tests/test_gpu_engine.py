@@ -38,7 +38,7 @@ def test_engine_matches_oracle(pkg, oracle, H, native):
     sc = pkg.scenes.make_scene(1, n=30000, width=320, height=240, parity_variant=True)
     ref = oracle.pipeline(sc)
     eng = host.Engine(sc, fuse_tile_count=native, visible_list=native, packed_rows=native, overwrite_world_grads=native,
-                      packed_vscreen=native)
+                      packed_vscreen=native, tile_sort=native)
     eng.forward()
     eng.backward()
     g1 = _check(eng, ref, sc)

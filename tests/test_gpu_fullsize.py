@@ -112,7 +112,7 @@ def test_full_size_properties(pkg, oracle, H, cfg):
     rgb2, _, T2 = eng.render()
     assert np.array_equal(rgb, rgb2) and np.array_equal(T, T2)
     ref = host.Engine(sc, fuse_tile_count=False, visible_list=False, packed_rows=False, overwrite_world_grads=False,
-                      packed_vscreen=False)
+                      packed_vscreen=False, tile_sort=False)
     ref.forward()
     ref.backward()
     assert np.array_equal(ref.cache("sorted_ids").view(np.uint64), keys)

@@ -30,11 +30,11 @@ def _grad_close(got, ref, abs_scale, name, max_bad=0, rtol=GRAD_RTOL, afrac=2e-6
 
 
 def _compare(gpu, oracle, sc, label, fused_count=False, use_list=False, use_packed=False, mask=None, variant=None,
-             use_vrows=False):
+             use_vrows=False, tile_sort=False):
     live = None if mask is None else oracle.compute_tile_active(mask, sc.width, sc.height)
     r = oracle.pipeline(sc, tile_active=live, variant=variant)
     print(f"[{label}] N={sc.n} {sc.width}x{sc.height} visible={r['proj']['visible']} K={r['isect_ids'].size}", flush=True)
-    g = GpuRun(gpu, sc, use_list=use_list, use_packed=use_packed, use_vrows=use_vrows)
+    g = GpuRun(gpu, sc, use_list=use_list, use_packed=use_packed, use_vrows=use_vrows, tile_sort=tile_sort)
     if mask is not None:
         g.set_tile_mask(mask)
         assert np.array_equal(g.host("tile_active"), live)
@@ -211,6 +211,23 @@ def test_huge_splats_cooperative_key_write(gpu, oracle):
     g, r = _compare(gpu, oracle, sc, "huge", fused_count=True, use_list=True)
     assert r["counts"].max() > 500
     _compare(gpu, oracle, sc, "huge-nolist")
+
+
+def test_tile_segmented_sort(gpu, oracle):
+    """ssr_sort_tile_pairs in place of the whole-key sort and the offsets kernel: the same sorted keys,
+    values and tile ranges, and so the same images and gradients."""
+    _compare(gpu, oracle, gpu.scenes.tiny_scene(n=400, width=72, height=56, seed=3), "tiny-seg", tile_sort=True)
+    _compare(gpu, oracle, gpu.scenes.tiny_scene(n=300, width=16, height=16, seed=6), "one-tile-seg", tile_sort=True)
+    sc = gpu.scenes.tiny_scene(n=600, width=640, height=400, seed=13)
+    sc.log_scales[::7] += 2.5          # tiles with thousands of entries: the larger segment classes
+    sc.means[::50, 2] = -3.6
+    _compare(gpu, oracle, sc, "huge-seg", fused_count=True, use_list=True, tile_sort=True)
+    _compare(gpu, oracle, gpu.scenes.make_scene(1), "cfg1-seg", fused_count=True, use_list=True, use_packed=True,
+             use_vrows=True, tile_sort=True)
+    _compare(gpu, oracle, gpu.scenes.make_scene(5, n=40000, width=1024, height=512), "cfg5/eq-seg", tile_sort=True)
+    mask = np.zeros((30, 50), np.uint8)
+    mask[4:20, 8:30] = 1
+    _compare(gpu, oracle, gpu.scenes.tiny_scene(n=900, width=160, height=96, seed=41), "mask-seg", mask=mask, tile_sort=True)
 
 
 def test_tiny_equirect(gpu, oracle):

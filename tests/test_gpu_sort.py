@@ -58,6 +58,92 @@ def test_sort_already_sorted_and_reversed(L):
     assert np.array_equal(ko, keys) and np.array_equal(vo, vals[::-1])
 
 
+def _sort_tiles(L, keys, vals, n_tiles):
+    lib = L.load()
+    n = keys.size
+    ka, kb = L.DeviceArray.from_host(keys), L.DeviceArray((max(n, 1),), np.int64)
+    va, vb = L.DeviceArray.from_host(vals), L.DeviceArray((max(n, 1),), np.int32)
+    off = L.DeviceArray((n_tiles,), np.int32)
+    sb = lib.ssr_sort_tile_scratch_bytes(n, n_tiles)
+    scratch = L.DeviceArray((max(sb, 16),), np.uint8)
+    sel = C.c_int(-1)
+    L.check(lib.ssr_sort_tile_pairs(ka.ptr, kb.ptr, va.ptr, vb.ptr, n, n_tiles, off.ptr, C.byref(sel), scratch.ptr, sb,
+                                    None))
+    k, v = (kb, vb) if sel.value else (ka, va)
+    return k.to_host()[:n], v.to_host()[:n], off.to_host()
+
+
+def _tile_keys(rng, n_tiles, lengths, depth_bits):
+    """Keys (tile << 32) | depth in a random input order; `lengths[t]` entries for tile t."""
+    tiles = np.repeat(np.arange(n_tiles, dtype=np.int64), lengths)
+    n = tiles.size
+    depth = depth_bits(n)
+    keys = (tiles << 32) | depth.astype(np.int64)
+    perm = rng.permutation(n)
+    return keys[perm]
+
+
+@pytest.mark.parametrize("case", ["uniform", "ragged", "long", "one_tile", "dups", "single_entries", "many_tiles", "narrow",
+                                  "constant", "many_tiles_ragged"])
+def test_sort_tile_pairs(L, case):
+    """The tile-segmented sort against numpy's stable sort of the whole key, and its offsets against
+    searchsorted: segment lengths on both sides of every size class (1, 512, 1024, 8192), empty tiles,
+    duplicate depths (stability), up to 65536 tiles (16 tile bits: two partition passes)."""
+    rng = np.random.default_rng(sum(map(ord, case)))
+    rand32 = lambda n: rng.integers(0, 1 << 32, n, dtype=np.int64)
+    if case == "uniform":
+        n_tiles, lengths, bits = 2500, rng.integers(0, 900, 2500), rand32
+    elif case == "ragged":
+        n_tiles = 700
+        lengths = rng.choice([0, 0, 1, 2, 63, 64, 65, 255, 256, 257, 511, 512, 513, 1023, 1024, 1025, 2000, 4095, 4096, 4097, 5000, 8191, 8192, 8193, 9000],
+                             n_tiles)
+        bits = rand32
+    elif case == "long":
+        n_tiles, lengths, bits = 40, rng.integers(3000, 30000, 40), rand32
+        lengths[7] = 0
+        lengths[11] = 70001
+    elif case == "one_tile":
+        n_tiles, lengths, bits = 1, np.array([12345]), rand32
+    elif case == "dups":
+        n_tiles, lengths = 300, rng.integers(0, 6000, 300)
+        bits = lambda n: rng.choice(np.array([0, 1, 0x40000000, 0x40000001, 0xFFFFFFFF, 0x3F800000], np.int64), n)
+    elif case == "narrow":     # digits that are constant inside a tile: passes the segment sort skips
+        n_tiles, lengths = 400, rng.integers(0, 3000, 400)
+        lengths[3] = 12000
+        bits = lambda n: 0x40A00000 + (rng.integers(0, 1 << 16, n, dtype=np.int64) << rng.choice([0, 8]))
+    elif case == "constant":   # one depth per tile
+        n_tiles, lengths = 300, rng.integers(0, 2500, 300)
+        lengths[5] = 9000
+        bits = lambda n: np.full(n, 0x3F800000, np.int64)
+    elif case == "many_tiles_ragged":   # enough tiles for the one-wavefront-per-tile kernel, every size class
+        n_tiles = 20000
+        sizes = np.array([0, 1, 2, 63, 64, 65, 255, 256, 257, 511, 512, 513, 1023, 1024, 1025, 4097, 9000])
+        prob = np.where(sizes <= 513, 1.0, 0.02)
+        lengths, bits = rng.choice(sizes, n_tiles, p=prob / prob.sum()), rand32
+    elif case == "single_entries":
+        n_tiles, lengths, bits = 5000, rng.integers(0, 2, 5000), rand32
+    else:
+        n_tiles, lengths, bits = 65536, rng.integers(0, 40, 65536), rand32
+    keys = _tile_keys(rng, n_tiles, lengths, bits)
+    vals = np.arange(keys.size, dtype=np.int32)       # input position: exposes any instability
+    ko, vo, off = _sort_tiles(L, keys, vals, n_tiles)
+    order = np.argsort(keys.view(np.uint64), kind="stable")
+    assert np.array_equal(ko, keys[order])
+    assert np.array_equal(vo, vals[order])
+    assert np.array_equal(off, np.searchsorted(keys[order] >> 32, np.arange(n_tiles), side="left").astype(np.int32))
+
+
+def test_sort_tile_pairs_empty_and_errors(L):
+    lib = L.load()
+    ko, vo, off = _sort_tiles(L, np.zeros(0, np.int64), np.zeros(0, np.int32), 77)
+    assert ko.size == 0 and np.array_equal(off, np.zeros(77, np.int32))
+    ko, vo, off = _sort_tiles(L, np.array([(5 << 32) | 9], np.int64), np.array([3], np.int32), 8)
+    assert ko[0] == (5 << 32) | 9 and vo[0] == 3 and np.array_equal(off, [0, 0, 0, 0, 0, 0, 1, 1])
+    sel = C.c_int(0)
+    assert lib.ssr_sort_tile_pairs(None, None, None, None, 10, 100, None, C.byref(sel), None, 0, None) != 0
+    assert lib.ssr_last_error() != b""
+
+
 @pytest.mark.parametrize("n", [1, 2, 255, 256, 2047, 2048, 2049, 1_000_003, 10_000_019])
 def test_inclusive_sum_i64(L, n):
     lib = L.load()
