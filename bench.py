@@ -22,16 +22,18 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E peak
 
 
-def algorithmic_bytes(N, V, K, K_f, K_b, P, T, S):
+def algorithmic_bytes(N, V, K, K_f, K_b, P, T, S, sort_sweeps):
     """Minimum HBM bytes per stage for one iteration: every array an algorithm of this shape must
     read or write once. N splats, V visible, K splat-tile pairs, K_f / K_b pairs the forward /
-    backward actually need, P pixels, T tiles, S bytes of higher-order SH storage per splat."""
+    backward actually need, P pixels, T tiles, S bytes of higher-order SH storage per splat;
+    sort_sweeps = times the sort reads and writes the whole (key, value) array: one per 8-bit digit
+    of the whole key, or one per digit of the tile bits plus one for the per-tile segment sort."""
     return {
         "K1": N * (44 + 20) + V * (12 + S + 40 + 4),
         "K2": N * 16 + V * (24 + 8) + (N - V) * 8,
         "K3": N * 16,
         "K4": N * 16 + V * (24 + 4 + 16) + K * 12,
-        "K5": 6 * K * 24,
+        "K5": sort_sweeps * K * 24,
         "K6": K * 8 + T * 4,
         "K7": K_f * 44 + P * 24,
         "K8": P * 32 + K_b * 44 + K_b * 40 + N * 40,
@@ -198,7 +200,10 @@ def main():
     K_b = tile_need(eng.cache("offsets"), eng.cache("last_ids"), K, sc.width, sc.height)
     K_f = K_b   # lower bound of the forward's need (it also reads the splat that ends a pixel)
     S = 180 if sc.sh_codec == 0 else (47 if sc.sh_codec == 3 else 45 + 8 * 45 / 256)
-    ab = algorithmic_bytes(sc.n, V, K, K_f, K_b, P, T, S)
+    tile_bits = max(T - 1, 0).bit_length()
+    tile_sort = native and not args.whole_key_sort
+    sort_sweeps = (tile_bits + 7) // 8 + 1 if tile_sort else (32 + tile_bits + 7) // 8
+    ab = algorithmic_bytes(sc.n, V, K, K_f, K_b, P, T, S, sort_sweeps)
     total_bytes = sum(ab.values())
     dom = max(acc, key=acc.get)
     dom_gbs = ab[dom] / (acc[dom] * 1e-3) / 1e9 if acc[dom] > 0 else 0.0
@@ -222,7 +227,8 @@ def main():
                                f"{'pinhole' if sc.camera_model == 0 else 'equirectangular'}, SH3 "
                                f"{['fp32', 'ref-q8', 'ref-q16', 'int8*fp16scale'][sc.sh_codec]}, tile 16x16, seed {pkg.scenes.CONFIGS[cfg]['seed']:#x}",
                    "visible": V, "n_isects": K, "K_b": K_b, "tiles": T, "pixels": P,
-                   "stage_order": ("fused tile count, visible-splat work list, packed fragment rows, packed gradient rows, plain-store gradients" if native else "reference order")
+                   "stage_order": ("fused tile count, visible-splat work list, packed fragment rows, packed gradient rows, plain-store gradients"
+                                   + (", tile-segmented sort" if tile_sort else "") if native else "reference order")
                                   + (", packed projection outputs" if args.packed_projection else "")
                                   + (", projection backward fused with Adam" if args.fused_optimizer else "")
                                   + (f", compositing variants dist_type={args.dist_type} median={int(args.median)} accum_mode={args.accum_mode}" if variants else ""),

@@ -37,7 +37,10 @@ extern "C" {
 typedef void* ssr_stream_t;
 typedef void* ssr_event_t;
 
-enum { SSR_CAM_PINHOLE = 0, SSR_CAM_EQUIRECT = 3 };       /* CameraModelType, src/core/Common.cuh */
+enum { SSR_CAM_PINHOLE = 0, SSR_CAM_FISHEYE = 1, SSR_CAM_EQUISOLID = 2, SSR_CAM_EQUIRECT = 3 };   /* CameraModelType, src/core/Common.cuh */
+/* CameraDistortionType (src/core/CameraModel.h; coefficient order per tier:
+ * src/shaders/projection_utils.slang:242-295). Pairs accepted: src/kernels/projection/CameraVariants.cuh:11-22. */
+enum { SSR_LENS_NONE = 0, SSR_LENS_OPENCV = 1, SSR_LENS_THIN_PRISM = 2, SSR_LENS_RATIONAL = 3 };
 enum { SSR_SH_F32 = 0, SSR_SH_REF_Q8 = 1, SSR_SH_REF_Q16 = 2, SSR_SH_I8_F16SCALE = 3 };
 enum { SSR_DIST_NONE = 0, SSR_DIST_D = 1, SSR_DIST_RGB_D = 2 };   /* DistortionType, src/primitives/Primitive.cuh:24-32 */
 enum { SSR_ACCUM_NONE = 0, SSR_ACCUM_MAX = 1, SSR_ACCUM_SUM = 2, SSR_ACCUM_AVG = 3 };   /* DensifyAccumMode, :37-42 */
@@ -84,6 +87,9 @@ typedef struct {
     uint32_t width, height;
     const float* viewmats;  /* device [C,4,4] row-major world->camera */
     const float* intrins;   /* device [C,4] fx,fy,cx,cy */
+    const float* dist_coeffs;   /* device [C,8] lens coefficients in the tier's order; unused (may be
+                                 * NULL) with SSR_LENS_NONE */
+    int32_t distortion;     /* SSR_LENS_* */
 } ssr_camera;
 
 /* ---- K1: projection_3dgs_forward (src/kernels/projection/ProjectionFwd.cuh:18-36,

@@ -8,6 +8,7 @@
 // function names the reference source it follows.
 #include "ssr_oracle.h"
 #include "../include/ssr_math.h"
+#include "../include/ssr_camera.h"
 
 #include <algorithm>
 #include <cmath>
@@ -31,7 +32,13 @@ struct Cam {
     float R[3][3];
     float t[3];
     float fx, fy, cx, cy;
+    int tier;
+    float dc[8];
 };
+
+// PINHOLE without lens distortion and EQUIRECTANGULAR are written out by hand below; the other
+// (model, tier) pairs use the differentiated model functions of include/ssr_camera.h.
+bool lens_path(const Cam& c) { return !((c.model == OR_CAM_PINHOLE && c.tier == OR_LENS_NONE) || c.model == OR_CAM_EQUIRECT); }
 
 Cam load_cam(const or_camera* c) {
     // src/kernels/projection/ProjectionFwd_kernel.cuh:52-60
@@ -42,6 +49,8 @@ Cam load_cam(const or_camera* c) {
         k.t[i] = c->viewmat[4 * i + 3];
     }
     k.fx = c->fx; k.fy = c->fy; k.cx = c->cx; k.cy = c->cy;
+    k.tier = c->distortion;
+    for (int i = 0; i < 8; i++) k.dc[i] = (c->distortion != OR_LENS_NONE) ? c->dist_coeffs[i] : 0.0f;
     return k;
 }
 
@@ -243,7 +252,32 @@ Proj project(const Cam& cam, const float mean[3], const float quat[4], const flo
             p.covc[i][j] = (tmp[i][0] * cam.R[j][0] + tmp[i][1] * cam.R[j][1]) + tmp[i][2] * cam.R[j][2];
 
     float (*J)[3] = p.J;
-    if (cam.model == OR_CAM_PINHOLE) {
+    if (lens_path(cam)) {
+        // persp / fisheye / equisolid _proj<D, assume_valid> and _proj_jac<D>
+        // (projection_utils.slang:345-358,414-427,446-459 and :362-375,463-493): the point is
+        // dropped when the lens map is not locally invertible there (is_valid_distortion, :310-321);
+        // otherwise uv and its Jacobian come from one first-order evaluation of the model.
+        typedef SsrJet<3, 1> Jet;
+        Jet u, v, du, dv;
+        ssr_model_normalised<Jet>(cam.model, ssr_jet_seed<3, 1>(x, 0), ssr_jet_seed<3, 1>(y, 1), ssr_jet_seed<3, 1>(z, 2), u, v);
+        if (!assume_valid && !ssr_distortion_valid(cam.tier, cam.dc, u.v, v.v)) return p;
+        ssr_distort<Jet>(cam.tier, cam.dc, u, v, du, dv);
+        const Jet px = du * cam.fx + cam.cx, py = dv * cam.fy + cam.cy;
+        p.xy[0] = px.v; p.xy[1] = py.v;
+        for (int k = 0; k < 3; k++) { J[0][k] = px.d[k]; J[1][k] = py.d[k]; }
+        if (cam.model == OR_CAM_PINHOLE) {   // the clamp of persp_proj_3dgs, primitive_3dgs.slang:84-95
+            float Wf = (float)cam.W;
+            float lim_pos = Wf + 0.3f * (0.5f * Wf);
+            float lim_neg = 0.3f * (0.5f * Wf);
+            float rz = 1.f / z;
+            float max_x = (-((-lim_neg) - cam.cx)) * rz, min_x = (-(lim_pos - cam.cx)) * rz;
+            float max_y = (-((-lim_neg) - cam.cy)) * rz, min_y = (-(lim_pos - cam.cy)) * rz;
+            p.clamp_lo[0] = J[0][2] < min_x; p.clamp_hi[0] = !p.clamp_lo[0] && J[0][2] > max_x;
+            p.clamp_lo[1] = J[1][2] < min_y; p.clamp_hi[1] = !p.clamp_lo[1] && J[1][2] > max_y;
+            J[0][2] = ssr_min(ssr_max(J[0][2], min_x), max_x);
+            J[1][2] = ssr_min(ssr_max(J[1][2], min_y), max_y);
+        }
+    } else if (cam.model == OR_CAM_PINHOLE) {
         // persp_proj_3dgs, primitive_3dgs.slang:63-99; persp_proj_uv / _jac,
         // projection_utils.slang:331-375. The valid test (z < 0) is covered by the z <= 0 cull.
         float z2 = z * z;
@@ -282,6 +316,16 @@ Proj project(const Cam& cam, const float mean[3], const float quat[4], const flo
     for (int i = 0; i < 2; i++)
         for (int j = 0; j < 2; j++)
             p.c2[i][j] = (jc[i][0] * J[j][0] + jc[i][1] * J[j][1]) + jc[i][2] * J[j][2];
+    if (!assume_valid && (cam.model == OR_CAM_FISHEYE || cam.model == OR_CAM_EQUISOLID)) {
+        // primitive_3dgs.slang:509-514: behind the lens (z < 0) yet still visibly opaque at the image
+        // centre -- dropped; evaluated on the covariance before the blur
+        const float m0 = p.xy[0] - cam.cx, m1 = p.xy[1] - cam.cy;
+        const float idet = 1.0f / (p.c2[0][0] * p.c2[1][1] - p.c2[0][1] * p.c2[1][0]);
+        const float i00 = p.c2[1][1] * idet, i01 = (-p.c2[0][1]) * idet, i10 = (-p.c2[1][0]) * idet, i11 = p.c2[0][0] * idet;
+        const float q = (i00 * m0 + i01 * m1) * m0 + (i10 * m0 + i11 * m1) * m1;
+        const float seen = p.opac * ssr_exp(-0.5f * q);
+        if (z < 0.0f && seen > kAlphaThreshold) return p;
+    }
     // add_blur, primitive_3dgs.slang:398-405 (not antialiased: eps 0.3)
     p.c2[0][0] = p.c2[0][0] + 0.3f;
     p.c2[1][1] = p.c2[1][1] + 0.3f;
@@ -300,7 +344,9 @@ Proj project(const Cam& cam, const float mean[3], const float quat[4], const flo
         return p;
     p.aabb[0] = xmin; p.aabb[1] = ymin; p.aabb[2] = xmax; p.aabb[3] = ymax;
     // get_sorting_depth, projection_utils.slang:1012-1029
-    p.sort_depth = (cam.model == OR_CAM_PINHOLE) ? z : dot3(p.mc, p.mc);
+    if (cam.model == OR_CAM_PINHOLE) p.sort_depth = z;
+    else if (cam.model == OR_CAM_EQUIRECT) p.sort_depth = dot3(p.mc, p.mc);
+    else p.sort_depth = ((z * z) * z) * z + ((1.0f / 512.0f) * (x * x + y * y)) * (x * x + y * y);
     float campos[3];
     for (int i = 0; i < 3; i++)
         campos[i] = -((cam.R[0][i] * cam.t[0] + cam.R[1][i] * cam.t[1]) + cam.R[2][i] * cam.t[2]);
@@ -1139,7 +1185,29 @@ void or_projection_bwd(int64_t N, int sh_degree, const float* means, const float
                 vS[k][l] = s;
             }
         const float vm0 = v_xy[2 * g], vm1 = v_xy[2 * g + 1];
-        if (cam.model == OR_CAM_PINHOLE) {
+        if (lens_path(cam)) {
+            // bwd_diff of *_proj_uv and of its forward-mode Jacobian (projection_utils.slang:362-375,
+            // 463-493): v_p = J^T v_uv + sum_ij v_J[i][j] dJ[i][j]/dp, with dJ/dp the Hessians of the
+            // two pixel coordinates; a clamped J[i][2] (perspective only) depends on z through its bound.
+            typedef SsrJet<3, 2> Jet;
+            Jet px, py;
+            ssr_model_pixel<Jet>(cam.model, cam.tier, cam.dc, cam.fx, cam.fy, cam.cx, cam.cy, ssr_jet_seed<3, 2>(x, 0),
+                                 ssr_jet_seed<3, 2>(y, 1), ssr_jet_seed<3, 2>(z, 2), px, py);
+            const float iz2 = 1.0f / (z * z);
+            const float Wf = (float)cam.W;
+            const float lim_pos = Wf + 0.3f * (0.5f * Wf), lim_neg = 0.3f * (0.5f * Wf);
+            const float bound_lo[2] = {-(lim_pos - cam.cx), -(lim_pos - cam.cy)}, bound_hi[2] = {lim_neg + cam.cx, lim_neg + cam.cy};
+            for (int i = 0; i < 2; i++) {
+                const Jet& f = i == 0 ? px : py;
+                const float vm = i == 0 ? vm0 : vm1;
+                for (int k = 0; k < 3; k++) vmc[k] += vm * f.d[k];
+                for (int j = 0; j < 3; j++) {
+                    if (j == 2 && p.clamp_lo[i]) { vmc[2] += vJ[i][2] * bound_lo[i] * (-iz2); continue; }
+                    if (j == 2 && p.clamp_hi[i]) { vmc[2] += vJ[i][2] * bound_hi[i] * (-iz2); continue; }
+                    for (int k = 0; k < 3; k++) vmc[k] += vJ[i][j] * f.h[j <= k ? ssr_jet_idx<3>(j, k) : ssr_jet_idx<3>(k, j)];
+                }
+            }
+        } else if (cam.model == OR_CAM_PINHOLE) {
             const float z2 = z * z, iz = 1.0f / z, iz2 = 1.0f / z2;
             vmc[2] += vJ[0][0] * (-cam.fx * iz2) + vJ[1][1] * (-cam.fy * iz2);
             const float Wf = (float)cam.W;

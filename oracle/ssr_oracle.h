@@ -25,7 +25,8 @@
 extern "C" {
 #endif
 
-enum { OR_CAM_PINHOLE = 0, OR_CAM_EQUIRECT = 3 };            /* src/core/Common.cuh CameraModelType */
+enum { OR_CAM_PINHOLE = 0, OR_CAM_FISHEYE = 1, OR_CAM_EQUISOLID = 2, OR_CAM_EQUIRECT = 3 };   /* src/core/Common.cuh CameraModelType */
+enum { OR_LENS_NONE = 0, OR_LENS_OPENCV = 1, OR_LENS_THIN_PRISM = 2, OR_LENS_RATIONAL = 3 };   /* CameraDistortionType, src/shaders/projection_utils.slang:220-225 */
 enum { OR_SH_F32 = 0, OR_SH_REF_Q8 = 1, OR_SH_REF_Q16 = 2, OR_SH_I8_F16SCALE = 3 };
 
 typedef struct {
@@ -33,6 +34,8 @@ typedef struct {
     uint32_t width, height;
     float viewmat[16];      /* row-major world->camera [R t; 0 1] */
     float fx, fy, cx, cy;
+    int32_t distortion;     /* OR_LENS_* */
+    float dist_coeffs[8];   /* in the tier's own order, src/shaders/projection_utils.slang:242-295 */
 } or_camera;
 
 typedef struct {

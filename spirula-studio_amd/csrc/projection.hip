@@ -47,7 +47,7 @@ __device__ __forceinline__ void sh_colour(const ssr_world& W, const ssr_sh_quant
 // listed splats, so the expensive part runs on dense wavefronts however sparse visibility is.
 // (Running phase 2 as a kernel of its own over the global list was measured and is slower in every
 // configuration, sparse or dense.)
-template <int kDegree>
+template <int kDegree, bool kLens>
 __global__ __launch_bounds__(kProjBlock) void projection_fwd_kernel(ssr_projection_fwd_params P) {
     __shared__ int s_list[kProjBlock];
     __shared__ int s_count;
@@ -61,7 +61,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_fwd_kernel(ssr_projecti
         float mean[3], quat[4], ls[3], logit;
         load_splat(P.world, g, mean, quat, ls, logit);
         ProjD p;
-        project<false>(cam, mean, quat, ls, logit, p);
+        project<false, kLens>(cam, mean, quat, ls, logit, p);
         float bb[4] = {p.aabb[0], p.aabb[1], p.aabb[2], p.aabb[3]};
         bb[0] = ssr_min(ssr_max(bb[0], 0.0f), cam.Wf - 1.0f);
         bb[1] = ssr_min(ssr_max(bb[1], 0.0f), cam.Hf - 1.0f);
@@ -184,6 +184,7 @@ inline size_t packed_stage_layout(int64_t n, void* base, PackedStage* st) {
 // projected geometry of the visible splats is kept: compacted in splat order within the
 // workgroup's segment of the staging area (ballot ranks inside a wavefront, wavefront totals through
 // LDS), so that the second pass never touches a culled splat.
+template <bool kLens>
 __global__ __launch_bounds__(kProjBlock) void projection_packed_mask_kernel(ssr_projection_packed_params P, PackedStage S) {
     __shared__ int s_wave[kProjBlock / 64];
     const int64_t block0 = (int64_t)blockIdx.x * kProjBlock;
@@ -195,7 +196,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_packed_mask_kernel(ssr_
     if (g < P.num_splats) {
         float mean[3], quat[4], ls[3], logit;
         load_splat(P.world, g, mean, quat, ls, logit);
-        project<false>(cam, mean, quat, ls, logit, p);
+        project<false, kLens>(cam, mean, quat, ls, logit, p);
         bb[0] = ssr_min(ssr_max(p.aabb[0], 0.0f), cam.Wf - 1.0f);
         bb[1] = ssr_min(ssr_max(p.aabb[1], 0.0f), cam.Hf - 1.0f);
         bb[2] = ssr_min(ssr_max(p.aabb[2], 0.0f), cam.Wf - 1.0f);
@@ -338,14 +339,14 @@ __device__ __forceinline__ VScreenD vscreen_of(const ssr_screen& s, const float*
     return VScreenD{s.xy, s.depth, s.conic, s.opac, s.rgb, 2, 1, 3, 1, 3};
 }
 
-template <int kDegree, class ShSink>
+template <int kDegree, bool kLens, class ShSink>
 __device__ __forceinline__ void projection_vjp(const CamD& cam, const ssr_world& W, const ssr_sh_quant& Q, int64_t g,
                                                const VScreenD& VS, int64_t r, WorldGradD& out, ShSink&& sh_sink) {
     constexpr int kCoef = kDegree * (kDegree + 2);
     float mean[3], quat[4], ls[3], logit;
     load_splat(W, g, mean, quat, ls, logit);
     ProjD p;
-    project<true>(cam, mean, quat, ls, logit, p);
+    project<true, kLens>(cam, mean, quat, ls, logit, p);
     const float x = p.mc[0], y = p.mc[1], z = p.mc[2];
     float vmc[3] = {0.f, 0.f, 0.f};
     // conic = inverse(cov2d)
@@ -386,7 +387,31 @@ __device__ __forceinline__ void projection_vjp(const CamD& cam, const ssr_world&
             vS[k][l] = s;
         }
     const float vm0 = VS.xy[VS.s_xy * r], vm1 = VS.xy[VS.s_xy * r + 1];
-    if (cam.model == SSR_CAM_PINHOLE) {
+    if (kLens) {
+        // uv, J and dJ/dp of the model from one second-order evaluation: v_p = J^T v_uv + sum_ij v_J[i][j] dJ[i][j]/dp.
+        // A clamped J[i][2] of the perspective camera is a function of z alone (its bound).
+        typedef SsrJet<3, 2> Jet;
+        Jet px, py;
+        ssr_model_pixel<Jet>(cam.model, cam.tier, cam.dc, cam.fx, cam.fy, cam.cx, cam.cy, ssr_jet_seed<3, 2>(x, 0),
+                             ssr_jet_seed<3, 2>(y, 1), ssr_jet_seed<3, 2>(z, 2), px, py);
+        const float iz2 = 1.0f / (z * z);
+        const float lim_pos = cam.Wf + 0.3f * (0.5f * cam.Wf), lim_neg = 0.3f * (0.5f * cam.Wf);
+        const float bound_lo[2] = {-(lim_pos - cam.cx), -(lim_pos - cam.cy)}, bound_hi[2] = {lim_neg + cam.cx, lim_neg + cam.cy};
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const Jet& f = i == 0 ? px : py;
+            const float vm = i == 0 ? vm0 : vm1;
+#pragma unroll
+            for (int k = 0; k < 3; k++) vmc[k] += vm * f.d[k];
+#pragma unroll
+            for (int j = 0; j < 3; j++) {
+                if (j == 2 && p.clamp_lo[i]) { vmc[2] += vJ[i][2] * bound_lo[i] * (-iz2); continue; }
+                if (j == 2 && p.clamp_hi[i]) { vmc[2] += vJ[i][2] * bound_hi[i] * (-iz2); continue; }
+#pragma unroll
+                for (int k = 0; k < 3; k++) vmc[k] += vJ[i][j] * f.h[j <= k ? ssr_jet_idx<3>(j, k) : ssr_jet_idx<3>(k, j)];
+            }
+        }
+    } else if (cam.model == SSR_CAM_PINHOLE) {
         const float z2 = z * z, iz = 1.0f / z, iz2 = 1.0f / z2;
         vmc[2] += vJ[0][0] * (-cam.fx * iz2) + vJ[1][1] * (-cam.fy * iz2);
         const float lim_pos = cam.Wf + 0.3f * (0.5f * cam.Wf), lim_neg = 0.3f * (0.5f * cam.Wf);
@@ -544,7 +569,7 @@ __device__ __forceinline__ void projection_vjp(const CamD& cam, const ssr_world&
     out.logit = vlogit;
 }
 
-template <int kDegree, bool kAccumulate>
+template <int kDegree, bool kAccumulate, bool kLens>
 __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projection_bwd_params P) {
     const int64_t i = (int64_t)blockIdx.x * kProjBlock + threadIdx.x;
     if (i >= (P.packed_gaussian_ids ? P.num_packed : (P.visible_ids ? P.n_visible : P.num_splats))) return;
@@ -569,7 +594,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
     const CamD cam = load_camera(P.camera);
     WorldGradD wg;
     float* vsh = V.features_sh + g * (int64_t)V.sh_stride;
-    projection_vjp<kDegree>(cam, P.world, P.sh, g, vscreen_of(P.v_screen, P.v_rows), r, wg, [&](int j, float Yj, const float vc[3]) {
+    projection_vjp<kDegree, kLens>(cam, P.world, P.sh, g, vscreen_of(P.v_screen, P.v_rows), r, wg, [&](int j, float Yj, const float vc[3]) {
         const float tv[3] = {Yj * vc[0], Yj * vc[1], Yj * vc[2]};
         const float d2 = dot3(tv, tv);
         const bool ok = ssr_isfinite(d2) && d2 != 0.0f;   // harmonics.slang:397-403
@@ -610,7 +635,7 @@ __device__ __forceinline__ float adam_step(float x, float v, float lr, const Ada
 // (Y_j * v_colour), so only its factors (15 + 3 floats) go to LDS. Phase 2, the workgroup streams
 // over its 256 x 3 kCoef SH coefficients in memory order: parameter and both moments are read and
 // written fully coalesced, the gradient is rebuilt from the factors in LDS.
-template <int kDegree>
+template <int kDegree, bool kLens>
 __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_kernel(ssr_fpbo_params P, AdamD scalar_adam) {
     constexpr int kCoef = kDegree * (kDegree + 2);
     constexpr int kY = kCoef > 0 ? kCoef : 1;
@@ -650,7 +675,7 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
             ssr_sh_quant none;
             none.codec = SSR_SH_F32; none.packed = nullptr; none.bounds = nullptr; none.bounds_stride = 0;
             none.num_sh_buffer = 0; none.scale_f16 = nullptr;
-            projection_vjp<kDegree>(cam, W, none, g, vscreen_of(P.v_screen, P.v_rows), g, pg, [&](int j, float Yj, const float vc[3]) {
+            projection_vjp<kDegree, kLens>(cam, W, none, g, vscreen_of(P.v_screen, P.v_rows), g, pg, [&](int j, float Yj, const float vc[3]) {
                 s_Y[threadIdx.x][j] = Yj;
                 if (j == 0) { s_vc[threadIdx.x][0] = vc[0]; s_vc[threadIdx.x][1] = vc[1]; s_vc[threadIdx.x][2] = vc[2]; }
             });
@@ -765,8 +790,10 @@ static int check_common(const char* where, int64_t n, int sh_degree, const ssr_w
                         const ssr_camera& cam) {
     SSR_REQUIRE(n >= 0 && n < (int64_t)1 << 31, where, "num_splats must be in [0, 2^31)");
     SSR_REQUIRE(sh_degree >= 0 && sh_degree <= 3, where, "SH degree must be 0..3");
-    SSR_REQUIRE(cam.camera_model == SSR_CAM_PINHOLE || cam.camera_model == SSR_CAM_EQUIRECT, where,
-                "unsupported camera model (PINHOLE and EQUIRECTANGULAR without distortion are built)");
+    SSR_REQUIRE(ssr_camera_variant_supported(cam.camera_model, cam.distortion), where,
+                "unsupported camera model / lens distortion pair (PINHOLE: none, opencv, thin prism, rational; FISHEYE and "
+                "EQUISOLID: none, opencv, thin prism; EQUIRECTANGULAR: none)");
+    SSR_REQUIRE(cam.distortion == SSR_LENS_NONE || cam.dist_coeffs, where, "null lens coefficients");
     SSR_REQUIRE(cam.num_cameras == 1, where, "exactly one camera per call is supported");
     SSR_REQUIRE(cam.width > 0 && cam.height > 0, where, "empty image");
     SSR_REQUIRE(cam.viewmats && cam.intrins, where, "null camera pointer");
@@ -811,12 +838,17 @@ extern "C" int ssr_projection_fwd(const ssr_projection_fwd_params* p, ssr_stream
     SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->packed_rows) & 15) == 0, "ssr_projection_fwd", "packed_rows must be 16-byte aligned");
     const dim3 grid((unsigned)ceil_div(p->num_splats, kProjBlock)), block(kProjBlock);
     hipStream_t s = as_stream(stream);
+    const bool lens = camera_needs_lens_path(p->camera.camera_model, p->camera.distortion);
+#define SSR_LAUNCH_FWD(D)                                                                          \
+    if (lens) hipLaunchKernelGGL((projection_fwd_kernel<D, true>), grid, block, 0, s, *p);         \
+    else hipLaunchKernelGGL((projection_fwd_kernel<D, false>), grid, block, 0, s, *p)
     switch (p->sh_degree) {
-        case 0: hipLaunchKernelGGL(projection_fwd_kernel<0>, grid, block, 0, s, *p); break;
-        case 1: hipLaunchKernelGGL(projection_fwd_kernel<1>, grid, block, 0, s, *p); break;
-        case 2: hipLaunchKernelGGL(projection_fwd_kernel<2>, grid, block, 0, s, *p); break;
-        default: hipLaunchKernelGGL(projection_fwd_kernel<3>, grid, block, 0, s, *p); break;
+        case 0: SSR_LAUNCH_FWD(0); break;
+        case 1: SSR_LAUNCH_FWD(1); break;
+        case 2: SSR_LAUNCH_FWD(2); break;
+        default: SSR_LAUNCH_FWD(3); break;
     }
+#undef SSR_LAUNCH_FWD
     SSR_CHECK_LAUNCH("ssr_projection_fwd");
     return 0;
 }
@@ -853,7 +885,10 @@ extern "C" int ssr_projection_packed_mask(const ssr_projection_packed_params* p,
     PackedStage st;
     packed_stage_layout(p->num_splats, p->scratch, &st);
     const int64_t nb = ceil_div(p->num_splats, kProjBlock);
-    hipLaunchKernelGGL(projection_packed_mask_kernel, dim3((unsigned)nb), dim3(kProjBlock), 0, s, *p, st);
+    if (camera_needs_lens_path(p->camera.camera_model, p->camera.distortion))
+        hipLaunchKernelGGL(projection_packed_mask_kernel<true>, dim3((unsigned)nb), dim3(kProjBlock), 0, s, *p, st);
+    else
+        hipLaunchKernelGGL(projection_packed_mask_kernel<false>, dim3((unsigned)nb), dim3(kProjBlock), 0, s, *p, st);
     SSR_CHECK_LAUNCH(where);
     hipLaunchKernelGGL(packed_block_scan_kernel, dim3(1), dim3(kScanOneBlock), 0, s, (const int32_t*)st.block_counts, nb,
                        st.block_offsets, p->nnz);
@@ -914,9 +949,15 @@ extern "C" int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream
     const int64_t work = packed ? p->num_packed : (p->visible_ids ? p->n_visible : p->num_splats);
     const dim3 grid((unsigned)ceil_div(work, kProjBlock)), block(kProjBlock);
     hipStream_t s = as_stream(stream);
-#define SSR_LAUNCH_BWD(D)                                                                          \
-    if (p->accumulate) hipLaunchKernelGGL((projection_bwd_kernel<D, true>), grid, block, 0, s, *p); \
-    else hipLaunchKernelGGL((projection_bwd_kernel<D, false>), grid, block, 0, s, *p)
+    const bool lens = camera_needs_lens_path(p->camera.camera_model, p->camera.distortion);
+#define SSR_LAUNCH_BWD(D)                                                                                     \
+    if (lens) {                                                                                               \
+        if (p->accumulate) hipLaunchKernelGGL((projection_bwd_kernel<D, true, true>), grid, block, 0, s, *p);  \
+        else hipLaunchKernelGGL((projection_bwd_kernel<D, false, true>), grid, block, 0, s, *p);               \
+    } else {                                                                                                  \
+        if (p->accumulate) hipLaunchKernelGGL((projection_bwd_kernel<D, true, false>), grid, block, 0, s, *p); \
+        else hipLaunchKernelGGL((projection_bwd_kernel<D, false, false>), grid, block, 0, s, *p);              \
+    }
     switch (p->sh_degree) {
         case 0: SSR_LAUNCH_BWD(0); break;
         case 1: SSR_LAUNCH_BWD(1); break;
@@ -951,12 +992,17 @@ extern "C" int ssr_fused_projection_bwd_optimizer(const ssr_fpbo_params* p, ssr_
     ad.b2c = (float)(1.0 / (1.0 - pow(0.999, (double)p->step)));
     const dim3 grid((unsigned)ceil_div(p->num_splats, kProjBlock)), block(kProjBlock);
     hipStream_t s = as_stream(stream);
+    const bool lens = camera_needs_lens_path(p->camera.camera_model, p->camera.distortion);
+#define SSR_LAUNCH_FPBO(D)                                                                                       \
+    if (lens) hipLaunchKernelGGL((fused_projection_bwd_optimizer_kernel<D, true>), grid, block, 0, s, *p, ad);    \
+    else hipLaunchKernelGGL((fused_projection_bwd_optimizer_kernel<D, false>), grid, block, 0, s, *p, ad)
     switch (p->sh_degree) {
-        case 0: hipLaunchKernelGGL(fused_projection_bwd_optimizer_kernel<0>, grid, block, 0, s, *p, ad); break;
-        case 1: hipLaunchKernelGGL(fused_projection_bwd_optimizer_kernel<1>, grid, block, 0, s, *p, ad); break;
-        case 2: hipLaunchKernelGGL(fused_projection_bwd_optimizer_kernel<2>, grid, block, 0, s, *p, ad); break;
-        default: hipLaunchKernelGGL(fused_projection_bwd_optimizer_kernel<3>, grid, block, 0, s, *p, ad); break;
+        case 0: SSR_LAUNCH_FPBO(0); break;
+        case 1: SSR_LAUNCH_FPBO(1); break;
+        case 2: SSR_LAUNCH_FPBO(2); break;
+        default: SSR_LAUNCH_FPBO(3); break;
     }
+#undef SSR_LAUNCH_FPBO
     SSR_CHECK_LAUNCH(where);
     return 0;
 }

@@ -1,25 +1,34 @@
 // projection_device.h -- per-Gaussian projection and SH colour as device functions, shared by the
 // forward (K1) and backward (K9) kernels.
 //
-// Follows projection_3dgs<camera_model, DistNone, assume_valid, eval3d=false>
-// (src/shaders/primitive_3dgs.slang:419-578), persp_proj_3dgs (:63-99), equirect_proj_3dgs
-// (:194-211), quat_scale_to_covar / covarW2C / inverse (src/shaders/projection_utils.slang:69-174),
+// Follows projection_3dgs<camera_model, D, assume_valid, eval3d=false>
+// (src/shaders/primitive_3dgs.slang:419-578), persp_proj_3dgs (:63-99), fisheye_proj_3dgs /
+// equisolid_proj_3dgs (:148-192), equirect_proj_3dgs (:194-211), quat_scale_to_covar / covarW2C / inverse (src/shaders/projection_utils.slang:69-174),
 // view_radius_3dgs (:1033-1043) and sh_coeffs_to_color (src/shaders/harmonics.slang:154-251).
 //
 // Every expression is evaluated in the order written, without contraction, so that the outputs
 // that feed tile keys (extents, sorting depth, conic, opacity) have one defined bit pattern.
 #pragma once
 #include "common.h"
+#include "../../include/ssr_camera.h"
 
 namespace ssr {
 
 struct CamD {
     int model;
+    int tier;          // lens distortion tier, SSR_LENS_*
     float Wf, Hf;
     float R[3][3];
     float t[3];
     float fx, fy, cx, cy;
+    float dc[8];       // lens coefficients (zero without distortion)
 };
+
+// PINHOLE without lens distortion and EQUIRECTANGULAR have hand-written Jacobians; every other pair
+// goes through the differentiated model functions of ssr_camera.h (kLens instantiations).
+__host__ __device__ __forceinline__ bool camera_needs_lens_path(int model, int tier) {
+    return !((model == SSR_CAM_PINHOLE && tier == SSR_LENS_NONE) || model == SSR_CAM_EQUIRECT);
+}
 
 __device__ __forceinline__ CamD load_camera(const ssr_camera& c) {
     // src/kernels/projection/ProjectionFwd_kernel.cuh:52-60 (row-major [R t; 0 1])
@@ -33,6 +42,9 @@ __device__ __forceinline__ CamD load_camera(const ssr_camera& c) {
         k.t[i] = c.viewmats[4 * i + 3];
     }
     k.fx = c.intrins[0]; k.fy = c.intrins[1]; k.cx = c.intrins[2]; k.cy = c.intrins[3];
+    k.tier = c.distortion;
+#pragma unroll
+    for (int i = 0; i < 8; i++) k.dc[i] = (c.distortion != SSR_LENS_NONE) ? c.dist_coeffs[i] : 0.0f;
     return k;
 }
 
@@ -59,7 +71,22 @@ __device__ __forceinline__ float view_radius(const float mean[3], const float ls
     return radius / (ssr_max(dist, radius) + ssr_sqrt(ssr_max(dist * dist - radius * radius, 0.0f)));
 }
 
-template <bool kAssumeValid>
+// J[.][2] of a perspective camera is clamped to the cone of the (enlarged) image,
+// src/shaders/primitive_3dgs.slang:84-95; the y limits reuse the x limits as written there.
+__device__ __forceinline__ void clamp_pinhole_jacobian(const CamD& cam, float z, ProjD& p) {
+    float (*J)[3] = p.J;
+    const float lim_pos = cam.Wf + 0.3f * (0.5f * cam.Wf);
+    const float lim_neg = 0.3f * (0.5f * cam.Wf);
+    const float rz = 1.f / z;
+    const float max_x = (-((-lim_neg) - cam.cx)) * rz, min_x = (-(lim_pos - cam.cx)) * rz;
+    const float max_y = (-((-lim_neg) - cam.cy)) * rz, min_y = (-(lim_pos - cam.cy)) * rz;
+    p.clamp_lo[0] = J[0][2] < min_x; p.clamp_hi[0] = !p.clamp_lo[0] && J[0][2] > max_x;
+    p.clamp_lo[1] = J[1][2] < min_y; p.clamp_hi[1] = !p.clamp_lo[1] && J[1][2] > max_y;
+    J[0][2] = ssr_min(ssr_max(J[0][2], min_x), max_x);
+    J[1][2] = ssr_min(ssr_max(J[1][2], min_y), max_y);
+}
+
+template <bool kAssumeValid, bool kLens = false>
 __device__ __forceinline__ void project(const CamD& cam, const float mean[3], const float quat[4],
                                         const float ls[3], float logit, ProjD& p) {
     p.valid = false;
@@ -115,22 +142,26 @@ __device__ __forceinline__ void project(const CamD& cam, const float mean[3], co
 
     float (*J)[3] = p.J;
     p.clamp_lo[0] = p.clamp_lo[1] = p.clamp_hi[0] = p.clamp_hi[1] = false;
-    if (cam.model == SSR_CAM_PINHOLE) {
+    if (kLens) {
+        // *_proj<D, assume_valid> and *_proj_jac<D>: uv and its Jacobian from one first-order evaluation
+        typedef SsrJet<3, 1> Jet;
+        const Jet jx = ssr_jet_seed<3, 1>(x, 0), jy = ssr_jet_seed<3, 1>(y, 1), jz = ssr_jet_seed<3, 1>(z, 2);
+        Jet u, v, du, dv;
+        ssr_model_normalised<Jet>(cam.model, jx, jy, jz, u, v);
+        if (!kAssumeValid && !ssr_distortion_valid(cam.tier, cam.dc, u.v, v.v)) return;
+        ssr_distort<Jet>(cam.tier, cam.dc, u, v, du, dv);
+        const Jet px = du * cam.fx + cam.cx, py = dv * cam.fy + cam.cy;
+        p.xy[0] = px.v; p.xy[1] = py.v;
+#pragma unroll
+        for (int k = 0; k < 3; k++) { J[0][k] = px.d[k]; J[1][k] = py.d[k]; }
+        if (cam.model == SSR_CAM_PINHOLE) clamp_pinhole_jacobian(cam, z, p);
+    } else if (cam.model == SSR_CAM_PINHOLE) {
         const float z2 = z * z;
         p.xy[0] = cam.fx * (x / z) + cam.cx;
         p.xy[1] = cam.fy * (y / z) + cam.cy;
         J[0][0] = (z / z2) * cam.fx; J[0][1] = 0.0f; J[0][2] = ((0.0f - x) / z2) * cam.fx;
         J[1][0] = 0.0f; J[1][1] = (z / z2) * cam.fy; J[1][2] = ((0.0f - y) / z2) * cam.fy;
-        const float lim_pos = cam.Wf + 0.3f * (0.5f * cam.Wf);
-        const float lim_neg = 0.3f * (0.5f * cam.Wf);
-        const float rz = 1.f / z;
-        // the y limits reuse the x limits (src/shaders/primitive_3dgs.slang:92-93)
-        const float max_x = (-((-lim_neg) - cam.cx)) * rz, min_x = (-(lim_pos - cam.cx)) * rz;
-        const float max_y = (-((-lim_neg) - cam.cy)) * rz, min_y = (-(lim_pos - cam.cy)) * rz;
-        p.clamp_lo[0] = J[0][2] < min_x; p.clamp_hi[0] = !p.clamp_lo[0] && J[0][2] > max_x;
-        p.clamp_lo[1] = J[1][2] < min_y; p.clamp_hi[1] = !p.clamp_lo[1] && J[1][2] > max_y;
-        J[0][2] = ssr_min(ssr_max(J[0][2], min_x), max_x);
-        J[1][2] = ssr_min(ssr_max(J[1][2], min_y), max_y);
+        clamp_pinhole_jacobian(cam, z, p);
     } else {
         const float h2 = x * x + z * z;
         const float h = ssr_sqrt(h2);
@@ -153,6 +184,16 @@ __device__ __forceinline__ void project(const CamD& cam, const float mean[3], co
 #pragma unroll
         for (int j = 0; j < 2; j++)
             p.c2[i][j] = (jc[i][0] * J[j][0] + jc[i][1] * J[j][1]) + jc[i][2] * J[j][2];
+    if (kLens && !kAssumeValid && (cam.model == SSR_CAM_FISHEYE || cam.model == SSR_CAM_EQUISOLID)) {
+        // a splat behind a wide lens that still reaches the image centre with visible opacity is dropped,
+        // src/shaders/primitive_3dgs.slang:509-514 (before the blur is added)
+        const float m0 = p.xy[0] - cam.cx, m1 = p.xy[1] - cam.cy;
+        const float idet = 1.0f / (p.c2[0][0] * p.c2[1][1] - p.c2[0][1] * p.c2[1][0]);
+        const float i00 = p.c2[1][1] * idet, i01 = (-p.c2[0][1]) * idet, i10 = (-p.c2[1][0]) * idet, i11 = p.c2[0][0] * idet;
+        const float q = (i00 * m0 + i01 * m1) * m0 + (i10 * m0 + i11 * m1) * m1;
+        const float seen = p.opac * ssr_exp(-0.5f * q);
+        if (z < 0.0f && seen > kAlphaThreshold) return;
+    }
     p.c2[0][0] = p.c2[0][0] + 0.3f;   // add_blur, not antialiased
     p.c2[1][1] = p.c2[1][1] + 0.3f;
     const float det = p.c2[0][0] * p.c2[1][1] - p.c2[0][1] * p.c2[1][0];
@@ -169,7 +210,10 @@ __device__ __forceinline__ void project(const CamD& cam, const float mean[3], co
     const float xmin = p.xy[0] - rx, xmax = p.xy[0] + rx, ymin = p.xy[1] - ry, ymax = p.xy[1] + ry;
     if (xmax <= 0 || xmin >= cam.Wf || ymax <= 0 || ymin >= cam.Hf) return;
     p.aabb[0] = xmin; p.aabb[1] = ymin; p.aabb[2] = xmax; p.aabb[3] = ymax;
-    p.sort_depth = (cam.model == SSR_CAM_PINHOLE) ? z : dot3(p.mc, p.mc);
+    // get_sorting_depth, src/shaders/projection_utils.slang:1012-1029
+    if (cam.model == SSR_CAM_PINHOLE) p.sort_depth = z;
+    else if (cam.model == SSR_CAM_EQUIRECT) p.sort_depth = dot3(p.mc, p.mc);
+    else p.sort_depth = ((z * z) * z) * z + ((1.0f / 512.0f) * (x * x + y * y)) * (x * x + y * y);
     float campos[3];
 #pragma unroll
     for (int i = 0; i < 3; i++)

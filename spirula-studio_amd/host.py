@@ -21,7 +21,7 @@ SYMBOLS = {
     "ssrh_set_options": (C.c_int, [C.c_int] * 8),
     "ssrh_set_data_3dgs": (C.c_int, [C.c_int64, vp, vp, vp, vp, vp, vp, C.c_int]),
     "ssrh_set_sh_value_quant": (C.c_int, [C.c_int, vp, C.c_int64, C.c_int, vp, C.c_int64, C.c_int, C.c_int64]),
-    "ssrh_set_camera_params": (C.c_int, [C.c_int, C.c_int, C.c_char_p, C.c_char_p, vp, vp, C.c_int]),
+    "ssrh_set_camera_params": (C.c_int, [C.c_int, C.c_int, C.c_char_p, C.c_char_p, vp, vp, vp, C.c_int]),
     "ssrh_backward_with_variants": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, C.c_int]),
     "ssrh_backward_fused_optimizer": (C.c_int, [vp, vp, vp, vp, C.c_int]),
     "ssrh_copy_params_to_host": (C.c_int, [vp, vp, vp, vp, vp, vp]),
@@ -60,7 +60,8 @@ def check(rc):
         raise _lib.SsrError(load().ssrh_last_error().decode() or f"host error {rc}")
 
 
-_MODEL = {0: b"PINHOLE", 3: b"EQUIRECTANGULAR"}
+_MODEL = {0: b"PINHOLE", 1: b"FISHEYE", 2: b"EQUISOLID", 3: b"EQUIRECTANGULAR"}
+_LENS = {0: b"NONE", 1: b"OPENCV", 2: b"THIN_PRISM", 3: b"RATIONAL"}
 
 CACHE = dict(aabb=(0, np.float32), sort_depth=(1, np.float32), xy=(2, np.float32), depth=(3, np.float32),
              conic=(4, np.float32), opac=(5, np.float32), rgb=(6, np.float32), sorted_ids=(7, np.int64),
@@ -108,8 +109,10 @@ class Engine:
             check(self.h.ssrh_set_sh_value_quant(bits, packed.ctypes.data, packed.size, packed.itemsize,
                                                  bounds.ctypes.data, bounds.shape[0], be, scene.sh_bounds_stride))
         vm, it = f32(scene.viewmat), f32(scene.intrins)
-        check(self.h.ssrh_set_camera_params(scene.width, scene.height, _MODEL[scene.camera_model], b"NONE",
-                                            vm.ctypes.data, it.ctypes.data, 1))
+        tier = int(getattr(scene, "distortion", 0))
+        dc = f32(np.zeros(8) if getattr(scene, "dist_coeffs", None) is None else scene.dist_coeffs)
+        check(self.h.ssrh_set_camera_params(scene.width, scene.height, _MODEL[scene.camera_model], _LENS[tier],
+                                            vm.ctypes.data, it.ctypes.data, dc.ctypes.data, 1))
         # cotangents resident on the device
         self.d_vrgb = _lib.DeviceArray.from_host(f32(scene.v_rgb))
         self.d_vdepth = _lib.DeviceArray.from_host(f32(scene.v_depth))

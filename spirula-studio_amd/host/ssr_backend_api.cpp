@@ -51,15 +51,24 @@ struct StageTimer {
     }
 };
 
+// camera_model_from_name / camera_distortion_from_name (src/core/CameraModel.h:64-71,165-183), with the
+// lower-case spellings this harness has always accepted
 int camera_model_of(const std::string& m) {
-    if (m == "PINHOLE" || m == "pinhole") return SSR_CAM_PINHOLE;
+    if (m == "PINHOLE" || m == "pinhole" || m == "SIMPLE_PINHOLE" || m == "SIMPLE_RADIAL" || m == "RADIAL" || m == "OPENCV")
+        return SSR_CAM_PINHOLE;
+    if (m == "FISHEYE" || m == "fisheye" || m == "SIMPLE_FISHEYE" || m == "SIMPLE_RADIAL_FISHEYE" || m == "RADIAL_FISHEYE" ||
+        m == "OPENCV_FISHEYE" || m == "THIN_PRISM_FISHEYE")
+        return SSR_CAM_FISHEYE;
+    if (m == "EQUISOLID" || m == "equisolid") return SSR_CAM_EQUISOLID;
     if (m == "EQUIRECTANGULAR" || m == "equirectangular" || m == "EQUIRECT") return SSR_CAM_EQUIRECT;
-    throw std::runtime_error("projection: camera model '" + m + "' is not built in this backend "
-                             "(PINHOLE and EQUIRECTANGULAR are)");
+    throw std::runtime_error("projection: unknown camera model '" + m + "'");
 }
-void require_no_distortion(const std::string& d) {
-    if (!(d == "NONE" || d == "none" || d.empty()))
-        throw std::runtime_error("projection: distortion tier '" + d + "' is not built in this backend (NONE is)");
+int lens_tier_of(const std::string& d) {
+    if (d == "NONE" || d == "none" || d.empty()) return SSR_LENS_NONE;
+    if (d == "OPENCV" || d == "opencv") return SSR_LENS_OPENCV;
+    if (d == "THIN_PRISM" || d == "thin_prism") return SSR_LENS_THIN_PRISM;
+    if (d == "RATIONAL" || d == "rational") return SSR_LENS_RATIONAL;
+    throw std::runtime_error("projection: unknown distortion tier '" + d + "'");
 }
 
 ssr_world world_of(const std::vector<DeviceTensorFloatND>& s) {
@@ -97,10 +106,21 @@ ssr_sh_quant sh_of(const std::optional<TorchTensorView>& packed, const std::opti
     }
     return q;
 }
-ssr_camera camera_of(const std::string& model, const TorchTensorView& viewmats, const TorchTensorView& intrins,
-                     uint32_t w, uint32_t h) {
+ssr_camera camera_of(const std::string& model, const std::string& distortion, const TorchTensorView& dist_coeffs,
+                     const TorchTensorView& viewmats, const TorchTensorView& intrins, uint32_t w, uint32_t h) {
     ssr_camera c;
     c.camera_model = camera_model_of(model);
+    c.distortion = lens_tier_of(distortion);
+    // camera_distortion_is_compiled, src/core/CameraModel.h:154-162
+    const bool wide = c.camera_model == SSR_CAM_FISHEYE || c.camera_model == SSR_CAM_EQUISOLID;
+    if ((wide && c.distortion == SSR_LENS_RATIONAL) || (c.camera_model == SSR_CAM_EQUIRECT && c.distortion != SSR_LENS_NONE))
+        throw std::runtime_error("projection: camera model '" + model + "' has no '" + distortion + "' distortion tier");
+    c.dist_coeffs = (const float*)std::get<0>(dist_coeffs);
+    if (c.distortion != SSR_LENS_NONE) {
+        const auto& ds = std::get<2>(dist_coeffs);
+        if (!c.dist_coeffs || ds.size() != 2 || ds[1] != 8)
+            throw std::runtime_error("projection: distortion needs a [num_cameras, 8] coefficient tensor");
+    }
     const auto& shape = std::get<2>(viewmats);
     c.num_cameras = shape.empty() ? 0u : (uint32_t)shape[0];
     if (c.num_cameras != 1) throw std::runtime_error("this backend runs one camera per call (got " + std::to_string(c.num_cameras) + ")");
@@ -204,18 +224,17 @@ std::tuple<DeviceTensor2D<float4>, DeviceTensor2D<float>, std::vector<DeviceTens
 projection_3dgs_forward(const int64_t num_splats, const int max_sh_degree,
                         const std::vector<DeviceTensorFloatND>& in_splats, TorchTensorView viewmats,
                         TorchTensorView intrins, const uint32_t image_width, const uint32_t image_height,
-                        const std::string camera_model, const std::string distortion, const TorchTensorView,
+                        const std::string camera_model, const std::string distortion, const TorchTensorView dist_coeffs,
                         DeviceVector<float> radii, const std::optional<TorchTensorView> sh_value_packed,
                         const std::optional<TorchTensorView> sh_value_bounds, const uint32_t num_sh_buffer,
                         const int sh_value_bits, const int64_t sh_bounds_stride) {
-    require_no_distortion(distortion);
     ssr_projection_fwd_params p;
     std::memset(&p, 0, sizeof(p));
     p.num_splats = num_splats;
     p.sh_degree = max_sh_degree;
     p.world = world_of(in_splats);
     p.sh = sh_of(sh_value_packed, sh_value_bounds, num_sh_buffer, sh_value_bits, sh_bounds_stride);
-    p.camera = camera_of(camera_model, viewmats, intrins, image_width, image_height);
+    p.camera = camera_of(camera_model, distortion, dist_coeffs, viewmats, intrins, image_width, image_height);
     const int64_t C = 1, N = num_splats;
 
     DeviceTensor2D<float4> aabb; aabb.resize(PoolSlot::ProjAabb, C, N);
@@ -266,18 +285,17 @@ std::tuple<DeviceVector<int32_t>, DeviceVector<int32_t>, DeviceVector<float4>, D
 projection_3dgs_packed_forward(const int64_t num_splats, const int max_sh_degree,
                                const std::vector<DeviceTensorFloatND>& in_splats, TorchTensorView viewmats,
                                TorchTensorView intrins, const uint32_t image_width, const uint32_t image_height,
-                               const std::string camera_model, const std::string distortion, const TorchTensorView,
+                               const std::string camera_model, const std::string distortion, const TorchTensorView dist_coeffs,
                                DeviceVector<float> radii, const std::optional<TorchTensorView> sh_value_packed,
                                const std::optional<TorchTensorView> sh_value_bounds, const uint32_t num_sh_buffer,
                                const int sh_value_bits, const int64_t sh_bounds_stride) {
-    require_no_distortion(distortion);
     ssr_projection_packed_params p;
     std::memset(&p, 0, sizeof(p));
     p.num_splats = num_splats;
     p.sh_degree = max_sh_degree;
     p.world = world_of(in_splats);
     p.sh = sh_of(sh_value_packed, sh_value_bounds, num_sh_buffer, sh_value_bits, sh_bounds_stride);
-    p.camera = camera_of(camera_model, viewmats, intrins, image_width, image_height);
+    p.camera = camera_of(camera_model, distortion, dist_coeffs, viewmats, intrins, image_width, image_height);
     p.radii = radii.data_ptr();
     p.scratch_bytes = ssr_projection_packed_scratch_bytes(num_splats);
     p.scratch = DevicePool::global().acquire<uint8_t>(PoolSlot::ProjPackedScratch, p.scratch_bytes);
@@ -564,14 +582,13 @@ rasterize_to_pixels_3dgs_bwd(int64_t num_splats, std::vector<DeviceTensorFloatND
 void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
                               const std::vector<DeviceTensorFloatND>& splats_world, TorchTensorView viewmats,
                               TorchTensorView intrins, const uint32_t image_width, const uint32_t image_height,
-                              const std::string camera_model, const std::string distortion, const TorchTensorView,
+                              const std::string camera_model, const std::string distortion, const TorchTensorView dist_coeffs,
                               const DeviceVector<int32_t> camera_ids, const DeviceVector<int32_t> gaussian_ids,
                               const DeviceTensor2D<float4> aabb, const std::vector<DeviceTensorFloatND>& v_splats_screen,
                               const std::vector<DeviceTensorFloatND>& v_splats_world, DeviceTensor2D<float>* v_viewmats,
                               const std::optional<TorchTensorView> sh_value_packed,
                               const std::optional<TorchTensorView> sh_value_bounds, const uint32_t num_sh_buffer,
                               const int sh_value_bits, const int64_t sh_bounds_stride) {
-    require_no_distortion(distortion);
     if (v_viewmats) throw std::runtime_error("projection_3dgs_backward: camera pose gradients are not built in this backend");
     const bool is_packed = camera_ids.data_ptr() && gaussian_ids.data_ptr();   // src/kernels/projection/ProjectionBwd.cu:80
     g_bwd_list = nullptr; g_bwd_count = 0;
@@ -584,7 +601,7 @@ void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
     p.sh_degree = max_sh_degree;
     p.world = world_of(splats_world);
     p.sh = sh_of(sh_value_packed, sh_value_bounds, num_sh_buffer, sh_value_bits, sh_bounds_stride);
-    p.camera = camera_of(camera_model, viewmats, intrins, image_width, image_height);
+    p.camera = camera_of(camera_model, distortion, dist_coeffs, viewmats, intrins, image_width, image_height);
     p.aabb = (const float*)aabb.data_ptr();
     p.v_screen = screen_of(v_splats_screen);
     if (g_vrows && p.v_screen.xy == g_vrows_for_xy) p.v_rows = g_vrows;
@@ -606,7 +623,7 @@ void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
 void fused_projection_bwd_optimizer_3dgs(
     const int64_t num_splats, const int max_sh_degree, std::vector<DeviceTensorFloatND> splats_world,
     TorchTensorView viewmats, TorchTensorView intrins, const uint32_t image_width, const uint32_t image_height,
-    const std::string camera_model, const std::string distortion, const TorchTensorView,
+    const std::string camera_model, const std::string distortion, const TorchTensorView dist_coeffs,
     const DeviceVector<int32_t> camera_ids, const DeviceVector<int32_t> gaussian_ids, DeviceTensorFloatND aabb,
     const std::vector<DeviceTensorFloatND> v_splats_world, const std::vector<DeviceTensorFloatND> v_splats_screen,
     const std::vector<DeviceTensorFloatND> g1_splats_world, const std::vector<DeviceTensorFloatND> g2_splats_world,
@@ -619,7 +636,6 @@ void fused_projection_bwd_optimizer_3dgs(
     const float quat_norm_reg_weight, const float sh_reg_weight, bool use_scale_agnostic_mean, bool color_trust_linear,
     float, std::variant<int32_t, TorchTensorView> step, int quantization_level) {
     const char* w = "fused_projection_bwd_optimizer_3dgs: ";
-    require_no_distortion(distortion);
     if (camera_ids.data_ptr() || gaussian_ids.data_ptr()) throw std::runtime_error(std::string(w) + "packed mode is not built in this backend");
     if (sh_packed || non_sh.enabled || quantization_level != 0) throw std::runtime_error(std::string(w) + "quantized Adam state is not built in this backend");
     if (sh_value_packed) throw std::runtime_error(std::string(w) + "value-quantized SH is not built in this backend");
@@ -632,7 +648,7 @@ void fused_projection_bwd_optimizer_3dgs(
     p.num_splats = num_splats;
     p.sh_degree = max_sh_degree;
     p.world = world_of(splats_world);
-    p.camera = camera_of(camera_model, viewmats, intrins, image_width, image_height);
+    p.camera = camera_of(camera_model, distortion, dist_coeffs, viewmats, intrins, image_width, image_height);
     p.aabb = aabb.data_ptr();
     p.v_screen = screen_of(v_splats_screen);
     if (g_vrows && p.v_screen.xy == g_vrows_for_xy) p.v_rows = g_vrows;

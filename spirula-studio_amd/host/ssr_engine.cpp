@@ -401,12 +401,14 @@ int ssrh_set_sh_value_quant(int bits, const void* packed, int64_t packed_count, 
     return guard([&] { set_sh_value_quant(bits, tv(packed, (uint32_t)packed_elem, {packed_count}), tv(bounds, (uint32_t)bounds_elem, {bounds_count}), bounds_stride); });
 }
 
+// dist_coeffs: [num_cameras, 8] lens coefficients in the tier's order, or NULL for all zeros
 int ssrh_set_camera_params(int width, int height, const char* model, const char* distortion, const float* viewmats,
-                           const float* intrins, int num_cameras) {
+                           const float* intrins, const float* dist_coeffs, int num_cameras) {
     return guard([&] {
         static const float zero_coeffs[8 * 16] = {0};
+        if (!dist_coeffs && num_cameras > 16) throw std::runtime_error("set_camera_params: pass dist_coeffs for more than 16 cameras");
         set_camera_params(width, height, model, distortion, tv(viewmats, 4, {num_cameras, 4, 4}), tv(intrins, 4, {num_cameras, 4}),
-                          tv(zero_coeffs, 4, {num_cameras, 8}));
+                          tv(dist_coeffs ? dist_coeffs : zero_coeffs, 4, {num_cameras, 8}));
     });
 }
 

@@ -13,7 +13,8 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 SO_PATH = os.path.join(_HERE, "csrc", "libssr_hip.so")
 
-CAM_PINHOLE, CAM_EQUIRECT = 0, 3
+CAM_PINHOLE, CAM_FISHEYE, CAM_EQUISOLID, CAM_EQUIRECT = 0, 1, 2, 3
+LENS_NONE, LENS_OPENCV, LENS_THIN_PRISM, LENS_RATIONAL = 0, 1, 2, 3
 SH_F32, SH_REF_Q8, SH_REF_Q16, SH_I8_F16SCALE = 0, 1, 2, 3
 H2D, D2H, D2D, H2H, AUTO = 0, 1, 2, 3, 4
 
@@ -36,7 +37,8 @@ class ShQuant(C.Structure):
 
 class Camera(C.Structure):
     _fields_ = [("camera_model", C.c_int32), ("num_cameras", C.c_uint32), ("width", C.c_uint32),
-                ("height", C.c_uint32), ("viewmats", vp), ("intrins", vp)]
+                ("height", C.c_uint32), ("viewmats", vp), ("intrins", vp), ("dist_coeffs", vp),
+                ("distortion", C.c_int32)]
 
 
 class ProjectionFwdParams(C.Structure):

@@ -19,7 +19,17 @@ import os
 import numpy as np
 
 CAM_PINHOLE = 0         # src/core/Common.cuh CameraModelType
+CAM_FISHEYE = 1
+CAM_EQUISOLID = 2
 CAM_EQUIRECT = 3
+LENS_NONE, LENS_OPENCV, LENS_THIN_PRISM, LENS_RATIONAL = 0, 1, 2, 3   # CameraDistortionType, src/core/CameraModel.h:37-42
+# mild coefficient sets per tier (each in its own order), strong enough to move pixels by several percent
+LENS_PRESETS = {
+    0: [0, 0, 0, 0, 0, 0, 0, 0],
+    1: [0.05, -0.01, 0.002, -0.001, 0, 0, 0, 0],                        # k1 k2 p1 p2
+    2: [0.04, -0.008, 0.001, -0.0002, 0.001, -0.0015, 0.0008, -0.0005],  # k1 k2 k3 k4 p1 p2 sx1 sy1
+    3: [0.06, 0.01, 0.001, 0.02, 0.005, 0.0005, 0.001, -0.001],          # k1 k2 k3 k4 k5 k6 p1 p2
+}
 
 SH_F32 = 0              # fp32 coefficients
 SH_REF_Q8 = 1           # uint8 codes + per-block fp32 (min,max), src/core/Tensor.h:1313-1392
@@ -119,6 +129,8 @@ class Scene:
     sh_bounds: np.ndarray | None = None      # [n_bounds,2] float32 (reference codecs)
     sh_bounds_stride: int = 0
     sh_scale_f16: np.ndarray | None = None   # [N] float16 (int8 codec)
+    distortion: int = 0                      # lens distortion tier (LENS_*)
+    dist_coeffs: np.ndarray | None = None    # [8] float32 in the tier's own order
 
     @property
     def tile_w(self) -> int:
@@ -303,12 +315,23 @@ def subset(sc: Scene, idx: np.ndarray) -> Scene:
     return out
 
 
+def with_lens(sc: Scene, tier: int) -> Scene:
+    """The scene seen through a lens of the given distortion tier."""
+    return dataclasses.replace(sc, distortion=int(tier), dist_coeffs=np.array(LENS_PRESETS[int(tier)], np.float32))
+
+
 def tiny_scene(n: int = 300, width: int = 64, height: int = 48, seed: int = 7,
                camera_model: int = CAM_PINHOLE, big: bool = True) -> Scene:
     """A small scene with large, overlapping splats (many tiles per splat, early termination)."""
     if camera_model == CAM_PINHOLE:
         means = uniform(seed, 0, 3 * n, -1.0, 1.0).reshape(n, 3)
         t, f = (0, 0, 4), float(width)
+    elif camera_model in (CAM_FISHEYE, CAM_EQUISOLID):
+        # splats all around a camera whose image width spans 180 degrees: those behind it fall outside
+        d = normal(seed, 0, 3 * n, 0.0, 1.0).reshape(n, 3).astype(np.float64)
+        d /= np.maximum(np.sqrt((d * d).sum(axis=1, keepdims=True)), 1e-12)
+        means = (d * uniform(seed, 7, n, 2.0, 6.0).astype(np.float64)[:, None]).astype(np.float32)
+        t, f = (0, 0, 0), width / math.pi
     else:
         d = normal(seed, 0, 3 * n, 0.0, 1.0).reshape(n, 3).astype(np.float64)
         d /= np.maximum(np.sqrt((d * d).sum(axis=1, keepdims=True)), 1e-12)

@@ -83,6 +83,11 @@ class GpuRun:
         c.camera_model, c.num_cameras = self.sc.camera_model, 1
         c.width, c.height = self.sc.width, self.sc.height
         c.viewmats, c.intrins = self.ptr("viewmat"), self.ptr("intrins")
+        c.distortion = int(getattr(self.sc, "distortion", 0))
+        if "dist_coeffs" not in self.d:
+            dc = getattr(self.sc, "dist_coeffs", None)
+            self.d["dist_coeffs"] = self.L.DeviceArray.from_host(np.zeros(8, np.float32) if dc is None else np.asarray(dc, np.float32))
+        c.dist_coeffs = self.ptr("dist_coeffs")
         return c
 
     def screen(self, prefix=""):

@@ -14,7 +14,7 @@ _SO = os.path.join(_ROOT, "oracle", "libssr_oracle.so")
 class OrCamera(C.Structure):
     _fields_ = [("model", C.c_int32), ("width", C.c_uint32), ("height", C.c_uint32),
                 ("viewmat", C.c_float * 16), ("fx", C.c_float), ("fy", C.c_float),
-                ("cx", C.c_float), ("cy", C.c_float)]
+                ("cx", C.c_float), ("cy", C.c_float), ("distortion", C.c_int32), ("dist_coeffs", C.c_float * 8)]
 
 
 class OrShSource(C.Structure):
@@ -54,6 +54,10 @@ def camera_of(scene) -> OrCamera:
     for i in range(16):
         cam.viewmat[i] = float(vm[i])
     cam.fx, cam.fy, cam.cx, cam.cy = [float(v) for v in scene.intrins]
+    cam.distortion = int(getattr(scene, "distortion", 0))
+    dc = np.zeros(8, np.float32) if getattr(scene, "dist_coeffs", None) is None else np.asarray(scene.dist_coeffs, np.float32)
+    for i in range(8):
+        cam.dist_coeffs[i] = float(dc[i])
     return cam
 
 

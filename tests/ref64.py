@@ -18,7 +18,80 @@ def quat_rot(q):
         [2 * (x * z - w * y), 2 * (y * z + w * x), 1 - 2 * (x * x + y * y)]])
 
 
-def project(mean, quat, log_scale, logit, viewmat, intr, width, model, f32_consts=True):
+def lens_distort(tier, c, u, v):
+    """The distortion tiers of src/shaders/projection_utils.slang:235-295, written from the COLMAP model
+    definitions (OPENCV, THIN_PRISM_FISHEYE radial-first, FULL_OPENCV); works on complex numbers."""
+    if tier == 0:
+        return u, v
+    r2 = u * u + v * v
+    if tier == 1:
+        k1, k2, p1, p2 = c[:4]
+        radial, sx, sy = 1 + k1 * r2 + k2 * r2 ** 2, 0.0, 0.0
+    elif tier == 2:
+        k1, k2, k3, k4, p1, p2, sx, sy = c[:8]
+        radial = 1 + k1 * r2 + k2 * r2 ** 2 + k3 * r2 ** 3 + k4 * r2 ** 4
+    else:
+        k1, k2, k3, k4, k5, k6, p1, p2 = c[:8]
+        radial = (1 + k1 * r2 + k2 * r2 ** 2 + k3 * r2 ** 3) / (1 + k4 * r2 + k5 * r2 ** 2 + k6 * r2 ** 3)
+        sx = sy = 0.0
+    du = u * radial + 2 * p1 * u * v + p2 * (r2 + 2 * u * u) + sx * r2
+    dv = v * radial + 2 * p2 * u * v + p1 * (r2 + 2 * v * v) + sy * r2
+    return du, dv
+
+
+def model_normalised(model, x, y, z):
+    """(x/z, y/z); equidistant fisheye theta * (x, y)/r; equisolid 2 sin(theta/2) * (x, y)/r. Complex-safe:
+    inputs may carry an infinitesimal imaginary part (complex-step differentiation)."""
+    import cmath
+    if model == 0:
+        return x / z, y / z
+    r = cmath.sqrt(x * x + y * y)
+    # atan2 under complex-step differentiation: the real angle, plus i times its differential
+    rr, zr = complex(r).real, complex(z).real
+    theta = complex(math.atan2(rr, zr), (zr * complex(r).imag - rr * complex(z).imag) / (rr * rr + zr * zr))
+    if abs(r) < 1e-12:
+        k = 1.0 / z
+    elif model == 1:
+        k = theta / r
+    else:
+        k = 2 * cmath.sin(0.5 * theta) / r
+    return x * k, y * k
+
+
+def model_pixel(model, tier, coeffs, intr, p):
+    fx, fy, cx, cy = [float(v) for v in intr]
+    u, v = model_normalised(model, p[0], p[1], p[2])
+    du, dv = lens_distort(tier, [float(c) for c in coeffs], u, v)
+    return fx * du + cx, fy * dv + cy
+
+
+def model_jacobian(model, tier, coeffs, intr, p):
+    """d pixel / d p by complex-step differentiation (no subtraction, so exact to rounding)."""
+    J = np.zeros((2, 3))
+    h = 1e-30
+    for k in range(3):
+        q = [complex(v) for v in p]
+        q[k] += 1j * h
+        a, b = model_pixel(model, tier, coeffs, intr, q)
+        J[0, k], J[1, k] = a.imag / h, b.imag / h
+    return J
+
+
+def lens_valid(tier, coeffs, u, v):
+    """is_valid_distortion (src/shaders/projection_utils.slang:310-321), with central differences."""
+    if tier == 0:
+        return True, 1.0
+    c = [float(x) for x in coeffs]
+    h = 1e-6
+    a1, b1 = lens_distort(tier, c, u + h, v); a0, b0 = lens_distort(tier, c, u - h, v)
+    c1, d1 = lens_distort(tier, c, u, v + h); c0, d0 = lens_distort(tier, c, u, v - h)
+    j00, j10, j01, j11 = (a1 - a0) / (2 * h), (b1 - b0) / (2 * h), (c1 - c0) / (2 * h), (d1 - d0) / (2 * h)
+    jdet = min(j00 * j11 - j01 * j10, j00, j11)
+    du, dv = lens_distort(tier, c, u, v)
+    return (0.25 < jdet < 4.0) and (u * du + v * dv >= 0), jdet
+
+
+def project(mean, quat, log_scale, logit, viewmat, intr, width, model, f32_consts=True, tier=0, coeffs=None):
     """Returns xy(2), depth, conic(3), opac, plus cov2d (blurred) and the tile extents."""
     R, t = viewmat[:3, :3].astype(np.float64), viewmat[:3, 3].astype(np.float64)
     fx, fy, cx, cy = [float(v) for v in intr]
@@ -28,29 +101,42 @@ def project(mean, quat, log_scale, logit, viewmat, intr, width, model, f32_const
     S = np.diag(np.exp(log_scale))
     cov = Rq @ S @ S @ Rq.T
     covc = R @ cov @ R.T
-    if model == 0:
+    coeffs = np.zeros(8) if coeffs is None else np.asarray(coeffs, np.float64)
+    extra = {}
+    if model in (1, 2) or tier != 0:
+        a, b = model_pixel(model, tier, coeffs, intr, [complex(v) for v in pc])
+        xy = np.array([a.real, b.real])
+        J = model_jacobian(model, tier, coeffs, intr, pc)
+        u, v = model_normalised(model, complex(x), complex(y), complex(z))
+        extra["lens_valid"], extra["lens_jdet"] = lens_valid(tier, coeffs, u.real, v.real)
+    elif model == 0:
         xy = np.array([fx * x / z + cx, fy * y / z + cy])
         J = np.array([[fx / z, 0, -fx * x / z ** 2], [0, fy / z, -fy * y / z ** 2]])
-        c03 = float(np.float32(0.3)) if f32_consts else 0.3
-        lim_pos = width + c03 * (0.5 * width)
-        lim_neg = c03 * (0.5 * width)
-        # y limits reuse the x limits (src/shaders/primitive_3dgs.slang:92-93)
-        J[0, 2] = min(max(J[0, 2], -(lim_pos - cx) / z), (lim_neg + cx) / z)
-        J[1, 2] = min(max(J[1, 2], -(lim_pos - cy) / z), (lim_neg + cy) / z)
     else:
         h = math.hypot(x, z)
         r2 = x * x + y * y + z * z
         xy = np.array([fx * math.atan2(x, z) + cx, fy * math.atan2(y, h) + cy])
         J = np.array([[fx * z / h ** 2, 0, -fx * x / h ** 2],
                       [-fy * x * y / (h * r2), fy * h / r2, -fy * z * y / (h * r2)]])
+    if model == 0:
+        c03 = float(np.float32(0.3)) if f32_consts else 0.3
+        lim_pos = width + c03 * (0.5 * width)
+        lim_neg = c03 * (0.5 * width)
+        # y limits reuse the x limits (src/shaders/primitive_3dgs.slang:92-93)
+        J[0, 2] = min(max(J[0, 2], -(lim_pos - cx) / z), (lim_neg + cx) / z)
+        J[1, 2] = min(max(J[1, 2], -(lim_pos - cy) / z), (lim_neg + cy) / z)
     c2 = J @ covc @ J.T
+    opac = 1.0 / (1.0 + math.exp(-logit))
+    if model in (1, 2):
+        # the weight the unblurred splat still has at the image centre (src/shaders/primitive_3dgs.slang:509-514)
+        m = xy - np.array([cx, cy])
+        extra["centre_weight"] = opac * math.exp(-0.5 * float(m @ np.linalg.inv(c2) @ m))
     eps = float(np.float32(0.3)) if f32_consts else 0.3
     c2 = c2 + eps * np.eye(2)
     inv = np.linalg.inv(c2)
-    opac = 1.0 / (1.0 + math.exp(-logit))
     depth = float(np.linalg.norm(pc))
     return dict(xy=xy, depth=depth, conic=np.array([inv[0, 0], inv[0, 1], inv[1, 1]]), opac=opac,
-                cov2d=c2, pc=pc)
+                cov2d=c2, pc=pc, **extra)
 
 
 def real_sh_deg3(d):

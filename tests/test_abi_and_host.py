@@ -54,8 +54,17 @@ def test_argument_checks_without_device(L):
     p.num_splats, p.sh_degree = 10, 7
     assert lib.ssr_projection_fwd(C.byref(p), None) != 0 and b"SH degree" in lib.ssr_last_error()
     p.sh_degree = 3
-    p.camera.camera_model, p.camera.num_cameras, p.camera.width, p.camera.height = 1, 1, 8, 8
+    p.camera.camera_model, p.camera.num_cameras, p.camera.width, p.camera.height = 7, 1, 8, 8
     assert lib.ssr_projection_fwd(C.byref(p), None) != 0 and b"camera model" in lib.ssr_last_error()
+    # pairs the reference does not instantiate (src/kernels/projection/CameraVariants.cuh:11-22)
+    for model, tier in [(1, 3), (2, 3), (3, 1), (0, 4)]:
+        p.camera.camera_model, p.camera.distortion = model, tier
+        assert lib.ssr_projection_fwd(C.byref(p), None) != 0 and b"camera model" in lib.ssr_last_error()
+    p.camera.camera_model, p.camera.distortion = 1, 2
+    p.camera.viewmats = p.camera.intrins = 16     # non-null, never read: the coefficient check comes first
+    assert lib.ssr_projection_fwd(C.byref(p), None) != 0 and b"lens coefficients" in lib.ssr_last_error()
+    p.camera.viewmats = p.camera.intrins = None
+    p.camera.distortion = 0
     p.camera.camera_model, p.camera.num_cameras = 0, 2
     p.camera.viewmats = p.camera.intrins = 16
     assert lib.ssr_projection_fwd(C.byref(p), None) != 0 and b"one camera" in lib.ssr_last_error()

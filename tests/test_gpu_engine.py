@@ -68,6 +68,25 @@ def test_engine_quantized_and_equirect(pkg, oracle, H):
     _check(eng, ref, sc)
 
 
+def test_engine_wide_lens_cameras(pkg, oracle, H):
+    """The engine on a fisheye with a thin-prism lens and on a pinhole with the rational model: camera model
+    and distortion arrive as the reference's strings plus a [1, 8] coefficient row."""
+    host, lib = H
+    S = pkg.scenes
+    for model, tier in [(S.CAM_FISHEYE, S.LENS_THIN_PRISM), (S.CAM_EQUISOLID, S.LENS_NONE), (S.CAM_PINHOLE, S.LENS_RATIONAL)]:
+        sc = S.tiny_scene(n=3000, width=256, height=192, seed=51, camera_model=model)
+        if model == S.CAM_PINHOLE:
+            sc.intrins = np.array([150.0, 155.0, 128.0, 96.0], np.float32)
+            sc.viewmat[2, 3] = 2.6
+        sc = S.with_lens(sc, tier)
+        ref = oracle.pipeline(sc)
+        assert ref["proj"]["visible"] > 100
+        eng = host.Engine(sc)
+        eng.forward()
+        eng.backward()
+        _check(eng, ref, sc)
+
+
 def test_engine_overwrite_without_list(pkg, oracle, H):
     host, lib = H
     sc = pkg.scenes.make_scene(4, n=40000, width=480, height=270)
@@ -94,7 +113,7 @@ def test_lazy_gradient_zeroing_follows_the_camera(pkg, oracle, H):
     # look the other way: a different set of splats is visible
     sc.viewmat = np.array([[-1, 0, 0, 0], [0, 1, 0, 0], [0, 0, -1, 0.5], [0, 0, 0, 1]], np.float32)
     vm, it = np.ascontiguousarray(sc.viewmat), np.ascontiguousarray(sc.intrins, np.float32)
-    host.check(eng.h.ssrh_set_camera_params(sc.width, sc.height, b"PINHOLE", b"NONE", vm.ctypes.data, it.ctypes.data, 1))
+    host.check(eng.h.ssrh_set_camera_params(sc.width, sc.height, b"PINHOLE", b"NONE", vm.ctypes.data, it.ctypes.data, None, 1))
     eng.forward()
     eng.backward()
     ref2 = oracle.pipeline(sc)
@@ -160,7 +179,7 @@ def test_engine_packed_follows_the_camera_and_handles_nothing_visible(pkg, oracl
     def look(viewmat):
         sc.viewmat = np.asarray(viewmat, np.float32)
         vm, it = np.ascontiguousarray(sc.viewmat), np.ascontiguousarray(sc.intrins, np.float32)
-        host.check(eng.h.ssrh_set_camera_params(sc.width, sc.height, b"PINHOLE", b"NONE", vm.ctypes.data, it.ctypes.data, 1))
+        host.check(eng.h.ssrh_set_camera_params(sc.width, sc.height, b"PINHOLE", b"NONE", vm.ctypes.data, it.ctypes.data, None, 1))
         eng.forward()
         eng.backward()
         r = oracle.pipeline_packed(sc)
@@ -292,9 +311,12 @@ def test_unsupported_variants_raise(pkg, H):
     for dist in (3, 4):   # DN, RGB_DN: the 3dgs pixel has no normal channel
         assert h.ssrh_forward_3dgs(b"3dgs", 3, 0, 0, dist) != 0
         assert b"normal" in h.ssrh_last_error()
-    assert h.ssrh_set_camera_params(32, 32, b"FISHEYE", b"NONE", None, None, 1) == 0
-    assert h.ssrh_forward_3dgs(b"3dgs", 3, 0, 0, 0) != 0
-    assert b"FISHEYE" in h.ssrh_last_error()
+    vm, it = np.ascontiguousarray(sc.viewmat, np.float32), np.ascontiguousarray(sc.intrins, np.float32)
+    for model, lens, word in [(b"FISHEYE", b"RATIONAL", b"RATIONAL"), (b"EQUIRECTANGULAR", b"OPENCV", b"OPENCV"),
+                              (b"ORTHOGRAPHIC", b"NONE", b"ORTHOGRAPHIC"), (b"PINHOLE", b"BROWN", b"BROWN")]:
+        assert h.ssrh_set_camera_params(32, 32, model, lens, vm.ctypes.data, it.ctypes.data, None, 1) == 0
+        assert h.ssrh_forward_3dgs(b"3dgs", 3, 0, 0, 0) != 0
+        assert word in h.ssrh_last_error()
 
 
 def test_runtime_contract(pkg, H):

@@ -2,6 +2,8 @@
 inputs. Bars: tile keys / sorted ids / tile ranges bit-exact; images max-abs 1e-4 per channel;
 gradients 1e-3 relative (with a floor proportional to the sum of |terms|, since float atomics add
 in a different order)."""
+import math
+
 import numpy as np
 import pytest
 
@@ -230,6 +232,48 @@ def test_tile_segmented_sort(gpu, oracle):
     _compare(gpu, oracle, gpu.scenes.tiny_scene(n=900, width=160, height=96, seed=41), "mask-seg", mask=mask, tile_sort=True)
 
 
+CAMERA_PAIRS = [(0, 1), (0, 2), (0, 3), (1, 0), (1, 1), (1, 2), (2, 0), (2, 1), (2, 2)]
+
+
+def _lens_scene(gpu, model, tier, n=1500, seed=31, width=200, height=144):
+    S = gpu.scenes
+    sc = S.tiny_scene(n=n, width=width, height=height, seed=seed, camera_model=model)
+    if model == S.CAM_PINHOLE:   # a wide field of view, where the lens terms are not small
+        sc.intrins = np.array([0.6 * width, 0.62 * width, 0.5 * width, 0.5 * height], np.float32)
+        sc.viewmat[2, 3] = 2.6
+    return S.with_lens(sc, tier)
+
+
+@pytest.mark.parametrize("model,tier", CAMERA_PAIRS)
+def test_camera_variants(gpu, oracle, model, tier):
+    """FISHEYE / EQUISOLID and the lens-distortion tiers (every pair of
+    src/kernels/projection/CameraVariants.cuh:11-22 beyond the two hand-written ones): K1 bit-exact, and
+    through the whole path to the gradients."""
+    sc = _lens_scene(gpu, model, tier)
+    g, r = _compare(gpu, oracle, sc, f"model{model}-lens{tier}")
+    assert r["proj"]["visible"] > 100
+    _compare(gpu, oracle, sc, f"model{model}-lens{tier}-native", fused_count=True, use_list=True, use_packed=True,
+             use_vrows=True, tile_sort=True)
+
+
+def test_camera_variants_strong_lens_and_packed(gpu, oracle):
+    """A lens strong enough that is_valid_distortion drops part of the field; the packed projection on a
+    wide lens; a larger fisheye frame."""
+    sc = _lens_scene(gpu, 1, 2, n=2500, seed=37)
+    sc.dist_coeffs = (sc.dist_coeffs * np.float32(8.0)).astype(np.float32)
+    _compare(gpu, oracle, sc, "fisheye-strong-prism")
+    sc = _lens_scene(gpu, 0, 3, n=2500, seed=38)
+    sc.dist_coeffs = (sc.dist_coeffs * np.float32(-8.0)).astype(np.float32)
+    _compare(gpu, oracle, sc, "pinhole-strong-rational", fused_count=True, use_list=True)
+    _compare_packed(gpu, oracle, _lens_scene(gpu, 2, 1, n=2000, seed=39), "equisolid-opencv-packed", fused_count=True)
+    _compare_packed(gpu, oracle, _lens_scene(gpu, 0, 2, n=2000, seed=40), "pinhole-prism-packed", use_packed=True)
+    sc = gpu.scenes.make_scene(5, n=40000, width=768, height=768)
+    sc.camera_model = gpu.scenes.CAM_FISHEYE
+    sc.intrins = np.array([768 / math.pi, 768 / math.pi, 384, 384], np.float32)
+    _compare(gpu, oracle, gpu.scenes.with_lens(sc, 1), "cfg5-as-fisheye", fused_count=True, use_list=True, use_packed=True,
+             use_vrows=True, tile_sort=True)
+
+
 def test_tiny_equirect(gpu, oracle):
     _compare(gpu, oracle, gpu.scenes.tiny_scene(n=600, width=128, height=64, seed=4, camera_model=3), "tiny-eq")
 
@@ -322,7 +366,7 @@ def test_tile_skip_mask(gpu, oracle):
     assert r["counts"].max() > 96
 
 
-@pytest.mark.parametrize("cfg", ["tiny", "cfg2", "equirect-steps"])
+@pytest.mark.parametrize("cfg", ["tiny", "cfg2", "equirect-steps", "fisheye-prism"])
 def test_fused_projection_bwd_optimizer(gpu, oracle, cfg):
     """K9 fused with Adam (fused_projection_bwd_optimizer_3dgs, fp32 state): both sides are fed the
     SAME screen gradients (the device's), so only the arithmetic of the fused kernel is compared."""
@@ -335,6 +379,8 @@ def test_fused_projection_bwd_optimizer(gpu, oracle, cfg):
         sc.quats *= np.linspace(0.5, 2.0, sc.n)[:, None].astype(np.float32)
     elif cfg == "cfg2":
         sc = gpu.scenes.make_scene(2, n=40000, width=480, height=270, parity_variant=True)
+    elif cfg == "fisheye-prism":
+        sc = _lens_scene(gpu, 1, 2, n=3000, seed=43)
     else:
         sc = gpu.scenes.make_scene(5, n=30000, width=512, height=256)
     g = GpuRun(gpu, sc)
