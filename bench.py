@@ -12,6 +12,7 @@ kernel that takes the most time, and a `cpu_baseline` object (the CPU oracle tim
 """
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -95,6 +96,10 @@ def main():
                     help="run the stages exactly as the reference does (separate count pass, atomic K9 into zero-filled buffers)")
     ap.add_argument("--whole-key-sort", action="store_true",
                     help="six whole-array digit passes + the offsets kernel instead of the tile-segmented sort")
+    ap.add_argument("--lens", choices=["none", "opencv", "thin_prism", "rational"], default="none",
+                    help="widened row: the scene's camera with a lens-distortion tier (mild preset coefficients)")
+    ap.add_argument("--fisheye", action="store_true",
+                    help="widened row: view the scene through an equidistant fisheye spanning 180 degrees of the image width")
     ap.add_argument("--packed-projection", action="store_true",
                     help="run the packed form of the projection (compacted nnz-row outputs; the reference's training default)")
     ap.add_argument("--fused-optimizer", action="store_true",
@@ -131,6 +136,12 @@ def main():
     cfg = args.config
     t_gen = time.time()
     sc = pkg.scenes.make_scene(cfg, n=args.n)
+    if args.fisheye:
+        sc.camera_model = pkg.scenes.CAM_FISHEYE
+        f = sc.width / math.pi
+        sc.intrins = np.array([f, f, sc.width / 2.0, sc.height / 2.0], np.float32)
+    if args.lens != "none":
+        sc = pkg.scenes.with_lens(sc, ["none", "opencv", "thin_prism", "rational"].index(args.lens))
     t_gen = time.time() - t_gen
     native = not args.reference_order
     eng = host.Engine(sc, fuse_tile_count=native, visible_list=native and not args.packed_projection, packed_rows=native,
@@ -224,7 +235,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"config {cfg}: {sc.name}, N={sc.n}, {sc.width}x{sc.height}, "
-                               f"{'pinhole' if sc.camera_model == 0 else 'equirectangular'}, SH3 "
+                               f"{['pinhole', 'fisheye', 'equisolid', 'equirectangular'][sc.camera_model]}"
+                               f"{'' if not sc.distortion else ' + ' + args.lens + ' lens'}, SH3 "
                                f"{['fp32', 'ref-q8', 'ref-q16', 'int8*fp16scale'][sc.sh_codec]}, tile 16x16, seed {pkg.scenes.CONFIGS[cfg]['seed']:#x}",
                    "visible": V, "n_isects": K, "K_b": K_b, "tiles": T, "pixels": P,
                    "stage_order": ("fused tile count, visible-splat work list, packed fragment rows, packed gradient rows, plain-store gradients"

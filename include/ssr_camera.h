@@ -197,25 +197,27 @@ SSR_HD SsrJet<N, O> ssr_jet_sin_quarter(const SsrJet<N, O>& a) {
 template <class T>
 SSR_HD void ssr_distort(int tier, const float* c, const T& u, const T& v, T& ou, T& ov) {
     if (tier == SSR_TIER_NONE) { ou = u; ov = v; return; }
+    // all eight read up front, so that the tier selects among values, not among addresses
+    const float c0 = c[0], c1 = c[1], c2 = c[2], c3 = c[3], c4 = c[4], c5 = c[5], c6 = c[6], c7 = c[7];
     const T r2 = u * u + v * v;
     const T uv = u * v;
-    T radial, tx, ty;
-    float p1, p2;
+    T radial;
+    float p1, p2, s1 = 0.0f, s2 = 0.0f;
     if (tier == SSR_TIER_OPENCV) {             // k1 k2 p1 p2
-        radial = r2 * (r2 * c[1] + c[0]) + 1.0f;
-        p1 = c[2]; p2 = c[3];
+        radial = r2 * (r2 * c1 + c0) + 1.0f;
+        p1 = c2; p2 = c3;
     } else if (tier == SSR_TIER_THIN_PRISM) {  // k1 k2 k3 k4 p1 p2 sx1 sy1
-        radial = r2 * (r2 * (r2 * (r2 * c[3] + c[2]) + c[1]) + c[0]) + 1.0f;
-        p1 = c[4]; p2 = c[5];
+        radial = r2 * (r2 * (r2 * (r2 * c3 + c2) + c1) + c0) + 1.0f;
+        p1 = c4; p2 = c5; s1 = c6; s2 = c7;
     } else {                                   // k1 k2 k3 k4 k5 k6 p1 p2; k4..k6 in the denominator
-        const T num = r2 * (r2 * (r2 * c[2] + c[1]) + c[0]) + 1.0f;
-        const T den = r2 * (r2 * (r2 * c[5] + c[4]) + c[3]) + 1.0f;
+        const T num = r2 * (r2 * (r2 * c2 + c1) + c0) + 1.0f;
+        const T den = r2 * (r2 * (r2 * c5 + c4) + c3) + 1.0f;
         radial = num / den;
-        p1 = c[6]; p2 = c[7];
+        p1 = c6; p2 = c7;
     }
-    tx = uv * (2.0f * p1) + (r2 + (u * u) * 2.0f) * p2;
-    ty = uv * (2.0f * p2) + (r2 + (v * v) * 2.0f) * p1;
-    if (tier == SSR_TIER_THIN_PRISM) { tx = tx + r2 * c[6]; ty = ty + r2 * c[7]; }
+    T tx = uv * (2.0f * p1) + (r2 + (u * u) * 2.0f) * p2;
+    T ty = uv * (2.0f * p2) + (r2 + (v * v) * 2.0f) * p1;
+    if (tier == SSR_TIER_THIN_PRISM) { tx = tx + r2 * s1; ty = ty + r2 * s2; }
     ou = u * radial + tx;
     ov = v * radial + ty;
 }
