@@ -318,8 +318,11 @@ int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream_t stream);
  * the 236 B/splat gradient round trip through HBM disappears. Quaternions take the Riemannian
  * step (gradient projected on the tangent of the unit sphere, result re-normalised). Splats that
  * are not visible still decay their moments, as in the reference.
- * Built: fp32 parameters and moments, one camera, non-packed, regularizers mcmc_opacity,
- * mcmc_scale, scale ratio, quaternion norm and SH/DC magnitude. Not built (rejected): quantized
+ * Built: fp32 parameters and moments, one camera, non-packed and packed (aabb and v_screen holding
+ * the nnz compacted rows of the packed projection; the reference sorts the rows by splat and walks a
+ * per-splat range, FusedProjectionBwdOptim.cu:160-212 -- with one camera a splat has at most one
+ * row, found through packed_row_of), regularizers mcmc_opacity, mcmc_scale, scale ratio,
+ * quaternion norm and SH/DC magnitude. Not built (rejected): quantized
  * Adam state, value-quantized SH, effective-rank regularizer, scale-agnostic mean step,
  * colour trust region. */
 typedef struct {
@@ -339,8 +342,15 @@ typedef struct {
     float mcmc_opacity_reg_weight, mcmc_scale_reg_weight, quat_norm_reg_weight, sh_reg_weight;
     int32_t step;               /* Adam step (>= 1) when `steps` is NULL */
     const int32_t* steps;       /* optional per-splat step [N] */
+    const int32_t* packed_row_of;   /* packed mode: [N], row of aabb / v_screen / v_rows that belongs to
+                                       splat g, or -1 (ssr_packed_row_map); NULL = row g */
 } ssr_fpbo_params;
 int ssr_fused_projection_bwd_optimizer(const ssr_fpbo_params* p, ssr_stream_t stream);
+/* row_of[g] = i where gaussian_ids[i] == g, -1 for splats without a packed row (one camera, so ids
+ * are unique); the per-splat lookup the packed mode above needs (FusedProjectionBwdOptim.cu:160-212
+ * builds the multi-camera form of it with a sort). */
+int ssr_packed_row_map(const int32_t* gaussian_ids, int64_t nnz, int64_t num_splats, int32_t* row_of,
+                       ssr_stream_t stream);
 
 /* Zeroes the gradient rows of the listed splats only (the rows a previous ssr_projection_bwd run
  * over that list wrote), instead of refilling all N rows. No counterpart in the reference, which

@@ -668,14 +668,17 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
         for (int i = 0; i < 4; i++) wg.quat[i] = VI.quats ? VI.quats[4 * g + i] : 0.f;
         wg.logit = VI.opacity_logits ? VI.opacity_logits[g] : 0.f;
 
-        const float4 bb = reinterpret_cast<const float4*>(P.aabb)[g];
+        // the row that holds this splat's aabb and screen gradients: g, or its packed row (none: skipped)
+        const int64_t row = P.packed_row_of ? (int64_t)P.packed_row_of[g] : g;
+        float4 bb = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (row >= 0) bb = reinterpret_cast<const float4*>(P.aabb)[row];
         if (!(bb.z <= bb.x || bb.w <= bb.y)) {   // FusedProjectionBwdOptim_kernel.cuh:271-272
             const CamD cam = load_camera(P.camera);
             WorldGradD pg;
             ssr_sh_quant none;
             none.codec = SSR_SH_F32; none.packed = nullptr; none.bounds = nullptr; none.bounds_stride = 0;
             none.num_sh_buffer = 0; none.scale_f16 = nullptr;
-            projection_vjp<kDegree, kLens>(cam, W, none, g, vscreen_of(P.v_screen, P.v_rows), g, pg, [&](int j, float Yj, const float vc[3]) {
+            projection_vjp<kDegree, kLens>(cam, W, none, g, vscreen_of(P.v_screen, P.v_rows), row, pg, [&](int j, float Yj, const float vc[3]) {
                 s_Y[threadIdx.x][j] = Yj;
                 if (j == 0) { s_vc[threadIdx.x][0] = vc[0]; s_vc[threadIdx.x][1] = vc[1]; s_vc[threadIdx.x][2] = vc[2]; }
             });
@@ -768,6 +771,14 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
 // (3 mean, 4 quat, 3 scale, 1 opacity, 3 dc, sh_stride SH).
 // Rows of splats that are visible now (non-empty aabb) are skipped when `aabb` is given: the
 // projection backward that follows overwrites them.
+__global__ __launch_bounds__(kProjBlock) void packed_row_map_kernel(const int32_t* __restrict__ gaussian_ids, int64_t nnz,
+                                                                    int64_t num_splats, int32_t* __restrict__ row_of) {
+    const int64_t i = (int64_t)blockIdx.x * kProjBlock + threadIdx.x;
+    if (i >= nnz) return;
+    const int32_t g = gaussian_ids[i];
+    if (g >= 0 && g < num_splats) row_of[g] = (int32_t)i;
+}
+
 __global__ __launch_bounds__(kProjBlock) void zero_world_rows_kernel(ssr_world V, const int32_t* __restrict__ ids, int64_t n,
                                                                      const float4* __restrict__ aabb) {
     const int64_t row = (int64_t)blockIdx.x * (kProjBlock / 64) + (threadIdx.x >> 6);
@@ -966,6 +977,20 @@ extern "C" int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream
     }
 #undef SSR_LAUNCH_BWD
     SSR_CHECK_LAUNCH("ssr_projection_bwd");
+    return 0;
+}
+
+extern "C" int ssr_packed_row_map(const int32_t* gaussian_ids, int64_t nnz, int64_t num_splats, int32_t* row_of,
+                                  ssr_stream_t stream) {
+    const char* where = "ssr_packed_row_map";
+    SSR_REQUIRE(num_splats >= 0 && num_splats < (int64_t)1 << 31 && nnz >= 0 && nnz <= num_splats, where, "counts out of range");
+    if (num_splats == 0) return 0;
+    SSR_REQUIRE(row_of && (nnz == 0 || gaussian_ids), where, "null buffer");
+    if (ssr_fill_u32(row_of, 0xffffffffu, num_splats, stream)) return 1;
+    if (nnz == 0) return 0;
+    hipLaunchKernelGGL(packed_row_map_kernel, dim3((unsigned)ceil_div(nnz, kProjBlock)), dim3(kProjBlock), 0, as_stream(stream),
+                       gaussian_ids, nnz, num_splats, row_of);
+    SSR_CHECK_LAUNCH(where);
     return 0;
 }
 

@@ -636,7 +636,7 @@ void fused_projection_bwd_optimizer_3dgs(
     const float quat_norm_reg_weight, const float sh_reg_weight, bool use_scale_agnostic_mean, bool color_trust_linear,
     float, std::variant<int32_t, TorchTensorView> step, int quantization_level) {
     const char* w = "fused_projection_bwd_optimizer_3dgs: ";
-    if (camera_ids.data_ptr() || gaussian_ids.data_ptr()) throw std::runtime_error(std::string(w) + "packed mode is not built in this backend");
+    const bool is_packed = camera_ids.data_ptr() && gaussian_ids.data_ptr();   // src/kernels/optim/FusedProjectionBwdOptim.cu:160
     if (sh_packed || non_sh.enabled || quantization_level != 0) throw std::runtime_error(std::string(w) + "quantized Adam state is not built in this backend");
     if (sh_value_packed) throw std::runtime_error(std::string(w) + "value-quantized SH is not built in this backend");
     if (erank_reg_weight != 0.0f || erank_reg_weight_s3 != 0.0f) throw std::runtime_error(std::string(w) + "the effective-rank regularizer is not built in this backend");
@@ -668,5 +668,11 @@ void fused_projection_bwd_optimizer_3dgs(
         p.steps = (const int32_t*)std::get<0>(std::get<TorchTensorView>(step));
     }
     StageTimer t(&g_times.k9);
+    if (is_packed) {   // aabb and v_splats_screen hold nnz compacted rows: find each splat's row
+        int32_t* row_of = DevicePool::global().acquire<int32_t>(PoolSlot::FusedProjBwdRowOf, (size_t)num_splats);
+        ok(ssr_packed_row_map(gaussian_ids.data_ptr(), (int64_t)gaussian_ids.size(), num_splats, row_of, nullptr),
+           "fused_projection_bwd_optimizer_3dgs/row map");
+        p.packed_row_of = row_of;
+    }
     ok(ssr_fused_projection_bwd_optimizer(&p, nullptr), "fused_projection_bwd_optimizer_3dgs");
 }

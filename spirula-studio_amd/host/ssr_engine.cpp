@@ -282,7 +282,6 @@ void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorVi
     auto& E = engine();
     if (std::get<0>(E.fwd.renders).data_ptr() == nullptr)
         throw std::runtime_error("engine_backward_fused_optimizer: forward_3dgs must be called first");
-    if (E.packed) throw std::runtime_error("engine_backward_fused_optimizer: packed projection is not built for the fused optimizer");
     const int64_t n = E.max_num_splats;
     if (!E.optim.adam_ready) {
         const PoolSlot s1[6] = {PoolSlot::AdamG1Means, PoolSlot::AdamG1Quats, PoolSlot::AdamG1Scales, PoolSlot::AdamG1Opacities,
@@ -304,13 +303,22 @@ void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorVi
     }
     E.grad.v_screen = raster_backward(v_render_rgb, v_render_depth, v_render_Ts);
     const int64_t W = E.camera.width, H = E.camera.height;
+    DeviceVector<int32_t> cam_ids, gauss_ids;
+    DeviceTensorFloatND aabb((float*)E.fwd.aabb.data_ptr(), {E.fwd.aabb.numel(), 4});
+    if (E.packed && E.fwd.gaussian_ids.size() > 0) {
+        cam_ids = E.fwd.camera_ids; gauss_ids = E.fwd.gaussian_ids;   // aabb and v_screen hold the nnz packed rows
+    } else if (E.packed) {
+        // nothing visible: every splat still takes its moment decay, so run the plain form on empty extents
+        float* zero = DevicePool::global().acquire<float>(PoolSlot::EngZeroAabb, (size_t)(E.cur_num_splats * 4));
+        backend::memset_async(zero, 0, (size_t)(E.cur_num_splats * 4) * sizeof(float));
+        aabb = DeviceTensorFloatND(zero, {E.cur_num_splats, 4});
+    }
     fused_projection_bwd_optimizer_3dgs(
         E.cur_num_splats, E.sh_degree, E.fwd.splats_w, E.camera.viewmats, E.camera.intrins, (uint32_t)W, (uint32_t)H,
-        E.camera.model_str, E.camera.distortion_str, E.camera.dist_coeffs, DeviceVector<int32_t>{}, DeviceVector<int32_t>{},
-        DeviceTensorFloatND((float*)E.fwd.aabb.data_ptr(), {E.fwd.aabb.numel(), 4}), {}, E.grad.v_screen, E.optim.g1, E.optim.g2,
-        std::nullopt, std::nullopt, E.world.sh_packed, E.world.sh_bounds, NonShQuantState{}, E.optim.radii,
-        E.optim.densify_score, hyper[0], hyper[1], hyper[2], hyper[3], hyper[4], hyper[5], hyper[6], hyper[7], hyper[8],
-        hyper[9], 0.0f, 0.0f, hyper[10], hyper[11], false, false, 0.0f, (int32_t)step, 0);
+        E.camera.model_str, E.camera.distortion_str, E.camera.dist_coeffs, cam_ids, gauss_ids, aabb, {}, E.grad.v_screen,
+        E.optim.g1, E.optim.g2, std::nullopt, std::nullopt, E.world.sh_packed, E.world.sh_bounds, NonShQuantState{},
+        E.optim.radii, E.optim.densify_score, hyper[0], hyper[1], hyper[2], hyper[3], hyper[4], hyper[5], hyper[6], hyper[7],
+        hyper[8], hyper[9], 0.0f, 0.0f, hyper[10], hyper[11], false, false, 0.0f, (int32_t)step, 0);
 }
 
 void engine_copy_params_to_host(TorchTensorView means, TorchTensorView quats, TorchTensorView scales,

@@ -91,7 +91,7 @@ class FpboParams(C.Structure):
                 ("max_gauss_ratio", C.c_float), ("scale_regularization_weight", C.c_float),
                 ("mcmc_opacity_reg_weight", C.c_float), ("mcmc_scale_reg_weight", C.c_float),
                 ("quat_norm_reg_weight", C.c_float), ("sh_reg_weight", C.c_float),
-                ("step", C.c_int32), ("steps", vp)]
+                ("step", C.c_int32), ("steps", vp), ("packed_row_of", vp)]
 
 
 # every symbol include/ssr_backend.h declares: (name, restype, argtypes)
@@ -117,6 +117,7 @@ SYMBOLS = {
     "ssr_raster_bwd": (_i32, [C.POINTER(RasterBwdParams), vp]),
     "ssr_projection_bwd": (_i32, [C.POINTER(ProjectionBwdParams), vp]),
     "ssr_fused_projection_bwd_optimizer": (_i32, [C.POINTER(FpboParams), vp]),
+    "ssr_packed_row_map": (_i32, [vp, _i64, _i64, vp, vp]),
     "ssr_zero_world_rows": (_i32, [C.POINTER(World), vp, _i64, vp, vp]),
     "ssr_fill_u32": (_i32, [vp, _u32, _i64, vp]),
     "ssr_init": (_i32, [_i32]),

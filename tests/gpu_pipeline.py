@@ -349,6 +349,13 @@ class GpuRun:
         if steps is not None:
             self.d["steps"] = D.from_host(np.ascontiguousarray(steps, np.int32))
             p.steps = self.ptr("steps")
+        if self.packed_projection:   # aabb and v_screen hold the nnz packed rows
+            self.d["row_of"] = D((self.n,), np.int32)
+            self.check(self.lib.ssr_packed_row_map(self.ptr("gaussian_ids") if self.rows else None, self.rows, self.n,
+                                                   self.ptr("row_of"), None))
+            p.packed_row_of = self.ptr("row_of")
+        if self.use_vrows:
+            p.v_rows = self.ptr("v_rows")
         self.check(self.lib.ssr_fused_projection_bwd_optimizer(C.byref(p), None))
         self.check(self.lib.ssr_device_synchronize())
         out = lambda pre: {k: self.host(pre + k) for k in keys}

@@ -197,6 +197,33 @@ def test_engine_packed_follows_the_camera_and_handles_nothing_visible(pkg, oracl
     look([[1, 0, 0, 0], [0, 1, 0, 0], [0, 0, 1, 0], [0, 0, 0, 1]])             # and back
 
 
+def test_engine_packed_fused_optimizer_with_nothing_visible(pkg, oracle, H):
+    """No packed rows at all: no projection gradient, but every splat still decays its moments and takes
+    the regularizer step (the reference's kernel runs over all N splats whatever is visible)."""
+    host, lib = H
+    sc = pkg.scenes.tiny_scene(n=2000, width=96, height=64, seed=71)
+    sc.viewmat = np.array([[1, 0, 0, 0], [0, 1, 0, 0], [0, 0, 1, -1000.0], [0, 0, 0, 1]], np.float32)   # all behind
+    eng = host.Engine(sc, packed_projection=True)
+    eng.forward()
+    assert eng.n_isects == 0
+    h = dict(lr_means=1.6e-4, lr_quats=1e-3, lr_scales=5e-3, lr_opacs=5e-2, lr_features_dc=2.5e-3, lr_features_sh=1.25e-4,
+             max_gauss_ratio=6.0, scale_regularization_weight=0.01, mcmc_opacity_reg_weight=0.01, mcmc_scale_reg_weight=0.01,
+             quat_norm_reg_weight=0.02, sh_reg_weight=0.05)
+    before = eng.params()
+    eng.backward_fused_optimizer(h, 1)
+    after = eng.params()
+    P = {k: np.ascontiguousarray(before[k], np.float32).copy() for k in oracle.WORLD_KEYS}
+    g1 = {k: np.zeros_like(v) for k, v in P.items()}
+    g2 = {k: np.zeros_like(v) for k, v in P.items()}
+    vs = dict(v_xy=np.zeros((sc.n, 2), np.float32), v_depth=np.zeros(sc.n, np.float32), v_conic=np.zeros((sc.n, 3), np.float32),
+              v_opac=np.zeros(sc.n, np.float32), v_rgb=np.zeros((sc.n, 3), np.float32))
+    oracle.fused_projection_bwd_optimizer(sc, np.zeros((sc.n, 4), np.float32), vs, P, g1, g2, h, step=1)
+    assert np.array_equal(after["means"], before["means"])    # no gradient reaches the means
+    assert np.abs(after["opacity_logits"] - before["opacity_logits"]).max() > 0.01    # the opacity regularizer moved it
+    for k in oracle.WORLD_KEYS:
+        assert np.abs(after[k].astype(np.float64) - P[k]).max() <= 0.05 * 5e-2, k
+
+
 def test_engine_tile_mask_is_one_shot(pkg, oracle, H):
     host, lib = H
     sc = pkg.scenes.make_scene(1, n=20000, width=320, height=240, parity_variant=True)
@@ -221,19 +248,24 @@ def test_engine_tile_mask_is_one_shot(pkg, oracle, H):
             _check(eng, oracle.pipeline(sc), sc)
 
 
-def test_engine_fused_optimizer_training_steps(pkg, oracle, H):
+@pytest.mark.parametrize("packed", [False, True])
+def test_engine_fused_optimizer_training_steps(pkg, oracle, H, packed):
     """Three training steps with the projection backward folded into Adam, against the oracle running
-    the same loop (forward, compositing backward, fused optimizer) on its own copy of the parameters."""
+    the same loop (forward, compositing backward, fused optimizer) on its own copy of the parameters;
+    also on the packed projection outputs (forward_3dgs(packed=true), the reference's training default),
+    where the splats behind the camera have no row and only decay their moments."""
     import copy
     host, lib = H
     sc = pkg.scenes.make_scene(1, n=20000, width=320, height=240, parity_variant=True)
+    if packed:
+        sc.means[::3, 2] = -10.0
     ref_sc = copy.deepcopy(sc)
     h = dict(lr_means=1.6e-4, lr_quats=1e-3, lr_scales=5e-3, lr_opacs=5e-2, lr_features_dc=2.5e-3,
              lr_features_sh=1.25e-4, max_gauss_ratio=6.0, scale_regularization_weight=0.01,
              mcmc_opacity_reg_weight=0.01, mcmc_scale_reg_weight=0.01, quat_norm_reg_weight=0.02, sh_reg_weight=0.05)
     lrs = dict(means="lr_means", quats="lr_quats", log_scales="lr_scales", opacity_logits="lr_opacs",
                features_dc="lr_features_dc", features_sh="lr_features_sh")
-    eng = host.Engine(sc)
+    eng = host.Engine(sc, packed_projection=packed)
     P = {k: np.ascontiguousarray(getattr(ref_sc, k), np.float32).copy() for k in oracle.WORLD_KEYS}
     g1 = {k: np.zeros_like(v) for k, v in P.items()}
     g2 = {k: np.zeros_like(v) for k, v in P.items()}

@@ -366,7 +366,7 @@ def test_tile_skip_mask(gpu, oracle):
     assert r["counts"].max() > 96
 
 
-@pytest.mark.parametrize("cfg", ["tiny", "cfg2", "equirect-steps", "fisheye-prism"])
+@pytest.mark.parametrize("cfg", ["tiny", "cfg2", "equirect-steps", "fisheye-prism", "tiny-packed", "cfg4-packed"])
 def test_fused_projection_bwd_optimizer(gpu, oracle, cfg):
     """K9 fused with Adam (fused_projection_bwd_optimizer_3dgs, fp32 state): both sides are fed the
     SAME screen gradients (the device's), so only the arithmetic of the fused kernel is compared."""
@@ -381,12 +381,30 @@ def test_fused_projection_bwd_optimizer(gpu, oracle, cfg):
         sc = gpu.scenes.make_scene(2, n=40000, width=480, height=270, parity_variant=True)
     elif cfg == "fisheye-prism":
         sc = _lens_scene(gpu, 1, 2, n=3000, seed=43)
+    elif cfg == "tiny-packed":
+        sc = gpu.scenes.tiny_scene(n=900, width=96, height=64, seed=61)
+        sc.means[::4, 2] = -10.0
+    elif cfg == "cfg4-packed":
+        sc = gpu.scenes.make_scene(4, n=60000, width=480, height=270, sh_codec=0)   # mostly culled
     else:
         sc = gpu.scenes.make_scene(5, n=30000, width=512, height=256)
-    g = GpuRun(gpu, sc)
+    packed = cfg.endswith("packed")
+    g = GpuRun(gpu, sc, packed_projection=packed)
     g.projection_fwd(); g.tiles(); g.raster_fwd(); g.raster_bwd()
     vs = {k: g.host(k) for k in ["v_xy", "v_depth", "v_conic", "v_opac", "v_rgb"]}
     aabb = g.host("aabb")
+    if packed:   # the packed mode is the plain one renumbered: give the oracle the rows scattered back to splats
+        ids = g.host("gaussian_ids")[:g.rows]
+        assert 0 < g.rows < sc.n and np.all(np.diff(ids) > 0)
+        row_of = np.full(sc.n, -1, np.int32)
+        row_of[ids] = np.arange(g.rows, dtype=np.int32)
+        full = np.zeros((sc.n, 4), np.float32)
+        full[ids] = aabb[:g.rows]
+        aabb = full
+        for k in vs:
+            full = np.zeros((sc.n,) + vs[k].shape[1:], np.float32)
+            full[ids] = vs[k][:g.rows]
+            vs[k] = full
     P = {k: np.ascontiguousarray(getattr(sc, k), np.float32).copy() for k in oracle.WORLD_KEYS}
     g1 = {k: rng.normal(0, 1e-3, P[k].shape).astype(np.float32) for k in oracle.WORLD_KEYS}
     g2 = {k: rng.uniform(1e-7, 1e-5, P[k].shape).astype(np.float32) for k in oracle.WORLD_KEYS}
@@ -408,6 +426,8 @@ def test_fused_projection_bwd_optimizer(gpu, oracle, cfg):
         a, b = dP[k].astype(np.float64), P[k].astype(np.float64)
         assert np.abs(a - b).max() <= 0.02 * h[lrs[k]] * 40 + 1e-6, (k, float(np.abs(a - b).max()))
     assert np.allclose(dscore, score, rtol=1e-3, atol=1e-9)
+    if packed:
+        assert np.array_equal(g.host("row_of"), row_of)
 
 
 def _variant_cotangents(sc, seed=1):
