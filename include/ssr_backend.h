@@ -321,9 +321,9 @@ int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream_t stream);
  * Built: fp32 parameters and moments, one camera, non-packed and packed (aabb and v_screen holding
  * the nnz compacted rows of the packed projection; the reference sorts the rows by splat and walks a
  * per-splat range, FusedProjectionBwdOptim.cu:160-212 -- with one camera a splat has at most one
- * row, found through packed_row_of), regularizers mcmc_opacity, mcmc_scale, scale ratio,
- * quaternion norm and SH/DC magnitude. Not built (rejected): quantized
- * Adam state, value-quantized SH, effective-rank regularizer, scale-agnostic mean step,
+ * row, found through packed_row_of), regularizers mcmc_opacity, mcmc_scale, scale ratio, effective
+ * rank, quaternion norm and SH/DC magnitude. Not built (rejected): quantized
+ * Adam state, value-quantized SH, scale-agnostic mean step,
  * colour trust region. */
 typedef struct {
     int64_t num_splats;
@@ -342,6 +342,7 @@ typedef struct {
     float mcmc_opacity_reg_weight, mcmc_scale_reg_weight, quat_norm_reg_weight, sh_reg_weight;
     int32_t step;               /* Adam step (>= 1) when `steps` is NULL */
     const int32_t* steps;       /* optional per-splat step [N] */
+    float erank_reg_weight, erank_reg_weight_s3;   /* effective-rank regularizer of the scales */
     const int32_t* packed_row_of;   /* packed mode: [N], row of aabb / v_screen / v_rows that belongs to
                                        splat g, or -1 (ssr_packed_row_map); NULL = row g */
 } ssr_fpbo_params;

@@ -160,6 +160,32 @@ SSR_HD SsrJet<N, O> ssr_jet_sqrt(const SsrJet<N, O>& a) {
     const float f1 = 0.5f / ssr_sqrt(m);
     return ssr_jet_apply(a, f, f1, a.v > 1e-7f ? -0.5f * (f1 / m) : 0.0f);
 }
+template <int N, int O>
+SSR_HD SsrJet<N, O> operator-(const SsrJet<N, O>& a, const SsrJet<N, O>& b) { return a + b * -1.0f; }
+template <int N, int O>
+SSR_HD SsrJet<N, O> ssr_jet_exp(const SsrJet<N, O>& a) {
+    const float f = ssr_exp(a.v);
+    return ssr_jet_apply(a, f, f, f);
+}
+template <int N, int O>
+SSR_HD SsrJet<N, O> ssr_jet_log(const SsrJet<N, O>& a) {
+    const float i = 1.0f / a.v;
+    return ssr_jet_apply(a, ssr_log(a.v), i, -(i * i));
+}
+// max / min: the derivative follows the selected operand; on a tie each side takes half
+// (the rule of the reference's differentiated max, src/generated/per_splat_losses.cuh:19-45)
+template <int N, int O>
+SSR_HD SsrJet<N, O> ssr_jet_max(const SsrJet<N, O>& a, const SsrJet<N, O>& b) {
+    if (a.v > b.v) return a;
+    if (a.v < b.v) return b;
+    return (a + b) * 0.5f;
+}
+template <int N, int O>
+SSR_HD SsrJet<N, O> ssr_jet_min(const SsrJet<N, O>& a, const SsrJet<N, O>& b) {
+    if (a.v < b.v) return a;
+    if (a.v > b.v) return b;
+    return (a + b) * 0.5f;
+}
 // atan2(y, x)
 template <int N, int O>
 SSR_HD SsrJet<N, O> ssr_jet_atan2(const SsrJet<N, O>& y, const SsrJet<N, O>& x) {
@@ -265,4 +291,24 @@ SSR_HD void ssr_model_pixel(int model, int tier, const float* coeffs, float fx, 
     ssr_distort<T>(tier, coeffs, u, v, du, dv);
     px = du * fx + cx;
     py = dv * fy + cy;
+}
+
+// ---- effective-rank regularizer of the scales ------------------------------------------------------
+// erank_reg_3dgs (src/shaders/per_splat_losses.slang:3-15): with s_i the normalised squared scales,
+// reg = max(-log(exp(entropy(s)) - 0.99999), 0); loss = w * reg + w3 * s_min. Returns the loss, writes its
+// gradient with respect to the three log-scales.
+SSR_HD float ssr_erank_reg_grad(const float log_scales[3], float w, float w3, float grad[3]) {
+    typedef SsrJet<3, 1> Jet;
+    const Jet x = ssr_jet_exp(ssr_jet_seed<3, 1>(log_scales[0], 0) * 2.0f);
+    const Jet y = ssr_jet_exp(ssr_jet_seed<3, 1>(log_scales[1], 1) * 2.0f);
+    const Jet z = ssr_jet_exp(ssr_jet_seed<3, 1>(log_scales[2], 2) * 2.0f);
+    const Jet s = (x + y) + z;
+    const Jet s1 = ssr_jet_max(ssr_jet_max(x, y), z) / s;
+    const Jet s3 = ssr_jet_min(ssr_jet_min(x, y), z) / s;
+    const Jet s2 = (s1 * -1.0f + 1.0f) - s3;
+    const Jet r = ssr_jet_exp(((s1 * ssr_jet_log(s1)) * -1.0f - s2 * ssr_jet_log(s2)) - s3 * ssr_jet_log(s3));
+    const Jet reg = ssr_jet_max(ssr_jet_log(r + -0.99999f) * -1.0f, ssr_jet_const<3, 1>(0.0f));
+    const Jet loss = reg * w + s3 * w3;
+    grad[0] = loss.d[0]; grad[1] = loss.d[1]; grad[2] = loss.d[2];
+    return loss.v;
 }

@@ -510,7 +510,12 @@ void or_decode_sh(int64_t gid, const or_sh_source* sh, float* out45) { decode_sh
 // Fused projection backward + Adam, fp32 state (src/kernels/optim/FusedProjectionBwdOptim_kernel.cuh:232-710
 // with BLOCK_SIZE == 0, VALUE_BITS == 32, use_scale_agnostic_mean = color_trust_linear = false).
 // The data gradient is or_projection_bwd's; the regularizers are the closed-form derivatives of
-// src/shaders/per_splat_losses.slang:30-81 (effective-rank terms not included: weight 0).
+// src/shaders/per_splat_losses.slang:30-81; the effective-rank term (:3-15) is differentiated with the
+// first-order arithmetic of include/ssr_camera.h (ssr_erank_reg_grad).
+float or_erank_reg(const float* log_scales, float w, float w3, float* grad) {
+    return ssr_erank_reg_grad(log_scales, w, w3, grad);
+}
+
 void or_fused_projection_bwd_optimizer(int64_t N, int sh_degree,
     float* means, float* quats, float* log_scales, float* opacity_logits, float* features_dc, float* features_sh,
     const or_camera* cam, const float* aabb,
@@ -527,7 +532,7 @@ void or_fused_projection_bwd_optimizer(int64_t N, int sh_degree,
                       v_conic, v_opac, v_srgb, vm.data(), vq.data(), vs.data(), vo.data(), vd.data(), vsh.data());
     const float lr_means = hyper[0], lr_quats = hyper[1], lr_scales = hyper[2], lr_opacs = hyper[3], lr_dc = hyper[4],
                 lr_sh = hyper[5], max_ratio = hyper[6], scale_w = hyper[7], mcmc_o = hyper[8], mcmc_s = hyper[9],
-                qnorm_w = hyper[10], sh_w = hyper[11];
+                qnorm_w = hyper[10], sh_w = hyper[11], erank_w = hyper[12], erank_w3 = hyper[13];
     const float kBeta1 = 0.9f, kBeta2 = 0.999f, kEps = 1e-15f;
     const float sh_reg = sh_w * (1.0f / (float)(n_coef > 0 ? n_coef : 1));
 #pragma omp parallel for schedule(static)
@@ -574,6 +579,11 @@ void or_fused_projection_bwd_optimizer(int64_t N, int sh_degree,
         const float ratio = e[imax] / e[imin];
         const float rg = ratio > max_ratio ? scale_w * ratio : 0.0f;
         for (int i = 0; i < 3; i++) gs[i] += ms + (i == imax ? rg : 0.f) - (i == imin ? rg : 0.f);
+        if (erank_w != 0.0f || erank_w3 != 0.0f) {   // erank_reg_3dgs, per_splat_losses.slang:3-15,101
+            float ge[3];
+            ssr_erank_reg_grad(ls, erank_w, erank_w3, ge);
+            for (int i = 0; i < 3; i++) gs[i] += ge[i];
+        }
         const float qn = ssr_sqrt((q0[0] * q0[0] + q0[1] * q0[1]) + (q0[2] * q0[2] + q0[3] * q0[3]));
         const float qg = qnorm_w * ((1.0f - 1.0f / qn) / qn);
         for (int i = 0; i < 4; i++) gq[i] += qg * q0[i];

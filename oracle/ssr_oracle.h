@@ -132,13 +132,18 @@ void or_projection_bwd(int64_t N, int sh_degree,
  * src/kernels/optim/FusedProjectionBwdOptim_kernel.cuh:232-710): parameters and moments [N,...]
  * are updated in place. v_in (6 arrays, any may be NULL) are gradient contributions already
  * present. hyper = {lr_means, lr_quats, lr_scales, lr_opacs, lr_dc, lr_sh, max_gauss_ratio,
- * scale_reg_w, mcmc_opacity_w, mcmc_scale_w, quat_norm_w, sh_reg_w}. steps may be NULL (then `step`). */
+ * scale_reg_w, mcmc_opacity_w, mcmc_scale_w, quat_norm_w, sh_reg_w, erank_w, erank_w_s3}. steps may be NULL
+ * (then `step`). */
 void or_fused_projection_bwd_optimizer(int64_t N, int sh_degree,
     float* means, float* quats, float* log_scales, float* opacity_logits, float* features_dc, float* features_sh,
     const or_camera* cam, const float* aabb,
     const float* v_xy, const float* v_sdepth, const float* v_conic, const float* v_opac, const float* v_srgb,
     const float* const* v_in, float* const* g1, float* const* g2, float* densify_score,
     const float* hyper, int32_t step, const int32_t* steps);
+
+/* erank_reg_3dgs (src/shaders/per_splat_losses.slang:3-15): the loss for one splat's three log-scales and
+ * its gradient. */
+float or_erank_reg(const float* log_scales, float w, float w3, float* grad);
 
 /* Codecs (src/core/Tensor.h:1364-1392): block-wise (min,max) + uint8/uint16 codes. */
 void or_quantize_ref(int bits, int64_t n_cells, int64_t bounds_stride, const float* values,

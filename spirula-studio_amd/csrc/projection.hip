@@ -706,6 +706,12 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
             const float rg = ratio > P.max_gauss_ratio ? P.scale_regularization_weight * ratio : 0.0f;
 #pragma unroll
             for (int i = 0; i < 3; i++) wg.scale[i] += ms + (i == imax ? rg : 0.f) - (i == imin ? rg : 0.f);
+            if (P.erank_reg_weight != 0.0f || P.erank_reg_weight_s3 != 0.0f) {   // per_splat_losses.slang:3-15,101
+                float ge[3];
+                ssr_erank_reg_grad(ls, P.erank_reg_weight, P.erank_reg_weight_s3, ge);
+#pragma unroll
+                for (int i = 0; i < 3; i++) wg.scale[i] += ge[i];
+            }
             const float qn = ssr_sqrt((quat[0] * quat[0] + quat[1] * quat[1]) + (quat[2] * quat[2] + quat[3] * quat[3]));
             const float qg = P.quat_norm_reg_weight * ((1.0f - 1.0f / qn) / qn);
 #pragma unroll

@@ -639,7 +639,6 @@ void fused_projection_bwd_optimizer_3dgs(
     const bool is_packed = camera_ids.data_ptr() && gaussian_ids.data_ptr();   // src/kernels/optim/FusedProjectionBwdOptim.cu:160
     if (sh_packed || non_sh.enabled || quantization_level != 0) throw std::runtime_error(std::string(w) + "quantized Adam state is not built in this backend");
     if (sh_value_packed) throw std::runtime_error(std::string(w) + "value-quantized SH is not built in this backend");
-    if (erank_reg_weight != 0.0f || erank_reg_weight_s3 != 0.0f) throw std::runtime_error(std::string(w) + "the effective-rank regularizer is not built in this backend");
     if (use_scale_agnostic_mean) throw std::runtime_error(std::string(w) + "the scale-agnostic mean step is not built in this backend");
     if (color_trust_linear) throw std::runtime_error(std::string(w) + "the colour trust region is not built in this backend");
     if (num_splats == 0) return;
@@ -662,6 +661,7 @@ void fused_projection_bwd_optimizer_3dgs(
     p.max_gauss_ratio = max_gauss_ratio; p.scale_regularization_weight = scale_regularization_weight;
     p.mcmc_opacity_reg_weight = mcmc_opacity_reg_weight; p.mcmc_scale_reg_weight = mcmc_scale_reg_weight;
     p.quat_norm_reg_weight = quat_norm_reg_weight; p.sh_reg_weight = sh_reg_weight;
+    p.erank_reg_weight = erank_reg_weight; p.erank_reg_weight_s3 = erank_reg_weight_s3;
     if (const int32_t* s = std::get_if<int32_t>(&step)) {
         p.step = *s;
     } else {

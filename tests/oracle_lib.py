@@ -39,6 +39,7 @@ def lib():
         _lib.or_projection_fwd.restype = C.c_int64
         _lib.or_tile_write.restype = C.c_int64
         _lib.or_num_threads.restype = C.c_int
+        _lib.or_erank_reg.restype = C.c_float
     return _lib
 
 
@@ -228,7 +229,7 @@ def projection_bwd(scene, aabb, vs, sh_degree=3):
 
 HYPER = ["lr_means", "lr_quats", "lr_scales", "lr_opacs", "lr_features_dc", "lr_features_sh", "max_gauss_ratio",
          "scale_regularization_weight", "mcmc_opacity_reg_weight", "mcmc_scale_reg_weight", "quat_norm_reg_weight",
-         "sh_reg_weight"]
+         "sh_reg_weight", "erank_reg_weight", "erank_reg_weight_s3"]
 WORLD_KEYS = ["means", "quats", "log_scales", "opacity_logits", "features_dc", "features_sh"]
 
 
@@ -257,6 +258,14 @@ def fused_projection_bwd_optimizer(scene, aabb, vs, params, g1, g2, hyper, step=
         ptrs(v_in) if v_in is not None else None, ptrs(g1), ptrs(g2), _p(score), _p(hv), C.c_int32(step),
         _p(None if steps is None else np.ascontiguousarray(steps, np.int32)))
     return score
+
+
+def erank_reg(log_scales, w, w3):
+    """Loss and gradient of the effective-rank regularizer for one splat."""
+    ls = np.ascontiguousarray(log_scales, np.float32)
+    g = np.zeros(3, np.float32)
+    loss = lib().or_erank_reg(_p(ls), C.c_float(w), C.c_float(w3), _p(g))
+    return float(loss), g
 
 
 def pipeline(scene, sh_degree=3, backward=True, tile_active=None, variant=None):

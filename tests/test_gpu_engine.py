@@ -265,6 +265,8 @@ def test_engine_fused_optimizer_training_steps(pkg, oracle, H, packed):
              mcmc_opacity_reg_weight=0.01, mcmc_scale_reg_weight=0.01, quat_norm_reg_weight=0.02, sh_reg_weight=0.05)
     lrs = dict(means="lr_means", quats="lr_quats", log_scales="lr_scales", opacity_logits="lr_opacs",
                features_dc="lr_features_dc", features_sh="lr_features_sh")
+    if packed:
+        h.update(erank_reg_weight=0.05, erank_reg_weight_s3=0.01)
     eng = host.Engine(sc, packed_projection=packed)
     P = {k: np.ascontiguousarray(getattr(ref_sc, k), np.float32).copy() for k in oracle.WORLD_KEYS}
     g1 = {k: np.zeros_like(v) for k, v in P.items()}

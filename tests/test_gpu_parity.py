@@ -388,6 +388,8 @@ def test_fused_projection_bwd_optimizer(gpu, oracle, cfg):
         sc = gpu.scenes.make_scene(4, n=60000, width=480, height=270, sh_codec=0)   # mostly culled
     else:
         sc = gpu.scenes.make_scene(5, n=30000, width=512, height=256)
+    sc.log_scales[11] = [-2.5, -6.5, -6.6]                 # a needle
+    sc.log_scales[12] = [-3.0, -3.0, -3.0]                 # ties in the max and min of the scales
     packed = cfg.endswith("packed")
     g = GpuRun(gpu, sc, packed_projection=packed)
     g.projection_fwd(); g.tiles(); g.raster_fwd(); g.raster_bwd()
@@ -412,6 +414,8 @@ def test_fused_projection_bwd_optimizer(gpu, oracle, cfg):
     h = dict(lr_means=1.6e-4, lr_quats=1e-3, lr_scales=5e-3, lr_opacs=5e-2, lr_features_dc=2.5e-3,
              lr_features_sh=1.25e-4, max_gauss_ratio=6.0, scale_regularization_weight=0.01,
              mcmc_opacity_reg_weight=0.01, mcmc_scale_reg_weight=0.01, quat_norm_reg_weight=0.02, sh_reg_weight=0.05)
+    if cfg in ("tiny", "cfg4-packed", "fisheye-prism"):   # with the effective-rank regularizer (needles and blobs both occur)
+        h.update(erank_reg_weight=0.1, erank_reg_weight_s3=0.01)
     steps = rng.integers(1, 400, sc.n).astype(np.int32) if cfg == "equirect-steps" else None
     dP, d1, d2, dscore = g.fused_optimizer(g1, g2, h, step=37, steps=steps, v_in=v_in)
     score = oracle.fused_projection_bwd_optimizer(sc, aabb, vs, P, g1, g2, h, step=37, steps=steps, v_in=v_in)

@@ -9,6 +9,16 @@ B1, B2, EPS = 0.9, 0.999, 1e-15
 KSH0 = 0.28209479177387814
 
 
+def _erank64(ls, w, w3):
+    """erank_reg_3dgs, src/shaders/per_splat_losses.slang:3-15, in float64."""
+    x = np.exp(2.0 * np.asarray(ls, np.float64))
+    s = np.sort(x / x.sum())
+    s3, s1 = s[0], s[2]
+    s2 = 1.0 - s1 - s3
+    r = np.exp(-s1 * np.log(s1) - s2 * np.log(s2) - s3 * np.log(s3))
+    return w * max(-np.log(r - 0.99999), 0.0) + w3 * s3
+
+
 def _losses64(ls, logit, quat, dc, sh, h, n_coef):
     """Sum of the per-splat regularizers with v_loss = 1, in float64."""
     e = np.exp(ls)
@@ -23,6 +33,8 @@ def _losses64(ls, logit, quat, dc, sh, h, n_coef):
     lim = 0.5 / KSH0
     loss += 0.5 * h["sh_reg_weight"] * (np.maximum(np.abs(dc) - lim, 0) ** 2).sum()
     loss += 0.5 * h["sh_reg_weight"] / max(n_coef, 1) * (sh ** 2).sum()
+    if h.get("erank_reg_weight", 0.0) or h.get("erank_reg_weight_s3", 0.0):
+        loss += _erank64(ls, h.get("erank_reg_weight", 0.0), h.get("erank_reg_weight_s3", 0.0))
     return loss
 
 
@@ -50,7 +62,10 @@ def test_fused_optimizer_against_float64_adam(pkg, oracle, per_splat_steps):
     v_in = {"means": rng.normal(0, 1e-3, (sc.n, 3)).astype(np.float32), "opacity_logits": None}
     h = dict(lr_means=1.6e-4, lr_quats=1e-3, lr_scales=5e-3, lr_opacs=5e-2, lr_features_dc=2.5e-3,
              lr_features_sh=1.25e-4, max_gauss_ratio=6.0, scale_regularization_weight=0.01,
-             mcmc_opacity_reg_weight=0.01, mcmc_scale_reg_weight=0.01, quat_norm_reg_weight=0.02, sh_reg_weight=0.05)
+             mcmc_opacity_reg_weight=0.01, mcmc_scale_reg_weight=0.01, quat_norm_reg_weight=0.02, sh_reg_weight=0.05,
+             erank_reg_weight=0.1, erank_reg_weight_s3=0.01)
+    sc.log_scales[9] = [-3.0, -3.0 - 1e-3, -7.0]   # nearly a needle... a disc: effective rank close to 2
+    sc.log_scales[11] = [-2.5, -6.5, -6.6]         # a needle: effective rank close to 1, the log term is large
     steps = rng.integers(1, 400, sc.n).astype(np.int32) if per_splat_steps else None
     step = 37
     P0 = {k: v.astype(np.float64) for k, v in P.items()}
@@ -110,3 +125,39 @@ def test_zero_learning_rates_and_weights_leave_parameters_alone(pkg, oracle):
     # moments took the gradient: g1 = 0.1 v
     assert np.allclose(g1["means"], 0.1 * r["grads"]["v_means"], rtol=1e-5, atol=1e-12)
     assert np.allclose(g2["features_sh"], 0.001 * r["grads"]["v_sh"] ** 2, rtol=1e-4, atol=1e-20)
+
+
+def test_effective_rank_regularizer(oracle):
+    """Loss and gradient of erank_reg_3dgs against its float64 definition and central differences; the
+    -log term switches off once exp(entropy) - 0.99999 reaches 1; on ties the derivative of max / min is
+    shared between the tied operands, as the reference's differentiated max does
+    (src/generated/per_splat_losses.cuh:19-45)."""
+    rng = np.random.default_rng(4)
+    n_on = n_off = 0
+    for _ in range(300):
+        ls = rng.uniform(-7, -1, 3)
+        u = rng.random()
+        if u < 0.35:
+            ls[1:] = ls[0] - rng.uniform(2.0, 5.0, 2)    # needle-like: rank near 1, the log term is active
+        elif u < 0.7:
+            ls = ls[0] + rng.uniform(-0.4, 0.4, 3)       # blob-like: rank well above 2, the log term is off
+        w, w3 = float(rng.uniform(0, 0.2)), float(rng.uniform(0, 0.05))
+        ls32 = ls.astype(np.float32).astype(np.float64)
+        loss, g = oracle.erank_reg(ls32, w, w3)
+        want = _erank64(ls32, w, w3)
+        x = np.exp(2 * ls32); s = np.sort(x / x.sum())
+        r = np.exp(-(s * np.log(s)).sum())
+        if abs(r - 1.99999) < 1e-3:
+            continue                                    # at the switch
+        n_on += r < 1.99999
+        n_off += r > 1.99999
+        assert np.isclose(loss, want, rtol=2e-4, atol=1e-6)
+        fd = _fd(lambda v: _erank64(v, w, w3), ls32, eps=1e-5)
+        assert np.allclose(g, fd, rtol=2e-3, atol=2e-4 * (np.abs(fd).max() + 1e-3)), (ls32, g, fd)
+    assert n_on > 50 and n_off > 50
+    # isotropic: entropy is stationary, and d s_min / d l = 2 s_min (weights - s) with the tie weights (1/4, 1/4, 1/2)
+    loss, g = oracle.erank_reg(np.array([-3.0, -3.0, -3.0]), 0.0, 1.0)
+    assert np.isclose(loss, 1 / 3, rtol=1e-6)
+    assert np.allclose(g, 2 / 3 * (np.array([0.25, 0.25, 0.5]) - 1 / 3), atol=1e-6)
+    loss, g = oracle.erank_reg(np.array([-3.0, -3.0, -3.0]), 1.0, 0.0)
+    assert loss == 0.0 and not np.any(g)               # rank 3: the log term is off
