@@ -322,9 +322,8 @@ int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream_t stream);
  * the nnz compacted rows of the packed projection; the reference sorts the rows by splat and walks a
  * per-splat range, FusedProjectionBwdOptim.cu:160-212 -- with one camera a splat has at most one
  * row, found through packed_row_of), regularizers mcmc_opacity, mcmc_scale, scale ratio, effective
- * rank, quaternion norm and SH/DC magnitude. Not built (rejected): quantized
- * Adam state, value-quantized SH, scale-agnostic mean step,
- * colour trust region. */
+ * rank, quaternion norm and SH/DC magnitude; the scale-agnostic step of the means. Not built
+ * (rejected): quantized Adam state, value-quantized SH, colour trust region. */
 typedef struct {
     int64_t num_splats;
     int32_t sh_degree;
@@ -343,6 +342,9 @@ typedef struct {
     int32_t step;               /* Adam step (>= 1) when `steps` is NULL */
     const int32_t* steps;       /* optional per-splat step [N] */
     float erank_reg_weight, erank_reg_weight_s3;   /* effective-rank regularizer of the scales */
+    const float* scale_agnostic_radii;   /* optional [N] apparent radii of the forward (its `radii` output): when
+                                            given, the means take the scale-agnostic step
+                                            (use_scale_agnostic_mean, FusedProjectionBwdOptim_kernel.cuh:519-534) */
     const int32_t* packed_row_of;   /* packed mode: [N], row of aabb / v_screen / v_rows that belongs to
                                        splat g, or -1 (ssr_packed_row_map); NULL = row g */
 } ssr_fpbo_params;

@@ -521,7 +521,7 @@ void or_fused_projection_bwd_optimizer(int64_t N, int sh_degree,
     const or_camera* cam, const float* aabb,
     const float* v_xy, const float* v_sdepth, const float* v_conic, const float* v_opac, const float* v_srgb,
     const float* const* v_in, float* const* g1, float* const* g2, float* densify_score,
-    const float* hyper, int32_t step, const int32_t* steps) {
+    const float* hyper, int32_t step, const int32_t* steps, const float* radii) {
     const int n_coef = sh_degree * (sh_degree + 2);
     std::vector<float> vm((size_t)N * 3), vq((size_t)N * 4), vs((size_t)N * 3), vo((size_t)N), vd((size_t)N * 3),
         vsh((size_t)N * 45);
@@ -591,6 +591,22 @@ void or_fused_projection_bwd_optimizer(int64_t N, int sh_degree,
         for (int i = 0; i < 3; i++)
             gd[i] += sh_w * (ssr_max(features_dc[3 * g + i] - lim, 0.0f) + ssr_min(features_dc[3 * g + i] + lim, 0.0f));
         const float smax = ssr_max(ssr_max(ls[0], ls[1]), ls[2]);
+        // use_scale_agnostic_mean (FusedProjectionBwdOptim_kernel.cuh:519-534), from the parameters as they were:
+        // num = apply_covar_to_vec(quat, exp(0.5 log_scale), v_mean) * sqrt(2 log(max(255 sigmoid(opacity), 1.00001)))
+        // (projection_utils.slang:151-162, the rotation from the stored quaternion as it is), den = 0.6 radii
+        float sa_num[3] = {0.f, 0.f, 0.f}, sa_den = 0.f;
+        if (radii) {
+            float Rm[3][3], M[3][3], cov[3][3];
+            quat_to_rot(q0, Rm);
+            const float hs[3] = {ssr_exp(0.5f * ls[0]), ssr_exp(0.5f * ls[1]), ssr_exp(0.5f * ls[2])};
+            for (int i = 0; i < 3; i++)
+                for (int j = 0; j < 3; j++) M[i][j] = Rm[i][j] * hs[j];
+            for (int i = 0; i < 3; i++)
+                for (int j = 0; j < 3; j++) cov[i][j] = (M[i][0] * M[j][0] + M[i][1] * M[j][1]) + M[i][2] * M[j][2];
+            const float extent = ssr_sqrt(2.0f * ssr_log(ssr_max(255.0f * ssr_sigmoid(logit), 1.00001f)));
+            for (int i = 0; i < 3; i++) sa_num[i] = ((cov[i][0] * gm[0] + cov[i][1] * gm[1]) + cov[i][2] * gm[2]) * extent;
+            sa_den = radii[g] * 0.6f;
+        }
         // scales
         float new_ls[3];
         for (int i = 0; i < 3; i++) new_ls[i] = adam(ls[i], gs[i], lr_scales, g1[2] + 3 * g + i, g2[2] + 3 * g + i);
@@ -608,7 +624,18 @@ void or_fused_projection_bwd_optimizer(int64_t N, int sh_degree,
         for (int i = 0; i < 3; i++) log_scales[3 * g + i] = new_ls[i];
         opacity_logits[g] = adam(logit, go, lr_opacs, g1[3] + g, g2[3] + g);
         if (densify_score) densify_score[g] = ssr_exp(smax) * ssr_sqrt(dot3(gm, gm));
-        for (int i = 0; i < 3; i++) means[3 * g + i] = adam(means[3 * g + i], gm[i], lr_means, g1[0] + 3 * g + i, g2[0] + 3 * g + i);
+        for (int i = 0; i < 3; i++) {
+            if (radii) {
+                float* g1p = g1[0] + 3 * g + i;
+                float* g2p = g2[0] + 3 * g + i;
+                const float a = kBeta1 * *g1p + (1.f - kBeta1) * sa_num[i];
+                const float b = kBeta2 * *g2p + (1.f - kBeta2) * (((gm[i] * gm[i]) * sa_den) * sa_den);
+                *g1p = a; *g2p = b;
+                means[3 * g + i] = means[3 * g + i] - ((lr_means * b1c) * a) / (ssr_sqrt(b * b2c) + kEps);
+            } else {
+                means[3 * g + i] = adam(means[3 * g + i], gm[i], lr_means, g1[0] + 3 * g + i, g2[0] + 3 * g + i);
+            }
+        }
         for (int i = 0; i < 3; i++)
             features_dc[3 * g + i] = adam(features_dc[3 * g + i], gd[i], lr_dc, g1[4] + 3 * g + i, g2[4] + 3 * g + i);
     }

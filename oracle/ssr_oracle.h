@@ -139,7 +139,8 @@ void or_fused_projection_bwd_optimizer(int64_t N, int sh_degree,
     const or_camera* cam, const float* aabb,
     const float* v_xy, const float* v_sdepth, const float* v_conic, const float* v_opac, const float* v_srgb,
     const float* const* v_in, float* const* g1, float* const* g2, float* densify_score,
-    const float* hyper, int32_t step, const int32_t* steps);
+    const float* hyper, int32_t step, const int32_t* steps,
+    const float* radii /* optional [N]: the forward's radii; given = the scale-agnostic step of the means */);
 
 /* erank_reg_3dgs (src/shaders/per_splat_losses.slang:3-15): the loss for one splat's three log-scales and
  * its gradient. */

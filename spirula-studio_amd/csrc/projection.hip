@@ -745,9 +745,45 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
             const float smax = ssr_max(ssr_max(ls[0], ls[1]), ls[2]);
             P.densify_score[g] = ssr_exp(smax) * ssr_sqrt(dot3(wg.mean, wg.mean));
         }
+        if (P.scale_agnostic_radii) {
+            // use_scale_agnostic_mean (FusedProjectionBwdOptim_kernel.cuh:519-534): the first moment takes the
+            // gradient pushed through the splat's own covariance R diag(exp(log_scale)) R^T (R from the stored,
+            // un-normalised quaternion, as apply_covar_to_vec does) times its opacity-aware extent, the second
+            // moment the gradient scaled by 0.6 x the splat's apparent radius
+            const float w = quat[0], qx = quat[1], qy = quat[2], qz = quat[3];
+            const float x2 = qx * qx, y2 = qy * qy, z2 = qz * qz, xy = qx * qy, xz = qx * qz, yz = qy * qz;
+            const float wx = w * qx, wy = w * qy, wz = w * qz;
+            const float R[3][3] = {{1.f - 2.f * (y2 + z2), 2.f * (xy - wz), 2.f * (xz + wy)},
+                                   {2.f * (xy + wz), 1.f - 2.f * (x2 + z2), 2.f * (yz - wx)},
+                                   {2.f * (xz - wy), 2.f * (yz + wx), 1.f - 2.f * (x2 + y2)}};
+            const float hs[3] = {ssr_exp(0.5f * ls[0]), ssr_exp(0.5f * ls[1]), ssr_exp(0.5f * ls[2])};
+            float M[3][3], cov[3][3];
 #pragma unroll
-        for (int i = 0; i < 3; i++)
-            W.means[3 * g + i] = adam_step(mean[i], wg.mean[i], P.lr_means, ad, P.g1.means + 3 * g + i, P.g2.means + 3 * g + i);
+            for (int i = 0; i < 3; i++)
+#pragma unroll
+                for (int j = 0; j < 3; j++) M[i][j] = R[i][j] * hs[j];
+#pragma unroll
+            for (int i = 0; i < 3; i++)
+#pragma unroll
+                for (int j = 0; j < 3; j++) cov[i][j] = (M[i][0] * M[j][0] + M[i][1] * M[j][1]) + M[i][2] * M[j][2];
+            const float extent = ssr_sqrt(2.0f * ssr_log(ssr_max(255.0f * ssr_sigmoid(logit), 1.00001f)));
+            const float den = P.scale_agnostic_radii[g] * 0.6f;
+            constexpr float kBeta1 = 0.9f, kBeta2 = 0.999f, kEps = 1e-15f;
+#pragma unroll
+            for (int i = 0; i < 3; i++) {
+                const float num = ((cov[i][0] * wg.mean[0] + cov[i][1] * wg.mean[1]) + cov[i][2] * wg.mean[2]) * extent;
+                float* g1p = P.g1.means + 3 * g + i;
+                float* g2p = P.g2.means + 3 * g + i;
+                const float m1 = kBeta1 * *g1p + (1.f - kBeta1) * num;
+                const float m2 = kBeta2 * *g2p + (1.f - kBeta2) * (((wg.mean[i] * wg.mean[i]) * den) * den);
+                *g1p = m1; *g2p = m2;
+                W.means[3 * g + i] = mean[i] - ((P.lr_means * ad.b1c) * m1) / (ssr_sqrt(m2 * ad.b2c) + kEps);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 3; i++)
+                W.means[3 * g + i] = adam_step(mean[i], wg.mean[i], P.lr_means, ad, P.g1.means + 3 * g + i, P.g2.means + 3 * g + i);
+        }
 #pragma unroll
         for (int i = 0; i < 3; i++)
             W.features_dc[3 * g + i] = adam_step(dc[i], wg.dc[i], P.lr_features_dc, ad, P.g1.features_dc + 3 * g + i, P.g2.features_dc + 3 * g + i);
@@ -773,10 +809,6 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
     }
 }
 
-// One wavefront per listed splat: lane l zeroes float l of its 59-float gradient row
-// (3 mean, 4 quat, 3 scale, 1 opacity, 3 dc, sh_stride SH).
-// Rows of splats that are visible now (non-empty aabb) are skipped when `aabb` is given: the
-// projection backward that follows overwrites them.
 __global__ __launch_bounds__(kProjBlock) void packed_row_map_kernel(const int32_t* __restrict__ gaussian_ids, int64_t nnz,
                                                                     int64_t num_splats, int32_t* __restrict__ row_of) {
     const int64_t i = (int64_t)blockIdx.x * kProjBlock + threadIdx.x;
@@ -785,6 +817,10 @@ __global__ __launch_bounds__(kProjBlock) void packed_row_map_kernel(const int32_
     if (g >= 0 && g < num_splats) row_of[g] = (int32_t)i;
 }
 
+// One wavefront per listed splat: lane l zeroes float l of its 59-float gradient row
+// (3 mean, 4 quat, 3 scale, 1 opacity, 3 dc, sh_stride SH).
+// Rows of splats that are visible now (non-empty aabb) are skipped when `aabb` is given: the
+// projection backward that follows overwrites them.
 __global__ __launch_bounds__(kProjBlock) void zero_world_rows_kernel(ssr_world V, const int32_t* __restrict__ ids, int64_t n,
                                                                      const float4* __restrict__ aabb) {
     const int64_t row = (int64_t)blockIdx.x * (kProjBlock / 64) + (threadIdx.x >> 6);

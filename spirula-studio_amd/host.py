@@ -23,7 +23,7 @@ SYMBOLS = {
     "ssrh_set_sh_value_quant": (C.c_int, [C.c_int, vp, C.c_int64, C.c_int, vp, C.c_int64, C.c_int, C.c_int64]),
     "ssrh_set_camera_params": (C.c_int, [C.c_int, C.c_int, C.c_char_p, C.c_char_p, vp, vp, vp, C.c_int]),
     "ssrh_backward_with_variants": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, C.c_int]),
-    "ssrh_backward_fused_optimizer": (C.c_int, [vp, vp, vp, vp, C.c_int]),
+    "ssrh_backward_fused_optimizer": (C.c_int, [vp, vp, vp, vp, C.c_int, C.c_int]),
     "ssrh_copy_params_to_host": (C.c_int, [vp, vp, vp, vp, vp, vp]),
     "ssrh_set_tile_mask": (C.c_int, [vp, C.c_int, C.c_int]),
     "ssrh_forward_3dgs": (C.c_int, [C.c_char_p, C.c_int, C.c_int, C.c_int, C.c_int]),
@@ -148,11 +148,12 @@ class Engine:
              "scale_regularization_weight", "mcmc_opacity_reg_weight", "mcmc_scale_reg_weight", "quat_norm_reg_weight",
              "sh_reg_weight", "erank_reg_weight", "erank_reg_weight_s3"]
 
-    def backward_fused_optimizer(self, hyper, step):
+    def backward_fused_optimizer(self, hyper, step, scale_agnostic_mean=False):
         """Compositing backward, then the projection backward fused with the Adam step: the engine's
         parameters and its Adam moments are updated in place (fp32 SH only)."""
         hv = np.array([hyper.get(k, 0.0) for k in self.HYPER], np.float32)
-        check(self.h.ssrh_backward_fused_optimizer(self.d_vrgb.ptr, self.d_vdepth.ptr, self.d_vT.ptr, hv.ctypes.data, int(step)))
+        check(self.h.ssrh_backward_fused_optimizer(self.d_vrgb.ptr, self.d_vdepth.ptr, self.d_vT.ptr, hv.ctypes.data, int(step),
+                                                   int(scale_agnostic_mean)))
 
     def params(self):
         n = self.sc.n

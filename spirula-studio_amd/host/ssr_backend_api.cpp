@@ -629,7 +629,7 @@ void fused_projection_bwd_optimizer_3dgs(
     const std::vector<DeviceTensorFloatND> g1_splats_world, const std::vector<DeviceTensorFloatND> g2_splats_world,
     const std::optional<TorchTensorView> sh_packed, const std::optional<TorchTensorView>,
     const std::optional<TorchTensorView> sh_value_packed, const std::optional<TorchTensorView>, NonShQuantState non_sh,
-    DeviceVector<float>, DeviceVector<float> densify_score, const float lr_means, const float lr_quats,
+    DeviceVector<float> radii, DeviceVector<float> densify_score, const float lr_means, const float lr_quats,
     const float lr_scales, const float lr_opacs, const float lr_features_dc, const float lr_features_sh,
     const float max_gauss_ratio, const float scale_regularization_weight, const float mcmc_opacity_reg_weight,
     const float mcmc_scale_reg_weight, const float erank_reg_weight, const float erank_reg_weight_s3,
@@ -639,7 +639,6 @@ void fused_projection_bwd_optimizer_3dgs(
     const bool is_packed = camera_ids.data_ptr() && gaussian_ids.data_ptr();   // src/kernels/optim/FusedProjectionBwdOptim.cu:160
     if (sh_packed || non_sh.enabled || quantization_level != 0) throw std::runtime_error(std::string(w) + "quantized Adam state is not built in this backend");
     if (sh_value_packed) throw std::runtime_error(std::string(w) + "value-quantized SH is not built in this backend");
-    if (use_scale_agnostic_mean) throw std::runtime_error(std::string(w) + "the scale-agnostic mean step is not built in this backend");
     if (color_trust_linear) throw std::runtime_error(std::string(w) + "the colour trust region is not built in this backend");
     if (num_splats == 0) return;
     ssr_fpbo_params p;
@@ -662,6 +661,10 @@ void fused_projection_bwd_optimizer_3dgs(
     p.mcmc_opacity_reg_weight = mcmc_opacity_reg_weight; p.mcmc_scale_reg_weight = mcmc_scale_reg_weight;
     p.quat_norm_reg_weight = quat_norm_reg_weight; p.sh_reg_weight = sh_reg_weight;
     p.erank_reg_weight = erank_reg_weight; p.erank_reg_weight_s3 = erank_reg_weight_s3;
+    if (use_scale_agnostic_mean) {
+        if (!radii.data_ptr()) throw std::runtime_error(std::string(w) + "the scale-agnostic mean step needs the forward's radii");
+        p.scale_agnostic_radii = radii.data_ptr();
+    }
     if (const int32_t* s = std::get_if<int32_t>(&step)) {
         p.step = *s;
     } else {

@@ -278,7 +278,7 @@ void engine_backward_with_variants(TorchTensorView v_render_rgb, TorchTensorView
 }
 
 void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
-                                     TorchTensorView v_render_Ts, const float hyper[14], int step) {
+                                     TorchTensorView v_render_Ts, const float hyper[14], int step, bool scale_agnostic_mean) {
     auto& E = engine();
     if (std::get<0>(E.fwd.renders).data_ptr() == nullptr)
         throw std::runtime_error("engine_backward_fused_optimizer: forward_3dgs must be called first");
@@ -318,7 +318,7 @@ void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorVi
         E.camera.model_str, E.camera.distortion_str, E.camera.dist_coeffs, cam_ids, gauss_ids, aabb, {}, E.grad.v_screen,
         E.optim.g1, E.optim.g2, std::nullopt, std::nullopt, E.world.sh_packed, E.world.sh_bounds, NonShQuantState{},
         E.optim.radii, E.optim.densify_score, hyper[0], hyper[1], hyper[2], hyper[3], hyper[4], hyper[5], hyper[6], hyper[7],
-        hyper[8], hyper[9], hyper[12], hyper[13], hyper[10], hyper[11], false, false, 0.0f, (int32_t)step, 0);
+        hyper[8], hyper[9], hyper[12], hyper[13], hyper[10], hyper[11], scale_agnostic_mean, false, 0.0f, (int32_t)step, 0);
 }
 
 void engine_copy_params_to_host(TorchTensorView means, TorchTensorView quats, TorchTensorView scales,
@@ -445,10 +445,12 @@ int ssrh_backward_with_variants(const float* v_rgb, const float* v_depth, const 
     });
 }
 
-int ssrh_backward_fused_optimizer(const float* v_rgb, const float* v_depth, const float* v_Ts, const float* hyper14, int step) {
+int ssrh_backward_fused_optimizer(const float* v_rgb, const float* v_depth, const float* v_Ts, const float* hyper14, int step,
+                                  int scale_agnostic_mean) {
     return guard([&] {
         const int64_t C = engine().camera.num, H = engine().camera.height, W = engine().camera.width;
-        engine_backward_fused_optimizer(tv(v_rgb, 4, {C, H, W, 3}), tv(v_depth, 4, {C, H, W, 1}), tv(v_Ts, 4, {C, H, W, 1}), hyper14, step);
+        engine_backward_fused_optimizer(tv(v_rgb, 4, {C, H, W, 3}), tv(v_depth, 4, {C, H, W, 1}), tv(v_Ts, 4, {C, H, W, 1}), hyper14, step,
+                                        scale_agnostic_mean != 0);
     });
 }
 

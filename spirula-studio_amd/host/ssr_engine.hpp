@@ -83,8 +83,10 @@ void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorV
 // then fused_projection_bwd_optimizer_3dgs on the engine's parameters with Adam moments kept in pool
 // slots (zero on first use). hyper: lr_means, lr_quats, lr_scales, lr_opacs, lr_dc, lr_sh,
 // max_gauss_ratio, scale_reg_w, mcmc_opacity_w, mcmc_scale_w, quat_norm_w, sh_reg_w, erank_w, erank_w_s3.
+// scale_agnostic_mean: OptimConfig::use_scale_agnostic_mean (the means step on the forward's radii).
 void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
-                                     TorchTensorView v_render_Ts, const float hyper[14], int step);
+                                     TorchTensorView v_render_Ts, const float hyper[14], int step,
+                                     bool scale_agnostic_mean = false);
 // engine_backward_from_render_grad with the cotangents of the variants of the forward that ran
 // (any may be a null view): distortion image, median depth, and a pixel weight map to accumulate
 // per splat (the reference feeds these from its loss, src/engine/EngineLoss.cpp:138-216).

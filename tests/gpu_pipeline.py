@@ -326,7 +326,7 @@ class GpuRun:
             p.packed_gaussian_ids, p.num_packed = self.ptr("gaussian_ids"), self.rows
         self.check(self.lib.ssr_projection_bwd(C.byref(p), None))
 
-    def fused_optimizer(self, g1, g2, hyper, step=1, steps=None, v_in=None):
+    def fused_optimizer(self, g1, g2, hyper, step=1, steps=None, v_in=None, scale_agnostic=False):
         """ssr_fused_projection_bwd_optimizer on the device copies of the parameters (fp32 SH);
         g1 / g2 are host dicts keyed like the world arrays. Returns (params, g1, g2, score) from the device."""
         D = self.L.DeviceArray
@@ -356,6 +356,8 @@ class GpuRun:
             p.packed_row_of = self.ptr("row_of")
         if self.use_vrows:
             p.v_rows = self.ptr("v_rows")
+        if scale_agnostic:
+            p.scale_agnostic_radii = self.ptr("radii")
         self.check(self.lib.ssr_fused_projection_bwd_optimizer(C.byref(p), None))
         self.check(self.lib.ssr_device_synchronize())
         out = lambda pre: {k: self.host(pre + k) for k in keys}

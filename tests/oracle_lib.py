@@ -234,7 +234,7 @@ WORLD_KEYS = ["means", "quats", "log_scales", "opacity_logits", "features_dc", "
 
 
 def fused_projection_bwd_optimizer(scene, aabb, vs, params, g1, g2, hyper, step=1, steps=None, v_in=None,
-                                   sh_degree=3, densify=True):
+                                   sh_degree=3, densify=True, radii=None):
     """Updates params / g1 / g2 (dicts of float32 arrays keyed by WORLD_KEYS, fp32 SH [N,15,3]) in place
     and returns the densification score."""
     n = scene.n
@@ -256,7 +256,8 @@ def fused_projection_bwd_optimizer(scene, aabb, vs, params, g1, g2, hyper, step=
         C.c_int64(n), C.c_int(sh_degree), *[_p(params[k]) for k in WORLD_KEYS], C.byref(cam), _p(aabb),
         _p(vs["v_xy"]), _p(vs["v_depth"]), _p(vs["v_conic"]), _p(vs["v_opac"]), _p(vs["v_rgb"]),
         ptrs(v_in) if v_in is not None else None, ptrs(g1), ptrs(g2), _p(score), _p(hv), C.c_int32(step),
-        _p(None if steps is None else np.ascontiguousarray(steps, np.int32)))
+        _p(None if steps is None else np.ascontiguousarray(steps, np.int32)),
+        _p(None if radii is None else np.ascontiguousarray(radii, np.float32)))
     return score
 
 

@@ -197,6 +197,40 @@ def test_engine_packed_follows_the_camera_and_handles_nothing_visible(pkg, oracl
     look([[1, 0, 0, 0], [0, 1, 0, 0], [0, 0, 1, 0], [0, 0, 0, 1]])             # and back
 
 
+@pytest.mark.parametrize("packed", [False, True])
+def test_engine_fused_optimizer_scale_agnostic_means(pkg, oracle, H, packed):
+    """One step with OptimConfig::use_scale_agnostic_mean (the reference's default): the means move by
+    lr * (covariance-weighted gradient) / (gradient x 0.6 radii). A component whose own gradient is almost
+    zero takes a huge, rounding-dependent step in the reference too, so the steps are compared relatively
+    and a small fraction of such components is allowed to differ."""
+    host, lib = H
+    sc = pkg.scenes.make_scene(1, n=20000, width=320, height=240, parity_variant=True)
+    if packed:
+        sc.means[::3, 2] = -10.0
+    h = dict(lr_means=1.6e-4, lr_quats=1e-3, lr_scales=5e-3, lr_opacs=5e-2, lr_features_dc=2.5e-3, lr_features_sh=1.25e-4,
+             max_gauss_ratio=6.0, scale_regularization_weight=0.01, mcmc_opacity_reg_weight=0.01, mcmc_scale_reg_weight=0.01,
+             quat_norm_reg_weight=0.02, sh_reg_weight=0.05)
+    eng = host.Engine(sc, packed_projection=packed)
+    eng.forward()
+    eng.backward_fused_optimizer(h, 1, scale_agnostic_mean=True)
+    got = eng.params()
+    P = {k: np.ascontiguousarray(getattr(sc, k), np.float32).copy() for k in oracle.WORLD_KEYS}
+    g1 = {k: np.zeros_like(v) for k, v in P.items()}
+    g2 = {k: np.zeros_like(v) for k, v in P.items()}
+    r = oracle.pipeline(sc, backward=True)
+    oracle.fused_projection_bwd_optimizer(sc, r["proj"]["aabb"], r["vscreen"], P, g1, g2, h, step=1, radii=r["proj"]["radii"])
+    want = P["means"].astype(np.float64) - sc.means
+    step = got["means"].astype(np.float64) - sc.means
+    vis = r["proj"]["aabb"][:, 2] > r["proj"]["aabb"][:, 0]
+    assert not np.any(step[~vis]) and not np.any(want[~vis])          # no gradient, no step
+    assert np.abs(want[vis]).max() > 10 * h["lr_means"]                # not the plain Adam step
+    far = np.abs(step - want) > 0.05 * np.abs(want) + 1e-7
+    assert far[vis].mean() < 0.01, float(far[vis].mean())
+    for k in ["quats", "log_scales", "opacity_logits", "features_dc"]:  # the other parameters take the plain step
+        d = np.abs(got[k].astype(np.float64) - P[k])
+        assert (d > 0.05 * 5e-2).mean() < 2e-3, k
+
+
 def test_engine_packed_fused_optimizer_with_nothing_visible(pkg, oracle, H):
     """No packed rows at all: no projection gradient, but every splat still decays its moments and takes
     the regularizer step (the reference's kernel runs over all N splats whatever is visible)."""

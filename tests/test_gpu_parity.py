@@ -417,8 +417,10 @@ def test_fused_projection_bwd_optimizer(gpu, oracle, cfg):
     if cfg in ("tiny", "cfg4-packed", "fisheye-prism"):   # with the effective-rank regularizer (needles and blobs both occur)
         h.update(erank_reg_weight=0.1, erank_reg_weight_s3=0.01)
     steps = rng.integers(1, 400, sc.n).astype(np.int32) if cfg == "equirect-steps" else None
-    dP, d1, d2, dscore = g.fused_optimizer(g1, g2, h, step=37, steps=steps, v_in=v_in)
-    score = oracle.fused_projection_bwd_optimizer(sc, aabb, vs, P, g1, g2, h, step=37, steps=steps, v_in=v_in)
+    sa = cfg in ("tiny", "cfg4-packed", "cfg2")   # the scale-agnostic step of the means (the reference's default)
+    dP, d1, d2, dscore = g.fused_optimizer(g1, g2, h, step=37, steps=steps, v_in=v_in, scale_agnostic=sa)
+    score = oracle.fused_projection_bwd_optimizer(sc, aabb, vs, P, g1, g2, h, step=37, steps=steps, v_in=v_in,
+                                                  radii=g.host("radii") if sa else None)
     lrs = dict(means="lr_means", quats="lr_quats", log_scales="lr_scales", opacity_logits="lr_opacs",
                features_dc="lr_features_dc", features_sh="lr_features_sh")
     for k in oracle.WORLD_KEYS:

@@ -47,8 +47,16 @@ def _fd(f, x, eps=1e-6):
     return g
 
 
-@pytest.mark.parametrize("per_splat_steps", [False, True])
-def test_fused_optimizer_against_float64_adam(pkg, oracle, per_splat_steps):
+def _rot_raw(q):
+    """normalized_quat_to_rotmat (src/shaders/projection_utils.slang:69-88) applied to the quaternion as stored."""
+    w, x, y, z = q
+    return np.array([[1 - 2 * (y * y + z * z), 2 * (x * y - w * z), 2 * (x * z + w * y)],
+                     [2 * (x * y + w * z), 1 - 2 * (x * x + z * z), 2 * (y * z - w * x)],
+                     [2 * (x * z - w * y), 2 * (y * z + w * x), 1 - 2 * (x * x + y * y)]])
+
+
+@pytest.mark.parametrize("per_splat_steps,scale_agnostic", [(False, False), (True, False), (False, True)])
+def test_fused_optimizer_against_float64_adam(pkg, oracle, per_splat_steps, scale_agnostic):
     sc = pkg.scenes.tiny_scene(n=120, width=96, height=64, seed=51)
     sc.means[::4, 2] = -10.0                     # culled splats still decay their moments
     sc.log_scales[5] = [-2.0, -4.5, -3.0]        # ratio e^2.5 > max_gauss_ratio
@@ -71,8 +79,9 @@ def test_fused_optimizer_against_float64_adam(pkg, oracle, per_splat_steps):
     P0 = {k: v.astype(np.float64) for k, v in P.items()}
     G1 = {k: v.astype(np.float64) for k, v in g1.items()}
     G2 = {k: v.astype(np.float64) for k, v in g2.items()}
+    radii = r["proj"]["radii"] if scale_agnostic else None
     score = oracle.fused_projection_bwd_optimizer(sc, r["proj"]["aabb"], r["vscreen"], P, g1, g2, h, step=step,
-                                                  steps=steps, v_in=v_in)
+                                                  steps=steps, v_in=v_in, radii=radii)
     # ---- float64 expectation ----
     gr = r["grads"]
     data = dict(means=gr["v_means"] + v_in["means"], quats=gr["v_quats"], log_scales=gr["v_scales"],
@@ -99,6 +108,13 @@ def test_fused_optimizer_against_float64_adam(pkg, oracle, per_splat_steps):
                 v = v - np.dot(x, v) * x
             m1 = B1 * G1[k][g] + (1 - B1) * v
             m2 = B2 * G2[k][g] + (1 - B2) * v * v
+            if k == "means" and scale_agnostic:
+                # use_scale_agnostic_mean, FusedProjectionBwdOptim_kernel.cuh:519-534
+                Rm = _rot_raw(q)
+                cov = Rm @ np.diag(np.exp(ls)) @ Rm.T
+                extent = np.sqrt(2 * np.log(max(255.0 / (1 + np.exp(-lo)), 1.00001)))
+                m1 = B1 * G1[k][g] + (1 - B1) * (cov @ v) * extent
+                m2 = B2 * G2[k][g] + (1 - B2) * v * v * (0.6 * float(radii[g])) ** 2
             lr = h["lr_" + {"log_scales": "scales", "opacity_logits": "opacs"}.get(k, k)]
             new = x - lr * c1[g] * m1 / (np.sqrt(m2 * c2[g]) + EPS)
             if k == "quats":
