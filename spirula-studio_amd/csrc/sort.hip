@@ -16,8 +16,8 @@ namespace ssr {
 
 constexpr int kSortBlock = 256;                         // 4 wavefronts
 constexpr int kSortWaves = kSortBlock / 64;
-constexpr int kSortRounds = 16;                         // keys per lane
-constexpr int kSortTile = kSortBlock * kSortRounds;     // 4096 keys per workgroup
+constexpr int kSortRounds = 8;                          // keys per lane
+constexpr int kSortTile = kSortBlock * kSortRounds;     // 2048 keys per workgroup
 constexpr int kRadix = 256;
 
 __device__ __forceinline__ uint32_t digit_of(uint64_t key, int shift, uint32_t mask) {
@@ -146,7 +146,7 @@ __global__ __launch_bounds__(kSortBlock) void sort_scatter_kernel(
         off[r] = prev + rank;
     }
     __syncthreads();
-    {   // thread t owns digit t: per-wave counts become positions, inside this workgroup's 4096 keys in digit
+    {   // thread t owns digit t: per-wave counts become positions, inside this workgroup's keys in digit
         // order, of each wave's first key of the digit; s_shift[t] = where the digit's run goes in the output
         // minus where it starts in that order
         const uint32_t d = threadIdx.x;

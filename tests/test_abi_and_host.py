@@ -47,7 +47,7 @@ def test_argument_checks_without_device(L):
     assert lib.ssr_sort_end_bit(2500) == 44 and lib.ssr_sort_end_bit(8160) == 45
     assert lib.ssr_sort_end_bit(32400) == 47 and lib.ssr_sort_end_bit(32768) == 48
     assert lib.ssr_scan_scratch_bytes(0) == 0 and lib.ssr_scan_scratch_bytes(2049) == 16
-    assert lib.ssr_sort_scratch_bytes(0) == 0 and lib.ssr_sort_scratch_bytes(4097) == (2 * 256 + 256) * 4
+    assert lib.ssr_sort_scratch_bytes(0) == 0 and lib.ssr_sort_scratch_bytes(4097) == (3 * 256 + 256) * 4   # three 2048-key blocks
     assert lib.ssr_projection_fwd(None, None) != 0 and b"null params" in lib.ssr_last_error()
     assert lib.ssr_last_error() == b""                     # cleared by the read
     p = L.ProjectionFwdParams()
