@@ -93,7 +93,7 @@ __global__ __launch_bounds__(kSortBlock) void sort_scan_rows_kernel(uint32_t* __
 
 __global__ __launch_bounds__(kSortBlock) void sort_scatter_kernel(
     const uint64_t* __restrict__ keys_in, const int32_t* __restrict__ vals_in, uint64_t* __restrict__ keys_out,
-    int32_t* __restrict__ vals_out, int64_t n, int shift, uint32_t mask, int n_bits, uint32_t n_blocks,
+    int32_t* __restrict__ vals_out, int64_t n, int shift, uint32_t mask, uint32_t n_blocks,
     const uint32_t* __restrict__ hist, const uint32_t* __restrict__ totals) {
     __shared__ uint32_t wcount[kSortWaves][kRadix];   // per-wave running digit counts, then bases
     __shared__ uint32_t ws[kSortWaves], ws2[kSortWaves];
@@ -522,7 +522,7 @@ static int sort_pairs_impl(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, in
                            shift == begin_bit ? clear4 : nullptr);
         hipLaunchKernelGGL(sort_scan_rows_kernel, dim3(kRadix), dim3(kSortBlock), 0, s, hist, nb, totals);
         hipLaunchKernelGGL(sort_scatter_kernel, dim3(nb), dim3(kSortBlock), 0, s, k[cur], v[cur], k[cur ^ 1], v[cur ^ 1], n,
-                           shift, mask, bits, nb, hist, totals);
+                           shift, mask, nb, hist, totals);
         cur ^= 1;
     }
     SSR_CHECK_LAUNCH("ssr_sort_pairs_u64_i32");
