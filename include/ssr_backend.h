@@ -323,7 +323,8 @@ int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream_t stream);
  * per-splat range, FusedProjectionBwdOptim.cu:160-212 -- with one camera a splat has at most one
  * row, found through packed_row_of), regularizers mcmc_opacity, mcmc_scale, scale ratio, effective
  * rank, quaternion norm and SH/DC magnitude; the scale-agnostic step of the means. Not built
- * (rejected): quantized Adam state, value-quantized SH, colour trust region. */
+ * (rejected): quantized state of the non-SH parameters, 4-bit moments / 8-bit values, colour trust
+ * region. */
 typedef struct {
     int64_t num_splats;
     int32_t sh_degree;
@@ -347,6 +348,17 @@ typedef struct {
                                             (use_scale_agnostic_mean, FusedProjectionBwdOptim_kernel.cuh:519-534) */
     const int32_t* packed_row_of;   /* packed mode: [N], row of aabb / v_screen / v_rows that belongs to
                                        splat g, or -1 (ssr_packed_row_map); NULL = row g */
+    /* Quantized SH state, the reference's quantization level 1 (QUANT_BITS 8, VALUE_BITS 16;
+     * FusedProjectionBwdOptim_kernel.cuh:709-1030, codecs src/core/Tensor.h:936-1133,1300-1405): when
+     * sh_state_packed is given, the SH coefficients live in sh_value_packed (16-bit codes, one (min,max)
+     * per block of 256 splats) and their Adam moments in sh_state_packed (u, log_s bytes, one float4 of
+     * bounds per block), num_sh_buffer coefficients per splat in both; world / g1 / g2 .features_sh are
+     * then not used. All four arrays are updated in place; all-zero state arrays are the zero moments. */
+    uint16_t* sh_state_packed;      /* [N * 3 * num_sh_buffer] */
+    float* sh_state_bounds;         /* float4[ceil(N / 256)] */
+    uint16_t* sh_value_packed;      /* [N * 3 * num_sh_buffer] */
+    float* sh_value_bounds;         /* float2[ceil(N / 256)] */
+    uint32_t num_sh_buffer;
 } ssr_fpbo_params;
 int ssr_fused_projection_bwd_optimizer(const ssr_fpbo_params* p, ssr_stream_t stream);
 /* row_of[g] = i where gaussian_ids[i] == g, -1 for splats without a packed row (one camera, so ids

@@ -1,0 +1,68 @@
+// ssr_quant.h -- the block-wise codecs of the quantized optimizer state, one definition for the host
+// restatement and the device kernels.
+//
+// QuantizedAdamState<8, 256> (src/core/Tensor.h:936-1133): per cell two bytes, the linearly quantized
+// u = g1 / (sqrt(g2) + eps) and log_s = log1p(sqrt(g2) / eps), against per-block bounds
+// (u_min, u_max, log_s_min, log_s_max). QuantizedTensor<16, 256> (src/core/Tensor.h:1300-1405): one
+// 16-bit linear code per cell against per-block (min, max). Both are endpoint-exact and keep 0 <-> 0.
+//
+// log1p / expm1 are built on ssr_log / ssr_exp (the reference calls the CUDA math library), so codes can
+// differ from the reference's by one step where its log1pf rounds differently; here host and device
+// agree bit for bit.
+#pragma once
+
+#include "ssr_math.h"
+
+#define SSR_ADAMQ_EPS 1e-15f   /* QuantizedAdamState::kEps, the Adam denominator's epsilon */
+
+SSR_HD float ssr_log1p(float x) {   // x >= 0
+    const float u = 1.0f + x;
+    if (u == 1.0f) return x;
+    return ssr_log(u) * (x / (u - 1.0f));
+}
+SSR_HD float ssr_expm1(float y) {
+    const float u = ssr_exp(y);
+    if (u == 1.0f) return y;
+    const float um1 = u - 1.0f;
+    if (um1 == -1.0f) return -1.0f;
+    return um1 * (y / ssr_log(u));
+}
+// roundf (half away from zero) for the codes; negative inputs only need to land at or below zero
+SSR_HD float ssr_round_code(float x) {
+    const float r = ssr_floor(x);
+    return (x - r >= 0.5f) ? r + 1.0f : r;
+}
+
+// (g1, g2) -> (u, log_s): QuantizedAdamState::g1g2_to_us / forward_sqrt_g2
+SSR_HD void ssr_adamq_to_us(float g1, float g2, float* u, float* log_s) {
+    const float sq = ssr_sqrt(ssr_max(g2, 0.0f));
+    *u = g1 / (sq + SSR_ADAMQ_EPS);
+    *log_s = ssr_log1p(ssr_max(sq, 0.0f) * (1.0f / SSR_ADAMQ_EPS));
+}
+// code = u_q | s_q << 8 against bounds mm = (u_min, u_max, log_s_min, log_s_max): encode_g1g2_code
+SSR_HD uint32_t ssr_adamq_encode(float g1, float g2, const float mm[4]) {
+    float u, ls;
+    ssr_adamq_to_us(g1, g2, &u, &ls);
+    const float ur = ssr_max(mm[1] - mm[0], SSR_ADAMQ_EPS), sr = ssr_max(mm[3] - mm[2], SSR_ADAMQ_EPS);
+    const float uq = ssr_min(ssr_max(ssr_round_code((255.0f * (u - mm[0])) / ur), 0.0f), 255.0f);
+    const float sq = ssr_min(ssr_max(ssr_round_code((255.0f * (ls - mm[2])) / sr), 0.0f), 255.0f);
+    return (uint32_t)uq | ((uint32_t)sq << 8);
+}
+// decode_g1g2
+SSR_HD void ssr_adamq_decode(uint32_t code, const float mm[4], float* g1, float* g2) {
+    const float kInv = 1.0f / 255.0f;
+    const float u = mm[0] + (mm[1] - mm[0]) * ((float)(code & 255u) * kInv);
+    const float ls = mm[2] + (mm[3] - mm[2]) * ((float)((code >> 8) & 255u) * kInv);
+    const float sq = SSR_ADAMQ_EPS * ssr_expm1(ls);
+    *g1 = u * (sq + SSR_ADAMQ_EPS);
+    *g2 = sq * sq;
+}
+
+// QuantizedTensor<16>::encode_v_code / decode_v against bounds (lo, hi)
+SSR_HD uint32_t ssr_q16_encode(float v, float lo, float hi) {
+    const float range = ssr_max(hi - lo, 1e-30f);
+    return (uint32_t)ssr_min(ssr_max(ssr_round_code((65535.0f * (v - lo)) / range), 0.0f), 65535.0f);
+}
+SSR_HD float ssr_q16_decode(uint32_t code, float lo, float hi) {
+    return lo + (hi - lo) * ((float)code * (1.0f / 65535.0f));
+}

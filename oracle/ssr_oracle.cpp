@@ -9,6 +9,7 @@
 #include "ssr_oracle.h"
 #include "../include/ssr_math.h"
 #include "../include/ssr_camera.h"
+#include "../include/ssr_quant.h"
 
 #include <algorithm>
 #include <cmath>
@@ -516,8 +517,18 @@ float or_erank_reg(const float* log_scales, float w, float w3, float* grad) {
     return ssr_erank_reg_grad(log_scales, w, w3, grad);
 }
 
-void or_fused_projection_bwd_optimizer(int64_t N, int sh_degree,
+void or_quant_codec(int op, int64_t n, float* a, float* b, const float* mm, uint32_t* codes) {
+    for (int64_t i = 0; i < n; i++) {
+        if (op == 0) codes[i] = ssr_adamq_encode(a[i], b[i], mm);
+        else if (op == 1) ssr_adamq_decode(codes[i], mm, a + i, b + i);
+        else if (op == 2) codes[i] = ssr_q16_encode(a[i], mm[0], mm[1]);
+        else a[i] = ssr_q16_decode(codes[i], mm[0], mm[1]);
+    }
+}
+
+static void fused_optimizer_impl(int64_t N, int sh_degree,
     float* means, float* quats, float* log_scales, float* opacity_logits, float* features_dc, float* features_sh,
+    const or_sh_quant_state* q,
     const or_camera* cam, const float* aabb,
     const float* v_xy, const float* v_sdepth, const float* v_conic, const float* v_opac, const float* v_srgb,
     const float* const* v_in, float* const* g1, float* const* g2, float* densify_score,
@@ -528,6 +539,12 @@ void or_fused_projection_bwd_optimizer(int64_t N, int sh_degree,
     or_sh_source src;
     memset(&src, 0, sizeof(src));
     src.codec = OR_SH_F32; src.sh_f32 = features_sh; src.num_sh_buffer = 15;
+    if (q) {
+        // the view-direction gradient is taken against the decoded coefficients
+        // (FusedProjectionBwdOptim_kernel.cuh:289-310)
+        src.codec = OR_SH_REF_Q16; src.sh_f32 = nullptr; src.packed = reinterpret_cast<const uint8_t*>(q->value_packed); src.bounds = q->value_bounds;
+        src.num_sh_buffer = q->num_sh_buffer; src.bounds_stride = (int64_t)256 * 3 * q->num_sh_buffer;
+    }
     or_projection_bwd(N, sh_degree, means, quats, log_scales, opacity_logits, features_dc, &src, cam, aabb, v_xy, v_sdepth,
                       v_conic, v_opac, v_srgb, vm.data(), vq.data(), vs.data(), vo.data(), vd.data(), vsh.data());
     const float lr_means = hyper[0], lr_quats = hyper[1], lr_scales = hyper[2], lr_opacs = hyper[3], lr_dc = hyper[4],
@@ -561,8 +578,8 @@ void or_fused_projection_bwd_optimizer(int64_t N, int sh_degree,
         }
         for (int i = 0; i < 4; i++) gq[i] = vin(1, 4 * g + i) + vq[4 * g + i];
         go = vin(3, g) + vo[g];
-        // SH
-        for (int i = 0; i < 3 * n_coef; i++) {
+        // SH (fp32 state; the quantized state is updated block by block below)
+        for (int i = 0; !q && i < 3 * n_coef; i++) {
             float* x = features_sh + 45 * g + i;
             *x = adam(*x, vsh[45 * g + i] + sh_reg * *x, lr_sh, g1[5] + 45 * g + i, g2[5] + 45 * g + i);
         }
@@ -639,6 +656,94 @@ void or_fused_projection_bwd_optimizer(int64_t N, int sh_degree,
         for (int i = 0; i < 3; i++)
             features_dc[3 * g + i] = adam(features_dc[3 * g + i], gd[i], lr_dc, g1[4] + 3 * g + i, g2[4] + 3 * g + i);
     }
+    if (!q) return;
+    // ---- SH coefficients and moments in the quantized state, FusedProjectionBwdOptim_kernel.cuh:709-1030 ----
+    // Per block of 256 splats: decode moments and values against the block's OLD bounds, take the Adam step in
+    // fp32, reduce min / max of the new (u, log_s) and of the new values over the block, store those as the NEW
+    // bounds, encode against them. Coefficients above the active degree are re-encoded as zeros, and the new
+    // bounds are widened to contain zero when there are any (:842-861, :925-938).
+    const int64_t R = 3 * (int64_t)q->num_sh_buffer;
+    const int64_t n_blocks = (N + 255) / 256;
+#pragma omp parallel for schedule(static)
+    for (int64_t blk = 0; blk < n_blocks; blk++) {
+        const int64_t g0 = blk * 256, g1e = (g0 + 256 < N) ? g0 + 256 : N;
+        const int n_here = (int)(g1e - g0);
+        float old_mm[4], new_mm[4] = {1e30f, -1e30f, 1e30f, -1e30f};
+        for (int k = 0; k < 4; k++) old_mm[k] = q->state_bounds[4 * blk + k];
+        const float old_lo = q->value_bounds[2 * blk], old_hi = q->value_bounds[2 * blk + 1];
+        float new_lo = 1e30f, new_hi = -1e30f;
+        std::vector<float> ng1((size_t)n_here * 3 * n_coef), ng2(ng1.size()), nx(ng1.size());
+        for (int s = 0; s < n_here; s++) {
+            const int64_t g = g0 + s;
+            float b1c, b2c;
+            if (steps) {
+                const float t = (float)steps[g];
+                b1c = 1.0f / (1.0f - ssr_exp(t * -0.105360515657826301f));
+                b2c = 1.0f / (1.0f - ssr_exp(t * -0.00100050033358353350f));
+            } else {
+                b1c = (float)(1.0 / (1.0 - pow(0.9, (double)step)));
+                b2c = (float)(1.0 / (1.0 - pow(0.999, (double)step)));
+            }
+            for (int i = 0; i < 3 * n_coef; i++) {
+                const int64_t cell = R * g + i;
+                float m1, m2;
+                ssr_adamq_decode(q->state_packed[cell], old_mm, &m1, &m2);
+                const float x = ssr_q16_decode(q->value_packed[cell], old_lo, old_hi);
+                const float v = vsh[45 * g + i] + sh_reg * x;
+                const float a = kBeta1 * m1 + (1.f - kBeta1) * v;
+                const float b = kBeta2 * m2 + (1.f - kBeta2) * (v * v);
+                const float xn = x - ((lr_sh * b1c) * a) / (ssr_sqrt(b * b2c) + kEps);
+                const size_t o = (size_t)s * 3 * n_coef + i;
+                ng1[o] = a; ng2[o] = b; nx[o] = xn;
+                float u, ls;
+                ssr_adamq_to_us(a, b, &u, &ls);
+                new_mm[0] = ssr_min(new_mm[0], u); new_mm[1] = ssr_max(new_mm[1], u);
+                new_mm[2] = ssr_min(new_mm[2], ls); new_mm[3] = ssr_max(new_mm[3], ls);
+                new_lo = ssr_min(new_lo, xn); new_hi = ssr_max(new_hi, xn);
+            }
+            if (R > 3 * n_coef) {
+                new_lo = ssr_min(new_lo, 0.0f); new_hi = ssr_max(new_hi, 0.0f);
+                new_mm[0] = ssr_min(new_mm[0], 0.0f); new_mm[1] = ssr_max(new_mm[1], 0.0f);
+                new_mm[2] = ssr_min(new_mm[2], 0.0f);
+            }
+        }
+        for (int k = 0; k < 4; k++) q->state_bounds[4 * blk + k] = new_mm[k];
+        q->value_bounds[2 * blk] = new_lo; q->value_bounds[2 * blk + 1] = new_hi;
+        for (int s = 0; s < n_here; s++) {
+            const int64_t g = g0 + s;
+            for (int64_t i = 0; i < R; i++) {
+                const int64_t cell = R * g + i;
+                if (i < 3 * n_coef) {
+                    const size_t o = (size_t)s * 3 * n_coef + (size_t)i;
+                    q->state_packed[cell] = (uint16_t)ssr_adamq_encode(ng1[o], ng2[o], new_mm);
+                    q->value_packed[cell] = (uint16_t)ssr_q16_encode(nx[o], new_lo, new_hi);
+                } else {
+                    q->state_packed[cell] = (uint16_t)ssr_adamq_encode(0.0f, 0.0f, new_mm);
+                    q->value_packed[cell] = (uint16_t)ssr_q16_encode(0.0f, new_lo, new_hi);
+                }
+            }
+        }
+    }
+}
+
+void or_fused_projection_bwd_optimizer(int64_t N, int sh_degree,
+    float* means, float* quats, float* log_scales, float* opacity_logits, float* features_dc, float* features_sh,
+    const or_camera* cam, const float* aabb,
+    const float* v_xy, const float* v_sdepth, const float* v_conic, const float* v_opac, const float* v_srgb,
+    const float* const* v_in, float* const* g1, float* const* g2, float* densify_score,
+    const float* hyper, int32_t step, const int32_t* steps, const float* radii) {
+    fused_optimizer_impl(N, sh_degree, means, quats, log_scales, opacity_logits, features_dc, features_sh, nullptr, cam, aabb,
+                         v_xy, v_sdepth, v_conic, v_opac, v_srgb, v_in, g1, g2, densify_score, hyper, step, steps, radii);
+}
+
+void or_fused_projection_bwd_optimizer_q(int64_t N, int sh_degree,
+    float* means, float* quats, float* log_scales, float* opacity_logits, float* features_dc, const or_sh_quant_state* q,
+    const or_camera* cam, const float* aabb,
+    const float* v_xy, const float* v_sdepth, const float* v_conic, const float* v_opac, const float* v_srgb,
+    const float* const* v_in, float* const* g1, float* const* g2, float* densify_score,
+    const float* hyper, int32_t step, const int32_t* steps, const float* radii) {
+    fused_optimizer_impl(N, sh_degree, means, quats, log_scales, opacity_logits, features_dc, nullptr, q, cam, aabb,
+                         v_xy, v_sdepth, v_conic, v_opac, v_srgb, v_in, g1, g2, densify_score, hyper, step, steps, radii);
 }
 
 

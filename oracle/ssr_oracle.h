@@ -142,6 +142,29 @@ void or_fused_projection_bwd_optimizer(int64_t N, int sh_degree,
     const float* hyper, int32_t step, const int32_t* steps,
     const float* radii /* optional [N]: the forward's radii; given = the scale-agnostic step of the means */);
 
+/* The quantized SH state of the fused optimizer at the reference's quantization level 1
+ * (src/kernels/optim/FusedProjectionBwdOptim_kernel.cuh:709-1030 with QUANT_BITS = 8, VALUE_BITS = 16):
+ * per block of 256 splats, Adam moments as QuantizedAdamState<8,256> cells (2 bytes: u, log_s; bounds
+ * float4) and SH values as QuantizedTensor<16,256> cells (bounds float2); num_sh_buffer coefficients per
+ * splat in both buffers. Pass to or_fused_projection_bwd_optimizer_q. */
+typedef struct {
+    uint16_t* state_packed;     /* [N * 3 * num_sh_buffer] u_q | s_q << 8 */
+    float* state_bounds;        /* float4[ceil(N / 256)] */
+    uint16_t* value_packed;     /* [N * 3 * num_sh_buffer] */
+    float* value_bounds;        /* float2[ceil(N / 256)] */
+    uint32_t num_sh_buffer;
+} or_sh_quant_state;
+/* As or_fused_projection_bwd_optimizer, with the SH coefficients and their moments held in q. */
+void or_fused_projection_bwd_optimizer_q(int64_t N, int sh_degree,
+    float* means, float* quats, float* log_scales, float* opacity_logits, float* features_dc, const or_sh_quant_state* q,
+    const or_camera* cam, const float* aabb,
+    const float* v_xy, const float* v_sdepth, const float* v_conic, const float* v_opac, const float* v_srgb,
+    const float* const* v_in, float* const* g1, float* const* g2, float* densify_score,
+    const float* hyper, int32_t step, const int32_t* steps, const float* radii);
+/* The codecs on arrays: op 0 Adam-state encode (a = g1, b = g2, mm float4 -> codes), 1 Adam-state decode
+ * (codes -> a = g1, b = g2), 2 value encode (a = v, mm float2 -> codes), 3 value decode (codes -> a). */
+void or_quant_codec(int op, int64_t n, float* a, float* b, const float* mm, uint32_t* codes);
+
 /* erank_reg_3dgs (src/shaders/per_splat_losses.slang:3-15): the loss for one splat's three log-scales and
  * its gradient. */
 float or_erank_reg(const float* log_scales, float w, float w3, float* grad);

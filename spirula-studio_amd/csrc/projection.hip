@@ -15,6 +15,7 @@
 #include <string.h>
 
 #include "projection_device.h"
+#include "../../include/ssr_quant.h"
 #include "raster_device.h"
 
 namespace ssr {
@@ -635,13 +636,14 @@ __device__ __forceinline__ float adam_step(float x, float v, float lr, const Ada
 // (Y_j * v_colour), so only its factors (15 + 3 floats) go to LDS. Phase 2, the workgroup streams
 // over its 256 x 3 kCoef SH coefficients in memory order: parameter and both moments are read and
 // written fully coalesced, the gradient is rebuilt from the factors in LDS.
-template <int kDegree, bool kLens>
+template <int kDegree, bool kLens, bool kQuant>
 __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_kernel(ssr_fpbo_params P, AdamD scalar_adam) {
     constexpr int kCoef = kDegree * (kDegree + 2);
     constexpr int kY = kCoef > 0 ? kCoef : 1;
     __shared__ float s_Y[kProjBlock][kY + 1];   // +1: odd row pitch, conflict-free column reads
     __shared__ float s_vc[kProjBlock][3];
     __shared__ float s_b1c[kProjBlock], s_b2c[kProjBlock];
+    __shared__ float s_red[kProjBlock / 64][6];   // quantized state: per-wave min / max of the new bounds
     const int64_t block0 = (int64_t)blockIdx.x * kProjBlock;
     const int64_t g = block0 + threadIdx.x;
     const ssr_world& W = P.world;
@@ -678,6 +680,10 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
             ssr_sh_quant none;
             none.codec = SSR_SH_F32; none.packed = nullptr; none.bounds = nullptr; none.bounds_stride = 0;
             none.num_sh_buffer = 0; none.scale_f16 = nullptr;
+            if (kQuant) {   // the view-direction gradient is taken against the decoded 16-bit coefficients
+                none.codec = SSR_SH_REF_Q16; none.packed = P.sh_value_packed; none.bounds = P.sh_value_bounds;
+                none.num_sh_buffer = P.num_sh_buffer; none.bounds_stride = (int64_t)kProjBlock * 3 * P.num_sh_buffer;
+            }
             projection_vjp<kDegree, kLens>(cam, W, none, g, vscreen_of(P.v_screen, P.v_rows), row, pg, [&](int j, float Yj, const float vc[3]) {
                 s_Y[threadIdx.x][j] = Yj;
                 if (j == 0) { s_vc[threadIdx.x][0] = vc[0]; s_vc[threadIdx.x][1] = vc[1]; s_vc[threadIdx.x][2] = vc[2]; }
@@ -796,6 +802,99 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
     const int n_here = rest < kProjBlock ? (int)rest : kProjBlock;
     const float sh_reg = P.sh_reg_weight * (1.0f / (float)kY);
     constexpr int kPer = 3 * kCoef;
+    if (kQuant) {
+        // Quantized state (FusedProjectionBwdOptim_kernel.cuh:709-1030 at QUANT_BITS 8, VALUE_BITS 16): moments and
+        // values of this block's cells are decoded against the block's old bounds, stepped in fp32, and encoded
+        // against the min / max of the results. The workgroup walks the cells in memory order twice -- once for
+        // the new bounds, once (recomputing the same step from the same old codes) to encode -- rather than
+        // holding 3 x 45 results per thread.
+        const int R = 3 * (int)P.num_sh_buffer;                    // cells per splat
+        const int64_t cell0 = block0 * R;
+        const int n_cells = n_here * R;
+        float old_mm[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) old_mm[k] = P.sh_state_bounds[4 * blockIdx.x + k];
+        const float old_lo = P.sh_value_bounds[2 * blockIdx.x], old_hi = P.sh_value_bounds[2 * blockIdx.x + 1];
+        auto step_cell = [&](int sp, int k, float& m1, float& m2, float& xn) {
+            const int64_t cell = cell0 + (int64_t)sp * R + k;
+            ssr_adamq_decode(P.sh_state_packed[cell], old_mm, &m1, &m2);
+            const float x = ssr_q16_decode(P.sh_value_packed[cell], old_lo, old_hi);
+            const int j = k / 3, c = k - 3 * j;
+            const float v = s_Y[sp][j] * s_vc[sp][c] + sh_reg * x;
+            constexpr float kBeta1 = 0.9f, kBeta2 = 0.999f, kEps = 1e-15f;
+            m1 = kBeta1 * m1 + (1.f - kBeta1) * v;
+            m2 = kBeta2 * m2 + (1.f - kBeta2) * (v * v);
+            xn = x - ((P.lr_features_sh * s_b1c[sp]) * m1) / (ssr_sqrt(m2 * s_b2c[sp]) + kEps);
+        };
+        float mn[3] = {1e30f, 1e30f, 1e30f}, mx[3] = {-1e30f, -1e30f, -1e30f};   // u, log_s, value
+        {
+            int sp = (int)threadIdx.x / R, k = (int)threadIdx.x - sp * R;
+            const int dsp = kProjBlock / R, dk = kProjBlock - dsp * R;
+            for (int e = threadIdx.x; e < n_cells; e += kProjBlock) {
+                if (k < kPer) {
+                    float m1, m2, xn, u, ls;
+                    step_cell(sp, k, m1, m2, xn);
+                    ssr_adamq_to_us(m1, m2, &u, &ls);
+                    mn[0] = ssr_min(mn[0], u); mx[0] = ssr_max(mx[0], u);
+                    mn[1] = ssr_min(mn[1], ls); mx[1] = ssr_max(mx[1], ls);
+                    mn[2] = ssr_min(mn[2], xn); mx[2] = ssr_max(mx[2], xn);
+                }
+                sp += dsp; k += dk;
+                if (k >= R) { k -= R; sp++; }
+            }
+        }
+        if (R > kPer && n_here > 0) {   // coefficients above the active degree are re-encoded as zeros: cover zero
+            mn[0] = ssr_min(mn[0], 0.0f); mx[0] = ssr_max(mx[0], 0.0f);
+            mn[1] = ssr_min(mn[1], 0.0f);
+            mn[2] = ssr_min(mn[2], 0.0f); mx[2] = ssr_max(mx[2], 0.0f);
+        }
+#pragma unroll
+        for (int k = 0; k < 3; k++) {
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) {
+                mn[k] = ssr_min(mn[k], __shfl_xor(mn[k], d, 64));
+                mx[k] = ssr_max(mx[k], __shfl_xor(mx[k], d, 64));
+            }
+        }
+        __syncthreads();   // s_red is free (first use), and every wavefront has finished reading the old codes
+        if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+            for (int k = 0; k < 3; k++) { s_red[threadIdx.x >> 6][2 * k] = mn[k]; s_red[threadIdx.x >> 6][2 * k + 1] = mx[k]; }
+        }
+        __syncthreads();
+        float new_mm[4], new_lo, new_hi;
+        {
+            float a[6];
+#pragma unroll
+            for (int k = 0; k < 6; k++) {
+                a[k] = s_red[0][k];
+#pragma unroll
+                for (int w = 1; w < kProjBlock / 64; w++) a[k] = (k & 1) ? ssr_max(a[k], s_red[w][k]) : ssr_min(a[k], s_red[w][k]);
+            }
+            new_mm[0] = a[0]; new_mm[1] = a[1]; new_mm[2] = a[2]; new_mm[3] = a[3]; new_lo = a[4]; new_hi = a[5];
+        }
+        // second walk: the same step from the same old codes, encoded against the new bounds. A cell is read and
+        // written by the same thread, and the bounds are written only after every thread has them in registers.
+        {
+            int sp = (int)threadIdx.x / R, k = (int)threadIdx.x - sp * R;
+            const int dsp = kProjBlock / R, dk = kProjBlock - dsp * R;
+            for (int e = threadIdx.x; e < n_cells; e += kProjBlock) {
+                const int64_t cell = cell0 + (int64_t)sp * R + k;
+                float m1 = 0.0f, m2 = 0.0f, xn = 0.0f;
+                if (k < kPer) step_cell(sp, k, m1, m2, xn);
+                P.sh_state_packed[cell] = (uint16_t)ssr_adamq_encode(m1, m2, new_mm);
+                P.sh_value_packed[cell] = (uint16_t)ssr_q16_encode(xn, new_lo, new_hi);
+                sp += dsp; k += dk;
+                if (k >= R) { k -= R; sp++; }
+            }
+        }
+        if (threadIdx.x == 0) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) P.sh_state_bounds[4 * blockIdx.x + k] = new_mm[k];
+            P.sh_value_bounds[2 * blockIdx.x] = new_lo; P.sh_value_bounds[2 * blockIdx.x + 1] = new_hi;
+        }
+        return;
+    }
     for (int e = threadIdx.x; e < n_here * kPer; e += kProjBlock) {
         const int sp = e / kPer, i = e - sp * kPer;
         const int j = i / 3, c = i - 3 * j;
@@ -1041,16 +1140,26 @@ extern "C" int ssr_fused_projection_bwd_optimizer(const ssr_fpbo_params* p, ssr_
     SSR_REQUIRE(p, where, "null params");
     ssr_sh_quant none;
     memset(&none, 0, sizeof(none));
+    if (p->sh_state_packed) {   // the coefficients are read from the 16-bit value codes
+        none.codec = SSR_SH_REF_Q16; none.packed = p->sh_value_packed; none.bounds = p->sh_value_bounds;
+        none.num_sh_buffer = p->num_sh_buffer;
+    }
     int e = check_common(where, p->num_splats, p->sh_degree, p->world, none, p->camera);
     if (e) return e;
     if (p->num_splats == 0) return 0;
     SSR_REQUIRE(p->aabb && (reinterpret_cast<uintptr_t>(p->aabb) & 15) == 0, where, "aabb must be non-null and 16-byte aligned");
     SSR_REQUIRE(p->v_rows || (p->v_screen.xy && p->v_screen.depth && p->v_screen.conic && p->v_screen.opac && p->v_screen.rgb), where,
                 "null v_screen buffer");
+    const bool quant = p->sh_state_packed != nullptr;
     for (const ssr_world* w : {&p->world, &p->g1, &p->g2}) {
         SSR_REQUIRE(w->means && w->quats && w->log_scales && w->opacity_logits && w->features_dc, where, "null parameter or moment buffer");
-        SSR_REQUIRE(p->sh_degree == 0 || (w->features_sh && w->sh_stride >= 3 * p->sh_degree * (p->sh_degree + 2)), where,
+        SSR_REQUIRE(quant || p->sh_degree == 0 || (w->features_sh && w->sh_stride >= 3 * p->sh_degree * (p->sh_degree + 2)), where,
                     "features_sh missing or sh_stride too small");
+    }
+    if (quant) {
+        SSR_REQUIRE(p->sh_state_bounds && p->sh_value_packed && p->sh_value_bounds, where, "null quantized SH state buffer");
+        SSR_REQUIRE((int)p->num_sh_buffer >= p->sh_degree * (p->sh_degree + 2) && p->num_sh_buffer <= 15u, where,
+                    "num_sh_buffer must cover the SH degree (at most 15)");
     }
     SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->world.quats) & 15) == 0, where, "quats must be 16-byte aligned");
     SSR_REQUIRE(p->steps || p->step >= 1, where, "Adam step must be >= 1");
@@ -1060,9 +1169,14 @@ extern "C" int ssr_fused_projection_bwd_optimizer(const ssr_fpbo_params* p, ssr_
     const dim3 grid((unsigned)ceil_div(p->num_splats, kProjBlock)), block(kProjBlock);
     hipStream_t s = as_stream(stream);
     const bool lens = camera_needs_lens_path(p->camera.camera_model, p->camera.distortion);
-#define SSR_LAUNCH_FPBO(D)                                                                                       \
-    if (lens) hipLaunchKernelGGL((fused_projection_bwd_optimizer_kernel<D, true>), grid, block, 0, s, *p, ad);    \
-    else hipLaunchKernelGGL((fused_projection_bwd_optimizer_kernel<D, false>), grid, block, 0, s, *p, ad)
+#define SSR_LAUNCH_FPBO(D)                                                                                              \
+    if (quant) {                                                                                                        \
+        if (lens) hipLaunchKernelGGL((fused_projection_bwd_optimizer_kernel<D, true, true>), grid, block, 0, s, *p, ad);  \
+        else hipLaunchKernelGGL((fused_projection_bwd_optimizer_kernel<D, false, true>), grid, block, 0, s, *p, ad);      \
+    } else {                                                                                                            \
+        if (lens) hipLaunchKernelGGL((fused_projection_bwd_optimizer_kernel<D, true, false>), grid, block, 0, s, *p, ad); \
+        else hipLaunchKernelGGL((fused_projection_bwd_optimizer_kernel<D, false, false>), grid, block, 0, s, *p, ad);     \
+    }
     switch (p->sh_degree) {
         case 0: SSR_LAUNCH_FPBO(0); break;
         case 1: SSR_LAUNCH_FPBO(1); break;

@@ -23,7 +23,8 @@ SYMBOLS = {
     "ssrh_set_sh_value_quant": (C.c_int, [C.c_int, vp, C.c_int64, C.c_int, vp, C.c_int64, C.c_int, C.c_int64]),
     "ssrh_set_camera_params": (C.c_int, [C.c_int, C.c_int, C.c_char_p, C.c_char_p, vp, vp, vp, C.c_int]),
     "ssrh_backward_with_variants": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, C.c_int]),
-    "ssrh_backward_fused_optimizer": (C.c_int, [vp, vp, vp, vp, C.c_int, C.c_int]),
+    "ssrh_backward_fused_optimizer": (C.c_int, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int]),
+    "ssrh_copy_sh_quant_state": (C.c_int, [vp, vp, vp, vp]),
     "ssrh_copy_params_to_host": (C.c_int, [vp, vp, vp, vp, vp, vp]),
     "ssrh_set_tile_mask": (C.c_int, [vp, C.c_int, C.c_int]),
     "ssrh_forward_3dgs": (C.c_int, [C.c_char_p, C.c_int, C.c_int, C.c_int, C.c_int]),
@@ -148,12 +149,21 @@ class Engine:
              "scale_regularization_weight", "mcmc_opacity_reg_weight", "mcmc_scale_reg_weight", "quat_norm_reg_weight",
              "sh_reg_weight", "erank_reg_weight", "erank_reg_weight_s3"]
 
-    def backward_fused_optimizer(self, hyper, step, scale_agnostic_mean=False):
+    def backward_fused_optimizer(self, hyper, step, scale_agnostic_mean=False, quantization_level=0):
         """Compositing backward, then the projection backward fused with the Adam step: the engine's
         parameters and its Adam moments are updated in place (fp32 SH only)."""
         hv = np.array([hyper.get(k, 0.0) for k in self.HYPER], np.float32)
         check(self.h.ssrh_backward_fused_optimizer(self.d_vrgb.ptr, self.d_vdepth.ptr, self.d_vT.ptr, hv.ctypes.data, int(step),
-                                                   int(scale_agnostic_mean)))
+                                                   int(scale_agnostic_mean), int(quantization_level)))
+
+    def sh_quant_state(self):
+        """Quantization level 1: the engine's SH moments and values as host arrays."""
+        n, R = self.sc.n, 45
+        nb = (n + 255) // 256
+        q = dict(state_packed=np.zeros(n * R, np.uint16), state_bounds=np.zeros((nb, 4), np.float32),
+                 value_packed=np.zeros(n * R, np.uint16), value_bounds=np.zeros((nb, 2), np.float32), num_sh_buffer=15)
+        check(self.h.ssrh_copy_sh_quant_state(*[q[k].ctypes.data for k in ["state_packed", "state_bounds", "value_packed", "value_bounds"]]))
+        return q
 
     def params(self):
         n = self.sc.n

@@ -627,8 +627,8 @@ void fused_projection_bwd_optimizer_3dgs(
     const DeviceVector<int32_t> camera_ids, const DeviceVector<int32_t> gaussian_ids, DeviceTensorFloatND aabb,
     const std::vector<DeviceTensorFloatND> v_splats_world, const std::vector<DeviceTensorFloatND> v_splats_screen,
     const std::vector<DeviceTensorFloatND> g1_splats_world, const std::vector<DeviceTensorFloatND> g2_splats_world,
-    const std::optional<TorchTensorView> sh_packed, const std::optional<TorchTensorView>,
-    const std::optional<TorchTensorView> sh_value_packed, const std::optional<TorchTensorView>, NonShQuantState non_sh,
+    const std::optional<TorchTensorView> sh_packed, const std::optional<TorchTensorView> sh_quant_bounds,
+    const std::optional<TorchTensorView> sh_value_packed, const std::optional<TorchTensorView> sh_value_bounds, NonShQuantState non_sh,
     DeviceVector<float> radii, DeviceVector<float> densify_score, const float lr_means, const float lr_quats,
     const float lr_scales, const float lr_opacs, const float lr_features_dc, const float lr_features_sh,
     const float max_gauss_ratio, const float scale_regularization_weight, const float mcmc_opacity_reg_weight,
@@ -637,8 +637,14 @@ void fused_projection_bwd_optimizer_3dgs(
     float, std::variant<int32_t, TorchTensorView> step, int quantization_level) {
     const char* w = "fused_projection_bwd_optimizer_3dgs: ";
     const bool is_packed = camera_ids.data_ptr() && gaussian_ids.data_ptr();   // src/kernels/optim/FusedProjectionBwdOptim.cu:160
-    if (sh_packed || non_sh.enabled || quantization_level != 0) throw std::runtime_error(std::string(w) + "quantized Adam state is not built in this backend");
-    if (sh_value_packed) throw std::runtime_error(std::string(w) + "value-quantized SH is not built in this backend");
+    // quantization_level: 0 = fp32 SH and moments; 1 = 16-bit SH values, 8-bit moments
+    // (src/kernels/optim/FusedProjectionBwdOptim_kernel.cuh:1104-1111; validation as FusedProjectionBwdOptim.cu:386-400)
+    if (quantization_level != 0 && quantization_level != 1) throw std::runtime_error(std::string(w) + "quantization_level must be 0 or 1");
+    if (non_sh.enabled) throw std::runtime_error(std::string(w) + "quantized state of the non-SH parameters is not built in this backend");
+    const bool quant = quantization_level == 1;
+    if (quant && !(sh_packed && sh_quant_bounds && sh_value_packed && sh_value_bounds))
+        throw std::runtime_error(std::string(w) + "quantization level 1 needs the packed SH state, the packed SH values and both bounds");
+    if (!quant && (sh_packed || sh_value_packed)) throw std::runtime_error(std::string(w) + "packed SH buffers given at quantization level 0");
     if (color_trust_linear) throw std::runtime_error(std::string(w) + "the colour trust region is not built in this backend");
     if (num_splats == 0) return;
     ssr_fpbo_params p;
@@ -646,6 +652,13 @@ void fused_projection_bwd_optimizer_3dgs(
     p.num_splats = num_splats;
     p.sh_degree = max_sh_degree;
     p.world = world_of(splats_world);
+    if (quant) {
+        p.sh_state_packed = (uint16_t*)std::get<0>(*sh_packed);
+        p.sh_state_bounds = (float*)std::get<0>(*sh_quant_bounds);
+        p.sh_value_packed = (uint16_t*)std::get<0>(*sh_value_packed);
+        p.sh_value_bounds = (float*)std::get<0>(*sh_value_bounds);
+        p.num_sh_buffer = (uint32_t)(splats_world[5].channels() / 3);   // the buffers' stride, not the active degree
+    }
     p.camera = camera_of(camera_model, distortion, dist_coeffs, viewmats, intrins, image_width, image_height);
     p.aabb = aabb.data_ptr();
     p.v_screen = screen_of(v_splats_screen);

@@ -278,7 +278,8 @@ void engine_backward_with_variants(TorchTensorView v_render_rgb, TorchTensorView
 }
 
 void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
-                                     TorchTensorView v_render_Ts, const float hyper[14], int step, bool scale_agnostic_mean) {
+                                     TorchTensorView v_render_Ts, const float hyper[14], int step, bool scale_agnostic_mean,
+                                     int quantization_level) {
     auto& E = engine();
     if (std::get<0>(E.fwd.renders).data_ptr() == nullptr)
         throw std::runtime_error("engine_backward_fused_optimizer: forward_3dgs must be called first");
@@ -301,6 +302,24 @@ void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorVi
         E.optim.densify_score.resize(PoolSlot::EngDensifyScore, n);
         E.optim.adam_ready = true;
     }
+    std::optional<TorchTensorView> sh_state, sh_state_bounds, sh_values, sh_value_bounds;
+    if (quantization_level == 1) {
+        // OptimConfig::quantization_level 1: the SH values are the engine's 16-bit codes (set_sh_value_quant with one
+        // bound per 256 splats), updated in place; their moments live in two pool slots, all zeros at first
+        const int64_t R = 3 * (int64_t)E.num_sh, nb = (n + 255) / 256;
+        if (E.world.sh_value_bits != 16 || !E.world.sh_packed || E.world.sh_bounds_stride != 256 * R)
+            throw std::runtime_error("engine_backward_fused_optimizer: quantization level 1 needs 16-bit SH values with one bound per 256 splats");
+        uint8_t* st = DevicePool::global().acquire<uint8_t>(PoolSlot::AdamShStatePacked, (size_t)(n * R * 2));
+        float* sb = DevicePool::global().acquire<float>(PoolSlot::AdamShStateBounds, (size_t)(nb * 4));
+        if (!E.optim.sh_state_ready) {
+            backend::memset_async(st, 0, (size_t)(n * R * 2));
+            backend::memset_async(sb, 0, (size_t)(nb * 4) * sizeof(float));
+            E.optim.sh_state_ready = true;
+        }
+        sh_state = TorchTensorView{(uint64_t)(uintptr_t)st, 1u, std::vector<int64_t>{n * R * 2}};
+        sh_state_bounds = TorchTensorView{(uint64_t)(uintptr_t)sb, 4u, std::vector<int64_t>{nb, 4}};
+        sh_values = E.world.sh_packed; sh_value_bounds = E.world.sh_bounds;
+    }
     E.grad.v_screen = raster_backward(v_render_rgb, v_render_depth, v_render_Ts);
     const int64_t W = E.camera.width, H = E.camera.height;
     DeviceVector<int32_t> cam_ids, gauss_ids;
@@ -316,9 +335,9 @@ void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorVi
     fused_projection_bwd_optimizer_3dgs(
         E.cur_num_splats, E.sh_degree, E.fwd.splats_w, E.camera.viewmats, E.camera.intrins, (uint32_t)W, (uint32_t)H,
         E.camera.model_str, E.camera.distortion_str, E.camera.dist_coeffs, cam_ids, gauss_ids, aabb, {}, E.grad.v_screen,
-        E.optim.g1, E.optim.g2, std::nullopt, std::nullopt, E.world.sh_packed, E.world.sh_bounds, NonShQuantState{},
+        E.optim.g1, E.optim.g2, sh_state, sh_state_bounds, sh_values, sh_value_bounds, NonShQuantState{},
         E.optim.radii, E.optim.densify_score, hyper[0], hyper[1], hyper[2], hyper[3], hyper[4], hyper[5], hyper[6], hyper[7],
-        hyper[8], hyper[9], hyper[12], hyper[13], hyper[10], hyper[11], scale_agnostic_mean, false, 0.0f, (int32_t)step, 0);
+        hyper[8], hyper[9], hyper[12], hyper[13], hyper[10], hyper[11], scale_agnostic_mean, false, 0.0f, (int32_t)step, quantization_level);
 }
 
 void engine_copy_params_to_host(TorchTensorView means, TorchTensorView quats, TorchTensorView scales,
@@ -420,6 +439,24 @@ int ssrh_set_camera_params(int width, int height, const char* model, const char*
     });
 }
 
+// Quantization level 1: copies the SH state to the host (any pointer may be NULL): moments [N * 3 * num_sh] uint16
+// cells and float4 bounds per 256 splats, values [N * 3 * num_sh] uint16 codes and float2 bounds per 256 splats.
+int ssrh_copy_sh_quant_state(uint16_t* state_packed, float* state_bounds, uint16_t* value_packed, float* value_bounds) {
+    return guard([&] {
+        auto& E = engine();
+        const int64_t n = E.max_num_splats, R = 3 * (int64_t)E.num_sh, nb = (n + 255) / 256;
+        auto get = [](void* dst, const void* src, size_t bytes) {
+            if (dst && src && bytes) backend::memcpy_sync(dst, src, bytes, backend::MemcpyKind::DeviceToHost);
+        };
+        if (E.optim.sh_state_ready) {
+            get(state_packed, DevicePool::global().acquire<uint8_t>(PoolSlot::AdamShStatePacked, (size_t)(n * R * 2)), (size_t)(n * R * 2));
+            get(state_bounds, DevicePool::global().acquire<float>(PoolSlot::AdamShStateBounds, (size_t)(nb * 4)), (size_t)(nb * 4) * sizeof(float));
+        }
+        if (E.world.sh_packed) get(value_packed, (const void*)std::get<0>(*E.world.sh_packed), (size_t)(n * R * 2));
+        if (E.world.sh_bounds) get(value_bounds, (const void*)std::get<0>(*E.world.sh_bounds), (size_t)(nb * 2) * sizeof(float));
+    });
+}
+
 int ssrh_set_tile_mask(const uint8_t* mask, int h_mask, int w_mask) {
     return guard([&] { engine_set_tile_mask(tv(mask, 1, {1, h_mask, w_mask})); });
 }
@@ -446,11 +483,11 @@ int ssrh_backward_with_variants(const float* v_rgb, const float* v_depth, const 
 }
 
 int ssrh_backward_fused_optimizer(const float* v_rgb, const float* v_depth, const float* v_Ts, const float* hyper14, int step,
-                                  int scale_agnostic_mean) {
+                                  int scale_agnostic_mean, int quantization_level) {
     return guard([&] {
         const int64_t C = engine().camera.num, H = engine().camera.height, W = engine().camera.width;
         engine_backward_fused_optimizer(tv(v_rgb, 4, {C, H, W, 3}), tv(v_depth, 4, {C, H, W, 1}), tv(v_Ts, 4, {C, H, W, 1}), hyper14, step,
-                                        scale_agnostic_mean != 0);
+                                        scale_agnostic_mean != 0, quantization_level);
     });
 }
 

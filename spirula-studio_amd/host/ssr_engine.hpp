@@ -35,6 +35,7 @@ struct EngineState {
     struct {
         DeviceVector<float> radii; bool skip_grad_zero = false;
         bool adam_ready = false;
+        bool sh_state_ready = false;   // quantization level 1: the 8-bit SH moments have been zeroed
         std::vector<DeviceTensorFloatND> g1, g2;   // Adam moments, shaped like the world tensors
         DeviceVector<float> densify_score;
     } optim;
@@ -84,9 +85,11 @@ void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorV
 // slots (zero on first use). hyper: lr_means, lr_quats, lr_scales, lr_opacs, lr_dc, lr_sh,
 // max_gauss_ratio, scale_reg_w, mcmc_opacity_w, mcmc_scale_w, quat_norm_w, sh_reg_w, erank_w, erank_w_s3.
 // scale_agnostic_mean: OptimConfig::use_scale_agnostic_mean (the means step on the forward's radii).
+// quantization_level 1: SH values stay the 16-bit codes of set_sh_value_quant (one bound per 256 splats) and are
+// updated in place, their moments are 8-bit cells in pool slots (OptimConfig::quantization_level).
 void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
                                      TorchTensorView v_render_Ts, const float hyper[14], int step,
-                                     bool scale_agnostic_mean = false);
+                                     bool scale_agnostic_mean = false, int quantization_level = 0);
 // engine_backward_from_render_grad with the cotangents of the variants of the forward that ran
 // (any may be a null view): distortion image, median depth, and a pixel weight map to accumulate
 // per splat (the reference feeds these from its loss, src/engine/EngineLoss.cpp:138-216).

@@ -92,7 +92,8 @@ class FpboParams(C.Structure):
                 ("mcmc_opacity_reg_weight", C.c_float), ("mcmc_scale_reg_weight", C.c_float),
                 ("quat_norm_reg_weight", C.c_float), ("sh_reg_weight", C.c_float),
                 ("step", C.c_int32), ("steps", vp), ("erank_reg_weight", C.c_float), ("erank_reg_weight_s3", C.c_float),
-                ("scale_agnostic_radii", vp), ("packed_row_of", vp)]
+                ("scale_agnostic_radii", vp), ("packed_row_of", vp), ("sh_state_packed", vp), ("sh_state_bounds", vp),
+                ("sh_value_packed", vp), ("sh_value_bounds", vp), ("num_sh_buffer", C.c_uint32)]
 
 
 # every symbol include/ssr_backend.h declares: (name, restype, argtypes)

@@ -326,13 +326,16 @@ class GpuRun:
             p.packed_gaussian_ids, p.num_packed = self.ptr("gaussian_ids"), self.rows
         self.check(self.lib.ssr_projection_bwd(C.byref(p), None))
 
-    def fused_optimizer(self, g1, g2, hyper, step=1, steps=None, v_in=None, scale_agnostic=False):
+    def fused_optimizer(self, g1, g2, hyper, step=1, steps=None, v_in=None, scale_agnostic=False, quant_state=None):
         """ssr_fused_projection_bwd_optimizer on the device copies of the parameters (fp32 SH);
         g1 / g2 are host dicts keyed like the world arrays. Returns (params, g1, g2, score) from the device."""
         D = self.L.DeviceArray
         keys = ["means", "quats", "log_scales", "opacity_logits", "features_dc", "features_sh"]
         for pre, src in (("m1_", g1), ("m2_", g2)):
             for k in keys:
+                if quant_state is not None and k == "features_sh":
+                    self.d[pre + k] = None
+                    continue
                 self.d[pre + k] = D.from_host(np.ascontiguousarray(src[k], np.float32))
         for k in keys:
             a = None if v_in is None else v_in.get(k)
@@ -358,10 +361,29 @@ class GpuRun:
             p.v_rows = self.ptr("v_rows")
         if scale_agnostic:
             p.scale_agnostic_radii = self.ptr("radii")
+        if quant_state is not None:
+            # the reference's quantization level 1: SH values are the scene's 16-bit codes (one (min, max) per 256
+            # splats, which the forward already read), their moments the 8-bit (u, log_s) cells given here
+            assert self.sc.sh_codec == 2 and self.sc.sh_bounds_stride == 256 * 45
+            self.d["sh_state_packed"] = D.from_host(np.ascontiguousarray(quant_state["state_packed"], np.uint16))
+            self.d["sh_state_bounds"] = D.from_host(np.ascontiguousarray(quant_state["state_bounds"], np.float32))
+            p.sh_state_packed, p.sh_state_bounds = self.ptr("sh_state_packed"), self.ptr("sh_state_bounds")
+            p.sh_value_packed, p.sh_value_bounds = self.ptr("sh_packed"), self.ptr("sh_bounds")
+            p.num_sh_buffer = 15
+            w = p.world
+            w.features_sh = None
+            p.world = w
         self.check(self.lib.ssr_fused_projection_bwd_optimizer(C.byref(p), None))
         self.check(self.lib.ssr_device_synchronize())
+        if quant_state is not None:
+            keys = keys[:5]
         out = lambda pre: {k: self.host(pre + k) for k in keys}
-        return out(""), out("m1_"), out("m2_"), self.host("score")
+        res = out(""), out("m1_"), out("m2_"), self.host("score")
+        if quant_state is not None:
+            q = dict(state_packed=self.host("sh_state_packed"), state_bounds=self.host("sh_state_bounds"),
+                     value_packed=self.host("sh_packed").view(np.uint16), value_bounds=self.host("sh_bounds"), num_sh_buffer=15)
+            return res + (q,)
+        return res
 
     def run_all(self, backward=True, fused_count=False):
         self.projection_fwd(fused_count)

@@ -261,6 +261,94 @@ def fused_projection_bwd_optimizer(scene, aabb, vs, params, g1, g2, hyper, step=
     return score
 
 
+class OrShQuantState(C.Structure):
+    _fields_ = [("state_packed", C.c_void_p), ("state_bounds", C.c_void_p), ("value_packed", C.c_void_p),
+                ("value_bounds", C.c_void_p), ("num_sh_buffer", C.c_uint32)]
+
+
+def quant_codec(op, a=None, b=None, mm=None, codes=None):
+    """The codecs of the quantized optimizer state on arrays: op 0 Adam-state encode (g1, g2 -> codes),
+    1 decode (codes -> g1, g2), 2 16-bit value encode, 3 value decode."""
+    mm = np.ascontiguousarray(mm, np.float32)
+    if op in (0, 2):
+        a = np.ascontiguousarray(a, np.float32)
+        b = np.ascontiguousarray(a if b is None else b, np.float32)
+        codes = np.zeros(a.size, np.uint32)
+        lib().or_quant_codec(C.c_int(op), C.c_int64(a.size), _p(a), _p(b), _p(mm), _p(codes))
+        return codes
+    codes = np.ascontiguousarray(codes, np.uint32)
+    a = np.zeros(codes.size, np.float32)
+    b = np.zeros(codes.size, np.float32)
+    lib().or_quant_codec(C.c_int(op), C.c_int64(codes.size), _p(a), _p(b), _p(mm), _p(codes))
+    return (a, b) if op == 1 else a
+
+
+def quantize_sh_state(features_sh, num_sh_buffer=15):
+    """fp32 SH [N, num_sh_buffer, 3] -> the level-1 state: 16-bit values against per-256-splat (min, max),
+    all-zero moments (packed zeros with zero bounds decode to g1 = g2 = 0)."""
+    n = features_sh.shape[0]
+    R = 3 * num_sh_buffer
+    flat = np.ascontiguousarray(features_sh, np.float32).reshape(n, R)
+    nb = (n + 255) // 256
+    vb = np.zeros((nb, 2), np.float32)
+    vp = np.zeros(n * R, np.uint16)
+    for blk in range(nb):
+        rows = flat[blk * 256:(blk + 1) * 256]
+        vb[blk] = [rows.min(), rows.max()]
+        vp[blk * 256 * R: blk * 256 * R + rows.size] = quant_codec(2, rows.reshape(-1), mm=vb[blk]).astype(np.uint16)
+    return dict(state_packed=np.zeros(n * R, np.uint16), state_bounds=np.zeros((nb, 4), np.float32), value_packed=vp,
+                value_bounds=vb, num_sh_buffer=num_sh_buffer)
+
+
+def decode_sh_values(q, n):
+    R = 3 * q["num_sh_buffer"]
+    out = np.zeros((n, R), np.float32)
+    for blk in range((n + 255) // 256):
+        c = q["value_packed"][blk * 256 * R: min((blk + 1) * 256, n) * R]
+        out[blk * 256: blk * 256 + c.size // R] = quant_codec(3, codes=c.astype(np.uint32), mm=q["value_bounds"][blk]).reshape(-1, R)
+    return out.reshape(n, q["num_sh_buffer"], 3)
+
+
+def decode_sh_moments(q, n):
+    R = 3 * q["num_sh_buffer"]
+    g1, g2 = np.zeros((n, R), np.float32), np.zeros((n, R), np.float32)
+    for blk in range((n + 255) // 256):
+        c = q["state_packed"][blk * 256 * R: min((blk + 1) * 256, n) * R]
+        a, b = quant_codec(1, codes=c.astype(np.uint32), mm=q["state_bounds"][blk])
+        g1[blk * 256: blk * 256 + c.size // R] = a.reshape(-1, R)
+        g2[blk * 256: blk * 256 + c.size // R] = b.reshape(-1, R)
+    return g1, g2
+
+
+def fused_projection_bwd_optimizer_q(scene, aabb, vs, params, q, g1, g2, hyper, step=1, steps=None, v_in=None,
+                                     sh_degree=3, densify=True, radii=None):
+    """The fused optimizer with the SH coefficients and their moments in the quantized state q (updated in
+    place); params / g1 / g2 hold the five non-SH arrays (a features_sh entry is ignored)."""
+    n = scene.n
+    cam = camera_of(scene)
+
+    def ptrs(d):
+        arr = (C.c_void_p * 6)()
+        for i, k in enumerate(WORLD_KEYS):
+            a = None if d is None or k == "features_sh" else d.get(k)
+            arr[i] = None if a is None else a.ctypes.data
+        return arr
+    hv = np.array([hyper.get(k, 0.0) for k in HYPER], np.float32)
+    score = np.zeros(n, np.float32) if densify else None
+    st = OrShQuantState()
+    for k in ["state_packed", "state_bounds", "value_packed", "value_bounds"]:
+        assert q[k].flags.c_contiguous
+        setattr(st, k, q[k].ctypes.data)
+    st.num_sh_buffer = q["num_sh_buffer"]
+    lib().or_fused_projection_bwd_optimizer_q(
+        C.c_int64(n), C.c_int(sh_degree), *[_p(params[k]) for k in WORLD_KEYS[:5]], C.byref(st), C.byref(cam), _p(aabb),
+        _p(vs["v_xy"]), _p(vs["v_depth"]), _p(vs["v_conic"]), _p(vs["v_opac"]), _p(vs["v_rgb"]),
+        ptrs(v_in) if v_in is not None else None, ptrs(g1), ptrs(g2), _p(score), _p(hv), C.c_int32(step),
+        _p(None if steps is None else np.ascontiguousarray(steps, np.int32)),
+        _p(None if radii is None else np.ascontiguousarray(radii, np.float32)))
+    return score
+
+
 def erank_reg(log_scales, w, w3):
     """Loss and gradient of the effective-rank regularizer for one splat."""
     ls = np.ascontiguousarray(log_scales, np.float32)

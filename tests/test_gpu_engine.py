@@ -231,6 +231,68 @@ def test_engine_fused_optimizer_scale_agnostic_means(pkg, oracle, H, packed):
         assert (d > 0.05 * 5e-2).mean() < 2e-3, k
 
 
+@pytest.mark.parametrize("packed", [False, True])
+def test_engine_fused_optimizer_quantization_level_1(pkg, oracle, H, packed):
+    """Training steps at OptimConfig::quantization_level 1 (the reference's default): the engine keeps the SH
+    coefficients as 16-bit codes that the forward reads and the fused optimizer rewrites in place, and their Adam
+    moments as 8-bit cells; against the oracle running the same loop on its own copy."""
+    host, lib = H
+    S = pkg.scenes
+    sc = S.make_scene(1, n=20000, width=320, height=240, parity_variant=True, sh_codec=0)
+    if packed:
+        sc.means[::3, 2] = -10.0
+    S.apply_sh_codec(sc, 2, bounds_stride=256 * 45)
+    h = dict(lr_means=1.6e-4, lr_quats=1e-3, lr_scales=5e-3, lr_opacs=5e-2, lr_features_dc=2.5e-3, lr_features_sh=2.5e-3,
+             max_gauss_ratio=6.0, scale_regularization_weight=0.01, mcmc_opacity_reg_weight=0.01, mcmc_scale_reg_weight=0.01,
+             quat_norm_reg_weight=0.02, sh_reg_weight=0.05)
+    n, R = sc.n, 45
+    nb = (n + 255) // 256
+    eng = host.Engine(sc, packed_projection=packed)
+    import copy
+    ref = copy.deepcopy(sc)        # keeps the 16-bit codec: the oracle's forward decodes ref.sh_packed / ref.sh_bounds
+    q = dict(state_packed=np.zeros(n * R, np.uint16), state_bounds=np.zeros((nb, 4), np.float32),
+             value_packed=np.ascontiguousarray(sc.sh_packed).view(np.uint16).copy(),
+             value_bounds=np.ascontiguousarray(sc.sh_bounds, np.float32).reshape(nb, 2).copy(), num_sh_buffer=15)
+    P = {k: np.ascontiguousarray(getattr(sc, k), np.float32).copy() for k in oracle.WORLD_KEYS[:5]}
+    g1 = {k: np.zeros_like(v) for k, v in P.items()}
+    g2 = {k: np.zeros_like(v) for k, v in P.items()}
+    start = oracle.decode_sh_values(q, n)
+    for step in (1, 2, 3):
+        eng.forward()
+        eng.backward_fused_optimizer(h, step, quantization_level=1)
+        for k in P:
+            setattr(ref, k, P[k])
+        ref.sh_packed, ref.sh_bounds = q["value_packed"].copy(), q["value_bounds"].copy()
+        r = oracle.pipeline(ref, backward=True)
+        oracle.fused_projection_bwd_optimizer_q(ref, r["proj"]["aabb"], r["vscreen"], P, q, g1, g2, h, step=step)
+        eq = eng.sh_quant_state()
+        got, want = oracle.decode_sh_values(eq, n), oracle.decode_sh_values(q, n)
+        far = np.abs(got - want) > 0.05 * h["lr_features_sh"] + 1e-6
+        assert far.mean() < 5e-3, (step, float(far.mean()))
+        assert np.abs(got - want).max() <= 2.5 * step * h["lr_features_sh"] + 1e-5
+        assert np.allclose(eq["value_bounds"], q["value_bounds"], atol=2.5 * step * h["lr_features_sh"])
+        m1, m2 = oracle.decode_sh_moments(eq, n)
+        w1, w2 = oracle.decode_sh_moments(q, n)
+        assert np.isfinite(m1).all() and np.isfinite(m2).all()
+        scale = np.abs(w1).max(axis=1, keepdims=True) + 1e-12
+        assert ((np.abs(m1 - w1) > 0.05 * scale + 1e-9).mean()) < 0.02, step
+    assert np.abs(want - start).max() > 2 * h["lr_features_sh"]          # the coefficients moved, step after step
+    eng.forward()                                                      # and the forward renders the updated codes
+    for k in P:
+        setattr(ref, k, P[k])
+    ref.sh_packed, ref.sh_bounds = q["value_packed"].copy(), q["value_bounds"].copy()
+    r = oracle.pipeline(ref, backward=False)
+    rgb, depth, T = eng.render()
+    assert np.abs(rgb - r["fwd"]["rgb"]).max() < 0.05      # three sign-sensitive first Adam steps apart
+    # exactly what the engine now holds, rendered by the oracle: the forward reads the rewritten codes and bounds
+    got_p, got_q = eng.params(), eng.sh_quant_state()
+    for k in P:
+        setattr(ref, k, got_p[k])
+    ref.sh_packed, ref.sh_bounds = got_q["value_packed"], got_q["value_bounds"]
+    r = oracle.pipeline(ref, backward=False)
+    assert np.abs(rgb - r["fwd"]["rgb"]).max() < 1e-4
+
+
 def test_engine_packed_fused_optimizer_with_nothing_visible(pkg, oracle, H):
     """No packed rows at all: no projection gradient, but every splat still decays its moments and takes
     the regularizer step (the reference's kernel runs over all N splats whatever is visible)."""

@@ -436,6 +436,82 @@ def test_fused_projection_bwd_optimizer(gpu, oracle, cfg):
         assert np.array_equal(g.host("row_of"), row_of)
 
 
+@pytest.mark.parametrize("cfg", ["tiny", "tiny-deg1-packed-steps", "cfg3"])
+def test_fused_optimizer_quantized_sh_state(gpu, oracle, cfg):
+    """The fused optimizer at the reference's quantization level 1: SH values as 16-bit codes and their Adam
+    moments as 8-bit (u, log_s) cells, both against per-256-splat bounds that are recomputed every step
+    (FusedProjectionBwdOptim_kernel.cuh:709-1030). Two consecutive steps against the oracle, both sides fed the
+    device's screen gradients; the second step starts from non-zero moments. Codes may differ by one where the
+    two sides' gradients differ in the last bit."""
+    rng = np.random.default_rng(17)
+    S = gpu.scenes
+    deg, packed = 3, False
+    if cfg == "tiny":
+        sc = S.tiny_scene(n=700, width=96, height=64, seed=83)        # two full blocks and a partial one
+        sc.means[::4, 2] = -10.0
+    elif cfg == "tiny-deg1-packed-steps":
+        sc = S.tiny_scene(n=1100, width=96, height=64, seed=84)
+        sc.means[::3, 2] = -10.0
+        deg, packed = 1, True                                          # coefficients above degree 1 are re-encoded as zeros
+    else:
+        sc = S.make_scene(3, n=30000, width=320, height=192, sh_codec=0)
+    S.apply_sh_codec(sc, 2, bounds_stride=256 * 45)
+    h = dict(lr_means=1.6e-4, lr_quats=1e-3, lr_scales=5e-3, lr_opacs=5e-2, lr_features_dc=2.5e-3, lr_features_sh=2.5e-3,
+             max_gauss_ratio=6.0, scale_regularization_weight=0.01, mcmc_opacity_reg_weight=0.01, mcmc_scale_reg_weight=0.01,
+             quat_norm_reg_weight=0.02, sh_reg_weight=0.05)
+    n, R = sc.n, 45
+    nb = (n + 255) // 256
+    steps = rng.integers(1, 60, n).astype(np.int32) if "steps" in cfg else None
+    q = dict(state_packed=np.zeros(n * R, np.uint16), state_bounds=np.zeros((nb, 4), np.float32),
+             value_packed=np.ascontiguousarray(sc.sh_packed).view(np.uint16).copy(),
+             value_bounds=np.ascontiguousarray(sc.sh_bounds, np.float32).reshape(nb, 2).copy(), num_sh_buffer=15)
+    P = {k: np.ascontiguousarray(getattr(sc, k), np.float32).copy() for k in oracle.WORLD_KEYS[:5]}
+    g1 = {k: np.zeros_like(v) for k, v in P.items()}
+    g2 = {k: np.zeros_like(v) for k, v in P.items()}
+    for t in (1, 2):
+        # the scene both sides start this step from
+        for k in P:
+            setattr(sc, k, P[k].copy())
+        sc.sh_packed, sc.sh_bounds = q["value_packed"].copy(), q["value_bounds"].copy()
+        g = GpuRun(gpu, sc, sh_degree=deg, packed_projection=packed)
+        g.projection_fwd(); g.tiles(); g.raster_fwd(); g.raster_bwd()
+        vs = {k: g.host(k) for k in ["v_xy", "v_depth", "v_conic", "v_opac", "v_rgb"]}
+        aabb = g.host("aabb")
+        if packed:
+            ids = g.host("gaussian_ids")[:g.rows]
+            full = np.zeros((n, 4), np.float32); full[ids] = aabb[:g.rows]; aabb = full
+            for k in vs:
+                full = np.zeros((n,) + vs[k].shape[1:], np.float32); full[ids] = vs[k][:g.rows]; vs[k] = full
+        dP, d1, d2, dscore, dq = g.fused_optimizer(g1, g2, h, step=t, steps=steps, quant_state=q)
+        oq = {k: (v.copy() if isinstance(v, np.ndarray) else v) for k, v in q.items()}
+        oP = {k: v.copy() for k, v in P.items()}
+        o1 = {k: v.copy() for k, v in g1.items()}
+        o2 = {k: v.copy() for k, v in g2.items()}
+        oracle.fused_projection_bwd_optimizer_q(sc, aabb, vs, oP, oq, o1, o2, h, step=t, steps=steps, sh_degree=deg)
+        assert np.allclose(dq["value_bounds"], oq["value_bounds"], rtol=1e-5, atol=1e-8)
+        assert np.allclose(dq["state_bounds"], oq["state_bounds"], rtol=1e-4, atol=1e-6)
+        for key, width in [("value_packed", 16), ("state_packed", 8)]:
+            a, b = dq[key].astype(np.int64), oq[key].astype(np.int64)
+            if width == 16:
+                d = np.abs(a - b)
+                assert d.max() <= 2 and (d > 0).mean() < 0.02, (key, int(d.max()), float((d > 0).mean()))
+            else:
+                du, ds = np.abs((a & 255) - (b & 255)), np.abs((a >> 8) - (b >> 8))
+                assert max(du.max(), ds.max()) <= 1 and max((du > 0).mean(), (ds > 0).mean()) < 0.01, (key, t)
+        for k in P:   # the non-SH parameters take the fp32 path
+            assert np.abs(dP[k].astype(np.float64) - oP[k]).max() <= 0.02 * 5e-2 * 40 + 1e-6, k
+        if deg < 3:   # coefficients above the active degree: zero values, zero moments
+            vals = oracle.decode_sh_values(dq, n).reshape(n, 15, 3)
+            m1, m2 = oracle.decode_sh_moments(dq, n)
+            step = (dq["value_bounds"][:, 1] - dq["value_bounds"][:, 0]).max() / 65535
+            assert np.abs(vals[:, deg * (deg + 2):]).max() <= step
+            assert not np.any(m2.reshape(n, 15, 3)[:, deg * (deg + 2):])
+        # carry the DEVICE's state into the next step
+        P, g1, g2, q = dP, d1, d2, dq
+    vals0 = oracle.decode_sh_values(dict(q, value_packed=np.ascontiguousarray(sc.sh_packed).view(np.uint16), value_bounds=sc.sh_bounds), n)
+    assert np.abs(oracle.decode_sh_values(q, n) - vals0).max() > 1e-4    # the coefficients did move
+
+
 def _variant_cotangents(sc, seed=1):
     rng = np.random.default_rng(seed)
     h, w = sc.height, sc.width
