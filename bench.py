@@ -105,6 +105,10 @@ def main():
     ap.add_argument("--fused-optimizer", action="store_true",
                     help="backward = compositing backward + projection backward fused with the Adam step "
                          "(the reference's FPBO mode); K9 then includes the optimizer's 1.4 kB/splat of traffic")
+    ap.add_argument("--quantization-level", type=int, default=0, choices=[0, 1],
+                    help="with --fused-optimizer: 1 = SH values as 16-bit codes and their Adam moments as 8-bit cells "
+                         "(the reference's default level); the scene's SH is then stored at 16 bits, one bound per 256 splats")
+    ap.add_argument("--scale-agnostic-mean", action="store_true", help="with --fused-optimizer: the scale-agnostic step of the means")
     ap.add_argument("--dist-type", type=int, default=0, help="compositing variant: 1 depth distortion, 2 rgb + depth distortion")
     ap.add_argument("--median", action="store_true", help="compositing variant: also render the median depth and back-propagate it")
     ap.add_argument("--accum-mode", type=int, default=0, help="compositing variant: accumulate a pixel weight map per splat (1 max, 2 sum, 3 avg)")
@@ -136,6 +140,10 @@ def main():
     cfg = args.config
     t_gen = time.time()
     sc = pkg.scenes.make_scene(cfg, n=args.n)
+    if args.fused_optimizer and args.quantization_level == 1:
+        if sc.sh_codec != 0:
+            sc = pkg.scenes.make_scene(cfg, n=args.n, sh_codec=0)
+        pkg.scenes.apply_sh_codec(sc, 2, bounds_stride=256 * 45)
     if args.fisheye:
         sc.camera_model = pkg.scenes.CAM_FISHEYE
         f = sc.width / math.pi
@@ -167,7 +175,8 @@ def main():
                                                          vcot["amap"].ptr if args.accum_mode else None, args.accum_mode))
         elif args.fused_optimizer:
             adam_step[0] += 1
-            eng.backward_fused_optimizer(hyper, adam_step[0])
+            eng.backward_fused_optimizer(hyper, adam_step[0], scale_agnostic_mean=args.scale_agnostic_mean,
+                                         quantization_level=args.quantization_level)
         else:
             eng.backward()
 
@@ -242,7 +251,8 @@ def main():
                    "stage_order": ("fused tile count, visible-splat work list, packed fragment rows, packed gradient rows, plain-store gradients"
                                    + (", tile-segmented sort" if tile_sort else "") if native else "reference order")
                                   + (", packed projection outputs" if args.packed_projection else "")
-                                  + (", projection backward fused with Adam" if args.fused_optimizer else "")
+                                  + (", projection backward fused with Adam" + (" (quantized SH state)" if args.quantization_level else "")
+                                     if args.fused_optimizer else "")
                                   + (f", compositing variants dist_type={args.dist_type} median={int(args.median)} accum_mode={args.accum_mode}" if variants else ""),
                    "device_ms_per_iter_median": float(np.median(ms))},
         "hbm_roofline_frac_whole_iteration": total_bytes / (float(np.median(ms)) * 1e-3) / 1e9 / HBM_PEAK_GBS,

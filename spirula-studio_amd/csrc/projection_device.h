@@ -249,7 +249,48 @@ __device__ __forceinline__ void decode_sh(const ssr_world& w, const ssr_sh_quant
                                                    : (int64_t)256 * 3 * (int64_t)q.num_sh_buffer;
         const bool q16 = q.codec == SSR_SH_REF_Q16;
         const float inv = q16 ? (1.0f / 65535.0f) : (1.0f / 255.0f);
-        // bounds change at most once every `stride` cells: track the current block incrementally
+        // one bound per 256 splats is the layout the optimizer keeps: the splat's cells then share a block,
+        // and the block is gid / 256 (no 64-bit division, no per-cell test)
+        if (stride == (int64_t)256 * 3 * (int64_t)q.num_sh_buffer) {
+            const int64_t blk = gid >> 8;
+            const float lo = q.bounds[2 * blk], hi = q.bounds[2 * blk + 1];
+            if (q16 && n > 1 && (reinterpret_cast<uintptr_t>(q.packed) & 3) == 0) {
+                // 16-bit codes through aligned 32-bit loads (half as many memory instructions): the splat's first
+                // code sits in the low or the high half of its first word, by the parity of `base`
+                const uint16_t* p16 = reinterpret_cast<const uint16_t*>(q.packed) + base;
+                const bool odd = (base & 1) != 0;
+                const uint32_t* p32 = reinterpret_cast<const uint32_t*>(p16 - (odd ? 1 : 0));
+                constexpr int kWords = (n + 1) / 2 + ((n & 1) ? 0 : 1);   // words touched when the run starts in a high half
+                uint32_t w[kWords];
+#pragma unroll
+                for (int k = 0; k < kWords - 1; k++) w[k] = p32[k];
+                // the last word is only partly this splat's: take it whole when the run reaches into its high half,
+                // else just the one code (the bytes after it may lie beyond the array)
+                {
+                    constexpr int kLast = kWords - 1;
+                    // odd start: the run is halves 1..n of these words; even start: halves 0..n-1
+                    const bool need = odd ? (2 * kLast <= n) : (2 * kLast <= n - 1);
+                    const bool whole = odd ? (2 * kLast + 1 <= n) : (2 * kLast + 1 <= n - 1);
+                    w[kLast] = 0u;
+                    if (need) w[kLast] = whole ? p32[kLast] : (uint32_t)reinterpret_cast<const uint16_t*>(p32)[2 * kLast];
+                }
+#pragma unroll
+                for (int i = 0; i < n; i++) {
+                    const uint32_t even_code = (w[i >> 1] >> (16 * (i & 1))) & 0xffffu;
+                    const uint32_t odd_code = (w[(i + 1) >> 1] >> (16 * ((i + 1) & 1))) & 0xffffu;
+                    out[i] = lo + (hi - lo) * ((float)(odd ? odd_code : even_code) * inv);
+                }
+                return;
+            }
+#pragma unroll
+            for (int i = 0; i < n; i++) {
+                const float v = q16 ? (float)reinterpret_cast<const uint16_t*>(q.packed)[base + i]
+                                    : (float)reinterpret_cast<const uint8_t*>(q.packed)[base + i];
+                out[i] = lo + (hi - lo) * (v * inv);
+            }
+            return;
+        }
+        // otherwise bounds change at most once every `stride` cells: track the current block incrementally
         int64_t blk = base / stride;
         int64_t next = (blk + 1) * stride;
         float lo = q.bounds[2 * blk], hi = q.bounds[2 * blk + 1];
