@@ -48,14 +48,21 @@ SSR_HD uint32_t ssr_adamq_encode(float g1, float g2, const float mm[4]) {
     const float sq = ssr_min(ssr_max(ssr_round_code((255.0f * (ls - mm[2])) / sr), 0.0f), 255.0f);
     return (uint32_t)uq | ((uint32_t)sq << 8);
 }
-// decode_g1g2
-SSR_HD void ssr_adamq_decode(uint32_t code, const float mm[4], float* g1, float* g2) {
+// decode_g1g2, in two steps: sqrt(g2) depends on the 8-bit log_s code alone, so a kernel can tabulate it per
+// block (256 entries) instead of evaluating expm1 per cell
+SSR_HD float ssr_adamq_decode_sqrt_g2(uint32_t s_code, const float mm[4]) {
+    const float kInv = 1.0f / 255.0f;
+    const float ls = mm[2] + (mm[3] - mm[2]) * ((float)s_code * kInv);
+    return SSR_ADAMQ_EPS * ssr_expm1(ls);
+}
+SSR_HD void ssr_adamq_decode_with(uint32_t code, const float mm[4], float sq, float* g1, float* g2) {
     const float kInv = 1.0f / 255.0f;
     const float u = mm[0] + (mm[1] - mm[0]) * ((float)(code & 255u) * kInv);
-    const float ls = mm[2] + (mm[3] - mm[2]) * ((float)((code >> 8) & 255u) * kInv);
-    const float sq = SSR_ADAMQ_EPS * ssr_expm1(ls);
     *g1 = u * (sq + SSR_ADAMQ_EPS);
     *g2 = sq * sq;
+}
+SSR_HD void ssr_adamq_decode(uint32_t code, const float mm[4], float* g1, float* g2) {
+    ssr_adamq_decode_with(code, mm, ssr_adamq_decode_sqrt_g2((code >> 8) & 255u, mm), g1, g2);
 }
 
 // QuantizedTensor<16>::encode_v_code / decode_v against bounds (lo, hi)

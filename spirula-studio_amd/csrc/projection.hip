@@ -644,6 +644,7 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
     __shared__ float s_vc[kProjBlock][3];
     __shared__ float s_b1c[kProjBlock], s_b2c[kProjBlock];
     __shared__ float s_red[kProjBlock / 64][6];   // quantized state: per-wave min / max of the new bounds
+    __shared__ float s_sqrt_g2[kQuant ? 256 : 1];  // quantized state: sqrt(g2) of each 8-bit log_s code under the old bounds
     const int64_t block0 = (int64_t)blockIdx.x * kProjBlock;
     const int64_t g = block0 + threadIdx.x;
     const ssr_world& W = P.world;
@@ -796,6 +797,13 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
     }
     s_b1c[threadIdx.x] = ad.b1c; s_b2c[threadIdx.x] = ad.b2c;
     if (kCoef == 0) return;
+    float old_mm[4] = {0.f, 0.f, 0.f, 0.f};
+    if (kQuant) {
+        static_assert(!kQuant || kProjBlock == 256, "one table entry per thread");
+#pragma unroll
+        for (int k = 0; k < 4; k++) old_mm[k] = P.sh_state_bounds[4 * blockIdx.x + k];
+        s_sqrt_g2[threadIdx.x] = ssr_adamq_decode_sqrt_g2(threadIdx.x, old_mm);
+    }
     __syncthreads();
     // phase 2: SH coefficients of the workgroup's splats in memory order (FusedProjectionBwdOptim_kernel.cuh:667-710)
     const int64_t rest = P.num_splats - block0;
@@ -811,13 +819,11 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
         const int R = 3 * (int)P.num_sh_buffer;                    // cells per splat
         const int64_t cell0 = block0 * R;
         const int n_cells = n_here * R;
-        float old_mm[4];
-#pragma unroll
-        for (int k = 0; k < 4; k++) old_mm[k] = P.sh_state_bounds[4 * blockIdx.x + k];
         const float old_lo = P.sh_value_bounds[2 * blockIdx.x], old_hi = P.sh_value_bounds[2 * blockIdx.x + 1];
         auto step_cell = [&](int sp, int k, float& m1, float& m2, float& xn) {
             const int64_t cell = cell0 + (int64_t)sp * R + k;
-            ssr_adamq_decode(P.sh_state_packed[cell], old_mm, &m1, &m2);
+            const uint32_t code = P.sh_state_packed[cell];
+            ssr_adamq_decode_with(code, old_mm, s_sqrt_g2[code >> 8], &m1, &m2);
             const float x = ssr_q16_decode(P.sh_value_packed[cell], old_lo, old_hi);
             const int j = k / 3, c = k - 3 * j;
             const float v = s_Y[sp][j] * s_vc[sp][c] + sh_reg * x;
