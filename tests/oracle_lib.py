@@ -44,7 +44,10 @@ def lib():
 
 
 def _p(a):
-    return None if a is None else a.ctypes.data_as(C.c_void_p)
+    if a is None:
+        return None
+    assert a.flags["C_CONTIGUOUS"], "the oracle reads raw row-major buffers"
+    return a.ctypes.data_as(C.c_void_p)
 
 
 def camera_of(scene) -> OrCamera:
@@ -399,7 +402,7 @@ def pack_projection(p):
     return q
 
 
-def pipeline_packed(scene, sh_degree=3, backward=True, tile_active=None):
+def pipeline_packed(scene, sh_degree=3, backward=True, tile_active=None, variant=None):
     """The iteration with packed projection outputs (engine path with packed=true,
     src/engine/EngineForward.cpp:119-162,215-217): every later stage sees nnz rows, flatten ids are
     packed row numbers, v_screen has nnz rows, and the projection backward maps row i to splat
@@ -414,11 +417,15 @@ def pipeline_packed(scene, sh_degree=3, backward=True, tile_active=None):
     n_tiles = scene.tile_w * scene.tile_h
     sk, sv = sort_pairs(ids, flat, 0, 32 + tile_n_bits(n_tiles))
     offs = tile_offsets(sk, n_tiles)
-    f = raster_fwd(m, p, w, h, offs, sv)
+    va = variant or {}
+    f = raster_fwd(m, p, w, h, offs, sv, va.get("dist_type", 0), va.get("median", False))
     out = dict(proj=p, full_proj=full, counts=counts, cum=cum, isect_ids=ids, flatten_ids=flat, pads=pads,
                sorted_ids=sk, sorted_flat=sv, offsets=offs, fwd=f)
     if backward:
-        vs = raster_bwd(m, p, w, h, offs, sv, f, scene.v_rgb, scene.v_depth, scene.v_T)
+        vs = raster_bwd(m, p, w, h, offs, sv, f, scene.v_rgb, scene.v_depth, scene.v_T,
+                        dist_type=va.get("dist_type", 0), v_dist_rgb=va.get("v_dist_rgb"), v_dist_depth=va.get("v_dist_depth"),
+                        v_median=va.get("v_median") if va.get("median") else None, accum_mode=va.get("accum_mode", 0),
+                        accum_map=va.get("accum_map"), gaussian_ids=p["gaussian_ids"], n_world=n)
         out["vscreen"] = vs
         shapes = dict(v_xy=(n, 2), v_depth=(n,), v_conic=(n, 3), v_opac=(n,), v_rgb=(n, 3))
         spread = {}

@@ -117,13 +117,15 @@ def _compare(gpu, oracle, sc, label, fused_count=False, use_list=False, use_pack
     return g, r
 
 
-def _compare_packed(gpu, oracle, sc, label, fused_count=False, use_packed=False, read_nnz=True):
+def _compare_packed(gpu, oracle, sc, label, fused_count=False, use_packed=False, read_nnz=True, variant=None):
     """Packed projection outputs (nnz compacted rows) through every later stage."""
-    r = oracle.pipeline_packed(sc)
+    r = oracle.pipeline_packed(sc, variant=variant)
     q = r["proj"]
     m = q["visible"]
     print(f"[{label}] N={sc.n} {sc.width}x{sc.height} nnz={m} K={r['isect_ids'].size}", flush=True)
-    g = GpuRun(gpu, sc, use_packed=use_packed, packed_projection=True, read_nnz=read_nnz).run_all(fused_count=fused_count)
+    g = GpuRun(gpu, sc, use_packed=use_packed, packed_projection=True, read_nnz=read_nnz)
+    g.variant = variant or {}
+    g.run_all(fused_count=fused_count)
     assert g.nnz == m
     # K1 packed: ids exact and ascending, rows bit-exact, rows past nnz untouched
     assert np.array_equal(g.host("gaussian_ids")[:m], q["gaussian_ids"])
@@ -148,10 +150,21 @@ def _compare_packed(gpu, oracle, sc, label, fused_count=False, use_packed=False,
     dd = np.abs(g.host("r_depth") - f["depth"])
     assert (dd <= IMG_TOL * np.maximum(1.0, np.abs(f["depth"]))).all()
     assert np.array_equal(g.host("r_last"), f["last_ids"])
+    va = variant or {}
+    if va.get("dist_type"):
+        assert np.abs(g.host("r_dist_depth") - f["dist_depth"]).max() <= IMG_TOL
+        if va["dist_type"] == 2:
+            assert np.abs(g.host("r_dist_rgb") - f["dist_rgb"]).max() <= IMG_TOL
+    if va.get("median"):
+        assert (np.abs(g.host("r_median") - f["median"]) <= IMG_TOL * np.maximum(1.0, np.abs(f["median"]))).all()
     vs = r["vscreen"]
+    if va.get("accum_mode"):   # indexed by world splat through gaussian_ids
+        assert np.allclose(g.host("accum_weight"), vs["accum_weight"], rtol=1e-3, atol=1e-6)
     ab = vs["abs_terms"]
+    kw = dict(afrac=3e-5) if va.get("dist_type") else {}   # see _compare
+    assert not va.get("median"), "median rows: use _compare's tolerance handling"
     for k, cols in [("v_xy", slice(0, 2)), ("v_depth", 2), ("v_conic", slice(3, 6)), ("v_opac", 6), ("v_rgb", slice(7, 10))]:
-        _grad_close(g.host(k)[:m], vs[k], ab[:, cols], k)
+        _grad_close(g.host(k)[:m], vs[k], ab[:, cols], k, **kw)
     gr = r["grads"]
     vis = np.zeros(sc.n, bool)
     vis[q["gaussian_ids"]] = True

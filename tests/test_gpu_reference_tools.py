@@ -1,0 +1,240 @@
+"""The 3dgs rows of the reference's backend parity tools on their own inputs (src/backend/tests/render_parity.cpp,
+raster_bwd_parity.cpp, accum_weight_map.cpp), one camera of the tools' two-camera batch per run: the GPU path
+through the C ABI against the oracle, and accum_weight_map's own expectations on the GPU path."""
+import numpy as np
+import pytest
+
+import reference_tools as R
+from gpu_pipeline import GpuRun
+from test_gpu_parity import _compare, _compare_packed, gpu  # noqa: F401  (gpu: module fixture)
+
+pytestmark = pytest.mark.gpu
+
+PINHOLE, FISHEYE, EQUISOLID, EQUIRECT = 0, 1, 2, 3
+NONE, OPENCV, THIN_PRISM, RATIONAL = 0, 1, 2, 3
+
+
+# render_parity.cpp:186-196, rows with prim == 0: (packed, camera model, tier, dist_type, median)
+@pytest.mark.parametrize("packed,model,tier,dist_type,median", [(False, PINHOLE, OPENCV, 2, True), (False, FISHEYE, THIN_PRISM, 1, False),
+                                                              (True, EQUIRECT, NONE, 0, False)])
+@pytest.mark.parametrize("cam", [0, 1])
+def test_render_parity_rows(gpu, oracle, packed, model, tier, dist_type, median, cam):
+    sc, _ = R.tool_scene(gpu, R.SEED_RENDER, cam, model, tier)
+    z3, z1 = np.zeros((sc.height, sc.width, 3), np.float32), np.zeros((sc.height, sc.width), np.float32)
+    va = dict(dist_type=dist_type, median=median, v_dist_rgb=z3, v_dist_depth=z1, v_median=z1)
+    label = f"render_parity model {model} tier {tier} cam {cam}"
+    if packed:
+        _compare_packed(gpu, oracle, sc, label, fused_count=True, variant=va)
+    else:
+        _compare(gpu, oracle, sc, label, fused_count=True, use_list=True, use_packed=True, variant=va)
+
+
+# raster_bwd_parity.cpp:176-181, rows with prim == 0: (packed, camera model, tier, dist_type, median, accumulation mode)
+@pytest.mark.parametrize("packed,model,tier,dist_type,median,accum", [(False, PINHOLE, NONE, 0, False, 0), (False, PINHOLE, OPENCV, 2, True, 1),
+                                                                    (True, FISHEYE, THIN_PRISM, 1, False, 2),
+                                                                    (True, FISHEYE, THIN_PRISM, 1, False, 3)])
+@pytest.mark.parametrize("cam", [0, 1])
+def test_raster_bwd_parity_rows(gpu, oracle, packed, model, tier, dist_type, median, accum, cam):
+    _, rng = R.tool_world(R.SEED_RASTER_BWD)
+    ct = R.raster_bwd_cotangents(rng)
+    sc, _ = R.tool_scene(gpu, R.SEED_RASTER_BWD, cam, model, tier, cotangents=ct)
+    va = dict(dist_type=dist_type, median=median, accum_mode=accum, v_dist_rgb=ct["v_dist_rgb"][cam], v_dist_depth=ct["v_dist_depth"][cam],
+              v_median=ct["v_median"][cam], accum_map=ct["accum_map"][cam])
+    label = f"raster_bwd_parity model {model} tier {tier} dist {dist_type} accum {accum} cam {cam}"
+    if packed:
+        _compare_packed(gpu, oracle, sc, label, fused_count=True, use_packed=True, variant=va)
+    else:
+        _compare(gpu, oracle, sc, label, fused_count=True, use_list=True, use_packed=True, use_vrows=True, variant=va)
+
+
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("mode", [1, 2, 3])
+def test_accum_weight_map_reaches_the_right_splats(gpu, oracle, packed, mode):
+    """accum_weight_map.cpp run_mode(): known loss maps planted on the real forward chain, the per-splat score read back."""
+    centres = {}
+    runs = {}
+    for cam in (0, 1):
+        sc, _ = R.tool_scene(gpu, R.SEED_RASTER_BWD, cam)
+        g = GpuRun(gpu, sc, use_packed=True, packed_projection=packed)
+        g.projection_fwd(fused_count=True)
+        g.tiles(fused_count=True)
+        g.raster_fwd()
+        xy = np.full((sc.n, 2), -1e9, np.float32)
+        if packed:   # packed rows go back through gaussian_ids, the mapping under test
+            xy[g.host("gaussian_ids")[:g.nnz]] = g.host("xy")[:g.nnz]
+        else:
+            aabb = g.host("aabb")
+            vis = aabb[:, 2] > aabb[:, 0]
+            xy[vis] = g.host("xy")[vis]
+        centres[cam], runs[cam] = xy, g
+    for cam in (0, 1):
+        g, sc = runs[cam], runs[cam].sc
+
+        def run(amap):
+            g.variant = dict(accum_mode=mode, accum_map=amap)
+            g.raster_bwd()
+            return R.accum_finalize(g.host("accum_weight"), sc.n, mode)
+        R.accum_weight_map_checks(run, centres[cam], centres[1 - cam], mode, f"gpu {'packed' if packed else 'plain'} mode {mode} cam {cam}")
+
+
+# fpbo_parity.cpp:160-162, the two fp32-state 3dgs rows: PINHOLE without a lens and with the OpenCV tier, all five
+# non-SH world gradients present, densify score on, two consecutive steps (10, then 11)
+@pytest.mark.parametrize("row,tier", [(0, NONE), (1, OPENCV)])
+@pytest.mark.parametrize("cam", [0, 1])
+def test_fpbo_parity_rows(gpu, oracle, row, tier, cam):
+    sc, rng = R.tool_scene(gpu, R.SEED_FPBO, cam, PINHOLE, tier, n=R.N_FPBO)
+    for _ in range(row + 1):   # row 1 draws after row 0
+        vs2, v_world, g1, g2 = R.fpbo_row_inputs(rng)
+    vs = {k: np.ascontiguousarray(v[cam]) for k, v in vs2.items()}
+    g = GpuRun(gpu, sc)
+    g.projection_fwd()
+    D = gpu.lib.DeviceArray
+    for k, v in vs.items():
+        g.d[k] = D.from_host(v)
+    aabb = g.host("aabb")
+    assert 100 < (aabb[:, 2] > aabb[:, 0]).sum() < sc.n
+    P = {k: np.ascontiguousarray(getattr(sc, k), np.float32).copy() for k in oracle.WORLD_KEYS}
+    o1 = {k: v.copy() for k, v in g1.items()}
+    o2 = {k: v.copy() for k, v in g2.items()}
+    h = R.FPBO_HYPER
+    lrs = dict(means="lr_means", quats="lr_quats", log_scales="lr_scales", opacity_logits="lr_opacs",
+               features_dc="lr_features_dc", features_sh="lr_features_sh")
+    d1, d2 = g1, g2
+    for step in (10, 11):
+        dP, d1, d2, dscore = g.fused_optimizer(d1, d2, h, step=step, v_in=v_world)
+        score = oracle.fused_projection_bwd_optimizer(sc, aabb, vs, P, o1, o2, h, step=step, v_in=v_world)
+        for k in oracle.WORLD_KEYS:
+            a, b = d1[k].reshape(sc.n, -1).astype(np.float64), o1[k].reshape(sc.n, -1).astype(np.float64)
+            assert (np.abs(a - b) <= 1e-3 * np.abs(b) + 1e-4 * (np.abs(b).max(axis=1, keepdims=True) + 1e-12)).all(), ("g1", k, step)
+            a, b = d2[k].reshape(sc.n, -1).astype(np.float64), o2[k].reshape(sc.n, -1).astype(np.float64)
+            assert (np.abs(a - b) <= 2e-3 * np.abs(b) + 1e-12).all(), ("g2", k, step)
+            a, b = dP[k].astype(np.float64), P[k].astype(np.float64)
+            assert np.abs(a - b).max() <= 0.02 * h[lrs[k]] * 40 + 1e-6, (k, step, float(np.abs(a - b).max()))
+        assert np.allclose(dscore, score, rtol=1e-3, atol=1e-9)
+    assert np.abs(P["means"] - sc.means).max() > 1e-5   # two steps did move the splats
+
+
+# projection_parity.cpp:120-160 with prim == 0: every camera model at SH degree 0 without a lens and at degree 3 with
+# each of its compiled tiers
+@pytest.mark.parametrize("model", [PINHOLE, FISHEYE, EQUISOLID, EQUIRECT])
+@pytest.mark.parametrize("cam", [0, 1])
+def test_projection_parity_rows(gpu, oracle, model, cam):
+    for deg, tiers in [(0, [NONE]), (3, R.COMPILED_TIERS[model])]:
+        for tier in tiers:
+            sc, _ = R.tool_scene(gpu, R.SEED_PROJ, cam, model, tier)
+            want = oracle.projection_fwd(sc, deg)
+            g = GpuRun(gpu, sc, sh_degree=deg)
+            g.projection_fwd()
+            got = g.proj_host()
+            vis = want["aabb"][:, 2] > want["aabb"][:, 0]
+            print(f"[projection_parity model {model} tier {tier} degree {deg} cam {cam}] visible={int(vis.sum())}", flush=True)
+            assert 50 < vis.sum() < sc.n
+            for k in ["aabb", "sort_depth", "radii"]:
+                assert np.array_equal(got[k].view(np.uint32), want[k].view(np.uint32)), (k, tier, deg)
+            for k in ["xy", "depth", "conic", "opac", "rgb"]:
+                assert np.array_equal(got[k][vis].view(np.uint32), want[k][vis].view(np.uint32)), (k, tier, deg)
+
+
+# projection_parity.cpp:201-215 with prim == 0 (PINHOLE): 8- and 16-bit SH value codes, bounds per 256 cells and per
+# 256 splats, the tier rotating through the four configurations
+@pytest.mark.parametrize("cam", [0, 1])
+def test_projection_parity_quantized_rows(gpu, oracle, cam):
+    _, rng = R.tool_world(R.SEED_PROJ)
+    q = R.projection_quant_inputs(rng)
+    qcfg = 0
+    for bits in (8, 16):
+        for per_block in (0, 1):
+            tier = R.COMPILED_TIERS[PINHOLE][qcfg % 4]
+            qcfg += 1
+            sc, _ = R.tool_scene(gpu, R.SEED_PROJ, cam, PINHOLE, tier)
+            sc.sh_codec = 1 if bits == 8 else 2
+            sc.sh_packed = q["q8"] if bits == 8 else q["q16"]
+            sc.sh_bounds = q["bounds_block"] if per_block else q["bounds_cell"]
+            sc.sh_bounds_stride = 0 if per_block else 256      # 0: the fused optimizer's layout, as the tool passes it
+            want = oracle.projection_fwd(sc, 3)
+            g = GpuRun(gpu, sc)
+            g.projection_fwd()
+            got = g.proj_host()
+            vis = want["aabb"][:, 2] > want["aabb"][:, 0]
+            for k in ["aabb", "sort_depth", "radii"]:
+                assert np.array_equal(got[k].view(np.uint32), want[k].view(np.uint32)), (k, bits, per_block)
+            for k in ["xy", "depth", "conic", "opac", "rgb"]:
+                assert np.array_equal(got[k][vis].view(np.uint32), want[k][vis].view(np.uint32)), (k, bits, per_block)
+            # the colours do come from the codes: decode by the codec's definition and compare with an fp32 run
+            stride = 256 * 45 if per_block else 256
+            b = sc.sh_bounds[np.arange(sc.n * 45) // stride]
+            qmax = np.float32(255.0 if bits == 8 else 65535.0)
+            dec = (b[:, 0] + (b[:, 1] - b[:, 0]) * (sc.sh_packed.astype(np.float32) * (np.float32(1.0) / qmax))).astype(np.float32)
+            sc32, _ = R.tool_scene(gpu, R.SEED_PROJ, cam, PINHOLE, tier)
+            sc32.features_sh = dec.reshape(sc.n, 15, 3)
+            w32 = oracle.projection_fwd(sc32, 3)
+            assert np.array_equal(w32["rgb"][vis].view(np.uint32), want["rgb"][vis].view(np.uint32)), (bits, per_block)
+
+
+def _k9_direct(gpu, oracle, sc, vs, label, packed=False):
+    """ssr_projection_bwd fed given screen gradients (rows: splats, or packed rows), against the oracle."""
+    g = GpuRun(gpu, sc, packed_projection=packed)
+    g.projection_fwd()
+    D = gpu.lib.DeviceArray
+    aabb = g.host("aabb")
+    if packed:
+        ids = g.host("gaussian_ids")[:g.rows]
+        full_aabb = np.zeros((sc.n, 4), np.float32)
+        full_aabb[ids] = aabb[:g.rows]
+        full_vs = {}
+        for k, v in vs.items():
+            assert v.shape[0] == g.rows
+            full_vs[k] = np.zeros((sc.n,) + v.shape[1:], np.float32)
+            full_vs[k][ids] = v
+    else:
+        full_aabb, full_vs = aabb, vs
+    for k, v in vs.items():
+        g.d[k] = D.from_host(np.ascontiguousarray(v))
+    g.projection_bwd()
+    want = oracle.projection_bwd(sc, full_aabb, full_vs)
+    vis = full_aabb[:, 2] > full_aabb[:, 0]
+    print(f"[{label}] visible={int(vis.sum())}", flush=True)
+    assert 50 < vis.sum() < sc.n
+    for k, o in [("w_means", "v_means"), ("w_quats", "v_quats"), ("w_log_scales", "v_scales"),
+                 ("w_opacity_logits", "v_opacities"), ("w_features_dc", "v_dc"), ("w_features_sh", "v_sh")]:
+        got, ref = g.host(k).astype(np.float64).reshape(sc.n, -1), want[o].astype(np.float64).reshape(sc.n, -1)
+        scale = np.abs(ref).max(axis=1, keepdims=True) + 1e-30
+        floor = 2e-5 * (np.abs(ref).mean() + 1e-12)
+        assert (np.abs(got - ref) <= 2e-3 * scale + floor).all(), (k, float((np.abs(got - ref) / scale).max()))
+        assert not np.any(got[~vis]), k
+        # and inside the tool's own acceptance band (proj_bwd_parity.cpp:327)
+        assert (np.abs(got - ref) <= 5e-3 + 1e-3 * np.abs(ref)).all(), k
+
+
+# proj_bwd_parity.cpp:171-180, rows with prim == 0 (the camera-pose gradient some of them also ask for is not built
+# here): screen gradients drawn by the tool, not produced by the compositing backward
+@pytest.mark.parametrize("cam", [0, 1])
+def test_proj_bwd_parity_rows(gpu, oracle, cam):
+    n = R.N_TOOL
+    _, rng = R.tool_world(R.SEED_PROJ_BWD)
+    q = R.projection_quant_inputs(rng)          # the tool draws its codes and bounds before the rows (:126-142)
+    # rows 0 and 1: PINHOLE without a lens / with the OpenCV tier, C * N rows each, camera-major
+    for tier in (NONE, OPENCV):
+        vs2 = R.screen_gradients(rng, R.C_TOOL * n)
+        vs = {k: np.ascontiguousarray(v.reshape((R.C_TOOL, n) + v.shape[1:])[cam]) for k, v in vs2.items()}
+        sc, _ = R.tool_scene(gpu, R.SEED_PROJ_BWD, cam, PINHOLE, tier)
+        _k9_direct(gpu, oracle, sc, vs, f"proj_bwd_parity PINHOLE tier {tier} cam {cam}")
+    R.screen_gradients(rng, R.C_TOOL * n)        # row 2 (another primitive) draws the same amount
+    # row 3: packed, EQUISOLID + OpenCV; the tool's rows are camera 0's visible splats, then camera 1's
+    nnz = []
+    for c in range(R.C_TOOL):
+        sc_c, _ = R.tool_scene(gpu, R.SEED_PROJ_BWD, c, EQUISOLID, OPENCV)
+        a = oracle.projection_fwd(sc_c)["aabb"]
+        nnz.append(int(((a[:, 2] - a[:, 0] > np.float32(1e-3)) & (a[:, 3] - a[:, 1] > np.float32(1e-3))).sum()))
+    vs2 = R.screen_gradients(rng, sum(nnz))
+    lo = sum(nnz[:cam])
+    vs = {k: np.ascontiguousarray(v[lo:lo + nnz[cam]]) for k, v in vs2.items()}
+    sc, _ = R.tool_scene(gpu, R.SEED_PROJ_BWD, cam, EQUISOLID, OPENCV)
+    _k9_direct(gpu, oracle, sc, vs, f"proj_bwd_parity packed EQUISOLID OPENCV cam {cam}", packed=True)
+    # row 6: 8-bit SH codes, bounds per 256 cells, thin-prism lens (two rows of another primitive draw in between:
+    # the gradients here have the tool's ranges, not its exact stream)
+    vs2 = R.screen_gradients(rng, R.C_TOOL * n)
+    vs = {k: np.ascontiguousarray(v.reshape((R.C_TOOL, n) + v.shape[1:])[cam]) for k, v in vs2.items()}
+    sc, _ = R.tool_scene(gpu, R.SEED_PROJ_BWD, cam, PINHOLE, THIN_PRISM)
+    sc.sh_codec, sc.sh_packed, sc.sh_bounds, sc.sh_bounds_stride = 1, q["q8"], q["bounds_cell"], 256
+    _k9_direct(gpu, oracle, sc, vs, f"proj_bwd_parity q8 THIN_PRISM cam {cam}")
