@@ -110,6 +110,8 @@ def main():
                     help="with --fused-optimizer: 1 = SH values as 16-bit codes and their Adam moments as 8-bit cells "
                          "(the reference's default level); the scene's SH is then stored at 16 bits, one bound per 256 splats")
     ap.add_argument("--scale-agnostic-mean", action="store_true", help="with --fused-optimizer: the scale-agnostic step of the means")
+    ap.add_argument("--non-sh-optim-bits", type=int, default=32, choices=[32, 16],
+                    help="with --quantization-level 1: 16 = the moments of the non-SH tensors as 16-bit cells too (what the reference's trainer sets)")
     ap.add_argument("--dist-type", type=int, default=0, help="compositing variant: 1 depth distortion, 2 rgb + depth distortion")
     ap.add_argument("--median", action="store_true", help="compositing variant: also render the median depth and back-propagate it")
     ap.add_argument("--accum-mode", type=int, default=0, help="compositing variant: accumulate a pixel weight map per splat (1 max, 2 sum, 3 avg)")
@@ -177,7 +179,7 @@ def main():
         elif args.fused_optimizer:
             adam_step[0] += 1
             eng.backward_fused_optimizer(hyper, adam_step[0], scale_agnostic_mean=args.scale_agnostic_mean,
-                                         quantization_level=args.quantization_level)
+                                         quantization_level=args.quantization_level, non_sh_optim_bits=args.non_sh_optim_bits)
         else:
             eng.backward()
 
@@ -253,7 +255,7 @@ def main():
                    "stage_order": ("fused tile count, visible-splat work list, packed fragment rows, packed gradient rows, plain-store gradients"
                                    + (", tile-segmented sort" if tile_sort else "") if native else "reference order")
                                   + (", packed projection outputs" if args.packed_projection else "")
-                                  + (", projection backward fused with Adam" + (" (quantized SH state)" if args.quantization_level else "")
+                                  + (", projection backward fused with Adam" + ((" (quantized SH state" + (" and non-SH moments)" if args.non_sh_optim_bits == 16 else ")")) if args.quantization_level else "")
                                      if args.fused_optimizer else "")
                                   + (f", compositing variants dist_type={args.dist_type} median={int(args.median)} accum_mode={args.accum_mode}" if variants else ""),
                    "device_ms_per_iter_median": float(np.median(ms))},

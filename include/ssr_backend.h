@@ -322,9 +322,9 @@ int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream_t stream);
  * the nnz compacted rows of the packed projection; the reference sorts the rows by splat and walks a
  * per-splat range, FusedProjectionBwdOptim.cu:160-212 -- with one camera a splat has at most one
  * row, found through packed_row_of), regularizers mcmc_opacity, mcmc_scale, scale ratio, effective
- * rank, quaternion norm and SH/DC magnitude; the scale-agnostic step of the means. Not built
- * (rejected): quantized state of the non-SH parameters, 4-bit moments / 8-bit values, colour trust
- * region. */
+ * rank, quaternion norm and SH/DC magnitude; the scale-agnostic step of the means; the quantized SH
+ * state and the quantized moments of the non-SH tensors (below). Not built (rejected): the colour
+ * trust region of the linear-colour preset. */
 typedef struct {
     int64_t num_splats;
     int32_t sh_degree;
@@ -359,6 +359,14 @@ typedef struct {
     uint16_t* sh_value_packed;      /* [N * 3 * num_sh_buffer] */
     float* sh_value_bounds;         /* float2[ceil(N / 256)] */
     uint32_t num_sh_buffer;
+    /* Quantized Adam state of the five non-SH tensors (NonShQuantState, 16-bit codec;
+     * FusedProjectionBwdOptim_kernel.cuh:97-143,373-638), which the reference turns on together with the
+     * quantized SH state: per parameter one 32-bit cell (u code | log_s code << 16), per tensor one float4
+     * of bounds per block of 256 splats, in the order means, quats, log_scales, opacity_logits, features_dc.
+     * All ten given (then the matching members of g1 / g2 are not used) or all NULL; all-zero arrays are
+     * the zero moments. The parameters themselves stay fp32. */
+    uint32_t* non_sh_packed[5];     /* [N * 3], [N * 4], [N * 3], [N], [N * 3] */
+    float* non_sh_bounds[5];        /* float4[ceil(N / 256)] each */
 } ssr_fpbo_params;
 int ssr_fused_projection_bwd_optimizer(const ssr_fpbo_params* p, ssr_stream_t stream);
 /* row_of[g] = i where gaussian_ids[i] == g, -1 for splats without a packed row (one camera, so ids

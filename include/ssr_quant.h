@@ -1,9 +1,9 @@
 // ssr_quant.h -- the block-wise codecs of the quantized optimizer state, one definition for the host
 // restatement and the device kernels.
 //
-// QuantizedAdamState<8, 256> (src/core/Tensor.h:936-1133): per cell two bytes, the linearly quantized
-// u = g1 / (sqrt(g2) + eps) and log_s = log1p(sqrt(g2) / eps), against per-block bounds
-// (u_min, u_max, log_s_min, log_s_max). QuantizedTensor<16, 256> (src/core/Tensor.h:1300-1405): one
+// QuantizedAdamState<8, 256> and <16, 256> (src/core/Tensor.h:936-1133): per cell two codes (bytes, or
+// 16-bit halves of a word), the linearly quantized u = g1 / (sqrt(g2) + eps) and
+// log_s = log1p(sqrt(g2) / eps), against per-block bounds (u_min, u_max, log_s_min, log_s_max). QuantizedTensor<16, 256> (src/core/Tensor.h:1300-1405): one
 // 16-bit linear code per cell against per-block (min, max). Both are endpoint-exact and keep 0 <-> 0.
 //
 // log1p / expm1 are built on ssr_log / ssr_exp (the reference calls the CUDA math library), so codes can
@@ -39,17 +39,27 @@ SSR_HD void ssr_adamq_to_us(float g1, float g2, float* u, float* log_s) {
     *u = g1 / (sq + SSR_ADAMQ_EPS);
     *log_s = ssr_log1p(ssr_max(sq, 0.0f) * (1.0f / SSR_ADAMQ_EPS));
 }
-// code = u_q | s_q << 8 against bounds mm = (u_min, u_max, log_s_min, log_s_max): encode_g1g2_code
-SSR_HD uint32_t ssr_adamq_encode(float g1, float g2, const float mm[4]) {
+// The two codes of one cell against bounds mm = (u_min, u_max, log_s_min, log_s_max) at qmax = 2^bits - 1
+// levels: encode_us. The 8-bit state keeps them as u_q | s_q << 8, the 16-bit state as u_q | s_q << 16.
+SSR_HD void ssr_adamq_codes(float g1, float g2, const float mm[4], float qmax, uint32_t* u_q, uint32_t* s_q) {
     float u, ls;
     ssr_adamq_to_us(g1, g2, &u, &ls);
     const float ur = ssr_max(mm[1] - mm[0], SSR_ADAMQ_EPS), sr = ssr_max(mm[3] - mm[2], SSR_ADAMQ_EPS);
-    const float uq = ssr_min(ssr_max(ssr_round_code((255.0f * (u - mm[0])) / ur), 0.0f), 255.0f);
-    const float sq = ssr_min(ssr_max(ssr_round_code((255.0f * (ls - mm[2])) / sr), 0.0f), 255.0f);
-    return (uint32_t)uq | ((uint32_t)sq << 8);
+    *u_q = (uint32_t)ssr_min(ssr_max(ssr_round_code((qmax * (u - mm[0])) / ur), 0.0f), qmax);
+    *s_q = (uint32_t)ssr_min(ssr_max(ssr_round_code((qmax * (ls - mm[2])) / sr), 0.0f), qmax);
 }
-// decode_g1g2, in two steps: sqrt(g2) depends on the 8-bit log_s code alone, so a kernel can tabulate it per
-// block (256 entries) instead of evaluating expm1 per cell
+SSR_HD uint32_t ssr_adamq_encode(float g1, float g2, const float mm[4]) {     // 8-bit cell: encode_g1g2_code
+    uint32_t uq, sq;
+    ssr_adamq_codes(g1, g2, mm, 255.0f, &uq, &sq);
+    return uq | (sq << 8);
+}
+SSR_HD uint32_t ssr_adamq16_encode(float g1, float g2, const float mm[4]) {   // 16-bit cell
+    uint32_t uq, sq;
+    ssr_adamq_codes(g1, g2, mm, 65535.0f, &uq, &sq);
+    return uq | (sq << 16);
+}
+// decode_g1g2, in two steps: sqrt(g2) depends on the log_s code alone, so a kernel can tabulate it per
+// block (256 entries for the 8-bit state) instead of evaluating expm1 per cell
 SSR_HD float ssr_adamq_decode_sqrt_g2(uint32_t s_code, const float mm[4]) {
     const float kInv = 1.0f / 255.0f;
     const float ls = mm[2] + (mm[3] - mm[2]) * ((float)s_code * kInv);
@@ -63,6 +73,14 @@ SSR_HD void ssr_adamq_decode_with(uint32_t code, const float mm[4], float sq, fl
 }
 SSR_HD void ssr_adamq_decode(uint32_t code, const float mm[4], float* g1, float* g2) {
     ssr_adamq_decode_with(code, mm, ssr_adamq_decode_sqrt_g2((code >> 8) & 255u, mm), g1, g2);
+}
+SSR_HD void ssr_adamq16_decode(uint32_t code, const float mm[4], float* g1, float* g2) {
+    const float kInv = 1.0f / 65535.0f;
+    const float u = mm[0] + (mm[1] - mm[0]) * ((float)(code & 65535u) * kInv);
+    const float ls = mm[2] + (mm[3] - mm[2]) * ((float)(code >> 16) * kInv);
+    const float sq = SSR_ADAMQ_EPS * ssr_expm1(ls);
+    *g1 = u * (sq + SSR_ADAMQ_EPS);
+    *g2 = sq * sq;
 }
 
 // QuantizedTensor<16>::encode_v_code / decode_v against bounds (lo, hi)

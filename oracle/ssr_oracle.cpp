@@ -522,18 +522,39 @@ void or_quant_codec(int op, int64_t n, float* a, float* b, const float* mm, uint
         if (op == 0) codes[i] = ssr_adamq_encode(a[i], b[i], mm);
         else if (op == 1) ssr_adamq_decode(codes[i], mm, a + i, b + i);
         else if (op == 2) codes[i] = ssr_q16_encode(a[i], mm[0], mm[1]);
-        else a[i] = ssr_q16_decode(codes[i], mm[0], mm[1]);
+        else if (op == 3) a[i] = ssr_q16_decode(codes[i], mm[0], mm[1]);
+        else if (op == 4) codes[i] = ssr_adamq16_encode(a[i], b[i], mm);
+        else ssr_adamq16_decode(codes[i], mm, a + i, b + i);
     }
 }
 
 static void fused_optimizer_impl(int64_t N, int sh_degree,
     float* means, float* quats, float* log_scales, float* opacity_logits, float* features_dc, float* features_sh,
-    const or_sh_quant_state* q,
+    const or_sh_quant_state* q, const or_non_sh_quant_state* nq,
     const or_camera* cam, const float* aabb,
     const float* v_xy, const float* v_sdepth, const float* v_conic, const float* v_opac, const float* v_srgb,
-    const float* const* v_in, float* const* g1, float* const* g2, float* densify_score,
+    const float* const* v_in, float* const* g1_in, float* const* g2_in, float* densify_score,
     const float* hyper, int32_t step, const int32_t* steps, const float* radii) {
     const int n_coef = sh_degree * (sh_degree + 2);
+    // Quantized non-SH state (NonShQuantState, FusedProjectionBwdOptim_kernel.cuh:97-143,373-638): the moments of the
+    // five non-SH tensors are decoded against each block's OLD bounds into fp32, the step below runs on those, and
+    // afterwards each block's min / max of the new (u, log_s) become its NEW bounds, against which they are encoded.
+    static const int kPrims[5] = {3, 4, 3, 1, 3};
+    const int64_t n_blocks_ns = (N + 255) / 256;
+    std::vector<float> dq1[5], dq2[5];
+    float* g1[6];
+    float* g2[6];
+    for (int t = 0; t < 6; t++) { g1[t] = g1_in ? g1_in[t] : nullptr; g2[t] = g2_in ? g2_in[t] : nullptr; }
+    if (nq) {
+        for (int t = 0; t < 5; t++) {
+            dq1[t].resize((size_t)N * kPrims[t]); dq2[t].resize((size_t)N * kPrims[t]);
+            for (int64_t g = 0; g < N; g++)
+                for (int i = 0; i < kPrims[t]; i++)
+                    ssr_adamq16_decode(nq->packed[t][kPrims[t] * g + i], nq->bounds[t] + 4 * (g / 256), &dq1[t][kPrims[t] * g + i],
+                                       &dq2[t][kPrims[t] * g + i]);
+            g1[t] = dq1[t].data(); g2[t] = dq2[t].data();
+        }
+    }
     std::vector<float> vm((size_t)N * 3), vq((size_t)N * 4), vs((size_t)N * 3), vo((size_t)N), vd((size_t)N * 3),
         vsh((size_t)N * 45);
     or_sh_source src;
@@ -656,6 +677,21 @@ static void fused_optimizer_impl(int64_t N, int sh_degree,
         for (int i = 0; i < 3; i++)
             features_dc[3 * g + i] = adam(features_dc[3 * g + i], gd[i], lr_dc, g1[4] + 3 * g + i, g2[4] + 3 * g + i);
     }
+    if (nq) {
+        for (int t = 0; t < 5; t++)
+            for (int64_t blk = 0; blk < n_blocks_ns; blk++) {
+                const int64_t c0 = blk * 256 * kPrims[t], c1 = std::min<int64_t>(N, blk * 256 + 256) * kPrims[t];
+                float mm[4] = {1e30f, -1e30f, 1e30f, -1e30f};
+                for (int64_t c = c0; c < c1; c++) {
+                    float u, ls;
+                    ssr_adamq_to_us(dq1[t][c], dq2[t][c], &u, &ls);
+                    mm[0] = ssr_min(mm[0], u); mm[1] = ssr_max(mm[1], u);
+                    mm[2] = ssr_min(mm[2], ls); mm[3] = ssr_max(mm[3], ls);
+                }
+                for (int k = 0; k < 4; k++) nq->bounds[t][4 * blk + k] = mm[k];
+                for (int64_t c = c0; c < c1; c++) nq->packed[t][c] = ssr_adamq16_encode(dq1[t][c], dq2[t][c], mm);
+            }
+    }
     if (!q) return;
     // ---- SH coefficients and moments in the quantized state, FusedProjectionBwdOptim_kernel.cuh:709-1030 ----
     // Per block of 256 splats: decode moments and values against the block's OLD bounds, take the Adam step in
@@ -732,17 +768,18 @@ void or_fused_projection_bwd_optimizer(int64_t N, int sh_degree,
     const float* v_xy, const float* v_sdepth, const float* v_conic, const float* v_opac, const float* v_srgb,
     const float* const* v_in, float* const* g1, float* const* g2, float* densify_score,
     const float* hyper, int32_t step, const int32_t* steps, const float* radii) {
-    fused_optimizer_impl(N, sh_degree, means, quats, log_scales, opacity_logits, features_dc, features_sh, nullptr, cam, aabb,
+    fused_optimizer_impl(N, sh_degree, means, quats, log_scales, opacity_logits, features_dc, features_sh, nullptr, nullptr, cam, aabb,
                          v_xy, v_sdepth, v_conic, v_opac, v_srgb, v_in, g1, g2, densify_score, hyper, step, steps, radii);
 }
 
 void or_fused_projection_bwd_optimizer_q(int64_t N, int sh_degree,
     float* means, float* quats, float* log_scales, float* opacity_logits, float* features_dc, const or_sh_quant_state* q,
+    const or_non_sh_quant_state* nq,
     const or_camera* cam, const float* aabb,
     const float* v_xy, const float* v_sdepth, const float* v_conic, const float* v_opac, const float* v_srgb,
     const float* const* v_in, float* const* g1, float* const* g2, float* densify_score,
     const float* hyper, int32_t step, const int32_t* steps, const float* radii) {
-    fused_optimizer_impl(N, sh_degree, means, quats, log_scales, opacity_logits, features_dc, nullptr, q, cam, aabb,
+    fused_optimizer_impl(N, sh_degree, means, quats, log_scales, opacity_logits, features_dc, nullptr, q, nq, cam, aabb,
                          v_xy, v_sdepth, v_conic, v_opac, v_srgb, v_in, g1, g2, densify_score, hyper, step, steps, radii);
 }
 

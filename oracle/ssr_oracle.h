@@ -154,15 +154,26 @@ typedef struct {
     float* value_bounds;        /* float2[ceil(N / 256)] */
     uint32_t num_sh_buffer;
 } or_sh_quant_state;
-/* As or_fused_projection_bwd_optimizer, with the SH coefficients and their moments held in q. */
+/* The quantized Adam state of the five non-SH tensors (NonShQuantState,
+ * src/kernels/optim/FusedProjectionBwdOptim_kernel.cuh:97-143,373-638): QuantizedAdamState<16,256> cells
+ * (u code | log_s code << 16), one float4 of bounds per 256 splats and tensor; order means, quats,
+ * log_scales, opacity_logits, features_dc. */
+typedef struct {
+    uint32_t* packed[5];        /* [N * 3], [N * 4], [N * 3], [N], [N * 3] */
+    float* bounds[5];           /* float4[ceil(N / 256)] each */
+} or_non_sh_quant_state;
+/* As or_fused_projection_bwd_optimizer, with the SH coefficients and their moments held in q and, when nq is
+ * given, the moments of the non-SH tensors in nq (g1 / g2 entries 0..4 are then not used). */
 void or_fused_projection_bwd_optimizer_q(int64_t N, int sh_degree,
     float* means, float* quats, float* log_scales, float* opacity_logits, float* features_dc, const or_sh_quant_state* q,
+    const or_non_sh_quant_state* nq,
     const or_camera* cam, const float* aabb,
     const float* v_xy, const float* v_sdepth, const float* v_conic, const float* v_opac, const float* v_srgb,
     const float* const* v_in, float* const* g1, float* const* g2, float* densify_score,
     const float* hyper, int32_t step, const int32_t* steps, const float* radii);
 /* The codecs on arrays: op 0 Adam-state encode (a = g1, b = g2, mm float4 -> codes), 1 Adam-state decode
- * (codes -> a = g1, b = g2), 2 value encode (a = v, mm float2 -> codes), 3 value decode (codes -> a). */
+ * (codes -> a = g1, b = g2), 2 value encode (a = v, mm float2 -> codes), 3 value decode (codes -> a), 4 / 5 the
+ * 16-bit Adam-state encode / decode. */
 void or_quant_codec(int op, int64_t n, float* a, float* b, const float* mm, uint32_t* codes);
 
 /* erank_reg_3dgs (src/shaders/per_splat_losses.slang:3-15): the loss for one splat's three log-scales and

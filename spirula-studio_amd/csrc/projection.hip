@@ -623,20 +623,34 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
 // ---- projection backward fused with Adam ---------------------------------------------------------
 struct AdamD { float b1c, b2c; };   // 1/(1-beta1^t), 1/(1-beta2^t)
 
-__device__ __forceinline__ float adam_step(float x, float v, float lr, const AdamD& a, float* g1p, float* g2p) {
+// one Adam step on values: the moments are updated in place, the stepped parameter is returned
+__device__ __forceinline__ float adam_core(float x, float v, float lr, const AdamD& a, float& g1, float& g2) {
     constexpr float kBeta1 = 0.9f, kBeta2 = 0.999f, kEps = 1e-15f;
-    const float g1 = kBeta1 * *g1p + (1.f - kBeta1) * v;
-    const float g2 = kBeta2 * *g2p + (1.f - kBeta2) * (v * v);
-    *g1p = g1; *g2p = g2;
+    g1 = kBeta1 * g1 + (1.f - kBeta1) * v;
+    g2 = kBeta2 * g2 + (1.f - kBeta2) * (v * v);
     return x - ((lr * a.b1c) * g1) / (ssr_sqrt(g2 * a.b2c) + kEps);
 }
+__device__ __forceinline__ float adam_step(float x, float v, float lr, const AdamD& a, float* g1p, float* g2p) {
+    float g1 = *g1p, g2 = *g2p;
+    const float r = adam_core(x, v, lr, a, g1, g2);
+    *g1p = g1; *g2p = g2;
+    return r;
+}
+
+// The five non-SH tensors in the order of the quantized non-SH state: means, quats, log_scales, opacity_logits,
+// features_dc; kNsOff = first of a tensor's parameters among a splat's 14, kNsPrims = how many it has.
+__device__ __forceinline__ float* non_sh_tensor(const ssr_world& w, int t) {
+    return t == 0 ? w.means : t == 1 ? w.quats : t == 2 ? w.log_scales : t == 3 ? w.opacity_logits : w.features_dc;
+}
+__device__ __forceinline__ constexpr int ns_off(int t) { return t == 0 ? 0 : t == 1 ? 3 : t == 2 ? 7 : t == 3 ? 10 : 11; }
+__device__ __forceinline__ constexpr int ns_prims(int t) { return t == 1 ? 4 : t == 3 ? 1 : 3; }
 
 // Two phases per workgroup of 256 splats. Phase 1, one thread per splat: projection VJP in
 // registers, regularizers, Adam on the 14 non-SH parameters; the SH gradient is rank one
 // (Y_j * v_colour), so only its factors (15 + 3 floats) go to LDS. Phase 2, the workgroup streams
 // over its 256 x 3 kCoef SH coefficients in memory order: parameter and both moments are read and
 // written fully coalesced, the gradient is rebuilt from the factors in LDS.
-template <int kDegree, bool kLens, bool kQuant>
+template <int kDegree, bool kLens, bool kQuant, bool kNsq>
 __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_kernel(ssr_fpbo_params P, AdamD scalar_adam) {
     constexpr int kCoef = kDegree * (kDegree + 2);
     constexpr int kY = kCoef > 0 ? kCoef : 1;
@@ -645,6 +659,7 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
     __shared__ float s_b1c[kProjBlock], s_b2c[kProjBlock];
     __shared__ float s_red[kProjBlock / 64][6];   // quantized state: per-wave min / max of the new bounds
     __shared__ float s_sqrt_g2[kQuant ? 256 : 1];  // quantized state: sqrt(g2) of each 8-bit log_s code under the old bounds
+    __shared__ float s_ns[kNsq ? kProjBlock / 64 : 1][20];   // quantized non-SH state: per-wave (min, max) x (u, log_s) x 5 tensors
     const int64_t block0 = (int64_t)blockIdx.x * kProjBlock;
     const int64_t g = block0 + threadIdx.x;
     const ssr_world& W = P.world;
@@ -652,6 +667,52 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
 #pragma unroll
     for (int j = 0; j < kY; j++) s_Y[threadIdx.x][j] = 0.f;
     s_vc[threadIdx.x][0] = s_vc[threadIdx.x][1] = s_vc[threadIdx.x][2] = 0.f;
+    // Moments of the 14 non-SH parameters: fp32 arrays, or (NonShQuantState, FusedProjectionBwdOptim_kernel.cuh:97-143,
+    // 373-638) 16-bit (u, log_s) cells decoded against the block's old bounds, kept in registers after the step
+    // and encoded once the block's new bounds are known.
+    float ns_g1[kNsq ? 14 : 1], ns_g2[kNsq ? 14 : 1];
+    float ns_mm[kNsq ? 5 : 1][4];
+    if (kNsq) {
+#pragma unroll
+        for (int t = 0; t < 5; t++) { ns_mm[t][0] = 1e30f; ns_mm[t][1] = -1e30f; ns_mm[t][2] = 1e30f; ns_mm[t][3] = -1e30f; }
+#pragma unroll
+        for (int i = 0; i < 14; i++) { ns_g1[i] = 0.f; ns_g2[i] = 0.f; }
+    }
+    float ns_old[kNsq ? 5 : 1][4];
+    if (kNsq) {
+#pragma unroll
+        for (int t = 0; t < 5; t++)
+#pragma unroll
+            for (int k = 0; k < 4; k++) ns_old[t][k] = P.non_sh_bounds[t][4 * blockIdx.x + k];
+    }
+    auto fetch_moments = [&](int t, int i, float& m1, float& m2) {
+        if (kNsq) {
+            ssr_adamq16_decode(P.non_sh_packed[t][(int64_t)ns_prims(t) * g + i], ns_old[t], &m1, &m2);
+        } else {
+            m1 = non_sh_tensor(P.g1, t)[(int64_t)ns_prims(t) * g + i];
+            m2 = non_sh_tensor(P.g2, t)[(int64_t)ns_prims(t) * g + i];
+        }
+    };
+    auto keep_moments = [&](int t, int i, float m1, float m2) {
+        if (kNsq) {
+            ns_g1[ns_off(t) + i] = m1; ns_g2[ns_off(t) + i] = m2;
+            float u, ls;
+            ssr_adamq_to_us(m1, m2, &u, &ls);
+            ns_mm[t][0] = ssr_min(ns_mm[t][0], u); ns_mm[t][1] = ssr_max(ns_mm[t][1], u);
+            ns_mm[t][2] = ssr_min(ns_mm[t][2], ls); ns_mm[t][3] = ssr_max(ns_mm[t][3], ls);
+        } else {
+            non_sh_tensor(P.g1, t)[(int64_t)ns_prims(t) * g + i] = m1;
+            non_sh_tensor(P.g2, t)[(int64_t)ns_prims(t) * g + i] = m2;
+        }
+    };
+    // Adam on parameter i of tensor t: returns the stepped value
+    auto step_param = [&](int t, int i, float x, float v, float lr) {
+        float m1, m2;
+        fetch_moments(t, i, m1, m2);
+        const float r = adam_core(x, v, lr, ad, m1, m2);
+        keep_moments(t, i, m1, m2);
+        return r;
+    };
     if (g < P.num_splats) {
         if (P.steps) {   // per-splat step: beta^t = exp(t ln beta)
             const float t = (float)P.steps[g];
@@ -730,8 +791,7 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
 
         // scales, quats (Riemannian), opacity, means, dc -- FusedProjectionBwdOptim_kernel.cuh:390-612
 #pragma unroll
-        for (int i = 0; i < 3; i++)
-            W.log_scales[3 * g + i] = adam_step(ls[i], wg.scale[i], P.lr_scales, ad, P.g1.log_scales + 3 * g + i, P.g2.log_scales + 3 * g + i);
+        for (int i = 0; i < 3; i++) W.log_scales[3 * g + i] = step_param(2, i, ls[i], wg.scale[i], P.lr_scales);
         {
             const float n2 = (quat[0] * quat[0] + quat[1] * quat[1]) + (quat[2] * quat[2] + quat[3] * quat[3]);
             const float inv = 1.0f / ssr_sqrt(n2);
@@ -742,12 +802,12 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
 #pragma unroll
             for (int i = 0; i < 4; i++) v[i] = wg.quat[i] - d * q[i];
 #pragma unroll
-            for (int i = 0; i < 4; i++) q[i] = adam_step(q[i], v[i], P.lr_quats, ad, P.g1.quats + 4 * g + i, P.g2.quats + 4 * g + i);
+            for (int i = 0; i < 4; i++) q[i] = step_param(1, i, q[i], v[i], P.lr_quats);
             const float m2 = (q[0] * q[0] + q[1] * q[1]) + (q[2] * q[2] + q[3] * q[3]);
             const float minv = 1.0f / ssr_sqrt(m2);
             *reinterpret_cast<float4*>(W.quats + 4 * g) = make_float4(q[0] * minv, q[1] * minv, q[2] * minv, q[3] * minv);
         }
-        W.opacity_logits[g] = adam_step(logit, wg.logit, P.lr_opacs, ad, P.g1.opacity_logits + g, P.g2.opacity_logits + g);
+        W.opacity_logits[g] = step_param(3, 0, logit, wg.logit, P.lr_opacs);
         if (P.densify_score) {
             const float smax = ssr_max(ssr_max(ls[0], ls[1]), ls[2]);
             P.densify_score[g] = ssr_exp(smax) * ssr_sqrt(dot3(wg.mean, wg.mean));
@@ -779,21 +839,53 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
 #pragma unroll
             for (int i = 0; i < 3; i++) {
                 const float num = ((cov[i][0] * wg.mean[0] + cov[i][1] * wg.mean[1]) + cov[i][2] * wg.mean[2]) * extent;
-                float* g1p = P.g1.means + 3 * g + i;
-                float* g2p = P.g2.means + 3 * g + i;
-                const float m1 = kBeta1 * *g1p + (1.f - kBeta1) * num;
-                const float m2 = kBeta2 * *g2p + (1.f - kBeta2) * (((wg.mean[i] * wg.mean[i]) * den) * den);
-                *g1p = m1; *g2p = m2;
+                float m1, m2;
+                fetch_moments(0, i, m1, m2);
+                m1 = kBeta1 * m1 + (1.f - kBeta1) * num;
+                m2 = kBeta2 * m2 + (1.f - kBeta2) * (((wg.mean[i] * wg.mean[i]) * den) * den);
+                keep_moments(0, i, m1, m2);
                 W.means[3 * g + i] = mean[i] - ((P.lr_means * ad.b1c) * m1) / (ssr_sqrt(m2 * ad.b2c) + kEps);
             }
         } else {
 #pragma unroll
-            for (int i = 0; i < 3; i++)
-                W.means[3 * g + i] = adam_step(mean[i], wg.mean[i], P.lr_means, ad, P.g1.means + 3 * g + i, P.g2.means + 3 * g + i);
+            for (int i = 0; i < 3; i++) W.means[3 * g + i] = step_param(0, i, mean[i], wg.mean[i], P.lr_means);
         }
 #pragma unroll
-        for (int i = 0; i < 3; i++)
-            W.features_dc[3 * g + i] = adam_step(dc[i], wg.dc[i], P.lr_features_dc, ad, P.g1.features_dc + 3 * g + i, P.g2.features_dc + 3 * g + i);
+        for (int i = 0; i < 3; i++) W.features_dc[3 * g + i] = step_param(4, i, dc[i], wg.dc[i], P.lr_features_dc);
+    }
+    if (kNsq) {
+        // new bounds of the block: every thread takes part (those past the last splat hold the neutral element),
+        // then each splat's 14 cells are encoded against them
+#pragma unroll
+        for (int t = 0; t < 5; t++) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                float v = ns_mm[t][k];
+#pragma unroll
+                for (int d = 32; d >= 1; d >>= 1) v = (k & 1) ? ssr_max(v, __shfl_xor(v, d, 64)) : ssr_min(v, __shfl_xor(v, d, 64));
+                if ((threadIdx.x & 63) == 0) s_ns[threadIdx.x >> 6][4 * t + k] = v;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < 5; t++) {
+            float mm[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                mm[k] = s_ns[0][4 * t + k];
+#pragma unroll
+                for (int w = 1; w < kProjBlock / 64; w++) mm[k] = (k & 1) ? ssr_max(mm[k], s_ns[w][4 * t + k]) : ssr_min(mm[k], s_ns[w][4 * t + k]);
+            }
+            if (threadIdx.x == 0) {
+#pragma unroll
+                for (int k = 0; k < 4; k++) P.non_sh_bounds[t][4 * blockIdx.x + k] = mm[k];
+            }
+            if (g < P.num_splats) {
+#pragma unroll
+                for (int i = 0; i < ns_prims(t); i++)
+                    P.non_sh_packed[t][(int64_t)ns_prims(t) * g + i] = ssr_adamq16_encode(ns_g1[ns_off(t) + i], ns_g2[ns_off(t) + i], mm);
+            }
+        }
     }
     s_b1c[threadIdx.x] = ad.b1c; s_b2c[threadIdx.x] = ad.b2c;
     if (kCoef == 0) return;
@@ -1157,8 +1249,14 @@ extern "C" int ssr_fused_projection_bwd_optimizer(const ssr_fpbo_params* p, ssr_
     SSR_REQUIRE(p->v_rows || (p->v_screen.xy && p->v_screen.depth && p->v_screen.conic && p->v_screen.opac && p->v_screen.rgb), where,
                 "null v_screen buffer");
     const bool quant = p->sh_state_packed != nullptr;
+    int n_ns = 0;
+    for (int t = 0; t < 5; t++) n_ns += (p->non_sh_packed[t] != nullptr) + (p->non_sh_bounds[t] != nullptr);
+    SSR_REQUIRE(n_ns == 0 || n_ns == 10, where, "the quantized non-SH state needs all five packed and all five bounds arrays");
+    const bool nsq = n_ns == 10;
+    SSR_REQUIRE(!nsq || quant, where, "the quantized non-SH state is built together with the quantized SH state only");
     for (const ssr_world* w : {&p->world, &p->g1, &p->g2}) {
-        SSR_REQUIRE(w->means && w->quats && w->log_scales && w->opacity_logits && w->features_dc, where, "null parameter or moment buffer");
+        SSR_REQUIRE((nsq && w != &p->world) || (w->means && w->quats && w->log_scales && w->opacity_logits && w->features_dc), where,
+                    "null parameter or moment buffer");
         SSR_REQUIRE(quant || p->sh_degree == 0 || (w->features_sh && w->sh_stride >= 3 * p->sh_degree * (p->sh_degree + 2)), where,
                     "features_sh missing or sh_stride too small");
     }
@@ -1175,13 +1273,15 @@ extern "C" int ssr_fused_projection_bwd_optimizer(const ssr_fpbo_params* p, ssr_
     const dim3 grid((unsigned)ceil_div(p->num_splats, kProjBlock)), block(kProjBlock);
     hipStream_t s = as_stream(stream);
     const bool lens = camera_needs_lens_path(p->camera.camera_model, p->camera.distortion);
-#define SSR_LAUNCH_FPBO(D)                                                                                              \
-    if (quant) {                                                                                                        \
-        if (lens) hipLaunchKernelGGL((fused_projection_bwd_optimizer_kernel<D, true, true>), grid, block, 0, s, *p, ad);  \
-        else hipLaunchKernelGGL((fused_projection_bwd_optimizer_kernel<D, false, true>), grid, block, 0, s, *p, ad);      \
-    } else {                                                                                                            \
-        if (lens) hipLaunchKernelGGL((fused_projection_bwd_optimizer_kernel<D, true, false>), grid, block, 0, s, *p, ad); \
-        else hipLaunchKernelGGL((fused_projection_bwd_optimizer_kernel<D, false, false>), grid, block, 0, s, *p, ad);     \
+#define SSR_LAUNCH_FPBO_Q(D, L)                                                                                             \
+    if (nsq) hipLaunchKernelGGL((fused_projection_bwd_optimizer_kernel<D, L, true, true>), grid, block, 0, s, *p, ad);          \
+    else if (quant) hipLaunchKernelGGL((fused_projection_bwd_optimizer_kernel<D, L, true, false>), grid, block, 0, s, *p, ad);  \
+    else hipLaunchKernelGGL((fused_projection_bwd_optimizer_kernel<D, L, false, false>), grid, block, 0, s, *p, ad);
+#define SSR_LAUNCH_FPBO(D)           \
+    if (lens) {                      \
+        SSR_LAUNCH_FPBO_Q(D, true)   \
+    } else {                         \
+        SSR_LAUNCH_FPBO_Q(D, false)  \
     }
     switch (p->sh_degree) {
         case 0: SSR_LAUNCH_FPBO(0); break;
@@ -1190,6 +1290,7 @@ extern "C" int ssr_fused_projection_bwd_optimizer(const ssr_fpbo_params* p, ssr_
         default: SSR_LAUNCH_FPBO(3); break;
     }
 #undef SSR_LAUNCH_FPBO
+#undef SSR_LAUNCH_FPBO_Q
     SSR_CHECK_LAUNCH(where);
     return 0;
 }

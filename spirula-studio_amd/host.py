@@ -23,7 +23,8 @@ SYMBOLS = {
     "ssrh_set_sh_value_quant": (C.c_int, [C.c_int, vp, C.c_int64, C.c_int, vp, C.c_int64, C.c_int, C.c_int64]),
     "ssrh_set_camera_params": (C.c_int, [C.c_int, C.c_int, C.c_char_p, C.c_char_p, vp, vp, vp, C.c_int]),
     "ssrh_backward_with_variants": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, C.c_int]),
-    "ssrh_backward_fused_optimizer": (C.c_int, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int]),
+    "ssrh_backward_fused_optimizer": (C.c_int, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_int]),
+    "ssrh_copy_non_sh_quant_state": (C.c_int, [vp, vp]),
     "ssrh_copy_sh_quant_state": (C.c_int, [vp, vp, vp, vp]),
     "ssrh_copy_params_to_host": (C.c_int, [vp, vp, vp, vp, vp, vp]),
     "ssrh_set_tile_mask": (C.c_int, [vp, C.c_int, C.c_int]),
@@ -149,12 +150,23 @@ class Engine:
              "scale_regularization_weight", "mcmc_opacity_reg_weight", "mcmc_scale_reg_weight", "quat_norm_reg_weight",
              "sh_reg_weight", "erank_reg_weight", "erank_reg_weight_s3"]
 
-    def backward_fused_optimizer(self, hyper, step, scale_agnostic_mean=False, quantization_level=0):
+    def backward_fused_optimizer(self, hyper, step, scale_agnostic_mean=False, quantization_level=0, non_sh_optim_bits=32):
         """Compositing backward, then the projection backward fused with the Adam step: the engine's
-        parameters and its Adam moments are updated in place (fp32 SH only)."""
+        parameters and its Adam moments are updated in place. quantization_level 1: quantized SH values and
+        moments; non_sh_optim_bits 16 (with level 1): the other moments as 16-bit cells too."""
         hv = np.array([hyper.get(k, 0.0) for k in self.HYPER], np.float32)
         check(self.h.ssrh_backward_fused_optimizer(self.d_vrgb.ptr, self.d_vdepth.ptr, self.d_vT.ptr, hv.ctypes.data, int(step),
-                                                   int(scale_agnostic_mean), int(quantization_level)))
+                                                   int(scale_agnostic_mean), int(quantization_level), int(non_sh_optim_bits)))
+
+    def non_sh_quant_state(self):
+        """non_sh_optim_bits 16: the engine's quantized non-SH moments, per tensor (means, quats, log_scales,
+        opacity_logits, features_dc) the 32-bit cells and the [blocks, 4] bounds."""
+        n = self.sc.n
+        nb = (n + 255) // 256
+        pk, bd = np.zeros(n * 14, np.uint32), np.zeros((5, nb, 4), np.float32)
+        check(self.h.ssrh_copy_non_sh_quant_state(pk.ctypes.data, bd.ctypes.data))
+        off = [0, 3, 7, 10, 11, 14]
+        return dict(packed=[pk[n * off[t]: n * off[t + 1]].copy() for t in range(5)], bounds=[bd[t].copy() for t in range(5)])
 
     def sh_quant_state(self):
         """Quantization level 1: the engine's SH moments and values as host arrays."""

@@ -640,7 +640,6 @@ void fused_projection_bwd_optimizer_3dgs(
     // quantization_level: 0 = fp32 SH and moments; 1 = 16-bit SH values, 8-bit moments
     // (src/kernels/optim/FusedProjectionBwdOptim_kernel.cuh:1104-1111; validation as FusedProjectionBwdOptim.cu:386-400)
     if (quantization_level != 0 && quantization_level != 1) throw std::runtime_error(std::string(w) + "quantization_level must be 0 or 1");
-    if (non_sh.enabled) throw std::runtime_error(std::string(w) + "quantized state of the non-SH parameters is not built in this backend");
     const bool quant = quantization_level == 1;
     if (quant && !(sh_packed && sh_quant_bounds && sh_value_packed && sh_value_bounds))
         throw std::runtime_error(std::string(w) + "quantization level 1 needs the packed SH state, the packed SH values and both bounds");
@@ -658,6 +657,15 @@ void fused_projection_bwd_optimizer_3dgs(
         p.sh_value_packed = (uint16_t*)std::get<0>(*sh_value_packed);
         p.sh_value_bounds = (float*)std::get<0>(*sh_value_bounds);
         p.num_sh_buffer = (uint32_t)(splats_world[5].channels() / 3);   // the buffers' stride, not the active degree
+        if (non_sh.enabled) {   // read only at a quantized level, as in the kernel (FusedProjectionBwdOptim_kernel.cuh:378)
+            uint8_t* pk[5] = {non_sh.means_packed, non_sh.quats_packed, non_sh.scales_packed, non_sh.opacities_packed, non_sh.features_dc_packed};
+            float* bd[5] = {non_sh.means_bounds, non_sh.quats_bounds, non_sh.scales_bounds, non_sh.opacities_bounds, non_sh.features_dc_bounds};
+            for (int t = 0; t < 5; t++) {
+                if (!pk[t] || !bd[t]) throw std::runtime_error(std::string(w) + "non_sh.enabled with a null buffer");
+                p.non_sh_packed[t] = reinterpret_cast<uint32_t*>(pk[t]);
+                p.non_sh_bounds[t] = bd[t];
+            }
+        }
     }
     p.camera = camera_of(camera_model, distortion, dist_coeffs, viewmats, intrins, image_width, image_height);
     p.aabb = aabb.data_ptr();
@@ -665,8 +673,8 @@ void fused_projection_bwd_optimizer_3dgs(
     if (g_vrows && p.v_screen.xy == g_vrows_for_xy) p.v_rows = g_vrows;
     if (!v_splats_world.empty()) p.v_world_in = world_of(v_splats_world);
     p.v_world_in.features_sh = nullptr;   // not read (FusedProjectionBwdOptim_kernel.cuh:250-255)
-    p.g1 = world_of(g1_splats_world);
-    p.g2 = world_of(g2_splats_world);
+    if (!g1_splats_world.empty()) p.g1 = world_of(g1_splats_world);
+    if (!g2_splats_world.empty()) p.g2 = world_of(g2_splats_world);
     p.densify_score = densify_score.data_ptr();
     p.lr_means = lr_means; p.lr_quats = lr_quats; p.lr_scales = lr_scales; p.lr_opacs = lr_opacs;
     p.lr_features_dc = lr_features_dc; p.lr_features_sh = lr_features_sh;

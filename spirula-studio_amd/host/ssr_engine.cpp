@@ -279,7 +279,7 @@ void engine_backward_with_variants(TorchTensorView v_render_rgb, TorchTensorView
 
 void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
                                      TorchTensorView v_render_Ts, const float hyper[14], int step, bool scale_agnostic_mean,
-                                     int quantization_level) {
+                                     int quantization_level, int non_sh_optim_bits) {
     auto& E = engine();
     if (std::get<0>(E.fwd.renders).data_ptr() == nullptr)
         throw std::runtime_error("engine_backward_fused_optimizer: forward_3dgs must be called first");
@@ -320,6 +320,28 @@ void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorVi
         sh_state_bounds = TorchTensorView{(uint64_t)(uintptr_t)sb, 4u, std::vector<int64_t>{nb, 4}};
         sh_values = E.world.sh_packed; sh_value_bounds = E.world.sh_bounds;
     }
+    // OptimConfig::non_sh_optim_bits (src/engine/EngineConfig.h:120; the trainer sets 16 at every quantized level,
+    // src/app/TrainerCore.cpp:383): the moments of the five non-SH tensors as 16-bit cells in two pool slots, tensor
+    // after tensor, all zeros at first; read at a quantized level only (src/engine/EngineDensify.cpp:179-193)
+    if (non_sh_optim_bits != 32 && non_sh_optim_bits != 16)
+        throw std::runtime_error("engine_backward_fused_optimizer: non_sh_optim_bits must be 32 (off) or 16");
+    NonShQuantState non_sh;
+    if (non_sh_optim_bits == 16 && quantization_level == 1) {
+        const int64_t nb = (n + 255) / 256;
+        uint8_t* pk = DevicePool::global().acquire<uint8_t>(PoolSlot::AdamNonShPacked, (size_t)(n * 14 * 4));
+        float* bd = DevicePool::global().acquire<float>(PoolSlot::AdamNonShBounds, (size_t)(5 * nb * 4));
+        if (!E.optim.non_sh_state_ready) {
+            backend::memset_async(pk, 0, (size_t)(n * 14 * 4));
+            backend::memset_async(bd, 0, (size_t)(5 * nb * 4) * sizeof(float));
+            E.optim.non_sh_state_ready = true;
+        }
+        non_sh.enabled = true;
+        non_sh.means_packed = pk;                 non_sh.means_bounds = bd;
+        non_sh.quats_packed = pk + n * 3 * 4;     non_sh.quats_bounds = bd + nb * 4;
+        non_sh.scales_packed = pk + n * 7 * 4;    non_sh.scales_bounds = bd + 2 * nb * 4;
+        non_sh.opacities_packed = pk + n * 10 * 4; non_sh.opacities_bounds = bd + 3 * nb * 4;
+        non_sh.features_dc_packed = pk + n * 11 * 4; non_sh.features_dc_bounds = bd + 4 * nb * 4;
+    }
     E.grad.v_screen = raster_backward(v_render_rgb, v_render_depth, v_render_Ts);
     const int64_t W = E.camera.width, H = E.camera.height;
     DeviceVector<int32_t> cam_ids, gauss_ids;
@@ -335,7 +357,7 @@ void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorVi
     fused_projection_bwd_optimizer_3dgs(
         E.cur_num_splats, E.sh_degree, E.fwd.splats_w, E.camera.viewmats, E.camera.intrins, (uint32_t)W, (uint32_t)H,
         E.camera.model_str, E.camera.distortion_str, E.camera.dist_coeffs, cam_ids, gauss_ids, aabb, {}, E.grad.v_screen,
-        E.optim.g1, E.optim.g2, sh_state, sh_state_bounds, sh_values, sh_value_bounds, NonShQuantState{},
+        E.optim.g1, E.optim.g2, sh_state, sh_state_bounds, sh_values, sh_value_bounds, non_sh,
         E.optim.radii, E.optim.densify_score, hyper[0], hyper[1], hyper[2], hyper[3], hyper[4], hyper[5], hyper[6], hyper[7],
         hyper[8], hyper[9], hyper[12], hyper[13], hyper[10], hyper[11], scale_agnostic_mean, false, 0.0f, (int32_t)step, quantization_level);
 }
@@ -483,11 +505,27 @@ int ssrh_backward_with_variants(const float* v_rgb, const float* v_depth, const 
 }
 
 int ssrh_backward_fused_optimizer(const float* v_rgb, const float* v_depth, const float* v_Ts, const float* hyper14, int step,
-                                  int scale_agnostic_mean, int quantization_level) {
+                                  int scale_agnostic_mean, int quantization_level, int non_sh_optim_bits) {
     return guard([&] {
         const int64_t C = engine().camera.num, H = engine().camera.height, W = engine().camera.width;
         engine_backward_fused_optimizer(tv(v_rgb, 4, {C, H, W, 3}), tv(v_depth, 4, {C, H, W, 1}), tv(v_Ts, 4, {C, H, W, 1}), hyper14, step,
-                                        scale_agnostic_mean != 0, quantization_level);
+                                        scale_agnostic_mean != 0, quantization_level, non_sh_optim_bits);
+    });
+}
+
+// non_sh_optim_bits 16: copies the quantized non-SH moments to the host: 14 * N 32-bit cells (means, quats, scales,
+// opacities, dc, tensor after tensor) and 5 x ceil(N / 256) float4 bounds in the same order.
+int ssrh_copy_non_sh_quant_state(uint32_t* packed, float* bounds) {
+    return guard([&] {
+        auto& E = engine();
+        const int64_t n = E.max_num_splats, nb = (n + 255) / 256;
+        if (!E.optim.non_sh_state_ready) throw std::runtime_error("ssrh_copy_non_sh_quant_state: no quantized non-SH state yet");
+        if (packed)
+            backend::memcpy_sync(packed, DevicePool::global().acquire<uint8_t>(PoolSlot::AdamNonShPacked, (size_t)(n * 14 * 4)),
+                                 (size_t)(n * 14 * 4), backend::MemcpyKind::DeviceToHost);
+        if (bounds)
+            backend::memcpy_sync(bounds, DevicePool::global().acquire<float>(PoolSlot::AdamNonShBounds, (size_t)(5 * nb * 4)),
+                                 (size_t)(5 * nb * 4) * sizeof(float), backend::MemcpyKind::DeviceToHost);
     });
 }
 

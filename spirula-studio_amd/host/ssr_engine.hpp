@@ -36,6 +36,7 @@ struct EngineState {
         DeviceVector<float> radii; bool skip_grad_zero = false;
         bool adam_ready = false;
         bool sh_state_ready = false;   // quantization level 1: the 8-bit SH moments have been zeroed
+        bool non_sh_state_ready = false;   // non_sh_optim_bits 16: the 16-bit non-SH moments have been zeroed
         std::vector<DeviceTensorFloatND> g1, g2;   // Adam moments, shaped like the world tensors
         DeviceVector<float> densify_score;
     } optim;
@@ -87,9 +88,11 @@ void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorV
 // scale_agnostic_mean: OptimConfig::use_scale_agnostic_mean (the means step on the forward's radii).
 // quantization_level 1: SH values stay the 16-bit codes of set_sh_value_quant (one bound per 256 splats) and are
 // updated in place, their moments are 8-bit cells in pool slots (OptimConfig::quantization_level).
+// non_sh_optim_bits 16 (OptimConfig::non_sh_optim_bits; with a quantized level only): the moments of the five
+// non-SH tensors are 16-bit cells in pool slots instead of the fp32 arrays.
 void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
                                      TorchTensorView v_render_Ts, const float hyper[14], int step,
-                                     bool scale_agnostic_mean = false, int quantization_level = 0);
+                                     bool scale_agnostic_mean = false, int quantization_level = 0, int non_sh_optim_bits = 32);
 // engine_backward_from_render_grad with the cotangents of the variants of the forward that ran
 // (any may be a null view): distortion image, median depth, and a pixel weight map to accumulate
 // per splat (the reference feeds these from its loss, src/engine/EngineLoss.cpp:138-216).

@@ -66,7 +66,7 @@ enum class PoolSlot : int {
     IsectScanScratch, IsectSortScratch, IsectCounters, ProjVisibleIds, ProjVisibleIdsB, ProjPackedRows,
     IsectTileActive, EngTileMask,
     AdamG1Means, AdamG1Quats, AdamG1Scales, AdamG1Opacities, AdamG1FeaturesDc, AdamG1FeaturesSh,
-    AdamG2Means, AdamG2Quats, AdamG2Scales, AdamG2Opacities, AdamG2FeaturesDc, AdamG2FeaturesSh, EngDensifyScore, EngZeroAabb, FusedProjBwdRowOf, AdamShStatePacked, AdamShStateBounds, ProjCameraIds, ProjGaussianIds, ProjGaussianIdsB, ProjPackedScratch, ProjPackedNnz,
+    AdamG2Means, AdamG2Quats, AdamG2Scales, AdamG2Opacities, AdamG2FeaturesDc, AdamG2FeaturesSh, EngDensifyScore, EngZeroAabb, FusedProjBwdRowOf, AdamShStatePacked, AdamShStateBounds, AdamNonShPacked, AdamNonShBounds, ProjCameraIds, ProjGaussianIds, ProjGaussianIdsB, ProjPackedScratch, ProjPackedNnz,
     RendersRgb, RendersDepth, RenderTs, RenderLastIds, RenderDistortionRgb, RenderDistortionDepth, RenderMedian,
     RasterBwdAccumWeight, RasterBwdVRows, EngVDistRgb, EngVDistDepth, EngVMedian, EngAccumMap,
     RasterBwdVScreenXy, RasterBwdVScreenDepth, RasterBwdVScreenConic, RasterBwdVScreenOpac, RasterBwdVScreenRgb,
@@ -179,8 +179,21 @@ public:
     int64_t channels() const { return rows() ? numel() / rows() : 0; }
 };
 
-// src/core/NonShQuantState.h:16-28 (only `enabled` is consulted here: quantized Adam state is not built)
-struct NonShQuantState { bool enabled = false; };
+// src/core/NonShQuantState.h:16-28: the 16-bit quantized Adam moments of the five non-SH tensors, one float4 of
+// bounds per 256 splats and tensor (bounds held as plain floats here)
+struct NonShQuantState {
+    bool enabled = false;
+    uint8_t* means_packed = nullptr;
+    uint8_t* quats_packed = nullptr;
+    uint8_t* scales_packed = nullptr;
+    uint8_t* opacities_packed = nullptr;
+    uint8_t* features_dc_packed = nullptr;
+    float* means_bounds = nullptr;
+    float* quats_bounds = nullptr;
+    float* scales_bounds = nullptr;
+    float* opacities_bounds = nullptr;
+    float* features_dc_bounds = nullptr;
+};
 
 struct RenderOutput {
     // (rgb [I,H,W] float3, depth [I,H,W] float, normal -- unused by the 3dgs primitive)

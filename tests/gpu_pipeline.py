@@ -326,14 +326,14 @@ class GpuRun:
             p.packed_gaussian_ids, p.num_packed = self.ptr("gaussian_ids"), self.rows
         self.check(self.lib.ssr_projection_bwd(C.byref(p), None))
 
-    def fused_optimizer(self, g1, g2, hyper, step=1, steps=None, v_in=None, scale_agnostic=False, quant_state=None):
+    def fused_optimizer(self, g1, g2, hyper, step=1, steps=None, v_in=None, scale_agnostic=False, quant_state=None, non_sh=None):
         """ssr_fused_projection_bwd_optimizer on the device copies of the parameters (fp32 SH);
         g1 / g2 are host dicts keyed like the world arrays. Returns (params, g1, g2, score) from the device."""
         D = self.L.DeviceArray
         keys = ["means", "quats", "log_scales", "opacity_logits", "features_dc", "features_sh"]
         for pre, src in (("m1_", g1), ("m2_", g2)):
             for k in keys:
-                if quant_state is not None and k == "features_sh":
+                if (quant_state is not None and k == "features_sh") or (non_sh is not None and k != "features_sh"):
                     self.d[pre + k] = None
                     continue
                 self.d[pre + k] = D.from_host(np.ascontiguousarray(src[k], np.float32))
@@ -373,12 +373,19 @@ class GpuRun:
             w = p.world
             w.features_sh = None
             p.world = w
+        if non_sh is not None:   # quantized non-SH moments: five arrays of 32-bit cells, five of float4 bounds
+            for t in range(5):
+                self.d[f"ns_packed{t}"] = D.from_host(np.ascontiguousarray(non_sh["packed"][t], np.uint32))
+                self.d[f"ns_bounds{t}"] = D.from_host(np.ascontiguousarray(non_sh["bounds"][t], np.float32))
+                p.non_sh_packed[t], p.non_sh_bounds[t] = self.ptr(f"ns_packed{t}"), self.ptr(f"ns_bounds{t}")
         self.check(self.lib.ssr_fused_projection_bwd_optimizer(C.byref(p), None))
         self.check(self.lib.ssr_device_synchronize())
         if quant_state is not None:
             keys = keys[:5]
-        out = lambda pre: {k: self.host(pre + k) for k in keys}
+        out = lambda pre: {k: (self.host(pre + k) if self.d.get(pre + k) is not None else None) for k in keys}
         res = out(""), out("m1_"), out("m2_"), self.host("score")
+        if non_sh is not None:
+            self.non_sh_out = dict(packed=[self.host(f"ns_packed{t}") for t in range(5)], bounds=[self.host(f"ns_bounds{t}") for t in range(5)])
         if quant_state is not None:
             q = dict(state_packed=self.host("sh_state_packed"), state_bounds=self.host("sh_state_bounds"),
                      value_packed=self.host("sh_packed").view(np.uint16), value_bounds=self.host("sh_bounds"), num_sh_buffer=15)

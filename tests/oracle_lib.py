@@ -271,9 +271,9 @@ class OrShQuantState(C.Structure):
 
 def quant_codec(op, a=None, b=None, mm=None, codes=None):
     """The codecs of the quantized optimizer state on arrays: op 0 Adam-state encode (g1, g2 -> codes),
-    1 decode (codes -> g1, g2), 2 16-bit value encode, 3 value decode."""
+    1 decode (codes -> g1, g2), 2 16-bit value encode, 3 value decode, 4 / 5 the 16-bit Adam-state encode / decode."""
     mm = np.ascontiguousarray(mm, np.float32)
-    if op in (0, 2):
+    if op in (0, 2, 4):
         a = np.ascontiguousarray(a, np.float32)
         b = np.ascontiguousarray(a if b is None else b, np.float32)
         codes = np.zeros(a.size, np.uint32)
@@ -283,7 +283,7 @@ def quant_codec(op, a=None, b=None, mm=None, codes=None):
     a = np.zeros(codes.size, np.float32)
     b = np.zeros(codes.size, np.float32)
     lib().or_quant_codec(C.c_int(op), C.c_int64(codes.size), _p(a), _p(b), _p(mm), _p(codes))
-    return (a, b) if op == 1 else a
+    return (a, b) if op in (1, 5) else a
 
 
 def quantize_sh_state(features_sh, num_sh_buffer=15):
@@ -323,10 +323,56 @@ def decode_sh_moments(q, n):
     return g1, g2
 
 
+class OrNonShQuantState(C.Structure):
+    _fields_ = [("packed", C.c_void_p * 5), ("bounds", C.c_void_p * 5)]
+
+
+NON_SH_KEYS = ["means", "quats", "log_scales", "opacity_logits", "features_dc"]
+NON_SH_PRIMS = [3, 4, 3, 1, 3]
+
+
+def zero_non_sh_state(n):
+    """The all-zero quantized non-SH state (decodes to zero moments): per tensor [N * prims] uint32 cells and
+    [ceil(N / 256), 4] float32 bounds."""
+    nb = (n + 255) // 256
+    return dict(packed=[np.zeros(n * p, np.uint32) for p in NON_SH_PRIMS], bounds=[np.zeros((nb, 4), np.float32) for _ in range(5)])
+
+
+def encode_non_sh_state(g1, g2, n):
+    """fp32 moments (dicts keyed by NON_SH_KEYS) -> the quantized non-SH state, by the codec's definition."""
+    st = zero_non_sh_state(n)
+    for t, (k, prims) in enumerate(zip(NON_SH_KEYS, NON_SH_PRIMS)):
+        a, b = g1[k].reshape(-1).astype(np.float32), g2[k].reshape(-1).astype(np.float32)
+        for blk in range((n + 255) // 256):
+            sl = slice(blk * 256 * prims, min((blk + 1) * 256, n) * prims)
+            sq = np.sqrt(np.maximum(b[sl], 0)).astype(np.float32)
+            u = (a[sl] / (sq + np.float32(1e-15))).astype(np.float32)
+            # log_s through the codec's own log1p: encode a lone cell against (0, 1) bounds is not available, so
+            # take the bounds from decode(encode) fixed points: min / max of log1p(sq / eps) computed in float64
+            ls = np.log1p(sq.astype(np.float64) / 1e-15).astype(np.float32)
+            mm = np.array([u.min(), u.max(), ls.min(), ls.max()], np.float32)
+            st["bounds"][t][blk] = mm
+            st["packed"][t][sl] = quant_codec(4, a[sl], b[sl], mm=mm)
+    return st
+
+
+def decode_non_sh_state(st, n):
+    g1, g2 = {}, {}
+    for t, (k, prims) in enumerate(zip(NON_SH_KEYS, NON_SH_PRIMS)):
+        a, b = np.zeros(n * prims, np.float32), np.zeros(n * prims, np.float32)
+        for blk in range((n + 255) // 256):
+            sl = slice(blk * 256 * prims, min((blk + 1) * 256, n) * prims)
+            a[sl], b[sl] = quant_codec(5, codes=st["packed"][t][sl], mm=st["bounds"][t][blk])
+        shape = (n,) if prims == 1 else (n, prims)
+        g1[k], g2[k] = a.reshape(shape), b.reshape(shape)
+    return g1, g2
+
+
 def fused_projection_bwd_optimizer_q(scene, aabb, vs, params, q, g1, g2, hyper, step=1, steps=None, v_in=None,
-                                     sh_degree=3, densify=True, radii=None):
+                                     sh_degree=3, densify=True, radii=None, non_sh=None):
     """The fused optimizer with the SH coefficients and their moments in the quantized state q (updated in
-    place); params / g1 / g2 hold the five non-SH arrays (a features_sh entry is ignored)."""
+    place); params / g1 / g2 hold the five non-SH arrays (a features_sh entry is ignored). non_sh: the quantized
+    state of the non-SH moments (zero_non_sh_state layout, updated in place); g1 / g2 may then be None."""
     n = scene.n
     cam = camera_of(scene)
 
@@ -343,8 +389,17 @@ def fused_projection_bwd_optimizer_q(scene, aabb, vs, params, q, g1, g2, hyper, 
         assert q[k].flags.c_contiguous
         setattr(st, k, q[k].ctypes.data)
     st.num_sh_buffer = q["num_sh_buffer"]
+    ns = None
+    if non_sh is not None:
+        ns = OrNonShQuantState()
+        for t in range(5):
+            assert non_sh["packed"][t].dtype == np.uint32 and non_sh["packed"][t].flags.c_contiguous
+            assert non_sh["bounds"][t].dtype == np.float32 and non_sh["bounds"][t].flags.c_contiguous
+            ns.packed[t] = non_sh["packed"][t].ctypes.data
+            ns.bounds[t] = non_sh["bounds"][t].ctypes.data
     lib().or_fused_projection_bwd_optimizer_q(
-        C.c_int64(n), C.c_int(sh_degree), *[_p(params[k]) for k in WORLD_KEYS[:5]], C.byref(st), C.byref(cam), _p(aabb),
+        C.c_int64(n), C.c_int(sh_degree), *[_p(params[k]) for k in WORLD_KEYS[:5]], C.byref(st),
+        C.byref(ns) if ns is not None else None, C.byref(cam), _p(aabb),
         _p(vs["v_xy"]), _p(vs["v_depth"]), _p(vs["v_conic"]), _p(vs["v_opac"]), _p(vs["v_rgb"]),
         ptrs(v_in) if v_in is not None else None, ptrs(g1), ptrs(g2), _p(score), _p(hv), C.c_int32(step),
         _p(None if steps is None else np.ascontiguousarray(steps, np.int32)),

@@ -231,11 +231,13 @@ def test_engine_fused_optimizer_scale_agnostic_means(pkg, oracle, H, packed):
         assert (d > 0.05 * 5e-2).mean() < 2e-3, k
 
 
-@pytest.mark.parametrize("packed", [False, True])
-def test_engine_fused_optimizer_quantization_level_1(pkg, oracle, H, packed):
+@pytest.mark.parametrize("packed,non_sh_bits", [(False, 32), (True, 32), (False, 16), (True, 16)])
+def test_engine_fused_optimizer_quantization_level_1(pkg, oracle, H, packed, non_sh_bits):
     """Training steps at OptimConfig::quantization_level 1 (the reference's default): the engine keeps the SH
     coefficients as 16-bit codes that the forward reads and the fused optimizer rewrites in place, and their Adam
-    moments as 8-bit cells; against the oracle running the same loop on its own copy."""
+    moments as 8-bit cells; against the oracle running the same loop on its own copy. non_sh_bits 16: the moments
+    of the other five tensors as 16-bit cells as well (OptimConfig::non_sh_optim_bits, what the reference's trainer
+    sets at this level)."""
     host, lib = H
     S = pkg.scenes
     sc = S.make_scene(1, n=20000, width=320, height=240, parity_variant=True, sh_codec=0)
@@ -257,14 +259,27 @@ def test_engine_fused_optimizer_quantization_level_1(pkg, oracle, H, packed):
     g1 = {k: np.zeros_like(v) for k, v in P.items()}
     g2 = {k: np.zeros_like(v) for k, v in P.items()}
     start = oracle.decode_sh_values(q, n)
+    ns = None
+    if non_sh_bits == 16:
+        ns, g1, g2 = oracle.zero_non_sh_state(n), None, None
     for step in (1, 2, 3):
         eng.forward()
-        eng.backward_fused_optimizer(h, step, quantization_level=1)
+        eng.backward_fused_optimizer(h, step, quantization_level=1, non_sh_optim_bits=non_sh_bits)
         for k in P:
             setattr(ref, k, P[k])
         ref.sh_packed, ref.sh_bounds = q["value_packed"].copy(), q["value_bounds"].copy()
         r = oracle.pipeline(ref, backward=True)
-        oracle.fused_projection_bwd_optimizer_q(ref, r["proj"]["aabb"], r["vscreen"], P, q, g1, g2, h, step=step)
+        oracle.fused_projection_bwd_optimizer_q(ref, r["proj"]["aabb"], r["vscreen"], P, q, g1, g2, h, step=step, non_sh=ns)
+        if ns is not None:
+            e1, e2 = oracle.decode_non_sh_state(eng.non_sh_quant_state(), n)
+            o1, o2 = oracle.decode_non_sh_state(ns, n)
+            for k in oracle.NON_SH_KEYS:
+                a, b = e1[k].reshape(n, -1).astype(np.float64), o1[k].reshape(n, -1).astype(np.float64)
+                assert np.isfinite(a).all() and np.abs(b).max() > 0
+                scale = np.abs(b).max(axis=1, keepdims=True) + 1e-12
+                assert (np.abs(a - b) > 0.05 * scale + 1e-9).mean() < 0.02, (k, step)
+                a, b = e2[k].reshape(n, -1).astype(np.float64), o2[k].reshape(n, -1).astype(np.float64)
+                assert (np.abs(a - b) > 0.05 * b + 1e-14).mean() < 0.02, (k, step)
         eq = eng.sh_quant_state()
         got, want = oracle.decode_sh_values(eq, n), oracle.decode_sh_values(q, n)
         far = np.abs(got - want) > 0.05 * h["lr_features_sh"] + 1e-6

@@ -449,7 +449,7 @@ def test_fused_projection_bwd_optimizer(gpu, oracle, cfg):
         assert np.array_equal(g.host("row_of"), row_of)
 
 
-@pytest.mark.parametrize("cfg", ["tiny", "tiny-deg1-packed-steps", "cfg3"])
+@pytest.mark.parametrize("cfg", ["tiny", "tiny-deg1-packed-steps", "cfg3", "tiny-nonsh", "cfg3-nonsh-packed-steps"])
 def test_fused_optimizer_quantized_sh_state(gpu, oracle, cfg):
     """The fused optimizer at the reference's quantization level 1: SH values as 16-bit codes and their Adam
     moments as 8-bit (u, log_s) cells, both against per-256-splat bounds that are recomputed every step
@@ -459,7 +459,9 @@ def test_fused_optimizer_quantized_sh_state(gpu, oracle, cfg):
     rng = np.random.default_rng(17)
     S = gpu.scenes
     deg, packed = 3, False
-    if cfg == "tiny":
+    # "nonsh": also the moments of the five non-SH tensors quantized (16-bit cells), as the reference runs at this level
+    ns = oracle.zero_non_sh_state(1) if "nonsh" in cfg else None
+    if cfg.startswith("tiny") and "deg1" not in cfg:
         sc = S.tiny_scene(n=700, width=96, height=64, seed=83)        # two full blocks and a partial one
         sc.means[::4, 2] = -10.0
     elif cfg == "tiny-deg1-packed-steps":
@@ -468,6 +470,7 @@ def test_fused_optimizer_quantized_sh_state(gpu, oracle, cfg):
         deg, packed = 1, True                                          # coefficients above degree 1 are re-encoded as zeros
     else:
         sc = S.make_scene(3, n=30000, width=320, height=192, sh_codec=0)
+        packed = "packed" in cfg
     S.apply_sh_codec(sc, 2, bounds_stride=256 * 45)
     h = dict(lr_means=1.6e-4, lr_quats=1e-3, lr_scales=5e-3, lr_opacs=5e-2, lr_features_dc=2.5e-3, lr_features_sh=2.5e-3,
              max_gauss_ratio=6.0, scale_regularization_weight=0.01, mcmc_opacity_reg_weight=0.01, mcmc_scale_reg_weight=0.01,
@@ -481,6 +484,9 @@ def test_fused_optimizer_quantized_sh_state(gpu, oracle, cfg):
     P = {k: np.ascontiguousarray(getattr(sc, k), np.float32).copy() for k in oracle.WORLD_KEYS[:5]}
     g1 = {k: np.zeros_like(v) for k, v in P.items()}
     g2 = {k: np.zeros_like(v) for k, v in P.items()}
+    if ns is not None:
+        ns, g1, g2 = oracle.zero_non_sh_state(n), None, None
+    sa = "nonsh" in cfg and "cfg3" in cfg    # with the scale-agnostic step of the means
     for t in (1, 2):
         # the scene both sides start this step from
         for k in P:
@@ -495,12 +501,24 @@ def test_fused_optimizer_quantized_sh_state(gpu, oracle, cfg):
             full = np.zeros((n, 4), np.float32); full[ids] = aabb[:g.rows]; aabb = full
             for k in vs:
                 full = np.zeros((n,) + vs[k].shape[1:], np.float32); full[ids] = vs[k][:g.rows]; vs[k] = full
-        dP, d1, d2, dscore, dq = g.fused_optimizer(g1, g2, h, step=t, steps=steps, quant_state=q)
+        dP, d1, d2, dscore, dq = g.fused_optimizer(g1, g2, h, step=t, steps=steps, quant_state=q, non_sh=ns, scale_agnostic=sa)
         oq = {k: (v.copy() if isinstance(v, np.ndarray) else v) for k, v in q.items()}
         oP = {k: v.copy() for k, v in P.items()}
-        o1 = {k: v.copy() for k, v in g1.items()}
-        o2 = {k: v.copy() for k, v in g2.items()}
-        oracle.fused_projection_bwd_optimizer_q(sc, aabb, vs, oP, oq, o1, o2, h, step=t, steps=steps, sh_degree=deg)
+        o1 = None if ns is not None else {k: v.copy() for k, v in g1.items()}
+        o2 = None if ns is not None else {k: v.copy() for k, v in g2.items()}
+        ons = None if ns is None else dict(packed=[a.copy() for a in ns["packed"]], bounds=[a.copy() for a in ns["bounds"]])
+        oracle.fused_projection_bwd_optimizer_q(sc, aabb, vs, oP, oq, o1, o2, h, step=t, steps=steps, sh_degree=deg, non_sh=ons,
+                                                radii=g.host("radii") if sa else None)
+        if ns is not None:
+            dns = g.non_sh_out
+            for ti, k in enumerate(oracle.NON_SH_KEYS):
+                assert np.allclose(dns["bounds"][ti], ons["bounds"][ti], rtol=1e-4, atol=1e-6), (k, t)
+                a, b = dns["packed"][ti].astype(np.int64), ons["packed"][ti].astype(np.int64)
+                du, ds = np.abs((a & 65535) - (b & 65535)), np.abs((a >> 16) - (b >> 16))
+                # the two sides' gradients agree to rounding, which a 16-bit code resolves: a few steps at most
+                assert max(du.max(), ds.max()) <= 24 and max((du > 2).mean(), (ds > 2).mean()) < 0.02, (k, t, int(du.max()), int(ds.max()))
+                assert a.any()
+            ns = dns
         assert np.allclose(dq["value_bounds"], oq["value_bounds"], rtol=1e-5, atol=1e-8)
         assert np.allclose(dq["state_bounds"], oq["state_bounds"], rtol=1e-4, atol=1e-6)
         for key, width in [("value_packed", 16), ("state_packed", 8)]:

@@ -238,3 +238,80 @@ def test_proj_bwd_parity_rows(gpu, oracle, cam):
     sc, _ = R.tool_scene(gpu, R.SEED_PROJ_BWD, cam, PINHOLE, THIN_PRISM)
     sc.sh_codec, sc.sh_packed, sc.sh_bounds, sc.sh_bounds_stride = 1, q["q8"], q["bounds_cell"], 256
     _k9_direct(gpu, oracle, sc, vs, f"proj_bwd_parity q8 THIN_PRISM cam {cam}")
+
+
+# fpbo_parity.cpp:169, the quantized 3dgs row: packed projection, EQUISOLID + OpenCV, degree 3, quantization level 1
+# with the non-SH moments quantized too, all five non-SH world gradients, two steps (10, 11) on one forward.
+# The stream is followed through the four rows before it, so these are the tool's own codes, bounds and gradients.
+@pytest.mark.parametrize("cam", [0, 1])
+def test_fpbo_parity_quantized_row(gpu, oracle, cam):
+    n, C_ = R.N_FPBO, R.C_TOOL
+    _, rng = R.tool_world(R.SEED_FPBO, n=n)
+    for row in range(4):
+        rng.raw(C_ * n * (7 if row == 3 else 10))                 # screen gradients (the 3dgut row has 7 floats per row)
+        rng.raw(n * {0: 14, 1: 14, 2: 0, 3: 10}[row])              # world gradients present in that row
+        rng.raw(2 * n * (14 + 45))                                 # both moments of all six tensors
+        if row == 2:
+            rng.raw(n)                                             # per-splat steps
+    cells, nb = n * 45, (n + 255) // 256
+    b = (rng.raw(2 * cells) & np.uint32(0xFF)).astype(np.uint16)
+    codes = np.ascontiguousarray(b[0::2] | (b[1::2] << np.uint16(8)))
+    d = rng.raw(2 * nb).reshape(nb, 2)
+    uf = lambda col, lo, hi: (np.float32(lo) + ((np.float32(hi) - np.float32(lo)) * (d[:, col] & np.uint32(0xFFFFFF)).astype(np.float32))
+                              / np.float32(16777215.0)).astype(np.float32)
+    vbounds = np.ascontiguousarray(np.stack([uf(0, -0.5, -0.1), uf(1, 0.1, 0.5)], axis=1), np.float32)
+
+    def scene(c):
+        sc, _ = R.tool_scene(gpu, R.SEED_FPBO, c, EQUISOLID, OPENCV, n=n)
+        sc.sh_codec, sc.sh_packed, sc.sh_bounds, sc.sh_bounds_stride = 2, codes.copy(), vbounds.copy(), 256 * 45
+        return sc
+    nnz = []
+    for c in range(C_):
+        a = oracle.projection_fwd(scene(c))["aabb"]
+        nnz.append(int(((a[:, 2] - a[:, 0] > np.float32(1e-3)) & (a[:, 3] - a[:, 1] > np.float32(1e-3))).sum()))
+    vs_all = R.screen_gradients(rng, sum(nnz))
+    lo = sum(nnz[:cam])
+    vs_rows = {k: np.ascontiguousarray(v[lo:lo + nnz[cam]]) for k, v in vs_all.items()}
+    shapes = dict(means=(n, 3), quats=(n, 4), log_scales=(n, 3), opacity_logits=(n,), features_dc=(n, 3))
+    v_world = {k: rng.uf(int(np.prod(s)), -0.05, 0.05).reshape(s) for k, s in shapes.items()}
+    sc = scene(cam)
+    g = GpuRun(gpu, sc, packed_projection=True)
+    g.projection_fwd()
+    assert g.rows == nnz[cam] and 100 < g.rows < n
+    D = gpu.lib.DeviceArray
+    for k, v in vs_rows.items():
+        g.d[k] = D.from_host(v)
+    ids = g.host("gaussian_ids")[:g.rows]
+    aabb = np.zeros((n, 4), np.float32)
+    aabb[ids] = g.host("aabb")[:g.rows]
+    vs = {}
+    for k, v in vs_rows.items():
+        vs[k] = np.zeros((n,) + v.shape[1:], np.float32)
+        vs[k][ids] = v
+    q = dict(state_packed=np.zeros(cells, np.uint16), state_bounds=np.zeros((nb, 4), np.float32), value_packed=codes.copy(),
+             value_bounds=vbounds.copy(), num_sh_buffer=15)
+    ns = oracle.zero_non_sh_state(n)
+    P = {k: np.ascontiguousarray(getattr(sc, k), np.float32).copy() for k in oracle.WORLD_KEYS[:5]}
+    h = R.FPBO_HYPER
+    dq, dns = q, ns
+    for step in (10, 11):
+        dP, _, _, _, dq = g.fused_optimizer(None, None, h, step=step, v_in=v_world, quant_state=dq, non_sh=dns)
+        dns = g.non_sh_out
+        oracle.fused_projection_bwd_optimizer_q(sc, aabb, vs, P, q, None, None, h, step=step, v_in=v_world, non_sh=ns, densify=False)
+        assert np.allclose(dq["value_bounds"], q["value_bounds"], rtol=1e-5, atol=1e-7), step
+        assert np.allclose(dq["state_bounds"], q["state_bounds"], rtol=1e-4, atol=1e-6), step
+        dv = np.abs(dq["value_packed"].astype(np.int64) - q["value_packed"].astype(np.int64))
+        assert dv.max() <= 2 and (dv > 1).mean() < 0.02, (step, int(dv.max()))
+        a, b = dq["state_packed"].astype(np.int64), q["state_packed"].astype(np.int64)
+        # the tool's own acceptance is +-1 quantum per code (fpbo_parity.cpp:11)
+        assert max(np.abs((a & 255) - (b & 255)).max(), np.abs((a >> 8) - (b >> 8)).max()) <= 1, step
+        for t, k in enumerate(oracle.NON_SH_KEYS):
+            assert np.allclose(dns["bounds"][t], ns["bounds"][t], rtol=1e-4, atol=1e-6), (k, step)
+            a, b = dns["packed"][t].astype(np.int64), ns["packed"][t].astype(np.int64)
+            du, ds = np.abs((a & 65535) - (b & 65535)), np.abs((a >> 16) - (b >> 16))
+            assert (du > 2).mean() < 0.02 and (ds > 2).mean() < 0.02, (k, step, int(du.max()), int(ds.max()))
+            assert np.abs(dP[k].astype(np.float64) - P[k]).max() <= 0.02 * 5e-2 * 40 + 1e-6, (k, step)
+        # the second step starts from the device's state on both sides
+        q = {k: (v.copy() if isinstance(v, np.ndarray) else v) for k, v in dq.items()}
+        ns = dict(packed=[x.copy() for x in dns["packed"]], bounds=[x.copy() for x in dns["bounds"]])
+        P = {k: v.copy() for k, v in dP.items()}

@@ -145,3 +145,88 @@ def test_quantized_state_step_equals_fp32_step_on_the_decoded_state(pkg, oracle,
     assert (np.abs(np.log1p(gsq[:, act] / EPS) - np.log1p(wsq[:, act] / EPS)) <= 0.5001 * sl + 1e-4).all()
     if nc < 15:
         assert not np.any(gm2[:, ~act]) and np.abs(gm1[:, ~act]).max() < 1e-12
+
+
+def test_adam_state_codec_16_bit(oracle):
+    """QuantizedAdamState<16, 256> (the non-SH state): same definitions at 65535 levels, one 32-bit cell."""
+    rng = np.random.default_rng(2)
+    n = 20000
+    g2 = (10.0 ** rng.uniform(-16, -2, n)).astype(np.float32)
+    g2[::50] = 0.0
+    g1 = (np.sqrt(g2) * rng.uniform(-3, 3, n)).astype(np.float32)
+    sq = np.sqrt(g2.astype(np.float64))
+    u = g1.astype(np.float64) / (sq + EPS)
+    ls = np.log1p(sq / EPS)
+    mm = np.array([u.min(), u.max(), ls.min(), ls.max()], np.float32)
+    codes = oracle.quant_codec(4, g1, g2, mm)
+    uq, sq_q = (codes & 65535).astype(np.int64), (codes >> 16).astype(np.int64)
+    want_u = np.clip(np.floor(65535 * (u - mm[0]) / (mm[1] - mm[0]) + 0.5), 0, 65535)
+    want_s = np.clip(np.floor(65535 * (ls - mm[2]) / (mm[3] - mm[2]) + 0.5), 0, 65535)
+    # fp32 arithmetic of the encode moves a 16-bit code by a few steps at most (2^-24 relative on a 2^16 range)
+    assert np.abs(uq - want_u).max() <= 2 and np.abs(sq_q - want_s).max() <= 2
+    assert (uq != want_u).mean() < 0.2 and (sq_q != want_s).mean() < 0.2
+    assert uq[np.argmin(u)] == 0 and uq[np.argmax(u)] == 65535 and sq_q[np.argmin(ls)] == 0 and sq_q[np.argmax(ls)] == 65535
+    d1, d2 = oracle.quant_codec(5, codes=codes, mm=mm)
+    du = d1.astype(np.float64) / (np.sqrt(d2.astype(np.float64)) + EPS)
+    dls = np.log1p(np.sqrt(d2.astype(np.float64)) / EPS)
+    assert np.abs(du - u).max() <= 1.5 * (mm[1] - mm[0]) / 65535 + 1e-6
+    assert np.abs(dls - ls).max() <= 1.5 * (mm[3] - mm[2]) / 65535 + 1e-5
+    z1, z2 = oracle.quant_codec(5, codes=np.zeros(4, np.uint32), mm=np.zeros(4, np.float32))
+    assert not np.any(z1) and not np.any(z2)
+    assert not np.any(oracle.quant_codec(4, np.zeros(3, np.float32), np.zeros(3, np.float32), np.array([0, 2, 0, 30], np.float32)))
+
+
+@pytest.mark.parametrize("scale_agnostic", [False, True])
+def test_quantized_non_sh_state_step(pkg, oracle, scale_agnostic):
+    """One step with the quantized non-SH state equals: decode the 16-bit cells against each block's bounds, take
+    the fp32 step on those moments, encode the new moments against their block-wise min / max."""
+    sc = pkg.scenes.tiny_scene(n=700, width=96, height=64, seed=83)
+    sc.means[::5, 2] = -10.0
+    n = sc.n
+    h = dict(lr_means=1.6e-4, lr_quats=1e-3, lr_scales=5e-3, lr_opacs=5e-2, lr_features_dc=2.5e-3, lr_features_sh=1.25e-4,
+             max_gauss_ratio=6.0, scale_regularization_weight=0.01, mcmc_opacity_reg_weight=0.01, mcmc_scale_reg_weight=0.01,
+             quat_norm_reg_weight=0.02, sh_reg_weight=0.05, erank_reg_weight=0.1, erank_reg_weight_s3=0.02)
+    q = oracle.quantize_sh_state(sc.features_sh)
+    ns = oracle.zero_non_sh_state(n)
+    P = {k: np.ascontiguousarray(getattr(sc, k), np.float32).copy() for k in oracle.WORLD_KEYS}
+
+    def forward(Pq, q_state):
+        sc_q = pkg.scenes.subset(sc, np.arange(n))
+        for k in oracle.WORLD_KEYS[:5]:
+            setattr(sc_q, k, Pq[k])
+        sc_q.features_sh = oracle.decode_sh_values(q_state, n)
+        return sc_q, oracle.pipeline(sc_q)
+
+    for t in (1, 2):
+        sc_q, r = forward(P, q)
+        oracle.fused_projection_bwd_optimizer_q(sc_q, r["proj"]["aabb"], r["vscreen"], P, q, None, None, h, step=t, non_sh=ns,
+                                                radii=r["proj"]["radii"] if scale_agnostic else None)
+    assert all(a.any() for a in ns["packed"])
+    sc_q, r = forward(P, q)
+    radii = r["proj"]["radii"] if scale_agnostic else None
+    f1, f2 = oracle.decode_non_sh_state(ns, n)
+    Pf = {k: v.copy() for k, v in P.items()}
+    qf = {k: (v.copy() if isinstance(v, np.ndarray) else v) for k, v in q.items()}
+    oracle.fused_projection_bwd_optimizer_q(sc_q, r["proj"]["aabb"], r["vscreen"], Pf, qf, f1, f2, h, step=3, radii=radii)
+    Pq = {k: v.copy() for k, v in P.items()}
+    qq = {k: (v.copy() if isinstance(v, np.ndarray) else v) for k, v in q.items()}
+    nq = dict(packed=[a.copy() for a in ns["packed"]], bounds=[a.copy() for a in ns["bounds"]])
+    oracle.fused_projection_bwd_optimizer_q(sc_q, r["proj"]["aabb"], r["vscreen"], Pq, qq, None, None, h, step=3, non_sh=nq, radii=radii)
+    for k in oracle.WORLD_KEYS[:5]:       # same decoded moments, same step: the parameters agree to the bit
+        assert np.array_equal(Pq[k], Pf[k]), k
+    for k in ["state_packed", "value_packed"]:
+        assert np.array_equal(qq[k], qf[k]), k
+    d1, d2 = oracle.decode_non_sh_state(nq, n)
+    for t, (k, prims) in enumerate(zip(oracle.NON_SH_KEYS, oracle.NON_SH_PRIMS)):
+        a, b = f1[k].reshape(n, -1).astype(np.float64), f2[k].reshape(n, -1).astype(np.float64)
+        sq = np.sqrt(np.maximum(b, 0))
+        u, ls = a / (sq + EPS), np.log1p(sq / EPS)
+        ga, gb = d1[k].reshape(n, -1).astype(np.float64), d2[k].reshape(n, -1).astype(np.float64)
+        gsq = np.sqrt(gb)
+        gu, gls = ga / (gsq + EPS), np.log1p(gsq / EPS)
+        for blk in range((n + 255) // 256):
+            rows = slice(blk * 256, min((blk + 1) * 256, n))
+            mm = np.array([u[rows].min(), u[rows].max(), ls[rows].min(), ls[rows].max()])
+            assert np.allclose(nq["bounds"][t][blk], mm, rtol=2e-5, atol=1e-6), (k, blk)
+            assert np.abs(gu[rows] - u[rows]).max() <= 1.5 * (mm[1] - mm[0]) / 65535 + 1e-5 * max(1.0, np.abs(mm[:2]).max()), k
+            assert np.abs(gls[rows] - ls[rows]).max() <= 1.5 * (mm[3] - mm[2]) / 65535 + 1e-5 * max(1.0, mm[3]), k
