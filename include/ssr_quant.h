@@ -5,6 +5,8 @@
 // 16-bit halves of a word), the linearly quantized u = g1 / (sqrt(g2) + eps) and
 // log_s = log1p(sqrt(g2) / eps), against per-block bounds (u_min, u_max, log_s_min, log_s_max). QuantizedTensor<16, 256> (src/core/Tensor.h:1300-1405): one
 // 16-bit linear code per cell against per-block (min, max). Both are endpoint-exact and keep 0 <-> 0.
+// The encoders multiply by levels / range (the reference divides, under fast-math): codes can differ from a
+// correctly rounded quotient at a rounding tie only.
 //
 // log1p / expm1 are built on ssr_log / ssr_exp (the reference calls the CUDA math library), so codes can
 // differ from the reference's by one step where its log1pf rounds differently; here host and device
@@ -18,7 +20,9 @@
 SSR_HD float ssr_log1p(float x) {   // x >= 0
     const float u = 1.0f + x;
     if (u == 1.0f) return x;
-    return ssr_log(u) * (x / (u - 1.0f));
+    const float um1 = u - 1.0f;
+    if (um1 == x) return ssr_log(u);   // the correction factor x / (u - 1) is exactly 1 (always so from 2^25 on)
+    return ssr_log(u) * (x / um1);
 }
 SSR_HD float ssr_expm1(float y) {
     const float u = ssr_exp(y);
@@ -44,9 +48,10 @@ SSR_HD void ssr_adamq_to_us(float g1, float g2, float* u, float* log_s) {
 SSR_HD void ssr_adamq_codes(float g1, float g2, const float mm[4], float qmax, uint32_t* u_q, uint32_t* s_q) {
     float u, ls;
     ssr_adamq_to_us(g1, g2, &u, &ls);
-    const float ur = ssr_max(mm[1] - mm[0], SSR_ADAMQ_EPS), sr = ssr_max(mm[3] - mm[2], SSR_ADAMQ_EPS);
-    *u_q = (uint32_t)ssr_min(ssr_max(ssr_round_code((qmax * (u - mm[0])) / ur), 0.0f), qmax);
-    *s_q = (uint32_t)ssr_min(ssr_max(ssr_round_code((qmax * (ls - mm[2])) / sr), 0.0f), qmax);
+    // codes per unit of u / log_s: depends on the bounds alone, so a loop over a block's cells divides once
+    const float ku = qmax / ssr_max(mm[1] - mm[0], SSR_ADAMQ_EPS), ks = qmax / ssr_max(mm[3] - mm[2], SSR_ADAMQ_EPS);
+    *u_q = (uint32_t)ssr_min(ssr_max(ssr_round_code((u - mm[0]) * ku), 0.0f), qmax);
+    *s_q = (uint32_t)ssr_min(ssr_max(ssr_round_code((ls - mm[2]) * ks), 0.0f), qmax);
 }
 SSR_HD uint32_t ssr_adamq_encode(float g1, float g2, const float mm[4]) {     // 8-bit cell: encode_g1g2_code
     uint32_t uq, sq;
@@ -85,8 +90,8 @@ SSR_HD void ssr_adamq16_decode(uint32_t code, const float mm[4], float* g1, floa
 
 // QuantizedTensor<16>::encode_v_code / decode_v against bounds (lo, hi)
 SSR_HD uint32_t ssr_q16_encode(float v, float lo, float hi) {
-    const float range = ssr_max(hi - lo, 1e-30f);
-    return (uint32_t)ssr_min(ssr_max(ssr_round_code((65535.0f * (v - lo)) / range), 0.0f), 65535.0f);
+    const float k = 65535.0f / ssr_max(hi - lo, 1e-30f);
+    return (uint32_t)ssr_min(ssr_max(ssr_round_code((v - lo) * k), 0.0f), 65535.0f);
 }
 SSR_HD float ssr_q16_decode(uint32_t code, float lo, float hi) {
     return lo + (hi - lo) * ((float)code * (1.0f / 65535.0f));

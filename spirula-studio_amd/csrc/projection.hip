@@ -933,9 +933,11 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
                     float m1, m2, xn, u, ls;
                     step_cell(sp, k, m1, m2, xn);
                     ssr_adamq_to_us(m1, m2, &u, &ls);
-                    mn[0] = ssr_min(mn[0], u); mx[0] = ssr_max(mx[0], u);
-                    mn[1] = ssr_min(mn[1], ls); mx[1] = ssr_max(mx[1], ls);
-                    mn[2] = ssr_min(mn[2], xn); mx[2] = ssr_max(mx[2], xn);
+                    // the running bounds are never NaN (a NaN candidate loses every comparison), so the plain
+                    // comparisons give what ssr_min / ssr_max give
+                    mn[0] = (u < mn[0]) ? u : mn[0]; mx[0] = (u > mx[0]) ? u : mx[0];
+                    mn[1] = (ls < mn[1]) ? ls : mn[1]; mx[1] = (ls > mx[1]) ? ls : mx[1];
+                    mn[2] = (xn < mn[2]) ? xn : mn[2]; mx[2] = (xn > mx[2]) ? xn : mx[2];
                 }
                 sp += dsp; k += dk;
                 if (k >= R) { k -= R; sp++; }
