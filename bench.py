@@ -232,10 +232,13 @@ def main():
     dom = max(acc, key=acc.get)
     dom_gbs = ab[dom] / (acc[dom] * 1e-3) / 1e9 if acc[dom] > 0 else 0.0
     traffic = None
+    valu_inst = None     # profiled VALU wavefront instructions per launch of the dominant kernel (plain path only)
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(tpath):
         try:
             traffic = json.load(open(tpath)).get(f"config{cfg}", {}).get(dom)
+            if native and not (variants or args.fused_optimizer or args.packed_projection or args.lens != "none" or args.fisheye):
+                valu_inst = json.load(open(tpath)).get(f"config{cfg}_valu_wave_instructions", {}).get(dom)
         except Exception:
             traffic = None
 
@@ -268,6 +271,11 @@ def main():
                      "frac": dom_gbs / HBM_PEAK_GBS, "traffic": traffic,
                      "algorithmic_bytes_per_launch": ab[dom], "avg_launch_ms": acc[dom]},
     }
+    if valu_inst:
+        # the dominant kernel is bound by vector-instruction issue, which neither "hbm" nor "mfma" names: a wavefront
+        # instruction holds one of the chip's 1024 SIMDs for 4 cycles; share of the measured duration at 2.4 GHz
+        out["roofline"]["valu_issue"] = {"wave_instructions_per_launch": valu_inst,
+                                         "frac_of_issue_slots": valu_inst * 4 / 1024 / (acc[dom] * 1e-3 * 2.4e9)}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(pkg, cfg)
     print(json.dumps(out))
