@@ -280,7 +280,7 @@ typedef struct {
 int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t stream);
 
 /* ---- K9: projection_3dgs_backward (src/kernels/projection/ProjectionBwd.cuh:18-46, kernel
- * src/kernels/projection/ProjectionBwd_kernel.cuh:16-130), v_viewmats = NULL. accumulate != 0:
+ * src/kernels/projection/ProjectionBwd_kernel.cuh:16-130). accumulate != 0:
  * gradients are added into v_world (the reference's behaviour; caller zero-fills,
  * src/engine/EngineLoss.cpp:120-127). accumulate == 0: every row of v_world is overwritten
  * (zeros for culled splats), which gives the same values with C = 1 and needs no zero-fill. */
@@ -306,6 +306,11 @@ typedef struct {
     const int32_t* packed_gaussian_ids;
     int64_t num_packed;
     const float* v_rows;    /* optional: ssr_raster_bwd's row output; when given, v_screen is not read */
+    /* Optional gradient of the camera pose (the reference's v_viewmats, ProjectionBwd_kernel.cuh:89-127): 16
+     * floats laid out like the row-major [R|t] view matrix; the sums over all processed splats of dL/dR (rows
+     * 0..2, columns 0..2) and dL/dt (column 3) are ADDED to it (caller zero-fills), the last row is not touched.
+     * Both the projection and the SH view direction contribute. Computed by a second pass over the splats. */
+    float* v_viewmat;
 } ssr_projection_bwd_params;
 int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream_t stream);
 

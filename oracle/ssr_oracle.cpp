@@ -1324,9 +1324,19 @@ void or_projection_bwd(int64_t N, int sh_degree, const float* means, const float
     const or_sh_source* sh, const or_camera* camera, const float* aabb, const float* v_xy,
     const float* v_sdepth, const float* v_conic, const float* v_opac, const float* v_srgb,
     float* v_means, float* v_quats, float* v_scales, float* v_opacities, float* v_dc, float* v_sh) {
+    or_projection_bwd_pose(N, sh_degree, means, quats, log_scales, opacity_logits, features_dc, sh, camera, aabb, v_xy, v_sdepth,
+                           v_conic, v_opac, v_srgb, v_means, v_quats, v_scales, v_opacities, v_dc, v_sh, nullptr);
+}
+
+void or_projection_bwd_pose(int64_t N, int sh_degree, const float* means, const float* quats,
+    const float* log_scales, const float* opacity_logits, const float* features_dc,
+    const or_sh_source* sh, const or_camera* camera, const float* aabb, const float* v_xy,
+    const float* v_sdepth, const float* v_conic, const float* v_opac, const float* v_srgb,
+    float* v_means, float* v_quats, float* v_scales, float* v_opacities, float* v_dc, float* v_sh, float* v_viewmat) {
     const Cam cam = load_cam(camera);
     const int n_coef = sh_degree * (sh_degree + 2);
     auto fin = [](float v) { return ssr_isfinite(v) ? v : 0.0f; };
+    std::vector<float> pose(v_viewmat ? (size_t)N * 12 : 0, 0.0f);   // per-splat dL/dR (9) and dL/dt (3), summed below
 #pragma omp parallel for schedule(static)
     for (int64_t g = 0; g < N; g++) {
         const float* bb = aabb + 4 * g;
@@ -1529,12 +1539,39 @@ void or_projection_bwd(int64_t N, int sh_degree, const float* means, const float
             vdir[1] = (vy - dn * Y) * b.inorm;
             vdir[2] = (vz - dn * Z) * b.inorm;
         }
+        if (v_viewmat) {
+            // mean_c = R mean + t, cov_c = R cov R^T, view direction = mean + R^T t (primitive_3dgs.slang:434-436,
+            // harmonics.slang:145-149): dL/dt = v_mean_c + R v_dir, dL/dR = v_mean_c mean^T + (vS + vS^T) R cov + t v_dir^T
+            float cov[3][3], RS[3][3];
+            for (int a = 0; a < 3; a++)
+                for (int j = 0; j < 3; j++) cov[a][j] = (p.M[a][0] * p.M[j][0] + p.M[a][1] * p.M[j][1]) + p.M[a][2] * p.M[j][2];
+            for (int k = 0; k < 3; k++)
+                for (int j = 0; j < 3; j++) RS[k][j] = (cam.R[k][0] * cov[0][j] + cam.R[k][1] * cov[1][j]) + cam.R[k][2] * cov[2][j];
+            float* out = pose.data() + 12 * g;
+            for (int i = 0; i < 3; i++) {
+                out[9 + i] = vmc[i] + ((cam.R[i][0] * vdir[0] + cam.R[i][1] * vdir[1]) + cam.R[i][2] * vdir[2]);
+                for (int j = 0; j < 3; j++) {
+                    float s = vmc[i] * mean[j] + cam.t[i] * vdir[j];
+                    for (int k = 0; k < 3; k++) s += (vS[i][k] + vS[k][i]) * RS[k][j];
+                    out[3 * i + j] = s;
+                }
+            }
+        }
         // World::atomicStore, PrimitiveBase3DGS.cuh:75-83: per-component finite filter
         for (int i = 0; i < 3; i++) v_means[3 * g + i] += fin(vmean[i] + vdir[i]);
         for (int i = 0; i < 4; i++) v_quats[4 * g + i] += fin(vquat[i]);
         for (int i = 0; i < 3; i++) v_scales[3 * g + i] += fin(vscale[i]);
         v_opacities[g] += fin(vlogit);
         for (int i = 0; i < 3; i++) v_dc[3 * g + i] += fin(vdcl[i]);
+    }
+    if (v_viewmat) {   // summed in double, in splat order (the kernels add floats in an unspecified order)
+        double acc[12] = {0};
+        for (int64_t g = 0; g < N; g++)
+            for (int k = 0; k < 12; k++) acc[k] += pose[12 * g + k];
+        for (int i = 0; i < 3; i++) {
+            for (int j = 0; j < 3; j++) v_viewmat[4 * i + j] += (float)acc[3 * i + j];
+            v_viewmat[4 * i + 3] += (float)acc[9 + i];
+        }
     }
 }
 

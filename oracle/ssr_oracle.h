@@ -127,6 +127,15 @@ void or_projection_bwd(int64_t N, int sh_degree,
     const float* v_xy, const float* v_sdepth, const float* v_conic, const float* v_opac,
     const float* v_srgb,
     float* v_means, float* v_quats, float* v_scales, float* v_opacities, float* v_dc, float* v_sh);
+/* As or_projection_bwd, and the camera-pose gradient (the reference's v_viewmats,
+ * src/kernels/projection/ProjectionBwd_kernel.cuh:89-127): the sums over the processed splats of dL/dR and dL/dt
+ * are added to v_viewmat (16 floats, row-major [R|t]; may be NULL). */
+void or_projection_bwd_pose(int64_t N, int sh_degree,
+    const float* means, const float* quats, const float* log_scales, const float* opacity_logits,
+    const float* features_dc, const or_sh_source* sh, const or_camera* cam, const float* aabb,
+    const float* v_xy, const float* v_sdepth, const float* v_conic, const float* v_opac,
+    const float* v_srgb,
+    float* v_means, float* v_quats, float* v_scales, float* v_opacities, float* v_dc, float* v_sh, float* v_viewmat);
 
 /* K9 fused with Adam (fp32-state branch of fused_projection_bwd_optimizer_3dgs,
  * src/kernels/optim/FusedProjectionBwdOptim_kernel.cuh:232-710): parameters and moments [N,...]

@@ -340,9 +340,13 @@ __device__ __forceinline__ VScreenD vscreen_of(const ssr_screen& s, const float*
     return VScreenD{s.xy, s.depth, s.conic, s.opac, s.rgb, 2, 1, 3, 1, 3};
 }
 
-template <int kDegree, bool kLens, class ShSink>
+// dL/dR and dL/dt of the world-to-camera transform, one splat's share
+struct PoseGradD { float R[3][3], t[3]; };
+
+template <int kDegree, bool kLens, bool kPose = false, class ShSink>
 __device__ __forceinline__ void projection_vjp(const CamD& cam, const ssr_world& W, const ssr_sh_quant& Q, int64_t g,
-                                               const VScreenD& VS, int64_t r, WorldGradD& out, ShSink&& sh_sink) {
+                                               const VScreenD& VS, int64_t r, WorldGradD& out, ShSink&& sh_sink,
+                                               PoseGradD* pose = nullptr) {
     constexpr int kCoef = kDegree * (kDegree + 2);
     float mean[3], quat[4], ls[3], logit;
     load_splat(W, g, mean, quat, ls, logit);
@@ -568,6 +572,31 @@ __device__ __forceinline__ void projection_vjp(const CamD& cam, const ssr_world&
 #pragma unroll
     for (int i = 0; i < 4; i++) out.quat[i] = vquat[i];
     out.logit = vlogit;
+    if (kPose) {
+        // mean_c = R mean + t, cov_c = R cov R^T (cov = M M^T), view direction = mean + R^T t
+        // (src/shaders/primitive_3dgs.slang:434-436, src/shaders/harmonics.slang:145-149):
+        //   dL/dt = v_mean_c + R v_dir,   dL/dR = v_mean_c mean^T + (v_cov_c + v_cov_c^T) R cov + t v_dir^T
+        float cov[3][3], RS[3][3];
+#pragma unroll
+        for (int a = 0; a < 3; a++)
+#pragma unroll
+            for (int j = 0; j < 3; j++) cov[a][j] = (p.M[a][0] * p.M[j][0] + p.M[a][1] * p.M[j][1]) + p.M[a][2] * p.M[j][2];
+#pragma unroll
+        for (int k = 0; k < 3; k++)
+#pragma unroll
+            for (int j = 0; j < 3; j++) RS[k][j] = (cam.R[k][0] * cov[0][j] + cam.R[k][1] * cov[1][j]) + cam.R[k][2] * cov[2][j];
+#pragma unroll
+        for (int i = 0; i < 3; i++) {
+            pose->t[i] = vmc[i] + ((cam.R[i][0] * vdir[0] + cam.R[i][1] * vdir[1]) + cam.R[i][2] * vdir[2]);
+#pragma unroll
+            for (int j = 0; j < 3; j++) {
+                float s = vmc[i] * mean[j] + cam.t[i] * vdir[j];
+#pragma unroll
+                for (int k = 0; k < 3; k++) s += (vS[i][k] + vS[k][i]) * RS[k][j];
+                pose->R[i][j] = s;
+            }
+        }
+    }
 }
 
 template <int kDegree, bool kAccumulate, bool kLens>
@@ -618,6 +647,51 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
     put<kAccumulate>(V.opacity_logits + g, fin(wg.logit));
 #pragma unroll
     for (int i = 0; i < 3; i++) put<kAccumulate>(V.features_dc + 3 * g + i, fin(wg.dc[i]));
+}
+
+// Camera-pose gradient: the same VJP once more, keeping only dL/dR and dL/dt, summed over the workgroup and added
+// to the 16-float view-matrix gradient with one atomic per entry and workgroup (the reference sums per warp,
+// ProjectionBwd_kernel.cuh:108-127).
+template <int kDegree, bool kLens>
+__global__ __launch_bounds__(kProjBlock) void projection_pose_bwd_kernel(ssr_projection_bwd_params P) {
+    __shared__ float s_part[kProjBlock / 64][12];
+    const int64_t i = (int64_t)blockIdx.x * kProjBlock + threadIdx.x;
+    const int64_t n_rows = P.packed_gaussian_ids ? P.num_packed : (P.visible_ids ? P.n_visible : P.num_splats);
+    float v[12];
+#pragma unroll
+    for (int k = 0; k < 12; k++) v[k] = 0.f;
+    if (i < n_rows) {
+        const int64_t g = P.packed_gaussian_ids ? (int64_t)P.packed_gaussian_ids[i] : (P.visible_ids ? (int64_t)P.visible_ids[i] : i);
+        const int64_t r = P.packed_gaussian_ids ? i : g;
+        float4 bb = make_float4(0.f, 0.f, 1.f, 1.f);
+        if (!P.packed_gaussian_ids) bb = reinterpret_cast<const float4*>(P.aabb)[g];
+        if (!(bb.z <= bb.x || bb.w <= bb.y)) {
+            const CamD cam = load_camera(P.camera);
+            WorldGradD wg;
+            PoseGradD pg;
+            projection_vjp<kDegree, kLens, true>(cam, P.world, P.sh, g, vscreen_of(P.v_screen, P.v_rows), r, wg,
+                                                 [](int, float, const float*) {}, &pg);
+#pragma unroll
+            for (int a = 0; a < 3; a++) {
+#pragma unroll
+                for (int b = 0; b < 3; b++) v[4 * a + b] = pg.R[a][b];
+                v[4 * a + 3] = pg.t[a];
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 12; k++) {
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) v[k] += __shfl_xor(v[k], d, 64);
+        if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6][k] = v[k];
+    }
+    __syncthreads();
+    if (threadIdx.x < 12) {
+        float s = s_part[0][threadIdx.x];
+#pragma unroll
+        for (int w = 1; w < kProjBlock / 64; w++) s += s_part[w][threadIdx.x];
+        atomicAdd(P.v_viewmat + threadIdx.x, s);
+    }
 }
 
 // ---- projection backward fused with Adam ---------------------------------------------------------
@@ -1218,6 +1292,19 @@ extern "C" int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream
     }
 #undef SSR_LAUNCH_BWD
     SSR_CHECK_LAUNCH("ssr_projection_bwd");
+    if (p->v_viewmat) {
+#define SSR_LAUNCH_POSE(D)                                                                            \
+    if (lens) hipLaunchKernelGGL((projection_pose_bwd_kernel<D, true>), grid, block, 0, s, *p);        \
+    else hipLaunchKernelGGL((projection_pose_bwd_kernel<D, false>), grid, block, 0, s, *p);
+        switch (p->sh_degree) {
+            case 0: SSR_LAUNCH_POSE(0); break;
+            case 1: SSR_LAUNCH_POSE(1); break;
+            case 2: SSR_LAUNCH_POSE(2); break;
+            default: SSR_LAUNCH_POSE(3); break;
+        }
+#undef SSR_LAUNCH_POSE
+        SSR_CHECK_LAUNCH("ssr_projection_bwd (camera pose)");
+    }
     return 0;
 }
 

@@ -25,6 +25,7 @@ SYMBOLS = {
     "ssrh_backward_with_variants": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, C.c_int]),
     "ssrh_backward_fused_optimizer": (C.c_int, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_int]),
     "ssrh_copy_non_sh_quant_state": (C.c_int, [vp, vp]),
+    "ssrh_backward_with_pose_grad": (C.c_int, [vp, vp, vp, vp]),
     "ssrh_copy_sh_quant_state": (C.c_int, [vp, vp, vp, vp]),
     "ssrh_copy_params_to_host": (C.c_int, [vp, vp, vp, vp, vp, vp]),
     "ssrh_set_tile_mask": (C.c_int, [vp, C.c_int, C.c_int]),
@@ -145,6 +146,12 @@ class Engine:
 
     def backward(self):
         check(self.h.ssrh_backward_from_render_grad(self.d_vrgb.ptr, self.d_vdepth.ptr, self.d_vT.ptr))
+
+    def backward_with_pose_grad(self):
+        """The backward plus the camera-pose gradient: returns dL/d[R|t] as [4,4] (last row zero)."""
+        out = np.zeros((4, 4), np.float32)
+        check(self.h.ssrh_backward_with_pose_grad(self.d_vrgb.ptr, self.d_vdepth.ptr, self.d_vT.ptr, out.ctypes.data))
+        return out
 
     HYPER = ["lr_means", "lr_quats", "lr_scales", "lr_opacs", "lr_features_dc", "lr_features_sh", "max_gauss_ratio",
              "scale_regularization_weight", "mcmc_opacity_reg_weight", "mcmc_scale_reg_weight", "quat_norm_reg_weight",

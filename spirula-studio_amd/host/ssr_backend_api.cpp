@@ -589,7 +589,7 @@ void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
                               const std::optional<TorchTensorView> sh_value_packed,
                               const std::optional<TorchTensorView> sh_value_bounds, const uint32_t num_sh_buffer,
                               const int sh_value_bits, const int64_t sh_bounds_stride) {
-    if (v_viewmats) throw std::runtime_error("projection_3dgs_backward: camera pose gradients are not built in this backend");
+
     const bool is_packed = camera_ids.data_ptr() && gaussian_ids.data_ptr();   // src/kernels/projection/ProjectionBwd.cu:80
     g_bwd_list = nullptr; g_bwd_count = 0;
     if (num_splats == 0) return;   // ProjectionBwd.cu:86-87
@@ -607,6 +607,7 @@ void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
     if (g_vrows && p.v_screen.xy == g_vrows_for_xy) p.v_rows = g_vrows;
     p.v_world = world_of(v_splats_world);
     p.accumulate = g_opts.overwrite_world_grads ? 0 : 1;
+    if (v_viewmats) p.v_viewmat = v_viewmats->data_ptr();   // [C = 1, 16]: accumulated into, as the reference does
     if (is_packed) {
         p.aabb = nullptr;
         p.packed_gaussian_ids = gaussian_ids.data_ptr(); p.num_packed = camera_ids.size();

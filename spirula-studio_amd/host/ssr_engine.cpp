@@ -226,7 +226,7 @@ std::vector<DeviceTensorFloatND> raster_backward(TorchTensorView v_render_rgb, T
 }  // namespace
 
 void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
-                                      TorchTensorView v_render_Ts) {
+                                      TorchTensorView v_render_Ts, DeviceTensor2D<float>* v_viewmats) {
     auto& E = engine();
     if (std::get<0>(E.fwd.renders).data_ptr() == nullptr)
         throw std::runtime_error("engine_backward_from_render_grad: forward_3dgs must be called first");
@@ -242,7 +242,7 @@ void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorV
     projection_3dgs_backward(
         E.cur_num_splats, E.sh_degree, E.fwd.splats_w, E.camera.viewmats, E.camera.intrins, (uint32_t)W, (uint32_t)H,
         E.camera.model_str, E.camera.distortion_str, E.camera.dist_coeffs, E.fwd.camera_ids, E.fwd.gaussian_ids,
-        E.fwd.aabb, vs, v_world, nullptr, E.world.sh_packed, E.world.sh_bounds, (uint32_t)E.num_sh, E.world.sh_value_bits,
+        E.fwd.aabb, vs, v_world, v_viewmats, E.world.sh_packed, E.world.sh_bounds, (uint32_t)E.num_sh, E.world.sh_value_bits,
         E.world.sh_bounds_stride);
     E.grad.dirty_list = ssr_ext::last_backward_list(&E.grad.dirty_count);
     E.grad.dirty_key = (const void*)E.grad.means.data_ptr();
@@ -491,6 +491,19 @@ int ssrh_backward_from_render_grad(const float* v_rgb, const float* v_depth, con
     return guard([&] {
         const int64_t C = engine().camera.num, H = engine().camera.height, W = engine().camera.width;
         engine_backward_from_render_grad(tv(v_rgb, 4, {C, H, W, 3}), tv(v_depth, 4, {C, H, W, 1}), tv(v_Ts, 4, {C, H, W, 1}));
+    });
+}
+
+// The backward with the camera-pose gradient as well (the launch function's v_viewmats; the reference's engine
+// itself always passes null): out16 receives dL/d[R|t] as a row-major 4x4 whose last row is zero.
+int ssrh_backward_with_pose_grad(const float* v_rgb, const float* v_depth, const float* v_Ts, float* out16) {
+    return guard([&] {
+        const int64_t C = engine().camera.num, H = engine().camera.height, W = engine().camera.width;
+        float* d = DevicePool::global().acquire<float>(PoolSlot::EngPoseGrad, 16);
+        backend::memset_async(d, 0, 16 * sizeof(float));
+        DeviceTensor2D<float> vm(d, 1, 16);
+        engine_backward_from_render_grad(tv(v_rgb, 4, {C, H, W, 3}), tv(v_depth, 4, {C, H, W, 1}), tv(v_Ts, 4, {C, H, W, 1}), &vm);
+        backend::memcpy_sync(out16, d, 16 * sizeof(float), backend::MemcpyKind::DeviceToHost);
     });
 }
 

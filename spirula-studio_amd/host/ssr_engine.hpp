@@ -79,7 +79,7 @@ void set_camera_params(int width, int height, std::string camera_model, std::str
 void engine_set_tile_mask(TorchTensorView mask);
 void forward_3dgs(std::string primitive, int sh_degree, bool packed, bool output_median, int dist_type_int);
 void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
-                                      TorchTensorView v_render_Ts);
+                                      TorchTensorView v_render_Ts, DeviceTensor2D<float>* v_viewmats = nullptr);
 // Backward with the projection backward folded into the optimizer step
 // (engine().optim.use_fused_proj_bwd_optim, src/engine/EngineLoss.cpp:286-290): compositing backward,
 // then fused_projection_bwd_optimizer_3dgs on the engine's parameters with Adam moments kept in pool

@@ -71,7 +71,8 @@ class ProjectionBwdParams(C.Structure):
     _fields_ = [("num_splats", C.c_int64), ("sh_degree", C.c_int32), ("world", World),
                 ("sh", ShQuant), ("camera", Camera), ("aabb", vp), ("v_screen", Screen),
                 ("v_world", World), ("accumulate", C.c_int32), ("visible_ids", vp),
-                ("n_visible", C.c_int64), ("packed_gaussian_ids", vp), ("num_packed", C.c_int64), ("v_rows", vp)]
+                ("n_visible", C.c_int64), ("packed_gaussian_ids", vp), ("num_packed", C.c_int64), ("v_rows", vp),
+                ("v_viewmat", vp)]
 
 
 class ProjectionPackedParams(C.Structure):

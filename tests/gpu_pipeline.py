@@ -298,7 +298,8 @@ class GpuRun:
             for k, sl in [("v_xy", slice(0, 2)), ("v_depth", 2), ("v_conic", slice(3, 6)), ("v_opac", 6), ("v_rgb", slice(7, 10))]:
                 self.d[k] = D.from_host(np.ascontiguousarray(rows[:, sl]))
 
-    def projection_bwd(self, accumulate=True, poison=False):
+    def projection_bwd(self, accumulate=True, poison=False, pose=False):
+        """pose=True: also the camera-pose gradient, read back with host("v_viewmat") as [4,4]."""
         D = self.L.DeviceArray
         n = self.n
         for k, shape in [("w_means", (n, 3)), ("w_quats", (n, 4)), ("w_log_scales", (n, 3)),
@@ -319,6 +320,10 @@ class GpuRun:
         if self.use_vrows:
             p.v_rows = self.ptr("v_rows")
             p.v_screen = self.L.Screen()   # not read
+        if pose:
+            self.d["v_viewmat"] = D((4, 4), np.float32)
+            self.d["v_viewmat"].fill_zero()
+            p.v_viewmat = self.ptr("v_viewmat")
         if self.packed_projection:
             if self.rows == 0:   # nothing visible: the launcher has nothing to run (ProjectionBwd.cu:86-97)
                 return

@@ -214,19 +214,22 @@ def raster_bwd(n, scr, w, h, offsets, flat, fwd, v_rgb, v_depth, v_T, with_abs=T
     return g
 
 
-def projection_bwd(scene, aabb, vs, sh_degree=3):
+def projection_bwd(scene, aabb, vs, sh_degree=3, pose=False):
+    """pose=True: also the camera-pose gradient, g["v_viewmat"] [4,4] laid out like the [R|t] view matrix."""
     n = scene.n
     keep = []
     cam, sh = camera_of(scene), sh_source_of(scene, keep)
     g = dict(v_means=np.zeros((n, 3), np.float32), v_quats=np.zeros((n, 4), np.float32),
              v_scales=np.zeros((n, 3), np.float32), v_opacities=np.zeros(n, np.float32),
              v_dc=np.zeros((n, 3), np.float32), v_sh=np.zeros((n, 15, 3), np.float32))
-    lib().or_projection_bwd(
+    if pose:
+        g["v_viewmat"] = np.zeros((4, 4), np.float32)
+    lib().or_projection_bwd_pose(
         C.c_int64(n), C.c_int(sh_degree), _p(scene.means), _p(scene.quats), _p(scene.log_scales),
         _p(scene.opacity_logits), _p(scene.features_dc), C.byref(sh), C.byref(cam), _p(aabb),
         _p(vs["v_xy"]), _p(vs["v_depth"]), _p(vs["v_conic"]), _p(vs["v_opac"]), _p(vs["v_rgb"]),
         _p(g["v_means"]), _p(g["v_quats"]), _p(g["v_scales"]), _p(g["v_opacities"]), _p(g["v_dc"]),
-        _p(g["v_sh"]))
+        _p(g["v_sh"]), _p(g.get("v_viewmat")))
     return g
 
 

@@ -171,8 +171,9 @@ def test_projection_parity_quantized_rows(gpu, oracle, cam):
             assert np.array_equal(w32["rgb"][vis].view(np.uint32), want["rgb"][vis].view(np.uint32)), (bits, per_block)
 
 
-def _k9_direct(gpu, oracle, sc, vs, label, packed=False):
-    """ssr_projection_bwd fed given screen gradients (rows: splats, or packed rows), against the oracle."""
+def _k9_direct(gpu, oracle, sc, vs, label, packed=False, pose=False):
+    """ssr_projection_bwd fed given screen gradients (rows: splats, or packed rows), against the oracle.
+    pose: also the camera-pose gradient (the rows of the tool that ask for v_viewmats)."""
     g = GpuRun(gpu, sc, packed_projection=packed)
     g.projection_fwd()
     D = gpu.lib.DeviceArray
@@ -190,8 +191,14 @@ def _k9_direct(gpu, oracle, sc, vs, label, packed=False):
         full_aabb, full_vs = aabb, vs
     for k, v in vs.items():
         g.d[k] = D.from_host(np.ascontiguousarray(v))
-    g.projection_bwd()
-    want = oracle.projection_bwd(sc, full_aabb, full_vs)
+    g.projection_bwd(pose=pose)
+    want = oracle.projection_bwd(sc, full_aabb, full_vs, pose=pose)
+    if pose:
+        got_vm, want_vm = g.host("v_viewmat").astype(np.float64), want.pop("v_viewmat").astype(np.float64)
+        print(f"[{label}] dL/dt = {want_vm[:3, 3]}", flush=True)
+        assert not np.any(got_vm[3]) and np.abs(want_vm[:3]).min() > 0
+        assert np.abs(got_vm - want_vm).max() <= 1e-3 * np.abs(want_vm).max(), (got_vm, want_vm)
+        assert (np.abs(got_vm - want_vm) <= 5e-3 + 1e-3 * np.abs(want_vm)).all()     # the tool's band
     vis = full_aabb[:, 2] > full_aabb[:, 0]
     print(f"[{label}] visible={int(vis.sum())}", flush=True)
     assert 50 < vis.sum() < sc.n
@@ -206,8 +213,8 @@ def _k9_direct(gpu, oracle, sc, vs, label, packed=False):
         assert (np.abs(got - ref) <= 5e-3 + 1e-3 * np.abs(ref)).all(), k
 
 
-# proj_bwd_parity.cpp:171-180, rows with prim == 0 (the camera-pose gradient some of them also ask for is not built
-# here): screen gradients drawn by the tool, not produced by the compositing backward
+# proj_bwd_parity.cpp:171-180, rows with prim == 0, the first two with the camera-pose gradient: screen gradients drawn by
+# the tool, not produced by the compositing backward
 @pytest.mark.parametrize("cam", [0, 1])
 def test_proj_bwd_parity_rows(gpu, oracle, cam):
     n = R.N_TOOL
@@ -218,7 +225,7 @@ def test_proj_bwd_parity_rows(gpu, oracle, cam):
         vs2 = R.screen_gradients(rng, R.C_TOOL * n)
         vs = {k: np.ascontiguousarray(v.reshape((R.C_TOOL, n) + v.shape[1:])[cam]) for k, v in vs2.items()}
         sc, _ = R.tool_scene(gpu, R.SEED_PROJ_BWD, cam, PINHOLE, tier)
-        _k9_direct(gpu, oracle, sc, vs, f"proj_bwd_parity PINHOLE tier {tier} cam {cam}")
+        _k9_direct(gpu, oracle, sc, vs, f"proj_bwd_parity PINHOLE tier {tier} cam {cam}", pose=True)
     R.screen_gradients(rng, R.C_TOOL * n)        # row 2 (another primitive) draws the same amount
     # row 3: packed, EQUISOLID + OpenCV; the tool's rows are camera 0's visible splats, then camera 1's
     nnz = []
@@ -230,7 +237,7 @@ def test_proj_bwd_parity_rows(gpu, oracle, cam):
     lo = sum(nnz[:cam])
     vs = {k: np.ascontiguousarray(v[lo:lo + nnz[cam]]) for k, v in vs2.items()}
     sc, _ = R.tool_scene(gpu, R.SEED_PROJ_BWD, cam, EQUISOLID, OPENCV)
-    _k9_direct(gpu, oracle, sc, vs, f"proj_bwd_parity packed EQUISOLID OPENCV cam {cam}", packed=True)
+    _k9_direct(gpu, oracle, sc, vs, f"proj_bwd_parity packed EQUISOLID OPENCV cam {cam}", packed=True, pose=True)
     # row 6: 8-bit SH codes, bounds per 256 cells, thin-prism lens (two rows of another primitive draw in between:
     # the gradients here have the tool's ranges, not its exact stream)
     vs2 = R.screen_gradients(rng, R.C_TOOL * n)

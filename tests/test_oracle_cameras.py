@@ -230,3 +230,46 @@ def test_pinhole_clamp_with_a_lens_routes_to_the_bound(pkg, oracle):
                  sc.features_dc[g].astype(np.float64), sc.features_sh[g].astype(np.float64)]
             fd[k] = (_loss64(sc, g, v, mp, *a) - _loss64(sc, g, v, mm, *a)) / (2 * h)
         np.testing.assert_allclose(g_or["v_means"][g], fd, rtol=2e-3, atol=2e-3 * np.abs(fd).max())
+
+
+@pytest.mark.parametrize("model,tier", [(0, 0), (0, 1), (0, 3), (1, 2), (2, 0), (3, 0)])
+def test_camera_pose_gradient_matches_finite_differences(pkg, oracle, model, tier):
+    """dL/dR and dL/dt of the view matrix (the reference's v_viewmats: the projection through mean_c = R mean + t and
+    cov_c = R cov R^T, the colour through the view direction mean + R^T t), summed over the splats, against central
+    differences of the float64 loss in each of the twelve entries (R perturbed entry by entry, not kept orthonormal:
+    that is the derivative the reference's autodiff forms)."""
+    sc = _scene(pkg, model, tier, n=120, seed=37)
+    rng = np.random.default_rng(9)
+    o = oracle.projection_fwd(sc)
+    n = sc.n
+    v = dict(v_xy=rng.normal(0, 1, (n, 2)).astype(np.float32), v_depth=rng.normal(0, 1, n).astype(np.float32),
+             v_conic=rng.normal(0, 1, (n, 3)).astype(np.float32), v_opac=rng.normal(0, 1, n).astype(np.float32),
+             v_rgb=rng.normal(0, 1, (n, 3)).astype(np.float32))
+    vis = np.nonzero(o["aabb"][:, 2] > o["aabb"][:, 0])[0]
+    assert len(vis) > 20
+    got = oracle.projection_bwd(sc, o["aabb"], v, pose=True)["v_viewmat"].astype(np.float64)
+    assert not np.any(got[3])
+    # the same world gradients with and without the pose output
+    plain = oracle.projection_bwd(sc, o["aabb"], v)
+    with_pose = oracle.projection_bwd(sc, o["aabb"], v, pose=True)
+    for k in plain:
+        assert np.array_equal(plain[k], with_pose[k]), k
+
+    def total(vm):
+        import dataclasses
+        s2 = dataclasses.replace(sc, viewmat=vm)
+        return sum(_loss64(s2, g, v, sc.means[g].astype(np.float64), sc.quats[g].astype(np.float64), sc.log_scales[g].astype(np.float64),
+                           float(sc.opacity_logits[g]), sc.features_dc[g].astype(np.float64), sc.features_sh[g].astype(np.float64))
+                   for g in vis)
+    fd = np.zeros((4, 4))
+    base = sc.viewmat.astype(np.float64)
+    for i in range(3):
+        for j in range(4):
+            h = 1e-6 * max(1.0, abs(base[i, j]))
+            vp, vm_ = base.copy(), base.copy()
+            vp[i, j] += h
+            vm_[i, j] -= h
+            fd[i, j] = (total(vp) - total(vm_)) / (2 * h)
+    scale = np.abs(fd).max()
+    assert scale > 1e-3
+    assert np.abs(got - fd).max() <= 3e-3 * scale, (got, fd)
