@@ -328,8 +328,7 @@ int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream_t stream);
  * per-splat range, FusedProjectionBwdOptim.cu:160-212 -- with one camera a splat has at most one
  * row, found through packed_row_of), regularizers mcmc_opacity, mcmc_scale, scale ratio, effective
  * rank, quaternion norm and SH/DC magnitude; the scale-agnostic step of the means; the quantized SH
- * state and the quantized moments of the non-SH tensors (below). Not built (rejected): the colour
- * trust region of the linear-colour preset. */
+ * state, the quantized moments of the non-SH tensors and the colour trust region (below). */
 typedef struct {
     int64_t num_splats;
     int32_t sh_degree;
@@ -372,6 +371,13 @@ typedef struct {
      * the zero moments. The parameters themselves stay fp32. */
     uint32_t* non_sh_packed[5];     /* [N * 3], [N * 4], [N * 3], [N], [N * 3] */
     float* non_sh_bounds[5];        /* float4[ceil(N / 256)] each */
+    /* Colour trust region of the linear-colour preset (color_trust_linear, eps_tr;
+     * FusedProjectionBwdOptim_kernel.cuh:551-596,651-705,774-794): the DC colour steps in the space of
+     * splat_dc_encode with its gradient divided by the slope of the sRGB curve at the DC colour and the step
+     * clipped to kSh0 sqrt(2 eps_tr / opacity); the SH gradients are divided by the same slopes and their steps
+     * clipped to kSh0 sqrt(4 eps_tr colour / opacity) per channel. */
+    int32_t color_trust_linear;
+    float eps_tr;
 } ssr_fpbo_params;
 int ssr_fused_projection_bwd_optimizer(const ssr_fpbo_params* p, ssr_stream_t stream);
 /* row_of[g] = i where gaussian_ids[i] == g, -1 for splats without a packed row (one camera, so ids

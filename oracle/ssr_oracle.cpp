@@ -10,6 +10,7 @@
 #include "../include/ssr_math.h"
 #include "../include/ssr_camera.h"
 #include "../include/ssr_quant.h"
+#include "../include/ssr_colour.h"
 
 #include <algorithm>
 #include <cmath>
@@ -528,6 +529,11 @@ void or_quant_codec(int op, int64_t n, float* a, float* b, const float* mm, uint
     }
 }
 
+void or_colour_map(int op, int64_t n, const float* x, float* y) {
+    for (int64_t i = 0; i < n; i++)
+        y[i] = op == 0 ? ssr_srgb_slope(x[i]) : op == 1 ? ssr_splat_dc_encode(x[i]) : ssr_splat_dc_decode(x[i]);
+}
+
 static void fused_optimizer_impl(int64_t N, int sh_degree,
     float* means, float* quats, float* log_scales, float* opacity_logits, float* features_dc, float* features_sh,
     const or_sh_quant_state* q, const or_non_sh_quant_state* nq,
@@ -571,6 +577,16 @@ static void fused_optimizer_impl(int64_t N, int sh_degree,
     const float lr_means = hyper[0], lr_quats = hyper[1], lr_scales = hyper[2], lr_opacs = hyper[3], lr_dc = hyper[4],
                 lr_sh = hyper[5], max_ratio = hyper[6], scale_w = hyper[7], mcmc_o = hyper[8], mcmc_s = hyper[9],
                 qnorm_w = hyper[10], sh_w = hyper[11], erank_w = hyper[12], erank_w3 = hyper[13];
+    // colour trust region (FusedProjectionBwdOptim_kernel.cuh:551-596,651-705,774-794): per splat the slope of the
+    // sRGB curve at its DC colour and the clip of its SH steps, from the parameters as they were
+    const bool ctl = hyper[14] != 0.0f;
+    const float eps_tr = hyper[15];
+    const float kSh0 = 0.28209479177387814f;
+    std::vector<float> ctl_slope(ctl ? (size_t)N * 3 : 0), ctl_clip(ctl ? (size_t)N * 3 : 0);
+    auto clip_step = [](float delta, float clip) {
+        delta = ssr_min(ssr_max(delta, -clip), clip);
+        return ssr_isfinite(delta) ? delta : 0.0f;
+    };
     const float kBeta1 = 0.9f, kBeta2 = 0.999f, kEps = 1e-15f;
     const float sh_reg = sh_w * (1.0f / (float)(n_coef > 0 ? n_coef : 1));
 #pragma omp parallel for schedule(static)
@@ -599,10 +615,26 @@ static void fused_optimizer_impl(int64_t N, int sh_degree,
         }
         for (int i = 0; i < 4; i++) gq[i] = vin(1, 4 * g + i) + vq[4 * g + i];
         go = vin(3, g) + vo[g];
+        if (ctl) {
+            const float inv_opac = 1.0f / ssr_max(ssr_sigmoid(opacity_logits[g]), 1e-12f);
+            for (int c = 0; c < 3; c++) {
+                const float c_dc = kSh0 * features_dc[3 * g + c] + 0.5f;
+                ctl_slope[3 * g + c] = ssr_srgb_slope(c_dc);
+                const float cc = ssr_max(c_dc, (1.0f / 255.0f) * (1.0f / 255.0f));
+                ctl_clip[3 * g + c] = kSh0 * ssr_sqrt(((4.0f * eps_tr) * cc) * inv_opac);
+            }
+        }
         // SH (fp32 state; the quantized state is updated block by block below)
         for (int i = 0; !q && i < 3 * n_coef; i++) {
             float* x = features_sh + 45 * g + i;
-            *x = adam(*x, vsh[45 * g + i] + sh_reg * *x, lr_sh, g1[5] + 45 * g + i, g2[5] + 45 * g + i);
+            float v = vsh[45 * g + i] + sh_reg * *x;
+            if (ctl) {
+                v = v / ctl_slope[3 * g + i % 3];
+                const float delta = adam(0.0f, v, lr_sh, g1[5] + 45 * g + i, g2[5] + 45 * g + i);
+                *x = *x + clip_step(delta, ctl_clip[3 * g + i % 3]);
+            } else {
+                *x = adam(*x, v, lr_sh, g1[5] + 45 * g + i, g2[5] + 45 * g + i);
+            }
         }
         const float* ls = log_scales + 3 * g;
         const float* q0 = quats + 4 * g;
@@ -674,8 +706,16 @@ static void fused_optimizer_impl(int64_t N, int sh_degree,
                 means[3 * g + i] = adam(means[3 * g + i], gm[i], lr_means, g1[0] + 3 * g + i, g2[0] + 3 * g + i);
             }
         }
-        for (int i = 0; i < 3; i++)
-            features_dc[3 * g + i] = adam(features_dc[3 * g + i], gd[i], lr_dc, g1[4] + 3 * g + i, g2[4] + 3 * g + i);
+        for (int i = 0; i < 3; i++) {
+            if (ctl) {
+                const float dc = features_dc[3 * g + i];
+                const float delta = adam(0.0f, gd[i] / ctl_slope[3 * g + i], lr_dc, g1[4] + 3 * g + i, g2[4] + 3 * g + i);
+                const float clip = kSh0 * ssr_sqrt((2.0f * eps_tr) / ssr_max(sg, 1e-12f));
+                features_dc[3 * g + i] = ssr_splat_dc_decode(ssr_splat_dc_encode(dc) + clip_step(delta, clip));
+            } else {
+                features_dc[3 * g + i] = adam(features_dc[3 * g + i], gd[i], lr_dc, g1[4] + 3 * g + i, g2[4] + 3 * g + i);
+            }
+        }
     }
     if (nq) {
         for (int t = 0; t < 5; t++)
@@ -725,10 +765,13 @@ static void fused_optimizer_impl(int64_t N, int sh_degree,
                 float m1, m2;
                 ssr_adamq_decode(q->state_packed[cell], old_mm, &m1, &m2);
                 const float x = ssr_q16_decode(q->value_packed[cell], old_lo, old_hi);
-                const float v = vsh[45 * g + i] + sh_reg * x;
+                float v = vsh[45 * g + i] + sh_reg * x;
+                if (ctl) v = v / ctl_slope[3 * g + i % 3];
                 const float a = kBeta1 * m1 + (1.f - kBeta1) * v;
                 const float b = kBeta2 * m2 + (1.f - kBeta2) * (v * v);
-                const float xn = x - ((lr_sh * b1c) * a) / (ssr_sqrt(b * b2c) + kEps);
+                float delta = 0.0f - ((lr_sh * b1c) * a) / (ssr_sqrt(b * b2c) + kEps);
+                if (ctl) delta = clip_step(delta, ctl_clip[3 * g + i % 3]);
+                const float xn = x + delta;
                 const size_t o = (size_t)s * 3 * n_coef + i;
                 ng1[o] = a; ng2[o] = b; nx[o] = xn;
                 float u, ls;

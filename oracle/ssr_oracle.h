@@ -141,7 +141,8 @@ void or_projection_bwd_pose(int64_t N, int sh_degree,
  * src/kernels/optim/FusedProjectionBwdOptim_kernel.cuh:232-710): parameters and moments [N,...]
  * are updated in place. v_in (6 arrays, any may be NULL) are gradient contributions already
  * present. hyper = {lr_means, lr_quats, lr_scales, lr_opacs, lr_dc, lr_sh, max_gauss_ratio,
- * scale_reg_w, mcmc_opacity_w, mcmc_scale_w, quat_norm_w, sh_reg_w, erank_w, erank_w_s3}. steps may be NULL
+ * scale_reg_w, mcmc_opacity_w, mcmc_scale_w, quat_norm_w, sh_reg_w, erank_w, erank_w_s3, color_trust_linear (0 / 1),
+ * eps_tr} (16 floats). steps may be NULL
  * (then `step`). */
 void or_fused_projection_bwd_optimizer(int64_t N, int sh_degree,
     float* means, float* quats, float* log_scales, float* opacity_logits, float* features_dc, float* features_sh,
@@ -184,6 +185,10 @@ void or_fused_projection_bwd_optimizer_q(int64_t N, int sh_degree,
  * (codes -> a = g1, b = g2), 2 value encode (a = v, mm float2 -> codes), 3 value decode (codes -> a), 4 / 5 the
  * 16-bit Adam-state encode / decode. */
 void or_quant_codec(int op, int64_t n, float* a, float* b, const float* mm, uint32_t* codes);
+
+/* The colour maps of the colour trust region on arrays: op 0 slope of the sRGB curve, 1 splat_dc_encode,
+ * 2 splat_dc_decode (src/shaders/pixel_wise.slang:60-115). */
+void or_colour_map(int op, int64_t n, const float* x, float* y);
 
 /* erank_reg_3dgs (src/shaders/per_splat_losses.slang:3-15): the loss for one splat's three log-scales and
  * its gradient. */

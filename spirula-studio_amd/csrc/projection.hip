@@ -12,10 +12,12 @@
 // One thread per Gaussian, 256 threads (4 wavefronts) per workgroup. Both kernels are bound by
 // HBM traffic (236 B in, 60 B out per visible splat forward; 472 B in/out backward).
 #include <math.h>
+#include <type_traits>
 #include <string.h>
 
 #include "projection_device.h"
 #include "../../include/ssr_quant.h"
+#include "../../include/ssr_colour.h"
 #include "raster_device.h"
 
 namespace ssr {
@@ -734,6 +736,8 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
     __shared__ float s_red[kProjBlock / 64][6];   // quantized state: per-wave min / max of the new bounds
     __shared__ float s_sqrt_g2[kQuant ? 256 : 1];  // quantized state: sqrt(g2) of each 8-bit log_s code under the old bounds
     __shared__ float s_ns[kNsq ? kProjBlock / 64 : 1][20];   // quantized non-SH state: per-wave (min, max) x (u, log_s) x 5 tensors
+    __shared__ float s_ctl[kProjBlock][6];         // colour trust region: per splat the sRGB slope (3) and the SH step clip (3)
+    const bool ctl = P.color_trust_linear != 0;
     const int64_t block0 = (int64_t)blockIdx.x * kProjBlock;
     const int64_t g = block0 + threadIdx.x;
     const ssr_world& W = P.world;
@@ -924,8 +928,38 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
 #pragma unroll
             for (int i = 0; i < 3; i++) W.means[3 * g + i] = step_param(0, i, mean[i], wg.mean[i], P.lr_means);
         }
+        // features_dc: the plain step, or (colour trust region, FusedProjectionBwdOptim_kernel.cuh:551-596) the step in the
+        // space of splat_dc_encode, gradient divided by the slope of the sRGB curve at the DC colour, clipped
+        constexpr float kSh0 = 0.28209479177387814f;
+        float slope[3] = {1.f, 1.f, 1.f};
+        if (ctl) {
+            const float opac = ssr_sigmoid(logit);
+            const float inv_opac = 1.0f / ssr_max(opac, 1e-12f);
 #pragma unroll
-        for (int i = 0; i < 3; i++) W.features_dc[3 * g + i] = step_param(4, i, dc[i], wg.dc[i], P.lr_features_dc);
+            for (int c = 0; c < 3; c++) {
+                const float c_dc = kSh0 * dc[c] + 0.5f;
+                slope[c] = ssr_srgb_slope(c_dc);
+                s_ctl[threadIdx.x][c] = slope[c];
+                const float cc = ssr_max(c_dc, (1.0f / 255.0f) * (1.0f / 255.0f));
+                s_ctl[threadIdx.x][3 + c] = kSh0 * ssr_sqrt(((4.0f * P.eps_tr) * cc) * inv_opac);   // :656-666
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 3; i++) {
+            const float v = ctl ? wg.dc[i] / slope[i] : wg.dc[i];
+            float delta = step_param(4, i, 0.0f, v, P.lr_features_dc);   // 0 - step: the step itself, exactly
+            if (ctl) {
+                const float clip = kSh0 * ssr_sqrt((2.0f * P.eps_tr) / ssr_max(ssr_sigmoid(logit), 1e-12f));
+                delta = ssr_min(ssr_max(delta, -clip), clip);
+                delta = ssr_isfinite(delta) ? delta : 0.0f;
+                W.features_dc[3 * g + i] = ssr_splat_dc_decode(ssr_splat_dc_encode(dc[i]) + delta);
+            } else {
+                W.features_dc[3 * g + i] = dc[i] + delta;
+            }
+        }
+    } else if (ctl) {
+#pragma unroll
+        for (int c = 0; c < 6; c++) s_ctl[threadIdx.x][c] = 1.0f;
     }
     if (kNsq) {
         // new bounds of the block: every thread takes part (those past the last splat hold the neutral element),
@@ -976,6 +1010,9 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
     const int n_here = rest < kProjBlock ? (int)rest : kProjBlock;
     const float sh_reg = P.sh_reg_weight * (1.0f / (float)kY);
     constexpr int kPer = 3 * kCoef;
+    // the colour trust region is a uniform choice: two copies of the loops, so that the plain one stays free of the branch
+    auto phase2 = [&](auto ctl_tag) {
+    constexpr bool kCtl = decltype(ctl_tag)::value;
     if (kQuant) {
         // Quantized state (FusedProjectionBwdOptim_kernel.cuh:709-1030 at QUANT_BITS 8, VALUE_BITS 16): moments and
         // values of this block's cells are decoded against the block's old bounds, stepped in fp32, and encoded
@@ -992,11 +1029,18 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
             ssr_adamq_decode_with(code, old_mm, s_sqrt_g2[code >> 8], &m1, &m2);
             const float x = ssr_q16_decode(P.sh_value_packed[cell], old_lo, old_hi);
             const int j = k / 3, c = k - 3 * j;
-            const float v = s_Y[sp][j] * s_vc[sp][c] + sh_reg * x;
+            float v = s_Y[sp][j] * s_vc[sp][c] + sh_reg * x;
+            if (kCtl) v = v / s_ctl[sp][c];
             constexpr float kBeta1 = 0.9f, kBeta2 = 0.999f, kEps = 1e-15f;
             m1 = kBeta1 * m1 + (1.f - kBeta1) * v;
             m2 = kBeta2 * m2 + (1.f - kBeta2) * (v * v);
-            xn = x - ((P.lr_features_sh * s_b1c[sp]) * m1) / (ssr_sqrt(m2 * s_b2c[sp]) + kEps);
+            float delta = 0.0f - ((P.lr_features_sh * s_b1c[sp]) * m1) / (ssr_sqrt(m2 * s_b2c[sp]) + kEps);
+            if (kCtl) {   // FusedProjectionBwdOptim_kernel.cuh:787-794
+                const float clip = s_ctl[sp][3 + c];
+                delta = ssr_min(ssr_max(delta, -clip), clip);
+                delta = ssr_isfinite(delta) ? delta : 0.0f;
+            }
+            xn = x + delta;
         };
         float mn[3] = {1e30f, 1e30f, 1e30f}, mx[3] = {-1e30f, -1e30f, -1e30f};   // u, log_s, value
         {
@@ -1075,11 +1119,24 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
         const int64_t row = block0 + sp;
         float* xp = W.features_sh + row * W.sh_stride + i;
         const float x = *xp;
-        const float v = s_Y[sp][j] * s_vc[sp][c] + sh_reg * x;
+        float v = s_Y[sp][j] * s_vc[sp][c] + sh_reg * x;
+        if (kCtl) v = v / s_ctl[sp][c];     // FusedProjectionBwdOptim_kernel.cuh:694-705
         AdamD a;
         a.b1c = s_b1c[sp]; a.b2c = s_b2c[sp];
-        *xp = adam_step(x, v, P.lr_features_sh, a, P.g1.features_sh + row * P.g1.sh_stride + i, P.g2.features_sh + row * P.g2.sh_stride + i);
+        float* g1p = P.g1.features_sh + row * P.g1.sh_stride + i;
+        float* g2p = P.g2.features_sh + row * P.g2.sh_stride + i;
+        float m1 = *g1p, m2 = *g2p;
+        float delta = adam_core(0.0f, v, P.lr_features_sh, a, m1, m2);   // 0 - step: the step itself, exactly
+        if (kCtl) {
+            const float clip = s_ctl[sp][3 + c];
+            delta = ssr_min(ssr_max(delta, -clip), clip);
+            delta = ssr_isfinite(delta) ? delta : 0.0f;
+        }
+        *xp = x + delta;
+        *g1p = m1; *g2p = m2;
     }
+    };
+    if (ctl) phase2(std::true_type{}); else phase2(std::false_type{});
 }
 
 __global__ __launch_bounds__(kProjBlock) void packed_row_map_kernel(const int32_t* __restrict__ gaussian_ids, int64_t nnz,

@@ -155,7 +155,7 @@ class Engine:
 
     HYPER = ["lr_means", "lr_quats", "lr_scales", "lr_opacs", "lr_features_dc", "lr_features_sh", "max_gauss_ratio",
              "scale_regularization_weight", "mcmc_opacity_reg_weight", "mcmc_scale_reg_weight", "quat_norm_reg_weight",
-             "sh_reg_weight", "erank_reg_weight", "erank_reg_weight_s3"]
+             "sh_reg_weight", "erank_reg_weight", "erank_reg_weight_s3", "color_trust_linear", "eps_tr"]
 
     def backward_fused_optimizer(self, hyper, step, scale_agnostic_mean=False, quantization_level=0, non_sh_optim_bits=32):
         """Compositing backward, then the projection backward fused with the Adam step: the engine's

@@ -635,7 +635,7 @@ void fused_projection_bwd_optimizer_3dgs(
     const float max_gauss_ratio, const float scale_regularization_weight, const float mcmc_opacity_reg_weight,
     const float mcmc_scale_reg_weight, const float erank_reg_weight, const float erank_reg_weight_s3,
     const float quat_norm_reg_weight, const float sh_reg_weight, bool use_scale_agnostic_mean, bool color_trust_linear,
-    float, std::variant<int32_t, TorchTensorView> step, int quantization_level) {
+    float eps_tr, std::variant<int32_t, TorchTensorView> step, int quantization_level) {
     const char* w = "fused_projection_bwd_optimizer_3dgs: ";
     const bool is_packed = camera_ids.data_ptr() && gaussian_ids.data_ptr();   // src/kernels/optim/FusedProjectionBwdOptim.cu:160
     // quantization_level: 0 = fp32 SH and moments; 1 = 16-bit SH values, 8-bit moments
@@ -645,7 +645,6 @@ void fused_projection_bwd_optimizer_3dgs(
     if (quant && !(sh_packed && sh_quant_bounds && sh_value_packed && sh_value_bounds))
         throw std::runtime_error(std::string(w) + "quantization level 1 needs the packed SH state, the packed SH values and both bounds");
     if (!quant && (sh_packed || sh_value_packed)) throw std::runtime_error(std::string(w) + "packed SH buffers given at quantization level 0");
-    if (color_trust_linear) throw std::runtime_error(std::string(w) + "the colour trust region is not built in this backend");
     if (num_splats == 0) return;
     ssr_fpbo_params p;
     std::memset(&p, 0, sizeof(p));
@@ -683,6 +682,7 @@ void fused_projection_bwd_optimizer_3dgs(
     p.mcmc_opacity_reg_weight = mcmc_opacity_reg_weight; p.mcmc_scale_reg_weight = mcmc_scale_reg_weight;
     p.quat_norm_reg_weight = quat_norm_reg_weight; p.sh_reg_weight = sh_reg_weight;
     p.erank_reg_weight = erank_reg_weight; p.erank_reg_weight_s3 = erank_reg_weight_s3;
+    p.color_trust_linear = color_trust_linear ? 1 : 0; p.eps_tr = eps_tr;
     if (use_scale_agnostic_mean) {
         if (!radii.data_ptr()) throw std::runtime_error(std::string(w) + "the scale-agnostic mean step needs the forward's radii");
         p.scale_agnostic_radii = radii.data_ptr();

@@ -108,9 +108,9 @@ void projection_3dgs_backward(
     const std::optional<TorchTensorView> sh_value_bounds,
     const uint32_t num_sh_buffer, const int sh_value_bits, const int64_t sh_bounds_stride);
 
-// src/kernels/optim/FusedProjectionBwdOptim.cuh:18-62. fp32 parameters and Adam state, one camera,
-// non-packed; quantized state / value-quantized SH / effective-rank regularizer / scale-agnostic mean /
-// colour trust region throw.
+// src/kernels/optim/FusedProjectionBwdOptim.cuh:18-62: every argument is honoured (plain and packed rows,
+// all regularizers, scale-agnostic mean step, colour trust region, quantization levels 0 and 1 with the
+// non-SH quantized moments); one camera per call.
 void fused_projection_bwd_optimizer_3dgs(
     const int64_t num_splats, const int max_sh_degree,
     std::vector<DeviceTensorFloatND> splats_world,

@@ -278,7 +278,7 @@ void engine_backward_with_variants(TorchTensorView v_render_rgb, TorchTensorView
 }
 
 void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
-                                     TorchTensorView v_render_Ts, const float hyper[14], int step, bool scale_agnostic_mean,
+                                     TorchTensorView v_render_Ts, const float hyper[16], int step, bool scale_agnostic_mean,
                                      int quantization_level, int non_sh_optim_bits) {
     auto& E = engine();
     if (std::get<0>(E.fwd.renders).data_ptr() == nullptr)
@@ -359,7 +359,8 @@ void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorVi
         E.camera.model_str, E.camera.distortion_str, E.camera.dist_coeffs, cam_ids, gauss_ids, aabb, {}, E.grad.v_screen,
         E.optim.g1, E.optim.g2, sh_state, sh_state_bounds, sh_values, sh_value_bounds, non_sh,
         E.optim.radii, E.optim.densify_score, hyper[0], hyper[1], hyper[2], hyper[3], hyper[4], hyper[5], hyper[6], hyper[7],
-        hyper[8], hyper[9], hyper[12], hyper[13], hyper[10], hyper[11], scale_agnostic_mean, false, 0.0f, (int32_t)step, quantization_level);
+        hyper[8], hyper[9], hyper[12], hyper[13], hyper[10], hyper[11], scale_agnostic_mean, hyper[14] != 0.0f, hyper[15], (int32_t)step,
+        quantization_level);
 }
 
 void engine_copy_params_to_host(TorchTensorView means, TorchTensorView quats, TorchTensorView scales,
@@ -517,11 +518,11 @@ int ssrh_backward_with_variants(const float* v_rgb, const float* v_depth, const 
     });
 }
 
-int ssrh_backward_fused_optimizer(const float* v_rgb, const float* v_depth, const float* v_Ts, const float* hyper14, int step,
+int ssrh_backward_fused_optimizer(const float* v_rgb, const float* v_depth, const float* v_Ts, const float* hyper16, int step,
                                   int scale_agnostic_mean, int quantization_level, int non_sh_optim_bits) {
     return guard([&] {
         const int64_t C = engine().camera.num, H = engine().camera.height, W = engine().camera.width;
-        engine_backward_fused_optimizer(tv(v_rgb, 4, {C, H, W, 3}), tv(v_depth, 4, {C, H, W, 1}), tv(v_Ts, 4, {C, H, W, 1}), hyper14, step,
+        engine_backward_fused_optimizer(tv(v_rgb, 4, {C, H, W, 3}), tv(v_depth, 4, {C, H, W, 1}), tv(v_Ts, 4, {C, H, W, 1}), hyper16, step,
                                         scale_agnostic_mean != 0, quantization_level, non_sh_optim_bits);
     });
 }

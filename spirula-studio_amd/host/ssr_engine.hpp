@@ -84,14 +84,15 @@ void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorV
 // (engine().optim.use_fused_proj_bwd_optim, src/engine/EngineLoss.cpp:286-290): compositing backward,
 // then fused_projection_bwd_optimizer_3dgs on the engine's parameters with Adam moments kept in pool
 // slots (zero on first use). hyper: lr_means, lr_quats, lr_scales, lr_opacs, lr_dc, lr_sh,
-// max_gauss_ratio, scale_reg_w, mcmc_opacity_w, mcmc_scale_w, quat_norm_w, sh_reg_w, erank_w, erank_w_s3.
+// max_gauss_ratio, scale_reg_w, mcmc_opacity_w, mcmc_scale_w, quat_norm_w, sh_reg_w, erank_w, erank_w_s3,
+// color_trust_linear (0 / 1), eps_tr.
 // scale_agnostic_mean: OptimConfig::use_scale_agnostic_mean (the means step on the forward's radii).
 // quantization_level 1: SH values stay the 16-bit codes of set_sh_value_quant (one bound per 256 splats) and are
 // updated in place, their moments are 8-bit cells in pool slots (OptimConfig::quantization_level).
 // non_sh_optim_bits 16 (OptimConfig::non_sh_optim_bits; with a quantized level only): the moments of the five
 // non-SH tensors are 16-bit cells in pool slots instead of the fp32 arrays.
 void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorView v_render_depth,
-                                     TorchTensorView v_render_Ts, const float hyper[14], int step,
+                                     TorchTensorView v_render_Ts, const float hyper[16], int step,
                                      bool scale_agnostic_mean = false, int quantization_level = 0, int non_sh_optim_bits = 32);
 // engine_backward_from_render_grad with the cotangents of the variants of the forward that ran
 // (any may be a null view): distortion image, median depth, and a pixel weight map to accumulate

@@ -95,7 +95,7 @@ class FpboParams(C.Structure):
                 ("step", C.c_int32), ("steps", vp), ("erank_reg_weight", C.c_float), ("erank_reg_weight_s3", C.c_float),
                 ("scale_agnostic_radii", vp), ("packed_row_of", vp), ("sh_state_packed", vp), ("sh_state_bounds", vp),
                 ("sh_value_packed", vp), ("sh_value_bounds", vp), ("num_sh_buffer", C.c_uint32),
-                ("non_sh_packed", vp * 5), ("non_sh_bounds", vp * 5)]
+                ("non_sh_packed", vp * 5), ("non_sh_bounds", vp * 5), ("color_trust_linear", C.c_int32), ("eps_tr", C.c_float)]
 
 
 # every symbol include/ssr_backend.h declares: (name, restype, argtypes)

@@ -235,7 +235,7 @@ def projection_bwd(scene, aabb, vs, sh_degree=3, pose=False):
 
 HYPER = ["lr_means", "lr_quats", "lr_scales", "lr_opacs", "lr_features_dc", "lr_features_sh", "max_gauss_ratio",
          "scale_regularization_weight", "mcmc_opacity_reg_weight", "mcmc_scale_reg_weight", "quat_norm_reg_weight",
-         "sh_reg_weight", "erank_reg_weight", "erank_reg_weight_s3"]
+         "sh_reg_weight", "erank_reg_weight", "erank_reg_weight_s3", "color_trust_linear", "eps_tr"]
 WORLD_KEYS = ["means", "quats", "log_scales", "opacity_logits", "features_dc", "features_sh"]
 
 
@@ -408,6 +408,14 @@ def fused_projection_bwd_optimizer_q(scene, aabb, vs, params, q, g1, g2, hyper, 
         _p(None if steps is None else np.ascontiguousarray(steps, np.int32)),
         _p(None if radii is None else np.ascontiguousarray(radii, np.float32)))
     return score
+
+
+def colour_map(op, x):
+    """op 0: slope of the sRGB curve, 1: splat_dc_encode, 2: splat_dc_decode."""
+    x = np.ascontiguousarray(x, np.float32)
+    y = np.zeros_like(x)
+    lib().or_colour_map(C.c_int(op), C.c_int64(x.size), _p(x), _p(y))
+    return y
 
 
 def erank_reg(log_scales, w, w3):

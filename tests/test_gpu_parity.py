@@ -379,18 +379,18 @@ def test_tile_skip_mask(gpu, oracle):
     assert r["counts"].max() > 96
 
 
-@pytest.mark.parametrize("cfg", ["tiny", "cfg2", "equirect-steps", "fisheye-prism", "tiny-packed", "cfg4-packed"])
+@pytest.mark.parametrize("cfg", ["tiny", "cfg2", "equirect-steps", "fisheye-prism", "tiny-packed", "cfg4-packed", "tiny-ctl", "cfg2-ctl"])
 def test_fused_projection_bwd_optimizer(gpu, oracle, cfg):
     """K9 fused with Adam (fused_projection_bwd_optimizer_3dgs, fp32 state): both sides are fed the
     SAME screen gradients (the device's), so only the arithmetic of the fused kernel is compared."""
     rng = np.random.default_rng(11)
-    if cfg == "tiny":
+    if cfg in ("tiny", "tiny-ctl"):
         sc = gpu.scenes.tiny_scene(n=900, width=96, height=64, seed=61)
         sc.means[::4, 2] = -10.0
         sc.log_scales[5] = [-2.0, -4.5, -3.0]
         sc.features_dc[7] = [2.5, -2.2, 0.1]
         sc.quats *= np.linspace(0.5, 2.0, sc.n)[:, None].astype(np.float32)
-    elif cfg == "cfg2":
+    elif cfg in ("cfg2", "cfg2-ctl"):
         sc = gpu.scenes.make_scene(2, n=40000, width=480, height=270, parity_variant=True)
     elif cfg == "fisheye-prism":
         sc = _lens_scene(gpu, 1, 2, n=3000, seed=43)
@@ -429,6 +429,8 @@ def test_fused_projection_bwd_optimizer(gpu, oracle, cfg):
              mcmc_opacity_reg_weight=0.01, mcmc_scale_reg_weight=0.01, quat_norm_reg_weight=0.02, sh_reg_weight=0.05)
     if cfg in ("tiny", "cfg4-packed", "fisheye-prism"):   # with the effective-rank regularizer (needles and blobs both occur)
         h.update(erank_reg_weight=0.1, erank_reg_weight_s3=0.01)
+    if cfg.endswith("ctl"):   # the colour trust region, with rates at which its clips bind
+        h.update(color_trust_linear=1, eps_tr=1e-4, lr_features_dc=2.5e-2, lr_features_sh=1.25e-2)
     steps = rng.integers(1, 400, sc.n).astype(np.int32) if cfg == "equirect-steps" else None
     sa = cfg in ("tiny", "cfg4-packed", "cfg2")   # the scale-agnostic step of the means (the reference's default)
     dP, d1, d2, dscore = g.fused_optimizer(g1, g2, h, step=37, steps=steps, v_in=v_in, scale_agnostic=sa)
@@ -445,11 +447,21 @@ def test_fused_projection_bwd_optimizer(gpu, oracle, cfg):
         a, b = dP[k].astype(np.float64), P[k].astype(np.float64)
         assert np.abs(a - b).max() <= 0.02 * h[lrs[k]] * 40 + 1e-6, (k, float(np.abs(a - b).max()))
     assert np.allclose(dscore, score, rtol=1e-3, atol=1e-9)
+    if cfg.endswith("ctl"):   # the clipped steps themselves: both sides land on the same values, and the clips did bind
+        k0 = 0.28209479177387814
+        for k in ("features_dc", "features_sh"):
+            assert np.abs(dP[k].astype(np.float64) - P[k]).max() <= 3e-5, (k, float(np.abs(dP[k].astype(np.float64) - P[k]).max()))
+        opac = 1 / (1 + np.exp(-sc.opacity_logits.astype(np.float64)))
+        c_dc = np.maximum(k0 * sc.features_dc.astype(np.float64) + 0.5, (1 / 255.0) ** 2)
+        clip = k0 * np.sqrt(4e-4 * c_dc / np.maximum(opac, 1e-12)[:, None])
+        moved = np.abs(dP["features_sh"].astype(np.float64) - sc.features_sh)
+        assert (moved <= clip[:, None, :] * (1 + 1e-4) + 1e-7).all()
+        assert (moved >= clip[:, None, :] * (1 - 1e-3)).mean() > 0.02
     if packed:
         assert np.array_equal(g.host("row_of"), row_of)
 
 
-@pytest.mark.parametrize("cfg", ["tiny", "tiny-deg1-packed-steps", "cfg3", "tiny-nonsh", "cfg3-nonsh-packed-steps"])
+@pytest.mark.parametrize("cfg", ["tiny", "tiny-deg1-packed-steps", "cfg3", "tiny-nonsh", "cfg3-nonsh-packed-steps", "tiny-nonsh-ctl"])
 def test_fused_optimizer_quantized_sh_state(gpu, oracle, cfg):
     """The fused optimizer at the reference's quantization level 1: SH values as 16-bit codes and their Adam
     moments as 8-bit (u, log_s) cells, both against per-256-splat bounds that are recomputed every step
@@ -475,6 +487,8 @@ def test_fused_optimizer_quantized_sh_state(gpu, oracle, cfg):
     h = dict(lr_means=1.6e-4, lr_quats=1e-3, lr_scales=5e-3, lr_opacs=5e-2, lr_features_dc=2.5e-3, lr_features_sh=2.5e-3,
              max_gauss_ratio=6.0, scale_regularization_weight=0.01, mcmc_opacity_reg_weight=0.01, mcmc_scale_reg_weight=0.01,
              quat_norm_reg_weight=0.02, sh_reg_weight=0.05)
+    if cfg.endswith("ctl"):
+        h.update(color_trust_linear=1, eps_tr=1e-4, lr_features_dc=2.5e-2, lr_features_sh=1.25e-2)
     n, R = sc.n, 45
     nb = (n + 255) // 256
     steps = rng.integers(1, 60, n).astype(np.int32) if "steps" in cfg else None

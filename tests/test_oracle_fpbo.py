@@ -177,3 +177,105 @@ def test_effective_rank_regularizer(oracle):
     assert np.allclose(g, 2 / 3 * (np.array([0.25, 0.25, 0.5]) - 1 / 3), atol=1e-6)
     loss, g = oracle.erank_reg(np.array([-3.0, -3.0, -3.0]), 1.0, 0.0)
     assert loss == 0.0 and not np.any(g)               # rank 3: the log term is off
+
+
+def test_colour_maps_of_the_trust_region(oracle):
+    """ssr_srgb_slope against central differences of the sRGB transfer curve in float64; splat_dc_decode inverts
+    splat_dc_encode, the map has slope 1 at colour 0.5 and continues linearly below colour 0
+    (src/shaders/pixel_wise.slang:60-115)."""
+    x = np.concatenate([np.linspace(-0.2, 0.0031, 40), np.linspace(0.0032, 2.0, 400)]).astype(np.float32)
+    curve = lambda v: np.where(v < 0.0031308, 12.92 * v, 1.055 * np.maximum(v, 1e-300) ** (1 / 2.4) - 0.055)
+    h = 1e-7
+    want = (curve(x.astype(np.float64) + h) - curve(x.astype(np.float64) - h)) / (2 * h)
+    got = oracle.colour_map(0, x)
+    keep = np.abs(x.astype(np.float64) - 0.0031308) > 1e-5      # the curve's two branches meet with different slopes
+    assert np.abs(got[keep] / want[keep] - 1).max() < 2e-5
+    assert np.all(got[x < 0.0031308] == np.float32(12.92))
+    dc = np.linspace(-4.0, 6.0, 2001).astype(np.float32)      # colours from below 0 to above 2
+    enc = oracle.colour_map(1, dc)
+    back = oracle.colour_map(2, enc)
+    assert np.abs(back - dc).max() < 5e-6
+    assert np.all(np.diff(enc) > 0)
+    k = 0.28209479177387814
+    # slope 1 at colour 0.5 (dc = 0) and constant slope k / a * s / k = s / a below colour 0
+    e = oracle.colour_map(1, np.array([-1e-3, 1e-3], np.float32)).astype(np.float64)
+    assert abs((e[1] - e[0]) / 2e-3 - 1.0) < 2e-3
+    a = 1 / 255.0
+    s = np.sqrt(0.5 + a * a)
+    low = oracle.colour_map(1, np.array([-3.0, -2.5], np.float32)).astype(np.float64)      # colours -0.35, -0.21
+    assert abs((low[1] - low[0]) / 0.5 - s / a) < 1e-2 * s / a
+    # float64 definitions
+    u = k * dc.astype(np.float64) + 0.5
+    w = np.where(u >= 0, 2 * np.sqrt(np.maximum(u, 0) + a * a), 2 * a + u / a)
+    want_enc = (w - 2 * s) * s / k
+    # below colour 0 the map multiplies the fp32 rounding of the colour by s / (a k) = 640
+    assert (np.abs(enc - want_enc) <= 2e-6 * np.abs(want_enc) + 1e-4).all()
+
+
+@pytest.mark.parametrize("quantized", [False, True])
+def test_colour_trust_region_against_float64(pkg, oracle, quantized):
+    """color_trust_linear (FusedProjectionBwdOptim_kernel.cuh:551-596,651-705,774-794): DC and SH steps of the oracle
+    against a float64 restatement built from the pinned gradients, the float64 colour maps and the clip radii."""
+    sc = pkg.scenes.tiny_scene(n=300, width=96, height=64, seed=57)
+    sc.features_dc[3] = [-2.0, 0.4, 3.0]          # a colour below 0 (linear continuation) and one above 1
+    sc.opacity_logits[5] = -9.0                   # nearly transparent: wide clip
+    n = sc.n
+    rng = np.random.default_rng(4)
+    h = dict(lr_means=1.6e-4, lr_quats=1e-3, lr_scales=5e-3, lr_opacs=5e-2, lr_features_dc=2.5e-2, lr_features_sh=1.25e-2,
+             max_gauss_ratio=6.0, scale_regularization_weight=0.01, mcmc_opacity_reg_weight=0.01, mcmc_scale_reg_weight=0.01,
+             quat_norm_reg_weight=0.02, sh_reg_weight=0.05, color_trust_linear=1.0, eps_tr=1e-4)     # large rates: the clips bind
+    step = 5
+    k0 = 0.28209479177387814
+    if quantized:
+        q = oracle.quantize_sh_state(sc.features_sh)
+        sc.features_sh = oracle.decode_sh_values(q, n)
+    r = oracle.pipeline(sc)
+    P = {k: np.ascontiguousarray(getattr(sc, k), np.float32).copy() for k in oracle.WORLD_KEYS}
+    g1 = {k: rng.normal(0, 1e-3, P[k].shape).astype(np.float32) for k in oracle.WORLD_KEYS}
+    g2 = {k: rng.uniform(1e-7, 1e-5, P[k].shape).astype(np.float32) for k in oracle.WORLD_KEYS}
+    P0 = {k: v.astype(np.float64) for k, v in P.items()}
+    G1 = {k: v.astype(np.float64) for k, v in g1.items()}
+    G2 = {k: v.astype(np.float64) for k, v in g2.items()}
+    if quantized:
+        G1["features_sh"][:] = 0; G2["features_sh"][:] = 0        # the quantized state starts from zero moments
+        oracle.fused_projection_bwd_optimizer_q(sc, r["proj"]["aabb"], r["vscreen"], P, q, g1, g2, h, step=step)
+        new_sh = oracle.decode_sh_values(q, n).astype(np.float64)
+        tol_sh = ((q["value_bounds"][:, 1] - q["value_bounds"][:, 0]) / 65535).repeat(256)[:n, None, None] * 0.51 + 1e-6
+    else:
+        oracle.fused_projection_bwd_optimizer(sc, r["proj"]["aabb"], r["vscreen"], P, g1, g2, h, step=step)
+        new_sh = P["features_sh"].astype(np.float64)
+        tol_sh = 1e-6
+    gr = r["grads"]
+    c1, c2 = 1 / (1 - B1 ** step), 1 / (1 - B2 ** step)
+    a = 1 / 255.0
+    s = np.sqrt(0.5 + a * a)
+    enc = lambda dc: ((np.where(k0 * dc + 0.5 >= 0, 2 * np.sqrt(np.maximum(k0 * dc + 0.5, 0) + a * a), 2 * a + (k0 * dc + 0.5) / a)) - 2 * s) * s / k0
+    def dec(x):
+        w = x * k0 / s + 2 * s
+        return (np.where(w >= 2 * a, 0.25 * w * w - a * a, (w - 2 * a) * a) - 0.5) / k0
+    slope = lambda c: np.where(c < 0.0031308, 12.92, 1.055 / 2.4 * np.maximum(c, 1e-300) ** (1 / 2.4 - 1))
+    n_clipped_dc = n_clipped_sh = 0
+    for g in range(n):
+        dc, sh, lo = P0["features_dc"][g], P0["features_sh"][g], P0["opacity_logits"][g]
+        opac = 1 / (1 + np.exp(-lo))
+        c_dc = k0 * dc + 0.5
+        sl = slope(c_dc)
+        lim = 0.5 / k0
+        v = (gr["v_dc"][g].astype(np.float64) + h["sh_reg_weight"] * (np.maximum(dc - lim, 0) + np.minimum(dc + lim, 0))) / sl
+        m1 = B1 * G1["features_dc"][g] + (1 - B1) * v
+        m2 = B2 * G2["features_dc"][g] + (1 - B2) * v * v
+        delta = -h["lr_features_dc"] * c1 * m1 / (np.sqrt(m2 * c2) + EPS)
+        clip = k0 * np.sqrt(2 * h["eps_tr"] / max(opac, 1e-12))
+        n_clipped_dc += int((np.abs(delta) > clip).sum())
+        want = dec(enc(dc) + np.clip(delta, -clip, clip))
+        assert np.allclose(P["features_dc"][g], want, rtol=2e-5, atol=2e-5), (g, P["features_dc"][g], want)
+        v = (gr["v_sh"][g].astype(np.float64) + h["sh_reg_weight"] / 15 * sh) / sl[None, :]
+        m1 = B1 * G1["features_sh"][g] + (1 - B1) * v
+        m2 = B2 * G2["features_sh"][g] + (1 - B2) * v * v
+        delta = -h["lr_features_sh"] * c1 * m1 / (np.sqrt(m2 * c2) + EPS)
+        clip = k0 * np.sqrt(4 * h["eps_tr"] * np.maximum(c_dc, a * a) / max(opac, 1e-12))
+        n_clipped_sh += int((np.abs(delta) > clip[None, :]).sum())
+        want = sh + np.clip(delta, -clip[None, :], clip[None, :])
+        t = tol_sh if np.isscalar(tol_sh) else tol_sh[g]
+        assert (np.abs(new_sh[g] - want) <= t + 2e-5 * np.abs(want)).all(), (g, np.abs(new_sh[g] - want).max())
+    assert n_clipped_dc > 20 and n_clipped_sh > 200        # the trust region did bind
