@@ -117,6 +117,10 @@ typedef struct {
      * 16-byte aligned, [C*N,12]. The compositing kernels gather a splat from it with one or two
      * cache lines instead of five (same values, so same results). */
     float* packed_rows;
+    /* The antialiased ("mip") variant of the primitive (src/shaders/primitive_3dgs.slang:528-543, the runtime
+     * `antialiased` argument of the same projection function): screen-space blur 0.1 instead of 0.3 and the opacity
+     * multiplied by sqrt(det cov2d / det (cov2d + blur)); everything after the projection is unchanged. */
+    int32_t antialiased;
 } ssr_projection_fwd_params;
 int ssr_projection_fwd(const ssr_projection_fwd_params* p, ssr_stream_t stream);
 
@@ -149,6 +153,10 @@ typedef struct {
     ssr_screen screen;          /* [nnz] rows */
     int64_t* tiles_per_splat;   /* optional [nnz]: fused K2 */
     float* packed_rows;         /* optional [nnz,12]: 48-byte fragment rows, as in ssr_projection_fwd_params */
+    /* The antialiased ("mip") variant of the primitive (src/shaders/primitive_3dgs.slang:528-543, the runtime
+     * `antialiased` argument of the same projection function): screen-space blur 0.1 instead of 0.3 and the opacity
+     * multiplied by sqrt(det cov2d / det (cov2d + blur)); everything after the projection is unchanged. */
+    int32_t antialiased;
 } ssr_projection_packed_params;
 size_t ssr_projection_packed_scratch_bytes(int64_t num_splats);
 int ssr_projection_packed_mask(const ssr_projection_packed_params* p, ssr_stream_t stream);
@@ -311,6 +319,10 @@ typedef struct {
      * 0..2, columns 0..2) and dL/dt (column 3) are ADDED to it (caller zero-fills), the last row is not touched.
      * Both the projection and the SH view direction contribute. Computed by a second pass over the splats. */
     float* v_viewmat;
+    /* The antialiased ("mip") variant of the primitive (src/shaders/primitive_3dgs.slang:528-543, the runtime
+     * `antialiased` argument of the same projection function): screen-space blur 0.1 instead of 0.3 and the opacity
+     * multiplied by sqrt(det cov2d / det (cov2d + blur)); everything after the projection is unchanged. */
+    int32_t antialiased;
 } ssr_projection_bwd_params;
 int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream_t stream);
 
@@ -378,6 +390,10 @@ typedef struct {
      * clipped to kSh0 sqrt(4 eps_tr colour / opacity) per channel. */
     int32_t color_trust_linear;
     float eps_tr;
+    /* The antialiased ("mip") variant of the primitive (src/shaders/primitive_3dgs.slang:528-543, the runtime
+     * `antialiased` argument of the same projection function): screen-space blur 0.1 instead of 0.3 and the opacity
+     * multiplied by sqrt(det cov2d / det (cov2d + blur)); everything after the projection is unchanged. */
+    int32_t antialiased;
 } ssr_fpbo_params;
 int ssr_fused_projection_bwd_optimizer(const ssr_fpbo_params* p, ssr_stream_t stream);
 /* row_of[g] = i where gaussian_ids[i] == g, -1 for splats without a packed row (one camera, so ids

@@ -36,6 +36,7 @@ struct Cam {
     float fx, fy, cx, cy;
     int tier;
     float dc[8];
+    bool aa;   // antialiased ("mip") variant
 };
 
 // PINHOLE without lens distortion and EQUIRECTANGULAR are written out by hand below; the other
@@ -53,6 +54,7 @@ Cam load_cam(const or_camera* c) {
     k.fx = c->fx; k.fy = c->fy; k.cx = c->cx; k.cy = c->cy;
     k.tier = c->distortion;
     for (int i = 0; i < 8; i++) k.dc[i] = (c->distortion != OR_LENS_NONE) ? c->dist_coeffs[i] : 0.0f;
+    k.aa = c->antialiased != 0;
     return k;
 }
 
@@ -191,6 +193,7 @@ struct Proj {
     // intermediates reused by the VJP
     float mc[3], qn[4], qinv, s[3], Rq[3][3], M[3][3], J[2][3], covc[3][3];
     float c2[2][2];   // blurred 2D covariance
+    float sig, comp, det_orig, det_blur, c2o[2];   // antialiased variant: sigmoid(logit), compensation, determinants, pre-blur diagonal
     bool clamp_lo[2], clamp_hi[2];
 };
 
@@ -328,11 +331,21 @@ Proj project(const Cam& cam, const float mean[3], const float quat[4], const flo
         const float seen = p.opac * ssr_exp(-0.5f * q);
         if (z < 0.0f && seen > kAlphaThreshold) return p;
     }
-    // add_blur, primitive_3dgs.slang:398-405 (not antialiased: eps 0.3)
-    p.c2[0][0] = p.c2[0][0] + 0.3f;
-    p.c2[1][1] = p.c2[1][1] + 0.3f;
+    // add_blur, primitive_3dgs.slang:398-405,528-543: eps 0.3, or 0.1 in the antialiased variant, which also scales
+    // the opacity by sqrt(max(0, det before / det after))
+    const float eps2d = cam.aa ? 0.1f : 0.3f;
+    p.det_orig = p.c2[0][0] * p.c2[1][1] - p.c2[0][1] * p.c2[1][0];
+    p.c2o[0] = p.c2[0][0]; p.c2o[1] = p.c2[1][1];
+    p.c2[0][0] = p.c2[0][0] + eps2d;
+    p.c2[1][1] = p.c2[1][1] + eps2d;
     float det = p.c2[0][0] * p.c2[1][1] - p.c2[0][1] * p.c2[1][0];
+    p.det_blur = det;
     if (!assume_valid && det <= 0.f) return p;
+    p.sig = p.opac; p.comp = 1.0f;
+    if (cam.aa) {
+        p.comp = ssr_sqrt(ssr_max(0.0f, p.det_orig / det));
+        p.opac = p.opac * p.comp;
+    }
     float invdet = 1.0f / det;   // inverse(), projection_utils.slang:164-174
     p.conic[0] = p.c2[1][1] * invdet;
     p.conic[1] = (-p.c2[0][1]) * invdet;
@@ -1399,6 +1412,18 @@ void or_projection_bwd_pose(int64_t N, int sh_degree, const float* means, const 
         vC[1][1] = inv * g00 + c00 * v_det;
         vC[0][1] = -(inv * g01) - c10 * v_det;
         vC[1][0] = -(c01 * v_det);
+        if (cam.aa) {
+            // opacity = sigmoid(logit) * sqrt(max(0, det_orig / det_blur)): through both determinants to the 2D covariance
+            const float ratio = p.det_orig / p.det_blur;
+            const float v_comp = v_opac[g] * p.sig;
+            const float v_ratio = ratio > 0.0f ? v_comp * (0.5f / ssr_sqrt(ssr_max(1e-7f, ratio))) : 0.0f;
+            const float v_do = v_ratio / p.det_blur;
+            const float v_db = -((v_ratio * p.det_orig) / (p.det_blur * p.det_blur));
+            vC[0][0] += v_do * p.c2o[1] + v_db * c11;
+            vC[1][1] += v_do * p.c2o[0] + v_db * c00;
+            vC[0][1] += (v_do + v_db) * (-c10);
+            vC[1][0] += (v_do + v_db) * (-c01);
+        }
         // --- cov2d = J covc J^T ---
         float vJ[2][3], vS[3][3];
         for (int i = 0; i < 2; i++)
@@ -1516,7 +1541,7 @@ void or_projection_bwd_pose(int64_t N, int sh_degree, const float* means, const 
         const float qd = ((p.qn[0] * vqn[0] + p.qn[1] * vqn[1]) + p.qn[2] * vqn[2]) + p.qn[3] * vqn[3];
         float vquat[4];
         for (int i = 0; i < 4; i++) vquat[i] = (vqn[i] - p.qn[i] * qd) * p.qinv;
-        const float vlogit = v_opac[g] * (p.opac * (1.0f - p.opac));
+        const float vlogit = (v_opac[g] * p.comp) * (p.sig * (1.0f - p.sig));
 
         // --- SH colour VJP, harmonics.slang:373-649,1087-1126 ---
         float coef[45];

@@ -36,6 +36,8 @@ typedef struct {
     float fx, fy, cx, cy;
     int32_t distortion;     /* OR_LENS_* */
     float dist_coeffs[8];   /* in the tier's own order, src/shaders/projection_utils.slang:242-295 */
+    int32_t antialiased;    /* the "mip" variant of the primitive (the projection function's runtime `antialiased`
+                               argument, src/shaders/primitive_3dgs.slang:528-543); carried here for convenience */
 } or_camera;
 
 typedef struct {

@@ -59,7 +59,8 @@ __global__ __launch_bounds__(kProjBlock) void projection_fwd_kernel(ssr_projecti
     __syncthreads();
     const int64_t block0 = (int64_t)blockIdx.x * kProjBlock;
     const int64_t g = block0 + threadIdx.x;
-    const CamD cam = load_camera(P.camera);
+    CamD cam = load_camera(P.camera);
+    cam.aa = P.antialiased != 0;
     if (g < P.num_splats) {
         float mean[3], quat[4], ls[3], logit;
         load_splat(P.world, g, mean, quat, ls, logit);
@@ -192,7 +193,8 @@ __global__ __launch_bounds__(kProjBlock) void projection_packed_mask_kernel(ssr_
     __shared__ int s_wave[kProjBlock / 64];
     const int64_t block0 = (int64_t)blockIdx.x * kProjBlock;
     const int64_t g = block0 + threadIdx.x;
-    const CamD cam = load_camera(P.camera);
+    CamD cam = load_camera(P.camera);
+    cam.aa = P.antialiased != 0;
     bool vis = false;
     ProjD p;
     float bb[4] = {0.f, 0.f, 0.f, 0.f};
@@ -282,7 +284,8 @@ __global__ __launch_bounds__(kProjBlock) void projection_packed_emit_kernel(ssr_
     }
     const int64_t src = lo * kProjBlock + (j - S.block_offsets[lo]);
     const int64_t N = P.num_splats;
-    const CamD cam = load_camera(P.camera);
+    CamD cam = load_camera(P.camera);
+    cam.aa = P.antialiased != 0;
     const float4 bb4 = S.aabb[src];
     const float2 xy = S.xy[src];
     const float conic[3] = {S.conic[src], S.conic[N + src], S.conic[2 * N + src]};
@@ -368,6 +371,19 @@ __device__ __forceinline__ void projection_vjp(const CamD& cam, const ssr_world&
     vC[1][1] = inv * g00 + c00 * v_det;
     vC[0][1] = -(inv * g01) - c10 * v_det;
     vC[1][0] = -(c01 * v_det);
+    if (cam.aa) {
+        // opacity = sigmoid(logit) * sqrt(max(0, det_orig / det_blur)): the gradient of the opacity reaches the 2D
+        // covariance through both determinants (sqrt derivative guarded at 1e-7, max(0, .) passes where positive)
+        const float ratio = p.det_orig / p.det_blur;
+        const float v_comp = VS.opac[VS.s_opac * r] * p.sig;
+        const float v_ratio = ratio > 0.0f ? v_comp * (0.5f / ssr_sqrt(ssr_max(1e-7f, ratio))) : 0.0f;
+        const float v_do = v_ratio / p.det_blur;
+        const float v_db = -((v_ratio * p.det_orig) / (p.det_blur * p.det_blur));
+        vC[0][0] += v_do * p.c2o[1] + v_db * c11;
+        vC[1][1] += v_do * p.c2o[0] + v_db * c00;
+        vC[0][1] += (v_do + v_db) * (-c10);
+        vC[1][0] += (v_do + v_db) * (-c01);
+    }
     // cov2d = J covc J^T
     float vJ[2][3], vS[3][3];
 #pragma unroll
@@ -504,7 +520,7 @@ __device__ __forceinline__ void projection_vjp(const CamD& cam, const ssr_world&
     float vquat[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) vquat[i] = (vqn[i] - p.qn[i] * qd) * p.qinv;
-    const float vlogit = VS.opac[VS.s_opac * r] * (p.opac * (1.0f - p.opac));
+    const float vlogit = (VS.opac[VS.s_opac * r] * p.comp) * (p.sig * (1.0f - p.sig));
 
     // SH colour VJP (src/shaders/harmonics.slang:373-649,1087-1126)
     float coef[kCoef > 0 ? 3 * kCoef : 1];
@@ -623,7 +639,8 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
         }
         return;
     }
-    const CamD cam = load_camera(P.camera);
+    CamD cam = load_camera(P.camera);
+    cam.aa = P.antialiased != 0;
     WorldGradD wg;
     float* vsh = V.features_sh + g * (int64_t)V.sh_stride;
     projection_vjp<kDegree, kLens>(cam, P.world, P.sh, g, vscreen_of(P.v_screen, P.v_rows), r, wg, [&](int j, float Yj, const float vc[3]) {
@@ -668,7 +685,8 @@ __global__ __launch_bounds__(kProjBlock) void projection_pose_bwd_kernel(ssr_pro
         float4 bb = make_float4(0.f, 0.f, 1.f, 1.f);
         if (!P.packed_gaussian_ids) bb = reinterpret_cast<const float4*>(P.aabb)[g];
         if (!(bb.z <= bb.x || bb.w <= bb.y)) {
-            const CamD cam = load_camera(P.camera);
+            CamD cam = load_camera(P.camera);
+    cam.aa = P.antialiased != 0;
             WorldGradD wg;
             PoseGradD pg;
             projection_vjp<kDegree, kLens, true>(cam, P.world, P.sh, g, vscreen_of(P.v_screen, P.v_rows), r, wg,
@@ -815,7 +833,8 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
         float4 bb = make_float4(0.f, 0.f, 0.f, 0.f);
         if (row >= 0) bb = reinterpret_cast<const float4*>(P.aabb)[row];
         if (!(bb.z <= bb.x || bb.w <= bb.y)) {   // FusedProjectionBwdOptim_kernel.cuh:271-272
-            const CamD cam = load_camera(P.camera);
+            CamD cam = load_camera(P.camera);
+    cam.aa = P.antialiased != 0;
             WorldGradD pg;
             ssr_sh_quant none;
             none.codec = SSR_SH_F32; none.packed = nullptr; none.bounds = nullptr; none.bounds_stride = 0;

@@ -22,6 +22,7 @@ struct CamD {
     float t[3];
     float fx, fy, cx, cy;
     float dc[8];       // lens coefficients (zero without distortion)
+    bool aa;           // antialiased ("mip") variant: set by the kernel from its parameters, not part of the camera
 };
 
 // PINHOLE without lens distortion and EQUIRECTANGULAR have hand-written Jacobians; every other pair
@@ -33,6 +34,7 @@ __host__ __device__ __forceinline__ bool camera_needs_lens_path(int model, int t
 __device__ __forceinline__ CamD load_camera(const ssr_camera& c) {
     // src/kernels/projection/ProjectionFwd_kernel.cuh:52-60 (row-major [R t; 0 1])
     CamD k;
+    k.aa = false;
     k.model = c.camera_model;
     k.Wf = (float)c.width; k.Hf = (float)c.height;
 #pragma unroll
@@ -53,6 +55,7 @@ struct ProjD {
     float aabb[4];
     float sort_depth, radius;
     float xy[2], depth, conic[3], opac;
+    float sig, comp, det_orig, det_blur, c2o[2];   // antialiased variant: sigmoid(logit), the compensation factor, both determinants, the diagonal before the blur
     // intermediates for the VJP
     float mc[3], qn[4], qinv, s[3], Rq[3][3], M[3][3], J[2][3], covc[3][3], c2[2][2];
     bool clamp_lo[2], clamp_hi[2];
@@ -194,10 +197,21 @@ __device__ __forceinline__ void project(const CamD& cam, const float mean[3], co
         const float seen = p.opac * ssr_exp(-0.5f * q);
         if (z < 0.0f && seen > kAlphaThreshold) return;
     }
-    p.c2[0][0] = p.c2[0][0] + 0.3f;   // add_blur, not antialiased
-    p.c2[1][1] = p.c2[1][1] + 0.3f;
+    // add_blur (src/shaders/primitive_3dgs.slang:398-405,528-543): the antialiased variant blurs less and scales
+    // the opacity by sqrt(det before / det after)
+    const float eps2d = cam.aa ? 0.1f : 0.3f;
+    p.det_orig = p.c2[0][0] * p.c2[1][1] - p.c2[0][1] * p.c2[1][0];
+    p.c2o[0] = p.c2[0][0]; p.c2o[1] = p.c2[1][1];
+    p.c2[0][0] = p.c2[0][0] + eps2d;
+    p.c2[1][1] = p.c2[1][1] + eps2d;
     const float det = p.c2[0][0] * p.c2[1][1] - p.c2[0][1] * p.c2[1][0];
+    p.det_blur = det;
     if (!kAssumeValid && det <= 0.f) return;
+    p.sig = p.opac; p.comp = 1.0f;
+    if (cam.aa) {
+        p.comp = ssr_sqrt(ssr_max(0.0f, p.det_orig / det));
+        p.opac = p.opac * p.comp;
+    }
     const float invdet = 1.0f / det;
     p.conic[0] = p.c2[1][1] * invdet;
     p.conic[1] = (-p.c2[0][1]) * invdet;

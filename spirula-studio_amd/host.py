@@ -130,7 +130,9 @@ class Engine:
         check(self.h.ssrh_set_tile_mask(mask.ctypes.data, mask.shape[0], mask.shape[1]))
 
     def forward(self):
-        check(self.h.ssrh_forward_3dgs(b"3dgs", self.sh_degree, int(self.packed_projection), int(self.output_median),
+        """The scene's `antialiased` flag selects the reference's "mip" primitive."""
+        primitive = b"mip" if getattr(self.sc, "antialiased", False) else b"3dgs"
+        check(self.h.ssrh_forward_3dgs(primitive, self.sh_degree, int(self.packed_projection), int(self.output_median),
                                        int(self.dist_type)))
 
     def set_variants(self, dist_type=0, median=False):

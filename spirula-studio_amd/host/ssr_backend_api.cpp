@@ -6,6 +6,11 @@
 
 #include "../../include/ssr_backend.h"
 
+// set for the duration of a projection_mip_* / fused_projection_bwd_optimizer_mip call (ssr_detail::AntialiasedScope)
+static thread_local bool g_antialiased = false;
+ssr_detail::AntialiasedScope::AntialiasedScope() { g_antialiased = true; }
+ssr_detail::AntialiasedScope::~AntialiasedScope() { g_antialiased = false; }
+
 namespace {
 
 [[noreturn]] void throw_last(const char* where) {
@@ -232,6 +237,7 @@ projection_3dgs_forward(const int64_t num_splats, const int max_sh_degree,
     std::memset(&p, 0, sizeof(p));
     p.num_splats = num_splats;
     p.sh_degree = max_sh_degree;
+    p.antialiased = g_antialiased ? 1 : 0;
     p.world = world_of(in_splats);
     p.sh = sh_of(sh_value_packed, sh_value_bounds, num_sh_buffer, sh_value_bits, sh_bounds_stride);
     p.camera = camera_of(camera_model, distortion, dist_coeffs, viewmats, intrins, image_width, image_height);
@@ -293,6 +299,7 @@ projection_3dgs_packed_forward(const int64_t num_splats, const int max_sh_degree
     std::memset(&p, 0, sizeof(p));
     p.num_splats = num_splats;
     p.sh_degree = max_sh_degree;
+    p.antialiased = g_antialiased ? 1 : 0;
     p.world = world_of(in_splats);
     p.sh = sh_of(sh_value_packed, sh_value_bounds, num_sh_buffer, sh_value_bits, sh_bounds_stride);
     p.camera = camera_of(camera_model, distortion, dist_coeffs, viewmats, intrins, image_width, image_height);
@@ -599,6 +606,7 @@ void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
     std::memset(&p, 0, sizeof(p));
     p.num_splats = num_splats;
     p.sh_degree = max_sh_degree;
+    p.antialiased = g_antialiased ? 1 : 0;
     p.world = world_of(splats_world);
     p.sh = sh_of(sh_value_packed, sh_value_bounds, num_sh_buffer, sh_value_bits, sh_bounds_stride);
     p.camera = camera_of(camera_model, distortion, dist_coeffs, viewmats, intrins, image_width, image_height);
@@ -650,6 +658,7 @@ void fused_projection_bwd_optimizer_3dgs(
     std::memset(&p, 0, sizeof(p));
     p.num_splats = num_splats;
     p.sh_degree = max_sh_degree;
+    p.antialiased = g_antialiased ? 1 : 0;
     p.world = world_of(splats_world);
     if (quant) {
         p.sh_state_packed = (uint16_t*)std::get<0>(*sh_packed);

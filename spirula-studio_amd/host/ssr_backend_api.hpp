@@ -139,6 +139,19 @@ void fused_projection_bwd_optimizer_3dgs(
     bool use_scale_agnostic_mean, bool color_trust_linear, float eps_tr,
     std::variant<int32_t, TorchTensorView> step, int quantization_level);
 
+// The antialiased ("mip") primitive: the reference's projection_mip_* / rasterize_to_pixels_mip_* /
+// fused_projection_bwd_optimizer_mip (src/kernels/projection/ProjectionFwd.cuh, ProjectionPackedFwd.cuh, ProjectionBwd.cuh,
+// src/kernels/raster/RasterizationFwd.cuh, RasterizationBwd.cuh, src/kernels/optim/FusedProjectionBwdOptim.cuh) are the 3dgs
+// functions instantiated with antialiased = true (src/primitives/Primitive3DGS.cuh:20): same arguments, the projection's
+// runtime flag set; compositing does not depend on it.
+namespace ssr_detail { struct AntialiasedScope { AntialiasedScope(); ~AntialiasedScope(); }; }
+template <class... A> auto projection_mip_forward(A&&... a) { ssr_detail::AntialiasedScope s; return projection_3dgs_forward(std::forward<A>(a)...); }
+template <class... A> auto projection_mip_packed_forward(A&&... a) { ssr_detail::AntialiasedScope s; return projection_3dgs_packed_forward(std::forward<A>(a)...); }
+template <class... A> void projection_mip_backward(A&&... a) { ssr_detail::AntialiasedScope s; projection_3dgs_backward(std::forward<A>(a)...); }
+template <class... A> void fused_projection_bwd_optimizer_mip(A&&... a) { ssr_detail::AntialiasedScope s; fused_projection_bwd_optimizer_3dgs(std::forward<A>(a)...); }
+template <class... A> auto rasterize_to_pixels_mip_fwd(A&&... a) { return rasterize_to_pixels_3dgs_fwd(std::forward<A>(a)...); }
+template <class... A> auto rasterize_to_pixels_mip_bwd(A&&... a) { return rasterize_to_pixels_3dgs_bwd(std::forward<A>(a)...); }
+
 // ---- extensions of this backend (no counterpart in the reference) ----
 namespace ssr_ext {
 // Work the reference does that this backend can skip with identical results:

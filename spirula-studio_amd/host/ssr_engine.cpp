@@ -121,7 +121,11 @@ void engine_set_tile_mask(TorchTensorView mask) {
 }
 
 void forward_3dgs(std::string primitive, int sh_degree, bool packed, bool output_median, int dist_type_int) {
-    if (primitive != "3dgs") throw std::runtime_error("forward_3dgs: primitive '" + primitive + "' is not built in this backend");
+    // "mip" is the antialiased 3dgs (src/engine/EngineForward.cpp:135,181,268 call the *_mip_* instantiations)
+    if (primitive != "3dgs" && primitive != "mip")
+        throw std::runtime_error("forward_3dgs: primitive '" + primitive + "' is not built in this backend");
+    std::optional<ssr_detail::AntialiasedScope> antialiased;
+    if (primitive == "mip") antialiased.emplace();
     auto& E = engine();
     if (!E.world.initialized) throw std::runtime_error("forward_3dgs: set_data_3dgs must be called first");
     E.primitive = primitive; E.sh_degree = sh_degree; E.packed = packed;
@@ -239,6 +243,8 @@ void engine_backward_from_render_grad(TorchTensorView v_render_rgb, TorchTensorV
         DeviceTensorFloatND(E.grad.means), DeviceTensorFloatND(E.grad.quats), DeviceTensorFloatND(E.grad.scales),
         DeviceTensorFloatND((float*)E.grad.opacities.data_ptr(), {E.grad.opacities.size(), 1}),
         DeviceTensorFloatND(E.grad.features_dc), DeviceTensorFloatND(E.grad.features_sh)};
+    std::optional<ssr_detail::AntialiasedScope> antialiased;
+    if (E.primitive == "mip") antialiased.emplace();
     projection_3dgs_backward(
         E.cur_num_splats, E.sh_degree, E.fwd.splats_w, E.camera.viewmats, E.camera.intrins, (uint32_t)W, (uint32_t)H,
         E.camera.model_str, E.camera.distortion_str, E.camera.dist_coeffs, E.fwd.camera_ids, E.fwd.gaussian_ids,
@@ -267,6 +273,8 @@ void engine_backward_with_variants(TorchTensorView v_render_rgb, TorchTensorView
         DeviceTensorFloatND(E.grad.means), DeviceTensorFloatND(E.grad.quats), DeviceTensorFloatND(E.grad.scales),
         DeviceTensorFloatND((float*)E.grad.opacities.data_ptr(), {E.grad.opacities.size(), 1}),
         DeviceTensorFloatND(E.grad.features_dc), DeviceTensorFloatND(E.grad.features_sh)};
+    std::optional<ssr_detail::AntialiasedScope> antialiased;
+    if (E.primitive == "mip") antialiased.emplace();
     projection_3dgs_backward(
         E.cur_num_splats, E.sh_degree, E.fwd.splats_w, E.camera.viewmats, E.camera.intrins, (uint32_t)E.camera.width,
         (uint32_t)E.camera.height, E.camera.model_str, E.camera.distortion_str, E.camera.dist_coeffs, E.fwd.camera_ids,
@@ -354,6 +362,8 @@ void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorVi
         backend::memset_async(zero, 0, (size_t)(E.cur_num_splats * 4) * sizeof(float));
         aabb = DeviceTensorFloatND(zero, {E.cur_num_splats, 4});
     }
+    std::optional<ssr_detail::AntialiasedScope> antialiased;
+    if (E.primitive == "mip") antialiased.emplace();
     fused_projection_bwd_optimizer_3dgs(
         E.cur_num_splats, E.sh_degree, E.fwd.splats_w, E.camera.viewmats, E.camera.intrins, (uint32_t)W, (uint32_t)H,
         E.camera.model_str, E.camera.distortion_str, E.camera.dist_coeffs, cam_ids, gauss_ids, aabb, {}, E.grad.v_screen,

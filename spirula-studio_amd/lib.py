@@ -45,7 +45,8 @@ class ProjectionFwdParams(C.Structure):
     _fields_ = [("num_splats", C.c_int64), ("sh_degree", C.c_int32), ("world", World),
                 ("sh", ShQuant), ("camera", Camera), ("aabb", vp), ("sort_depth", vp),
                 ("radii", vp), ("screen", Screen), ("tiles_per_splat", vp), ("visible_ids", vp),
-                ("visible_count", vp), ("packed_rows", vp)]
+                ("visible_count", vp), ("packed_rows", vp),
+                ("antialiased", C.c_int32)]
 
 
 class RasterFwdParams(C.Structure):
@@ -72,7 +73,8 @@ class ProjectionBwdParams(C.Structure):
                 ("sh", ShQuant), ("camera", Camera), ("aabb", vp), ("v_screen", Screen),
                 ("v_world", World), ("accumulate", C.c_int32), ("visible_ids", vp),
                 ("n_visible", C.c_int64), ("packed_gaussian_ids", vp), ("num_packed", C.c_int64), ("v_rows", vp),
-                ("v_viewmat", vp)]
+                ("v_viewmat", vp),
+                ("antialiased", C.c_int32)]
 
 
 class ProjectionPackedParams(C.Structure):
@@ -80,7 +82,8 @@ class ProjectionPackedParams(C.Structure):
                 ("sh", ShQuant), ("camera", Camera), ("radii", vp), ("scratch", vp),
                 ("scratch_bytes", C.c_size_t), ("nnz", vp), ("max_rows", C.c_int64),
                 ("camera_ids", vp), ("gaussian_ids", vp), ("aabb", vp), ("sort_depth", vp),
-                ("screen", Screen), ("tiles_per_splat", vp), ("packed_rows", vp)]
+                ("screen", Screen), ("tiles_per_splat", vp), ("packed_rows", vp),
+                ("antialiased", C.c_int32)]
 
 
 class FpboParams(C.Structure):
@@ -95,7 +98,8 @@ class FpboParams(C.Structure):
                 ("step", C.c_int32), ("steps", vp), ("erank_reg_weight", C.c_float), ("erank_reg_weight_s3", C.c_float),
                 ("scale_agnostic_radii", vp), ("packed_row_of", vp), ("sh_state_packed", vp), ("sh_state_bounds", vp),
                 ("sh_value_packed", vp), ("sh_value_bounds", vp), ("num_sh_buffer", C.c_uint32),
-                ("non_sh_packed", vp * 5), ("non_sh_bounds", vp * 5), ("color_trust_linear", C.c_int32), ("eps_tr", C.c_float)]
+                ("non_sh_packed", vp * 5), ("non_sh_bounds", vp * 5), ("color_trust_linear", C.c_int32), ("eps_tr", C.c_float),
+                ("antialiased", C.c_int32)]
 
 
 # every symbol include/ssr_backend.h declares: (name, restype, argtypes)

@@ -131,6 +131,7 @@ class Scene:
     sh_scale_f16: np.ndarray | None = None   # [N] float16 (int8 codec)
     distortion: int = 0                      # lens distortion tier (LENS_*)
     dist_coeffs: np.ndarray | None = None    # [8] float32 in the tier's own order
+    antialiased: bool = False                # the "mip" variant of the primitive (blur 0.1, opacity compensation)
 
     @property
     def tile_w(self) -> int:

@@ -116,6 +116,7 @@ class GpuRun:
         self.d["nnz"] = D((1,), np.int64)
         p = self.L.ProjectionPackedParams()
         p.num_splats, p.sh_degree = n, self.sh_degree
+        p.antialiased = 1 if getattr(self.sc, "antialiased", False) else 0
         p.world, p.sh, p.camera = self.world(), self.shq(), self.camera()
         p.radii, p.scratch, p.scratch_bytes, p.nnz = self.ptr("radii"), self.ptr("pk_scratch"), sb, self.ptr("nnz")
         self.check(self.lib.ssr_projection_packed_mask(C.byref(p), None))
@@ -153,6 +154,7 @@ class GpuRun:
             self.d[k].fill_zero()
         p = self.L.ProjectionFwdParams()
         p.num_splats, p.sh_degree = self.n, self.sh_degree
+        p.antialiased = 1 if getattr(self.sc, "antialiased", False) else 0
         p.world, p.sh, p.camera = self.world(), self.shq(), self.camera()
         p.aabb, p.sort_depth, p.radii = self.ptr("aabb"), self.ptr("sort_depth"), self.ptr("radii")
         p.screen = self.screen()
@@ -312,6 +314,7 @@ class GpuRun:
                 self.d[k].fill_zero()
         p = self.L.ProjectionBwdParams()
         p.num_splats, p.sh_degree = n, self.sh_degree
+        p.antialiased = 1 if getattr(self.sc, "antialiased", False) else 0
         p.world, p.sh, p.camera = self.world(), self.shq(), self.camera()
         p.aabb, p.v_screen, p.v_world = self.ptr("aabb"), self.screen("v_"), self.world("w_")
         p.accumulate = 1 if accumulate else 0
@@ -348,6 +351,7 @@ class GpuRun:
         self.d["score"] = D((self.n,), np.float32)
         p = self.L.FpboParams()
         p.num_splats, p.sh_degree = self.n, self.sh_degree
+        p.antialiased = 1 if getattr(self.sc, "antialiased", False) else 0
         p.world, p.camera, p.aabb = self.world(), self.camera(), self.ptr("aabb")
         p.v_screen, p.v_world_in, p.g1, p.g2 = self.screen("v_"), self.world("vi_"), self.world("m1_"), self.world("m2_")
         p.densify_score = self.ptr("score")

@@ -14,7 +14,8 @@ _SO = os.path.join(_ROOT, "oracle", "libssr_oracle.so")
 class OrCamera(C.Structure):
     _fields_ = [("model", C.c_int32), ("width", C.c_uint32), ("height", C.c_uint32),
                 ("viewmat", C.c_float * 16), ("fx", C.c_float), ("fy", C.c_float),
-                ("cx", C.c_float), ("cy", C.c_float), ("distortion", C.c_int32), ("dist_coeffs", C.c_float * 8)]
+                ("cx", C.c_float), ("cy", C.c_float), ("distortion", C.c_int32), ("dist_coeffs", C.c_float * 8),
+                ("antialiased", C.c_int32)]
 
 
 class OrShSource(C.Structure):
@@ -62,6 +63,7 @@ def camera_of(scene) -> OrCamera:
     dc = np.zeros(8, np.float32) if getattr(scene, "dist_coeffs", None) is None else np.asarray(scene.dist_coeffs, np.float32)
     for i in range(8):
         cam.dist_coeffs[i] = float(dc[i])
+    cam.antialiased = 1 if getattr(scene, "antialiased", False) else 0
     return cam
 
 

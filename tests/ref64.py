@@ -91,7 +91,7 @@ def lens_valid(tier, coeffs, u, v):
     return (0.25 < jdet < 4.0) and (u * du + v * dv >= 0), jdet
 
 
-def project(mean, quat, log_scale, logit, viewmat, intr, width, model, f32_consts=True, tier=0, coeffs=None):
+def project(mean, quat, log_scale, logit, viewmat, intr, width, model, f32_consts=True, tier=0, coeffs=None, antialiased=False):
     """Returns xy(2), depth, conic(3), opac, plus cov2d (blurred) and the tile extents."""
     R, t = viewmat[:3, :3].astype(np.float64), viewmat[:3, 3].astype(np.float64)
     fx, fy, cx, cy = [float(v) for v in intr]
@@ -131,8 +131,14 @@ def project(mean, quat, log_scale, logit, viewmat, intr, width, model, f32_const
         # the weight the unblurred splat still has at the image centre (src/shaders/primitive_3dgs.slang:509-514)
         m = xy - np.array([cx, cy])
         extra["centre_weight"] = opac * math.exp(-0.5 * float(m @ np.linalg.inv(c2) @ m))
-    eps = float(np.float32(0.3)) if f32_consts else 0.3
+    # screen-space blur; the antialiased ("mip") variant blurs less and rescales the opacity by the square root of
+    # the ratio of the determinants, so that a splat keeps its integrated weight (src/shaders/primitive_3dgs.slang:398-405,528-543)
+    blur = 0.1 if antialiased else 0.3
+    eps = float(np.float32(blur)) if f32_consts else blur
+    det_before = float(np.linalg.det(c2))
     c2 = c2 + eps * np.eye(2)
+    if antialiased:
+        opac = opac * math.sqrt(max(0.0, det_before / float(np.linalg.det(c2))))
     inv = np.linalg.inv(c2)
     depth = float(np.linalg.norm(pc))
     return dict(xy=xy, depth=depth, conic=np.array([inv[0, 0], inv[0, 1], inv[1, 1]]), opac=opac,

@@ -97,7 +97,7 @@ def tool_lens(tier: int, cam: int) -> np.ndarray:
     return (np.float32(1.0 - 0.3 * (cam % 3)) * row).astype(np.float32)
 
 
-def tool_scene(pkg, seed: int, cam: int, model: int = 0, tier: int = 0, n: int = N_TOOL, cotangents=None):
+def tool_scene(pkg, seed: int, cam: int, model: int = 0, tier: int = 0, n: int = N_TOOL, cotangents=None, mip: bool = False):
     """One camera of a tool's two-camera batch as a scene of this package. cotangents: dict with the [C,H,W,..]
     arrays the tool draws (raster_bwd_cotangents), of which camera `cam`'s slice is used."""
     w, rng = tool_world(seed, n)
@@ -107,7 +107,7 @@ def tool_scene(pkg, seed: int, cam: int, model: int = 0, tier: int = 0, n: int =
     ct = cotangents or {}
     sc = pkg.scenes.Scene(name=f"tool-{seed}-cam{cam}", n=n, width=W_TOOL, height=H_TOOL, camera_model=model, viewmat=vm,
                           intrins=intr, v_rgb=ct["v_rgb"][cam] if ct else z3, v_depth=ct["v_depth"][cam] if ct else z1,
-                          v_T=ct["v_T"][cam] if ct else z1, distortion=tier, dist_coeffs=tool_lens(tier, cam), **w)
+                          v_T=ct["v_T"][cam] if ct else z1, distortion=tier, dist_coeffs=tool_lens(tier, cam), antialiased=mip, **w)
     return sc, rng
 
 

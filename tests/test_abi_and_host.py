@@ -132,3 +132,25 @@ def test_codecs_match_the_oracle_encoders(pkg, oracle):
     assert np.array_equal(scale.view(np.uint16), osc)
     assert np.array_equal(codes, oc)
     assert np.abs(dec - v).max() <= float(scale.astype(np.float32).max()) * 0.51
+
+
+def test_ctypes_structures_match_the_header(pkg, tmp_path):
+    """Every parameter structure of include/ssr_backend.h has the same size and the same offset of its last
+    member in the Python mirror as the C compiler gives it."""
+    import ctypes as C
+    import subprocess
+    from spirula_studio_amd import lib
+    pairs = [("ssr_world", lib.World), ("ssr_screen", lib.Screen), ("ssr_sh_quant", lib.ShQuant), ("ssr_camera", lib.Camera),
+             ("ssr_projection_fwd_params", lib.ProjectionFwdParams), ("ssr_projection_packed_params", lib.ProjectionPackedParams),
+             ("ssr_raster_fwd_params", lib.RasterFwdParams), ("ssr_raster_bwd_params", lib.RasterBwdParams),
+             ("ssr_projection_bwd_params", lib.ProjectionBwdParams), ("ssr_fpbo_params", lib.FpboParams)]
+    src = tmp_path / "sizes.c"
+    body = "".join(f'    printf("%zu %zu\\n", sizeof({c}), offsetof({c}, {py._fields_[-1][0]}));\n' for c, py in pairs)
+    src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "ssr_backend.h"\nint main(void) {\n' + body + "    return 0;\n}\n")
+    exe = tmp_path / "sizes"
+    subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split("\n")
+    for (c, py), line in zip(pairs, out):
+        size, off = [int(v) for v in line.split()]
+        assert C.sizeof(py) == size, (c, C.sizeof(py), size)
+        assert getattr(py, py._fields_[-1][0]).offset == off, (c, py._fields_[-1][0])

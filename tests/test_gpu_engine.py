@@ -1,5 +1,7 @@
 """GPU: the C++ host layer (reference-shaped launch functions + engine call order) against the
 oracle, in both stage orders, and the behaviours the engine relies on."""
+import dataclasses
+
 import numpy as np
 import pytest
 
@@ -85,6 +87,41 @@ def test_engine_wide_lens_cameras(pkg, oracle, H):
         eng.forward()
         eng.backward()
         _check(eng, ref, sc)
+
+
+@pytest.mark.parametrize("packed", [False, True])
+def test_engine_mip_primitive(pkg, oracle, H, packed):
+    """forward_3dgs("mip"): the antialiased variant through the engine, the backward, and two fused optimizer
+    steps (the reference instantiates the same functions with antialiased = true)."""
+    host, lib = H
+    S = pkg.scenes
+    sc = S.tiny_scene(n=3000, width=256, height=192, seed=59)
+    sc.log_scales -= 2.0
+    sc.antialiased = True
+    ref = oracle.pipeline_packed(sc) if packed else oracle.pipeline(sc)
+    plain = oracle.pipeline(dataclasses.replace(sc, antialiased=False), backward=False)
+    assert np.abs(plain["fwd"]["rgb"] - ref["fwd"]["rgb"]).max() > 0.02         # a different image than "3dgs"
+    eng = host.Engine(sc, packed_projection=packed)
+    eng.forward()
+    eng.backward()
+    _check(eng, ref, sc)
+    h = dict(lr_means=1.6e-4, lr_quats=1e-3, lr_scales=5e-3, lr_opacs=5e-2, lr_features_dc=2.5e-3, lr_features_sh=1.25e-4,
+             max_gauss_ratio=6.0, scale_regularization_weight=0.01, mcmc_opacity_reg_weight=0.01, mcmc_scale_reg_weight=0.01,
+             quat_norm_reg_weight=0.02, sh_reg_weight=0.05)
+    eng2 = host.Engine(sc, packed_projection=packed)
+    eng2.forward()
+    eng2.backward_fused_optimizer(h, 1)
+    P = {k: np.ascontiguousarray(getattr(sc, k), np.float32).copy() for k in oracle.WORLD_KEYS}
+    g1 = {k: np.zeros_like(v) for k, v in P.items()}
+    g2 = {k: np.zeros_like(v) for k, v in P.items()}
+    r = oracle.pipeline(sc)
+    oracle.fused_projection_bwd_optimizer(sc, r["proj"]["aabb"], r["vscreen"], P, g1, g2, h, step=1)
+    got = eng2.params()
+    lrs = dict(means="lr_means", quats="lr_quats", log_scales="lr_scales", opacity_logits="lr_opacs",
+               features_dc="lr_features_dc", features_sh="lr_features_sh")
+    for k in oracle.WORLD_KEYS:      # first Adam step: +-lr per element, sign decided by the gradient
+        far = np.abs(got[k].astype(np.float64) - P[k]) > 0.05 * h[lrs[k]]
+        assert far.mean() < 5e-3, (k, float(far.mean()))
 
 
 @pytest.mark.parametrize("packed", [False, True])

@@ -2,6 +2,7 @@
 inputs. Bars: tile keys / sorted ids / tile ranges bit-exact; images max-abs 1e-4 per channel;
 gradients 1e-3 relative (with a floor proportional to the sum of |terms|, since float atomics add
 in a different order)."""
+import dataclasses
 import math
 
 import numpy as np
@@ -287,6 +288,24 @@ def test_camera_variants_strong_lens_and_packed(gpu, oracle):
              use_vrows=True, tile_sort=True)
 
 
+@pytest.mark.parametrize("model,tier,packed", [(0, 0, False), (0, 0, True), (0, 1, False), (1, 2, False), (3, 0, True)])
+def test_antialiased_variant(gpu, oracle, model, tier, packed):
+    """The antialiased ("mip") variant of the primitive through the whole iteration: blur 0.1 and the opacity
+    compensation in the projection, its gradient in the projection backward."""
+    sc = _lens_scene(gpu, model, tier, n=2500, seed=35)
+    sc.log_scales -= 2.2          # a pixel or two on screen: the blur and its compensation matter
+    sc.antialiased = True
+    plain = oracle.projection_fwd(dataclasses.replace(sc, antialiased=False))
+    if packed:
+        g, r = _compare_packed(gpu, oracle, sc, f"mip-{model}-{tier}-packed", fused_count=True, use_packed=True)
+        opac = r["full_proj"]["opac"]
+    else:
+        g, r = _compare(gpu, oracle, sc, f"mip-{model}-{tier}", fused_count=True, use_list=True, use_packed=True, use_vrows=True)
+        opac = r["proj"]["opac"]
+    both = (plain["aabb"][:, 2] > plain["aabb"][:, 0]) & (r["full_proj" if packed else "proj"]["aabb"][:, 2] > 0)
+    assert both.sum() > 100 and (opac[both] < 0.9 * plain["opac"][both]).mean() > 0.1     # the compensation is at work
+
+
 def test_tiny_equirect(gpu, oracle):
     _compare(gpu, oracle, gpu.scenes.tiny_scene(n=600, width=128, height=64, seed=4, camera_model=3), "tiny-eq")
 
@@ -379,13 +398,16 @@ def test_tile_skip_mask(gpu, oracle):
     assert r["counts"].max() > 96
 
 
-@pytest.mark.parametrize("cfg", ["tiny", "cfg2", "equirect-steps", "fisheye-prism", "tiny-packed", "cfg4-packed", "tiny-ctl", "cfg2-ctl"])
+@pytest.mark.parametrize("cfg", ["tiny", "cfg2", "equirect-steps", "fisheye-prism", "tiny-packed", "cfg4-packed", "tiny-ctl", "cfg2-ctl", "tiny-mip"])
 def test_fused_projection_bwd_optimizer(gpu, oracle, cfg):
     """K9 fused with Adam (fused_projection_bwd_optimizer_3dgs, fp32 state): both sides are fed the
     SAME screen gradients (the device's), so only the arithmetic of the fused kernel is compared."""
     rng = np.random.default_rng(11)
-    if cfg in ("tiny", "tiny-ctl"):
+    if cfg in ("tiny", "tiny-ctl", "tiny-mip"):
         sc = gpu.scenes.tiny_scene(n=900, width=96, height=64, seed=61)
+        if cfg == "tiny-mip":      # the antialiased primitive (fused_projection_bwd_optimizer_mip)
+            sc.log_scales -= 1.5
+            sc.antialiased = True
         sc.means[::4, 2] = -10.0
         sc.log_scales[5] = [-2.0, -4.5, -3.0]
         sc.features_dc[7] = [2.5, -2.2, 0.1]

@@ -14,12 +14,13 @@ PINHOLE, FISHEYE, EQUISOLID, EQUIRECT = 0, 1, 2, 3
 NONE, OPENCV, THIN_PRISM, RATIONAL = 0, 1, 2, 3
 
 
-# render_parity.cpp:186-196, rows with prim == 0: (packed, camera model, tier, dist_type, median)
-@pytest.mark.parametrize("packed,model,tier,dist_type,median", [(False, PINHOLE, OPENCV, 2, True), (False, FISHEYE, THIN_PRISM, 1, False),
-                                                              (True, EQUIRECT, NONE, 0, False)])
+# render_parity.cpp:186-196, rows with prim == 0 (3dgs) and 1 (mip): (mip, packed, camera model, tier, dist_type, median)
+@pytest.mark.parametrize("mip,packed,model,tier,dist_type,median", [(False, False, PINHOLE, OPENCV, 2, True), (True, False, PINHOLE, NONE, 2, True),
+                                                                  (False, False, FISHEYE, THIN_PRISM, 1, False),
+                                                                  (False, True, EQUIRECT, NONE, 0, False)])
 @pytest.mark.parametrize("cam", [0, 1])
-def test_render_parity_rows(gpu, oracle, packed, model, tier, dist_type, median, cam):
-    sc, _ = R.tool_scene(gpu, R.SEED_RENDER, cam, model, tier)
+def test_render_parity_rows(gpu, oracle, mip, packed, model, tier, dist_type, median, cam):
+    sc, _ = R.tool_scene(gpu, R.SEED_RENDER, cam, model, tier, mip=mip)
     z3, z1 = np.zeros((sc.height, sc.width, 3), np.float32), np.zeros((sc.height, sc.width), np.float32)
     va = dict(dist_type=dist_type, median=median, v_dist_rgb=z3, v_dist_depth=z1, v_median=z1)
     label = f"render_parity model {model} tier {tier} cam {cam}"
@@ -118,10 +119,11 @@ def test_fpbo_parity_rows(gpu, oracle, row, tier, cam):
 # each of its compiled tiers
 @pytest.mark.parametrize("model", [PINHOLE, FISHEYE, EQUISOLID, EQUIRECT])
 @pytest.mark.parametrize("cam", [0, 1])
-def test_projection_parity_rows(gpu, oracle, model, cam):
+@pytest.mark.parametrize("mip", [False, True])      # prim 0 and prim 1 of the tool's sweep
+def test_projection_parity_rows(gpu, oracle, model, cam, mip):
     for deg, tiers in [(0, [NONE]), (3, R.COMPILED_TIERS[model])]:
         for tier in tiers:
-            sc, _ = R.tool_scene(gpu, R.SEED_PROJ, cam, model, tier)
+            sc, _ = R.tool_scene(gpu, R.SEED_PROJ, cam, model, tier, mip=mip)
             want = oracle.projection_fwd(sc, deg)
             g = GpuRun(gpu, sc, sh_degree=deg)
             g.projection_fwd()
@@ -171,10 +173,10 @@ def test_projection_parity_quantized_rows(gpu, oracle, cam):
             assert np.array_equal(w32["rgb"][vis].view(np.uint32), want["rgb"][vis].view(np.uint32)), (bits, per_block)
 
 
-def _k9_direct(gpu, oracle, sc, vs, label, packed=False, pose=False):
+def _k9_direct(gpu, oracle, sc, vs, label, packed=False, pose=False, sh_degree=3):
     """ssr_projection_bwd fed given screen gradients (rows: splats, or packed rows), against the oracle.
     pose: also the camera-pose gradient (the rows of the tool that ask for v_viewmats)."""
-    g = GpuRun(gpu, sc, packed_projection=packed)
+    g = GpuRun(gpu, sc, packed_projection=packed, sh_degree=sh_degree)
     g.projection_fwd()
     D = gpu.lib.DeviceArray
     aabb = g.host("aabb")
@@ -192,7 +194,7 @@ def _k9_direct(gpu, oracle, sc, vs, label, packed=False, pose=False):
     for k, v in vs.items():
         g.d[k] = D.from_host(np.ascontiguousarray(v))
     g.projection_bwd(pose=pose)
-    want = oracle.projection_bwd(sc, full_aabb, full_vs, pose=pose)
+    want = oracle.projection_bwd(sc, full_aabb, full_vs, sh_degree=sh_degree, pose=pose)
     if pose:
         got_vm, want_vm = g.host("v_viewmat").astype(np.float64), want.pop("v_viewmat").astype(np.float64)
         print(f"[{label}] dL/dt = {want_vm[:3, 3]}", flush=True)
@@ -226,7 +228,11 @@ def test_proj_bwd_parity_rows(gpu, oracle, cam):
         vs = {k: np.ascontiguousarray(v.reshape((R.C_TOOL, n) + v.shape[1:])[cam]) for k, v in vs2.items()}
         sc, _ = R.tool_scene(gpu, R.SEED_PROJ_BWD, cam, PINHOLE, tier)
         _k9_direct(gpu, oracle, sc, vs, f"proj_bwd_parity PINHOLE tier {tier} cam {cam}", pose=True)
-    R.screen_gradients(rng, R.C_TOOL * n)        # row 2 (another primitive) draws the same amount
+    # row 2: the mip primitive, FISHEYE + thin prism, SH degree 2
+    vs2 = R.screen_gradients(rng, R.C_TOOL * n)
+    vs = {k: np.ascontiguousarray(v.reshape((R.C_TOOL, n) + v.shape[1:])[cam]) for k, v in vs2.items()}
+    sc, _ = R.tool_scene(gpu, R.SEED_PROJ_BWD, cam, FISHEYE, THIN_PRISM, mip=True)
+    _k9_direct(gpu, oracle, sc, vs, f"proj_bwd_parity mip FISHEYE THIN_PRISM cam {cam}", sh_degree=2)
     # row 3: packed, EQUISOLID + OpenCV; the tool's rows are camera 0's visible splats, then camera 1's
     nnz = []
     for c in range(R.C_TOOL):

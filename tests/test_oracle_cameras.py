@@ -2,6 +2,7 @@
 src/kernels/projection/CameraVariants.cuh:11-22 beyond PINHOLE/None and EQUIRECTANGULAR) against
 closed forms and an independent float64 restatement whose Jacobian comes from complex-step
 differentiation, and the backward against finite differences of that restatement."""
+import dataclasses
 import math
 
 import numpy as np
@@ -273,3 +274,94 @@ def test_camera_pose_gradient_matches_finite_differences(pkg, oracle, model, tie
     scale = np.abs(fd).max()
     assert scale > 1e-3
     assert np.abs(got - fd).max() <= 3e-3 * scale, (got, fd)
+
+
+# ---- the antialiased ("mip") variant of the primitive: same projection function, runtime flag ----
+
+def _aa_scene(pkg, model, tier, n=300, seed=41):
+    sc = _scene(pkg, model, tier, n=n, seed=seed)
+    sc.log_scales -= 1.2          # small on screen: the blur matters, compensation well below 1
+    sc.antialiased = True
+    return sc
+
+
+@pytest.mark.parametrize("model,tier", [(0, 0), (0, 2), (1, 1), (3, 0)])
+def test_antialiased_forward_matches_float64(pkg, oracle, model, tier):
+    sc = _aa_scene(pkg, model, tier)
+    o = oracle.projection_fwd(sc)
+    plain = oracle.projection_fwd(dataclasses.replace(sc, antialiased=False))
+    vis = o["aabb"][:, 2] > o["aabb"][:, 0]
+    assert vis.sum() > 40
+    comps = []
+    for g in np.nonzero(vis)[0][:120]:
+        r = ref64.project(sc.means[g].astype(np.float64), sc.quats[g].astype(np.float64), sc.log_scales[g].astype(np.float64),
+                          float(sc.opacity_logits[g]), sc.viewmat, sc.intrins, sc.width, sc.camera_model, tier=sc.distortion,
+                          coeffs=sc.dist_coeffs, antialiased=True)
+        np.testing.assert_allclose(o["xy"][g], r["xy"], rtol=2e-5, atol=3e-3)
+        np.testing.assert_allclose(o["conic"][g], r["conic"], rtol=1e-3, atol=2e-6)
+        np.testing.assert_allclose(o["opac"][g], r["opac"], rtol=2e-4, atol=1e-7)
+        # closed form of the compensation: the blurred splat keeps the integrated weight of the unblurred one,
+        # opacity * 2 pi sqrt(det) is the same before and after
+        c2 = r["cov2d"]
+        before = c2 - np.float32(0.1) * np.eye(2)
+        sig = 1 / (1 + math.exp(-float(sc.opacity_logits[g])))
+        assert abs(o["opac"][g] * math.sqrt(np.linalg.det(c2)) - sig * math.sqrt(max(np.linalg.det(before), 0))) <= 2e-4 * sig * math.sqrt(np.linalg.det(c2))
+        comps.append(o["opac"][g] / sig)
+        if plain["aabb"][g, 2] > plain["aabb"][g, 0]:
+            assert o["opac"][g] <= plain["opac"][g] * (1 + 1e-6)          # never brighter than the plain variant
+            assert o["conic"][g, 0] >= plain["conic"][g, 0] * (1 - 1e-6)   # and sharper (blur 0.1 instead of 0.3)
+    assert min(comps) < 0.7 and max(comps) > 0.8      # the compensation spans a wide range in the scene
+
+
+@pytest.mark.parametrize("model,tier", [(0, 0), (0, 1), (2, 2), (3, 0)])
+def test_antialiased_backward_matches_finite_differences(pkg, oracle, model, tier):
+    sc = _aa_scene(pkg, model, tier, n=160, seed=43)
+    rng = np.random.default_rng(11)
+    o = oracle.projection_fwd(sc)
+    n = sc.n
+    v = dict(v_xy=rng.normal(0, 1, (n, 2)).astype(np.float32), v_depth=rng.normal(0, 1, n).astype(np.float32),
+             v_conic=rng.normal(0, 1, (n, 3)).astype(np.float32), v_opac=rng.normal(0, 3, n).astype(np.float32),
+             v_rgb=rng.normal(0, 1, (n, 3)).astype(np.float32))
+    g_or = oracle.projection_bwd(sc, o["aabb"], v, pose=True)
+    vis = np.nonzero(o["aabb"][:, 2] > o["aabb"][:, 0])[0]
+    assert len(vis) > 20
+
+    def loss(g, mean, quat, ls, logit, viewmat=None):
+        r = ref64.project(mean, quat, ls, logit, sc.viewmat if viewmat is None else viewmat, sc.intrins, sc.width, sc.camera_model,
+                          tier=sc.distortion, coeffs=sc.dist_coeffs, antialiased=True)
+        col = ref64.sh_color(mean, sc.viewmat if viewmat is None else viewmat, sc.features_dc[g].astype(np.float64),
+                             sc.features_sh[g].astype(np.float64))
+        f64 = lambda a: np.asarray(a, np.float64)
+        return float(f64(v["v_xy"][g]) @ r["xy"] + f64(v["v_depth"][g]) * r["depth"] + f64(v["v_conic"][g]) @ r["conic"]
+                     + f64(v["v_opac"][g]) * r["opac"] + f64(v["v_rgb"][g]) @ col)
+    for g in vis[:20]:
+        args = [sc.means[g].astype(np.float64), sc.quats[g].astype(np.float64), sc.log_scales[g].astype(np.float64),
+                np.array([float(sc.opacity_logits[g])])]
+        for ai, name in enumerate(["v_means", "v_quats", "v_scales", "v_opacities"]):
+            got = np.asarray(g_or[name][g], np.float64).reshape(-1)
+            fd = np.zeros_like(got)
+            for k in range(args[ai].size):
+                h = 1e-6 * max(1.0, abs(args[ai][k]))
+                ap, am = [x.copy() for x in args], [x.copy() for x in args]
+                ap[ai][k] += h
+                am[ai][k] -= h
+                fd[k] = (loss(g, ap[0], ap[1], ap[2], float(ap[3][0])) - loss(g, am[0], am[1], am[2], float(am[3][0]))) / (2 * h)
+            assert np.abs(got - fd).max() <= 2e-3 * (np.abs(fd).max() + 1e-6), (g, name, got, fd)
+    # the opacity gradient reaches the scales through the compensation: with only v_opac set the scale gradient is not zero
+    v0 = {k: np.zeros_like(a) for k, a in v.items()}
+    v0["v_opac"] = v["v_opac"]
+    assert np.abs(oracle.projection_bwd(sc, o["aabb"], v0)["v_scales"][vis]).max() > 1e-3
+    assert not np.any(oracle.projection_bwd(dataclasses.replace(sc, antialiased=False), o["aabb"], v0)["v_scales"])
+    # and the camera pose
+    fd = np.zeros((4, 4))
+    base = sc.viewmat.astype(np.float64)
+    tot = lambda vm: sum(loss(g, sc.means[g].astype(np.float64), sc.quats[g].astype(np.float64), sc.log_scales[g].astype(np.float64),
+                              float(sc.opacity_logits[g]), vm) for g in vis)
+    for i in range(3):
+        for j in range(4):
+            h = 1e-6 * max(1.0, abs(base[i, j]))
+            vp, vm_ = base.copy(), base.copy()
+            vp[i, j] += h
+            vm_[i, j] -= h
+            fd[i, j] = (tot(vp) - tot(vm_)) / (2 * h)
+    assert np.abs(g_or["v_viewmat"].astype(np.float64) - fd).max() <= 3e-3 * np.abs(fd).max()
