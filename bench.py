@@ -110,6 +110,7 @@ def main():
                     help="with --fused-optimizer: 1 = SH values as 16-bit codes and their Adam moments as 8-bit cells "
                          "(the reference's default level); the scene's SH is then stored at 16 bits, one bound per 256 splats")
     ap.add_argument("--scale-agnostic-mean", action="store_true", help="with --fused-optimizer: the scale-agnostic step of the means")
+    ap.add_argument("--mip", action="store_true", help="the antialiased primitive (blur 0.1, opacity compensation)")
     ap.add_argument("--non-sh-optim-bits", type=int, default=32, choices=[32, 16],
                     help="with --quantization-level 1: 16 = the moments of the non-SH tensors as 16-bit cells too (what the reference's trainer sets)")
     ap.add_argument("--dist-type", type=int, default=0, help="compositing variant: 1 depth distortion, 2 rgb + depth distortion")
@@ -153,6 +154,8 @@ def main():
         sc.intrins = np.array([f, f, sc.width / 2.0, sc.height / 2.0], np.float32)
     if args.lens != "none":
         sc = pkg.scenes.with_lens(sc, ["none", "opencv", "thin_prism", "rational"].index(args.lens))
+    if args.mip:
+        sc.antialiased = True
     t_gen = time.time() - t_gen
     native = not args.reference_order
     eng = host.Engine(sc, fuse_tile_count=native, visible_list=native and not args.packed_projection, packed_rows=native,
@@ -237,7 +240,7 @@ def main():
     if os.path.exists(tpath):
         try:
             traffic = json.load(open(tpath)).get(f"config{cfg}", {}).get(dom)
-            if native and not (variants or args.fused_optimizer or args.packed_projection or args.lens != "none" or args.fisheye):
+            if native and not (variants or args.fused_optimizer or args.packed_projection or args.lens != "none" or args.fisheye or args.mip):
                 valu_inst = json.load(open(tpath)).get(f"config{cfg}_valu_wave_instructions", {}).get(dom)
         except Exception:
             traffic = None
@@ -257,6 +260,7 @@ def main():
                    "visible": V, "n_isects": K, "K_b": K_b, "tiles": T, "pixels": P,
                    "stage_order": ("fused tile count, visible-splat work list, packed fragment rows, packed gradient rows, plain-store gradients"
                                    + (", tile-segmented sort" if tile_sort else "") if native else "reference order")
+                                  + (", antialiased (mip) primitive" if args.mip else "")
                                   + (", packed projection outputs" if args.packed_projection else "")
                                   + (", projection backward fused with Adam" + ((" (quantized SH state" + (" and non-SH moments)" if args.non_sh_optim_bits == 16 else ")")) if args.quantization_level else "")
                                      if args.fused_optimizer else "")

@@ -624,9 +624,10 @@ int ssrh_time_iterations(int sh_degree, int packed, const float* v_rgb_dev, cons
                          int iters, float* ms_out) {
     return guard([&] {
         ssr_event_t a = ssr_event_create(), b = ssr_event_create();
+        const std::string primitive = engine().primitive.empty() ? "3dgs" : engine().primitive;   // as the last forward
         for (int i = 0; i < iters; i++) {
             ssr_event_record(a, nullptr);
-            forward_3dgs("3dgs", sh_degree, packed != 0, false, 0);
+            forward_3dgs(primitive, sh_degree, packed != 0, false, 0);
             const int64_t C = engine().camera.num, H = engine().camera.height, W = engine().camera.width;
             engine_backward_from_render_grad(tv(v_rgb_dev, 4, {C, H, W, 3}), tv(v_depth_dev, 4, {C, H, W, 1}), tv(v_Ts_dev, 4, {C, H, W, 1}));
             ssr_event_record(b, nullptr);

@@ -328,3 +328,48 @@ def test_fpbo_parity_quantized_row(gpu, oracle, cam):
         q = {k: (v.copy() if isinstance(v, np.ndarray) else v) for k, v in dq.items()}
         ns = dict(packed=[x.copy() for x in dns["packed"]], bounds=[x.copy() for x in dns["bounds"]])
         P = {k: v.copy() for k, v in dP.items()}
+
+
+# fpbo_parity.cpp:163, the mip row: unpacked, FISHEYE + thin prism, SH degree 2, fp32 state, the scale-agnostic step of the
+# means, no world gradients, per-splat steps (then step 11 for everyone on the second call), no densify score
+@pytest.mark.parametrize("cam", [0, 1])
+def test_fpbo_parity_mip_row(gpu, oracle, cam):
+    n = R.N_FPBO
+    sc, rng = R.tool_scene(gpu, R.SEED_FPBO, cam, FISHEYE, THIN_PRISM, n=n, mip=True)
+    for _ in range(2):                      # rows 0 and 1 draw first
+        R.fpbo_row_inputs(rng)
+    vs2 = R.screen_gradients(rng, R.C_TOOL * n)
+    vs = {k: np.ascontiguousarray(v.reshape((R.C_TOOL, n) + v.shape[1:])[cam]) for k, v in vs2.items()}
+    keys = oracle.WORLD_KEYS
+    shapes = [(n, 3), (n, 4), (n, 3), (n,), (n, 3), (n, 15, 3)]
+    g1, g2 = {}, {}
+    for k, s in zip(keys, shapes):          # no world gradients in this row (vw_mask 0): the moments follow directly
+        g1[k] = rng.uf(int(np.prod(s)), -0.02, 0.02).reshape(s)
+        g2[k] = rng.uf(int(np.prod(s)), 0.0, 4e-4).reshape(s)
+    steps = (1 + rng.raw(n) % np.uint32(50)).astype(np.int32)
+    g = GpuRun(gpu, sc, sh_degree=2)
+    g.projection_fwd()
+    D = gpu.lib.DeviceArray
+    for k, v in vs.items():
+        g.d[k] = D.from_host(v)
+    aabb, radii = g.host("aabb"), g.host("radii")
+    assert 100 < (aabb[:, 2] > aabb[:, 0]).sum() < n
+    P = {k: np.ascontiguousarray(getattr(sc, k), np.float32).copy() for k in keys}
+    o1 = {k: v.copy() for k, v in g1.items()}
+    o2 = {k: v.copy() for k, v in g2.items()}
+    h = R.FPBO_HYPER
+    lrs = dict(means="lr_means", quats="lr_quats", log_scales="lr_scales", opacity_logits="lr_opacs",
+               features_dc="lr_features_dc", features_sh="lr_features_sh")
+    d1, d2 = g1, g2
+    for call, st in enumerate([steps, None]):
+        dP, d1, d2, _ = g.fused_optimizer(d1, d2, h, step=11, steps=st, scale_agnostic=True)
+        oracle.fused_projection_bwd_optimizer(sc, aabb, vs, P, o1, o2, h, step=11, steps=st, sh_degree=2, radii=radii, densify=False)
+        for k in keys:
+            a, b = d1[k].reshape(n, -1).astype(np.float64), o1[k].reshape(n, -1).astype(np.float64)
+            assert (np.abs(a - b) <= 1e-3 * np.abs(b) + 1e-4 * (np.abs(b).max(axis=1, keepdims=True) + 1e-12)).all(), ("g1", k, call)
+            a, b = d2[k].reshape(n, -1).astype(np.float64), o2[k].reshape(n, -1).astype(np.float64)
+            assert (np.abs(a - b) <= 2e-3 * np.abs(b) + 1e-12).all(), ("g2", k, call)
+            far = np.abs(dP[k].astype(np.float64) - P[k]) > 0.02 * h[lrs[k]] + 1e-7
+            assert far.mean() < 2e-3, (k, call, float(far.mean()))
+        # the coefficients above degree 2 are left alone
+        assert np.array_equal(dP["features_sh"][:, 8:], sc.features_sh[:, 8:])
