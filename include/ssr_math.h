@@ -84,19 +84,8 @@ SSR_HD float ssr_exp(float x) {
     return (y * ssr_pow2i(k1)) * ssr_pow2i(k2);
 }
 
-// natural log. log(0) = -inf, log(x<0) = NaN, log(inf) = inf; subnormal inputs are handled.
-SSR_HD float ssr_log(float x) {
-    if (!(x == x)) return x;
-    if (x < 0.0f) return ssr_u2f(0x7fc00000u);
-    if (x == 0.0f) return ssr_u2f(0xff800000u);
-    uint32_t u = ssr_f2u(x);
-    if (u == 0x7f800000u) return x;
-    int e = 0;
-    if (u < 0x00800000u) {                      // subnormal: scale by 2^23 (exact)
-        x = x * 8388608.0f;
-        u = ssr_f2u(x);
-        e = -23;
-    }
+// log of a normal positive finite number whose bits are u, with e added to the exponent
+SSR_HD float ssr_log_core(uint32_t u, int e) {
     e += (int)(u >> 23) - 126;                  // x = m * 2^e, m in [0.5, 1)
     float m = ssr_u2f((u & 0x007fffffu) | 0x3f000000u);
     if (m < 0.707106781186547524f) {
@@ -122,6 +111,28 @@ SSR_HD float ssr_log(float x) {
     float r = m + y;
     r = ssr_fma(fe, 0.693359375f, r);
     return r;
+}
+
+// natural log. log(0) = -inf, log(x<0) = NaN, log(inf) = inf; subnormal inputs are handled.
+SSR_HD float ssr_log(float x) {
+    if (!(x == x)) return x;
+    if (x < 0.0f) return ssr_u2f(0x7fc00000u);
+    if (x == 0.0f) return ssr_u2f(0xff800000u);
+    uint32_t u = ssr_f2u(x);
+    if (u == 0x7f800000u) return x;
+    int e = 0;
+    if (u < 0x00800000u) {                      // subnormal: scale by 2^23 (exact)
+        x = x * 8388608.0f;
+        u = ssr_f2u(x);
+        e = -23;
+    }
+    return ssr_log_core(u, e);
+}
+
+// ssr_log for x >= 1 (or NaN): the same value with the tests for zero, negative and subnormal inputs left out
+SSR_HD float ssr_log_ge1(float x) {
+    if (!(x < 3.0e38f)) return ssr_log(x);      // infinity, NaN and the last binade take the general path
+    return ssr_log_core(ssr_f2u(x), 0);
 }
 
 // atan(x) for finite x, result in (-pi/2, pi/2).

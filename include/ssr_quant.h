@@ -20,9 +20,9 @@
 SSR_HD float ssr_log1p(float x) {   // x >= 0
     const float u = 1.0f + x;
     if (u == 1.0f) return x;
-    const float um1 = u - 1.0f;
-    if (um1 == x) return ssr_log(u);   // the correction factor x / (u - 1) is exactly 1 (always so from 2^25 on)
-    return ssr_log(u) * (x / um1);
+    const float um1 = u - 1.0f;        // u > 1 from here on
+    if (um1 == x) return ssr_log_ge1(u);   // the correction factor x / (u - 1) is exactly 1 (always so from 2^25 on)
+    return ssr_log_ge1(u) * (x / um1);
 }
 SSR_HD float ssr_expm1(float y) {
     const float u = ssr_exp(y);
