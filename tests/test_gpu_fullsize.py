@@ -152,3 +152,69 @@ def test_full_size_properties(pkg, oracle, H, cfg):
     g2 = eng2.grads()
     for k in g1:
         close(0.5 * g2[k], g1[k], ("linear", k))
+
+
+def test_full_size_default_training_step(pkg, oracle, H):
+    """The reference trainer's default step at the headline size (config 2, 1 M splats): packed projection, fused
+    optimizer at quantization level 1 with 16-bit non-SH moments, scale-agnostic mean step. Checked through what
+    holds at any size: every block's bounds are the exact extremes of what it stores (each block contains the codes
+    0 and full scale of every quantity), a first Adam step moves every visible coefficient by the learning rate,
+    and the run agrees with the fp32-state step on the same scene up to the codecs' resolution."""
+    host, lib = H
+    S = pkg.scenes
+    sc = S.make_scene(2)
+    S.apply_sh_codec(sc, 2, bounds_stride=256 * 45)
+    n, R = sc.n, 45
+    nb = (n + 255) // 256
+    h = dict(lr_means=1.6e-4, lr_quats=1e-3, lr_scales=5e-3, lr_opacs=5e-2, lr_features_dc=2.5e-3, lr_features_sh=1.25e-3,
+             max_gauss_ratio=10.0, scale_regularization_weight=0.1, mcmc_opacity_reg_weight=0.01, mcmc_scale_reg_weight=0.01,
+             erank_reg_weight=0.1, erank_reg_weight_s3=0.02, quat_norm_reg_weight=0.01, sh_reg_weight=0.05)
+    eng = host.Engine(sc, packed_projection=True)
+    eng.forward()
+    q0 = eng.sh_quant_state()
+    v0 = oracle.decode_sh_values(q0, n)
+    eng.backward_fused_optimizer(h, 1, scale_agnostic_mean=True, quantization_level=1, non_sh_optim_bits=16)
+    q1 = eng.sh_quant_state()
+    ns = eng.non_sh_quant_state()
+    ids = eng.cache("gaussian_ids")
+    vis = np.zeros(n, bool)
+    vis[ids] = True
+    print(f"[full default step] N={n} visible={int(vis.sum())}", flush=True)
+    assert 0.5 * n < vis.sum() < n
+    # ---- every block holds both endpoints of each stored quantity ----
+    full = n // 256
+    codes = q1["value_packed"][: full * 256 * R].reshape(full, 256 * R)
+    assert (codes.min(axis=1) == 0).all() and (codes.max(axis=1) == 65535).all()
+    st = q1["state_packed"][: full * 256 * R].reshape(full, 256 * R)
+    assert ((st & 255).min(axis=1) == 0).all() and ((st & 255).max(axis=1) == 255).all()
+    assert ((st >> 8).min(axis=1) == 0).all() and ((st >> 8).max(axis=1) == 255).all()
+    for t, prims in enumerate(oracle.NON_SH_PRIMS):
+        c = ns["packed"][t][: full * 256 * prims].reshape(full, 256 * prims)
+        assert ((c & 65535).min(axis=1) == 0).all() and ((c & 65535).max(axis=1) == 65535).all(), t
+        assert ((c >> 16).min(axis=1) == 0).all() and ((c >> 16).max(axis=1) == 65535).all(), t
+    vb = q1["value_bounds"]
+    assert np.isfinite(vb).all() and (vb[:, 1] >= vb[:, 0]).all() and np.isfinite(q1["state_bounds"]).all()
+    # ---- first Adam step from zero moments: +-lr for every coefficient with a gradient ----
+    v1 = oracle.decode_sh_values(q1, n)
+    step = (vb[:, 1] - vb[:, 0]) / 65535
+    tol = np.repeat(step, 256)[:n, None, None] * 0.51 + 2e-6
+    moved = np.abs(v1.astype(np.float64) - v0)
+    assert (moved <= h["lr_features_sh"] * 1.001 + tol).all()
+    assert (np.abs(moved[vis] - h["lr_features_sh"]) <= tol[vis]).mean() > 0.98     # visible splats: a full step (the regularizer alone moves the rest)
+    # ---- against the fp32-state step on the same scene ----
+    ref = S.make_scene(2)
+    ref.features_sh = v0.copy()
+    pq = eng.params()                      # before the next engine takes the (single) engine state over
+    e32 = host.Engine(ref, packed_projection=True)
+    e32.forward()
+    e32.backward_fused_optimizer(h, 1, scale_agnostic_mean=True)
+    p32 = e32.params()
+    for k, lr in [("means", None), ("quats", "lr_quats"), ("log_scales", "lr_scales"), ("opacity_logits", "lr_opacs"), ("features_dc", "lr_features_dc")]:
+        d = np.abs(p32[k].astype(np.float64) - pq[k])
+        if lr is None:      # the scale-agnostic step of the means is not bounded by the rate; compare relatively
+            s = np.abs(p32[k].astype(np.float64) - ref.means)
+            assert (d > 0.02 * s + 1e-6).mean() < 1e-3, k
+        else:
+            assert (d > 0.02 * h[lr]).mean() < 1e-3, (k, float((d > 0.02 * h[lr]).mean()))
+    d = np.abs(p32["features_sh"].astype(np.float64) - v1)
+    assert (d > tol + 0.02 * h["lr_features_sh"]).mean() < 1e-3
