@@ -1042,11 +1042,14 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
         const int64_t cell0 = block0 * R;
         const int n_cells = n_here * R;
         const float old_lo = P.sh_value_bounds[2 * blockIdx.x], old_hi = P.sh_value_bounds[2 * blockIdx.x + 1];
+        // the block's cells through 32-bit offsets from its first cell: cell (sp, k) is at sp * R + k
+        uint16_t* const state_cells = P.sh_state_packed + cell0;
+        uint16_t* const value_cells = P.sh_value_packed + cell0;
         auto step_cell = [&](int sp, int k, float& m1, float& m2, float& xn) {
-            const int64_t cell = cell0 + (int64_t)sp * R + k;
-            const uint32_t code = P.sh_state_packed[cell];
+            const int cell = sp * R + k;
+            const uint32_t code = state_cells[cell];
             ssr_adamq_decode_with(code, old_mm, s_sqrt_g2[code >> 8], &m1, &m2);
-            const float x = ssr_q16_decode(P.sh_value_packed[cell], old_lo, old_hi);
+            const float x = ssr_q16_decode(value_cells[cell], old_lo, old_hi);
             const int j = k / 3, c = k - 3 * j;
             float v = s_Y[sp][j] * s_vc[sp][c] + sh_reg * x;
             if (kCtl) v = v / s_ctl[sp][c];
@@ -1116,11 +1119,10 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
             int sp = (int)threadIdx.x / R, k = (int)threadIdx.x - sp * R;
             const int dsp = kProjBlock / R, dk = kProjBlock - dsp * R;
             for (int e = threadIdx.x; e < n_cells; e += kProjBlock) {
-                const int64_t cell = cell0 + (int64_t)sp * R + k;
                 float m1 = 0.0f, m2 = 0.0f, xn = 0.0f;
                 if (k < kPer) step_cell(sp, k, m1, m2, xn);
-                P.sh_state_packed[cell] = (uint16_t)ssr_adamq_encode(m1, m2, new_mm);
-                P.sh_value_packed[cell] = (uint16_t)ssr_q16_encode(xn, new_lo, new_hi);
+                state_cells[e] = (uint16_t)ssr_adamq_encode(m1, m2, new_mm);     // e == sp * R + k
+                value_cells[e] = (uint16_t)ssr_q16_encode(xn, new_lo, new_hi);
                 sp += dsp; k += dk;
                 if (k >= R) { k -= R; sp++; }
             }
