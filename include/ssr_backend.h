@@ -18,7 +18,8 @@
  *    cleared) by ssr_last_error(), like the reference's sticky backend::last_error()
  *    (src/backend/api/BackendRuntime.h:98). Nothing calls exit().
  *  - Supported variant: primitive "3dgs" (not antialiased), camera PINHOLE or EQUIRECTANGULAR,
- *    distortion NONE, one camera (C = 1), SH degree 0..3, dist_type None / D / RGB_D, median
+ *    distortion NONE, one camera per projection launch (the host layer loops over a [C,4,4] set;
+ *    tiling and compositing take the C images in one launch), SH degree 0..3, dist_type None / D / RGB_D, median
  *    depth, accumulation weights; both the [C,N] layout and the packed (compacted, nnz rows) layout of
  *    the projection outputs. Anything else is rejected with an error, as the reference
  *    rejects an uncompiled variant (src/kernels/projection/ProjectionFwd.cu:84-89).
@@ -191,6 +192,14 @@ int ssr_tile_write(int64_t n, const float* aabb, const float* sort_depth, const 
                    uint32_t width, uint32_t height, int64_t* isect_ids, int32_t* flatten_ids,
                    const int32_t* visible_ids, int64_t n_visible, const int32_t* tile_active,
                    ssr_stream_t stream);
+/* The same over the rows of several images at once: row r belongs to image r / rows_per_image
+ * and its keys carry tile ids offset by image * tiles-per-image (the reference's
+ * (camera_id * n_tiles + tile) key, IntersectTile.cu:215-262). n must be a multiple of
+ * rows_per_image; no work list and no tile-skip map here. */
+int ssr_tile_write_images(int64_t n, int64_t rows_per_image, const float* aabb, const float* sort_depth,
+                          const float* xy, const float* conic, const float* opac, const int64_t* cum_tiles,
+                          uint32_t width, uint32_t height, int64_t* isect_ids, int32_t* flatten_ids,
+                          ssr_stream_t stream);
 /* sort_pairs<int64,int32> with CUB DoubleBuffer semantics (src/backend/common/SortScan.h:42-56;
  * call site IntersectTile.cu:486-493): stable on bits [begin_bit,end_bit); *selector says which
  * of the (a,b) buffers holds the result. */
@@ -238,6 +247,11 @@ typedef struct {
     float* distortion_rgb;      /* [H,W,3], RGB_D */
     float* distortion_depth;    /* [H,W], D and RGB_D */
     float* render_median;       /* optional [H,W] */
+    /* Images rendered by one launch (0 counts as 1). Image c owns tiles [c T, (c+1) T) of
+     * tile_offsets (T = tiles of one image) and pixels [c H W, (c+1) H W) of every per-pixel
+     * buffer; the splat rows stay global, as the reference's [C,N,...] layout has them
+     * (RasterizationFwd.cu grid = {C, tile_h, tile_w}). */
+    int32_t num_images;
 } ssr_raster_fwd_params;
 int ssr_raster_fwd(const ssr_raster_fwd_params* p, ssr_stream_t stream);
 
@@ -284,6 +298,7 @@ typedef struct {
     const int32_t* gaussian_ids;      /* optional [num_splats] (packed projection) */
     int64_t num_world;                /* rows per lane of accum_weight */
     float* accum_weight;              /* [num_world] or [2 num_world] (AVG) */
+    int32_t num_images;               /* as in ssr_raster_fwd_params; accum_mode needs one image */
 } ssr_raster_bwd_params;
 int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t stream);
 

@@ -86,16 +86,18 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
     __shared__ float s_acc[kBatch * kAccCh];
     // distortion composites ln(max(z, 1e-6)): a per-splat value, taken once when the fragment is staged
     [[maybe_unused]] __shared__ float s_lz[kDist != SSR_DIST_NONE ? kBatch : 1];
-    const int n_tiles = tile_w * tile_h;
+    // images stack in the tile space: image c owns tiles [c tile_w tile_h, (c+1) tile_w tile_h)
+    const int n_tiles = tile_w * tile_h * (P.num_images > 1 ? P.num_images : 1);
     const int tile = xcd_tile_of(blockIdx.x, n_tiles);
     if (tile >= n_tiles) return;
     const int tid = threadIdx.x, lane = tid & 63, mt = tid >> 6;
-    const int ty = tile / tile_w, tx = tile - ty * tile_w;
+    const int gy = tile / tile_w, tx = tile - gy * tile_w;
+    const int img = gy / tile_h, ty = gy - img * tile_h;
     const int j = tx * kTile + (mt & 1) * kMicro + (lane & 7);
     const int i = ty * kTile + (mt >> 1) * kMicro + (lane >> 3);
     const float px = (float)j + 0.5f, py = (float)i + 0.5f;
     const bool inside = (uint32_t)i < P.height && (uint32_t)j < P.width;
-    const int64_t pid = (int64_t)i * P.width + j;
+    const int64_t pid = ((int64_t)img * P.height + i) * P.width + j;
 
     // per-pixel state (RasterizationEval3DBwd_kernel.cuh:186-232)
     const int32_t bin_final = inside ? P.last_ids[pid] : -1;
@@ -367,7 +369,11 @@ extern "C" int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t strea
         SSR_REQUIRE(p->num_world > 0, "ssr_raster_bwd", "num_world must be positive");
     }
     const int tw = (int)ceil_div(p->width, kTile), th = (int)ceil_div(p->height, kTile);
-    const dim3 grid((unsigned)xcd_grid_size(tw * th)), block(kRasterBlock);
+    SSR_REQUIRE(p->num_images >= 0, "ssr_raster_bwd", "negative num_images");
+    const int nimg = p->num_images > 1 ? p->num_images : 1;
+    SSR_REQUIRE((int64_t)tw * th * nimg < (int64_t)1 << 30, "ssr_raster_bwd", "too many tiles");
+    SSR_REQUIRE(nimg == 1 || p->accum_mode == SSR_ACCUM_NONE, "ssr_raster_bwd", "weight accumulation takes one image per call");
+    const dim3 grid((unsigned)xcd_grid_size(tw * th * nimg)), block(kRasterBlock);
     hipStream_t st = as_stream(stream);
     const bool med = p->v_render_median != nullptr;
 #define SSR_BWD(D, M, A) hipLaunchKernelGGL((raster_bwd_kernel<D, M, A>), grid, block, 0, st, *p, tw, th)

@@ -17,11 +17,13 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_kernel(ssr_raster_fwd
     __shared__ FragLds frags[kBatch];
     // distortion composites ln(max(z, 1e-6)): a per-splat value, taken once when the fragment is staged
     [[maybe_unused]] __shared__ float s_lz[kDist != SSR_DIST_NONE ? kBatch : 1];
-    const int n_tiles = tile_w * tile_h;
+    // images stack in the tile space: image c owns tiles [c tile_w tile_h, (c+1) tile_w tile_h)
+    const int n_tiles = tile_w * tile_h * (P.num_images > 1 ? P.num_images : 1);
     const int tile = xcd_tile_of(blockIdx.x, n_tiles);
     if (tile >= n_tiles) return;   // whole workgroup leaves together
     const int tid = threadIdx.x, lane = tid & 63, mt = tid >> 6;
-    const int ty = tile / tile_w, tx = tile - ty * tile_w;
+    const int gy = tile / tile_w, tx = tile - gy * tile_w;
+    const int img = gy / tile_h, ty = gy - img * tile_h;
     const int j = tx * kTile + (mt & 1) * kMicro + (lane & 7);
     const int i = ty * kTile + (mt >> 1) * kMicro + (lane >> 3);
     const float px = (float)j + 0.5f, py = (float)i + 0.5f;
@@ -94,7 +96,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_kernel(ssr_raster_fwd
         }
     }
     if (inside) {
-        const int64_t pid = (int64_t)i * P.width + j;
+        const int64_t pid = ((int64_t)img * P.height + i) * P.width + j;
         P.render_T[pid] = T;
         const float invW = 1.0f / ssr_max(1.0f - T, 1e-10f);
         float* o = P.render_rgb + 3 * pid;
@@ -140,7 +142,10 @@ extern "C" int ssr_raster_fwd(const ssr_raster_fwd_params* p, ssr_stream_t strea
     SSR_REQUIRE(p->dist_type == SSR_DIST_NONE || p->distortion_depth, "ssr_raster_fwd", "null distortion_depth");
     SSR_REQUIRE(p->dist_type != SSR_DIST_RGB_D || p->distortion_rgb, "ssr_raster_fwd", "null distortion_rgb");
     const int tw = (int)ceil_div(p->width, kTile), th = (int)ceil_div(p->height, kTile);
-    const dim3 grid((unsigned)xcd_grid_size(tw * th)), block(kRasterBlock);
+    SSR_REQUIRE(p->num_images >= 0, "ssr_raster_fwd", "negative num_images");
+    const int nimg = p->num_images > 1 ? p->num_images : 1;
+    SSR_REQUIRE((int64_t)tw * th * nimg < (int64_t)1 << 30, "ssr_raster_fwd", "too many tiles");
+    const dim3 grid((unsigned)xcd_grid_size(tw * th * nimg)), block(kRasterBlock);
     hipStream_t s = as_stream(stream);
 #define SSR_FWD(D, M) hipLaunchKernelGGL((raster_fwd_kernel<D, M>), grid, block, 0, s, *p, tw, th)
     const bool med = p->render_median != nullptr;

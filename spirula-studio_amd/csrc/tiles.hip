@@ -74,7 +74,8 @@ __global__ __launch_bounds__(kTileBlock) void tile_write_kernel(
     int64_t n, const float4* __restrict__ aabb, const float* __restrict__ sort_depth,
     const float2* __restrict__ xy, const float* __restrict__ conic, const float* __restrict__ opac,
     const int64_t* __restrict__ cum, int tile_w, int tile_h, int64_t* __restrict__ isect_ids,
-    int32_t* __restrict__ flatten_ids, const int32_t* __restrict__ visible_ids, const int32_t* __restrict__ live) {
+    int32_t* __restrict__ flatten_ids, const int32_t* __restrict__ visible_ids, const int32_t* __restrict__ live,
+    uint32_t rows_per_image) {
     const int64_t i = (int64_t)blockIdx.x * kTileBlock + threadIdx.x;
     const int lane = threadIdx.x & 63;
     const bool in_range = i < n;
@@ -83,6 +84,9 @@ __global__ __launch_bounds__(kTileBlock) void tile_write_kernel(
     TileGeomD tg;
     uint32_t du = 0;
     bool visible = false;
+    // several images in one launch: row g belongs to image g / rows_per_image, whose tiles follow
+    // the earlier images' in the key space
+    const int tile_base = rows_per_image ? (int)((uint32_t)g / rows_per_image) * (tile_w * tile_h) : 0;
     if (in_range) {
         cur = g == 0 ? 0 : cum[g - 1];
         end = cum[g];
@@ -103,7 +107,7 @@ __global__ __launch_bounds__(kTileBlock) void tile_write_kernel(
         for_each_tile(tg, [&](int lo, int hi, int fixed, bool rows) {
             for (int v = lo; v < hi && cur < end; v++) {
                 if (live && !tile_is_live(live, tile_w, fixed, v, rows)) continue;
-                const int64_t tile_id = rows ? ((int64_t)fixed * tile_w + v) : ((int64_t)v * tile_w + fixed);
+                const int64_t tile_id = tile_base + (rows ? ((int64_t)fixed * tile_w + v) : ((int64_t)v * tile_w + fixed));
                 isect_ids[cur] = (int64_t)(((uint64_t)tile_id << 32) | (uint64_t)du);
                 flatten_ids[cur] = (int32_t)g;
                 ++cur;
@@ -130,6 +134,7 @@ __global__ __launch_bounds__(kTileBlock) void tile_write_kernel(
         sg.by_rows = __shfl((int)tg.by_rows, src, 64) != 0;
         const uint32_t sdu = (uint32_t)__shfl((int)du, src, 64);
         const int32_t sgid = (int32_t)__shfl((int)g, src, 64);
+        const int sbase = __shfl(tile_base, src, 64);
         int64_t scur = ((int64_t)__shfl((int)(cur >> 32), src, 64) << 32) | (uint32_t)__shfl((int)(uint32_t)cur, src, 64);
         const int64_t send = ((int64_t)__shfl((int)(end >> 32), src, 64) << 32) | (uint32_t)__shfl((int)(uint32_t)end, src, 64);
         const int b0 = sg.by_rows ? sg.ymin : sg.xmin, b1 = sg.by_rows ? sg.ymax : sg.xmax;
@@ -142,7 +147,7 @@ __global__ __launch_bounds__(kTileBlock) void tile_write_kernel(
             int64_t pos = scur + (inc - c);
             for (int v = lo; v < hi && pos < send; v++) {
                 if (live && !tile_is_live(live, tile_w, r, v, sg.by_rows)) continue;
-                const int64_t tile_id = sg.by_rows ? ((int64_t)r * tile_w + v) : ((int64_t)v * tile_w + r);
+                const int64_t tile_id = sbase + (sg.by_rows ? ((int64_t)r * tile_w + v) : ((int64_t)v * tile_w + r));
                 isect_ids[pos] = (int64_t)(((uint64_t)tile_id << 32) | (uint64_t)sdu);
                 flatten_ids[pos] = sgid;
                 pos++;
@@ -324,8 +329,32 @@ int ssr_tile_write(int64_t n, const float* aabb, const float* sort_depth, const 
     const int64_t work = visible_ids ? n_visible : n;
     hipLaunchKernelGGL(tile_write_kernel, dim3((unsigned)ceil_div(work, kTileBlock)), dim3(kTileBlock), 0, as_stream(stream),
                        work, reinterpret_cast<const float4*>(aabb), sort_depth, reinterpret_cast<const float2*>(xy), conic, opac,
-                       cum_tiles, tw, th, isect_ids, flatten_ids, visible_ids, tile_active);
+                       cum_tiles, tw, th, isect_ids, flatten_ids, visible_ids, tile_active, 0u);
     SSR_CHECK_LAUNCH("ssr_tile_write");
+    return 0;
+}
+
+int ssr_tile_write_images(int64_t n, int64_t rows_per_image, const float* aabb, const float* sort_depth,
+                          const float* xy, const float* conic, const float* opac, const int64_t* cum_tiles,
+                          uint32_t width, uint32_t height, int64_t* isect_ids, int32_t* flatten_ids,
+                          ssr_stream_t stream) {
+    SSR_REQUIRE(n >= 0 && n < (int64_t)1 << 31, "ssr_tile_write_images", "count out of range");
+    if (n == 0) return 0;
+    SSR_REQUIRE(rows_per_image > 0 && n % rows_per_image == 0, "ssr_tile_write_images",
+                "n must be a positive multiple of rows_per_image");
+    SSR_REQUIRE(aabb && sort_depth && xy && conic && opac && cum_tiles, "ssr_tile_write_images", "null pointer");
+    SSR_REQUIRE(isect_ids && flatten_ids, "ssr_tile_write_images", "null output (n_isects == 0 needs no call)");
+    SSR_REQUIRE(width > 0 && height > 0, "ssr_tile_write_images", "empty image");
+    SSR_REQUIRE((reinterpret_cast<uintptr_t>(aabb) & 15) == 0 && (reinterpret_cast<uintptr_t>(xy) & 7) == 0,
+                "ssr_tile_write_images", "aabb must be 16-byte and xy 8-byte aligned");
+    const int tw = (int)ceil_div(width, kTile), th = (int)ceil_div(height, kTile);
+    SSR_REQUIRE((n / rows_per_image) * (int64_t)tw * th < (int64_t)1 << 31, "ssr_tile_write_images",
+                "tile ids of all images must fit 31 bits");
+    hipLaunchKernelGGL(tile_write_kernel, dim3((unsigned)ceil_div(n, kTileBlock)), dim3(kTileBlock), 0, as_stream(stream),
+                       n, reinterpret_cast<const float4*>(aabb), sort_depth, reinterpret_cast<const float2*>(xy), conic, opac,
+                       cum_tiles, tw, th, isect_ids, flatten_ids, (const int32_t*)nullptr, (const int32_t*)nullptr,
+                       (uint32_t)rows_per_image);
+    SSR_CHECK_LAUNCH("ssr_tile_write_images");
     return 0;
 }
 

@@ -111,11 +111,16 @@ class Engine:
             be = bounds.itemsize if scene.sh_codec == 3 else 8
             check(self.h.ssrh_set_sh_value_quant(bits, packed.ctypes.data, packed.size, packed.itemsize,
                                                  bounds.ctypes.data, bounds.shape[0], be, scene.sh_bounds_stride))
+        # a [C,4,4] viewmat (with [C,4] intrins, [C,8] coefficients and [C,H,W,...] cotangents) renders C
+        # cameras in one pass; a [4,4] one is the single camera
         vm, it = f32(scene.viewmat), f32(scene.intrins)
+        self.num_cameras = vm.shape[0] if vm.ndim == 3 else 1
         tier = int(getattr(scene, "distortion", 0))
-        dc = f32(np.zeros(8) if getattr(scene, "dist_coeffs", None) is None else scene.dist_coeffs)
+        dc = f32(np.zeros(8 * self.num_cameras) if getattr(scene, "dist_coeffs", None) is None else scene.dist_coeffs)
+        assert vm.size == 16 * self.num_cameras and it.size == 4 * self.num_cameras and dc.size == 8 * self.num_cameras
         check(self.h.ssrh_set_camera_params(scene.width, scene.height, _MODEL[scene.camera_model], _LENS[tier],
-                                            vm.ctypes.data, it.ctypes.data, dc.ctypes.data, 1))
+                                            vm.ctypes.data, it.ctypes.data, dc.ctypes.data, self.num_cameras))
+        assert np.size(scene.v_T) == self.num_cameras * scene.height * scene.width
         # cotangents resident on the device
         self.d_vrgb = _lib.DeviceArray.from_host(f32(scene.v_rgb))
         self.d_vdepth = _lib.DeviceArray.from_host(f32(scene.v_depth))
@@ -151,9 +156,9 @@ class Engine:
 
     def backward_with_pose_grad(self):
         """The backward plus the camera-pose gradient: returns dL/d[R|t] as [4,4] (last row zero)."""
-        out = np.zeros((4, 4), np.float32)
+        out = np.zeros((self.num_cameras, 4, 4), np.float32)
         check(self.h.ssrh_backward_with_pose_grad(self.d_vrgb.ptr, self.d_vdepth.ptr, self.d_vT.ptr, out.ctypes.data))
-        return out
+        return out if self.num_cameras > 1 else out[0]
 
     HYPER = ["lr_means", "lr_quats", "lr_scales", "lr_opacs", "lr_features_dc", "lr_features_sh", "max_gauss_ratio",
              "scale_regularization_weight", "mcmc_opacity_reg_weight", "mcmc_scale_reg_weight", "quat_norm_reg_weight",
@@ -212,7 +217,8 @@ class Engine:
 
     def render(self):
         h, w = self.sc.height, self.sc.width
-        rgb, depth, T = np.zeros((h, w, 3), np.float32), np.zeros((h, w), np.float32), np.zeros((h, w), np.float32)
+        lead = (self.num_cameras,) if self.num_cameras > 1 else ()
+        rgb, depth, T = np.zeros(lead + (h, w, 3), np.float32), np.zeros(lead + (h, w), np.float32), np.zeros(lead + (h, w), np.float32)
         check(self.h.ssrh_copy_render_to_host(rgb.ctypes.data, depth.ctypes.data, T.ctypes.data))
         return rgb, depth, T
 

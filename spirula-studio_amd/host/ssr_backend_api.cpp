@@ -112,7 +112,8 @@ ssr_sh_quant sh_of(const std::optional<TorchTensorView>& packed, const std::opti
     return q;
 }
 ssr_camera camera_of(const std::string& model, const std::string& distortion, const TorchTensorView& dist_coeffs,
-                     const TorchTensorView& viewmats, const TorchTensorView& intrins, uint32_t w, uint32_t h) {
+                     const TorchTensorView& viewmats, const TorchTensorView& intrins, uint32_t w, uint32_t h,
+                     bool several_ok = false) {
     ssr_camera c;
     c.camera_model = camera_model_of(model);
     c.distortion = lens_tier_of(distortion);
@@ -128,11 +129,30 @@ ssr_camera camera_of(const std::string& model, const std::string& distortion, co
     }
     const auto& shape = std::get<2>(viewmats);
     c.num_cameras = shape.empty() ? 0u : (uint32_t)shape[0];
-    if (c.num_cameras != 1) throw std::runtime_error("this backend runs one camera per call (got " + std::to_string(c.num_cameras) + ")");
+    if (c.num_cameras < 1 || (c.num_cameras != 1 && !several_ok))
+        throw std::runtime_error("this entry point runs one camera per call (got " + std::to_string(c.num_cameras) + ")");
     c.width = w; c.height = h;
     c.viewmats = (const float*)std::get<0>(viewmats);
     c.intrins = (const float*)std::get<0>(intrins);
     return c;
+}
+// Camera i of a [C, ...] set, as a one-camera set: the kernels take one camera per launch
+ssr_camera camera_at(const ssr_camera& all, uint32_t i) {
+    ssr_camera c = all;
+    c.num_cameras = 1;
+    c.viewmats = all.viewmats + 16 * (size_t)i;
+    c.intrins = all.intrins + 4 * (size_t)i;
+    if (all.dist_coeffs) c.dist_coeffs = all.dist_coeffs + 8 * (size_t)i;
+    return c;
+}
+ssr_screen screen_rows_from(const ssr_screen& s, int64_t row) {
+    ssr_screen o = s;
+    if (s.xy) o.xy = s.xy + 2 * row;
+    if (s.depth) o.depth = s.depth + row;
+    if (s.conic) o.conic = s.conic + 3 * row;
+    if (s.opac) o.opac = s.opac + row;
+    if (s.rgb) o.rgb = s.rgb + 3 * row;
+    return o;
 }
 
 }  // namespace
@@ -240,8 +260,10 @@ projection_3dgs_forward(const int64_t num_splats, const int max_sh_degree,
     p.antialiased = g_antialiased ? 1 : 0;
     p.world = world_of(in_splats);
     p.sh = sh_of(sh_value_packed, sh_value_bounds, num_sh_buffer, sh_value_bits, sh_bounds_stride);
-    p.camera = camera_of(camera_model, distortion, dist_coeffs, viewmats, intrins, image_width, image_height);
-    const int64_t C = 1, N = num_splats;
+    // Several cameras ([C,4,4] viewmats): one projection launch per camera into row block c of the
+    // [C,N,...] outputs (the reference's single launch covers C*N rows, ProjectionFwd_kernel.cuh:60-110).
+    const ssr_camera cameras = camera_of(camera_model, distortion, dist_coeffs, viewmats, intrins, image_width, image_height, true);
+    const int64_t C = cameras.num_cameras, N = num_splats;
 
     DeviceTensor2D<float4> aabb; aabb.resize(PoolSlot::ProjAabb, C, N);
     DeviceTensor2D<float> depths; depths.resize(PoolSlot::ProjDepths, C, N);
@@ -261,7 +283,7 @@ projection_3dgs_forward(const int64_t num_splats, const int max_sh_degree,
     g_counters = DevicePool::global().acquire<int64_t>(PoolSlot::IsectCounters, 2);
     g_visible_ids = nullptr;
     g_n_visible = -1;
-    if (g_opts.visible_list) {
+    if (g_opts.visible_list && C == 1) {   // one list and one counter: a single camera's
         g_list_toggle ^= 1;
         g_visible_ids = DevicePool::global().acquire<int32_t>(
             g_list_toggle ? PoolSlot::ProjVisibleIdsB : PoolSlot::ProjVisibleIds, (size_t)(C * N));
@@ -278,7 +300,15 @@ projection_3dgs_forward(const int64_t num_splats, const int max_sh_degree,
     }
     {
         StageTimer t(&g_times.k1);
-        ok(ssr_projection_fwd(&p, nullptr), "projection_3dgs_forward");
+        const ssr_projection_fwd_params all = p;
+        for (int64_t c = 0; c < C; c++) {
+            p.camera = camera_at(cameras, (uint32_t)c);
+            p.aabb = all.aabb + 4 * c * N; p.sort_depth = all.sort_depth + c * N;
+            p.screen = screen_rows_from(all.screen, c * N);
+            if (all.tiles_per_splat) p.tiles_per_splat = all.tiles_per_splat + c * N;
+            if (all.packed_rows) p.packed_rows = all.packed_rows + 12 * c * N;
+            ok(ssr_projection_fwd(&p, nullptr), "projection_3dgs_forward");
+        }
     }
     std::vector<DeviceTensorFloatND> screen = {
         DeviceTensorFloatND(xy, {C * N, 2}), DeviceTensorFloatND(dp, {C * N, 1}), DeviceTensorFloatND(cn, {C * N, 3}),
@@ -380,8 +410,11 @@ do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, 
     // the single camera this backend runs, every image id is 0 and the array itself is not read.
     if (!proj_xy || !proj_conic || !proj_opac)
         throw std::runtime_error("do_intersect_tile_generic: AABB mode is not built in this backend (ellipse mode is)");
-    if (I != 1) throw std::runtime_error("do_intersect_tile_generic: this backend runs one image per call");
+    if (I < 1) throw std::runtime_error("do_intersect_tile_generic: no image");
+    if (I > 1 && (image_ids || tile_active))
+        throw std::runtime_error("do_intersect_tile_generic: packed rows and the tile-skip map take one image per call");
     const int64_t total = depths.numel();
+    if (total % I != 0) throw std::runtime_error("do_intersect_tile_generic: rows are not a multiple of the image count");
     const uint32_t tile_w = (image_width + 15) / 16, tile_h = (image_height + 15) / 16;
     const uint32_t n_tiles = tile_w * tile_h * I;
 
@@ -422,6 +455,11 @@ do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, 
     DeviceVector<int32_t> flat_a, flat_b; flat_a.resize(PoolSlot::IsectFlatA, n_isects); flat_b.resize(PoolSlot::IsectFlatB, n_isects);
     {
         StageTimer t(&g_times.k4);
+        if (I > 1)   // keys carry image * tiles + tile (IntersectTile.cu:215-262)
+            ok(ssr_tile_write_images(total, total / I, aabb.data_ptr(), depths.data_ptr(), proj_xy->data_ptr(),
+                                     proj_conic->data_ptr(), proj_opac->data_ptr(), cum.data_ptr(), image_width, image_height,
+                                     ids_a.data_ptr(), flat_a.data_ptr(), nullptr), "do_intersect_tile_generic/write");
+        else
         ok(ssr_tile_write(total, aabb.data_ptr(), depths.data_ptr(), proj_xy->data_ptr(), proj_conic->data_ptr(),
                           proj_opac->data_ptr(), cum.data_ptr(), image_width, image_height, ids_a.data_ptr(),
                           flat_a.data_ptr(), g_visible_ids, g_visible_ids ? g_n_visible : 0, tile_active, nullptr),
@@ -461,7 +499,8 @@ rasterize_to_pixels_3dgs_fwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     if (dist_type == DistortionType::DN || dist_type == DistortionType::RGB_DN)
         throw std::runtime_error("rasterize_to_pixels_3dgs_fwd: normal distortion needs a normal channel, which the 3dgs pixel does not have");
     const int64_t I = tile_offsets.size<0>();
-    if (I != 1) throw std::runtime_error("rasterize_to_pixels_3dgs_fwd: this backend runs one image per call");
+    if (I < 1) throw std::runtime_error("rasterize_to_pixels_3dgs_fwd: no image");
+    if (I > 1 && gaussian_ids.data_ptr()) throw std::runtime_error("rasterize_to_pixels_3dgs_fwd: packed rows take one image per call");
     RenderOutput::TensorTuple renders;
     std::get<0>(renders).resize(PoolSlot::RendersRgb, I, image_height, image_width);
     std::get<1>(renders).resize(PoolSlot::RendersDepth, I, image_height, image_width);
@@ -469,7 +508,8 @@ rasterize_to_pixels_3dgs_fwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     DeviceTensor3D<int32_t> last; last.resize(PoolSlot::RenderLastIds, I, image_height, image_width);
     ssr_raster_fwd_params p;
     std::memset(&p, 0, sizeof(p));
-    p.num_splats = num_splats;
+    p.num_splats = I > 1 && !splats_s.empty() ? splats_s[0].rows() : num_splats;   // [C,N] rows
+    p.num_images = (int32_t)I;
     if (flatten_ids.size() > 0) p.screen = screen_of(splats_s);
     p.width = image_width; p.height = image_height;
     p.tile_offsets = tile_offsets.data_ptr(); p.flatten_ids = flatten_ids.data_ptr(); p.n_isects = flatten_ids.size();
@@ -545,7 +585,11 @@ rasterize_to_pixels_3dgs_bwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     }
     ssr_raster_bwd_params p;
     std::memset(&p, 0, sizeof(p));
-    p.num_splats = num_splats;
+    const int64_t I = tile_offsets.size<0>();
+    if (I > 1 && (gaussian_ids.data_ptr() || accum_mode != DensifyAccumMode::None))
+        throw std::runtime_error("rasterize_to_pixels_3dgs_bwd: packed rows and weight accumulation take one image per call");
+    p.num_splats = I > 1 && !splats_s.empty() ? splats_s[0].rows() : num_splats;   // [C,N] rows
+    p.num_images = (int32_t)I;
     p.screen = screen_of(splats_s);
     p.width = image_width; p.height = image_height;
     p.tile_offsets = tile_offsets.data_ptr(); p.flatten_ids = flatten_ids.data_ptr(); p.n_isects = flatten_ids.size();
@@ -609,13 +653,15 @@ void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
     p.antialiased = g_antialiased ? 1 : 0;
     p.world = world_of(splats_world);
     p.sh = sh_of(sh_value_packed, sh_value_bounds, num_sh_buffer, sh_value_bits, sh_bounds_stride);
-    p.camera = camera_of(camera_model, distortion, dist_coeffs, viewmats, intrins, image_width, image_height);
+    const ssr_camera cameras = camera_of(camera_model, distortion, dist_coeffs, viewmats, intrins, image_width, image_height, !is_packed);
+    const int64_t C = cameras.num_cameras;
+    p.camera = camera_at(cameras, 0);
     p.aabb = (const float*)aabb.data_ptr();
     p.v_screen = screen_of(v_splats_screen);
     if (g_vrows && p.v_screen.xy == g_vrows_for_xy) p.v_rows = g_vrows;
     p.v_world = world_of(v_splats_world);
     p.accumulate = g_opts.overwrite_world_grads ? 0 : 1;
-    if (v_viewmats) p.v_viewmat = v_viewmats->data_ptr();   // [C = 1, 16]: accumulated into, as the reference does
+    if (v_viewmats) p.v_viewmat = v_viewmats->data_ptr();   // [C, 16]: accumulated into, as the reference does
     if (is_packed) {
         p.aabb = nullptr;
         p.packed_gaussian_ids = gaussian_ids.data_ptr(); p.num_packed = camera_ids.size();
@@ -627,6 +673,19 @@ void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
     }
     StageTimer t(&g_times.k9);
     ok(ssr_projection_bwd(&p, nullptr), "projection_3dgs_backward");
+    // further cameras: one launch each over row block c of the [C,N,...] gradients, added into the
+    // world gradients the first launch wrote (the reference's single launch sums them with
+    // atomicStore, src/kernels/projection/ProjectionBwd_kernel.cuh:107)
+    const ssr_projection_bwd_params first = p;
+    for (int64_t c = 1; c < C; c++) {
+        p.camera = camera_at(cameras, (uint32_t)c);
+        p.aabb = first.aabb + 4 * c * num_splats;
+        p.v_screen = screen_rows_from(first.v_screen, c * num_splats);
+        if (first.v_rows) p.v_rows = first.v_rows + 12 * c * num_splats;
+        if (first.v_viewmat) p.v_viewmat = first.v_viewmat + 16 * c;
+        p.accumulate = 1;
+        ok(ssr_projection_bwd(&p, nullptr), "projection_3dgs_backward");
+    }
 }
 
 void fused_projection_bwd_optimizer_3dgs(

@@ -510,11 +510,11 @@ int ssrh_backward_from_render_grad(const float* v_rgb, const float* v_depth, con
 int ssrh_backward_with_pose_grad(const float* v_rgb, const float* v_depth, const float* v_Ts, float* out16) {
     return guard([&] {
         const int64_t C = engine().camera.num, H = engine().camera.height, W = engine().camera.width;
-        float* d = DevicePool::global().acquire<float>(PoolSlot::EngPoseGrad, 16);
-        backend::memset_async(d, 0, 16 * sizeof(float));
-        DeviceTensor2D<float> vm(d, 1, 16);
+        float* d = DevicePool::global().acquire<float>(PoolSlot::EngPoseGrad, (size_t)(16 * C));
+        backend::memset_async(d, 0, (size_t)(16 * C) * sizeof(float));
+        DeviceTensor2D<float> vm(d, C, 16);
         engine_backward_from_render_grad(tv(v_rgb, 4, {C, H, W, 3}), tv(v_depth, 4, {C, H, W, 1}), tv(v_Ts, 4, {C, H, W, 1}), &vm);
-        backend::memcpy_sync(out16, d, 16 * sizeof(float), backend::MemcpyKind::DeviceToHost);
+        backend::memcpy_sync(out16, d, (size_t)(16 * C) * sizeof(float), backend::MemcpyKind::DeviceToHost);
     });
 }
 

@@ -54,7 +54,8 @@ class RasterFwdParams(C.Structure):
                 ("height", C.c_uint32), ("tile_offsets", vp), ("flatten_ids", vp),
                 ("n_isects", C.c_int64), ("render_rgb", vp), ("render_depth", vp),
                 ("render_T", vp), ("last_ids", vp), ("packed_rows", vp), ("dist_type", C.c_int32),
-                ("distortion_rgb", vp), ("distortion_depth", vp), ("render_median", vp)]
+                ("distortion_rgb", vp), ("distortion_depth", vp), ("render_median", vp),
+                ("num_images", C.c_int32)]
 
 
 class RasterBwdParams(C.Structure):
@@ -65,7 +66,8 @@ class RasterBwdParams(C.Structure):
                 ("v_screen", Screen), ("packed_rows", vp), ("v_rows", vp), ("dist_type", C.c_int32), ("render_rgb", vp),
                 ("distortion_rgb", vp), ("distortion_depth", vp), ("v_distortion_rgb", vp),
                 ("v_distortion_depth", vp), ("v_render_median", vp), ("accum_mode", C.c_int32),
-                ("accum_weight_map", vp), ("gaussian_ids", vp), ("num_world", C.c_int64), ("accum_weight", vp)]
+                ("accum_weight_map", vp), ("gaussian_ids", vp), ("num_world", C.c_int64), ("accum_weight", vp),
+                ("num_images", C.c_int32)]
 
 
 class ProjectionBwdParams(C.Structure):
@@ -115,6 +117,7 @@ SYMBOLS = {
     "ssr_inclusive_sum_i64": (_i32, [vp, vp, _i64, vp, vp, _sz, vp]),
     "ssr_read_i64": (_i32, [vp, C.POINTER(C.c_int64), _i32, vp]),
     "ssr_tile_write": (_i32, [_i64, vp, vp, vp, vp, vp, vp, _u32, _u32, vp, vp, vp, _i64, vp, vp]),
+    "ssr_tile_write_images": (_i32, [_i64, _i64, vp, vp, vp, vp, vp, vp, _u32, _u32, vp, vp, vp]),
     "ssr_sort_scratch_bytes": (_sz, [_i64]),
     "ssr_sort_pairs_u64_i32": (_i32, [vp, vp, vp, vp, _i64, _i32, _i32, C.POINTER(C.c_int), vp, _sz, vp]),
     "ssr_tile_offsets": (_i32, [_i64, vp, _u32, vp, vp]),

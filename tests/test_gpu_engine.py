@@ -572,3 +572,92 @@ def test_runtime_contract(pkg, H):
     for e in (ev, e0, e1):
         L.ssr_event_destroy(e)
     L.ssr_device_free(d); L.ssr_device_free(d2); L.ssr_host_free_pinned(p)
+
+
+@pytest.mark.parametrize("native", [False, True])
+def test_engine_two_cameras(pkg, oracle, H, native):
+    """[C = 2] viewmats through the adapter (the reference's entry points take [C,4,4] cameras and render C
+    images in one pass: ProjectionFwd_kernel.cuh:60-110, IntersectTile.cu:215-262, RasterizationFwd.cu grid
+    {C, tile_h, tile_w}). Against the oracle run once per camera: image c's keys carry tile ids offset by
+    c * tiles and row ids offset by c * N, its pixels and last ids are the single camera's, the world
+    gradients and radii combine both cameras, and each camera gets its own pose gradient."""
+    import copy
+    host, lib = H
+    S = pkg.scenes
+    base = S.tiny_scene(n=3000, width=250, height=180, seed=71)   # ragged edge tiles in both directions
+    cams = []
+    for k, (ang, t) in enumerate([(0.2, (0.3, -0.2, 3.0)), (-0.35, (-0.4, 0.1, 3.4))]):
+        c, s_ = np.cos(ang), np.sin(ang)
+        vm = np.array([[c, 0, s_, t[0]], [0, 1, 0, t[1]], [-s_, 0, c, t[2]], [0, 0, 0, 1]], np.float32)
+        it = np.array([150.0 + 20 * k, 155.0 - 10 * k, 125.0, 90.0 + 5 * k], np.float32)
+        cams.append((vm, it))
+    rng = np.random.default_rng(5)
+    h, w, n = base.height, base.width, base.n
+    v_rgb = rng.standard_normal((2, h, w, 3)).astype(np.float32)
+    v_depth = rng.standard_normal((2, h, w)).astype(np.float32)
+    v_T = rng.standard_normal((2, h, w)).astype(np.float32)
+    refs, poses = [], []
+    for k, (vm, it) in enumerate(cams):
+        sc = copy.deepcopy(base)
+        sc.viewmat, sc.intrins = vm, it
+        sc.v_rgb, sc.v_depth, sc.v_T = v_rgb[k], v_depth[k], v_T[k]
+        ref = oracle.pipeline(sc)
+        assert ref["proj"]["visible"] > 100 and ref["sorted_ids"].size > 1000
+        refs.append(ref)
+        poses.append(oracle.projection_bwd(sc, ref["proj"]["aabb"], ref["vscreen"], pose=True)["v_viewmat"].astype(np.float64))
+    both = copy.deepcopy(base)
+    both.viewmat = np.stack([c[0] for c in cams])
+    both.intrins = np.stack([c[1] for c in cams])
+    both.v_rgb, both.v_depth, both.v_T = v_rgb, v_depth, v_T
+    eng = host.Engine(both, fuse_tile_count=native, visible_list=native, packed_rows=native, overwrite_world_grads=native,
+                      packed_vscreen=native, tile_sort=native)
+    tiles = ((w + 15) // 16) * ((h + 15) // 16)
+    for rep in range(2):   # the second pass: zero-fills honoured, nothing accumulates
+        eng.forward()
+        got_pose = eng.backward_with_pose_grad().astype(np.float64)
+        n0 = refs[0]["sorted_ids"].size
+        assert eng.n_isects == n0 + refs[1]["sorted_ids"].size
+        assert np.array_equal(eng.cache("sorted_ids"),
+                              np.concatenate([refs[0]["sorted_ids"], refs[1]["sorted_ids"] + (np.int64(tiles) << 32)]))
+        assert np.array_equal(eng.cache("sorted_flat"), np.concatenate([refs[0]["sorted_flat"], refs[1]["sorted_flat"] + n]))
+        assert np.array_equal(eng.cache("offsets"),
+                              np.concatenate([refs[0]["offsets"].reshape(-1), refs[1]["offsets"].reshape(-1) + n0]))
+        assert np.array_equal(eng.cache("aabb").reshape(2, n, 4), np.stack([r["proj"]["aabb"] for r in refs]))
+        assert np.array_equal(eng.cache("radii"), np.maximum(refs[0]["proj"]["radii"], refs[1]["proj"]["radii"]))
+        rgb, depth, T = eng.render()
+        last = eng.cache("last_ids").reshape(2, h, w)
+        for k in range(2):
+            assert np.abs(rgb[k] - refs[k]["fwd"]["rgb"]).max() <= 1e-4
+            assert np.abs(depth[k] - refs[k]["fwd"]["depth"]).max() <= 1e-4 * max(1.0, np.abs(refs[k]["fwd"]["depth"]).max())
+            assert np.abs(T[k] - refs[k]["fwd"]["T"]).max() <= 1e-4
+            # last_ids are positions in the whole sorted list (image 1's run starts at n0); a pixel no
+            # fragment reached keeps 0 and T = 1
+            reached = refs[k]["fwd"]["T"] < 1.0
+            assert np.array_equal(last[k], np.where(reached, refs[k]["fwd"]["last_ids"] + (n0 if k else 0), 0))
+            assert np.abs(got_pose[k] - poses[k]).max() <= 2e-3 * np.abs(poses[k]).max(), (k, got_pose[k], poses[k])
+        g = eng.grads()
+        for key, v in g.items():
+            r = sum(ref["grads"][key].astype(np.float64) for ref in refs).reshape(n, -1)
+            scale = sum(np.abs(ref["grads"][key].astype(np.float64)).reshape(n, -1).max(axis=1, keepdims=True) for ref in refs)
+            err = np.abs(v.reshape(n, -1) - r)
+            assert (err <= 2e-3 * scale + 2e-5 * (np.abs(r).mean() + 1e-12)).all(), key
+
+
+def test_two_cameras_are_refused_where_one_is_required(pkg, H):
+    """Packed projection, the fused optimizer and the tile-skip map take one camera per call: a [2,4,4]
+    camera set raises instead of rendering the first camera only."""
+    import copy
+    host, lib = H
+    sc = pkg.scenes.tiny_scene(n=500, width=64, height=48, seed=3)
+    sc.viewmat = np.stack([sc.viewmat, sc.viewmat])
+    sc.intrins = np.stack([sc.intrins, sc.intrins])
+    for name in ["v_rgb", "v_depth", "v_T"]:
+        setattr(sc, name, np.stack([getattr(sc, name)] * 2))
+    eng = host.Engine(sc, packed_projection=True)
+    with pytest.raises(lib.SsrError, match="one camera per call"):
+        eng.forward()
+    eng = host.Engine(sc)
+    eng.forward()
+    hyper = dict.fromkeys(host.Engine.HYPER, 0.0)
+    with pytest.raises(lib.SsrError, match="one camera per call"):
+        eng.backward_fused_optimizer(hyper, 1)
