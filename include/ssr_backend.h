@@ -298,7 +298,8 @@ typedef struct {
     const int32_t* gaussian_ids;      /* optional [num_splats] (packed projection) */
     int64_t num_world;                /* rows per lane of accum_weight */
     float* accum_weight;              /* [num_world] or [2 num_world] (AVG) */
-    int32_t num_images;               /* as in ssr_raster_fwd_params; accum_mode needs one image */
+    int32_t num_images;               /* as in ssr_raster_fwd_params; with accum_mode, screen row r
+                                       * adds into world row r % num_world */
 } ssr_raster_bwd_params;
 int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t stream);
 

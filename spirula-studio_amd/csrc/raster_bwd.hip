@@ -74,6 +74,13 @@ __device__ __forceinline__ void atomic_max_f32(float* p, float v) {
 // kDist (SSR_DIST_*), kMedian and kAccum (SSR_ACCUM_*) select the variants
 // (RasterizationEval3DBwd_kernel.cuh:150-172,207-279,433-585); <0, false, 0> is the plain kernel and
 // compiles to exactly the code it had without them.
+// Row of accum_weight a screen row adds into: its world row. Packed rows carry it in gaussian_ids;
+// [C,N] rows are c * N + n (RasterizationEval3DBwd_kernel.cuh:368).
+__device__ __forceinline__ int64_t accum_row(const ssr_raster_bwd_params& P, uint32_t g) {
+    if (P.gaussian_ids) return (int64_t)P.gaussian_ids[g];
+    return P.num_images > 1 ? (int64_t)(g % (uint32_t)P.num_world) : (int64_t)g;
+}
+
 template <int kDist, bool kMedian, int kAccum>
 __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd_params P, int tile_w, int tile_h) {
     __shared__ FragLds frags[kBatch];
@@ -186,7 +193,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
                 if (a != 0.0f || b != 0.0f) {
                     s_acc[tid * kAccCh + 10] = 0.0f; s_acc[tid * kAccCh + 11] = 0.0f;
                     const uint32_t g = (uint32_t)s_ids[tid];
-                    const int64_t wid = P.gaussian_ids ? (int64_t)P.gaussian_ids[g] : (int64_t)g;
+                    const int64_t wid = accum_row(P, g);
                     if (a != 0.0f) atomicAdd(P.accum_weight + wid, a);
                     if (kAccum == SSR_ACCUM_AVG && b != 0.0f) atomicAdd(P.accum_weight + P.num_world + wid, b);
                 }
@@ -209,7 +216,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
         add(P.v_screen.opac + g, v[6]);
         add(P.v_screen.rgb + 3u * g, v[7]); add(P.v_screen.rgb + 3u * g + 1u, v[8]); add(P.v_screen.rgb + 3u * g + 2u, v[9]);
         if constexpr (kAccCh == 12) {
-            const int64_t wid = P.gaussian_ids ? (int64_t)P.gaussian_ids[g] : (int64_t)g;
+            const int64_t wid = accum_row(P, g);
             add(P.accum_weight + wid, v[10]);
             if constexpr (kAccum == SSR_ACCUM_AVG) add(P.accum_weight + P.num_world + wid, v[11]);
         }
@@ -306,7 +313,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
                 if constexpr (kMedian) t_d += v_depth_median;
                 [[maybe_unused]] int64_t wid = 0;
                 if constexpr (kAccum != SSR_ACCUM_NONE) {   // :553-562,574-585
-                    wid = P.gaussian_ids ? (int64_t)P.gaussian_ids[s_ids[k]] : (int64_t)s_ids[k];
+                    wid = accum_row(P, (uint32_t)s_ids[k]);
                     if constexpr (kAccum == SSR_ACCUM_MAX) {
                         const float mx = wave_max_f32(amap * w);   // inactive lanes contribute map * 0; the running max starts at 0
                         if (lane == 0) atomic_max_f32(P.accum_weight + wid, ssr_max(mx, 0.0f));
@@ -372,7 +379,8 @@ extern "C" int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t strea
     SSR_REQUIRE(p->num_images >= 0, "ssr_raster_bwd", "negative num_images");
     const int nimg = p->num_images > 1 ? p->num_images : 1;
     SSR_REQUIRE((int64_t)tw * th * nimg < (int64_t)1 << 30, "ssr_raster_bwd", "too many tiles");
-    SSR_REQUIRE(nimg == 1 || p->accum_mode == SSR_ACCUM_NONE, "ssr_raster_bwd", "weight accumulation takes one image per call");
+    SSR_REQUIRE(nimg == 1 || p->accum_mode == SSR_ACCUM_NONE || (p->num_world < ((int64_t)1 << 31) && p->num_splats == nimg * p->num_world),
+                "ssr_raster_bwd", "several images accumulate per world row: num_splats must be num_images * num_world");
     const dim3 grid((unsigned)xcd_grid_size(tw * th * nimg)), block(kRasterBlock);
     hipStream_t st = as_stream(stream);
     const bool med = p->v_render_median != nullptr;

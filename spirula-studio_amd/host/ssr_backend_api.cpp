@@ -586,8 +586,8 @@ rasterize_to_pixels_3dgs_bwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     ssr_raster_bwd_params p;
     std::memset(&p, 0, sizeof(p));
     const int64_t I = tile_offsets.size<0>();
-    if (I > 1 && (gaussian_ids.data_ptr() || accum_mode != DensifyAccumMode::None))
-        throw std::runtime_error("rasterize_to_pixels_3dgs_bwd: packed rows and weight accumulation take one image per call");
+    if (I > 1 && gaussian_ids.data_ptr())
+        throw std::runtime_error("rasterize_to_pixels_3dgs_bwd: packed rows take one image per call");
     p.num_splats = I > 1 && !splats_s.empty() ? splats_s[0].rows() : num_splats;   // [C,N] rows
     p.num_images = (int32_t)I;
     p.screen = screen_of(splats_s);

@@ -661,3 +661,59 @@ def test_two_cameras_are_refused_where_one_is_required(pkg, H):
     hyper = dict.fromkeys(host.Engine.HYPER, 0.0)
     with pytest.raises(lib.SsrError, match="one camera per call"):
         eng.backward_fused_optimizer(hyper, 1)
+
+
+@pytest.mark.parametrize("accum_mode", [1, 3])
+def test_engine_two_cameras_variants(pkg, oracle, H, accum_mode):
+    """Two cameras with the distortion images, median depth and accumulation weights: per-pixel outputs are
+    each camera's own, the weights of both cameras land in the splat's one world row
+    (RasterizationEval3DBwd_kernel.cuh:368: row % N) -- summed for SUM/AVG, the larger for MAX."""
+    import copy
+    host, lib = H
+    S = pkg.scenes
+    base = S.tiny_scene(n=2500, width=200, height=150, seed=77)
+    h, w, n = base.height, base.width, base.n
+    rng = np.random.default_rng(9)
+    vms, its = [], []
+    for k, ang in enumerate([0.15, -0.3]):
+        c, s_ = np.cos(ang), np.sin(ang)
+        vms.append(np.array([[c, 0, s_, 0.2 - 0.5 * k], [0, 1, 0, 0.1 * k], [-s_, 0, c, 3.0 + 0.3 * k], [0, 0, 0, 1]], np.float32))
+        its.append(np.array([140.0 + 15 * k, 145.0, 100.0, 75.0 - 4 * k], np.float32))
+    cot = dict(v_rgb=rng.standard_normal((2, h, w, 3)), v_depth=rng.standard_normal((2, h, w)), v_T=rng.standard_normal((2, h, w)),
+               v_dist_rgb=rng.uniform(-1, 1, (2, h, w, 3)), v_dist_depth=rng.uniform(-1, 1, (2, h, w)),
+               accum_map=rng.uniform(0, 1, (2, h, w)))
+    cot = {k: v.astype(np.float32) for k, v in cot.items()}
+    refs, meds = [], []
+    for k in range(2):
+        sc = copy.deepcopy(base)
+        sc.viewmat, sc.intrins = vms[k], its[k]
+        sc.v_rgb, sc.v_depth, sc.v_T = cot["v_rgb"][k], cot["v_depth"][k], cot["v_T"][k]
+        va = dict(dist_type=2, median=False, accum_mode=accum_mode, v_dist_rgb=cot["v_dist_rgb"][k],
+                  v_dist_depth=cot["v_dist_depth"][k], accum_map=cot["accum_map"][k])
+        refs.append(oracle.pipeline(sc, variant=va))
+        meds.append(oracle.pipeline(sc, backward=False, variant=dict(median=True))["fwd"]["median"])
+        assert refs[-1]["proj"]["visible"] > 100
+    both = copy.deepcopy(base)
+    both.viewmat, both.intrins = np.stack(vms), np.stack(its)
+    both.v_rgb, both.v_depth, both.v_T = cot["v_rgb"], cot["v_depth"], cot["v_T"]
+    eng = host.Engine(both)
+    eng.set_variants(dist_type=2, median=True)
+    eng.forward()
+    eng.backward_with_variants(cot["v_dist_rgb"], cot["v_dist_depth"], None, cot["accum_map"], accum_mode=accum_mode)
+    dist_rgb, dist_depth = eng.cache("dist_rgb").reshape(2, h, w, 3), eng.cache("dist_depth").reshape(2, h, w)
+    median = eng.cache("median").reshape(2, h, w)
+    for k in range(2):
+        assert np.abs(dist_rgb[k] - refs[k]["fwd"]["dist_rgb"]).max() <= 1e-4
+        assert np.abs(dist_depth[k] - refs[k]["fwd"]["dist_depth"]).max() <= 1e-4
+        assert (np.abs(median[k] - meds[k]) <= 1e-4 * np.maximum(1, np.abs(meds[k]))).all()
+    aw = eng.cache("accum_weight")
+    a0, a1 = (r["vscreen"]["accum_weight"] for r in refs)
+    want = np.maximum(a0, a1) if accum_mode == 1 else a0 + a1
+    assert aw.size == want.size == (2 * n if accum_mode == 3 else n)
+    assert (a0[:n] > 0).sum() > 100 and (a1[:n] > 0).sum() > 100 and ((a0[:n] > 0) != (a1[:n] > 0)).sum() > 10
+    assert np.allclose(aw, want, rtol=1e-3, atol=1e-6)
+    g = eng.grads()
+    for key, v in g.items():
+        r = sum(ref["grads"][key].astype(np.float64) for ref in refs).reshape(n, -1)
+        scale = sum(np.abs(ref["grads"][key].astype(np.float64)).reshape(n, -1).max(axis=1, keepdims=True) for ref in refs)
+        assert (np.abs(v.reshape(n, -1) - r) <= 2e-3 * scale + 2e-5 * (np.abs(r).mean() + 1e-12)).all(), key
