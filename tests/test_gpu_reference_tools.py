@@ -373,3 +373,49 @@ def test_fpbo_parity_mip_row(gpu, oracle, cam):
             assert far.mean() < 2e-3, (k, call, float(far.mean()))
         # the coefficients above degree 2 are left alone
         assert np.array_equal(dP["features_sh"][:, 8:], sc.features_sh[:, 8:])
+
+
+@pytest.mark.parametrize("model,tier,dist_type,median,accum", [(PINHOLE, NONE, 0, False, 0), (PINHOLE, OPENCV, 2, True, 1),
+                                                              (FISHEYE, THIN_PRISM, 1, False, 3)])
+def test_raster_bwd_parity_rows_as_the_tool_batches_them(gpu, oracle, model, tier, dist_type, median, accum):
+    """The tool's two cameras in ONE call, as raster_bwd_parity.cpp runs them (C = 2 viewmats, [C,H,W,..]
+    cotangents, per-camera lens rows), through the host layer's reference-shaped launch functions; checked
+    against the oracle run once per camera."""
+    import dataclasses
+    from spirula_studio_amd import host
+    host.load()
+    _, rng = R.tool_world(R.SEED_RASTER_BWD)
+    ct = R.raster_bwd_cotangents(rng)
+    scs = [R.tool_scene(gpu, R.SEED_RASTER_BWD, cam, model, tier, cotangents=ct)[0] for cam in (0, 1)]
+    refs = []
+    for cam, sc in enumerate(scs):
+        va = dict(dist_type=dist_type, median=False, accum_mode=accum, v_dist_rgb=ct["v_dist_rgb"][cam],
+                  v_dist_depth=ct["v_dist_depth"][cam], accum_map=ct["accum_map"][cam])
+        refs.append(oracle.pipeline(sc, variant=va))
+        assert refs[-1]["proj"]["visible"] > 100
+    both = dataclasses.replace(scs[0], viewmat=np.stack([s.viewmat for s in scs]), intrins=np.stack([s.intrins for s in scs]),
+                               dist_coeffs=np.stack([s.dist_coeffs for s in scs]), v_rgb=ct["v_rgb"], v_depth=ct["v_depth"], v_T=ct["v_T"])
+    eng = host.Engine(both)
+    eng.set_variants(dist_type=dist_type, median=median)
+    eng.forward()
+    eng.backward_with_variants(ct["v_dist_rgb"] if dist_type == 2 else None, ct["v_dist_depth"] if dist_type else None, None,
+                               ct["accum_map"] if accum else None, accum_mode=accum)
+    n, h, w = both.n, both.height, both.width
+    tiles = ((w + 15) // 16) * ((h + 15) // 16)
+    n0 = refs[0]["sorted_ids"].size
+    assert np.array_equal(eng.cache("sorted_ids"), np.concatenate([refs[0]["sorted_ids"], refs[1]["sorted_ids"] + (np.int64(tiles) << 32)]))
+    assert np.array_equal(eng.cache("sorted_flat"), np.concatenate([refs[0]["sorted_flat"], refs[1]["sorted_flat"] + n]))
+    assert np.array_equal(eng.cache("offsets"), np.concatenate([refs[0]["offsets"].reshape(-1), refs[1]["offsets"].reshape(-1) + n0]))
+    rgb, depth, T = eng.render()
+    for cam in (0, 1):
+        assert np.abs(rgb[cam] - refs[cam]["fwd"]["rgb"]).max() <= 1e-4
+        assert np.abs(T[cam] - refs[cam]["fwd"]["T"]).max() <= 1e-4
+        if dist_type:
+            assert np.abs(eng.cache("dist_depth").reshape(2, h, w)[cam] - refs[cam]["fwd"]["dist_depth"]).max() <= 1e-4
+    if accum:
+        a0, a1 = (r["vscreen"]["accum_weight"] for r in refs)
+        assert np.allclose(eng.cache("accum_weight"), np.maximum(a0, a1) if accum == 1 else a0 + a1, rtol=1e-3, atol=1e-6)
+    for key, v in eng.grads().items():
+        r = sum(ref["grads"][key].astype(np.float64) for ref in refs).reshape(n, -1)
+        scale = sum(np.abs(ref["grads"][key].astype(np.float64)).reshape(n, -1).max(axis=1, keepdims=True) for ref in refs)
+        assert (np.abs(v.reshape(n, -1) - r) <= 2e-3 * scale + 2e-5 * (np.abs(r).mean() + 1e-12)).all(), key
