@@ -116,6 +116,8 @@ def main():
     ap.add_argument("--dist-type", type=int, default=0, help="compositing variant: 1 depth distortion, 2 rgb + depth distortion")
     ap.add_argument("--median", action="store_true", help="compositing variant: also render the median depth and back-propagate it")
     ap.add_argument("--accum-mode", type=int, default=0, help="compositing variant: accumulate a pixel weight map per splat (1 max, 2 sum, 3 avg)")
+    ap.add_argument("--cameras", type=int, default=1,
+                    help="render C cameras per iteration in one call ([C,N] layout, plain path only); an iteration is then C images")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run device copies / fills of known size (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE) and exit")
     args = ap.parse_args()
@@ -156,6 +158,21 @@ def main():
         sc = pkg.scenes.with_lens(sc, ["none", "opencv", "thin_prism", "rational"].index(args.lens))
     if args.mip:
         sc.antialiased = True
+    ncam = args.cameras
+    if ncam > 1:
+        if args.packed_projection or args.fused_optimizer or args.dist_type or args.median or args.accum_mode:
+            sys.exit("bench.py: --cameras runs the plain forward + backward only")
+        vms = []
+        for k in range(ncam):   # the same view, each camera a little further along x
+            vm = np.array(sc.viewmat, np.float32).copy()
+            vm[0, 3] += 0.05 * k
+            vms.append(vm)
+        sc.viewmat = np.stack(vms)
+        sc.intrins = np.stack([np.asarray(sc.intrins, np.float32)] * ncam)
+        if getattr(sc, "dist_coeffs", None) is not None:
+            sc.dist_coeffs = np.stack([np.asarray(sc.dist_coeffs, np.float32)] * ncam)
+        for name in ("v_rgb", "v_depth", "v_T"):
+            setattr(sc, name, np.ascontiguousarray(np.stack([np.asarray(getattr(sc, name), np.float32)] * ncam)))
     t_gen = time.time() - t_gen
     native = not args.reference_order
     eng = host.Engine(sc, fuse_tile_count=native, visible_list=native and not args.packed_projection, packed_rows=native,
@@ -221,16 +238,20 @@ def main():
     aabb = eng.cache("aabb").reshape(-1, 4)
     V = int((aabb[:, 2] > aabb[:, 0]).sum())   # packed form: every one of its nnz rows
     K = eng.n_isects
-    P = sc.width * sc.height
-    T = sc.tile_w * sc.tile_h
-    K_b = tile_need(eng.cache("offsets"), eng.cache("last_ids"), K, sc.width, sc.height)
+    P1, T1 = sc.width * sc.height, sc.tile_w * sc.tile_h
+    P, T = ncam * P1, ncam * T1    # several cameras: C images of pixels and of tiles, C*N projected rows
+    offs, last = eng.cache("offsets"), eng.cache("last_ids")
+    K_b = 0
+    for c in range(ncam):   # positions in offsets and last_ids are absolute, so each image is taken with its own end
+        end = int(offs[(c + 1) * T1]) if c + 1 < ncam else K
+        K_b += tile_need(offs[c * T1:(c + 1) * T1], last[c * P1:(c + 1) * P1], end, sc.width, sc.height)
     K_f = K_b   # lower bound of the forward's need (it also reads the splat that ends a pixel)
     S = 180 if sc.sh_codec == 0 else (47 if sc.sh_codec == 3 else 45 + 8 * 45 / 256)
     tile_bits = max(T - 1, 0).bit_length()
     tile_sort = native and not args.whole_key_sort
     sort_sweeps = (32 + tile_bits + 7) // 8
     sort_sweeps_done = (tile_bits + 7) // 8 + 1 if tile_sort else sort_sweeps
-    ab = algorithmic_bytes(sc.n, V, K, K_f, K_b, P, T, S, sort_sweeps)
+    ab = algorithmic_bytes(ncam * sc.n, V, K, K_f, K_b, P, T, S, sort_sweeps)
     total_bytes = sum(ab.values())
     dom = max(acc, key=acc.get)
     dom_gbs = ab[dom] / (acc[dom] * 1e-3) / 1e9 if acc[dom] > 0 else 0.0
@@ -239,8 +260,8 @@ def main():
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(tpath):
         try:
-            traffic = json.load(open(tpath)).get(f"config{cfg}", {}).get(dom)
-            if native and not (variants or args.fused_optimizer or args.packed_projection or args.lens != "none" or args.fisheye or args.mip):
+            traffic = json.load(open(tpath)).get(f"config{cfg}", {}).get(dom) if ncam == 1 else None
+            if native and ncam == 1 and not (variants or args.fused_optimizer or args.packed_projection or args.lens != "none" or args.fisheye or args.mip):
                 valu_inst = json.load(open(tpath)).get(f"config{cfg}_valu_wave_instructions", {}).get(dom)
         except Exception:
             traffic = None
@@ -261,6 +282,7 @@ def main():
                    "stage_order": ("fused tile count, visible-splat work list, packed fragment rows, packed gradient rows, plain-store gradients"
                                    + (", tile-segmented sort" if tile_sort else "") if native else "reference order")
                                   + (", antialiased (mip) primitive" if args.mip else "")
+                                  + (f", {ncam} cameras per iteration in one call" if ncam > 1 else "")
                                   + (", packed projection outputs" if args.packed_projection else "")
                                   + (", projection backward fused with Adam" + ((" (quantized SH state" + (" and non-SH moments)" if args.non_sh_optim_bits == 16 else ")")) if args.quantization_level else "")
                                      if args.fused_optimizer else "")
@@ -281,7 +303,7 @@ def main():
         out["roofline"]["valu_issue"] = {"wave_instructions_per_launch": valu_inst,
                                          "frac_of_issue_slots": valu_inst * 4 / 1024 / (acc[dom] * 1e-3 * 2.4e9)}
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(pkg, cfg)
+        out["cpu_baseline"] = cpu_baseline(pkg, cfg)   # one camera of the configuration
     print(json.dumps(out))
 
 

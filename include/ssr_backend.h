@@ -306,7 +306,8 @@ int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t stream);
 /* ---- K9: projection_3dgs_backward (src/kernels/projection/ProjectionBwd.cuh:18-46, kernel
  * src/kernels/projection/ProjectionBwd_kernel.cuh:16-130). accumulate != 0:
  * gradients are added into v_world (the reference's behaviour; caller zero-fills,
- * src/engine/EngineLoss.cpp:120-127). accumulate == 0: every row of v_world is overwritten
+ * src/engine/EngineLoss.cpp:120-127) with a plain read-add-write: a launch holds one camera, so one
+ * thread owns a row, and launches that share v_world must be ordered on a stream. accumulate == 0: every row of v_world is overwritten
  * (zeros for culled splats), which gives the same values with C = 1 and needs no zero-fill. */
 typedef struct {
     int64_t num_splats;

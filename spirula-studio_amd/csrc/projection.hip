@@ -323,9 +323,11 @@ __global__ __launch_bounds__(kProjBlock) void projection_packed_emit_kernel(ssr_
 
 __device__ __forceinline__ float fin(float v) { return ssr_isfinite(v) ? v : 0.0f; }
 
+// A launch handles one camera, so exactly one thread owns a world row: adding into it needs no atomic
+// (the reference's launch covers C cameras at once and adds atomically); the sum is the same float.
 template <bool kAccumulate>
 __device__ __forceinline__ void put(float* p, float v) {
-    if (kAccumulate) { if (v != 0.0f) atomicAdd(p, v); }
+    if (kAccumulate) { if (v != 0.0f) *p += v; }
     else *p = v;
 }
 
@@ -649,7 +651,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
         const bool ok = ssr_isfinite(d2) && d2 != 0.0f;   // harmonics.slang:397-403
 #pragma unroll
         for (int c = 0; c < 3; c++) {
-            if (kAccumulate) { if (ok) atomicAdd(vsh + 3 * j + c, tv[c]); }
+            if (kAccumulate) { if (ok) vsh[3 * j + c] += tv[c]; }
             else vsh[3 * j + c] = ok ? tv[c] : 0.0f;
         }
     });
