@@ -165,7 +165,7 @@ struct Options {
     // K1 also writes each visible screen row as one 48-byte record; the compositing kernels gather
     // from it when they are handed the screen buffers of that same projection.
     bool packed_rows = false;
-    // K9 stores gradients instead of atomically adding them (with several cameras the first
+    // K9 stores gradients instead of adding them into zero-filled rows (with several cameras the first
     // camera's launch stores and the others add). Without the visible list every row is overwritten (zeros for
     // culled splats) and the caller may skip its zero-fill; with the list only visible rows are
     // stored and the zero-fill is still needed.
