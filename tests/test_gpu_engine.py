@@ -661,6 +661,10 @@ def test_two_cameras_are_refused_where_one_is_required(pkg, H):
     hyper = dict.fromkeys(host.Engine.HYPER, 0.0)
     with pytest.raises(lib.SsrError, match="one camera per call"):
         eng.backward_fused_optimizer(hyper, 1)
+    # the C ABI's own check: rows must split evenly over the images
+    L = lib.load()
+    with pytest.raises(lib.SsrError, match="rows_per_image"):
+        lib.check(L.ssr_tile_write_images(10, 3, None, None, None, None, None, None, 64, 48, None, None, None))
 
 
 @pytest.mark.parametrize("accum_mode", [1, 3])
