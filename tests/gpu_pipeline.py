@@ -8,6 +8,29 @@ import ctypes as C
 import numpy as np
 
 
+WORLD_GRAD_RTOL = 1e-3   # the bar for parameter gradients: 1e-3 of the row's largest entry
+MARGINS = {}             # label -> largest err / rowmax seen, for the report at the end of a run
+
+
+def world_grad_check(got, ref, n, name, rtol=WORLD_GRAD_RTOL, bad_frac=0.0, scale=None):
+    """Parameter-gradient bar: |got - ref| <= rtol * max|ref row| + a floor of 2e-5 of the tensor's
+    mean magnitude (rows whose terms cancel). Prints the largest observed error relative to the row
+    maximum, with and without the floor, so that the margin is on record."""
+    got = np.asarray(got, np.float64).reshape(n, -1)
+    ref = np.asarray(ref, np.float64).reshape(n, -1)
+    if scale is None:   # a caller that sums several cameras passes the sum of their row maxima
+        scale = np.abs(ref).max(axis=1, keepdims=True)
+    scale = scale + 1e-30
+    floor = 2e-5 * (np.abs(ref).mean() + 1e-12)
+    err = np.abs(got - ref)
+    raw = float((err / scale).max()) if err.size else 0.0
+    over = float((np.maximum(err - floor, 0.0) / scale).max()) if err.size else 0.0
+    MARGINS[name] = max(MARGINS.get(name, 0.0), over)
+    print(f"  grad {name}: max err/rowmax {raw:.3e}, beyond the floor {over:.3e} (bar {rtol:.0e})", flush=True)
+    bad = err > rtol * scale + floor
+    assert bad.mean() <= bad_frac, (name, over, float(bad.mean()))
+
+
 class GpuRun:
     def __init__(self, pkg, scene, sh_degree=3, use_list=False, use_packed=False, packed_projection=False,
                  read_nnz=True, use_vrows=False, tile_sort=False):

@@ -5,6 +5,8 @@ import dataclasses
 import numpy as np
 import pytest
 
+from gpu_pipeline import world_grad_check
+
 pytestmark = pytest.mark.gpu
 
 
@@ -27,10 +29,7 @@ def _check(eng, ref, sc):
     assert np.array_equal(eng.cache("last_ids").reshape(sc.height, sc.width), ref["fwd"]["last_ids"])
     g = eng.grads()
     for k, v in g.items():
-        r = ref["grads"][k].astype(np.float64).reshape(sc.n, -1)
-        scale = np.abs(r).max(axis=1, keepdims=True)
-        err = np.abs(v.reshape(sc.n, -1) - r)
-        assert (err <= 2e-3 * scale + 2e-5 * (np.abs(r).mean() + 1e-12)).all(), k
+        world_grad_check(v, ref["grads"][k], sc.n, f"engine/{k}")
     return g
 
 
@@ -144,7 +143,8 @@ def test_engine_camera_pose_gradient(pkg, oracle, H, packed):
     got = eng.backward_with_pose_grad().astype(np.float64)
     _check(eng, ref, sc)
     assert not np.any(got[3]) and np.abs(want[:3]).min() > 0
-    assert np.abs(got - want).max() <= 2e-3 * np.abs(want).max(), (got, want)
+    print(f"  pose gradient: max err / max {np.abs(got - want).max() / np.abs(want).max():.3e}", flush=True)
+    assert np.abs(got - want).max() <= 1e-3 * np.abs(want).max(), (got, want)
     # accumulated into, not overwritten: a second backward on a fresh buffer gives the same sums again
     again = eng.backward_with_pose_grad().astype(np.float64)
     assert np.abs(again - got).max() <= 1e-4 * np.abs(want).max()
@@ -206,10 +206,7 @@ def _check_packed(eng, ref, sc):
     assert eng.cache("v_xy").size == 2 * m
     g = eng.grads()
     for k, v in g.items():
-        r = ref["grads"][k].astype(np.float64).reshape(sc.n, -1)
-        scale = np.abs(r).max(axis=1, keepdims=True)
-        err = np.abs(v.reshape(sc.n, -1) - r)
-        assert (err <= 2e-3 * scale + 2e-5 * (np.abs(r).mean() + 1e-12)).all(), k
+        world_grad_check(v, ref["grads"][k], sc.n, f"engine/{k}")
     return g
 
 
@@ -500,10 +497,7 @@ def test_engine_compositing_variants(pkg, oracle, H, packed):
     assert np.allclose(aw, r["vscreen"]["accum_weight"], rtol=1e-3, atol=1e-6) and (aw[:sc.n] > 0).sum() > 100
     g = eng.grads()
     for k, v in g.items():
-        ref = r["grads"][k].astype(np.float64).reshape(sc.n, -1)
-        scale = np.abs(ref).max(axis=1, keepdims=True)
-        err = np.abs(v.reshape(sc.n, -1) - ref)
-        assert (err <= 2e-3 * scale + 2e-5 * (np.abs(ref).mean() + 1e-12)).all(), k
+        world_grad_check(v, r["grads"][k], sc.n, f"engine-variants/{k}")
     # a forward with distortion needs its cotangent in the backward
     assert eng.h.ssrh_backward_from_render_grad(eng.d_vrgb.ptr, eng.d_vdepth.ptr, eng.d_vT.ptr) != 0
     assert b"distortion" in eng.h.ssrh_last_error()
@@ -634,13 +628,13 @@ def test_engine_two_cameras(pkg, oracle, H, native):
             # fragment reached keeps 0 and T = 1
             reached = refs[k]["fwd"]["T"] < 1.0
             assert np.array_equal(last[k], np.where(reached, refs[k]["fwd"]["last_ids"] + (n0 if k else 0), 0))
-            assert np.abs(got_pose[k] - poses[k]).max() <= 2e-3 * np.abs(poses[k]).max(), (k, got_pose[k], poses[k])
+            print(f"  pose gradient {k}: max err / max {np.abs(got_pose[k] - poses[k]).max() / np.abs(poses[k]).max():.3e}", flush=True)
+            assert np.abs(got_pose[k] - poses[k]).max() <= 1e-3 * np.abs(poses[k]).max(), (k, got_pose[k], poses[k])
         g = eng.grads()
         for key, v in g.items():
             r = sum(ref["grads"][key].astype(np.float64) for ref in refs).reshape(n, -1)
             scale = sum(np.abs(ref["grads"][key].astype(np.float64)).reshape(n, -1).max(axis=1, keepdims=True) for ref in refs)
-            err = np.abs(v.reshape(n, -1) - r)
-            assert (err <= 2e-3 * scale + 2e-5 * (np.abs(r).mean() + 1e-12)).all(), key
+            world_grad_check(v, r, n, f"two-cameras/{key}", scale=scale)
 
 
 def test_two_cameras_are_refused_where_one_is_required(pkg, H):
@@ -720,4 +714,4 @@ def test_engine_two_cameras_variants(pkg, oracle, H, accum_mode):
     for key, v in g.items():
         r = sum(ref["grads"][key].astype(np.float64) for ref in refs).reshape(n, -1)
         scale = sum(np.abs(ref["grads"][key].astype(np.float64)).reshape(n, -1).max(axis=1, keepdims=True) for ref in refs)
-        assert (np.abs(v.reshape(n, -1) - r) <= 2e-3 * scale + 2e-5 * (np.abs(r).mean() + 1e-12)).all(), key
+        world_grad_check(v, r, n, f"two-cameras-variants/{key}", scale=scale)

@@ -6,6 +6,7 @@ import numpy as np
 import pytest
 
 import ref64
+from gpu_pipeline import world_grad_check
 
 pytestmark = pytest.mark.gpu
 
@@ -122,10 +123,7 @@ def test_full_size_properties(pkg, oracle, H, cfg):
     g3 = ref.grads()
 
     def close(a, b, what):
-        a, b = a.reshape(n, -1).astype(np.float64), b.reshape(n, -1).astype(np.float64)
-        scale = np.abs(b).max(axis=1, keepdims=True)
-        bad = np.abs(a - b) > 2e-3 * scale + 2e-5 * (np.abs(b).mean() + 1e-12)
-        assert bad.mean() < 1e-5, (what, float(bad.mean()))
+        world_grad_check(a, b, n, f"config{cfg}/{what[0]}/{what[1]}")
 
     for k in g1:
         close(g1b[k], g1[k], ("idempotent", k))

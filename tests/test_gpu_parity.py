@@ -8,7 +8,7 @@ import math
 import numpy as np
 import pytest
 
-from gpu_pipeline import GpuRun
+from gpu_pipeline import GpuRun, world_grad_check
 
 pytestmark = pytest.mark.gpu
 
@@ -107,13 +107,8 @@ def _compare(gpu, oracle, sc, label, fused_count=False, use_list=False, use_pack
     gr = r["grads"]
     for k, o in [("w_means", "v_means"), ("w_quats", "v_quats"), ("w_log_scales", "v_scales"),
                  ("w_opacity_logits", "v_opacities"), ("w_features_dc", "v_dc"), ("w_features_sh", "v_sh")]:
-        got, ref = g.host(k).astype(np.float64), gr[o].astype(np.float64)
-        rows = ref.reshape(sc.n, -1)
-        scale = np.abs(rows).max(axis=1, keepdims=True) + 1e-30
-        err = np.abs(got.reshape(sc.n, -1) - rows)
-        # per-row relative bar, with a floor for rows whose inputs cancel
-        floor = 2e-5 * (np.abs(rows).mean() + 1e-12)
-        assert (err <= 2 * GRAD_RTOL * scale + floor).all(), (k, float((err / scale).max()))
+        got = g.host(k)
+        world_grad_check(got, gr[o], sc.n, f"{label}/{k}")
         assert not np.any(got[~vis]), k
     return g, r
 
@@ -171,12 +166,8 @@ def _compare_packed(gpu, oracle, sc, label, fused_count=False, use_packed=False,
     vis[q["gaussian_ids"]] = True
     for k, o in [("w_means", "v_means"), ("w_quats", "v_quats"), ("w_log_scales", "v_scales"),
                  ("w_opacity_logits", "v_opacities"), ("w_features_dc", "v_dc"), ("w_features_sh", "v_sh")]:
-        got, ref = g.host(k).astype(np.float64), gr[o].astype(np.float64)
-        rows = ref.reshape(sc.n, -1)
-        scale = np.abs(rows).max(axis=1, keepdims=True) + 1e-30
-        err = np.abs(got.reshape(sc.n, -1) - rows)
-        floor = 2e-5 * (np.abs(rows).mean() + 1e-12)
-        assert (err <= 2 * GRAD_RTOL * scale + floor).all(), (k, float((err / scale).max()))
+        got = g.host(k)
+        world_grad_check(got, gr[o], sc.n, f"{label}/{k}")
         assert not np.any(got[~vis]), k
     return g, r
 

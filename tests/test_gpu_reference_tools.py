@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import reference_tools as R
-from gpu_pipeline import GpuRun
+from gpu_pipeline import GpuRun, world_grad_check
 from test_gpu_parity import _compare, _compare_packed, gpu  # noqa: F401  (gpu: module fixture)
 
 pytestmark = pytest.mark.gpu
@@ -207,9 +207,7 @@ def _k9_direct(gpu, oracle, sc, vs, label, packed=False, pose=False, sh_degree=3
     for k, o in [("w_means", "v_means"), ("w_quats", "v_quats"), ("w_log_scales", "v_scales"),
                  ("w_opacity_logits", "v_opacities"), ("w_features_dc", "v_dc"), ("w_features_sh", "v_sh")]:
         got, ref = g.host(k).astype(np.float64).reshape(sc.n, -1), want[o].astype(np.float64).reshape(sc.n, -1)
-        scale = np.abs(ref).max(axis=1, keepdims=True) + 1e-30
-        floor = 2e-5 * (np.abs(ref).mean() + 1e-12)
-        assert (np.abs(got - ref) <= 2e-3 * scale + floor).all(), (k, float((np.abs(got - ref) / scale).max()))
+        world_grad_check(got, ref, sc.n, f"{label}/{k}")
         assert not np.any(got[~vis]), k
         # and inside the tool's own acceptance band (proj_bwd_parity.cpp:327)
         assert (np.abs(got - ref) <= 5e-3 + 1e-3 * np.abs(ref)).all(), k
