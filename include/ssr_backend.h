@@ -182,6 +182,14 @@ size_t ssr_scan_scratch_bytes(int64_t n);
  * read back in one copy. */
 int ssr_inclusive_sum_i64(const int64_t* in, int64_t* out, int64_t n, int64_t* total_out,
                           void* scratch, size_t scratch_bytes, ssr_stream_t stream);
+/* The same scan for callers that cannot allocate device memory or pass a workspace (code under
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in the
+ * reference. The block sums live in a 512 KiB array inside the library (one copy per GPU, held until
+ * the process ends), so n is limited to 2^27 = 134 217 728 elements; a larger n is rejected with an
+ * error. Same kernels and same results as ssr_inclusive_sum_i64. Calls on one GPU share that
+ * array: calls that overlap in time on one GPU (different streams, different threads) race. */
+int ssr_inclusive_sum_i64_static(const int64_t* in, int64_t* out, int64_t n, int64_t* total_out,
+                                 ssr_stream_t stream);
 /* The reference's blocking readback of n_isects (8 bytes, IntersectTile.cu:432-436); `count`
  * consecutive values are copied. */
 int ssr_read_i64(const int64_t* device_values, int64_t* host_values, int count, ssr_stream_t stream);

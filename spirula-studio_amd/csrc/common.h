@@ -24,6 +24,10 @@ inline hipStream_t as_stream(ssr_stream_t s) { return reinterpret_cast<hipStream
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Resolves the current device's address of the scan workspace that ssr_inclusive_sum_i64_static
+// uses (tiles.hip); ssr_init calls it so that the first scan does not pay for it.
+int warm_static_scan();
+
 }  // namespace ssr
 
 #define SSR_CHECK_LAUNCH(where)                                       \

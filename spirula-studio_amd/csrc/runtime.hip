@@ -85,7 +85,9 @@ int ssr_init(int device) {
     e = check_hip(hipGetDeviceProperties(&prop, device), "ssr_init/hipGetDeviceProperties");
     if (e) return e;
     g_device_name = std::string(prop.name) + " (" + prop.gcnArchName + ")";
-    return check_hip(hipFree(nullptr), "ssr_init/context");
+    e = check_hip(hipFree(nullptr), "ssr_init/context");
+    if (e) return e;
+    return warm_static_scan();
 }
 
 const char* ssr_device_name(void) { return g_device_name.c_str(); }

@@ -4,6 +4,7 @@
 // K6 follows intersect_offset_kernel (:271-307). Keys are (tile_id << 32) | depth bits with
 // depth bits = bits(|sorting depth|) ^ 0x80000000 (:190-196); values are flat splat indices.
 #include "projection_device.h"
+#include <mutex>
 
 namespace ssr {
 
@@ -236,6 +237,42 @@ __global__ __launch_bounds__(kScanBlock) void scan_down_kernel(const int64_t* __
     }
 }
 
+// ---- scan workspace held by the library itself (ssr_inclusive_sum_i64_static) ----
+
+// Block sums of the largest scan the allocation-free entry point accepts: 65 536 blocks of 2048
+// elements = 2^27 elements, 512 KiB. Every GPU the library runs on holds its own copy of this array
+// at its own address for the life of the process. The name below is only the host-side handle of
+// the symbol; host code uses the address hipGetSymbolAddress returns for the current device.
+constexpr int64_t kStaticScanBlocks = 65536;
+static __device__ __align__(256) int64_t scan_static_scratch[kStaticScanBlocks];
+
+constexpr int kMaxDevices = 64;
+static int64_t* g_static_scan_ptr[kMaxDevices];   // per device, null until resolved
+static std::mutex g_static_scan_mutex;
+
+// Resolves (once per device, with that device current) the device address of the array above.
+static int static_scan_pointer(int64_t** out) {
+    int dev = -1;
+    int e = check_hip(hipGetDevice(&dev), "ssr_inclusive_sum_i64_static/hipGetDevice");
+    if (e) return e;
+    if (dev < 0 || dev >= kMaxDevices) return fail("ssr_inclusive_sum_i64_static", "device index out of range");
+    std::lock_guard<std::mutex> lock(g_static_scan_mutex);
+    if (!g_static_scan_ptr[dev]) {
+        void* p = nullptr;
+        e = check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scan_static_scratch)), "ssr_inclusive_sum_i64_static/hipGetSymbolAddress");
+        if (e) return e;
+        if (!p) return fail("ssr_inclusive_sum_i64_static", "the scan workspace has no device address");
+        g_static_scan_ptr[dev] = static_cast<int64_t*>(p);
+    }
+    *out = g_static_scan_ptr[dev];
+    return 0;
+}
+
+int warm_static_scan() {
+    int64_t* p = nullptr;
+    return static_scan_pointer(&p);
+}
+
 // ---- K6 ----
 
 __global__ __launch_bounds__(kTileBlock) void tile_offsets_kernel(int64_t n_isects, const int64_t* __restrict__ ids,
@@ -307,6 +344,25 @@ int ssr_inclusive_sum_i64(const int64_t* in, int64_t* out, int64_t n, int64_t* t
     hipLaunchKernelGGL(scan_spine_kernel, dim3(1), dim3(kScanBlock), 0, s, sums, nb);
     hipLaunchKernelGGL(scan_down_kernel, dim3((unsigned)nb), dim3(kScanBlock), 0, s, in, n, sums, out, total_out);
     SSR_CHECK_LAUNCH("ssr_inclusive_sum_i64");
+    return 0;
+}
+
+int ssr_inclusive_sum_i64_static(const int64_t* in, int64_t* out, int64_t n, int64_t* total_out, ssr_stream_t stream) {
+    SSR_REQUIRE(n >= 0, "ssr_inclusive_sum_i64_static", "negative count");
+    SSR_REQUIRE(n <= kStaticScanBlocks * (int64_t)kScanTile, "ssr_inclusive_sum_i64_static",
+                "count exceeds the built-in workspace (2^27 elements); use ssr_inclusive_sum_i64 with caller scratch");
+    if (n == 0) return 0;
+    SSR_REQUIRE(in && out, "ssr_inclusive_sum_i64_static", "null pointer");
+    int64_t* sums = nullptr;
+    const int e = static_scan_pointer(&sums);
+    if (e) return e;
+    // Nothing to clear: the first kernel writes every block sum the other two read.
+    const int64_t nb = ceil_div(n, kScanTile);
+    hipStream_t s = as_stream(stream);
+    hipLaunchKernelGGL(scan_reduce_kernel, dim3((unsigned)nb), dim3(kScanBlock), 0, s, in, n, sums);
+    hipLaunchKernelGGL(scan_spine_kernel, dim3(1), dim3(kScanBlock), 0, s, sums, nb);
+    hipLaunchKernelGGL(scan_down_kernel, dim3((unsigned)nb), dim3(kScanBlock), 0, s, in, n, sums, out, total_out);
+    SSR_CHECK_LAUNCH("ssr_inclusive_sum_i64_static");
     return 0;
 }
 

@@ -115,6 +115,7 @@ SYMBOLS = {
     "ssr_compute_tile_active": (_i32, [vp, _i32, _i32, _u32, _u32, vp, vp]),
     "ssr_scan_scratch_bytes": (_sz, [_i64]),
     "ssr_inclusive_sum_i64": (_i32, [vp, vp, _i64, vp, vp, _sz, vp]),
+    "ssr_inclusive_sum_i64_static": (_i32, [vp, vp, _i64, vp, vp]),
     "ssr_read_i64": (_i32, [vp, C.POINTER(C.c_int64), _i32, vp]),
     "ssr_tile_write": (_i32, [_i64, vp, vp, vp, vp, vp, vp, _u32, _u32, vp, vp, vp, _i64, vp, vp]),
     "ssr_tile_write_images": (_i32, [_i64, _i64, vp, vp, vp, vp, vp, vp, _u32, _u32, vp, vp, vp]),
