@@ -314,8 +314,9 @@ int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t stream);
 /* ---- K9: projection_3dgs_backward (src/kernels/projection/ProjectionBwd.cuh:18-46, kernel
  * src/kernels/projection/ProjectionBwd_kernel.cuh:16-130). accumulate != 0:
  * gradients are added into v_world (the reference's behaviour; caller zero-fills,
- * src/engine/EngineLoss.cpp:120-127) with a plain read-add-write: a launch holds one camera, so one
- * thread owns a row, and launches that share v_world must be ordered on a stream. accumulate == 0: every row of v_world is overwritten
+ * src/engine/EngineLoss.cpp:120-127). Over [N] rows or a visible list the add is a plain
+ * read-add-write: a launch holds one camera, so one thread owns a row. Launches that share v_world
+ * must be ordered on one stream (two launches on different streams race). accumulate == 0: every row of v_world is overwritten
  * (zeros for culled splats), which gives the same values with C = 1 and needs no zero-fill. */
 typedef struct {
     int64_t num_splats;
@@ -348,6 +349,11 @@ typedef struct {
      * `antialiased` argument of the same projection function): screen-space blur 0.1 instead of 0.3 and the opacity
      * multiplied by sqrt(det cov2d / det (cov2d + blur)); everything after the projection is unchanged. */
     int32_t antialiased;
+    /* Packed mode with accumulate != 0: non-zero declares that packed_gaussian_ids names no splat twice
+     * (the rows of ONE camera), which lets the launch add with a plain read-add-write. Zero (the
+     * default) adds atomically, as the reference does, so that lists holding several cameras' rows
+     * stay correct. Store mode (accumulate == 0) always needs unique ids. */
+    int32_t packed_ids_unique;
 } ssr_projection_bwd_params;
 int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream_t stream);
 
@@ -459,7 +465,8 @@ int ssr_event_destroy(ssr_event_t ev);
 const char* ssr_last_error(void);               /* returns and clears; "" when none */
 
 /* Diagnostics: include/ssr_math.h evaluated on the device (op: 0 exp, 1 log, 2 atan2(a,b),
- * 3 sigmoid), to check that host and device produce identical bits. */
+ * 3 sigmoid, 4 / 5 Adam's inverse bias correction for beta1 / beta2 at step a), to check that host
+ * and device produce identical bits. */
 int ssr_debug_math(int op, int64_t n, const float* a, const float* b, float* out,
                    ssr_stream_t stream);
 

@@ -175,6 +175,21 @@ SSR_HD float ssr_atan2(float y, float x) {
 
 SSR_HD float ssr_sigmoid(float x) { return 1.0f / (1.0f + ssr_exp(-x)); }
 
+// Adam's inverse bias corrections 1 / (1 - beta^t) for beta1 = 0.9f and beta2 = 0.999f, evaluated as the
+// reference does in float (src/kernels/optim/FusedProjectionBwdOptim_kernel.cuh:369-370:
+// 1.0f / (1.0f - powf(beta, step)), beta being the FLOAT constant: 0.999f is 0.99900001287..., and
+// ln 0.999f differs from ln 0.999 by 1.3e-5 relative, which would scale every step at small t).
+// beta^t = exp(t ln beta) with ln beta split into two floats, so that the product keeps its low bits:
+// within about 1.5 ulp of the power, the accuracy class of a device powf.
+SSR_HD float ssr_pow_split(float t, float ln_hi, float ln_lo) {
+    const float x = t * ln_hi;
+    const float rest = ssr_fma(t, ln_hi, -x) + t * ln_lo;   // t ln beta - x
+    const float e = ssr_exp(x);
+    return ssr_fma(e, rest, e);                              // e^x (1 + rest)
+}
+SSR_HD float ssr_adam_inv_bias1(float t) { return 1.0f / (1.0f - ssr_pow_split(t, -0.10536054521799088f, 3.0692108854424305e-09f)); }
+SSR_HD float ssr_adam_inv_bias2(float t) { return 1.0f / (1.0f - ssr_pow_split(t, -0.0010004874784499407f, 3.235708576077023e-11f)); }
+
 // float -> int32 / uint32 conversions with saturating, NaN -> 0 semantics. The reference casts
 // floor()/ceil() results that can be NaN or negative (src/kernels/tile/IntersectTile.cu:72-75,
 // 208-213); CUDA's conversion saturates while the C cast is undefined there, so the behaviour is

@@ -515,6 +515,8 @@ void or_math(int op, int64_t n, const float* a, const float* b, float* out) {
             case 0: out[i] = ssr_exp(a[i]); break;
             case 1: out[i] = ssr_log(a[i]); break;
             case 2: out[i] = ssr_atan2(a[i], b[i]); break;
+            case 4: out[i] = ssr_adam_inv_bias1(a[i]); break;
+            case 5: out[i] = ssr_adam_inv_bias2(a[i]); break;
             default: out[i] = ssr_sigmoid(a[i]); break;
         }
     }
@@ -607,11 +609,11 @@ static void fused_optimizer_impl(int64_t N, int sh_degree,
         float b1c, b2c;
         if (steps) {
             const float t = (float)steps[g];
-            b1c = 1.0f / (1.0f - ssr_exp(t * -0.105360515657826301f));
-            b2c = 1.0f / (1.0f - ssr_exp(t * -0.00100050033358353350f));
+            b1c = ssr_adam_inv_bias1(t);   // FusedProjectionBwdOptim_kernel.cuh:369-370, float constants
+            b2c = ssr_adam_inv_bias2(t);
         } else {
-            b1c = (float)(1.0 / (1.0 - pow(0.9, (double)step)));
-            b2c = (float)(1.0 / (1.0 - pow(0.999, (double)step)));
+            b1c = ssr_adam_inv_bias1((float)step);
+            b2c = ssr_adam_inv_bias2((float)step);
         }
         auto adam = [&](float x, float v, float lr, float* g1p, float* g2p) {
             const float a = kBeta1 * *g1p + (1.f - kBeta1) * v;
@@ -767,11 +769,11 @@ static void fused_optimizer_impl(int64_t N, int sh_degree,
             float b1c, b2c;
             if (steps) {
                 const float t = (float)steps[g];
-                b1c = 1.0f / (1.0f - ssr_exp(t * -0.105360515657826301f));
-                b2c = 1.0f / (1.0f - ssr_exp(t * -0.00100050033358353350f));
+                b1c = ssr_adam_inv_bias1(t);
+                b2c = ssr_adam_inv_bias2(t);
             } else {
-                b1c = (float)(1.0 / (1.0 - pow(0.9, (double)step)));
-                b2c = (float)(1.0 / (1.0 - pow(0.999, (double)step)));
+                b1c = ssr_adam_inv_bias1((float)step);
+                b2c = ssr_adam_inv_bias2((float)step);
             }
             for (int i = 0; i < 3 * n_coef; i++) {
                 const int64_t cell = R * g + i;

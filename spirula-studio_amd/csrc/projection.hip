@@ -323,12 +323,15 @@ __global__ __launch_bounds__(kProjBlock) void projection_packed_emit_kernel(ssr_
 
 __device__ __forceinline__ float fin(float v) { return ssr_isfinite(v) ? v : 0.0f; }
 
-// A launch handles one camera, so exactly one thread owns a world row: adding into it needs no atomic
-// (the reference's launch covers C cameras at once and adds atomically); the sum is the same float.
-template <bool kAccumulate>
+// How K9 leaves a value in the world gradients. kPutStore overwrites; kPutAdd is a plain
+// read-add-write, valid when exactly one thread of the launch owns the row (one camera and, in packed
+// mode, no splat id listed twice) -- the sum is the same float an atomic would give; kPutAtomic is the
+// reference's atomic add (its launch covers C cameras at once), used when rows may repeat.
+enum { kPutStore = 0, kPutAdd = 1, kPutAtomic = 2 };
+template <int kMode>
 __device__ __forceinline__ void put(float* p, float v) {
-    if (kAccumulate) { if (v != 0.0f) *p += v; }
-    else *p = v;
+    if (kMode == kPutStore) *p = v;
+    else if (v != 0.0f) { if (kMode == kPutAtomic) atomicAdd(p, v); else *p += v; }
 }
 
 // Gradient of one splat's screen row with respect to its world row (everything K9 computes before
@@ -545,41 +548,30 @@ __device__ __forceinline__ void projection_vjp(const CamD& cam, const ssr_world&
         for (int j = 0; j < kCoef; j++) {
             sh_sink(j, b.Y[j], vc);
         }
-        auto cd = [&](int j) { return (coef[3 * j] * vc[0] + coef[3 * j + 1] * vc[1]) + coef[3 * j + 2] * vc[2]; };
+        // gY(j) = dL/dY_j. With Y(l, +-m) = A(z) {Re, Im} w^m, w = x + i y, and d w^m = m w^(m-1) dw:
+        //   dL/dx += m A (g_c Re w^(m-1) + g_s Im w^(m-1)),  dL/dy += m A (g_s Re w^(m-1) - g_c Im w^(m-1)),
+        //   dL/dz += A'(z) (g_c Re w^m + g_s Im w^m);        zonal terms B(z) add B'(z) g to dL/dz only.
+        auto gY = [&](int j) { return (coef[3 * j] * vc[0] + coef[3 * j + 1] * vc[1]) + coef[3 * j + 2] * vc[2]; };
         const float X = b.x, Y = b.y, Z = b.z;
-        float vx = -0.48860251190292f * cd(2), vy = -0.48860251190292f * cd(0), vz = 0.48860251190292f * cd(1);
+        float vx = 0.0f, vy = 0.0f, vz = 0.0f;
+        auto order = [&](int m, float A, float dA, float gc, float gs) {
+            const float mA = (float)m * A;
+            vx += mA * (gc * b.re[m - 1] + gs * b.im[m - 1]);
+            vy += mA * (gs * b.re[m - 1] - gc * b.im[m - 1]);
+            vz += dA * (gc * b.re[m] + gs * b.im[m]);
+        };
+        order(1, -shk::k1, 0.0f, gY(2), gY(0));
+        vz += shk::k1 * gY(1);
         if (kDegree >= 2) {
-            const float z2 = Z * Z;
-            const float fTmp0B = -1.092548430592079f * Z;
-            const float fC1 = X * X - Y * Y, fS1 = 2.f * X * Y;
-            const float fC1_x = 2.f * X, fC1_y = -2.f * Y, fS1_x = 2.f * Y, fS1_y = 2.f * X;
-            const float pSH6_z = 2.f * 0.9461746957575601f * Z;
-            const float pSH7_x = fTmp0B, pSH7_z = -1.092548430592079f * X;
-            const float pSH5_y = fTmp0B, pSH5_z = -1.092548430592079f * Y;
-            const float pSH8_x = 0.5462742152960395f * fC1_x, pSH8_y = 0.5462742152960395f * fC1_y;
-            const float pSH4_x = 0.5462742152960395f * fS1_x, pSH4_y = 0.5462742152960395f * fS1_y;
-            vx += pSH4_x * cd(3) + pSH8_x * cd(7) + pSH7_x * cd(6);
-            vy += pSH4_y * cd(3) + pSH8_y * cd(7) + pSH5_y * cd(4);
-            vz += pSH6_z * cd(5) + pSH7_z * cd(6) + pSH5_z * cd(4);
+            order(2, shk::k22, 0.0f, gY(7), gY(3));
+            order(1, -shk::k21 * Z, -shk::k21, gY(6), gY(4));
+            vz += (2.0f * shk::k20a * Z) * gY(5);
             if (kDegree >= 3) {
-                const float fTmp0C = -2.285228997322329f * z2 + 0.4570457994644658f;
-                const float fTmp1B = 1.445305721320277f * Z;
-                const float fTmp0C_z = -2.285228997322329f * 2.f * Z;
-                const float fTmp1B_z = 1.445305721320277f;
-                const float fC2_x = fC1 + X * fC1_x - Y * fS1_x;
-                const float fC2_y = X * fC1_y - fS1 - Y * fS1_y;
-                const float fS2_x = fS1 + X * fS1_x + Y * fC1_x;
-                const float fS2_y = X * fS1_y + fC1 + Y * fC1_y;
-                const float pSH12_z = 3.f * 1.865881662950577f * z2 - 1.119528997770346f;
-                const float pSH13_x = fTmp0C, pSH13_z = fTmp0C_z * X;
-                const float pSH11_y = fTmp0C, pSH11_z = fTmp0C_z * Y;
-                const float pSH14_x = fTmp1B * fC1_x, pSH14_y = fTmp1B * fC1_y, pSH14_z = fTmp1B_z * fC1;
-                const float pSH10_x = fTmp1B * fS1_x, pSH10_y = fTmp1B * fS1_y, pSH10_z = fTmp1B_z * fS1;
-                const float pSH15_x = -0.5900435899266435f * fC2_x, pSH15_y = -0.5900435899266435f * fC2_y;
-                const float pSH9_x = -0.5900435899266435f * fS2_x, pSH9_y = -0.5900435899266435f * fS2_y;
-                vx += pSH9_x * cd(8) + pSH15_x * cd(14) + pSH10_x * cd(9) + pSH14_x * cd(13) + pSH13_x * cd(12);
-                vy += pSH9_y * cd(8) + pSH15_y * cd(14) + pSH10_y * cd(9) + pSH14_y * cd(13) + pSH11_y * cd(10);
-                vz += pSH12_z * cd(11) + pSH13_z * cd(12) + pSH11_z * cd(10) + pSH14_z * cd(13) + pSH10_z * cd(9);
+                const float zz = Z * Z;
+                order(3, -shk::k33, 0.0f, gY(14), gY(8));
+                order(2, shk::k32 * Z, shk::k32, gY(13), gY(9));
+                order(1, shk::k31b - shk::k31a * zz, -2.0f * shk::k31a * Z, gY(12), gY(10));
+                vz += (3.0f * shk::k30a * zz - shk::k30b) * gY(11);
             }
         }
         const float dn = (vx * X + vy * Y) + vz * Z;
@@ -619,8 +611,9 @@ __device__ __forceinline__ void projection_vjp(const CamD& cam, const ssr_world&
     }
 }
 
-template <int kDegree, bool kAccumulate, bool kLens>
+template <int kDegree, int kPut, bool kLens>
 __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projection_bwd_params P) {
+    constexpr bool kAccumulate = kPut != kPutStore;
     const int64_t i = (int64_t)blockIdx.x * kProjBlock + threadIdx.x;
     if (i >= (P.packed_gaussian_ids ? P.num_packed : (P.visible_ids ? P.n_visible : P.num_splats))) return;
     // g: row of the splat in world / v_world; r: its row in v_screen (ProjectionBwd_kernel.cuh:51-63)
@@ -651,8 +644,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
         const bool ok = ssr_isfinite(d2) && d2 != 0.0f;   // harmonics.slang:397-403
 #pragma unroll
         for (int c = 0; c < 3; c++) {
-            if (kAccumulate) { if (ok) vsh[3 * j + c] += tv[c]; }
-            else vsh[3 * j + c] = ok ? tv[c] : 0.0f;
+            put<kPut>(vsh + 3 * j + c, ok ? tv[c] : 0.0f);
         }
     });
     if (!kAccumulate) {   // coefficients above the active degree receive nothing
@@ -660,14 +652,14 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
     }
     // World::atomicStore (src/primitives/PrimitiveBase3DGS.cuh:75-83): per-component finite filter
 #pragma unroll
-    for (int i = 0; i < 3; i++) put<kAccumulate>(V.means + 3 * g + i, fin(wg.mean[i]));
+    for (int i = 0; i < 3; i++) put<kPut>(V.means + 3 * g + i, fin(wg.mean[i]));
 #pragma unroll
-    for (int i = 0; i < 4; i++) put<kAccumulate>(V.quats + 4 * g + i, fin(wg.quat[i]));
+    for (int i = 0; i < 4; i++) put<kPut>(V.quats + 4 * g + i, fin(wg.quat[i]));
 #pragma unroll
-    for (int i = 0; i < 3; i++) put<kAccumulate>(V.log_scales + 3 * g + i, fin(wg.scale[i]));
-    put<kAccumulate>(V.opacity_logits + g, fin(wg.logit));
+    for (int i = 0; i < 3; i++) put<kPut>(V.log_scales + 3 * g + i, fin(wg.scale[i]));
+    put<kPut>(V.opacity_logits + g, fin(wg.logit));
 #pragma unroll
-    for (int i = 0; i < 3; i++) put<kAccumulate>(V.features_dc + 3 * g + i, fin(wg.dc[i]));
+    for (int i = 0; i < 3; i++) put<kPut>(V.features_dc + 3 * g + i, fin(wg.dc[i]));
 }
 
 // Camera-pose gradient: the same VJP once more, keeping only dL/dR and dL/dt, summed over the workgroup and added
@@ -814,8 +806,8 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
     if (g < P.num_splats) {
         if (P.steps) {   // per-splat step: beta^t = exp(t ln beta)
             const float t = (float)P.steps[g];
-            ad.b1c = 1.0f / (1.0f - ssr_exp(t * -0.105360515657826301f));
-            ad.b2c = 1.0f / (1.0f - ssr_exp(t * -0.00100050033358353350f));
+            ad.b1c = ssr_adam_inv_bias1(t);
+            ad.b2c = ssr_adam_inv_bias2(t);
         }
         // gradient contributions that are already there (World::atomicLoad, FusedProjectionBwdOptim_kernel.cuh:250-251)
         WorldGradD wg;
@@ -1356,14 +1348,16 @@ extern "C" int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream
     const dim3 grid((unsigned)ceil_div(work, kProjBlock)), block(kProjBlock);
     hipStream_t s = as_stream(stream);
     const bool lens = camera_needs_lens_path(p->camera.camera_model, p->camera.distortion);
-#define SSR_LAUNCH_BWD(D)                                                                                     \
-    if (lens) {                                                                                               \
-        if (p->accumulate) hipLaunchKernelGGL((projection_bwd_kernel<D, true, true>), grid, block, 0, s, *p);  \
-        else hipLaunchKernelGGL((projection_bwd_kernel<D, false, true>), grid, block, 0, s, *p);               \
-    } else {                                                                                                  \
-        if (p->accumulate) hipLaunchKernelGGL((projection_bwd_kernel<D, true, false>), grid, block, 0, s, *p); \
-        else hipLaunchKernelGGL((projection_bwd_kernel<D, false, false>), grid, block, 0, s, *p);              \
+    // accumulating over packed rows: a caller's id list may name a splat more than once (rows of several
+    // cameras), so add atomically unless the caller vouches for unique ids
+    const int put_mode = !p->accumulate ? kPutStore : ((packed && !p->packed_ids_unique) ? kPutAtomic : kPutAdd);
+#define SSR_LAUNCH_BWD_L(D, L)                                                                                          \
+    switch (put_mode) {                                                                                                 \
+        case kPutStore: hipLaunchKernelGGL((projection_bwd_kernel<D, kPutStore, L>), grid, block, 0, s, *p); break;       \
+        case kPutAdd: hipLaunchKernelGGL((projection_bwd_kernel<D, kPutAdd, L>), grid, block, 0, s, *p); break;           \
+        default: hipLaunchKernelGGL((projection_bwd_kernel<D, kPutAtomic, L>), grid, block, 0, s, *p); break;             \
     }
+#define SSR_LAUNCH_BWD(D) if (lens) { SSR_LAUNCH_BWD_L(D, true) } else { SSR_LAUNCH_BWD_L(D, false) }
     switch (p->sh_degree) {
         case 0: SSR_LAUNCH_BWD(0); break;
         case 1: SSR_LAUNCH_BWD(1); break;
@@ -1371,6 +1365,7 @@ extern "C" int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream
         default: SSR_LAUNCH_BWD(3); break;
     }
 #undef SSR_LAUNCH_BWD
+#undef SSR_LAUNCH_BWD_L
     SSR_CHECK_LAUNCH("ssr_projection_bwd");
     if (p->v_viewmat) {
 #define SSR_LAUNCH_POSE(D)                                                                            \
@@ -1437,8 +1432,8 @@ extern "C" int ssr_fused_projection_bwd_optimizer(const ssr_fpbo_params* p, ssr_
     SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->world.quats) & 15) == 0, where, "quats must be 16-byte aligned");
     SSR_REQUIRE(p->steps || p->step >= 1, where, "Adam step must be >= 1");
     AdamD ad;
-    ad.b1c = (float)(1.0 / (1.0 - pow(0.9, (double)p->step)));
-    ad.b2c = (float)(1.0 / (1.0 - pow(0.999, (double)p->step)));
+    ad.b1c = ssr_adam_inv_bias1((float)p->step);
+    ad.b2c = ssr_adam_inv_bias2((float)p->step);
     const dim3 grid((unsigned)ceil_div(p->num_splats, kProjBlock)), block(kProjBlock);
     hipStream_t s = as_stream(stream);
     const bool lens = camera_needs_lens_path(p->camera.camera_model, p->camera.distortion);

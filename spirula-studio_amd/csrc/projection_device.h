@@ -322,7 +322,24 @@ __device__ __forceinline__ void decode_sh(const ssr_world& w, const ssr_sh_quant
     }
 }
 
-struct ShBasisD { float Y[15]; float x, y, z, inorm; };
+// Real spherical harmonics of bands 1..3 in the product form
+//   Y(l, +m) = A_lm(z) Re (x + i y)^m,   Y(l, -m) = A_lm(z) Im (x + i y)^m,   Y(l, 0) = B_l(z),
+// with the sign and ordering convention of src/shaders/harmonics.slang:172-217 (index j runs -l..l
+// inside band l). The colour feeds bit-exact tile keys downstream, so each Y_j is formed by the
+// operations the oracle uses; (x + i y)^m comes from the complex-power recurrence (x y + y x is
+// exactly 2 x y). The direction gradient in projection_vjp differentiates the same product form.
+struct ShBasisD {
+    float Y[15];
+    float x, y, z, inorm;
+    float re[4], im[4];   // Re / Im (x + i y)^m, m = 0..3
+};
+
+namespace shk {   // normalisation constants of the product form
+constexpr float k1 = 0.48860251190292f;
+constexpr float k20a = 0.9461746957575601f, k20b = 0.3153915652525201f, k21 = 1.092548430592079f, k22 = 0.5462742152960395f;
+constexpr float k30a = 1.865881662950577f, k30b = 1.119528997770346f, k31a = 2.285228997322329f, k31b = 0.4570457994644658f,
+                k32 = 1.445305721320277f, k33 = 0.5900435899266435f;
+}  // namespace shk
 
 template <int kDegree>
 __device__ __forceinline__ void sh_basis(const float dir[3], ShBasisD& b) {
@@ -331,32 +348,34 @@ __device__ __forceinline__ void sh_basis(const float dir[3], ShBasisD& b) {
     b.inorm = 1.0f / ssr_sqrt((dir[0] * dir[0] + dir[1] * dir[1]) + dir[2] * dir[2]);
     const float x = dir[0] * b.inorm, y = dir[1] * b.inorm, z = dir[2] * b.inorm;
     b.x = x; b.y = y; b.z = z;
+    b.re[0] = 1.0f; b.im[0] = 0.0f; b.re[1] = x; b.im[1] = y;
+#pragma unroll
+    for (int m = 1; m < 3; m++) {
+        b.re[m + 1] = x * b.re[m] - y * b.im[m];
+        b.im[m + 1] = x * b.im[m] + y * b.re[m];
+    }
     if (kDegree < 1) return;
-    b.Y[0] = -0.48860251190292f * y;
-    b.Y[1] = 0.48860251190292f * z;
-    b.Y[2] = -0.48860251190292f * x;
+    b.Y[0] = -shk::k1 * b.im[1];
+    b.Y[1] = shk::k1 * z;
+    b.Y[2] = -shk::k1 * b.re[1];
     if (kDegree < 2) return;
-    const float z2 = z * z;
-    const float fTmp0B = -1.092548430592079f * z;
-    const float fC1 = x * x - y * y;
-    const float fS1 = 2.f * x * y;
-    b.Y[3] = 0.5462742152960395f * fS1;
-    b.Y[4] = fTmp0B * y;
-    b.Y[5] = 0.9461746957575601f * z2 - 0.3153915652525201f;
-    b.Y[6] = fTmp0B * x;
-    b.Y[7] = 0.5462742152960395f * fC1;
+    const float zz = z * z;
+    const float a21 = -shk::k21 * z;
+    b.Y[3] = shk::k22 * b.im[2];
+    b.Y[4] = a21 * b.im[1];
+    b.Y[5] = shk::k20a * zz - shk::k20b;
+    b.Y[6] = a21 * b.re[1];
+    b.Y[7] = shk::k22 * b.re[2];
     if (kDegree < 3) return;
-    const float fTmp0C = -2.285228997322329f * z2 + 0.4570457994644658f;
-    const float fTmp1B = 1.445305721320277f * z;
-    const float fC2 = x * fC1 - y * fS1;
-    const float fS2 = x * fS1 + y * fC1;
-    b.Y[8] = -0.5900435899266435f * fS2;
-    b.Y[9] = fTmp1B * fS1;
-    b.Y[10] = fTmp0C * y;
-    b.Y[11] = z * (1.865881662950577f * z2 - 1.119528997770346f);
-    b.Y[12] = fTmp0C * x;
-    b.Y[13] = fTmp1B * fC1;
-    b.Y[14] = -0.5900435899266435f * fC2;
+    const float a31 = -shk::k31a * zz + shk::k31b;
+    const float a32 = shk::k32 * z;
+    b.Y[8] = -shk::k33 * b.im[3];
+    b.Y[9] = a32 * b.im[2];
+    b.Y[10] = a31 * b.im[1];
+    b.Y[11] = z * (shk::k30a * zz - shk::k30b);
+    b.Y[12] = a31 * b.re[1];
+    b.Y[13] = a32 * b.re[2];
+    b.Y[14] = -shk::k33 * b.re[3];
 }
 
 // colour before the +0.5 shift (src/shaders/harmonics.slang:154-223)

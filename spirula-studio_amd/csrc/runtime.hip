@@ -52,6 +52,8 @@ __global__ void debug_math_kernel(int op, int64_t n, const float* a, const float
         case 0: r = ssr_exp(a[i]); break;
         case 1: r = ssr_log(a[i]); break;
         case 2: r = ssr_atan2(a[i], b[i]); break;
+        case 4: r = ssr_adam_inv_bias1(a[i]); break;
+        case 5: r = ssr_adam_inv_bias2(a[i]); break;
         default: r = ssr_sigmoid(a[i]); break;
     }
     out[i] = r;

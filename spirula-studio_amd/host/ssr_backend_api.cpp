@@ -665,6 +665,7 @@ void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
     if (is_packed) {
         p.aabb = nullptr;
         p.packed_gaussian_ids = gaussian_ids.data_ptr(); p.num_packed = camera_ids.size();
+        p.packed_ids_unique = 1;   // one camera per call: the packed projection lists a splat once
         g_bwd_list = gaussian_ids.data_ptr(); g_bwd_count = camera_ids.size();
     } else if (g_visible_ids && g_n_visible >= 0) {
         // the rows that end up non-zero are the listed ones either way

@@ -76,7 +76,7 @@ class ProjectionBwdParams(C.Structure):
                 ("v_world", World), ("accumulate", C.c_int32), ("visible_ids", vp),
                 ("n_visible", C.c_int64), ("packed_gaussian_ids", vp), ("num_packed", C.c_int64), ("v_rows", vp),
                 ("v_viewmat", vp),
-                ("antialiased", C.c_int32)]
+                ("antialiased", C.c_int32), ("packed_ids_unique", C.c_int32)]
 
 
 class ProjectionPackedParams(C.Structure):

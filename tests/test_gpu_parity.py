@@ -186,6 +186,12 @@ def test_device_math_is_bit_identical_to_host(gpu, oracle):
         got = do.to_host()
         want = oracle.math(op, x, b)
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), op
+    # Adam's inverse bias corrections (ops 4, 5) at integer steps
+    t = np.concatenate([np.arange(1, 20000), [50000, 1000000]]).astype(np.float32)
+    dt, dr = L.DeviceArray.from_host(t), L.DeviceArray(t.shape, np.float32)
+    for op in (4, 5):
+        L.check(lib.ssr_debug_math(op, t.size, dt.ptr, dt.ptr, dr.ptr, None))
+        assert np.array_equal(dr.to_host().view(np.uint32), oracle.math(op, t).view(np.uint32)), op
 
 
 def test_tiny_pinhole(gpu, oracle):
@@ -333,6 +339,31 @@ def test_packed_projection_tiny(gpu, oracle):
     _compare_packed(gpu, oracle, gpu.scenes.tiny_scene(n=700, width=96, height=64, seed=21), "pk-tiny")
     _compare_packed(gpu, oracle, gpu.scenes.tiny_scene(n=900, width=80, height=48, seed=22), "pk-tiny-fused",
                     fused_count=True, use_packed=True)
+
+
+def test_packed_backward_adds_repeated_ids(gpu, oracle):
+    """A packed id list that names splats twice (the rows of two cameras in one list): the accumulating
+    projection backward adds atomically by default, so both rows of a splat reach its world row; with
+    ids declared unique the plain read-add-write is used and gives the single-camera result."""
+    D = gpu.lib.DeviceArray
+    g, r = _compare_packed(gpu, oracle, gpu.scenes.tiny_scene(n=900, width=96, height=64, seed=29), "pk-repeat")
+    m = g.rows // 3
+    assert m > 50
+    once = {k: g.host(k).copy() for k in ["w_means", "w_quats", "w_log_scales", "w_opacity_logits", "w_features_dc", "w_features_sh"]}
+    ids = g.host("gaussian_ids")[:m]
+    keep = np.zeros(g.n, bool)
+    keep[ids] = True
+    for k in ["gaussian_ids", "v_xy", "v_depth", "v_conic", "v_opac", "v_rgb"]:
+        a = g.host(k)[:m]
+        g.d[k] = D.from_host(np.concatenate([a, a]))
+    g.rows = 2 * m
+    g.use_vrows = False
+    g.projection_bwd(accumulate=True)
+    for k, v in once.items():
+        got = g.host(k)
+        assert np.array_equal(got[keep], 2.0 * v[keep]), k      # x + x is exact, whichever row lands first
+        assert not np.any(got[~keep]), k
+    assert np.abs(once["w_means"][keep]).max() > 0
 
 
 def test_packed_projection_without_readback(gpu, oracle):

@@ -5,7 +5,7 @@ differences of the loss definitions of src/shaders/per_splat_losses.slang:30-81.
 import numpy as np
 import pytest
 
-B1, B2, EPS = 0.9, 0.999, 1e-15
+B1, B2, EPS = float(np.float32(0.9)), float(np.float32(0.999)), 1e-15   # the reference's float constants
 KSH0 = 0.28209479177387814
 
 

@@ -55,3 +55,23 @@ def test_sigmoid(oracle):
     got = oracle.math(3, x)
     want = 1 / (1 + np.exp(-x.astype(np.float64)))
     assert np.abs(got - want).max() < 1.5e-7
+
+
+def test_adam_inverse_bias_corrections(oracle):
+    """1 / (1 - beta^t) with the reference's FLOAT betas (FusedProjectionBwdOptim_kernel.cuh:369-370): against
+    float64 powers of float32(0.9) / float32(0.999). The power is within 2 ulp, so the correction is within
+    2 ulp of the power's spacing divided by (1 - beta^t) -- and nowhere near the 1.3e-5 by which a correction
+    built on the double constant 0.999 is off at small t."""
+    t = np.concatenate([np.arange(1, 3000), np.array([5000, 30000, 100000, 1000000])]).astype(np.float32)
+    for op, beta in ((4, np.float32(0.9)), (5, np.float32(0.999))):
+        p = float(beta) ** t.astype(np.float64)
+        want = 1.0 / (1.0 - p)
+        got = oracle.math(op, t).astype(np.float64)
+        ulp_p = np.maximum(np.spacing(p.astype(np.float32)).astype(np.float64), 2.0 ** -25)   # 1 - p rounds at 2^-24 or finer
+        bound = 2.5 * ulp_p / (1.0 - p) + 2e-7
+        assert (np.abs(got / want - 1.0) <= bound).all(), (op, float(np.abs(got / want - 1.0).max()))
+    # t = 1: the power is the float constant itself and 1 - beta is exact (the reference's value)
+    assert oracle.math(4, np.array([1], np.float32))[0] == np.float32(1.0) / (np.float32(1.0) - np.float32(0.9))
+    assert oracle.math(5, np.array([1], np.float32))[0] == np.float32(1.0) / (np.float32(1.0) - np.float32(0.999))
+    wrong = 1.0 / (1.0 - 0.999 ** 2.0)    # the double-constant form misses by > 5e-6 at t = 2
+    assert abs(oracle.math(5, np.array([2], np.float32))[0] / wrong - 1.0) > 5e-6
