@@ -1178,6 +1178,72 @@ void or_raster_fwd_ex(int64_t N, const float* xy, const float* depth, const floa
     if (stats) { stats[0] = kf; stats[1] = kb; stats[2] = vis_f; stats[3] = vis_b; stats[4] = prod_b; }
 }
 
+// Lane statistics of the compositing backward (a measurement aid, not a restatement of the reference):
+// how many of the pixels a (splat, pixel-block) visit covers actually composite the splat (alpha > 1/255
+// and sorted index <= the pixel's last_id), for square blocks of 8, 4 and 2 pixels inside the 8x8
+// sub-tiles the reference's footprint test keeps. A block is visited when the sub-tile test passes,
+// the sorted index does not exceed the largest last_id of the block's sub-tile, and the ellipse
+// alpha >= 1/255 reaches the box of the block's pixel centres.
+// out[0..2] = visits at block size 8, 4, 2; out[3] = compositing (pixel, splat) pairs;
+// out[4..6] = visits with at least one compositing pixel, per block size.
+void or_raster_lane_stats(const float* xy, const float* depth, const float* conic, const float* opac, const float* rgb,
+    uint32_t width, uint32_t height, const int32_t* tile_offsets, const int32_t* flatten_ids, int64_t n_isects,
+    const int32_t* last_ids, int64_t* out) {
+    const int tw = (int)((width + kTile - 1) / kTile), th = (int)((height + kTile - 1) / kTile);
+    const int n_tiles = tw * th;
+    int64_t v8 = 0, v4 = 0, v2 = 0, pairs = 0, p8 = 0, p4 = 0, p2 = 0;
+#pragma omp parallel for schedule(dynamic, 4) reduction(+ : v8, v4, v2, pairs, p8, p4, p2)
+    for (int tile = 0; tile < n_tiles; tile++) {
+        const int ty = tile / tw, tx = tile % tw;
+        const int32_t start = tile_offsets[tile];
+        const int32_t end = (tile == n_tiles - 1) ? (int32_t)n_isects : tile_offsets[tile + 1];
+        int32_t mt_last[4] = {-1, -1, -1, -1};
+        for (int py_ = 0; py_ < kTile; py_++)
+            for (int px_ = 0; px_ < kTile; px_++) {
+                const uint32_t i = ty * kTile + py_, j = tx * kTile + px_;
+                if (i >= height || j >= width) continue;
+                const int mt = (py_ / kMicro) * 2 + (px_ / kMicro);
+                mt_last[mt] = std::max(mt_last[mt], last_ids[(int64_t)i * width + j]);
+            }
+        for (int32_t k = start; k < end; k++) {
+            const int32_t g = flatten_ids[k];
+            const Frag f = load_frag(g, xy, depth, conic, opac, rgb);
+            if (!(f.opac > kAlphaThreshold)) continue;
+            const float kk = 0.5f / ssr_log(f.opac / kAlphaThreshold);
+            const float ic[3] = {f.cx * kk, f.cy * kk, f.cz * kk};
+            for (int mt = 0; mt < 4; mt++) {
+                if (k > mt_last[mt]) continue;
+                const int ox = tx * kTile + (mt & 1) * kMicro, oy = ty * kTile + (mt >> 1) * kMicro;
+                if (!micro_hit(xy + 2 * g, conic + 3 * g, f.opac, (float)ox, (float)oy)) continue;
+                bool act[8][8];
+                for (int y = 0; y < 8; y++)
+                    for (int x = 0; x < 8; x++) {
+                        const uint32_t i = oy + y, j = ox + x;
+                        act[y][x] = false;
+                        if (i >= height || j >= width) continue;
+                        float dx, dy, vis, sigma;
+                        const float alpha = eval_alpha(f, (float)j + 0.5f, (float)i + 0.5f, dx, dy, vis, sigma);
+                        act[y][x] = alpha > kAlphaThreshold && k <= last_ids[(int64_t)i * width + j];
+                    }
+                for (int bs = 8; bs >= 2; bs >>= 1) {
+                    for (int by = 0; by < 8; by += bs)
+                        for (int bx = 0; bx < 8; bx += bs) {
+                            const float x0 = (float)(ox + bx) + 0.5f - f.x, y0 = (float)(oy + by) + 0.5f - f.y;
+                            if (bs < 8 && !ellipse_box_overlap(ic, x0, x0 + (float)(bs - 1), y0, y0 + (float)(bs - 1))) continue;
+                            int n_act = 0;
+                            for (int y = by; y < by + bs; y++)
+                                for (int x = bx; x < bx + bs; x++) n_act += act[y][x] ? 1 : 0;
+                            if (bs == 8) { v8++; pairs += n_act; p8 += n_act > 0; }
+                            else if (bs == 4) { v4++; p4 += n_act > 0; }
+                            else { v2++; p2 += n_act > 0; }
+                        }
+                }
+            }
+        }
+    }
+    out[0] = v8; out[1] = v4; out[2] = v2; out[3] = pairs; out[4] = p8; out[5] = p4; out[6] = p2;
+}
+
 // rasterize_to_pixels_bwd_kernel (IS_EVAL3D=0, dist_type=None, no median, no accum weights),
 // src/kernels/raster/RasterizationEval3DBwd_kernel.cuh:107-584, fragment VJPs from
 // src/primitives/Primitive3DGS.cuh:262-300. Partial sums are formed per (splat, 8x8 sub-tile)

@@ -93,6 +93,10 @@ void or_raster_fwd(int64_t N, const float* xy, const float* depth, const float* 
 
 /* K8. v_* outputs are ACCUMULATED into (caller zero-fills). abs_* (optional, may be NULL) receive
  * the sum of absolute values of the same terms in double, as an error scale for comparisons. */
+/* measurement aid: lane statistics of the compositing backward for pixel blocks of 8, 4 and 2 */
+void or_raster_lane_stats(const float* xy, const float* depth, const float* conic, const float* opac, const float* rgb,
+    uint32_t width, uint32_t height, const int32_t* tile_offsets, const int32_t* flatten_ids, int64_t n_isects,
+    const int32_t* last_ids, int64_t* out);
 void or_raster_bwd(int64_t N, const float* xy, const float* depth, const float* conic,
     const float* opac, const float* rgb, uint32_t width, uint32_t height,
     const int32_t* tile_offsets, const int32_t* flatten_ids, int64_t n_isects,

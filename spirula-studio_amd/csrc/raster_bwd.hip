@@ -21,6 +21,7 @@
 // dropped and zeros skipped as there (src/core/Common.cuh:791-856). The scan starts at the tile's largest
 // last_id rather than at the end of the range; splats beyond it are skipped by every pixel anyway.
 #include "raster_device.h"
+#include <stdlib.h>
 
 namespace ssr {
 
@@ -341,6 +342,293 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
     flush_slot();
 }
 
+// ---- the row-granular plain kernel --------------------------------------------------------------
+//
+// Same per-pixel arithmetic, different walk: a wavefront's four 16-lane rows each hold one 4x4-pixel
+// block of the wavefront's 8x8 sub-tile and walk their OWN list of the staged fragments -- those whose
+// block bit is set (raster_device.h) and whose sorted index does not exceed the block's largest
+// last_id. A splat of a few pixels' radius touches about half of the blocks of the sub-tiles it
+// touches, so far fewer lanes idle than when all 64 lanes visit every fragment of the sub-tile.
+// Lists are built per batch by the wavefront that walks them (ballot + rank, slot numbers as bytes).
+// The ten per-splat sums are reduced inside each row by a transposing reduction over the four lane
+// bits (row_ror:8, row_half_mirror, two quad permutations): every level halves the number of live
+// registers by keeping one channel in the lanes with the bit clear and another in those with it
+// set, so 29 operations leave each of ten lanes of the row holding one finished channel.
+// What is summed are moments of u = vis * v_alpha: (u, u dx, u dy, u dx^2, u dx dy, u dy^2) and the four
+// colour / depth weights; the gradients of position, conic and opacity are linear in them and are
+// formed once per fragment when its sums leave LDS.
+// exp(-sigma) comes from the hardware exponential; whenever a lane's alpha falls within 4e-5 relative
+// of the 1/255 threshold or of the 0.999 gate, the wavefront re-evaluates with the bit-defined
+// exponential, so every decision is the one the forward took.
+
+template <int kCtrl>
+__device__ __forceinline__ float dpp_full(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, 0xf, 0xf, true));
+}
+// lanes with `sel` clear end with a[l] + a[partner], lanes with it set with b[l] + b[partner]
+template <int kCtrl>
+__device__ __forceinline__ float fold_pair(float a, float b, bool sel) {
+    const float keep = sel ? b : a, send = sel ? a : b;
+    return keep + dpp_full<kCtrl>(send);
+}
+constexpr int kDppRor8 = 0x128, kDppHalfMirror = 0x141, kDppQuadXor2 = 0x4E, kDppQuadXor1 = 0xB1;
+
+constexpr int kRowBatch = 128;   // fragments staged per batch by the row-granular kernel
+
+__global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raster_bwd_params P, int tile_w, int tile_h) {
+    __shared__ FragLds frags[kRowBatch];
+    __shared__ int32_t s_ids[kRowBatch];
+    __shared__ int s_wave_max[4];
+    // Moment sums per (wavefront, fragment, channel). Each wavefront adds into its own copy with a plain
+    // read-add-write: a float atomic in LDS costs about three cycles per active lane on this hardware,
+    // which at forty lanes a step would make LDS, not arithmetic, the limit of this kernel.
+    __shared__ float s_acc[4 * kRowBatch * 10];
+    __shared__ uint8_t s_bits[2 * kRowBatch];                       // block bits of sub-tiles {0,1} and {2,3}
+    __shared__ uint8_t s_list[kBlocksPerTile * kRowBatch + 16];
+    const int n_tiles = tile_w * tile_h * (P.num_images > 1 ? P.num_images : 1);
+    const int tile = xcd_tile_of(blockIdx.x, n_tiles);
+    if (tile >= n_tiles) return;
+    const int tid = threadIdx.x, lane = tid & 63, mt = tid >> 6, row = lane >> 4, l16 = lane & 15;
+    const int gy = tile / tile_w, tx = tile - gy * tile_w;
+    const int img = gy / tile_h, ty = gy - img * tile_h;
+    const int j = tx * kTile + (mt & 1) * kMicro + (row & 1) * kBlock + (l16 & 3);
+    const int i = ty * kTile + (mt >> 1) * kMicro + (row >> 1) * kBlock + (l16 >> 2);
+    const float px = (float)j + 0.5f, py = (float)i + 0.5f;
+    const bool inside = (uint32_t)i < P.height && (uint32_t)j < P.width;
+    const int64_t pid = ((int64_t)img * P.height + i) * P.width + j;
+
+    const int32_t bin_final = inside ? P.last_ids[pid] : -1;
+    float T1 = inside ? P.render_T[pid] : 0.0f;
+    float vT1 = inside ? P.v_render_T[pid] : 0.0f;
+    float vr = 0.f, vg = 0.f, vb = 0.f, vd = 0.f;
+    if (inside) {
+        const float* v = P.v_render_rgb + 3 * pid;
+        vr = v[0]; vg = v[1]; vb = v[2];
+        vd = P.v_render_depth[pid];
+        const float inv_alpha = 1.0f / ssr_max(1.0f - T1, 1e-10f);
+        vT1 = vT1 + (P.render_depth[pid] * vd) * inv_alpha;
+        vd = vd * inv_alpha;
+    }
+
+    const int32_t range_start = P.tile_offsets[tile];
+    const int32_t range_end = (tile == n_tiles - 1) ? (int32_t)P.n_isects : P.tile_offsets[tile + 1];
+    // largest last_id per block (row), per wavefront, per tile
+    int row_last = bin_final;
+#pragma unroll
+    for (int d = 8; d >= 1; d >>= 1) row_last = max(row_last, __shfl_xor(row_last, d, 16));
+    const int blk_last[4] = {__builtin_amdgcn_readlane(row_last, 0), __builtin_amdgcn_readlane(row_last, 16),
+                             __builtin_amdgcn_readlane(row_last, 32), __builtin_amdgcn_readlane(row_last, 48)};
+    const int wave_last = max(max(blk_last[0], blk_last[1]), max(blk_last[2], blk_last[3]));
+    if (lane == 0) s_wave_max[mt] = wave_last;
+    __syncthreads();
+    const int tile_last = max(max(s_wave_max[0], s_wave_max[1]), max(s_wave_max[2], s_wave_max[3]));
+    const float tile_x0 = (float)(tx * kTile), tile_y0 = (float)(ty * kTile);
+
+    // which finished channel this lane holds after the reduction (see the fold order below): -1 none
+    const bool b3 = (l16 & 8) != 0, b2 = (l16 & 4) != 0, b1 = (l16 & 2) != 0, b0 = (l16 & 1) != 0;
+    int chan = -1;
+    if (!b0) chan = 4 * (b1 ? 1 : 0) + 2 * (b2 ? 1 : 0) + (b3 ? 1 : 0);
+    else if (!b1 && !b2) chan = 8 + (b3 ? 1 : 0);
+    for (int e = tid; e < 4 * kRowBatch * 10; e += kRasterBlock) s_acc[e] = 0.0f;
+    float* my_acc = s_acc + mt * (kRowBatch * 10);
+
+    // Two neighbouring threads own fragment slot t / 2: they add up the four wavefronts' moment sums, turn
+    // them into the ten gradient channels (x, y, depth, conic[3], opac, rgb[3]) and leave those in the first
+    // copy; then all threads move the batch to global memory in the order of the destination rows, so that
+    // a row's atomics travel as one or two requests.
+    auto flush = [&]() {
+        {
+            const int slot = tid >> 1;
+            const bool geom = (tid & 1) == 0;   // this thread: u, ux, uy, uxx, uxy, uyy; its neighbour: the colour / depth weights
+            float m[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            const int c0 = geom ? 0 : 6, nc = geom ? 6 : 4;
+#pragma unroll
+            for (int w = 0; w < 4; w++)
+#pragma unroll
+                for (int c = 0; c < 6; c++)
+                    if (c < nc) { m[c] += s_acc[(w * kRowBatch + slot) * 10 + c0 + c]; }
+#pragma unroll
+            for (int w = 1; w < 4; w++)
+#pragma unroll
+                for (int c = 0; c < 6; c++)
+                    if (c < nc) s_acc[(w * kRowBatch + slot) * 10 + c0 + c] = 0.0f;
+            float o[6];
+            if (geom) {
+                const float4 q0 = frags[slot].q0, q1 = frags[slot].q1;
+                const float k = -q1.y;                       // v_sigma = -(opac vis) v_alpha = k u
+                const float sx = k * m[1], sy = k * m[2];
+                o[0] = ssr_fma(q0.z + q0.z, sx, q0.w * sy);  // conic.x = 2 * (0.5 conic.x), conic.z likewise
+                o[1] = ssr_fma(q0.w, sx, (q1.x + q1.x) * sy);
+                o[2] = (0.5f * k) * m[3]; o[3] = k * m[4]; o[4] = (0.5f * k) * m[5];
+                o[5] = m[0];
+            } else {
+                o[0] = m[3]; o[1] = m[0]; o[2] = m[1]; o[3] = m[2]; o[4] = 0.f; o[5] = 0.f;
+            }
+            // both threads of a slot sit in one wavefront, so every read above precedes these writes
+            float* dst = s_acc + slot * 10;
+            if (geom) {
+                dst[0] = ssr_isfinite(o[0]) ? o[0] : 0.f; dst[1] = ssr_isfinite(o[1]) ? o[1] : 0.f;
+                dst[3] = ssr_isfinite(o[2]) ? o[2] : 0.f; dst[4] = ssr_isfinite(o[3]) ? o[3] : 0.f;
+                dst[5] = ssr_isfinite(o[4]) ? o[4] : 0.f; dst[6] = ssr_isfinite(o[5]) ? o[5] : 0.f;
+            } else {
+                dst[2] = ssr_isfinite(o[0]) ? o[0] : 0.f;
+                dst[7] = ssr_isfinite(o[1]) ? o[1] : 0.f; dst[8] = ssr_isfinite(o[2]) ? o[2] : 0.f;
+                dst[9] = ssr_isfinite(o[3]) ? o[3] : 0.f;
+            }
+        }
+        __syncthreads();
+        if (P.v_rows) {
+            for (int e = tid; e < kRowBatch * 10; e += kRasterBlock) {
+                const int slot = e / 10, ch = e - slot * 10;
+                const float x = s_acc[e];
+                if (x != 0.0f) {
+                    s_acc[e] = 0.0f;
+                    atomicAdd(P.v_rows + (int64_t)12 * s_ids[slot] + ch, x);
+                }
+            }
+        } else if (tid < kRowBatch) {
+            float v[10];
+            bool any = false;
+#pragma unroll
+            for (int c = 0; c < 10; c++) { v[c] = s_acc[tid * 10 + c]; any |= v[c] != 0.0f; }
+            if (any) {
+#pragma unroll
+                for (int c = 0; c < 10; c++) s_acc[tid * 10 + c] = 0.0f;
+                const int64_t g = s_ids[tid];
+                auto add = [](float* p, float x) { if (x != 0.0f) atomicAdd(p, x); };
+                add(P.v_screen.xy + 2 * g, v[0]); add(P.v_screen.xy + 2 * g + 1, v[1]);
+                add(P.v_screen.depth + g, v[2]);
+                add(P.v_screen.conic + 3 * g, v[3]); add(P.v_screen.conic + 3 * g + 1, v[4]); add(P.v_screen.conic + 3 * g + 2, v[5]);
+                add(P.v_screen.opac + g, v[6]);
+                add(P.v_screen.rgb + 3 * g, v[7]); add(P.v_screen.rgb + 3 * g + 1, v[8]); add(P.v_screen.rgb + 3 * g + 2, v[9]);
+            }
+        }
+        __syncthreads();   // s_ids, frags and s_acc are free for the next batch
+    };
+
+    const uint8_t* my_list = s_list + (4 * mt + row) * kRowBatch;
+    bool first = true;
+    for (int32_t hi = min(range_end - 1, tile_last); hi >= range_start; hi -= kRowBatch) {
+        // Explicit wait for this wavefront's LDS traffic (the read-add-writes and float atomics of the walk):
+        // the compiler does not place one ahead of this loop-header barrier on the path that leaves the walk,
+        // and a pending float atomic is overtaken by the reads that follow the barrier.
+        __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
+        __syncthreads();   // previous batch fully consumed (first pass: the zero fill of s_acc is complete)
+        if (!first) flush();   // its sums leave before the slots are reused
+        first = false;
+        {
+            // slot t holds sorted index hi - t: ascending t is back to front. Thread pair (slot, half) shares the staging.
+            const int slot = tid & (kRowBatch - 1), half = tid >> 7;
+            const int32_t idx = hi - slot;
+            uint32_t bits8 = 0;
+            if (idx >= range_start) {
+                const int32_t g = P.flatten_ids[idx];
+                const FragLds f = stage_fragment_half(P.screen, P.packed_rows, g, tile_x0, tile_y0, half, bits8);
+                if (half == 0) { s_ids[slot] = g; frags[slot] = f; }
+            }
+            s_bits[half * kRowBatch + slot] = (uint8_t)bits8;
+        }
+        __syncthreads();
+        // this wavefront's four lists: slots whose block bit is set and whose sorted index hi - slot is
+        // not beyond the block's largest last_id
+        const int n_batch = min(kRowBatch, hi - range_start + 1);
+        int cnt[4] = {0, 0, 0, 0};
+        for (int c = 0; c * 64 < n_batch; c++) {
+            const int slot = c * 64 + lane;
+            const uint32_t bits = (uint32_t)s_bits[(mt >> 1) * kRowBatch + slot] >> (4 * (mt & 1));
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const bool in = ((bits >> r) & 1u) != 0 && hi - slot <= blk_last[r];
+                const uint64_t bal = __ballot(in);
+                if (in) s_list[(4 * mt + r) * kRowBatch + cnt[r] + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(bal >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)bal, 0u))] = (uint8_t)slot;
+                cnt[r] += __builtin_popcountll(bal);
+            }
+        }
+        // the lists are written and read by this wavefront only: order its LDS accesses, no workgroup barrier
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        const int my_cnt = row == 0 ? cnt[0] : row == 1 ? cnt[1] : row == 2 ? cnt[2] : cnt[3];
+        const int n_steps = max(max(cnt[0], cnt[1]), max(cnt[2], cnt[3]));
+        // Steps in which two rows of this wavefront sit on the same fragment: their read-add-writes would
+        // overwrite each other, so those steps add atomically. One bit per step, found here (lane = step).
+        uint64_t clash_lo = 0, clash_hi = 0;
+        {
+            const uint8_t* base = s_list + 4 * mt * kRowBatch;
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                const int stp = c * 64 + lane;
+                const int e0 = stp < cnt[0] ? (int)base[stp] : -1, e1 = stp < cnt[1] ? (int)base[kRowBatch + stp] : -2,
+                          e2 = stp < cnt[2] ? (int)base[2 * kRowBatch + stp] : -3, e3 = stp < cnt[3] ? (int)base[3 * kRowBatch + stp] : -4;
+                const bool cl = (e0 == e1) | (e0 == e2) | (e0 == e3) | (e1 == e2) | (e1 == e3) | (e2 == e3);
+                const uint64_t m = (c * 64 < n_steps) ? __ballot(cl) : 0ull;
+                if (c == 0) clash_lo = m; else clash_hi = m;
+            }
+        }
+        // Two-deep software pipeline: the list byte of step st + 2 and the fragment of step st + 1 are in
+        // flight while step st computes, so that the two dependent LDS latencies hide behind arithmetic.
+        int k_next = 0 < my_cnt ? (int)my_list[0] : 0;
+        int k_next2 = 1 < my_cnt ? (int)my_list[1] : 0;
+        float4 n0 = frags[k_next].q0, n1 = frags[k_next].q1;
+        float2 n2a = make_float2(frags[k_next].q2.x, frags[k_next].q2.y);
+        float n2w = frags[k_next].q2.w;
+#pragma unroll 2
+        for (int st = 0; st < n_steps; st++) {
+            const bool in_list = st < my_cnt;
+            const int k = k_next;
+            const float4 q0 = n0, q1 = n1;
+            const float4 q2 = make_float4(n2a.x, n2a.y, 0.0f, n2w);
+            k_next = k_next2;
+            k_next2 = st + 2 < my_cnt ? (int)my_list[st + 2] : 0;
+            n0 = frags[k_next].q0; n1 = frags[k_next].q1;
+            n2a = make_float2(frags[k_next].q2.x, frags[k_next].q2.y);
+            n2w = frags[k_next].q2.w;
+            const int32_t sorted_idx = hi - k;
+            const float dx = q0.x - px, dy = q0.y - py;
+            const float sigma = ssr_fma(q0.z * dx, dx, ssr_fma(q1.x * dy, dy, (q0.w * dx) * dy));
+            const bool in_range = !(sigma < 0.f || sigma > q2.w);
+            float vis = in_range ? __builtin_amdgcn_exp2f(sigma * -1.44269504088896341f) : 0.0f;
+            float ov = q1.y * vis;
+            const bool near_edge = in_list & ((ssr_fabs(ov - kAlphaThreshold) <= 1.6e-7f) | (ssr_fabs(ov - 0.999f) <= 4e-5f));
+            if (__ballot(near_edge) != 0ull) {   // decisions exactly as the forward took them
+                vis = in_range ? exp_neg_small(-sigma) : 0.0f;
+                ov = q1.y * vis;
+            }
+            const float alpha = ssr_min(0.999f, ov);
+            const bool active = in_list && sorted_idx <= bin_final && alpha > kAlphaThreshold;
+            if (__ballot(active) == 0ull) continue;
+            // inactive lanes run with alpha = 0 and v_alpha = 0: T and v_T unchanged, every term zero
+            const float a = active ? alpha : 0.0f;
+            const float T0 = T1 * __builtin_amdgcn_rcpf(1.0f - a);
+            const float dv = ssr_fma(q2.y, vd, ssr_fma(q2.x, vb, ssr_fma(q1.w, vg, q1.z * vr))) - vT1;
+            const float w = a * T0;
+            // evaluate_alpha_vjp gate (src/primitives/Primitive3DGS.cuh:273); sigma >= 0 holds when active
+            const float v_alpha = (active && ov <= 0.999f) ? T0 * dv : 0.0f;
+            vT1 = ssr_fma(a, dv, vT1);
+            T1 = T0;
+            const float u = vis * v_alpha;
+            const float ux = u * dx, uy = u * dy;
+            const float uxx = ux * dx, uxy = ux * dy, uyy = uy * dy;
+            const float wr = vr * w, wg = vg * w, wb = vb * w, wd = vd * w;
+            // channels 0..9 = u, ux, uy, uxx, uxy, uyy, wr, wg, wb, wd
+            const float r0 = fold_pair<kDppRor8>(u, ux, b3), r1 = fold_pair<kDppRor8>(uy, uxx, b3),
+                        r2 = fold_pair<kDppRor8>(uxy, uyy, b3), r3 = fold_pair<kDppRor8>(wr, wg, b3),
+                        r4 = fold_pair<kDppRor8>(wb, wd, b3);
+            const float s0 = fold_pair<kDppHalfMirror>(r0, r1, b2), s1 = fold_pair<kDppHalfMirror>(r2, r3, b2),
+                        s2 = r4 + dpp_full<kDppHalfMirror>(r4);
+            const float t0 = fold_pair<kDppQuadXor2>(s0, s1, b1), t1 = s2 + dpp_full<kDppQuadXor2>(s2);
+            const float fin_sum = fold_pair<kDppQuadXor1>(t0, t1, b0);
+            const bool mine = chan >= 0 && in_list && ssr_isfinite(fin_sum) && fin_sum != 0.0f;
+            const bool clash = (((st < 64 ? clash_lo : clash_hi) >> (st & 63)) & 1ull) != 0;
+            float* cell = my_acc + k * 10 + (chan >= 0 ? chan : 0);
+            if (clash) { if (mine) atomicAdd(cell, fin_sum); }
+            else if (mine) *cell += fin_sum;
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0), as at the head of the loop
+    __syncthreads();
+    if (!first) flush();
+}
+
 }  // namespace ssr
 
 using namespace ssr;
@@ -393,6 +681,14 @@ extern "C" int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t strea
         default: SSR_BWD(D, M, SSR_ACCUM_NONE); break;           \
     }
 #define SSR_BWD_M(D) if (med) { SSR_BWD_A(D, true) } else { SSR_BWD_A(D, false) }
+    // The plain variant runs the row-granular kernel; SSR_RASTER_WAVE_VISITS=1 in the environment
+    // selects the one-wavefront-per-visit kernel instead (for comparisons).
+    static const bool wave_visits = getenv("SSR_RASTER_WAVE_VISITS") != nullptr;
+    if (p->dist_type == SSR_DIST_NONE && !med && p->accum_mode == SSR_ACCUM_NONE && !wave_visits) {
+        hipLaunchKernelGGL(raster_bwd_rows_kernel, grid, block, 0, st, *p, tw, th);
+        SSR_CHECK_LAUNCH("ssr_raster_bwd");
+        return 0;
+    }
     switch (p->dist_type) {
         case SSR_DIST_D: SSR_BWD_M(SSR_DIST_D) break;
         case SSR_DIST_RGB_D: SSR_BWD_M(SSR_DIST_RGB_D) break;

@@ -61,7 +61,7 @@ constexpr int kPackedRowFloats = 12;
 // Brings splat `g` into the staged form and computes its sub-tile footprint mask, either from a
 // packed row or by gathering the five screen arrays.
 __device__ __forceinline__ FragLds stage_fragment(const ssr_screen& s, const float* __restrict__ packed, int32_t g,
-                                                  float tile_x0, float tile_y0) {
+                                                  float tile_x0, float tile_y0, float* kk_out = nullptr) {
     FragLds f;
     float cut, kk;
     if (packed) {
@@ -93,7 +93,113 @@ __device__ __forceinline__ FragLds stage_fragment(const ssr_screen& s, const flo
         }
     }
     f.q2.z = __uint_as_float(hits);
+    if (kk_out) *kk_out = kk;
     return f;
+}
+
+// ---- 4x4-pixel blocks: the row-granular kernels ------------------------------------------------
+//
+// The row-granular variants of K7 / K8 cut a 16x16 tile into sixteen 4x4-pixel blocks. Block id =
+// 4 * sub_tile + quadrant (sub_tile m as above, quadrant = (y bit 2) * 2 + (x bit 2) inside it), so the
+// four 16-lane rows of wavefront m own the four blocks of sub-tile m. Every staged fragment carries a
+// 16-bit block mask in the upper half of the word that holds the 4-bit sub-tile mask: bit b is set when
+// the reference's sub-tile test passes for b's sub-tile AND the alpha >= 1/255 ellipse, grown by a
+// margin far above rounding, reaches the box of b's pixel centres -- a superset of the blocks in which
+// any pixel composites the splat, so the pixel results are those of the sub-tile walk.
+constexpr int kBlock = 4;
+constexpr int kBlocksPerTile = 16;
+
+// Block bits of the two block rows (bands of four pixel-centre lines) of tile half `half` (sub-tiles 2 half
+// and 2 half + 1): bit 4 (column >> 1) + 2 band + (column & 1), i.e. 4 (m & 1) + quadrant. Conservative test
+// of "the ellipse q(d) = a dx^2 + 2 b dx dy + c dy^2 <= 1 + margin reaches a pixel centre of the block": the
+// part of the ellipse inside the band dy in [Y0, Y1] is convex, so its extent in x is one interval --
+// between the band's two end lines, or out to the ellipse's extreme points when those lie inside the band --
+// and a block is reached exactly when its centres' x range meets that interval. The margin (1e-3) is far
+// above the rounding of this arithmetic and of the alpha evaluation; a degenerate conic keeps every block.
+__device__ __forceinline__ uint32_t block_bits_of_half(float a, float b, float c, float x, float y, float tile_x0,
+                                                       float tile_y0, int half) {
+    const float t = 1.001f;
+    const float det = a * c - b * b;
+    if (!(det > 0.0f) || !(a > 0.0f) || !(c > 0.0f)) return 0xFFu;
+    const float inv_det = __builtin_amdgcn_rcpf(det), inv_a = __builtin_amdgcn_rcpf(a);
+    const float ymax = __builtin_amdgcn_sqrtf((a * t) * inv_det) * 1.0001f;
+    const float xmax = __builtin_amdgcn_sqrtf((c * t) * inv_det) * 1.0001f;
+    const float y_r = -(b * __builtin_amdgcn_rcpf(c)) * xmax;   // dy at which dx is largest; -y_r where it is smallest
+    const float nba = -b * inv_a, at = a * t;
+    uint32_t bits = 0;
+#pragma unroll
+    for (int band = 0; band < 2; band++) {
+        const float Y0 = (tile_y0 + (float)(half * kMicro + band * kBlock) + 0.5f) - y, Y1 = Y0 + (float)(kBlock - 1);
+        const float yl = __builtin_fmaxf(Y0, -ymax), yh = __builtin_fminf(Y1, ymax);
+        if (!(yl <= yh)) continue;
+        const float hl = __builtin_amdgcn_sqrtf(__builtin_fmaxf(ssr_fma(-det * yl, yl, at), 0.0f)) * inv_a * 1.0001f + 1e-4f;
+        const float hh = __builtin_amdgcn_sqrtf(__builtin_fmaxf(ssr_fma(-det * yh, yh, at), 0.0f)) * inv_a * 1.0001f + 1e-4f;
+        const float cl = nba * yl, ch = nba * yh;
+        float xr = __builtin_fmaxf(cl + hl, ch + hh), xl = __builtin_fminf(cl - hl, ch - hh);
+        if (yl <= y_r && y_r <= yh) xr = xmax;
+        if (yl <= -y_r && -y_r <= yh) xl = -xmax;
+#pragma unroll
+        for (int col = 0; col < 4; col++) {
+            const float X0 = (tile_x0 + (float)(col * kBlock) + 0.5f) - x;
+            if (X0 <= xr && X0 + (float)(kBlock - 1) >= xl) bits |= 1u << (4 * (col >> 1) + 2 * band + (col & 1));
+        }
+    }
+    return bits;
+}
+
+// Stages splat g for the row-granular backward, where two threads share a fragment: thread `half`
+// (0 / 1) runs the reference's sub-tile test for sub-tiles 2 half and 2 half + 1 and the block tests of
+// those that pass; it returns their eight block bits (bit 4 (m & 1) + quadrant). The fragment record
+// itself is the same from either thread.
+__device__ __forceinline__ FragLds stage_fragment_half(const ssr_screen& s, const float* __restrict__ packed, int32_t g,
+                                                       float tile_x0, float tile_y0, int half, uint32_t& bits8) {
+    FragLds f;
+    float cut, kk;
+    if (packed) {
+        const float4* row = reinterpret_cast<const float4*>(packed) + 3 * (int64_t)g;
+        f.q0 = row[0]; f.q1 = row[1];
+        const float4 r2 = row[2];
+        f.q2 = make_float4(r2.x, r2.y, 0.0f, r2.z);
+        cut = r2.z; kk = r2.w;
+    } else {
+        const float2 xy = *reinterpret_cast<const float2*>(s.xy + 2 * (int64_t)g);
+        const float* cn = s.conic + 3 * (int64_t)g;
+        const float opac = s.opac[g];
+        const float* rg = s.rgb + 3 * (int64_t)g;
+        fragment_constants(opac, cut, kk);
+        f.q0 = make_float4(xy.x, xy.y, 0.5f * cn[0], cn[1]);
+        f.q1 = make_float4(0.5f * cn[2], opac, rg[0], rg[1]);
+        f.q2 = make_float4(rg[2], s.depth[g], 0.0f, cut);
+    }
+    bits8 = 0;
+    if (f.q1.y > kAlphaThreshold) {
+        const float ic[3] = {(f.q0.z + f.q0.z) * kk, f.q0.w * kk, (f.q1.x + f.q1.x) * kk};
+        const float x = f.q0.x, y = f.q0.y;
+        uint32_t sub = 0;   // the reference's test for the two sub-tiles of this half
+#pragma unroll
+        for (int mm = 0; mm < 2; mm++) {
+            const int m = 2 * half + mm;
+            const float sx0 = tile_x0 + (float)((m & 1) * kMicro), sy0 = tile_y0 + (float)((m >> 1) * kMicro);
+            if (ellipse_box_overlap(ic, sx0 - x, (sx0 + (float)kMicro) - x, sy0 - y, (sy0 + (float)kMicro) - y)) sub |= 0xFu << (4 * mm);
+        }
+        if (sub) bits8 = sub & block_bits_of_half(ic[0], ic[1], ic[2], x, y, tile_x0, tile_y0, half);
+    }
+    return f;
+}
+
+// Adds the block mask to a fragment staged by stage_fragment (bits 16..31 of the mask word; bit 4 m + quadrant).
+__device__ __forceinline__ void add_block_mask(FragLds& f, float kk, float tile_x0, float tile_y0) {
+    const uint32_t hits = __float_as_uint(f.q2.z);
+    uint32_t blocks = 0;
+    if (hits) {
+        const float a = (f.q0.z + f.q0.z) * kk, b = f.q0.w * kk, c = (f.q1.x + f.q1.x) * kk;
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const uint32_t sub = ((hits >> (2 * half)) & 1u ? 0x0Fu : 0u) | ((hits >> (2 * half + 1)) & 1u ? 0xF0u : 0u);
+            if (sub) blocks |= (sub & block_bits_of_half(a, b, c, f.q0.x, f.q0.y, tile_x0, tile_y0, half)) << (8 * half);
+        }
+    }
+    f.q2.z = __uint_as_float(hits | (blocks << 16));
 }
 
 // exp(x) for x in [-87, 0] (and NaN): the same operations as ssr_exp() on that range, where its

@@ -7,6 +7,7 @@
 // WITHOUT adding this splat; else accumulate rgb*alpha*T, depth*alpha*T and remember the sorted
 // index. Outputs rgb, depth / max(1-T, 1e-10), T and last_id.
 #include "raster_device.h"
+#include <stdlib.h>
 
 namespace ssr {
 
@@ -117,6 +118,116 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_kernel(ssr_raster_fwd
     }
 }
 
+// The row-granular plain kernel: the same per-pixel arithmetic, but each 16-lane row of a wavefront
+// holds one 4x4-pixel block and walks its own list of the staged fragments whose block bit is set
+// (raster_device.h), instead of all 64 lanes visiting every fragment that reaches the 8x8 sub-tile.
+// Lists are built per batch by the wavefront that walks them (ballot + rank, slot numbers as bytes).
+__global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raster_fwd_params P, int tile_w, int tile_h) {
+    __shared__ FragLds frags[kBatch];
+    __shared__ uint8_t s_list[kBlocksPerTile * kBatch + 16];
+    const int n_tiles = tile_w * tile_h * (P.num_images > 1 ? P.num_images : 1);
+    const int tile = xcd_tile_of(blockIdx.x, n_tiles);
+    if (tile >= n_tiles) return;
+    const int tid = threadIdx.x, lane = tid & 63, mt = tid >> 6, row = lane >> 4, l16 = lane & 15;
+    const int gy = tile / tile_w, tx = tile - gy * tile_w;
+    const int img = gy / tile_h, ty = gy - img * tile_h;
+    const int j = tx * kTile + (mt & 1) * kMicro + (row & 1) * kBlock + (l16 & 3);
+    const int i = ty * kTile + (mt >> 1) * kMicro + (row >> 1) * kBlock + (l16 >> 2);
+    const float px = (float)j + 0.5f, py = (float)i + 0.5f;
+    const bool inside = (uint32_t)i < P.height && (uint32_t)j < P.width;
+    bool done = !inside;
+
+    const int32_t range_start = P.tile_offsets[tile];
+    const int32_t range_end = (tile == n_tiles - 1) ? (int32_t)P.n_isects : P.tile_offsets[tile + 1];
+    float T = 1.0f, cr = 0.f, cg = 0.f, cb = 0.f, cd = 0.f;
+    uint32_t cur_idx = 0;
+    const float tile_x0 = (float)(tx * kTile), tile_y0 = (float)(ty * kTile);
+    const uint8_t* my_list = s_list + (4 * mt + row) * kBatch;
+
+    for (int32_t batch_start = range_start; batch_start < range_end; batch_start += kBatch) {
+        // all pixels of the tile finished: stop (this barrier also fences reuse of the LDS batch)
+        if (__syncthreads_count(done) >= kRasterBlock) break;
+        const int32_t idx = batch_start + tid;
+        if (idx < range_end) {
+            float kk;
+            FragLds f = stage_fragment(P.screen, P.packed_rows, P.flatten_ids[idx], tile_x0, tile_y0, &kk);
+            add_block_mask(f, kk, tile_x0, tile_y0);
+            frags[tid] = f;
+        } else {
+            frags[tid].q2 = make_float4(0.f, 0.f, 0.f, 0.f);   // empty masks
+        }
+        __syncthreads();
+        const int n_batch = min(kBatch, range_end - batch_start);
+        // a row whose sixteen pixels are finished needs no list
+        const uint64_t live = __ballot(!done);
+        const bool row_live[4] = {(live & 0xFFFFull) != 0, (live & 0xFFFF0000ull) != 0, (live & 0xFFFF00000000ull) != 0,
+                                  (live & 0xFFFF000000000000ull) != 0};
+        int cnt[4] = {0, 0, 0, 0};
+        if (live != 0ull) {
+            for (int c = 0; c * 64 < n_batch; c++) {
+                const int slot = c * 64 + lane;
+                const uint32_t bits = __float_as_uint(frags[slot].q2.z) >> (16 + 4 * mt);
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    if (!row_live[r]) continue;
+                    const bool in = ((bits >> r) & 1u) != 0;
+                    const uint64_t bal = __ballot(in);
+                    if (in) s_list[(4 * mt + r) * kBatch + cnt[r] + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(bal >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)bal, 0u))] = (uint8_t)slot;
+                    cnt[r] += __builtin_popcountll(bal);
+                }
+            }
+        }
+        // the lists are written and read by this wavefront only: order its LDS accesses, no workgroup barrier
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        const int my_cnt = row == 0 ? cnt[0] : row == 1 ? cnt[1] : row == 2 ? cnt[2] : cnt[3];
+        const int n_steps = max(max(cnt[0], cnt[1]), max(cnt[2], cnt[3]));
+        // Two-deep software pipeline: the list byte of step st + 2 and the fragment of step st + 1 are in
+        // flight while step st computes, so that the two dependent LDS latencies hide behind arithmetic.
+        int k_next = 0 < my_cnt ? (int)my_list[0] : 0;
+        int k_next2 = 1 < my_cnt ? (int)my_list[1] : 0;
+        float4 n0 = frags[k_next].q0, n1 = frags[k_next].q1;
+        float2 n2a = make_float2(frags[k_next].q2.x, frags[k_next].q2.y);
+        float n2w = frags[k_next].q2.w;
+#pragma unroll 2
+        for (int st = 0; st < n_steps; st++) {
+            if (__ballot(!done) == 0ull) break;   // this sub-tile is finished
+            const bool in_list = st < my_cnt;
+            const int k = k_next;
+            const float4 q0 = n0, q1 = n1;
+            const float4 q2 = make_float4(n2a.x, n2a.y, 0.0f, n2w);
+            k_next = k_next2;
+            k_next2 = st + 2 < my_cnt ? (int)my_list[st + 2] : 0;
+            n0 = frags[k_next].q0; n1 = frags[k_next].q1;
+            n2a = make_float2(frags[k_next].q2.x, frags[k_next].q2.y);
+            n2w = frags[k_next].q2.w;
+            float dx, dy, vis, sigma;
+            const float alpha = eval_alpha_fast(q0, q1, q2.w, px, py, dx, dy, vis, sigma);
+            if (!done && in_list && alpha > kAlphaThreshold) {
+                const float next_T = T * (1.0f - alpha);
+                if (next_T > kTransmitThreshold) {
+                    const float w = alpha * T;
+                    cr = ssr_fma(q1.z, w, cr); cg = ssr_fma(q1.w, w, cg); cb = ssr_fma(q2.x, w, cb);
+                    cd = ssr_fma(q2.y, w, cd);
+                    cur_idx = (uint32_t)(batch_start + k);
+                    T = next_T;
+                } else {
+                    done = true;
+                }
+            }
+        }
+    }
+    if (inside) {
+        const int64_t pid = ((int64_t)img * P.height + i) * P.width + j;
+        P.render_T[pid] = T;
+        const float invW = 1.0f / ssr_max(1.0f - T, 1e-10f);
+        float* o = P.render_rgb + 3 * pid;
+        o[0] = cr; o[1] = cg; o[2] = cb;
+        P.render_depth[pid] = cd * invW;
+        P.last_ids[pid] = (int32_t)cur_idx;
+    }
+}
+
 }  // namespace ssr
 
 using namespace ssr;
@@ -149,6 +260,14 @@ extern "C" int ssr_raster_fwd(const ssr_raster_fwd_params* p, ssr_stream_t strea
     hipStream_t s = as_stream(stream);
 #define SSR_FWD(D, M) hipLaunchKernelGGL((raster_fwd_kernel<D, M>), grid, block, 0, s, *p, tw, th)
     const bool med = p->render_median != nullptr;
+    // The plain variant runs the row-granular kernel; SSR_RASTER_WAVE_VISITS=1 in the environment
+    // selects the one-wavefront-per-visit kernel instead (for comparisons).
+    static const bool wave_visits = getenv("SSR_RASTER_WAVE_VISITS") != nullptr;
+    if (p->dist_type == SSR_DIST_NONE && !med && !wave_visits) {
+        hipLaunchKernelGGL(raster_fwd_rows_kernel, grid, block, 0, s, *p, tw, th);
+        SSR_CHECK_LAUNCH("ssr_raster_fwd");
+        return 0;
+    }
     switch (p->dist_type) {
         case SSR_DIST_D: if (med) SSR_FWD(SSR_DIST_D, true); else SSR_FWD(SSR_DIST_D, false); break;
         case SSR_DIST_RGB_D: if (med) SSR_FWD(SSR_DIST_RGB_D, true); else SSR_FWD(SSR_DIST_RGB_D, false); break;

@@ -191,6 +191,18 @@ def raster_fwd(n, scr, w, h, offsets, flat, dist_type=0, median=False):
     return o
 
 
+def raster_lane_stats(scr, w, h, offsets, flat, last_ids):
+    """Lane statistics of the compositing backward: visits per block size and compositing pairs."""
+    out = np.zeros(7, np.int64)
+    last_ids = np.ascontiguousarray(last_ids, np.int32)
+    lib().or_raster_lane_stats(_p(scr["xy"]), _p(scr["depth"]), _p(scr["conic"]), _p(scr["opac"]), _p(scr["rgb"]),
+                               C.c_uint32(w), C.c_uint32(h), _p(offsets), _p(flat), C.c_int64(flat.size),
+                               _p(last_ids), _p(out))
+    v8, v4, v2, pairs, p8, p4, p2 = (int(x) for x in out)
+    return dict(visits={8: v8, 4: v4, 2: v2}, productive={8: p8, 4: p4, 2: p2}, pairs=pairs,
+                utilisation={8: pairs / max(1, 64 * v8), 4: pairs / max(1, 16 * v4), 2: pairs / max(1, 4 * v2)})
+
+
 def raster_bwd(n, scr, w, h, offsets, flat, fwd, v_rgb, v_depth, v_T, with_abs=True, dist_type=0,
                v_dist_rgb=None, v_dist_depth=None, v_median=None, accum_mode=0, accum_map=None,
                gaussian_ids=None, n_world=None):
