@@ -564,64 +564,90 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
                 if (c == 0) clash_lo = m; else clash_hi = m;
             }
         }
-        // Two-deep software pipeline: the list byte of step st + 2 and the fragment of step st + 1 are in
-        // flight while step st computes, so that the two dependent LDS latencies hide behind arithmetic.
-        int k_next = 0 < my_cnt ? (int)my_list[0] : 0;
-        int k_next2 = 1 < my_cnt ? (int)my_list[1] : 0;
-        float4 n0 = frags[k_next].q0, n1 = frags[k_next].q1;
-        float2 n2a = make_float2(frags[k_next].q2.x, frags[k_next].q2.y);
-        float n2w = frags[k_next].q2.w;
-#pragma unroll 2
-        for (int st = 0; st < n_steps; st++) {
+        // One step of a row: fragment k (registers q*) against the row's sixteen pixels.
+        auto step = [&](int st, int k, const float4& q0, const float4& q1, const float2& q2, float cut) {
             const bool in_list = st < my_cnt;
-            const int k = k_next;
-            const float4 q0 = n0, q1 = n1;
-            const float4 q2 = make_float4(n2a.x, n2a.y, 0.0f, n2w);
-            k_next = k_next2;
-            k_next2 = st + 2 < my_cnt ? (int)my_list[st + 2] : 0;
-            n0 = frags[k_next].q0; n1 = frags[k_next].q1;
-            n2a = make_float2(frags[k_next].q2.x, frags[k_next].q2.y);
-            n2w = frags[k_next].q2.w;
             const int32_t sorted_idx = hi - k;
             const float dx = q0.x - px, dy = q0.y - py;
             const float sigma = ssr_fma(q0.z * dx, dx, ssr_fma(q1.x * dy, dy, (q0.w * dx) * dy));
-            const bool in_range = !(sigma < 0.f || sigma > q2.w);
+            const bool in_range = !(sigma < 0.f || sigma > cut);
             float vis = in_range ? __builtin_amdgcn_exp2f(sigma * -1.44269504088896341f) : 0.0f;
             float ov = q1.y * vis;
             const bool near_edge = in_list & ((ssr_fabs(ov - kAlphaThreshold) <= 1.6e-7f) | (ssr_fabs(ov - 0.999f) <= 4e-5f));
-            if (__ballot(near_edge) != 0ull) {   // decisions exactly as the forward took them
+            if (__builtin_amdgcn_ballot_w64(near_edge) != 0ull) {   // decisions exactly as the forward took them
                 vis = in_range ? exp_neg_small(-sigma) : 0.0f;
                 ov = q1.y * vis;
             }
             const float alpha = ssr_min(0.999f, ov);
-            const bool active = in_list && sorted_idx <= bin_final && alpha > kAlphaThreshold;
-            if (__ballot(active) == 0ull) continue;
-            // inactive lanes run with alpha = 0 and v_alpha = 0: T and v_T unchanged, every term zero
-            const float a = active ? alpha : 0.0f;
-            const float T0 = T1 * __builtin_amdgcn_rcpf(1.0f - a);
-            const float dv = ssr_fma(q2.y, vd, ssr_fma(q2.x, vb, ssr_fma(q1.w, vg, q1.z * vr))) - vT1;
-            const float w = a * T0;
-            // evaluate_alpha_vjp gate (src/primitives/Primitive3DGS.cuh:273); sigma >= 0 holds when active
-            const float v_alpha = (active && ov <= 0.999f) ? T0 * dv : 0.0f;
-            vT1 = ssr_fma(a, dv, vT1);
-            T1 = T0;
-            const float u = vis * v_alpha;
-            const float ux = u * dx, uy = u * dy;
-            const float uxx = ux * dx, uxy = ux * dy, uyy = uy * dy;
-            const float wr = vr * w, wg = vg * w, wb = vb * w, wd = vd * w;
-            // channels 0..9 = u, ux, uy, uxx, uxy, uyy, wr, wg, wb, wd
-            const float r0 = fold_pair<kDppRor8>(u, ux, b3), r1 = fold_pair<kDppRor8>(uy, uxx, b3),
-                        r2 = fold_pair<kDppRor8>(uxy, uyy, b3), r3 = fold_pair<kDppRor8>(wr, wg, b3),
-                        r4 = fold_pair<kDppRor8>(wb, wd, b3);
-            const float s0 = fold_pair<kDppHalfMirror>(r0, r1, b2), s1 = fold_pair<kDppHalfMirror>(r2, r3, b2),
-                        s2 = r4 + dpp_full<kDppHalfMirror>(r4);
-            const float t0 = fold_pair<kDppQuadXor2>(s0, s1, b1), t1 = s2 + dpp_full<kDppQuadXor2>(s2);
-            const float fin_sum = fold_pair<kDppQuadXor1>(t0, t1, b0);
-            const bool mine = chan >= 0 && in_list && ssr_isfinite(fin_sum) && fin_sum != 0.0f;
-            const bool clash = (((st < 64 ? clash_lo : clash_hi) >> (st & 63)) & 1ull) != 0;
-            float* cell = my_acc + k * 10 + (chan >= 0 ? chan : 0);
-            if (clash) { if (mine) atomicAdd(cell, fin_sum); }
-            else if (mine) *cell += fin_sum;
+            const bool active = in_list & (sorted_idx <= bin_final) & (alpha > kAlphaThreshold);
+            if (__builtin_amdgcn_ballot_w64(active) != 0ull) {
+                // inactive lanes run with alpha = 0 and v_alpha = 0: T and v_T unchanged, every term zero
+                const float a = active ? alpha : 0.0f;
+                const float T0 = T1 * __builtin_amdgcn_rcpf(1.0f - a);
+                const float dv = ssr_fma(q2.y, vd, ssr_fma(q2.x, vb, ssr_fma(q1.w, vg, q1.z * vr))) - vT1;
+                const float w = a * T0;
+                // evaluate_alpha_vjp gate (src/primitives/Primitive3DGS.cuh:273); sigma >= 0 holds when active
+                const float v_alpha = (active & (ov <= 0.999f)) ? T0 * dv : 0.0f;
+                vT1 = ssr_fma(a, dv, vT1);
+                T1 = T0;
+                const float u = vis * v_alpha;
+                const float ux = u * dx, uy = u * dy;
+                const float uxx = ux * dx, uxy = ux * dy, uyy = uy * dy;
+                const float wr = vr * w, wg = vg * w, wb = vb * w, wd = vd * w;
+                // Channels 0..9 = u, ux, uy, uxx, uxy, uyy, wr, wg, wb, wd. The first two levels of the transposing
+                // reduction as bank-masked DPP adds (one instruction per channel and level, against three per pair with
+                // selects): lanes 0-7 of a row take the even channel of a pair, lanes 8-15 the odd one; then lane groups
+                // of four likewise with the half-mirror pairing. s_nop covers the two wait states a DPP read needs
+                // after a write of its source by the instruction before; inside the block the reads trail the writes.
+                float r0, r1, r2, r3, r4, s0, s1, s2;
+                asm volatile(
+                    "s_nop 1\n\t"
+                    "v_add_f32_dpp %0, %8, %8 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+                    "v_add_f32_dpp %0, %9, %9 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                    "v_add_f32_dpp %1, %10, %10 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+                    "v_add_f32_dpp %1, %11, %11 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                    "v_add_f32_dpp %2, %12, %12 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+                    "v_add_f32_dpp %2, %13, %13 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                    "v_add_f32_dpp %3, %14, %14 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+                    "v_add_f32_dpp %3, %15, %15 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                    "v_add_f32_dpp %4, %16, %16 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+                    "v_add_f32_dpp %4, %17, %17 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                    "v_add_f32_dpp %5, %0, %0 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+                    "v_add_f32_dpp %5, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+                    "v_add_f32_dpp %6, %2, %2 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+                    "v_add_f32_dpp %6, %3, %3 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+                    "v_add_f32_dpp %7, %4, %4 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+                    : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3), "=&v"(r4), "=&v"(s0), "=&v"(s1), "=&v"(s2)
+                    : "v"(u), "v"(ux), "v"(uy), "v"(uxx), "v"(uxy), "v"(uyy), "v"(wr), "v"(wg), "v"(wb), "v"(wd));
+                const float t0 = fold_pair<kDppQuadXor2>(s0, s1, b1), t1 = s2 + dpp_full<kDppQuadXor2>(s2);
+                const float fin_sum = fold_pair<kDppQuadXor1>(t0, t1, b0);
+                const bool mine = (chan >= 0) & in_list & ssr_isfinite(fin_sum) & (fin_sum != 0.0f);
+                const bool clash = (((st < 64 ? clash_lo : clash_hi) >> (st & 63)) & 1ull) != 0;
+                float* cell = my_acc + k * 10 + (chan >= 0 ? chan : 0);
+                if (clash) { if (mine) atomicAdd(cell, fin_sum); }
+                else if (mine) *cell += fin_sum;
+            }
+        };
+        // Software pipeline, two steps per trip: list bytes run two steps ahead of their use and the fragment of the
+        // next step loads while the current one computes, so that the two dependent LDS latencies hide behind
+        // arithmetic; the two fragment register sets alternate, so nothing is copied between steps.
+        auto list_at = [&](int st) { return st < my_cnt ? (int)my_list[st] : 0; };
+        int k0 = list_at(0), k1 = list_at(1), k2 = list_at(2);
+        float4 a0 = frags[k0].q0, a1 = frags[k0].q1;
+        float2 a2 = make_float2(frags[k0].q2.x, frags[k0].q2.y);
+        float aw = frags[k0].q2.w;
+        for (int st = 0; st < n_steps; st += 2) {
+            const float4 c0 = frags[k1].q0, c1 = frags[k1].q1;
+            const float2 c2 = make_float2(frags[k1].q2.x, frags[k1].q2.y);
+            const float cw = frags[k1].q2.w;
+            const int k3 = list_at(st + 3);
+            step(st, k0, a0, a1, a2, aw);
+            a0 = frags[k2].q0; a1 = frags[k2].q1;
+            a2 = make_float2(frags[k2].q2.x, frags[k2].q2.y);
+            aw = frags[k2].q2.w;
+            const int k4 = list_at(st + 4);
+            if (st + 1 < n_steps) step(st + 1, k1, c0, c1, c2, cw);
+            k0 = k2; k1 = k3; k2 = k4;
         }
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0), as at the head of the loop

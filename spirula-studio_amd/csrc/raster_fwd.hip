@@ -182,39 +182,41 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raste
         __builtin_amdgcn_wave_barrier();
         const int my_cnt = row == 0 ? cnt[0] : row == 1 ? cnt[1] : row == 2 ? cnt[2] : cnt[3];
         const int n_steps = max(max(cnt[0], cnt[1]), max(cnt[2], cnt[3]));
-        // Two-deep software pipeline: the list byte of step st + 2 and the fragment of step st + 1 are in
-        // flight while step st computes, so that the two dependent LDS latencies hide behind arithmetic.
-        int k_next = 0 < my_cnt ? (int)my_list[0] : 0;
-        int k_next2 = 1 < my_cnt ? (int)my_list[1] : 0;
-        float4 n0 = frags[k_next].q0, n1 = frags[k_next].q1;
-        float2 n2a = make_float2(frags[k_next].q2.x, frags[k_next].q2.y);
-        float n2w = frags[k_next].q2.w;
-#pragma unroll 2
-        for (int st = 0; st < n_steps; st++) {
-            if (__ballot(!done) == 0ull) break;   // this sub-tile is finished
-            const bool in_list = st < my_cnt;
-            const int k = k_next;
-            const float4 q0 = n0, q1 = n1;
-            const float4 q2 = make_float4(n2a.x, n2a.y, 0.0f, n2w);
-            k_next = k_next2;
-            k_next2 = st + 2 < my_cnt ? (int)my_list[st + 2] : 0;
-            n0 = frags[k_next].q0; n1 = frags[k_next].q1;
-            n2a = make_float2(frags[k_next].q2.x, frags[k_next].q2.y);
-            n2w = frags[k_next].q2.w;
+        // One step of a row: fragment k (registers q*) against the row's sixteen pixels, branch-free
+        auto step = [&](int st, int k, const float4& q0, const float4& q1, const float2& q2, float cut) {
             float dx, dy, vis, sigma;
-            const float alpha = eval_alpha_fast(q0, q1, q2.w, px, py, dx, dy, vis, sigma);
-            if (!done && in_list && alpha > kAlphaThreshold) {
-                const float next_T = T * (1.0f - alpha);
-                if (next_T > kTransmitThreshold) {
-                    const float w = alpha * T;
-                    cr = ssr_fma(q1.z, w, cr); cg = ssr_fma(q1.w, w, cg); cb = ssr_fma(q2.x, w, cb);
-                    cd = ssr_fma(q2.y, w, cd);
-                    cur_idx = (uint32_t)(batch_start + k);
-                    T = next_T;
-                } else {
-                    done = true;
-                }
-            }
+            const float alpha = eval_alpha_fast(q0, q1, cut, px, py, dx, dy, vis, sigma);
+            const bool hit = !done & (st < my_cnt) & (alpha > kAlphaThreshold);
+            const float next_T = T * (1.0f - alpha);
+            const bool keep = hit & (next_T > kTransmitThreshold);
+            const float w = keep ? alpha * T : 0.0f;   // a fragment that is not composited adds zero
+            cr = ssr_fma(q1.z, w, cr); cg = ssr_fma(q1.w, w, cg); cb = ssr_fma(q2.x, w, cb);
+            cd = ssr_fma(q2.y, w, cd);
+            cur_idx = keep ? (uint32_t)(batch_start + k) : cur_idx;
+            T = keep ? next_T : T;
+            done = done | (hit & !keep);
+        };
+        // Software pipeline, two steps per trip: list bytes run two steps ahead of their use and the fragment of the
+        // next step loads while the current one computes, so that the two dependent LDS latencies hide behind
+        // arithmetic; the two fragment register sets alternate, so nothing is copied between steps.
+        auto list_at = [&](int st) { return st < my_cnt ? (int)my_list[st] : 0; };
+        int k0 = list_at(0), k1 = list_at(1), k2 = list_at(2);
+        float4 a0 = frags[k0].q0, a1 = frags[k0].q1;
+        float2 a2 = make_float2(frags[k0].q2.x, frags[k0].q2.y);
+        float aw = frags[k0].q2.w;
+        for (int st = 0; st < n_steps; st += 2) {
+            if (__builtin_amdgcn_ballot_w64(!done) == 0ull) break;   // this sub-tile is finished
+            const float4 c0 = frags[k1].q0, c1 = frags[k1].q1;
+            const float2 c2 = make_float2(frags[k1].q2.x, frags[k1].q2.y);
+            const float cw = frags[k1].q2.w;
+            const int k3 = list_at(st + 3);
+            step(st, k0, a0, a1, a2, aw);
+            a0 = frags[k2].q0; a1 = frags[k2].q1;
+            a2 = make_float2(frags[k2].q2.x, frags[k2].q2.y);
+            aw = frags[k2].q2.w;
+            const int k4 = list_at(st + 4);
+            step(st + 1, k1, c0, c1, c2, cw);   // beyond the lists every row is out of its list: nothing happens
+            k0 = k2; k1 = k3; k2 = k4;
         }
     }
     if (inside) {
