@@ -57,32 +57,58 @@ def tile_need(offsets, last_ids, n_isects, width, height):
     return int(need.sum())
 
 
-def cpu_baseline(pkg, cfg, budget_s=20.0):
-    """The CPU oracle on this host's cores, on a bounded sample of the same workload."""
+def _time_oracle(oracle_lib, sc, threads, min_iters, budget_s):
+    """Seconds per iteration of the CPU oracle's forward+backward on `threads` threads, and its last result."""
+    oracle_lib.lib().or_set_num_threads(threads)
+    t0 = time.time()
+    iters, res = 0, None
+    while iters < min_iters or (time.time() - t0 < budget_s and iters < 20):
+        res = oracle_lib.pipeline(sc)
+        iters += 1
+        if time.time() - t0 > 3 * budget_s:
+            break
+    return (time.time() - t0) / iters, iters, res
+
+
+def lavapipe_status():
+    """The baseline BASELINE.json asks for is the reference's Vulkan path on Mesa lavapipe. It needs the reference
+    tree, slangc and a Vulkan loader with the lavapipe ICD on this host; say what is missing instead of a number."""
+    import glob
+    import shutil
+    missing = []
+    if not os.path.isdir("/root/reference/src/backend/vulkan"):
+        missing.append("the reference source tree (only this repository travels to the GPU box)")
+    if not shutil.which("slangc"):
+        missing.append("slangc (the reference compiles its shaders to SPIR-V at build time and commits none)")
+    if not (glob.glob("/usr/lib/x86_64-linux-gnu/libvulkan.so*") or glob.glob("/usr/lib64/libvulkan.so*")):
+        missing.append("a Vulkan loader")
+    if not (glob.glob("/usr/share/vulkan/icd.d/lvp_icd*.json") or glob.glob("/etc/vulkan/icd.d/lvp_icd*.json")):
+        missing.append("the lavapipe ICD")
+    return "unavailable: missing " + "; ".join(missing) if missing else "present but not driven by this harness"
+
+
+def cpu_baseline(pkg, cfg, sc):
+    """The CPU oracle (this repository's restatement, not the reference implementation) on this host's cores, on
+    the stated workload itself: whole iterations of configuration `cfg` on every core; for the headline
+    configuration also one iteration on a single thread and configuration 1 on every core. Returns the JSON
+    object and K_f, the number of (splat, tile) pairs the forward needs, which only the oracle records."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import oracle_lib
-    full = pkg.scenes.CONFIGS[cfg]
-    # sample: the same scene at 1/8 of the splats and 1/8 of the pixels keeps the per-tile load
-    frac = 8
-    n = max(1000, full["n"] // frac)
-    w = max(64, int(full["w"] / frac ** 0.5) // 16 * 16)
-    h = max(64, int(full["h"] / frac ** 0.5) // 16 * 16)
-    sc = pkg.scenes.make_scene(cfg, n=n, width=w, height=h)
-    oracle_lib.lib()
-    cores = oracle_lib.lib().or_num_threads()
-    t0 = time.time()
-    iters = 0
-    while True:
-        oracle_lib.pipeline(sc)
-        iters += 1
-        if time.time() - t0 > budget_s or iters >= 50:
-            break
-    dt = (time.time() - t0) / iters
-    # whole-config rate estimated from the sample: work scales with splats and with pixels
-    est = 1.0 / (dt * frac)
-    return {"value": est, "unit": "iters/s", "cores": cores, "kind": "port",
-            "sample": f"{iters} iteration(s) of config {cfg} at N={n}, {w}x{h} (1/{frac} of the splats and of "
-                      f"the pixels): {dt * 1e3:.1f} ms each; value = sample rate / {frac}"}
+    L = oracle_lib.lib()
+    cores = L.or_num_threads()
+    dt, iters, res = _time_oracle(oracle_lib, sc, cores, 3 if sc.n <= 1_000_000 else 1, 10.0)
+    out = {"value": 1.0 / dt, "unit": "iters/s", "cores": cores, "kind": "port",
+           "sample": f"{iters} whole iteration(s) of config {cfg} (N={sc.n}, {sc.width}x{sc.height}) on {cores} threads: "
+                     f"{dt * 1e3:.0f} ms each; own CPU oracle, not the reference implementation",
+           "lavapipe": lavapipe_status()}
+    if cfg == 2:
+        dt1, it1, _ = _time_oracle(oracle_lib, sc, 1, 1, 0.0)
+        out["single_thread"] = {"value": 1.0 / dt1, "unit": "iters/s", "cores": 1, "sample": f"{it1} iteration(s), {dt1 * 1e3:.0f} ms each"}
+        sc1 = pkg.scenes.make_scene(1)
+        dtc, itc, _ = _time_oracle(oracle_lib, sc1, cores, 3, 3.0)
+        out["config1"] = {"value": 1.0 / dtc, "unit": "iters/s", "cores": cores, "sample": f"{itc} iteration(s) of config 1, {dtc * 1e3:.0f} ms each"}
+    L.or_set_num_threads(cores)
+    return out, int(res["fwd"]["K_f"])
 
 
 def main():
@@ -245,7 +271,15 @@ def main():
     for c in range(ncam):   # positions in offsets and last_ids are absolute, so each image is taken with its own end
         end = int(offs[(c + 1) * T1]) if c + 1 < ncam else K
         K_b += tile_need(offs[c * T1:(c + 1) * T1], last[c * P1:(c + 1) * P1], end, sc.width, sc.height)
-    K_f = K_b   # lower bound of the forward's need (it also reads the splat that ends a pixel)
+    # K_f, the pairs the forward needs (it also reads the splat that ends a pixel), is recorded by the CPU oracle only:
+    # taken from the cpu_baseline leg when that runs on this very scene, else bounded below by K_b
+    K_f, cpu = K_b, None
+    plain_scene = not (args.fisheye or args.lens != "none" or args.mip or ncam > 1 or args.n)
+    if not args.no_cpu_baseline:
+        if plain_scene and not (args.fused_optimizer and args.quantization_level == 1):
+            cpu, K_f = cpu_baseline(pkg, cfg, sc)
+        else:
+            cpu, _ = cpu_baseline(pkg, cfg, pkg.scenes.make_scene(cfg))
     S = 180 if sc.sh_codec == 0 else (47 if sc.sh_codec == 3 else 45 + 8 * 45 / 256)
     tile_bits = max(T - 1, 0).bit_length()
     tile_sort = native and not args.whole_key_sort
@@ -278,7 +312,7 @@ def main():
                                f"{['pinhole', 'fisheye', 'equisolid', 'equirectangular'][sc.camera_model]}"
                                f"{'' if not sc.distortion else ' + ' + args.lens + ' lens'}, SH3 "
                                f"{['fp32', 'ref-q8', 'ref-q16', 'int8*fp16scale'][sc.sh_codec]}, tile 16x16, seed {pkg.scenes.CONFIGS[cfg]['seed']:#x}",
-                   "visible": V, "n_isects": K, "K_b": K_b, "tiles": T, "pixels": P,
+                   "visible": V, "n_isects": K, "K_f": K_f, "K_b": K_b, "tiles": T, "pixels": P,
                    "stage_order": ("fused tile count, visible-splat work list, packed fragment rows, packed gradient rows, plain-store gradients"
                                    + (", tile-segmented sort" if tile_sort else "") if native else "reference order")
                                   + (", antialiased (mip) primitive" if args.mip else "")
@@ -302,8 +336,8 @@ def main():
         # instruction holds one of the chip's 1024 SIMDs for 4 cycles; share of the measured duration at 2.4 GHz
         out["roofline"]["valu_issue"] = {"wave_instructions_per_launch": valu_inst,
                                          "frac_of_issue_slots": valu_inst * 4 / 1024 / (acc[dom] * 1e-3 * 2.4e9)}
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(pkg, cfg)   # one camera of the configuration
+    if cpu is not None:
+        out["cpu_baseline"] = cpu   # one camera of the configuration
     print(json.dumps(out))
 
 

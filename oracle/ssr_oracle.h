@@ -6,11 +6,12 @@
  * product library never links, loads or calls it. Only tests, the smoke check and the
  * cpu_baseline leg of the benchmark may use it.
  *
- * Parity unpinned: the opacity side of the median-depth gradient in or_raster_bwd_ex. The reference's
- * backward omits the far splat's own opacity term by its own statement
- * (src/kernels/raster/RasterizationEval3DBwd_kernel.cuh:433-440), so it is not the derivative of the
- * forward and no finite difference can check it; it is restated as read. Every other function is
- * checked against closed forms, float64 restatements or finite differences by tests/test_oracle_*.py.
+ * Every function is checked against closed forms, float64 restatements or finite differences by
+ * tests/test_oracle_*.py; nothing is left unpinned. The median-depth gradient of or_raster_bwd_ex omits the
+ * far splat's own opacity term, as the reference states it does
+ * (src/kernels/raster/RasterizationEval3DBwd_kernel.cuh:433-440): it is the gradient of the median with
+ * ln(1 - alpha_far) held fixed, and is checked against finite differences of that function
+ * (tests/test_oracle_raster_variants.py). or_raster_lane_stats is a measurement aid, not a restatement.
  *
  * Every pointer is a host pointer. Arrays use the reference's layouts
  * (src/primitives/PrimitiveBase3DGS.cuh:87-139,187-225):

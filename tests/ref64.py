@@ -254,3 +254,45 @@ def composite_ex(px, py, frags, dist_type=0):
     else:
         out["depth"] = (w * z).sum() / W
     return out
+
+
+def median_plan(px, py, frags):
+    """What the median-depth backward of the reference freezes at one pixel (RasterizationEval3DBwd_kernel.cuh:433-470):
+    the composited splats in order, the far member of the crossing of T = 1/2 (first composited splat after which
+    T < 1/2), the near member (the composited splat before it, None when the far one is the first) and
+    d0 = ln(1 - alpha_far). None when T never crosses 1/2 among the composited splats (a crossing splat that also
+    ends the pixel is not composited, and the backward never visits it)."""
+    K = len(frags["opac"])
+    T, chain = 1.0, []
+    for k in range(K):
+        dx, dy = frags["xy"][k, 0] - px, frags["xy"][k, 1] - py
+        a, b, c = frags["conic"][k]
+        sigma = 0.5 * (a * dx * dx + c * dy * dy) + b * dx * dy
+        if sigma < 0:
+            continue
+        alpha = min(0.999, frags["opac"][k] * math.exp(-sigma))
+        if alpha <= ALPHA_T:
+            continue
+        nT = T * (1 - alpha)
+        if nT <= 1e-4:
+            break
+        if T >= 0.5 and nT < 0.5:
+            return dict(chain=list(chain), near=chain[-1] if chain else None, far=k, d0=math.log(1 - alpha))
+        chain.append(k)
+        T = nT
+    return None
+
+
+def median_surrogate(px, py, frags, plan):
+    """The function whose gradient the reference's median backward is: z_near + (z_far - z_near) (ln 1/2 - a) / d0 with
+    a = sum over the composited splats up to the near one of ln(1 - alpha_j), and d0 (the far splat's own ln(1 - alpha))
+    held at its value of the unperturbed scene -- "the far splat's own opacity term is omitted"."""
+    a = 0.0
+    for k in plan["chain"]:
+        dx, dy = frags["xy"][k, 0] - px, frags["xy"][k, 1] - py
+        ca, cb, cc = frags["conic"][k]
+        sigma = 0.5 * (ca * dx * dx + cc * dy * dy) + cb * dx * dy
+        a += math.log(1 - min(0.999, frags["opac"][k] * math.exp(-sigma)))
+    z_n = frags["depth"][plan["near"]] if plan["near"] is not None else 0.0
+    z_f = frags["depth"][plan["far"]]
+    return z_n + (z_f - z_n) * (math.log(0.5) - a) / plan["d0"]

@@ -83,15 +83,14 @@ def _compare(gpu, oracle, sc, label, fused_count=False, use_list=False, use_pack
         assert np.allclose(aw, vs["accum_weight"], rtol=1e-3, atol=1e-6)
         assert (aw[:sc.n] > 0).sum() > 10
     ab = vs["abs_terms"]
-    # The median's backward finds the crossing of T = 1/2 on the transmittance it reconstructs by undoing
-    # the recursion; a pixel whose T sits within rounding of 1/2 can attribute it to the neighbouring
-    # splat on either side (the reference's own backward has the same property against its forward),
-    # so with the median on a handful of elements may disagree.
-    # The interpolation weight f = (ln 1/2 - ln T0) / (ln T1 - ln T0) divides by ln(1 - alpha), as small as
-    # 0.004: rounding of the reconstructed T (1e-6 relative) moves f by up to 3e-4, so the median's own
-    # terms are compared at that conditioning rather than at the bar of the plain path.
-    mb = 8 if va.get("median") else 0
-    kw = dict(rtol=1e-2, afrac=1e-3) if mb else {}
+    # The median's backward finds the crossing of T = 1/2 on the transmittance it reconstructs by undoing the
+    # recursion; a pixel whose T sits within rounding of 1/2 can attribute it to the neighbouring splat on either
+    # side (the reference's own backward has the same property against its forward), so two elements may disagree.
+    # The median's terms are not part of the |term| sums that set the floor, and its interpolation weight divides
+    # by ln(1 - alpha) >= 0.004, so the floor is raised to 1e-4 of those sums; the relative bar stays at 1e-3.
+    # (Measured on the MI355X: nothing beyond 1e-3 relative + 3e-5 of the sums except two elements in one case.)
+    mb = 2 if va.get("median") else 0
+    kw = dict(rtol=GRAD_RTOL, afrac=1e-4) if mb else {}
     if va.get("dist_type") and not mb:
         # the distortion terms contain (c W - C), a difference of nearly equal numbers whose rounding is
         # not part of the |term| sums that set the floor: widen the floor for these runs

@@ -117,6 +117,76 @@ def test_median_backward_depth_gradient(pkg, oracle):
     assert np.abs(vs["v_opac"]).max() > 0 and not np.any(vs["v_rgb"])
 
 
+def test_median_backward_is_the_gradient_of_its_surrogate(pkg, oracle):
+    """Every part of the median gradient, opacity side included. The reference's backward leaves out the far splat's
+    own opacity term on purpose (RasterizationEval3DBwd_kernel.cuh:433-440), so it is not the gradient of the forward;
+    it IS the gradient of the forward with d0 = ln(1 - alpha_far) held fixed: z_near + (z_far - z_near)(ln 1/2 - a)/d0,
+    a = ln T before the far splat. That surrogate is written out independently in float64 (ref64.median_surrogate) and
+    differentiated by central differences with respect to every screen attribute of sampled splats; the oracle's
+    v_xy, v_conic, v_opac and v_depth must equal it."""
+    sc = _scene(pkg, n=60, w=32, h=32, seed=9)
+    sc.v_rgb[:] = 0; sc.v_depth[:] = 0; sc.v_T[:] = 0      # median cotangent only
+    cot = _cot(sc)
+    r = oracle.pipeline(sc, variant=dict(median=True, **cot))
+    vs, p = r["vscreen"], r["proj"]
+    tiles = [(t, *_tile_frags(r, sc, t)) for t in range(sc.tile_w * sc.tile_h)]
+    plans, n_plans = {}, 0
+    for t, s, fr, g in tiles:
+        ty, tx = divmod(t, sc.tile_w)
+        for py in range(ty * 16, min(ty * 16 + 16, sc.height)):
+            for px in range(tx * 16, min(tx * 16 + 16, sc.width)):
+                plans[(py, px)] = ref64.median_plan(px + 0.5, py + 0.5, fr)
+                n_plans += plans[(py, px)] is not None
+    assert n_plans > 100
+
+    def total(override=None):
+        tot = 0.0
+        for t, s, fr, g in tiles:
+            if override is not None:
+                gi, key, k, val = override
+                if not np.any(g == gi):
+                    continue
+                fr = {kk: vv.copy() for kk, vv in fr.items()}
+                for j in np.nonzero(g == gi)[0]:
+                    fr[key].reshape(len(g), -1)[j, k] = val
+            ty, tx = divmod(t, sc.tile_w)
+            for py in range(ty * 16, min(ty * 16 + 16, sc.height)):
+                for px in range(tx * 16, min(tx * 16 + 16, sc.width)):
+                    pl = plans[(py, px)]
+                    if pl is not None:
+                        tot += float(cot["v_median"][py, px]) * ref64.median_surrogate(px + 0.5, py + 0.5, fr, pl)
+        return tot
+
+    used = np.unique(r["sorted_flat"])
+    rng = np.random.default_rng(2)
+    names = [("xy", "v_xy"), ("depth", "v_depth"), ("conic", "v_conic"), ("opac", "v_opac")]
+    checked = dict(v_xy=0, v_depth=0, v_conic=0, v_opac=0)
+    for gi in rng.choice(used, size=min(8, used.size), replace=False):
+        for key, vname in names:
+            base = p[key][gi].astype(np.float64).reshape(-1)
+            got = np.asarray(vs[vname][gi], np.float64).reshape(-1)
+            fd = np.zeros_like(base)
+            for k in range(base.size):
+                h = 1e-5 * max(1.0, abs(base[k]))
+                fd[k] = (total((gi, key, k, base[k] + h)) - total((gi, key, k, base[k] - h))) / (2 * h)
+            # float32 kernel arithmetic against float64 differences; terms of both signs add up per splat
+            scale = max(np.abs(fd).max(), np.abs(got).max())
+            assert np.abs(got - fd).max() <= 3e-3 * scale + 1e-7, (gi, key, got, fd)
+            checked[vname] += int(np.abs(fd).max() > 1e-6)
+    assert min(checked.values()) >= 2, checked     # every kind of gradient was really exercised
+    assert not np.any(vs["v_rgb"])
+    # and the surrogate is not the forward: differences of the forward's own median disagree with the oracle on the
+    # opacity of some sampled splat (the omitted term), so a backward that "fixed" the omission would fail above
+    differs = 0
+    for gi in rng.choice(used, size=min(8, used.size), replace=False):
+        base = float(p["opac"][gi])
+        h = 1e-5
+        fd_true = (_total(sc, r, tiles, cot, 0, True, (gi, "opac", 0, base + h)) -
+                   _total(sc, r, tiles, cot, 0, True, (gi, "opac", 0, base - h))) / (2 * h)
+        differs += abs(fd_true - float(vs["v_opac"][gi])) > 0.05 * max(abs(fd_true), abs(float(vs["v_opac"][gi])), 1e-6)
+    assert differs >= 2, differs
+
+
 @pytest.mark.parametrize("mode", [1, 2, 3])
 def test_accumulated_pixel_weights(pkg, oracle, mode):
     """accum_weight[splat] = max / sum over pixels of map[pixel] * alpha * T_before (Avg: also the
