@@ -147,7 +147,7 @@ typedef struct {
     size_t scratch_bytes;
     int64_t* nnz;               /* device scalar: written by _mask, read by _emit */
     int64_t max_rows;           /* _emit: capacity of the arrays below, in rows (>= *nnz) */
-    int32_t* camera_ids;        /* [nnz] all zero with one camera */
+    int32_t* camera_ids;        /* [nnz] every entry = camera_index */
     int32_t* gaussian_ids;      /* [nnz] ascending */
     float* aabb;                /* [nnz,4] */
     float* sort_depth;          /* [nnz] */
@@ -158,6 +158,10 @@ typedef struct {
      * `antialiased` argument of the same projection function): screen-space blur 0.1 instead of 0.3 and the opacity
      * multiplied by sqrt(det cov2d / det (cov2d + blur)); everything after the projection is unchanged. */
     int32_t antialiased;
+    /* Value written into camera_ids (0 for a single camera). A camera set is packed by one mask / emit pair per
+     * camera, each emit writing its rows behind the previous camera's, so that the rows are ordered by
+     * (camera, splat) as the reference's single scan over C * N leaves them (ProjectionPackedFwd.cu:64-158). */
+    int32_t camera_index;
 } ssr_projection_packed_params;
 size_t ssr_projection_packed_scratch_bytes(int64_t num_splats);
 int ssr_projection_packed_mask(const ssr_projection_packed_params* p, ssr_stream_t stream);
@@ -200,13 +204,20 @@ int ssr_tile_write(int64_t n, const float* aabb, const float* sort_depth, const 
                    uint32_t width, uint32_t height, int64_t* isect_ids, int32_t* flatten_ids,
                    const int32_t* visible_ids, int64_t n_visible, const int32_t* tile_active,
                    ssr_stream_t stream);
-/* The same over the rows of several images at once: row r belongs to image r / rows_per_image
- * and its keys carry tile ids offset by image * tiles-per-image (the reference's
- * (camera_id * n_tiles + tile) key, IntersectTile.cu:215-262). n must be a multiple of
- * rows_per_image; no work list and no tile-skip map here. */
-int ssr_tile_write_images(int64_t n, int64_t rows_per_image, const float* aabb, const float* sort_depth,
-                          const float* xy, const float* conic, const float* opac, const int64_t* cum_tiles,
-                          uint32_t width, uint32_t height, int64_t* isect_ids, int32_t* flatten_ids,
+/* The count and the key write over the rows of several images at once. Row r belongs to image
+ * image_ids[r] when image_ids is given (packed rows: the camera_ids of the packed projection), else to image
+ * r / rows_per_image (the [C,N] layout; n must then be num_images * rows_per_image). Its keys carry tile ids
+ * offset by image * tiles-per-image (the reference's (camera_id * n_tiles + tile) key, IntersectTile.cu:215-262),
+ * and tile_active, when given, holds one [tile_h, tile_w] block per image (IntersectTile.cuh:18-22). No work
+ * list here. */
+int ssr_tile_count_images(int64_t n, int64_t rows_per_image, const int32_t* image_ids, int32_t num_images,
+                          const float* aabb, const float* xy, const float* conic, const float* opac,
+                          uint32_t width, uint32_t height, const int32_t* tile_active, int64_t* tiles_per_splat,
+                          ssr_stream_t stream);
+int ssr_tile_write_images(int64_t n, int64_t rows_per_image, const int32_t* image_ids, int32_t num_images,
+                          const float* aabb, const float* sort_depth, const float* xy, const float* conic,
+                          const float* opac, const int64_t* cum_tiles, uint32_t width, uint32_t height,
+                          int64_t* isect_ids, int32_t* flatten_ids, const int32_t* tile_active,
                           ssr_stream_t stream);
 /* sort_pairs<int64,int32> with CUB DoubleBuffer semantics (src/backend/common/SortScan.h:42-56;
  * call site IntersectTile.cu:486-493): stable on bits [begin_bit,end_bit); *selector says which
@@ -425,6 +436,12 @@ typedef struct {
      * `antialiased` argument of the same projection function): screen-space blur 0.1 instead of 0.3 and the opacity
      * multiplied by sqrt(det cov2d / det (cov2d + blur)); everything after the projection is unchanged. */
     int32_t antialiased;
+    /* Optional [N, v_sh_in_stride] fp32: gradient contributions to the higher-order SH coefficients that are already
+     * there, added to this camera's before the step (coefficient k of splat g at g * v_sh_in_stride + k). This is how
+     * a camera batch is summed: the other cameras' projection backward adds into v_world_in and v_sh_in first
+     * (the reference sums the cameras inside its kernel, FusedProjectionBwdOptim_kernel.cuh:262-330). */
+    const float* v_sh_in;
+    int32_t v_sh_in_stride;
 } ssr_fpbo_params;
 int ssr_fused_projection_bwd_optimizer(const ssr_fpbo_params* p, ssr_stream_t stream);
 /* row_of[g] = i where gaussian_ids[i] == g, -1 for splats without a packed row (one camera, so ids

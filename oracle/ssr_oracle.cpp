@@ -596,6 +596,10 @@ static void fused_optimizer_impl(int64_t N, int sh_degree,
     // sRGB curve at its DC colour and the clip of its SH steps, from the parameters as they were
     const bool ctl = hyper[14] != 0.0f;
     const float eps_tr = hyper[15];
+    // hyper[16] != 0: v_in[5] holds SH-gradient contributions that are already there (the other cameras of a batch,
+    // which the reference sums inside its kernel, FusedProjectionBwdOptim_kernel.cuh:262-330) and is added; the
+    // reference's own v_splats_world input carries none for SH, so the default leaves it unread
+    const bool sh_in = hyper[16] != 0.0f && v_in && v_in[5];
     const float kSh0 = 0.28209479177387814f;
     std::vector<float> ctl_slope(ctl ? (size_t)N * 3 : 0), ctl_clip(ctl ? (size_t)N * 3 : 0);
     auto clip_step = [](float delta, float clip) {
@@ -642,7 +646,7 @@ static void fused_optimizer_impl(int64_t N, int sh_degree,
         // SH (fp32 state; the quantized state is updated block by block below)
         for (int i = 0; !q && i < 3 * n_coef; i++) {
             float* x = features_sh + 45 * g + i;
-            float v = vsh[45 * g + i] + sh_reg * *x;
+            float v = (vsh[45 * g + i] + (sh_in ? v_in[5][45 * g + i] : 0.0f)) + sh_reg * *x;
             if (ctl) {
                 v = v / ctl_slope[3 * g + i % 3];
                 const float delta = adam(0.0f, v, lr_sh, g1[5] + 45 * g + i, g2[5] + 45 * g + i);
@@ -780,7 +784,7 @@ static void fused_optimizer_impl(int64_t N, int sh_degree,
                 float m1, m2;
                 ssr_adamq_decode(q->state_packed[cell], old_mm, &m1, &m2);
                 const float x = ssr_q16_decode(q->value_packed[cell], old_lo, old_hi);
-                float v = vsh[45 * g + i] + sh_reg * x;
+                float v = (vsh[45 * g + i] + (sh_in ? v_in[5][45 * g + i] : 0.0f)) + sh_reg * x;
                 if (ctl) v = v / ctl_slope[3 * g + i % 3];
                 const float a = kBeta1 * m1 + (1.f - kBeta1) * v;
                 const float b = kBeta2 * m2 + (1.f - kBeta2) * (v * v);

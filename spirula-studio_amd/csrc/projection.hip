@@ -291,7 +291,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_packed_emit_kernel(ssr_
     const float conic[3] = {S.conic[src], S.conic[N + src], S.conic[2 * N + src]};
     const float opac = S.opac[src], depth = S.depth[src];
     const int32_t g = S.gid[src];
-    P.camera_ids[j] = 0;
+    P.camera_ids[j] = P.camera_index;
     P.gaussian_ids[j] = g;
     reinterpret_cast<float4*>(P.aabb)[j] = bb4;
     P.sort_depth[j] = S.sort_depth[src];
@@ -1045,7 +1045,9 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
             ssr_adamq_decode_with(code, old_mm, s_sqrt_g2[code >> 8], &m1, &m2);
             const float x = ssr_q16_decode(value_cells[cell], old_lo, old_hi);
             const int j = k / 3, c = k - 3 * j;
-            float v = s_Y[sp][j] * s_vc[sp][c] + sh_reg * x;
+            float v = s_Y[sp][j] * s_vc[sp][c];
+            if (P.v_sh_in) v = v + P.v_sh_in[(block0 + sp) * (int64_t)P.v_sh_in_stride + k];
+            v = v + sh_reg * x;
             if (kCtl) v = v / s_ctl[sp][c];
             constexpr float kBeta1 = 0.9f, kBeta2 = 0.999f, kEps = 1e-15f;
             m1 = kBeta1 * m1 + (1.f - kBeta1) * v;
@@ -1134,7 +1136,9 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
         const int64_t row = block0 + sp;
         float* xp = W.features_sh + row * W.sh_stride + i;
         const float x = *xp;
-        float v = s_Y[sp][j] * s_vc[sp][c] + sh_reg * x;
+        float v = s_Y[sp][j] * s_vc[sp][c];
+        if (P.v_sh_in) v = v + P.v_sh_in[row * (int64_t)P.v_sh_in_stride + i];
+        v = v + sh_reg * x;
         if (kCtl) v = v / s_ctl[sp][c];     // FusedProjectionBwdOptim_kernel.cuh:694-705
         AdamD a;
         a.b1c = s_b1c[sp]; a.b2c = s_b2c[sp];

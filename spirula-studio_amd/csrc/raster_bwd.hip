@@ -678,6 +678,8 @@ extern "C" int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t strea
     SSR_REQUIRE(p->v_rows || (p->v_screen.xy && p->v_screen.depth && p->v_screen.conic && p->v_screen.opac && p->v_screen.rgb),
                 "ssr_raster_bwd", "null v_screen buffer");
     SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->v_rows) & 15) == 0, "ssr_raster_bwd", "v_rows must be 16-byte aligned");
+    // the variant kernels address a gradient row as 12 * row in 32 bits
+    SSR_REQUIRE(!p->v_rows || p->num_splats <= (int64_t)(0xFFFFFFFFu / 12u), "ssr_raster_bwd", "with v_rows, num_splats must not exceed 357913941");
     SSR_REQUIRE(p->dist_type >= SSR_DIST_NONE && p->dist_type <= SSR_DIST_RGB_D, "ssr_raster_bwd",
                 "dist_type must be NONE, D or RGB_D (the 3dgs pixel has no normal channel)");
     if (p->dist_type != SSR_DIST_NONE)
@@ -693,8 +695,9 @@ extern "C" int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t strea
     SSR_REQUIRE(p->num_images >= 0, "ssr_raster_bwd", "negative num_images");
     const int nimg = p->num_images > 1 ? p->num_images : 1;
     SSR_REQUIRE((int64_t)tw * th * nimg < (int64_t)1 << 30, "ssr_raster_bwd", "too many tiles");
-    SSR_REQUIRE(nimg == 1 || p->accum_mode == SSR_ACCUM_NONE || (p->num_world < ((int64_t)1 << 31) && p->num_splats == nimg * p->num_world),
-                "ssr_raster_bwd", "several images accumulate per world row: num_splats must be num_images * num_world");
+    SSR_REQUIRE(nimg == 1 || p->accum_mode == SSR_ACCUM_NONE || p->gaussian_ids ||
+                    (p->num_world < ((int64_t)1 << 31) && p->num_splats == nimg * p->num_world),
+                "ssr_raster_bwd", "several images accumulate per world row: num_splats must be num_images * num_world (or gaussian_ids given)");
     const dim3 grid((unsigned)xcd_grid_size(tw * th * nimg)), block(kRasterBlock);
     hipStream_t st = as_stream(stream);
     const bool med = p->v_render_median != nullptr;

@@ -13,11 +13,15 @@ constexpr int kTileBlock = 256;
 __global__ __launch_bounds__(kTileBlock) void tile_count_kernel(
     int64_t n, const float4* __restrict__ aabb, const float2* __restrict__ xy,
     const float* __restrict__ conic, const float* __restrict__ opac, int tile_w, int tile_h,
-    const int32_t* __restrict__ live, int64_t* __restrict__ tiles_per_splat) {
+    const int32_t* __restrict__ live, int64_t* __restrict__ tiles_per_splat, uint32_t rows_per_image,
+    const int32_t* __restrict__ image_ids) {
     const int64_t g = (int64_t)blockIdx.x * kTileBlock + threadIdx.x;
     if (g >= n) return;
     const float4 a = aabb[g];
     if (a.z <= a.x || a.w <= a.y) { tiles_per_splat[g] = 0; return; }
+    // several images: row g belongs to image image_ids[g] (packed rows) or g / rows_per_image, and the
+    // tile-skip map holds one [tile_h, tile_w] block per image
+    if (live) live += (int64_t)(image_ids ? image_ids[g] : (rows_per_image ? (int)((uint32_t)g / rows_per_image) : 0)) * (tile_w * tile_h);
     const float bb[4] = {a.x, a.y, a.z, a.w};
     const float2 c = xy[g];
     const float cxy[2] = {c.x, c.y};
@@ -75,8 +79,8 @@ __global__ __launch_bounds__(kTileBlock) void tile_write_kernel(
     int64_t n, const float4* __restrict__ aabb, const float* __restrict__ sort_depth,
     const float2* __restrict__ xy, const float* __restrict__ conic, const float* __restrict__ opac,
     const int64_t* __restrict__ cum, int tile_w, int tile_h, int64_t* __restrict__ isect_ids,
-    int32_t* __restrict__ flatten_ids, const int32_t* __restrict__ visible_ids, const int32_t* __restrict__ live,
-    uint32_t rows_per_image) {
+    int32_t* __restrict__ flatten_ids, const int32_t* __restrict__ visible_ids, const int32_t* __restrict__ live_all,
+    uint32_t rows_per_image, const int32_t* __restrict__ image_ids) {
     const int64_t i = (int64_t)blockIdx.x * kTileBlock + threadIdx.x;
     const int lane = threadIdx.x & 63;
     const bool in_range = i < n;
@@ -85,9 +89,11 @@ __global__ __launch_bounds__(kTileBlock) void tile_write_kernel(
     TileGeomD tg;
     uint32_t du = 0;
     bool visible = false;
-    // several images in one launch: row g belongs to image g / rows_per_image, whose tiles follow
-    // the earlier images' in the key space
-    const int tile_base = rows_per_image ? (int)((uint32_t)g / rows_per_image) * (tile_w * tile_h) : 0;
+    // several images in one launch: row g belongs to image image_ids[g] (packed rows) or g / rows_per_image;
+    // its tiles follow the earlier images' in the key space, and its block of the tile-skip map is its own
+    const int image = (in_range && image_ids) ? image_ids[g] : (rows_per_image ? (int)((uint32_t)g / rows_per_image) : 0);
+    const int tile_base = image * (tile_w * tile_h);
+    const int32_t* live = live_all ? live_all + tile_base : nullptr;
     if (in_range) {
         cur = g == 0 ? 0 : cum[g - 1];
         end = cum[g];
@@ -136,6 +142,7 @@ __global__ __launch_bounds__(kTileBlock) void tile_write_kernel(
         const uint32_t sdu = (uint32_t)__shfl((int)du, src, 64);
         const int32_t sgid = (int32_t)__shfl((int)g, src, 64);
         const int sbase = __shfl(tile_base, src, 64);
+        const int32_t* slive = live_all ? live_all + sbase : nullptr;
         int64_t scur = ((int64_t)__shfl((int)(cur >> 32), src, 64) << 32) | (uint32_t)__shfl((int)(uint32_t)cur, src, 64);
         const int64_t send = ((int64_t)__shfl((int)(end >> 32), src, 64) << 32) | (uint32_t)__shfl((int)(uint32_t)end, src, 64);
         const int b0 = sg.by_rows ? sg.ymin : sg.xmin, b1 = sg.by_rows ? sg.ymax : sg.xmax;
@@ -143,11 +150,11 @@ __global__ __launch_bounds__(kTileBlock) void tile_write_kernel(
             const int r = base + lane;
             int lo = 0, hi = 0;
             if (r < b1) tile_band_interval(sg, r, lo, hi);
-            const int c = live ? count_live(live, tile_w, lo, hi, r, sg.by_rows) : max(hi - lo, 0);
+            const int c = slive ? count_live(slive, tile_w, lo, hi, r, sg.by_rows) : max(hi - lo, 0);
             const int inc = wave_inclusive_scan_i32(c, lane);
             int64_t pos = scur + (inc - c);
             for (int v = lo; v < hi && pos < send; v++) {
-                if (live && !tile_is_live(live, tile_w, r, v, sg.by_rows)) continue;
+                if (slive && !tile_is_live(slive, tile_w, r, v, sg.by_rows)) continue;
                 const int64_t tile_id = sbase + (sg.by_rows ? ((int64_t)r * tile_w + v) : ((int64_t)v * tile_w + r));
                 isect_ids[pos] = (int64_t)(((uint64_t)tile_id << 32) | (uint64_t)sdu);
                 flatten_ids[pos] = sgid;
@@ -321,8 +328,29 @@ int ssr_tile_count(int64_t n, const float* aabb, const float* xy, const float* c
     const int tw = (int)ceil_div(width, kTile), th = (int)ceil_div(height, kTile);
     hipLaunchKernelGGL(tile_count_kernel, dim3((unsigned)ceil_div(n, kTileBlock)), dim3(kTileBlock), 0, as_stream(stream),
                        n, reinterpret_cast<const float4*>(aabb), reinterpret_cast<const float2*>(xy), conic, opac, tw, th,
-                       tile_active, tiles_per_splat);
+                       tile_active, tiles_per_splat, 0u, (const int32_t*)nullptr);
     SSR_CHECK_LAUNCH("ssr_tile_count");
+    return 0;
+}
+
+int ssr_tile_count_images(int64_t n, int64_t rows_per_image, const int32_t* image_ids, int32_t num_images, const float* aabb,
+                          const float* xy, const float* conic, const float* opac, uint32_t width, uint32_t height,
+                          const int32_t* tile_active, int64_t* tiles_per_splat, ssr_stream_t stream) {
+    SSR_REQUIRE(n >= 0 && n < (int64_t)1 << 31, "ssr_tile_count_images", "count out of range");
+    if (n == 0) return 0;
+    SSR_REQUIRE(num_images >= 1, "ssr_tile_count_images", "num_images must be at least 1");
+    SSR_REQUIRE(image_ids || (rows_per_image > 0 && rows_per_image * num_images == n), "ssr_tile_count_images",
+                "without image_ids, n must be num_images * rows_per_image");
+    SSR_REQUIRE(aabb && xy && conic && opac && tiles_per_splat, "ssr_tile_count_images", "null pointer");
+    SSR_REQUIRE(width > 0 && height > 0, "ssr_tile_count_images", "empty image");
+    SSR_REQUIRE((reinterpret_cast<uintptr_t>(aabb) & 15) == 0 && (reinterpret_cast<uintptr_t>(xy) & 7) == 0,
+                "ssr_tile_count_images", "aabb must be 16-byte and xy 8-byte aligned");
+    const int tw = (int)ceil_div(width, kTile), th = (int)ceil_div(height, kTile);
+    SSR_REQUIRE((int64_t)num_images * tw * th < (int64_t)1 << 31, "ssr_tile_count_images", "tile ids of all images must fit 31 bits");
+    hipLaunchKernelGGL(tile_count_kernel, dim3((unsigned)ceil_div(n, kTileBlock)), dim3(kTileBlock), 0, as_stream(stream),
+                       n, reinterpret_cast<const float4*>(aabb), reinterpret_cast<const float2*>(xy), conic, opac, tw, th,
+                       tile_active, tiles_per_splat, image_ids ? 0u : (uint32_t)rows_per_image, image_ids);
+    SSR_CHECK_LAUNCH("ssr_tile_count_images");
     return 0;
 }
 
@@ -385,31 +413,32 @@ int ssr_tile_write(int64_t n, const float* aabb, const float* sort_depth, const 
     const int64_t work = visible_ids ? n_visible : n;
     hipLaunchKernelGGL(tile_write_kernel, dim3((unsigned)ceil_div(work, kTileBlock)), dim3(kTileBlock), 0, as_stream(stream),
                        work, reinterpret_cast<const float4*>(aabb), sort_depth, reinterpret_cast<const float2*>(xy), conic, opac,
-                       cum_tiles, tw, th, isect_ids, flatten_ids, visible_ids, tile_active, 0u);
+                       cum_tiles, tw, th, isect_ids, flatten_ids, visible_ids, tile_active, 0u, (const int32_t*)nullptr);
     SSR_CHECK_LAUNCH("ssr_tile_write");
     return 0;
 }
 
-int ssr_tile_write_images(int64_t n, int64_t rows_per_image, const float* aabb, const float* sort_depth,
-                          const float* xy, const float* conic, const float* opac, const int64_t* cum_tiles,
-                          uint32_t width, uint32_t height, int64_t* isect_ids, int32_t* flatten_ids,
-                          ssr_stream_t stream) {
+int ssr_tile_write_images(int64_t n, int64_t rows_per_image, const int32_t* image_ids, int32_t num_images,
+                          const float* aabb, const float* sort_depth, const float* xy, const float* conic, const float* opac,
+                          const int64_t* cum_tiles, uint32_t width, uint32_t height, int64_t* isect_ids, int32_t* flatten_ids,
+                          const int32_t* tile_active, ssr_stream_t stream) {
     SSR_REQUIRE(n >= 0 && n < (int64_t)1 << 31, "ssr_tile_write_images", "count out of range");
     if (n == 0) return 0;
-    SSR_REQUIRE(rows_per_image > 0 && n % rows_per_image == 0, "ssr_tile_write_images",
-                "n must be a positive multiple of rows_per_image");
+    SSR_REQUIRE(num_images >= 1, "ssr_tile_write_images", "num_images must be at least 1");
+    SSR_REQUIRE(image_ids || (rows_per_image > 0 && rows_per_image * num_images == n), "ssr_tile_write_images",
+                "without image_ids, n must be num_images * rows_per_image");
     SSR_REQUIRE(aabb && sort_depth && xy && conic && opac && cum_tiles, "ssr_tile_write_images", "null pointer");
     SSR_REQUIRE(isect_ids && flatten_ids, "ssr_tile_write_images", "null output (n_isects == 0 needs no call)");
     SSR_REQUIRE(width > 0 && height > 0, "ssr_tile_write_images", "empty image");
     SSR_REQUIRE((reinterpret_cast<uintptr_t>(aabb) & 15) == 0 && (reinterpret_cast<uintptr_t>(xy) & 7) == 0,
                 "ssr_tile_write_images", "aabb must be 16-byte and xy 8-byte aligned");
     const int tw = (int)ceil_div(width, kTile), th = (int)ceil_div(height, kTile);
-    SSR_REQUIRE((n / rows_per_image) * (int64_t)tw * th < (int64_t)1 << 31, "ssr_tile_write_images",
+    SSR_REQUIRE((int64_t)num_images * tw * th < (int64_t)1 << 31, "ssr_tile_write_images",
                 "tile ids of all images must fit 31 bits");
     hipLaunchKernelGGL(tile_write_kernel, dim3((unsigned)ceil_div(n, kTileBlock)), dim3(kTileBlock), 0, as_stream(stream),
                        n, reinterpret_cast<const float4*>(aabb), sort_depth, reinterpret_cast<const float2*>(xy), conic, opac,
-                       cum_tiles, tw, th, isect_ids, flatten_ids, (const int32_t*)nullptr, (const int32_t*)nullptr,
-                       (uint32_t)rows_per_image);
+                       cum_tiles, tw, th, isect_ids, flatten_ids, (const int32_t*)nullptr, tile_active,
+                       image_ids ? 0u : (uint32_t)rows_per_image, image_ids);
     SSR_CHECK_LAUNCH("ssr_tile_write_images");
     return 0;
 }

@@ -130,9 +130,10 @@ class Engine:
         check(self.h.ssrh_set_options(*self.opts, int(on), self.packed_vscreen, self.tile_sort))
 
     def set_tile_mask(self, mask):
-        """Tile-skip map for the next forward only, from a [h_mask, w_mask] byte mask."""
+        """Tile-skip map for the next forward only, from a [h_mask, w_mask] byte mask (one camera) or a
+        [C, h_mask, w_mask] stack with one mask per camera of the set."""
         mask = np.ascontiguousarray(mask, np.uint8)
-        check(self.h.ssrh_set_tile_mask(mask.ctypes.data, mask.shape[0], mask.shape[1]))
+        check(self.h.ssrh_set_tile_mask(mask.ctypes.data, mask.shape[-2], mask.shape[-1]))
 
     def forward(self):
         """The scene's `antialiased` flag selects the reference's "mip" primitive."""

@@ -32,6 +32,7 @@ int32_t* g_visible_ids = nullptr;    // device work list of the last projection 
 float* g_packed_rows = nullptr;      // packed screen rows of the last projection (null: off)
 const float* g_packed_for_xy = nullptr;   // the screen.xy buffer those rows mirror
 bool g_packed_mode = false;          // the last projection was the packed form
+std::vector<int64_t> g_packed_counts;   // ... and its rows per camera (rows are ordered by camera, then splat)
 int g_list_toggle = 0;               // which of the two visible-list buffers the last projection used
 float* g_vrows = nullptr;             // packed gradient rows of the last compositing backward (null: off)
 const float* g_vrows_for_xy = nullptr; // the v_screen.xy buffer they stand in for
@@ -332,19 +333,33 @@ projection_3dgs_packed_forward(const int64_t num_splats, const int max_sh_degree
     p.antialiased = g_antialiased ? 1 : 0;
     p.world = world_of(in_splats);
     p.sh = sh_of(sh_value_packed, sh_value_bounds, num_sh_buffer, sh_value_bits, sh_bounds_stride);
-    p.camera = camera_of(camera_model, distortion, dist_coeffs, viewmats, intrins, image_width, image_height);
+    // Several cameras: one mask / emit pair per camera, each camera's rows behind the previous camera's, which is
+    // the (camera, splat) order the reference's single scan over C * N leaves (ProjectionPackedFwd.cu:64-158). Every
+    // camera stages into its own part of the scratch slot, so that all masks run before the one readback of the
+    // C row counts.
+    const ssr_camera cameras = camera_of(camera_model, distortion, dist_coeffs, viewmats, intrins, image_width, image_height, true);
+    const int64_t C = cameras.num_cameras;
     p.radii = radii.data_ptr();
     p.scratch_bytes = ssr_projection_packed_scratch_bytes(num_splats);
-    p.scratch = DevicePool::global().acquire<uint8_t>(PoolSlot::ProjPackedScratch, p.scratch_bytes);
-    p.nnz = DevicePool::global().acquire<int64_t>(PoolSlot::ProjPackedNnz, 1);
+    const size_t scratch_stride = (p.scratch_bytes + 255) & ~(size_t)255;
+    uint8_t* scratch = DevicePool::global().acquire<uint8_t>(PoolSlot::ProjPackedScratch, scratch_stride * (size_t)C);
+    int64_t* nnz_dev = DevicePool::global().acquire<int64_t>(PoolSlot::ProjPackedNnz, (size_t)C);
     // the work list and its counters belong to the non-packed form
     g_packed_mode = true;
     g_visible_ids = nullptr; g_n_visible = -1; g_counters = nullptr;
     g_counts_fused = false; g_packed_rows = nullptr; g_packed_for_xy = nullptr;
     StageTimer t(&g_times.k1);
-    ok(ssr_projection_packed_mask(&p, nullptr), "projection_3dgs_packed_forward/mask");
+    for (int64_t c = 0; c < C; c++) {
+        p.camera = camera_at(cameras, (uint32_t)c);
+        p.scratch = scratch + scratch_stride * (size_t)c;
+        p.nnz = nnz_dev + c;
+        ok(ssr_projection_packed_mask(&p, nullptr), "projection_3dgs_packed_forward/mask");
+    }
+    std::vector<int64_t> counts((size_t)C, 0);
+    if (num_splats > 0) ok(ssr_read_i64(nnz_dev, counts.data(), (int)C, nullptr), "projection_3dgs_packed_forward/readback");
     int64_t nnz = 0;
-    if (num_splats > 0) ok(ssr_read_i64(p.nnz, &nnz, 1, nullptr), "projection_3dgs_packed_forward/readback");
+    for (int64_t v : counts) nnz += v;
+    g_packed_counts = counts;
     g_n_visible = nnz;
     DeviceVector<int32_t> camera_ids, gaussian_ids;
     DeviceVector<float4> aabb;
@@ -369,21 +384,33 @@ projection_3dgs_packed_forward(const int64_t num_splats, const int max_sh_degree
     std::vector<DeviceTensorFloatND> screen = {
         DeviceTensorFloatND(xy, {nnz, 2}), DeviceTensorFloatND(dp, {nnz, 1}), DeviceTensorFloatND(cn, {nnz, 3}),
         DeviceTensorFloatND(op, {nnz, 1}), DeviceTensorFloatND(rg, {nnz, 3})};
-    {
-        p.max_rows = nnz;
-        p.camera_ids = camera_ids.data_ptr(); p.gaussian_ids = gaussian_ids.data_ptr();
-        p.aabb = (float*)aabb.data_ptr(); p.sort_depth = depths.data_ptr();
-        p.screen.xy = xy; p.screen.depth = dp; p.screen.conic = cn; p.screen.opac = op; p.screen.rgb = rg;
-        if (g_opts.fuse_tile_count) {
-            p.tiles_per_splat = DevicePool::global().acquire<int64_t>(PoolSlot::IsectTilesPerSplat, (size_t)nnz);
-            g_counts_fused = true;
+    int64_t* tiles = nullptr;
+    if (g_opts.fuse_tile_count) {
+        tiles = DevicePool::global().acquire<int64_t>(PoolSlot::IsectTilesPerSplat, (size_t)nnz);
+        g_counts_fused = true;
+    }
+    if (g_opts.packed_rows) {
+        g_packed_rows = DevicePool::global().acquire<float>(PoolSlot::ProjPackedRows, (size_t)(nnz * 12));
+        g_packed_for_xy = xy;
+    }
+    int64_t row0 = 0;
+    for (int64_t c = 0; c < C; c++) {
+        const int64_t rows = counts[(size_t)c];
+        if (rows > 0) {
+            p.camera = camera_at(cameras, (uint32_t)c);
+            p.camera_index = (int32_t)c;
+            p.scratch = scratch + scratch_stride * (size_t)c;
+            p.nnz = nnz_dev + c;
+            p.max_rows = rows;
+            p.camera_ids = camera_ids.data_ptr() + row0; p.gaussian_ids = gaussian_ids.data_ptr() + row0;
+            p.aabb = (float*)aabb.data_ptr() + 4 * row0; p.sort_depth = depths.data_ptr() + row0;
+            p.screen.xy = xy + 2 * row0; p.screen.depth = dp + row0; p.screen.conic = cn + 3 * row0;
+            p.screen.opac = op + row0; p.screen.rgb = rg + 3 * row0;
+            p.tiles_per_splat = tiles ? tiles + row0 : nullptr;
+            p.packed_rows = g_packed_rows ? g_packed_rows + 12 * row0 : nullptr;
+            ok(ssr_projection_packed_emit(&p, nullptr), "projection_3dgs_packed_forward/emit");
         }
-        if (g_opts.packed_rows) {
-            g_packed_rows = DevicePool::global().acquire<float>(PoolSlot::ProjPackedRows, (size_t)(nnz * 12));
-            g_packed_for_xy = xy;
-            p.packed_rows = g_packed_rows;
-        }
-        ok(ssr_projection_packed_emit(&p, nullptr), "projection_3dgs_packed_forward/emit");
+        row0 += rows;
     }
     return std::make_tuple(camera_ids, gaussian_ids, aabb, depths, screen);
 }
@@ -393,11 +420,14 @@ int64_t intersect_tile_count(int width, int height) {
 }
 
 void compute_tile_active(TorchTensorView mask, int I, int width, int height, int32_t* tile_active) {
-    if (I != 1) throw std::runtime_error("compute_tile_active: this backend runs one image per call");
+    if (I < 1) throw std::runtime_error("compute_tile_active: no image");
     const auto& ms = std::get<2>(mask);
-    if (ms.size() != 3) throw std::runtime_error("compute_tile_active: mask must be [I, H_mask, W_mask]");
-    ok(ssr_compute_tile_active((const uint8_t*)std::get<0>(mask), (int32_t)ms[1], (int32_t)ms[2], (uint32_t)width,
-                               (uint32_t)height, tile_active, nullptr), "compute_tile_active");
+    if (ms.size() != 3 || ms[0] != I) throw std::runtime_error("compute_tile_active: mask must be [I, H_mask, W_mask]");
+    const int64_t tiles = intersect_tile_count(width, height);
+    for (int i = 0; i < I; i++)   // one [tile_h, tile_w] block per image (IntersectTile.cuh:18-22)
+        ok(ssr_compute_tile_active((const uint8_t*)std::get<0>(mask) + (size_t)i * (size_t)(ms[1] * ms[2]), (int32_t)ms[1],
+                                   (int32_t)ms[2], (uint32_t)width, (uint32_t)height, tile_active + (size_t)i * (size_t)tiles, nullptr),
+           "compute_tile_active");
 }
 
 std::tuple<DeviceVector<int64_t>, DeviceVector<int32_t>, DeviceTensor3D<int32_t>>
@@ -411,10 +441,9 @@ do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, 
     if (!proj_xy || !proj_conic || !proj_opac)
         throw std::runtime_error("do_intersect_tile_generic: AABB mode is not built in this backend (ellipse mode is)");
     if (I < 1) throw std::runtime_error("do_intersect_tile_generic: no image");
-    if (I > 1 && (image_ids || tile_active))
-        throw std::runtime_error("do_intersect_tile_generic: packed rows and the tile-skip map take one image per call");
     const int64_t total = depths.numel();
-    if (total % I != 0) throw std::runtime_error("do_intersect_tile_generic: rows are not a multiple of the image count");
+    const int32_t* img_ids = (image_ids && I > 1) ? image_ids->data_ptr() : nullptr;   // packed rows of several cameras
+    if (!img_ids && total % I != 0) throw std::runtime_error("do_intersect_tile_generic: rows are not a multiple of the image count");
     const uint32_t tile_w = (image_width + 15) / 16, tile_h = (image_height + 15) / 16;
     const uint32_t n_tiles = tile_w * tile_h * I;
 
@@ -422,6 +451,11 @@ do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, 
     // counts fused into the projection know nothing of a tile-skip map: count again when one is given
     if (!g_counts_fused || tile_active) {
         StageTimer t(&g_times.k2);
+        if (I > 1)
+            ok(ssr_tile_count_images(total, img_ids ? 0 : total / I, img_ids, (int32_t)I, aabb.data_ptr(), proj_xy->data_ptr(),
+                                     proj_conic->data_ptr(), proj_opac->data_ptr(), image_width, image_height, tile_active,
+                                     tiles_per_splat.data_ptr(), nullptr), "do_intersect_tile_generic/count");
+        else
         ok(ssr_tile_count(total, aabb.data_ptr(), proj_xy->data_ptr(), proj_conic->data_ptr(), proj_opac->data_ptr(),
                           image_width, image_height, tile_active, tiles_per_splat.data_ptr(), nullptr), "do_intersect_tile_generic/count");
     } else {
@@ -456,9 +490,10 @@ do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, 
     {
         StageTimer t(&g_times.k4);
         if (I > 1)   // keys carry image * tiles + tile (IntersectTile.cu:215-262)
-            ok(ssr_tile_write_images(total, total / I, aabb.data_ptr(), depths.data_ptr(), proj_xy->data_ptr(),
-                                     proj_conic->data_ptr(), proj_opac->data_ptr(), cum.data_ptr(), image_width, image_height,
-                                     ids_a.data_ptr(), flat_a.data_ptr(), nullptr), "do_intersect_tile_generic/write");
+            ok(ssr_tile_write_images(total, img_ids ? 0 : total / I, img_ids, (int32_t)I, aabb.data_ptr(), depths.data_ptr(),
+                                     proj_xy->data_ptr(), proj_conic->data_ptr(), proj_opac->data_ptr(), cum.data_ptr(),
+                                     image_width, image_height, ids_a.data_ptr(), flat_a.data_ptr(), tile_active, nullptr),
+               "do_intersect_tile_generic/write");
         else
         ok(ssr_tile_write(total, aabb.data_ptr(), depths.data_ptr(), proj_xy->data_ptr(), proj_conic->data_ptr(),
                           proj_opac->data_ptr(), cum.data_ptr(), image_width, image_height, ids_a.data_ptr(),
@@ -500,7 +535,6 @@ rasterize_to_pixels_3dgs_fwd(int64_t num_splats, std::vector<DeviceTensorFloatND
         throw std::runtime_error("rasterize_to_pixels_3dgs_fwd: normal distortion needs a normal channel, which the 3dgs pixel does not have");
     const int64_t I = tile_offsets.size<0>();
     if (I < 1) throw std::runtime_error("rasterize_to_pixels_3dgs_fwd: no image");
-    if (I > 1 && gaussian_ids.data_ptr()) throw std::runtime_error("rasterize_to_pixels_3dgs_fwd: packed rows take one image per call");
     RenderOutput::TensorTuple renders;
     std::get<0>(renders).resize(PoolSlot::RendersRgb, I, image_height, image_width);
     std::get<1>(renders).resize(PoolSlot::RendersDepth, I, image_height, image_width);
@@ -508,7 +542,7 @@ rasterize_to_pixels_3dgs_fwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     DeviceTensor3D<int32_t> last; last.resize(PoolSlot::RenderLastIds, I, image_height, image_width);
     ssr_raster_fwd_params p;
     std::memset(&p, 0, sizeof(p));
-    p.num_splats = I > 1 && !splats_s.empty() ? splats_s[0].rows() : num_splats;   // [C,N] rows
+    p.num_splats = I > 1 && !splats_s.empty() ? splats_s[0].rows() : num_splats;   // [C,N] rows, or the packed rows of C cameras
     p.num_images = (int32_t)I;
     if (flatten_ids.size() > 0) p.screen = screen_of(splats_s);
     p.width = image_width; p.height = image_height;
@@ -586,8 +620,6 @@ rasterize_to_pixels_3dgs_bwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     ssr_raster_bwd_params p;
     std::memset(&p, 0, sizeof(p));
     const int64_t I = tile_offsets.size<0>();
-    if (I > 1 && gaussian_ids.data_ptr())
-        throw std::runtime_error("rasterize_to_pixels_3dgs_bwd: packed rows take one image per call");
     p.num_splats = I > 1 && !splats_s.empty() ? splats_s[0].rows() : num_splats;   // [C,N] rows
     p.num_images = (int32_t)I;
     p.screen = screen_of(splats_s);
@@ -653,7 +685,7 @@ void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
     p.antialiased = g_antialiased ? 1 : 0;
     p.world = world_of(splats_world);
     p.sh = sh_of(sh_value_packed, sh_value_bounds, num_sh_buffer, sh_value_bits, sh_bounds_stride);
-    const ssr_camera cameras = camera_of(camera_model, distortion, dist_coeffs, viewmats, intrins, image_width, image_height, !is_packed);
+    const ssr_camera cameras = camera_of(camera_model, distortion, dist_coeffs, viewmats, intrins, image_width, image_height, true);
     const int64_t C = cameras.num_cameras;
     p.camera = camera_at(cameras, 0);
     p.aabb = (const float*)aabb.data_ptr();
@@ -673,6 +705,44 @@ void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
         if (!ssr_ext::backward_overwrites_all_rows(num_splats)) { p.visible_ids = g_visible_ids; p.n_visible = g_n_visible; }
     }
     StageTimer t(&g_times.k9);
+    if (is_packed && C > 1) {
+        // Packed rows of several cameras are ordered by camera: one launch per camera over its run of rows, the first
+        // in the mode the options ask for, the others adding (the reference's single launch adds atomically,
+        // ProjectionBwd_kernel.cuh:107). The runs are those of the packed projection that produced the rows; rows
+        // that did not come from it are split by reading camera_ids back.
+        const int64_t total = camera_ids.size();
+        std::vector<int64_t> counts = g_packed_counts;
+        int64_t sum = 0;
+        for (int64_t v : counts) sum += v;
+        if ((int64_t)counts.size() != C || sum != total) {
+            std::vector<int32_t> host_ids((size_t)total);
+            backend::memcpy_sync(host_ids.data(), camera_ids.data_ptr(), (size_t)total * sizeof(int32_t), backend::MemcpyKind::DeviceToHost);
+            counts.assign((size_t)C, 0);
+            int32_t prev = 0;
+            for (int32_t c : host_ids) {
+                if (c < prev || c >= C) throw std::runtime_error("projection_3dgs_backward: packed rows must be ordered by camera id");
+                counts[(size_t)c]++; prev = c;
+            }
+        }
+        const ssr_projection_bwd_params all = p;
+        int64_t row0 = 0;
+        bool first_launch = true;
+        for (int64_t c = 0; c < C; c++) {
+            const int64_t rows = counts[(size_t)c];
+            if (rows > 0) {
+                p.camera = camera_at(cameras, (uint32_t)c);
+                p.packed_gaussian_ids = all.packed_gaussian_ids + row0; p.num_packed = rows;
+                p.v_screen = screen_rows_from(all.v_screen, row0);
+                if (all.v_rows) p.v_rows = all.v_rows + 12 * row0;
+                if (all.v_viewmat) p.v_viewmat = all.v_viewmat + 16 * c;
+                p.accumulate = first_launch ? all.accumulate : 1;
+                ok(ssr_projection_bwd(&p, nullptr), "projection_3dgs_backward");
+                first_launch = false;
+            }
+            row0 += rows;
+        }
+        return;
+    }
     ok(ssr_projection_bwd(&p, nullptr), "projection_3dgs_backward");
     // further cameras: one launch each over row block c of the [C,N,...] gradients, added into the
     // world gradients the first launch wrote (the reference's single launch sums them with
@@ -736,12 +806,72 @@ void fused_projection_bwd_optimizer_3dgs(
             }
         }
     }
-    p.camera = camera_of(camera_model, distortion, dist_coeffs, viewmats, intrins, image_width, image_height);
+    const ssr_camera cameras = camera_of(camera_model, distortion, dist_coeffs, viewmats, intrins, image_width, image_height, true);
+    const int64_t C = cameras.num_cameras;
+    p.camera = camera_at(cameras, 0);
     p.aabb = aabb.data_ptr();
     p.v_screen = screen_of(v_splats_screen);
     if (g_vrows && p.v_screen.xy == g_vrows_for_xy) p.v_rows = g_vrows;
     if (!v_splats_world.empty()) p.v_world_in = world_of(v_splats_world);
     p.v_world_in.features_sh = nullptr;   // not read (FusedProjectionBwdOptim_kernel.cuh:250-255)
+    // rows of camera 0 in the packed layout (all of them with one camera)
+    int64_t rows0 = is_packed ? (int64_t)gaussian_ids.size() : 0;
+    StageTimer t(&g_times.k9);
+    if (C > 1) {
+        // A camera batch: the reference walks every camera's row of a splat inside its kernel and steps once with
+        // the sum (FusedProjectionBwdOptim.cu:160-212, FusedProjectionBwdOptim_kernel.cuh:262-330). Here the
+        // projection backward of cameras 1..C-1 adds into a scratch copy of the incoming gradients, SH included,
+        // and the fused kernel runs camera 0 on top of that sum.
+        const int64_t N = num_splats, S = splats_world[5].channels();
+        float* tmp = DevicePool::global().acquire<float>(PoolSlot::FusedMultiCamGrad, (size_t)(N * (14 + S)));
+        ssr_world acc;
+        acc.means = tmp; acc.quats = tmp + 3 * N; acc.log_scales = tmp + 7 * N; acc.opacity_logits = tmp + 10 * N;
+        acc.features_dc = tmp + 11 * N; acc.features_sh = tmp + 14 * N; acc.sh_stride = (int32_t)S;
+        backend::memset_async(tmp, 0, (size_t)(N * (14 + S)) * sizeof(float));
+        const float* src[5] = {p.v_world_in.means, p.v_world_in.quats, p.v_world_in.log_scales, p.v_world_in.opacity_logits, p.v_world_in.features_dc};
+        float* dst[5] = {acc.means, acc.quats, acc.log_scales, acc.opacity_logits, acc.features_dc};
+        const int64_t width5[5] = {3, 4, 3, 1, 3};
+        for (int i = 0; i < 5; i++)
+            if (src[i]) backend::memcpy_async(dst[i], src[i], (size_t)(N * width5[i]) * sizeof(float), backend::MemcpyKind::DeviceToDevice);
+        std::vector<int64_t> counts;
+        if (is_packed) {
+            counts = g_packed_counts;
+            int64_t sum = 0;
+            for (int64_t v : counts) sum += v;
+            if ((int64_t)counts.size() != C || sum != (int64_t)camera_ids.size())
+                throw std::runtime_error(std::string(w) + "the packed rows of a camera batch must come from the preceding projection_3dgs_packed_forward");
+            rows0 = counts[0];
+        }
+        ssr_projection_bwd_params b;
+        std::memset(&b, 0, sizeof(b));
+        b.num_splats = N; b.sh_degree = max_sh_degree; b.antialiased = p.antialiased;
+        b.world = p.world;
+        if (quant) {   // the coefficients are the 16-bit value codes, one bound per 256 splats
+            b.sh.codec = SSR_SH_REF_Q16; b.sh.packed = p.sh_value_packed; b.sh.bounds = p.sh_value_bounds;
+            b.sh.num_sh_buffer = p.num_sh_buffer; b.sh.bounds_stride = (int64_t)256 * 3 * p.num_sh_buffer;
+        }
+        b.v_world = acc; b.accumulate = 1; b.packed_ids_unique = 1;
+        int64_t row = rows0;
+        for (int64_t c = 1; c < C; c++) {
+            b.camera = camera_at(cameras, (uint32_t)c);
+            if (is_packed) {
+                const int64_t rows = counts[(size_t)c];
+                b.packed_gaussian_ids = gaussian_ids.data_ptr() + row; b.num_packed = rows;
+                b.v_screen = screen_rows_from(p.v_screen, row);
+                b.v_rows = p.v_rows ? p.v_rows + 12 * row : nullptr;
+                row += rows;
+                if (rows == 0) continue;
+            } else {
+                b.aabb = p.aabb + 4 * c * N;
+                b.v_screen = screen_rows_from(p.v_screen, c * N);
+                b.v_rows = p.v_rows ? p.v_rows + 12 * c * N : nullptr;
+            }
+            ok(ssr_projection_bwd(&b, nullptr), "fused_projection_bwd_optimizer_3dgs/other cameras");
+        }
+        p.v_world_in = acc;
+        p.v_world_in.features_sh = nullptr;
+        p.v_sh_in = acc.features_sh; p.v_sh_in_stride = (int32_t)S;
+    }
     if (!g1_splats_world.empty()) p.g1 = world_of(g1_splats_world);
     if (!g2_splats_world.empty()) p.g2 = world_of(g2_splats_world);
     p.densify_score = densify_score.data_ptr();
@@ -761,10 +891,9 @@ void fused_projection_bwd_optimizer_3dgs(
     } else {
         p.steps = (const int32_t*)std::get<0>(std::get<TorchTensorView>(step));
     }
-    StageTimer t(&g_times.k9);
-    if (is_packed) {   // aabb and v_splats_screen hold nnz compacted rows: find each splat's row
+    if (is_packed) {   // aabb and v_splats_screen hold nnz compacted rows: find each splat's row (camera 0's rows)
         int32_t* row_of = DevicePool::global().acquire<int32_t>(PoolSlot::FusedProjBwdRowOf, (size_t)num_splats);
-        ok(ssr_packed_row_map(gaussian_ids.data_ptr(), (int64_t)gaussian_ids.size(), num_splats, row_of, nullptr),
+        ok(ssr_packed_row_map(gaussian_ids.data_ptr(), rows0, num_splats, row_of, nullptr),
            "fused_projection_bwd_optimizer_3dgs/row map");
         p.packed_row_of = row_of;
     }

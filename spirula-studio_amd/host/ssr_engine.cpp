@@ -491,7 +491,8 @@ int ssrh_copy_sh_quant_state(uint16_t* state_packed, float* state_bounds, uint16
 }
 
 int ssrh_set_tile_mask(const uint8_t* mask, int h_mask, int w_mask) {
-    return guard([&] { engine_set_tile_mask(tv(mask, 1, {1, h_mask, w_mask})); });
+    // one mask per camera of the current camera set, [C, h_mask, w_mask]
+    return guard([&] { engine_set_tile_mask(tv(mask, 1, {std::max<int64_t>(1, engine().camera.num), h_mask, w_mask})); });
 }
 
 int ssrh_forward_3dgs(const char* primitive, int sh_degree, int packed, int output_median, int dist_type) {

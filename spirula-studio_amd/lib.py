@@ -85,7 +85,7 @@ class ProjectionPackedParams(C.Structure):
                 ("scratch_bytes", C.c_size_t), ("nnz", vp), ("max_rows", C.c_int64),
                 ("camera_ids", vp), ("gaussian_ids", vp), ("aabb", vp), ("sort_depth", vp),
                 ("screen", Screen), ("tiles_per_splat", vp), ("packed_rows", vp),
-                ("antialiased", C.c_int32)]
+                ("antialiased", C.c_int32), ("camera_index", C.c_int32)]
 
 
 class FpboParams(C.Structure):
@@ -101,7 +101,7 @@ class FpboParams(C.Structure):
                 ("scale_agnostic_radii", vp), ("packed_row_of", vp), ("sh_state_packed", vp), ("sh_state_bounds", vp),
                 ("sh_value_packed", vp), ("sh_value_bounds", vp), ("num_sh_buffer", C.c_uint32),
                 ("non_sh_packed", vp * 5), ("non_sh_bounds", vp * 5), ("color_trust_linear", C.c_int32), ("eps_tr", C.c_float),
-                ("antialiased", C.c_int32)]
+                ("antialiased", C.c_int32), ("v_sh_in", vp), ("v_sh_in_stride", C.c_int32)]
 
 
 # every symbol include/ssr_backend.h declares: (name, restype, argtypes)
@@ -118,7 +118,8 @@ SYMBOLS = {
     "ssr_inclusive_sum_i64_static": (_i32, [vp, vp, _i64, vp, vp]),
     "ssr_read_i64": (_i32, [vp, C.POINTER(C.c_int64), _i32, vp]),
     "ssr_tile_write": (_i32, [_i64, vp, vp, vp, vp, vp, vp, _u32, _u32, vp, vp, vp, _i64, vp, vp]),
-    "ssr_tile_write_images": (_i32, [_i64, _i64, vp, vp, vp, vp, vp, vp, _u32, _u32, vp, vp, vp]),
+    "ssr_tile_count_images": (_i32, [_i64, _i64, vp, _i32, vp, vp, vp, vp, _u32, _u32, vp, vp, vp]),
+    "ssr_tile_write_images": (_i32, [_i64, _i64, vp, _i32, vp, vp, vp, vp, vp, vp, _u32, _u32, vp, vp, vp, vp]),
     "ssr_sort_scratch_bytes": (_sz, [_i64]),
     "ssr_sort_pairs_u64_i32": (_i32, [vp, vp, vp, vp, _i64, _i32, _i32, C.POINTER(C.c_int), vp, _sz, vp]),
     "ssr_tile_offsets": (_i32, [_i64, vp, _u32, vp, vp]),

@@ -249,7 +249,7 @@ def projection_bwd(scene, aabb, vs, sh_degree=3, pose=False):
 
 HYPER = ["lr_means", "lr_quats", "lr_scales", "lr_opacs", "lr_features_dc", "lr_features_sh", "max_gauss_ratio",
          "scale_regularization_weight", "mcmc_opacity_reg_weight", "mcmc_scale_reg_weight", "quat_norm_reg_weight",
-         "sh_reg_weight", "erank_reg_weight", "erank_reg_weight_s3", "color_trust_linear", "eps_tr"]
+         "sh_reg_weight", "erank_reg_weight", "erank_reg_weight_s3", "color_trust_linear", "eps_tr", "v_in_sh"]
 WORLD_KEYS = ["means", "quats", "log_scales", "opacity_logits", "features_dc", "features_sh"]
 
 

@@ -637,28 +637,140 @@ def test_engine_two_cameras(pkg, oracle, H, native):
             world_grad_check(v, r, n, f"two-cameras/{key}", scale=scale)
 
 
-def test_two_cameras_are_refused_where_one_is_required(pkg, H):
-    """Packed projection, the fused optimizer and the tile-skip map take one camera per call: a [2,4,4]
-    camera set raises instead of rendering the first camera only."""
+def _two_camera_scene(pkg, n=3000, seed=71, cull_every=0):
+    """A scene, two cameras that see different subsets of it, per-camera cotangents, and the scene with both."""
     import copy
+    S = pkg.scenes
+    base = S.tiny_scene(n=n, width=250, height=180, seed=seed)
+    if cull_every:
+        base.means[::cull_every, 2] = -10.0
+    cams = []
+    # the second camera looks past the scene's edge, so that each camera sees splats the other does not
+    for k, (ang, t) in enumerate([(0.2, (0.9, -0.2, 2.2)), (-0.35, (-1.1, 0.1, 2.4))]):
+        c, s_ = np.cos(ang), np.sin(ang)
+        vm = np.array([[c, 0, s_, t[0]], [0, 1, 0, t[1]], [-s_, 0, c, t[2]], [0, 0, 0, 1]], np.float32)
+        it = np.array([150.0 + 20 * k, 155.0 - 10 * k, 125.0, 90.0 + 5 * k], np.float32)
+        cams.append((vm, it))
+    rng = np.random.default_rng(5)
+    h, w = base.height, base.width
+    v_rgb = rng.standard_normal((2, h, w, 3)).astype(np.float32)
+    v_depth = rng.standard_normal((2, h, w)).astype(np.float32)
+    v_T = rng.standard_normal((2, h, w)).astype(np.float32)
+    singles = []
+    for k, (vm, it) in enumerate(cams):
+        sc = copy.deepcopy(base)
+        sc.viewmat, sc.intrins = vm, it
+        sc.v_rgb, sc.v_depth, sc.v_T = v_rgb[k], v_depth[k], v_T[k]
+        singles.append(sc)
+    both = copy.deepcopy(base)
+    both.viewmat = np.stack([c[0] for c in cams])
+    both.intrins = np.stack([c[1] for c in cams])
+    both.v_rgb, both.v_depth, both.v_T = v_rgb, v_depth, v_T
+    return base, singles, both
+
+
+@pytest.mark.parametrize("native", [False, True])
+def test_engine_two_cameras_packed_projection(pkg, oracle, H, native):
+    """The packed projection over a camera batch (ProjectionPackedFwd_kernel.cuh:37-47,119-135: one scan over C * N):
+    rows ordered by (camera, splat), camera_ids saying which image a row belongs to, and every later stage on
+    those rows; against the oracle's packed chain run once per camera."""
     host, lib = H
-    sc = pkg.scenes.tiny_scene(n=500, width=64, height=48, seed=3)
-    sc.viewmat = np.stack([sc.viewmat, sc.viewmat])
-    sc.intrins = np.stack([sc.intrins, sc.intrins])
-    for name in ["v_rgb", "v_depth", "v_T"]:
-        setattr(sc, name, np.stack([getattr(sc, name)] * 2))
-    eng = host.Engine(sc, packed_projection=True)
-    with pytest.raises(lib.SsrError, match="one camera per call"):
+    base, singles, both = _two_camera_scene(pkg, cull_every=4)
+    n, h, w = base.n, base.height, base.width
+    refs = [oracle.pipeline_packed(sc) for sc in singles]
+    m = [r["proj"]["visible"] for r in refs]
+    assert min(m) > 100 and m[0] != m[1]
+    eng = host.Engine(both, packed_projection=True, fuse_tile_count=native, packed_rows=native, overwrite_world_grads=native,
+                      packed_vscreen=native, tile_sort=native)
+    tiles = ((w + 15) // 16) * ((h + 15) // 16)
+    for rep in range(2):
         eng.forward()
-    eng = host.Engine(sc)
+        eng.backward()
+        assert np.array_equal(eng.cache("gaussian_ids"), np.concatenate([r["proj"]["gaussian_ids"] for r in refs]))
+        assert np.array_equal(eng.cache("camera_ids"), np.repeat([0, 1], m).astype(np.int32))
+        assert np.array_equal(eng.cache("aabb").reshape(-1, 4), np.concatenate([r["proj"]["aabb"] for r in refs]))
+        n0 = refs[0]["sorted_ids"].size
+        assert eng.n_isects == n0 + refs[1]["sorted_ids"].size
+        assert np.array_equal(eng.cache("sorted_ids"),
+                              np.concatenate([refs[0]["sorted_ids"], refs[1]["sorted_ids"] + (np.int64(tiles) << 32)]))
+        assert np.array_equal(eng.cache("sorted_flat"), np.concatenate([refs[0]["sorted_flat"], refs[1]["sorted_flat"] + m[0]]))
+        rgb, depth, T = eng.render()
+        for k in range(2):
+            assert np.abs(rgb[k] - refs[k]["fwd"]["rgb"]).max() <= 1e-4
+            assert np.abs(T[k] - refs[k]["fwd"]["T"]).max() <= 1e-4
+        g = eng.grads()
+        for key, v in g.items():
+            r = sum(ref["grads"][key].astype(np.float64) for ref in refs).reshape(n, -1)
+            scale = sum(np.abs(ref["grads"][key].astype(np.float64)).reshape(n, -1).max(axis=1, keepdims=True) for ref in refs)
+            world_grad_check(v, r, n, f"two-cameras-packed/{key}", scale=scale)
+
+
+def test_engine_two_cameras_tile_mask(pkg, oracle, H):
+    """compute_tile_active on an [I = 2, H_mask, W_mask] mask (IntersectTile.cuh:18-22) and both tile passes with one
+    [tile_h, tile_w] block of the map per image: each image's keys are its own camera's masked keys."""
+    host, lib = H
+    base, singles, both = _two_camera_scene(pkg)
+    h, w = base.height, base.width
+    tiles = ((w + 15) // 16) * ((h + 15) // 16)
+    rng = np.random.default_rng(9)
+    masks = (rng.uniform(size=(2, 23, 31)) > 0.55).astype(np.uint8)
+    refs = []
+    for k, sc in enumerate(singles):
+        live = oracle.compute_tile_active(masks[k], w, h)
+        assert 0 < live.sum() < live.size
+        refs.append(oracle.pipeline(sc, tile_active=live))
+    eng = host.Engine(both)
+    eng.set_tile_mask(masks)
     eng.forward()
-    hyper = dict.fromkeys(host.Engine.HYPER, 0.0)
-    with pytest.raises(lib.SsrError, match="one camera per call"):
-        eng.backward_fused_optimizer(hyper, 1)
-    # the C ABI's own check: rows must split evenly over the images
-    L = lib.load()
-    with pytest.raises(lib.SsrError, match="rows_per_image"):
-        lib.check(L.ssr_tile_write_images(10, 3, None, None, None, None, None, None, 64, 48, None, None, None))
+    n0 = refs[0]["sorted_ids"].size
+    assert eng.n_isects == n0 + refs[1]["sorted_ids"].size
+    assert np.array_equal(eng.cache("sorted_ids"),
+                          np.concatenate([refs[0]["sorted_ids"], refs[1]["sorted_ids"] + (np.int64(tiles) << 32)]))
+    assert np.array_equal(eng.cache("sorted_flat"), np.concatenate([refs[0]["sorted_flat"], refs[1]["sorted_flat"] + base.n]))
+    rgb, depth, T = eng.render()
+    for k in range(2):
+        assert np.abs(rgb[k] - refs[k]["fwd"]["rgb"]).max() <= 1e-4
+
+
+@pytest.mark.parametrize("packed", [False, True])
+def test_engine_two_cameras_fused_optimizer(pkg, oracle, H, packed):
+    """The fused optimizer over a camera batch: one Adam step on the SUM of both cameras' gradients
+    (FusedProjectionBwdOptim.cu:160-212 gathers every camera's row of a splat; FusedProjectionBwdOptim_kernel.cuh:262-330
+    sums them). Oracle: camera 1's projection backward as incoming gradients (SH included) of the fused step of
+    camera 0."""
+    host, lib = H
+    base, singles, both = _two_camera_scene(pkg, n=4000, seed=72, cull_every=5 if packed else 0)
+    n = base.n
+    hy = dict(lr_means=1.6e-4, lr_quats=1e-3, lr_scales=5e-3, lr_opacs=5e-2, lr_features_dc=2.5e-3, lr_features_sh=1.25e-3,
+              max_gauss_ratio=6.0, scale_regularization_weight=0.01, mcmc_opacity_reg_weight=0.01, mcmc_scale_reg_weight=0.01,
+              quat_norm_reg_weight=0.02, sh_reg_weight=0.05)
+    eng = host.Engine(both, packed_projection=packed)
+    eng.forward()
+    eng.backward_fused_optimizer(hy, 3)
+    got = eng.params()
+    refs = [oracle.pipeline(sc) for sc in singles]
+    P = {k: np.ascontiguousarray(getattr(base, k), np.float32).copy() for k in oracle.WORLD_KEYS}
+    g1 = {k: np.zeros_like(v) for k, v in P.items()}
+    g2 = {k: np.zeros_like(v) for k, v in P.items()}
+    other = refs[1]["grads"]
+    v_in = dict(means=other["v_means"], quats=other["v_quats"], log_scales=other["v_scales"], opacity_logits=other["v_opacities"],
+                features_dc=other["v_dc"], features_sh=other["v_sh"])
+    v_in = {k: np.ascontiguousarray(v, np.float32) for k, v in v_in.items()}
+    oracle.fused_projection_bwd_optimizer(singles[0], refs[0]["proj"]["aabb"], refs[0]["vscreen"], P, g1, g2,
+                                          dict(hy, v_in_sh=1.0), step=3, v_in=v_in)
+    lrs = dict(means="lr_means", quats="lr_quats", log_scales="lr_scales", opacity_logits="lr_opacs",
+               features_dc="lr_features_dc", features_sh="lr_features_sh")
+    vis1_only = (refs[1]["proj"]["aabb"][:, 2] > refs[1]["proj"]["aabb"][:, 0]) & ~(refs[0]["proj"]["aabb"][:, 2] > refs[0]["proj"]["aabb"][:, 0])
+    assert vis1_only.sum() > 20       # splats only the second camera sees: their step comes from its gradients alone
+    for k in oracle.WORLD_KEYS:
+        step_got = got[k].astype(np.float64) - getattr(base, k)
+        step_want = P[k].astype(np.float64) - getattr(base, k)
+        # a first Adam step moves every parameter by about lr whatever the gradient's size, so a wrong gradient SIGN
+        # or a missing camera shows as a difference of the order of lr
+        far = np.abs(step_got - step_want) > 0.02 * hy[lrs[k]] + 1e-7
+        assert far.mean() < 2e-3, (k, float(far.mean()))
+        moved = np.abs(step_want.reshape(n, -1)[vis1_only]).max(axis=1) > 0.5 * hy[lrs[k]]
+        assert moved.mean() > 0.5, k      # (a visible splat that no pixel composites has no gradient and stays)
 
 
 @pytest.mark.parametrize("accum_mode", [1, 3])
