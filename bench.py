@@ -129,6 +129,8 @@ def main():
                     help="widened row: view the scene through an equidistant fisheye spanning 180 degrees of the image width")
     ap.add_argument("--packed-projection", action="store_true",
                     help="run the packed form of the projection (compacted nnz-row outputs; the reference's training default)")
+    ap.add_argument("--dense-projection", action="store_true",
+                    help="config 4: keep the [N]-row projection outputs instead of the packed rows its sparse view defaults to")
     ap.add_argument("--fused-optimizer", action="store_true",
                     help="backward = compositing backward + projection backward fused with the Adam step "
                          "(the reference's FPBO mode); K9 then includes the optimizer's 1.4 kB/splat of traffic")
@@ -170,6 +172,10 @@ def main():
         return
 
     cfg = args.config
+    # config 4 looks out from inside the scene and sees an eighth of it: the reference's packed projection (compacted
+    # nnz-row outputs) is its mode for such views and the faster one here, so it is this config's default
+    if cfg == 4 and not (args.dense_projection or args.reference_order or args.cameras > 1):
+        args.packed_projection = True
     t_gen = time.time()
     sc = pkg.scenes.make_scene(cfg, n=args.n)
     if args.fused_optimizer and args.quantization_level == 1:

@@ -453,10 +453,13 @@ int ssr_packed_row_map(const int32_t* gaussian_ids, int64_t nnz, int64_t num_spl
 /* Zeroes the gradient rows of the listed splats only (the rows a previous ssr_projection_bwd run
  * over that list wrote), instead of refilling all N rows. No counterpart in the reference, which
  * always refills (src/engine/EngineLoss.cpp:120-127).
- * skip_visible_aabb (optional, [N,4]): rows of splats whose aabb is non-empty are left alone, for use
- * right before an ssr_projection_bwd in store mode that overwrites exactly those rows. */
+ * Rows that an ssr_projection_bwd in store mode is about to overwrite can be left alone, named either way:
+ * skip_visible_aabb (optional, [N,4]): splats whose aabb is non-empty;
+ * skip_sorted_ids (optional, n_skip ascending splat ids, e.g. one camera's packed gaussian_ids): splats in
+ * that list, found by bisection. */
 int ssr_zero_world_rows(const ssr_world* v_world, const int32_t* ids, int64_t n,
-                        const float* skip_visible_aabb, ssr_stream_t stream);
+                        const float* skip_visible_aabb, const int32_t* skip_sorted_ids, int64_t n_skip,
+                        ssr_stream_t stream);
 
 /* ---- K10 and runtime (src/backend/api/BackendRuntime.h:29-168). */
 int ssr_fill_u32(void* dst, uint32_t value, int64_t count, ssr_stream_t stream);

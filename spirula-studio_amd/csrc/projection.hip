@@ -230,28 +230,54 @@ __global__ __launch_bounds__(kProjBlock) void projection_packed_mask_kernel(ssr_
     atomic_max_nonneg(P.radii + g, p.radius);   // ProjectionPackedFwd_kernel.cuh:183
 }
 
-// Exclusive scan of the workgroup counts by ONE workgroup: each thread sums a contiguous run, the
-// 1024 run totals are scanned in LDS, then each thread writes its run's offsets. The counts are
-// N/256 values (39k for ten million splats), so one workgroup is enough and saves two launches.
+// Exclusive scan of the workgroup counts by ONE workgroup (the counts are N/256 values, 39k for ten million
+// splats; one workgroup saves two launches). It walks the counts in tiles of 4096: every thread holds four
+// consecutive values, a wavefront scans its 256 with shuffles, the sixteen wavefront totals are scanned by
+// each thread from LDS, and a running total carries from tile to tile. The next tile's loads are issued
+// before the current tile is scanned.
 constexpr int kScanOneBlock = 1024;
 __global__ __launch_bounds__(kScanOneBlock) void packed_block_scan_kernel(const int32_t* __restrict__ counts, int64_t nb,
                                                                           int64_t* __restrict__ offsets, int64_t* __restrict__ nnz) {
-    __shared__ long long s_part[kScanOneBlock];
-    const int64_t run = (nb + kScanOneBlock - 1) / kScanOneBlock;
-    const int64_t lo = (int64_t)threadIdx.x * run, hi = lo + run < nb ? lo + run : nb;
-    long long sum = 0;
-    for (int64_t i = lo; i < hi; i++) sum += counts[i];
-    s_part[threadIdx.x] = sum;
-    __syncthreads();
-    for (int d = 1; d < kScanOneBlock; d <<= 1) {   // Hillis-Steele inclusive scan
-        const long long v = (int)threadIdx.x >= d ? s_part[threadIdx.x - d] : 0;
+    __shared__ int s_wave[2][kScanOneBlock / 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    auto load4 = [&](int64_t base, int v[4]) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) v[k] = base + k < nb ? counts[base + k] : 0;
+    };
+    long long carry = 0;
+    int cur[4], nxt[4];
+    load4((int64_t)threadIdx.x * 4, cur);
+    int parity = 0;
+    for (int64_t tile0 = 0; tile0 < nb; tile0 += 4 * kScanOneBlock, parity ^= 1) {
+        const int64_t base = tile0 + (int64_t)threadIdx.x * 4;
+        load4(base + 4 * kScanOneBlock, nxt);
+        const int mine = (cur[0] + cur[1]) + (cur[2] + cur[3]);
+        int incl = mine;   // inclusive scan over the wavefront
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int up = __shfl_up(incl, d, 64);
+            if (lane >= d) incl += up;
+        }
+        if (lane == 63) s_wave[parity][wave] = incl;
         __syncthreads();
-        s_part[threadIdx.x] += v;
-        __syncthreads();
+        int before = 0, total = 0;
+#pragma unroll
+        for (int w = 0; w < kScanOneBlock / 64; w++) {
+            const int t = s_wave[parity][w];
+            if (w < wave) before += t;
+            total += t;
+        }
+        long long acc = carry + before + (incl - mine);
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            if (base + k < nb) offsets[base + k] = acc;
+            acc += cur[k];
+        }
+        carry += total;
+#pragma unroll
+        for (int k = 0; k < 4; k++) cur[k] = nxt[k];
     }
-    long long acc = s_part[threadIdx.x] - sum;
-    for (int64_t i = lo; i < hi; i++) { offsets[i] = acc; acc += counts[i]; }
-    if (threadIdx.x == kScanOneBlock - 1) { offsets[nb] = s_part[threadIdx.x]; *nnz = s_part[threadIdx.x]; }
+    if (threadIdx.x == 0) { offsets[nb] = carry; *nnz = carry; }
 }
 
 // Pass 2 (projection_packed_fwd_kernel, ProjectionPackedFwd_kernel.cuh:97-184): one thread per
@@ -1168,24 +1194,73 @@ __global__ __launch_bounds__(kProjBlock) void packed_row_map_kernel(const int32_
 
 // One wavefront per listed splat: lane l zeroes float l of its 59-float gradient row
 // (3 mean, 4 quat, 3 scale, 1 opacity, 3 dc, sh_stride SH).
-// Rows of splats that are visible now (non-empty aabb) are skipped when `aabb` is given: the
-// projection backward that follows overwrites them.
+// Rows of splats that are visible now (non-empty aabb when `aabb` is given, member of the ascending list
+// `keep` when that is given) are skipped: the projection backward that follows overwrites them.
+// A workgroup takes 256 listed rows. First every thread decides about one row: the `keep` list is bracketed
+// once per workgroup by the smallest and largest id of its rows (two searches with uniform arguments; lists
+// that ascend together, as two packed projections' do, leave a bracket of a few hundred entries), and each
+// thread bisects inside the bracket. Then the rows that remain are zeroed, one wavefront per row.
 __global__ __launch_bounds__(kProjBlock) void zero_world_rows_kernel(ssr_world V, const int32_t* __restrict__ ids, int64_t n,
-                                                                     const float4* __restrict__ aabb) {
-    const int64_t row = (int64_t)blockIdx.x * (kProjBlock / 64) + (threadIdx.x >> 6);
-    if (row >= n) return;
-    const int lane = threadIdx.x & 63;
-    const int64_t g = ids[row];
-    if (aabb) {
+                                                                     const float4* __restrict__ aabb,
+                                                                     const int32_t* __restrict__ keep, int64_t n_keep) {
+    __shared__ int s_rows[kProjBlock];
+    __shared__ int s_count;
+    __shared__ int s_lo[kProjBlock / 64], s_hi[kProjBlock / 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (threadIdx.x == 0) s_count = 0;
+    const int64_t row = (int64_t)blockIdx.x * kProjBlock + threadIdx.x;
+    const bool valid = row < n;
+    const int g = valid ? ids[row] : 0;
+    bool alive = valid;
+    if (aabb && alive) {
         const float4 bb = aabb[g];
-        if (!(bb.z <= bb.x || bb.w <= bb.y)) return;
+        alive = bb.z <= bb.x || bb.w <= bb.y;
     }
-    if (lane < 3) V.means[3 * g + lane] = 0.f;
-    else if (lane < 7) V.quats[4 * g + lane - 3] = 0.f;
-    else if (lane < 10) V.log_scales[3 * g + lane - 7] = 0.f;
-    else if (lane < 11) V.opacity_logits[g] = 0.f;
-    else if (lane < 14) V.features_dc[3 * g + lane - 11] = 0.f;
-    for (int k = lane; k < V.sh_stride; k += 64) V.features_sh[g * (int64_t)V.sh_stride + k] = 0.f;
+    if (keep && n_keep > 0) {
+        int gmin = valid ? g : 0x7fffffff, gmax = valid ? g : -1;
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) {
+            gmin = min(gmin, __shfl_xor(gmin, d, 64));
+            gmax = max(gmax, __shfl_xor(gmax, d, 64));
+        }
+        if (lane == 0) { s_lo[wave] = gmin; s_hi[wave] = gmax; }
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < kProjBlock / 64; w++) { gmin = min(gmin, s_lo[w]); gmax = max(gmax, s_hi[w]); }
+        int64_t lo = 0, hi = n_keep;       // first entry >= gmin
+        while (lo < hi) {
+            const int64_t mid = (lo + hi) >> 1;
+            if (keep[mid] < gmin) lo = mid + 1; else hi = mid;
+        }
+        const int64_t first = lo;
+        hi = n_keep;                       // first entry > gmax
+        while (lo < hi) {
+            const int64_t mid = (lo + hi) >> 1;
+            if (keep[mid] <= gmax) lo = mid + 1; else hi = mid;
+        }
+        if (alive) {
+            int64_t a = first, b = lo;     // first entry >= g inside the bracket
+            while (a < b) {
+                const int64_t mid = (a + b) >> 1;
+                if (keep[mid] < g) a = mid + 1; else b = mid;
+            }
+            if (a < lo && keep[a] == g) alive = false;
+        }
+    } else {
+        __syncthreads();
+    }
+    if (alive) s_rows[atomicAdd(&s_count, 1)] = g;
+    __syncthreads();
+    const int count = s_count;
+    for (int k = wave; k < count; k += kProjBlock / 64) {
+        const int64_t z = s_rows[k];
+        if (lane < 3) V.means[3 * z + lane] = 0.f;
+        else if (lane < 7) V.quats[4 * z + lane - 3] = 0.f;
+        else if (lane < 10) V.log_scales[3 * z + lane - 7] = 0.f;
+        else if (lane < 11) V.opacity_logits[z] = 0.f;
+        else if (lane < 14) V.features_dc[3 * z + lane - 11] = 0.f;
+        for (int c = lane; c < V.sh_stride; c += 64) V.features_sh[z * (int64_t)V.sh_stride + c] = 0.f;
+    }
 }
 
 static int check_common(const char* where, int64_t n, int sh_degree, const ssr_world& w, const ssr_sh_quant& sh,
@@ -1464,16 +1539,17 @@ extern "C" int ssr_fused_projection_bwd_optimizer(const ssr_fpbo_params* p, ssr_
 }
 
 extern "C" int ssr_zero_world_rows(const ssr_world* v_world, const int32_t* ids, int64_t n, const float* skip_visible_aabb,
-                                   ssr_stream_t stream) {
+                                   const int32_t* skip_sorted_ids, int64_t n_skip, ssr_stream_t stream) {
     SSR_REQUIRE(v_world, "ssr_zero_world_rows", "null world");
     SSR_REQUIRE(n >= 0 && n < (int64_t)1 << 31, "ssr_zero_world_rows", "count out of range");
     if (n == 0) return 0;
     SSR_REQUIRE(ids, "ssr_zero_world_rows", "null ids");
+    SSR_REQUIRE(n_skip >= 0 && (n_skip == 0 || skip_sorted_ids), "ssr_zero_world_rows", "skip list: negative count or null ids");
     const ssr_world& v = *v_world;
     SSR_REQUIRE(v.means && v.quats && v.log_scales && v.opacity_logits && v.features_dc && (v.features_sh || v.sh_stride == 0),
                 "ssr_zero_world_rows", "null buffer");
-    hipLaunchKernelGGL(zero_world_rows_kernel, dim3((unsigned)ceil_div(n, kProjBlock / 64)), dim3(kProjBlock), 0, as_stream(stream),
-                       v, ids, n, reinterpret_cast<const float4*>(skip_visible_aabb));
+    hipLaunchKernelGGL(zero_world_rows_kernel, dim3((unsigned)ceil_div(n, kProjBlock)), dim3(kProjBlock), 0, as_stream(stream),
+                       v, ids, n, reinterpret_cast<const float4*>(skip_visible_aabb), skip_sorted_ids, n_skip);
     SSR_CHECK_LAUNCH("ssr_zero_world_rows");
     return 0;
 }

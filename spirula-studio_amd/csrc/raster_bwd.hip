@@ -371,7 +371,7 @@ __device__ __forceinline__ float fold_pair(float a, float b, bool sel) {
     const float keep = sel ? b : a, send = sel ? a : b;
     return keep + dpp_full<kCtrl>(send);
 }
-constexpr int kDppRor8 = 0x128, kDppHalfMirror = 0x141, kDppQuadXor2 = 0x4E, kDppQuadXor1 = 0xB1;
+constexpr int kDppQuadXor2 = 0x4E, kDppQuadXor1 = 0xB1;
 
 constexpr int kRowBatch = 128;   // fragments staged per batch by the row-granular kernel
 

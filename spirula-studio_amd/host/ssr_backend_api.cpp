@@ -239,9 +239,10 @@ bool backward_overwrites_all_rows(int64_t num_splats) {
 }
 const int32_t* last_backward_list(int64_t* count) { if (count) *count = g_bwd_count; return g_bwd_list; }
 void zero_world_rows(const std::vector<DeviceTensorFloatND>& v, const int32_t* ids, int64_t n,
-                     const DeviceTensor2D<float4>* aabb) {
+                     const DeviceTensor2D<float4>* aabb, const int32_t* sorted_now, int64_t n_now) {
     ssr_world w = world_of(v);
-    ok(ssr_zero_world_rows(&w, ids, n, aabb ? (const float*)aabb->data_ptr() : nullptr, nullptr), "zero_world_rows");
+    ok(ssr_zero_world_rows(&w, ids, n, aabb ? (const float*)aabb->data_ptr() : nullptr, sorted_now, sorted_now ? n_now : 0, nullptr),
+       "zero_world_rows");
 }
 }  // namespace ssr_ext
 

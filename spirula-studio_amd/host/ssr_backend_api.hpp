@@ -199,7 +199,8 @@ const int32_t* last_backward_list(int64_t* count);
 // its zero-fill.
 bool backward_overwrites_all_rows(int64_t num_splats);
 // Zeroes the rows of `ids` in six world-gradient tensors (ordered as v_splats_world).
-// With `aabb` given, rows of currently visible splats are skipped (a store-mode backward overwrites them).
+// Rows of currently visible splats are skipped (a store-mode backward overwrites them): those with a non-empty
+// `aabb` row, or those named in the ascending id list `sorted_now` (one camera's packed gaussian_ids).
 void zero_world_rows(const std::vector<DeviceTensorFloatND>& v_splats_world, const int32_t* ids, int64_t n,
-                     const DeviceTensor2D<float4>* aabb);
+                     const DeviceTensor2D<float4>* aabb, const int32_t* sorted_now = nullptr, int64_t n_now = 0);
 }  // namespace ssr_ext

@@ -55,7 +55,10 @@ void alloc_grad_buffers() {
             DeviceTensorFloatND((float*)g.opacities.data_ptr(), {g.opacities.size(), 1}),
             DeviceTensorFloatND(g.features_dc), DeviceTensorFloatND(g.features_sh)};
         if (g.dirty_count > 0)
-            ssr_ext::zero_world_rows(v_world, g.dirty_list, g.dirty_count, engine().packed ? nullptr : &engine().fwd.aabb);
+            // one camera's packed ids ascend, which is what the skip list needs
+            ssr_ext::zero_world_rows(v_world, g.dirty_list, g.dirty_count, engine().packed ? nullptr : &engine().fwd.aabb,
+                                     engine().packed && engine().camera.num == 1 ? engine().fwd.gaussian_ids.data_ptr() : nullptr,
+                                     engine().fwd.gaussian_ids.size());
         return;
     }
     g.means.zero(); g.quats.zero(); g.scales.zero(); g.opacities.zero(); g.features_dc.zero(); g.features_sh.zero();

@@ -131,7 +131,7 @@ SYMBOLS = {
     "ssr_projection_bwd": (_i32, [C.POINTER(ProjectionBwdParams), vp]),
     "ssr_fused_projection_bwd_optimizer": (_i32, [C.POINTER(FpboParams), vp]),
     "ssr_packed_row_map": (_i32, [vp, _i64, _i64, vp, vp]),
-    "ssr_zero_world_rows": (_i32, [C.POINTER(World), vp, _i64, vp, vp]),
+    "ssr_zero_world_rows": (_i32, [C.POINTER(World), vp, _i64, vp, vp, _i64, vp]),
     "ssr_fill_u32": (_i32, [vp, _u32, _i64, vp]),
     "ssr_init": (_i32, [_i32]),
     "ssr_device_count": (_i32, []),

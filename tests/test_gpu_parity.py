@@ -2,6 +2,7 @@
 inputs. Bars: tile keys / sorted ids / tile ranges bit-exact; images max-abs 1e-4 per channel;
 gradients 1e-3 relative (with a floor proportional to the sum of |terms|, since float atomics add
 in a different order)."""
+import ctypes as C
 import dataclasses
 import math
 
@@ -363,6 +364,48 @@ def test_packed_backward_adds_repeated_ids(gpu, oracle):
         assert np.array_equal(got[keep], 2.0 * v[keep]), k      # x + x is exact, whichever row lands first
         assert not np.any(got[~keep]), k
     assert np.abs(once["w_means"][keep]).max() > 0
+
+
+def test_zero_world_rows_skip_lists(gpu):
+    """ssr_zero_world_rows zeroes exactly the listed rows, minus the rows its skip lists name (non-empty aabb rows,
+    members of an ascending id list): checked against numpy on random lists, with an empty skip list, a skip list
+    that covers everything, and ids at both ends of the range."""
+    L = gpu.lib
+    lib = L.load()
+    rng = np.random.default_rng(77)
+    n, S = 5000, 45
+    shapes = dict(means=(n, 3), quats=(n, 4), log_scales=(n, 3), opacity_logits=(n,), features_dc=(n, 3), features_sh=(n, S))
+    for case in range(5):
+        host = {k: rng.uniform(1, 2, sh).astype(np.float32) for k, sh in shapes.items()}
+        dev = {k: L.DeviceArray.from_host(v) for k, v in host.items()}
+        w = L.World()
+        for k in shapes:
+            setattr(w, k, dev[k].ptr)
+        w.sh_stride = S
+        ids = np.unique(np.concatenate([rng.choice(n, 900, replace=False), [0, n - 1]])).astype(np.int32)
+        rng.shuffle(ids)
+        keep = {0: np.zeros(0, np.int32), 1: np.arange(n, dtype=np.int32), 2: np.array([0, n - 1], np.int32)}.get(
+            case, np.sort(rng.choice(n, 1500, replace=False)).astype(np.int32))
+        aabb = np.zeros((n, 4), np.float32)
+        if case == 4:
+            vis = rng.random(n) < 0.3
+            aabb[vis] = [1.0, 2.0, 5.0, 7.0]
+        d_ids, d_keep, d_aabb = L.DeviceArray.from_host(ids), L.DeviceArray.from_host(np.concatenate([keep, [0]]).astype(np.int32)), L.DeviceArray.from_host(aabb)
+        L.check(lib.ssr_zero_world_rows(C.byref(w), d_ids.ptr, ids.size, d_aabb.ptr if case == 4 else None,
+                                        d_keep.ptr if keep.size else None, keep.size, None))
+        L.check(lib.ssr_device_synchronize())
+        gone = np.zeros(n, bool)
+        gone[ids] = True
+        gone[keep] = False
+        if case == 4:
+            gone &= ~vis
+        assert gone.any() or case == 1
+        for k in shapes:
+            want = host[k].copy()
+            want[gone] = 0.0
+            assert np.array_equal(dev[k].to_host(), want), (case, k)
+    e = lib.ssr_zero_world_rows(C.byref(w), d_ids.ptr, ids.size, None, None, 5, None)
+    assert e != 0 and b"skip list" in lib.ssr_last_error()
 
 
 def test_packed_projection_without_readback(gpu, oracle):
