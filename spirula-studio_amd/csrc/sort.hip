@@ -353,8 +353,8 @@ __device__ __forceinline__ void seg_sort_lds(uint64_t* keys, int32_t* vals, int6
 
 // Work lists of the tiles whose segments are too long for the direct kernel, by size class:
 // counts[c] entries in list[c]; class 0 up to kSegCap0 keys, class 1 up to kSegCap1, class 2 beyond.
-struct SegLists { uint32_t* counts; uint32_t* list[3]; };
-constexpr int kSegCap0 = 4 * 64 * 4;           // four wavefronts, 4 keys per lane
+struct SegLists { uint32_t* counts; uint32_t* list[3]; bool has_class0; };
+constexpr int kSegCap0 = 4 * 64 * 8;           // four wavefronts, 8 keys per lane
 constexpr int kSegCap1 = 16 * 64 * 8;          // sixteen wavefronts, 8 keys per lane
 
 // One workgroup of kWaves wavefronts per tile: sorts segments of 2..64*kWaves*kRounds keys, lists the
@@ -378,7 +378,8 @@ __global__ __launch_bounds__(kWaves * 64) void sort_segments_direct_kernel(uint6
     if (len <= 1) return;
     if (len > kCap) {
         if (threadIdx.x == 0) {
-            const int c = len > kSegCap1 ? 2 : len > kSegCap0 ? 1 : 0;
+            // class 0 exists only where a kernel for it follows: otherwise everything up to kSegCap1 is class 1
+            const int c = len > kSegCap1 ? 2 : (len > kSegCap0 || !lists.has_class0) ? 1 : 0;
             lists.list[c][atomicAdd(&lists.counts[c], 1u)] = tile;
         }
         return;
@@ -394,12 +395,13 @@ __global__ __launch_bounds__(256) void sort_segments_small_kernel(uint64_t* keys
     __shared__ uint32_t ws[kRadix / 64];
     __shared__ uint32_t wor[4];
     __shared__ uint2 buf[kSegCap0];
+    static_assert(kSegCap0 == 4 * 64 * 8, "class 0 is sorted by four wavefronts with 8 keys per lane");
     const uint32_t count = lists.counts[0];
     for (uint32_t idx = blockIdx.x; idx < count; idx += gridDim.x) {
         const uint32_t tile = lists.list[0][idx];
         const int64_t s = tile_offsets[tile];
         const int64_t e = tile + 1 < n_tiles ? (int64_t)tile_offsets[tile + 1] : n;
-        seg_sort_lds<4, 4>(keys, vals, s, (int)(e - s), wcount, ws, wor, buf);
+        seg_sort_lds<4, 8>(keys, vals, s, (int)(e - s), wcount, ws, wor, buf);
         __syncthreads();   // LDS is reused by the next segment
     }
 }
@@ -454,8 +456,10 @@ __device__ __forceinline__ void seg_sort_global(uint64_t* keys, int32_t* vals, u
     }
 }
 
-// Workgroups of sixteen wavefronts take the listed segments of class 1 (in LDS), then of class 2
-// (through global memory), in turn.
+// Workgroups of sixteen wavefronts take the listed segments of class 2 (through global memory), then of class 1
+// (in LDS), longest class first, each workgroup drawing its next segment from a shared cursor when it has
+// finished one (segment lengths differ eightfold, so a fixed assignment leaves workgroups idle at the end).
+// lists.counts[3] is the cursor: zero at launch.
 __global__ __launch_bounds__(kSegGlobalWaves * 64) void sort_segments_long_kernel(
     uint64_t* keys, int32_t* vals, uint64_t* keys_alt, int32_t* vals_alt, const int32_t* __restrict__ tile_offsets,
     uint32_t n_tiles, int64_t n, SegLists lists) {
@@ -463,20 +467,20 @@ __global__ __launch_bounds__(kSegGlobalWaves * 64) void sort_segments_long_kerne
     __shared__ uint32_t ws[kRadix / 64];
     __shared__ uint32_t wor[kSegGlobalWaves];
     __shared__ uint2 buf[kSegCap1];
+    __shared__ uint32_t s_next;
     static_assert(kSegCap1 == kSegGlobalWaves * 64 * 8, "class 1 is sorted by sixteen wavefronts with 8 keys per lane");
     const uint32_t count1 = lists.counts[1], count2 = lists.counts[2];
-    for (uint32_t idx = blockIdx.x; idx < count1; idx += gridDim.x) {
-        const uint32_t tile = lists.list[1][idx];
+    for (;;) {
+        if (threadIdx.x == 0) s_next = atomicAdd(&lists.counts[3], 1u);
+        __syncthreads();
+        const uint32_t idx = s_next;
+        if (idx >= count1 + count2) break;   // the same value in every thread: the workgroup leaves together
+        const uint32_t tile = idx < count2 ? lists.list[2][idx] : lists.list[1][idx - count2];
         const int64_t s = tile_offsets[tile];
         const int64_t e = tile + 1 < n_tiles ? (int64_t)tile_offsets[tile + 1] : n;
-        seg_sort_lds<kSegGlobalWaves, 8>(keys, vals, s, (int)(e - s), wcount, ws, wor, buf);
-        __syncthreads();   // LDS is reused by the next segment
-    }
-    for (uint32_t idx = blockIdx.x; idx < count2; idx += gridDim.x) {
-        const uint32_t tile = lists.list[2][idx];
-        const int64_t s = tile_offsets[tile];
-        const int64_t e = tile + 1 < n_tiles ? (int64_t)tile_offsets[tile + 1] : n;
-        seg_sort_global(keys, vals, keys_alt, vals_alt, s, (int)(e - s), wcount, ws);
+        if (idx < count2) seg_sort_global(keys, vals, keys_alt, vals_alt, s, (int)(e - s), wcount, ws);
+        else seg_sort_lds<kSegGlobalWaves, 8>(keys, vals, s, (int)(e - s), wcount, ws, wor, buf);
+        __syncthreads();   // LDS, s_next included, is reused by the next segment
     }
 }
 
@@ -569,18 +573,25 @@ int ssr_sort_tile_pairs(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, int32
     uint64_t* kc = reinterpret_cast<uint64_t*>(k[cur]);
     uint64_t* ka = reinterpret_cast<uint64_t*>(k[cur ^ 1]);
     const bool lone_waves = n_tiles >= 16384;   // at least two rounds of one-wavefront workgroups on 256 compute units
+    lists.has_class0 = lone_waves;
     if (lone_waves) {
         hipLaunchKernelGGL((sort_segments_direct_kernel<1, 8>), dim3(n_tiles), dim3(64), 0, s, kc, v[cur], tile_offsets, n_tiles,
                            n, lists);
-        // the listed segments: fixed grids, a workgroup with no list entry ends at once
-        if (n > 512)
-            hipLaunchKernelGGL(sort_segments_small_kernel, dim3(n_tiles < 2048 ? n_tiles : 2048), dim3(256), 0, s, kc, v[cur],
-                               tile_offsets, n_tiles, n, lists);
     } else {
-        hipLaunchKernelGGL((sort_segments_direct_kernel<4, 4>), dim3(n_tiles), dim3(256), 0, s, kc, v[cur], tile_offsets,
-                           n_tiles, n, lists);
+        // 8 keys per lane sort segments of up to 2048 keys directly, at the price of a slower kernel for short
+        // segments: worth it where the mean segment is long
+        if (n / n_tiles > 512)
+            hipLaunchKernelGGL((sort_segments_direct_kernel<4, 8>), dim3(n_tiles), dim3(256), 0, s, kc, v[cur], tile_offsets,
+                               n_tiles, n, lists);
+        else
+            hipLaunchKernelGGL((sort_segments_direct_kernel<4, 4>), dim3(n_tiles), dim3(256), 0, s, kc, v[cur], tile_offsets,
+                               n_tiles, n, lists);
     }
-    if (n > kSegCap0)
+    // the listed segments: fixed grids, a workgroup with no list entry ends at once
+    if (lone_waves && n > 512)   // four wavefronts sort class 0 directly otherwise
+        hipLaunchKernelGGL(sort_segments_small_kernel, dim3(n_tiles < 2048 ? n_tiles : 2048), dim3(256), 0, s, kc, v[cur],
+                           tile_offsets, n_tiles, n, lists);
+    if (n > (lone_waves ? kSegCap0 : 1024))
         hipLaunchKernelGGL(sort_segments_long_kernel, dim3(n_tiles < 512 ? n_tiles : 512), dim3(kSegGlobalWaves * 64), 0, s, kc,
                            v[cur], ka, v[cur ^ 1], tile_offsets, n_tiles, n, lists);
     SSR_CHECK_LAUNCH("ssr_sort_tile_pairs");
