@@ -188,17 +188,65 @@ inline size_t packed_stage_layout(int64_t n, void* base, PackedStage* st) {
 // projected geometry of the visible splats is kept: compacted in splat order within the
 // workgroup's segment of the staging area (ballot ranks inside a wavefront, wavefront totals through
 // LDS), so that the second pass never touches a culled splat.
+// A pinhole view is sparse when the camera stands inside the scene, and this kernel is bound by the projection's
+// arithmetic, not by memory: so a first pass reads only the mean and the scales, rejects what is certainly
+// behind the camera or off the image, and, when under five eighths of the workgroup's splats remain, compacts
+// them in splat order so that the projection runs on dense wavefronts. The test is one-sided: z <= 0 is the
+// projection's own rule on the identically computed z; the screen radius is bounded by
+// 3.33 sqrt(s_max^2 |J row|^2 + blur) with |J row|^2 <= (f^2 + L^2) / z^2, L the clamp of J[.][2]
+// (clamp_pinhole_jacobian), enlarged by 1 % and a pixel, so whatever is rejected here the projection's
+// off-image test rejects as well; anything unordered (NaN) is kept.
+__device__ __forceinline__ bool pinhole_may_be_visible(const CamD& cam, const ssr_world& W, int64_t g) {
+    const float* m = W.means + 3 * g;
+    const float mean[3] = {m[0], m[1], m[2]};
+    float mc[3];
+#pragma unroll
+    for (int i = 0; i < 3; i++)
+        mc[i] = ((cam.R[i][0] * mean[0] + cam.R[i][1] * mean[1]) + cam.R[i][2] * mean[2]) + cam.t[i];
+    const float z = mc[2];
+    if (z <= 0.0f) return false;
+    const float* sc = W.log_scales + 3 * g;
+    const float smax = __builtin_amdgcn_exp2f(ssr_max(sc[0], ssr_max(sc[1], sc[2])) * 1.44269504f) * 1.001f;   // hardware exp2, an ulp off at most
+    const float lim_pos = cam.Wf + 0.3f * (0.5f * cam.Wf), lim_neg = 0.3f * (0.5f * cam.Wf);
+    const float Lx = ssr_max(lim_pos - cam.cx, lim_neg + cam.cx), Ly = ssr_max(lim_pos - cam.cy, lim_neg + cam.cy);
+    const float rz = 1.0f / z, sz = smax * rz;
+    const float Rx = 3.33f * 1.01f * ssr_sqrt((sz * sz) * (cam.fx * cam.fx + Lx * Lx) + 0.3f) + 1.0f;
+    const float Ry = 3.33f * 1.01f * ssr_sqrt((sz * sz) * (cam.fy * cam.fy + Ly * Ly) + 0.3f) + 1.0f;
+    const float u = cam.fx * (mc[0] * rz) + cam.cx, v = cam.fy * (mc[1] * rz) + cam.cy;
+    return !(u + Rx < 0.0f || u - Rx > cam.Wf || v + Ry < 0.0f || v - Ry > cam.Hf);
+}
+
 template <bool kLens>
 __global__ __launch_bounds__(kProjBlock) void projection_packed_mask_kernel(ssr_projection_packed_params P, PackedStage S) {
     __shared__ int s_wave[kProjBlock / 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t block0 = (int64_t)blockIdx.x * kProjBlock;
-    const int64_t g = block0 + threadIdx.x;
+    int64_t g = block0 + threadIdx.x;
     CamD cam = load_camera(P.camera);
     cam.aa = P.antialiased != 0;
+    bool work = g < P.num_splats;
+    if (!kLens && cam.model == SSR_CAM_PINHOLE) {
+        __shared__ int s_pre[kProjBlock / 64];
+        __shared__ int s_cand[kProjBlock];
+        const bool keep = work && pinhole_may_be_visible(cam, P.world, g);
+        const unsigned long long km = __ballot(keep);
+        if (lane == 0) s_pre[wave] = __popcll(km);
+        __syncthreads();
+        int kbase = 0, ktotal = 0;
+#pragma unroll
+        for (int w = 0; w < kProjBlock / 64; w++) { if (w < wave) kbase += s_pre[w]; ktotal += s_pre[w]; }
+        work = keep;
+        if (ktotal * 8 <= kProjBlock * 5) {   // the same for the whole workgroup
+            if (keep) s_cand[kbase + __popcll(km & ((1ull << lane) - 1ull))] = threadIdx.x;
+            __syncthreads();
+            work = (int)threadIdx.x < ktotal;   // candidates stay in splat order, so the ranks below do too
+            if (work) g = block0 + s_cand[threadIdx.x];
+        }
+    }
     bool vis = false;
     ProjD p;
     float bb[4] = {0.f, 0.f, 0.f, 0.f};
-    if (g < P.num_splats) {
+    if (work) {
         float mean[3], quat[4], ls[3], logit;
         load_splat(P.world, g, mean, quat, ls, logit);
         project<false, kLens>(cam, mean, quat, ls, logit, p);
@@ -209,7 +257,6 @@ __global__ __launch_bounds__(kProjBlock) void projection_packed_mask_kernel(ssr_
         vis = bb[2] - bb[0] > 1e-3f && bb[3] - bb[1] > 1e-3f;   // ProjectionPackedFwd_kernel.cuh:93
     }
     const unsigned long long m = __ballot(vis);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int rank = __popcll(m & ((1ull << lane) - 1ull));
     if (lane == 0) s_wave[wave] = __popcll(m);
     __syncthreads();
@@ -240,18 +287,21 @@ __global__ __launch_bounds__(kScanOneBlock) void packed_block_scan_kernel(const 
                                                                           int64_t* __restrict__ offsets, int64_t* __restrict__ nnz) {
     __shared__ int s_wave[2][kScanOneBlock / 64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    auto load4 = [&](int64_t base, int v[4]) {
+    constexpr int kPer = 4;
+    auto load_run = [&](int64_t base, int v[kPer]) {
 #pragma unroll
-        for (int k = 0; k < 4; k++) v[k] = base + k < nb ? counts[base + k] : 0;
+        for (int k = 0; k < kPer; k++) v[k] = base + k < nb ? counts[base + k] : 0;
     };
     long long carry = 0;
-    int cur[4], nxt[4];
-    load4((int64_t)threadIdx.x * 4, cur);
+    int cur[kPer], nxt[kPer];
+    load_run((int64_t)threadIdx.x * kPer, cur);
     int parity = 0;
-    for (int64_t tile0 = 0; tile0 < nb; tile0 += 4 * kScanOneBlock, parity ^= 1) {
-        const int64_t base = tile0 + (int64_t)threadIdx.x * 4;
-        load4(base + 4 * kScanOneBlock, nxt);
-        const int mine = (cur[0] + cur[1]) + (cur[2] + cur[3]);
+    for (int64_t tile0 = 0; tile0 < nb; tile0 += kPer * kScanOneBlock, parity ^= 1) {
+        const int64_t base = tile0 + (int64_t)threadIdx.x * kPer;
+        load_run(base + kPer * kScanOneBlock, nxt);
+        int mine = 0;
+#pragma unroll
+        for (int k = 0; k < kPer; k++) mine += cur[k];
         int incl = mine;   // inclusive scan over the wavefront
 #pragma unroll
         for (int d = 1; d < 64; d <<= 1) {
@@ -269,13 +319,13 @@ __global__ __launch_bounds__(kScanOneBlock) void packed_block_scan_kernel(const 
         }
         long long acc = carry + before + (incl - mine);
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
+        for (int k = 0; k < kPer; k++) {
             if (base + k < nb) offsets[base + k] = acc;
             acc += cur[k];
         }
         carry += total;
 #pragma unroll
-        for (int k = 0; k < 4; k++) cur[k] = nxt[k];
+        for (int k = 0; k < kPer; k++) cur[k] = nxt[k];
     }
     if (threadIdx.x == 0) { offsets[nb] = carry; *nnz = carry; }
 }
@@ -1194,6 +1244,30 @@ __global__ __launch_bounds__(kProjBlock) void packed_row_map_kernel(const int32_
 
 // One wavefront per listed splat: lane l zeroes float l of its 59-float gradient row
 // (3 mean, 4 quat, 3 scale, 1 opacity, 3 dc, sh_stride SH).
+// The first index i in [0, n] with a[i] >= x in the ascending array a, searched outwards from `start` in doubling
+// steps and then by bisection: a few probes when the answer is near the guess, the usual logarithm otherwise.
+__device__ __forceinline__ int64_t first_at_or_above(const int32_t* __restrict__ a, int64_t n, int64_t start, int x) {
+    if (n <= 0) return 0;
+    start = start < 0 ? 0 : (start >= n ? n - 1 : start);
+    int64_t lo, hi, step = 1;
+    if (a[start] < x) {          // the answer lies to the right of start
+        lo = start + 1;
+        int64_t i = start + step;
+        while (i < n && a[i] < x) { lo = i + 1; step <<= 1; i = start + step; }
+        hi = i < n ? i : n;
+    } else {                     // at start or to its left
+        hi = start;
+        int64_t i = start - step;
+        while (i >= 0 && a[i] >= x) { hi = i; step <<= 1; i = start - step; }
+        lo = i >= 0 ? i + 1 : 0;
+    }
+    while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (a[mid] < x) lo = mid + 1; else hi = mid;
+    }
+    return lo;
+}
+
 // Rows of splats that are visible now (non-empty aabb when `aabb` is given, member of the ascending list
 // `keep` when that is given) are skipped: the projection backward that follows overwrites them.
 // A workgroup takes 256 listed rows. First every thread decides about one row: the `keep` list is bracketed
@@ -1227,17 +1301,11 @@ __global__ __launch_bounds__(kProjBlock) void zero_world_rows_kernel(ssr_world V
         __syncthreads();
 #pragma unroll
         for (int w = 0; w < kProjBlock / 64; w++) { gmin = min(gmin, s_lo[w]); gmax = max(gmax, s_hi[w]); }
-        int64_t lo = 0, hi = n_keep;       // first entry >= gmin
-        while (lo < hi) {
-            const int64_t mid = (lo + hi) >> 1;
-            if (keep[mid] < gmin) lo = mid + 1; else hi = mid;
-        }
-        const int64_t first = lo;
-        hi = n_keep;                       // first entry > gmax
-        while (lo < hi) {
-            const int64_t mid = (lo + hi) >> 1;
-            if (keep[mid] <= gmax) lo = mid + 1; else hi = mid;
-        }
+        // lists of two views of one scene name much the same splats at much the same places: guess, then gallop
+        const int64_t row0 = (int64_t)blockIdx.x * kProjBlock;
+        const int64_t first = first_at_or_above(keep, n_keep, row0 * n_keep / n, gmin);
+        const int64_t rows_here = n - row0 < kProjBlock ? n - row0 : kProjBlock;
+        const int64_t lo = first_at_or_above(keep, n_keep, first + rows_here, gmax + 1);   // ids stay below 2^31 - 1
         if (alive) {
             int64_t a = first, b = lo;     // first entry >= g inside the bracket
             while (a < b) {

@@ -470,6 +470,7 @@ __global__ __launch_bounds__(kSegGlobalWaves * 64) void sort_segments_long_kerne
     __shared__ uint32_t s_next;
     static_assert(kSegCap1 == kSegGlobalWaves * 64 * 8, "class 1 is sorted by sixteen wavefronts with 8 keys per lane");
     const uint32_t count1 = lists.counts[1], count2 = lists.counts[2];
+    if (count1 + count2 == 0) return;   // nothing listed: no workgroup touches the cursor
     for (;;) {
         if (threadIdx.x == 0) s_next = atomicAdd(&lists.counts[3], 1u);
         __syncthreads();

@@ -424,6 +424,29 @@ def test_packed_projection_sparse_and_dense(gpu, oracle):
     _compare_packed(gpu, oracle, sc, "pk-cfg5")
 
 
+def test_packed_projection_first_pass_cull(gpu, oracle):
+    """The packed mask kernel first rejects splats from the mean and the scales alone and compacts the rest when
+    few remain: it may only reject what the projection rejects. Splats straddling every image edge with centres
+    far off the image, very large splats, splats just in front of and just behind the camera plane, workgroups
+    on both sides of the compaction threshold: rows, ids and the whole chain as the oracle's."""
+    S = gpu.scenes
+    sc = S.tiny_scene(n=3000, width=96, height=64, seed=31)
+    sc.means[:, :2] *= 8.0                      # most centres off the image, many footprints reaching back in
+    sc.log_scales[::5] += 2.0                   # some very large ones
+    g, r = _compare_packed(gpu, oracle, sc, "pk-cull-edges", fused_count=True)
+    assert 0 < g.nnz < 0.8 * sc.n
+    sc = S.tiny_scene(n=2048, width=96, height=64, seed=32)
+    cam_z = (sc.means @ sc.viewmat[2, :3]) + sc.viewmat[2, 3]
+    sc.means -= np.outer(cam_z - np.where(np.arange(sc.n) % 2, 1e-3, -1e-3) * (1 + np.arange(sc.n) % 7), sc.viewmat[2, :3]) * (np.arange(sc.n) % 3 == 0)[:, None]
+    _compare_packed(gpu, oracle, sc, "pk-cull-camera-plane")
+    sc = S.tiny_scene(n=256 * 6, width=96, height=64, seed=33)
+    blk = np.arange(sc.n) // 256
+    for b, share in enumerate([0.0, 0.3, 0.6, 0.65, 0.9, 1.0]):   # share of a workgroup's splats in front of the camera
+        idx = np.where(blk == b)[0]
+        sc.means[idx[int(share * idx.size):], 2] = -10.0
+    _compare_packed(gpu, oracle, sc, "pk-cull-threshold", fused_count=True)
+
+
 def test_packed_projection_all_culled_and_empty(gpu, oracle):
     sc = gpu.scenes.tiny_scene(n=300, width=40, height=24, seed=1)
     sc.means[:, 2] = -10.0
