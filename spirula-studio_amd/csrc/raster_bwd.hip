@@ -376,7 +376,7 @@ constexpr int kDppQuadXor2 = 0x4E, kDppQuadXor1 = 0xB1;
 constexpr int kRowBatch = 128;   // fragments staged per batch by the row-granular kernel
 
 __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raster_bwd_params P, int tile_w, int tile_h) {
-    __shared__ FragLds frags[kRowBatch];
+    __shared__ FragLds frags[kRowBatch + 1];   // the last one is the blank fragment that ends every list
     __shared__ int32_t s_ids[kRowBatch];
     __shared__ int s_wave_max[4];
     // Moment sums per (wavefront, fragment, channel). Each wavefront adds into its own copy with a plain
@@ -430,7 +430,16 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
     if (!b0) chan = 4 * (b1 ? 1 : 0) + 2 * (b2 ? 1 : 0) + (b3 ? 1 : 0);
     else if (!b1 && !b2) chan = 8 + (b3 ? 1 : 0);
     for (int e = tid; e < 4 * kRowBatch * 10; e += kRasterBlock) s_acc[e] = 0.0f;
+    // A list is read without asking where it ends: behind its entries stands slot kRowBatch, a fragment of opacity
+    // zero, which no pixel takes up and whose sums stay zero. The tail of the last list is filled here, the rest by
+    // each wavefront before it builds its lists (the first barrier of the batch loop orders this with the reads).
+    for (int e = tid; e < (int)sizeof(s_list); e += kRasterBlock) s_list[e] = (uint8_t)kRowBatch;
+    if (tid == 0) {
+        const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+        frags[kRowBatch].q0 = z; frags[kRowBatch].q1 = z; frags[kRowBatch].q2 = z;
+    }
     float* my_acc = s_acc + mt * (kRowBatch * 10);
+    char* my_cells = reinterpret_cast<char*>(my_acc + (chan >= 0 ? chan : 0));   // + 40 bytes per fragment slot
 
     // Two neighbouring threads own fragment slot t / 2: they add up the four wavefronts' moment sums, turn
     // them into the ten gradient channels (x, y, depth, conic[3], opac, rgb[3]) and leave those in the first
@@ -533,6 +542,8 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
         // not beyond the block's largest last_id
         const int n_batch = min(kRowBatch, hi - range_start + 1);
         int cnt[4] = {0, 0, 0, 0};
+        static_assert(4 * kRowBatch == 64 * 8, "one 8-byte store per lane blanks the wavefront's four lists");
+        reinterpret_cast<uint64_t*>(s_list + 4 * mt * kRowBatch)[lane] = 0x0101010101010101ull * (uint64_t)kRowBatch;
         for (int c = 0; c * 64 < n_batch; c++) {
             const int slot = c * 64 + lane;
             const uint32_t bits = (uint32_t)s_bits[(mt >> 1) * kRowBatch + slot] >> (4 * (mt & 1));
@@ -547,7 +558,6 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
         // the lists are written and read by this wavefront only: order its LDS accesses, no workgroup barrier
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        const int my_cnt = row == 0 ? cnt[0] : row == 1 ? cnt[1] : row == 2 ? cnt[2] : cnt[3];
         const int n_steps = max(max(cnt[0], cnt[1]), max(cnt[2], cnt[3]));
         // Steps in which two rows of this wavefront sit on the same fragment: their read-add-writes would
         // overwrite each other, so those steps add atomically. One bit per step, found here (lane = step).
@@ -565,21 +575,26 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
             }
         }
         // One step of a row: fragment k (registers q*) against the row's sixteen pixels.
+        const int k_min = hi - bin_final;
         auto step = [&](int st, int k, const float4& q0, const float4& q1, const float2& q2, float cut) {
-            const bool in_list = st < my_cnt;
-            const int32_t sorted_idx = hi - k;
             const float dx = q0.x - px, dy = q0.y - py;
             const float sigma = ssr_fma(q0.z * dx, dx, ssr_fma(q1.x * dy, dy, (q0.w * dx) * dy));
-            const bool in_range = !(sigma < 0.f || sigma > cut);
+            // a lane on a fragment behind its pixel's last one (sorted index hi - k > bin_final) runs with vis = 0, and
+            // the blank fragment past the end of a list has opacity zero: alpha = 0 either way, and one comparison
+            // decides about the lane
+            const bool in_range = (k >= k_min) & !(sigma < 0.f || sigma > cut);
             float vis = in_range ? __builtin_amdgcn_exp2f(sigma * -1.44269504088896341f) : 0.0f;
             float ov = q1.y * vis;
-            const bool near_edge = in_list & ((ssr_fabs(ov - kAlphaThreshold) <= 1.6e-7f) | (ssr_fabs(ov - 0.999f) <= 4e-5f));
+            const bool near_edge = (ssr_fabs(ov - kAlphaThreshold) <= 1.6e-7f) | (ssr_fabs(ov - 0.999f) <= 4e-5f);
             if (__builtin_amdgcn_ballot_w64(near_edge) != 0ull) {   // decisions exactly as the forward took them
                 vis = in_range ? exp_neg_small(-sigma) : 0.0f;
                 ov = q1.y * vis;
             }
-            const float alpha = ssr_min(0.999f, ov);
-            const bool active = in_list & (sorted_idx <= bin_final) & (alpha > kAlphaThreshold);
+            // min(0.999, ov) as the one instruction it is (a NaN ov gives 0.999, as ssr_min does); the compiler's own
+            // minimum spends a second instruction on quieting a signalling NaN first
+            float alpha;
+            asm("v_min_f32 %0, %1, %2" : "=v"(alpha) : "s"(0.999f), "v"(ov));
+            const bool active = alpha > kAlphaThreshold;
             if (__builtin_amdgcn_ballot_w64(active) != 0ull) {
                 // inactive lanes run with alpha = 0 and v_alpha = 0: T and v_T unchanged, every term zero
                 const float a = active ? alpha : 0.0f;
@@ -621,9 +636,9 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
                     : "v"(u), "v"(ux), "v"(uy), "v"(uxx), "v"(uxy), "v"(uyy), "v"(wr), "v"(wg), "v"(wb), "v"(wd));
                 const float t0 = fold_pair<kDppQuadXor2>(s0, s1, b1), t1 = s2 + dpp_full<kDppQuadXor2>(s2);
                 const float fin_sum = fold_pair<kDppQuadXor1>(t0, t1, b0);
-                const bool mine = (chan >= 0) & in_list & ssr_isfinite(fin_sum) & (fin_sum != 0.0f);
+                const bool mine = (chan >= 0) & ssr_isfinite(fin_sum) & (fin_sum != 0.0f);
                 const bool clash = (((st < 64 ? clash_lo : clash_hi) >> (st & 63)) & 1ull) != 0;
-                float* cell = my_acc + k * 10 + (chan >= 0 ? chan : 0);
+                float* cell = reinterpret_cast<float*>(my_cells + __umul24((unsigned)k, 40u));
                 if (clash) { if (mine) atomicAdd(cell, fin_sum); }
                 else if (mine) *cell += fin_sum;
             }
@@ -631,20 +646,24 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
         // Software pipeline, two steps per trip: list bytes run two steps ahead of their use and the fragment of the
         // next step loads while the current one computes, so that the two dependent LDS latencies hide behind
         // arithmetic; the two fragment register sets alternate, so nothing is copied between steps.
-        auto list_at = [&](int st) { return st < my_cnt ? (int)my_list[st] : 0; };
+        auto list_at = [&](int st) { return (int)my_list[st]; };   // past the end: some valid slot, never used
+        // slots are below 128: a 24-bit multiply (full rate) addresses the fragment, not the quarter-rate 32-bit one
+        auto frag_of = [&](int k) -> const FragLds& {
+            return *reinterpret_cast<const FragLds*>(reinterpret_cast<const char*>(frags) + __umul24((unsigned)k, (unsigned)sizeof(FragLds)));
+        };
         int k0 = list_at(0), k1 = list_at(1), k2 = list_at(2);
-        float4 a0 = frags[k0].q0, a1 = frags[k0].q1;
-        float2 a2 = make_float2(frags[k0].q2.x, frags[k0].q2.y);
-        float aw = frags[k0].q2.w;
+        float4 a0 = frag_of(k0).q0, a1 = frag_of(k0).q1;
+        float2 a2 = make_float2(frag_of(k0).q2.x, frag_of(k0).q2.y);
+        float aw = frag_of(k0).q2.w;
         for (int st = 0; st < n_steps; st += 2) {
-            const float4 c0 = frags[k1].q0, c1 = frags[k1].q1;
-            const float2 c2 = make_float2(frags[k1].q2.x, frags[k1].q2.y);
-            const float cw = frags[k1].q2.w;
+            const float4 c0 = frag_of(k1).q0, c1 = frag_of(k1).q1;
+            const float2 c2 = make_float2(frag_of(k1).q2.x, frag_of(k1).q2.y);
+            const float cw = frag_of(k1).q2.w;
             const int k3 = list_at(st + 3);
             step(st, k0, a0, a1, a2, aw);
-            a0 = frags[k2].q0; a1 = frags[k2].q1;
-            a2 = make_float2(frags[k2].q2.x, frags[k2].q2.y);
-            aw = frags[k2].q2.w;
+            a0 = frag_of(k2).q0; a1 = frag_of(k2).q1;
+            a2 = make_float2(frag_of(k2).q2.x, frag_of(k2).q2.y);
+            aw = frag_of(k2).q2.w;
             const int k4 = list_at(st + 4);
             if (st + 1 < n_steps) step(st + 1, k1, c0, c1, c2, cw);
             k0 = k2; k1 = k3; k2 = k4;

@@ -135,7 +135,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raste
     const int i = ty * kTile + (mt >> 1) * kMicro + (row >> 1) * kBlock + (l16 >> 2);
     const float px = (float)j + 0.5f, py = (float)i + 0.5f;
     const bool inside = (uint32_t)i < P.height && (uint32_t)j < P.width;
-    bool done = !inside;
+    int alive = inside ? 1 : 0;   // 0 once the pixel has stopped compositing (an int: the loop tests it with one compare)
 
     const int32_t range_start = P.tile_offsets[tile];
     const int32_t range_end = (tile == n_tiles - 1) ? (int32_t)P.n_isects : P.tile_offsets[tile + 1];
@@ -143,10 +143,13 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raste
     uint32_t cur_idx = 0;
     const float tile_x0 = (float)(tx * kTile), tile_y0 = (float)(ty * kTile);
     const uint8_t* my_list = s_list + (4 * mt + row) * kBatch;
+    // list entries are read a few steps ahead without asking whether the list reaches that far: every byte is a valid
+    // slot from the start (the first barrier of the batch loop orders this with the first reads)
+    for (int e = tid; e < (int)sizeof(s_list); e += kRasterBlock) s_list[e] = 0;
 
     for (int32_t batch_start = range_start; batch_start < range_end; batch_start += kBatch) {
         // all pixels of the tile finished: stop (this barrier also fences reuse of the LDS batch)
-        if (__syncthreads_count(done) >= kRasterBlock) break;
+        if (__syncthreads_count(alive == 0) >= kRasterBlock) break;
         const int32_t idx = batch_start + tid;
         if (idx < range_end) {
             float kk;
@@ -159,7 +162,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raste
         __syncthreads();
         const int n_batch = min(kBatch, range_end - batch_start);
         // a row whose sixteen pixels are finished needs no list
-        const uint64_t live = __ballot(!done);
+        const uint64_t live = __ballot(alive != 0);
         const bool row_live[4] = {(live & 0xFFFFull) != 0, (live & 0xFFFF0000ull) != 0, (live & 0xFFFF00000000ull) != 0,
                                   (live & 0xFFFF000000000000ull) != 0};
         int cnt[4] = {0, 0, 0, 0};
@@ -186,7 +189,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raste
         auto step = [&](int st, int k, const float4& q0, const float4& q1, const float2& q2, float cut) {
             float dx, dy, vis, sigma;
             const float alpha = eval_alpha_fast(q0, q1, cut, px, py, dx, dy, vis, sigma);
-            const bool hit = !done & (st < my_cnt) & (alpha > kAlphaThreshold);
+            const bool hit = (alive != 0) & (st < my_cnt) & (alpha > kAlphaThreshold);
             const float next_T = T * (1.0f - alpha);
             const bool keep = hit & (next_T > kTransmitThreshold);
             const float w = keep ? alpha * T : 0.0f;   // a fragment that is not composited adds zero
@@ -194,26 +197,30 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raste
             cd = ssr_fma(q2.y, w, cd);
             cur_idx = keep ? (uint32_t)(batch_start + k) : cur_idx;
             T = keep ? next_T : T;
-            done = done | (hit & !keep);
+            alive = (hit & !keep) ? 0 : alive;
         };
         // Software pipeline, two steps per trip: list bytes run two steps ahead of their use and the fragment of the
         // next step loads while the current one computes, so that the two dependent LDS latencies hide behind
         // arithmetic; the two fragment register sets alternate, so nothing is copied between steps.
-        auto list_at = [&](int st) { return st < my_cnt ? (int)my_list[st] : 0; };
+        auto list_at = [&](int st) { return (int)my_list[st]; };   // past the end: some valid slot, never used
+        // slots are below 256: a 24-bit multiply (full rate) addresses the fragment, not the quarter-rate 32-bit one
+        auto frag_of = [&](int k) -> const FragLds& {
+            return *reinterpret_cast<const FragLds*>(reinterpret_cast<const char*>(frags) + __umul24((unsigned)k, (unsigned)sizeof(FragLds)));
+        };
         int k0 = list_at(0), k1 = list_at(1), k2 = list_at(2);
-        float4 a0 = frags[k0].q0, a1 = frags[k0].q1;
-        float2 a2 = make_float2(frags[k0].q2.x, frags[k0].q2.y);
-        float aw = frags[k0].q2.w;
+        float4 a0 = frag_of(k0).q0, a1 = frag_of(k0).q1;
+        float2 a2 = make_float2(frag_of(k0).q2.x, frag_of(k0).q2.y);
+        float aw = frag_of(k0).q2.w;
         for (int st = 0; st < n_steps; st += 2) {
-            if (__builtin_amdgcn_ballot_w64(!done) == 0ull) break;   // this sub-tile is finished
-            const float4 c0 = frags[k1].q0, c1 = frags[k1].q1;
-            const float2 c2 = make_float2(frags[k1].q2.x, frags[k1].q2.y);
-            const float cw = frags[k1].q2.w;
+            if (__builtin_amdgcn_ballot_w64(alive != 0) == 0ull) break;   // this sub-tile is finished
+            const float4 c0 = frag_of(k1).q0, c1 = frag_of(k1).q1;
+            const float2 c2 = make_float2(frag_of(k1).q2.x, frag_of(k1).q2.y);
+            const float cw = frag_of(k1).q2.w;
             const int k3 = list_at(st + 3);
             step(st, k0, a0, a1, a2, aw);
-            a0 = frags[k2].q0; a1 = frags[k2].q1;
-            a2 = make_float2(frags[k2].q2.x, frags[k2].q2.y);
-            aw = frags[k2].q2.w;
+            a0 = frag_of(k2).q0; a1 = frag_of(k2).q1;
+            a2 = make_float2(frag_of(k2).q2.x, frag_of(k2).q2.y);
+            aw = frag_of(k2).q2.w;
             const int k4 = list_at(st + 4);
             step(st + 1, k1, c0, c1, c2, cw);   // beyond the lists every row is out of its list: nothing happens
             k0 = k2; k1 = k3; k2 = k4;
