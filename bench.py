@@ -296,15 +296,31 @@ def main():
     dom = max(acc, key=acc.get)
     dom_gbs = ab[dom] / (acc[dom] * 1e-3) / 1e9 if acc[dom] > 0 else 0.0
     traffic = None
-    valu_inst = None     # profiled VALU wavefront instructions per launch of the dominant kernel (plain path only)
+    valu_inst = None     # profiled VALU wavefront instructions per launch of the dominant kernel
+    prof = {}
+    # the profiles were taken with this script's default arguments for each config: they describe no other variant
+    default_run = (native and ncam == 1 and tile_sort and args.packed_projection == (cfg == 4) and not args.n and
+                   not (variants or args.fused_optimizer or args.lens != "none" or args.fisheye or args.mip))
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-    if os.path.exists(tpath):
+    if default_run and os.path.exists(tpath):
         try:
-            traffic = json.load(open(tpath)).get(f"config{cfg}", {}).get(dom) if ncam == 1 else None
-            if native and ncam == 1 and not (variants or args.fused_optimizer or args.packed_projection or args.lens != "none" or args.fisheye or args.mip):
-                valu_inst = json.load(open(tpath)).get(f"config{cfg}_valu_wave_instructions", {}).get(dom)
+            prof = json.load(open(tpath))
+            traffic = prof.get(f"config{cfg}", {}).get(dom)
+            valu_inst = prof.get(f"config{cfg}_valu_wave_instructions", {}).get(dom)
         except Exception:
-            traffic = None
+            prof, traffic, valu_inst = {}, None, None
+    # What the sort really does, beside the charged figure of stage_algorithmic_GBs (which prices the reference's
+    # whole-key sweeps): pairs per second through the whole stage, the sweeps done, and the HBM bytes the profile saw
+    sort_info = {"pairs": K, "ms": acc.get("K5", 0.0) + acc.get("K6", 0.0),
+                 "Gpairs_per_s": K / ((acc.get("K5", 0.0) + acc.get("K6", 0.0)) * 1e-3) / 1e9 if acc.get("K5", 0.0) > 0 else None,
+                 "key_sweeps_done": sort_sweeps_done, "key_sweeps_charged": sort_sweeps,
+                 "hbm_bytes_profiled": prof.get(f"config{cfg}", {}).get("K5"),
+                 "hbm_GBs_profiled": (prof[f"config{cfg}"]["K5"] / (acc["K5"] * 1e-3) / 1e9
+                                      if prof.get(f"config{cfg}", {}).get("K5") and acc.get("K5", 0.0) > 0 else None)}
+    at = prof.get(f"config{cfg}_l2_atomic_requests", {})
+    atomic_info = {"l2_atomic_requests_profiled": at or None,
+                   "K8_G_atomic_requests_per_s": (at["K8"] / (acc["K8"] * 1e-3) / 1e9 if at.get("K8") and acc.get("K8", 0.0) > 0 else None),
+                   "note": "K8 adds a fragment's ten gradient floats as one or two row requests (TCC_ATOMIC_sum counts requests, not floats)"}
 
     out = {
         "metric": "fwd+bwd raster iters/sec at 1M SH3 1080p; % of HBM roofline",
@@ -331,6 +347,8 @@ def main():
         "hbm_roofline_frac_whole_iteration": total_bytes / (float(np.median(ms)) * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "algorithmic_bytes_per_iter": total_bytes,
         "sort_sweeps": {"charged": sort_sweeps, "done": sort_sweeps_done},
+        "sort": sort_info,
+        "atomics": atomic_info,
         "stage_ms": {k: round(v, 4) for k, v in acc.items()},
         "stage_algorithmic_GBs": {k: round(ab[k] / (acc[k] * 1e-3) / 1e9, 1) if acc[k] > 0 else None for k in acc},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": dom_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",

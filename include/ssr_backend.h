@@ -17,12 +17,16 @@
  *  - Return value 0 = success. Non-zero = error; the message is kept per thread and returned (and
  *    cleared) by ssr_last_error(), like the reference's sticky backend::last_error()
  *    (src/backend/api/BackendRuntime.h:98). Nothing calls exit().
- *  - Supported variant: primitive "3dgs" (not antialiased), camera PINHOLE or EQUIRECTANGULAR,
- *    distortion NONE, one camera per projection launch (the host layer loops over a [C,4,4] set;
- *    tiling and compositing take the C images in one launch), SH degree 0..3, dist_type None / D / RGB_D, median
- *    depth, accumulation weights; both the [C,N] layout and the packed (compacted, nnz rows) layout of
- *    the projection outputs. Anything else is rejected with an error, as the reference
- *    rejects an uncompiled variant (src/kernels/projection/ProjectionFwd.cu:84-89).
+ *  - Supported variants: primitives "3dgs" and "mip" (the antialiased one: `antialiased` in the projection
+ *    parameter blocks); camera PINHOLE with lens NONE / OPENCV / THIN_PRISM / RATIONAL, FISHEYE and EQUISOLID
+ *    with NONE / OPENCV / THIN_PRISM, EQUIRECTANGULAR with NONE (the reference's own table,
+ *    src/kernels/projection/CameraVariants.cuh:11-22; ssr_camera_variant_supported answers for a pair);
+ *    SH degree 0..3 in fp32 or one of the quantised codecs; dist_type None / D / RGB_D, median depth,
+ *    accumulation weights; the [C,N] layout and the packed (compacted, nnz rows) layout of the projection
+ *    outputs; the projection backward alone or fused with the Adam step. One camera per projection launch:
+ *    the host layer loops over a [C,4,4] set (packed rows ordered by camera, then splat), while tiling,
+ *    sorting and compositing take the C images in one launch. Anything else is rejected with an error, as the
+ *    reference rejects an uncompiled variant (src/kernels/projection/ProjectionFwd.cu:84-89).
  *  - Layouts are the reference's (src/primitives/PrimitiveBase3DGS.cuh:87-139,187-225).
  */
 #ifndef SSR_BACKEND_H
