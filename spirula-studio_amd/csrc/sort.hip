@@ -573,7 +573,9 @@ int ssr_sort_tile_pairs(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, int32
     hipStream_t s = as_stream(stream);
     uint64_t* kc = reinterpret_cast<uint64_t*>(k[cur]);
     uint64_t* ka = reinterpret_cast<uint64_t*>(k[cur ^ 1]);
-    const bool lone_waves = n_tiles >= 16384;   // at least two rounds of one-wavefront workgroups on 256 compute units
+    // one wavefront per tile: at least two rounds of such workgroups on 256 compute units, and segments that mostly fit
+    // its 512 keys (a mean of 336 does, config 5; a mean of 411 with a third of the tiles above 512 does not)
+    const bool lone_waves = n_tiles >= 16384 && n / n_tiles <= 384;
     lists.has_class0 = lone_waves;
     if (lone_waves) {
         hipLaunchKernelGGL((sort_segments_direct_kernel<1, 8>), dim3(n_tiles), dim3(64), 0, s, kc, v[cur], tile_offsets, n_tiles,

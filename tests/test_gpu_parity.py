@@ -437,7 +437,7 @@ def test_packed_projection_first_pass_cull(gpu, oracle):
     assert 0 < g.nnz < 0.8 * sc.n
     sc = S.tiny_scene(n=2048, width=96, height=64, seed=32)
     cam_z = (sc.means @ sc.viewmat[2, :3]) + sc.viewmat[2, 3]
-    sc.means -= np.outer(cam_z - np.where(np.arange(sc.n) % 2, 1e-3, -1e-3) * (1 + np.arange(sc.n) % 7), sc.viewmat[2, :3]) * (np.arange(sc.n) % 3 == 0)[:, None]
+    sc.means -= np.outer(cam_z - np.where(np.arange(sc.n) % 2, 2e-2, -2e-2) * (1 + np.arange(sc.n) % 7), sc.viewmat[2, :3]) * (np.arange(sc.n) % 3 == 0)[:, None]
     _compare_packed(gpu, oracle, sc, "pk-cull-camera-plane")
     sc = S.tiny_scene(n=256 * 6, width=96, height=64, seed=33)
     blk = np.arange(sc.n) // 256
