@@ -12,7 +12,7 @@ WORLD_GRAD_RTOL = 1e-3   # the bar for parameter gradients: 1e-3 of the row's la
 MARGINS = {}             # label -> largest err / rowmax seen, for the report at the end of a run
 
 
-def world_grad_check(got, ref, n, name, rtol=WORLD_GRAD_RTOL, bad_frac=0.0, scale=None):
+def world_grad_check(got, ref, n, name, rtol=WORLD_GRAD_RTOL, bad_frac=0.0, scale=None, row_floor=None):
     """Parameter-gradient bar: |got - ref| <= rtol * max|ref row| + a floor of 2e-5 of the tensor's
     mean magnitude (rows whose terms cancel). Prints the largest observed error relative to the row
     maximum, with and without the floor, so that the margin is on record."""
@@ -22,6 +22,8 @@ def world_grad_check(got, ref, n, name, rtol=WORLD_GRAD_RTOL, bad_frac=0.0, scal
         scale = np.abs(ref).max(axis=1, keepdims=True)
     scale = scale + 1e-30
     floor = 2e-5 * (np.abs(ref).mean() + 1e-12)
+    if row_floor is not None:   # what the summation-order floor of a screen gradient becomes in this row
+        floor = floor + np.asarray(row_floor, np.float64).reshape(n, 1)
     err = np.abs(got - ref)
     raw = float((err / scale).max()) if err.size else 0.0
     over = float((np.maximum(err - floor, 0.0) / scale).max()) if err.size else 0.0
