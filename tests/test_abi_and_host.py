@@ -74,6 +74,20 @@ def test_argument_checks_without_device(L):
     assert lib.ssr_memcpy(None, None, 0, 0, None, 0) == 0
     assert lib.ssr_fill_u32(None, 0, 0, None) == 0
     assert lib.ssr_tile_offsets(-1, None, 4, None, None) != 0 and lib.ssr_last_error() != b""
+    # gradient rows are addressed as 12 * row in 32 bits: more rows than that are refused, not wrapped
+    b = L.RasterBwdParams()
+    b.width = b.height = 16
+    b.n_isects = 1
+    for f in ("tile_offsets", "flatten_ids", "render_T", "last_ids", "render_depth", "v_render_rgb", "v_render_depth",
+              "v_render_T", "packed_rows", "v_rows"):
+        setattr(b, f, 16)          # non-null, aligned, never read: the check comes before any launch
+    b.num_splats = 0xFFFFFFFF // 12 + 1
+    assert lib.ssr_raster_bwd(C.byref(b), None) != 0 and b"357913941" in lib.ssr_last_error()
+    b.num_splats = 1 << 30
+    assert lib.ssr_raster_bwd(C.byref(b), None) != 0 and b"2^30" in lib.ssr_last_error()
+    # the allocation-free scan refuses what its fixed scratch cannot hold
+    assert lib.ssr_inclusive_sum_i64_static(16, 16, (1 << 27) + 1, None, None) != 0 and b"static" in lib.ssr_last_error()
+    assert lib.ssr_zero_world_rows(None, None, 0, None, None, 0, None) != 0 and b"null world" in lib.ssr_last_error()
 
 
 def test_missing_library_fails_loudly(pkg, monkeypatch):
