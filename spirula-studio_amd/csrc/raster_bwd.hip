@@ -375,14 +375,21 @@ constexpr int kDppQuadXor2 = 0x4E, kDppQuadXor1 = 0xB1;
 
 constexpr int kRowBatch = 128;   // fragments staged per batch by the row-granular kernel
 
+// kAccum: the pixel-weight accumulation of the densifier (RasterizationEval3DBwd_kernel.cuh:553-562,574-585). Sum and
+// average ride as two more channels (map * w and w) through the same reduction, in lanes that hold copies otherwise;
+// the maximum takes a reduction of its own.
+template <int kAccum>
 __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raster_bwd_params P, int tile_w, int tile_h) {
+    constexpr bool kSums = kAccum == SSR_ACCUM_SUM || kAccum == SSR_ACCUM_AVG;
+    constexpr int kCh = kSums ? 12 : 10;   // channels per fragment slot
     __shared__ FragLds frags[kRowBatch + 1];   // the last one is the blank fragment that ends every list
     __shared__ int32_t s_ids[kRowBatch];
     __shared__ int s_wave_max[4];
     // Moment sums per (wavefront, fragment, channel). Each wavefront adds into its own copy with a plain
     // read-add-write: a float atomic in LDS costs about three cycles per active lane on this hardware,
     // which at forty lanes a step would make LDS, not arithmetic, the limit of this kernel.
-    __shared__ float s_acc[4 * kRowBatch * 10];
+    __shared__ float s_acc[4 * kRowBatch * kCh];
+    [[maybe_unused]] __shared__ float s_max[kAccum == SSR_ACCUM_MAX ? 4 * kRowBatch : 1];   // per wavefront and slot: largest map * w
     __shared__ uint8_t s_bits[2 * kRowBatch];                       // block bits of sub-tiles {0,1} and {2,3}
     __shared__ uint8_t s_list[kBlocksPerTile * kRowBatch + 16];
     const int n_tiles = tile_w * tile_h * (P.num_images > 1 ? P.num_images : 1);
@@ -409,6 +416,8 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
         vT1 = vT1 + (P.render_depth[pid] * vd) * inv_alpha;
         vd = vd * inv_alpha;
     }
+    [[maybe_unused]] float amap = 0.0f;
+    if constexpr (kAccum != SSR_ACCUM_NONE) amap = inside ? P.accum_weight_map[pid] : 0.0f;
 
     const int32_t range_start = P.tile_offsets[tile];
     const int32_t range_end = (tile == n_tiles - 1) ? (int32_t)P.n_isects : P.tile_offsets[tile + 1];
@@ -428,8 +437,9 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
     const bool b3 = (l16 & 8) != 0, b2 = (l16 & 4) != 0, b1 = (l16 & 2) != 0, b0 = (l16 & 1) != 0;
     int chan = -1;
     if (!b0) chan = 4 * (b1 ? 1 : 0) + 2 * (b2 ? 1 : 0) + (b3 ? 1 : 0);
-    else if (!b1 && !b2) chan = 8 + (b3 ? 1 : 0);
-    for (int e = tid; e < 4 * kRowBatch * 10; e += kRasterBlock) s_acc[e] = 0.0f;
+    else if (!b1 && (!b2 || kSums)) chan = 8 + 2 * (b2 ? 1 : 0) + (b3 ? 1 : 0);
+    for (int e = tid; e < 4 * kRowBatch * kCh; e += kRasterBlock) s_acc[e] = 0.0f;
+    if constexpr (kAccum == SSR_ACCUM_MAX) { for (int e = tid; e < 4 * kRowBatch; e += kRasterBlock) s_max[e] = 0.0f; }
     // A list is read without asking where it ends: behind its entries stands slot kRowBatch, a fragment of opacity
     // zero, which no pixel takes up and whose sums stay zero. The tail of the last list is filled here, the rest by
     // each wavefront before it builds its lists (the first barrier of the batch loop orders this with the reads).
@@ -438,8 +448,8 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
         const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
         frags[kRowBatch].q0 = z; frags[kRowBatch].q1 = z; frags[kRowBatch].q2 = z;
     }
-    float* my_acc = s_acc + mt * (kRowBatch * 10);
-    char* my_cells = reinterpret_cast<char*>(my_acc + (chan >= 0 ? chan : 0));   // + 40 bytes per fragment slot
+    float* my_acc = s_acc + mt * (kRowBatch * kCh);
+    char* my_cells = reinterpret_cast<char*>(my_acc + (chan >= 0 ? chan : 0));   // + 4 kCh bytes per fragment slot
 
     // Two neighbouring threads own fragment slot t / 2: they add up the four wavefronts' moment sums, turn
     // them into the ten gradient channels (x, y, depth, conic[3], opac, rgb[3]) and leave those in the first
@@ -450,17 +460,17 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
             const int slot = tid >> 1;
             const bool geom = (tid & 1) == 0;   // this thread: u, ux, uy, uxx, uxy, uyy; its neighbour: the colour / depth weights
             float m[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            const int c0 = geom ? 0 : 6, nc = geom ? 6 : 4;
+            const int c0 = geom ? 0 : 6, nc = geom ? 6 : kCh - 6;
 #pragma unroll
             for (int w = 0; w < 4; w++)
 #pragma unroll
                 for (int c = 0; c < 6; c++)
-                    if (c < nc) { m[c] += s_acc[(w * kRowBatch + slot) * 10 + c0 + c]; }
+                    if (c < nc) { m[c] += s_acc[(w * kRowBatch + slot) * kCh + c0 + c]; }
 #pragma unroll
             for (int w = 1; w < 4; w++)
 #pragma unroll
                 for (int c = 0; c < 6; c++)
-                    if (c < nc) s_acc[(w * kRowBatch + slot) * 10 + c0 + c] = 0.0f;
+                    if (c < nc) s_acc[(w * kRowBatch + slot) * kCh + c0 + c] = 0.0f;
             float o[6];
             if (geom) {
                 const float4 q0 = frags[slot].q0, q1 = frags[slot].q1;
@@ -474,7 +484,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
                 o[0] = m[3]; o[1] = m[0]; o[2] = m[1]; o[3] = m[2]; o[4] = 0.f; o[5] = 0.f;
             }
             // both threads of a slot sit in one wavefront, so every read above precedes these writes
-            float* dst = s_acc + slot * 10;
+            float* dst = s_acc + slot * kCh;
             if (geom) {
                 dst[0] = ssr_isfinite(o[0]) ? o[0] : 0.f; dst[1] = ssr_isfinite(o[1]) ? o[1] : 0.f;
                 dst[3] = ssr_isfinite(o[2]) ? o[2] : 0.f; dst[4] = ssr_isfinite(o[3]) ? o[3] : 0.f;
@@ -483,15 +493,16 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
                 dst[2] = ssr_isfinite(o[0]) ? o[0] : 0.f;
                 dst[7] = ssr_isfinite(o[1]) ? o[1] : 0.f; dst[8] = ssr_isfinite(o[2]) ? o[2] : 0.f;
                 dst[9] = ssr_isfinite(o[3]) ? o[3] : 0.f;
+                if constexpr (kSums) { dst[10] = ssr_isfinite(m[4]) ? m[4] : 0.f; dst[11] = ssr_isfinite(m[5]) ? m[5] : 0.f; }
             }
         }
         __syncthreads();
         if (P.v_rows) {
             for (int e = tid; e < kRowBatch * 10; e += kRasterBlock) {
                 const int slot = e / 10, ch = e - slot * 10;
-                const float x = s_acc[e];
+                const float x = s_acc[slot * kCh + ch];
                 if (x != 0.0f) {
-                    s_acc[e] = 0.0f;
+                    s_acc[slot * kCh + ch] = 0.0f;
                     atomicAdd(P.v_rows + (int64_t)12 * s_ids[slot] + ch, x);
                 }
             }
@@ -499,10 +510,10 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
             float v[10];
             bool any = false;
 #pragma unroll
-            for (int c = 0; c < 10; c++) { v[c] = s_acc[tid * 10 + c]; any |= v[c] != 0.0f; }
+            for (int c = 0; c < 10; c++) { v[c] = s_acc[tid * kCh + c]; any |= v[c] != 0.0f; }
             if (any) {
 #pragma unroll
-                for (int c = 0; c < 10; c++) s_acc[tid * 10 + c] = 0.0f;
+                for (int c = 0; c < 10; c++) s_acc[tid * kCh + c] = 0.0f;
                 const int64_t g = s_ids[tid];
                 auto add = [](float* p, float x) { if (x != 0.0f) atomicAdd(p, x); };
                 add(P.v_screen.xy + 2 * g, v[0]); add(P.v_screen.xy + 2 * g + 1, v[1]);
@@ -510,6 +521,25 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
                 add(P.v_screen.conic + 3 * g, v[3]); add(P.v_screen.conic + 3 * g + 1, v[4]); add(P.v_screen.conic + 3 * g + 2, v[5]);
                 add(P.v_screen.opac + g, v[6]);
                 add(P.v_screen.rgb + 3 * g, v[7]); add(P.v_screen.rgb + 3 * g + 1, v[8]); add(P.v_screen.rgb + 3 * g + 2, v[9]);
+            }
+        }
+        if constexpr (kSums) {   // the weight sums of slot t leave with thread t
+            if (tid < kRowBatch) {
+                const float a = s_acc[tid * kCh + 10], b = s_acc[tid * kCh + 11];
+                if (a != 0.0f || b != 0.0f) {
+                    s_acc[tid * kCh + 10] = 0.0f; s_acc[tid * kCh + 11] = 0.0f;
+                    const int64_t wid = accum_row(P, (uint32_t)s_ids[tid]);
+                    if (a != 0.0f) atomicAdd(P.accum_weight + wid, a);
+                    if (kAccum == SSR_ACCUM_AVG && b != 0.0f) atomicAdd(P.accum_weight + P.num_world + wid, b);
+                }
+            }
+        }
+        if constexpr (kAccum == SSR_ACCUM_MAX) {
+            if (tid < kRowBatch) {
+                float mx = 0.0f;
+#pragma unroll
+                for (int w = 0; w < 4; w++) { mx = ssr_max(mx, s_max[w * kRowBatch + tid]); s_max[w * kRowBatch + tid] = 0.0f; }
+                if (mx > 0.0f) atomic_max_f32(P.accum_weight + accum_row(P, (uint32_t)s_ids[tid]), mx);   // the running maximum starts at 0
             }
         }
         __syncthreads();   // s_ids, frags and s_acc are free for the next batch
@@ -615,6 +645,34 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
                 // of four likewise with the half-mirror pairing. s_nop covers the two wait states a DPP read needs
                 // after a write of its source by the instruction before; inside the block the reads trail the writes.
                 float r0, r1, r2, r3, r4, s0, s1, s2;
+                if constexpr (kSums) {
+                    // a sixth pair (map * w, w): its first level joins the others, its second shares s2's instruction
+                    // slot pattern (banks 1 and 3), and the quad levels below carry it at no cost
+                    const float aw = amap * w;
+                    float r5;
+                    asm volatile(
+                        "s_nop 1\n\t"
+                        "v_add_f32_dpp %0, %9, %9 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+                        "v_add_f32_dpp %0, %10, %10 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                        "v_add_f32_dpp %1, %11, %11 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+                        "v_add_f32_dpp %1, %12, %12 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                        "v_add_f32_dpp %2, %13, %13 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+                        "v_add_f32_dpp %2, %14, %14 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                        "v_add_f32_dpp %3, %15, %15 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+                        "v_add_f32_dpp %3, %16, %16 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                        "v_add_f32_dpp %4, %17, %17 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+                        "v_add_f32_dpp %4, %18, %18 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                        "v_add_f32_dpp %5, %19, %19 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+                        "v_add_f32_dpp %5, %20, %20 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                        "v_add_f32_dpp %6, %0, %0 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+                        "v_add_f32_dpp %6, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+                        "v_add_f32_dpp %7, %2, %2 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+                        "v_add_f32_dpp %7, %3, %3 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+                        "v_add_f32_dpp %8, %4, %4 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+                        "v_add_f32_dpp %8, %5, %5 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+                        : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3), "=&v"(r4), "=&v"(r5), "=&v"(s0), "=&v"(s1), "=&v"(s2)
+                        : "v"(u), "v"(ux), "v"(uy), "v"(uxx), "v"(uxy), "v"(uyy), "v"(wr), "v"(wg), "v"(wb), "v"(wd), "v"(aw), "v"(w));
+                } else {
                 asm volatile(
                     "s_nop 1\n\t"
                     "v_add_f32_dpp %0, %8, %8 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
@@ -634,13 +692,26 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
                     "v_add_f32_dpp %7, %4, %4 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
                     : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3), "=&v"(r4), "=&v"(s0), "=&v"(s1), "=&v"(s2)
                     : "v"(u), "v"(ux), "v"(uy), "v"(uxx), "v"(uxy), "v"(uyy), "v"(wr), "v"(wg), "v"(wb), "v"(wd));
+                }
                 const float t0 = fold_pair<kDppQuadXor2>(s0, s1, b1), t1 = s2 + dpp_full<kDppQuadXor2>(s2);
                 const float fin_sum = fold_pair<kDppQuadXor1>(t0, t1, b0);
                 const bool mine = (chan >= 0) & ssr_isfinite(fin_sum) & (fin_sum != 0.0f);
                 const bool clash = (((st < 64 ? clash_lo : clash_hi) >> (st & 63)) & 1ull) != 0;
-                float* cell = reinterpret_cast<float*>(my_cells + __umul24((unsigned)k, 40u));
+                float* cell = reinterpret_cast<float*>(my_cells + __umul24((unsigned)k, 4u * kCh));
                 if (clash) { if (mine) atomicAdd(cell, fin_sum); }
                 else if (mine) *cell += fin_sum;
+                if constexpr (kAccum == SSR_ACCUM_MAX) {   // inactive lanes contribute map * 0
+                    float mx = amap * w;
+                    mx = ssr_max(mx, dpp_full<0x128>(mx));   // row_ror:8
+                    mx = ssr_max(mx, dpp_full<0x141>(mx));   // row_half_mirror
+                    mx = ssr_max(mx, dpp_full<kDppQuadXor2>(mx));
+                    mx = ssr_max(mx, dpp_full<kDppQuadXor1>(mx));
+                    if (l16 == 0 && mx > 0.0f) {   // non-negative floats order as their bit patterns
+                        int* mc = reinterpret_cast<int*>(s_max + mt * kRowBatch + k);
+                        if (clash) atomicMax(mc, __float_as_int(mx));
+                        else *mc = max(*mc, __float_as_int(mx));
+                    }
+                }
             }
         };
         // Software pipeline, two steps per trip: list bytes run two steps ahead of their use and the fragment of the
@@ -732,8 +803,13 @@ extern "C" int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t strea
     // The plain variant runs the row-granular kernel; SSR_RASTER_WAVE_VISITS=1 in the environment
     // selects the one-wavefront-per-visit kernel instead (for comparisons).
     static const bool wave_visits = getenv("SSR_RASTER_WAVE_VISITS") != nullptr;
-    if (p->dist_type == SSR_DIST_NONE && !med && p->accum_mode == SSR_ACCUM_NONE && !wave_visits) {
-        hipLaunchKernelGGL(raster_bwd_rows_kernel, grid, block, 0, st, *p, tw, th);
+    if (p->dist_type == SSR_DIST_NONE && !med && !wave_visits) {
+        switch (p->accum_mode) {
+            case SSR_ACCUM_MAX: hipLaunchKernelGGL(raster_bwd_rows_kernel<SSR_ACCUM_MAX>, grid, block, 0, st, *p, tw, th); break;
+            case SSR_ACCUM_SUM: hipLaunchKernelGGL(raster_bwd_rows_kernel<SSR_ACCUM_SUM>, grid, block, 0, st, *p, tw, th); break;
+            case SSR_ACCUM_AVG: hipLaunchKernelGGL(raster_bwd_rows_kernel<SSR_ACCUM_AVG>, grid, block, 0, st, *p, tw, th); break;
+            default: hipLaunchKernelGGL(raster_bwd_rows_kernel<SSR_ACCUM_NONE>, grid, block, 0, st, *p, tw, th); break;
+        }
         SSR_CHECK_LAUNCH("ssr_raster_bwd");
         return 0;
     }
