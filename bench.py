@@ -215,7 +215,13 @@ def main():
     hyper = dict(lr_means=1.6e-6, lr_quats=1e-5, lr_scales=5e-5, lr_opacs=5e-4, lr_features_dc=2.5e-5, lr_features_sh=1.25e-6)
     adam_step = [0]
 
-    variants = args.dist_type or args.median or args.accum_mode
+    # the accumulation of the loss map rides with the fused optimizer as the trainer's step does; alone, or with
+    # distortion / median, it goes through the variants' backward
+    fused_accum = bool(args.fused_optimizer and args.accum_mode and not (args.dist_type or args.median))
+    variants = (args.dist_type or args.median or args.accum_mode) and not fused_accum
+    if fused_accum:
+        amap_dev = lib.DeviceArray.from_host(np.random.default_rng(1).uniform(0, 1, (ncam, sc.height, sc.width)).astype(np.float32))
+        eng.set_loss_map(amap_dev.ptr, args.accum_mode)
     if variants:
         rng = np.random.default_rng(1)
         eng.set_variants(args.dist_type, args.median)
@@ -342,7 +348,8 @@ def main():
                                   + (", packed projection outputs" if args.packed_projection else "")
                                   + (", projection backward fused with Adam" + ((" (quantized SH state" + (" and non-SH moments)" if args.non_sh_optim_bits == 16 else ")")) if args.quantization_level else "")
                                      if args.fused_optimizer else "")
-                                  + (f", compositing variants dist_type={args.dist_type} median={int(args.median)} accum_mode={args.accum_mode}" if variants else ""),
+                                  + (f", compositing variants dist_type={args.dist_type} median={int(args.median)} accum_mode={args.accum_mode}" if variants else "")
+                                  + (f", loss map accumulated per splat (accum_mode={args.accum_mode})" if fused_accum else ""),
                    "device_ms_per_iter_median": float(np.median(ms))},
         "hbm_roofline_frac_whole_iteration": total_bytes / (float(np.median(ms)) * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "algorithmic_bytes_per_iter": total_bytes,

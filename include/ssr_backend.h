@@ -301,7 +301,9 @@ typedef struct {
      * splat as ONE row (x, y, depth, conic[3], opac, rgb[3], 2 pad) instead of five arrays, so that
      * its atomics land in one or two cache lines instead of five. When given, v_screen is not
      * written; ssr_projection_bwd / ssr_fused_projection_bwd_optimizer read the rows through their
-     * own v_rows field. No counterpart in the reference. */
+     * own v_rows field. With accum_mode sum or avg (and neither distortion nor median) the two spare
+     * floats of a row carry that row's weight sums on their way to accum_weight; the readers ignore
+     * them. No counterpart in the reference. */
     float* v_rows;
     /* Variants (RasterizationEval3DBwd_kernel.cuh:150-172,207-279,433-585). With dist_type set:
      * render_rgb and distortion_* are the forward's outputs, v_distortion_* the cotangents of the

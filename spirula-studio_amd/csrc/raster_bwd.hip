@@ -379,19 +379,23 @@ constexpr int kRowBatch = 128;   // fragments staged per batch by the row-granul
 // average ride as two more channels (map * w and w) through the same reduction, in lanes that hold copies otherwise;
 // the maximum takes a reduction of its own.
 template <int kAccum>
-__global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raster_bwd_params P, int tile_w, int tile_h) {
+__device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params& P, int tile_w, int tile_h) {
     constexpr bool kSums = kAccum == SSR_ACCUM_SUM || kAccum == SSR_ACCUM_AVG;
     constexpr int kCh = kSums ? 12 : 10;   // channels per fragment slot
-    __shared__ FragLds frags[kRowBatch + 1];   // the last one is the blank fragment that ends every list
-    __shared__ int32_t s_ids[kRowBatch];
+    // Fragments per batch: with twelve channels in four copies a batch of 128 would take 33 KB of LDS and leave four
+    // workgroups per compute unit instead of five, which costs this latency-bound kernel more than the shorter batch
+    constexpr int kB = kSums ? 112 : kRowBatch;
+    static_assert(kB <= 128 && 2 * kB <= kRasterBlock && (4 * kB) % 8 == 0, "two threads stage a fragment; a wavefront blanks its lists with 8-byte stores");
+    __shared__ FragLds frags[kB + 1];   // the last one is the blank fragment that ends every list
+    __shared__ int32_t s_ids[kB];
     __shared__ int s_wave_max[4];
     // Moment sums per (wavefront, fragment, channel). Each wavefront adds into its own copy with a plain
     // read-add-write: a float atomic in LDS costs about three cycles per active lane on this hardware,
     // which at forty lanes a step would make LDS, not arithmetic, the limit of this kernel.
-    __shared__ float s_acc[4 * kRowBatch * kCh];
-    [[maybe_unused]] __shared__ float s_max[kAccum == SSR_ACCUM_MAX ? 4 * kRowBatch : 1];   // per wavefront and slot: largest map * w
-    __shared__ uint8_t s_bits[2 * kRowBatch];                       // block bits of sub-tiles {0,1} and {2,3}
-    __shared__ uint8_t s_list[kBlocksPerTile * kRowBatch + 16];
+    __shared__ float s_acc[4 * kB * kCh];
+    [[maybe_unused]] __shared__ float s_max[kAccum == SSR_ACCUM_MAX ? 4 * kB : 1];   // per wavefront and slot: largest map * w
+    __shared__ uint8_t s_bits[2 * kB];                       // block bits of sub-tiles {0,1} and {2,3}
+    __shared__ __attribute__((aligned(8))) uint8_t s_list[kBlocksPerTile * kB + 16];
     const int n_tiles = tile_w * tile_h * (P.num_images > 1 ? P.num_images : 1);
     const int tile = xcd_tile_of(blockIdx.x, n_tiles);
     if (tile >= n_tiles) return;
@@ -438,17 +442,17 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
     int chan = -1;
     if (!b0) chan = 4 * (b1 ? 1 : 0) + 2 * (b2 ? 1 : 0) + (b3 ? 1 : 0);
     else if (!b1 && (!b2 || kSums)) chan = 8 + 2 * (b2 ? 1 : 0) + (b3 ? 1 : 0);
-    for (int e = tid; e < 4 * kRowBatch * kCh; e += kRasterBlock) s_acc[e] = 0.0f;
-    if constexpr (kAccum == SSR_ACCUM_MAX) { for (int e = tid; e < 4 * kRowBatch; e += kRasterBlock) s_max[e] = 0.0f; }
-    // A list is read without asking where it ends: behind its entries stands slot kRowBatch, a fragment of opacity
+    for (int e = tid; e < 4 * kB * kCh; e += kRasterBlock) s_acc[e] = 0.0f;
+    if constexpr (kAccum == SSR_ACCUM_MAX) { for (int e = tid; e < 4 * kB; e += kRasterBlock) s_max[e] = 0.0f; }
+    // A list is read without asking where it ends: behind its entries stands slot kB, a fragment of opacity
     // zero, which no pixel takes up and whose sums stay zero. The tail of the last list is filled here, the rest by
     // each wavefront before it builds its lists (the first barrier of the batch loop orders this with the reads).
-    for (int e = tid; e < (int)sizeof(s_list); e += kRasterBlock) s_list[e] = (uint8_t)kRowBatch;
+    for (int e = tid; e < (int)sizeof(s_list); e += kRasterBlock) s_list[e] = (uint8_t)kB;
     if (tid == 0) {
         const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
-        frags[kRowBatch].q0 = z; frags[kRowBatch].q1 = z; frags[kRowBatch].q2 = z;
+        frags[kB].q0 = z; frags[kB].q1 = z; frags[kB].q2 = z;
     }
-    float* my_acc = s_acc + mt * (kRowBatch * kCh);
+    float* my_acc = s_acc + mt * (kB * kCh);
     char* my_cells = reinterpret_cast<char*>(my_acc + (chan >= 0 ? chan : 0));   // + 4 kCh bytes per fragment slot
 
     // Two neighbouring threads own fragment slot t / 2: they add up the four wavefronts' moment sums, turn
@@ -456,7 +460,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
     // copy; then all threads move the batch to global memory in the order of the destination rows, so that
     // a row's atomics travel as one or two requests.
     auto flush = [&]() {
-        {
+        if (tid < 2 * kB) {
             const int slot = tid >> 1;
             const bool geom = (tid & 1) == 0;   // this thread: u, ux, uy, uxx, uxy, uyy; its neighbour: the colour / depth weights
             float m[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -465,12 +469,12 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
             for (int w = 0; w < 4; w++)
 #pragma unroll
                 for (int c = 0; c < 6; c++)
-                    if (c < nc) { m[c] += s_acc[(w * kRowBatch + slot) * kCh + c0 + c]; }
+                    if (c < nc) { m[c] += s_acc[(w * kB + slot) * kCh + c0 + c]; }
 #pragma unroll
             for (int w = 1; w < 4; w++)
 #pragma unroll
                 for (int c = 0; c < 6; c++)
-                    if (c < nc) s_acc[(w * kRowBatch + slot) * kCh + c0 + c] = 0.0f;
+                    if (c < nc) s_acc[(w * kB + slot) * kCh + c0 + c] = 0.0f;
             float o[6];
             if (geom) {
                 const float4 q0 = frags[slot].q0, q1 = frags[slot].q1;
@@ -498,15 +502,18 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
         }
         __syncthreads();
         if (P.v_rows) {
-            for (int e = tid; e < kRowBatch * 10; e += kRasterBlock) {
-                const int slot = e / 10, ch = e - slot * 10;
+            // with weight sums, those leave in the row's two spare floats: the same cache line and request as the ten
+            // gradients (atomics of their own to the weight arrays double this kernel's L2 atomic requests);
+            // accum_from_rows_kernel moves them on afterwards
+            for (int e = tid; e < kB * kCh; e += kRasterBlock) {
+                const int slot = e / kCh, ch = e - slot * kCh;
                 const float x = s_acc[slot * kCh + ch];
                 if (x != 0.0f) {
                     s_acc[slot * kCh + ch] = 0.0f;
                     atomicAdd(P.v_rows + (int64_t)12 * s_ids[slot] + ch, x);
                 }
             }
-        } else if (tid < kRowBatch) {
+        } else if (tid < kB) {
             float v[10];
             bool any = false;
 #pragma unroll
@@ -523,8 +530,8 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
                 add(P.v_screen.rgb + 3 * g, v[7]); add(P.v_screen.rgb + 3 * g + 1, v[8]); add(P.v_screen.rgb + 3 * g + 2, v[9]);
             }
         }
-        if constexpr (kSums) {   // the weight sums of slot t leave with thread t
-            if (tid < kRowBatch) {
+        if constexpr (kSums) {   // without gradient rows the weight sums of slot t leave with thread t
+            if (!P.v_rows && tid < kB) {
                 const float a = s_acc[tid * kCh + 10], b = s_acc[tid * kCh + 11];
                 if (a != 0.0f || b != 0.0f) {
                     s_acc[tid * kCh + 10] = 0.0f; s_acc[tid * kCh + 11] = 0.0f;
@@ -535,19 +542,19 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
             }
         }
         if constexpr (kAccum == SSR_ACCUM_MAX) {
-            if (tid < kRowBatch) {
+            if (tid < kB) {
                 float mx = 0.0f;
 #pragma unroll
-                for (int w = 0; w < 4; w++) { mx = ssr_max(mx, s_max[w * kRowBatch + tid]); s_max[w * kRowBatch + tid] = 0.0f; }
+                for (int w = 0; w < 4; w++) { mx = ssr_max(mx, s_max[w * kB + tid]); s_max[w * kB + tid] = 0.0f; }
                 if (mx > 0.0f) atomic_max_f32(P.accum_weight + accum_row(P, (uint32_t)s_ids[tid]), mx);   // the running maximum starts at 0
             }
         }
         __syncthreads();   // s_ids, frags and s_acc are free for the next batch
     };
 
-    const uint8_t* my_list = s_list + (4 * mt + row) * kRowBatch;
+    const uint8_t* my_list = s_list + (4 * mt + row) * kB;
     bool first = true;
-    for (int32_t hi = min(range_end - 1, tile_last); hi >= range_start; hi -= kRowBatch) {
+    for (int32_t hi = min(range_end - 1, tile_last); hi >= range_start; hi -= kB) {
         // Explicit wait for this wavefront's LDS traffic (the read-add-writes and float atomics of the walk):
         // the compiler does not place one ahead of this loop-header barrier on the path that leaves the walk,
         // and a pending float atomic is overtaken by the reads that follow the barrier.
@@ -557,31 +564,31 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
         first = false;
         {
             // slot t holds sorted index hi - t: ascending t is back to front. Thread pair (slot, half) shares the staging.
-            const int slot = tid & (kRowBatch - 1), half = tid >> 7;
+            const int half = tid >= kB ? 1 : 0, slot = tid - half * kB;   // threads past 2 kB stage nothing
             const int32_t idx = hi - slot;
             uint32_t bits8 = 0;
-            if (idx >= range_start) {
+            if (idx >= range_start && tid < 2 * kB) {
                 const int32_t g = P.flatten_ids[idx];
                 const FragLds f = stage_fragment_half(P.screen, P.packed_rows, g, tile_x0, tile_y0, half, bits8);
                 if (half == 0) { s_ids[slot] = g; frags[slot] = f; }
             }
-            s_bits[half * kRowBatch + slot] = (uint8_t)bits8;
+            if (tid < 2 * kB) s_bits[half * kB + slot] = (uint8_t)bits8;
         }
         __syncthreads();
         // this wavefront's four lists: slots whose block bit is set and whose sorted index hi - slot is
         // not beyond the block's largest last_id
-        const int n_batch = min(kRowBatch, hi - range_start + 1);
+        const int n_batch = min(kB, hi - range_start + 1);
         int cnt[4] = {0, 0, 0, 0};
-        static_assert(4 * kRowBatch == 64 * 8, "one 8-byte store per lane blanks the wavefront's four lists");
-        reinterpret_cast<uint64_t*>(s_list + 4 * mt * kRowBatch)[lane] = 0x0101010101010101ull * (uint64_t)kRowBatch;
+        if (lane < 4 * kB / 8)   // 8-byte stores blank the wavefront's four lists
+            reinterpret_cast<uint64_t*>(s_list + 4 * mt * kB)[lane] = 0x0101010101010101ull * (uint64_t)kB;
         for (int c = 0; c * 64 < n_batch; c++) {
             const int slot = c * 64 + lane;
-            const uint32_t bits = (uint32_t)s_bits[(mt >> 1) * kRowBatch + slot] >> (4 * (mt & 1));
+            const uint32_t bits = (uint32_t)s_bits[(mt >> 1) * kB + slot] >> (4 * (mt & 1));
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const bool in = ((bits >> r) & 1u) != 0 && hi - slot <= blk_last[r];
+                const bool in = slot < kB && ((bits >> r) & 1u) != 0 && hi - slot <= blk_last[r];
                 const uint64_t bal = __ballot(in);
-                if (in) s_list[(4 * mt + r) * kRowBatch + cnt[r] + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(bal >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)bal, 0u))] = (uint8_t)slot;
+                if (in) s_list[(4 * mt + r) * kB + cnt[r] + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(bal >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)bal, 0u))] = (uint8_t)slot;
                 cnt[r] += __builtin_popcountll(bal);
             }
         }
@@ -593,12 +600,12 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
         // overwrite each other, so those steps add atomically. One bit per step, found here (lane = step).
         uint64_t clash_lo = 0, clash_hi = 0;
         {
-            const uint8_t* base = s_list + 4 * mt * kRowBatch;
+            const uint8_t* base = s_list + 4 * mt * kB;
 #pragma unroll
             for (int c = 0; c < 2; c++) {
                 const int stp = c * 64 + lane;
-                const int e0 = stp < cnt[0] ? (int)base[stp] : -1, e1 = stp < cnt[1] ? (int)base[kRowBatch + stp] : -2,
-                          e2 = stp < cnt[2] ? (int)base[2 * kRowBatch + stp] : -3, e3 = stp < cnt[3] ? (int)base[3 * kRowBatch + stp] : -4;
+                const int e0 = stp < cnt[0] ? (int)base[stp] : -1, e1 = stp < cnt[1] ? (int)base[kB + stp] : -2,
+                          e2 = stp < cnt[2] ? (int)base[2 * kB + stp] : -3, e3 = stp < cnt[3] ? (int)base[3 * kB + stp] : -4;
                 const bool cl = (e0 == e1) | (e0 == e2) | (e0 == e3) | (e1 == e2) | (e1 == e3) | (e2 == e3);
                 const uint64_t m = (c * 64 < n_steps) ? __ballot(cl) : 0ull;
                 if (c == 0) clash_lo = m; else clash_hi = m;
@@ -707,7 +714,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
                     mx = ssr_max(mx, dpp_full<kDppQuadXor2>(mx));
                     mx = ssr_max(mx, dpp_full<kDppQuadXor1>(mx));
                     if (l16 == 0 && mx > 0.0f) {   // non-negative floats order as their bit patterns
-                        int* mc = reinterpret_cast<int*>(s_max + mt * kRowBatch + k);
+                        int* mc = reinterpret_cast<int*>(s_max + mt * kB + k);
                         if (clash) atomicMax(mc, __float_as_int(mx));
                         else *mc = max(*mc, __float_as_int(mx));
                     }
@@ -743,6 +750,30 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
     __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0), as at the head of the loop
     __syncthreads();
     if (!first) flush();
+}
+
+
+template <int kAccum>
+__global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raster_bwd_params P, int tile_w, int tile_h) {
+    raster_bwd_rows_body<kAccum>(P, tile_w, tile_h);
+}
+// The average keeps one register more than five wavefronts per SIMD allow (104 against 102): hold the compiler to
+// five, which it reaches without spilling; the other instantiations are below the limit already.
+__global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(5))) void raster_bwd_rows_avg_kernel(
+    ssr_raster_bwd_params P, int tile_w, int tile_h) {
+    raster_bwd_rows_body<SSR_ACCUM_AVG>(P, tile_w, tile_h);
+}
+
+// Moves the weight sums that raster_bwd_rows_kernel left in floats 10 and 11 of the gradient rows to the weight
+// arrays: row r belongs to world row accum_row(r); rows of several cameras may share one, hence the atomic.
+__global__ __launch_bounds__(256) void accum_from_rows_kernel(ssr_raster_bwd_params P, int avg) {
+    const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (r >= P.num_splats) return;
+    const float2 ab = *reinterpret_cast<const float2*>(P.v_rows + 12 * r + 10);
+    if (ab.x == 0.0f && ab.y == 0.0f) return;
+    const int64_t wid = accum_row(P, (uint32_t)r);
+    if (ab.x != 0.0f) atomicAdd(P.accum_weight + wid, ab.x);
+    if (avg && ab.y != 0.0f) atomicAdd(P.accum_weight + P.num_world + wid, ab.y);
 }
 
 }  // namespace ssr
@@ -807,9 +838,12 @@ extern "C" int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t strea
         switch (p->accum_mode) {
             case SSR_ACCUM_MAX: hipLaunchKernelGGL(raster_bwd_rows_kernel<SSR_ACCUM_MAX>, grid, block, 0, st, *p, tw, th); break;
             case SSR_ACCUM_SUM: hipLaunchKernelGGL(raster_bwd_rows_kernel<SSR_ACCUM_SUM>, grid, block, 0, st, *p, tw, th); break;
-            case SSR_ACCUM_AVG: hipLaunchKernelGGL(raster_bwd_rows_kernel<SSR_ACCUM_AVG>, grid, block, 0, st, *p, tw, th); break;
+            case SSR_ACCUM_AVG: hipLaunchKernelGGL(raster_bwd_rows_avg_kernel, grid, block, 0, st, *p, tw, th); break;
             default: hipLaunchKernelGGL(raster_bwd_rows_kernel<SSR_ACCUM_NONE>, grid, block, 0, st, *p, tw, th); break;
         }
+        if (p->v_rows && (p->accum_mode == SSR_ACCUM_SUM || p->accum_mode == SSR_ACCUM_AVG))
+            hipLaunchKernelGGL(accum_from_rows_kernel, dim3((unsigned)ceil_div(p->num_splats, 256)), dim3(256), 0, st, *p,
+                               p->accum_mode == SSR_ACCUM_AVG ? 1 : 0);
         SSR_CHECK_LAUNCH("ssr_raster_bwd");
         return 0;
     }

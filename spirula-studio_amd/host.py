@@ -29,6 +29,7 @@ SYMBOLS = {
     "ssrh_copy_sh_quant_state": (C.c_int, [vp, vp, vp, vp]),
     "ssrh_copy_params_to_host": (C.c_int, [vp, vp, vp, vp, vp, vp]),
     "ssrh_set_tile_mask": (C.c_int, [vp, C.c_int, C.c_int]),
+    "ssrh_set_loss_map": (C.c_int, [vp, C.c_int]),
     "ssrh_forward_3dgs": (C.c_int, [C.c_char_p, C.c_int, C.c_int, C.c_int, C.c_int]),
     "ssrh_backward_from_render_grad": (C.c_int, [vp, vp, vp]),
     "ssrh_copy_render_to_host": (C.c_int, [vp, vp, vp]),
@@ -164,6 +165,11 @@ class Engine:
     HYPER = ["lr_means", "lr_quats", "lr_scales", "lr_opacs", "lr_features_dc", "lr_features_sh", "max_gauss_ratio",
              "scale_regularization_weight", "mcmc_opacity_reg_weight", "mcmc_scale_reg_weight", "quat_norm_reg_weight",
              "sh_reg_weight", "erank_reg_weight", "erank_reg_weight_s3", "color_trust_linear", "eps_tr"]
+
+    def set_loss_map(self, device_ptr, accum_mode):
+        """The [C,H,W] loss map (a device pointer that stays valid) the fused training step accumulates per splat:
+        accum_mode 1 max, 2 sum, 3 avg; None or 0 switches it off."""
+        check(self.h.ssrh_set_loss_map(device_ptr, int(accum_mode)))
 
     def backward_fused_optimizer(self, hyper, step, scale_agnostic_mean=False, quantization_level=0, non_sh_optim_bits=32):
         """Compositing backward, then the projection backward fused with the Adam step: the engine's

@@ -353,7 +353,12 @@ void engine_backward_fused_optimizer(TorchTensorView v_render_rgb, TorchTensorVi
         non_sh.opacities_packed = pk + n * 10 * 4; non_sh.opacities_bounds = bd + 3 * nb * 4;
         non_sh.features_dc_packed = pk + n * 11 * 4; non_sh.features_dc_bounds = bd + 4 * nb * 4;
     }
-    E.grad.v_screen = raster_backward(v_render_rgb, v_render_depth, v_render_Ts);
+    VariantGrads vg;   // the training step's loss map, when one is set: accumulated per splat as the densifier's score
+    if (std::get<0>(E.optim.loss_map) && E.optim.loss_map_accum_mode != 0) {
+        vg.accum_map = E.optim.loss_map;
+        vg.accum_mode = (DensifyAccumMode)E.optim.loss_map_accum_mode;
+    }
+    E.grad.v_screen = raster_backward(v_render_rgb, v_render_depth, v_render_Ts, vg);
     const int64_t W = E.camera.width, H = E.camera.height;
     DeviceVector<int32_t> cam_ids, gauss_ids;
     DeviceTensorFloatND aabb((float*)E.fwd.aabb.data_ptr(), {E.fwd.aabb.numel(), 4});
@@ -529,6 +534,18 @@ int ssrh_backward_with_variants(const float* v_rgb, const float* v_depth, const 
         engine_backward_with_variants(tv(v_rgb, 4, {C, H, W, 3}), tv(v_depth, 4, {C, H, W, 1}), tv(v_Ts, 4, {C, H, W, 1}),
                                       tv(v_dist_rgb, 4, {C, H, W, 3}), tv(v_dist_depth, 4, {C, H, W, 1}), tv(v_median, 4, {C, H, W, 1}),
                                       tv(accum_map, 4, {C, H, W, 1}), accum_mode);
+    });
+}
+
+// The loss map [C,H,W] (device or host pointer, kept by the caller until the backward has run) that the fused
+// training step accumulates per splat with `accum_mode` (1 max, 2 sum, 3 avg); null or mode 0 switches it off.
+int ssrh_set_loss_map(const float* map, int accum_mode) {
+    return guard([&] {
+        auto& E = engine();
+        if (accum_mode < 0 || accum_mode > 3) throw std::runtime_error("ssrh_set_loss_map: accum_mode must be 0..3");
+        const int64_t C = E.camera.num, H = E.camera.height, W = E.camera.width;
+        E.optim.loss_map = map ? tv(map, 4, {C, H, W}) : TorchTensorView{0, 4, {}};
+        E.optim.loss_map_accum_mode = map ? accum_mode : 0;
     });
 }
 

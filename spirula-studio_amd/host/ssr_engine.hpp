@@ -39,6 +39,10 @@ struct EngineState {
         bool non_sh_state_ready = false;   // non_sh_optim_bits 16: the 16-bit non-SH moments have been zeroed
         std::vector<DeviceTensorFloatND> g1, g2;   // Adam moments, shaped like the world tensors
         DeviceVector<float> densify_score;
+        // the loss map of the training step and how the compositing backward accumulates it per splat
+        // (cfg.loss.loss_map_accum_mode, src/engine/EngineTrainStep.cpp:256-258); null map: no accumulation
+        TorchTensorView loss_map{0, 4, {}};
+        int loss_map_accum_mode = 0;
     } optim;
     struct {
         std::vector<DeviceTensorFloatND> splats_w, splats_s;

@@ -291,6 +291,38 @@ def test_engine_fused_optimizer_scale_agnostic_means(pkg, oracle, H, packed):
         assert (d > 0.05 * 5e-2).mean() < 2e-3, k
 
 
+@pytest.mark.parametrize("packed,accum_mode", [(False, 3), (True, 3), (False, 1), (True, 2)])
+def test_engine_fused_step_accumulates_the_loss_map(pkg, oracle, H, packed, accum_mode):
+    """The training step of the reference accumulates its loss map per splat in the same compositing backward that
+    feeds the fused optimizer (EngineTrainStep.cpp:256-258): with a map set, the engine's fused step leaves the
+    oracle's accumulated weights, and the parameters take exactly the step they take without a map."""
+    host, lib = H
+    sc = pkg.scenes.make_scene(1, n=20000, width=320, height=240, parity_variant=True)
+    if packed:
+        sc.means[::3, 2] = -10.0
+    h = dict(lr_means=1.6e-4, lr_quats=1e-3, lr_scales=5e-3, lr_opacs=5e-2, lr_features_dc=2.5e-3, lr_features_sh=1.25e-4)
+    amap = np.random.default_rng(5).uniform(0, 1, (sc.height, sc.width)).astype(np.float32)
+    d_map = lib.DeviceArray.from_host(amap)
+    kw = dict(fuse_tile_count=True, visible_list=not packed, packed_rows=True, overwrite_world_grads=True,
+              packed_projection=packed, packed_vscreen=True, tile_sort=True)
+    eng = host.Engine(sc, **kw)
+    eng.set_loss_map(d_map.ptr, accum_mode)
+    eng.forward()
+    eng.backward_fused_optimizer(h, 1)
+    aw = eng.cache("accum_weight")
+    got = eng.params()
+    r = oracle.pipeline(sc, backward=True, variant=dict(dist_type=0, median=False, accum_mode=accum_mode, accum_map=amap))
+    ref = r["vscreen"]["accum_weight"]
+    assert np.allclose(aw[:ref.size], ref, rtol=1e-3, atol=1e-6) and (aw[:sc.n] > 0).sum() > 1000
+    eng.set_loss_map(None, 0)
+    plain = host.Engine(sc, **kw)
+    plain.forward()
+    plain.backward_fused_optimizer(h, 1)
+    base = plain.params()
+    for k in oracle.WORLD_KEYS:   # the map adds outputs, it changes no gradient (summation order aside)
+        assert np.allclose(got[k], base[k], rtol=1e-4, atol=1e-6), k
+
+
 @pytest.mark.parametrize("packed,non_sh_bits", [(False, 32), (True, 32), (False, 16), (True, 16)])
 def test_engine_fused_optimizer_quantization_level_1(pkg, oracle, H, packed, non_sh_bits):
     """Training steps at OptimConfig::quantization_level 1 (the reference's default): the engine keeps the SH
