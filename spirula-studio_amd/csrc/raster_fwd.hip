@@ -122,8 +122,11 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_kernel(ssr_raster_fwd
 // holds one 4x4-pixel block and walks its own list of the staged fragments whose block bit is set
 // (raster_device.h), instead of all 64 lanes visiting every fragment that reaches the 8x8 sub-tile.
 // Lists are built per batch by the wavefront that walks them (ballot + rank, slot numbers as bytes).
+template <int kDist, bool kMedian>
 __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raster_fwd_params P, int tile_w, int tile_h) {
     __shared__ FragLds frags[kBatch];
+    // distortion composites ln(max(z, 1e-6)): a per-splat value, taken once when the fragment is staged
+    [[maybe_unused]] __shared__ float s_lz[kDist != SSR_DIST_NONE ? kBatch : 1];
     __shared__ uint8_t s_list[kBlocksPerTile * kBatch + 16];
     const int n_tiles = tile_w * tile_h * (P.num_images > 1 ? P.num_images : 1);
     const int tile = xcd_tile_of(blockIdx.x, n_tiles);
@@ -140,6 +143,8 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raste
     const int32_t range_start = P.tile_offsets[tile];
     const int32_t range_end = (tile == n_tiles - 1) ? (int32_t)P.n_isects : P.tile_offsets[tile + 1];
     float T = 1.0f, cr = 0.f, cg = 0.f, cb = 0.f, cd = 0.f;
+    [[maybe_unused]] float s2r = 0.f, s2g = 0.f, s2b = 0.f, s2d = 0.f;           // second moments (distortion)
+    [[maybe_unused]] float median = 0.f, med_prev_z = 0.f, med_prev_T = 1.0f;   // median depth
     uint32_t cur_idx = 0;
     const float tile_x0 = (float)(tx * kTile), tile_y0 = (float)(ty * kTile);
     const uint8_t* my_list = s_list + (4 * mt + row) * kBatch;
@@ -156,6 +161,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raste
             FragLds f = stage_fragment(P.screen, P.packed_rows, P.flatten_ids[idx], tile_x0, tile_y0, &kk);
             add_block_mask(f, kk, tile_x0, tile_y0);
             frags[tid] = f;
+            if constexpr (kDist != SSR_DIST_NONE) s_lz[tid] = ssr_log(ssr_max(f.q2.y, 1e-6f));
         } else {
             frags[tid].q2 = make_float4(0.f, 0.f, 0.f, 0.f);   // empty masks
         }
@@ -191,10 +197,29 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raste
             const float alpha = eval_alpha_fast(q0, q1, cut, px, py, dx, dy, vis, sigma);
             const bool hit = (alive != 0) & (st < my_cnt) & (alpha > kAlphaThreshold);
             const float next_T = T * (1.0f - alpha);
+            if constexpr (kMedian) {   // before the early-out, so a splat that ends the pixel still counts
+                const bool cross = hit & (med_prev_T >= 0.5f) & (next_T < 0.5f);
+                if (__builtin_amdgcn_ballot_w64(cross) != 0ull) {   // once per pixel: rarely any lane
+                    const float a = ssr_log(med_prev_T), b = ssr_log(next_T), d = b - a;
+                    const float fr = (ssr_fabs(d) > 1e-20f) ? (-0.6931471805599453f - a) / d : 0.0f;
+                    median = cross ? med_prev_z + (q2.y - med_prev_z) * fr : median;
+                }
+                med_prev_T = hit ? next_T : med_prev_T;
+                med_prev_z = hit ? q2.y : med_prev_z;
+            }
             const bool keep = hit & (next_T > kTransmitThreshold);
             const float w = keep ? alpha * T : 0.0f;   // a fragment that is not composited adds zero
+            float zd = q2.y;
+            if constexpr (kDist != SSR_DIST_NONE) {
+                zd = s_lz[k];
+                if constexpr (kDist == SSR_DIST_RGB_D) {
+                    s2r = ssr_fma(q1.z * q1.z, w, s2r); s2g = ssr_fma(q1.w * q1.w, w, s2g);
+                    s2b = ssr_fma(q2.x * q2.x, w, s2b);
+                }
+                s2d = ssr_fma(zd * zd, w, s2d);
+            }
             cr = ssr_fma(q1.z, w, cr); cg = ssr_fma(q1.w, w, cg); cb = ssr_fma(q2.x, w, cb);
-            cd = ssr_fma(q2.y, w, cd);
+            cd = ssr_fma(zd, w, cd);
             cur_idx = keep ? (uint32_t)(batch_start + k) : cur_idx;
             T = keep ? next_T : T;
             alive = (hit & !keep) ? 0 : alive;
@@ -232,7 +257,18 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raste
         const float invW = 1.0f / ssr_max(1.0f - T, 1e-10f);
         float* o = P.render_rgb + 3 * pid;
         o[0] = cr; o[1] = cg; o[2] = cb;
-        P.render_depth[pid] = cd * invW;
+        if constexpr (kMedian) P.render_median[pid] = median;
+        if constexpr (kDist != SSR_DIST_NONE) {   // D = W S - C^2 on the raw accumulators
+            const float W = 1.0f - T;
+            if constexpr (kDist == SSR_DIST_RGB_D) {
+                float* d = P.distortion_rgb + 3 * pid;
+                d[0] = s2r * W - cr * cr; d[1] = s2g * W - cg * cg; d[2] = s2b * W - cb * cb;
+            }
+            P.distortion_depth[pid] = s2d * W - cd * cd;
+            P.render_depth[pid] = ssr_exp(cd * invW);
+        } else {
+            P.render_depth[pid] = cd * invW;
+        }
         P.last_ids[pid] = (int32_t)cur_idx;
     }
 }
@@ -269,11 +305,17 @@ extern "C" int ssr_raster_fwd(const ssr_raster_fwd_params* p, ssr_stream_t strea
     hipStream_t s = as_stream(stream);
 #define SSR_FWD(D, M) hipLaunchKernelGGL((raster_fwd_kernel<D, M>), grid, block, 0, s, *p, tw, th)
     const bool med = p->render_median != nullptr;
-    // The plain variant runs the row-granular kernel; SSR_RASTER_WAVE_VISITS=1 in the environment
-    // selects the one-wavefront-per-visit kernel instead (for comparisons).
+    // Every variant runs the row-granular kernel; SSR_RASTER_WAVE_VISITS=1 in the environment selects the
+    // one-wavefront-per-visit kernel instead (for comparisons).
     static const bool wave_visits = getenv("SSR_RASTER_WAVE_VISITS") != nullptr;
-    if (p->dist_type == SSR_DIST_NONE && !med && !wave_visits) {
-        hipLaunchKernelGGL(raster_fwd_rows_kernel, grid, block, 0, s, *p, tw, th);
+    if (!wave_visits) {
+#define SSR_FWD_ROWS(D, M) hipLaunchKernelGGL((raster_fwd_rows_kernel<D, M>), grid, block, 0, s, *p, tw, th)
+        switch (p->dist_type) {
+            case SSR_DIST_D: if (med) SSR_FWD_ROWS(SSR_DIST_D, true); else SSR_FWD_ROWS(SSR_DIST_D, false); break;
+            case SSR_DIST_RGB_D: if (med) SSR_FWD_ROWS(SSR_DIST_RGB_D, true); else SSR_FWD_ROWS(SSR_DIST_RGB_D, false); break;
+            default: if (med) SSR_FWD_ROWS(SSR_DIST_NONE, true); else SSR_FWD_ROWS(SSR_DIST_NONE, false); break;
+        }
+#undef SSR_FWD_ROWS
         SSR_CHECK_LAUNCH("ssr_raster_fwd");
         return 0;
     }
