@@ -301,7 +301,7 @@ typedef struct {
      * splat as ONE row (x, y, depth, conic[3], opac, rgb[3], 2 pad) instead of five arrays, so that
      * its atomics land in one or two cache lines instead of five. When given, v_screen is not
      * written; ssr_projection_bwd / ssr_fused_projection_bwd_optimizer read the rows through their
-     * own v_rows field. With accum_mode sum or avg (and neither distortion nor median) the two spare
+     * own v_rows field. With accum_mode sum or avg the two spare
      * floats of a row carry that row's weight sums on their way to accum_weight; the readers ignore
      * them. No counterpart in the reference. */
     float* v_rows;

@@ -378,7 +378,7 @@ constexpr int kRowBatch = 128;   // fragments staged per batch by the row-granul
 // kAccum: the pixel-weight accumulation of the densifier (RasterizationEval3DBwd_kernel.cuh:553-562,574-585). Sum and
 // average ride as two more channels (map * w and w) through the same reduction, in lanes that hold copies otherwise;
 // the maximum takes a reduction of its own.
-template <int kAccum>
+template <int kDist, bool kMedian, int kAccum>
 __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params& P, int tile_w, int tile_h) {
     constexpr bool kSums = kAccum == SSR_ACCUM_SUM || kAccum == SSR_ACCUM_AVG;
     constexpr int kCh = kSums ? 12 : 10;   // channels per fragment slot
@@ -395,6 +395,9 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
     __shared__ float s_acc[4 * kB * kCh];
     [[maybe_unused]] __shared__ float s_max[kAccum == SSR_ACCUM_MAX ? 4 * kB : 1];   // per wavefront and slot: largest map * w
     __shared__ uint8_t s_bits[2 * kB];                       // block bits of sub-tiles {0,1} and {2,3}
+    // distortion composites ln(max(z, 1e-6)): the value and the factor d ln z / dz per staged fragment
+    [[maybe_unused]] __shared__ float s_lz[kDist != SSR_DIST_NONE ? kB + 1 : 1];
+    [[maybe_unused]] __shared__ float s_iz[kDist != SSR_DIST_NONE ? kB + 1 : 1];
     __shared__ __attribute__((aligned(8))) uint8_t s_list[kBlocksPerTile * kB + 16];
     const int n_tiles = tile_w * tile_h * (P.num_images > 1 ? P.num_images : 1);
     const int tile = xcd_tile_of(blockIdx.x, n_tiles);
@@ -416,9 +419,41 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
         const float* v = P.v_render_rgb + 3 * pid;
         vr = v[0]; vg = v[1]; vb = v[2];
         vd = P.v_render_depth[pid];
+    }
+    // totals of the forward held constant during the sweep (distortion), median state
+    [[maybe_unused]] float Cr = 0.f, Cg = 0.f, Cb = 0.f, Cd = 0.f, Sr = 0.f, Sg = 0.f, Sb = 0.f, Sd = 0.f;
+    [[maybe_unused]] float vDr = 0.f, vDg = 0.f, vDb = 0.f, vDd = 0.f, Wd = 0.f;
+    [[maybe_unused]] float med_v = 0.f, pend_zgrad = 0.f, pend_zfar = 0.f, pend_Tfar = 0.f;
+    {
         const float inv_alpha = 1.0f / ssr_max(1.0f - T1, 1e-10f);
-        vT1 = vT1 + (P.render_depth[pid] * vd) * inv_alpha;
-        vd = vd * inv_alpha;
+        const float exp_depth = inside ? P.render_depth[pid] : 0.0f;
+        if constexpr (kDist != SSR_DIST_NONE) {
+            // log-depth render: depth = exp(C_lnz / W)  (RasterizationEval3DBwd_kernel.cuh:212-218)
+            const float m = ssr_log(ssr_max(exp_depth, 1e-6f));
+            vT1 = vT1 + ((exp_depth * vd) * m) * inv_alpha;
+            vd = vd * (exp_depth * inv_alpha);
+            // C, S = (D + C^2) / W, W and the distortion cotangent (:228-257)
+            Cd = m * ssr_max(1.0f - T1, 1e-10f);
+            Wd = inside ? (1.0f - T1) : 0.0f;
+            const float invW = Wd > 1e-10f ? (1.0f / Wd) : 0.0f;
+            float Dd = 0.f, Dr = 0.f, Dg = 0.f, Db = 0.f;
+            if (inside) {
+                Dd = P.distortion_depth[pid]; vDd = P.v_distortion_depth[pid];
+                if constexpr (kDist == SSR_DIST_RGB_D) {
+                    const float* c = P.render_rgb + 3 * pid; Cr = c[0]; Cg = c[1]; Cb = c[2];
+                    const float* d = P.distortion_rgb + 3 * pid; Dr = d[0]; Dg = d[1]; Db = d[2];
+                    const float* v = P.v_distortion_rgb + 3 * pid; vDr = v[0]; vDg = v[1]; vDb = v[2];
+                }
+            }
+            Sd = (Dd + Cd * Cd) * invW;
+            if constexpr (kDist == SSR_DIST_RGB_D) {
+                Sr = (Dr + Cr * Cr) * invW; Sg = (Dg + Cg * Cg) * invW; Sb = (Db + Cb * Cb) * invW;
+            }
+        } else {
+            vT1 = vT1 + (exp_depth * vd) * inv_alpha;
+            vd = vd * inv_alpha;
+        }
+        if constexpr (kMedian) med_v = inside ? P.v_render_median[pid] : 0.0f;
     }
     [[maybe_unused]] float amap = 0.0f;
     if constexpr (kAccum != SSR_ACCUM_NONE) amap = inside ? P.accum_weight_map[pid] : 0.0f;
@@ -451,6 +486,7 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
     if (tid == 0) {
         const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
         frags[kB].q0 = z; frags[kB].q1 = z; frags[kB].q2 = z;
+        if constexpr (kDist != SSR_DIST_NONE) { s_iz[kB] = 0.0f; s_lz[kB] = 0.0f; }
     }
     float* my_acc = s_acc + mt * (kB * kCh);
     char* my_cells = reinterpret_cast<char*>(my_acc + (chan >= 0 ? chan : 0));   // + 4 kCh bytes per fragment slot
@@ -570,7 +606,13 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
             if (idx >= range_start && tid < 2 * kB) {
                 const int32_t g = P.flatten_ids[idx];
                 const FragLds f = stage_fragment_half(P.screen, P.packed_rows, g, tile_x0, tile_y0, half, bits8);
-                if (half == 0) { s_ids[slot] = g; frags[slot] = f; }
+                if (half == 0) {
+                    s_ids[slot] = g; frags[slot] = f;
+                    if constexpr (kDist != SSR_DIST_NONE) {
+                        s_lz[slot] = ssr_log(ssr_max(f.q2.y, 1e-6f));
+                        s_iz[slot] = 1.0f / ssr_max(f.q2.y, 1e-6f);   // d/d ln z -> d/dz
+                    }
+                }
             }
             if (tid < 2 * kB) s_bits[half * kB + slot] = (uint8_t)bits8;
         }
@@ -636,8 +678,43 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
                 // inactive lanes run with alpha = 0 and v_alpha = 0: T and v_T unchanged, every term zero
                 const float a = active ? alpha : 0.0f;
                 const float T0 = T1 * __builtin_amdgcn_rcpf(1.0f - a);
-                const float dv = ssr_fma(q2.y, vd, ssr_fma(q2.x, vb, ssr_fma(q1.w, vg, q1.z * vr))) - vT1;
+                [[maybe_unused]] float v_depth_median = 0.0f;
+                if constexpr (kMedian) {   // RasterizationEval3DBwd_kernel.cuh:433-470
+                    if (active && pend_Tfar > 0.0f) {   // near member of the crossing found at the previous active splat
+                        v_depth_median += pend_zgrad;
+                        const float dba = ssr_log(pend_Tfar) - ssr_log(T1);
+                        const float inv = (ssr_fabs(dba) > 1e-20f) ? (-1.0f / dba) : 0.0f;
+                        vT1 += ((med_v * (pend_zfar - q2.y)) * inv) / T1;
+                        pend_Tfar = 0.0f;
+                    }
+                    if (active && T0 >= 0.5f && T1 < 0.5f) {   // far member: post-splat T drops below 1/2 here
+                        const float la = ssr_log(T0), d = ssr_log(T1) - la;
+                        const float fr = (ssr_fabs(d) > 1e-20f) ? (-0.6931471805599453f - la) / d : 0.0f;
+                        v_depth_median += fr * med_v;
+                        pend_zgrad = (1.0f - fr) * med_v;
+                        pend_zfar = q2.y;
+                        pend_Tfar = T1;
+                    }
+                }
+                const float cr = q1.z, cg = q1.w, cb = q2.x;
+                float cdp = q2.y;
+                if constexpr (kDist != SSR_DIST_NONE) cdp = s_lz[k];
+                float dv = ssr_fma(cdp, vd, ssr_fma(cb, vb, ssr_fma(cg, vg, cr * vr))) - vT1;
                 const float w = a * T0;
+                [[maybe_unused]] float xr = 0.f, xg = 0.f, xb = 0.f, xd = 0.f;   // distortion part of the colour gradient
+                if constexpr (kDist != SSR_DIST_NONE) {   // closed form D = W S - C^2 (:497-517)
+                    float gsum = 0.0f;
+                    const float w2 = 2.0f * w;
+                    if constexpr (kDist == SSR_DIST_RGB_D) {
+                        xr = ((cr * Wd - Cr) * vDr) * w2; xg = ((cg * Wd - Cg) * vDg) * w2; xb = ((cb * Wd - Cb) * vDb) * w2;
+                        gsum += ((Sr + (cr * cr) * Wd) - (cr * Cr) * 2.0f) * vDr;
+                        gsum += ((Sg + (cg * cg) * Wd) - (cg * Cg) * 2.0f) * vDg;
+                        gsum += ((Sb + (cb * cb) * Wd) - (cb * Cb) * 2.0f) * vDb;
+                    }
+                    xd = ((cdp * Wd - Cd) * vDd) * w2;
+                    gsum += ((Sd + (cdp * cdp) * Wd) - (cdp * Cd) * 2.0f) * vDd;
+                    dv += gsum;   // v_alpha gains T0 g and v_T0 gains alpha g, exactly where dv enters
+                }
                 // evaluate_alpha_vjp gate (src/primitives/Primitive3DGS.cuh:273); sigma >= 0 holds when active
                 const float v_alpha = (active & (ov <= 0.999f)) ? T0 * dv : 0.0f;
                 vT1 = ssr_fma(a, dv, vT1);
@@ -645,7 +722,12 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
                 const float u = vis * v_alpha;
                 const float ux = u * dx, uy = u * dy;
                 const float uxx = ux * dx, uxy = ux * dy, uyy = uy * dy;
-                const float wr = vr * w, wg = vg * w, wb = vb * w, wd = vd * w;
+                float wr = vr * w, wg = vg * w, wb = vb * w, wd = vd * w;
+                if constexpr (kDist != SSR_DIST_NONE) {
+                    if constexpr (kDist == SSR_DIST_RGB_D) { wr += xr; wg += xg; wb += xb; }
+                    wd = (wd + xd) * s_iz[k];
+                }
+                if constexpr (kMedian) wd += v_depth_median;
                 // Channels 0..9 = u, ux, uy, uxx, uxy, uyy, wr, wg, wb, wd. The first two levels of the transposing
                 // reduction as bank-masked DPP adds (one instruction per channel and level, against three per pair with
                 // selects): lanes 0-7 of a row take the even channel of a pair, lanes 8-15 the odd one; then lane groups
@@ -753,15 +835,15 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
 }
 
 
-template <int kAccum>
+template <int kDist, bool kMedian, int kAccum>
 __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raster_bwd_params P, int tile_w, int tile_h) {
-    raster_bwd_rows_body<kAccum>(P, tile_w, tile_h);
+    raster_bwd_rows_body<kDist, kMedian, kAccum>(P, tile_w, tile_h);
 }
-// The average keeps one register more than five wavefronts per SIMD allow (104 against 102): hold the compiler to
-// five, which it reaches without spilling; the other instantiations are below the limit already.
+// The plain average keeps one register more than five wavefronts per SIMD allow (104 against 102): hold the compiler
+// to five, which it reaches without spilling; the other plain instantiations are below the limit already.
 __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(5))) void raster_bwd_rows_avg_kernel(
     ssr_raster_bwd_params P, int tile_w, int tile_h) {
-    raster_bwd_rows_body<SSR_ACCUM_AVG>(P, tile_w, tile_h);
+    raster_bwd_rows_body<SSR_DIST_NONE, false, SSR_ACCUM_AVG>(P, tile_w, tile_h);
 }
 
 // Moves the weight sums that raster_bwd_rows_kernel left in floats 10 and 11 of the gradient rows to the weight
@@ -834,13 +916,26 @@ extern "C" int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t strea
     // The plain variant runs the row-granular kernel; SSR_RASTER_WAVE_VISITS=1 in the environment
     // selects the one-wavefront-per-visit kernel instead (for comparisons).
     static const bool wave_visits = getenv("SSR_RASTER_WAVE_VISITS") != nullptr;
-    if (p->dist_type == SSR_DIST_NONE && !med && !wave_visits) {
-        switch (p->accum_mode) {
-            case SSR_ACCUM_MAX: hipLaunchKernelGGL(raster_bwd_rows_kernel<SSR_ACCUM_MAX>, grid, block, 0, st, *p, tw, th); break;
-            case SSR_ACCUM_SUM: hipLaunchKernelGGL(raster_bwd_rows_kernel<SSR_ACCUM_SUM>, grid, block, 0, st, *p, tw, th); break;
-            case SSR_ACCUM_AVG: hipLaunchKernelGGL(raster_bwd_rows_avg_kernel, grid, block, 0, st, *p, tw, th); break;
-            default: hipLaunchKernelGGL(raster_bwd_rows_kernel<SSR_ACCUM_NONE>, grid, block, 0, st, *p, tw, th); break;
+    if (!wave_visits) {
+#define SSR_ROWS(D, M, A) hipLaunchKernelGGL((raster_bwd_rows_kernel<D, M, A>), grid, block, 0, st, *p, tw, th)
+#define SSR_ROWS_A(D, M)                                          \
+    switch (p->accum_mode) {                                      \
+        case SSR_ACCUM_MAX: SSR_ROWS(D, M, SSR_ACCUM_MAX); break;   \
+        case SSR_ACCUM_SUM: SSR_ROWS(D, M, SSR_ACCUM_SUM); break;   \
+        case SSR_ACCUM_AVG: SSR_ROWS(D, M, SSR_ACCUM_AVG); break;   \
+        default: SSR_ROWS(D, M, SSR_ACCUM_NONE); break;             \
+    }
+#define SSR_ROWS_M(D) if (med) { SSR_ROWS_A(D, true) } else { SSR_ROWS_A(D, false) }
+        if (p->dist_type == SSR_DIST_NONE && !med && p->accum_mode == SSR_ACCUM_AVG)
+            hipLaunchKernelGGL(raster_bwd_rows_avg_kernel, grid, block, 0, st, *p, tw, th);
+        else switch (p->dist_type) {
+            case SSR_DIST_D: SSR_ROWS_M(SSR_DIST_D); break;
+            case SSR_DIST_RGB_D: SSR_ROWS_M(SSR_DIST_RGB_D); break;
+            default: SSR_ROWS_M(SSR_DIST_NONE); break;
         }
+#undef SSR_ROWS_M
+#undef SSR_ROWS_A
+#undef SSR_ROWS
         if (p->v_rows && (p->accum_mode == SSR_ACCUM_SUM || p->accum_mode == SSR_ACCUM_AVG))
             hipLaunchKernelGGL(accum_from_rows_kernel, dim3((unsigned)ceil_div(p->num_splats, 256)), dim3(256), 0, st, *p,
                                p->accum_mode == SSR_ACCUM_AVG ? 1 : 0);

@@ -321,7 +321,14 @@ class GpuRun:
             for k in ["v_xy", "v_depth", "v_conic", "v_opac", "v_rgb"]:
                 assert np.all(self.host(k).view(np.uint32) == 0x7fc12345), k
             rows = self.host("v_rows")
-            assert not np.any(rows[:, 10:])
+            if p.accum_mode in (2, 3):   # the weight sums travel in the two spare floats of a row
+                aw = self.host("accum_weight")
+                if not self.packed_projection:   # row = world row: the sums, as they were moved on
+                    assert np.allclose(rows[:, 10], aw[:self.n], rtol=1e-6, atol=0)
+                    if p.accum_mode == 3:
+                        assert np.allclose(rows[:, 11], aw[self.n:], rtol=1e-6, atol=0)
+            else:
+                assert not np.any(rows[:, 10:])
             for k, sl in [("v_xy", slice(0, 2)), ("v_depth", 2), ("v_conic", slice(3, 6)), ("v_opac", 6), ("v_rgb", slice(7, 10))]:
                 self.d[k] = D.from_host(np.ascontiguousarray(rows[:, sl]))
 
