@@ -233,6 +233,14 @@ int ssr_sort_pairs_u64_i32(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, in
 /* intersect_offset_kernel (IntersectTile.cu:271-307); zero-fills when n_isects == 0 (:448-451). */
 int ssr_tile_offsets(int64_t n_isects, const int64_t* sorted_ids, uint32_t n_tiles,
                      int32_t* offsets, ssr_stream_t stream);
+/* Launch order for the compositing kernels (their optional tile_order field): order[n_tiles] receives all tile
+ * ids by descending fragment count (in classes of 32 fragments; the order inside a class is arbitrary). Workgroup
+ * w of a compositing launch takes order[w]: workgroups start in index order and are dealt round-robin to the XCDs,
+ * so the longest tiles start first and every XCD gets the same mix. scratch: ssr_tile_order_scratch_bytes.
+ * No counterpart in the reference (its grid is one block per tile in index order). */
+size_t ssr_tile_order_scratch_bytes(uint32_t n_tiles);
+int ssr_tile_order(const int32_t* tile_offsets, uint32_t n_tiles, int64_t n_isects, int32_t* order, void* scratch,
+                   size_t scratch_bytes, ssr_stream_t stream);
 /* Number of key bits the sort must cover: 32 + tile_n_bits (IntersectTile.cu:489-490). */
 int ssr_sort_end_bit(uint32_t n_tiles);
 /* The sort of IntersectTile.cu:486-493 and the offsets of :271-307 in one call, for keys of the
@@ -275,6 +283,7 @@ typedef struct {
      * buffer; the splat rows stay global, as the reference's [C,N,...] layout has them
      * (RasterizationFwd.cu grid = {C, tile_h, tile_w}). */
     int32_t num_images;
+    const int32_t* tile_order;  /* optional: ssr_tile_order's output for these tile_offsets; NULL = tiles in index order, one contiguous band per XCD */
 } ssr_raster_fwd_params;
 int ssr_raster_fwd(const ssr_raster_fwd_params* p, ssr_stream_t stream);
 
@@ -325,6 +334,7 @@ typedef struct {
     float* accum_weight;              /* [num_world] or [2 num_world] (AVG) */
     int32_t num_images;               /* as in ssr_raster_fwd_params; with accum_mode, screen row r
                                        * adds into world row r % num_world */
+    const int32_t* tile_order;        /* optional, as in ssr_raster_fwd_params */
 } ssr_raster_bwd_params;
 int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t stream);
 

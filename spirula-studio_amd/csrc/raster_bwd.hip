@@ -96,8 +96,8 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd
     [[maybe_unused]] __shared__ float s_lz[kDist != SSR_DIST_NONE ? kBatch : 1];
     // images stack in the tile space: image c owns tiles [c tile_w tile_h, (c+1) tile_w tile_h)
     const int n_tiles = tile_w * tile_h * (P.num_images > 1 ? P.num_images : 1);
-    const int tile = xcd_tile_of(blockIdx.x, n_tiles);
-    if (tile >= n_tiles) return;
+    const int tile = tile_of_workgroup(P.tile_order, blockIdx.x, n_tiles);
+    if (tile < 0 || tile >= n_tiles) return;
     const int tid = threadIdx.x, lane = tid & 63, mt = tid >> 6;
     const int gy = tile / tile_w, tx = tile - gy * tile_w;
     const int img = gy / tile_h, ty = gy - img * tile_h;
@@ -400,8 +400,8 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
     [[maybe_unused]] __shared__ float s_iz[kDist != SSR_DIST_NONE ? kB + 1 : 1];
     __shared__ __attribute__((aligned(8))) uint8_t s_list[kBlocksPerTile * kB + 16];
     const int n_tiles = tile_w * tile_h * (P.num_images > 1 ? P.num_images : 1);
-    const int tile = xcd_tile_of(blockIdx.x, n_tiles);
-    if (tile >= n_tiles) return;
+    const int tile = tile_of_workgroup(P.tile_order, blockIdx.x, n_tiles);
+    if (tile < 0 || tile >= n_tiles) return;
     const int tid = threadIdx.x, lane = tid & 63, mt = tid >> 6, row = lane >> 4, l16 = lane & 15;
     const int gy = tile / tile_w, tx = tile - gy * tile_w;
     const int img = gy / tile_h, ty = gy - img * tile_h;

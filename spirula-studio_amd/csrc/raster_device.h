@@ -244,5 +244,11 @@ __device__ __forceinline__ int xcd_tile_of(int wg, int n_tiles) {
     return (wg & 7) * chunk + (wg >> 3);
 }
 inline int xcd_grid_size(int n_tiles) { return ((n_tiles + 7) >> 3) * 8; }
+// With a caller's launch order (ssr_tile_order: all tiles, longest first) workgroup w takes its w-th entry: the
+// round-robin dealing then gives every XCD the same mix of long and short tiles.
+__device__ __forceinline__ int tile_of_workgroup(const int32_t* __restrict__ order, int wg, int n_tiles) {
+    if (!order) return xcd_tile_of(wg, n_tiles);
+    return wg < n_tiles ? order[wg] : -1;
+}
 
 }  // namespace ssr

@@ -20,8 +20,8 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_kernel(ssr_raster_fwd
     [[maybe_unused]] __shared__ float s_lz[kDist != SSR_DIST_NONE ? kBatch : 1];
     // images stack in the tile space: image c owns tiles [c tile_w tile_h, (c+1) tile_w tile_h)
     const int n_tiles = tile_w * tile_h * (P.num_images > 1 ? P.num_images : 1);
-    const int tile = xcd_tile_of(blockIdx.x, n_tiles);
-    if (tile >= n_tiles) return;   // whole workgroup leaves together
+    const int tile = tile_of_workgroup(P.tile_order, blockIdx.x, n_tiles);
+    if (tile < 0 || tile >= n_tiles) return;   // whole workgroup leaves together
     const int tid = threadIdx.x, lane = tid & 63, mt = tid >> 6;
     const int gy = tile / tile_w, tx = tile - gy * tile_w;
     const int img = gy / tile_h, ty = gy - img * tile_h;
@@ -129,8 +129,8 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raste
     [[maybe_unused]] __shared__ float s_lz[kDist != SSR_DIST_NONE ? kBatch : 1];
     __shared__ uint8_t s_list[kBlocksPerTile * kBatch + 16];
     const int n_tiles = tile_w * tile_h * (P.num_images > 1 ? P.num_images : 1);
-    const int tile = xcd_tile_of(blockIdx.x, n_tiles);
-    if (tile >= n_tiles) return;
+    const int tile = tile_of_workgroup(P.tile_order, blockIdx.x, n_tiles);
+    if (tile < 0 || tile >= n_tiles) return;
     const int tid = threadIdx.x, lane = tid & 63, mt = tid >> 6, row = lane >> 4, l16 = lane & 15;
     const int gy = tile / tile_w, tx = tile - gy * tile_w;
     const int img = gy / tile_h, ty = gy - img * tile_h;

@@ -298,6 +298,65 @@ __global__ __launch_bounds__(kTileBlock) void tile_offsets_kernel(int64_t n_isec
     }
 }
 
+// Launch order of the compositing workgroups: all tiles by descending fragment count. Workgroups are dispatched in
+// index order as compute units free up, and dealt round-robin to the eight XCDs, so with this order the long tiles
+// of a clustered scene start at once instead of forming the tail of the launch, and every XCD receives the same
+// mix of loads (contiguous bands of tiles per XCD, which keep a band's splat rows in one L2, left whole XCDs idle
+// at the end: measured, the balance is worth far more than the locality). A counting sort in 256 classes of 32
+// fragments: workgroups of 1024 tiles count their classes into a table; a second kernel turns the table into
+// positions and scatters. The order inside a class does not matter.
+constexpr int kOrderBlock = 1024;
+__device__ __forceinline__ uint32_t tile_class(const int32_t* __restrict__ offsets, uint32_t t, uint32_t n_tiles, int64_t n_isects) {
+    const int64_t e = t + 1 < n_tiles ? (int64_t)offsets[t + 1] : n_isects;
+    const int64_t len = e - offsets[t];
+    return 255u - (uint32_t)min((int64_t)255, len >> 5);   // class 0 holds the longest tiles
+}
+// counts[block][256]: how many tiles of each class the workgroup's 1024 tiles hold
+__global__ __launch_bounds__(kOrderBlock) void tile_order_count_kernel(const int32_t* __restrict__ offsets, uint32_t n_tiles,
+                                                                       int64_t n_isects, uint32_t* __restrict__ counts) {
+    __shared__ uint32_t s_count[256];
+    if (threadIdx.x < 256) s_count[threadIdx.x] = 0;
+    __syncthreads();
+    const uint32_t t = blockIdx.x * kOrderBlock + threadIdx.x;
+    if (t < n_tiles) atomicAdd(&s_count[tile_class(offsets, t, n_tiles, n_isects)], 1u);
+    __syncthreads();
+    if (threadIdx.x < 256) counts[blockIdx.x * 256 + threadIdx.x] = s_count[threadIdx.x];
+}
+// Every workgroup sums the table for itself (a few dozen rows): the size of each class and what the workgroups
+// before it hold of it give, after a scan over the classes, where its own tiles of that class go.
+__global__ __launch_bounds__(kOrderBlock) void tile_order_scatter_kernel(const int32_t* __restrict__ offsets, uint32_t n_tiles,
+                                                                         int64_t n_isects, const uint32_t* __restrict__ counts,
+                                                                         int32_t* __restrict__ order) {
+    __shared__ uint32_t s_next[256];
+    __shared__ uint32_t s_wave[4];
+    if (threadIdx.x < 256) {
+        uint32_t total = 0, before = 0;
+        for (uint32_t b = 0; b < gridDim.x; b++) {
+            const uint32_t c = counts[b * 256 + threadIdx.x];
+            total += c;
+            if (b < blockIdx.x) before += c;
+        }
+        uint32_t incl = total;   // exclusive scan over the 256 classes: four wavefronts, then their totals
+        const int lane = threadIdx.x & 63;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t up = __shfl_up(incl, d, 64);
+            if (lane >= d) incl += up;
+        }
+        if (lane == 63) s_wave[threadIdx.x >> 6] = incl;
+        s_next[threadIdx.x] = incl - total + before;
+    }
+    __syncthreads();
+    if (threadIdx.x < 256) {
+        uint32_t add = 0;
+        for (uint32_t w = 0; w < (threadIdx.x >> 6); w++) add += s_wave[w];
+        s_next[threadIdx.x] += add;
+    }
+    __syncthreads();
+    const uint32_t t = blockIdx.x * kOrderBlock + threadIdx.x;
+    if (t < n_tiles) order[atomicAdd(&s_next[tile_class(offsets, t, n_tiles, n_isects)], 1u)] = (int32_t)t;
+}
+
 }  // namespace ssr
 
 using namespace ssr;
@@ -459,6 +518,26 @@ int ssr_tile_offsets(int64_t n_isects, const int64_t* sorted_ids, uint32_t n_til
     hipLaunchKernelGGL(tile_offsets_kernel, dim3((unsigned)ceil_div(n_isects, kTileBlock)), dim3(kTileBlock), 0,
                        as_stream(stream), n_isects, sorted_ids, (int64_t)n_tiles, offsets);
     SSR_CHECK_LAUNCH("ssr_tile_offsets");
+    return 0;
+}
+
+size_t ssr_tile_order_scratch_bytes(uint32_t n_tiles) {
+    return 256 * (size_t)ceil_div((int64_t)n_tiles, kOrderBlock) * sizeof(uint32_t);
+}
+
+int ssr_tile_order(const int32_t* tile_offsets, uint32_t n_tiles, int64_t n_isects, int32_t* order, void* scratch,
+                   size_t scratch_bytes, ssr_stream_t stream) {
+    SSR_REQUIRE(n_tiles < (1u << 30), "ssr_tile_order", "too many tiles");
+    if (n_tiles == 0) return 0;
+    SSR_REQUIRE(tile_offsets && order, "ssr_tile_order", "null pointer");
+    SSR_REQUIRE(n_isects >= 0, "ssr_tile_order", "negative count");
+    SSR_REQUIRE(scratch && scratch_bytes >= ssr_tile_order_scratch_bytes(n_tiles), "ssr_tile_order", "scratch too small");
+    uint32_t* counts = static_cast<uint32_t*>(scratch);
+    const dim3 grid((unsigned)ceil_div((int64_t)n_tiles, kOrderBlock)), block(kOrderBlock);
+    hipLaunchKernelGGL(tile_order_count_kernel, grid, block, 0, as_stream(stream), tile_offsets, n_tiles, n_isects, counts);
+    hipLaunchKernelGGL(tile_order_scatter_kernel, grid, block, 0, as_stream(stream), tile_offsets, n_tiles, n_isects,
+                       (const uint32_t*)counts, order);
+    SSR_CHECK_LAUNCH("ssr_tile_order");
     return 0;
 }
 

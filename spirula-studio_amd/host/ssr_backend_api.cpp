@@ -35,6 +35,8 @@ bool g_packed_mode = false;          // the last projection was the packed form
 std::vector<int64_t> g_packed_counts;   // ... and its rows per camera (rows are ordered by camera, then splat)
 int g_list_toggle = 0;               // which of the two visible-list buffers the last projection used
 float* g_vrows = nullptr;             // packed gradient rows of the last compositing backward (null: off)
+const int32_t* g_tile_order = nullptr;       // launch order of the compositing workgroups for the offsets below (null: off)
+const int32_t* g_tile_order_for = nullptr;   // the tile_offsets that order was made from
 const float* g_vrows_for_xy = nullptr; // the v_screen.xy buffer they stand in for
 const int32_t* g_bwd_list = nullptr; // list of the last projection backward
 int64_t g_bwd_count = 0;
@@ -442,6 +444,7 @@ do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, 
     if (!proj_xy || !proj_conic || !proj_opac)
         throw std::runtime_error("do_intersect_tile_generic: AABB mode is not built in this backend (ellipse mode is)");
     if (I < 1) throw std::runtime_error("do_intersect_tile_generic: no image");
+    g_tile_order = nullptr; g_tile_order_for = nullptr;
     const int64_t total = depths.numel();
     const int32_t* img_ids = (image_ids && I > 1) ? image_ids->data_ptr() : nullptr;   // packed rows of several cameras
     if (!img_ids && total % I != 0) throw std::runtime_error("do_intersect_tile_generic: rows are not a multiple of the image count");
@@ -519,6 +522,14 @@ do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, 
         StageTimer t(&g_times.k6);
         ok(ssr_tile_offsets(n_isects, ids_out.data_ptr(), n_tiles, offsets.data_ptr(), nullptr), "do_intersect_tile_generic/offsets");
     }
+    if (g_opts.tile_sort) {   // the native stage order also launches each XCD's longest tiles first
+        StageTimer t(&g_times.k6);   // the offsets themselves came out of the sort
+        // one slot: the order, then the scratch of the counting sort behind it
+        const size_t sb = ssr_tile_order_scratch_bytes(n_tiles);
+        int32_t* order = DevicePool::global().acquire<int32_t>(PoolSlot::IsectTileOrder, (size_t)n_tiles + sb / sizeof(int32_t));
+        ok(ssr_tile_order(offsets.data_ptr(), n_tiles, n_isects, order, order + n_tiles, sb, nullptr), "do_intersect_tile_generic/order");
+        g_tile_order = order; g_tile_order_for = offsets.data_ptr();
+    }
     return std::make_tuple(ids_out, flat_out, offsets);
 }
 
@@ -548,6 +559,7 @@ rasterize_to_pixels_3dgs_fwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     if (flatten_ids.size() > 0) p.screen = screen_of(splats_s);
     p.width = image_width; p.height = image_height;
     p.tile_offsets = tile_offsets.data_ptr(); p.flatten_ids = flatten_ids.data_ptr(); p.n_isects = flatten_ids.size();
+    if (g_tile_order && g_tile_order_for == p.tile_offsets) p.tile_order = g_tile_order;
     p.render_rgb = (float*)std::get<0>(renders).data_ptr(); p.render_depth = std::get<1>(renders).data_ptr();
     p.render_T = Ts.data_ptr(); p.last_ids = last.data_ptr();
     if (g_packed_rows && p.screen.xy == g_packed_for_xy) p.packed_rows = g_packed_rows;
@@ -626,6 +638,7 @@ rasterize_to_pixels_3dgs_bwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     p.screen = screen_of(splats_s);
     p.width = image_width; p.height = image_height;
     p.tile_offsets = tile_offsets.data_ptr(); p.flatten_ids = flatten_ids.data_ptr(); p.n_isects = flatten_ids.size();
+    if (g_tile_order && g_tile_order_for == p.tile_offsets) p.tile_order = g_tile_order;
     p.render_T = render_Ts.data_ptr(); p.last_ids = last_ids.data_ptr(); p.render_depth = std::get<1>(render_outputs_tuple).data_ptr();
     p.v_render_rgb = (const float*)std::get<0>(v_render_outputs).data_ptr();
     p.v_render_depth = std::get<1>(v_render_outputs).data_ptr();

@@ -55,7 +55,7 @@ class RasterFwdParams(C.Structure):
                 ("n_isects", C.c_int64), ("render_rgb", vp), ("render_depth", vp),
                 ("render_T", vp), ("last_ids", vp), ("packed_rows", vp), ("dist_type", C.c_int32),
                 ("distortion_rgb", vp), ("distortion_depth", vp), ("render_median", vp),
-                ("num_images", C.c_int32)]
+                ("num_images", C.c_int32), ("tile_order", vp)]
 
 
 class RasterBwdParams(C.Structure):
@@ -67,7 +67,7 @@ class RasterBwdParams(C.Structure):
                 ("distortion_rgb", vp), ("distortion_depth", vp), ("v_distortion_rgb", vp),
                 ("v_distortion_depth", vp), ("v_render_median", vp), ("accum_mode", C.c_int32),
                 ("accum_weight_map", vp), ("gaussian_ids", vp), ("num_world", C.c_int64), ("accum_weight", vp),
-                ("num_images", C.c_int32)]
+                ("num_images", C.c_int32), ("tile_order", vp)]
 
 
 class ProjectionBwdParams(C.Structure):
@@ -123,6 +123,8 @@ SYMBOLS = {
     "ssr_sort_scratch_bytes": (_sz, [_i64]),
     "ssr_sort_pairs_u64_i32": (_i32, [vp, vp, vp, vp, _i64, _i32, _i32, C.POINTER(C.c_int), vp, _sz, vp]),
     "ssr_tile_offsets": (_i32, [_i64, vp, _u32, vp, vp]),
+    "ssr_tile_order_scratch_bytes": (C.c_size_t, [C.c_uint32]),
+    "ssr_tile_order": (_i32, [vp, C.c_uint32, _i64, vp, vp, C.c_size_t, vp]),
     "ssr_sort_end_bit": (_i32, [_u32]),
     "ssr_sort_tile_scratch_bytes": (_sz, [_i64, _u32]),
     "ssr_sort_tile_pairs": (_i32, [vp, vp, vp, vp, _i64, _u32, vp, C.POINTER(C.c_int), vp, _sz, vp]),

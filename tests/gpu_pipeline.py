@@ -243,9 +243,26 @@ class GpuRun:
         if not (self.tile_sort and K):
             self.check(self.lib.ssr_tile_offsets(K, self.ptr(self.keys), n_tiles, self.ptr("offsets"), None))
 
+    def order_tiles(self):
+        """ssr_tile_order on the current offsets, checked here: a permutation of the tiles whose fragment counts fall
+        class by class (32 fragments a class, everything from 8160 up in the first)."""
+        D = self.L.DeviceArray
+        n_tiles = self.sc.tile_w * self.sc.tile_h
+        sb = self.lib.ssr_tile_order_scratch_bytes(n_tiles)
+        self.d["tile_order"], self.d["tile_order_scratch"] = D((n_tiles,), np.int32), D((sb,), np.uint8)
+        self.check(self.lib.ssr_tile_order(self.ptr("offsets"), n_tiles, self.K, self.ptr("tile_order"),
+                                           self.ptr("tile_order_scratch"), sb, None))
+        order = self.host("tile_order")
+        assert np.array_equal(np.sort(order), np.arange(n_tiles))
+        offs = self.host("offsets").ravel().astype(np.int64)
+        cls = np.minimum(np.diff(np.concatenate([offs, [self.K]])) >> 5, 255)[order]
+        assert np.all(cls[1:] <= cls[:-1])
+
     def raster_fwd(self):
         sc, D = self.sc, self.L.DeviceArray
         h, w = sc.height, sc.width
+        if self.tile_sort and self.K:   # the native stage order also launches the longest tiles first
+            self.order_tiles()
         for k, shape, dt in [("r_rgb", (h, w, 3), np.float32), ("r_depth", (h, w), np.float32),
                              ("r_T", (h, w), np.float32), ("r_last", (h, w), np.int32)]:
             self.d[k] = D(shape, dt)
@@ -268,6 +285,7 @@ class GpuRun:
         if va.get("median"):
             self.d["r_median"] = D((h, w), np.float32)
             p.render_median = self.ptr("r_median")
+        p.tile_order = self.ptr("tile_order")
         self.check(self.lib.ssr_raster_fwd(C.byref(p), None))
 
     def raster_bwd(self, v_rgb=None, v_depth=None, v_T=None):
@@ -316,6 +334,7 @@ class GpuRun:
             p.accum_weight_map, p.accum_weight, p.num_world = self.ptr("accum_map"), self.ptr("accum_weight"), self.n
             if self.packed_projection:
                 p.gaussian_ids = self.ptr("gaussian_ids")
+        p.tile_order = self.ptr("tile_order")
         self.check(self.lib.ssr_raster_bwd(C.byref(p), None))
         if self.use_vrows and n:   # unpack for the comparisons, after checking the arrays were left alone
             for k in ["v_xy", "v_depth", "v_conic", "v_opac", "v_rgb"]:

@@ -88,6 +88,9 @@ def test_argument_checks_without_device(L):
     # the allocation-free scan refuses what its fixed scratch cannot hold
     assert lib.ssr_inclusive_sum_i64_static(16, 16, (1 << 27) + 1, None, None) != 0 and b"static" in lib.ssr_last_error()
     assert lib.ssr_zero_world_rows(None, None, 0, None, None, 0, None) != 0 and b"null world" in lib.ssr_last_error()
+    assert lib.ssr_tile_order_scratch_bytes(8160) == 8 * 256 * 4
+    assert lib.ssr_tile_order(16, 100, 5, 16, None, 0, None) != 0 and b"scratch" in lib.ssr_last_error()
+    assert lib.ssr_tile_order(None, 0, 0, None, None, 0, None) == 0
 
 
 def test_missing_library_fails_loudly(pkg, monkeypatch):
