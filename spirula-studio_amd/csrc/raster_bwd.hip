@@ -9,63 +9,28 @@
 //     T0 = T1/(1-alpha); v_alpha = T0 (c.v_c) - v_T1 T0; v_c_k = alpha T0 v_c;
 //     v_T0 = alpha (c.v_c) + v_T1 (1-alpha)
 //
-// Native schedule instead of the reference's 32-lane systolic sweep: a wavefront holds the 64
-// pixels of one 8x8 sub-tile in its lanes (state in registers, no LDS traffic for it); fragments
-// are staged per 16x16 tile in LDS, back to front, shared by the tile's 4 wavefronts; each
-// wavefront walks the fragments whose footprint bit is set. The ten per-splat sums are reduced
-// across the wavefront by a transposing reduction: v_permlane32_swap and v_permlane16_swap (gfx950)
-// each fold one level of TWO channels at once, leaving 3 registers that hold one channel per
-// 16-lane row; 4 DPP steps per register finish the rows (28 operations instead of 60). Ten lanes
-// then issue ONE float atomic instruction per (splat, sub-tile) -- the same number of atomic
-// operations as the reference (src/primitives/PrimitiveBase3DGS.cuh:177-183), non-finite sums
-// dropped and zeros skipped as there (src/core/Common.cuh:791-856). The scan starts at the tile's largest
-// last_id rather than at the end of the range; splats beyond it are skipped by every pixel anyway.
+// Native schedule instead of the reference's 32-lane systolic sweep: one workgroup per 16x16 tile, a wavefront per
+// 8x8 sub-tile, and within it each 16-lane row holds one 4x4-pixel block (pixel state in registers). Fragments are
+// staged per tile in LDS, back to front, shared by the tile's four wavefronts; every row walks its OWN list of the
+// staged fragments -- those whose block bit is set (raster_device.h) and whose sorted index does not exceed the
+// block's largest last_id. A splat of a few pixels' radius touches about half of the blocks of the sub-tiles it
+// touches, so far fewer lanes idle than when all 64 lanes visit every fragment of the sub-tile. Lists are built per
+// batch by the wavefront that walks them (ballot + rank, slot numbers as bytes). The scan starts at the tile's
+// largest last_id rather than at the end of the range; splats beyond it are skipped by every pixel anyway.
+// The ten per-splat sums are reduced inside each row by a transposing reduction over the four lane bits (row_ror:8,
+// row_half_mirror, two quad permutations): every level halves the number of live registers by keeping one channel in
+// the lanes with the bit clear and another in those with it set, so 23 operations leave each of ten lanes of the
+// row holding one finished channel. What is summed are moments of u = vis * v_alpha: (u, u dx, u dy, u dx^2,
+// u dx dy, u dy^2) and the four colour / depth weights; the gradients of position, conic and opacity are linear in
+// them and are formed once per fragment when its sums leave LDS for global memory -- one set of atomics per (splat,
+// tile), non-finite sums dropped and zeros skipped as in the reference (src/core/Common.cuh:791-856).
+// exp(-sigma) comes from the hardware exponential; whenever a lane's alpha falls within 1.6e-7 of the 1/255
+// threshold or within 4e-5 of the 0.999 gate, the wavefront re-evaluates with the bit-defined exponential, so every
+// decision is the one the forward took.
 #include "raster_device.h"
-#include <stdlib.h>
 
 namespace ssr {
 
-template <int kCtrl>
-__device__ __forceinline__ float dpp_get(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, 0xf, 0xf, true));
-}
-
-// lanes 0..31: a[l] + a[l+32]; lanes 32..63: b[l-32] + b[l]
-__device__ __forceinline__ float fold32(float a, float b) {
-    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
-    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-}
-// rows (16 lanes each): row0 = a.row0 + a.row1, row1 = b.row0 + b.row1, row2 = a.row2 + a.row3,
-// row3 = b.row2 + b.row3
-__device__ __forceinline__ float fold16(float a, float b) {
-    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
-    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-}
-// every lane of a row receives the sum over its row
-__device__ __forceinline__ float row_sum(float v) {
-    v += dpp_get<0xB1>(v);     // quad_perm [1,0,3,2]
-    v += dpp_get<0x4E>(v);     // quad_perm [2,3,0,1]
-    v += dpp_get<0x141>(v);    // row_half_mirror
-    v += dpp_get<0x140>(v);    // row_mirror
-    return v;
-}
-
-__device__ __forceinline__ int wave_max_i32(int v) {
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) v = max(v, __shfl_xor(v, d, 64));
-    return v;
-}
-
-__device__ __forceinline__ float wave_sum_f32(float v) {
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
-    return v;
-}
-__device__ __forceinline__ float wave_max_f32(float v) {
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) v = ssr_max(v, __shfl_xor(v, d, 64));
-    return v;
-}
 // float atomic max through the integer orderings (src/core/Common.cuh:784-788)
 __device__ __forceinline__ void atomic_max_f32(float* p, float v) {
     if (__float_as_int(v) >= 0) atomicMax(reinterpret_cast<int*>(p), __float_as_int(v));
@@ -81,285 +46,6 @@ __device__ __forceinline__ int64_t accum_row(const ssr_raster_bwd_params& P, uin
     if (P.gaussian_ids) return (int64_t)P.gaussian_ids[g];
     return P.num_images > 1 ? (int64_t)(g % (uint32_t)P.num_world) : (int64_t)g;
 }
-
-template <int kDist, bool kMedian, int kAccum>
-__global__ __launch_bounds__(kRasterBlock) void raster_bwd_kernel(ssr_raster_bwd_params P, int tile_w, int tile_h) {
-    __shared__ FragLds frags[kBatch];
-    __shared__ int32_t s_ids[kBatch];
-    __shared__ int s_wave_max[4];
-    // Per-fragment gradient sums of the whole tile: the four wavefronts (sub-tiles) add their reduced
-    // sums here with LDS atomics, and each staged fragment goes to global memory once per batch --
-    // one set of global atomics per (splat, tile) instead of one per (splat, sub-tile).
-    constexpr int kAccCh = (kAccum == SSR_ACCUM_SUM || kAccum == SSR_ACCUM_AVG) ? 12 : 10;
-    __shared__ float s_acc[kBatch * kAccCh];
-    // distortion composites ln(max(z, 1e-6)): a per-splat value, taken once when the fragment is staged
-    [[maybe_unused]] __shared__ float s_lz[kDist != SSR_DIST_NONE ? kBatch : 1];
-    // images stack in the tile space: image c owns tiles [c tile_w tile_h, (c+1) tile_w tile_h)
-    const int n_tiles = tile_w * tile_h * (P.num_images > 1 ? P.num_images : 1);
-    const int tile = tile_of_workgroup(P.tile_order, blockIdx.x, n_tiles);
-    if (tile < 0 || tile >= n_tiles) return;
-    const int tid = threadIdx.x, lane = tid & 63, mt = tid >> 6;
-    const int gy = tile / tile_w, tx = tile - gy * tile_w;
-    const int img = gy / tile_h, ty = gy - img * tile_h;
-    const int j = tx * kTile + (mt & 1) * kMicro + (lane & 7);
-    const int i = ty * kTile + (mt >> 1) * kMicro + (lane >> 3);
-    const float px = (float)j + 0.5f, py = (float)i + 0.5f;
-    const bool inside = (uint32_t)i < P.height && (uint32_t)j < P.width;
-    const int64_t pid = ((int64_t)img * P.height + i) * P.width + j;
-
-    // per-pixel state (RasterizationEval3DBwd_kernel.cuh:186-232)
-    const int32_t bin_final = inside ? P.last_ids[pid] : -1;
-    float T1 = inside ? P.render_T[pid] : 0.0f;
-    float vT1 = inside ? P.v_render_T[pid] : 0.0f;
-    float vr = 0.f, vg = 0.f, vb = 0.f, vd = 0.f;
-    if (inside) {
-        const float* v = P.v_render_rgb + 3 * pid;
-        vr = v[0]; vg = v[1]; vb = v[2];
-        vd = P.v_render_depth[pid];
-    }
-    // totals of the forward held constant during the sweep (distortion), median state, weight map
-    [[maybe_unused]] float Cr = 0.f, Cg = 0.f, Cb = 0.f, Cd = 0.f, Sr = 0.f, Sg = 0.f, Sb = 0.f, Sd = 0.f;
-    [[maybe_unused]] float vDr = 0.f, vDg = 0.f, vDb = 0.f, vDd = 0.f, Wd = 0.f;
-    [[maybe_unused]] float med_v = 0.f, pend_zgrad = 0.f, pend_zfar = 0.f, pend_Tfar = 0.f, amap = 0.f;
-    {
-        const float inv_alpha = 1.0f / ssr_max(1.0f - T1, 1e-10f);
-        const float exp_depth = inside ? P.render_depth[pid] : 0.0f;
-        if constexpr (kDist != SSR_DIST_NONE) {
-            // log-depth render: depth = exp(C_lnz / W)  (RasterizationEval3DBwd_kernel.cuh:212-218)
-            const float m = ssr_log(ssr_max(exp_depth, 1e-6f));
-            vT1 = vT1 + ((exp_depth * vd) * m) * inv_alpha;
-            vd = vd * (exp_depth * inv_alpha);
-            // C, S = (D + C^2) / W, W and the distortion cotangent (:228-257)
-            Cd = m * ssr_max(1.0f - T1, 1e-10f);
-            Wd = inside ? (1.0f - T1) : 0.0f;
-            const float invW = Wd > 1e-10f ? (1.0f / Wd) : 0.0f;
-            float Dd = 0.f, Dr = 0.f, Dg = 0.f, Db = 0.f;
-            if (inside) {
-                Dd = P.distortion_depth[pid]; vDd = P.v_distortion_depth[pid];
-                if constexpr (kDist == SSR_DIST_RGB_D) {
-                    const float* c = P.render_rgb + 3 * pid; Cr = c[0]; Cg = c[1]; Cb = c[2];
-                    const float* d = P.distortion_rgb + 3 * pid; Dr = d[0]; Dg = d[1]; Db = d[2];
-                    const float* v = P.v_distortion_rgb + 3 * pid; vDr = v[0]; vDg = v[1]; vDb = v[2];
-                }
-            }
-            Sd = (Dd + Cd * Cd) * invW;
-            if constexpr (kDist == SSR_DIST_RGB_D) {
-                Sr = (Dr + Cr * Cr) * invW; Sg = (Dg + Cg * Cg) * invW; Sb = (Db + Cb * Cb) * invW;
-            }
-        } else {
-            vT1 = vT1 + (exp_depth * vd) * inv_alpha;
-            vd = vd * inv_alpha;
-        }
-        if constexpr (kMedian) med_v = inside ? P.v_render_median[pid] : 0.0f;
-        if constexpr (kAccum != SSR_ACCUM_NONE) amap = inside ? P.accum_weight_map[pid] : 0.0f;
-    }
-
-    const int32_t range_start = P.tile_offsets[tile];
-    const int32_t range_end = (tile == n_tiles - 1) ? (int32_t)P.n_isects : P.tile_offsets[tile + 1];
-    const int wave_last = wave_max_i32(bin_final);
-    if (lane == 0) s_wave_max[mt] = wave_last;
-    __syncthreads();
-    const int tile_last = max(max(s_wave_max[0], s_wave_max[1]), max(s_wave_max[2], s_wave_max[3]));
-    const float tile_x0 = (float)(tx * kTile), tile_y0 = (float)(ty * kTile);
-
-    // After the reduction, row r of register j holds channel kChan[j][r] in all its lanes; lane
-    // 16 r + j (j < 3) adds that channel. Destination = base + stride * splat, fixed per lane.
-    //   channels: 0,1 xy  2 depth  3,4,5 conic  6 opac  7,8,9 rgb
-    const int row = lane >> 4, sub = lane & 15;
-    int chan = -1;
-    if (sub == 0) chan = row == 0 ? 0 : row == 1 ? 2 : row == 2 ? 1 : 3;
-    else if (sub == 1) chan = row == 0 ? 4 : row == 1 ? 6 : row == 2 ? 5 : 7;
-    else if (sub == 2 && (row & 1) == 0) chan = row == 0 ? 8 : 9;
-    else if (sub == 2 && (kAccum == SSR_ACCUM_SUM || kAccum == SSR_ACCUM_AVG) && (row == 1 || kAccum == SSR_ACCUM_AVG))
-        chan = row == 1 ? 10 : 11;   // the weight sums ride in the two spare rows of the third register
-#pragma unroll
-    for (int c = 0; c < kAccCh; c++) s_acc[tid * kAccCh + c] = 0.0f;
-    // Thread t owns fragment slot t: it moves that slot's sums to global memory (zeros skipped, as in
-    // src/core/Common.cuh:791-856) and clears them. Called between two barriers.
-    auto flush_slot = [&]() {
-        if (P.v_rows) {
-            // all 256 slots x 10 channels in memory order of the destination rows: the lanes of one
-            // instruction cover whole rows, so a row's atomics travel as one or two requests
-            __syncthreads();   // slot owners differ from readers here: wait for every wavefront's sums
-            for (int e = tid; e < kBatch * 10; e += kRasterBlock) {
-                const int slot = e / 10, ch = e - slot * 10;
-                const float x = s_acc[slot * kAccCh + ch];
-                if (x != 0.0f) {
-                    s_acc[slot * kAccCh + ch] = 0.0f;
-                    atomicAdd(P.v_rows + 12u * (uint32_t)s_ids[slot] + (uint32_t)ch, x);
-                }
-            }
-            if constexpr (kAccCh == 12) {
-                const float a = s_acc[tid * kAccCh + 10], b = s_acc[tid * kAccCh + 11];
-                if (a != 0.0f || b != 0.0f) {
-                    s_acc[tid * kAccCh + 10] = 0.0f; s_acc[tid * kAccCh + 11] = 0.0f;
-                    const uint32_t g = (uint32_t)s_ids[tid];
-                    const int64_t wid = accum_row(P, g);
-                    if (a != 0.0f) atomicAdd(P.accum_weight + wid, a);
-                    if (kAccum == SSR_ACCUM_AVG && b != 0.0f) atomicAdd(P.accum_weight + P.num_world + wid, b);
-                }
-            }
-            __syncthreads();   // s_ids and s_acc are free for the next batch
-            return;
-        }
-        float v[kAccCh];
-        bool any = false;
-#pragma unroll
-        for (int c = 0; c < kAccCh; c++) { v[c] = s_acc[tid * kAccCh + c]; any |= v[c] != 0.0f; }
-        if (!any) return;
-#pragma unroll
-        for (int c = 0; c < kAccCh; c++) s_acc[tid * kAccCh + c] = 0.0f;
-        const uint32_t g = (uint32_t)s_ids[tid];   // < 2^30 rows, so every index below fits 32 bits
-        auto add = [](float* p, float x) { if (x != 0.0f) atomicAdd(p, x); };
-        add(P.v_screen.xy + 2u * g, v[0]); add(P.v_screen.xy + 2u * g + 1u, v[1]);
-        add(P.v_screen.depth + g, v[2]);
-        add(P.v_screen.conic + 3u * g, v[3]); add(P.v_screen.conic + 3u * g + 1u, v[4]); add(P.v_screen.conic + 3u * g + 2u, v[5]);
-        add(P.v_screen.opac + g, v[6]);
-        add(P.v_screen.rgb + 3u * g, v[7]); add(P.v_screen.rgb + 3u * g + 1u, v[8]); add(P.v_screen.rgb + 3u * g + 2u, v[9]);
-        if constexpr (kAccCh == 12) {
-            const int64_t wid = accum_row(P, g);
-            add(P.accum_weight + wid, v[10]);
-            if constexpr (kAccum == SSR_ACCUM_AVG) add(P.accum_weight + P.num_world + wid, v[11]);
-        }
-    };
-
-    for (int32_t hi = min(range_end - 1, tile_last); hi >= range_start; hi -= kBatch) {
-        __syncthreads();   // previous batch fully consumed
-        flush_slot();      // its sums leave before the slot is reused (first pass: all zero)
-        const int32_t idx = hi - tid;   // LDS slot t holds sorted index hi - t: ascending t is back to front
-        if (idx >= range_start) {
-            const int32_t g = P.flatten_ids[idx];
-            s_ids[tid] = g;
-            frags[tid] = stage_fragment(P.screen, P.packed_rows, g, tile_x0, tile_y0);
-            if constexpr (kDist != SSR_DIST_NONE) s_lz[tid] = ssr_log(ssr_max(frags[tid].q2.y, 1e-6f));
-        } else {
-            frags[tid].q2 = make_float4(0.f, 0.f, 0.f, 0.f);
-        }
-        __syncthreads();
-        const int n_batch = min(kBatch, hi - range_start + 1);
-        for (int c = 0; c * 64 < n_batch; c++) {
-            if (hi - c * 64 - 63 > wave_last) continue;   // nothing in this chunk is <= any last_id here
-            const uint32_t my_hits = __float_as_uint(frags[c * 64 + lane].q2.z);
-            uint64_t m = __ballot((my_hits >> mt) & 1u);
-            while (m) {
-                const int t = __builtin_ctzll(m);
-                m &= m - 1;
-                const int k = c * 64 + t;
-                const int32_t sorted_idx = hi - k;
-                if (sorted_idx > wave_last) continue;
-                const float4 q0 = frags[k].q0, q1 = frags[k].q1, q2 = frags[k].q2;
-                float dx, dy, vis, sigma;
-                const float alpha = eval_alpha_fast(q0, q1, q2.w, px, py, dx, dy, vis, sigma);
-                const bool active = sorted_idx <= bin_final && alpha > kAlphaThreshold;
-                if (__ballot(active) == 0ull) continue;
-                // Branch-free per-lane terms: an inactive lane runs with alpha = 0 and v_alpha = 0, which
-                // leaves its T and v_T unchanged (T/(1-0) = T, v_T + 0*(..) = v_T) and makes every term zero.
-                const float cr = q1.z, cg = q1.w, cb = q2.x;
-                float cdp = q2.y;
-                const float a = active ? alpha : 0.0f;
-                // 1/(1-alpha) by the hardware reciprocal (1 ulp): gradients are compared at 1e-3
-                const float T0 = T1 * __builtin_amdgcn_rcpf(1.0f - a);
-                [[maybe_unused]] float v_depth_median = 0.0f;
-                if constexpr (kMedian) {   // RasterizationEval3DBwd_kernel.cuh:433-470
-                    if (active && pend_Tfar > 0.0f) {   // near member of the crossing found at the previous active splat
-                        v_depth_median += pend_zgrad;
-                        const float dba = ssr_log(pend_Tfar) - ssr_log(T1);
-                        const float inv = (ssr_fabs(dba) > 1e-20f) ? (-1.0f / dba) : 0.0f;
-                        vT1 += ((med_v * (pend_zfar - q2.y)) * inv) / T1;
-                        pend_Tfar = 0.0f;
-                    }
-                    if (active && T0 >= 0.5f && T1 < 0.5f) {   // far member: post-splat T drops below 1/2 here
-                        const float la = ssr_log(T0), d = ssr_log(T1) - la;
-                        const float fr = (ssr_fabs(d) > 1e-20f) ? (-0.6931471805599453f - la) / d : 0.0f;
-                        v_depth_median += fr * med_v;
-                        pend_zgrad = (1.0f - fr) * med_v;
-                        pend_zfar = q2.y;
-                        pend_Tfar = T1;
-                    }
-                }
-                if constexpr (kDist != SSR_DIST_NONE) cdp = s_lz[k];
-                float dv = ssr_fma(cdp, vd, ssr_fma(cb, vb, ssr_fma(cg, vg, cr * vr))) - vT1;
-                const float w = a * T0;
-                [[maybe_unused]] float xr = 0.f, xg = 0.f, xb = 0.f, xd = 0.f;   // distortion part of the colour gradient
-                if constexpr (kDist != SSR_DIST_NONE) {   // closed form D = W S - C^2 (:497-517)
-                    float gsum = 0.0f;
-                    const float w2 = 2.0f * w;
-                    if constexpr (kDist == SSR_DIST_RGB_D) {
-                        xr = ((cr * Wd - Cr) * vDr) * w2; xg = ((cg * Wd - Cg) * vDg) * w2; xb = ((cb * Wd - Cb) * vDb) * w2;
-                        gsum += ((Sr + (cr * cr) * Wd) - (cr * Cr) * 2.0f) * vDr;
-                        gsum += ((Sg + (cg * cg) * Wd) - (cg * Cg) * 2.0f) * vDg;
-                        gsum += ((Sb + (cb * cb) * Wd) - (cb * Cb) * 2.0f) * vDb;
-                    }
-                    xd = ((cdp * Wd - Cd) * vDd) * w2;
-                    gsum += ((Sd + (cdp * cdp) * Wd) - (cdp * Cd) * 2.0f) * vDd;
-                    dv += gsum;   // v_alpha gains T0 g and v_T0 gains alpha g, exactly where dv enters
-                }
-                const float ov = q1.y * vis;
-                // evaluate_alpha_vjp gate (src/primitives/Primitive3DGS.cuh:273); sigma >= 0 holds when active
-                const float v_alpha = (active && ov <= 0.999f) ? T0 * dv : 0.0f;
-                vT1 = ssr_fma(a, dv, vT1);
-                T1 = T0;
-                const float v_sigma = (-ov) * v_alpha;
-                const float vsx = v_sigma * dx, vsy = v_sigma * dy;
-                const float t_ca = (0.5f * vsx) * dx, t_cb = vsx * dy, t_cc = (0.5f * vsy) * dy;
-                // conic.x = 2 * (0.5 conic.x), conic.z likewise
-                const float t_x = ssr_fma(q0.z + q0.z, vsx, q0.w * vsy);
-                const float t_y = ssr_fma(q0.w, vsx, (q1.x + q1.x) * vsy);
-                const float t_o = vis * v_alpha;
-                float t_r = vr * w, t_g = vg * w, t_b = vb * w, t_d = vd * w;
-                if constexpr (kDist != SSR_DIST_NONE) {
-                    if constexpr (kDist == SSR_DIST_RGB_D) { t_r += xr; t_g += xg; t_b += xb; }
-                    t_d = (t_d + xd) * (1.0f / ssr_max(q2.y, 1e-6f));   // d/d ln z -> d/dz
-                }
-                if constexpr (kMedian) t_d += v_depth_median;
-                [[maybe_unused]] int64_t wid = 0;
-                if constexpr (kAccum != SSR_ACCUM_NONE) {   // :553-562,574-585
-                    wid = accum_row(P, (uint32_t)s_ids[k]);
-                    if constexpr (kAccum == SSR_ACCUM_MAX) {
-                        const float mx = wave_max_f32(amap * w);   // inactive lanes contribute map * 0; the running max starts at 0
-                        if (lane == 0) atomic_max_f32(P.accum_weight + wid, ssr_max(mx, 0.0f));
-                    }
-                }
-                // transposing reduction: 10 channels -> 3 registers with one channel per row
-                const float ra_ = fold32(t_x, t_y), rb_ = fold32(t_d, t_ca), rc_ = fold32(t_cb, t_cc),
-                            rd_ = fold32(t_o, t_r), re_ = fold32(t_g, t_b);
-                const float s1 = row_sum(fold16(ra_, rb_));   // rows: x, d, y, ca      -> channels 0,2,1,3
-                const float s2 = row_sum(fold16(rc_, rd_));   // rows: cb, o, cc, r     -> channels 4,6,5,7
-                float s3;
-                if constexpr (kAccum == SSR_ACCUM_SUM || kAccum == SSR_ACCUM_AVG) {
-                    // the weight sums ride in the two spare rows of the third register
-                    const float rf_ = fold32(amap * w, w);
-                    s3 = row_sum(fold16(re_, rf_));           // rows: g, sum map w, b, sum w -> channels 8,10,9,11
-                } else {
-                    s3 = row_sum(fold16(re_, re_));           // rows: g, g, b, b       -> channels 8,8,9,9
-                }
-                float mine = sub == 0 ? s1 : (sub == 1 ? s2 : s3);
-                if (chan >= 0 && ssr_isfinite(mine) && mine != 0.0f) atomicAdd(&s_acc[k * kAccCh + chan], mine);
-            }
-        }
-    }
-    __syncthreads();
-    flush_slot();
-}
-
-// ---- the row-granular plain kernel --------------------------------------------------------------
-//
-// Same per-pixel arithmetic, different walk: a wavefront's four 16-lane rows each hold one 4x4-pixel
-// block of the wavefront's 8x8 sub-tile and walk their OWN list of the staged fragments -- those whose
-// block bit is set (raster_device.h) and whose sorted index does not exceed the block's largest
-// last_id. A splat of a few pixels' radius touches about half of the blocks of the sub-tiles it
-// touches, so far fewer lanes idle than when all 64 lanes visit every fragment of the sub-tile.
-// Lists are built per batch by the wavefront that walks them (ballot + rank, slot numbers as bytes).
-// The ten per-splat sums are reduced inside each row by a transposing reduction over the four lane
-// bits (row_ror:8, row_half_mirror, two quad permutations): every level halves the number of live
-// registers by keeping one channel in the lanes with the bit clear and another in those with it
-// set, so 29 operations leave each of ten lanes of the row holding one finished channel.
-// What is summed are moments of u = vis * v_alpha: (u, u dx, u dy, u dx^2, u dx dy, u dy^2) and the four
-// colour / depth weights; the gradients of position, conic and opacity are linear in them and are
-// formed once per fragment when its sums leave LDS.
-// exp(-sigma) comes from the hardware exponential; whenever a lane's alpha falls within 4e-5 relative
-// of the 1/255 threshold or of the 0.999 gate, the wavefront re-evaluates with the bit-defined
-// exponential, so every decision is the one the forward took.
 
 template <int kCtrl>
 __device__ __forceinline__ float dpp_full(float v) {
@@ -664,7 +350,7 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
             const bool in_range = (k >= k_min) & !(sigma < 0.f || sigma > cut);
             float vis = in_range ? __builtin_amdgcn_exp2f(sigma * -1.44269504088896341f) : 0.0f;
             float ov = q1.y * vis;
-            const bool near_edge = (ssr_fabs(ov - kAlphaThreshold) <= 1.6e-7f) | (ssr_fabs(ov - 0.999f) <= 4e-5f);
+            const bool near_edge = ((int)(ssr_fabs(ov - kAlphaThreshold) <= 1.6e-7f) | (int)(ssr_fabs(ov - 0.999f) <= 4e-5f)) != 0;
             if (__builtin_amdgcn_ballot_w64(near_edge) != 0ull) {   // decisions exactly as the forward took them
                 vis = in_range ? exp_neg_small(-sigma) : 0.0f;
                 ov = q1.y * vis;
@@ -904,19 +590,6 @@ extern "C" int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t strea
     const dim3 grid((unsigned)xcd_grid_size(tw * th * nimg)), block(kRasterBlock);
     hipStream_t st = as_stream(stream);
     const bool med = p->v_render_median != nullptr;
-#define SSR_BWD(D, M, A) hipLaunchKernelGGL((raster_bwd_kernel<D, M, A>), grid, block, 0, st, *p, tw, th)
-#define SSR_BWD_A(D, M)                                        \
-    switch (p->accum_mode) {                                   \
-        case SSR_ACCUM_MAX: SSR_BWD(D, M, SSR_ACCUM_MAX); break; \
-        case SSR_ACCUM_SUM: SSR_BWD(D, M, SSR_ACCUM_SUM); break; \
-        case SSR_ACCUM_AVG: SSR_BWD(D, M, SSR_ACCUM_AVG); break; \
-        default: SSR_BWD(D, M, SSR_ACCUM_NONE); break;           \
-    }
-#define SSR_BWD_M(D) if (med) { SSR_BWD_A(D, true) } else { SSR_BWD_A(D, false) }
-    // The plain variant runs the row-granular kernel; SSR_RASTER_WAVE_VISITS=1 in the environment
-    // selects the one-wavefront-per-visit kernel instead (for comparisons).
-    static const bool wave_visits = getenv("SSR_RASTER_WAVE_VISITS") != nullptr;
-    if (!wave_visits) {
 #define SSR_ROWS(D, M, A) hipLaunchKernelGGL((raster_bwd_rows_kernel<D, M, A>), grid, block, 0, st, *p, tw, th)
 #define SSR_ROWS_A(D, M)                                          \
     switch (p->accum_mode) {                                      \
@@ -926,30 +599,19 @@ extern "C" int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t strea
         default: SSR_ROWS(D, M, SSR_ACCUM_NONE); break;             \
     }
 #define SSR_ROWS_M(D) if (med) { SSR_ROWS_A(D, true) } else { SSR_ROWS_A(D, false) }
-        if (p->dist_type == SSR_DIST_NONE && !med && p->accum_mode == SSR_ACCUM_AVG)
-            hipLaunchKernelGGL(raster_bwd_rows_avg_kernel, grid, block, 0, st, *p, tw, th);
-        else switch (p->dist_type) {
-            case SSR_DIST_D: SSR_ROWS_M(SSR_DIST_D); break;
-            case SSR_DIST_RGB_D: SSR_ROWS_M(SSR_DIST_RGB_D); break;
-            default: SSR_ROWS_M(SSR_DIST_NONE); break;
-        }
+    if (p->dist_type == SSR_DIST_NONE && !med && p->accum_mode == SSR_ACCUM_AVG)
+        hipLaunchKernelGGL(raster_bwd_rows_avg_kernel, grid, block, 0, st, *p, tw, th);
+    else switch (p->dist_type) {
+        case SSR_DIST_D: SSR_ROWS_M(SSR_DIST_D); break;
+        case SSR_DIST_RGB_D: SSR_ROWS_M(SSR_DIST_RGB_D); break;
+        default: SSR_ROWS_M(SSR_DIST_NONE); break;
+    }
 #undef SSR_ROWS_M
 #undef SSR_ROWS_A
 #undef SSR_ROWS
-        if (p->v_rows && (p->accum_mode == SSR_ACCUM_SUM || p->accum_mode == SSR_ACCUM_AVG))
-            hipLaunchKernelGGL(accum_from_rows_kernel, dim3((unsigned)ceil_div(p->num_splats, 256)), dim3(256), 0, st, *p,
-                               p->accum_mode == SSR_ACCUM_AVG ? 1 : 0);
-        SSR_CHECK_LAUNCH("ssr_raster_bwd");
-        return 0;
-    }
-    switch (p->dist_type) {
-        case SSR_DIST_D: SSR_BWD_M(SSR_DIST_D) break;
-        case SSR_DIST_RGB_D: SSR_BWD_M(SSR_DIST_RGB_D) break;
-        default: SSR_BWD_M(SSR_DIST_NONE) break;
-    }
-#undef SSR_BWD_M
-#undef SSR_BWD_A
-#undef SSR_BWD
+    if (p->v_rows && (p->accum_mode == SSR_ACCUM_SUM || p->accum_mode == SSR_ACCUM_AVG))
+        hipLaunchKernelGGL(accum_from_rows_kernel, dim3((unsigned)ceil_div(p->num_splats, 256)), dim3(256), 0, st, *p,
+                           p->accum_mode == SSR_ACCUM_AVG ? 1 : 0);
     SSR_CHECK_LAUNCH("ssr_raster_bwd");
     return 0;
 }

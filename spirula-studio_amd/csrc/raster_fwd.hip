@@ -7,121 +7,14 @@
 // WITHOUT adding this splat; else accumulate rgb*alpha*T, depth*alpha*T and remember the sorted
 // index. Outputs rgb, depth / max(1-T, 1e-10), T and last_id.
 #include "raster_device.h"
-#include <stdlib.h>
 
 namespace ssr {
 
-// kDist (SSR_DIST_*) and kMedian select the variants (RasterizationEval3DFwd_kernel.cuh:143-148,245-307);
-// <0, false> is the plain kernel and compiles to exactly the code it had without them.
-template <int kDist, bool kMedian>
-__global__ __launch_bounds__(kRasterBlock) void raster_fwd_kernel(ssr_raster_fwd_params P, int tile_w, int tile_h) {
-    __shared__ FragLds frags[kBatch];
-    // distortion composites ln(max(z, 1e-6)): a per-splat value, taken once when the fragment is staged
-    [[maybe_unused]] __shared__ float s_lz[kDist != SSR_DIST_NONE ? kBatch : 1];
-    // images stack in the tile space: image c owns tiles [c tile_w tile_h, (c+1) tile_w tile_h)
-    const int n_tiles = tile_w * tile_h * (P.num_images > 1 ? P.num_images : 1);
-    const int tile = tile_of_workgroup(P.tile_order, blockIdx.x, n_tiles);
-    if (tile < 0 || tile >= n_tiles) return;   // whole workgroup leaves together
-    const int tid = threadIdx.x, lane = tid & 63, mt = tid >> 6;
-    const int gy = tile / tile_w, tx = tile - gy * tile_w;
-    const int img = gy / tile_h, ty = gy - img * tile_h;
-    const int j = tx * kTile + (mt & 1) * kMicro + (lane & 7);
-    const int i = ty * kTile + (mt >> 1) * kMicro + (lane >> 3);
-    const float px = (float)j + 0.5f, py = (float)i + 0.5f;
-    const bool inside = (uint32_t)i < P.height && (uint32_t)j < P.width;
-    bool done = !inside;
-
-    const int32_t range_start = P.tile_offsets[tile];
-    const int32_t range_end = (tile == n_tiles - 1) ? (int32_t)P.n_isects : P.tile_offsets[tile + 1];
-
-    float T = 1.0f, cr = 0.f, cg = 0.f, cb = 0.f, cd = 0.f;
-    [[maybe_unused]] float s2r = 0.f, s2g = 0.f, s2b = 0.f, s2d = 0.f;           // second moments (distortion)
-    [[maybe_unused]] float median = 0.f, med_prev_z = 0.f, med_prev_T = 1.0f;   // median depth
-    uint32_t cur_idx = 0;
-    const float tile_x0 = (float)(tx * kTile), tile_y0 = (float)(ty * kTile);
-
-    for (int32_t batch_start = range_start; batch_start < range_end; batch_start += kBatch) {
-        // all pixels of the tile finished: stop (this barrier also fences reuse of the LDS batch)
-        if (__syncthreads_count(done) >= kRasterBlock) break;
-        const int32_t idx = batch_start + tid;
-        if (idx < range_end) {
-            frags[tid] = stage_fragment(P.screen, P.packed_rows, P.flatten_ids[idx], tile_x0, tile_y0);
-            if constexpr (kDist != SSR_DIST_NONE) s_lz[tid] = ssr_log(ssr_max(frags[tid].q2.y, 1e-6f));
-        } else {
-            frags[tid].q2 = make_float4(0.f, 0.f, 0.f, 0.f);   // empty footprint mask
-        }
-        __syncthreads();
-        const int n_batch = min(kBatch, range_end - batch_start);
-        for (int c = 0; c * 64 < n_batch; c++) {
-            if (__ballot(!done) == 0ull) break;   // this sub-tile is finished
-            const uint32_t my_hits = __float_as_uint(frags[c * 64 + lane].q2.z);
-            uint64_t m = __ballot((my_hits >> mt) & 1u);
-            while (m) {
-                const int t = __builtin_ctzll(m);
-                m &= m - 1;
-                const int k = c * 64 + t;
-                const float4 q0 = frags[k].q0, q1 = frags[k].q1, q2 = frags[k].q2;
-                float dx, dy, vis, sigma;
-                const float alpha = eval_alpha_fast(q0, q1, q2.w, px, py, dx, dy, vis, sigma);
-                if (!done && alpha > kAlphaThreshold) {
-                    const float next_T = T * (1.0f - alpha);
-                    if constexpr (kMedian) {   // before the early-out, so a splat that ends the pixel still counts
-                        if (med_prev_T >= 0.5f && next_T < 0.5f) {
-                            const float a = ssr_log(med_prev_T), b = ssr_log(next_T), d = b - a;
-                            const float fr = (ssr_fabs(d) > 1e-20f) ? (-0.6931471805599453f - a) / d : 0.0f;
-                            median = med_prev_z + (q2.y - med_prev_z) * fr;
-                        }
-                        med_prev_T = next_T;
-                        med_prev_z = q2.y;
-                    }
-                    if (next_T > kTransmitThreshold) {
-                        const float w = alpha * T;
-                        float zd = q2.y;
-                        if constexpr (kDist != SSR_DIST_NONE) {
-                            zd = s_lz[k];
-                            if constexpr (kDist == SSR_DIST_RGB_D) {
-                                s2r = ssr_fma(q1.z * q1.z, w, s2r); s2g = ssr_fma(q1.w * q1.w, w, s2g);
-                                s2b = ssr_fma(q2.x * q2.x, w, s2b);
-                            }
-                            s2d = ssr_fma(zd * zd, w, s2d);
-                        }
-                        cr = ssr_fma(q1.z, w, cr); cg = ssr_fma(q1.w, w, cg); cb = ssr_fma(q2.x, w, cb);
-                        cd = ssr_fma(zd, w, cd);
-                        cur_idx = (uint32_t)(batch_start + k);
-                        T = next_T;
-                    } else {
-                        done = true;
-                    }
-                }
-            }
-        }
-    }
-    if (inside) {
-        const int64_t pid = ((int64_t)img * P.height + i) * P.width + j;
-        P.render_T[pid] = T;
-        const float invW = 1.0f / ssr_max(1.0f - T, 1e-10f);
-        float* o = P.render_rgb + 3 * pid;
-        o[0] = cr; o[1] = cg; o[2] = cb;
-        if constexpr (kMedian) P.render_median[pid] = median;
-        if constexpr (kDist != SSR_DIST_NONE) {   // D = W S - C^2 on the raw accumulators
-            const float W = 1.0f - T;
-            if constexpr (kDist == SSR_DIST_RGB_D) {
-                float* d = P.distortion_rgb + 3 * pid;
-                d[0] = s2r * W - cr * cr; d[1] = s2g * W - cg * cg; d[2] = s2b * W - cb * cb;
-            }
-            P.distortion_depth[pid] = s2d * W - cd * cd;
-            P.render_depth[pid] = ssr_exp(cd * invW);
-        } else {
-            P.render_depth[pid] = cd * invW;
-        }
-        P.last_ids[pid] = (int32_t)cur_idx;
-    }
-}
-
-// The row-granular plain kernel: the same per-pixel arithmetic, but each 16-lane row of a wavefront
-// holds one 4x4-pixel block and walks its own list of the staged fragments whose block bit is set
-// (raster_device.h), instead of all 64 lanes visiting every fragment that reaches the 8x8 sub-tile.
-// Lists are built per batch by the wavefront that walks them (ballot + rank, slot numbers as bytes).
+// One workgroup per 16x16 tile, a wavefront per 8x8 sub-tile; each 16-lane row of a wavefront holds one 4x4-pixel
+// block and walks its own list of the staged fragments whose block bit is set (raster_device.h), so that lanes do
+// not visit fragments that only reach other parts of the sub-tile. Lists are built per batch by the wavefront that
+// walks them (ballot + rank, slot numbers as bytes). kDist (SSR_DIST_*) and kMedian select the variants
+// (RasterizationEval3DFwd_kernel.cuh:143-148,245-307): per-lane accumulators only.
 template <int kDist, bool kMedian>
 __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raster_fwd_params P, int tile_w, int tile_h) {
     __shared__ FragLds frags[kBatch];
@@ -303,28 +196,14 @@ extern "C" int ssr_raster_fwd(const ssr_raster_fwd_params* p, ssr_stream_t strea
     SSR_REQUIRE((int64_t)tw * th * nimg < (int64_t)1 << 30, "ssr_raster_fwd", "too many tiles");
     const dim3 grid((unsigned)xcd_grid_size(tw * th * nimg)), block(kRasterBlock);
     hipStream_t s = as_stream(stream);
-#define SSR_FWD(D, M) hipLaunchKernelGGL((raster_fwd_kernel<D, M>), grid, block, 0, s, *p, tw, th)
     const bool med = p->render_median != nullptr;
-    // Every variant runs the row-granular kernel; SSR_RASTER_WAVE_VISITS=1 in the environment selects the
-    // one-wavefront-per-visit kernel instead (for comparisons).
-    static const bool wave_visits = getenv("SSR_RASTER_WAVE_VISITS") != nullptr;
-    if (!wave_visits) {
 #define SSR_FWD_ROWS(D, M) hipLaunchKernelGGL((raster_fwd_rows_kernel<D, M>), grid, block, 0, s, *p, tw, th)
-        switch (p->dist_type) {
-            case SSR_DIST_D: if (med) SSR_FWD_ROWS(SSR_DIST_D, true); else SSR_FWD_ROWS(SSR_DIST_D, false); break;
-            case SSR_DIST_RGB_D: if (med) SSR_FWD_ROWS(SSR_DIST_RGB_D, true); else SSR_FWD_ROWS(SSR_DIST_RGB_D, false); break;
-            default: if (med) SSR_FWD_ROWS(SSR_DIST_NONE, true); else SSR_FWD_ROWS(SSR_DIST_NONE, false); break;
-        }
-#undef SSR_FWD_ROWS
-        SSR_CHECK_LAUNCH("ssr_raster_fwd");
-        return 0;
-    }
     switch (p->dist_type) {
-        case SSR_DIST_D: if (med) SSR_FWD(SSR_DIST_D, true); else SSR_FWD(SSR_DIST_D, false); break;
-        case SSR_DIST_RGB_D: if (med) SSR_FWD(SSR_DIST_RGB_D, true); else SSR_FWD(SSR_DIST_RGB_D, false); break;
-        default: if (med) SSR_FWD(SSR_DIST_NONE, true); else SSR_FWD(SSR_DIST_NONE, false); break;
+        case SSR_DIST_D: if (med) SSR_FWD_ROWS(SSR_DIST_D, true); else SSR_FWD_ROWS(SSR_DIST_D, false); break;
+        case SSR_DIST_RGB_D: if (med) SSR_FWD_ROWS(SSR_DIST_RGB_D, true); else SSR_FWD_ROWS(SSR_DIST_RGB_D, false); break;
+        default: if (med) SSR_FWD_ROWS(SSR_DIST_NONE, true); else SSR_FWD_ROWS(SSR_DIST_NONE, false); break;
     }
-#undef SSR_FWD
+#undef SSR_FWD_ROWS
     SSR_CHECK_LAUNCH("ssr_raster_fwd");
     return 0;
 }
