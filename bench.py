@@ -144,6 +144,9 @@ def main():
     ap.add_argument("--dist-type", type=int, default=0, help="compositing variant: 1 depth distortion, 2 rgb + depth distortion")
     ap.add_argument("--median", action="store_true", help="compositing variant: also render the median depth and back-propagate it")
     ap.add_argument("--accum-mode", type=int, default=0, help="compositing variant: accumulate a pixel weight map per splat (1 max, 2 sum, 3 avg)")
+    ap.add_argument("--deferred-counts", action="store_true",
+                    help="after the first iteration the forward does not wait for the intersection count: key arrays sized "
+                         "from the previous count, overflow checked before the backward uses the counts")
     ap.add_argument("--cameras", type=int, default=1,
                     help="render C cameras per iteration in one call ([C,N] layout, plain path only); an iteration is then C images")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -209,7 +212,7 @@ def main():
     native = not args.reference_order
     eng = host.Engine(sc, fuse_tile_count=native, visible_list=native and not args.packed_projection, packed_rows=native,
                       overwrite_world_grads=native, packed_projection=args.packed_projection, packed_vscreen=native,
-                      tile_sort=native and not args.whole_key_sort)
+                      tile_sort=native and not args.whole_key_sort, deferred_counts=args.deferred_counts)
     L = lib.load()
 
     hyper = dict(lr_means=1.6e-6, lr_quats=1e-5, lr_scales=5e-5, lr_opacs=5e-4, lr_features_dc=2.5e-5, lr_features_sh=1.25e-6)

@@ -223,6 +223,30 @@ int ssr_tile_write_images(int64_t n, int64_t rows_per_image, const int32_t* imag
                           const float* opac, const int64_t* cum_tiles, uint32_t width, uint32_t height,
                           int64_t* isect_ids, int32_t* flatten_ids, const int32_t* tile_active,
                           ssr_stream_t stream);
+/* The key write for a caller that does not read the counts back (the reference blocks on n_isects,
+ * IntersectTile.cu:432-436; no counterpart there). isect_ids / flatten_ids hold `capacity` entries, sized from an
+ * earlier iteration; the real number of keys stays on the device (the scan's total), and so does the work list's
+ * length *n_visible when visible_ids is given. Keys are those of ssr_tile_write / ssr_tile_write_images; none is
+ * written at or beyond `capacity`, so a count above the capacity loses keys but touches no memory outside the
+ * arrays: the caller compares the count with its capacity once it has read it (asynchronously) and repeats the
+ * iteration with larger arrays if it did not fit. Entries from the real count up to `capacity` are not written;
+ * ssr_sort_tile_pairs_capped and the compositing launches (tile_offsets_closed) never read them. */
+typedef struct {
+    int64_t n;                      /* rows: splats, or num_images * rows_per_image, or packed rows */
+    int64_t rows_per_image;         /* with num_images > 1 and no image_ids */
+    const int32_t* image_ids;       /* optional, [n]: packed rows of several images */
+    int32_t num_images;
+    const float* aabb; const float* sort_depth; const float* xy; const float* conic; const float* opac;
+    const int64_t* cum_tiles;       /* [n] inclusive scan of the counts */
+    uint32_t width, height;
+    int64_t* isect_ids;             /* [capacity] */
+    int32_t* flatten_ids;           /* [capacity] */
+    int64_t capacity;
+    const int32_t* visible_ids;     /* optional work list (one image) ... */
+    const int64_t* n_visible;       /* ... and its length, on the device (the launch covers n rows) */
+    const int32_t* tile_active;
+} ssr_tile_write_capped_params;
+int ssr_tile_write_capped(const ssr_tile_write_capped_params* p, ssr_stream_t stream);
 /* sort_pairs<int64,int32> with CUB DoubleBuffer semantics (src/backend/common/SortScan.h:42-56;
  * call site IntersectTile.cu:486-493): stable on bits [begin_bit,end_bit); *selector says which
  * of the (a,b) buffers holds the result. */
@@ -239,6 +263,8 @@ int ssr_tile_offsets(int64_t n_isects, const int64_t* sorted_ids, uint32_t n_til
  * so the longest tiles start first and every XCD gets the same mix. scratch: ssr_tile_order_scratch_bytes.
  * No counterpart in the reference (its grid is one block per tile in index order). */
 size_t ssr_tile_order_scratch_bytes(uint32_t n_tiles);
+/* n_isects < 0: tile_offsets holds n_tiles + 1 entries, the last one ending the last tile
+ * (ssr_sort_tile_pairs_capped). */
 int ssr_tile_order(const int32_t* tile_offsets, uint32_t n_tiles, int64_t n_isects, int32_t* order, void* scratch,
                    size_t scratch_bytes, ssr_stream_t stream);
 /* Number of key bits the sort must cover: 32 + tile_n_bits (IntersectTile.cu:489-490). */
@@ -253,6 +279,19 @@ size_t ssr_sort_tile_scratch_bytes(int64_t n, uint32_t n_tiles);
 int ssr_sort_tile_pairs(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, int32_t* vals_b,
                         int64_t n, uint32_t n_tiles, int32_t* tile_offsets, int* selector,
                         void* scratch, size_t scratch_bytes, ssr_stream_t stream);
+/* The same over arrays of `capacity` entries of which the first *n_isects (device; clamped to capacity) are
+ * keys, as ssr_tile_write_capped leaves them. tile_offsets holds n_tiles + 1 entries; tile_offsets[n_tiles]
+ * receives that number, the end of the last tile. The first tile_offsets[n_tiles] entries of the result and
+ * tile_offsets[0..n_tiles) are those of ssr_sort_tile_pairs on the keys; the entries behind them are unspecified.
+ * Launches are sized for `capacity`; workgroups behind the count leave at once.
+ * Scratch: ssr_sort_tile_scratch_bytes(capacity, n_tiles). No counterpart in the reference. */
+int ssr_sort_tile_pairs_capped(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, int32_t* vals_b,
+                               int64_t capacity, const int64_t* n_isects, uint32_t n_tiles, int32_t* tile_offsets,
+                               int* selector, void* scratch, size_t scratch_bytes, ssr_stream_t stream);
+/* ssr_tile_offsets over the first *n_isects (device) of `capacity` sorted keys, with the one entry more:
+ * offsets[n_tiles] = min(*n_isects, capacity). */
+int ssr_tile_offsets_capped(int64_t capacity, const int64_t* n_isects, const int64_t* sorted_ids, uint32_t n_tiles,
+                            int32_t* offsets, ssr_stream_t stream);
 
 /* ---- K7: rasterize_to_pixels_3dgs_fwd (src/kernels/raster/RasterizationFwd.cuh:18-38, kernel
  * src/kernels/raster/RasterizationEval3DFwd_kernel.cuh:48-313, IS_EVAL3D=0). */
@@ -284,6 +323,7 @@ typedef struct {
      * (RasterizationFwd.cu grid = {C, tile_h, tile_w}). */
     int32_t num_images;
     const int32_t* tile_order;  /* optional: ssr_tile_order's output for these tile_offsets; NULL = tiles in index order, one contiguous band per XCD */
+    int32_t tile_offsets_closed; /* nonzero: tile_offsets holds one more entry, the end of the last tile (ssr_sort_tile_pairs_capped); n_isects is then only the capacity of flatten_ids */
 } ssr_raster_fwd_params;
 int ssr_raster_fwd(const ssr_raster_fwd_params* p, ssr_stream_t stream);
 
@@ -335,6 +375,7 @@ typedef struct {
     int32_t num_images;               /* as in ssr_raster_fwd_params; with accum_mode, screen row r
                                        * adds into world row r % num_world */
     const int32_t* tile_order;        /* optional, as in ssr_raster_fwd_params */
+    int32_t tile_offsets_closed;      /* as in ssr_raster_fwd_params */
 } ssr_raster_bwd_params;
 int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t stream);
 

@@ -1207,7 +1207,7 @@ __global__ __launch_bounds__(kProjBlock) void fused_projection_bwd_optimizer_ker
         return;
     }
     for (int e = threadIdx.x; e < n_here * kPer; e += kProjBlock) {
-        const int sp = e / kPer, i = e - sp * kPer;
+        const int sp = e / (kPer > 0 ? kPer : 1), i = e - sp * kPer;   // degree 0: no trip
         const int j = i / 3, c = i - 3 * j;
         const int64_t row = block0 + sp;
         float* xp = W.features_sh + row * W.sh_stride + i;

@@ -305,6 +305,8 @@ __device__ __forceinline__ void decode_sh(const ssr_world& w, const ssr_sh_quant
             return;
         }
         // otherwise bounds change at most once every `stride` cells: track the current block incrementally
+        // (cells advance by one and `stride` is at least one, so a cell that reaches `next` is exactly `next`
+        // and its block is the following one: one division for the splat, none per cell)
         int64_t blk = base / stride;
         int64_t next = (blk + 1) * stride;
         float lo = q.bounds[2 * blk], hi = q.bounds[2 * blk + 1];
@@ -312,7 +314,7 @@ __device__ __forceinline__ void decode_sh(const ssr_world& w, const ssr_sh_quant
         for (int i = 0; i < n; i++) {
             const int64_t cell = base + i;
             if (cell >= next) {
-                blk = cell / stride; next = (blk + 1) * stride;
+                blk += 1; next += stride;
                 lo = q.bounds[2 * blk]; hi = q.bounds[2 * blk + 1];
             }
             const float v = q16 ? (float)reinterpret_cast<const uint16_t*>(q.packed)[cell]

@@ -145,7 +145,7 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
     if constexpr (kAccum != SSR_ACCUM_NONE) amap = inside ? P.accum_weight_map[pid] : 0.0f;
 
     const int32_t range_start = P.tile_offsets[tile];
-    const int32_t range_end = (tile == n_tiles - 1) ? (int32_t)P.n_isects : P.tile_offsets[tile + 1];
+    const int32_t range_end = (tile == n_tiles - 1 && !P.tile_offsets_closed) ? (int32_t)P.n_isects : P.tile_offsets[tile + 1];
     // largest last_id per block (row), per wavefront, per tile
     int row_last = bin_final;
 #pragma unroll

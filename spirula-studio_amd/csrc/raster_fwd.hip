@@ -34,7 +34,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raste
     int alive = inside ? 1 : 0;   // 0 once the pixel has stopped compositing (an int: the loop tests it with one compare)
 
     const int32_t range_start = P.tile_offsets[tile];
-    const int32_t range_end = (tile == n_tiles - 1) ? (int32_t)P.n_isects : P.tile_offsets[tile + 1];
+    const int32_t range_end = (tile == n_tiles - 1 && !P.tile_offsets_closed) ? (int32_t)P.n_isects : P.tile_offsets[tile + 1];
     float T = 1.0f, cr = 0.f, cg = 0.f, cb = 0.f, cd = 0.f;
     [[maybe_unused]] float s2r = 0.f, s2g = 0.f, s2b = 0.f, s2d = 0.f;           // second moments (distortion)
     [[maybe_unused]] float median = 0.f, med_prev_z = 0.f, med_prev_T = 1.0f;   // median depth

@@ -46,11 +46,16 @@ __device__ __forceinline__ void wave_match_digit(uint32_t d, uint32_t varying, b
 }
 
 // hist[d * n_blocks + block]
-__global__ __launch_bounds__(kSortBlock) void sort_hist_kernel(const uint64_t* __restrict__ keys, int64_t n, int shift,
+// n_dev (optional): the real number of keys, on the device, where the host only knows an upper bound n; workgroups
+// behind it leave at once.
+__global__ __launch_bounds__(kSortBlock) void sort_hist_kernel(const uint64_t* __restrict__ keys, int64_t n,
+                                                               const int64_t* __restrict__ n_dev, int shift,
                                                                uint32_t mask, uint32_t n_blocks,
                                                                uint32_t* __restrict__ hist, uint32_t* clear4) {
     __shared__ uint32_t lh[kRadix];
+    if (n_dev) n = min(n, *n_dev);
     if (clear4 && blockIdx.x == 0 && threadIdx.x < 4) clear4[threadIdx.x] = 0;   // counters of a later kernel on this stream
+    if ((int64_t)blockIdx.x * kSortTile >= n) return;   // behind the keys: its column is never read (sort_scan_rows_kernel)
     lh[threadIdx.x] = 0;
     __syncthreads();
     const int64_t base = (int64_t)blockIdx.x * kSortTile;
@@ -64,12 +69,17 @@ __global__ __launch_bounds__(kSortBlock) void sort_hist_kernel(const uint64_t* _
 }
 
 // One workgroup per digit: exclusive scan of its row of per-workgroup counts; row total out.
+// (rows of n_blocks columns; only the columns of workgroups that hold keys were written: the first n_used)
 __global__ __launch_bounds__(kSortBlock) void sort_scan_rows_kernel(uint32_t* __restrict__ hist, uint32_t n_blocks,
-                                                                    uint32_t* __restrict__ totals) {
+                                                                    uint32_t* __restrict__ totals, int64_t n,
+                                                                    const int64_t* __restrict__ n_dev) {
     __shared__ uint32_t ws[kSortWaves];
     uint32_t* row = hist + (size_t)blockIdx.x * n_blocks;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     uint32_t carry = 0;
+    if (n_dev) n = min(n, *n_dev);
+    const uint32_t n_used = (uint32_t)((n + kSortTile - 1) / kSortTile);
+    n_blocks = min(n_blocks, n_used);
     for (uint32_t start = 0; start < n_blocks; start += kSortBlock) {
         const uint32_t i = start + threadIdx.x;
         const uint32_t v = i < n_blocks ? row[i] : 0;
@@ -93,8 +103,10 @@ __global__ __launch_bounds__(kSortBlock) void sort_scan_rows_kernel(uint32_t* __
 
 __global__ __launch_bounds__(kSortBlock) void sort_scatter_kernel(
     const uint64_t* __restrict__ keys_in, const int32_t* __restrict__ vals_in, uint64_t* __restrict__ keys_out,
-    int32_t* __restrict__ vals_out, int64_t n, int shift, uint32_t mask, uint32_t n_blocks,
+    int32_t* __restrict__ vals_out, int64_t n, const int64_t* __restrict__ n_dev, int shift, uint32_t mask, uint32_t n_blocks,
     const uint32_t* __restrict__ hist, const uint32_t* __restrict__ totals) {
+    if (n_dev) n = min(n, *n_dev);
+    if ((int64_t)blockIdx.x * kSortTile >= n) return;   // nothing of this workgroup's is real (the whole workgroup leaves)
     __shared__ uint32_t wcount[kSortWaves][kRadix];   // per-wave running digit counts, then bases
     __shared__ uint32_t ws[kSortWaves], ws2[kSortWaves];
     __shared__ uint32_t s_shift[kRadix];
@@ -357,6 +369,12 @@ struct SegLists { uint32_t* counts; uint32_t* list[3]; bool has_class0; };
 constexpr int kSegCap0 = 4 * 64 * 8;           // four wavefronts, 8 keys per lane
 constexpr int kSegCap1 = 16 * 64 * 8;          // sixteen wavefronts, 8 keys per lane
 
+// End of tile `tile`'s segment. n < 0: the offsets hold one entry more, which ends the last tile (the host does
+// not know the number of keys).
+__device__ __forceinline__ int64_t seg_end(const int32_t* __restrict__ tile_offsets, uint32_t tile, uint32_t n_tiles, int64_t n) {
+    return (tile + 1 < n_tiles || n < 0) ? (int64_t)tile_offsets[tile + 1] : n;
+}
+
 // One workgroup of kWaves wavefronts per tile: sorts segments of 2..64*kWaves*kRounds keys, lists the
 // longer ones. These kernels are bound by instruction issue: one wavefront per tile executes the fewest
 // instructions per key, but its tiles take long, so it pays only when there are several rounds of
@@ -373,7 +391,7 @@ __global__ __launch_bounds__(kWaves * 64) void sort_segments_direct_kernel(uint6
     __shared__ uint2 buf[kCap];
     const uint32_t tile = blockIdx.x;
     const int64_t s = tile_offsets[tile];
-    const int64_t e = tile + 1 < n_tiles ? (int64_t)tile_offsets[tile + 1] : n;
+    const int64_t e = seg_end(tile_offsets, tile, n_tiles, n);
     const int len = (int)(e - s);
     if (len <= 1) return;
     if (len > kCap) {
@@ -400,7 +418,7 @@ __global__ __launch_bounds__(256) void sort_segments_small_kernel(uint64_t* keys
     for (uint32_t idx = blockIdx.x; idx < count; idx += gridDim.x) {
         const uint32_t tile = lists.list[0][idx];
         const int64_t s = tile_offsets[tile];
-        const int64_t e = tile + 1 < n_tiles ? (int64_t)tile_offsets[tile + 1] : n;
+        const int64_t e = seg_end(tile_offsets, tile, n_tiles, n);
         seg_sort_lds<4, 8>(keys, vals, s, (int)(e - s), wcount, ws, wor, buf);
         __syncthreads();   // LDS is reused by the next segment
     }
@@ -478,7 +496,7 @@ __global__ __launch_bounds__(kSegGlobalWaves * 64) void sort_segments_long_kerne
         if (idx >= count1 + count2) break;   // the same value in every thread: the workgroup leaves together
         const uint32_t tile = idx < count2 ? lists.list[2][idx] : lists.list[1][idx - count2];
         const int64_t s = tile_offsets[tile];
-        const int64_t e = tile + 1 < n_tiles ? (int64_t)tile_offsets[tile + 1] : n;
+        const int64_t e = seg_end(tile_offsets, tile, n_tiles, n);
         if (idx < count2) seg_sort_global(keys, vals, keys_alt, vals_alt, s, (int)(e - s), wcount, ws);
         else seg_sort_lds<kSegGlobalWaves, 8>(keys, vals, s, (int)(e - s), wcount, ws, wor, buf);
         __syncthreads();   // LDS, s_next included, is reused by the next segment
@@ -505,7 +523,7 @@ size_t ssr_sort_tile_scratch_bytes(int64_t n, uint32_t n_tiles) {
 // clear4 (optional): four counters that the first kernel launched here sets to zero
 static int sort_pairs_impl(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, int32_t* vals_b, int64_t n, int begin_bit,
                            int end_bit, int* selector, void* scratch, size_t scratch_bytes, ssr_stream_t stream,
-                           uint32_t* clear4) {
+                           uint32_t* clear4, const int64_t* n_dev = nullptr) {
     SSR_REQUIRE(selector, "ssr_sort_pairs_u64_i32", "null selector");
     *selector = 0;
     SSR_REQUIRE(n >= 0 && n < (int64_t)1 << 31, "ssr_sort_pairs_u64_i32", "count out of range");
@@ -523,11 +541,11 @@ static int sort_pairs_impl(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, in
     for (int shift = begin_bit; shift < end_bit; shift += 8) {
         const int bits = end_bit - shift < 8 ? end_bit - shift : 8;
         const uint32_t mask = (1u << bits) - 1u;
-        hipLaunchKernelGGL(sort_hist_kernel, dim3(nb), dim3(kSortBlock), 0, s, k[cur], n, shift, mask, nb, hist,
+        hipLaunchKernelGGL(sort_hist_kernel, dim3(nb), dim3(kSortBlock), 0, s, k[cur], n, n_dev, shift, mask, nb, hist,
                            shift == begin_bit ? clear4 : nullptr);
-        hipLaunchKernelGGL(sort_scan_rows_kernel, dim3(kRadix), dim3(kSortBlock), 0, s, hist, nb, totals);
+        hipLaunchKernelGGL(sort_scan_rows_kernel, dim3(kRadix), dim3(kSortBlock), 0, s, hist, nb, totals, n, n_dev);
         hipLaunchKernelGGL(sort_scatter_kernel, dim3(nb), dim3(kSortBlock), 0, s, k[cur], v[cur], k[cur ^ 1], v[cur ^ 1], n,
-                           shift, mask, nb, hist, totals);
+                           n_dev, shift, mask, nb, hist, totals);
         cur ^= 1;
     }
     SSR_CHECK_LAUNCH("ssr_sort_pairs_u64_i32");
@@ -542,9 +560,11 @@ int ssr_sort_pairs_u64_i32(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, in
                            nullptr);
 }
 
-int ssr_sort_tile_pairs(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, int32_t* vals_b, int64_t n,
-                        uint32_t n_tiles, int32_t* tile_offsets, int* selector, void* scratch, size_t scratch_bytes,
-                        ssr_stream_t stream) {
+// n_dev: only the first *n_dev (device) of the n entries are keys; tile_offsets then has n_tiles + 1 entries
+static int sort_tile_pairs_impl(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, int32_t* vals_b, int64_t n,
+                                uint32_t n_tiles, int32_t* tile_offsets, int* selector, void* scratch, size_t scratch_bytes,
+                                ssr_stream_t stream, const int64_t* n_dev) {
+    const bool closed = n_dev != nullptr;
     SSR_REQUIRE(selector, "ssr_sort_tile_pairs", "null selector");
     *selector = 0;
     SSR_REQUIRE(n >= 0 && n < (int64_t)1 << 31, "ssr_sort_tile_pairs", "count out of range");
@@ -559,7 +579,8 @@ int ssr_sort_tile_pairs(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, int32
     }
     const int end_bit = ssr_sort_end_bit(n_tiles);
     if (n > 0 && end_bit > 32) {   // partition by tile: stable on the tile bits only
-        if (sort_pairs_impl(keys_a, keys_b, vals_a, vals_b, n, 32, end_bit, selector, scratch, scratch_bytes, stream, lists.counts))
+        if (sort_pairs_impl(keys_a, keys_b, vals_a, vals_b, n, 32, end_bit, selector, scratch, scratch_bytes, stream, lists.counts,
+                            n_dev))
             return 1;
     } else if (n > 0) {
         SSR_REQUIRE(keys_a && keys_b && vals_a && vals_b, "ssr_sort_tile_pairs", "null buffer");
@@ -568,14 +589,18 @@ int ssr_sort_tile_pairs(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, int32
     const int cur = *selector;
     int64_t* k[2] = {keys_a, keys_b};
     int32_t* v[2] = {vals_a, vals_b};
-    if (ssr_tile_offsets(n, k[cur], n_tiles, tile_offsets, stream)) return 1;
+    if (closed ? ssr_tile_offsets_capped(n, n_dev, k[cur], n_tiles, tile_offsets, stream)
+               : ssr_tile_offsets(n, k[cur], n_tiles, tile_offsets, stream))
+        return 1;
     if (n <= 1) return 0;
+    const int64_t n_host = n;   // sizes the launches
+    if (closed) n = -1;         // the kernels end the last tile at tile_offsets[n_tiles]
     hipStream_t s = as_stream(stream);
     uint64_t* kc = reinterpret_cast<uint64_t*>(k[cur]);
     uint64_t* ka = reinterpret_cast<uint64_t*>(k[cur ^ 1]);
     // one wavefront per tile: at least two rounds of such workgroups on 256 compute units, and segments that mostly fit
     // its 512 keys (a mean of 336 does, config 5; a mean of 411 with a third of the tiles above 512 does not)
-    const bool lone_waves = n_tiles >= 16384 && n / n_tiles <= 384;
+    const bool lone_waves = n_tiles >= 16384 && n_host / n_tiles <= 384;
     lists.has_class0 = lone_waves;
     if (lone_waves) {
         hipLaunchKernelGGL((sort_segments_direct_kernel<1, 8>), dim3(n_tiles), dim3(64), 0, s, kc, v[cur], tile_offsets, n_tiles,
@@ -583,7 +608,7 @@ int ssr_sort_tile_pairs(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, int32
     } else {
         // 8 keys per lane sort segments of up to 2048 keys directly, at the price of a slower kernel for short
         // segments: worth it where the mean segment is long
-        if (n / n_tiles > 512)
+        if (n_host / n_tiles > 512)
             hipLaunchKernelGGL((sort_segments_direct_kernel<4, 8>), dim3(n_tiles), dim3(256), 0, s, kc, v[cur], tile_offsets,
                                n_tiles, n, lists);
         else
@@ -591,14 +616,31 @@ int ssr_sort_tile_pairs(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, int32
                                n_tiles, n, lists);
     }
     // the listed segments: fixed grids, a workgroup with no list entry ends at once
-    if (lone_waves && n > 512)   // four wavefronts sort class 0 directly otherwise
+    if (lone_waves && n_host > 512)   // four wavefronts sort class 0 directly otherwise
         hipLaunchKernelGGL(sort_segments_small_kernel, dim3(n_tiles < 2048 ? n_tiles : 2048), dim3(256), 0, s, kc, v[cur],
                            tile_offsets, n_tiles, n, lists);
-    if (n > (lone_waves ? kSegCap0 : 1024))
+    if (n_host > (lone_waves ? kSegCap0 : 1024))
         hipLaunchKernelGGL(sort_segments_long_kernel, dim3(n_tiles < 512 ? n_tiles : 512), dim3(kSegGlobalWaves * 64), 0, s, kc,
                            v[cur], ka, v[cur ^ 1], tile_offsets, n_tiles, n, lists);
     SSR_CHECK_LAUNCH("ssr_sort_tile_pairs");
     return 0;
+}
+
+int ssr_sort_tile_pairs(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, int32_t* vals_b, int64_t n,
+                        uint32_t n_tiles, int32_t* tile_offsets, int* selector, void* scratch, size_t scratch_bytes,
+                        ssr_stream_t stream) {
+    return sort_tile_pairs_impl(keys_a, keys_b, vals_a, vals_b, n, n_tiles, tile_offsets, selector, scratch, scratch_bytes,
+                                stream, nullptr);
+}
+
+int ssr_sort_tile_pairs_capped(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, int32_t* vals_b, int64_t capacity,
+                               const int64_t* n_isects, uint32_t n_tiles, int32_t* tile_offsets, int* selector, void* scratch,
+                               size_t scratch_bytes, ssr_stream_t stream) {
+    SSR_REQUIRE(n_tiles > 0 && n_tiles < 0x7fffffffu, "ssr_sort_tile_pairs_capped", "tile count out of range");
+    SSR_REQUIRE(capacity > 0, "ssr_sort_tile_pairs_capped", "capacity must be positive");
+    SSR_REQUIRE(n_isects, "ssr_sort_tile_pairs_capped", "null count");
+    return sort_tile_pairs_impl(keys_a, keys_b, vals_a, vals_b, capacity, n_tiles, tile_offsets, selector, scratch, scratch_bytes,
+                                stream, n_isects);
 }
 
 }  // extern "C"

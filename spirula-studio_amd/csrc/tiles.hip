@@ -75,15 +75,26 @@ __device__ __forceinline__ int wave_inclusive_scan_i32(int v, int lane) {
     return v;
 }
 
-__global__ __launch_bounds__(kTileBlock) void tile_write_kernel(
-    int64_t n, const float4* __restrict__ aabb, const float* __restrict__ sort_depth,
-    const float2* __restrict__ xy, const float* __restrict__ conic, const float* __restrict__ opac,
-    const int64_t* __restrict__ cum, int tile_w, int tile_h, int64_t* __restrict__ isect_ids,
-    int32_t* __restrict__ flatten_ids, const int32_t* __restrict__ visible_ids, const int32_t* __restrict__ live_all,
-    uint32_t rows_per_image, const int32_t* __restrict__ image_ids) {
-    const int64_t i = (int64_t)blockIdx.x * kTileBlock + threadIdx.x;
+struct TileWriteArgs {
+    const float4* __restrict__ aabb; const float* __restrict__ sort_depth; const float2* __restrict__ xy;
+    const float* __restrict__ conic; const float* __restrict__ opac; const int64_t* __restrict__ cum;
+    int tile_w, tile_h;
+    int64_t* __restrict__ isect_ids; int32_t* __restrict__ flatten_ids;
+    const int32_t* __restrict__ visible_ids; const int32_t* __restrict__ live_all;
+    uint32_t rows_per_image; const int32_t* __restrict__ image_ids;
+};
+
+// Keys of work item i (row i, or the row visible_ids[i]); the whole wavefront calls this together. kCapped: no
+// key is written at or beyond position `capacity`.
+template <bool kCapped>
+__device__ __forceinline__ void tile_write_row(const TileWriteArgs& A, int64_t i, bool in_range, int64_t capacity) {
+    const float4* __restrict__ aabb = A.aabb; const float* __restrict__ sort_depth = A.sort_depth;
+    const float2* __restrict__ xy = A.xy; const float* __restrict__ conic = A.conic; const float* __restrict__ opac = A.opac;
+    const int64_t* __restrict__ cum = A.cum; const int tile_w = A.tile_w, tile_h = A.tile_h;
+    int64_t* __restrict__ isect_ids = A.isect_ids; int32_t* __restrict__ flatten_ids = A.flatten_ids;
+    const int32_t* __restrict__ visible_ids = A.visible_ids; const int32_t* __restrict__ live_all = A.live_all;
+    const uint32_t rows_per_image = A.rows_per_image; const int32_t* __restrict__ image_ids = A.image_ids;
     const int lane = threadIdx.x & 63;
-    const bool in_range = i < n;
     const int64_t g = in_range ? (visible_ids ? (int64_t)visible_ids[i] : i) : 0;
     int64_t cur = 0, end = 0;
     TileGeomD tg;
@@ -97,6 +108,7 @@ __global__ __launch_bounds__(kTileBlock) void tile_write_kernel(
     if (in_range) {
         cur = g == 0 ? 0 : cum[g - 1];
         end = cum[g];
+        if (kCapped) { cur = min(cur, capacity); end = min(end, capacity); }
         const float4 a = aabb[g];
         visible = !(a.z <= a.x || a.w <= a.y);
         if (visible) {
@@ -167,6 +179,22 @@ __global__ __launch_bounds__(kTileBlock) void tile_write_kernel(
             flatten_ids[pos] = sgid;
         }
     }
+}
+
+__global__ __launch_bounds__(kTileBlock) void tile_write_kernel(int64_t n, TileWriteArgs A) {
+    const int64_t i = (int64_t)blockIdx.x * kTileBlock + threadIdx.x;
+    tile_write_row<false>(A, i, i < n, 0);
+}
+
+// The key write when the host does not know the counts: the arrays hold `capacity` entries, and the work list's
+// length, when there is a list, is *n_visible (device): the launch covers all n rows and the threads behind the
+// list's end leave at once. No key is written at or beyond `capacity`.
+__global__ __launch_bounds__(kTileBlock) void tile_write_capped_kernel(int64_t n, TileWriteArgs A, int64_t capacity,
+                                                                       const int64_t* __restrict__ n_visible) {
+    const int64_t i = (int64_t)blockIdx.x * kTileBlock + threadIdx.x;
+    const int64_t work = (A.visible_ids && n_visible) ? min(*n_visible, n) : n;
+    if ((int64_t)blockIdx.x * kTileBlock >= work) return;
+    tile_write_row<true>(A, i, i < work, capacity);
 }
 
 // ---- int64 inclusive scan: per-block reduce, single-block scan of the block sums, downsweep ----
@@ -282,9 +310,16 @@ int warm_static_scan() {
 
 // ---- K6 ----
 
-__global__ __launch_bounds__(kTileBlock) void tile_offsets_kernel(int64_t n_isects, const int64_t* __restrict__ ids,
-                                                                  int64_t n_tiles, int32_t* __restrict__ offsets) {
+// n_dev (optional): the real number of keys, on the device, where the host only knows an upper bound n_isects.
+__global__ __launch_bounds__(kTileBlock) void tile_offsets_kernel(int64_t n_isects, const int64_t* __restrict__ n_dev,
+                                                                  const int64_t* __restrict__ ids, int64_t n_tiles,
+                                                                  int32_t* __restrict__ offsets) {
     const int64_t idx = (int64_t)blockIdx.x * kTileBlock + threadIdx.x;
+    if (n_dev) {
+        n_isects = min(n_isects, *n_dev);
+        if (n_isects == 0 && idx == 0)   // no key: nobody below writes anything
+            for (int64_t i = 0; i < n_tiles; ++i) offsets[i] = 0;
+    }
     if (idx >= n_isects) return;
     const int64_t tile = ids[idx] >> 32;
     if (idx == 0)
@@ -307,7 +342,7 @@ __global__ __launch_bounds__(kTileBlock) void tile_offsets_kernel(int64_t n_isec
 // positions and scatters. The order inside a class does not matter.
 constexpr int kOrderBlock = 1024;
 __device__ __forceinline__ uint32_t tile_class(const int32_t* __restrict__ offsets, uint32_t t, uint32_t n_tiles, int64_t n_isects) {
-    const int64_t e = t + 1 < n_tiles ? (int64_t)offsets[t + 1] : n_isects;
+    const int64_t e = (t + 1 < n_tiles || n_isects < 0) ? (int64_t)offsets[t + 1] : n_isects;   // < 0: one entry more
     const int64_t len = e - offsets[t];
     return 255u - (uint32_t)min((int64_t)255, len >> 5);   // class 0 holds the longest tiles
 }
@@ -470,9 +505,10 @@ int ssr_tile_write(int64_t n, const float* aabb, const float* sort_depth, const 
                 "ssr_tile_write", "aabb must be 16-byte and xy 8-byte aligned");
     const int tw = (int)ceil_div(width, kTile), th = (int)ceil_div(height, kTile);
     const int64_t work = visible_ids ? n_visible : n;
+    const TileWriteArgs A = {reinterpret_cast<const float4*>(aabb), sort_depth, reinterpret_cast<const float2*>(xy), conic, opac,
+                             cum_tiles, tw, th, isect_ids, flatten_ids, visible_ids, tile_active, 0u, nullptr};
     hipLaunchKernelGGL(tile_write_kernel, dim3((unsigned)ceil_div(work, kTileBlock)), dim3(kTileBlock), 0, as_stream(stream),
-                       work, reinterpret_cast<const float4*>(aabb), sort_depth, reinterpret_cast<const float2*>(xy), conic, opac,
-                       cum_tiles, tw, th, isect_ids, flatten_ids, visible_ids, tile_active, 0u, (const int32_t*)nullptr);
+                       work, A);
     SSR_CHECK_LAUNCH("ssr_tile_write");
     return 0;
 }
@@ -494,11 +530,40 @@ int ssr_tile_write_images(int64_t n, int64_t rows_per_image, const int32_t* imag
     const int tw = (int)ceil_div(width, kTile), th = (int)ceil_div(height, kTile);
     SSR_REQUIRE((int64_t)num_images * tw * th < (int64_t)1 << 31, "ssr_tile_write_images",
                 "tile ids of all images must fit 31 bits");
-    hipLaunchKernelGGL(tile_write_kernel, dim3((unsigned)ceil_div(n, kTileBlock)), dim3(kTileBlock), 0, as_stream(stream),
-                       n, reinterpret_cast<const float4*>(aabb), sort_depth, reinterpret_cast<const float2*>(xy), conic, opac,
-                       cum_tiles, tw, th, isect_ids, flatten_ids, (const int32_t*)nullptr, tile_active,
-                       image_ids ? 0u : (uint32_t)rows_per_image, image_ids);
+    const TileWriteArgs A = {reinterpret_cast<const float4*>(aabb), sort_depth, reinterpret_cast<const float2*>(xy), conic, opac,
+                             cum_tiles, tw, th, isect_ids, flatten_ids, nullptr, tile_active,
+                             image_ids ? 0u : (uint32_t)rows_per_image, image_ids};
+    hipLaunchKernelGGL(tile_write_kernel, dim3((unsigned)ceil_div(n, kTileBlock)), dim3(kTileBlock), 0, as_stream(stream), n, A);
     SSR_CHECK_LAUNCH("ssr_tile_write_images");
+    return 0;
+}
+
+int ssr_tile_write_capped(const ssr_tile_write_capped_params* p, ssr_stream_t stream) {
+    SSR_REQUIRE(p, "ssr_tile_write_capped", "null params");
+    SSR_REQUIRE(p->n >= 0 && p->n < (int64_t)1 << 31, "ssr_tile_write_capped", "count out of range");
+    SSR_REQUIRE(p->capacity >= 0 && p->capacity < (int64_t)1 << 31, "ssr_tile_write_capped", "capacity out of range");
+    if (p->n == 0 || p->capacity == 0) return 0;
+    SSR_REQUIRE(p->num_images >= 1, "ssr_tile_write_capped", "num_images must be at least 1");
+    SSR_REQUIRE(p->num_images == 1 || p->image_ids || (p->rows_per_image > 0 && p->rows_per_image * p->num_images == p->n),
+                "ssr_tile_write_capped", "without image_ids, n must be num_images * rows_per_image");
+    SSR_REQUIRE(p->num_images == 1 || !p->visible_ids, "ssr_tile_write_capped", "the work list is for one image");
+    SSR_REQUIRE(p->aabb && p->sort_depth && p->xy && p->conic && p->opac && p->cum_tiles, "ssr_tile_write_capped", "null pointer");
+    SSR_REQUIRE(p->isect_ids && p->flatten_ids, "ssr_tile_write_capped", "null output");
+    SSR_REQUIRE(!p->visible_ids || p->n_visible, "ssr_tile_write_capped", "a work list needs its device count");
+    SSR_REQUIRE(p->width > 0 && p->height > 0, "ssr_tile_write_capped", "empty image");
+    SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->aabb) & 15) == 0 && (reinterpret_cast<uintptr_t>(p->xy) & 7) == 0,
+                "ssr_tile_write_capped", "aabb must be 16-byte and xy 8-byte aligned");
+    const int tw = (int)ceil_div(p->width, kTile), th = (int)ceil_div(p->height, kTile);
+    SSR_REQUIRE((int64_t)p->num_images * tw * th < (int64_t)1 << 31, "ssr_tile_write_capped",
+                "tile ids of all images must fit 31 bits");
+    const bool images = p->num_images > 1;
+    const TileWriteArgs A = {reinterpret_cast<const float4*>(p->aabb), p->sort_depth, reinterpret_cast<const float2*>(p->xy),
+                             p->conic, p->opac, p->cum_tiles, tw, th, p->isect_ids, p->flatten_ids, p->visible_ids,
+                             p->tile_active, (images && !p->image_ids) ? (uint32_t)p->rows_per_image : 0u,
+                             images ? p->image_ids : nullptr};
+    hipLaunchKernelGGL(tile_write_capped_kernel, dim3((unsigned)ceil_div(p->n, kTileBlock)), dim3(kTileBlock), 0,
+                       as_stream(stream), p->n, A, p->capacity, p->n_visible);
+    SSR_CHECK_LAUNCH("ssr_tile_write_capped");
     return 0;
 }
 
@@ -516,8 +581,19 @@ int ssr_tile_offsets(int64_t n_isects, const int64_t* sorted_ids, uint32_t n_til
     if (n_isects == 0) return ssr_fill_u32(offsets, 0u, n_tiles, stream);   // IntersectTile.cu:448-451
     SSR_REQUIRE(sorted_ids, "ssr_tile_offsets", "null keys");
     hipLaunchKernelGGL(tile_offsets_kernel, dim3((unsigned)ceil_div(n_isects, kTileBlock)), dim3(kTileBlock), 0,
-                       as_stream(stream), n_isects, sorted_ids, (int64_t)n_tiles, offsets);
+                       as_stream(stream), n_isects, (const int64_t*)nullptr, sorted_ids, (int64_t)n_tiles, offsets);
     SSR_CHECK_LAUNCH("ssr_tile_offsets");
+    return 0;
+}
+
+int ssr_tile_offsets_capped(int64_t capacity, const int64_t* n_isects, const int64_t* sorted_ids, uint32_t n_tiles,
+                            int32_t* offsets, ssr_stream_t stream) {
+    SSR_REQUIRE(capacity > 0 && capacity < (int64_t)1 << 31, "ssr_tile_offsets_capped", "capacity out of range");
+    SSR_REQUIRE(n_tiles > 0 && n_tiles < 0x7fffffffu, "ssr_tile_offsets_capped", "tile count out of range");
+    SSR_REQUIRE(offsets && sorted_ids && n_isects, "ssr_tile_offsets_capped", "null pointer");
+    hipLaunchKernelGGL(tile_offsets_kernel, dim3((unsigned)ceil_div(capacity, kTileBlock)), dim3(kTileBlock), 0,
+                       as_stream(stream), capacity, n_isects, sorted_ids, (int64_t)n_tiles + 1, offsets);
+    SSR_CHECK_LAUNCH("ssr_tile_offsets_capped");
     return 0;
 }
 
@@ -530,7 +606,6 @@ int ssr_tile_order(const int32_t* tile_offsets, uint32_t n_tiles, int64_t n_isec
     SSR_REQUIRE(n_tiles < (1u << 30), "ssr_tile_order", "too many tiles");
     if (n_tiles == 0) return 0;
     SSR_REQUIRE(tile_offsets && order, "ssr_tile_order", "null pointer");
-    SSR_REQUIRE(n_isects >= 0, "ssr_tile_order", "negative count");
     SSR_REQUIRE(scratch && scratch_bytes >= ssr_tile_order_scratch_bytes(n_tiles), "ssr_tile_order", "scratch too small");
     uint32_t* counts = static_cast<uint32_t*>(scratch);
     const dim3 grid((unsigned)ceil_div((int64_t)n_tiles, kOrderBlock)), block(kOrderBlock);

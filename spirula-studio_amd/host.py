@@ -30,6 +30,8 @@ SYMBOLS = {
     "ssrh_copy_params_to_host": (C.c_int, [vp, vp, vp, vp, vp, vp]),
     "ssrh_set_tile_mask": (C.c_int, [vp, C.c_int, C.c_int]),
     "ssrh_set_loss_map": (C.c_int, [vp, C.c_int]),
+    "ssrh_set_deferred_counts": (C.c_int, [C.c_int, C.c_int64]),
+    "ssrh_deferred_capacity": (C.c_int64, []),
     "ssrh_forward_3dgs": (C.c_int, [C.c_char_p, C.c_int, C.c_int, C.c_int, C.c_int]),
     "ssrh_backward_from_render_grad": (C.c_int, [vp, vp, vp]),
     "ssrh_copy_render_to_host": (C.c_int, [vp, vp, vp]),
@@ -81,9 +83,11 @@ class Engine:
 
     def __init__(self, scene, device=0, fuse_tile_count=True, visible_list=True, packed_rows=True, overwrite_world_grads=True,
                  stage_profiling=False, sh_degree=3, packed_projection=False, packed_vscreen=True,
-                 tile_sort=True):
+                 tile_sort=True, deferred_counts=False):
         """packed_projection: forward_3dgs(packed=true), the compacted projection outputs of
-        projection_3dgs_packed_forward (the visible-splat work list then has no role)."""
+        projection_3dgs_packed_forward (the visible-splat work list then has no role).
+        deferred_counts (with tile_sort): after the first iteration the forward no longer waits for the
+        intersection count; see set_deferred_counts."""
         self.h = load()
         self.packed_projection = bool(packed_projection)
         self.dist_type, self.output_median = 0, False   # variants of the next forward (set_variants)
@@ -96,6 +100,7 @@ class Engine:
         self.packed_vscreen = int(packed_vscreen)
         self.tile_sort = int(tile_sort)
         check(self.h.ssrh_set_options(*self.opts, int(stage_profiling), self.packed_vscreen, self.tile_sort))
+        self.set_deferred_counts(deferred_counts, 0)
         f32 = lambda a: np.ascontiguousarray(a, np.float32)
         self._keep = [f32(scene.means), f32(scene.quats), f32(scene.log_scales), f32(scene.opacity_logits),
                       f32(scene.features_dc), f32(scene.features_sh)]
@@ -166,6 +171,17 @@ class Engine:
              "scale_regularization_weight", "mcmc_opacity_reg_weight", "mcmc_scale_reg_weight", "quat_norm_reg_weight",
              "sh_reg_weight", "erank_reg_weight", "erank_reg_weight_s3", "color_trust_linear", "eps_tr"]
 
+    def set_deferred_counts(self, on, capacity=None):
+        """on: the forward sizes its key arrays from the previous iteration's intersection count (plus 1/16 and
+        65536 entries) and leaves the count on the device instead of waiting for it; the backward (or n_isects)
+        raises if the count turned out larger, and the iteration must then be repeated (the next forward reads its
+        count). capacity: entries for the next forward's arrays; 0 makes it read its count; None keeps the current."""
+        check(self.h.ssrh_set_deferred_counts(int(bool(on)), -1 if capacity is None else int(capacity)))
+
+    @property
+    def deferred_capacity(self):
+        return int(self.h.ssrh_deferred_capacity())
+
     def set_loss_map(self, device_ptr, accum_mode):
         """The [C,H,W] loss map (a device pointer that stays valid) the fused training step accumulates per splat:
         accum_mode 1 max, 2 sum, 3 avg; None or 0 switches it off."""
@@ -220,7 +236,10 @@ class Engine:
 
     @property
     def n_isects(self):
-        return int(self.h.ssrh_last_n_isects())
+        v = int(self.h.ssrh_last_n_isects())
+        if v == -2:
+            check(1)
+        return v
 
     def render(self):
         h, w = self.sc.height, self.sc.width

@@ -40,6 +40,17 @@ const int32_t* g_tile_order_for = nullptr;   // the tile_offsets that order was 
 const float* g_vrows_for_xy = nullptr; // the v_screen.xy buffer they stand in for
 const int32_t* g_bwd_list = nullptr; // list of the last projection backward
 int64_t g_bwd_count = 0;
+// Counts left on the device (Options::deferred_counts): the key arrays of the next intersection are sized from
+// g_deferred_capacity (0: unknown, that call reads the count as the reference does), the counters travel to pinned
+// memory behind the scan, and resolve_counts() waits for them when somebody needs the numbers.
+int64_t g_deferred_capacity = 0;
+int64_t g_deferred_used = 0;          // capacity of the arrays the pending counts belong to
+bool g_counts_pending = false;
+int64_t* g_counts_host = nullptr;     // pinned [2]
+ssr_event_t g_counts_event = nullptr;
+const int32_t* g_offsets_closed = nullptr;   // tile_offsets with one more entry, the end of the last tile (null: none)
+
+int64_t capacity_for(int64_t n_isects) { return n_isects + n_isects / 16 + 65536; }
 
 struct StageTimer {
     ssr_event_t a = nullptr, b = nullptr;
@@ -231,9 +242,27 @@ namespace ssr_ext {
 Options& options() { return g_opts; }
 void set_stage_profiling(bool on) { g_profile = on; }
 StageTimes last_stage_times() { return g_times; }
-int64_t last_n_isects() { return g_n_isects; }
-int64_t last_n_visible() { return g_n_visible; }
+void resolve_counts() {
+    if (!g_counts_pending) return;
+    g_counts_pending = false;
+    ok(ssr_event_synchronize(g_counts_event), "resolve_counts");
+    g_n_isects = g_counts_host[0];
+    if (g_visible_ids) g_n_visible = g_counts_host[1];
+    const int64_t used = g_deferred_used;
+    if (g_n_isects > used) {
+        g_deferred_capacity = 0;   // the next intersection reads its count and sizes from it
+        throw std::runtime_error("resolve_counts: " + std::to_string(g_n_isects) + " intersections did not fit the " +
+                                 std::to_string(used) + " the arrays were sized for; the images and gradients of this "
+                                 "iteration miss fragments: repeat it");
+    }
+    g_deferred_capacity = capacity_for(g_n_isects);
+}
+void set_deferred_capacity(int64_t capacity) { g_deferred_capacity = capacity < 0 ? 0 : capacity; }
+int64_t deferred_capacity() { return g_deferred_capacity; }
+int64_t last_n_isects() { resolve_counts(); return g_n_isects; }
+int64_t last_n_visible() { resolve_counts(); return g_n_visible; }
 bool backward_overwrites_all_rows(int64_t num_splats) {
+    resolve_counts();
     if (!g_opts.overwrite_world_grads) return false;
     if (g_packed_mode) return false;                       // packed rows: only listed splats are written
     if (!g_visible_ids || g_n_visible < 0) return true;    // no list: every row is visited
@@ -257,6 +286,7 @@ projection_3dgs_forward(const int64_t num_splats, const int max_sh_degree,
                         DeviceVector<float> radii, const std::optional<TorchTensorView> sh_value_packed,
                         const std::optional<TorchTensorView> sh_value_bounds, const uint32_t num_sh_buffer,
                         const int sh_value_bits, const int64_t sh_bounds_stride) {
+    try { ssr_ext::resolve_counts(); } catch (const std::runtime_error&) {}   // counts of an iteration nobody finished
     ssr_projection_fwd_params p;
     std::memset(&p, 0, sizeof(p));
     p.num_splats = num_splats;
@@ -329,6 +359,7 @@ projection_3dgs_packed_forward(const int64_t num_splats, const int max_sh_degree
                                DeviceVector<float> radii, const std::optional<TorchTensorView> sh_value_packed,
                                const std::optional<TorchTensorView> sh_value_bounds, const uint32_t num_sh_buffer,
                                const int sh_value_bits, const int64_t sh_bounds_stride) {
+    try { ssr_ext::resolve_counts(); } catch (const std::runtime_error&) {}   // counts of an iteration nobody finished
     ssr_projection_packed_params p;
     std::memset(&p, 0, sizeof(p));
     p.num_splats = num_splats;
@@ -433,6 +464,57 @@ void compute_tile_active(TorchTensorView mask, int I, int width, int height, int
            "compute_tile_active");
 }
 
+namespace {
+// K4-K6 in arrays of g_deferred_used entries, the counts staying on the device: the key write stops at the capacity,
+// the sort reads the count where it lies, and the offsets carry one more entry, the end of the last tile, which
+// the compositing launches read instead of a host count.
+std::tuple<DeviceVector<int64_t>, DeviceVector<int32_t>, DeviceTensor3D<int32_t>>
+intersect_tile_deferred(DeviceTensorFloatND& aabb, DeviceTensorFloatND& depths, DeviceTensorFloatND& proj_xy,
+                        DeviceTensorFloatND& proj_conic, DeviceTensorFloatND& proj_opac, uint32_t I, uint32_t image_width,
+                        uint32_t image_height, const int32_t* img_ids, const int32_t* tile_active, DeviceVector<int64_t>& cum,
+                        int64_t total) {
+    const uint32_t tile_w = (image_width + 15) / 16, tile_h = (image_height + 15) / 16;
+    const uint32_t n_tiles = tile_w * tile_h * I;
+    const int64_t cap = g_deferred_used;
+    if (cap >= ((int64_t)1 << 31)) throw std::runtime_error("do_intersect_tile_generic: capacity beyond 2^31-1 intersections");
+    int32_t* offs = DevicePool::global().acquire<int32_t>(PoolSlot::IsectOffsets, (size_t)n_tiles + 1);
+    DeviceTensor3D<int32_t> offsets(offs, I, tile_h, tile_w);
+    DeviceVector<int64_t> ids_a, ids_b; ids_a.resize(PoolSlot::IsectIdsA, cap); ids_b.resize(PoolSlot::IsectIdsB, cap);
+    DeviceVector<int32_t> flat_a, flat_b; flat_a.resize(PoolSlot::IsectFlatA, cap); flat_b.resize(PoolSlot::IsectFlatB, cap);
+    {
+        StageTimer t(&g_times.k4);
+        ssr_tile_write_capped_params p;
+        std::memset(&p, 0, sizeof(p));
+        p.n = total; p.num_images = (int32_t)I; p.rows_per_image = img_ids ? 0 : total / I; p.image_ids = img_ids;
+        p.aabb = aabb.data_ptr(); p.sort_depth = depths.data_ptr(); p.xy = proj_xy.data_ptr(); p.conic = proj_conic.data_ptr();
+        p.opac = proj_opac.data_ptr(); p.cum_tiles = cum.data_ptr(); p.width = image_width; p.height = image_height;
+        p.isect_ids = ids_a.data_ptr(); p.flatten_ids = flat_a.data_ptr(); p.capacity = cap;
+        if (g_visible_ids && I == 1) {
+            p.visible_ids = g_visible_ids; p.n_visible = g_counters + 1;
+        }
+        p.tile_active = tile_active;
+        ok(ssr_tile_write_capped(&p, nullptr), "do_intersect_tile_generic/write");
+    }
+    int selector = 0;
+    {
+        StageTimer t(&g_times.k5);
+        const size_t sb = ssr_sort_tile_scratch_bytes(cap, n_tiles);
+        void* scratch = DevicePool::global().acquire<uint8_t>(PoolSlot::IsectSortScratch, sb);
+        ok(ssr_sort_tile_pairs_capped(ids_a.data_ptr(), ids_b.data_ptr(), flat_a.data_ptr(), flat_b.data_ptr(), cap, g_counters,
+                                      n_tiles, offs, &selector, scratch, sb, nullptr), "do_intersect_tile_generic/tile_sort");
+    }
+    g_offsets_closed = offs;
+    {
+        StageTimer t(&g_times.k6);
+        const size_t sb = ssr_tile_order_scratch_bytes(n_tiles);
+        int32_t* order = DevicePool::global().acquire<int32_t>(PoolSlot::IsectTileOrder, (size_t)n_tiles + sb / sizeof(int32_t));
+        ok(ssr_tile_order(offs, n_tiles, -1, order, order + n_tiles, sb, nullptr), "do_intersect_tile_generic/order");
+        g_tile_order = order; g_tile_order_for = offs;
+    }
+    return std::make_tuple(selector ? ids_b : ids_a, selector ? flat_b : flat_a, offsets);
+}
+}  // namespace
+
 std::tuple<DeviceVector<int64_t>, DeviceVector<int32_t>, DeviceTensor3D<int32_t>>
 do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, DeviceTensorFloatND* proj_xy,
                           DeviceTensorFloatND* proj_conic, DeviceTensorFloatND* proj_opac, const uint32_t I,
@@ -444,7 +526,10 @@ do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, 
     if (!proj_xy || !proj_conic || !proj_opac)
         throw std::runtime_error("do_intersect_tile_generic: AABB mode is not built in this backend (ellipse mode is)");
     if (I < 1) throw std::runtime_error("do_intersect_tile_generic: no image");
-    g_tile_order = nullptr; g_tile_order_for = nullptr;
+    g_tile_order = nullptr; g_tile_order_for = nullptr; g_offsets_closed = nullptr;
+    if (g_counts_pending) {   // counts nobody asked for: settle them before the counters are reused
+        try { ssr_ext::resolve_counts(); } catch (const std::runtime_error&) {}
+    }
     const int64_t total = depths.numel();
     const int32_t* img_ids = (image_ids && I > 1) ? image_ids->data_ptr() : nullptr;   // packed rows of several cameras
     if (!img_ids && total % I != 0) throw std::runtime_error("do_intersect_tile_generic: rows are not a multiple of the image count");
@@ -475,14 +560,30 @@ do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, 
         if (!g_counters) g_counters = DevicePool::global().acquire<int64_t>(PoolSlot::IsectCounters, 2);
         ok(ssr_inclusive_sum_i64(tiles_per_splat.data_ptr(), cum.data_ptr(), total, g_counters, scratch, sb, nullptr),
            "do_intersect_tile_generic/scan");
-        if (total > 0) {
+        if (total > 0 && g_opts.deferred_counts && g_opts.tile_sort && g_deferred_capacity > 0) {
+            // the counts follow the scan to pinned memory; nobody waits here
+            if (!g_counts_host) {
+                g_counts_host = static_cast<int64_t*>(ssr_host_malloc_pinned(2 * sizeof(int64_t)));
+                g_counts_event = ssr_event_create();
+                if (!g_counts_host || !g_counts_event) throw_last("do_intersect_tile_generic/pinned counts");
+            }
+            ok(ssr_memcpy(g_counts_host, g_counters, 2 * sizeof(int64_t), 2 /* device to host */, nullptr, 1),
+               "do_intersect_tile_generic/counts");
+            ok(ssr_event_record(g_counts_event, nullptr), "do_intersect_tile_generic/counts");
+            g_counts_pending = true;
+            g_deferred_used = g_deferred_capacity;
+        } else if (total > 0) {
             int64_t both[2] = {0, 0};
             ok(ssr_read_i64(g_counters, both, g_visible_ids ? 2 : 1, nullptr), "do_intersect_tile_generic/readback");
             n_isects = both[0];
             if (g_visible_ids) g_n_visible = both[1];
         }
     }
+    if (g_counts_pending)
+        return intersect_tile_deferred(aabb, depths, *proj_xy, *proj_conic, *proj_opac, I, image_width, image_height, img_ids,
+                                       tile_active, cum, total);
     g_n_isects = n_isects;
+    if (g_opts.deferred_counts) g_deferred_capacity = capacity_for(n_isects);
     DeviceTensor3D<int32_t> offsets; offsets.resize(PoolSlot::IsectOffsets, I, tile_h, tile_w);
     if (n_isects == 0) {
         offsets.zero();
@@ -560,6 +661,7 @@ rasterize_to_pixels_3dgs_fwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     p.width = image_width; p.height = image_height;
     p.tile_offsets = tile_offsets.data_ptr(); p.flatten_ids = flatten_ids.data_ptr(); p.n_isects = flatten_ids.size();
     if (g_tile_order && g_tile_order_for == p.tile_offsets) p.tile_order = g_tile_order;
+    p.tile_offsets_closed = (g_offsets_closed && g_offsets_closed == p.tile_offsets) ? 1 : 0;
     p.render_rgb = (float*)std::get<0>(renders).data_ptr(); p.render_depth = std::get<1>(renders).data_ptr();
     p.render_T = Ts.data_ptr(); p.last_ids = last.data_ptr();
     if (g_packed_rows && p.screen.xy == g_packed_for_xy) p.packed_rows = g_packed_rows;
@@ -639,6 +741,7 @@ rasterize_to_pixels_3dgs_bwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     p.width = image_width; p.height = image_height;
     p.tile_offsets = tile_offsets.data_ptr(); p.flatten_ids = flatten_ids.data_ptr(); p.n_isects = flatten_ids.size();
     if (g_tile_order && g_tile_order_for == p.tile_offsets) p.tile_order = g_tile_order;
+    p.tile_offsets_closed = (g_offsets_closed && g_offsets_closed == p.tile_offsets) ? 1 : 0;
     p.render_T = render_Ts.data_ptr(); p.last_ids = last_ids.data_ptr(); p.render_depth = std::get<1>(render_outputs_tuple).data_ptr();
     p.v_render_rgb = (const float*)std::get<0>(v_render_outputs).data_ptr();
     p.v_render_depth = std::get<1>(v_render_outputs).data_ptr();
@@ -695,6 +798,7 @@ void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
     ssr_projection_bwd_params p;
     std::memset(&p, 0, sizeof(p));
     p.num_splats = num_splats;
+    ssr_ext::resolve_counts();   // the work list's length, when the forward left it on the device
     p.sh_degree = max_sh_degree;
     p.antialiased = g_antialiased ? 1 : 0;
     p.world = world_of(splats_world);
@@ -789,6 +893,7 @@ void fused_projection_bwd_optimizer_3dgs(
     const float quat_norm_reg_weight, const float sh_reg_weight, bool use_scale_agnostic_mean, bool color_trust_linear,
     float eps_tr, std::variant<int32_t, TorchTensorView> step, int quantization_level) {
     const char* w = "fused_projection_bwd_optimizer_3dgs: ";
+    ssr_ext::resolve_counts();   // no parameter is stepped on gradients of an intersection that did not fit
     const bool is_packed = camera_ids.data_ptr() && gaussian_ids.data_ptr();   // src/kernels/optim/FusedProjectionBwdOptim.cu:160
     // quantization_level: 0 = fp32 SH and moments; 1 = 16-bit SH values, 8-bit moments
     // (src/kernels/optim/FusedProjectionBwdOptim_kernel.cuh:1104-1111; validation as FusedProjectionBwdOptim.cu:386-400)

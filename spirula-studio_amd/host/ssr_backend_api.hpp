@@ -178,6 +178,15 @@ struct Options {
     // The key sort partitions by tile (the tile bits only) and then sorts each tile's range on the
     // depth bits with one workgroup per tile, instead of six whole-array digit passes; same result.
     bool tile_sort = false;
+    // With tile_sort: do_intersect_tile_generic does not wait for the intersection count (the reference blocks on
+    // it, IntersectTile.cu:432-436). The key arrays are sized from the previous call's count (plus 1/16 and 65536
+    // entries; or set_deferred_capacity), the count stays on the device and reaches the host asynchronously; the
+    // returned id vectors then have the capacity as their size; only their first last_n_isects() entries are keys.
+    // resolve_counts() waits for the numbers: it is called by everything here that needs them (last_n_isects,
+    // last_n_visible, backward_overwrites_all_rows, projection_3dgs_backward, the fused optimizer) and throws if
+    // the count did not fit; the images and gradients of that iteration are then incomplete and the next
+    // intersection reads its count again. The first call, and any call with capacity 0, blocks as before.
+    bool deferred_counts = false;
     // int8 codes x per-splat fp16 scale as SH storage (the benchmark's format): sh_value_bits == 8
     // with sh_value_bounds holding the fp16 scales when this is set.
     bool sh_int8_f16scale = false;
@@ -190,6 +199,9 @@ void set_stage_profiling(bool on);
 StageTimes last_stage_times();
 int64_t last_n_isects();
 int64_t last_n_visible();   // -1 when the visible list is off
+void resolve_counts();      // see Options::deferred_counts
+void set_deferred_capacity(int64_t capacity);
+int64_t deferred_capacity();
 // The list the last projection_3dgs_backward ran over (device pointer) and its length; it stays
 // intact until the projection after next (the two list buffers alternate). Null when it had none.
 const int32_t* last_backward_list(int64_t* count);

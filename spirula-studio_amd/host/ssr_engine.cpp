@@ -455,6 +455,16 @@ int ssrh_set_options(int fuse_tile_count, int visible_list, int packed_rows, int
     });
 }
 
+// on: the intersection count stays on the device between the forward's stages (Options::deferred_counts);
+// capacity >= 0 also sets the size of the next call's key arrays (0: that call reads its count).
+int ssrh_set_deferred_counts(int on, int64_t capacity) {
+    return guard([&] {
+        ssr_ext::options().deferred_counts = on != 0;
+        if (capacity >= 0) ssr_ext::set_deferred_capacity(capacity);
+    });
+}
+int64_t ssrh_deferred_capacity(void) { return ssr_ext::deferred_capacity(); }
+
 // host or device pointers; num_sh = coefficients per splat excluding DC (15 for SH3)
 int ssrh_set_data_3dgs(int64_t n, const float* means, const float* quats, const float* scales, const float* opacities,
                        const float* dc, const float* sh, int num_sh) {
@@ -627,8 +637,9 @@ int ssrh_cache_pointer(int which, void** ptr, int64_t* count) {
     });
 }
 
-int64_t ssrh_last_n_isects(void) { return ssr_ext::last_n_isects(); }
-int64_t ssrh_last_n_visible(void) { return ssr_ext::last_n_visible(); }
+// -2: the count did not fit the arrays it was left to (deferred counts); the message is in ssrh_last_error
+int64_t ssrh_last_n_isects(void) { int64_t v = -2; guard([&] { v = ssr_ext::last_n_isects(); }); return v; }
+int64_t ssrh_last_n_visible(void) { int64_t v = -2; guard([&] { v = ssr_ext::last_n_visible(); }); return v; }
 
 int ssrh_last_stage_times(float* out9) {
     return guard([&] {

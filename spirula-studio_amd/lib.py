@@ -55,7 +55,7 @@ class RasterFwdParams(C.Structure):
                 ("n_isects", C.c_int64), ("render_rgb", vp), ("render_depth", vp),
                 ("render_T", vp), ("last_ids", vp), ("packed_rows", vp), ("dist_type", C.c_int32),
                 ("distortion_rgb", vp), ("distortion_depth", vp), ("render_median", vp),
-                ("num_images", C.c_int32), ("tile_order", vp)]
+                ("num_images", C.c_int32), ("tile_order", vp), ("tile_offsets_closed", C.c_int32)]
 
 
 class RasterBwdParams(C.Structure):
@@ -67,7 +67,15 @@ class RasterBwdParams(C.Structure):
                 ("distortion_rgb", vp), ("distortion_depth", vp), ("v_distortion_rgb", vp),
                 ("v_distortion_depth", vp), ("v_render_median", vp), ("accum_mode", C.c_int32),
                 ("accum_weight_map", vp), ("gaussian_ids", vp), ("num_world", C.c_int64), ("accum_weight", vp),
-                ("num_images", C.c_int32), ("tile_order", vp)]
+                ("num_images", C.c_int32), ("tile_order", vp), ("tile_offsets_closed", C.c_int32)]
+
+
+class TileWriteCappedParams(C.Structure):
+    _fields_ = [("n", C.c_int64), ("rows_per_image", C.c_int64), ("image_ids", vp), ("num_images", C.c_int32),
+                ("aabb", vp), ("sort_depth", vp), ("xy", vp), ("conic", vp), ("opac", vp), ("cum_tiles", vp),
+                ("width", C.c_uint32), ("height", C.c_uint32), ("isect_ids", vp), ("flatten_ids", vp),
+                ("capacity", C.c_int64), ("visible_ids", vp), ("n_visible", vp),
+                ("tile_active", vp)]
 
 
 class ProjectionBwdParams(C.Structure):
@@ -120,6 +128,7 @@ SYMBOLS = {
     "ssr_tile_write": (_i32, [_i64, vp, vp, vp, vp, vp, vp, _u32, _u32, vp, vp, vp, _i64, vp, vp]),
     "ssr_tile_count_images": (_i32, [_i64, _i64, vp, _i32, vp, vp, vp, vp, _u32, _u32, vp, vp, vp]),
     "ssr_tile_write_images": (_i32, [_i64, _i64, vp, _i32, vp, vp, vp, vp, vp, vp, _u32, _u32, vp, vp, vp, vp]),
+    "ssr_tile_write_capped": (_i32, [C.POINTER(TileWriteCappedParams), vp]),
     "ssr_sort_scratch_bytes": (_sz, [_i64]),
     "ssr_sort_pairs_u64_i32": (_i32, [vp, vp, vp, vp, _i64, _i32, _i32, C.POINTER(C.c_int), vp, _sz, vp]),
     "ssr_tile_offsets": (_i32, [_i64, vp, _u32, vp, vp]),
@@ -128,6 +137,8 @@ SYMBOLS = {
     "ssr_sort_end_bit": (_i32, [_u32]),
     "ssr_sort_tile_scratch_bytes": (_sz, [_i64, _u32]),
     "ssr_sort_tile_pairs": (_i32, [vp, vp, vp, vp, _i64, _u32, vp, C.POINTER(C.c_int), vp, _sz, vp]),
+    "ssr_sort_tile_pairs_capped": (_i32, [vp, vp, vp, vp, _i64, vp, _u32, vp, C.POINTER(C.c_int), vp, _sz, vp]),
+    "ssr_tile_offsets_capped": (_i32, [_i64, vp, vp, _u32, vp, vp]),
     "ssr_raster_fwd": (_i32, [C.POINTER(RasterFwdParams), vp]),
     "ssr_raster_bwd": (_i32, [C.POINTER(RasterBwdParams), vp]),
     "ssr_projection_bwd": (_i32, [C.POINTER(ProjectionBwdParams), vp]),

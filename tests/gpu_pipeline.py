@@ -35,7 +35,7 @@ def world_grad_check(got, ref, n, name, rtol=WORLD_GRAD_RTOL, bad_frac=0.0, scal
 
 class GpuRun:
     def __init__(self, pkg, scene, sh_degree=3, use_list=False, use_packed=False, packed_projection=False,
-                 read_nnz=True, use_vrows=False, tile_sort=False):
+                 read_nnz=True, use_vrows=False, tile_sort=False, capacity=None):
         """use_packed: 48-byte fragment rows for the compositing kernels. packed_projection: the
         compacted (nnz-row) projection outputs of projection_3dgs_packed_forward; read_nnz=False
         sizes the outputs for all N splats instead of reading nnz back between the two calls."""
@@ -44,6 +44,10 @@ class GpuRun:
         self.packed_projection = packed_projection
         self.read_nnz = read_nnz
         self.tile_sort = tile_sort   # ssr_sort_tile_pairs instead of the whole-key sort + ssr_tile_offsets
+        # capacity (with tile_sort): the key arrays hold that many entries and nothing is read back between the scan
+        # and the compositing (ssr_tile_write_capped, ssr_sort_tile_pairs_capped, closed offsets)
+        self.capacity = capacity
+        assert capacity is None or tile_sort
         self.use_vrows = use_vrows   # one 12-float gradient row per splat between K8 and K9
         assert not (packed_projection and use_list)
         self.L = pkg.lib
@@ -203,6 +207,8 @@ class GpuRun:
         self.d["scan_scratch"] = D((max(sb, 8),), np.uint8)
         self.check(self.lib.ssr_inclusive_sum_i64(self.ptr("counts"), self.ptr("cum"), n, self.ptr("counters"),
                                                   self.ptr("scan_scratch"), sb, None))
+        if self.capacity is not None:
+            return self.tiles_capped()
         k = (C.c_int64 * 2)(0, 0)
         if n:
             self.check(self.lib.ssr_read_i64(self.ptr("counters"), k, 2, None))
@@ -243,6 +249,43 @@ class GpuRun:
         if not (self.tile_sort and K):
             self.check(self.lib.ssr_tile_offsets(K, self.ptr(self.keys), n_tiles, self.ptr("offsets"), None))
 
+    def tiles_capped(self):
+        """K4-K6 without knowing the counts on the host; self.K becomes the capacity, self.K_real the count read
+        back after everything was launched."""
+        sc, D = self.sc, self.L.DeviceArray
+        n, cap = self.rows, int(self.capacity)
+        n_tiles = sc.tile_w * sc.tile_h
+        self.d["offsets"] = D((n_tiles + 1,), np.int32)
+        for nm in ["keys_a", "keys_b"]:
+            self.d[nm] = D((cap,), np.int64)
+        for nm in ["vals_a", "vals_b"]:
+            self.d[nm] = D((cap,), np.int32)
+        p = self.L.TileWriteCappedParams()
+        p.n, p.num_images = n, 1
+        p.aabb, p.sort_depth, p.xy, p.conic, p.opac = (self.ptr("aabb"), self.ptr("sort_depth"), self.ptr("xy"),
+                                                       self.ptr("conic"), self.ptr("opac"))
+        p.cum_tiles, p.width, p.height = self.ptr("cum"), sc.width, sc.height
+        p.isect_ids, p.flatten_ids, p.capacity = self.ptr("keys_a"), self.ptr("vals_a"), cap
+        if self.use_list:
+            p.visible_ids, p.n_visible = self.ptr("vis_ids"), self.ptr("counters") + 8
+        p.tile_active = self.tile_active
+        self.check(self.lib.ssr_tile_write_capped(C.byref(p), None))
+        sb = self.lib.ssr_sort_tile_scratch_bytes(cap, n_tiles)
+        self.d["sort_scratch"] = D((sb,), np.uint8)
+        sel = C.c_int(0)
+        self.check(self.lib.ssr_sort_tile_pairs_capped(self.ptr("keys_a"), self.ptr("keys_b"), self.ptr("vals_a"),
+                                                       self.ptr("vals_b"), cap, self.ptr("counters"), n_tiles,
+                                                       self.ptr("offsets"),
+                                                       C.byref(sel), self.ptr("sort_scratch"), sb, None))
+        self.sel = sel.value
+        self.keys = "keys_b" if self.sel else "keys_a"
+        self.vals = "vals_b" if self.sel else "vals_a"
+        self.K = cap
+        k = (C.c_int64 * 2)(0, 0)
+        self.check(self.lib.ssr_read_i64(self.ptr("counters"), k, 2, None))
+        self.K_real = int(k[0])
+        self.V = int(k[1]) if self.use_list else None
+
     def order_tiles(self):
         """ssr_tile_order on the current offsets, checked here: a permutation of the tiles whose fragment counts fall
         class by class (32 fragments a class, everything from 8160 up in the first)."""
@@ -250,12 +293,13 @@ class GpuRun:
         n_tiles = self.sc.tile_w * self.sc.tile_h
         sb = self.lib.ssr_tile_order_scratch_bytes(n_tiles)
         self.d["tile_order"], self.d["tile_order_scratch"] = D((n_tiles,), np.int32), D((sb,), np.uint8)
-        self.check(self.lib.ssr_tile_order(self.ptr("offsets"), n_tiles, self.K, self.ptr("tile_order"),
+        closed = self.capacity is not None
+        self.check(self.lib.ssr_tile_order(self.ptr("offsets"), n_tiles, -1 if closed else self.K, self.ptr("tile_order"),
                                            self.ptr("tile_order_scratch"), sb, None))
         order = self.host("tile_order")
         assert np.array_equal(np.sort(order), np.arange(n_tiles))
         offs = self.host("offsets").ravel().astype(np.int64)
-        cls = np.minimum(np.diff(np.concatenate([offs, [self.K]])) >> 5, 255)[order]
+        cls = np.minimum(np.diff(offs if closed else np.concatenate([offs, [self.K]])) >> 5, 255)[order]
         assert np.all(cls[1:] <= cls[:-1])
 
     def raster_fwd(self):
@@ -286,6 +330,7 @@ class GpuRun:
             self.d["r_median"] = D((h, w), np.float32)
             p.render_median = self.ptr("r_median")
         p.tile_order = self.ptr("tile_order")
+        p.tile_offsets_closed = 1 if self.capacity is not None else 0
         self.check(self.lib.ssr_raster_fwd(C.byref(p), None))
 
     def raster_bwd(self, v_rgb=None, v_depth=None, v_T=None):
@@ -335,6 +380,7 @@ class GpuRun:
             if self.packed_projection:
                 p.gaussian_ids = self.ptr("gaussian_ids")
         p.tile_order = self.ptr("tile_order")
+        p.tile_offsets_closed = 1 if self.capacity is not None else 0
         self.check(self.lib.ssr_raster_bwd(C.byref(p), None))
         if self.use_vrows and n:   # unpack for the comparisons, after checking the arrays were left alone
             for k in ["v_xy", "v_depth", "v_conic", "v_opac", "v_rgb"]:

@@ -91,6 +91,26 @@ def test_argument_checks_without_device(L):
     assert lib.ssr_tile_order_scratch_bytes(8160) == 8 * 256 * 4
     assert lib.ssr_tile_order(16, 100, 5, 16, None, 0, None) != 0 and b"scratch" in lib.ssr_last_error()
     assert lib.ssr_tile_order(None, 0, 0, None, None, 0, None) == 0
+    # the entry points that leave the counts on the device
+    from spirula_studio_amd import lib as L
+    w = L.TileWriteCappedParams()
+    assert lib.ssr_tile_write_capped(None, None) != 0 and b"null params" in lib.ssr_last_error()
+    w.n, w.capacity, w.num_images = 10, 1 << 31, 1
+    assert lib.ssr_tile_write_capped(C.byref(w), None) != 0 and b"capacity" in lib.ssr_last_error()
+    w.capacity = 0
+    assert lib.ssr_tile_write_capped(C.byref(w), None) == 0      # nothing can be written: no launch
+    w.capacity, w.num_images = 100, 0
+    assert lib.ssr_tile_write_capped(C.byref(w), None) != 0 and b"num_images" in lib.ssr_last_error()
+    w.num_images, w.aabb, w.sort_depth, w.xy, w.conic, w.opac, w.cum_tiles = 1, 16, 16, 16, 16, 16, 16
+    w.isect_ids, w.flatten_ids, w.width, w.height, w.visible_ids = 16, 16, 64, 64, 16
+    assert lib.ssr_tile_write_capped(C.byref(w), None) != 0 and b"device count" in lib.ssr_last_error()
+    sel = C.c_int(0)
+    assert lib.ssr_sort_tile_pairs_capped(16, 16, 16, 16, 0, 16, 10, 16, C.byref(sel), 16, 1 << 20, None) != 0
+    assert b"capacity" in lib.ssr_last_error()
+    assert lib.ssr_sort_tile_pairs_capped(16, 16, 16, 16, 100, None, 10, 16, C.byref(sel), 16, 1 << 20, None) != 0
+    assert b"null count" in lib.ssr_last_error()
+    assert lib.ssr_tile_offsets_capped(100, None, 16, 10, 16, None) != 0 and b"null pointer" in lib.ssr_last_error()
+    assert lib.ssr_tile_offsets_capped(0, 16, 16, 10, 16, None) != 0 and b"capacity" in lib.ssr_last_error()
 
 
 def test_missing_library_fails_loudly(pkg, monkeypatch):

@@ -51,6 +51,95 @@ def test_engine_matches_oracle(pkg, oracle, H, native):
         assert np.allclose(g1[k], g2[k], rtol=2e-3, atol=1e-6)
 
 
+def _check_deferred(eng, ref, sc):
+    """_check for an iteration whose key arrays were sized without the count: the keys are their first n_isects entries."""
+    K = ref["sorted_ids"].size
+    assert eng.n_isects == K
+    ids, flat = eng.cache("sorted_ids"), eng.cache("sorted_flat")
+    assert ids.size == flat.size and ids.size > K
+    assert np.array_equal(ids[:K], ref["sorted_ids"]) and np.array_equal(flat[:K], ref["sorted_flat"])
+    assert np.array_equal(eng.cache("offsets"), ref["offsets"].ravel())
+    rgb, depth, T = eng.render()
+    assert np.abs(rgb - ref["fwd"]["rgb"]).max() <= 1e-4
+    assert np.abs(T - ref["fwd"]["T"]).max() <= 1e-4
+    assert np.array_equal(eng.cache("last_ids").reshape(sc.height, sc.width), ref["fwd"]["last_ids"])
+    for k, v in eng.grads().items():
+        world_grad_check(v, ref["grads"][k], sc.n, f"engine-deferred/{k}")
+
+
+@pytest.mark.parametrize("packed", [False, True])
+def test_engine_leaves_the_counts_on_the_device(pkg, oracle, H, packed):
+    """deferred_counts: the first iteration reads its intersection count as the reference does; the following ones
+    size the key arrays from the last count and wait for nothing between the projection and the compositing. Same
+    keys, ranges, image and gradients; a count that outgrows the arrays makes the backward raise before any gradient
+    is used, and the next iteration reads its count again."""
+    host, lib = H
+    sc = pkg.scenes.make_scene(1, n=30000, width=320, height=240, parity_variant=True)
+    if packed:
+        sc.means[::3, 2] = -10.0
+    ref = oracle.pipeline_packed(sc) if packed else oracle.pipeline(sc)
+    K = ref["sorted_ids"].size
+    eng = host.Engine(sc, packed_projection=packed, visible_list=not packed, deferred_counts=True)
+    assert eng.deferred_capacity == 0
+    eng.forward(); eng.backward()                     # blocking: learns the capacity
+    assert eng.n_isects == K and eng.cache("sorted_ids").size == K
+    assert eng.deferred_capacity == K + K // 16 + 65536
+    for _ in range(2):                                # deferred
+        eng.forward(); eng.backward()
+        if packed:
+            assert eng.n_isects == K and np.array_equal(eng.cache("sorted_ids")[:K], ref["sorted_ids"])
+            rgb, _, T = eng.render()
+            assert np.abs(rgb - ref["fwd"]["rgb"]).max() <= 1e-4
+            for k, v in eng.grads().items():
+                world_grad_check(v, ref["grads"][k], sc.n, f"engine-deferred-packed/{k}")
+        else:
+            _check_deferred(eng, ref, sc)
+        assert eng.cache("sorted_ids").size == K + K // 16 + 65536
+    # arrays too small for the count: the forward still runs (on the keys that fit), the backward refuses
+    eng.set_deferred_counts(True, capacity=K // 2)
+    eng.forward()
+    with pytest.raises(lib.SsrError, match="did not fit"):
+        eng.backward()
+    assert eng.deferred_capacity == 0
+    eng.forward(); eng.backward()                     # reads its count again
+    assert eng.n_isects == K and eng.cache("sorted_ids").size == K
+    for k, v in eng.grads().items():
+        world_grad_check(v, ref["grads"][k], sc.n, f"engine-after-overflow/{k}")
+    # the count query itself reports the overflow
+    eng.set_deferred_counts(True, capacity=K - 1)
+    eng.forward()
+    with pytest.raises(lib.SsrError, match="did not fit"):
+        eng.n_isects
+    eng.set_deferred_counts(False, 0)
+
+
+def test_engine_fused_step_refuses_an_intersection_that_did_not_fit(pkg, oracle, H):
+    """With the counts left on the device, the fused optimizer checks them before it steps: no parameter moves on
+    gradients that miss fragments, and the repeated iteration takes the step the blocking engine takes."""
+    host, lib = H
+    sc = pkg.scenes.make_scene(1, n=20000, width=320, height=240, parity_variant=True)
+    h = dict(lr_means=1.6e-4, lr_quats=1e-3, lr_scales=5e-3, lr_opacs=5e-2, lr_features_dc=2.5e-3, lr_features_sh=1.25e-4)
+    plain = host.Engine(sc)
+    plain.forward(); plain.backward_fused_optimizer(h, 1)
+    want = plain.params()
+    K = plain.n_isects
+    eng = host.Engine(sc, deferred_counts=True)
+    before = eng.params()
+    eng.set_deferred_counts(True, capacity=K // 3)
+    eng.forward()
+    with pytest.raises(lib.SsrError, match="did not fit"):
+        eng.backward_fused_optimizer(h, 1)
+    now = eng.params()
+    for k in oracle.WORLD_KEYS:
+        assert np.array_equal(now[k], before[k]), k
+    eng.set_deferred_counts(True, capacity=K + 1000)   # fits: nothing is read back before the step
+    eng.forward(); eng.backward_fused_optimizer(h, 1)
+    got = eng.params()
+    for k in oracle.WORLD_KEYS:
+        assert np.allclose(got[k], want[k], rtol=1e-4, atol=1e-6), k
+    eng.set_deferred_counts(False, 0)
+
+
 def test_engine_quantized_and_equirect(pkg, oracle, H):
     host, lib = H
     for cfg, kw in [(3, dict(n=20000, width=320, height=192)), (5, dict(n=30000, width=512, height=256))]:

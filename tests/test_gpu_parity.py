@@ -34,11 +34,14 @@ def _grad_close(got, ref, abs_scale, name, max_bad=0, rtol=GRAD_RTOL, afrac=2e-6
 
 
 def _compare(gpu, oracle, sc, label, fused_count=False, use_list=False, use_packed=False, mask=None, variant=None,
-             use_vrows=False, tile_sort=False):
+             use_vrows=False, tile_sort=False, spare=None):
+    """spare: run K4-K6 without reading the counts back, in arrays of K + spare entries (spare >= 0)."""
     live = None if mask is None else oracle.compute_tile_active(mask, sc.width, sc.height)
     r = oracle.pipeline(sc, tile_active=live, variant=variant)
     print(f"[{label}] N={sc.n} {sc.width}x{sc.height} visible={r['proj']['visible']} K={r['isect_ids'].size}", flush=True)
-    g = GpuRun(gpu, sc, use_list=use_list, use_packed=use_packed, use_vrows=use_vrows, tile_sort=tile_sort)
+    K = r["isect_ids"].size
+    g = GpuRun(gpu, sc, use_list=use_list, use_packed=use_packed, use_vrows=use_vrows, tile_sort=tile_sort,
+               capacity=None if spare is None else K + spare)
     if mask is not None:
         g.set_tile_mask(mask)
         assert np.array_equal(g.host("tile_active"), live)
@@ -57,12 +60,20 @@ def _compare(gpu, oracle, sc, label, fused_count=False, use_list=False, use_pack
     # K2..K6: bit-exact
     assert np.array_equal(g.host("counts"), r["counts"])
     assert np.array_equal(g.host("cum"), r["cum"])
-    assert g.K == r["isect_ids"].size
-    assert np.array_equal(g.unsorted_keys, r["isect_ids"])
-    assert np.array_equal(g.unsorted_vals, r["flatten_ids"])
-    assert np.array_equal(g.host(g.keys), r["sorted_ids"])
-    assert np.array_equal(g.host(g.vals), r["sorted_flat"])
-    assert np.array_equal(g.host("offsets"), r["offsets"])
+    if spare is None:
+        assert g.K == K
+        assert np.array_equal(g.unsorted_keys, r["isect_ids"])
+        assert np.array_equal(g.unsorted_vals, r["flatten_ids"])
+        assert np.array_equal(g.host(g.keys), r["sorted_ids"])
+        assert np.array_equal(g.host(g.vals), r["sorted_flat"])
+        assert np.array_equal(g.host("offsets"), r["offsets"])
+    else:   # the keys in front, one more offset
+        n_tiles = sc.tile_w * sc.tile_h
+        assert g.K_real == K and g.K == K + spare
+        assert np.array_equal(g.host(g.keys)[:K], r["sorted_ids"])
+        assert np.array_equal(g.host(g.vals)[:K], r["sorted_flat"])
+        assert np.array_equal(g.host("offsets")[:n_tiles], r["offsets"].ravel())
+        assert g.host("offsets")[n_tiles] == K
     # K7
     f = r["fwd"]
     assert np.abs(g.host("r_rgb") - f["rgb"]).max() <= IMG_TOL
@@ -117,6 +128,50 @@ def _compare(gpu, oracle, sc, label, fused_count=False, use_list=False, use_pack
         world_grad_check(got, gr[o], sc.n, f"{label}/{k}", row_floor=row_floor)
         assert not np.any(got[~vis]), k
     return g, r
+
+
+def test_counts_stay_on_the_device(gpu, oracle):
+    """K4-K8 in arrays sized without the counts (ssr_tile_write_capped, ssr_sort_tile_pairs_capped, closed offsets):
+    same keys, ranges, images and gradients as with the readback, whatever the spare room."""
+    _compare(gpu, oracle, gpu.scenes.tiny_scene(n=400, width=72, height=56, seed=3), "tiny-cap", tile_sort=True, spare=300)
+    _compare(gpu, oracle, gpu.scenes.tiny_scene(n=300, width=16, height=16, seed=6), "one-tile-cap", tile_sort=True, spare=1)
+    _compare(gpu, oracle, gpu.scenes.tiny_scene(n=400, width=72, height=56, seed=3), "exact-cap", tile_sort=True, spare=0)
+    # 128 x 128 tiles: a power of two
+    _compare(gpu, oracle, gpu.scenes.tiny_scene(n=60, width=2048, height=2048, seed=12), "pow2-cap", tile_sort=True, spare=5000)
+    sc = gpu.scenes.make_scene(2, n=30000, width=480, height=270)
+    _compare(gpu, oracle, sc, "cfg2-cap", fused_count=True, use_list=True, use_packed=True, use_vrows=True, tile_sort=True,
+             spare=70000)
+    huge = gpu.scenes.tiny_scene(n=600, width=640, height=400, seed=13)
+    huge.log_scales[::7] += 2.5          # splats that cover hundreds of tiles (the cooperative write)
+    huge.means[::50, 2] = -3.6
+    _compare(gpu, oracle, huge, "huge-cap", fused_count=True, use_list=True, tile_sort=True, spare=100)
+    none = gpu.scenes.tiny_scene(n=64, width=40, height=24, seed=1)
+    none.means[:, 2] = -10.0   # nothing in view: a count of zero that only the device knows
+    g, r = _compare(gpu, oracle, none, "all-culled-cap", tile_sort=True, spare=128)
+    assert g.K_real == 0 and not np.any(g.host("offsets")) and np.all(g.host("r_T") == 1.0)
+    g, r = _compare(gpu, oracle, none, "all-culled-cap-list", fused_count=True, use_list=True, tile_sort=True, spare=128)
+    assert g.K_real == 0 and g.V == 0 and np.all(g.host("r_T") == 1.0)
+
+
+def test_counts_beyond_the_capacity_lose_keys_only(gpu, oracle):
+    """More keys than the arrays hold: nothing outside the arrays is touched, every later stage runs on what fitted,
+    and the count that comes back says so."""
+    sc = gpu.scenes.tiny_scene(n=400, width=72, height=56, seed=3)
+    r = oracle.pipeline(sc)
+    K = r["isect_ids"].size
+    cap = K - K // 3
+    g = GpuRun(gpu, sc, tile_sort=True, capacity=cap)
+    g.run_all()
+    assert g.K_real == K and g.K == cap
+    n_tiles = sc.tile_w * sc.tile_h
+    keys, vals, offs = g.host(g.keys), g.host(g.vals), g.host("offsets")
+    assert offs[n_tiles] == cap and np.all(np.diff(offs) >= 0)
+    assert np.all((keys >> 32) < n_tiles) and np.all(np.diff(keys) >= 0)   # real keys only, sorted
+    # what fitted is what the key write puts below `cap`
+    keep = np.sort(r["isect_ids"][:cap], kind="stable")
+    assert np.array_equal(keys, keep)
+    assert vals.min() >= 0 and vals.max() < sc.n
+    assert np.isfinite(g.host("r_rgb")).all() and np.isfinite(g.host("w_means")).all()
 
 
 def _compare_packed(gpu, oracle, sc, label, fused_count=False, use_packed=False, read_nnz=True, variant=None):
