@@ -738,6 +738,112 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
     for (int i = 0; i < 3; i++) put<kPut>(V.features_dc + 3 * g + i, fin(wg.dc[i]));
 }
 
+// The degree-3 kernel with the SH gradient rows staged through LDS. A thread writing its own 180-byte row in
+// fifteen 12-byte pieces makes every store instruction of a wavefront touch 64 rows (90 cache lines for 768
+// bytes), and those partial-line writes, not the reads and not HBM, are what the kernel above waits for (the
+// texture-address unit 70 % busy, counted; staging the coefficient reads the same way made things slower).
+// Here every lane leaves its row in the wavefront's own 11.25 KB of LDS and the wavefront moves its 64 rows as one
+// run: sixteen-byte pieces in address order when the rows are consecutive (no work list), else 12-byte pieces
+// row after row through the lanes' row numbers. LDS operations of one wavefront execute in order, so no barrier
+// is involved. kPut: store or plain add (the atomic mode keeps the kernel above).
+constexpr int kShRow = 45;
+// piece e of a wavefront's 64 * 15 twelve-byte pieces lies in row e / 15 (the multiply-shift is exact below 960)
+__device__ __forceinline__ int sh_piece_row(int e) { return (int)(((uint32_t)e * 34953u) >> 19); }
+
+template <int kPut, bool kLens>
+__global__ __launch_bounds__(kProjBlock) void projection_bwd_staged_kernel(ssr_projection_bwd_params P) {
+    static_assert(kPut == kPutStore || kPut == kPutAdd, "atomic adds go element by element");
+    __shared__ __attribute__((aligned(16))) float s_sh[kProjBlock / 64][64 * kShRow];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float* my = s_sh[wave];
+    const int64_t n_rows = P.packed_gaussian_ids ? P.num_packed : (P.visible_ids ? P.n_visible : P.num_splats);
+    const int64_t i0 = (int64_t)blockIdx.x * kProjBlock + wave * 64;   // the wavefront's first work item
+    if (i0 >= n_rows) return;
+    const int64_t i = i0 + lane;
+    const bool in_range = i < n_rows;
+    const bool listed = P.packed_gaussian_ids || P.visible_ids;
+    const int64_t g = !in_range ? 0 : (P.packed_gaussian_ids ? (int64_t)P.packed_gaussian_ids[i] : (P.visible_ids ? (int64_t)P.visible_ids[i] : i));
+    const int64_t r = P.packed_gaussian_ids ? i : g;
+    float4 bb = make_float4(0.f, 0.f, 1.f, 1.f);
+    if (in_range && !P.packed_gaussian_ids) bb = reinterpret_cast<const float4*>(P.aabb)[g];
+    const bool valid = in_range && !(bb.z <= bb.x || bb.w <= bb.y);
+    ssr_world& V = P.v_world;
+    float* __restrict__ dst = V.features_sh;
+
+    // one splat per lane; its SH gradient row goes to LDS
+    float* mine = my + lane * kShRow;
+    WorldGradD wg;
+    if (valid) {
+        CamD cam = load_camera(P.camera);
+        cam.aa = P.antialiased != 0;
+        projection_vjp<3, kLens>(cam, P.world, P.sh, g, vscreen_of(P.v_screen, P.v_rows), r, wg, [&](int j, float Yj, const float vc[3]) {
+            const float tv[3] = {Yj * vc[0], Yj * vc[1], Yj * vc[2]};
+            const float d2 = dot3(tv, tv);
+            const bool ok = ssr_isfinite(d2) && d2 != 0.0f;   // harmonics.slang:397-403
+#pragma unroll
+            for (int c = 0; c < 3; c++) mine[3 * j + c] = ok ? tv[c] : 0.0f;
+        });
+    } else if (!listed) {
+        for (int k = 0; k < kShRow; k++) mine[k] = 0.0f;   // a culled row of a run that is written whole
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    // LDS -> the wavefront's gradient rows
+    if (!listed) {
+        const int count = (int)min((int64_t)64, n_rows - i0);   // rows of this wavefront
+        float4* __restrict__ d4 = reinterpret_cast<float4*>(dst + i0 * kShRow);
+        const int n4 = (count * kShRow) >> 2;   // whole pieces; at most three floats remain (a last, short wavefront)
+#pragma unroll
+        for (int t = 0; t < (64 * kShRow / 4 + 63) / 64; t++) {
+            const int e = t * 64 + lane;
+            if (e < n4) {
+                float4 v = reinterpret_cast<const float4*>(my)[e];
+                if (kPut == kPutAdd) { const float4 o = d4[e]; v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w; }
+                d4[e] = v;
+            }
+        }
+        if (lane < count * kShRow - 4 * n4) {
+            float* q = dst + i0 * kShRow + 4 * n4 + lane;
+            const float v = my[4 * n4 + lane];
+            *q = kPut == kPutAdd ? *q + v : v;
+        }
+    } else {
+        const int gl = valid ? (int)g : -1;
+#pragma unroll
+        for (int t = 0; t < kShRow / 3; t++) {
+            const int e = t * 64 + lane;
+            const int row = sh_piece_row(e), c3 = e - row * 15;
+            const int gr = __shfl(gl, row, 64);
+            if (gr >= 0) {
+                float* q = dst + (int64_t)gr * kShRow + 3 * c3;
+                const float* d = my + row * kShRow + 3 * c3;
+                if (kPut == kPutAdd) { q[0] += d[0]; q[1] += d[1]; q[2] += d[2]; }
+                else { q[0] = d[0]; q[1] = d[1]; q[2] = d[2]; }
+            }
+        }
+    }
+    // the other fourteen gradients, as in the kernel above
+    if (!valid) {
+        if (kPut == kPutStore && !listed && in_range) {
+#pragma unroll
+            for (int k = 0; k < 3; k++) { V.means[3 * g + k] = 0.f; V.log_scales[3 * g + k] = 0.f; V.features_dc[3 * g + k] = 0.f; }
+            *reinterpret_cast<float4*>(V.quats + 4 * g) = make_float4(0.f, 0.f, 0.f, 0.f);
+            V.opacity_logits[g] = 0.f;
+        }
+        return;
+    }
+#pragma unroll
+    for (int k = 0; k < 3; k++) put<kPut>(V.means + 3 * g + k, fin(wg.mean[k]));
+#pragma unroll
+    for (int k = 0; k < 4; k++) put<kPut>(V.quats + 4 * g + k, fin(wg.quat[k]));
+#pragma unroll
+    for (int k = 0; k < 3; k++) put<kPut>(V.log_scales + 3 * g + k, fin(wg.scale[k]));
+    put<kPut>(V.opacity_logits + g, fin(wg.logit));
+#pragma unroll
+    for (int k = 0; k < 3; k++) put<kPut>(V.features_dc + 3 * g + k, fin(wg.dc[k]));
+}
+
 // Camera-pose gradient: the same VJP once more, keeping only dL/dR and dL/dt, summed over the workgroup and added
 // to the 16-float view-matrix gradient with one atomic per entry and workgroup (the reference sums per warp,
 // ProjectionBwd_kernel.cuh:108-127).
@@ -1505,6 +1611,18 @@ extern "C" int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream
         default: hipLaunchKernelGGL((projection_bwd_kernel<D, kPutAtomic, L>), grid, block, 0, s, *p); break;             \
     }
 #define SSR_LAUNCH_BWD(D) if (lens) { SSR_LAUNCH_BWD_L(D, true) } else { SSR_LAUNCH_BWD_L(D, false) }
+    // degree 3 into gradient rows of 45 floats, 16-byte aligned: the kernel that stages those rows through LDS
+    const bool staged = p->sh_degree == 3 && v.sh_stride == kShRow && put_mode != kPutAtomic &&
+                        (reinterpret_cast<uintptr_t>(v.features_sh) & 15) == 0;
+    if (staged) {
+        if (put_mode == kPutStore) {
+            if (lens) hipLaunchKernelGGL((projection_bwd_staged_kernel<kPutStore, true>), grid, block, 0, s, *p);
+            else hipLaunchKernelGGL((projection_bwd_staged_kernel<kPutStore, false>), grid, block, 0, s, *p);
+        } else {
+            if (lens) hipLaunchKernelGGL((projection_bwd_staged_kernel<kPutAdd, true>), grid, block, 0, s, *p);
+            else hipLaunchKernelGGL((projection_bwd_staged_kernel<kPutAdd, false>), grid, block, 0, s, *p);
+        }
+    } else
     switch (p->sh_degree) {
         case 0: SSR_LAUNCH_BWD(0); break;
         case 1: SSR_LAUNCH_BWD(1); break;
