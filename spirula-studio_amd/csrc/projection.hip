@@ -429,13 +429,69 @@ __device__ __forceinline__ VScreenD vscreen_of(const ssr_screen& s, const float*
 // dL/dR and dL/dt of the world-to-camera transform, one splat's share
 struct PoseGradD { float R[3][3], t[3]; };
 
-template <int kDegree, bool kLens, bool kPose = false, class ShSink>
+template <int kDegree, bool kLens, bool kPose = false, bool kShFirst = false, class ShSink>
 __device__ __forceinline__ void projection_vjp(const CamD& cam, const ssr_world& W, const ssr_sh_quant& Q, int64_t g,
                                                const VScreenD& VS, int64_t r, WorldGradD& out, ShSink&& sh_sink,
                                                PoseGradD* pose = nullptr) {
     constexpr int kCoef = kDegree * (kDegree + 2);
     float mean[3], quat[4], ls[3], logit;
     load_splat(W, g, mean, quat, ls, logit);
+    float vc[3] = {0.f, 0.f, 0.f};
+    float vdir[3] = {0.f, 0.f, 0.f};
+    // (kShFirst: ahead of the geometry, whose live values then do not overlap the 45 coefficients)
+    auto sh_part = [&]() {
+        // SH colour VJP (src/shaders/harmonics.slang:373-649,1087-1126)
+        float coef[kCoef > 0 ? 3 * kCoef : 1];
+        if (kCoef > 0) decode_sh<kCoef>(W, Q, g, coef);
+        float dir[3];
+        view_dir(cam, mean, dir);
+        ShBasisD b;
+        sh_basis<kDegree>(dir, b);
+        const float* dcp = W.features_dc + 3 * g;
+        const float dc[3] = {dcp[0], dcp[1], dcp[2]};
+        float raw[3];
+        sh_color_raw<kDegree>(b, dc, coef, raw);
+        const float* vrg = VS.rgb + VS.s_rgb * r;
+    #pragma unroll
+        for (int c = 0; c < 3; c++) vc[c] = vrg[c] * (raw[c] >= -0.5f ? 1.0f : 0.0f);
+        if (kDegree >= 1) {
+    #pragma unroll
+            for (int j = 0; j < kCoef; j++) {
+                sh_sink(j, b.Y[j], vc);
+            }
+            // gY(j) = dL/dY_j. With Y(l, +-m) = A(z) {Re, Im} w^m, w = x + i y, and d w^m = m w^(m-1) dw:
+            //   dL/dx += m A (g_c Re w^(m-1) + g_s Im w^(m-1)),  dL/dy += m A (g_s Re w^(m-1) - g_c Im w^(m-1)),
+            //   dL/dz += A'(z) (g_c Re w^m + g_s Im w^m);        zonal terms B(z) add B'(z) g to dL/dz only.
+            auto gY = [&](int j) { return (coef[3 * j] * vc[0] + coef[3 * j + 1] * vc[1]) + coef[3 * j + 2] * vc[2]; };
+            const float X = b.x, Y = b.y, Z = b.z;
+            float vx = 0.0f, vy = 0.0f, vz = 0.0f;
+            auto order = [&](int m, float A, float dA, float gc, float gs) {
+                const float mA = (float)m * A;
+                vx += mA * (gc * b.re[m - 1] + gs * b.im[m - 1]);
+                vy += mA * (gs * b.re[m - 1] - gc * b.im[m - 1]);
+                vz += dA * (gc * b.re[m] + gs * b.im[m]);
+            };
+            order(1, -shk::k1, 0.0f, gY(2), gY(0));
+            vz += shk::k1 * gY(1);
+            if (kDegree >= 2) {
+                order(2, shk::k22, 0.0f, gY(7), gY(3));
+                order(1, -shk::k21 * Z, -shk::k21, gY(6), gY(4));
+                vz += (2.0f * shk::k20a * Z) * gY(5);
+                if (kDegree >= 3) {
+                    const float zz = Z * Z;
+                    order(3, -shk::k33, 0.0f, gY(14), gY(8));
+                    order(2, shk::k32 * Z, shk::k32, gY(13), gY(9));
+                    order(1, shk::k31b - shk::k31a * zz, -2.0f * shk::k31a * Z, gY(12), gY(10));
+                    vz += (3.0f * shk::k30a * zz - shk::k30b) * gY(11);
+                }
+            }
+            const float dn = (vx * X + vy * Y) + vz * Z;
+            vdir[0] = (vx - dn * X) * b.inorm;
+            vdir[1] = (vy - dn * Y) * b.inorm;
+            vdir[2] = (vz - dn * Z) * b.inorm;
+        }
+    };
+    if constexpr (kShFirst) sh_part();
     ProjD p;
     project<true, kLens>(cam, mean, quat, ls, logit, p);
     const float x = p.mc[0], y = p.mc[1], z = p.mc[2];
@@ -603,58 +659,7 @@ __device__ __forceinline__ void projection_vjp(const CamD& cam, const ssr_world&
     for (int i = 0; i < 4; i++) vquat[i] = (vqn[i] - p.qn[i] * qd) * p.qinv;
     const float vlogit = (VS.opac[VS.s_opac * r] * p.comp) * (p.sig * (1.0f - p.sig));
 
-    // SH colour VJP (src/shaders/harmonics.slang:373-649,1087-1126)
-    float coef[kCoef > 0 ? 3 * kCoef : 1];
-    if (kCoef > 0) decode_sh<kCoef>(W, Q, g, coef);
-    float dir[3];
-    view_dir(cam, mean, dir);
-    ShBasisD b;
-    sh_basis<kDegree>(dir, b);
-    const float* dcp = W.features_dc + 3 * g;
-    const float dc[3] = {dcp[0], dcp[1], dcp[2]};
-    float raw[3];
-    sh_color_raw<kDegree>(b, dc, coef, raw);
-    const float* vrg = VS.rgb + VS.s_rgb * r;
-    float vc[3];
-#pragma unroll
-    for (int c = 0; c < 3; c++) vc[c] = vrg[c] * (raw[c] >= -0.5f ? 1.0f : 0.0f);
-    float vdir[3] = {0.f, 0.f, 0.f};
-    if (kDegree >= 1) {
-#pragma unroll
-        for (int j = 0; j < kCoef; j++) {
-            sh_sink(j, b.Y[j], vc);
-        }
-        // gY(j) = dL/dY_j. With Y(l, +-m) = A(z) {Re, Im} w^m, w = x + i y, and d w^m = m w^(m-1) dw:
-        //   dL/dx += m A (g_c Re w^(m-1) + g_s Im w^(m-1)),  dL/dy += m A (g_s Re w^(m-1) - g_c Im w^(m-1)),
-        //   dL/dz += A'(z) (g_c Re w^m + g_s Im w^m);        zonal terms B(z) add B'(z) g to dL/dz only.
-        auto gY = [&](int j) { return (coef[3 * j] * vc[0] + coef[3 * j + 1] * vc[1]) + coef[3 * j + 2] * vc[2]; };
-        const float X = b.x, Y = b.y, Z = b.z;
-        float vx = 0.0f, vy = 0.0f, vz = 0.0f;
-        auto order = [&](int m, float A, float dA, float gc, float gs) {
-            const float mA = (float)m * A;
-            vx += mA * (gc * b.re[m - 1] + gs * b.im[m - 1]);
-            vy += mA * (gs * b.re[m - 1] - gc * b.im[m - 1]);
-            vz += dA * (gc * b.re[m] + gs * b.im[m]);
-        };
-        order(1, -shk::k1, 0.0f, gY(2), gY(0));
-        vz += shk::k1 * gY(1);
-        if (kDegree >= 2) {
-            order(2, shk::k22, 0.0f, gY(7), gY(3));
-            order(1, -shk::k21 * Z, -shk::k21, gY(6), gY(4));
-            vz += (2.0f * shk::k20a * Z) * gY(5);
-            if (kDegree >= 3) {
-                const float zz = Z * Z;
-                order(3, -shk::k33, 0.0f, gY(14), gY(8));
-                order(2, shk::k32 * Z, shk::k32, gY(13), gY(9));
-                order(1, shk::k31b - shk::k31a * zz, -2.0f * shk::k31a * Z, gY(12), gY(10));
-                vz += (3.0f * shk::k30a * zz - shk::k30b) * gY(11);
-            }
-        }
-        const float dn = (vx * X + vy * Y) + vz * Z;
-        vdir[0] = (vx - dn * X) * b.inorm;
-        vdir[1] = (vy - dn * Y) * b.inorm;
-        vdir[2] = (vz - dn * Z) * b.inorm;
-    }
+    if constexpr (!kShFirst) sh_part();
 #pragma unroll
     for (int i = 0; i < 3; i++) { out.mean[i] = vmean[i] + vdir[i]; out.scale[i] = vscale[i]; out.dc[i] = 0.2820947917738781f * vc[i]; }
 #pragma unroll
@@ -776,7 +781,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_staged_kernel(ssr_p
     if (valid) {
         CamD cam = load_camera(P.camera);
         cam.aa = P.antialiased != 0;
-        projection_vjp<3, kLens>(cam, P.world, P.sh, g, vscreen_of(P.v_screen, P.v_rows), r, wg, [&](int j, float Yj, const float vc[3]) {
+        projection_vjp<3, kLens, false, true>(cam, P.world, P.sh, g, vscreen_of(P.v_screen, P.v_rows), r, wg, [&](int j, float Yj, const float vc[3]) {
             const float tv[3] = {Yj * vc[0], Yj * vc[1], Yj * vc[2]};
             const float d2 = dot3(tv, tv);
             const bool ok = ssr_isfinite(d2) && d2 != 0.0f;   // harmonics.slang:397-403
