@@ -397,8 +397,10 @@ class GpuRun:
             for k, sl in [("v_xy", slice(0, 2)), ("v_depth", 2), ("v_conic", slice(3, 6)), ("v_opac", 6), ("v_rgb", slice(7, 10))]:
                 self.d[k] = D.from_host(np.ascontiguousarray(rows[:, sl]))
 
-    def projection_bwd(self, accumulate=True, poison=False, pose=False):
-        """pose=True: also the camera-pose gradient, read back with host("v_viewmat") as [4,4]."""
+    def projection_bwd(self, accumulate=True, poison=False, pose=False, misalign_sh_rows=False):
+        """pose=True: also the camera-pose gradient, read back with host("v_viewmat") as [4,4].
+        misalign_sh_rows: the SH gradient rows start 4 bytes into their buffer, which takes the launcher off the
+        kernel that stages them through LDS (it needs 16-byte alignment); read back with sh_rows_misaligned()."""
         D = self.L.DeviceArray
         n = self.n
         for k, shape in [("w_means", (n, 3)), ("w_quats", (n, 4)), ("w_log_scales", (n, 3)),
@@ -429,7 +431,18 @@ class GpuRun:
                 return
             p.aabb = None
             p.packed_gaussian_ids, p.num_packed = self.ptr("gaussian_ids"), self.rows
+        if misalign_sh_rows:
+            raw = D((n * 45 + 4,), np.float32)
+            if poison:
+                self.check(self.lib.ssr_fill_u32(raw.ptr, 0x7fc00000, n * 45 + 4, None))
+            else:
+                raw.fill_zero()
+            self.d["w_features_sh_raw"] = raw
+            p.v_world.features_sh = raw.ptr + 4
         self.check(self.lib.ssr_projection_bwd(C.byref(p), None))
+
+    def sh_rows_misaligned(self):
+        return self.d["w_features_sh_raw"].to_host()[1:1 + self.n * 45].reshape(self.n, 15, 3)
 
     def fused_optimizer(self, g1, g2, hyper, step=1, steps=None, v_in=None, scale_agnostic=False, quant_state=None, non_sh=None):
         """ssr_fused_projection_bwd_optimizer on the device copies of the parameters (fp32 SH);

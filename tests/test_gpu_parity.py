@@ -404,6 +404,29 @@ def test_empty_and_culled(gpu, oracle):
     assert np.all(g.host("r_T") == 1.0)
 
 
+@pytest.mark.parametrize("use_list,accumulate", [(False, False), (True, False), (False, True), (True, True)])
+def test_projection_backward_staged_rows_equal_plain_rows(gpu, oracle, use_list, accumulate):
+    """The projection backward that moves its SH gradient rows through LDS (16-byte aligned rows of 45 floats,
+    degree 3) and the one-thread-per-row kernel it stands in for give the same rows bit for bit: stored or added,
+    with and without a work list, culled rows zeroed or left alone alike."""
+    sc = gpu.scenes.make_scene(2, n=20011, width=480, height=270)   # the last wavefront is short
+    sc.means[::5, 2] = -20.0                                         # culled rows among the visible ones
+    g = GpuRun(gpu, sc, use_list=use_list, use_vrows=True)
+    g.run_all(backward=False, fused_count=True)
+    g.raster_bwd()
+    g.projection_bwd(accumulate=accumulate, poison=not accumulate)
+    staged = g.host("w_features_sh").copy()
+    others = {k: g.host(k).copy() for k in ["w_means", "w_quats", "w_log_scales", "w_opacity_logits", "w_features_dc"]}
+    g.projection_bwd(accumulate=accumulate, poison=not accumulate, misalign_sh_rows=True)
+    plain = g.sh_rows_misaligned()
+    assert np.array_equal(staged.view(np.uint32), plain.view(np.uint32))
+    aabb = g.host("aabb")
+    vis = aabb[:, 2] > aabb[:, 0]
+    assert 1000 < vis.sum() < sc.n - 1000 and np.any(staged[vis] != 0) and np.isfinite(staged[vis]).all()
+    for k, v in others.items():
+        assert np.array_equal(g.host(k).view(np.uint32), v.view(np.uint32)), k
+
+
 def test_packed_projection_tiny(gpu, oracle):
     """projection_3dgs_packed_forward: compacted rows in ascending splat order, then the whole chain."""
     _compare_packed(gpu, oracle, gpu.scenes.tiny_scene(n=700, width=96, height=64, seed=21), "pk-tiny")
