@@ -689,8 +689,8 @@ def test_runtime_contract(pkg, H):
     L.ssr_device_free(d); L.ssr_device_free(d2); L.ssr_host_free_pinned(p)
 
 
-@pytest.mark.parametrize("native", [False, True])
-def test_engine_two_cameras(pkg, oracle, H, native):
+@pytest.mark.parametrize("native,deferred", [(False, False), (True, False), (True, True)])
+def test_engine_two_cameras(pkg, oracle, H, native, deferred):
     """[C = 2] viewmats through the adapter (the reference's entry points take [C,4,4] cameras and render C
     images in one pass: ProjectionFwd_kernel.cuh:60-110, IntersectTile.cu:215-262, RasterizationFwd.cu grid
     {C, tile_h, tile_w}). Against the oracle run once per camera: image c's keys carry tile ids offset by
@@ -724,17 +724,20 @@ def test_engine_two_cameras(pkg, oracle, H, native):
     both.viewmat = np.stack([c[0] for c in cams])
     both.intrins = np.stack([c[1] for c in cams])
     both.v_rgb, both.v_depth, both.v_T = v_rgb, v_depth, v_T
+    # deferred: the second pass leaves the intersection count on the device (arrays sized from the first pass)
     eng = host.Engine(both, fuse_tile_count=native, visible_list=native, packed_rows=native, overwrite_world_grads=native,
-                      packed_vscreen=native, tile_sort=native)
+                      packed_vscreen=native, tile_sort=native, deferred_counts=deferred)
     tiles = ((w + 15) // 16) * ((h + 15) // 16)
     for rep in range(2):   # the second pass: zero-fills honoured, nothing accumulates
         eng.forward()
         got_pose = eng.backward_with_pose_grad().astype(np.float64)
         n0 = refs[0]["sorted_ids"].size
-        assert eng.n_isects == n0 + refs[1]["sorted_ids"].size
-        assert np.array_equal(eng.cache("sorted_ids"),
+        K = n0 + refs[1]["sorted_ids"].size
+        assert eng.n_isects == K
+        assert eng.cache("sorted_ids").size == (K + K // 16 + 65536 if deferred and rep else K)
+        assert np.array_equal(eng.cache("sorted_ids")[:K],
                               np.concatenate([refs[0]["sorted_ids"], refs[1]["sorted_ids"] + (np.int64(tiles) << 32)]))
-        assert np.array_equal(eng.cache("sorted_flat"), np.concatenate([refs[0]["sorted_flat"], refs[1]["sorted_flat"] + n]))
+        assert np.array_equal(eng.cache("sorted_flat")[:K], np.concatenate([refs[0]["sorted_flat"], refs[1]["sorted_flat"] + n]))
         assert np.array_equal(eng.cache("offsets"),
                               np.concatenate([refs[0]["offsets"].reshape(-1), refs[1]["offsets"].reshape(-1) + n0]))
         assert np.array_equal(eng.cache("aabb").reshape(2, n, 4), np.stack([r["proj"]["aabb"] for r in refs]))
