@@ -226,13 +226,17 @@ __device__ __forceinline__ int64_t block_exclusive_scan(int64_t v, int64_t& tota
     return base + inc - v;
 }
 
+// Item layout of the two passes over the data: a wavefront owns 8 x 64 consecutive items and reads them in eight
+// rounds, lane l taking item 64 r + l of its run, so that every load and store instruction covers one contiguous
+// 512 bytes (eight consecutive items per THREAD made each instruction touch 64 cache lines).
 __global__ __launch_bounds__(kScanBlock) void scan_reduce_kernel(const int64_t* __restrict__ in, int64_t n,
                                                                  int64_t* __restrict__ block_sums) {
     __shared__ int64_t lds[4];
-    const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)wave * (64 * kScanItems) + lane;
     int64_t s = 0;
 #pragma unroll
-    for (int i = 0; i < kScanItems; i++) { if (base + i < n) s += in[base + i]; }
+    for (int r = 0; r < kScanItems; r++) { if (base + 64 * r < n) s += in[base + 64 * r]; }
     int64_t total;
     block_exclusive_scan(s, total, lds);
     if (threadIdx.x == 0) block_sums[blockIdx.x] = total;
@@ -255,20 +259,30 @@ __global__ __launch_bounds__(kScanBlock) void scan_down_kernel(const int64_t* __
                                                                const int64_t* __restrict__ block_prefix,
                                                                int64_t* __restrict__ out, int64_t* __restrict__ total_out) {
     __shared__ int64_t lds[4];
-    const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)wave * (64 * kScanItems) + lane;
     int64_t v[kScanItems];
     int64_t s = 0;
 #pragma unroll
-    for (int i = 0; i < kScanItems; i++) { v[i] = base + i < n ? in[base + i] : 0; s += v[i]; }
-    int64_t total;
-    int64_t run = block_prefix[blockIdx.x] + block_exclusive_scan(s, total, lds);
+    for (int r = 0; r < kScanItems; r++) { v[r] = base + 64 * r < n ? in[base + 64 * r] : 0; s += v[r]; }
+    // what lies before this wavefront's run: the workgroup's prefix and the wavefronts before it
+    int64_t w = s;
 #pragma unroll
-    for (int i = 0; i < kScanItems; i++) {
-        run += v[i];
-        if (base + i < n) {
-            out[base + i] = run;
-            if (total_out && base + i == n - 1) *total_out = run;
+    for (int d = 32; d >= 1; d >>= 1) w += __shfl_xor(w, d, 64);
+    if (lane == 0) lds[wave] = w;
+    __syncthreads();
+    int64_t carry = block_prefix[blockIdx.x];
+#pragma unroll
+    for (int k = 0; k < kScanBlock / 64; k++) { if (k < wave) carry += lds[k]; }
+    // the run itself: an inclusive scan of each round of 64 items on top of the rounds before it
+#pragma unroll
+    for (int r = 0; r < kScanItems; r++) {
+        const int64_t inc = carry + wave_inclusive_scan(v[r], lane);
+        if (base + 64 * r < n) {
+            out[base + 64 * r] = inc;
+            if (total_out && base + 64 * r == n - 1) *total_out = inc;
         }
+        carry = __shfl(inc, 63, 64);
     }
 }
 
