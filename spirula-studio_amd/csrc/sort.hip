@@ -538,8 +538,11 @@ static int sort_pairs_impl(int64_t* keys_a, int64_t* keys_b, int32_t* vals_a, in
     uint64_t* k[2] = {reinterpret_cast<uint64_t*>(keys_a), reinterpret_cast<uint64_t*>(keys_b)};
     int32_t* v[2] = {vals_a, vals_b};
     int cur = 0;
-    for (int shift = begin_bit; shift < end_bit; shift += 8) {
-        const int bits = end_bit - shift < 8 ? end_bit - shift : 8;
+    // as few passes as 8-bit digits allow, the bits spread evenly over them (13 tile bits: 7 + 6, not 8 + 5): the
+    // scatter of a narrower digit writes longer runs, and no pass is left with the short runs of a full 256-way split
+    int passes = (end_bit - begin_bit + 7) / 8;
+    for (int shift = begin_bit, bits = 0; shift < end_bit; shift += bits, passes--) {
+        bits = (end_bit - shift + passes - 1) / passes;
         const uint32_t mask = (1u << bits) - 1u;
         hipLaunchKernelGGL(sort_hist_kernel, dim3(nb), dim3(kSortBlock), 0, s, k[cur], n, n_dev, shift, mask, nb, hist,
                            shift == begin_bit ? clear4 : nullptr);
