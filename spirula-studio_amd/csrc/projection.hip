@@ -149,7 +149,9 @@ __device__ __forceinline__ void sh_colour(const ssr_world& W, const ssr_sh_quant
 // ---- packed form -------------------------------------------------------------------------------
 // Staging area of the packed projection inside the caller's scratch buffer: per-workgroup visible
 // counts, their exclusive scan, and the geometry of the visible splats compacted within each
-// workgroup's own 256-row segment (structure of arrays, so both passes access it coalesced).
+// workgroup's own segment of kPackSeg rows (structure of arrays, so both passes access it coalesced).
+constexpr int kPackPer = 4;                       // splats per thread of the mask kernel
+constexpr int kPackSeg = kProjBlock * kPackPer;   // splats per workgroup of the mask kernel = rows of its segment
 struct PackedStage {
     int32_t* block_counts;    // [nb]
     int64_t* block_offsets;   // [nb + 1], block_offsets[nb] = nnz
@@ -165,7 +167,7 @@ struct PackedStage {
 __host__ __device__ inline size_t align16(size_t b) { return (b + 15) & ~(size_t)15; }
 
 inline size_t packed_stage_layout(int64_t n, void* base, PackedStage* st) {
-    const size_t nb = (size_t)ceil_div(n, kProjBlock), N = (size_t)n;
+    const size_t nb = (size_t)ceil_div(n, kPackSeg), N = (size_t)n;
     char* p = static_cast<char*>(base);
     size_t off = 0;
     auto take = [&](size_t bytes) { char* r = p ? p + off : nullptr; off += align16(bytes); return r; };
@@ -189,9 +191,9 @@ inline size_t packed_stage_layout(int64_t n, void* base, PackedStage* st) {
 // workgroup's segment of the staging area (ballot ranks inside a wavefront, wavefront totals through
 // LDS), so that the second pass never touches a culled splat.
 // A pinhole view is sparse when the camera stands inside the scene, and this kernel is bound by the projection's
-// arithmetic, not by memory: so a first pass reads only the mean and the scales, rejects what is certainly
-// behind the camera or off the image, and, when under five eighths of the workgroup's splats remain, compacts
-// them in splat order so that the projection runs on dense wavefronts. The test is one-sided: z <= 0 is the
+// arithmetic, not by memory: so a first pass over the workgroup's 1024 splats, four per thread, reads only the
+// mean and the scales and rejects what is certainly behind the camera or off the image; the rest are listed in
+// splat order and projected 256 at a time, on dense wavefronts. The test is one-sided: z <= 0 is the
 // projection's own rule on the identically computed z; the screen radius is bounded by
 // 3.33 sqrt(s_max^2 |J row|^2 + blur) with |J row|^2 <= (f^2 + L^2) / z^2, L the clamp of J[.][2]
 // (clamp_pinhole_jacobian), enlarged by 1 % and a pixel, so whatever is rejected here the projection's
@@ -209,72 +211,91 @@ __device__ __forceinline__ bool pinhole_may_be_visible(const CamD& cam, const ss
     const float smax = __builtin_amdgcn_exp2f(ssr_max(sc[0], ssr_max(sc[1], sc[2])) * 1.44269504f) * 1.001f;   // hardware exp2, an ulp off at most
     const float lim_pos = cam.Wf + 0.3f * (0.5f * cam.Wf), lim_neg = 0.3f * (0.5f * cam.Wf);
     const float Lx = ssr_max(lim_pos - cam.cx, lim_neg + cam.cx), Ly = ssr_max(lim_pos - cam.cy, lim_neg + cam.cy);
-    const float rz = 1.0f / z, sz = smax * rz;
-    const float Rx = 3.33f * 1.01f * ssr_sqrt((sz * sz) * (cam.fx * cam.fx + Lx * Lx) + 0.3f) + 1.0f;
-    const float Ry = 3.33f * 1.01f * ssr_sqrt((sz * sz) * (cam.fy * cam.fy + Ly * Ly) + 0.3f) + 1.0f;
+    // hardware reciprocal and square root (an ulp off): the 1 % and the pixel cover them
+    const float rz = __builtin_amdgcn_rcpf(z), sz = smax * rz;
+    const float Rx = 3.33f * 1.01f * __builtin_amdgcn_sqrtf((sz * sz) * (cam.fx * cam.fx + Lx * Lx) + 0.3f) + 1.0f;
+    const float Ry = 3.33f * 1.01f * __builtin_amdgcn_sqrtf((sz * sz) * (cam.fy * cam.fy + Ly * Ly) + 0.3f) + 1.0f;
     const float u = cam.fx * (mc[0] * rz) + cam.cx, v = cam.fy * (mc[1] * rz) + cam.cy;
     return !(u + Rx < 0.0f || u - Rx > cam.Wf || v + Ry < 0.0f || v - Ry > cam.Hf);
 }
 
 template <bool kLens>
 __global__ __launch_bounds__(kProjBlock) void projection_packed_mask_kernel(ssr_projection_packed_params P, PackedStage S) {
-    __shared__ int s_wave[kProjBlock / 64];
+    __shared__ int s_pre[kPackPer * (kProjBlock / 64)];   // candidates per (slice, wavefront)
+    __shared__ uint16_t s_cand[kPackSeg];                 // the candidates' offsets in the segment, in splat order
+    __shared__ int s_wave[2][kProjBlock / 64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int64_t block0 = (int64_t)blockIdx.x * kProjBlock;
-    int64_t g = block0 + threadIdx.x;
+    const int64_t block0 = (int64_t)blockIdx.x * kPackSeg;
+    const int n_here = (int)min((int64_t)kPackSeg, P.num_splats - block0);
     CamD cam = load_camera(P.camera);
     cam.aa = P.antialiased != 0;
-    bool work = g < P.num_splats;
-    if (!kLens && cam.model == SSR_CAM_PINHOLE) {
-        __shared__ int s_pre[kProjBlock / 64];
-        __shared__ int s_cand[kProjBlock];
-        const bool keep = work && pinhole_may_be_visible(cam, P.world, g);
-        const unsigned long long km = __ballot(keep);
-        if (lane == 0) s_pre[wave] = __popcll(km);
-        __syncthreads();
-        int kbase = 0, ktotal = 0;
+    const bool pretest = !kLens && cam.model == SSR_CAM_PINHOLE;
+    // 1. candidates: slice k of the segment is splats k * 256 .. k * 256 + 255, one per thread
+    unsigned long long km[kPackPer];
 #pragma unroll
-        for (int w = 0; w < kProjBlock / 64; w++) { if (w < wave) kbase += s_pre[w]; ktotal += s_pre[w]; }
-        work = keep;
-        if (ktotal * 8 <= kProjBlock * 5) {   // the same for the whole workgroup
-            if (keep) s_cand[kbase + __popcll(km & ((1ull << lane) - 1ull))] = threadIdx.x;
-            __syncthreads();
-            work = (int)threadIdx.x < ktotal;   // candidates stay in splat order, so the ranks below do too
-            if (work) g = block0 + s_cand[threadIdx.x];
-        }
+    for (int k = 0; k < kPackPer; k++) {
+        const int off = k * kProjBlock + (int)threadIdx.x;
+        const bool keep = off < n_here && (!pretest || pinhole_may_be_visible(cam, P.world, block0 + off));
+        km[k] = __ballot(keep);
+        if (lane == 0) s_pre[k * (kProjBlock / 64) + wave] = __popcll(km[k]);
     }
-    bool vis = false;
-    ProjD p;
-    float bb[4] = {0.f, 0.f, 0.f, 0.f};
-    if (work) {
-        float mean[3], quat[4], ls[3], logit;
-        load_splat(P.world, g, mean, quat, ls, logit);
-        project<false, kLens>(cam, mean, quat, ls, logit, p);
-        bb[0] = ssr_min(ssr_max(p.aabb[0], 0.0f), cam.Wf - 1.0f);
-        bb[1] = ssr_min(ssr_max(p.aabb[1], 0.0f), cam.Hf - 1.0f);
-        bb[2] = ssr_min(ssr_max(p.aabb[2], 0.0f), cam.Wf - 1.0f);
-        bb[3] = ssr_min(ssr_max(p.aabb[3], 0.0f), cam.Hf - 1.0f);
-        vis = bb[2] - bb[0] > 1e-3f && bb[3] - bb[1] > 1e-3f;   // ProjectionPackedFwd_kernel.cuh:93
-    }
-    const unsigned long long m = __ballot(vis);
-    const int rank = __popcll(m & ((1ull << lane) - 1ull));
-    if (lane == 0) s_wave[wave] = __popcll(m);
     __syncthreads();
-    int base = 0, total = 0;
+    int n_cand = 0;
 #pragma unroll
-    for (int w = 0; w < kProjBlock / 64; w++) { if (w < wave) base += s_wave[w]; total += s_wave[w]; }
-    if (threadIdx.x == 0) S.block_counts[blockIdx.x] = total;
-    if (!vis) return;
-    const int64_t d = block0 + base + rank;
+    for (int k = 0; k < kPackPer; k++) {
+        int before = n_cand;   // the slices before this one
+#pragma unroll
+        for (int w = 0; w < kProjBlock / 64; w++) {
+            const int c = s_pre[k * (kProjBlock / 64) + w];
+            if (w < wave) before += c;
+            n_cand += c;
+        }
+        if ((km[k] >> lane) & 1ull)
+            s_cand[before + __popcll(km[k] & ((1ull << lane) - 1ull))] = (uint16_t)(k * kProjBlock + (int)threadIdx.x);
+    }
+    __syncthreads();
+    // 2. the projection, 256 candidates a round; rounds and ranks keep the splat order
     const int64_t N = P.num_splats;
-    S.aabb[d] = make_float4(bb[0], bb[1], bb[2], bb[3]);
-    S.xy[d] = make_float2(p.xy[0], p.xy[1]);
-    S.conic[d] = p.conic[0]; S.conic[N + d] = p.conic[1]; S.conic[2 * N + d] = p.conic[2];
-    S.sort_depth[d] = p.sort_depth;
-    S.depth[d] = p.depth;
-    S.opac[d] = p.opac;
-    S.gid[d] = (int32_t)g;
-    atomic_max_nonneg(P.radii + g, p.radius);   // ProjectionPackedFwd_kernel.cuh:183
+    int n_out = 0;
+    for (int c0 = 0; c0 < n_cand; c0 += kProjBlock) {
+        const int c = c0 + (int)threadIdx.x;
+        bool vis = false;
+        ProjD p;
+        float bb[4] = {0.f, 0.f, 0.f, 0.f};
+        int64_t g = 0;
+        if (c < n_cand) {
+            g = block0 + s_cand[c];
+            float mean[3], quat[4], ls[3], logit;
+            load_splat(P.world, g, mean, quat, ls, logit);
+            project<false, kLens>(cam, mean, quat, ls, logit, p);
+            bb[0] = ssr_min(ssr_max(p.aabb[0], 0.0f), cam.Wf - 1.0f);
+            bb[1] = ssr_min(ssr_max(p.aabb[1], 0.0f), cam.Hf - 1.0f);
+            bb[2] = ssr_min(ssr_max(p.aabb[2], 0.0f), cam.Wf - 1.0f);
+            bb[3] = ssr_min(ssr_max(p.aabb[3], 0.0f), cam.Hf - 1.0f);
+            vis = bb[2] - bb[0] > 1e-3f && bb[3] - bb[1] > 1e-3f;   // ProjectionPackedFwd_kernel.cuh:93
+        }
+        const unsigned long long m = __ballot(vis);
+        const int rank = __popcll(m & ((1ull << lane) - 1ull));
+        int* totals = s_wave[(c0 / kProjBlock) & 1];   // two sets in turn: one barrier a round is enough
+        if (lane == 0) totals[wave] = __popcll(m);
+        __syncthreads();
+        int base = 0, total = 0;
+#pragma unroll
+        for (int w = 0; w < kProjBlock / 64; w++) { if (w < wave) base += totals[w]; total += totals[w]; }
+        if (vis) {
+            const int64_t d = block0 + n_out + base + rank;
+            S.aabb[d] = make_float4(bb[0], bb[1], bb[2], bb[3]);
+            S.xy[d] = make_float2(p.xy[0], p.xy[1]);
+            S.conic[d] = p.conic[0]; S.conic[N + d] = p.conic[1]; S.conic[2 * N + d] = p.conic[2];
+            S.sort_depth[d] = p.sort_depth;
+            S.depth[d] = p.depth;
+            S.opac[d] = p.opac;
+            S.gid[d] = (int32_t)g;
+            atomic_max_nonneg(P.radii + g, p.radius);   // ProjectionPackedFwd_kernel.cuh:183
+        }
+        n_out += total;
+    }
+    if (threadIdx.x == 0) S.block_counts[blockIdx.x] = n_out;
 }
 
 // Exclusive scan of the workgroup counts by ONE workgroup (the counts are N/256 values, 39k for ten million
@@ -348,7 +369,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_packed_emit_kernel(ssr_
     const int64_t nnz = *P.nnz < P.max_rows ? *P.nnz : P.max_rows;
     const int64_t j0 = (int64_t)blockIdx.x * kProjBlock;
     if (j0 >= nnz) return;
-    const int64_t nb = (P.num_splats + kProjBlock - 1) / kProjBlock;
+    const int64_t nb = (P.num_splats + kPackSeg - 1) / kPackSeg;
     const int64_t j1 = j0 + kProjBlock - 1 < nnz - 1 ? j0 + kProjBlock - 1 : nnz - 1;
     int64_t lo = last_block_at_or_before(S.block_offsets, nb, j0);
     int64_t hi = last_block_at_or_before(S.block_offsets, nb, j1) + 1;
@@ -358,7 +379,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_packed_emit_kernel(ssr_
         const int64_t mid = (lo + hi) >> 1;
         if (S.block_offsets[mid] <= j) lo = mid; else hi = mid;
     }
-    const int64_t src = lo * kProjBlock + (j - S.block_offsets[lo]);
+    const int64_t src = lo * kPackSeg + (j - S.block_offsets[lo]);
     const int64_t N = P.num_splats;
     CamD cam = load_camera(P.camera);
     cam.aa = P.antialiased != 0;
@@ -1540,7 +1561,7 @@ extern "C" int ssr_projection_packed_mask(const ssr_projection_packed_params* p,
     SSR_REQUIRE(p->radii, where, "null radii");
     PackedStage st;
     packed_stage_layout(p->num_splats, p->scratch, &st);
-    const int64_t nb = ceil_div(p->num_splats, kProjBlock);
+    const int64_t nb = ceil_div(p->num_splats, kPackSeg);
     if (camera_needs_lens_path(p->camera.camera_model, p->camera.distortion))
         hipLaunchKernelGGL(projection_packed_mask_kernel<true>, dim3((unsigned)nb), dim3(kProjBlock), 0, s, *p, st);
     else
