@@ -144,6 +144,9 @@ def main():
     ap.add_argument("--dist-type", type=int, default=0, help="compositing variant: 1 depth distortion, 2 rgb + depth distortion")
     ap.add_argument("--median", action="store_true", help="compositing variant: also render the median depth and back-propagate it")
     ap.add_argument("--accum-mode", type=int, default=0, help="compositing variant: accumulate a pixel weight map per splat (1 max, 2 sum, 3 avg)")
+    ap.add_argument("--packed-world-rows", action="store_true",
+                    help="with the packed projection: keep the visible splats' parameters (64 bytes each) for the projection backward")
+    ap.add_argument("--no-packed-world-rows", action="store_true", help="config 4: gather the parameters in the projection backward")
     ap.add_argument("--deferred-counts", action="store_true",
                     help="after the first iteration the forward does not wait for the intersection count: key arrays sized "
                          "from the previous count, overflow checked before the backward uses the counts")
@@ -179,6 +182,9 @@ def main():
     # nnz-row outputs) is its mode for such views and the faster one here, so it is this config's default
     if cfg == 4 and not (args.dense_projection or args.reference_order or args.cameras > 1):
         args.packed_projection = True
+        # ... and its visible splats are scattered over the parameter arrays: the packed projection keeps their
+        # parameters for the projection backward (not with the fused optimizer, which reads them where they live)
+        args.packed_world_rows = not (args.fused_optimizer or args.no_packed_world_rows)
     t_gen = time.time()
     sc = pkg.scenes.make_scene(cfg, n=args.n)
     if args.fused_optimizer and args.quantization_level == 1:
@@ -212,7 +218,8 @@ def main():
     native = not args.reference_order
     eng = host.Engine(sc, fuse_tile_count=native, visible_list=native and not args.packed_projection, packed_rows=native,
                       overwrite_world_grads=native, packed_projection=args.packed_projection, packed_vscreen=native,
-                      tile_sort=native and not args.whole_key_sort, deferred_counts=args.deferred_counts)
+                      tile_sort=native and not args.whole_key_sort, deferred_counts=args.deferred_counts,
+                      packed_world_rows=args.packed_world_rows)
     L = lib.load()
 
     hyper = dict(lr_means=1.6e-6, lr_quats=1e-5, lr_scales=5e-5, lr_opacs=5e-4, lr_features_dc=2.5e-5, lr_features_sh=1.25e-6)
@@ -311,7 +318,8 @@ def main():
     valu_inst = None     # profiled VALU wavefront instructions per launch of the dominant kernel
     prof = {}
     # the profiles were taken with this script's default arguments for each config: they describe no other variant
-    default_run = (native and ncam == 1 and tile_sort and args.packed_projection == (cfg == 4) and not args.n and
+    default_run = (native and ncam == 1 and tile_sort and args.packed_projection == (cfg == 4) and
+                   args.packed_world_rows == (cfg == 4) and not args.n and
                    not (variants or args.fused_optimizer or args.lens != "none" or args.fisheye or args.mip))
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if default_run and os.path.exists(tpath):
@@ -353,6 +361,7 @@ def main():
                                   + (", antialiased (mip) primitive" if args.mip else "")
                                   + (f", {ncam} cameras per iteration in one call" if ncam > 1 else "")
                                   + (", packed projection outputs" if args.packed_projection else "")
+                                  + (", parameter rows of the visible splats kept for the projection backward" if args.packed_world_rows else "")
                                   + (", projection backward fused with Adam" + ((" (quantized SH state" + (" and non-SH moments)" if args.non_sh_optim_bits == 16 else ")")) if args.quantization_level else "")
                                      if args.fused_optimizer else "")
                                   + (f", compositing variants dist_type={args.dist_type} median={int(args.median)} accum_mode={args.accum_mode}" if variants else "")

@@ -135,7 +135,7 @@ int ssr_projection_fwd(const ssr_projection_fwd_params* p, ssr_stream_t stream);
  * splat, in ascending splat order: camera_ids / gaussian_ids / aabb / sort_depth / screen, nnz rows.
  * The reference runs mask -> inclusive scan -> blocking readback of nnz -> a second full projection
  * that writes the compacted rows. Here the first call projects every splat once, compacts the
- * visible ones inside each 256-splat workgroup into `scratch`, and scans the workgroup counts into
+ * visible ones inside each workgroup's 1024-splat segment of `scratch`, and scans the workgroup counts into
  * *nnz; the second call evaluates SH colour for the nnz staged rows and places them. Between the
  * two the caller may read *nnz back (ssr_read_i64) to size its outputs, or skip the readback and
  * pass capacity num_splats as max_rows. Rows past *nnz are not written. radii is max-accumulated
@@ -166,8 +166,20 @@ typedef struct {
      * camera, each emit writing its rows behind the previous camera's, so that the rows are ordered by
      * (camera, splat) as the reference's single scan over C * N leaves them (ProjectionPackedFwd.cu:64-158). */
     int32_t camera_index;
+    /* Optional [4][world_rows_stride][4], 16-byte aligned: the parameters of each visible splat in the order of the
+     * packed rows, as four planes of 16-byte entries, (mean.xyz, opacity logit), (quat wxyz), (log_scale.xyz, dc.r),
+     * (dc.g, dc.b, 0, 0); entry i of every plane belongs to packed row i, world_rows_stride >= max_rows. Where a
+     * view sees a small, scattered part of the splats, ssr_projection_bwd reads these planes, consecutive lanes
+     * consecutive entries, instead of gathering 4- to 16-byte pieces of five arrays, one cache line each
+     * (ssr_projection_bwd_params::packed_world_rows). The mask call stages them when stage_world_rows is non-zero (the row count, and with it
+     * this array, is not known before); both calls then need stage_world_rows set and a scratch of
+     * ssr_projection_packed_scratch_bytes_world_rows(num_splats) bytes. No counterpart in the reference. */
+    float* world_rows;
+    int64_t world_rows_stride;
+    int32_t stage_world_rows;
 } ssr_projection_packed_params;
 size_t ssr_projection_packed_scratch_bytes(int64_t num_splats);
+size_t ssr_projection_packed_scratch_bytes_world_rows(int64_t num_splats);   /* with world_rows: 48 bytes per splat more */
 int ssr_projection_packed_mask(const ssr_projection_packed_params* p, ssr_stream_t stream);
 int ssr_projection_packed_emit(const ssr_projection_packed_params* p, ssr_stream_t stream);
 
@@ -422,6 +434,13 @@ typedef struct {
      * default) adds atomically, as the reference does, so that lists holding several cameras' rows
      * stay correct. Store mode (accumulate == 0) always needs unique ids. */
     int32_t packed_ids_unique;
+    /* Packed mode, optional [4][packed_world_stride][4]: the planes ssr_projection_packed_emit wrote into world_rows
+     * for these same packed rows (entry i of each plane = packed row i; packed_world_stride = its
+     * world_rows_stride). The parameters of row i are then read from here, not from `world` at
+     * packed_gaussian_ids[i] (the SH coefficients still are): the caller vouches that `world` has not changed
+     * since that projection. 16-byte aligned. */
+    const float* packed_world_rows;
+    int64_t packed_world_stride;
 } ssr_projection_bwd_params;
 int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream_t stream);
 

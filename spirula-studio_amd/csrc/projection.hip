@@ -42,7 +42,8 @@ __device__ __forceinline__ void atomic_max_nonneg(float* p, float v) {
 
 template <int kDegree>
 __device__ __forceinline__ void sh_colour(const ssr_world& W, const ssr_sh_quant& Q, const CamD& cam, int64_t g,
-                                          float* rgb_row, float* packed_row);
+                                          float* rgb_row, float* packed_row, const float* mean_in = nullptr,
+                                          float* dc_out = nullptr);
 
 // Two phases per workgroup of 256 splats. Phase 1: every thread projects its splat (44 B in) and
 // writes aabb / sorting depth / geometry row / tile count; splats that stay visible are appended
@@ -122,9 +123,10 @@ __global__ __launch_bounds__(kProjBlock) void projection_fwd_kernel(ssr_projecti
 // SH colour of one visible splat g: max(0.5 + sum_j Y_j c_j, 0) (src/shaders/harmonics.slang:1055-1066),
 // written to rgb_row[0..2] and, when given, to the colour slots of its 48-byte fragment row.
 template <int kDegree>
+// mean_in: the splat's mean where the caller holds it already; dc_out: receives the DC colour coefficients
 __device__ __forceinline__ void sh_colour(const ssr_world& W, const ssr_sh_quant& Q, const CamD& cam, int64_t g,
-                                          float* rgb_row, float* packed_row) {
-    const float* mp = W.means + 3 * g;
+                                          float* rgb_row, float* packed_row, const float* mean_in, float* dc_out) {
+    const float* mp = mean_in ? mean_in : W.means + 3 * g;
     const float mean[3] = {mp[0], mp[1], mp[2]};
     constexpr int kCoef = kDegree * (kDegree + 2);
     float coef[kCoef > 0 ? 3 * kCoef : 1];
@@ -135,6 +137,7 @@ __device__ __forceinline__ void sh_colour(const ssr_world& W, const ssr_sh_quant
     sh_basis<kDegree>(dir, b);
     const float* dcp = W.features_dc + 3 * g;
     const float dc[3] = {dcp[0], dcp[1], dcp[2]};
+    if (dc_out) { dc_out[0] = dc[0]; dc_out[1] = dc[1]; dc_out[2] = dc[2]; }
     float raw[3];
     sh_color_raw<kDegree>(b, dc, coef, raw);
     float col[3];
@@ -162,11 +165,12 @@ struct PackedStage {
     float* depth;             // [N]
     float* opac;              // [N]
     int32_t* gid;             // [N]
+    float4* world;            // optional [3][N]: (mean, logit), quat, (log_scale, 0) of the staged rows
 };
 
 __host__ __device__ inline size_t align16(size_t b) { return (b + 15) & ~(size_t)15; }
 
-inline size_t packed_stage_layout(int64_t n, void* base, PackedStage* st) {
+inline size_t packed_stage_layout(int64_t n, void* base, PackedStage* st, bool with_world = false) {
     const size_t nb = (size_t)ceil_div(n, kPackSeg), N = (size_t)n;
     char* p = static_cast<char*>(base);
     size_t off = 0;
@@ -174,7 +178,9 @@ inline size_t packed_stage_layout(int64_t n, void* base, PackedStage* st) {
     char* a0 = take(N * 16); char* a1 = take(N * 8); char* a2 = take(N * 12); char* a3 = take(N * 4);
     char* a4 = take(N * 4); char* a5 = take(N * 4); char* a6 = take(N * 4);
     char* a7 = take((nb + 1) * 8); char* a8 = take(nb * 4);
+    char* a9 = with_world ? take(N * 48) : nullptr;   // last, so that the layout without it is a prefix
     if (st) {
+        st->world = reinterpret_cast<float4*>(a9);
         st->aabb = reinterpret_cast<float4*>(a0); st->xy = reinterpret_cast<float2*>(a1);
         st->conic = reinterpret_cast<float*>(a2); st->sort_depth = reinterpret_cast<float*>(a3);
         st->depth = reinterpret_cast<float*>(a4); st->opac = reinterpret_cast<float*>(a5);
@@ -263,9 +269,9 @@ __global__ __launch_bounds__(kProjBlock) void projection_packed_mask_kernel(ssr_
         ProjD p;
         float bb[4] = {0.f, 0.f, 0.f, 0.f};
         int64_t g = 0;
+        float mean[3], quat[4], ls[3], logit;
         if (c < n_cand) {
             g = block0 + s_cand[c];
-            float mean[3], quat[4], ls[3], logit;
             load_splat(P.world, g, mean, quat, ls, logit);
             project<false, kLens>(cam, mean, quat, ls, logit, p);
             bb[0] = ssr_min(ssr_max(p.aabb[0], 0.0f), cam.Wf - 1.0f);
@@ -291,6 +297,11 @@ __global__ __launch_bounds__(kProjBlock) void projection_packed_mask_kernel(ssr_
             S.depth[d] = p.depth;
             S.opac[d] = p.opac;
             S.gid[d] = (int32_t)g;
+            if (S.world) {
+                S.world[d] = make_float4(mean[0], mean[1], mean[2], logit);
+                S.world[N + d] = make_float4(quat[0], quat[1], quat[2], quat[3]);
+                S.world[2 * N + d] = make_float4(ls[0], ls[1], ls[2], 0.0f);
+            }
             atomic_max_nonneg(P.radii + g, p.radius);   // ProjectionPackedFwd_kernel.cuh:183
         }
         n_out += total;
@@ -415,6 +426,19 @@ __global__ __launch_bounds__(kProjBlock) void projection_packed_emit_kernel(ssr_
         *reinterpret_cast<float2*>(&row[1]) = make_float2(0.5f * conic[2], opac);
         prow[9] = depth; prow[10] = cut; prow[11] = kk;
     }
+    if (P.world_rows) {   // the splat's parameters, plane by plane, for the projection backward
+        const float4 w0 = S.world[src], w2 = S.world[2 * N + src];
+        const float mean[3] = {w0.x, w0.y, w0.z};
+        float dc[3];
+        sh_colour<kDegree>(P.world, P.sh, cam, g, P.screen.rgb + 3 * j, prow, mean, dc);
+        float4* wr = reinterpret_cast<float4*>(P.world_rows) + j;
+        const int64_t plane = P.world_rows_stride;
+        wr[0] = w0;
+        wr[plane] = S.world[N + src];
+        wr[2 * plane] = make_float4(w2.x, w2.y, w2.z, dc[0]);
+        wr[3 * plane] = make_float4(dc[1], dc[2], 0.0f, 0.0f);
+        return;
+    }
     sh_colour<kDegree>(P.world, P.sh, cam, g, P.screen.rgb + 3 * j, prow);
 }
 
@@ -453,10 +477,21 @@ struct PoseGradD { float R[3][3], t[3]; };
 template <int kDegree, bool kLens, bool kPose = false, bool kShFirst = false, class ShSink>
 __device__ __forceinline__ void projection_vjp(const CamD& cam, const ssr_world& W, const ssr_sh_quant& Q, int64_t g,
                                                const VScreenD& VS, int64_t r, WorldGradD& out, ShSink&& sh_sink,
-                                               PoseGradD* pose = nullptr) {
+                                               PoseGradD* pose = nullptr, const float* world_row = nullptr,
+                                               int64_t world_plane = 0) {
     constexpr int kCoef = kDegree * (kDegree + 2);
     float mean[3], quat[4], ls[3], logit;
-    load_splat(W, g, mean, quat, ls, logit);
+    float dc[3];
+    if (world_row) {   // what ssr_projection_packed_emit left: the same values, four coalesced reads
+        const float4* wr = reinterpret_cast<const float4*>(world_row);
+        const float4 a = wr[0], b = wr[world_plane], c = wr[2 * world_plane], d = wr[3 * world_plane];
+        mean[0] = a.x; mean[1] = a.y; mean[2] = a.z; logit = a.w;
+        quat[0] = b.x; quat[1] = b.y; quat[2] = b.z; quat[3] = b.w;
+        ls[0] = c.x; ls[1] = c.y; ls[2] = c.z;
+        dc[0] = c.w; dc[1] = d.x; dc[2] = d.y;
+    } else {
+        load_splat(W, g, mean, quat, ls, logit);
+    }
     float vc[3] = {0.f, 0.f, 0.f};
     float vdir[3] = {0.f, 0.f, 0.f};
     // (kShFirst: ahead of the geometry, whose live values then do not overlap the 45 coefficients)
@@ -468,8 +503,10 @@ __device__ __forceinline__ void projection_vjp(const CamD& cam, const ssr_world&
         view_dir(cam, mean, dir);
         ShBasisD b;
         sh_basis<kDegree>(dir, b);
-        const float* dcp = W.features_dc + 3 * g;
-        const float dc[3] = {dcp[0], dcp[1], dcp[2]};
+        if (!world_row) {
+            const float* dcp = W.features_dc + 3 * g;
+            dc[0] = dcp[0]; dc[1] = dcp[1]; dc[2] = dcp[2];
+        }
         float raw[3];
         sh_color_raw<kDegree>(b, dc, coef, raw);
         const float* vrg = VS.rgb + VS.s_rgb * r;
@@ -748,7 +785,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_kernel(ssr_projecti
         for (int c = 0; c < 3; c++) {
             put<kPut>(vsh + 3 * j + c, ok ? tv[c] : 0.0f);
         }
-    });
+    }, nullptr, P.packed_world_rows ? P.packed_world_rows + 4 * r : nullptr, P.packed_world_stride);
     if (!kAccumulate) {   // coefficients above the active degree receive nothing
         for (int i = 3 * kCoef; i < V.sh_stride; i++) vsh[i] = 0.0f;
     }
@@ -808,7 +845,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_bwd_staged_kernel(ssr_p
             const bool ok = ssr_isfinite(d2) && d2 != 0.0f;   // harmonics.slang:397-403
 #pragma unroll
             for (int c = 0; c < 3; c++) mine[3 * j + c] = ok ? tv[c] : 0.0f;
-        });
+        }, nullptr, P.packed_world_rows ? P.packed_world_rows + 4 * r : nullptr, P.packed_world_stride);
     } else if (!listed) {
         for (int k = 0; k < kShRow; k++) mine[k] = 0.0f;   // a culled row of a run that is written whole
     }
@@ -1535,6 +1572,11 @@ extern "C" size_t ssr_projection_packed_scratch_bytes(int64_t num_splats) {
     return packed_stage_layout(num_splats, nullptr, nullptr);
 }
 
+extern "C" size_t ssr_projection_packed_scratch_bytes_world_rows(int64_t num_splats) {
+    if (num_splats <= 0) return 16;
+    return packed_stage_layout(num_splats, nullptr, nullptr, true);
+}
+
 static int check_packed(const char* where, const ssr_projection_packed_params* p) {
     SSR_REQUIRE(p, where, "null params");
     int e = check_common(where, p->num_splats, p->sh_degree, p->world, p->sh, p->camera);
@@ -1542,6 +1584,12 @@ static int check_packed(const char* where, const ssr_projection_packed_params* p
     SSR_REQUIRE(p->nnz, where, "null nnz");
     if (p->num_splats == 0) return 0;
     SSR_REQUIRE(p->scratch && (reinterpret_cast<uintptr_t>(p->scratch) & 15) == 0, where, "scratch must be non-null and 16-byte aligned");
+    if (p->stage_world_rows)
+        SSR_REQUIRE(p->scratch_bytes >= ssr_projection_packed_scratch_bytes_world_rows(p->num_splats), where,
+                    "scratch too small (with stage_world_rows it holds ssr_projection_packed_scratch_bytes_world_rows bytes)");
+    SSR_REQUIRE(!p->world_rows || p->stage_world_rows, where, "world_rows needs stage_world_rows set, in the mask call as well");
+    SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->world_rows) & 15) == 0, where, "world_rows must be 16-byte aligned");
+    SSR_REQUIRE(!p->world_rows || p->world_rows_stride >= p->max_rows, where, "world_rows_stride must be at least max_rows");
     SSR_REQUIRE(p->scratch_bytes >= ssr_projection_packed_scratch_bytes(p->num_splats), where, "scratch too small");
     SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->world.quats) & 15) == 0, where, "quats must be 16-byte aligned");
     return 0;
@@ -1560,7 +1608,7 @@ extern "C" int ssr_projection_packed_mask(const ssr_projection_packed_params* p,
     }
     SSR_REQUIRE(p->radii, where, "null radii");
     PackedStage st;
-    packed_stage_layout(p->num_splats, p->scratch, &st);
+    packed_stage_layout(p->num_splats, p->scratch, &st, p->stage_world_rows != 0);
     const int64_t nb = ceil_div(p->num_splats, kPackSeg);
     if (camera_needs_lens_path(p->camera.camera_model, p->camera.distortion))
         hipLaunchKernelGGL(projection_packed_mask_kernel<true>, dim3((unsigned)nb), dim3(kProjBlock), 0, s, *p, st);
@@ -1585,7 +1633,7 @@ extern "C" int ssr_projection_packed_emit(const ssr_projection_packed_params* p,
     SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->screen.xy) & 7) == 0, where, "screen.xy must be 8-byte aligned");
     SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->packed_rows) & 15) == 0, where, "packed_rows must be 16-byte aligned");
     PackedStage st;
-    packed_stage_layout(p->num_splats, p->scratch, &st);
+    packed_stage_layout(p->num_splats, p->scratch, &st, p->stage_world_rows != 0);
     const dim3 grid((unsigned)ceil_div(p->max_rows, kProjBlock)), block(kProjBlock);
     hipStream_t s = as_stream(stream);
     switch (p->sh_degree) {
@@ -1608,8 +1656,11 @@ extern "C" int ssr_projection_bwd(const ssr_projection_bwd_params* p, ssr_stream
         SSR_REQUIRE(!p->visible_ids, "ssr_projection_bwd", "packed mode takes no visible list");
         SSR_REQUIRE(p->num_packed >= 0 && p->num_packed <= p->num_splats, "ssr_projection_bwd", "num_packed out of range");
         if (p->num_packed == 0) return 0;
+        SSR_REQUIRE((reinterpret_cast<uintptr_t>(p->packed_world_rows) & 15) == 0, "ssr_projection_bwd", "packed_world_rows must be 16-byte aligned");
+        SSR_REQUIRE(!p->packed_world_rows || p->packed_world_stride >= p->num_packed, "ssr_projection_bwd", "packed_world_stride must be at least num_packed");
     } else {
         SSR_REQUIRE(p->aabb, "ssr_projection_bwd", "null aabb");   // ProjectionBwd.cu:89-97
+        SSR_REQUIRE(!p->packed_world_rows, "ssr_projection_bwd", "packed_world_rows belongs to packed mode");
     }
     SSR_REQUIRE(p->v_rows || (p->v_screen.xy && p->v_screen.depth && p->v_screen.conic && p->v_screen.opac && p->v_screen.rgb),
                 "ssr_projection_bwd", "null v_screen buffer");

@@ -31,6 +31,10 @@ int64_t* g_counters = nullptr;       // device [n_isects, n_visible], one readba
 int32_t* g_visible_ids = nullptr;    // device work list of the last projection (null: off)
 float* g_packed_rows = nullptr;      // packed screen rows of the last projection (null: off)
 const float* g_packed_for_xy = nullptr;   // the screen.xy buffer those rows mirror
+float* g_world_rows = nullptr;                 // parameter rows of the last packed projection (null: off)
+const int32_t* g_world_rows_for_ids = nullptr; // the gaussian_ids they follow
+const float* g_world_rows_for_means = nullptr; // the means tensor they were read from
+int64_t g_world_rows_count = 0;
 bool g_packed_mode = false;          // the last projection was the packed form
 std::vector<int64_t> g_packed_counts;   // ... and its rows per camera (rows are ordered by camera, then splat)
 int g_list_toggle = 0;               // which of the two visible-list buffers the last projection used
@@ -269,6 +273,7 @@ bool backward_overwrites_all_rows(int64_t num_splats) {
     return g_n_visible * 2 >= num_splats;
 }
 const int32_t* last_backward_list(int64_t* count) { if (count) *count = g_bwd_count; return g_bwd_list; }
+void forget_packed_world_rows() { g_world_rows = nullptr; g_world_rows_for_ids = nullptr; g_world_rows_for_means = nullptr; g_world_rows_count = 0; }
 void zero_world_rows(const std::vector<DeviceTensorFloatND>& v, const int32_t* ids, int64_t n,
                      const DeviceTensor2D<float4>* aabb, const int32_t* sorted_now, int64_t n_now) {
     ssr_world w = world_of(v);
@@ -310,6 +315,7 @@ projection_3dgs_forward(const int64_t num_splats, const int max_sh_degree,
     p.screen.xy = xy; p.screen.depth = dp; p.screen.conic = cn; p.screen.opac = op; p.screen.rgb = rg;
     g_counts_fused = false;
     g_packed_mode = false;
+    g_world_rows = nullptr; g_world_rows_for_ids = nullptr; g_world_rows_for_means = nullptr; g_world_rows_count = 0;
     if (g_opts.fuse_tile_count) {
         p.tiles_per_splat = DevicePool::global().acquire<int64_t>(PoolSlot::IsectTilesPerSplat, (size_t)(C * N));
         g_counts_fused = true;
@@ -374,7 +380,10 @@ projection_3dgs_packed_forward(const int64_t num_splats, const int max_sh_degree
     const ssr_camera cameras = camera_of(camera_model, distortion, dist_coeffs, viewmats, intrins, image_width, image_height, true);
     const int64_t C = cameras.num_cameras;
     p.radii = radii.data_ptr();
-    p.scratch_bytes = ssr_projection_packed_scratch_bytes(num_splats);
+    p.stage_world_rows = g_opts.packed_world_rows ? 1 : 0;
+    p.scratch_bytes = p.stage_world_rows ? ssr_projection_packed_scratch_bytes_world_rows(num_splats)
+                                         : ssr_projection_packed_scratch_bytes(num_splats);
+    g_world_rows = nullptr; g_world_rows_for_ids = nullptr; g_world_rows_for_means = nullptr; g_world_rows_count = 0;
     const size_t scratch_stride = (p.scratch_bytes + 255) & ~(size_t)255;
     uint8_t* scratch = DevicePool::global().acquire<uint8_t>(PoolSlot::ProjPackedScratch, scratch_stride * (size_t)C);
     int64_t* nnz_dev = DevicePool::global().acquire<int64_t>(PoolSlot::ProjPackedNnz, (size_t)C);
@@ -427,12 +436,20 @@ projection_3dgs_packed_forward(const int64_t num_splats, const int max_sh_degree
         g_packed_rows = DevicePool::global().acquire<float>(PoolSlot::ProjPackedRows, (size_t)(nnz * 12));
         g_packed_for_xy = xy;
     }
+    if (p.stage_world_rows) {
+        g_world_rows = DevicePool::global().acquire<float>(PoolSlot::ProjPackedWorldRows, (size_t)(nnz * 16));
+        g_world_rows_for_ids = gaussian_ids.data_ptr();
+        g_world_rows_for_means = p.world.means;
+        g_world_rows_count = nnz;
+    }
     int64_t row0 = 0;
     for (int64_t c = 0; c < C; c++) {
         const int64_t rows = counts[(size_t)c];
         if (rows > 0) {
             p.camera = camera_at(cameras, (uint32_t)c);
             p.camera_index = (int32_t)c;
+            p.world_rows = g_world_rows ? g_world_rows + 4 * row0 : nullptr;   // four planes of nnz entries
+            p.world_rows_stride = nnz;
             p.scratch = scratch + scratch_stride * (size_t)c;
             p.nnz = nnz_dev + c;
             p.max_rows = rows;
@@ -816,6 +833,9 @@ void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
         p.aabb = nullptr;
         p.packed_gaussian_ids = gaussian_ids.data_ptr(); p.num_packed = camera_ids.size();
         p.packed_ids_unique = 1;   // one camera per call: the packed projection lists a splat once
+        if (g_world_rows && gaussian_ids.data_ptr() == g_world_rows_for_ids && (int64_t)camera_ids.size() == g_world_rows_count &&
+            p.world.means == g_world_rows_for_means)
+            { p.packed_world_rows = g_world_rows; p.packed_world_stride = g_world_rows_count; }
         g_bwd_list = gaussian_ids.data_ptr(); g_bwd_count = camera_ids.size();
     } else if (g_visible_ids && g_n_visible >= 0) {
         // the rows that end up non-zero are the listed ones either way
@@ -852,6 +872,7 @@ void projection_3dgs_backward(const int64_t num_splats, const int max_sh_degree,
                 p.packed_gaussian_ids = all.packed_gaussian_ids + row0; p.num_packed = rows;
                 p.v_screen = screen_rows_from(all.v_screen, row0);
                 if (all.v_rows) p.v_rows = all.v_rows + 12 * row0;
+                if (all.packed_world_rows) p.packed_world_rows = all.packed_world_rows + 4 * row0;
                 if (all.v_viewmat) p.v_viewmat = all.v_viewmat + 16 * c;
                 p.accumulate = first_launch ? all.accumulate : 1;
                 ok(ssr_projection_bwd(&p, nullptr), "projection_3dgs_backward");
@@ -894,6 +915,7 @@ void fused_projection_bwd_optimizer_3dgs(
     float eps_tr, std::variant<int32_t, TorchTensorView> step, int quantization_level) {
     const char* w = "fused_projection_bwd_optimizer_3dgs: ";
     ssr_ext::resolve_counts();   // no parameter is stepped on gradients of an intersection that did not fit
+    ssr_ext::forget_packed_world_rows();   // the parameters change here
     const bool is_packed = camera_ids.data_ptr() && gaussian_ids.data_ptr();   // src/kernels/optim/FusedProjectionBwdOptim.cu:160
     // quantization_level: 0 = fp32 SH and moments; 1 = 16-bit SH values, 8-bit moments
     // (src/kernels/optim/FusedProjectionBwdOptim_kernel.cuh:1104-1111; validation as FusedProjectionBwdOptim.cu:386-400)

@@ -187,6 +187,12 @@ struct Options {
     // the count did not fit; the images and gradients of that iteration are then incomplete and the next
     // intersection reads its count again. The first call, and any call with capacity 0, blocks as before.
     bool deferred_counts = false;
+    // projection_3dgs_packed_forward also keeps the parameters of every visible splat, 64 bytes in four planes, in the
+    // order of the packed rows, and a projection_3dgs_backward that is handed the gaussian_ids and the parameter
+    // tensors of that call reads those planes instead of gathering from five arrays (it pays where a view sees a
+    // small, scattered part of the splats). For callers that do not change the parameters between a packed
+    // projection and its backward: tensors are recognised by their addresses, not by their contents.
+    bool packed_world_rows = false;
     // int8 codes x per-splat fp16 scale as SH storage (the benchmark's format): sh_value_bits == 8
     // with sh_value_bounds holding the fp16 scales when this is set.
     bool sh_int8_f16scale = false;
@@ -205,6 +211,9 @@ int64_t deferred_capacity();
 // The list the last projection_3dgs_backward ran over (device pointer) and its length; it stays
 // intact until the projection after next (the two list buffers alternate). Null when it had none.
 const int32_t* last_backward_list(int64_t* count);
+// Drops the parameter rows kept under Options::packed_world_rows: for a caller that writes new parameter values
+// into the same tensors between a packed projection and its backward.
+void forget_packed_world_rows();
 // True when the next projection_3dgs_backward (after the forward that just ran) will overwrite EVERY
 // row of v_splats_world -- store mode, and either no work list or so many visible splats (half or
 // more) that walking all rows is cheaper than a zero-fill plus the list. The caller may then skip

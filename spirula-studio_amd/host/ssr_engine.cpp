@@ -68,6 +68,7 @@ void alloc_grad_buffers() {
 
 void set_data_3dgs(int64_t num_splats, TorchTensorView means, TorchTensorView quats, TorchTensorView scales,
                    TorchTensorView opacities, TorchTensorView features_dc, TorchTensorView features_sh) {
+    ssr_ext::forget_packed_world_rows();   // new parameter values
     const int64_t max_num_splats = std::get<2>(means)[0];
     if (std::get<2>(quats)[0] != max_num_splats || std::get<2>(scales)[0] != max_num_splats ||
         std::get<2>(opacities)[0] != max_num_splats || std::get<2>(features_dc)[0] != max_num_splats ||
@@ -464,6 +465,12 @@ int ssrh_set_deferred_counts(int on, int64_t capacity) {
     });
 }
 int64_t ssrh_deferred_capacity(void) { return ssr_ext::deferred_capacity(); }
+
+// on: the packed projection keeps the parameters of the visible splats (64 bytes each, in four planes) and the projection backward
+// reads them (Options::packed_world_rows)
+int ssrh_set_packed_world_rows(int on) {
+    return guard([&] { ssr_ext::options().packed_world_rows = on != 0; });
+}
 
 // host or device pointers; num_sh = coefficients per splat excluding DC (15 for SH3)
 int ssrh_set_data_3dgs(int64_t n, const float* means, const float* quats, const float* scales, const float* opacities,

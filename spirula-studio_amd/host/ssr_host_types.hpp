@@ -66,7 +66,7 @@ enum class PoolSlot : int {
     IsectScanScratch, IsectSortScratch, IsectCounters, ProjVisibleIds, ProjVisibleIdsB, ProjPackedRows,
     IsectTileActive, EngTileMask, IsectTileOrder,
     AdamG1Means, AdamG1Quats, AdamG1Scales, AdamG1Opacities, AdamG1FeaturesDc, AdamG1FeaturesSh,
-    AdamG2Means, AdamG2Quats, AdamG2Scales, AdamG2Opacities, AdamG2FeaturesDc, AdamG2FeaturesSh, EngDensifyScore, EngZeroAabb, FusedProjBwdRowOf, AdamShStatePacked, AdamShStateBounds, AdamNonShPacked, AdamNonShBounds, EngPoseGrad, ProjCameraIds, ProjGaussianIds, ProjGaussianIdsB, ProjPackedScratch, ProjPackedNnz, FusedMultiCamGrad,
+    AdamG2Means, AdamG2Quats, AdamG2Scales, AdamG2Opacities, AdamG2FeaturesDc, AdamG2FeaturesSh, EngDensifyScore, EngZeroAabb, FusedProjBwdRowOf, AdamShStatePacked, AdamShStateBounds, AdamNonShPacked, AdamNonShBounds, EngPoseGrad, ProjCameraIds, ProjGaussianIds, ProjGaussianIdsB, ProjPackedScratch, ProjPackedNnz, ProjPackedWorldRows, FusedMultiCamGrad,
     RendersRgb, RendersDepth, RenderTs, RenderLastIds, RenderDistortionRgb, RenderDistortionDepth, RenderMedian,
     RasterBwdAccumWeight, RasterBwdVRows, EngVDistRgb, EngVDistDepth, EngVMedian, EngAccumMap,
     RasterBwdVScreenXy, RasterBwdVScreenDepth, RasterBwdVScreenConic, RasterBwdVScreenOpac, RasterBwdVScreenRgb,

@@ -84,7 +84,7 @@ class ProjectionBwdParams(C.Structure):
                 ("v_world", World), ("accumulate", C.c_int32), ("visible_ids", vp),
                 ("n_visible", C.c_int64), ("packed_gaussian_ids", vp), ("num_packed", C.c_int64), ("v_rows", vp),
                 ("v_viewmat", vp),
-                ("antialiased", C.c_int32), ("packed_ids_unique", C.c_int32)]
+                ("antialiased", C.c_int32), ("packed_ids_unique", C.c_int32), ("packed_world_rows", vp), ("packed_world_stride", C.c_int64)]
 
 
 class ProjectionPackedParams(C.Structure):
@@ -93,7 +93,7 @@ class ProjectionPackedParams(C.Structure):
                 ("scratch_bytes", C.c_size_t), ("nnz", vp), ("max_rows", C.c_int64),
                 ("camera_ids", vp), ("gaussian_ids", vp), ("aabb", vp), ("sort_depth", vp),
                 ("screen", Screen), ("tiles_per_splat", vp), ("packed_rows", vp),
-                ("antialiased", C.c_int32), ("camera_index", C.c_int32)]
+                ("antialiased", C.c_int32), ("camera_index", C.c_int32), ("world_rows", vp), ("world_rows_stride", C.c_int64), ("stage_world_rows", C.c_int32)]
 
 
 class FpboParams(C.Structure):
@@ -117,6 +117,7 @@ _i64, _u32, _i32, _sz = C.c_int64, C.c_uint32, C.c_int, C.c_size_t
 SYMBOLS = {
     "ssr_projection_fwd": (_i32, [C.POINTER(ProjectionFwdParams), vp]),
     "ssr_projection_packed_scratch_bytes": (_sz, [_i64]),
+    "ssr_projection_packed_scratch_bytes_world_rows": (_sz, [_i64]),
     "ssr_projection_packed_mask": (_i32, [C.POINTER(ProjectionPackedParams), vp]),
     "ssr_projection_packed_emit": (_i32, [C.POINTER(ProjectionPackedParams), vp]),
     "ssr_tile_count": (_i32, [_i64, vp, vp, vp, vp, _u32, _u32, vp, vp, vp]),

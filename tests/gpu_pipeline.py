@@ -35,7 +35,7 @@ def world_grad_check(got, ref, n, name, rtol=WORLD_GRAD_RTOL, bad_frac=0.0, scal
 
 class GpuRun:
     def __init__(self, pkg, scene, sh_degree=3, use_list=False, use_packed=False, packed_projection=False,
-                 read_nnz=True, use_vrows=False, tile_sort=False, capacity=None):
+                 read_nnz=True, use_vrows=False, tile_sort=False, capacity=None, world_rows=False):
         """use_packed: 48-byte fragment rows for the compositing kernels. packed_projection: the
         compacted (nnz-row) projection outputs of projection_3dgs_packed_forward; read_nnz=False
         sizes the outputs for all N splats instead of reading nnz back between the two calls."""
@@ -43,6 +43,10 @@ class GpuRun:
         self.use_packed = use_packed
         self.packed_projection = packed_projection
         self.read_nnz = read_nnz
+        # world_rows (with packed_projection): the projection also writes each visible splat's parameters (four
+        # planes of 16-byte entries), and the projection backward reads those
+        self.world_rows = world_rows
+        assert packed_projection or not world_rows
         self.tile_sort = tile_sort   # ssr_sort_tile_pairs instead of the whole-key sort + ssr_tile_offsets
         # capacity (with tile_sort): the key arrays hold that many entries and nothing is read back between the scan
         # and the compositing (ssr_tile_write_capped, ssr_sort_tile_pairs_capped, closed offsets)
@@ -140,7 +144,8 @@ class GpuRun:
         D = self.L.DeviceArray
         n = self.n
         self.d["radii"].fill_zero()
-        sb = self.lib.ssr_projection_packed_scratch_bytes(n)
+        sb = (self.lib.ssr_projection_packed_scratch_bytes_world_rows(n) if self.world_rows
+              else self.lib.ssr_projection_packed_scratch_bytes(n))
         self.d["pk_scratch"] = D((sb,), np.uint8)
         self.d["nnz"] = D((1,), np.int64)
         p = self.L.ProjectionPackedParams()
@@ -148,6 +153,7 @@ class GpuRun:
         p.antialiased = 1 if getattr(self.sc, "antialiased", False) else 0
         p.world, p.sh, p.camera = self.world(), self.shq(), self.camera()
         p.radii, p.scratch, p.scratch_bytes, p.nnz = self.ptr("radii"), self.ptr("pk_scratch"), sb, self.ptr("nnz")
+        p.stage_world_rows = 1 if self.world_rows else 0
         self.check(self.lib.ssr_projection_packed_mask(C.byref(p), None))
         if self.read_nnz:
             k = (C.c_int64 * 1)(0)
@@ -160,7 +166,8 @@ class GpuRun:
                               ("xy", (cap, 2), np.float32), ("depth", (cap,), np.float32),
                               ("conic", (cap, 3), np.float32), ("opac", (cap,), np.float32),
                               ("rgb", (cap, 3), np.float32), ("counts", (cap,), np.int64),
-                              ("cum", (cap,), np.int64), ("packed", (cap, 12), np.float32)]:
+                              ("cum", (cap,), np.int64), ("packed", (cap, 12), np.float32),
+                              ("world_rows", (4, cap, 4), np.float32)]:
             self.d[nm] = D(shape, dt)
             if cap:   # poison, so that rows past nnz are seen to stay untouched
                 self.check(self.lib.ssr_fill_u32(self.d[nm].ptr, 0x7fc12345, self.d[nm].nbytes // 4, None))
@@ -169,6 +176,8 @@ class GpuRun:
         p.aabb, p.sort_depth, p.screen = self.ptr("aabb"), self.ptr("sort_depth"), self.screen()
         p.tiles_per_splat = self.ptr("counts") if fused_count else None
         p.packed_rows = self.ptr("packed") if self.use_packed else None
+        p.world_rows = self.ptr("world_rows") if self.world_rows else None
+        p.world_rows_stride = cap
         self.check(self.lib.ssr_projection_packed_emit(C.byref(p), None))
         if not self.read_nnz:
             k = (C.c_int64 * 1)(0)
@@ -397,8 +406,8 @@ class GpuRun:
             for k, sl in [("v_xy", slice(0, 2)), ("v_depth", 2), ("v_conic", slice(3, 6)), ("v_opac", 6), ("v_rgb", slice(7, 10))]:
                 self.d[k] = D.from_host(np.ascontiguousarray(rows[:, sl]))
 
-    def projection_bwd(self, accumulate=True, poison=False, pose=False, misalign_sh_rows=False):
-        """pose=True: also the camera-pose gradient, read back with host("v_viewmat") as [4,4].
+    def projection_bwd(self, accumulate=True, poison=False, pose=False, misalign_sh_rows=False, use_world_rows=True):
+        """use_world_rows=False: gather the parameters although the projection left their rows. pose=True: also the camera-pose gradient, read back with host("v_viewmat") as [4,4].
         misalign_sh_rows: the SH gradient rows start 4 bytes into their buffer, which takes the launcher off the
         kernel that stages them through LDS (it needs 16-byte alignment); read back with sh_rows_misaligned()."""
         D = self.L.DeviceArray
@@ -431,6 +440,9 @@ class GpuRun:
                 return
             p.aabb = None
             p.packed_gaussian_ids, p.num_packed = self.ptr("gaussian_ids"), self.rows
+            if self.world_rows and use_world_rows:
+                p.packed_world_rows = self.ptr("world_rows")
+                p.packed_world_stride = self.cap
         if misalign_sh_rows:
             raw = D((n * 45 + 4,), np.float32)
             if poison:

@@ -48,6 +48,10 @@ def test_argument_checks_without_device(L):
     assert lib.ssr_sort_end_bit(32400) == 47 and lib.ssr_sort_end_bit(32768) == 48
     assert lib.ssr_scan_scratch_bytes(0) == 0 and lib.ssr_scan_scratch_bytes(2049) == 16
     assert lib.ssr_sort_scratch_bytes(0) == 0 and lib.ssr_sort_scratch_bytes(4097) == (3 * 256 + 256) * 4   # three 2048-key blocks
+    # the staging area of the packed projection: the parameter rows add 48 bytes per splat behind the rest
+    for n in (1, 1000, 1025, 10_000_000):
+        assert lib.ssr_projection_packed_scratch_bytes_world_rows(n) == lib.ssr_projection_packed_scratch_bytes(n) + 48 * n
+    assert lib.ssr_projection_packed_scratch_bytes_world_rows(0) == lib.ssr_projection_packed_scratch_bytes(0)
     assert lib.ssr_projection_fwd(None, None) != 0 and b"null params" in lib.ssr_last_error()
     assert lib.ssr_last_error() == b""                     # cleared by the read
     p = L.ProjectionFwdParams()

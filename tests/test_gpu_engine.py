@@ -314,10 +314,13 @@ def test_engine_packed_projection(pkg, oracle, H, native):
         _check_packed(eng, ref, sc)
 
 
-def test_engine_packed_follows_the_camera_and_handles_nothing_visible(pkg, oracle, H):
+@pytest.mark.parametrize("world_rows", [False, True], ids=["gathered", "world-rows"])
+def test_engine_packed_follows_the_camera_and_handles_nothing_visible(pkg, oracle, H, world_rows):
+    """world-rows: the packed projection keeps the visible splats' parameters (64 bytes each, in four planes) for the projection
+    backward (Options::packed_world_rows); the rows must follow every new projection."""
     host, lib = H
     sc = pkg.scenes.make_scene(4, n=60000, width=480, height=270)
-    eng = host.Engine(sc, packed_projection=True)
+    eng = host.Engine(sc, packed_projection=True, packed_world_rows=world_rows)
     for _ in range(2):
         eng.forward()
         eng.backward()
@@ -793,7 +796,7 @@ def _two_camera_scene(pkg, n=3000, seed=71, cull_every=0):
     return base, singles, both
 
 
-@pytest.mark.parametrize("native", [False, True])
+@pytest.mark.parametrize("native", [False, True, "world-rows"])
 def test_engine_two_cameras_packed_projection(pkg, oracle, H, native):
     """The packed projection over a camera batch (ProjectionPackedFwd_kernel.cuh:37-47,119-135: one scan over C * N):
     rows ordered by (camera, splat), camera_ids saying which image a row belongs to, and every later stage on
@@ -804,8 +807,10 @@ def test_engine_two_cameras_packed_projection(pkg, oracle, H, native):
     refs = [oracle.pipeline_packed(sc) for sc in singles]
     m = [r["proj"]["visible"] for r in refs]
     assert min(m) > 100 and m[0] != m[1]
+    world_rows = native == "world-rows"   # the parameter rows of both cameras, one run behind the other
+    native = bool(native)
     eng = host.Engine(both, packed_projection=True, fuse_tile_count=native, packed_rows=native, overwrite_world_grads=native,
-                      packed_vscreen=native, tile_sort=native)
+                      packed_vscreen=native, tile_sort=native, packed_world_rows=world_rows)
     tiles = ((w + 15) // 16) * ((h + 15) // 16)
     for rep in range(2):
         eng.forward()

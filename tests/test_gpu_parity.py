@@ -518,10 +518,10 @@ def test_packed_projection_sparse_and_dense(gpu, oracle):
 
 
 def test_packed_projection_first_pass_cull(gpu, oracle):
-    """The packed mask kernel first rejects splats from the mean and the scales alone and compacts the rest when
-    few remain: it may only reject what the projection rejects. Splats straddling every image edge with centres
-    far off the image, very large splats, splats just in front of and just behind the camera plane, workgroups
-    on both sides of the compaction threshold: rows, ids and the whole chain as the oracle's."""
+    """The packed mask kernel first rejects splats from the mean and the scales alone and lists the rest: it may
+    only reject what the projection rejects. Splats straddling every image edge with centres far off the image,
+    very large splats, splats just in front of and just behind the camera plane, 256-splat slices with every
+    share of candidates: rows, ids and the whole chain as the oracle's."""
     S = gpu.scenes
     sc = S.tiny_scene(n=3000, width=96, height=64, seed=31)
     sc.means[:, :2] *= 8.0                      # most centres off the image, many footprints reaching back in
@@ -540,6 +540,50 @@ def test_packed_projection_first_pass_cull(gpu, oracle):
     _compare_packed(gpu, oracle, sc, "pk-cull-threshold", fused_count=True)
 
 
+def test_packed_projection_world_rows(gpu, oracle):
+    """The optional parameter planes of the packed projection: entry i of the four planes holds the parameters of
+    splat gaussian_ids[i] bit for bit, entries past nnz stay untouched, every other output is what it is without them, and a
+    projection backward that reads the rows gives the same bits as one that gathers from the five arrays (store
+    and add mode, fp32 and int8 SH, with and without the gradient rows of the compositing backward)."""
+    S = gpu.scenes
+    cases = [("wr-tiny", S.tiny_scene(n=2500, width=96, height=64, seed=41), dict()),
+             ("wr-cfg4", S.make_scene(4, n=80000, width=480, height=270, sh_codec=3), dict(use_packed=True, use_vrows=True)),
+             ("wr-cfg2", S.make_scene(2, n=30000, width=480, height=270, parity_variant=True), dict(read_nnz=False))]
+    cases[0][1].means[::3, 2] = -10.0   # a third behind the camera
+    keys = ["w_means", "w_quats", "w_log_scales", "w_opacity_logits", "w_features_dc", "w_features_sh"]
+    for label, sc, kw in cases:
+        print(f"[{label}] N={sc.n}", flush=True)
+        runs = []
+        for wr in (False, True):
+            g = GpuRun(gpu, sc, packed_projection=True, world_rows=wr, **kw)
+            g.run_all(fused_count=True)
+            runs.append(g)
+        a, b = runs
+        m = b.nnz
+        assert a.nnz == m and 0 < m < sc.n
+        ids = b.host("gaussian_ids")[:m]
+        rows = b.host("world_rows")
+        want = np.zeros((m, 16), np.float32)
+        want[:, 0:3] = sc.means[ids]; want[:, 3] = np.ravel(sc.opacity_logits)[ids]
+        want[:, 4:8] = sc.quats[ids]; want[:, 8:11] = sc.log_scales[ids]; want[:, 11:14] = sc.features_dc[ids]
+        assert np.array_equal(rows[:, :m].view(np.uint32), want.reshape(m, 4, 4).transpose(1, 0, 2).view(np.uint32))
+        assert np.all(rows[:, m:].view(np.uint32) == 0x7fc12345)
+        for k in ["gaussian_ids", "aabb", "sort_depth", "xy", "depth", "conic", "opac", "rgb", "radii", "r_rgb", "r_last"]:
+            assert np.array_equal(a.host(k).view(np.uint32), b.host(k).view(np.uint32)), k
+        # the projection backward on ONE set of screen gradients (the compositing backward's atomics differ in the
+        # last bits from run to run), with and without the rows
+        vis = np.zeros(sc.n, bool); vis[ids] = True
+        for accumulate in (True, False):   # atomic adds into zeros (the plain kernel); stores over poison (the staged one)
+            got = []
+            for use in (True, False):
+                b.projection_bwd(accumulate=accumulate, poison=not accumulate, use_world_rows=use)
+                b.check(b.lib.ssr_device_synchronize())
+                got.append({k: b.host(k) for k in keys})
+            for k in keys:
+                assert np.array_equal(got[0][k][vis].view(np.uint32), got[1][k][vis].view(np.uint32)), (k, accumulate)
+                assert np.isfinite(got[0][k][vis]).all() and np.any(got[0][k][vis] != 0), k
+
+
 def test_packed_projection_all_culled_and_empty(gpu, oracle):
     sc = gpu.scenes.tiny_scene(n=300, width=40, height=24, seed=1)
     sc.means[:, 2] = -10.0
@@ -548,11 +592,22 @@ def test_packed_projection_all_culled_and_empty(gpu, oracle):
 
 
 def test_packed_projection_block_boundaries(gpu, oracle):
-    """Visibility patterns that leave whole 256-splat workgroups empty or full."""
+    """Visibility patterns that leave whole wavefront slices (256 splats) and whole workgroup segments (1024 splats)
+    of the mask kernel empty or full."""
     sc = gpu.scenes.tiny_scene(n=256 * 9 + 17, width=96, height=64, seed=24)
     blk = np.arange(sc.n) // 256
     sc.means[(blk == 0) | (blk == 3) | (blk == 4) | (blk == 9), 2] = -10.0   # culled blocks, incl. first and last
     g, r = _compare_packed(gpu, oracle, sc, "pk-blocks", fused_count=True)
+    assert 0 < g.nnz < sc.n
+    sc = gpu.scenes.tiny_scene(n=1024 * 5 + 300, width=96, height=64, seed=25)
+    seg = np.arange(sc.n) // 1024
+    sc.means[(seg == 0) | (seg == 2) | (seg == 5), 2] = -10.0   # culled segments: the first, one inside, the short last one
+    g, r = _compare_packed(gpu, oracle, sc, "pk-segments", fused_count=True)
+    assert 0 < g.nnz < sc.n
+    sc = gpu.scenes.tiny_scene(n=1024 * 3, width=96, height=64, seed=26)
+    seg = np.arange(sc.n) // 1024
+    sc.means[(seg == 1) & (np.arange(sc.n) % 1024 < 1023), 2] = -10.0   # one survivor at the end of a segment
+    g, r = _compare_packed(gpu, oracle, sc, "pk-segment-last-row")
     assert 0 < g.nnz < sc.n
 
 
