@@ -128,8 +128,9 @@ def test_full_size_properties(pkg, oracle, H, cfg):
     for k in g1:
         close(g1b[k], g1[k], ("idempotent", k))
         close(g3[k], g1[k], ("reference order", k))
-    # packed projection outputs: same image, same gradients, ids = the visible splats in order
-    pk = host.Engine(sc, packed_projection=True)
+    # packed projection outputs: same image, same gradients, ids = the visible splats in order (config 4 as the
+    # benchmark runs it: the projection backward reads the parameter rows that the packed projection keeps)
+    pk = host.Engine(sc, packed_projection=True, packed_world_rows=(cfg == 4))
     pk.forward()
     pk.backward()
     assert np.array_equal(pk.cache("gaussian_ids"), np.nonzero(vis)[0])
