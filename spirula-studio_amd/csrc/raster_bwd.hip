@@ -276,6 +276,13 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
 
     const uint8_t* my_list = s_list + (4 * mt + row) * kB;
     bool first = true;
+    // the splat id a thread stages next is read one batch ahead: the fragment gather of the next batch then waits for
+    // one memory round trip, not two in a row
+    int32_t g_ahead = 0;
+    {
+        const int32_t idx0 = min(range_end - 1, tile_last) - (tid >= kB ? tid - kB : tid);
+        if (idx0 >= range_start && tid < 2 * kB) g_ahead = P.flatten_ids[idx0];
+    }
     for (int32_t hi = min(range_end - 1, tile_last); hi >= range_start; hi -= kB) {
         // Explicit wait for this wavefront's LDS traffic (the read-add-writes and float atomics of the walk):
         // the compiler does not place one ahead of this loop-header barrier on the path that leaves the walk,
@@ -290,7 +297,7 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
             const int32_t idx = hi - slot;
             uint32_t bits8 = 0;
             if (idx >= range_start && tid < 2 * kB) {
-                const int32_t g = P.flatten_ids[idx];
+                const int32_t g = g_ahead;
                 const FragLds f = stage_fragment_half(P.screen, P.packed_rows, g, tile_x0, tile_y0, half, bits8);
                 if (half == 0) {
                     s_ids[slot] = g; frags[slot] = f;
@@ -301,6 +308,7 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
                 }
             }
             if (tid < 2 * kB) s_bits[half * kB + slot] = (uint8_t)bits8;
+            if (idx - kB >= range_start && tid < 2 * kB) g_ahead = P.flatten_ids[idx - kB];
         }
         __syncthreads();
         // this wavefront's four lists: slots whose block bit is set and whose sorted index hi - slot is

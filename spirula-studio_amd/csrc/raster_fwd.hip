@@ -45,19 +45,23 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raste
     // slot from the start (the first barrier of the batch loop orders this with the first reads)
     for (int e = tid; e < (int)sizeof(s_list); e += kRasterBlock) s_list[e] = 0;
 
+    // the splat id a thread stages next is read one batch ahead: the fragment gather of the next batch then waits for
+    // one memory round trip, not two in a row
+    int32_t g_ahead = range_start + tid < range_end ? P.flatten_ids[range_start + tid] : 0;
     for (int32_t batch_start = range_start; batch_start < range_end; batch_start += kBatch) {
         // all pixels of the tile finished: stop (this barrier also fences reuse of the LDS batch)
         if (__syncthreads_count(alive == 0) >= kRasterBlock) break;
         const int32_t idx = batch_start + tid;
         if (idx < range_end) {
             float kk;
-            FragLds f = stage_fragment(P.screen, P.packed_rows, P.flatten_ids[idx], tile_x0, tile_y0, &kk);
+            FragLds f = stage_fragment(P.screen, P.packed_rows, g_ahead, tile_x0, tile_y0, &kk);
             add_block_mask(f, kk, tile_x0, tile_y0);
             frags[tid] = f;
             if constexpr (kDist != SSR_DIST_NONE) s_lz[tid] = ssr_log(ssr_max(f.q2.y, 1e-6f));
         } else {
             frags[tid].q2 = make_float4(0.f, 0.f, 0.f, 0.f);   // empty masks
         }
+        if (idx + kBatch < range_end) g_ahead = P.flatten_ids[idx + kBatch];
         __syncthreads();
         const int n_batch = min(kBatch, range_end - batch_start);
         // a row whose sixteen pixels are finished needs no list
