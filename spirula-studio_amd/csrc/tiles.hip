@@ -329,17 +329,19 @@ __global__ __launch_bounds__(kTileBlock) void tile_offsets_kernel(int64_t n_isec
                                                                   const int64_t* __restrict__ ids, int64_t n_tiles,
                                                                   int32_t* __restrict__ offsets) {
     const int64_t idx = (int64_t)blockIdx.x * kTileBlock + threadIdx.x;
-    if (n_dev) {
-        n_isects = min(n_isects, *n_dev);
-        if (n_isects == 0 && idx == 0)   // no key: nobody below writes anything
-            for (int64_t i = 0; i < n_tiles; ++i) offsets[i] = 0;
+    if (n_dev) n_isects = min(n_isects, *n_dev);
+    // The tiles up to the first key's and those behind the last key's can be half the image (a scene that covers
+    // its middle): the first workgroup and the one that holds the last key fill them together, not one thread each.
+    if (blockIdx.x == 0) {
+        const int64_t upto = n_isects > 0 ? min((int64_t)(ids[0] >> 32) + 1, n_tiles) : (n_dev ? n_tiles : 0);   // no key: nobody below writes anything
+        for (int64_t i = threadIdx.x; i < upto; i += kTileBlock) offsets[i] = 0;
+    }
+    if (n_isects > 0 && (int64_t)blockIdx.x == (n_isects - 1) / kTileBlock) {
+        const int64_t from = (ids[n_isects - 1] >> 32) + 1;
+        for (int64_t i = from + threadIdx.x; i < n_tiles; i += kTileBlock) offsets[i] = (int32_t)n_isects;
     }
     if (idx >= n_isects) return;
     const int64_t tile = ids[idx] >> 32;
-    if (idx == 0)
-        for (int64_t i = 0; i < tile + 1 && i < n_tiles; ++i) offsets[i] = 0;
-    if (idx == n_isects - 1)
-        for (int64_t i = tile + 1; i < n_tiles; ++i) offsets[i] = (int32_t)n_isects;
     if (idx > 0) {
         const int64_t prev = ids[idx - 1] >> 32;
         if (prev != tile)
