@@ -362,6 +362,19 @@ __device__ __forceinline__ uint32_t tile_class(const int32_t* __restrict__ offse
     const int64_t len = e - offsets[t];
     return 255u - (uint32_t)min((int64_t)255, len >> 5);   // class 0 holds the longest tiles
 }
+// The lanes of this wavefront that hold the same class as this lane (live lanes only).
+__device__ __forceinline__ uint64_t wave_peers_u8(uint32_t cls, bool live) {
+    uint64_t peers = __ballot(live);
+#pragma unroll
+    for (int b = 0; b < 8; b++) {
+        const bool own = ((cls >> b) & 1u) != 0;
+        const uint64_t vote = __ballot(own);
+        peers &= own ? vote : ~vote;
+    }
+    return peers;
+}
+// Tiles of one class are many (most tiles of an image hold similar numbers of fragments): a wavefront adds once per
+// class it holds, not once per tile.
 // counts[block][256]: how many tiles of each class the workgroup's 1024 tiles hold
 __global__ __launch_bounds__(kOrderBlock) void tile_order_count_kernel(const int32_t* __restrict__ offsets, uint32_t n_tiles,
                                                                        int64_t n_isects, uint32_t* __restrict__ counts) {
@@ -369,7 +382,12 @@ __global__ __launch_bounds__(kOrderBlock) void tile_order_count_kernel(const int
     if (threadIdx.x < 256) s_count[threadIdx.x] = 0;
     __syncthreads();
     const uint32_t t = blockIdx.x * kOrderBlock + threadIdx.x;
-    if (t < n_tiles) atomicAdd(&s_count[tile_class(offsets, t, n_tiles, n_isects)], 1u);
+    {
+        const bool live = t < n_tiles;
+        const uint32_t cls = live ? tile_class(offsets, t, n_tiles, n_isects) : 0u;
+        const uint64_t peers = wave_peers_u8(cls, live);
+        if (live && (peers & ((1ull << (threadIdx.x & 63)) - 1ull)) == 0) atomicAdd(&s_count[cls], (uint32_t)__popcll(peers));
+    }
     __syncthreads();
     if (threadIdx.x < 256) counts[blockIdx.x * 256 + threadIdx.x] = s_count[threadIdx.x];
 }
@@ -382,7 +400,8 @@ __global__ __launch_bounds__(kOrderBlock) void tile_order_scatter_kernel(const i
     __shared__ uint32_t s_wave[4];
     if (threadIdx.x < 256) {
         uint32_t total = 0, before = 0;
-        for (uint32_t b = 0; b < gridDim.x; b++) {
+#pragma unroll 8
+        for (uint32_t b = 0; b < gridDim.x; b++) {   // (unrolled: the rows' loads in flight together)
             const uint32_t c = counts[b * 256 + threadIdx.x];
             total += c;
             if (b < blockIdx.x) before += c;
@@ -405,8 +424,17 @@ __global__ __launch_bounds__(kOrderBlock) void tile_order_scatter_kernel(const i
     }
     __syncthreads();
     const uint32_t t = blockIdx.x * kOrderBlock + threadIdx.x;
-    if (t < n_tiles) order[atomicAdd(&s_next[tile_class(offsets, t, n_tiles, n_isects)], 1u)] = (int32_t)t;
+    const bool live = t < n_tiles;
+    const int lane = threadIdx.x & 63;
+    const uint32_t cls = live ? tile_class(offsets, t, n_tiles, n_isects) : 0u;
+    const uint64_t peers = wave_peers_u8(cls, live);
+    const uint32_t rank = (uint32_t)__popcll(peers & ((1ull << lane) - 1ull));
+    uint32_t base = 0;
+    if (live && rank == 0) base = atomicAdd(&s_next[cls], (uint32_t)__popcll(peers));
+    base = __shfl(base, peers ? __ffsll((long long)peers) - 1 : 0, 64);   // from the class's first lane
+    if (live) order[base + rank] = (int32_t)t;
 }
+
 
 }  // namespace ssr
 

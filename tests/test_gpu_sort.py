@@ -144,6 +144,31 @@ def test_sort_tile_pairs_empty_and_errors(L):
     assert lib.ssr_last_error() != b""
 
 
+@pytest.mark.parametrize("n_tiles", [1, 2, 63, 1023, 1024, 1025, 8160, 32768, 65536, 65537, 131072 + 5])
+@pytest.mark.parametrize("closed", [False, True])
+def test_tile_order(L, n_tiles, closed):
+    """ssr_tile_order on synthetic tile ranges, on both sides of the size where one workgroup does it alone: a
+    permutation of the tiles, classes of 32 fragments in falling order (everything from 8160 fragments up in the
+    first). Lengths are drawn so that a few classes hold most tiles, as in an image, with empty and huge tiles
+    among them; closed: the ranges carry their own last entry instead of the count."""
+    lib = L.load()
+    rng = np.random.default_rng(n_tiles)
+    length = rng.choice([0, 1, 31, 32, 33, 100, 101, 102, 700, 8159, 8160, 20000], n_tiles,
+                        p=[.1, .05, .05, .05, .05, .3, .2, .1, .05, .02, .02, .01]).astype(np.int64)
+    ends = np.cumsum(length)
+    K = int(ends[-1])
+    offs = np.concatenate([[0], ends]).astype(np.int32)
+    assert ends[-1] < 2 ** 31
+    d_off = L.DeviceArray.from_host(offs if closed else offs[:-1])
+    sb = lib.ssr_tile_order_scratch_bytes(n_tiles)
+    order, scratch = L.DeviceArray((n_tiles,), np.int32), L.DeviceArray((max(sb, 16),), np.uint8)
+    L.check(lib.ssr_tile_order(d_off.ptr, n_tiles, -1 if closed else K, order.ptr, scratch.ptr, sb, None))
+    got = order.to_host()
+    assert np.array_equal(np.sort(got), np.arange(n_tiles))
+    cls = np.minimum(length >> 5, 255)[got]
+    assert np.all(cls[1:] <= cls[:-1])
+
+
 @pytest.mark.parametrize("n", [1, 2, 255, 256, 2047, 2048, 2049, 1_000_003, 10_000_019])
 def test_inclusive_sum_i64(L, n):
     lib = L.load()
