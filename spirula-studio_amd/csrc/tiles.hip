@@ -255,11 +255,21 @@ __global__ __launch_bounds__(kScanBlock) void scan_spine_kernel(int64_t* __restr
     }
 }
 
+// kSumTotals: block_prefix holds the workgroups' totals as scan_reduce_kernel left them, and every workgroup adds
+// up the ones before it for itself (a few loads per thread up to kScanSumBlocks workgroups): the spine kernel
+// between the two passes, a launch of four wavefronts, is then not needed.
+constexpr int64_t kScanSumBlocks = 4096;
+template <bool kSumTotals>
 __global__ __launch_bounds__(kScanBlock) void scan_down_kernel(const int64_t* __restrict__ in, int64_t n,
                                                                const int64_t* __restrict__ block_prefix,
                                                                int64_t* __restrict__ out, int64_t* __restrict__ total_out) {
     __shared__ int64_t lds[4];
+    [[maybe_unused]] __shared__ int64_t lds_before[4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    [[maybe_unused]] int64_t before = 0;
+    if constexpr (kSumTotals) {
+        for (int64_t b = threadIdx.x; b < (int64_t)blockIdx.x; b += kScanBlock) before += block_prefix[b];
+    }
     const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)wave * (64 * kScanItems) + lane;
     int64_t v[kScanItems];
     int64_t s = 0;
@@ -269,9 +279,16 @@ __global__ __launch_bounds__(kScanBlock) void scan_down_kernel(const int64_t* __
     int64_t w = s;
 #pragma unroll
     for (int d = 32; d >= 1; d >>= 1) w += __shfl_xor(w, d, 64);
+    if constexpr (kSumTotals) {
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) before += __shfl_xor(before, d, 64);
+        if (lane == 0) lds_before[wave] = before;
+    }
     if (lane == 0) lds[wave] = w;
     __syncthreads();
-    int64_t carry = block_prefix[blockIdx.x];
+    int64_t carry;
+    if constexpr (kSumTotals) carry = (lds_before[0] + lds_before[1]) + (lds_before[2] + lds_before[3]);
+    else carry = block_prefix[blockIdx.x];
 #pragma unroll
     for (int k = 0; k < kScanBlock / 64; k++) { if (k < wave) carry += lds[k]; }
     // the run itself: an inclusive scan of each round of 64 items on top of the rounds before it
@@ -507,8 +524,12 @@ int ssr_inclusive_sum_i64(const int64_t* in, int64_t* out, int64_t n, int64_t* t
     int64_t* sums = reinterpret_cast<int64_t*>(scratch);
     hipStream_t s = as_stream(stream);
     hipLaunchKernelGGL(scan_reduce_kernel, dim3((unsigned)nb), dim3(kScanBlock), 0, s, in, n, sums);
-    hipLaunchKernelGGL(scan_spine_kernel, dim3(1), dim3(kScanBlock), 0, s, sums, nb);
-    hipLaunchKernelGGL(scan_down_kernel, dim3((unsigned)nb), dim3(kScanBlock), 0, s, in, n, sums, out, total_out);
+    if (nb <= kScanSumBlocks) {
+        hipLaunchKernelGGL(scan_down_kernel<true>, dim3((unsigned)nb), dim3(kScanBlock), 0, s, in, n, sums, out, total_out);
+    } else {
+        hipLaunchKernelGGL(scan_spine_kernel, dim3(1), dim3(kScanBlock), 0, s, sums, nb);
+        hipLaunchKernelGGL(scan_down_kernel<false>, dim3((unsigned)nb), dim3(kScanBlock), 0, s, in, n, sums, out, total_out);
+    }
     SSR_CHECK_LAUNCH("ssr_inclusive_sum_i64");
     return 0;
 }
@@ -526,8 +547,12 @@ int ssr_inclusive_sum_i64_static(const int64_t* in, int64_t* out, int64_t n, int
     const int64_t nb = ceil_div(n, kScanTile);
     hipStream_t s = as_stream(stream);
     hipLaunchKernelGGL(scan_reduce_kernel, dim3((unsigned)nb), dim3(kScanBlock), 0, s, in, n, sums);
-    hipLaunchKernelGGL(scan_spine_kernel, dim3(1), dim3(kScanBlock), 0, s, sums, nb);
-    hipLaunchKernelGGL(scan_down_kernel, dim3((unsigned)nb), dim3(kScanBlock), 0, s, in, n, sums, out, total_out);
+    if (nb <= kScanSumBlocks) {
+        hipLaunchKernelGGL(scan_down_kernel<true>, dim3((unsigned)nb), dim3(kScanBlock), 0, s, in, n, sums, out, total_out);
+    } else {
+        hipLaunchKernelGGL(scan_spine_kernel, dim3(1), dim3(kScanBlock), 0, s, sums, nb);
+        hipLaunchKernelGGL(scan_down_kernel<false>, dim3((unsigned)nb), dim3(kScanBlock), 0, s, in, n, sums, out, total_out);
+    }
     SSR_CHECK_LAUNCH("ssr_inclusive_sum_i64_static");
     return 0;
 }

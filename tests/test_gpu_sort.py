@@ -169,7 +169,7 @@ def test_tile_order(L, n_tiles, closed):
     assert np.all(cls[1:] <= cls[:-1])
 
 
-@pytest.mark.parametrize("n", [1, 2, 255, 256, 2047, 2048, 2049, 1_000_003, 10_000_019])
+@pytest.mark.parametrize("n", [1, 2, 255, 256, 2047, 2048, 2049, 1_000_003, 8_388_608, 8_388_609, 10_000_019])
 def test_inclusive_sum_i64(L, n):
     lib = L.load()
     rng = np.random.default_rng(n)
