@@ -28,10 +28,11 @@ __device__ __forceinline__ uint32_t digit_of(uint64_t key, int shift, uint32_t m
 // peers), and the size of that peer group. One ballot per digit bit set in `varying` (the caller knows
 // the other bits to be the same in every live lane); a lane differs from this one when any bit's vote
 // disagrees with its own bit (vote XOR own bit, OR-ed over the bits).
+template <int kBits = 8>
 __device__ __forceinline__ void wave_match_digit(uint32_t d, uint32_t varying, bool live, uint32_t& rank, uint32_t& group) {
     uint32_t differ_lo = 0, differ_hi = 0;
 #pragma unroll
-    for (int b = 0; b < 8; b++) {
+    for (int b = 0; b < kBits; b++) {
         if ((varying >> b) & 1u) {
             const uint32_t own = (uint32_t)__builtin_amdgcn_sbfe((int)d, (uint32_t)b, 1u);   // 0 or ~0
             const uint64_t vote = __ballot(own != 0u);
@@ -216,9 +217,10 @@ __global__ __launch_bounds__(kSortBlock) void sort_scatter_kernel(
 
 // Ranks the wave's 64 keys of one round by `d` (8 bits): returns the number of earlier keys of this wave
 // with the same digit, and advances the wave's running count (wcount_row = this wave's 256 counters).
+template <int kBits = 8>
 __device__ __forceinline__ uint32_t seg_rank_round(uint32_t d, uint32_t varying, bool live, uint32_t* wcount_row) {
     uint32_t rank, group;
-    wave_match_digit(d, varying, live, rank, group);
+    wave_match_digit<kBits>(d, varying, live, rank, group);
     uint32_t prev = 0;
     if (live) prev = wcount_row[d];
     __builtin_amdgcn_wave_barrier();
@@ -227,27 +229,45 @@ __device__ __forceinline__ uint32_t seg_rank_round(uint32_t d, uint32_t varying,
     return prev + rank;
 }
 
-// Threads 0..255 own one digit each: per-wave counts become the segment-local position of each wave's
-// first key of that digit. Called by the whole workgroup (two barriers inside).
-template <int kWaves>
-__device__ __forceinline__ void seg_digit_bases(uint32_t (*wcount)[kRadix], uint32_t* ws) {
+// Per-wave digit counts become the segment-local position of each wave's first key of that digit. Called by the
+// whole workgroup (barriers inside). With at least as many digits as threads every thread owns a run of consecutive
+// digits; else threads 0..kRadixT-1 own one each.
+// radix_used: the digits in use (kRadixT, or fewer with the same divisibility), the others are not touched.
+template <int kWaves, int kRadixT = kRadix>
+__device__ __forceinline__ void seg_digit_bases(uint32_t (*wcount)[kRadixT], uint32_t* ws, int radix_used = kRadixT) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    if constexpr (kWaves == 1) {   // a lone wavefront: lane l owns digits 4l..4l+3, nothing to wait for
-        uint4 c = reinterpret_cast<uint4*>(wcount[0])[lane];
-        const uint32_t total = c.x + c.y + c.z + c.w;
+    constexpr int kThreads = kWaves * 64;
+    if constexpr (kRadixT >= kThreads) {
+        constexpr int kPer = kRadixT / kThreads;
+        static_assert(kPer * kThreads == kRadixT && kWaves <= kRadix / 64, "whole runs of digits; ws holds one total per wavefront");
+        const int per = radix_used / kThreads;   // this thread's digits: threadIdx.x * per .. + per - 1
+        uint32_t c[kWaves][kPer];
+        uint32_t total = 0;
+#pragma unroll
+        for (int j = 0; j < kPer; j++)
+#pragma unroll
+            for (int w = 0; w < kWaves; w++) { c[w][j] = j < per ? wcount[w][threadIdx.x * per + j] : 0u; total += c[w][j]; }
         uint32_t inc = total;
 #pragma unroll
         for (int d = 1; d < 64; d <<= 1) {
             const uint32_t o = __shfl_up(inc, d, 64);
             if (lane >= d) inc += o;
         }
-        uint4 b;
-        b.x = inc - total; b.y = b.x + c.x; b.z = b.y + c.y; b.w = b.z + c.z;
-        reinterpret_cast<uint4*>(wcount[0])[lane] = b;
+        uint32_t run = inc - total;
+        if constexpr (kWaves > 1) {
+            if (lane == 63) ws[wave] = inc;
+            __syncthreads();   // also: every count is read before any base is written
+#pragma unroll
+            for (int w = 0; w < kWaves; w++) { if (w < wave) run += ws[w]; }
+        }
+#pragma unroll
+        for (int j = 0; j < kPer; j++)
+#pragma unroll
+            for (int w = 0; w < kWaves; w++) { if (j < per) { wcount[w][threadIdx.x * per + j] = run; run += c[w][j]; } }
         __syncthreads();
         return;
     }
-    const bool owner = threadIdx.x < kRadix;
+    const bool owner = threadIdx.x < kRadixT;
     uint32_t total = 0, inc = 0;
     if (owner) {
 #pragma unroll
@@ -264,7 +284,7 @@ __device__ __forceinline__ void seg_digit_bases(uint32_t (*wcount)[kRadix], uint
     if (owner) {
         uint32_t run = inc - total;
 #pragma unroll
-        for (int w = 0; w < kRadix / 64; w++) { if (w < wave) run += ws[w]; }
+        for (int w = 0; w < kRadixT / 64; w++) { if (w < wave) run += ws[w]; }
 #pragma unroll
         for (int w = 0; w < kWaves; w++) {
             const uint32_t c = wcount[w][threadIdx.x];
@@ -289,11 +309,16 @@ __device__ __forceinline__ uint32_t seg_or_all(uint32_t x, uint32_t* wor) {
     return all;
 }
 
+constexpr int kSegWideFrom = 192;   // keys from which a segment takes the wider digits
 // The workgroup (kWaves wavefronts) sorts keys[s, s + len), len <= 64 * kWaves * kRounds, in place on the
-// low 32 key bits: keys in registers, one LDS round trip per digit pass.
-template <int kWaves, int kRounds>
-__device__ __forceinline__ void seg_sort_lds(uint64_t* keys, int32_t* vals, int64_t s, int len, uint32_t (*wcount)[kRadix],
-                                             uint32_t* ws, uint32_t* wor, uint2* buf) {
+// low 32 key bits: keys in registers, one LDS round trip per digit pass. Digits are 8 bits at bits 0, 8, 16, 24;
+// with kDigitBits = 9 (512 counters a wavefront) a segment of kSegWideFrom keys or more whose differing bits fit
+// fewer 9-bit digits takes those, cut evenly over the span (25 depth bits differ across a tile of the 1080p
+// benchmark scene: four 8-bit passes, three 9-bit ones).
+template <int kWaves, int kRounds, int kDigitBits = 8>
+__device__ __forceinline__ void seg_sort_lds(uint64_t* keys, int32_t* vals, int64_t s, int len,
+                                             uint32_t (*wcount)[1 << kDigitBits], uint32_t* ws, uint32_t* wor, uint2* buf) {
+    constexpr int kRadixT = 1 << kDigitBits;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int per_wave = ((len + kWaves - 1) / kWaves + 63) & ~63;   // contiguous run per wave
     const int rounds = per_wave >> 6;
@@ -313,29 +338,40 @@ __device__ __forceinline__ void seg_sort_lds(uint64_t* keys, int32_t* vals, int6
         differ |= key[r] ^ (uint32_t)key0;
     }
     differ = seg_or_all<kWaves>(differ, wor);
-    int last_shift = -1;   // the last pass that moves anything writes straight to the output
-#pragma unroll
-    for (int shift = 0; shift < 32; shift += 8) { if ((differ >> shift) & 255u) last_shift = shift; }
-    if (last_shift < 0) return;   // all keys equal: already in order
+    if (differ == 0) return;   // all keys equal: already in order
+    // 8-bit digits at bits 0, 8, 16, 24, those that are the same in every key skipped; or, where the counters allow
+    // wider digits and that saves a pass on a segment long enough to feel it, equal digits over the span
+    int lsb = 0, width = 8;
+    if constexpr (kDigitBits > 8) {
+        const int lo = __ffs((int)differ) - 1, span = 32 - __clz((int)differ) - lo;
+        const int wide = (span + kDigitBits - 1) / kDigitBits;
+        const int bytes = ((differ & 0xffu) != 0) + ((differ & 0xff00u) != 0) + ((differ & 0xff0000u) != 0) + ((differ >> 24) != 0);
+        if (len >= kSegWideFrom && wide < bytes) { lsb = lo; width = (span + wide - 1) / wide; }
+    }
+    const uint32_t mask = (1u << width) - 1u;
+    const int radix_used = width > 8 ? kRadixT : kRadix;
+    int last_shift = lsb;   // the last pass that moves anything writes straight to the output
+    for (int shift = lsb; shift < 32; shift += width) { if ((differ >> shift) & mask) last_shift = shift; }
 #pragma unroll 1
-    for (int shift = 0; shift <= last_shift; shift += 8) {
-        if (((differ >> shift) & 255u) == 0) continue;
-        wcount[wave][lane] = wcount[wave][lane + 64] = wcount[wave][lane + 128] = wcount[wave][lane + 192] = 0;
+    for (int shift = lsb; shift <= last_shift; shift += width) {
+        if (((differ >> shift) & mask) == 0) continue;
+#pragma unroll
+        for (int e = 0; e < kRadixT / 64; e++) { if (64 * e < radix_used) wcount[wave][lane + 64 * e] = 0; }
         __syncthreads();
 #pragma unroll
         for (int r = 0; r < kRounds; r++) {
             if (r < rounds) {
                 const bool live = first + r * 64 < len;
-                off[r] = seg_rank_round((key[r] >> shift) & 255u, (differ >> shift) & 255u, live, wcount[wave]);
+                off[r] = seg_rank_round<kDigitBits>((key[r] >> shift) & mask, (differ >> shift) & mask, live, wcount[wave]);
             }
         }
         __syncthreads();
-        seg_digit_bases<kWaves>(wcount, ws);
+        seg_digit_bases<kWaves, kRadixT>(wcount, ws, radix_used);
         if (shift == last_shift) {
 #pragma unroll
             for (int r = 0; r < kRounds; r++) {
                 if (r < rounds && first + r * 64 < len) {
-                    const uint32_t pos = wcount[wave][(key[r] >> shift) & 255u] + off[r];
+                    const uint32_t pos = wcount[wave][(key[r] >> shift) & mask] + off[r];
                     keys[s + pos] = ((uint64_t)hi << 32) | key[r];
                     vals[s + pos] = val[r];
                 }
@@ -344,7 +380,7 @@ __device__ __forceinline__ void seg_sort_lds(uint64_t* keys, int32_t* vals, int6
 #pragma unroll
             for (int r = 0; r < kRounds; r++) {
                 if (r < rounds && first + r * 64 < len) {
-                    const uint32_t pos = wcount[wave][(key[r] >> shift) & 255u] + off[r];
+                    const uint32_t pos = wcount[wave][(key[r] >> shift) & mask] + off[r];
                     buf[pos] = make_uint2(key[r], (uint32_t)val[r]);
                 }
             }
@@ -375,6 +411,10 @@ __device__ __forceinline__ int64_t seg_end(const int32_t* __restrict__ tile_offs
     return (tile + 1 < n_tiles || n < 0) ? (int64_t)tile_offsets[tile + 1] : n;
 }
 
+// Digit width of a segment sort: a lone wavefront sorts a segment of several rounds faster in three 9-bit passes than
+// in four 8-bit ones (config 5, 336 keys a tile: 105 -> 83 us); four wavefronts, whose passes are mostly barriers,
+// and short segments do not (measured: +1.5 us on configs 1 and 3, +3.5 on config 4's 100-key tiles).
+template <int kWaves> constexpr int seg_digit_bits() { return kWaves == 1 ? 9 : 8; }
 // One workgroup of kWaves wavefronts per tile: sorts segments of 2..64*kWaves*kRounds keys, lists the
 // longer ones. These kernels are bound by instruction issue: one wavefront per tile executes the fewest
 // instructions per key, but its tiles take long, so it pays only when there are several rounds of
@@ -385,7 +425,7 @@ __global__ __launch_bounds__(kWaves * 64) void sort_segments_direct_kernel(uint6
                                                                            uint32_t n_tiles, int64_t n, SegLists lists) {
     constexpr int kCap = kWaves * 64 * kRounds;
     static_assert(kCap <= kSegCap0, "class 0 starts above the direct kernel's capacity");
-    __shared__ __attribute__((aligned(16))) uint32_t wcount[kWaves][kRadix];
+    __shared__ __attribute__((aligned(16))) uint32_t wcount[kWaves][1 << seg_digit_bits<kWaves>()];
     __shared__ uint32_t ws[kRadix / 64];
     __shared__ uint32_t wor[kWaves];
     __shared__ uint2 buf[kCap];
@@ -402,7 +442,7 @@ __global__ __launch_bounds__(kWaves * 64) void sort_segments_direct_kernel(uint6
         }
         return;
     }
-    seg_sort_lds<kWaves, kRounds>(keys, vals, s, len, wcount, ws, wor, buf);
+    seg_sort_lds<kWaves, kRounds, seg_digit_bits<kWaves>()>(keys, vals, s, len, wcount, ws, wor, buf);
 }
 
 // Workgroups of four wavefronts take the listed segments of class 0 in turn.
