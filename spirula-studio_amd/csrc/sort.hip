@@ -74,30 +74,43 @@ __global__ __launch_bounds__(kSortBlock) void sort_hist_kernel(const uint64_t* _
 __global__ __launch_bounds__(kSortBlock) void sort_scan_rows_kernel(uint32_t* __restrict__ hist, uint32_t n_blocks,
                                                                     uint32_t* __restrict__ totals, int64_t n,
                                                                     const int64_t* __restrict__ n_dev) {
-    __shared__ uint32_t ws[kSortWaves];
+    __shared__ uint32_t ws[2][kSortWaves];   // two sets in turn: one barrier a chunk is enough
     uint32_t* row = hist + (size_t)blockIdx.x * n_blocks;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     uint32_t carry = 0;
     if (n_dev) n = min(n, *n_dev);
     const uint32_t n_used = (uint32_t)((n + kSortTile - 1) / kSortTile);
     n_blocks = min(n_blocks, n_used);
-    for (uint32_t start = 0; start < n_blocks; start += kSortBlock) {
-        const uint32_t i = start + threadIdx.x;
-        const uint32_t v = i < n_blocks ? row[i] : 0;
-        uint32_t inc = v;
+    // a row is a few thousand counts and this kernel nothing but their latency: eight chunks of 256 are loaded
+    // together, then scanned one after the other
+    constexpr int kAhead = 8;
+    int flip = 0;
+    for (uint32_t start = 0; start < n_blocks; start += kSortBlock * kAhead) {
+        uint32_t v[kAhead];
 #pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            const uint32_t o = __shfl_up(inc, d, 64);
-            if (lane >= d) inc += o;
+        for (int k = 0; k < kAhead; k++) {
+            const uint32_t i = start + k * kSortBlock + threadIdx.x;
+            v[k] = i < n_blocks ? row[i] : 0;
         }
-        if (lane == 63) ws[wave] = inc;
-        __syncthreads();
-        uint32_t base = 0, total = 0;
 #pragma unroll
-        for (int w = 0; w < kSortWaves; w++) { if (w < wave) base += ws[w]; total += ws[w]; }
-        if (i < n_blocks) row[i] = carry + base + inc - v;
-        carry += total;
-        __syncthreads();
+        for (int k = 0; k < kAhead; k++) {
+            if (start + k * kSortBlock >= n_blocks) break;   // the same for the whole workgroup
+            const uint32_t i = start + k * kSortBlock + threadIdx.x;
+            uint32_t inc = v[k];
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const uint32_t o = __shfl_up(inc, d, 64);
+                if (lane >= d) inc += o;
+            }
+            if (lane == 63) ws[flip][wave] = inc;
+            __syncthreads();
+            uint32_t base = 0, total = 0;
+#pragma unroll
+            for (int w = 0; w < kSortWaves; w++) { if (w < wave) base += ws[flip][w]; total += ws[flip][w]; }
+            if (i < n_blocks) row[i] = carry + base + inc - v[k];
+            carry += total;
+            flip ^= 1;
+        }
     }
     if (threadIdx.x == 0) totals[blockIdx.x] = carry;
 }
