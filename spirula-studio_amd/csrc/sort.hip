@@ -60,10 +60,16 @@ __global__ __launch_bounds__(kSortBlock) void sort_hist_kernel(const uint64_t* _
     lh[threadIdx.x] = 0;
     __syncthreads();
     const int64_t base = (int64_t)blockIdx.x * kSortTile;
-#pragma unroll 4
+    uint64_t k[kSortRounds];   // all loads ahead of the counting
+#pragma unroll
     for (int r = 0; r < kSortRounds; r++) {
         const int64_t i = base + r * kSortBlock + threadIdx.x;
-        if (i < n) atomicAdd(&lh[digit_of(keys[i], shift, mask)], 1u);
+        k[r] = i < n ? keys[i] : 0;
+    }
+#pragma unroll
+    for (int r = 0; r < kSortRounds; r++) {
+        const int64_t i = base + r * kSortBlock + threadIdx.x;
+        if (i < n) atomicAdd(&lh[digit_of(k[r], shift, mask)], 1u);
     }
     __syncthreads();
     hist[(size_t)threadIdx.x * n_blocks + blockIdx.x] = lh[threadIdx.x];
