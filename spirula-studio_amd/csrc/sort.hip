@@ -130,8 +130,11 @@ __global__ __launch_bounds__(kSortBlock) void sort_scatter_kernel(
     __shared__ uint32_t wcount[kSortWaves][kRadix];   // per-wave running digit counts, then bases
     __shared__ uint32_t ws[kSortWaves], ws2[kSortWaves];
     __shared__ uint32_t s_shift[kRadix];
+    // The pairs pass through LDS in digit order, keys first and the values after them through the same 16 KB:
+    // 21 KB a workgroup leave room for seven of them on a compute unit (29 KB for five), which is one round of
+    // workgroups instead of two for the 3.4 M keys of the 1080p benchmark scene.
     __shared__ uint64_t s_key[kSortTile];
-    __shared__ int32_t s_val[kSortTile];
+    int32_t* s_val = reinterpret_cast<int32_t*>(s_key);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
     for (int w = 0; w < kSortWaves; w++) wcount[w][threadIdx.x] = 0;
@@ -208,23 +211,34 @@ __global__ __launch_bounds__(kSortBlock) void sort_scatter_kernel(
     for (int r = 0; r < kSortRounds; r++) {
         const int64_t i = wave_base + r * 64 + lane;
         if (i < n) {
-            const uint32_t pos = wcount[wave][digit_of(key[r], shift, mask)] + off[r];
-            s_key[pos] = key[r];
-            s_val[pos] = val[r];
+            off[r] = wcount[wave][digit_of(key[r], shift, mask)] + off[r];   // the pair's place in digit order
+            s_key[off[r]] = key[r];
         }
     }
     __syncthreads();
     const int64_t block_base = (int64_t)blockIdx.x * kSortTile;
     const int block_n = (int)(n - block_base < kSortTile ? n - block_base : kSortTile);
+    uint32_t dst[kSortRounds];
 #pragma unroll
     for (int r = 0; r < kSortRounds; r++) {
         const int j = r * kSortBlock + threadIdx.x;
         if (j < block_n) {
             const uint64_t k = s_key[j];
-            const uint32_t pos = s_shift[digit_of(k, shift, mask)] + (uint32_t)j;
-            keys_out[pos] = k;
-            vals_out[pos] = s_val[j];
+            dst[r] = s_shift[digit_of(k, shift, mask)] + (uint32_t)j;
+            keys_out[dst[r]] = k;
         }
+    }
+    __syncthreads();   // the keys are out of LDS
+#pragma unroll
+    for (int r = 0; r < kSortRounds; r++) {
+        const int64_t i = wave_base + r * 64 + lane;
+        if (i < n) s_val[off[r]] = val[r];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < kSortRounds; r++) {
+        const int j = r * kSortBlock + threadIdx.x;
+        if (j < block_n) vals_out[dst[r]] = s_val[j];
     }
 }
 
