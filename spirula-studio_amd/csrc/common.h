@@ -28,6 +28,14 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // uses (tiles.hip); ssr_init calls it so that the first scan does not pay for it.
 int warm_static_scan();
 
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__) && !defined(__gfx942__) && !defined(__gfx90a__)
+#error "lds_wait() encodes s_waitcnt for the gfx9 family: on another target the same bits name other counters"
+#endif
+// Waits until every LDS (and scalar-memory) operation this wavefront has issued is complete: s_waitcnt lgkmcnt(0)
+// in the gfx9 encoding (vmcnt 63, expcnt 7 left alone). Placed ahead of a workgroup barrier that follows
+// non-returning LDS float atomics, whose completion the kernels here do not leave to the compiler.
+__device__ __forceinline__ void lds_wait() { __builtin_amdgcn_s_waitcnt(0xc07f); }
+
 }  // namespace ssr
 
 #define SSR_CHECK_LAUNCH(where)                                       \

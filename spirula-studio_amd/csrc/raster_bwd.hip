@@ -209,7 +209,9 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
             } else {
                 o[0] = m[3]; o[1] = m[0]; o[2] = m[1]; o[3] = m[2]; o[4] = 0.f; o[5] = 0.f;
             }
-            // both threads of a slot sit in one wavefront, so every read above precedes these writes
+            // both threads of a slot sit in one wavefront: order that wavefront's reads above before the writes below
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
             float* dst = s_acc + slot * kCh;
             if (geom) {
                 dst[0] = ssr_isfinite(o[0]) ? o[0] : 0.f; dst[1] = ssr_isfinite(o[1]) ? o[1] : 0.f;
@@ -287,7 +289,7 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
         // Explicit wait for this wavefront's LDS traffic (the read-add-writes and float atomics of the walk):
         // the compiler does not place one ahead of this loop-header barrier on the path that leaves the walk,
         // and a pending float atomic is overtaken by the reads that follow the barrier.
-        __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
+        lds_wait();
         __syncthreads();   // previous batch fully consumed (first pass: the zero fill of s_acc is complete)
         if (!first) flush();   // its sums leave before the slots are reused
         first = false;
@@ -319,10 +321,10 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
             reinterpret_cast<uint64_t*>(s_list + 4 * mt * kB)[lane] = 0x0101010101010101ull * (uint64_t)kB;
         for (int c = 0; c * 64 < n_batch; c++) {
             const int slot = c * 64 + lane;
-            const uint32_t bits = (uint32_t)s_bits[(mt >> 1) * kB + slot] >> (4 * (mt & 1));
+            const uint32_t bits = slot < kB ? (uint32_t)s_bits[(mt >> 1) * kB + slot] >> (4 * (mt & 1)) : 0u;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const bool in = slot < kB && ((bits >> r) & 1u) != 0 && hi - slot <= blk_last[r];
+                const bool in = ((bits >> r) & 1u) != 0 && hi - slot <= blk_last[r];
                 const uint64_t bal = __ballot(in);
                 if (in) s_list[(4 * mt + r) * kB + cnt[r] + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(bal >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)bal, 0u))] = (uint8_t)slot;
                 cnt[r] += __builtin_popcountll(bal);
@@ -523,7 +525,7 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
             k0 = k2; k1 = k3; k2 = k4;
         }
     }
-    __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0), as at the head of the loop
+    lds_wait();   // as at the head of the loop
     __syncthreads();
     if (!first) flush();
 }

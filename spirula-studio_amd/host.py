@@ -40,9 +40,12 @@ SYMBOLS = {
     "ssrh_cache_pointer": (C.c_int, [C.c_int, C.POINTER(vp), C.POINTER(C.c_int64)]),
     "ssrh_last_n_isects": (C.c_int64, []),
     "ssrh_last_n_visible": (C.c_int64, []),
+    "ssrh_short_frames": (C.c_int64, []),
     "ssrh_last_stage_times": (C.c_int, [vp]),
     "ssrh_time_iterations": (C.c_int, [C.c_int, C.c_int, vp, vp, vp, C.c_int, vp]),
     "ssrh_pool_bytes": (C.c_size_t, []),
+    "ssrh_sort_pairs_i64_i32": (C.c_int, [vp, vp, vp, vp, C.c_int64, C.c_int, C.c_int, C.POINTER(C.c_int)]),
+    "ssrh_inclusive_sum_i64": (C.c_int, [vp, vp, C.c_int64]),
 }
 
 _h = None
@@ -244,6 +247,11 @@ class Engine:
         if v == -2:
             check(1)
         return v
+
+    @property
+    def short_frames(self):
+        """Intersections so far that did not fit the arrays they were left to (deferred counts)."""
+        return int(self.h.ssrh_short_frames())
 
     def render(self):
         h, w = self.sc.height, self.sc.width

@@ -50,6 +50,7 @@ int64_t g_bwd_count = 0;
 int64_t g_deferred_capacity = 0;
 int64_t g_deferred_used = 0;          // capacity of the arrays the pending counts belong to
 bool g_counts_pending = false;
+int64_t g_short_frames = 0;           // intersections that did not fit their arrays, counted as they are found out
 int64_t* g_counts_host = nullptr;     // pinned [2]
 ssr_event_t g_counts_event = nullptr;
 const int32_t* g_offsets_closed = nullptr;   // tile_offsets with one more entry, the end of the last tile (null: none)
@@ -240,6 +241,33 @@ float event_elapsed_ms(Event* a, Event* b) {
     return ms;
 }
 
+
+// ---- src/backend/common/SortScan.h:53-60, the two instantiations of the tile-intersection stage ----
+template <>
+void sort_pairs<int64_t, int32_t>(DoubleBuffer<int64_t>& keys, DoubleBuffer<int32_t>& values, int64_t num_items,
+                                  int begin_bit, int end_bit, Stream stream) {
+    if (num_items < 0) throw std::runtime_error("sort_pairs: negative num_items");
+    if (num_items == 0 || end_bit <= begin_bit) return;   // nothing to order: the current buffers already hold the result
+    const size_t bytes = ssr_sort_scratch_bytes(num_items);
+    void* work = DevicePool::global().acquire<uint8_t>(PoolSlot::SeamSortScratch, bytes > 16 ? bytes : 16);
+    int moved = 0;   // 0: the result is where the input was, 1: in the alternate pair
+    if (ssr_sort_pairs_u64_i32(keys.current(), keys.alternate(), values.current(), values.alternate(), num_items, begin_bit,
+                               end_bit, &moved, work, bytes, stream) != 0)
+        throw std::runtime_error(std::string("sort_pairs: ") + ssr_last_error());
+    keys.selector ^= moved;
+    values.selector ^= moved;
+}
+
+template <>
+void inclusive_sum<int64_t>(const int64_t* in, int64_t* out, int64_t num_items, Stream stream) {
+    if (num_items < 0) throw std::runtime_error("inclusive_sum: negative num_items");
+    if (num_items == 0) return;
+    const size_t bytes = ssr_scan_scratch_bytes(num_items);
+    void* work = DevicePool::global().acquire<uint8_t>(PoolSlot::SeamScanScratch, bytes > 16 ? bytes : 16);
+    if (ssr_inclusive_sum_i64(in, out, num_items, nullptr, work, bytes, stream) != 0)
+        throw std::runtime_error(std::string("inclusive_sum: ") + ssr_last_error());
+}
+
 }  // namespace backend
 
 namespace ssr_ext {
@@ -255,6 +283,11 @@ void resolve_counts() {
     const int64_t used = g_deferred_used;
     if (g_n_isects > used) {
         g_deferred_capacity = 0;   // the next intersection reads its count and sizes from it
+        // Counted and left in the sticky error as well: a caller that only renders never asks for the counts, and the
+        // stages that settle them on its behalf must not lose the fact that a frame was short.
+        g_short_frames++;
+        g_sticky = "an intersection of " + std::to_string(g_n_isects) + " entries did not fit the " + std::to_string(used) +
+                   " its arrays were sized for (deferred counts): that frame misses fragments";
         throw std::runtime_error("resolve_counts: " + std::to_string(g_n_isects) + " intersections did not fit the " +
                                  std::to_string(used) + " the arrays were sized for; the images and gradients of this "
                                  "iteration miss fragments: repeat it");
@@ -263,6 +296,7 @@ void resolve_counts() {
 }
 void set_deferred_capacity(int64_t capacity) { g_deferred_capacity = capacity < 0 ? 0 : capacity; }
 int64_t deferred_capacity() { return g_deferred_capacity; }
+int64_t short_frames() { return g_short_frames; }
 int64_t last_n_isects() { resolve_counts(); return g_n_isects; }
 int64_t last_n_visible() { resolve_counts(); return g_n_visible; }
 bool backward_overwrites_all_rows(int64_t num_splats) {
@@ -291,7 +325,7 @@ projection_3dgs_forward(const int64_t num_splats, const int max_sh_degree,
                         DeviceVector<float> radii, const std::optional<TorchTensorView> sh_value_packed,
                         const std::optional<TorchTensorView> sh_value_bounds, const uint32_t num_sh_buffer,
                         const int sh_value_bits, const int64_t sh_bounds_stride) {
-    try { ssr_ext::resolve_counts(); } catch (const std::runtime_error&) {}   // counts of an iteration nobody finished
+    try { ssr_ext::resolve_counts(); } catch (const std::runtime_error&) {}   // an unfinished iteration's counts; a short one stays in short_frames() / last_error()
     ssr_projection_fwd_params p;
     std::memset(&p, 0, sizeof(p));
     p.num_splats = num_splats;
@@ -365,7 +399,7 @@ projection_3dgs_packed_forward(const int64_t num_splats, const int max_sh_degree
                                DeviceVector<float> radii, const std::optional<TorchTensorView> sh_value_packed,
                                const std::optional<TorchTensorView> sh_value_bounds, const uint32_t num_sh_buffer,
                                const int sh_value_bits, const int64_t sh_bounds_stride) {
-    try { ssr_ext::resolve_counts(); } catch (const std::runtime_error&) {}   // counts of an iteration nobody finished
+    try { ssr_ext::resolve_counts(); } catch (const std::runtime_error&) {}   // an unfinished iteration's counts; a short one stays in short_frames() / last_error()
     ssr_projection_packed_params p;
     std::memset(&p, 0, sizeof(p));
     p.num_splats = num_splats;
@@ -545,7 +579,7 @@ do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, 
     if (I < 1) throw std::runtime_error("do_intersect_tile_generic: no image");
     g_tile_order = nullptr; g_tile_order_for = nullptr; g_offsets_closed = nullptr;
     if (g_counts_pending) {   // counts nobody asked for: settle them before the counters are reused
-        try { ssr_ext::resolve_counts(); } catch (const std::runtime_error&) {}
+        try { ssr_ext::resolve_counts(); } catch (const std::runtime_error&) {}   // a short frame stays in short_frames() / last_error()
     }
     const int64_t total = depths.numel();
     const int32_t* img_ids = (image_ids && I > 1) ? image_ids->data_ptr() : nullptr;   // packed rows of several cameras

@@ -17,6 +17,7 @@
 // reference's sort scratch (src/backend/vulkan/SortScanVulkan.cpp:4-6).
 #pragma once
 #include "ssr_host_types.hpp"
+#include "ssr_sortscan.hpp"
 
 std::tuple<DeviceTensor2D<float4>, DeviceTensor2D<float>, std::vector<DeviceTensorFloatND>>
 projection_3dgs_forward(
@@ -110,7 +111,8 @@ void projection_3dgs_backward(
 
 // src/kernels/optim/FusedProjectionBwdOptim.cuh:18-62: every argument is honoured (plain and packed rows,
 // all regularizers, scale-agnostic mean step, colour trust region, quantization levels 0 and 1 with the
-// non-SH quantized moments); one camera per call.
+// non-SH quantized moments); with [C,4,4] cameras the other cameras'
+// world gradients are summed first and one Adam step is taken.
 void fused_projection_bwd_optimizer_3dgs(
     const int64_t num_splats, const int max_sh_degree,
     std::vector<DeviceTensorFloatND> splats_world,
@@ -186,6 +188,8 @@ struct Options {
     // last_n_visible, backward_overwrites_all_rows, projection_3dgs_backward, the fused optimizer) and throws if
     // the count did not fit; the images and gradients of that iteration are then incomplete and the next
     // intersection reads its count again. The first call, and any call with capacity 0, blocks as before.
+    // A caller that only renders asks for none of these: a short frame is then counted in short_frames(), left in
+    // backend::last_error(), and refused by engine_copy_render_to_host.
     bool deferred_counts = false;
     // projection_3dgs_packed_forward also keeps the parameters of every visible splat, 64 bytes in four planes, in the
     // order of the packed rows, and a projection_3dgs_backward that is handed the gaussian_ids and the parameter
@@ -206,6 +210,11 @@ StageTimes last_stage_times();
 int64_t last_n_isects();
 int64_t last_n_visible();   // -1 when the visible list is off
 void resolve_counts();      // see Options::deferred_counts
+// How many intersections so far turned out larger than the arrays they were left to (deferred counts). Each is also
+// reported by the resolve_counts() that finds it (an exception) and left in backend::last_error(); the stages that
+// settle an abandoned iteration's counts swallow the exception, so a caller that only renders learns of a short
+// frame here, or from engine_copy_render_to_host, which settles the counts before it hands out the image.
+int64_t short_frames();
 void set_deferred_capacity(int64_t capacity);
 int64_t deferred_capacity();
 // The list the last projection_3dgs_backward ran over (device pointer) and its length; it stays

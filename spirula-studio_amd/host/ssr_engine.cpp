@@ -68,28 +68,35 @@ void alloc_grad_buffers() {
 
 void set_data_3dgs(int64_t num_splats, TorchTensorView means, TorchTensorView quats, TorchTensorView scales,
                    TorchTensorView opacities, TorchTensorView features_dc, TorchTensorView features_sh) {
+    // Contract of src/engine/EngineSetup.cpp:11-47: the six tensors share their leading extent (the capacity),
+    // num_splats of those rows are live, and only the first call uploads -- later calls just move the counts.
+    struct Named { const char* name; const TorchTensorView* tv; };
+    const Named all[6] = {{"means", &means}, {"quats", &quats}, {"scales", &scales},
+                          {"opacities", &opacities}, {"features_dc", &features_dc}, {"features_sh", &features_sh}};
+    auto rows_of = [](const TorchTensorView& tv) { return std::get<2>(tv).empty() ? int64_t(0) : std::get<2>(tv)[0]; };
+    const int64_t capacity = rows_of(means);
+    for (const Named& t : all)
+        if (rows_of(*t.tv) != capacity)
+            throw std::runtime_error(std::string("set_data_3dgs: '") + t.name + "' has " + std::to_string(rows_of(*t.tv)) +
+                                     " rows where 'means' has " + std::to_string(capacity));
+    if (num_splats > capacity)
+        throw std::runtime_error("set_data_3dgs: num_splats " + std::to_string(num_splats) + " exceeds the " +
+                                 std::to_string(capacity) + " rows given");
     ssr_ext::forget_packed_world_rows();   // new parameter values
-    const int64_t max_num_splats = std::get<2>(means)[0];
-    if (std::get<2>(quats)[0] != max_num_splats || std::get<2>(scales)[0] != max_num_splats ||
-        std::get<2>(opacities)[0] != max_num_splats || std::get<2>(features_dc)[0] != max_num_splats ||
-        std::get<2>(features_sh)[0] != max_num_splats)
-        throw std::runtime_error("setData3DGS: max_num_splats mismatch across splat tensors");
-    if (max_num_splats < num_splats) throw std::runtime_error("setData3DGS: tensor size smaller than num_splats");
-    engine().cur_num_splats = num_splats;
-    engine().max_num_splats = max_num_splats;
-    auto sh_shape = std::get<2>(features_sh);
-    engine().num_sh = sh_shape.size() >= 2 ? (int)sh_shape[1] : 0;
-    if (engine().world.initialized) return;   // set once; later calls are no-ops (EngineSetup.cpp:36-37)
-    auto& w = engine().world;
+    auto& E = engine();
+    const auto& sh_dims = std::get<2>(features_sh);
+    E.num_sh = sh_dims.size() > 1 ? (int)sh_dims[1] : 0;
+    E.max_num_splats = capacity;
+    E.cur_num_splats = num_splats;
+    auto& w = E.world;
+    if (w.initialized) return;
     w.means = hv_to_dv<float3>(PoolSlot::WorldMeans, means);
     w.quats = hv_to_dv<float4>(PoolSlot::WorldQuats, quats);
     w.scales = hv_to_dv<float3>(PoolSlot::WorldScales, scales);
     w.opacities = hv_to_dv<float>(PoolSlot::WorldOpacities, opacities);
     w.features_dc = hv_to_dv<float3>(PoolSlot::WorldFeaturesDc, features_dc);
-    {
-        TorchTensorView d = device_copy_tv(PoolSlot::WorldFeaturesSh, features_sh);
-        w.features_sh = DeviceTensor2D<float3>((float3*)std::get<0>(d), max_num_splats, engine().num_sh);
-    }
+    const TorchTensorView sh_dev = device_copy_tv(PoolSlot::WorldFeaturesSh, features_sh);
+    w.features_sh = DeviceTensor2D<float3>((float3*)std::get<0>(sh_dev), capacity, E.num_sh);
     w.initialized = true;
 }
 
@@ -398,6 +405,9 @@ void engine_copy_params_to_host(TorchTensorView means, TorchTensorView quats, To
 
 void engine_copy_render_to_host(TorchTensorView out_rgb, TorchTensorView out_depth, TorchTensorView out_Ts,
                                 TorchTensorView, TorchTensorView) {
+    // the copies below wait for the device anyway: settle counts that were left there, so that an image whose
+    // intersection did not fit its arrays is refused instead of handed out with fragments missing
+    ssr_ext::resolve_counts();
     auto& f = engine().fwd;
     auto& rgb = std::get<0>(f.renders);
     auto& depth = std::get<1>(f.renders);
@@ -646,6 +656,7 @@ int ssrh_cache_pointer(int which, void** ptr, int64_t* count) {
 
 // -2: the count did not fit the arrays it was left to (deferred counts); the message is in ssrh_last_error
 int64_t ssrh_last_n_isects(void) { int64_t v = -2; guard([&] { v = ssr_ext::last_n_isects(); }); return v; }
+int64_t ssrh_short_frames(void) { return ssr_ext::short_frames(); }
 int64_t ssrh_last_n_visible(void) { int64_t v = -2; guard([&] { v = ssr_ext::last_n_visible(); }); return v; }
 
 int ssrh_last_stage_times(float* out9) {
@@ -679,5 +690,21 @@ int ssrh_time_iterations(int sh_degree, int packed, const float* v_rgb_dev, cons
 }
 
 size_t ssrh_pool_bytes(void) { return DevicePool::global().total_bytes(); }
+
+// The sort / scan seam (ssr_sortscan.hpp) for callers without C++: device arrays in, *selector_out says which
+// buffer of each pair holds the sorted data afterwards (0: keys_current / values_current).
+int ssrh_sort_pairs_i64_i32(int64_t* keys_current, int64_t* keys_alternate, int32_t* values_current, int32_t* values_alternate,
+                            int64_t num_items, int begin_bit, int end_bit, int* selector_out) {
+    return guard([&] {
+        backend::DoubleBuffer<int64_t> keys(keys_current, keys_alternate);
+        backend::DoubleBuffer<int32_t> values(values_current, values_alternate);
+        backend::sort_pairs<int64_t, int32_t>(keys, values, num_items, begin_bit, end_bit);
+        if (keys.selector != values.selector) throw std::runtime_error("sort_pairs left keys and values in different buffers");
+        if (selector_out) *selector_out = keys.selector;
+    });
+}
+int ssrh_inclusive_sum_i64(const int64_t* in, int64_t* out, int64_t num_items) {
+    return guard([&] { backend::inclusive_sum<int64_t>(in, out, num_items); });
+}
 
 }  // extern "C"

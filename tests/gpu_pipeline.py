@@ -8,14 +8,16 @@ import ctypes as C
 import numpy as np
 
 
-WORLD_GRAD_RTOL = 1e-3   # the bar for parameter gradients: 1e-3 of the row's largest entry
+WORLD_GRAD_RTOL = 1e-3   # the bar for parameter gradients, relative, per element
 MARGINS = {}             # label -> largest err / rowmax seen, for the report at the end of a run
 
 
-def world_grad_check(got, ref, n, name, rtol=WORLD_GRAD_RTOL, bad_frac=0.0, scale=None, row_floor=None):
-    """Parameter-gradient bar: |got - ref| <= rtol * max|ref row| + a floor of 2e-5 of the tensor's
-    mean magnitude (rows whose terms cancel). Prints the largest observed error relative to the row
-    maximum, with and without the floor, so that the margin is on record."""
+def world_grad_check(got, ref, n, name, rtol=WORLD_GRAD_RTOL, bad_frac=0.0, scale=None, row_floor=None, elem_floor=None):
+    """Parameter-gradient bar. With elem_floor (oracle_lib.world_grad_floors: what the summation order of the screen
+    gradients can move each element by): per element, |got - ref| <= rtol * |ref| + elem_floor. Without it (runs that
+    have no oracle chain to derive the floor from): |got - ref| <= rtol * max|ref row| + a floor of 2e-5 of the
+    tensor's mean magnitude. Either way the largest error relative to the row maximum is printed, with and without
+    the floor, so that the margin is on record."""
     got = np.asarray(got, np.float64).reshape(n, -1)
     ref = np.asarray(ref, np.float64).reshape(n, -1)
     if scale is None:   # a caller that sums several cameras passes the sum of their row maxima
@@ -28,9 +30,19 @@ def world_grad_check(got, ref, n, name, rtol=WORLD_GRAD_RTOL, bad_frac=0.0, scal
     raw = float((err / scale).max()) if err.size else 0.0
     over = float((np.maximum(err - floor, 0.0) / scale).max()) if err.size else 0.0
     MARGINS[name] = max(MARGINS.get(name, 0.0), over)
-    print(f"  grad {name}: max err/rowmax {raw:.3e}, beyond the floor {over:.3e} (bar {rtol:.0e})", flush=True)
-    bad = err > rtol * scale + floor
-    assert bad.mean() <= bad_frac, (name, over, float(bad.mean()))
+    if elem_floor is None:
+        print(f"  grad {name}: max err/rowmax {raw:.3e}, beyond the floor {over:.3e} (bar {rtol:.0e})", flush=True)
+        bad = err > rtol * scale + floor
+        assert bad.mean() <= bad_frac, (name, over, float(bad.mean()))
+        return
+    ef = np.asarray(elem_floor, np.float64).reshape(n, -1) + 1e-30
+    excess = np.maximum(err - ef, 0.0) / (np.abs(ref) + 1e-300)   # relative error left once the floor is taken off
+    worst = float(excess.max()) if err.size else 0.0
+    print(f"  grad {name}: max err/rowmax {raw:.3e}; per element beyond its floor {worst:.3e} of |ref| (bar {rtol:.0e})", flush=True)
+    bad = err > rtol * np.abs(ref) + ef
+    if bad.mean() > bad_frac:
+        i = np.argwhere(bad)[:4]
+        raise AssertionError((name, int(bad.sum()), [(tuple(ix), got[tuple(ix)], ref[tuple(ix)], ef[tuple(ix)]) for ix in i]))
 
 
 class GpuRun:

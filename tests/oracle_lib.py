@@ -247,6 +247,38 @@ def projection_bwd(scene, aabb, vs, sh_degree=3, pose=False):
     return g
 
 
+_SCREEN_CHANNELS = [("v_xy", 0), ("v_xy", 1), ("v_depth", None), ("v_conic", 0), ("v_conic", 1), ("v_conic", 2),
+                    ("v_opac", None), ("v_rgb", 0), ("v_rgb", 1), ("v_rgb", 2)]   # the order of abs_terms' columns
+
+
+def world_grad_floors(scene, r, sh_degree=3, afrac=2e-6, arith=4e-6):
+    """Per-element floor of the parameter gradients of pipeline result `r`: what the summation-order freedom of the
+    screen gradients becomes after the projection VJP. Screen channel j of a splat is a float sum of terms whose
+    magnitudes add up to abs_terms[:, j]; any order of that sum is right to afrac * abs_terms, and the VJP's own
+    arithmetic to `arith` of |J_ej v_j| per term. The VJP is linear and the splats are independent, so running it on
+    the cotangent (afrac * abs_terms_j + arith * |v_j|) e_j, one screen channel at a time, and adding the magnitudes
+    of the results gives sum_j |J_ej| (afrac abs_terms_j + arith |v_j|) for every element e at once."""
+    vs, aabb, n = r["vscreen"], r["proj"]["aabb"], scene.n
+    ab = vs["abs_terms"]
+    floors = None
+    for j, (name, col) in enumerate(_SCREEN_CHANNELS):
+        one = dict(v_xy=np.zeros((n, 2), np.float32), v_depth=np.zeros(n, np.float32), v_conic=np.zeros((n, 3), np.float32),
+                   v_opac=np.zeros(n, np.float32), v_rgb=np.zeros((n, 3), np.float32))
+        v = vs[name] if col is None else vs[name][:, col]
+        c = (afrac * ab[:, j] + arith * np.abs(v.astype(np.float64))).astype(np.float32)
+        if col is None:
+            one[name][:] = c
+        else:
+            one[name][:, col] = c
+        g = projection_bwd(scene, aabb, one, sh_degree)
+        if floors is None:
+            floors = {k: np.abs(a.astype(np.float64)) for k, a in g.items()}
+        else:
+            for k, a in g.items():
+                floors[k] += np.abs(a.astype(np.float64))
+    return floors
+
+
 HYPER = ["lr_means", "lr_quats", "lr_scales", "lr_opacs", "lr_features_dc", "lr_features_sh", "max_gauss_ratio",
          "scale_regularization_weight", "mcmc_opacity_reg_weight", "mcmc_scale_reg_weight", "quat_norm_reg_weight",
          "sh_reg_weight", "erank_reg_weight", "erank_reg_weight_s3", "color_trust_linear", "eps_tr", "v_in_sh"]

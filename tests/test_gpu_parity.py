@@ -114,18 +114,14 @@ def _compare(gpu, oracle, sc, label, fused_count=False, use_list=False, use_pack
     _grad_close(g.host("v_rgb"), vs["v_rgb"], ab[:, 7:10], "v_rgb", 3 * mb, **kw)
     if mb:   # K9 below would inherit those few rows
         return g, r
-    # K9, fed its own K8 output: compare with the oracle chain under a norm-relative bar
+    # K9, fed its own K8 output, against the oracle chain: 1e-3 relative per element, each element's floor being
+    # what the floors of the ten screen gradients become through the projection VJP
     gr = r["grads"]
+    floors = oracle.world_grad_floors(sc, r, afrac=kw.get("afrac", 2e-6))
     for k, o in [("w_means", "v_means"), ("w_quats", "v_quats"), ("w_log_scales", "v_scales"),
                  ("w_opacity_logits", "v_opacities"), ("w_features_dc", "v_dc"), ("w_features_sh", "v_sh")]:
         got = g.host(k)
-        row_floor = None
-        if k == "w_opacity_logits":
-            # this row is v_opac times the sigmoid's slope, and v_opac is a sum of cancelling terms held to a floor
-            # of 2e-6 of the sum of their magnitudes: the same floor, through the same factor, applies here
-            sg = 1.0 / (1.0 + np.exp(-sc.opacity_logits.astype(np.float64)))
-            row_floor = kw.get("afrac", 2e-6) * ab[:, 6] * sg * (1.0 - sg)
-        world_grad_check(got, gr[o], sc.n, f"{label}/{k}", row_floor=row_floor)
+        world_grad_check(got, gr[o], sc.n, f"{label}/{k}", elem_floor=floors[o])
         assert not np.any(got[~vis]), k
     return g, r
 

@@ -199,3 +199,39 @@ def test_argument_errors(L):
     assert lib.ssr_inclusive_sum_i64(None, None, 5, None, None, 0, None) != 0
     assert lib.ssr_last_error() != b""
     assert lib.ssr_sort_pairs_u64_i32(None, None, None, None, 0, 0, 8, C.byref(sel), None, 0, None) == 0
+
+
+# ---- the same ladder through the backend's C++ seam (backend::DoubleBuffer / sort_pairs / inclusive_sum) ----
+_SEAM_SIZES = [1, 100, 2048, 4097, 1 << 16, (1 << 20) + 123]          # vk_sortscan_test.cpp:185
+_SEAM_BITS = [(0, 64, (1 << 63) - 1), (0, 44, 1 << 44), (0, 49, 1 << 49), (8, 11, 1 << 20)]   # :190-199
+
+
+@pytest.mark.parametrize("n", _SEAM_SIZES)
+def test_seam_sort_pairs_and_scan(L, n):
+    """backend::sort_pairs<int64_t,int32_t> on backend::DoubleBuffer and backend::inclusive_sum<int64_t>
+    (src/backend/common/SortScan.h:42-60) against the stable CPU answers, on the sizes and bit ranges of
+    src/backend/vulkan/tests/vk_sortscan_test.cpp:185-201; the selector names the pair that holds the result."""
+    from spirula_studio_amd import host
+    h = host.load()
+    rng = np.random.default_rng(20260716 + n)
+    for b0, b1, key_range in _SEAM_BITS:
+        keys = rng.integers(0, key_range, n, dtype=np.int64)
+        vals = np.arange(n, dtype=np.int32)
+        kc, ka = L.DeviceArray.from_host(keys), L.DeviceArray((n,), np.int64)
+        vc, va = L.DeviceArray.from_host(vals), L.DeviceArray((n,), np.int32)
+        sel = C.c_int(-1)
+        host.check(h.ssrh_sort_pairs_i64_i32(kc.ptr, ka.ptr, vc.ptr, va.ptr, n, b0, b1, C.byref(sel)))
+        assert sel.value in (0, 1)
+        k, v = (ka, va) if sel.value else (kc, vc)
+        nb = b1 - b0
+        mask = np.uint64(0xFFFFFFFFFFFFFFFF) if nb >= 64 else np.uint64(((1 << nb) - 1) << b0)
+        order = np.argsort(keys.view(np.uint64) & mask, kind="stable")
+        assert np.array_equal(k.to_host(), keys[order]) and np.array_equal(v.to_host(), vals[order])
+    a = rng.integers(0, 1 << 33, n, dtype=np.int64)
+    da, do = L.DeviceArray.from_host(a), L.DeviceArray((n,), np.int64)
+    host.check(h.ssrh_inclusive_sum_i64(da.ptr, do.ptr, n))
+    assert np.array_equal(do.to_host(), np.cumsum(a))
+    # nothing to sort: the current buffers keep the data and the selector stays 0
+    sel = C.c_int(-1)
+    host.check(h.ssrh_sort_pairs_i64_i32(da.ptr, do.ptr, None, None, 0, 0, 44, C.byref(sel)))
+    assert sel.value == 0

@@ -37,8 +37,10 @@ def _static(L, a):
 
 def test_static_scan_matches_the_scratch_scan_twice(L):
     rng = np.random.default_rng(77)
-    # 3 000 017 elements use 1465 block sums; the second call uses 5 of them and must not see the rest
-    for n in (3_000_017, 9_001):
+    # 3 000 017 elements use 1465 block sums; the second call uses 5 of them and must not see the rest. 8 388 609
+    # elements are 4097 blocks, one more than a workgroup adds up for itself: the spine kernel then rewrites the
+    # static array in place, and the smaller call after it must see nothing of that either.
+    for n in (3_000_017, 9_001, 8_388_609, 70_001):
         a = rng.integers(0, 1 << 20, n, dtype=np.int64)
         a[::5] = 0
         a[3] = 1 << 41   # beyond 32 bits
