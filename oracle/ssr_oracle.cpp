@@ -1295,6 +1295,7 @@ void or_raster_bwd_ex(int64_t N, const float* xy, const float* depth, const floa
             int32_t bin_final[64];
             float Cc[64][4], Sc[64][4], vD[64][4], Wd[64], amap[64];
             float med_v[64], pend_zgrad[64], pend_zfar[64], pend_Tfar[64];
+            int undo_steps[64] = {0};   // per pixel: how many times T has been divided by (1 - alpha) so far
             for (int p = 0; p < 64; p++) {
                 const int pxi = bx + p % kMicro, pyi = by + p / kMicro;
                 const bool inside = pxi < (int)width && pyi < (int)height;
@@ -1393,6 +1394,11 @@ void or_raster_bwd_ex(int64_t N, const float* xy, const float* depth, const floa
                     }
                     vcol[3] += v_depth_median;
                     float t[10] = {0};
+                    // v_alpha is a difference, T0 (c . v_c) - v_T1 T0, often of nearly equal numbers: what rounding
+                    // moves in it scales with the two products, not with what is left of them. For the magnitude sums
+                    // the six channels that are linear in v_alpha are therefore taken at |T0 (c . v_c)| + |v_T1 T0|.
+                    const float v_alpha_mag = ssr_fabs(T0 * dotcv) + ssr_fabs(vT1p * T0);
+                    float tmag[10] = {0};
                     if (sigma >= 0.f && f.opac * vis <= 0.999f) {
                         const float v_sigma = (-f.opac) * vis * v_alpha;
                         t[3] = 0.5f * v_sigma * dx * dx;
@@ -1401,10 +1407,25 @@ void or_raster_bwd_ex(int64_t N, const float* xy, const float* depth, const floa
                         t[0] = v_sigma * (f.cx * dx + f.cy * dy);
                         t[1] = v_sigma * (f.cy * dx + f.cz * dy);
                         t[6] = vis * v_alpha;
+                        const float m_sigma = f.opac * vis * v_alpha_mag;
+                        tmag[3] = 0.5f * m_sigma * dx * dx;
+                        tmag[4] = ssr_fabs(m_sigma * dx * dy);
+                        tmag[5] = 0.5f * m_sigma * dy * dy;
+                        tmag[0] = m_sigma * (ssr_fabs(f.cx * dx) + ssr_fabs(f.cy * dy));
+                        tmag[1] = m_sigma * (ssr_fabs(f.cy * dx) + ssr_fabs(f.cz * dy));
+                        tmag[6] = vis * v_alpha_mag;
                     }
                     t[7] = vcol[0]; t[8] = vcol[1]; t[9] = vcol[2]; t[2] = vcol[3];
+                    tmag[7] = ssr_fabs(vcol[0]); tmag[8] = ssr_fabs(vcol[1]); tmag[9] = ssr_fabs(vcol[2]); tmag[2] = ssr_fabs(vcol[3]);
                     for (int q = 0; q < 10; q++) acc[q] += t[q];
-                    if (abs_terms) for (int q = 0; q < 10; q++) aacc[q] += std::fabs((double)t[q]);
+                    // Every term carries the rounding of the undo steps that produced its T0 and v_T1 (a division and
+                    // a product each, about two ulp a step, 1.2e-7): with the 2e-6 of the magnitude sum that tests
+                    // allow for summation order, a term n steps deep counts (1 + 0.06 n) times.
+                    if (abs_terms) {
+                        const double deep = 1.0 + 0.06 * undo_steps[p];
+                        for (int q = 0; q < 10; q++) aacc[q] += (double)ssr_max(ssr_fabs(t[q]), tmag[q]) * deep;
+                    }
+                    undo_steps[p]++;
                     if (accum_mode == 1) aw = ssr_max(aw, amap[p] * w);   // :553-562
                     else if (accum_mode) { aw += amap[p] * w; if (accum_mode == 3) aw_den += w; }
                     T1[p] = T0; vT1[p] = v_T0;

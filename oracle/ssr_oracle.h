@@ -104,7 +104,9 @@ void or_raster_bwd(int64_t N, const float* xy, const float* depth, const float* 
     const float* render_T, const int32_t* last_ids, const float* render_depth,
     const float* v_rgb, const float* v_depth, const float* v_T,
     float* v_xy, float* v_sdepth, float* v_conic, float* v_opac, float* v_srgb,
-    double* abs_terms /* [N,10] or NULL */);
+    double* abs_terms /* [N,10] or NULL: per output element the sum of term magnitudes (1 + 0.06 n), n = transmittance
+                         undo steps behind the term, a term that is linear in v_alpha taken at |T0 (c.v_c)| + |v_T1 T0|
+                         in place of their difference; 2e-6 of it bounds what summation order and rounding move */);
 
 /* K7 / K8 with their variants. dist_type: 0 none, 1 depth (D), 2 rgb + depth (RGB_D).
  * Forward: out_dist_rgb [H,W,3] (RGB_D), out_dist_depth [H,W] (D, RGB_D), out_median [H,W] or NULL.

@@ -27,6 +27,8 @@
 // exp(-sigma) comes from the hardware exponential; whenever a lane's alpha falls within 1.6e-7 of the 1/255
 // threshold or within 4e-5 of the 0.999 gate, the wavefront re-evaluates with the bit-defined exponential, so every
 // decision is the one the forward took.
+#include <stdlib.h>
+
 #include "raster_device.h"
 
 namespace ssr {
@@ -609,7 +611,10 @@ extern "C" int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t strea
         default: SSR_ROWS(D, M, SSR_ACCUM_NONE); break;             \
     }
 #define SSR_ROWS_M(D) if (med) { SSR_ROWS_A(D, true) } else { SSR_ROWS_A(D, false) }
-    if (p->dist_type == SSR_DIST_NONE && !med && p->accum_mode == SSR_ACCUM_AVG)
+    static const bool rows_only = getenv("SSR_BWD_ROWS") != nullptr;   // measurement switch: the row kernel for the plain variant too
+    if (p->dist_type == SSR_DIST_NONE && !med && p->accum_mode == SSR_ACCUM_NONE && !rows_only)
+        launch_raster_bwd_lanes(*p, tw, th, nimg, st);
+    else if (p->dist_type == SSR_DIST_NONE && !med && p->accum_mode == SSR_ACCUM_AVG)
         hipLaunchKernelGGL(raster_bwd_rows_avg_kernel, grid, block, 0, st, *p, tw, th);
     else switch (p->dist_type) {
         case SSR_DIST_D: SSR_ROWS_M(SSR_DIST_D); break;

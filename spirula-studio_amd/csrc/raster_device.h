@@ -251,4 +251,7 @@ __device__ __forceinline__ int tile_of_workgroup(const int32_t* __restrict__ ord
     return wg < n_tiles ? order[wg] : -1;
 }
 
+// K8's plain variant with one lane per fragment (raster_bwd_lanes.hip); validated arguments, launch only.
+int launch_raster_bwd_lanes(const ssr_raster_bwd_params& p, int tw, int th, int nimg, hipStream_t st);
+
 }  // namespace ssr

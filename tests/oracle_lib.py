@@ -251,13 +251,25 @@ _SCREEN_CHANNELS = [("v_xy", 0), ("v_xy", 1), ("v_depth", None), ("v_conic", 0),
                     ("v_opac", None), ("v_rgb", 0), ("v_rgb", 1), ("v_rgb", 2)]   # the order of abs_terms' columns
 
 
-def world_grad_floors(scene, r, sh_degree=3, afrac=2e-6, arith=4e-6):
-    """Per-element floor of the parameter gradients of pipeline result `r`: what the summation-order freedom of the
-    screen gradients becomes after the projection VJP. Screen channel j of a splat is a float sum of terms whose
-    magnitudes add up to abs_terms[:, j]; any order of that sum is right to afrac * abs_terms, and the VJP's own
-    arithmetic to `arith` of |J_ej v_j| per term. The VJP is linear and the splats are independent, so running it on
-    the cotangent (afrac * abs_terms_j + arith * |v_j|) e_j, one screen channel at a time, and adding the magnitudes
-    of the results gives sum_j |J_ej| (afrac abs_terms_j + arith |v_j|) for every element e at once."""
+def world_grad_floors(scene, r, sh_degree=3, afrac=2e-6, arith=4e-6, sens_draws=3, sens_rel=6e-7, sens_factor=4.0, row_ulps=32):
+    """Per-element floor of the parameter gradients of pipeline result `r`: how far two correct float32 evaluations
+    of the same chain may lie apart in that element. Two parts.
+
+    (a) What the summation-order freedom of the screen gradients becomes after the projection VJP. Screen channel j
+    of a splat is a float sum of terms whose magnitudes add up to abs_terms[:, j]; any order of that sum is right to
+    afrac * abs_terms, and the VJP's last sum to `arith` of |J_ej v_j| per term. The VJP is linear and the splats are
+    independent, so running it on the cotangent (afrac * abs_terms_j + arith * |v_j|) e_j, one screen channel at a
+    time, and adding the magnitudes of the results gives sum_j |J_ej| (afrac abs_terms_j + arith |v_j|) for every
+    element e at once.
+
+    (b) The conditioning of the VJP itself: an element that is a small difference of large intermediate products
+    (a scale gradient is a quadratic form of an indefinite matrix, say) is not defined to 1e-3 by float32 arithmetic
+    in any order. A backward-stable evaluation returns the exact result for inputs moved by a few ulp, so the
+    spread between correct evaluations is bounded by the element's sensitivity to such moves: the VJP is re-run
+    `sens_draws` times with every parameter and screen gradient multiplied by 1 +- sens_rel (about five ulp, random
+    signs) and sens_factor times the largest change seen is added to the floor. A well-conditioned element moves by
+    1e-6 of itself, far below the 1e-3 bar; one that cancels a thousandfold gets the thousandfold floor."""
+    import copy
     vs, aabb, n = r["vscreen"], r["proj"]["aabb"], scene.n
     ab = vs["abs_terms"]
     floors = None
@@ -276,6 +288,33 @@ def world_grad_floors(scene, r, sh_degree=3, afrac=2e-6, arith=4e-6):
         else:
             for k, a in g.items():
                 floors[k] += np.abs(a.astype(np.float64))
+    base = {k: a.astype(np.float64) for k, a in projection_bwd(scene, aabb, vs, sh_degree).items()}
+    rng = np.random.default_rng(20261125)
+    jiggle = lambda a: (a.astype(np.float64) * (1.0 + sens_rel * rng.choice([-1.0, 1.0], a.shape))).astype(np.float32)
+    spread = {k: np.zeros_like(a) for k, a in base.items()}
+    for _ in range(sens_draws):
+        sc2 = copy.copy(scene)
+        for k in ["means", "quats", "log_scales", "opacity_logits", "features_dc"]:
+            setattr(sc2, k, jiggle(getattr(scene, k)))
+        if getattr(scene, "sh_codec", 0) == 0 and getattr(scene, "features_sh", None) is not None:
+            sc2.features_sh = jiggle(scene.features_sh)
+        vs2 = {k: jiggle(vs[k]) for k in ["v_xy", "v_depth", "v_conic", "v_opac", "v_rgb"]}
+        g = projection_bwd(sc2, aabb, vs2, sh_degree)
+        for k, a in g.items():
+            spread[k] = np.maximum(spread[k], np.abs(a.astype(np.float64) - base[k]))
+    for k in floors:
+        floors[k] += sens_factor * spread[k]
+        # (c) the components of one row come out of shared matrix products (a quaternion gradient is tangent to the
+        # unit sphere, a scale gradient a diagonal of R^T M R): each inherits roundings of the size of an ulp of the
+        # row's largest entry, whatever its own size. row_ulps ulp of that entry are added (2e-6 of it, against the
+        # 1e-3 of the row maximum that a norm-wise bar would allow).
+        # (An SH gradient is basis value times colour gradient, entry by entry: what its entries share is the
+        # direction polynomial, so its "row" is the fifteen coefficients of one colour channel.)
+        if base[k].ndim == 3:
+            floors[k] += row_ulps * 6e-8 * np.abs(base[k]).max(axis=1, keepdims=True)
+        else:
+            rows = np.abs(base[k]).reshape(n, -1).max(axis=1)
+            floors[k] += (row_ulps * 6e-8 * rows).reshape((n,) + (1,) * (base[k].ndim - 1))
     return floors
 
 
