@@ -43,6 +43,29 @@ def algorithmic_bytes(N, V, K, K_f, K_b, P, T, S, sort_sweeps):
     }
 
 
+def done_bytes(ab, N, V, K, T, S, sort_sweeps_done, fused_count, tile_sort, listed, packed, k9_all_rows, world_rows):
+    """The same table for the work this build's stage order really does (the contract figures above price the
+    reference's stage order): the key array swept `sort_sweeps_done` times, no separate count pass when the projection
+    counts tiles itself, K4 and K9 over the visible rows only when a work list or the packed rows drive them, and K9's
+    gradient rows written once -- all N of them when the launch covers every splat (it stores zeros for culled
+    ones, so nothing is zero-filled beforehand), else the V visible ones plus as many re-zeroed from the iteration
+    before."""
+    d = dict(ab)
+    if fused_count:
+        d["K2"] = 0
+    rows = V if packed else N                      # rows the scan and the key write run over
+    d["K3"] = rows * 16
+    d["K4"] = (V * (4 if listed else 0) + (V if (listed or packed) else N) * 16 + V * 44 + K * 12)
+    d["K5"] = sort_sweeps_done * K * 24 + (K * 8 + T * 4 if tile_sort else 0)
+    if tile_sort:
+        d["K6"] = 0
+    reads = (V * (4 if listed else 0) if (listed or packed) else N * 16) + V * (56 + S + 40)
+    if packed and world_rows:
+        reads += 0                                 # the parameter planes replace the gathers one for one
+    d["K9"] = reads + (N * 236 if k9_all_rows else V * 236 * 2)
+    return d
+
+
 def tile_need(offsets, last_ids, n_isects, width, height):
     """K_b: per tile, (largest last_id over its pixels) - range start + 1, summed over tiles."""
     import numpy as np
@@ -111,72 +134,9 @@ def cpu_baseline(pkg, cfg, sc):
     return out, int(res["fwd"]["K_f"])
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--config", type=int, default=2, help="1..5 (BASELINE.json configs; 2 is the headline)")
-    ap.add_argument("--n", type=int, default=None, help="override the number of Gaussians")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--reference-order", action="store_true",
-                    help="run the stages exactly as the reference does (separate count pass, atomic K9 into zero-filled buffers)")
-    ap.add_argument("--whole-key-sort", action="store_true",
-                    help="six whole-array digit passes + the offsets kernel instead of the tile-segmented sort")
-    ap.add_argument("--lens", choices=["none", "opencv", "thin_prism", "rational"], default="none",
-                    help="widened row: the scene's camera with a lens-distortion tier (mild preset coefficients)")
-    ap.add_argument("--fisheye", action="store_true",
-                    help="widened row: view the scene through an equidistant fisheye spanning 180 degrees of the image width")
-    ap.add_argument("--packed-projection", action="store_true",
-                    help="run the packed form of the projection (compacted nnz-row outputs; the reference's training default)")
-    ap.add_argument("--dense-projection", action="store_true",
-                    help="config 4: keep the [N]-row projection outputs instead of the packed rows its sparse view defaults to")
-    ap.add_argument("--fused-optimizer", action="store_true",
-                    help="backward = compositing backward + projection backward fused with the Adam step "
-                         "(the reference's FPBO mode); K9 then includes the optimizer's 1.4 kB/splat of traffic")
-    ap.add_argument("--quantization-level", type=int, default=0, choices=[0, 1],
-                    help="with --fused-optimizer: 1 = SH values as 16-bit codes and their Adam moments as 8-bit cells "
-                         "(the reference's default level); the scene's SH is then stored at 16 bits, one bound per 256 splats")
-    ap.add_argument("--scale-agnostic-mean", action="store_true", help="with --fused-optimizer: the scale-agnostic step of the means")
-    ap.add_argument("--mip", action="store_true", help="the antialiased primitive (blur 0.1, opacity compensation)")
-    ap.add_argument("--non-sh-optim-bits", type=int, default=32, choices=[32, 16],
-                    help="with --quantization-level 1: 16 = the moments of the non-SH tensors as 16-bit cells too (what the reference's trainer sets)")
-    ap.add_argument("--dist-type", type=int, default=0, help="compositing variant: 1 depth distortion, 2 rgb + depth distortion")
-    ap.add_argument("--median", action="store_true", help="compositing variant: also render the median depth and back-propagate it")
-    ap.add_argument("--accum-mode", type=int, default=0, help="compositing variant: accumulate a pixel weight map per splat (1 max, 2 sum, 3 avg)")
-    ap.add_argument("--packed-world-rows", action="store_true",
-                    help="with the packed projection: keep the visible splats' parameters (64 bytes each) for the projection backward")
-    ap.add_argument("--no-packed-world-rows", action="store_true", help="config 4: gather the parameters in the projection backward")
-    ap.add_argument("--deferred-counts", action="store_true",
-                    help="after the first iteration the forward does not wait for the intersection count: key arrays sized "
-                         "from the previous count, overflow checked before the backward uses the counts")
-    ap.add_argument("--cameras", type=int, default=1,
-                    help="render C cameras per iteration in one call ([C,N] layout, plain path only); an iteration is then C images")
-    ap.add_argument("--copy-calibration", action="store_true",
-                    help="run device copies / fills of known size (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE) and exit")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build runs on one GPU; --gpus must be 1 (the path has no multi-GPU part)", file=sys.stderr)
-        sys.exit(2)
-
-    import numpy as np
-
-    import ssr_pkg
-    pkg = ssr_pkg.load()
-    from spirula_studio_amd import host, lib
-
-    if args.copy_calibration:
-        L = lib.load()
-        lib.check(L.ssr_init(0))
-        nbytes = 1 << 30
-        a, b = lib.DeviceArray((nbytes,), np.uint8), lib.DeviceArray((nbytes,), np.uint8)
-        for _ in range(5):
-            lib.check(L.ssr_fill_u32(a.ptr, 1, nbytes // 4, None))          # writes 1 GiB
-            lib.check(L.ssr_memcpy(b.ptr, a.ptr, nbytes, lib.D2D, None, 1))  # reads 1 GiB, writes 1 GiB
-        lib.check(L.ssr_device_synchronize())
-        print(json.dumps({"copy_calibration_bytes": nbytes, "launches": 5}))
-        return
-
+def run_config(args, pkg, host, lib, np, with_cpu):
+    """One configuration: builds the scene, times args.steps iterations, and returns the JSON object."""
+    L = lib.load()
     cfg = args.config
     # config 4 looks out from inside the scene and sees an eighth of it: the reference's packed projection (compacted
     # nnz-row outputs) is its mode for such views and the faster one here, so it is this config's default
@@ -220,7 +180,6 @@ def main():
                       overwrite_world_grads=native, packed_projection=args.packed_projection, packed_vscreen=native,
                       tile_sort=native and not args.whole_key_sort, deferred_counts=args.deferred_counts,
                       packed_world_rows=args.packed_world_rows)
-    L = lib.load()
 
     hyper = dict(lr_means=1.6e-6, lr_quats=1e-5, lr_scales=5e-5, lr_opacs=5e-4, lr_features_dc=2.5e-5, lr_features_sh=1.25e-6)
     adam_step = [0]
@@ -297,7 +256,7 @@ def main():
     # taken from the cpu_baseline leg when that runs on this very scene, else bounded below by K_b
     K_f, cpu = K_b, None
     plain_scene = not (args.fisheye or args.lens != "none" or args.mip or ncam > 1 or args.n)
-    if not args.no_cpu_baseline:
+    if with_cpu:
         if plain_scene and not (args.fused_optimizer and args.quantization_level == 1):
             cpu, K_f = cpu_baseline(pkg, cfg, sc)
         else:
@@ -312,8 +271,15 @@ def main():
         ab["K5"] += ab["K6"]
         ab["K6"] = 0
     total_bytes = sum(ab.values())
+    # ... and what this stage order really moves (done_bytes): K9 covers every row when the engine says its launch
+    # overwrites them all (store mode, not packed, no list or a list holding half the splats)
+    listed = native and not args.packed_projection
+    k9_all_rows = (not native) or (not args.packed_projection and V * 2 >= ncam * sc.n)
+    abd = done_bytes(ab, ncam * sc.n, V, K, T, S, sort_sweeps_done, fused_count=native, tile_sort=tile_sort, listed=listed,
+                     packed=args.packed_projection, k9_all_rows=k9_all_rows, world_rows=args.packed_world_rows) if native else dict(ab)
+    total_done = sum(abd.values())
     dom = max(acc, key=acc.get)
-    dom_gbs = ab[dom] / (acc[dom] * 1e-3) / 1e9 if acc[dom] > 0 else 0.0
+    dom_gbs = abd[dom] / (acc[dom] * 1e-3) / 1e9 if acc[dom] > 0 else 0.0
     traffic = None
     valu_inst = None     # profiled VALU wavefront instructions per launch of the dominant kernel
     prof = {}
@@ -367,16 +333,21 @@ def main():
                                   + (f", compositing variants dist_type={args.dist_type} median={int(args.median)} accum_mode={args.accum_mode}" if variants else "")
                                   + (f", loss map accumulated per splat (accum_mode={args.accum_mode})" if fused_accum else ""),
                    "device_ms_per_iter_median": float(np.median(ms))},
+        # two byte counts: the contract's (the reference's stage order: whole-key sort sweeps, a separate count pass,
+        # zero-filled gradient buffers) and the bytes of the work this stage order does; each over the same time
         "hbm_roofline_frac_whole_iteration": total_bytes / (float(np.median(ms)) * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "hbm_roofline_frac_whole_iteration_done": total_done / (float(np.median(ms)) * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "algorithmic_bytes_per_iter": total_bytes,
+        "algorithmic_bytes_done": total_done,
+        "stage_algorithmic_bytes_done": {k: int(abd[k]) for k in acc},
         "sort_sweeps": {"charged": sort_sweeps, "done": sort_sweeps_done},
         "sort": sort_info,
         "atomics": atomic_info,
         "stage_ms": {k: round(v, 4) for k, v in acc.items()},
-        "stage_algorithmic_GBs": {k: round(ab[k] / (acc[k] * 1e-3) / 1e9, 1) if acc[k] > 0 and ab[k] > 0 else None for k in acc},
+        "stage_algorithmic_GBs": {k: round(abd[k] / (acc[k] * 1e-3) / 1e9, 1) if acc[k] > 0 and abd[k] > 0 else None for k in acc},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": dom_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": dom_gbs / HBM_PEAK_GBS, "traffic": traffic,
-                     "algorithmic_bytes_per_launch": ab[dom], "avg_launch_ms": acc[dom]},
+                     "algorithmic_bytes_per_launch": abd[dom], "avg_launch_ms": acc[dom]},
     }
     if valu_inst:
         # the dominant kernel is bound by vector-instruction issue, which neither "hbm" nor "mfma" names: a wavefront
@@ -385,6 +356,100 @@ def main():
                                          "frac_of_issue_slots": valu_inst * 4 / 1024 / (acc[dom] * 1e-3 * 2.4e9)}
     if cpu is not None:
         out["cpu_baseline"] = cpu   # one camera of the configuration
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", type=int, default=2, help="1..5 (BASELINE.json configs; 2 is the headline)")
+    ap.add_argument("--n", type=int, default=None, help="override the number of Gaussians")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--reference-order", action="store_true",
+                    help="run the stages exactly as the reference does (separate count pass, atomic K9 into zero-filled buffers)")
+    ap.add_argument("--whole-key-sort", action="store_true",
+                    help="six whole-array digit passes + the offsets kernel instead of the tile-segmented sort")
+    ap.add_argument("--lens", choices=["none", "opencv", "thin_prism", "rational"], default="none",
+                    help="widened row: the scene's camera with a lens-distortion tier (mild preset coefficients)")
+    ap.add_argument("--fisheye", action="store_true",
+                    help="widened row: view the scene through an equidistant fisheye spanning 180 degrees of the image width")
+    ap.add_argument("--packed-projection", action="store_true",
+                    help="run the packed form of the projection (compacted nnz-row outputs; the reference's training default)")
+    ap.add_argument("--dense-projection", action="store_true",
+                    help="config 4: keep the [N]-row projection outputs instead of the packed rows its sparse view defaults to")
+    ap.add_argument("--fused-optimizer", action="store_true",
+                    help="backward = compositing backward + projection backward fused with the Adam step "
+                         "(the reference's FPBO mode); K9 then includes the optimizer's 1.4 kB/splat of traffic")
+    ap.add_argument("--quantization-level", type=int, default=0, choices=[0, 1],
+                    help="with --fused-optimizer: 1 = SH values as 16-bit codes and their Adam moments as 8-bit cells "
+                         "(the reference's default level); the scene's SH is then stored at 16 bits, one bound per 256 splats")
+    ap.add_argument("--scale-agnostic-mean", action="store_true", help="with --fused-optimizer: the scale-agnostic step of the means")
+    ap.add_argument("--mip", action="store_true", help="the antialiased primitive (blur 0.1, opacity compensation)")
+    ap.add_argument("--non-sh-optim-bits", type=int, default=32, choices=[32, 16],
+                    help="with --quantization-level 1: 16 = the moments of the non-SH tensors as 16-bit cells too (what the reference's trainer sets)")
+    ap.add_argument("--dist-type", type=int, default=0, help="compositing variant: 1 depth distortion, 2 rgb + depth distortion")
+    ap.add_argument("--median", action="store_true", help="compositing variant: also render the median depth and back-propagate it")
+    ap.add_argument("--accum-mode", type=int, default=0, help="compositing variant: accumulate a pixel weight map per splat (1 max, 2 sum, 3 avg)")
+    ap.add_argument("--packed-world-rows", action="store_true",
+                    help="with the packed projection: keep the visible splats' parameters (64 bytes each) for the projection backward")
+    ap.add_argument("--no-packed-world-rows", action="store_true", help="config 4: gather the parameters in the projection backward")
+    ap.add_argument("--deferred-counts", action="store_true",
+                    help="after the first iteration the forward does not wait for the intersection count: key arrays sized "
+                         "from the previous count, overflow checked before the backward uses the counts")
+    ap.add_argument("--cameras", type=int, default=1,
+                    help="render C cameras per iteration in one call ([C,N] layout, plain path only); an iteration is then C images")
+    ap.add_argument("--no-all-configs", action="store_true",
+                    help="headline run only: leave out the short runs of the other four configurations (all_configs)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run device copies / fills of known size (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE) and exit")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus must be 1 (the path has no multi-GPU part)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+
+    import ssr_pkg
+    pkg = ssr_pkg.load()
+    from spirula_studio_amd import host, lib
+
+    if args.copy_calibration:
+        L = lib.load()
+        lib.check(L.ssr_init(0))
+        nbytes = 1 << 30
+        a, b = lib.DeviceArray((nbytes,), np.uint8), lib.DeviceArray((nbytes,), np.uint8)
+        for _ in range(5):
+            lib.check(L.ssr_fill_u32(a.ptr, 1, nbytes // 4, None))          # writes 1 GiB
+            lib.check(L.ssr_memcpy(b.ptr, a.ptr, nbytes, lib.D2D, None, 1))  # reads 1 GiB, writes 1 GiB
+        lib.check(L.ssr_device_synchronize())
+        print(json.dumps({"copy_calibration_bytes": nbytes, "launches": 5}))
+        return
+
+    default_plain = not (args.reference_order or args.whole_key_sort or args.lens != "none" or args.fisheye or args.packed_projection
+                         or args.dense_projection or args.fused_optimizer or args.mip or args.dist_type or args.median
+                         or args.accum_mode or args.packed_world_rows or args.no_packed_world_rows or args.deferred_counts
+                         or args.cameras != 1 or args.n)
+    out = run_config(args, pkg, host, lib, np, with_cpu=not args.no_cpu_baseline)
+    if default_plain and not args.no_all_configs:
+        # the other four configurations of BASELINE.json, a short run each in this same process (no CPU leg; K_f then
+        # stands at its lower bound K_b): iterations/s and both roofline fractions per configuration
+        import copy
+        rows = []
+        for c in [1, 2, 3, 4, 5]:
+            if c == args.config:
+                r = out
+            else:
+                a2 = copy.copy(args)
+                a2.config, a2.steps, a2.warmup = c, min(args.steps, 10), min(args.warmup, 2)
+                r = run_config(a2, pkg, host, lib, np, with_cpu=False)
+            dom = r["roofline"]["kernel"]
+            rows.append({"workload": r["config"]["workload"], "ms_per_step": r["ms_per_step"], "iters_per_s": r["value"],
+                         "steps": r["steps"], "frac_contract": r["hbm_roofline_frac_whole_iteration"],
+                         "frac_done": r["hbm_roofline_frac_whole_iteration_done"], "dominant_kernel": dom,
+                         "dominant_kernel_ms": r["stage_ms"][dom], "dominant_kernel_frac": r["roofline"]["frac"]})
+        out["all_configs"] = rows
     print(json.dumps(out))
 
 

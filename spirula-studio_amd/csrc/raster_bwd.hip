@@ -27,8 +27,6 @@
 // exp(-sigma) comes from the hardware exponential; whenever a lane's alpha falls within 1.6e-7 of the 1/255
 // threshold or within 4e-5 of the 0.999 gate, the wavefront re-evaluates with the bit-defined exponential, so every
 // decision is the one the forward took.
-#include <stdlib.h>
-
 #include "raster_device.h"
 
 namespace ssr {
@@ -356,25 +354,40 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
         auto step = [&](int st, int k, const float4& q0, const float4& q1, const float2& q2, float cut) {
             const float dx = q0.x - px, dy = q0.y - py;
             const float sigma = ssr_fma(q0.z * dx, dx, ssr_fma(q1.x * dy, dy, (q0.w * dx) * dy));
-            // a lane on a fragment behind its pixel's last one (sorted index hi - k > bin_final) runs with vis = 0, and
-            // the blank fragment past the end of a list has opacity zero: alpha = 0 either way, and one comparison
-            // decides about the lane
-            const bool in_range = (k >= k_min) & !(sigma < 0.f || sigma > cut);
-            float vis = in_range ? __builtin_amdgcn_exp2f(sigma * -1.44269504088896341f) : 0.0f;
+            // alpha > 1/255 <=> sigma < ln(255 opac) = cut - 1e-3 (fragment_constants): decided by comparing sigma, except
+            // within 8e-6 of that bound, where the rounding of the exponential could decide; there, and where alpha
+            // comes within 4e-5 of the 0.999 cap, the wavefront re-evaluates with the bit-defined exponential, so that
+            // every decision is the forward's. A lane on a fragment behind its pixel's last one (sorted index
+            // hi - k > bin_final) is out; so is the blank fragment past the end of a list (cut 0: no sigma is below).
+            const uint32_t lo_bits = __float_as_uint(ssr_max(cut - 1.008e-3f, 0.0f));
+            const bool in_list = k >= k_min;
+            const bool below = __float_as_uint(sigma) < lo_bits;      // 0 <= sigma < bound - band
+            const uint64_t m_in = __builtin_amdgcn_ballot_w64(in_list), m_lo = __builtin_amdgcn_ballot_w64(below),
+                           m_off = __builtin_amdgcn_ballot_w64(sigma > cut - 0.992e-3f);
+            bool active = in_list & below;
+            float vis = active ? __builtin_amdgcn_exp2f(sigma * -1.44269504088896341f) : 0.0f;
             float ov = q1.y * vis;
-            const bool near_edge = ((int)(ssr_fabs(ov - kAlphaThreshold) <= 1.6e-7f) | (int)(ssr_fabs(ov - 0.999f) <= 4e-5f)) != 0;
-            if (__builtin_amdgcn_ballot_w64(near_edge) != 0ull) {   // decisions exactly as the forward took them
+            uint64_t unsure = m_in & ~(m_lo | m_off);
+            const bool sat_possible = __builtin_amdgcn_ballot_w64(q1.y >= 0.9989f) != 0ull;
+            if (sat_possible) unsure |= __builtin_amdgcn_ballot_w64(ssr_fabs(ov - 0.999f) <= 4e-5f);
+            float alpha = ov;
+            if (unsure != 0ull) {   // decisions exactly as the forward took them
+                const bool in_range = in_list & !(sigma < 0.f || sigma > cut);
                 vis = in_range ? exp_neg_small(-sigma) : 0.0f;
                 ov = q1.y * vis;
+                // min(0.999, ov) as the one instruction it is (a NaN ov gives 0.999, as ssr_min does); the compiler's own
+                // minimum spends a second instruction on quieting a signalling NaN first
+                asm("v_min_f32 %0, %1, %2" : "=v"(alpha) : "s"(0.999f), "v"(ov));
+                active = alpha > kAlphaThreshold;
+                alpha = active ? alpha : 0.0f;
+                vis = (active & (ov <= 0.999f)) ? vis : 0.0f;   // evaluate_alpha_vjp gate (src/primitives/Primitive3DGS.cuh:273)
+            } else if (sat_possible) {
+                asm("v_min_f32 %0, %1, %2" : "=v"(alpha) : "s"(0.999f), "v"(ov));
+                vis = ov <= 0.999f ? vis : 0.0f;                // the same gate; without a fragment near the cap it never closes
             }
-            // min(0.999, ov) as the one instruction it is (a NaN ov gives 0.999, as ssr_min does); the compiler's own
-            // minimum spends a second instruction on quieting a signalling NaN first
-            float alpha;
-            asm("v_min_f32 %0, %1, %2" : "=v"(alpha) : "s"(0.999f), "v"(ov));
-            const bool active = alpha > kAlphaThreshold;
             if (__builtin_amdgcn_ballot_w64(active) != 0ull) {
-                // inactive lanes run with alpha = 0 and v_alpha = 0: T and v_T unchanged, every term zero
-                const float a = active ? alpha : 0.0f;
+                // inactive lanes run with alpha = 0 and vis = 0: T and v_T unchanged, every term zero
+                const float a = alpha;
                 const float T0 = T1 * __builtin_amdgcn_rcpf(1.0f - a);
                 [[maybe_unused]] float v_depth_median = 0.0f;
                 if constexpr (kMedian) {   // RasterizationEval3DBwd_kernel.cuh:433-470
@@ -413,8 +426,7 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
                     gsum += ((Sd + (cdp * cdp) * Wd) - (cdp * Cd) * 2.0f) * vDd;
                     dv += gsum;   // v_alpha gains T0 g and v_T0 gains alpha g, exactly where dv enters
                 }
-                // evaluate_alpha_vjp gate (src/primitives/Primitive3DGS.cuh:273); sigma >= 0 holds when active
-                const float v_alpha = (active & (ov <= 0.999f)) ? T0 * dv : 0.0f;
+                const float v_alpha = T0 * dv;   // reaches the sums through vis, which is zero where the gate is closed
                 vT1 = ssr_fma(a, dv, vT1);
                 T1 = T0;
                 const float u = vis * v_alpha;
@@ -588,6 +600,7 @@ extern "C" int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t strea
     if (p->dist_type == SSR_DIST_RGB_D)
         SSR_REQUIRE(p->render_rgb && p->distortion_rgb && p->v_distortion_rgb, "ssr_raster_bwd", "null rgb distortion input");
     SSR_REQUIRE(p->accum_mode >= SSR_ACCUM_NONE && p->accum_mode <= SSR_ACCUM_AVG, "ssr_raster_bwd", "unknown accum_mode");
+    SSR_REQUIRE(p->schedule == SSR_BWD_SCHEDULE_ROWS || p->schedule == SSR_BWD_SCHEDULE_LANES, "ssr_raster_bwd", "unknown schedule");
     if (p->accum_mode != SSR_ACCUM_NONE) {
         SSR_REQUIRE(p->accum_weight_map && p->accum_weight, "ssr_raster_bwd", "null accumulation buffer");
         SSR_REQUIRE(p->num_world > 0, "ssr_raster_bwd", "num_world must be positive");
@@ -611,8 +624,7 @@ extern "C" int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t strea
         default: SSR_ROWS(D, M, SSR_ACCUM_NONE); break;             \
     }
 #define SSR_ROWS_M(D) if (med) { SSR_ROWS_A(D, true) } else { SSR_ROWS_A(D, false) }
-    static const bool rows_only = getenv("SSR_BWD_ROWS") != nullptr;   // measurement switch: the row kernel for the plain variant too
-    if (p->dist_type == SSR_DIST_NONE && !med && p->accum_mode == SSR_ACCUM_NONE && !rows_only)
+    if (p->schedule == SSR_BWD_SCHEDULE_LANES && p->dist_type == SSR_DIST_NONE && !med && p->accum_mode == SSR_ACCUM_NONE)
         launch_raster_bwd_lanes(*p, tw, th, nimg, st);
     else if (p->dist_type == SSR_DIST_NONE && !med && p->accum_mode == SSR_ACCUM_AVG)
         hipLaunchKernelGGL(raster_bwd_rows_avg_kernel, grid, block, 0, st, *p, tw, th);

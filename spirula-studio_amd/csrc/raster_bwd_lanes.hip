@@ -26,14 +26,13 @@
 namespace ssr {
 
 constexpr int kLB = 128;           // fragments staged per batch
-constexpr int kLCh = 12;           // floats per fragment slot: u, u dx, u dy, u dx^2, u dx dy, u dy^2, w_r, w_g, w_b, w_d, 2 unused
-typedef float float4v __attribute__((ext_vector_type(4)));
+constexpr int kLCh = 10;           // channels per fragment: u, u dx, u dy, u dx^2, u dx dy, u dy^2, w_r, w_g, w_b, w_d
 constexpr int kChunk = 16;         // fragments per row and chunk
 
 struct LanesShared {
     FragLds frags[kLB + 1];        // the last one is the blank fragment behind every list
     int32_t ids[kLB];
-    __attribute__((aligned(16))) float acc[(4 * kLB + 1) * kLCh];   // per wavefront and slot; the last row takes what blank fragments add (zeros)
+    float acc[(4 * kLB + 1) * kLCh];   // per wavefront and slot; the last row takes what blank fragments add (zeros)
     uint8_t bits[2 * kLB];
     __attribute__((aligned(16))) uint8_t list[kBlocksPerTile * kLB];
     // pixel state, index = 16 * block + 4 * row + column = thread id of the pixel's owner at set-up
@@ -222,18 +221,7 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
             const int4 lastq = *reinterpret_cast<const int4*>(S.last + pix0);
             float Tc[4] = {Tq.x, Tq.y, Tq.z, Tq.w}, vTc[4] = {vTq.x, vTq.y, vTq.z, vTq.w};
             const int lastc[4] = {lastq.x, lastq.y, lastq.z, lastq.w};
-            // Operands of the matrix instructions (v_mfma_f32_16x16x4_f32: D[i][j] += sum_k A[i][k] B[k][j]; a lane
-            // supplies A[l16][row] and B[row][l16] and receives D[4 row + 0..3][l16]):
-            //   g: A = the pixels' cotangents (pixel l16 of the block, channel `row`), B = the fragments' colours
-            //      (fragment l16, channel `row`): D[4 row + c][l16] = c_f . v_c for this lane's pixel (row, c);
-            //   sums: B = a per-lane value of pixel (row, c) and fragment l16, A selects the channel it belongs to and
-            //      weighs it: the moment sums with A = 1 in line `channel`, the colour sums with A = the cotangent
-            //      of pixel (row, c) in lines 6..9. D[channel][l16] then holds the sum over the block's pixels.
-            const float a_g = reinterpret_cast<const float*>(&S.v[blk_pix + l16])[row];
-            float a_col[4];
-#pragma unroll
-            for (int c = 0; c < 4; c++)
-                a_col[c] = (l16 >= 6 && l16 <= 9) ? reinterpret_cast<const float*>(&S.v[pix0 + c])[l16 - 6] : 0.0f;
+            const float4 vc[4] = {S.v[pix0], S.v[pix0 + 1], S.v[pix0 + 2], S.v[pix0 + 3]};
             const float px0 = tile_x0 + (float)((mt & 1) * kMicro + (q & 1) * kBlock) + 0.5f;
             const float py = tile_y0 + (float)((mt >> 1) * kMicro + (q >> 1) * kBlock + row) + 0.5f;
             const uint8_t* lst = S.list + (4 * mt + q) * kLB + l16;
@@ -242,9 +230,9 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
                 const int slot = (int)lst[ch];
                 const char* fp = reinterpret_cast<const char*>(S.frags) + __umul24((unsigned)slot, (unsigned)sizeof(FragLds));
                 const FragLds& F = *reinterpret_cast<const FragLds*>(fp);
-                const float4 q0 = F.q0;
-                const float cz = F.q1.x, opac = F.q1.y, cut = F.q2.w;
-                const float b_g = *reinterpret_cast<const float*>(fp + 24 + 4 * row);   // r, g, b, depth are floats 6..9 of the record
+                const float4 q0 = F.q0, q1 = F.q1;
+                const float2 q2 = make_float2(F.q2.x, F.q2.y);
+                const float cz = q1.x, opac = q1.y, cut = F.q2.w;
                 const int idx = hi - slot;
                 // alpha > 1/255 <=> sigma < ln(255 opac) = cut - 1e-3 (fragment_constants); the band around it in
                 // which the exponential's rounding could decide is +-8e-6
@@ -257,7 +245,10 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
                 constexpr bool kSat = decltype(sat_tag)::value;
                 const float dy = q0.y - py;
                 const float ty2 = cz * dy;
-                const float4v gq = __builtin_amdgcn_mfma_f32_16x16x4f32(a_g, b_g, float4v{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                float gq[4];   // c_f . v_c
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+                    gq[c] = ssr_fma(q2.y, vc[c].w, ssr_fma(q2.x, vc[c].z, ssr_fma(q1.w, vc[c].y, q1.z * vc[c].x)));
                 float a[4], visu[4], dx[4], om[4], bk[4];
 #pragma unroll
                 for (int c = 0; c < 4; c++) {
@@ -334,33 +325,37 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
                     : "=&v"(Tc[0]), "=&v"(Tc[1]), "=&v"(Tc[2]), "=&v"(Tc[3]), "=&v"(vTc[0]), "=&v"(vTc[1]), "=&v"(vTc[2]), "=&v"(vTc[3])
                     : "v"(T0[0]), "v"(T0[1]), "v"(T0[2]), "v"(T0[3]), "v"(vT0[0]), "v"(vT0[1]), "v"(vT0[2]), "v"(vT0[3]));
                 // per-lane sums over the four pixels of the row (the colour sums go through the matrix unit pixel by pixel)
-                float u[4], ux[4];
-                float4v dcol = {0.f, 0.f, 0.f, 0.f};
+                float u[4], ux[4], w[4];
 #pragma unroll
                 for (int c = 0; c < 4; c++) {
                     const float dv = gq[c] - vT1[c];
                     u[c] = visu[c] * (T0[c] * dv);
                     ux[c] = u[c] * dx[c];
-                    dcol = __builtin_amdgcn_mfma_f32_16x16x4f32(a_col[c], a[c] * T0[c], dcol, 0, 0, 0);
+                    w[c] = a[c] * T0[c];
                 }
                 const float U = (u[0] + u[1]) + (u[2] + u[3]), V1 = (ux[0] + ux[1]) + (ux[2] + ux[3]);
                 const float V2 = ssr_fma(ux[3], dx[3], ssr_fma(ux[2], dx[2], ssr_fma(ux[1], dx[1], ux[0] * dx[0])));
+                const float Wr = ssr_fma(vc[3].x, w[3], ssr_fma(vc[2].x, w[2], ssr_fma(vc[1].x, w[1], vc[0].x * w[0])));
+                const float Wg = ssr_fma(vc[3].y, w[3], ssr_fma(vc[2].y, w[2], ssr_fma(vc[1].y, w[1], vc[0].y * w[0])));
+                const float Wb = ssr_fma(vc[3].z, w[3], ssr_fma(vc[2].z, w[2], ssr_fma(vc[1].z, w[1], vc[0].z * w[0])));
+                const float Wd = ssr_fma(vc[3].w, w[3], ssr_fma(vc[2].w, w[2], ssr_fma(vc[1].w, w[1], vc[0].w * w[0])));
                 const float Uy = U * dy;
-                const float sel0 = l16 == 0 ? 1.0f : 0.0f, sel1 = l16 == 1 ? 1.0f : 0.0f, sel2 = l16 == 2 ? 1.0f : 0.0f,
-                            sel3 = l16 == 3 ? 1.0f : 0.0f, sel4 = l16 == 4 ? 1.0f : 0.0f, sel5 = l16 == 5 ? 1.0f : 0.0f;
-                float4v dmom = __builtin_amdgcn_mfma_f32_16x16x4f32(sel0, U, float4v{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-                dmom = __builtin_amdgcn_mfma_f32_16x16x4f32(sel1, V1, dmom, 0, 0, 0);
-                dmom = __builtin_amdgcn_mfma_f32_16x16x4f32(sel2, Uy, dmom, 0, 0, 0);
-                dmom = __builtin_amdgcn_mfma_f32_16x16x4f32(sel3, V2, dmom, 0, 0, 0);
-                dmom = __builtin_amdgcn_mfma_f32_16x16x4f32(sel4, V1 * dy, dmom, 0, 0, 0);
-                dmom = __builtin_amdgcn_mfma_f32_16x16x4f32(sel5, Uy * dy, dmom, 0, 0, 0);
-                // this lane now holds channels 4 row + 0..3 of its own fragment: rows 0..2 add them to the wavefront's copy
-                float4 add;
-                add.x = dmom[0] + dcol[0]; add.y = dmom[1] + dcol[1]; add.z = dmom[2] + dcol[2]; add.w = dmom[3] + dcol[3];
-                float4* cell = reinterpret_cast<float4*>((slot < kLB && row < 3 ? my_acc + __umul24((unsigned)slot, (unsigned)kLCh) + 4 * row : dump));
-                float4 cur = *cell;
-                cur.x += add.x; cur.y += add.y; cur.z += add.z; cur.w += add.w;
-                *cell = cur;
+                // the sum over the four pixel rows: channels in pairs through v_permlane16_swap (rows 0<->1, 2<->3), the
+                // pair sums in pairs through v_permlane32_swap; row r of R0 / R1 / R2 then holds channel r / 4 + r / 8 + r
+                auto fold16 = [](float x, float y) {
+                    const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(y), false, false);
+                    return __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+                };
+                auto fold32 = [](float x, float y) {
+                    const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(y), false, false);
+                    return __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+                };
+                const float R0 = fold32(fold16(U, V1), fold16(Uy, V2));                 // u, u dx, u dy, u dx^2
+                const float R1 = fold32(fold16(V1 * dy, Uy * dy), fold16(Wr, Wg));      // u dx dy, u dy^2, w_r, w_g
+                const float R2 = fold32(fold16(Wb, Wd), 0.0f);                          // w_b, w_d (rows 0, 1)
+                float* cell = (slot < kLB ? my_acc + __umul24((unsigned)slot, (unsigned)kLCh) : dump) + row;
+                cell[0] += R0; cell[4] += R1;
+                if (row < 2) cell[8] += R2;
                 };
                 if (sat_possible) chunk(std::true_type{}); else chunk(std::false_type{});
             }

@@ -67,7 +67,7 @@ class RasterBwdParams(C.Structure):
                 ("distortion_rgb", vp), ("distortion_depth", vp), ("v_distortion_rgb", vp),
                 ("v_distortion_depth", vp), ("v_render_median", vp), ("accum_mode", C.c_int32),
                 ("accum_weight_map", vp), ("gaussian_ids", vp), ("num_world", C.c_int64), ("accum_weight", vp),
-                ("num_images", C.c_int32), ("tile_order", vp), ("tile_offsets_closed", C.c_int32)]
+                ("num_images", C.c_int32), ("tile_order", vp), ("tile_offsets_closed", C.c_int32), ("schedule", C.c_int32)]
 
 
 class TileWriteCappedParams(C.Structure):

@@ -47,12 +47,13 @@ def world_grad_check(got, ref, n, name, rtol=WORLD_GRAD_RTOL, bad_frac=0.0, scal
 
 class GpuRun:
     def __init__(self, pkg, scene, sh_degree=3, use_list=False, use_packed=False, packed_projection=False,
-                 read_nnz=True, use_vrows=False, tile_sort=False, capacity=None, world_rows=False):
+                 read_nnz=True, use_vrows=False, tile_sort=False, capacity=None, world_rows=False, bwd_lanes=False):
         """use_packed: 48-byte fragment rows for the compositing kernels. packed_projection: the
         compacted (nnz-row) projection outputs of projection_3dgs_packed_forward; read_nnz=False
         sizes the outputs for all N splats instead of reading nnz back between the two calls."""
         self.use_list = use_list
         self.use_packed = use_packed
+        self.bwd_lanes = bwd_lanes   # SSR_BWD_SCHEDULE_LANES for the compositing backward (plain variant only)
         self.packed_projection = packed_projection
         self.read_nnz = read_nnz
         # world_rows (with packed_projection): the projection also writes each visible splat's parameters (four
@@ -402,6 +403,7 @@ class GpuRun:
                 p.gaussian_ids = self.ptr("gaussian_ids")
         p.tile_order = self.ptr("tile_order")
         p.tile_offsets_closed = 1 if self.capacity is not None else 0
+        p.schedule = 1 if self.bwd_lanes else 0
         self.check(self.lib.ssr_raster_bwd(C.byref(p), None))
         if self.use_vrows and n:   # unpack for the comparisons, after checking the arrays were left alone
             for k in ["v_xy", "v_depth", "v_conic", "v_opac", "v_rgb"]:

@@ -123,7 +123,11 @@ def test_full_size_properties(pkg, oracle, H, cfg):
     g3 = ref.grads()
 
     def close(a, b, what):
-        world_grad_check(a, b, n, f"config{cfg}/{what[0]}/{what[1]}")
+        # Two GPU runs against each other, without the oracle's magnitude sums to derive a floor from: an opacity
+        # gradient that cancels to a thousandth of its terms differs between two summation orders by more than 1e-3
+        # of itself, so a few elements per million may (the element-wise bar against the oracle, with floors, is
+        # test_gpu_parity.py::test_bench_configs_full_against_the_oracle).
+        world_grad_check(a, b, n, f"config{cfg}/{what[0]}/{what[1]}", bad_frac=1e-5)
 
     for k in g1:
         close(g1b[k], g1[k], ("idempotent", k))

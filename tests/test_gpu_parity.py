@@ -34,14 +34,15 @@ def _grad_close(got, ref, abs_scale, name, max_bad=0, rtol=GRAD_RTOL, afrac=2e-6
 
 
 def _compare(gpu, oracle, sc, label, fused_count=False, use_list=False, use_packed=False, mask=None, variant=None,
-             use_vrows=False, tile_sort=False, spare=None):
-    """spare: run K4-K6 without reading the counts back, in arrays of K + spare entries (spare >= 0)."""
+             use_vrows=False, tile_sort=False, spare=None, bwd_lanes=False):
+    """spare: run K4-K6 without reading the counts back, in arrays of K + spare entries (spare >= 0). bwd_lanes: the
+    compositing backward with one lane per fragment (SSR_BWD_SCHEDULE_LANES)."""
     live = None if mask is None else oracle.compute_tile_active(mask, sc.width, sc.height)
     r = oracle.pipeline(sc, tile_active=live, variant=variant)
     print(f"[{label}] N={sc.n} {sc.width}x{sc.height} visible={r['proj']['visible']} K={r['isect_ids'].size}", flush=True)
     K = r["isect_ids"].size
     g = GpuRun(gpu, sc, use_list=use_list, use_packed=use_packed, use_vrows=use_vrows, tile_sort=tile_sort,
-               capacity=None if spare is None else K + spare)
+               capacity=None if spare is None else K + spare, bwd_lanes=bwd_lanes)
     if mask is not None:
         g.set_tile_mask(mask)
         assert np.array_equal(g.host("tile_active"), live)
@@ -370,6 +371,32 @@ def test_config1_reduced(gpu, oracle):
 
 def test_config1_full(gpu, oracle):
     _compare(gpu, oracle, gpu.scenes.make_scene(1), "cfg1")
+    _compare(gpu, oracle, gpu.scenes.make_scene(1), "cfg1-lanes", use_packed=True, use_vrows=True, tile_sort=True, bwd_lanes=True)
+
+
+@pytest.mark.parametrize("lanes", [False, True])
+def test_backward_schedules(gpu, oracle, lanes):
+    """Both cuts of the compositing backward (a row per fragment, a lane per fragment) against the oracle on scenes
+    that stress what differs between them: large overlapping splats with early termination, an image that is no
+    multiple of the tile, opacities at the 0.999 cap (alpha capped, the exponent's gradient gated), one splat,
+    lists of exactly 16 / 17 / 128 / 129 fragments in a block, the equirectangular camera's small footprints."""
+    S = gpu.scenes
+    kw = dict(bwd_lanes=lanes)
+    _compare(gpu, oracle, S.tiny_scene(n=300, width=64, height=48, seed=11), f"sched{int(lanes)}-tiny", **kw)
+    _compare(gpu, oracle, S.tiny_scene(n=700, width=70, height=37, seed=12), f"sched{int(lanes)}-ragged", use_packed=True, use_vrows=True, **kw)
+    sc = S.tiny_scene(n=400, width=80, height=64, seed=13)
+    sc.opacity_logits[::3] = 9.0          # sigmoid 0.99988: the pixel under the centre saturates at 0.999
+    sc.opacity_logits[1::7] = 6.9         # 0.99899: inside the band around the cap
+    _compare(gpu, oracle, sc, f"sched{int(lanes)}-opaque", use_list=True, use_packed=True, use_vrows=True, tile_sort=True, **kw)
+    for n in (1, 16, 17, 128, 129, 257):  # every splat covers the one tile's every block: block lists of exactly n
+        sc = S.tiny_scene(n=n, width=16, height=16, seed=100 + n)
+        sc.means[:, :2] *= 0.02
+        sc.log_scales[:] = -1.0 + 0.2 * (sc.log_scales - sc.log_scales.mean())   # large, and not isotropic (an isotropic
+        # splat's quaternion gradient is zero but for rounding, which no relative bar can hold)
+        sc.opacity_logits[:] = -3.0       # faint: no pixel terminates, every fragment composites
+        _compare(gpu, oracle, sc, f"sched{int(lanes)}-list{n}", use_packed=True, use_vrows=True, **kw)
+    _compare(gpu, oracle, S.make_scene(5, n=20000, width=256, height=128, parity_variant=True), f"sched{int(lanes)}-equirect",
+             use_list=True, use_packed=True, use_vrows=True, tile_sort=True, **kw)
 
 
 @pytest.mark.parametrize("cfg", [2, 3, 4, 5])
@@ -378,7 +405,7 @@ def test_bench_configs_full_against_the_oracle(gpu, oracle, cfg):
     equirectangular 4096x2048) whole and at full size against the oracle, on the stage order the benchmark runs: every key, id, range and last id bit for bit, every pixel to 1e-4, every
     gradient row to 1e-3."""
     _compare(gpu, oracle, gpu.scenes.make_scene(cfg), f"cfg{cfg}-full", fused_count=True, use_list=True, use_packed=True,
-             use_vrows=True, tile_sort=True)
+             use_vrows=True, tile_sort=True, bwd_lanes=cfg == 2)   # the cut the engine picks for each (tiles per visible splat)
 
 
 @pytest.mark.parametrize("codec,stride", [(1, 256), (1, 0), (2, 256), (3, 0)])
