@@ -5,8 +5,11 @@
 
 One step = one forward+backward iteration of the path on a seeded synthetic scene whose inputs
 and pixel cotangents are already resident in HBM: zero radii -> projection+SH (with the tile
-count fused) -> int64 scan + 8-byte count readback -> key write -> 64-bit radix sort -> tile
-offsets -> compositing forward -> zero v_screen -> compositing backward -> projection backward.
+count fused) -> int64 scan (the first iteration reads the 16 bytes of counts back as the reference
+does, later ones leave them on the device; --blocking-counts reads them every time) -> key write ->
+64-bit radix sort -> tile offsets -> compositing forward -> zero the gradient rows -> compositing
+backward -> projection backward. After the headline configuration the other four run briefly in the
+same process (all_configs).
 Prints ONE JSON line: the metric of BASELINE.json (iterations/s), a `roofline` object for the
 kernel that takes the most time, and a `cpu_baseline` object (the CPU oracle timed on this host).
 """
@@ -176,9 +179,10 @@ def run_config(args, pkg, host, lib, np, with_cpu):
             setattr(sc, name, np.ascontiguousarray(np.stack([np.asarray(getattr(sc, name), np.float32)] * ncam)))
     t_gen = time.time() - t_gen
     native = not args.reference_order
+    deferred = native and not args.whole_key_sort and not args.blocking_counts and ncam == 1   # needs the tile-segmented sort
     eng = host.Engine(sc, fuse_tile_count=native, visible_list=native and not args.packed_projection, packed_rows=native,
                       overwrite_world_grads=native, packed_projection=args.packed_projection, packed_vscreen=native,
-                      tile_sort=native and not args.whole_key_sort, deferred_counts=args.deferred_counts,
+                      tile_sort=native and not args.whole_key_sort, deferred_counts=deferred,
                       packed_world_rows=args.packed_world_rows)
 
     hyper = dict(lr_means=1.6e-6, lr_quats=1e-5, lr_scales=5e-5, lr_opacs=5e-4, lr_features_dc=2.5e-5, lr_features_sh=1.25e-6)
@@ -323,7 +327,8 @@ def run_config(args, pkg, host, lib, np, with_cpu):
                                f"{['fp32', 'ref-q8', 'ref-q16', 'int8*fp16scale'][sc.sh_codec]}, tile 16x16, seed {pkg.scenes.CONFIGS[cfg]['seed']:#x}",
                    "visible": V, "n_isects": K, "K_f": K_f, "K_b": K_b, "tiles": T, "pixels": P,
                    "stage_order": ("fused tile count, visible-splat work list, packed fragment rows, packed gradient rows, plain-store gradients"
-                                   + (", tile-segmented sort" if tile_sort else "") if native else "reference order")
+                                   + (", tile-segmented sort" if tile_sort else "")
+                                   + (", intersection count left on the device after the first iteration" if deferred else "") if native else "reference order")
                                   + (", antialiased (mip) primitive" if args.mip else "")
                                   + (f", {ncam} cameras per iteration in one call" if ncam > 1 else "")
                                   + (", packed projection outputs" if args.packed_projection else "")
@@ -395,9 +400,10 @@ def main():
     ap.add_argument("--packed-world-rows", action="store_true",
                     help="with the packed projection: keep the visible splats' parameters (64 bytes each) for the projection backward")
     ap.add_argument("--no-packed-world-rows", action="store_true", help="config 4: gather the parameters in the projection backward")
-    ap.add_argument("--deferred-counts", action="store_true",
-                    help="after the first iteration the forward does not wait for the intersection count: key arrays sized "
-                         "from the previous count, overflow checked before the backward uses the counts")
+    ap.add_argument("--blocking-counts", action="store_true",
+                    help="wait for the intersection count between the scan and the key write in every iteration, as the reference "
+                         "does. Default: only the first iteration reads it; after that the key arrays are sized from the previous "
+                         "count, the count follows asynchronously, and an overflow is refused before the backward uses anything")
     ap.add_argument("--cameras", type=int, default=1,
                     help="render C cameras per iteration in one call ([C,N] layout, plain path only); an iteration is then C images")
     ap.add_argument("--no-all-configs", action="store_true",
@@ -429,7 +435,7 @@ def main():
 
     default_plain = not (args.reference_order or args.whole_key_sort or args.lens != "none" or args.fisheye or args.packed_projection
                          or args.dense_projection or args.fused_optimizer or args.mip or args.dist_type or args.median
-                         or args.accum_mode or args.packed_world_rows or args.no_packed_world_rows or args.deferred_counts
+                         or args.accum_mode or args.packed_world_rows or args.no_packed_world_rows or args.blocking_counts
                          or args.cameras != 1 or args.n)
     out = run_config(args, pkg, host, lib, np, with_cpu=not args.no_cpu_baseline)
     if default_plain and not args.no_all_configs:

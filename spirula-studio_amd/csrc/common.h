@@ -35,6 +35,18 @@ int warm_static_scan();
 // in the gfx9 encoding (vmcnt 63, expcnt 7 left alone). Placed ahead of a workgroup barrier that follows
 // non-returning LDS float atomics, whose completion the kernels here do not leave to the compiler.
 __device__ __forceinline__ void lds_wait() { __builtin_amdgcn_s_waitcnt(0xc07f); }
+// A workgroup barrier that orders LDS traffic only: every LDS operation of this wavefront is complete, then the
+// barrier. Unlike __syncthreads() it does not wait for vector-memory operations in flight (global atomics whose
+// results nobody reads, rows on their way from memory into LDS for a later batch) -- the release fence of
+// __syncthreads() would, at every barrier. Neither builtin may be moved across by the compiler, nor memory accesses
+// across them. Data that arrives in LDS from memory needs its own vmcnt wait ahead of the barrier that publishes it.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_s_barrier();
+}
+// Waits until every vector-memory operation this wavefront has issued is complete, loads into LDS included:
+// s_waitcnt vmcnt(0) in the gfx9 encoding (the six vmcnt bits are [3:0] and [15:14]).
+__device__ __forceinline__ void vmem_wait() { __builtin_amdgcn_s_waitcnt(0x0f70); }
 
 }  // namespace ssr
 

@@ -41,6 +41,8 @@ struct LanesShared {
     __attribute__((aligned(16))) int32_t last[256];
     float4 v[256];                 // v_r, v_g, v_b, v_depth / W
     int wave_max[4];
+    int cnt[kBlocksPerTile];       // list lengths of the batch
+    int next;                      // next block to hand out
 };
 
 __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) void raster_bwd_lanes_kernel(ssr_raster_bwd_params P, int tile_w, int tile_h) {
@@ -135,7 +137,7 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
                 dst[9] = ssr_isfinite(o[3]) ? o[3] : 0.f;
             }
         }
-        __syncthreads();
+        lds_barrier();
         if (P.v_rows) {
             for (int e = tid; e < kLB * kLCh; e += kRasterBlock) {
                 const int slot = e / kLCh, ch = e - slot * kLCh;
@@ -162,7 +164,7 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
                 add(P.v_screen.rgb + 3 * g, v[7]); add(P.v_screen.rgb + 3 * g + 1, v[8]); add(P.v_screen.rgb + 3 * g + 2, v[9]);
             }
         }
-        __syncthreads();
+        lds_barrier();
     };
 
     float* const my_acc = S.acc + mt * (kLB * kLCh);
@@ -175,9 +177,10 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
     }
     for (int32_t hi = min(range_end - 1, tile_last); hi >= range_start; hi -= kLB) {
         lds_wait();
-        __syncthreads();   // previous batch fully consumed
+        __syncthreads();   // previous batch fully consumed (and, this once per batch, memory operations complete)
         if (!first) flush();
         first = false;
+        if (tid == 0) S.next = 0;
         {
             const int half = tid >= kLB ? 1 : 0, slot = tid - half * kLB;
             const int32_t idx = hi - slot;
@@ -190,7 +193,7 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
             S.bits[half * kLB + slot] = (uint8_t)bits8;
             if (idx - kLB >= range_start) g_ahead = P.flatten_ids[idx - kLB];
         }
-        __syncthreads();
+        lds_barrier();
         const int n_batch = min(kLB, hi - range_start + 1);
         int cnt[4] = {0, 0, 0, 0};
         if (lane < 4 * kLB / 8)   // 8-byte stores blank the wavefront's four lists
@@ -206,15 +209,20 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
                 cnt[r] += __builtin_popcountll(bal);
             }
         }
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        __builtin_amdgcn_wave_barrier();
+        if (lane < 4) S.cnt[4 * mt + lane] = lane == 0 ? cnt[0] : lane == 1 ? cnt[1] : lane == 2 ? cnt[2] : cnt[3];
+        lds_barrier();   // every list of the tile is built
 
-        // ---- the walk: block q of this sub-tile, chunk by chunk; this lane = (pixel row `row`, list position l16) ----
-#pragma unroll 1
-        for (int q = 0; q < 4; q++) {
-            const int n_list = q == 0 ? cnt[0] : q == 1 ? cnt[1] : q == 2 ? cnt[2] : cnt[3];
+        // ---- the walk: the sixteen blocks are dealt to the wavefronts as they become free (a sub-tile's four blocks
+        // can hold most of a tile's work); this lane = (pixel row `row` of the block, list position l16) ----
+        for (;;) {
+            int blk = 0;
+            if (lane == 0) blk = atomicAdd(&S.next, 1);
+            blk = __builtin_amdgcn_readfirstlane(blk);
+            if (blk >= kBlocksPerTile) break;
+            const int n_list = S.cnt[blk];
             if (n_list == 0) continue;
-            const int blk_pix = (4 * mt + q) * 16;
+            const int bm = blk >> 2, q = blk & 3;   // sub-tile and quadrant of the block
+            const int blk_pix = blk * 16;
             const int pix0 = blk_pix + 4 * row;                // this lane's four pixels: pix0 + 0..3
             float4 Tq = *reinterpret_cast<const float4*>(S.T + pix0);
             float4 vTq = *reinterpret_cast<const float4*>(S.vT + pix0);
@@ -222,9 +230,9 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
             float Tc[4] = {Tq.x, Tq.y, Tq.z, Tq.w}, vTc[4] = {vTq.x, vTq.y, vTq.z, vTq.w};
             const int lastc[4] = {lastq.x, lastq.y, lastq.z, lastq.w};
             const float4 vc[4] = {S.v[pix0], S.v[pix0 + 1], S.v[pix0 + 2], S.v[pix0 + 3]};
-            const float px0 = tile_x0 + (float)((mt & 1) * kMicro + (q & 1) * kBlock) + 0.5f;
-            const float py = tile_y0 + (float)((mt >> 1) * kMicro + (q >> 1) * kBlock + row) + 0.5f;
-            const uint8_t* lst = S.list + (4 * mt + q) * kLB + l16;
+            const float px0 = tile_x0 + (float)((bm & 1) * kMicro + (q & 1) * kBlock) + 0.5f;
+            const float py = tile_y0 + (float)((bm >> 1) * kMicro + (q >> 1) * kBlock + row) + 0.5f;
+            const uint8_t* lst = S.list + blk * kLB + l16;
 #pragma unroll 1
             for (int ch = 0; ch < n_list; ch += kChunk) {
                 const int slot = (int)lst[ch];

@@ -147,6 +147,25 @@ __device__ __forceinline__ uint32_t block_bits_of_half(float a, float b, float c
     return bits;
 }
 
+// The eight block bits (bit 4 (m & 1) + quadrant) of tile half `half` (sub-tiles 2 half and 2 half + 1) for a fragment
+// given by the first two quarters of its row (x, y, 0.5 conic.x, conic.y | 0.5 conic.z, opac, ..) and its footprint
+// scale kk: the reference's sub-tile test, then the block tests of the sub-tiles that pass.
+__device__ __forceinline__ uint32_t fragment_block_bits_half(const float4& q0, const float4& q1, float kk, float tile_x0,
+                                                             float tile_y0, int half) {
+    if (!(q1.y > kAlphaThreshold)) return 0u;
+    // conic.x = 2 * (0.5 conic.x) exactly, conic.z likewise
+    const float ic[3] = {(q0.z + q0.z) * kk, q0.w * kk, (q1.x + q1.x) * kk};
+    const float x = q0.x, y = q0.y;
+    uint32_t sub = 0;   // the reference's test for the two sub-tiles of this half
+#pragma unroll
+    for (int mm = 0; mm < 2; mm++) {
+        const int m = 2 * half + mm;
+        const float sx0 = tile_x0 + (float)((m & 1) * kMicro), sy0 = tile_y0 + (float)((m >> 1) * kMicro);
+        if (ellipse_box_overlap(ic, sx0 - x, (sx0 + (float)kMicro) - x, sy0 - y, (sy0 + (float)kMicro) - y)) sub |= 0xFu << (4 * mm);
+    }
+    return sub ? sub & block_bits_of_half(ic[0], ic[1], ic[2], x, y, tile_x0, tile_y0, half) : 0u;
+}
+
 // Stages splat g for the row-granular backward, where two threads share a fragment: thread `half`
 // (0 / 1) runs the reference's sub-tile test for sub-tiles 2 half and 2 half + 1 and the block tests of
 // those that pass; it returns their eight block bits (bit 4 (m & 1) + quadrant). The fragment record
@@ -171,19 +190,7 @@ __device__ __forceinline__ FragLds stage_fragment_half(const ssr_screen& s, cons
         f.q1 = make_float4(0.5f * cn[2], opac, rg[0], rg[1]);
         f.q2 = make_float4(rg[2], s.depth[g], 0.0f, cut);
     }
-    bits8 = 0;
-    if (f.q1.y > kAlphaThreshold) {
-        const float ic[3] = {(f.q0.z + f.q0.z) * kk, f.q0.w * kk, (f.q1.x + f.q1.x) * kk};
-        const float x = f.q0.x, y = f.q0.y;
-        uint32_t sub = 0;   // the reference's test for the two sub-tiles of this half
-#pragma unroll
-        for (int mm = 0; mm < 2; mm++) {
-            const int m = 2 * half + mm;
-            const float sx0 = tile_x0 + (float)((m & 1) * kMicro), sy0 = tile_y0 + (float)((m >> 1) * kMicro);
-            if (ellipse_box_overlap(ic, sx0 - x, (sx0 + (float)kMicro) - x, sy0 - y, (sy0 + (float)kMicro) - y)) sub |= 0xFu << (4 * mm);
-        }
-        if (sub) bits8 = sub & block_bits_of_half(ic[0], ic[1], ic[2], x, y, tile_x0, tile_y0, half);
-    }
+    bits8 = fragment_block_bits_half(f.q0, f.q1, kk, tile_x0, tile_y0, half);
     return f;
 }
 
