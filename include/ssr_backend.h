@@ -336,6 +336,13 @@ typedef struct {
     int32_t num_images;
     const int32_t* tile_order;  /* optional: ssr_tile_order's output for these tile_offsets; NULL = tiles in index order, one contiguous band per XCD */
     int32_t tile_offsets_closed; /* nonzero: tile_offsets holds one more entry, the end of the last tile (ssr_sort_tile_pairs_capped); n_isects is then only the capacity of flatten_ids */
+    /* Optional [n_isects]: receives, for every sorted entry the forward stages, the 4x4-pixel blocks of its tile that the
+     * fragment can reach (bit 4 * sub_tile + quadrant; the reference's sub-tile test of RasterizationEval3DFwd_kernel.cuh:
+     * 203-209 and the block tests under it). The backward takes them from here (its block_masks field) instead of
+     * repeating the tests. Entries of batches the forward never reached (every pixel of the tile finished before them)
+     * are not written; the backward never reads them, since they lie behind every last_id. No counterpart in the
+     * reference. */
+    uint16_t* block_masks;
 } ssr_raster_fwd_params;
 int ssr_raster_fwd(const ssr_raster_fwd_params* p, ssr_stream_t stream);
 
@@ -396,6 +403,9 @@ typedef struct {
      * one for small footprints, whose block lists are too short to fill sixteen lanes. The variants always run ROWS.
      * No counterpart in the reference. */
     int32_t schedule;                 /* SSR_BWD_SCHEDULE_* */
+    /* Optional [n_isects]: the block masks ssr_raster_fwd left for these same tile_offsets / flatten_ids (its
+     * block_masks field). When given the sub-tile and block tests are not repeated; the results are the same. */
+    const uint16_t* block_masks;
 } ssr_raster_bwd_params;
 enum { SSR_BWD_SCHEDULE_ROWS = 0, SSR_BWD_SCHEDULE_LANES = 1 };
 int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t stream);

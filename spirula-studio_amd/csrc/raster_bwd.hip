@@ -300,7 +300,7 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
             uint32_t bits8 = 0;
             if (idx >= range_start && tid < 2 * kB) {
                 const int32_t g = g_ahead;
-                const FragLds f = stage_fragment_half(P.screen, P.packed_rows, g, tile_x0, tile_y0, half, bits8);
+                const FragLds f = stage_fragment_half(P.screen, P.packed_rows, g, tile_x0, tile_y0, half, bits8, P.block_masks ? P.block_masks + idx : nullptr);
                 if (half == 0) {
                     s_ids[slot] = g; frags[slot] = f;
                     if constexpr (kDist != SSR_DIST_NONE) {

@@ -187,7 +187,7 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
             uint32_t bits8 = 0;
             if (idx >= range_start) {
                 const int32_t g = g_ahead;
-                const FragLds f = stage_fragment_half(P.screen, P.packed_rows, g, tile_x0, tile_y0, half, bits8);
+                const FragLds f = stage_fragment_half(P.screen, P.packed_rows, g, tile_x0, tile_y0, half, bits8, P.block_masks ? P.block_masks + idx : nullptr);
                 if (half == 0) { S.ids[slot] = g; S.frags[slot] = f; }
             }
             S.bits[half * kLB + slot] = (uint8_t)bits8;

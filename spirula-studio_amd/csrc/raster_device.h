@@ -170,8 +170,10 @@ __device__ __forceinline__ uint32_t fragment_block_bits_half(const float4& q0, c
 // (0 / 1) runs the reference's sub-tile test for sub-tiles 2 half and 2 half + 1 and the block tests of
 // those that pass; it returns their eight block bits (bit 4 (m & 1) + quadrant). The fragment record
 // itself is the same from either thread.
+// `mask` (optional): the sixteen block bits the forward recorded for this sorted entry; the tests are then skipped.
 __device__ __forceinline__ FragLds stage_fragment_half(const ssr_screen& s, const float* __restrict__ packed, int32_t g,
-                                                       float tile_x0, float tile_y0, int half, uint32_t& bits8) {
+                                                       float tile_x0, float tile_y0, int half, uint32_t& bits8,
+                                                       const uint16_t* __restrict__ mask = nullptr) {
     FragLds f;
     float cut, kk;
     if (packed) {
@@ -190,7 +192,7 @@ __device__ __forceinline__ FragLds stage_fragment_half(const ssr_screen& s, cons
         f.q1 = make_float4(0.5f * cn[2], opac, rg[0], rg[1]);
         f.q2 = make_float4(rg[2], s.depth[g], 0.0f, cut);
     }
-    bits8 = fragment_block_bits_half(f.q0, f.q1, kk, tile_x0, tile_y0, half);
+    bits8 = mask ? ((uint32_t)*mask >> (8 * half)) & 0xFFu : fragment_block_bits_half(f.q0, f.q1, kk, tile_x0, tile_y0, half);
     return f;
 }
 

@@ -57,6 +57,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raste
             FragLds f = stage_fragment(P.screen, P.packed_rows, g_ahead, tile_x0, tile_y0, &kk);
             add_block_mask(f, kk, tile_x0, tile_y0);
             frags[tid] = f;
+            if (P.block_masks) P.block_masks[idx] = (uint16_t)(__float_as_uint(f.q2.z) >> 16);   // for the backward
             if constexpr (kDist != SSR_DIST_NONE) s_lz[tid] = ssr_log(ssr_max(f.q2.y, 1e-6f));
         } else {
             frags[tid].q2 = make_float4(0.f, 0.f, 0.f, 0.f);   // empty masks

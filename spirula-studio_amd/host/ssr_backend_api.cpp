@@ -41,6 +41,8 @@ int g_list_toggle = 0;               // which of the two visible-list buffers th
 float* g_vrows = nullptr;             // packed gradient rows of the last compositing backward (null: off)
 const int32_t* g_tile_order = nullptr;       // launch order of the compositing workgroups for the offsets below (null: off)
 const int32_t* g_tile_order_for = nullptr;   // the tile_offsets that order was made from
+const uint16_t* g_block_masks = nullptr;     // block masks the last compositing forward left (null: none)
+const int32_t* g_block_masks_for = nullptr;  // the flatten_ids they belong to
 const float* g_vrows_for_xy = nullptr; // the v_screen.xy buffer they stand in for
 const int32_t* g_bwd_list = nullptr; // list of the last projection backward
 int64_t g_bwd_count = 0;
@@ -578,6 +580,7 @@ do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, 
         throw std::runtime_error("do_intersect_tile_generic: AABB mode is not built in this backend (ellipse mode is)");
     if (I < 1) throw std::runtime_error("do_intersect_tile_generic: no image");
     g_tile_order = nullptr; g_tile_order_for = nullptr; g_offsets_closed = nullptr;
+    g_block_masks = nullptr; g_block_masks_for = nullptr;   // new keys: the last forward's block masks are void
     if (g_counts_pending) {   // counts nobody asked for: settle them before the counters are reused
         try { ssr_ext::resolve_counts(); } catch (const std::runtime_error&) {}   // a short frame stays in short_frames() / last_error()
     }
@@ -716,6 +719,12 @@ rasterize_to_pixels_3dgs_fwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     p.render_rgb = (float*)std::get<0>(renders).data_ptr(); p.render_depth = std::get<1>(renders).data_ptr();
     p.render_T = Ts.data_ptr(); p.last_ids = last.data_ptr();
     if (g_packed_rows && p.screen.xy == g_packed_for_xy) p.packed_rows = g_packed_rows;
+    g_block_masks = nullptr; g_block_masks_for = nullptr;
+    if (p.n_isects > 0) {   // the block masks of every staged entry, for the backward of these same keys
+        uint16_t* bm = DevicePool::global().acquire<uint16_t>(PoolSlot::IsectBlockMasks, (size_t)p.n_isects);
+        p.block_masks = bm;
+        g_block_masks = bm; g_block_masks_for = p.flatten_ids;
+    }
     // distortion channels present in dist_type only (RenderOutput::resizeDistortion, src/primitives/Primitive.cuh:88-101)
     RenderOutput::TensorTuple distortions;
     DeviceTensor3D<float> median;
@@ -793,6 +802,7 @@ rasterize_to_pixels_3dgs_bwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     p.tile_offsets = tile_offsets.data_ptr(); p.flatten_ids = flatten_ids.data_ptr(); p.n_isects = flatten_ids.size();
     if (g_tile_order && g_tile_order_for == p.tile_offsets) p.tile_order = g_tile_order;
     p.tile_offsets_closed = (g_offsets_closed && g_offsets_closed == p.tile_offsets) ? 1 : 0;
+    if (g_block_masks && g_block_masks_for == p.flatten_ids) p.block_masks = g_block_masks;
     {
         // The lane-per-fragment cut pays where a splat reaches several 4x4 blocks of a tile, which shows as tiles per
         // visible splat: three and more (measured: 3.7 on the 1M-splat 1080p scene, K8 0.50 -> 0.44 ms; 1.8 on the

@@ -64,7 +64,7 @@ enum class PoolSlot : int {
     ProjAabb, ProjDepths, ProjScreenXy, ProjScreenDepth, ProjScreenConic, ProjScreenOpac, ProjScreenRgb,
     IsectTilesPerSplat, IsectCumTiles, IsectIdsA, IsectIdsB, IsectFlatA, IsectFlatB, IsectOffsets,
     IsectScanScratch, IsectSortScratch, SeamSortScratch, SeamScanScratch, IsectCounters, ProjVisibleIds, ProjVisibleIdsB, ProjPackedRows,
-    IsectTileActive, EngTileMask, IsectTileOrder,
+    IsectTileActive, EngTileMask, IsectTileOrder, IsectBlockMasks,
     AdamG1Means, AdamG1Quats, AdamG1Scales, AdamG1Opacities, AdamG1FeaturesDc, AdamG1FeaturesSh,
     AdamG2Means, AdamG2Quats, AdamG2Scales, AdamG2Opacities, AdamG2FeaturesDc, AdamG2FeaturesSh, EngDensifyScore, EngZeroAabb, FusedProjBwdRowOf, AdamShStatePacked, AdamShStateBounds, AdamNonShPacked, AdamNonShBounds, EngPoseGrad, ProjCameraIds, ProjGaussianIds, ProjGaussianIdsB, ProjPackedScratch, ProjPackedNnz, ProjPackedWorldRows, FusedMultiCamGrad,
     RendersRgb, RendersDepth, RenderTs, RenderLastIds, RenderDistortionRgb, RenderDistortionDepth, RenderMedian,

@@ -55,7 +55,7 @@ class RasterFwdParams(C.Structure):
                 ("n_isects", C.c_int64), ("render_rgb", vp), ("render_depth", vp),
                 ("render_T", vp), ("last_ids", vp), ("packed_rows", vp), ("dist_type", C.c_int32),
                 ("distortion_rgb", vp), ("distortion_depth", vp), ("render_median", vp),
-                ("num_images", C.c_int32), ("tile_order", vp), ("tile_offsets_closed", C.c_int32)]
+                ("num_images", C.c_int32), ("tile_order", vp), ("tile_offsets_closed", C.c_int32), ("block_masks", vp)]
 
 
 class RasterBwdParams(C.Structure):
@@ -67,7 +67,7 @@ class RasterBwdParams(C.Structure):
                 ("distortion_rgb", vp), ("distortion_depth", vp), ("v_distortion_rgb", vp),
                 ("v_distortion_depth", vp), ("v_render_median", vp), ("accum_mode", C.c_int32),
                 ("accum_weight_map", vp), ("gaussian_ids", vp), ("num_world", C.c_int64), ("accum_weight", vp),
-                ("num_images", C.c_int32), ("tile_order", vp), ("tile_offsets_closed", C.c_int32), ("schedule", C.c_int32)]
+                ("num_images", C.c_int32), ("tile_order", vp), ("tile_offsets_closed", C.c_int32), ("schedule", C.c_int32), ("block_masks", vp)]
 
 
 class TileWriteCappedParams(C.Structure):

@@ -47,13 +47,14 @@ def world_grad_check(got, ref, n, name, rtol=WORLD_GRAD_RTOL, bad_frac=0.0, scal
 
 class GpuRun:
     def __init__(self, pkg, scene, sh_degree=3, use_list=False, use_packed=False, packed_projection=False,
-                 read_nnz=True, use_vrows=False, tile_sort=False, capacity=None, world_rows=False, bwd_lanes=False):
+                 read_nnz=True, use_vrows=False, tile_sort=False, capacity=None, world_rows=False, bwd_lanes=False, block_masks=False):
         """use_packed: 48-byte fragment rows for the compositing kernels. packed_projection: the
         compacted (nnz-row) projection outputs of projection_3dgs_packed_forward; read_nnz=False
         sizes the outputs for all N splats instead of reading nnz back between the two calls."""
         self.use_list = use_list
         self.use_packed = use_packed
         self.bwd_lanes = bwd_lanes   # SSR_BWD_SCHEDULE_LANES for the compositing backward (plain variant only)
+        self.block_masks = block_masks   # the forward records every entry's block mask and the backward reads them
         self.packed_projection = packed_projection
         self.read_nnz = read_nnz
         # world_rows (with packed_projection): the projection also writes each visible splat's parameters (four
@@ -353,6 +354,9 @@ class GpuRun:
             p.render_median = self.ptr("r_median")
         p.tile_order = self.ptr("tile_order")
         p.tile_offsets_closed = 1 if self.capacity is not None else 0
+        if self.block_masks and self.K > 0:
+            self.d["block_masks"] = D((self.K,), np.uint16)
+            p.block_masks = self.ptr("block_masks")
         self.check(self.lib.ssr_raster_fwd(C.byref(p), None))
 
     def raster_bwd(self, v_rgb=None, v_depth=None, v_T=None):
@@ -404,6 +408,8 @@ class GpuRun:
         p.tile_order = self.ptr("tile_order")
         p.tile_offsets_closed = 1 if self.capacity is not None else 0
         p.schedule = 1 if self.bwd_lanes else 0
+        if self.block_masks and "block_masks" in self.d:
+            p.block_masks = self.ptr("block_masks")
         self.check(self.lib.ssr_raster_bwd(C.byref(p), None))
         if self.use_vrows and n:   # unpack for the comparisons, after checking the arrays were left alone
             for k in ["v_xy", "v_depth", "v_conic", "v_opac", "v_rgb"]:

@@ -34,15 +34,16 @@ def _grad_close(got, ref, abs_scale, name, max_bad=0, rtol=GRAD_RTOL, afrac=2e-6
 
 
 def _compare(gpu, oracle, sc, label, fused_count=False, use_list=False, use_packed=False, mask=None, variant=None,
-             use_vrows=False, tile_sort=False, spare=None, bwd_lanes=False):
+             use_vrows=False, tile_sort=False, spare=None, bwd_lanes=False, block_masks=False):
     """spare: run K4-K6 without reading the counts back, in arrays of K + spare entries (spare >= 0). bwd_lanes: the
-    compositing backward with one lane per fragment (SSR_BWD_SCHEDULE_LANES)."""
+    compositing backward with one lane per fragment (SSR_BWD_SCHEDULE_LANES). block_masks: the forward records the
+    block mask of every staged entry and the backward reads them instead of repeating the tests."""
     live = None if mask is None else oracle.compute_tile_active(mask, sc.width, sc.height)
     r = oracle.pipeline(sc, tile_active=live, variant=variant)
     print(f"[{label}] N={sc.n} {sc.width}x{sc.height} visible={r['proj']['visible']} K={r['isect_ids'].size}", flush=True)
     K = r["isect_ids"].size
     g = GpuRun(gpu, sc, use_list=use_list, use_packed=use_packed, use_vrows=use_vrows, tile_sort=tile_sort,
-               capacity=None if spare is None else K + spare, bwd_lanes=bwd_lanes)
+               capacity=None if spare is None else K + spare, bwd_lanes=bwd_lanes, block_masks=block_masks)
     if mask is not None:
         g.set_tile_mask(mask)
         assert np.array_equal(g.host("tile_active"), live)
@@ -383,6 +384,8 @@ def test_backward_schedules(gpu, oracle, lanes):
     S = gpu.scenes
     kw = dict(bwd_lanes=lanes)
     _compare(gpu, oracle, S.tiny_scene(n=300, width=64, height=48, seed=11), f"sched{int(lanes)}-tiny", **kw)
+    _compare(gpu, oracle, S.tiny_scene(n=300, width=64, height=48, seed=11), f"sched{int(lanes)}-tiny-masks", block_masks=True, **kw)
+    kw["block_masks"] = True   # the rest with the forward's block masks handed to the backward, as the engine runs
     _compare(gpu, oracle, S.tiny_scene(n=700, width=70, height=37, seed=12), f"sched{int(lanes)}-ragged", use_packed=True, use_vrows=True, **kw)
     sc = S.tiny_scene(n=400, width=80, height=64, seed=13)
     sc.opacity_logits[::3] = 9.0          # sigmoid 0.99988: the pixel under the centre saturates at 0.999
@@ -405,7 +408,7 @@ def test_bench_configs_full_against_the_oracle(gpu, oracle, cfg):
     equirectangular 4096x2048) whole and at full size against the oracle, on the stage order the benchmark runs: every key, id, range and last id bit for bit, every pixel to 1e-4, every
     gradient row to 1e-3."""
     _compare(gpu, oracle, gpu.scenes.make_scene(cfg), f"cfg{cfg}-full", fused_count=True, use_list=True, use_packed=True,
-             use_vrows=True, tile_sort=True, bwd_lanes=cfg == 2)   # the cut the engine picks for each (tiles per visible splat)
+             use_vrows=True, tile_sort=True, bwd_lanes=cfg == 2, block_masks=True)   # the cut the engine picks for each (tiles per visible splat)
 
 
 @pytest.mark.parametrize("codec,stride", [(1, 256), (1, 0), (2, 256), (3, 0)])
