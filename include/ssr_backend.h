@@ -99,7 +99,7 @@ typedef struct {
 
 /* ---- K1: projection_3dgs_forward (src/kernels/projection/ProjectionFwd.cuh:18-36,
  * kernel src/kernels/projection/ProjectionFwd_kernel.cuh:17-111). Writes aabb/sort_depth for every
- * splat, the screen row and atomic-max radii only for visible ones. If tiles_per_splat is
+ * splat, the screen row and atomic-max radii only for visible ones (radii_store: every row). If tiles_per_splat is
  * non-NULL the tile count of K2 is produced in the same pass. */
 typedef struct {
     int64_t num_splats;
@@ -109,7 +109,7 @@ typedef struct {
     ssr_camera camera;
     float* aabb;            /* [C,N,4] */
     float* sort_depth;      /* [C,N] */
-    float* radii;           /* [N], caller zero-fills (src/engine/EngineForward.cpp:66-69) */
+    float* radii;           /* [N], caller zero-fills (src/engine/EngineForward.cpp:66-69) unless radii_store */
     ssr_screen screen;
     int64_t* tiles_per_splat; /* optional [C*N] */
     /* Optional work list (no counterpart in the reference's non-packed path): the indices of the
@@ -126,6 +126,13 @@ typedef struct {
      * `antialiased` argument of the same projection function): screen-space blur 0.1 instead of 0.3 and the opacity
      * multiplied by sqrt(det cov2d / det (cov2d + blur)); everything after the projection is unchanged. */
     int32_t antialiased;
+    /* Non-zero: radii[g] is stored -- the radius of a visible splat, 0 of a culled one -- instead of max-accumulated.
+     * For a launch that is the only writer of `radii` (one camera) this gives what the zero-fill and the atomic max
+     * give, and the caller needs no zero-fill. */
+    int32_t radii_store;
+    /* Optional: an int64 this launch sets to zero. A caller that alternates between two visible counters has the
+     * one of its NEXT projection cleared here, in place of a fill launch of its own before every projection. */
+    int64_t* clear_count;
 } ssr_projection_fwd_params;
 int ssr_projection_fwd(const ssr_projection_fwd_params* p, ssr_stream_t stream);
 

@@ -57,6 +57,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_fwd_kernel(ssr_projecti
     __shared__ int s_count;
     __shared__ long long s_base;
     if (threadIdx.x == 0) s_count = 0;
+    if (P.clear_count && blockIdx.x == 0 && threadIdx.x == 0) *P.clear_count = 0;
     __syncthreads();
     const int64_t block0 = (int64_t)blockIdx.x * kProjBlock;
     const int64_t g = block0 + threadIdx.x;
@@ -83,7 +84,9 @@ __global__ __launch_bounds__(kProjBlock) void projection_fwd_kernel(ssr_projecti
             P.screen.opac[g] = p.opac;
             aabb_out[g] = make_float4(bb[0], bb[1], bb[2], bb[3]);
             P.sort_depth[g] = p.sort_depth;
-            atomic_max_nonneg(P.radii + g, p.radius);
+            // stored: what the integer-ordered maximum with a zero leaves (a negative bit pattern loses to the zero)
+            if (P.radii_store) P.radii[g] = __float_as_int(p.radius) > 0 ? p.radius : 0.0f;
+            else atomic_max_nonneg(P.radii + g, p.radius);
             if (P.tiles_per_splat) {
                 const int tw = (int)((P.camera.width + kTile - 1) / kTile), th = (int)((P.camera.height + kTile - 1) / kTile);
                 TileGeomD tg;
@@ -104,6 +107,7 @@ __global__ __launch_bounds__(kProjBlock) void projection_fwd_kernel(ssr_projecti
             aabb_out[g] = make_float4(0.f, 0.f, 0.f, 0.f);
             P.sort_depth[g] = 0.0f;
             if (P.tiles_per_splat) P.tiles_per_splat[g] = 0;
+            if (P.radii_store) P.radii[g] = 0.0f;
         }
     }
     __syncthreads();

@@ -17,10 +17,16 @@ namespace ssr {
 // (RasterizationEval3DFwd_kernel.cuh:143-148,245-307): per-lane accumulators only.
 template <int kDist, bool kMedian>
 __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raster_fwd_params P, int tile_w, int tile_h) {
-    __shared__ FragLds frags[kBatch];
-    // distortion composites ln(max(z, 1e-6)): a per-splat value, taken once when the fragment is staged
-    [[maybe_unused]] __shared__ float s_lz[kDist != SSR_DIST_NONE ? kBatch : 1];
-    __shared__ uint8_t s_list[kBlocksPerTile * kBatch + 16];
+    // slot kBatch is a fragment of opacity zero: a list is padded with it up to the wavefront's step count, so that
+    // a step needs no test of its own for the end of its list
+    __shared__ FragLds frags[kBatch + 1];
+    // distortion composites ln(max(z, 1e-6)): a per-splat value, taken once when the fragment is staged (kept at the
+    // fragments' pitch, so that a list entry addresses it without a division)
+    [[maybe_unused]] __shared__ float s_lz[kDist != SSR_DIST_NONE ? (kBatch + 1) * 12 : 1];
+    // list entries are the fragments' byte offsets in `frags` (slot * 48 fits sixteen bits)
+    __shared__ uint16_t s_list[kBlocksPerTile * kBatch + 16];
+    static_assert(sizeof(FragLds) == 48 && kBatch * 48 < 65536, "list entries are 16-bit byte offsets of 48-byte fragments");
+    constexpr uint32_t kPadEntry = kBatch * 48;
     const int n_tiles = tile_w * tile_h * (P.num_images > 1 ? P.num_images : 1);
     const int tile = tile_of_workgroup(P.tile_order, blockIdx.x, n_tiles);
     if (tile < 0 || tile >= n_tiles) return;
@@ -31,26 +37,30 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raste
     const int i = ty * kTile + (mt >> 1) * kMicro + (row >> 1) * kBlock + (l16 >> 2);
     const float px = (float)j + 0.5f, py = (float)i + 0.5f;
     const bool inside = (uint32_t)i < P.height && (uint32_t)j < P.width;
-    int alive = inside ? 1 : 0;   // 0 once the pixel has stopped compositing (an int: the loop tests it with one compare)
 
     const int32_t range_start = P.tile_offsets[tile];
     const int32_t range_end = (tile == n_tiles - 1 && !P.tile_offsets_closed) ? (int32_t)P.n_isects : P.tile_offsets[tile + 1];
-    float T = 1.0f, cr = 0.f, cg = 0.f, cb = 0.f, cd = 0.f;
+    // The pixel's transmittance twice: T is the value that goes out; Tl is the same while the pixel composites and 0
+    // once it has stopped (or lies outside the image). A step then needs no flag: from Tl = 0 every product is 0,
+    // nothing passes the transmittance test and nothing is added.
+    float T = 1.0f, Tl = inside ? 1.0f : 0.0f, cr = 0.f, cg = 0.f, cb = 0.f, cd = 0.f;
     [[maybe_unused]] float s2r = 0.f, s2g = 0.f, s2b = 0.f, s2d = 0.f;           // second moments (distortion)
     [[maybe_unused]] float median = 0.f, med_prev_z = 0.f, med_prev_T = 1.0f;   // median depth
     uint32_t cur_idx = 0;
     const float tile_x0 = (float)(tx * kTile), tile_y0 = (float)(ty * kTile);
-    const uint8_t* my_list = s_list + (4 * mt + row) * kBatch;
-    // list entries are read a few steps ahead without asking whether the list reaches that far: every byte is a valid
-    // slot from the start (the first barrier of the batch loop orders this with the first reads)
-    for (int e = tid; e < (int)sizeof(s_list); e += kRasterBlock) s_list[e] = 0;
+    const uint16_t* my_list = s_list + (4 * mt + row) * kBatch;
+    // list entries are read a few steps ahead without asking whether the list reaches that far: every entry is a valid
+    // offset from the start (the first barrier of the batch loop orders this with the first reads)
+    for (int e = tid; e < (int)(sizeof(s_list) / sizeof(s_list[0])); e += kRasterBlock) s_list[e] = 0;
+    if (tid < 3) (&frags[kBatch].q0)[tid] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if constexpr (kDist != SSR_DIST_NONE) { if (tid == 0) s_lz[kBatch * 12] = 0.0f; }
 
     // the splat id a thread stages next is read one batch ahead: the fragment gather of the next batch then waits for
     // one memory round trip, not two in a row
     int32_t g_ahead = range_start + tid < range_end ? P.flatten_ids[range_start + tid] : 0;
     for (int32_t batch_start = range_start; batch_start < range_end; batch_start += kBatch) {
         // all pixels of the tile finished: stop (this barrier also fences reuse of the LDS batch)
-        if (__syncthreads_count(alive == 0) >= kRasterBlock) break;
+        if (__syncthreads_count(Tl == 0.0f) >= kRasterBlock) break;
         const int32_t idx = batch_start + tid;
         if (idx < range_end) {
             float kk;
@@ -58,7 +68,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raste
             add_block_mask(f, kk, tile_x0, tile_y0);
             frags[tid] = f;
             if (P.block_masks) P.block_masks[idx] = (uint16_t)(__float_as_uint(f.q2.z) >> 16);   // for the backward
-            if constexpr (kDist != SSR_DIST_NONE) s_lz[tid] = ssr_log(ssr_max(f.q2.y, 1e-6f));
+            if constexpr (kDist != SSR_DIST_NONE) s_lz[tid * 12] = ssr_log(ssr_max(f.q2.y, 1e-6f));
         } else {
             frags[tid].q2 = make_float4(0.f, 0.f, 0.f, 0.f);   // empty masks
         }
@@ -66,7 +76,7 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raste
         __syncthreads();
         const int n_batch = min(kBatch, range_end - batch_start);
         // a row whose sixteen pixels are finished needs no list
-        const uint64_t live = __ballot(alive != 0);
+        const uint64_t live = __ballot(Tl != 0.0f);
         const bool row_live[4] = {(live & 0xFFFFull) != 0, (live & 0xFFFF0000ull) != 0, (live & 0xFFFF00000000ull) != 0,
                                   (live & 0xFFFF000000000000ull) != 0};
         int cnt[4] = {0, 0, 0, 0};
@@ -79,37 +89,45 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raste
                     if (!row_live[r]) continue;
                     const bool in = ((bits >> r) & 1u) != 0;
                     const uint64_t bal = __ballot(in);
-                    if (in) s_list[(4 * mt + r) * kBatch + cnt[r] + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(bal >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)bal, 0u))] = (uint8_t)slot;
+                    if (in) s_list[(4 * mt + r) * kBatch + cnt[r] + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(bal >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)bal, 0u))] = (uint16_t)(slot * 48);
                     cnt[r] += __builtin_popcountll(bal);
                 }
             }
         }
+        // steps come in pairs: every list is padded to the even step count of the longest with the empty fragment
+        const int n_steps = (max(max(cnt[0], cnt[1]), max(cnt[2], cnt[3])) + 1) & ~1;
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+            for (int e = cnt[r] + lane; e < n_steps; e += 64) s_list[(4 * mt + r) * kBatch + e] = (uint16_t)kPadEntry;
         // the lists are written and read by this wavefront only: order its LDS accesses, no workgroup barrier
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        const int my_cnt = row == 0 ? cnt[0] : row == 1 ? cnt[1] : row == 2 ? cnt[2] : cnt[3];
-        const int n_steps = max(max(cnt[0], cnt[1]), max(cnt[2], cnt[3]));
-        // One step of a row: fragment k (registers q*) against the row's sixteen pixels, branch-free
-        auto step = [&](int st, int k, const float4& q0, const float4& q1, const float2& q2, float cut) {
+        uint32_t last_off = 0xFFFFFFFFu;   // offset of the last fragment this batch composited into the pixel
+        // One step of a row: the fragment at byte offset `off` (registers q*) against the row's sixteen pixels,
+        // branch-free. The same values as: hit = compositing && alpha > 1/255; keep = hit && T(1-alpha) > 1e-4;
+        // a kept fragment is added and T updated; a hit that is not kept ends the pixel.
+        auto step = [&](uint32_t off, const float4& q0, const float4& q1, const float2& q2, float cut) {
             float dx, dy, vis, sigma;
             const float alpha = eval_alpha_fast(q0, q1, cut, px, py, dx, dy, vis, sigma);
-            const bool hit = (alive != 0) & (st < my_cnt) & (alpha > kAlphaThreshold);
-            const float next_T = T * (1.0f - alpha);
+            const float a = alpha > kAlphaThreshold ? alpha : 0.0f;   // a skipped fragment: T (1 - 0) = T exactly
+            const float next_T = Tl * (1.0f - a);
             if constexpr (kMedian) {   // before the early-out, so a splat that ends the pixel still counts
+                const bool hit = (a > 0.0f) & (Tl > 0.0f);
                 const bool cross = hit & (med_prev_T >= 0.5f) & (next_T < 0.5f);
                 if (__builtin_amdgcn_ballot_w64(cross) != 0ull) {   // once per pixel: rarely any lane
-                    const float a = ssr_log(med_prev_T), b = ssr_log(next_T), d = b - a;
-                    const float fr = (ssr_fabs(d) > 1e-20f) ? (-0.6931471805599453f - a) / d : 0.0f;
+                    const float la = ssr_log(med_prev_T), lb = ssr_log(next_T), d = lb - la;
+                    const float fr = (ssr_fabs(d) > 1e-20f) ? (-0.6931471805599453f - la) / d : 0.0f;
                     median = cross ? med_prev_z + (q2.y - med_prev_z) * fr : median;
                 }
                 med_prev_T = hit ? next_T : med_prev_T;
                 med_prev_z = hit ? q2.y : med_prev_z;
             }
-            const bool keep = hit & (next_T > kTransmitThreshold);
-            const float w = keep ? alpha * T : 0.0f;   // a fragment that is not composited adds zero
+            // a compositing pixel has Tl > 1e-4, so a skipped fragment keeps it; a stopped one has next_T = 0
+            const bool keep = next_T > kTransmitThreshold;
+            const float w = keep ? a * Tl : 0.0f;   // a fragment that is not composited adds zero
             float zd = q2.y;
             if constexpr (kDist != SSR_DIST_NONE) {
-                zd = s_lz[k];
+                zd = s_lz[off >> 2];
                 if constexpr (kDist == SSR_DIST_RGB_D) {
                     s2r = ssr_fma(q1.z * q1.z, w, s2r); s2g = ssr_fma(q1.w * q1.w, w, s2g);
                     s2b = ssr_fma(q2.x * q2.x, w, s2b);
@@ -118,36 +136,37 @@ __global__ __launch_bounds__(kRasterBlock) void raster_fwd_rows_kernel(ssr_raste
             }
             cr = ssr_fma(q1.z, w, cr); cg = ssr_fma(q1.w, w, cg); cb = ssr_fma(q2.x, w, cb);
             cd = ssr_fma(zd, w, cd);
-            cur_idx = keep ? (uint32_t)(batch_start + k) : cur_idx;
+            last_off = w > 0.0f ? off : last_off;   // w > 0 exactly when the fragment was hit and kept (a > 1/255, Tl > 1e-4)
             T = keep ? next_T : T;
-            alive = (hit & !keep) ? 0 : alive;
+            Tl = keep ? next_T : 0.0f;
         };
-        // Software pipeline, two steps per trip: list bytes run two steps ahead of their use and the fragment of the
+        // Software pipeline, two steps per trip: list entries run two steps ahead of their use and the fragment of the
         // next step loads while the current one computes, so that the two dependent LDS latencies hide behind
         // arithmetic; the two fragment register sets alternate, so nothing is copied between steps.
-        auto list_at = [&](int st) { return (int)my_list[st]; };   // past the end: some valid slot, never used
-        // slots are below 256: a 24-bit multiply (full rate) addresses the fragment, not the quarter-rate 32-bit one
-        auto frag_of = [&](int k) -> const FragLds& {
-            return *reinterpret_cast<const FragLds*>(reinterpret_cast<const char*>(frags) + __umul24((unsigned)k, (unsigned)sizeof(FragLds)));
+        auto list_at = [&](int st) { return (uint32_t)my_list[st]; };   // past the padding: some valid offset, never used
+        auto frag_of = [&](uint32_t off) -> const FragLds& {
+            return *reinterpret_cast<const FragLds*>(reinterpret_cast<const char*>(frags) + off);
         };
-        int k0 = list_at(0), k1 = list_at(1), k2 = list_at(2);
+        uint32_t k0 = list_at(0), k1 = list_at(1), k2 = list_at(2);
         float4 a0 = frag_of(k0).q0, a1 = frag_of(k0).q1;
         float2 a2 = make_float2(frag_of(k0).q2.x, frag_of(k0).q2.y);
         float aw = frag_of(k0).q2.w;
-        for (int st = 0; st < n_steps; st += 2) {
-            if (__builtin_amdgcn_ballot_w64(alive != 0) == 0ull) break;   // this sub-tile is finished
+        int st = 0;
+        if (n_steps > 0 && live != 0ull) do {
             const float4 c0 = frag_of(k1).q0, c1 = frag_of(k1).q1;
             const float2 c2 = make_float2(frag_of(k1).q2.x, frag_of(k1).q2.y);
             const float cw = frag_of(k1).q2.w;
-            const int k3 = list_at(st + 3);
-            step(st, k0, a0, a1, a2, aw);
+            const uint32_t k3 = list_at(st + 3);
+            step(k0, a0, a1, a2, aw);
             a0 = frag_of(k2).q0; a1 = frag_of(k2).q1;
             a2 = make_float2(frag_of(k2).q2.x, frag_of(k2).q2.y);
             aw = frag_of(k2).q2.w;
-            const int k4 = list_at(st + 4);
-            step(st + 1, k1, c0, c1, c2, cw);   // beyond the lists every row is out of its list: nothing happens
+            const uint32_t k4 = list_at(st + 4);
+            step(k1, c0, c1, c2, cw);
             k0 = k2; k1 = k3; k2 = k4;
-        }
+            st += 2;
+        } while (st < n_steps && __builtin_amdgcn_ballot_w64(Tl != 0.0f) != 0ull);   // until this sub-tile is finished
+        if (last_off != 0xFFFFFFFFu) cur_idx = (uint32_t)batch_start + last_off / 48u;
     }
     if (inside) {
         const int64_t pid = ((int64_t)img * P.height + i) * P.width + j;

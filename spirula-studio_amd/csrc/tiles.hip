@@ -452,6 +452,61 @@ __global__ __launch_bounds__(kOrderBlock) void tile_order_scatter_kernel(const i
     if (live) order[base + rank] = (int32_t)t;
 }
 
+// The same order from one launch when the tiles are few enough for one workgroup to hold their classes in registers
+// (four per thread): count into LDS, scan the 256 classes, scatter. Measured: 2500 tiles 12.8 -> 9.0 us against the two
+// launches; at 8160 tiles one compute unit alone is the slower way (10 -> 17.7 us), hence the limit.
+constexpr int kOrderOnePer = 4;
+__global__ __launch_bounds__(kOrderBlock) void tile_order_one_kernel(const int32_t* __restrict__ offsets, uint32_t n_tiles,
+                                                                     int64_t n_isects, int32_t* __restrict__ order) {
+    __shared__ uint32_t s_next[256];
+    __shared__ uint32_t s_wave[4];
+    if (threadIdx.x < 256) s_next[threadIdx.x] = 0;
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    uint32_t cls[kOrderOnePer];
+#pragma unroll
+    for (int k = 0; k < kOrderOnePer; k++) {
+        const uint32_t t = (uint32_t)k * kOrderBlock + threadIdx.x;
+        cls[k] = t < n_tiles ? tile_class(offsets, t, n_tiles, n_isects) : 0u;
+    }
+#pragma unroll
+    for (int k = 0; k < kOrderOnePer; k++) {
+        if ((uint32_t)k * kOrderBlock >= n_tiles) break;   // the same for every thread
+        const bool live = (uint32_t)k * kOrderBlock + threadIdx.x < n_tiles;
+        const uint64_t peers = wave_peers_u8(cls[k], live);
+        if (live && (peers & ((1ull << lane) - 1ull)) == 0) atomicAdd(&s_next[cls[k]], (uint32_t)__popcll(peers));
+    }
+    __syncthreads();
+    uint32_t total = 0, incl = 0;
+    if (threadIdx.x < 256) {   // exclusive scan over the classes: four wavefronts, then their totals
+        total = incl = s_next[threadIdx.x];
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t up = __shfl_up(incl, d, 64);
+            if (lane >= d) incl += up;
+        }
+        if (lane == 63) s_wave[threadIdx.x >> 6] = incl;
+    }
+    __syncthreads();
+    if (threadIdx.x < 256) {
+        uint32_t add = 0;
+        for (uint32_t w = 0; w < (threadIdx.x >> 6); w++) add += s_wave[w];
+        s_next[threadIdx.x] = incl - total + add;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kOrderOnePer; k++) {
+        if ((uint32_t)k * kOrderBlock >= n_tiles) break;
+        const uint32_t t = (uint32_t)k * kOrderBlock + threadIdx.x;
+        const bool live = t < n_tiles;
+        const uint64_t peers = wave_peers_u8(cls[k], live);
+        const uint32_t rank = (uint32_t)__popcll(peers & ((1ull << lane) - 1ull));
+        uint32_t base = 0;
+        if (live && rank == 0) base = atomicAdd(&s_next[cls[k]], (uint32_t)__popcll(peers));
+        base = __shfl(base, peers ? __ffsll((long long)peers) - 1 : 0, 64);   // from the class's first lane
+        if (live) order[base + rank] = (int32_t)t;
+    }
+}
 
 }  // namespace ssr
 
@@ -676,6 +731,12 @@ int ssr_tile_order(const int32_t* tile_offsets, uint32_t n_tiles, int64_t n_isec
     if (n_tiles == 0) return 0;
     SSR_REQUIRE(tile_offsets && order, "ssr_tile_order", "null pointer");
     SSR_REQUIRE(scratch && scratch_bytes >= ssr_tile_order_scratch_bytes(n_tiles), "ssr_tile_order", "scratch too small");
+    if (n_tiles <= (uint32_t)(kOrderOnePer * kOrderBlock)) {
+        hipLaunchKernelGGL(tile_order_one_kernel, dim3(1), dim3(kOrderBlock), 0, as_stream(stream), tile_offsets, n_tiles, n_isects,
+                           order);
+        SSR_CHECK_LAUNCH("ssr_tile_order");
+        return 0;
+    }
     uint32_t* counts = static_cast<uint32_t*>(scratch);
     const dim3 grid((unsigned)ceil_div((int64_t)n_tiles, kOrderBlock)), block(kOrderBlock);
     hipLaunchKernelGGL(tile_order_count_kernel, grid, block, 0, as_stream(stream), tile_offsets, n_tiles, n_isects, counts);

@@ -27,7 +27,10 @@ ssr_ext::StageTimes g_times;
 int64_t g_n_isects = 0;
 int64_t g_n_visible = -1;
 bool g_counts_fused = false;         // the last projection already produced tile counts
-int64_t* g_counters = nullptr;       // device [n_isects, n_visible], one readback for both
+int64_t* g_counters = nullptr;       // device [n_isects, n_visible], one readback for both: one of the two pairs of the slot
+int64_t* g_counters_base = nullptr;  // the slot's two pairs; a projection with a visible list takes them in turn
+int g_counters_turn = 0;
+bool g_counters_clean[2] = {false, false};   // the pair's visible counter is known to be zero
 int32_t* g_visible_ids = nullptr;    // device work list of the last projection (null: off)
 float* g_packed_rows = nullptr;      // packed screen rows of the last projection (null: off)
 const float* g_packed_for_xy = nullptr;   // the screen.xy buffer those rows mirror
@@ -309,6 +312,7 @@ bool backward_overwrites_all_rows(int64_t num_splats) {
     return g_n_visible * 2 >= num_splats;
 }
 const int32_t* last_backward_list(int64_t* count) { if (count) *count = g_bwd_count; return g_bwd_list; }
+bool projection_stores_radii(int64_t cameras) { return cameras == 1; }
 void forget_packed_world_rows() { g_world_rows = nullptr; g_world_rows_for_ids = nullptr; g_world_rows_for_means = nullptr; g_world_rows_count = 0; }
 void zero_world_rows(const std::vector<DeviceTensorFloatND>& v, const int32_t* ids, int64_t n,
                      const DeviceTensor2D<float4>* aabb, const int32_t* sorted_now, int64_t n_now) {
@@ -317,6 +321,26 @@ void zero_world_rows(const std::vector<DeviceTensorFloatND>& v, const int32_t* i
        "zero_world_rows");
 }
 }  // namespace ssr_ext
+
+// The counters [n_isects, n_visible] live in one slot of two pairs, zeroed when the slot is first handed out.
+// next_turn: the caller is a projection that counts visible splats into the pair and has the other pair's counter
+// cleared by its kernel; otherwise the current pair is returned (only its n_isects is used).
+static int64_t* counters_pair(bool next_turn) {
+    int64_t* base = DevicePool::global().acquire<int64_t>(PoolSlot::IsectCounters, 4);
+    if (base != g_counters_base) {
+        g_counters_base = base;
+        g_counters_turn = 0;
+        backend::memset_async(base, 0, 4 * sizeof(int64_t));
+        g_counters_clean[0] = g_counters_clean[1] = true;
+    }
+    if (next_turn) {
+        g_counters_turn ^= 1;
+        // a projection that failed before its launch, or had no splats, has not cleared this pair
+        if (!g_counters_clean[g_counters_turn]) backend::memset_async(base + 2 * g_counters_turn, 0, 2 * sizeof(int64_t));
+        g_counters_clean[g_counters_turn] = false;   // about to count
+    }
+    return base + 2 * g_counters_turn;
+}
 
 // ---------------------------------------------------------------------------------------------
 std::tuple<DeviceTensor2D<float4>, DeviceTensor2D<float>, std::vector<DeviceTensorFloatND>>
@@ -356,16 +380,20 @@ projection_3dgs_forward(const int64_t num_splats, const int max_sh_degree,
         p.tiles_per_splat = DevicePool::global().acquire<int64_t>(PoolSlot::IsectTilesPerSplat, (size_t)(C * N));
         g_counts_fused = true;
     }
-    g_counters = DevicePool::global().acquire<int64_t>(PoolSlot::IsectCounters, 2);
+    g_counters = counters_pair(false);
     g_visible_ids = nullptr;
     g_n_visible = -1;
+    p.radii_store = C == 1 ? 1 : 0;   // the one writer of radii: same values as the caller's zero-fill and the maximum
     if (g_opts.visible_list && C == 1) {   // one list and one counter: a single camera's
         g_list_toggle ^= 1;
         g_visible_ids = DevicePool::global().acquire<int32_t>(
             g_list_toggle ? PoolSlot::ProjVisibleIdsB : PoolSlot::ProjVisibleIds, (size_t)(C * N));
-        backend::memset_async(g_counters, 0, 2 * sizeof(int64_t));
+        // the visible counter starts at zero: this projection clears the other pair's for the next one, as the
+        // one before did for this one (the pairs start out zeroed), so no fill is launched per projection
+        g_counters = counters_pair(true);
         p.visible_ids = g_visible_ids;
         p.visible_count = g_counters + 1;
+        p.clear_count = g_counters_base + 2 * (g_counters_turn ^ 1) + 1;
     }
     g_packed_rows = nullptr;
     g_packed_for_xy = nullptr;
@@ -385,6 +413,7 @@ projection_3dgs_forward(const int64_t num_splats, const int max_sh_degree,
             if (all.packed_rows) p.packed_rows = all.packed_rows + 12 * c * N;
             ok(ssr_projection_fwd(&p, nullptr), "projection_3dgs_forward");
         }
+        if (p.clear_count && N > 0) g_counters_clean[g_counters_turn ^ 1] = true;   // the launch went out
     }
     std::vector<DeviceTensorFloatND> screen = {
         DeviceTensorFloatND(xy, {C * N, 2}), DeviceTensorFloatND(dp, {C * N, 1}), DeviceTensorFloatND(cn, {C * N, 3}),
@@ -611,7 +640,7 @@ do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, 
         StageTimer t(&g_times.k3);
         const size_t sb = ssr_scan_scratch_bytes(total);
         void* scratch = DevicePool::global().acquire<uint8_t>(PoolSlot::IsectScanScratch, sb);
-        if (!g_counters) g_counters = DevicePool::global().acquire<int64_t>(PoolSlot::IsectCounters, 2);
+        if (!g_counters) g_counters = counters_pair(false);
         ok(ssr_inclusive_sum_i64(tiles_per_splat.data_ptr(), cum.data_ptr(), total, g_counters, scratch, sb, nullptr),
            "do_intersect_tile_generic/scan");
         if (total > 0 && g_opts.deferred_counts && g_opts.tile_sort && g_deferred_capacity > 0) {

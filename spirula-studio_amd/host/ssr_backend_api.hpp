@@ -223,6 +223,10 @@ const int32_t* last_backward_list(int64_t* count);
 // Drops the parameter rows kept under Options::packed_world_rows: for a caller that writes new parameter values
 // into the same tensors between a packed projection and its backward.
 void forget_packed_world_rows();
+// Whether projection_3dgs_forward with this many cameras stores every row of `radii` (one camera: its launch is the
+// only writer, so it stores what the caller's zero-fill and the atomic maximum would leave) -- a caller that
+// owns the buffer may then skip the fill.
+bool projection_stores_radii(int64_t cameras);
 // True when the next projection_3dgs_backward (after the forward that just ran) will overwrite EVERY
 // row of v_splats_world -- store mode, and either no work list or so many visible splats (half or
 // more) that walking all rows is cheaper than a zero-fill plus the list. The caller may then skip

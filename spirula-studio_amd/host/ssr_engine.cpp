@@ -146,9 +146,21 @@ void forward_3dgs(std::string primitive, int sh_degree, bool packed, bool output
         DeviceTensorFloatND((float*)E.world.opacities.data_ptr(), {E.world.opacities.size(), 1}),
         DeviceTensorFloatND(E.world.features_dc), DeviceTensorFloatND(E.world.features_sh)};
     E.fwd.splats_w = in_splats;
-    // radii: zeroed before projection, which accumulates with atomic max (EngineForward.cpp:66-69)
+    // radii: zeroed before projection, which accumulates with atomic max (EngineForward.cpp:66-69). A dense
+    // projection of one camera stores all N rows itself; the fill is then needed only for rows it does not reach
+    // (a new buffer, or fewer splats than the frame before).
     E.optim.radii.resize(PoolSlot::EngRadii, E.max_num_splats);
-    if (!E.optim.skip_grad_zero) E.optim.radii.zero();
+    {
+        static const float* zeroed_ptr = nullptr;
+        static int64_t zeroed_rows = 0, stored_rows = 0;
+        const bool stored = !packed && ssr_ext::projection_stores_radii(E.camera.num);
+        const bool covered = stored && zeroed_ptr == E.optim.radii.data_ptr() && zeroed_rows == E.max_num_splats && N >= stored_rows;
+        if (!covered && !E.optim.skip_grad_zero) {
+            E.optim.radii.zero();
+            zeroed_ptr = E.optim.radii.data_ptr(); zeroed_rows = E.max_num_splats;
+        }
+        stored_rows = stored ? N : E.max_num_splats;   // rows that may hold radii after this frame
+    }
 
     DeviceTensorFloatND aabb_nd, depths_nd;
     std::vector<DeviceTensorFloatND> screen;

@@ -46,7 +46,7 @@ class ProjectionFwdParams(C.Structure):
                 ("sh", ShQuant), ("camera", Camera), ("aabb", vp), ("sort_depth", vp),
                 ("radii", vp), ("screen", Screen), ("tiles_per_splat", vp), ("visible_ids", vp),
                 ("visible_count", vp), ("packed_rows", vp),
-                ("antialiased", C.c_int32)]
+                ("antialiased", C.c_int32), ("radii_store", C.c_int32), ("clear_count", vp)]
 
 
 class RasterFwdParams(C.Structure):

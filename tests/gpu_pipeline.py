@@ -202,9 +202,17 @@ class GpuRun:
     def projection_fwd(self, fused_count=False):
         if self.packed_projection:
             return self.projection_packed_fwd(fused_count)
-        for k in ["radii"]:
-            self.d[k].fill_zero()
+        # with the work list the launch stores every radius itself (radii_store): the buffer then starts out holding
+        # a large value in every row instead of the zero-fill, and a spare counter must come back cleared
+        store = bool(self.use_list)
+        if store:
+            self.check(self.lib.ssr_fill_u32(self.ptr("radii"), 0x7F000000, self.n, None))
+            self.d["spare_count"] = self.L.DeviceArray.from_host(np.array([12345], np.int64))
+        else:
+            self.d["radii"].fill_zero()
         p = self.L.ProjectionFwdParams()
+        p.radii_store = 1 if store else 0
+        p.clear_count = self.ptr("spare_count") if store else None
         p.num_splats, p.sh_degree = self.n, self.sh_degree
         p.antialiased = 1 if getattr(self.sc, "antialiased", False) else 0
         p.world, p.sh, p.camera = self.world(), self.shq(), self.camera()
@@ -218,6 +226,8 @@ class GpuRun:
             p.visible_ids = self.ptr("vis_ids")
             p.visible_count = self.d["counters"].ptr + 8
         self.check(self.lib.ssr_projection_fwd(C.byref(p), None))
+        if store:
+            assert int(self.host("spare_count")[0]) == 0, "clear_count was not cleared"
 
     def tiles(self, fused_count=False):
         sc, D = self.sc, self.L.DeviceArray

@@ -144,7 +144,7 @@ def test_sort_tile_pairs_empty_and_errors(L):
     assert lib.ssr_last_error() != b""
 
 
-@pytest.mark.parametrize("n_tiles", [1, 2, 63, 1023, 1024, 1025, 8160, 32768, 65536, 65537, 131072 + 5])
+@pytest.mark.parametrize("n_tiles", [1, 2, 63, 1023, 1024, 1025, 4095, 4096, 4097, 8160, 32768, 65536, 65537, 131072 + 5])
 @pytest.mark.parametrize("closed", [False, True])
 def test_tile_order(L, n_tiles, closed):
     """ssr_tile_order on synthetic tile ranges, on both sides of the size where one workgroup does it alone: a
