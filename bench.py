@@ -292,13 +292,16 @@ def run_config(args, pkg, host, lib, np, with_cpu):
                    args.packed_world_rows == (cfg == 4) and not args.n and
                    not (variants or args.fused_optimizer or args.lens != "none" or args.fisheye or args.mip))
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    prof, traffic, valu_inst, valu_busy, gpu_cycles = {}, None, None, None, None
     if default_run and os.path.exists(tpath):
         try:
             prof = json.load(open(tpath))
             traffic = prof.get(f"config{cfg}", {}).get(dom)
             valu_inst = prof.get(f"config{cfg}_valu_wave_instructions", {}).get(dom)
+            valu_busy = prof.get(f"config{cfg}_valu_busy_cycles_per_simd", {}).get(dom)
+            gpu_cycles = prof.get(f"config{cfg}_gpu_cycles", {}).get(dom)
         except Exception:
-            prof, traffic, valu_inst = {}, None, None
+            prof, traffic, valu_inst, valu_busy, gpu_cycles = {}, None, None, None, None
     # What the sort really does, beside the charged figure of stage_algorithmic_GBs (which prices the reference's
     # whole-key sweeps): pairs per second through the whole stage, the sweeps done, and the HBM bytes the profile saw
     sort_ms = acc.get("K5", 0.0) + (0.0 if tile_sort else acc.get("K6", 0.0))   # sort + tile offsets
@@ -354,11 +357,15 @@ def run_config(args, pkg, host, lib, np, with_cpu):
                      "frac": dom_gbs / HBM_PEAK_GBS, "traffic": traffic,
                      "algorithmic_bytes_per_launch": abd[dom], "avg_launch_ms": acc[dom]},
     }
-    if valu_inst:
-        # the dominant kernel is bound by vector-instruction issue, which neither "hbm" nor "mfma" names: a wavefront
-        # instruction holds one of the chip's 1024 SIMDs for 4 cycles; share of the measured duration at 2.4 GHz
+    if valu_inst and valu_busy and gpu_cycles:
+        # The dominant kernel is bound by vector-instruction issue, which neither "hbm" nor "mfma" names. From the
+        # committed profile of this configuration: wavefront instructions per launch, the SIMD cycles they occupy by
+        # instruction class (fp32 add/mul/fma 2.7, transcendental 7.8, the rest 4.1 cycles: measured rates,
+        # profiles/valu_issue_rates.md) spread over the 1024 SIMDs, and the kernel's own cycle count
+        # (GRBM_GUI_ACTIVE / 8) in the same profiling run. A model, and a lower bound where DPP forms are many.
         out["roofline"]["valu_issue"] = {"wave_instructions_per_launch": valu_inst,
-                                         "frac_of_issue_slots": valu_inst * 4 / 1024 / (acc[dom] * 1e-3 * 2.4e9)}
+                                         "modelled_busy_cycles_per_simd": valu_busy, "kernel_cycles": gpu_cycles,
+                                         "frac_of_issue_cycles": valu_busy / gpu_cycles}
     if cpu is not None:
         out["cpu_baseline"] = cpu   # one camera of the configuration
     return out

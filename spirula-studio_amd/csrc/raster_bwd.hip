@@ -624,7 +624,10 @@ extern "C" int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t strea
         default: SSR_ROWS(D, M, SSR_ACCUM_NONE); break;             \
     }
 #define SSR_ROWS_M(D) if (med) { SSR_ROWS_A(D, true) } else { SSR_ROWS_A(D, false) }
-    if (p->schedule == SSR_BWD_SCHEDULE_LANES && p->dist_type == SSR_DIST_NONE && !med && p->accum_mode == SSR_ACCUM_NONE)
+    // the lane-per-fragment cut covers the plain backward and, where the gradient rows carry them out, the weight sums
+    const bool sums = p->accum_mode == SSR_ACCUM_SUM || p->accum_mode == SSR_ACCUM_AVG;
+    if (p->schedule == SSR_BWD_SCHEDULE_LANES && p->dist_type == SSR_DIST_NONE && !med &&
+        (p->accum_mode == SSR_ACCUM_NONE || (sums && p->v_rows)))
         launch_raster_bwd_lanes(*p, tw, th, nimg, st);
     else if (p->dist_type == SSR_DIST_NONE && !med && p->accum_mode == SSR_ACCUM_AVG)
         hipLaunchKernelGGL(raster_bwd_rows_avg_kernel, grid, block, 0, st, *p, tw, th);

@@ -1,5 +1,5 @@
-// raster_bwd_lanes.hip -- K8, plain variant (no distortion, median or accumulation weights), with one LANE PER
-// FRAGMENT: the same sums as raster_bwd.hip (rasterize_to_pixels_bwd_kernel,
+// raster_bwd_lanes.hip -- K8 without distortion or median (plain, or with the loss-map weight sums of
+// accum_mode SUM / AVG, RasterizationEval3DBwd_kernel.cuh:520-538), with one LANE PER FRAGMENT: the same sums as raster_bwd.hip (rasterize_to_pixels_bwd_kernel,
 // src/kernels/raster/RasterizationEval3DBwd_kernel.cuh:423-494 with the fragment VJPs of
 // src/primitives/Primitive3DGS.cuh:262-300), cut differently.
 //
@@ -25,10 +25,12 @@
 
 namespace ssr {
 
-constexpr int kLB = 128;           // fragments staged per batch
-constexpr int kLCh = 10;           // channels per fragment: u, u dx, u dy, u dx^2, u dx dy, u dy^2, w_r, w_g, w_b, w_d
 constexpr int kChunk = 16;         // fragments per row and chunk
 
+// kLB fragments staged per batch; kLCh channels per fragment: u, u dx, u dy, u dx^2, u dx dy, u dy^2, w_r, w_g, w_b,
+// w_d and, with the weight sums, map * w and w. The sums' two channels are paid for with a shorter batch, so that four
+// workgroups still share a compute unit's LDS.
+template <int kLB, int kLCh, bool kSums>
 struct LanesShared {
     FragLds frags[kLB + 1];        // the last one is the blank fragment behind every list
     int32_t ids[kLB];
@@ -40,13 +42,17 @@ struct LanesShared {
     __attribute__((aligned(16))) float vT[256];
     __attribute__((aligned(16))) int32_t last[256];
     float4 v[256];                 // v_r, v_g, v_b, v_depth / W
+    float amap[kSums ? 256 : 1];   // the loss map's pixels (weight sums)
     int wave_max[4];
     int cnt[kBlocksPerTile];       // list lengths of the batch
     int next;                      // next block to hand out
 };
 
+template <bool kSums>
 __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) void raster_bwd_lanes_kernel(ssr_raster_bwd_params P, int tile_w, int tile_h) {
-    __shared__ LanesShared S;
+    constexpr int kLB = kSums ? 112 : 128, kLCh = kSums ? 12 : 10;
+    static_assert(kLB % kChunk == 0 && 2 * kLB <= kRasterBlock && kLB <= 255, "two staging threads per slot; slot numbers and the blank's are bytes");
+    __shared__ LanesShared<kLB, kLCh, kSums> S;
     const int n_tiles = tile_w * tile_h * (P.num_images > 1 ? P.num_images : 1);
     const int tile = tile_of_workgroup(P.tile_order, blockIdx.x, n_tiles);
     if (tile < 0 || tile >= n_tiles) return;
@@ -75,6 +81,7 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
         vT1 = vT1 + (out_depth * vd) * inv_alpha;
         vd = vd * inv_alpha;
         S.T[tid] = T1; S.vT[tid] = vT1; S.last[tid] = bin_final; S.v[tid] = make_float4(vr, vg, vb, vd);
+        if constexpr (kSums) S.amap[tid] = inside ? P.accum_weight_map[pid] : 0.0f;
         int row_last = bin_final;
 #pragma unroll
         for (int d = 8; d >= 1; d >>= 1) row_last = max(row_last, __shfl_xor(row_last, d, 16));
@@ -97,11 +104,11 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
     // (x, y, depth, conic[3], opac, rgb[3]) and leave them in the first copy; then all threads move the batch to
     // global memory in the order of the destination rows (raster_bwd.hip does the same).
     auto flush = [&]() {
-        {
+        if ((tid >> 1) < kLB) {
             const int slot = tid >> 1;
             const bool geom = (tid & 1) == 0;
             float m[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            const int c0 = geom ? 0 : 6, nc = geom ? 6 : 4;
+            const int c0 = geom ? 0 : 6, nc = geom ? 6 : kLCh - 6;
 #pragma unroll
             for (int w = 0; w < 4; w++)
 #pragma unroll
@@ -135,6 +142,7 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
                 dst[2] = ssr_isfinite(o[0]) ? o[0] : 0.f;
                 dst[7] = ssr_isfinite(o[1]) ? o[1] : 0.f; dst[8] = ssr_isfinite(o[2]) ? o[2] : 0.f;
                 dst[9] = ssr_isfinite(o[3]) ? o[3] : 0.f;
+                if constexpr (kSums) { dst[10] = ssr_isfinite(m[4]) ? m[4] : 0.f; dst[11] = ssr_isfinite(m[5]) ? m[5] : 0.f; }
             }
         }
         lds_barrier();
@@ -173,7 +181,7 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
     int32_t g_ahead = 0;
     {
         const int32_t idx0 = min(range_end - 1, tile_last) - (tid >= kLB ? tid - kLB : tid);
-        if (idx0 >= range_start) g_ahead = P.flatten_ids[idx0];
+        if (idx0 >= range_start && tid < 2 * kLB) g_ahead = P.flatten_ids[idx0];
     }
     for (int32_t hi = min(range_end - 1, tile_last); hi >= range_start; hi -= kLB) {
         lds_wait();
@@ -181,7 +189,7 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
         if (!first) flush();
         first = false;
         if (tid == 0) S.next = 0;
-        {
+        if (tid < 2 * kLB) {
             const int half = tid >= kLB ? 1 : 0, slot = tid - half * kLB;
             const int32_t idx = hi - slot;
             uint32_t bits8 = 0;
@@ -230,6 +238,8 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
             float Tc[4] = {Tq.x, Tq.y, Tq.z, Tq.w}, vTc[4] = {vTq.x, vTq.y, vTq.z, vTq.w};
             const int lastc[4] = {lastq.x, lastq.y, lastq.z, lastq.w};
             const float4 vc[4] = {S.v[pix0], S.v[pix0 + 1], S.v[pix0 + 2], S.v[pix0 + 3]};
+            [[maybe_unused]] float4 am = make_float4(0.f, 0.f, 0.f, 0.f);
+            if constexpr (kSums) am = *reinterpret_cast<const float4*>(S.amap + pix0);
             const float px0 = tile_x0 + (float)((bm & 1) * kMicro + (q & 1) * kBlock) + 0.5f;
             const float py = tile_y0 + (float)((bm >> 1) * kMicro + (q >> 1) * kBlock + row) + 0.5f;
             const uint8_t* lst = S.list + blk * kLB + l16;
@@ -360,10 +370,17 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
                 };
                 const float R0 = fold32(fold16(U, V1), fold16(Uy, V2));                 // u, u dx, u dy, u dx^2
                 const float R1 = fold32(fold16(V1 * dy, Uy * dy), fold16(Wr, Wg));      // u dx dy, u dy^2, w_r, w_g
-                const float R2 = fold32(fold16(Wb, Wd), 0.0f);                          // w_b, w_d (rows 0, 1)
                 float* cell = (slot < kLB ? my_acc + __umul24((unsigned)slot, (unsigned)kLCh) : dump) + row;
-                cell[0] += R0; cell[4] += R1;
-                if (row < 2) cell[8] += R2;
+                if constexpr (kSums) {   // rows 2 and 3 of the third register carry the weight sums: map * w and w
+                    const float Wa = ssr_fma(am.w, w[3], ssr_fma(am.z, w[2], ssr_fma(am.y, w[1], am.x * w[0])));
+                    const float Ww = (w[0] + w[1]) + (w[2] + w[3]);
+                    const float R2 = fold32(fold16(Wb, Wd), fold16(Wa, Ww));
+                    cell[0] += R0; cell[4] += R1; cell[8] += R2;
+                } else {
+                    const float R2 = fold32(fold16(Wb, Wd), 0.0f);                      // w_b, w_d (rows 0, 1)
+                    cell[0] += R0; cell[4] += R1;
+                    if (row < 2) cell[8] += R2;
+                }
                 };
                 if (sat_possible) chunk(std::true_type{}); else chunk(std::false_type{});
             }
@@ -381,7 +398,10 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
 
 int launch_raster_bwd_lanes(const ssr_raster_bwd_params& p, int tw, int th, int nimg, hipStream_t st) {
     const dim3 grid((unsigned)xcd_grid_size(tw * th * nimg)), block(kRasterBlock);
-    hipLaunchKernelGGL(raster_bwd_lanes_kernel, grid, block, 0, st, p, tw, th);
+    if (p.accum_mode == SSR_ACCUM_SUM || p.accum_mode == SSR_ACCUM_AVG)
+        hipLaunchKernelGGL(raster_bwd_lanes_kernel<true>, grid, block, 0, st, p, tw, th);
+    else
+        hipLaunchKernelGGL(raster_bwd_lanes_kernel<false>, grid, block, 0, st, p, tw, th);
     return 0;
 }
 

@@ -391,7 +391,15 @@ def test_backward_schedules(gpu, oracle, lanes):
     sc.opacity_logits[::3] = 9.0          # sigmoid 0.99988: the pixel under the centre saturates at 0.999
     sc.opacity_logits[1::7] = 6.9         # 0.99899: inside the band around the cap
     _compare(gpu, oracle, sc, f"sched{int(lanes)}-opaque", use_list=True, use_packed=True, use_vrows=True, tile_sort=True, **kw)
-    for n in (1, 16, 17, 128, 129, 257):  # every splat covers the one tile's every block: block lists of exactly n
+    # the loss-map weight sums (sum, avg) ride in the gradient rows' spare floats under either cut; batches of 112
+    for accum in (2, 3):
+        sc = S.tiny_scene(n=700, width=70, height=37, seed=14 + accum)
+        va = dict(dist_type=0, median=False, accum_mode=accum, **_variant_cotangents(sc, accum))
+        _compare(gpu, oracle, sc, f"sched{int(lanes)}-sums{accum}", use_packed=True, use_vrows=True, variant=va, **kw)
+    sc = S.make_scene(2, n=50000, width=480, height=270, parity_variant=True)
+    va = dict(dist_type=0, median=False, accum_mode=3, **_variant_cotangents(sc, 5))
+    _compare(gpu, oracle, sc, f"sched{int(lanes)}-sums-cfg2", fused_count=True, use_list=True, use_packed=True, use_vrows=True, tile_sort=True, variant=va, **kw)
+    for n in (1, 16, 17, 112, 113, 128, 129, 257):  # every splat covers the one tile's every block: block lists of exactly n
         sc = S.tiny_scene(n=n, width=16, height=16, seed=100 + n)
         sc.means[:, :2] *= 0.02
         sc.log_scales[:] = -1.0 + 0.2 * (sc.log_scales - sc.log_scales.mean())   # large, and not isotropic (an isotropic
