@@ -183,7 +183,8 @@ def run_config(args, pkg, host, lib, np, with_cpu):
     eng = host.Engine(sc, fuse_tile_count=native, visible_list=native and not args.packed_projection, packed_rows=native,
                       overwrite_world_grads=native, packed_projection=args.packed_projection, packed_vscreen=native,
                       tile_sort=native and not args.whole_key_sort, deferred_counts=deferred,
-                      packed_world_rows=args.packed_world_rows)
+                      packed_world_rows=args.packed_world_rows,
+                      backward_schedule={"auto": -1, "rows": 0, "lanes": 1}[args.backward_schedule])
 
     hyper = dict(lr_means=1.6e-6, lr_quats=1e-5, lr_scales=5e-5, lr_opacs=5e-4, lr_features_dc=2.5e-5, lr_features_sh=1.25e-6)
     adam_step = [0]
@@ -289,7 +290,7 @@ def run_config(args, pkg, host, lib, np, with_cpu):
     prof = {}
     # the profiles were taken with this script's default arguments for each config: they describe no other variant
     default_run = (native and ncam == 1 and tile_sort and args.packed_projection == (cfg == 4) and
-                   args.packed_world_rows == (cfg == 4) and not args.n and
+                   args.packed_world_rows == (cfg == 4) and not args.n and args.backward_schedule == "auto" and
                    not (variants or args.fused_optimizer or args.lens != "none" or args.fisheye or args.mip))
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     prof, traffic, valu_inst, valu_busy, gpu_cycles = {}, None, None, None, None
@@ -381,6 +382,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--reference-order", action="store_true",
                     help="run the stages exactly as the reference does (separate count pass, atomic K9 into zero-filled buffers)")
+    ap.add_argument("--backward-schedule", choices=["auto", "rows", "lanes"], default="auto",
+                    help="cut of the compositing backward: chosen from the tiles per visible splat, or forced")
     ap.add_argument("--whole-key-sort", action="store_true",
                     help="six whole-array digit passes + the offsets kernel instead of the tile-segmented sort")
     ap.add_argument("--lens", choices=["none", "opencv", "thin_prism", "rational"], default="none",

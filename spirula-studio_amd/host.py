@@ -33,6 +33,7 @@ SYMBOLS = {
     "ssrh_set_deferred_counts": (C.c_int, [C.c_int, C.c_int64]),
     "ssrh_deferred_capacity": (C.c_int64, []),
     "ssrh_set_packed_world_rows": (C.c_int, [C.c_int]),
+    "ssrh_set_backward_schedule": (C.c_int, [C.c_int]),
     "ssrh_forward_3dgs": (C.c_int, [C.c_char_p, C.c_int, C.c_int, C.c_int, C.c_int]),
     "ssrh_backward_from_render_grad": (C.c_int, [vp, vp, vp]),
     "ssrh_copy_render_to_host": (C.c_int, [vp, vp, vp]),
@@ -87,11 +88,12 @@ class Engine:
 
     def __init__(self, scene, device=0, fuse_tile_count=True, visible_list=True, packed_rows=True, overwrite_world_grads=True,
                  stage_profiling=False, sh_degree=3, packed_projection=False, packed_vscreen=True,
-                 tile_sort=True, deferred_counts=False, packed_world_rows=False):
+                 tile_sort=True, deferred_counts=False, packed_world_rows=False, backward_schedule=-1):
         """packed_projection: forward_3dgs(packed=true), the compacted projection outputs of
         projection_3dgs_packed_forward (the visible-splat work list then has no role).
         packed_world_rows (with packed_projection): that projection also keeps each visible splat's parameters as
         64 bytes in four planes, which the projection backward reads instead of gathering from five arrays.
+        backward_schedule: -1 lets the adapter choose the cut of the compositing backward, 0 / 1 force rows / lanes.
         deferred_counts (with tile_sort): after the first iteration the forward no longer waits for the
         intersection count; see set_deferred_counts."""
         self.h = load()
@@ -108,6 +110,7 @@ class Engine:
         check(self.h.ssrh_set_options(*self.opts, int(stage_profiling), self.packed_vscreen, self.tile_sort))
         self.set_deferred_counts(deferred_counts, 0)
         check(self.h.ssrh_set_packed_world_rows(int(bool(packed_world_rows))))
+        check(self.h.ssrh_set_backward_schedule(int(backward_schedule)))
         f32 = lambda a: np.ascontiguousarray(a, np.float32)
         self._keep = [f32(scene.means), f32(scene.quats), f32(scene.log_scales), f32(scene.opacity_logits),
                       f32(scene.features_dc), f32(scene.features_sh)]

@@ -834,11 +834,13 @@ rasterize_to_pixels_3dgs_bwd(int64_t num_splats, std::vector<DeviceTensorFloatND
     if (g_block_masks && g_block_masks_for == p.flatten_ids) p.block_masks = g_block_masks;
     {
         // The lane-per-fragment cut pays where a splat reaches several 4x4 blocks of a tile, which shows as tiles per
-        // visible splat: three and more (measured: 3.7 on the 1M-splat 1080p scene, K8 0.50 -> 0.44 ms; 1.8 on the
-        // 6M-splat equirectangular one, 1.50 -> 1.66 ms). The counts are the last ones the host has seen.
+        // visible splat. Measured (K8, rows / lanes, ms): 3.9 tiles per splat 0.109 / 0.080 (100k splats, 800x800);
+        // 3.7: 0.50 / 0.40 (1M, 1080p); 2.4: 0.592 / 0.558 (10M seen from inside, 4k); 1.9: 0.357 / 0.372 (3M, 1080p);
+        // 1.8: 1.45 / 1.57 (6M, equirectangular 4096x2048). The counts are the last ones the host has seen.
         const int64_t rows_seen = g_packed_mode ? p.num_splats : g_n_visible;
         const int64_t pairs_seen = g_n_isects > 0 ? g_n_isects : p.n_isects;
-        p.schedule = (rows_seen > 0 && pairs_seen >= 3 * rows_seen) ? SSR_BWD_SCHEDULE_LANES : SSR_BWD_SCHEDULE_ROWS;
+        p.schedule = (rows_seen > 0 && 5 * pairs_seen >= 11 * rows_seen) ? SSR_BWD_SCHEDULE_LANES : SSR_BWD_SCHEDULE_ROWS;
+        if (g_opts.backward_schedule >= 0) p.schedule = g_opts.backward_schedule ? SSR_BWD_SCHEDULE_LANES : SSR_BWD_SCHEDULE_ROWS;
     }
     p.render_T = render_Ts.data_ptr(); p.last_ids = last_ids.data_ptr(); p.render_depth = std::get<1>(render_outputs_tuple).data_ptr();
     p.v_render_rgb = (const float*)std::get<0>(v_render_outputs).data_ptr();

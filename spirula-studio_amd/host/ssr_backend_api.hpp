@@ -197,6 +197,10 @@ struct Options {
     // small, scattered part of the splats). For callers that do not change the parameters between a packed
     // projection and its backward: tensors are recognised by their addresses, not by their contents.
     bool packed_world_rows = false;
+    // Which cut of the compositing backward runs where both can (no distortion, no median; weight sums only with
+    // packed_vscreen): -1 lets the adapter choose from the tiles per visible splat it last saw, 0 a row of lanes per
+    // fragment (SSR_BWD_SCHEDULE_ROWS), 1 a lane per fragment (SSR_BWD_SCHEDULE_LANES).
+    int backward_schedule = -1;
     // int8 codes x per-splat fp16 scale as SH storage (the benchmark's format): sh_value_bits == 8
     // with sh_value_bounds holding the fp16 scales when this is set.
     bool sh_int8_f16scale = false;

@@ -494,6 +494,14 @@ int ssrh_set_packed_world_rows(int on) {
     return guard([&] { ssr_ext::options().packed_world_rows = on != 0; });
 }
 
+// -1: the adapter chooses the cut of the compositing backward; 0 / 1: rows / lanes (Options::backward_schedule)
+int ssrh_set_backward_schedule(int schedule) {
+    return guard([&] {
+        if (schedule < -1 || schedule > 1) throw std::runtime_error("ssrh_set_backward_schedule: -1 (auto), 0 (rows) or 1 (lanes)");
+        ssr_ext::options().backward_schedule = schedule;
+    });
+}
+
 // host or device pointers; num_sh = coefficients per splat excluding DC (15 for SH3)
 int ssrh_set_data_3dgs(int64_t n, const float* means, const float* quats, const float* scales, const float* opacities,
                        const float* dc, const float* sh, int num_sh) {

@@ -387,6 +387,31 @@ def test_engine_fused_optimizer_scale_agnostic_means(pkg, oracle, H, packed):
         assert (d > 0.05 * 5e-2).mean() < 2e-3, k
 
 
+@pytest.mark.parametrize("schedule", [0, 1])
+def test_engine_backward_schedule_forced(pkg, oracle, H, schedule):
+    """The engine with either cut of the compositing backward forced (the adapter otherwise picks one from the tiles
+    per visible splat): same keys, image and gradients, and the loss-map weight sums of the fused step."""
+    host, lib = H
+    sc = pkg.scenes.make_scene(1, n=30000, width=320, height=240, parity_variant=True)
+    ref = oracle.pipeline(sc)
+    eng = host.Engine(sc, backward_schedule=schedule)
+    for _ in range(2):
+        eng.forward()
+        eng.backward()
+        _check(eng, ref, sc)
+    amap = np.random.default_rng(6).uniform(0, 1, (sc.height, sc.width)).astype(np.float32)
+    d_map = lib.DeviceArray.from_host(amap)
+    eng.set_loss_map(d_map.ptr, 3)
+    eng.forward()
+    eng.backward_fused_optimizer(dict(lr_means=1.6e-4, lr_quats=1e-3, lr_scales=5e-3, lr_opacs=5e-2, lr_features_dc=2.5e-3,
+                                      lr_features_sh=1.25e-4), 1)
+    aw = eng.cache("accum_weight")
+    r = oracle.pipeline(sc, backward=True, variant=dict(dist_type=0, median=False, accum_mode=3, accum_map=amap))
+    want = r["vscreen"]["accum_weight"]
+    assert np.allclose(aw[:want.size], want, rtol=1e-3, atol=1e-6) and (aw[:sc.n] > 0).sum() > 1000
+    eng.set_loss_map(None, 0)
+
+
 @pytest.mark.parametrize("packed,accum_mode", [(False, 3), (True, 3), (False, 1), (True, 2)])
 def test_engine_fused_step_accumulates_the_loss_map(pkg, oracle, H, packed, accum_mode):
     """The training step of the reference accumulates its loss map per splat in the same compositing backward that

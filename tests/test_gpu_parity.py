@@ -416,7 +416,7 @@ def test_bench_configs_full_against_the_oracle(gpu, oracle, cfg):
     equirectangular 4096x2048) whole and at full size against the oracle, on the stage order the benchmark runs: every key, id, range and last id bit for bit, every pixel to 1e-4, every
     gradient row to 1e-3."""
     _compare(gpu, oracle, gpu.scenes.make_scene(cfg), f"cfg{cfg}-full", fused_count=True, use_list=True, use_packed=True,
-             use_vrows=True, tile_sort=True, bwd_lanes=cfg == 2, block_masks=True)   # the cut the engine picks for each (tiles per visible splat)
+             use_vrows=True, tile_sort=True, bwd_lanes=cfg in (2, 4), block_masks=True)   # the cut the engine picks for each (tiles per visible splat)
 
 
 @pytest.mark.parametrize("codec,stride", [(1, 256), (1, 0), (2, 256), (3, 0)])
