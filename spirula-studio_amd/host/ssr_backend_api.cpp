@@ -26,6 +26,8 @@ bool g_profile = false;
 ssr_ext::StageTimes g_times;
 int64_t g_n_isects = 0;
 int64_t g_n_visible = -1;
+int64_t g_seen_visible = -1;         // the last visible count the host learned, kept over the projections that follow it
+                                     // (g_n_visible starts unknown again with every projection)
 bool g_counts_fused = false;         // the last projection already produced tile counts
 int64_t* g_counters = nullptr;       // device [n_isects, n_visible], one readback for both: one of the two pairs of the slot
 int64_t* g_counters_base = nullptr;  // the slot's two pairs; a projection with a visible list takes them in turn
@@ -284,7 +286,7 @@ void resolve_counts() {
     g_counts_pending = false;
     ok(ssr_event_synchronize(g_counts_event), "resolve_counts");
     g_n_isects = g_counts_host[0];
-    if (g_visible_ids) g_n_visible = g_counts_host[1];
+    if (g_visible_ids) g_seen_visible = g_n_visible = g_counts_host[1];
     const int64_t used = g_deferred_used;
     if (g_n_isects > used) {
         g_deferred_capacity = 0;   // the next intersection reads its count and sizes from it
@@ -659,7 +661,7 @@ do_intersect_tile_generic(DeviceTensorFloatND aabb, DeviceTensorFloatND depths, 
             int64_t both[2] = {0, 0};
             ok(ssr_read_i64(g_counters, both, g_visible_ids ? 2 : 1, nullptr), "do_intersect_tile_generic/readback");
             n_isects = both[0];
-            if (g_visible_ids) g_n_visible = both[1];
+            if (g_visible_ids) g_seen_visible = g_n_visible = both[1];
         }
     }
     if (g_counts_pending)
@@ -836,8 +838,9 @@ rasterize_to_pixels_3dgs_bwd(int64_t num_splats, std::vector<DeviceTensorFloatND
         // The lane-per-fragment cut pays where a splat reaches several 4x4 blocks of a tile, which shows as tiles per
         // visible splat. Measured (K8, rows / lanes, ms): 3.9 tiles per splat 0.109 / 0.080 (100k splats, 800x800);
         // 3.7: 0.50 / 0.40 (1M, 1080p); 2.4: 0.592 / 0.558 (10M seen from inside, 4k); 1.9: 0.357 / 0.372 (3M, 1080p);
-        // 1.8: 1.45 / 1.57 (6M, equirectangular 4096x2048). The counts are the last ones the host has seen.
-        const int64_t rows_seen = g_packed_mode ? p.num_splats : g_n_visible;
+        // 1.8: 1.45 / 1.57 (6M, equirectangular 4096x2048). The counts are the last ones the host has seen (with deferred counts, the
+        // iteration before's: a backward that needs no count of its own does not wait for this iteration's).
+        const int64_t rows_seen = g_packed_mode ? p.num_splats : (g_n_visible >= 0 ? g_n_visible : g_seen_visible);
         const int64_t pairs_seen = g_n_isects > 0 ? g_n_isects : p.n_isects;
         p.schedule = (rows_seen > 0 && 5 * pairs_seen >= 11 * rows_seen) ? SSR_BWD_SCHEDULE_LANES : SSR_BWD_SCHEDULE_ROWS;
         if (g_opts.backward_schedule >= 0) p.schedule = g_opts.backward_schedule ? SSR_BWD_SCHEDULE_LANES : SSR_BWD_SCHEDULE_ROWS;
