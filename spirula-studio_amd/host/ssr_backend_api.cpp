@@ -329,7 +329,9 @@ void zero_world_rows(const std::vector<DeviceTensorFloatND>& v, const int32_t* i
 // cleared by its kernel; otherwise the current pair is returned (only its n_isects is used).
 static int64_t* counters_pair(bool next_turn) {
     int64_t* base = DevicePool::global().acquire<int64_t>(PoolSlot::IsectCounters, 4);
-    if (base != g_counters_base) {
+    static uint64_t generation = ~(uint64_t)0;
+    if (base != g_counters_base || generation != DevicePool::global().generation()) {
+        generation = DevicePool::global().generation();
         g_counters_base = base;
         g_counters_turn = 0;
         backend::memset_async(base, 0, 4 * sizeof(int64_t));

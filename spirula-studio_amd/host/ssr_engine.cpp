@@ -151,10 +151,13 @@ void forward_3dgs(std::string primitive, int sh_degree, bool packed, bool output
     // (a new buffer, or fewer splats than the frame before).
     E.optim.radii.resize(PoolSlot::EngRadii, E.max_num_splats);
     {
-        static const float* zeroed_ptr = nullptr;
-        static int64_t zeroed_rows = 0, stored_rows = 0;
+        const float*& zeroed_ptr = E.optim.radii_zeroed_ptr;
+        int64_t &zeroed_rows = E.optim.radii_zeroed_rows, &stored_rows = E.optim.radii_stored_rows;
         const bool stored = !packed && ssr_ext::projection_stores_radii(E.camera.num);
-        const bool covered = stored && zeroed_ptr == E.optim.radii.data_ptr() && zeroed_rows == E.max_num_splats && N >= stored_rows;
+        static uint64_t generation = ~(uint64_t)0;   // of the pool the buffer comes from
+        const bool same_pool = generation == DevicePool::global().generation();
+        generation = DevicePool::global().generation();
+        const bool covered = stored && same_pool && zeroed_ptr == E.optim.radii.data_ptr() && zeroed_rows == E.max_num_splats && N >= stored_rows;
         if (!covered && !E.optim.skip_grad_zero) {
             E.optim.radii.zero();
             zeroed_ptr = E.optim.radii.data_ptr(); zeroed_rows = E.max_num_splats;

@@ -34,6 +34,8 @@ struct EngineState {
     } camera;
     struct {
         DeviceVector<float> radii; bool skip_grad_zero = false;
+        // which rows of `radii` are known to hold zeros or the last projection's values (forward_3dgs)
+        const float* radii_zeroed_ptr = nullptr; int64_t radii_zeroed_rows = 0, radii_stored_rows = 0;
         bool adam_ready = false;
         bool sh_state_ready = false;   // quantization level 1: the 8-bit SH moments have been zeroed
         bool non_sh_state_ready = false;   // non_sh_optim_bits 16: the 16-bit non-SH moments have been zeroed

@@ -81,6 +81,7 @@ class DevicePool {
     struct Slot { void* ptr = nullptr; size_t cap = 0, used = 0; };
     std::vector<Slot> slots_;
     mutable std::mutex mu_;
+    uint64_t generation_ = 0;
     DevicePool() : slots_((size_t)PoolSlot::Count) {}
 public:
     static DevicePool& global() { static DevicePool p; return p; }
@@ -102,7 +103,11 @@ public:
     void free_all() {
         std::lock_guard<std::mutex> lock(mu_);
         for (auto& s : slots_) { if (s.ptr) backend::device_free(s.ptr); s = Slot{}; }
+        generation_++;
     }
+    // Changes whenever the pool has given its memory back: what a caller remembers about a slot's CONTENTS (a
+    // buffer it has zeroed once) holds only within one generation, whatever address the slot has afterwards.
+    uint64_t generation() const { std::lock_guard<std::mutex> l(mu_); return generation_; }
 };
 
 template <typename T>
