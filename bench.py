@@ -10,7 +10,7 @@ does, later ones leave them on the device; --blocking-counts reads them every ti
 64-bit radix sort -> tile offsets -> compositing forward -> zero the gradient rows -> compositing
 backward -> projection backward. After the headline configuration the other four run briefly in the
 same process (all_configs).
-Prints ONE JSON line: the metric of BASELINE.json (iterations/s), a `roofline` object for the
+Prints ONE JSON line: the benchmark's metric (forward+backward iterations/s), a `roofline` object for the
 kernel that takes the most time, and a `cpu_baseline` object (the CPU oracle timed on this host).
 """
 import argparse
@@ -97,7 +97,7 @@ def _time_oracle(oracle_lib, sc, threads, min_iters, budget_s):
 
 
 def lavapipe_status():
-    """The baseline BASELINE.json asks for is the reference's Vulkan path on Mesa lavapipe. It needs the reference
+    """The baseline the benchmark definition asks for is the reference's Vulkan path on Mesa lavapipe. It needs the reference
     tree, slangc and a Vulkan loader with the lavapipe ICD on this host; say what is missing instead of a number."""
     import glob
     import shutil
@@ -377,7 +377,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--config", type=int, default=2, help="1..5 (BASELINE.json configs; 2 is the headline)")
+    ap.add_argument("--config", type=int, default=2, help="1..5 (the five benchmark configurations; 2 is the headline)")
     ap.add_argument("--n", type=int, default=None, help="override the number of Gaussians")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--reference-order", action="store_true",
@@ -449,7 +449,7 @@ def main():
                          or args.cameras != 1 or args.n)
     out = run_config(args, pkg, host, lib, np, with_cpu=not args.no_cpu_baseline)
     if default_plain and not args.no_all_configs:
-        # the other four configurations of BASELINE.json, a short run each in this same process (no CPU leg; K_f then
+        # the other four benchmark configurations, a short run each in this same process (no CPU leg; K_f then
         # stands at its lower bound K_b): iterations/s and both roofline fractions per configuration
         import copy
         rows = []

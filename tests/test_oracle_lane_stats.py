@@ -1,6 +1,6 @@
 """Lane statistics of the compositing backward on the oracle's forward (CPU): of the pixels a (splat,
 pixel-block) visit covers, how many composite the splat, for blocks of 8x8 (one wavefront per visit), 4x4 and
-2x2 pixels. Run with -s to print the table; LANE_STATS_FULL=1 runs the BASELINE configs 2 and 5 at full size
+2x2 pixels. Run with -s to print the table; LANE_STATS_FULL=1 runs benchmark configurations 2 and 5 at full size
 (tens of seconds), otherwise reduced copies that keep the splat footprint in pixels."""
 import os
 
