@@ -60,6 +60,10 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
     const int gy = tile / tile_w, tx = tile - gy * tile_w;
     const int img = gy / tile_h, ty = gy - img * tile_h;
     const float tile_x0 = (float)(tx * kTile), tile_y0 = (float)(ty * kTile);
+    // the tile's range is asked for here, with the pixel state: behind the barrier below it would be one more memory
+    // round trip in the chain order -> range -> ids -> rows that every tile starts with
+    const int32_t range_start = P.tile_offsets[tile];
+    const int32_t range_end = (tile == n_tiles - 1 && !P.tile_offsets_closed) ? (int32_t)P.n_isects : P.tile_offsets[tile + 1];
     int wave_last;
     int blk_last[4];
     {   // set-up: thread = pixel (block `row` of sub-tile mt, pixel l16 of the block), as in raster_bwd.hip
@@ -97,8 +101,6 @@ __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(4,
     }
     __syncthreads();
     const int tile_last = max(max(S.wave_max[0], S.wave_max[1]), max(S.wave_max[2], S.wave_max[3]));
-    const int32_t range_start = P.tile_offsets[tile];
-    const int32_t range_end = (tile == n_tiles - 1 && !P.tile_offsets_closed) ? (int32_t)P.n_isects : P.tile_offsets[tile + 1];
 
     // Thread pairs own a slot: they add up the four wavefronts' sums, turn moments into the ten gradient channels
     // (x, y, depth, conic[3], opac, rgb[3]) and leave them in the first copy; then all threads move the batch to
