@@ -27,6 +27,8 @@
 // exp(-sigma) comes from the hardware exponential; whenever a lane's alpha falls within 1.6e-7 of the 1/255
 // threshold or within 4e-5 of the 0.999 gate, the wavefront re-evaluates with the bit-defined exponential, so every
 // decision is the one the forward took.
+#include <type_traits>
+
 #include "raster_device.h"
 
 namespace ssr {
@@ -293,6 +295,7 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
         __syncthreads();   // previous batch fully consumed (first pass: the zero fill of s_acc is complete)
         if (!first) flush();   // its sums leave before the slots are reused
         first = false;
+        bool near_cap = false;   // this thread's fragment can reach the 0.999 cap of alpha
         {
             // slot t holds sorted index hi - t: ascending t is back to front. Thread pair (slot, half) shares the staging.
             const int half = tid >= kB ? 1 : 0, slot = tid - half * kB;   // threads past 2 kB stage nothing
@@ -301,6 +304,7 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
             if (idx >= range_start && tid < 2 * kB) {
                 const int32_t g = g_ahead;
                 const FragLds f = stage_fragment_half(P.screen, P.packed_rows, g, tile_x0, tile_y0, half, bits8, P.block_masks ? P.block_masks + idx : nullptr);
+                near_cap = f.q1.y >= 0.9989f;
                 if (half == 0) {
                     s_ids[slot] = g; frags[slot] = f;
                     if constexpr (kDist != SSR_DIST_NONE) {
@@ -312,7 +316,9 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
             if (tid < 2 * kB) s_bits[half * kB + slot] = (uint8_t)bits8;
             if (idx - kB >= range_start && tid < 2 * kB) g_ahead = P.flatten_ids[idx - kB];
         }
-        __syncthreads();
+        // one answer per batch instead of a vote per step: batches without such a fragment (most) walk without the
+        // cap's operations
+        const bool sat_batch = __syncthreads_or(near_cap ? 1 : 0) != 0;
         // this wavefront's four lists: slots whose block bit is set and whose sorted index hi - slot is
         // not beyond the block's largest last_id
         const int n_batch = min(kB, hi - range_start + 1);
@@ -351,7 +357,9 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
         }
         // One step of a row: fragment k (registers q*) against the row's sixteen pixels.
         const int k_min = hi - bin_final;
-        auto step = [&](int st, int k, const float4& q0, const float4& q1, const float2& q2, float cut) {
+        uint64_t clash_run = clash_lo;   // bit 0: the step at hand
+        auto step = [&](auto sat_tag, int k, const float4& q0, const float4& q1, const float2& q2, float cut) {
+            constexpr bool kSat = decltype(sat_tag)::value;
             const float dx = q0.x - px, dy = q0.y - py;
             const float sigma = ssr_fma(q0.z * dx, dx, ssr_fma(q1.x * dy, dy, (q0.w * dx) * dy));
             // alpha > 1/255 <=> sigma < ln(255 opac) = cut - 1e-3 (fragment_constants): decided by comparing sigma, except
@@ -368,8 +376,7 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
             float vis = active ? __builtin_amdgcn_exp2f(sigma * -1.44269504088896341f) : 0.0f;
             float ov = q1.y * vis;
             uint64_t unsure = m_in & ~(m_lo | m_off);
-            const bool sat_possible = __builtin_amdgcn_ballot_w64(q1.y >= 0.9989f) != 0ull;
-            if (sat_possible) unsure |= __builtin_amdgcn_ballot_w64(ssr_fabs(ov - 0.999f) <= 4e-5f);
+            if constexpr (kSat) unsure |= __builtin_amdgcn_ballot_w64(ssr_fabs(ov - 0.999f) <= 4e-5f);
             float alpha = ov;
             if (unsure != 0ull) {   // decisions exactly as the forward took them
                 const bool in_range = in_list & !(sigma < 0.f || sigma > cut);
@@ -381,11 +388,11 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
                 active = alpha > kAlphaThreshold;
                 alpha = active ? alpha : 0.0f;
                 vis = (active & (ov <= 0.999f)) ? vis : 0.0f;   // evaluate_alpha_vjp gate (src/primitives/Primitive3DGS.cuh:273)
-            } else if (sat_possible) {
+            } else if constexpr (kSat) {
                 asm("v_min_f32 %0, %1, %2" : "=v"(alpha) : "s"(0.999f), "v"(ov));
                 vis = ov <= 0.999f ? vis : 0.0f;                // the same gate; without a fragment near the cap it never closes
             }
-            if (__builtin_amdgcn_ballot_w64(active) != 0ull) {
+            {   // (no vote on whether any lane is active: a step without one is rare, and the vote costs every step)
                 // inactive lanes run with alpha = 0 and vis = 0: T and v_T unchanged, every term zero
                 const float a = alpha;
                 const float T0 = T1 * __builtin_amdgcn_rcpf(1.0f - a);
@@ -495,7 +502,7 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
                 const float t0 = fold_pair<kDppQuadXor2>(s0, s1, b1), t1 = s2 + dpp_full<kDppQuadXor2>(s2);
                 const float fin_sum = fold_pair<kDppQuadXor1>(t0, t1, b0);
                 const bool mine = (chan >= 0) & ssr_isfinite(fin_sum) & (fin_sum != 0.0f);
-                const bool clash = (((st < 64 ? clash_lo : clash_hi) >> (st & 63)) & 1ull) != 0;
+                const bool clash = (clash_run & 1ull) != 0;
                 float* cell = reinterpret_cast<float*>(my_cells + __umul24((unsigned)k, 4u * kCh));
                 if (clash) { if (mine) atomicAdd(cell, fin_sum); }
                 else if (mine) *cell += fin_sum;
@@ -521,23 +528,29 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
         auto frag_of = [&](int k) -> const FragLds& {
             return *reinterpret_cast<const FragLds*>(reinterpret_cast<const char*>(frags) + __umul24((unsigned)k, (unsigned)sizeof(FragLds)));
         };
-        int k0 = list_at(0), k1 = list_at(1), k2 = list_at(2);
-        float4 a0 = frag_of(k0).q0, a1 = frag_of(k0).q1;
-        float2 a2 = make_float2(frag_of(k0).q2.x, frag_of(k0).q2.y);
-        float aw = frag_of(k0).q2.w;
-        for (int st = 0; st < n_steps; st += 2) {
-            const float4 c0 = frag_of(k1).q0, c1 = frag_of(k1).q1;
-            const float2 c2 = make_float2(frag_of(k1).q2.x, frag_of(k1).q2.y);
-            const float cw = frag_of(k1).q2.w;
-            const int k3 = list_at(st + 3);
-            step(st, k0, a0, a1, a2, aw);
-            a0 = frag_of(k2).q0; a1 = frag_of(k2).q1;
-            a2 = make_float2(frag_of(k2).q2.x, frag_of(k2).q2.y);
-            aw = frag_of(k2).q2.w;
-            const int k4 = list_at(st + 4);
-            if (st + 1 < n_steps) step(st + 1, k1, c0, c1, c2, cw);
-            k0 = k2; k1 = k3; k2 = k4;
-        }
+        auto walk = [&](auto sat_tag) {
+            int k0 = list_at(0), k1 = list_at(1), k2 = list_at(2);
+            float4 a0 = frag_of(k0).q0, a1 = frag_of(k0).q1;
+            float2 a2 = make_float2(frag_of(k0).q2.x, frag_of(k0).q2.y);
+            float aw = frag_of(k0).q2.w;
+            for (int st = 0; st < n_steps; st += 2) {
+                if (st == 64) clash_run = clash_hi;
+                const float4 c0 = frag_of(k1).q0, c1 = frag_of(k1).q1;
+                const float2 c2 = make_float2(frag_of(k1).q2.x, frag_of(k1).q2.y);
+                const float cw = frag_of(k1).q2.w;
+                const int k3 = list_at(st + 3);
+                step(sat_tag, k0, a0, a1, a2, aw);
+                clash_run >>= 1;
+                a0 = frag_of(k2).q0; a1 = frag_of(k2).q1;
+                a2 = make_float2(frag_of(k2).q2.x, frag_of(k2).q2.y);
+                aw = frag_of(k2).q2.w;
+                const int k4 = list_at(st + 4);
+                if (st + 1 < n_steps) step(sat_tag, k1, c0, c1, c2, cw);
+                clash_run >>= 1;
+                k0 = k2; k1 = k3; k2 = k4;
+            }
+        };
+        if (sat_batch) walk(std::true_type{}); else walk(std::false_type{});
     }
     lds_wait();   // as at the head of the loop
     __syncthreads();
