@@ -173,7 +173,8 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
     for (int e = tid; e < (int)sizeof(s_list); e += kRasterBlock) s_list[e] = (uint8_t)kB;
     if (tid == 0) {
         const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
-        frags[kB].q0 = z; frags[kB].q1 = z; frags[kB].q2 = z;
+        // the blank fragment: no opacity, and a conic that puts every pixel far beyond any band (its sigma is huge)
+        frags[kB].q0 = make_float4(0.f, 0.f, 1e30f, 0.f); frags[kB].q1 = z; frags[kB].q2 = z;
         if constexpr (kDist != SSR_DIST_NONE) { s_iz[kB] = 0.0f; s_lz[kB] = 0.0f; }
     }
     float* my_acc = s_acc + mt * (kB * kCh);
@@ -307,6 +308,8 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
                 near_cap = f.q1.y >= 0.9989f;
                 if (half == 0) {
                     s_ids[slot] = g; frags[slot] = f;
+                    // the lower edge of the band around sigma = ln(255 opac) = cut - 1e-3 in which the exact exponential decides
+                    frags[slot].q2.z = ssr_max(f.q2.w - 1.008e-3f, 0.0f);
                     if constexpr (kDist != SSR_DIST_NONE) {
                         s_lz[slot] = ssr_log(ssr_max(f.q2.y, 1e-6f));
                         s_iz[slot] = 1.0f / ssr_max(f.q2.y, 1e-6f);   // d/d ln z -> d/dz
@@ -358,7 +361,9 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
         // One step of a row: fragment k (registers q*) against the row's sixteen pixels.
         const int k_min = hi - bin_final;
         uint64_t clash_run = clash_lo;   // bit 0: the step at hand
-        auto step = [&](auto sat_tag, int k, const float4& q0, const float4& q1, const float2& q2, float cut) {
+        auto step = [&](auto sat_tag, int k, const float4& q0, const float4& q1, const float4& q2w) {
+            const float2 q2 = make_float2(q2w.x, q2w.y);
+            const float cut = q2w.w;
             constexpr bool kSat = decltype(sat_tag)::value;
             const float dx = q0.x - px, dy = q0.y - py;
             const float sigma = ssr_fma(q0.z * dx, dx, ssr_fma(q1.x * dy, dy, (q0.w * dx) * dy));
@@ -367,11 +372,11 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
             // comes within 4e-5 of the 0.999 cap, the wavefront re-evaluates with the bit-defined exponential, so that
             // every decision is the forward's. A lane on a fragment behind its pixel's last one (sorted index
             // hi - k > bin_final) is out; so is the blank fragment past the end of a list (cut 0: no sigma is below).
-            const uint32_t lo_bits = __float_as_uint(ssr_max(cut - 1.008e-3f, 0.0f));
+            const uint32_t lo_bits = __float_as_uint(q2w.z);   // max(cut - 1.008e-3, 0), left there when the fragment was staged
             const bool in_list = k >= k_min;
             const bool below = __float_as_uint(sigma) < lo_bits;      // 0 <= sigma < bound - band
             const uint64_t m_in = __builtin_amdgcn_ballot_w64(in_list), m_lo = __builtin_amdgcn_ballot_w64(below),
-                           m_off = __builtin_amdgcn_ballot_w64(sigma > cut - 0.992e-3f);
+                           m_off = __builtin_amdgcn_ballot_w64(sigma > q2w.z + 1.6e-5f);
             bool active = in_list & below;
             float vis = active ? __builtin_amdgcn_exp2f(sigma * -1.44269504088896341f) : 0.0f;
             float ov = q1.y * vis;
@@ -504,8 +509,10 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
                 const bool mine = (chan >= 0) & ssr_isfinite(fin_sum) & (fin_sum != 0.0f);
                 const bool clash = (clash_run & 1ull) != 0;
                 float* cell = reinterpret_cast<float*>(my_cells + __umul24((unsigned)k, 4u * kCh));
-                if (clash) { if (mine) atomicAdd(cell, fin_sum); }
-                else if (mine) *cell += fin_sum;
+                if (mine) {
+                    if (clash) atomicAdd(cell, fin_sum);
+                    else *cell += fin_sum;
+                }
                 if constexpr (kAccum == SSR_ACCUM_MAX) {   // inactive lanes contribute map * 0
                     float mx = amap * w;
                     mx = ssr_max(mx, dpp_full<0x128>(mx));   // row_ror:8
@@ -530,22 +537,16 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
         };
         auto walk = [&](auto sat_tag) {
             int k0 = list_at(0), k1 = list_at(1), k2 = list_at(2);
-            float4 a0 = frag_of(k0).q0, a1 = frag_of(k0).q1;
-            float2 a2 = make_float2(frag_of(k0).q2.x, frag_of(k0).q2.y);
-            float aw = frag_of(k0).q2.w;
+            float4 a0 = frag_of(k0).q0, a1 = frag_of(k0).q1, a2 = frag_of(k0).q2;
             for (int st = 0; st < n_steps; st += 2) {
                 if (st == 64) clash_run = clash_hi;
-                const float4 c0 = frag_of(k1).q0, c1 = frag_of(k1).q1;
-                const float2 c2 = make_float2(frag_of(k1).q2.x, frag_of(k1).q2.y);
-                const float cw = frag_of(k1).q2.w;
+                const float4 c0 = frag_of(k1).q0, c1 = frag_of(k1).q1, c2 = frag_of(k1).q2;
                 const int k3 = list_at(st + 3);
-                step(sat_tag, k0, a0, a1, a2, aw);
+                step(sat_tag, k0, a0, a1, a2);
                 clash_run >>= 1;
-                a0 = frag_of(k2).q0; a1 = frag_of(k2).q1;
-                a2 = make_float2(frag_of(k2).q2.x, frag_of(k2).q2.y);
-                aw = frag_of(k2).q2.w;
+                a0 = frag_of(k2).q0; a1 = frag_of(k2).q1; a2 = frag_of(k2).q2;
                 const int k4 = list_at(st + 4);
-                if (st + 1 < n_steps) step(sat_tag, k1, c0, c1, c2, cw);
+                if (st + 1 < n_steps) step(sat_tag, k1, c0, c1, c2);
                 clash_run >>= 1;
                 k0 = k2; k1 = k3; k2 = k4;
             }
