@@ -397,7 +397,11 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
                 asm("v_min_f32 %0, %1, %2" : "=v"(alpha) : "s"(0.999f), "v"(ov));
                 vis = ov <= 0.999f ? vis : 0.0f;                // the same gate; without a fragment near the cap it never closes
             }
-            {   // (no vote on whether any lane is active: a step without one is rare, and the vote costs every step)
+            // no vote on whether any lane is active (a step without one is rare, and the vote costs every step), except
+            // with the median, whose step is long enough for the vote to pay
+            bool any_active = true;
+            if constexpr (kMedian) any_active = __builtin_amdgcn_ballot_w64(active) != 0ull;
+            if (any_active) {
                 // inactive lanes run with alpha = 0 and vis = 0: T and v_T unchanged, every term zero
                 const float a = alpha;
                 const float T0 = T1 * __builtin_amdgcn_rcpf(1.0f - a);
@@ -551,7 +555,10 @@ __device__ __forceinline__ void raster_bwd_rows_body(const ssr_raster_bwd_params
                 k0 = k2; k1 = k3; k2 = k4;
             }
         };
-        if (sat_batch) walk(std::true_type{}); else walk(std::false_type{});
+        // (the median variants keep one instantiation, with the cap's operations: two cost them a wavefront per SIMD)
+        if constexpr (kMedian) walk(std::true_type{});
+        else if (sat_batch) walk(std::true_type{});
+        else walk(std::false_type{});
     }
     lds_wait();   // as at the head of the loop
     __syncthreads();
@@ -568,6 +575,12 @@ __global__ __launch_bounds__(kRasterBlock) void raster_bwd_rows_kernel(ssr_raste
 __global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(5))) void raster_bwd_rows_avg_kernel(
     ssr_raster_bwd_params P, int tile_w, int tile_h) {
     raster_bwd_rows_body<SSR_DIST_NONE, false, SSR_ACCUM_AVG>(P, tile_w, tile_h);
+}
+
+// The plain median likewise (106 registers without the limit).
+__global__ __launch_bounds__(kRasterBlock) __attribute__((amdgpu_waves_per_eu(5))) void raster_bwd_rows_median_kernel(
+    ssr_raster_bwd_params P, int tile_w, int tile_h) {
+    raster_bwd_rows_body<SSR_DIST_NONE, true, SSR_ACCUM_NONE>(P, tile_w, tile_h);
 }
 
 // Moves the weight sums that raster_bwd_rows_kernel left in floats 10 and 11 of the gradient rows to the weight
@@ -645,6 +658,8 @@ extern "C" int ssr_raster_bwd(const ssr_raster_bwd_params* p, ssr_stream_t strea
         launch_raster_bwd_lanes(*p, tw, th, nimg, st);
     else if (p->dist_type == SSR_DIST_NONE && !med && p->accum_mode == SSR_ACCUM_AVG)
         hipLaunchKernelGGL(raster_bwd_rows_avg_kernel, grid, block, 0, st, *p, tw, th);
+    else if (p->dist_type == SSR_DIST_NONE && med && p->accum_mode == SSR_ACCUM_NONE)
+        hipLaunchKernelGGL(raster_bwd_rows_median_kernel, grid, block, 0, st, *p, tw, th);
     else switch (p->dist_type) {
         case SSR_DIST_D: SSR_ROWS_M(SSR_DIST_D); break;
         case SSR_DIST_RGB_D: SSR_ROWS_M(SSR_DIST_RGB_D); break;
