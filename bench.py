@@ -458,7 +458,7 @@ def main():
                 r = out
             else:
                 a2 = copy.copy(args)
-                a2.config, a2.steps, a2.warmup = c, min(args.steps, 10), min(args.warmup, 2)
+                a2.config, a2.steps, a2.warmup = c, min(args.steps, 20), min(args.warmup, 5)
                 r = run_config(a2, pkg, host, lib, np, with_cpu=False)
             dom = r["roofline"]["kernel"]
             rows.append({"workload": r["config"]["workload"], "ms_per_step": r["ms_per_step"], "iters_per_s": r["value"],
